@@ -1,0 +1,293 @@
+"""ctypes binding of the CPU oracle (``libfnn_oracle.so``).
+
+TEST INFRASTRUCTURE ONLY.  Only ``tests/``, ``__graft_entry__.smoke()`` and the
+``cpu_baseline`` leg of ``bench.py`` may import this module; the shipped package
+never does.  It is the checker, not the thing measured or shipped.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+from dataclasses import dataclass, field
+from typing import Optional
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "libfnn_oracle.so")
+
+I8, I4, U8, U4, F8, F8R, F4, I4CB = range(8)
+ACT_NONE, ACT_RELU, ACT_GELU, ACT_SILU = range(4)
+DT_NAMES = {I8: "i8", I4: "i4", U8: "u8", U4: "u4", F8: "f8", F8R: "f8r", F4: "f4", I4CB: "i4cb"}
+MARGIN = 16
+
+
+def build(force: bool = False) -> str:
+    """Compile the oracle with gcc (strict IEEE flags live in the Makefile)."""
+    src = os.path.join(_HERE, "fnn_oracle.c")
+    if force or not os.path.exists(_SO) or os.path.getmtime(_SO) < os.path.getmtime(src):
+        subprocess.run(["make", "-C", _HERE, "-B", "libfnn_oracle.so"], check=True,
+                       stdout=subprocess.DEVNULL)
+    return _SO
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_SO):
+            build()
+        _lib = C.CDLL(_SO)
+        _proto(_lib)
+    return _lib
+
+
+_f32p = np.ctypeslib.ndpointer(dtype=np.float32, flags="C_CONTIGUOUS")
+_u32p = np.ctypeslib.ndpointer(dtype=np.uint32, flags="C_CONTIGUOUS")
+_u8p = np.ctypeslib.ndpointer(dtype=np.uint8, flags="C_CONTIGUOUS")
+_i32p = np.ctypeslib.ndpointer(dtype=np.int32, flags="C_CONTIGUOUS")
+_sz = C.c_size_t
+
+
+def _proto(l):
+    l.fnn_or_items.argtypes = [C.c_int]
+    l.fnn_or_unpack_word.argtypes = [C.c_int, C.c_uint32, _f32p]
+    l.fnn_or_pack_word.argtypes = [C.c_int, _f32p]
+    l.fnn_or_pack_word.restype = C.c_uint32
+    for n in ("e4m3", "e5m2"):
+        getattr(l, f"fnn_or_{n}_to_f32").argtypes = [C.c_uint8]
+        getattr(l, f"fnn_or_{n}_to_f32").restype = C.c_float
+        getattr(l, f"fnn_or_f32_to_{n}").argtypes = [C.c_float]
+        getattr(l, f"fnn_or_f32_to_{n}").restype = C.c_uint8
+    l.fnn_or_fp4_to_f32.argtypes = [C.c_uint8]
+    l.fnn_or_fp4_to_f32.restype = C.c_float
+    l.fnn_or_f32_to_fp4.argtypes = [C.c_float]
+    l.fnn_or_f32_to_fp4.restype = C.c_uint8
+    for n in ("i8x4_dot", "i4x8_dot", "f4x8_dot"):
+        getattr(l, f"fnn_or_{n}").argtypes = [C.c_uint32, C.c_uint32]
+        getattr(l, f"fnn_or_{n}").restype = C.c_int32
+    for n in ("i8x4_sum", "i4x8_sum"):
+        getattr(l, f"fnn_or_{n}").argtypes = [C.c_uint32]
+        getattr(l, f"fnn_or_{n}").restype = C.c_int32
+    l.fnn_or_packed_words.argtypes = [C.c_int, _sz, _sz]
+    l.fnn_or_packed_words.restype = _sz
+    l.fnn_or_from_f32_slice.argtypes = [C.c_int, _f32p, _sz, _sz, C.c_float, C.c_float, _u32p]
+    l.fnn_or_quant_per_channel_asym.argtypes = [C.c_int, _f32p, _sz, _sz, _u32p, _f32p, _f32p]
+    l.fnn_or_quant_per_channel_sym.argtypes = [C.c_int, _f32p, _sz, _sz, _u32p, _f32p, _f32p]
+    l.fnn_or_kmeans16.argtypes = [_f32p, _sz, C.c_int, _f32p]
+    l.fnn_or_quant_codebook.argtypes = [_f32p, _sz, _sz, _sz, _u32p, _f32p, _f32p]
+    l.fnn_or_transpose.argtypes = [_f32p, _sz, _sz, _f32p]
+    l.fnn_or_dequant.argtypes = [C.c_int, _u32p, _sz, _sz, C.c_void_p, _sz, C.c_void_p, _sz, _sz,
+                                 C.c_void_p, _f32p]
+    l.fnn_or_qmatmul.argtypes = [C.c_int, _u32p, _sz, _sz, C.c_void_p, _sz, C.c_void_p, _sz, _sz,
+                                 C.c_void_p, _f32p, _sz, _f32p, C.c_int, _sz, C.c_int]
+    l.fnn_or_bias_act.argtypes = [_f32p, _sz, _sz, C.c_void_p, C.c_int]
+    l.fnn_or_act.argtypes = [C.c_float, C.c_int]
+    l.fnn_or_act.restype = C.c_float
+    l.fnn_or_quantize_activations.argtypes = [_f32p, _sz, _u8p]
+    l.fnn_or_quantize_activations_calibrated.argtypes = [_f32p, _sz, C.c_float, C.c_float, _u8p]
+    l.fnn_or_qmatmul_i8act.argtypes = [C.c_int, _u32p, _sz, _sz, C.c_void_p, _sz, C.c_void_p, _sz,
+                                       _u8p, _sz, _sz, _f32p, C.c_void_p]
+    l.fnn_or_conv_out_size.argtypes = [_sz] * 5
+    l.fnn_or_conv_out_size.restype = _sz
+    l.fnn_or_qconv2d_i8.argtypes = [_f32p, _sz, _sz, _sz, _sz, _u32p, _sz, C.c_void_p, _sz,
+                                    C.c_void_p, _sz, C.c_void_p, _sz, _sz, _sz, _sz, _sz, _sz,
+                                    C.c_int, _f32p, C.c_void_p, C.c_void_p, C.c_void_p]
+    l.fnn_or_seeded_values.argtypes = [C.c_uint64, _sz, _f32p]
+
+
+def _ptr(a: Optional[np.ndarray]):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+def _f32(a) -> np.ndarray:
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+@dataclass
+class Packed:
+    """A packed weight as fastnn's PackedTensor holds it (packed_tensor.rs:95-126)."""
+    dt: int
+    rows: int
+    inner: int
+    words: np.ndarray                   # uint32, rows*ceil(inner/ITEMS) + 16
+    scales: np.ndarray                  # float32
+    zeros: np.ndarray                   # float32 (empty for the codebook type)
+    qblock: int = 0
+    codebook: Optional[np.ndarray] = None
+    extra: dict = field(default_factory=dict)
+
+    @property
+    def items(self) -> int:
+        return items(self.dt)
+
+    @property
+    def words_per_row(self) -> int:
+        return -(-self.inner // self.items)
+
+
+def items(dt: int) -> int:
+    return lib().fnn_or_items(dt)
+
+
+def unpack_word(dt: int, w: int) -> np.ndarray:
+    out = np.zeros(8, np.float32)
+    lib().fnn_or_unpack_word(dt, w & 0xFFFFFFFF, out)
+    return out[: items(dt)]
+
+
+def pack_word(dt: int, vals) -> int:
+    v = np.zeros(8, np.float32)
+    v[: len(vals)] = vals
+    return int(lib().fnn_or_pack_word(dt, v))
+
+
+def seeded_values(seed: int, n: int) -> np.ndarray:
+    out = np.zeros(n, np.float32)
+    lib().fnn_or_seeded_values(seed, n, out)
+    return out
+
+
+def from_f32_slice(dt: int, data, rows: int, inner: int, scale: float, zero: float) -> Packed:
+    data = _f32(data).reshape(-1)
+    words = np.zeros(lib().fnn_or_packed_words(dt, rows, inner), np.uint32)
+    lib().fnn_or_from_f32_slice(dt, data, rows, inner, scale, zero, words)
+    return Packed(dt, rows, inner, words, np.array([scale], np.float32),
+                  np.array([zero], np.float32))
+
+
+def quantize(dt: int, w_nk, qblock: int = 32) -> Packed:
+    """Quantise an [N,K] f32 matrix the way the reference's pass does for `dt`
+    (quantization.rs:170-260 integer types, :281-495 float/codebook types)."""
+    w = _f32(w_nk)
+    rows, inner = w.shape
+    flat = w.reshape(-1)
+    words = np.zeros(lib().fnn_or_packed_words(dt, rows, inner), np.uint32)
+    if dt == I4CB:
+        bpr = -(-inner // qblock)
+        scales = np.zeros(rows * bpr, np.float32)
+        cb = np.zeros(16, np.float32)
+        rc = lib().fnn_or_quant_codebook(flat, rows, inner, qblock, words, scales, cb)
+        if rc:
+            raise ValueError(f"codebook quantiser failed rc={rc}")
+        return Packed(dt, rows, inner, words, scales, np.zeros(0, np.float32), qblock, cb)
+    scales = np.zeros(rows, np.float32)
+    zeros = np.zeros(rows, np.float32)
+    if dt in (F8, F8R):
+        lib().fnn_or_quant_per_channel_sym(dt, flat, rows, inner, words, scales, zeros)
+    else:
+        lib().fnn_or_quant_per_channel_asym(dt, flat, rows, inner, words, scales, zeros)
+    return Packed(dt, rows, inner, words, scales, zeros)
+
+
+def quantize_kn(dt: int, w_kn, qblock: int = 32) -> Packed:
+    """Logical [K,N] weight -> transposed [N,K] -> packed (quantization.rs:144-156)."""
+    w = _f32(w_kn)
+    k, n = w.shape
+    t = np.zeros((n, k), np.float32)
+    lib().fnn_or_transpose(w.reshape(-1), k, n, t.reshape(-1))
+    return quantize(dt, t, qblock)
+
+
+def kmeans16(values, iters: int = 30) -> np.ndarray:
+    v = _f32(values).reshape(-1)
+    out = np.zeros(16, np.float32)
+    rc = lib().fnn_or_kmeans16(v, v.size, iters, out)
+    if rc:
+        raise ValueError(f"kmeans16 rc={rc}")
+    return out
+
+
+def dequant(p: Packed) -> np.ndarray:
+    out = np.zeros((p.rows, p.inner), np.float32)
+    rc = lib().fnn_or_dequant(p.dt, p.words, p.rows, p.inner, _ptr(p.scales), p.scales.size,
+                              _ptr(p.zeros) if p.zeros.size else None, p.zeros.size, p.qblock,
+                              _ptr(p.codebook), out.reshape(-1))
+    if rc:
+        raise ValueError(f"dequant rc={rc}")
+    return out
+
+
+def qmatmul(p: Packed, a, order: int = 2, k_tile: int = 0, bias=None, act: int = ACT_NONE,
+            i4cb_as_written: bool = False) -> np.ndarray:
+    """out[M,N] = act(A . deq(W)^T + bias); order 0 scalar f32, 1 AVX2-order f32, 2 f64 accumulate."""
+    a = _f32(a)
+    m, k = a.shape
+    assert k == p.inner
+    out = np.zeros((m, p.rows), np.float32)
+    rc = lib().fnn_or_qmatmul(p.dt, p.words, p.rows, k, _ptr(p.scales), p.scales.size,
+                              _ptr(p.zeros) if p.zeros.size else None, p.zeros.size, p.qblock,
+                              _ptr(p.codebook), a.reshape(-1), m, out.reshape(-1), order, k_tile,
+                              int(i4cb_as_written))
+    if rc:
+        raise ValueError(f"qmatmul rc={rc}")
+    if bias is not None or act != ACT_NONE:
+        b = None if bias is None else _f32(bias)
+        lib().fnn_or_bias_act(out.reshape(-1), m, p.rows, _ptr(b), act)
+    return out
+
+
+def act_fn(x: np.ndarray, act: int) -> np.ndarray:
+    x = _f32(x).copy()
+    lib().fnn_or_bias_act(x.reshape(-1), 1, x.size, None, act)
+    return x
+
+
+def quantize_activations(x, scale: Optional[float] = None, zp: float = 0.0) -> np.ndarray:
+    x = _f32(x).reshape(-1)
+    payload = np.zeros(8 + x.size, np.uint8)
+    if scale is None:
+        lib().fnn_or_quantize_activations(x, x.size, payload)
+    else:
+        lib().fnn_or_quantize_activations_calibrated(x, x.size, scale, zp, payload)
+    return payload
+
+
+def make_payload(scale: float, zp: float, q_i8) -> np.ndarray:
+    q = np.asarray(q_i8, dtype=np.int8).reshape(-1)
+    payload = np.zeros(8 + q.size, np.uint8)
+    payload[0:4] = np.frombuffer(np.float32(scale).tobytes(), np.uint8)
+    payload[4:8] = np.frombuffer(np.float32(zp).tobytes(), np.uint8)
+    payload[8:] = q.view(np.uint8)
+    return payload
+
+
+def qmatmul_i8act(p: Packed, payload: np.ndarray, m: int, want_acc: bool = False):
+    out = np.zeros((m, p.rows), np.float32)
+    acc = np.zeros((m, p.rows), np.int32) if want_acc else None
+    rc = lib().fnn_or_qmatmul_i8act(p.dt, p.words, p.rows, p.inner, _ptr(p.scales), p.scales.size,
+                                    _ptr(p.zeros) if p.zeros.size else None, p.zeros.size,
+                                    payload, payload.size, m, out.reshape(-1), _ptr(acc))
+    if rc:
+        raise ValueError(f"qmatmul_i8act rc={rc}")
+    return (out, acc) if want_acc else out
+
+
+def conv_out_size(inp, kernel, stride, pad, dil) -> int:
+    return int(lib().fnn_or_conv_out_size(inp, kernel, stride, pad, dil))
+
+
+def qconv2d_i8(x, p: Packed, kh: int, kw: int, stride: int, pad: int, dil: int, groups: int,
+               bias=None, act: int = ACT_NONE, want_acc: bool = False):
+    """x NCHW f32; p packed [OC, C/g*KH*KW] I8 weights."""
+    x = _f32(x)
+    b, c, h, w = x.shape
+    oc = p.rows
+    ho, wo = conv_out_size(h, kh, stride, pad, dil), conv_out_size(w, kw, stride, pad, dil)
+    y = np.zeros((b, oc, ho, wo), np.float32)
+    acc = np.zeros((b, oc, ho, wo), np.int32) if want_acc else None
+    sa = np.zeros(b * groups, np.float32)
+    za = np.zeros(b * groups, np.float32)
+    bb = None if bias is None else _f32(bias)
+    rc = lib().fnn_or_qconv2d_i8(x.reshape(-1), b, c, h, w, p.words, oc, _ptr(p.scales),
+                                 p.scales.size, _ptr(p.zeros), p.zeros.size, _ptr(bb), kh, kw,
+                                 stride, pad, dil, groups, act, y.reshape(-1), _ptr(acc),
+                                 _ptr(sa), _ptr(za))
+    if rc:
+        raise ValueError(f"qconv2d_i8 rc={rc}")
+    if want_acc:
+        return y, acc, sa, za
+    return y

@@ -1,0 +1,81 @@
+"""Pins the oracle's quantised Conv2d lowering: equals a float64 convolution of the
+dequantised operands, integer accumulators equal an exact integer convolution, and the
+im2col index formula is checked against torch's unfold."""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+
+def _qw(p, k):
+    kp = -(-k // 4)
+    w = p.words[: p.rows * kp].view(np.int8).reshape(p.rows, kp * 4)[:, :k]
+    return w.astype(np.int64)
+
+
+@pytest.mark.parametrize("cfg", [
+    dict(b=2, c=3, h=9, w=11, oc=4, kh=3, kw=3, stride=2, pad=1, dil=1, groups=1),
+    dict(b=1, c=4, h=8, w=8, oc=6, kh=1, kw=1, stride=1, pad=0, dil=1, groups=1),
+    dict(b=1, c=4, h=10, w=7, oc=4, kh=3, kw=2, stride=1, pad=2, dil=2, groups=2),
+    dict(b=1, c=5, h=6, w=6, oc=3, kh=3, kw=3, stride=1, pad=1, dil=1, groups=1),
+])
+@pytest.mark.parametrize("act", [0, 1, 3])
+def test_conv_matches_float_conv_of_dequantised(orc, cfg, act):
+    rng = np.random.default_rng(300)
+    b, c, h, w, oc, kh, kw = (cfg[x] for x in ("b", "c", "h", "w", "oc", "kh", "kw"))
+    stride, pad, dil, groups = cfg["stride"], cfg["pad"], cfg["dil"], cfg["groups"]
+    cg = c // groups
+    kk = cg * kh * kw
+    x = rng.uniform(0, 1, (b, c, h, w)).astype(np.float32)
+    wt = (rng.standard_normal((oc, kk)) * 0.1).astype(np.float32)
+    bias = (rng.standard_normal(oc) * 0.05).astype(np.float32)
+    p = orc.quantize(orc.I8, wt)
+    y, acc, sa, za = orc.qconv2d_i8(x, p, kh, kw, stride, pad, dil, groups, bias=bias, act=act, want_acc=True)
+    qw = _qw(p, kk)
+    ocg = oc // groups
+    for n in range(b):
+        for g in range(groups):
+            xs = torch.from_numpy(x[n:n + 1, g * cg:(g + 1) * cg].astype(np.float64))
+            col = F.unfold(xs, (kh, kw), dilation=dil, padding=pad, stride=stride)[0].numpy().T  # [P, K]
+            mn, mx = np.float32(col.min()), np.float32(col.max())
+            s = sa[n * groups + g]
+            z = za[n * groups + g]
+            assert s == np.float32(mx - mn) / np.float32(255.0)
+            assert z == np.float32(mn + np.float32(128.0) * s)
+            inv = np.float32(1.0) / s
+            t = (col.astype(np.float32) - z) * inv
+            qa = np.clip(np.sign(t) * np.floor(np.abs(t) + np.float32(0.5)), -128, 127).astype(np.int64)
+            for f in range(ocg):
+                ch = g * ocg + f
+                sab = np.float32(s * p.scales[ch])
+                bq = int(np.sign(bias[ch] / sab) * np.floor(abs(np.float32(bias[ch] / sab)) + 0.5))
+                want_acc = qa @ qw[ch] + bq
+                assert np.array_equal(acc[n, ch].reshape(-1), want_acc.astype(np.int32))
+                # float meaning: conv of dequantised operands + dequantised bias
+                da = qa * float(s) + float(z)
+                dw = qw[ch] * float(p.scales[ch]) + float(p.zeros[ch])
+                val = da @ dw + bq * float(sab)
+                if act == 1:
+                    val = np.maximum(val, 0)
+                elif act == 3:
+                    val = val / (1 + np.exp(-val))
+                got = y[n, ch].reshape(-1)
+                assert np.abs(got - val).max() <= 1e-4 * (np.abs(val).max() + 1), (cfg, ch)
+
+
+def test_conv_out_size(orc):
+    for (i, k, s, p, d) in [(640, 3, 2, 1, 1), (7, 3, 1, 0, 1), (5, 3, 1, 0, 3), (2, 5, 1, 0, 1), (8, 1, 1, 0, 1)]:
+        dk = (k - 1) * d + 1
+        want = (i + 2 * p - dk) // s + 1 if i + 2 * p >= dk else 0
+        assert orc.conv_out_size(i, k, s, p, d) == want
+
+
+def test_conv_constant_input_has_unit_scale(orc):
+    x = np.full((1, 2, 4, 4), 0.5, np.float32)
+    wt = np.ones((2, 2), np.float32) * 0.1
+    wt[0, 0] = -0.2
+    p = orc.quantize(orc.I8, wt)
+    y, acc, sa, za = orc.qconv2d_i8(x, p, 1, 1, 1, 0, 1, 1, want_acc=True)
+    assert sa[0] == 1.0 and za[0] == 0.0  # zero range -> scale 1, zero 0; 0.5 rounds to 1
+    deq = orc.dequant(p)
+    assert np.allclose(y[0, :, 0, 0], deq.sum(axis=1), atol=1e-5)
