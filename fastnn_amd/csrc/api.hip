@@ -1,0 +1,641 @@
+// C ABI of libfastnn_hip.so: context, device arena helpers, weight registry and the
+// entry points that enqueue the quantised MatMul / Conv2d kernels on the context's stream.
+// No exception or abort crosses this boundary; every failure becomes a status code plus a
+// message kept on the context.
+#include "common.h"
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <new>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "i8act.h"
+#include "mfma.h"
+
+struct fnn_hip_graph {
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+};
+
+struct Staging {
+    void *ptr = nullptr;
+    size_t cap = 0;
+};
+
+struct fnn_hip_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    std::string err;
+    std::unordered_map<uint64_t, fnn_hip_weight *> weights;
+    Staging st_a, st_out, st_bias, st_acc, st_tmp, st_tmp2;
+    float *scratch = nullptr;  // small reduction scratch (partials)
+    bool capturing = false;
+};
+
+namespace {
+
+thread_local std::string g_err;  // failures without a context
+
+int fail(fnn_hip_ctx *ctx, int code, const char *fmt, ...)
+{
+    char buf[1024];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    if (ctx) ctx->err = buf; else g_err = buf;
+    return code;
+}
+
+#define HIP_TRY(ctx, code, expr)                                                              \
+    do {                                                                                      \
+        hipError_t e__ = (expr);                                                              \
+        if (e__ != hipSuccess)                                                                \
+            return fail(ctx, code, "%s failed: %s", #expr, hipGetErrorString(e__));           \
+    } while (0)
+
+int ensure(fnn_hip_ctx *ctx, Staging &s, size_t bytes)
+{
+    if (bytes <= s.cap && s.ptr) return FNN_OK;
+    if (ctx->capturing) return fail(ctx, FNN_ERR_MEMORY, "staging growth during graph capture");
+    if (s.ptr) {
+        HIP_TRY(ctx, FNN_ERR_MEMORY, hipStreamSynchronize(ctx->stream));
+        HIP_TRY(ctx, FNN_ERR_MEMORY, hipFree(s.ptr));
+        s.ptr = nullptr;
+        s.cap = 0;
+    }
+    size_t cap = bytes < 4096 ? 4096 : bytes;
+    HIP_TRY(ctx, FNN_ERR_MEMORY, hipMalloc(&s.ptr, cap));
+    s.cap = cap;
+    return FNN_OK;
+}
+
+int items_of(int dt)
+{
+    switch (dt) {
+    case FNN_DT_I8: case FNN_DT_U8: case FNN_DT_F8: case FNN_DT_F8R: return 4;
+    case FNN_DT_I4: case FNN_DT_U4: case FNN_DT_F4: case FNN_DT_I4CB: return 8;
+    default: return 0;
+    }
+}
+
+const char *kernel_name_of(int dt)
+{
+    switch (dt) {
+    case FNN_DT_I8: return "matmul_i8";
+    case FNN_DT_I4: return "matmul_i4";
+    case FNN_DT_U8: return "matmul_u8";
+    case FNN_DT_U4: return "matmul_u4";
+    case FNN_DT_F8: return "matmul_f8";
+    case FNN_DT_F8R: return "matmul_f8r";
+    case FNN_DT_F4: return "matmul_f4";
+    case FNN_DT_I4CB: return "matmul_i4";
+    default: return "matmul_?";
+    }
+}
+
+void free_weight(fnn_hip_weight *w)
+{
+    if (!w) return;
+    if (w->words) (void)hipFree(w->words);
+    if (w->scales) (void)hipFree(w->scales);
+    if (w->zeros) (void)hipFree(w->zeros);
+    if (w->codebook) (void)hipFree(w->codebook);
+    if (w->row_qsum) (void)hipFree(w->row_qsum);
+    delete w;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *fnn_hip_version(void) { return "fastnn-hip 0.1 (gfx950)"; }
+
+int fnn_hip_device_count(void)
+{
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) return 0;
+    return n;
+}
+
+int fnn_hip_create(int device, fnn_hip_ctx **out)
+{
+    if (!out) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_hip_create: out is NULL");
+    *out = nullptr;
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess || n <= 0)
+        return fail(nullptr, FNN_ERR_MEMORY, "fnn_hip_create: no HIP device (%s)",
+                    e == hipSuccess ? "count 0" : hipGetErrorString(e));
+    if (device < 0 || device >= n)
+        return fail(nullptr, FNN_ERR_DISPATCH, "fnn_hip_create: device %d out of range [0,%d)", device, n);
+    fnn_hip_ctx *ctx = new (std::nothrow) fnn_hip_ctx();
+    if (!ctx) return fail(nullptr, FNN_ERR_MEMORY, "fnn_hip_create: out of host memory");
+    ctx->device = device;
+    if ((e = hipSetDevice(device)) != hipSuccess ||
+        (e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking)) != hipSuccess ||
+        (e = hipEventCreate(&ctx->ev0)) != hipSuccess || (e = hipEventCreate(&ctx->ev1)) != hipSuccess ||
+        (e = hipMalloc((void **)&ctx->scratch, 64 * 1024)) != hipSuccess) {
+        int rc = fail(nullptr, FNN_ERR_MEMORY, "fnn_hip_create: %s", hipGetErrorString(e));
+        fnn_hip_destroy(ctx);
+        return rc;
+    }
+    *out = ctx;
+    return FNN_OK;
+}
+
+void fnn_hip_destroy(fnn_hip_ctx *ctx)
+{
+    if (!ctx) return;
+    (void)hipSetDevice(ctx->device);
+    if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
+    for (auto &kv : ctx->weights) free_weight(kv.second);
+    for (Staging *s : {&ctx->st_a, &ctx->st_out, &ctx->st_bias, &ctx->st_acc, &ctx->st_tmp, &ctx->st_tmp2})
+        if (s->ptr) (void)hipFree(s->ptr);
+    if (ctx->scratch) (void)hipFree(ctx->scratch);
+    if (ctx->ev0) (void)hipEventDestroy(ctx->ev0);
+    if (ctx->ev1) (void)hipEventDestroy(ctx->ev1);
+    if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
+    delete ctx;
+}
+
+const char *fnn_hip_last_error(fnn_hip_ctx *ctx) { return ctx ? ctx->err.c_str() : g_err.c_str(); }
+
+int fnn_hip_sync(fnn_hip_ctx *ctx)
+{
+    if (!ctx) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_hip_sync: NULL context");
+    HIP_TRY(ctx, FNN_ERR_DISPATCH, hipStreamSynchronize(ctx->stream));
+    return FNN_OK;
+}
+
+int fnn_hip_malloc(fnn_hip_ctx *ctx, size_t bytes, void **dptr)
+{
+    if (!ctx || !dptr) return fail(ctx, FNN_ERR_MEMORY, "fnn_hip_malloc: NULL argument");
+    *dptr = nullptr;
+    HIP_TRY(ctx, FNN_ERR_MEMORY, hipSetDevice(ctx->device));
+    HIP_TRY(ctx, FNN_ERR_MEMORY, hipMalloc(dptr, bytes ? bytes : 1));
+    return FNN_OK;
+}
+
+int fnn_hip_free(fnn_hip_ctx *ctx, void *dptr)
+{
+    if (!ctx) return fail(nullptr, FNN_ERR_MEMORY, "fnn_hip_free: NULL context");
+    if (!dptr) return FNN_OK;
+    HIP_TRY(ctx, FNN_ERR_MEMORY, hipStreamSynchronize(ctx->stream));
+    HIP_TRY(ctx, FNN_ERR_MEMORY, hipFree(dptr));
+    return FNN_OK;
+}
+
+int fnn_hip_upload(fnn_hip_ctx *ctx, void *dst, const void *src, size_t bytes)
+{
+    if (!ctx || (bytes && (!dst || !src))) return fail(ctx, FNN_ERR_MEMORY, "fnn_hip_upload: NULL argument");
+    if (!bytes) return FNN_OK;
+    HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx->stream));
+    HIP_TRY(ctx, FNN_ERR_MEMORY, hipStreamSynchronize(ctx->stream));
+    return FNN_OK;
+}
+
+int fnn_hip_download(fnn_hip_ctx *ctx, void *dst, const void *src, size_t bytes)
+{
+    if (!ctx || (bytes && (!dst || !src))) return fail(ctx, FNN_ERR_MEMORY, "fnn_hip_download: NULL argument");
+    if (!bytes) return FNN_OK;
+    HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx->stream));
+    HIP_TRY(ctx, FNN_ERR_MEMORY, hipStreamSynchronize(ctx->stream));
+    return FNN_OK;
+}
+
+// Validation mirrors packed_tensor_from_meta (src/backend/cpu/matmul.rs:81-152).
+int fnn_hip_weight_register(fnn_hip_ctx *ctx, uint64_t key, int dtype, const uint32_t *words,
+                            size_t n_words, int64_t rows, int64_t inner, const float *scales,
+                            size_t n_scales, const float *zeros, size_t n_zeros,
+                            int quant_block_size, const float *codebook16, fnn_hip_weight **out)
+{
+    if (!ctx) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_hip_weight_register: NULL context");
+    if (out) *out = nullptr;
+    if (codebook16 && dtype == FNN_DT_I4) dtype = FNN_DT_I4CB;
+    const int items = items_of(dtype);
+    const char *kn = kernel_name_of(dtype);
+    if (!items) return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "unsupported packed dtype %d", dtype);
+    if (rows <= 0 || inner <= 0)
+        return fail(ctx, FNN_ERR_DISPATCH, "%s: invalid weight shape [%lld, %lld]", kn, (long long)rows, (long long)inner);
+    if (!scales || n_scales == 0)
+        return fail(ctx, FNN_ERR_DISPATCH, "%s: quantized weight metadata missing scales", kn);
+    if (n_zeros != 0 && n_zeros != n_scales && dtype != FNN_DT_I4CB)
+        return fail(ctx, FNN_ERR_DISPATCH,
+                    "%s: quantized weight metadata length mismatch: %zu scales vs %zu zero_points", kn,
+                    n_scales, n_zeros);
+    if (n_zeros != 0 && !zeros)
+        return fail(ctx, FNN_ERR_DISPATCH, "%s: zero_points pointer is NULL", kn);
+    const size_t urows = (size_t)rows;
+    const bool valid_len = n_scales == 1 || n_scales == urows ||
+                           (n_scales > 1 && urows > n_scales && urows % n_scales == 0) ||
+                           (quant_block_size > 0 && n_scales > urows && n_scales % urows == 0);
+    if (!valid_len)
+        return fail(ctx, FNN_ERR_DISPATCH,
+                    "%s: quantized weight metadata length %zu incompatible with shape [%lld, %lld] "
+                    "(expected 1, %lld, or a divisor of %lld)",
+                    kn, n_scales, (long long)rows, (long long)inner, (long long)rows, (long long)rows);
+    const int64_t kp = (inner + items - 1) / items;
+    const size_t expected = (size_t)(rows * kp);
+    if (!words || n_words < expected)
+        return fail(ctx, FNN_ERR_DISPATCH,
+                    "%s: quantized weight payload too short: got %zu packed words for shape [%lld, %lld], "
+                    "expected at least %zu",
+                    kn, words ? n_words : (size_t)0, (long long)rows, (long long)inner, expected);
+    int64_t bpr = 0;
+    if (dtype == FNN_DT_I4CB) {
+        if (!codebook16) return fail(ctx, FNN_ERR_DISPATCH, "%s: codebook weight without codebook", kn);
+        if (quant_block_size <= 0)
+            return fail(ctx, FNN_ERR_DISPATCH, "%s: codebook weight needs quant_block_size > 0", kn);
+        bpr = (inner + quant_block_size - 1) / quant_block_size;
+        if (n_scales < (size_t)(rows * bpr))
+            return fail(ctx, FNN_ERR_DISPATCH, "%s: codebook weight needs %lld block scales, got %zu", kn,
+                        (long long)(rows * bpr), n_scales);
+    } else if (quant_block_size > 0 && n_scales > urows) {
+        return fail(ctx, FNN_ERR_UNSUPPORTED_OP,
+                    "%s: per-block scales without a codebook are not produced by the quantisation pass", kn);
+    }
+    if (ctx->weights.count(key))
+        return fail(ctx, FNN_ERR_DISPATCH, "weight key %llu already registered", (unsigned long long)key);
+
+    HIP_TRY(ctx, FNN_ERR_MEMORY, hipSetDevice(ctx->device));
+    fnn_hip_weight *w = new (std::nothrow) fnn_hip_weight();
+    if (!w) return fail(ctx, FNN_ERR_MEMORY, "out of host memory");
+    memset(w, 0, sizeof(*w));
+    w->key = key; w->dtype = dtype; w->rows = rows; w->inner = inner; w->items = items; w->kp = kp;
+    w->qblock = (dtype == FNN_DT_I4CB) ? quant_block_size : 0;
+    w->bpr = bpr; w->ctx = ctx;
+
+    // device copy of the words, with the two value-preserving canonicalisations that let
+    // the hardware converts stand for the reference's decode tables:
+    //   F8: every exponent-15 byte decodes to NaN (src/dtypes/f8x4.rs:36) -> OCP NaN 0x7F/0xFF;
+    //   F4: nibble 0x8 decodes to +0.0 (src/dtypes/f4x8.rs:31-35) -> 0x0.
+    std::vector<uint32_t> host(expected);
+    memcpy(host.data(), words, expected * sizeof(uint32_t));
+    if (dtype == FNN_DT_F8) {
+        for (auto &x : host)
+            for (int i = 0; i < 4; i++)
+                if (((x >> (8 * i)) & 0x78u) == 0x78u) x |= (0x7Fu << (8 * i));
+    } else if (dtype == FNN_DT_F4) {
+        for (auto &x : host)
+            for (int i = 0; i < 8; i++)
+                if (((x >> (4 * i)) & 0xFu) == 0x8u) x &= ~(0xFu << (4 * i));
+    }
+    const size_t pad = 256;
+    hipError_t e;
+    auto bail = [&](const char *what) {
+        int rc = fail(ctx, FNN_ERR_MEMORY, "%s: %s", what, hipGetErrorString(e));
+        free_weight(w);
+        return rc;
+    };
+    if ((e = hipMalloc((void **)&w->words, expected * 4 + pad)) != hipSuccess) return bail("hipMalloc(words)");
+    if ((e = hipMemsetAsync(w->words, 0, expected * 4 + pad, ctx->stream)) != hipSuccess) return bail("hipMemset(words)");
+    if ((e = hipMemcpyAsync(w->words, host.data(), expected * 4, hipMemcpyHostToDevice, ctx->stream)) != hipSuccess)
+        return bail("hipMemcpy(words)");
+
+    // scales / zeros expanded to one entry per row (scale_for_row / zero_for_row,
+    // src/packed_tensor.rs:438-462; group rule src/backend/cpu/matmul.rs:147-149)
+    std::vector<float> sc, zr;
+    if (dtype == FNN_DT_I4CB) {
+        sc.assign(scales, scales + rows * bpr);
+        zr.assign((size_t)rows, 0.0f);
+    } else {
+        sc.resize((size_t)rows);
+        zr.resize((size_t)rows);
+        const size_t group = (n_scales > 1 && urows > n_scales) ? urows / n_scales : 1;
+        for (size_t r = 0; r < urows; r++) {
+            const size_t idx = (n_scales == 1) ? 0 : r / group;
+            sc[r] = scales[idx];
+            zr[r] = n_zeros ? zeros[idx] : 0.0f;
+        }
+    }
+    if ((e = hipMalloc((void **)&w->scales, sc.size() * 4 + 64)) != hipSuccess) return bail("hipMalloc(scales)");
+    if ((e = hipMalloc((void **)&w->zeros, zr.size() * 4 + 64)) != hipSuccess) return bail("hipMalloc(zeros)");
+    if ((e = hipMemcpyAsync(w->scales, sc.data(), sc.size() * 4, hipMemcpyHostToDevice, ctx->stream)) != hipSuccess)
+        return bail("hipMemcpy(scales)");
+    if ((e = hipMemcpyAsync(w->zeros, zr.data(), zr.size() * 4, hipMemcpyHostToDevice, ctx->stream)) != hipSuccess)
+        return bail("hipMemcpy(zeros)");
+    if (dtype == FNN_DT_I4CB) {
+        if ((e = hipMalloc((void **)&w->codebook, 64)) != hipSuccess) return bail("hipMalloc(codebook)");
+        if ((e = hipMemcpyAsync(w->codebook, codebook16, 64, hipMemcpyHostToDevice, ctx->stream)) != hipSuccess)
+            return bail("hipMemcpy(codebook)");
+    }
+    if ((e = hipStreamSynchronize(ctx->stream)) != hipSuccess) return bail("hipStreamSynchronize");
+    ctx->weights[key] = w;
+    if (out) *out = w;
+    return FNN_OK;
+}
+
+int fnn_hip_weight_lookup(fnn_hip_ctx *ctx, uint64_t key, fnn_hip_weight **out)
+{
+    if (!ctx || !out) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_weight_lookup: NULL argument");
+    auto it = ctx->weights.find(key);
+    *out = (it == ctx->weights.end()) ? nullptr : it->second;
+    if (!*out) return fail(ctx, FNN_ERR_DISPATCH, "weight key %llu not registered", (unsigned long long)key);
+    return FNN_OK;
+}
+
+int fnn_hip_weight_release(fnn_hip_ctx *ctx, fnn_hip_weight *w)
+{
+    if (!ctx || !w) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_weight_release: NULL argument");
+    auto it = ctx->weights.find(w->key);
+    if (it == ctx->weights.end() || it->second != w)
+        return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_weight_release: weight does not belong to this context");
+    HIP_TRY(ctx, FNN_ERR_DISPATCH, hipStreamSynchronize(ctx->stream));
+    ctx->weights.erase(it);
+    free_weight(w);
+    return FNN_OK;
+}
+
+int fnn_hip_dequant(fnn_hip_ctx *ctx, const fnn_hip_weight *w, float *out, int flags)
+{
+    if (!ctx || !w || !out) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_dequant: NULL argument");
+    const size_t bytes = (size_t)(w->rows * w->inner) * 4;
+    float *dout = out;
+    if (!(flags & FNN_FLAG_DEVICE_PTRS)) {
+        int rc = ensure(ctx, ctx->st_out, bytes);
+        if (rc) return rc;
+        dout = (float *)ctx->st_out.ptr;
+    }
+    HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_dequant(w, dout, ctx->stream));
+    if (!(flags & FNN_FLAG_DEVICE_PTRS)) {
+        HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(out, dout, bytes, hipMemcpyDeviceToHost, ctx->stream));
+        HIP_TRY(ctx, FNN_ERR_DISPATCH, hipStreamSynchronize(ctx->stream));
+    }
+    return FNN_OK;
+}
+
+int fnn_hip_qmatmul(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *a, int64_t m,
+                    const float *bias, int act, float *out, int flags)
+{
+    if (!ctx || !w) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_qmatmul: NULL context or weight");
+    const char *kn = kernel_name_of(w->dtype);
+    if (m < 0) return fail(ctx, FNN_ERR_DISPATCH, "%s: expected params [M,K,N], got M=%lld", kn, (long long)m);
+    if (m == 0) return FNN_OK;
+    if (!a || !out) return fail(ctx, FNN_ERR_DISPATCH, "%s: NULL activation or output pointer", kn);
+    if (act < FNN_ACT_NONE || act > FNN_ACT_SILU)
+        return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "%s: unknown activation %d", kn, act);
+    if ((flags & FNN_FLAG_I4CB_AS_WRITTEN) && w->dtype != FNN_DT_I4CB)
+        return fail(ctx, FNN_ERR_DISPATCH, "%s: as-written mode applies to codebook weights only", kn);
+    const int64_t n = w->rows, k = w->inner;
+    const bool dev = (flags & FNN_FLAG_DEVICE_PTRS) != 0;
+    const float *da = a, *dbias = bias;
+    float *dout = out;
+    if (!dev) {
+        int rc;
+        if ((rc = ensure(ctx, ctx->st_a, (size_t)(m * k) * 4))) return rc;
+        if ((rc = ensure(ctx, ctx->st_out, (size_t)(m * n) * 4))) return rc;
+        HIP_TRY(ctx, FNN_ERR_MEMORY,
+                hipMemcpyAsync(ctx->st_a.ptr, a, (size_t)(m * k) * 4, hipMemcpyHostToDevice, ctx->stream));
+        da = (const float *)ctx->st_a.ptr;
+        dout = (float *)ctx->st_out.ptr;
+        if (bias) {
+            if ((rc = ensure(ctx, ctx->st_bias, (size_t)n * 4))) return rc;
+            HIP_TRY(ctx, FNN_ERR_MEMORY,
+                    hipMemcpyAsync(ctx->st_bias.ptr, bias, (size_t)n * 4, hipMemcpyHostToDevice, ctx->stream));
+            dbias = (const float *)ctx->st_bias.ptr;
+        }
+    }
+    QMatmulArgs p;
+    p.words = w->words; p.scales = w->scales; p.zeros = w->zeros; p.codebook = w->codebook;
+    p.a = da; p.bias = dbias; p.out = dout;
+    p.m = m; p.n = n; p.k = k; p.kp = w->kp; p.bpr = w->bpr; p.qblock = w->qblock; p.act = act;
+    p.as_written = (flags & FNN_FLAG_I4CB_AS_WRITTEN) ? 1 : 0;
+
+    bool handled = false;
+    if (!(flags & FNN_FLAG_FORCE_GENERIC)) {
+        HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qgemv(w->dtype, p, ctx->stream, &handled));
+        if (!handled) {
+            int rc = fnn_mfma_qmatmul(ctx, ctx->stream, w, p, flags, &handled);
+            if (rc) return rc;
+        }
+    }
+    if (!handled) HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qgemm_generic(w->dtype, p, ctx->stream));
+    if (!dev) {
+        HIP_TRY(ctx, FNN_ERR_MEMORY,
+                hipMemcpyAsync(out, dout, (size_t)(m * n) * 4, hipMemcpyDeviceToHost, ctx->stream));
+        HIP_TRY(ctx, FNN_ERR_DISPATCH, hipStreamSynchronize(ctx->stream));
+    }
+    return FNN_OK;
+}
+
+int fnn_hip_quantize_activations(fnn_hip_ctx *ctx, const float *x, int64_t numel, float scale,
+                                 float zp, uint8_t *payload, int flags)
+{
+    if (!ctx || !x || !payload || numel < 0)
+        return fail(ctx, FNN_ERR_DISPATCH, "quantize_activations: NULL or invalid argument");
+    const bool dev = (flags & FNN_FLAG_DEVICE_PTRS) != 0;
+    const float *dx = x;
+    uint8_t *dp = payload;
+    if (!dev) {
+        int rc;
+        if ((rc = ensure(ctx, ctx->st_a, (size_t)numel * 4 + 16))) return rc;
+        if ((rc = ensure(ctx, ctx->st_out, (size_t)numel + 16))) return rc;
+        HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(ctx->st_a.ptr, x, (size_t)numel * 4, hipMemcpyHostToDevice, ctx->stream));
+        dx = (const float *)ctx->st_a.ptr;
+        dp = (uint8_t *)ctx->st_out.ptr;
+    }
+    HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_quantize_activations(dx, numel, scale, zp, dp, ctx->scratch, ctx->stream));
+    if (!dev) {
+        HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(payload, dp, (size_t)numel + 8, hipMemcpyDeviceToHost, ctx->stream));
+        HIP_TRY(ctx, FNN_ERR_DISPATCH, hipStreamSynchronize(ctx->stream));
+    }
+    return FNN_OK;
+}
+
+int fnn_hip_qmatmul_i8act(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const uint8_t *payload,
+                          int64_t m, float *out, int32_t *acc_out, int flags)
+{
+    if (!ctx || !w) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_qmatmul_i8act: NULL context or weight");
+    if (w->dtype != FNN_DT_I8 && w->dtype != FNN_DT_I4)
+        return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "matmul_*_i8: weight dtype %d has no I8-activation kernel", w->dtype);
+    const char *kn = (w->dtype == FNN_DT_I8) ? "matmul_i8_i8" : "matmul_i4_i8";
+    if (m < 0) return fail(ctx, FNN_ERR_DISPATCH, "%s: expected params [M,K,N]", kn);
+    if (m == 0) return FNN_OK;
+    if (!payload || !out) return fail(ctx, FNN_ERR_DISPATCH, "%s: NULL payload or output pointer", kn);
+    const int64_t n = w->rows, k = w->inner;
+    const bool dev = (flags & FNN_FLAG_DEVICE_PTRS) != 0;
+    const uint8_t *dp = payload;
+    float *dout = out;
+    int32_t *dacc = acc_out;
+    if (!dev) {
+        int rc;
+        if ((rc = ensure(ctx, ctx->st_a, (size_t)(m * k) + 8 + 16))) return rc;
+        if ((rc = ensure(ctx, ctx->st_out, (size_t)(m * n) * 4))) return rc;
+        HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(ctx->st_a.ptr, payload, (size_t)(m * k) + 8, hipMemcpyHostToDevice, ctx->stream));
+        dp = (const uint8_t *)ctx->st_a.ptr;
+        dout = (float *)ctx->st_out.ptr;
+        if (acc_out) {
+            if ((rc = ensure(ctx, ctx->st_acc, (size_t)(m * n) * 4))) return rc;
+            dacc = (int32_t *)ctx->st_acc.ptr;
+        }
+    }
+    I8ActArgs p;
+    p.words = w->words; p.scales = w->scales; p.zeros = w->zeros; p.payload = dp; p.out = dout;
+    p.acc_out = dacc; p.m = m; p.n = n; p.k = k; p.kp = w->kp;
+    bool handled = false;
+    if (!(flags & FNN_FLAG_FORCE_GENERIC)) {
+        int rc = fnn_mfma_qmatmul_i8act(ctx, ctx->stream, w, p, &handled);
+        if (rc) return rc;
+    }
+    if (!handled) HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qgemm_i8act_generic(w->dtype, p, ctx->stream));
+    if (!dev) {
+        HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(out, dout, (size_t)(m * n) * 4, hipMemcpyDeviceToHost, ctx->stream));
+        if (acc_out)
+            HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(acc_out, dacc, (size_t)(m * n) * 4, hipMemcpyDeviceToHost, ctx->stream));
+        HIP_TRY(ctx, FNN_ERR_DISPATCH, hipStreamSynchronize(ctx->stream));
+    }
+    return FNN_OK;
+}
+
+int fnn_hip_qconv2d(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *x, int64_t b, int64_t c,
+                    int64_t h, int64_t wd, int kh, int kw, int stride, int pad, int dil, int groups,
+                    const float *bias, int act, float *y, int32_t *acc_out, int flags)
+{
+    if (!ctx) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_hip_qconv2d: NULL context");
+    if (!w) return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8: missing weight_meta for quantized weight");
+    if (w->dtype != FNN_DT_I8)
+        return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "conv2d: only I8 weights have an integer conv kernel (dtype %d)", w->dtype);
+    if (groups <= 0) return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8: groups must be > 0");
+    if (b < 0 || c <= 0 || h <= 0 || wd <= 0 || kh <= 0 || kw <= 0 || stride <= 0 || dil <= 0 || pad < 0)
+        return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8: invalid geometry");
+    if (c % groups || w->rows % groups)
+        return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8: channels (%lld in, %lld out) not divisible by groups %d",
+                    (long long)c, (long long)w->rows, groups);
+    if (w->inner != (c / groups) * kh * kw)
+        return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8: weight inner dim %lld != C/g*KH*KW = %lld", (long long)w->inner,
+                    (long long)((c / groups) * kh * kw));
+    if (act < FNN_ACT_NONE || act > FNN_ACT_SILU) return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "conv2d_i8: unknown activation %d", act);
+    auto osz = [](int64_t in, int k, int s, int p, int d) -> int64_t {
+        int64_t dk = (int64_t)(k - 1) * d + 1;
+        return (in + 2 * p >= dk) ? (in + 2 * p - dk) / s + 1 : 0;
+    };
+    const int64_t ho = osz(h, kh, stride, pad, dil), wo = osz(wd, kw, stride, pad, dil);
+    const int64_t oc = w->rows;
+    if (b == 0 || ho == 0 || wo == 0) return FNN_OK;
+    if (!x || !y) return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8: NULL input or output pointer");
+    if (b * groups > 65535) return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "conv2d_i8: batch*groups > 65535");
+    const bool dev = (flags & FNN_FLAG_DEVICE_PTRS) != 0;
+    fnn_hip_weight *wm = const_cast<fnn_hip_weight *>(w);
+    if (!wm->row_qsum) {
+        if (ctx->capturing) return fail(ctx, FNN_ERR_MEMORY, "conv2d_i8: first use of a weight during graph capture");
+        HIP_TRY(ctx, FNN_ERR_MEMORY, hipMalloc((void **)&wm->row_qsum, (size_t)oc * 4 + 64));
+        HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_row_qsum(w, wm->row_qsum, ctx->stream));
+    }
+    const size_t xin = (size_t)(b * c * h * wd) * 4, yout = (size_t)(b * oc * ho * wo) * 4;
+    const float *dx = x, *dbias = bias;
+    float *dy = y;
+    int32_t *dacc = acc_out;
+    int rc;
+    if (!dev) {
+        if ((rc = ensure(ctx, ctx->st_a, xin))) return rc;
+        if ((rc = ensure(ctx, ctx->st_out, yout))) return rc;
+        HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(ctx->st_a.ptr, x, xin, hipMemcpyHostToDevice, ctx->stream));
+        dx = (const float *)ctx->st_a.ptr;
+        dy = (float *)ctx->st_out.ptr;
+        if (bias) {
+            if ((rc = ensure(ctx, ctx->st_bias, (size_t)oc * 4))) return rc;
+            HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(ctx->st_bias.ptr, bias, (size_t)oc * 4, hipMemcpyHostToDevice, ctx->stream));
+            dbias = (const float *)ctx->st_bias.ptr;
+        }
+        if (acc_out) {
+            if ((rc = ensure(ctx, ctx->st_acc, yout))) return rc;
+            dacc = (int32_t *)ctx->st_acc.ptr;
+        }
+    }
+    if ((rc = ensure(ctx, ctx->st_tmp, (size_t)(b * groups) * (QCONV_NPART * 2 + 4) * 4))) return rc;
+    QConvArgs p;
+    p.words = w->words; p.scales = w->scales; p.zeros = w->zeros; p.row_qsum = wm->row_qsum;
+    p.x = dx; p.bias = dbias; p.y = dy; p.acc_out = dacc;
+    p.minmax_partial = (float *)ctx->st_tmp.ptr;
+    p.actq = p.minmax_partial + (size_t)(b * groups) * QCONV_NPART * 2;
+    p.b = b; p.c = c; p.h = h; p.w = wd; p.oc = oc; p.ho = ho; p.wo = wo; p.kp = w->kp;
+    p.kh = kh; p.kw = kw; p.stride = stride; p.pad = pad; p.dil = dil; p.groups = groups; p.act = act;
+    HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qconv2d_i8(p, ctx->stream));
+    if (!dev) {
+        HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(y, dy, yout, hipMemcpyDeviceToHost, ctx->stream));
+        if (acc_out) HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(acc_out, dacc, yout, hipMemcpyDeviceToHost, ctx->stream));
+        HIP_TRY(ctx, FNN_ERR_DISPATCH, hipStreamSynchronize(ctx->stream));
+    }
+    return FNN_OK;
+}
+
+int fnn_hip_timer_start(fnn_hip_ctx *ctx)
+{
+    if (!ctx) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_hip_timer_start: NULL context");
+    HIP_TRY(ctx, FNN_ERR_DISPATCH, hipEventRecord(ctx->ev0, ctx->stream));
+    return FNN_OK;
+}
+
+int fnn_hip_timer_stop(fnn_hip_ctx *ctx, float *ms)
+{
+    if (!ctx || !ms) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_timer_stop: NULL argument");
+    HIP_TRY(ctx, FNN_ERR_DISPATCH, hipEventRecord(ctx->ev1, ctx->stream));
+    HIP_TRY(ctx, FNN_ERR_DISPATCH, hipEventSynchronize(ctx->ev1));
+    HIP_TRY(ctx, FNN_ERR_DISPATCH, hipEventElapsedTime(ms, ctx->ev0, ctx->ev1));
+    return FNN_OK;
+}
+
+int fnn_hip_graph_begin(fnn_hip_ctx *ctx)
+{
+    if (!ctx) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_hip_graph_begin: NULL context");
+    if (ctx->capturing) return fail(ctx, FNN_ERR_DISPATCH, "graph capture already active");
+    HIP_TRY(ctx, FNN_ERR_DISPATCH, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
+    ctx->capturing = true;
+    return FNN_OK;
+}
+
+int fnn_hip_graph_end(fnn_hip_ctx *ctx, fnn_hip_graph **out)
+{
+    if (!ctx || !out) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_graph_end: NULL argument");
+    if (!ctx->capturing) return fail(ctx, FNN_ERR_DISPATCH, "no graph capture active");
+    ctx->capturing = false;
+    fnn_hip_graph *g = new (std::nothrow) fnn_hip_graph();
+    if (!g) return fail(ctx, FNN_ERR_MEMORY, "out of host memory");
+    hipError_t e = hipStreamEndCapture(ctx->stream, &g->graph);
+    if (e == hipSuccess) e = hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+        if (g->graph) (void)hipGraphDestroy(g->graph);
+        delete g;
+        return fail(ctx, FNN_ERR_DISPATCH, "graph capture failed: %s", hipGetErrorString(e));
+    }
+    *out = g;
+    return FNN_OK;
+}
+
+int fnn_hip_graph_launch(fnn_hip_ctx *ctx, fnn_hip_graph *g)
+{
+    if (!ctx || !g) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_graph_launch: NULL argument");
+    HIP_TRY(ctx, FNN_ERR_DISPATCH, hipGraphLaunch(g->exec, ctx->stream));
+    return FNN_OK;
+}
+
+int fnn_hip_graph_destroy(fnn_hip_ctx *ctx, fnn_hip_graph *g)
+{
+    if (!g) return FNN_OK;
+    if (ctx && ctx->stream) (void)hipStreamSynchronize(ctx->stream);
+    if (g->exec) (void)hipGraphExecDestroy(g->exec);
+    if (g->graph) (void)hipGraphDestroy(g->graph);
+    delete g;
+    return FNN_OK;
+}
+
+}  // extern "C"
+
+// staging access for the MFMA translation unit
+int fnn_ctx_ensure_tmp(fnn_hip_ctx *ctx, int which, size_t bytes, void **ptr)
+{
+    Staging &s = which == 0 ? ctx->st_tmp : ctx->st_tmp2;
+    int rc = ensure(ctx, s, bytes);
+    if (rc) return rc;
+    *ptr = s.ptr;
+    return FNN_OK;
+}
+
+int fnn_ctx_fail(fnn_hip_ctx *ctx, int code, const char *msg) { return fail(ctx, code, "%s", msg); }

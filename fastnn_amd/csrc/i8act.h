@@ -1,0 +1,35 @@
+// Launch interfaces of the I8-activation and quantised-conv kernels.
+#pragma once
+#include "common.h"
+
+struct I8ActArgs {
+    const uint32_t *words;
+    const float *scales;    // [N]
+    const float *zeros;     // [N]
+    const uint8_t *payload; // [scale f32][zp f32][M*K i8]
+    float *out;             // [M,N]
+    int32_t *acc_out;       // [M,N] or null
+    int64_t m, n, k, kp;
+};
+
+struct QConvArgs {
+    const uint32_t *words;   // [OC, kp] I8 words
+    const float *scales;     // [OC]
+    const float *zeros;      // [OC]
+    const int32_t *row_qsum; // [OC] sum of q_w per output channel
+    const float *x;          // [B,C,H,W]
+    const float *bias;       // [OC] or null
+    float *y;                // [B,OC,Ho,Wo]
+    int32_t *acc_out;        // same shape as y, or null
+    float *minmax_partial;   // [B*G][NPART][2]
+    float *actq;             // [B*G][4]: sa, za, inv, unused
+    int64_t b, c, h, w, oc, ho, wo, kp;
+    int kh, kw, stride, pad, dil, groups, act;
+};
+constexpr int QCONV_NPART = 64;
+
+hipError_t launch_quantize_activations(const float *x, int64_t numel, float scale, float zp,
+                                       uint8_t *payload, float *scratch_partial, hipStream_t s);
+hipError_t launch_qgemm_i8act_generic(int dtype, const I8ActArgs &p, hipStream_t s);
+hipError_t launch_row_qsum(const fnn_hip_weight *w, int32_t *out, hipStream_t s);
+hipError_t launch_qconv2d_i8(const QConvArgs &p, hipStream_t s);

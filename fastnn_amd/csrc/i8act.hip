@@ -1,0 +1,168 @@
+// I8-activation path for gfx950: the "quantize_activations" kernel and the
+// "matmul_i8_i8" / "matmul_i4_i8" GEMMs with exact i32 accumulators
+// (src/backend/cpu/mod.rs:6928-7008, src/backend/cpu/microkernels/gemm.rs:1641-1975).
+#include "common.h"
+
+#include "i8act.h"
+
+namespace {
+
+__global__ void __launch_bounds__(256) absmax_partial_kernel(const float *x, int64_t numel, float *partial)
+{
+    __shared__ float sm[4];
+    float v = 0.0f;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < numel;
+         i += (int64_t)gridDim.x * blockDim.x)
+        v = fmaxf(v, fabsf(x[i]));  // fmaxf ignores NaN like f32::max
+    v = wave_max(v);
+    if ((threadIdx.x & 63) == 0) sm[threadIdx.x >> 6] = v;
+    __syncthreads();
+    if (threadIdx.x == 0) partial[blockIdx.x] = fmaxf(fmaxf(sm[0], sm[1]), fmaxf(sm[2], sm[3]));
+}
+
+// payload = [scale][zp][q...]; q = clamp(round((x - zp)/scale), -128, 127)
+__global__ void __launch_bounds__(256)
+quantize_act_kernel(const float *x, int64_t numel, const float *partial, int npartial, float scale_in,
+                    float zp, uint8_t *payload)
+{
+    __shared__ float s_scale;
+    if (threadIdx.x < 64) {
+        float scale = scale_in;
+        if (partial) {
+            float v = 0.0f;
+            for (int i = threadIdx.x; i < npartial; i += 64) v = fmaxf(v, partial[i]);
+            v = wave_max(v);
+            scale = (v == 0.0f) ? 1.0f : v / 127.0f;
+        }
+        if (threadIdx.x == 0) s_scale = scale;
+    }
+    __syncthreads();
+    const float scale = s_scale;
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        reinterpret_cast<float *>(payload)[0] = scale;
+        reinterpret_cast<float *>(payload)[1] = zp;
+    }
+    int8_t *q = reinterpret_cast<int8_t *>(payload + 8);
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < numel;
+         i += (int64_t)gridDim.x * blockDim.x) {
+        const float t = roundf((x[i] - zp) / scale);
+        // clamp keeps NaN and the saturating cast maps NaN to 0
+        const int qi = (t != t) ? 0 : (int)fminf(fmaxf(t, -128.0f), 127.0f);
+        q[i] = (int8_t)qi;
+    }
+}
+
+template <int DT>
+__device__ __forceinline__ void decode_int(uint32_t w, int *o)
+{
+    if constexpr (DT == FNN_DT_I8) {
+        o[0] = (int)(int8_t)(w & 0xff);
+        o[1] = (int)(int8_t)((w >> 8) & 0xff);
+        o[2] = (int)(int8_t)((w >> 16) & 0xff);
+        o[3] = (int)w >> 24;
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; i++) o[i] = ((int)(w << (28 - 4 * i))) >> 28;
+    }
+}
+
+constexpr int I8_MT = 4;
+
+// One wave per weight row and tile of 4 activation rows; lanes stride over packed words.
+template <int DT>
+__global__ void __launch_bounds__(256) qgemm_i8act_generic_kernel(I8ActArgs p)
+{
+    constexpr int EPW = (DT == FNN_DT_I8) ? 4 : 8;
+    const int lane = threadIdx.x & 63;
+    const int64_t n = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    const int64_t m0 = (int64_t)blockIdx.y * I8_MT;
+    if (n >= p.n) return;
+    const float sa = reinterpret_cast<const float *>(p.payload)[0];
+    const float za = reinterpret_cast<const float *>(p.payload)[1];
+    const int8_t *qa = reinterpret_cast<const int8_t *>(p.payload + 8);
+    const int64_t K = p.k;
+    int acc[I8_MT], qs[I8_MT];
+    float facc[I8_MT], fsum[I8_MT];
+#pragma unroll
+    for (int m = 0; m < I8_MT; m++) { acc[m] = qs[m] = 0; facc[m] = fsum[m] = 0.0f; }
+    const bool affine = (za != 0.0f);
+    for (int64_t wd = lane; wd < p.kp; wd += 64) {
+        int wq[EPW];
+        decode_int<DT>(p.words[n * p.kp + wd], wq);
+#pragma unroll
+        for (int e = 0; e < EPW; e++) {
+            const int64_t kk = wd * EPW + e;
+            if (kk < K) {
+#pragma unroll
+                for (int m = 0; m < I8_MT; m++) {
+                    if (m0 + m < p.m) {
+                        int q = qa[(m0 + m) * K + kk];
+                        if (affine) {
+                            float a = (float)q * sa + za;
+                            facc[m] += a * (float)wq[e];
+                            fsum[m] += a;
+                        } else {
+                            acc[m] += wq[e] * q;
+                            qs[m] += q;
+                        }
+                    }
+                }
+            }
+        }
+    }
+    const float sw = p.scales[n], zw = p.zeros[n];
+#pragma unroll
+    for (int m = 0; m < I8_MT; m++) {
+        if (m0 + m >= p.m) continue;
+        float res;
+        int a_tot = 0;
+        if (affine) {
+            float d = wave_sum(facc[m]);
+            float s = wave_sum(fsum[m]);
+            res = d * sw + zw * s;
+        } else {
+            a_tot = wave_sum_i32(acc[m]);
+            int q_tot = wave_sum_i32(qs[m]);
+            float dot = (float)a_tot * sa;
+            float input_sum = (float)q_tot * sa + (float)K * za;
+            res = dot * sw + zw * input_sum;
+        }
+        if (lane == 0) {
+            p.out[(m0 + m) * p.n + n] = res;
+            if (p.acc_out) p.acc_out[(m0 + m) * p.n + n] = a_tot;
+        }
+    }
+}
+
+}  // namespace
+
+hipError_t launch_quantize_activations(const float *x, int64_t numel, float scale, float zp,
+                                       uint8_t *payload, float *scratch_partial, hipStream_t s)
+{
+    int64_t blocks = (numel + 255) / 256;
+    if (blocks > 1024) blocks = 1024;
+    if (blocks < 1) blocks = 1;
+    const float *partial = nullptr;
+    if (!(scale > 0.0f)) {
+        hipLaunchKernelGGL(absmax_partial_kernel, dim3((unsigned)blocks), dim3(256), 0, s, x, numel,
+                           scratch_partial);
+        partial = scratch_partial;
+        zp = 0.0f;
+    }
+    hipLaunchKernelGGL(quantize_act_kernel, dim3((unsigned)blocks), dim3(256), 0, s, x, numel, partial,
+                       (int)blocks, scale, zp, payload);
+    return hipGetLastError();
+}
+
+hipError_t launch_qgemm_i8act_generic(int dtype, const I8ActArgs &p, hipStream_t s)
+{
+    const int wpb = 4;
+    dim3 grid((unsigned)((p.n + wpb - 1) / wpb), (unsigned)((p.m + I8_MT - 1) / I8_MT));
+    if (dtype == FNN_DT_I8)
+        hipLaunchKernelGGL((qgemm_i8act_generic_kernel<FNN_DT_I8>), grid, dim3(wpb * 64), 0, s, p);
+    else if (dtype == FNN_DT_I4)
+        hipLaunchKernelGGL((qgemm_i8act_generic_kernel<FNN_DT_I4>), grid, dim3(wpb * 64), 0, s, p);
+    else
+        return hipErrorInvalidValue;
+    return hipGetLastError();
+}

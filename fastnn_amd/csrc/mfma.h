@@ -1,0 +1,16 @@
+// MFMA GEMM entry points (matrix-core path for M >= 5 activation rows).
+#pragma once
+#include "common.h"
+#include "i8act.h"
+
+// context services implemented beside the C ABI
+int fnn_ctx_ensure_tmp(fnn_hip_ctx *ctx, int which, size_t bytes, void **ptr);
+int fnn_ctx_fail(fnn_hip_ctx *ctx, int code, const char *msg);
+
+// f32 activations x packed weights on f16 MFMA tiles; *handled = false when the shape
+// is left to the generic kernel.
+int fnn_mfma_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &p,
+                     int flags, bool *handled);
+// I8 activations x I8/I4 weights on int8 MFMA tiles with i32 accumulators.
+int fnn_mfma_qmatmul_i8act(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w,
+                           const I8ActArgs &p, bool *handled);

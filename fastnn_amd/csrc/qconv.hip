@@ -1,0 +1,200 @@
+// Quantised Conv2d (I8 weights, f32 NCHW activations) for gfx950:
+// conv2d_packed_i8x4 = im2col + per-(image,group) dynamic int8 activation quantisation +
+// integer GEMM with the fused 4-term dequantise, bias and activation
+// (src/backend/cpu/packed_conv.rs:125-232,444-625,1118-1196).
+//
+// The im2col matrix is never materialised: its (min,max) scan and the activation
+// quantisation are evaluated from the NCHW input through the index formula
+//   col[p, c*KH*KW + i*KW + j] = x[c, oh*s + i*d - pad, ow*s + j*d - pad]  (0 outside),
+// so the HBM traffic is the input, the weights and the output only.
+#include "common.h"
+
+#include "i8act.h"
+
+namespace {
+
+__device__ __forceinline__ float col_value(const float *xg, int64_t h, int64_t w, int kh, int kw,
+                                           int stride, int pad, int dil, int64_t wo, int64_t p,
+                                           int64_t e)
+{
+    const int64_t khw = (int64_t)kh * kw;
+    const int64_t ic = e / khw;
+    const int rem = (int)(e % khw);
+    const int i = rem / kw, j = rem % kw;
+    const int64_t oh = p / wo, ow = p % wo;
+    const int64_t ih = oh * stride + (int64_t)i * dil - pad;
+    const int64_t iw = ow * stride + (int64_t)j * dil - pad;
+    if (ih < 0 || ih >= h || iw < 0 || iw >= w) return 0.0f;
+    return xg[(ic * h + ih) * w + iw];
+}
+
+// min/max over the whole im2col matrix of one (image, group), padding zeros included
+// (src/backend/cpu/im2col.rs:496-507).
+__global__ void __launch_bounds__(256) conv_minmax_kernel(QConvArgs a)
+{
+    __shared__ float smn[4], smx[4];
+    const int bg = blockIdx.y;
+    const int64_t nn = bg / a.groups, g = bg % a.groups;
+    const int64_t cg = a.c / a.groups;
+    const int64_t kk = cg * a.kh * a.kw;
+    const int64_t np = a.ho * a.wo;
+    const float *xg = a.x + (nn * a.c + g * cg) * a.h * a.w;
+    float mn = INFINITY, mx = -INFINITY;
+    const int64_t total = np * kk;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (int64_t)gridDim.x * blockDim.x) {
+        // pixel-fastest order keeps neighbouring lanes on neighbouring input columns
+        const int64_t e = idx / np, p = idx % np;
+        const float v = col_value(xg, a.h, a.w, a.kh, a.kw, a.stride, a.pad, a.dil, a.wo, p, e);
+        mn = fminf(mn, v);
+        mx = fmaxf(mx, v);
+    }
+    mn = wave_min(mn);
+    mx = wave_max(mx);
+    if ((threadIdx.x & 63) == 0) { smn[threadIdx.x >> 6] = mn; smx[threadIdx.x >> 6] = mx; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float *dst = a.minmax_partial + ((int64_t)bg * QCONV_NPART + blockIdx.x) * 2;
+        dst[0] = fminf(fminf(smn[0], smn[1]), fminf(smn[2], smn[3]));
+        dst[1] = fmaxf(fmaxf(smx[0], smx[1]), fmaxf(smx[2], smx[3]));
+    }
+}
+
+// scale = range/255 (1 if range <= 0), zero = mn + 128*scale (0 if range <= 0), inv = 1/scale
+// (src/backend/cpu/packed_conv.rs:149-156)
+__global__ void __launch_bounds__(64) conv_actq_kernel(QConvArgs a, int nparts)
+{
+    const int bg = blockIdx.x;
+    float mn = INFINITY, mx = -INFINITY;
+    for (int i = threadIdx.x; i < nparts; i += 64) {
+        mn = fminf(mn, a.minmax_partial[((int64_t)bg * QCONV_NPART + i) * 2]);
+        mx = fmaxf(mx, a.minmax_partial[((int64_t)bg * QCONV_NPART + i) * 2 + 1]);
+    }
+    mn = wave_min(mn);
+    mx = wave_max(mx);
+    if (threadIdx.x == 0) {
+        const float range = mx - mn;
+        const float scale = (range > 0.0f) ? range / 255.0f : 1.0f;
+        const float zero = (range > 0.0f) ? mn + 128.0f * scale : 0.0f;
+        const float inv = (scale != 0.0f) ? 1.0f / scale : 0.0f;
+        a.actq[bg * 4 + 0] = scale;
+        a.actq[bg * 4 + 1] = zero;
+        a.actq[bg * 4 + 2] = inv;
+        a.actq[bg * 4 + 3] = 0.0f;
+    }
+}
+
+constexpr int CONV_OCT = 8;  // output channels per thread
+
+// One thread = one output pixel x CONV_OCT output channels of one (image, group).
+// acc = bias_q + sum q_a*q_w (i32, exact);
+// val = acc*sab + zw*(sa*sum q_a) + za*(sw*qb) + (za*zw)*K, left to right
+// (src/backend/cpu/packed_conv.rs:469-505).
+__global__ void __launch_bounds__(256) conv_i8_kernel(QConvArgs a)
+{
+    const int bg = blockIdx.z;
+    const int64_t nn = bg / a.groups, g = bg % a.groups;
+    const int64_t cg = a.c / a.groups, ocg = a.oc / a.groups;
+    const int64_t kk = cg * a.kh * a.kw;
+    const int64_t np = a.ho * a.wo;
+    const int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t f0 = (int64_t)blockIdx.y * CONV_OCT;
+    if (p >= np) return;
+    const float *xg = a.x + (nn * a.c + g * cg) * a.h * a.w;
+    const float sa = a.actq[bg * 4 + 0], za = a.actq[bg * 4 + 1], inv = a.actq[bg * 4 + 2];
+    int acc[CONV_OCT];
+#pragma unroll
+    for (int t = 0; t < CONV_OCT; t++) acc[t] = 0;
+    int qasum = 0;
+    const int8_t *wb = reinterpret_cast<const int8_t *>(a.words);
+    for (int64_t e = 0; e < kk; e++) {
+        const float v = col_value(xg, a.h, a.w, a.kh, a.kw, a.stride, a.pad, a.dil, a.wo, p, e);
+        const float t = roundf((v - za) * inv);
+        const int q = (t != t) ? 0 : (int)fminf(fmaxf(t, -128.0f), 127.0f);
+        qasum += q;
+#pragma unroll
+        for (int t2 = 0; t2 < CONV_OCT; t2++) {
+            const int64_t f = f0 + t2;
+            if (f < ocg) acc[t2] += q * (int)wb[((g * ocg + f) * a.kp) * 4 + e];
+        }
+    }
+    const float r = sa * (float)qasum;
+#pragma unroll
+    for (int t2 = 0; t2 < CONV_OCT; t2++) {
+        const int64_t f = f0 + t2;
+        if (f >= ocg) continue;
+        const int64_t ch = g * ocg + f;
+        const float sw = a.scales[ch], zw = a.zeros[ch];
+        const float sab = sa * sw;
+        int bias_q = 0;
+        if (a.bias) {
+            const float bq = roundf(a.bias[ch] / sab);
+            bias_q = (bq != bq) ? 0 : (bq >= 2147483648.0f ? 2147483647 : (bq <= -2147483648.0f ? (-2147483647 - 1) : (int)bq));
+        }
+        const int accv = acc[t2] + bias_q;
+        const float w_term = sw * (float)a.row_qsum[ch];
+        const float zp_prod = za * zw;
+        float val = (float)accv * sab;
+        val = val + zw * r;
+        val = val + za * w_term;
+        val = val + zp_prod * (float)kk;
+        if (a.act == FNN_ACT_RELU) val = fmaxf(val, 0.0f);
+        else if (a.act == FNN_ACT_SILU) val = val / (1.0f + expf(-val));
+        else if (a.act == FNN_ACT_GELU)
+            val = val * 0.5f * (1.0f + tanhf(val * 0.7978846f * (1.0f + 0.044715f * val * val)));
+        const int64_t o = (nn * a.oc + ch) * np + p;
+        a.y[o] = val;
+        if (a.acc_out) a.acc_out[o] = accv;
+    }
+}
+
+template <int BITS>
+__global__ void __launch_bounds__(256) row_qsum_kernel(const uint32_t *words, int64_t rows, int64_t kp, int32_t *out)
+{
+    const int lane = threadIdx.x & 63;
+    const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (r >= rows) return;
+    int s = 0;
+    for (int64_t wd = lane; wd < kp; wd += 64) {
+        const uint32_t w = words[r * kp + wd];
+        if (BITS == 8) {
+            s += (int)(int8_t)(w & 0xff) + (int)(int8_t)((w >> 8) & 0xff) + (int)(int8_t)((w >> 16) & 0xff) + ((int)w >> 24);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; i++) s += ((int)(w << (28 - 4 * i))) >> 28;
+        }
+    }
+    s = wave_sum_i32(s);
+    if (lane == 0) out[r] = s;
+}
+
+}  // namespace
+
+hipError_t launch_row_qsum(const fnn_hip_weight *w, int32_t *out, hipStream_t s)
+{
+    dim3 grid((unsigned)((w->rows + 3) / 4));
+    if (w->dtype == FNN_DT_I8)
+        hipLaunchKernelGGL((row_qsum_kernel<8>), grid, dim3(256), 0, s, w->words, w->rows, w->kp, out);
+    else if (w->dtype == FNN_DT_I4)
+        hipLaunchKernelGGL((row_qsum_kernel<4>), grid, dim3(256), 0, s, w->words, w->rows, w->kp, out);
+    else
+        return hipErrorInvalidValue;
+    return hipGetLastError();
+}
+
+hipError_t launch_qconv2d_i8(const QConvArgs &p, hipStream_t s)
+{
+    const int64_t bg = p.b * p.groups;
+    const int64_t cg = p.c / p.groups, ocg = p.oc / p.groups;
+    const int64_t np = p.ho * p.wo;
+    const int64_t total = np * cg * p.kh * p.kw;
+    if (bg == 0 || np == 0) return hipSuccess;
+    int64_t nparts = (total + 256 * 16 - 1) / (256 * 16);
+    if (nparts > QCONV_NPART) nparts = QCONV_NPART;
+    if (nparts < 1) nparts = 1;
+    hipLaunchKernelGGL(conv_minmax_kernel, dim3((unsigned)nparts, (unsigned)bg), dim3(256), 0, s, p);
+    hipLaunchKernelGGL(conv_actq_kernel, dim3((unsigned)bg), dim3(64), 0, s, p, (int)nparts);
+    dim3 grid((unsigned)((np + 255) / 256), (unsigned)((ocg + CONV_OCT - 1) / CONV_OCT), (unsigned)bg);
+    hipLaunchKernelGGL(conv_i8_kernel, grid, dim3(256), 0, s, p);
+    return hipGetLastError();
+}

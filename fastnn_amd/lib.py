@@ -1,0 +1,335 @@
+"""ctypes host layer over the C ABI of ``libfastnn_hip.so`` (include/fastnn_hip.h).
+
+Loading never falls back to a CPU path: if the shared library is missing or a GPU entry
+point fails, an exception is raised.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+from dataclasses import dataclass
+from typing import Optional
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libfastnn_hip.so")
+
+DT_I8, DT_I4, DT_U8, DT_U4, DT_F8, DT_F8R, DT_F4, DT_I4CB = range(8)
+ACT_NONE, ACT_RELU, ACT_GELU, ACT_SILU = range(4)
+FLAG_DEVICE_PTRS = 1
+FLAG_I4CB_AS_WRITTEN = 2
+FLAG_ACT_F16_SINGLE = 4
+FLAG_FORCE_GENERIC = 8
+
+STATUS_NAMES = {0: "Ok", 1: "Dispatch", 2: "Memory", 3: "UnsupportedOp", 4: "Compilation"}
+
+# every symbol include/fastnn_hip.h declares
+EXPORTED_SYMBOLS = [
+    "fnn_hip_device_count", "fnn_hip_create", "fnn_hip_destroy", "fnn_hip_last_error", "fnn_hip_sync",
+    "fnn_hip_malloc", "fnn_hip_free", "fnn_hip_upload", "fnn_hip_download",
+    "fnn_hip_weight_register", "fnn_hip_weight_lookup", "fnn_hip_weight_release", "fnn_hip_dequant",
+    "fnn_hip_qmatmul", "fnn_hip_quantize_activations", "fnn_hip_qmatmul_i8act", "fnn_hip_qconv2d",
+    "fnn_hip_timer_start", "fnn_hip_timer_stop",
+    "fnn_hip_graph_begin", "fnn_hip_graph_end", "fnn_hip_graph_launch", "fnn_hip_graph_destroy",
+    "fnn_packed_words", "fnn_quantize_weights", "fnn_transpose_kn_to_nk", "fnn_hip_version",
+]
+
+
+class FnnError(RuntimeError):
+    """A non-zero fnn_status; mirrors fastnn's BackendError variants."""
+
+    def __init__(self, status: int, message: str):
+        super().__init__(f"{STATUS_NAMES.get(status, status)} error: {message}")
+        self.status = status
+        self.kind = STATUS_NAMES.get(status, str(status))
+        self.message = message
+
+
+_lib = None
+
+
+def load_library(path: Optional[str] = None):
+    """Load libfastnn_hip.so; raises if it has not been built (no fallback)."""
+    global _lib
+    if _lib is not None and path is None:
+        return _lib
+    p = path or LIB_PATH
+    if not os.path.exists(p):
+        raise FileNotFoundError(
+            f"{p} not found: build it with `python -m fastnn_amd.build` (hipcc, gfx950). "
+            "There is no CPU fallback.")
+    lib = C.CDLL(p)
+    _prototype(lib)
+    if path is None:
+        _lib = lib
+    return lib
+
+
+_vp = C.c_void_p
+_i64 = C.c_int64
+_sz = C.c_size_t
+
+
+def _prototype(l):
+    l.fnn_hip_device_count.restype = C.c_int
+    l.fnn_hip_create.argtypes = [C.c_int, C.POINTER(_vp)]
+    l.fnn_hip_destroy.argtypes = [_vp]
+    l.fnn_hip_destroy.restype = None
+    l.fnn_hip_last_error.argtypes = [_vp]
+    l.fnn_hip_last_error.restype = C.c_char_p
+    l.fnn_hip_sync.argtypes = [_vp]
+    l.fnn_hip_malloc.argtypes = [_vp, _sz, C.POINTER(_vp)]
+    l.fnn_hip_free.argtypes = [_vp, _vp]
+    l.fnn_hip_upload.argtypes = [_vp, _vp, _vp, _sz]
+    l.fnn_hip_download.argtypes = [_vp, _vp, _vp, _sz]
+    l.fnn_hip_weight_register.argtypes = [_vp, C.c_uint64, C.c_int, _vp, _sz, _i64, _i64, _vp, _sz, _vp, _sz,
+                                          C.c_int, _vp, C.POINTER(_vp)]
+    l.fnn_hip_weight_lookup.argtypes = [_vp, C.c_uint64, C.POINTER(_vp)]
+    l.fnn_hip_weight_release.argtypes = [_vp, _vp]
+    l.fnn_hip_dequant.argtypes = [_vp, _vp, _vp, C.c_int]
+    l.fnn_hip_qmatmul.argtypes = [_vp, _vp, _vp, _i64, _vp, C.c_int, _vp, C.c_int]
+    l.fnn_hip_quantize_activations.argtypes = [_vp, _vp, _i64, C.c_float, C.c_float, _vp, C.c_int]
+    l.fnn_hip_qmatmul_i8act.argtypes = [_vp, _vp, _vp, _i64, _vp, _vp, C.c_int]
+    l.fnn_hip_qconv2d.argtypes = [_vp, _vp, _vp, _i64, _i64, _i64, _i64, C.c_int, C.c_int, C.c_int, C.c_int,
+                                  C.c_int, C.c_int, _vp, C.c_int, _vp, _vp, C.c_int]
+    l.fnn_hip_timer_start.argtypes = [_vp]
+    l.fnn_hip_timer_stop.argtypes = [_vp, C.POINTER(C.c_float)]
+    l.fnn_hip_graph_begin.argtypes = [_vp]
+    l.fnn_hip_graph_end.argtypes = [_vp, C.POINTER(_vp)]
+    l.fnn_hip_graph_launch.argtypes = [_vp, _vp]
+    l.fnn_hip_graph_destroy.argtypes = [_vp, _vp]
+    l.fnn_packed_words.argtypes = [C.c_int, _i64, _i64]
+    l.fnn_packed_words.restype = _sz
+    l.fnn_quantize_weights.argtypes = [C.c_int, _vp, _i64, _i64, C.c_int, _vp, _vp, _vp, _vp]
+    l.fnn_transpose_kn_to_nk.argtypes = [_vp, _i64, _i64, _vp]
+    l.fnn_transpose_kn_to_nk.restype = None
+    l.fnn_hip_version.restype = C.c_char_p
+
+
+def _np_ptr(a: Optional[np.ndarray]):
+    return None if a is None else a.ctypes.data_as(_vp)
+
+
+def _as_ptr(x):
+    """numpy array -> host pointer; int -> raw (device) pointer; None -> NULL."""
+    if x is None:
+        return None
+    if isinstance(x, np.ndarray):
+        return x.ctypes.data_as(_vp)
+    return _vp(int(x))
+
+
+@dataclass
+class PackedWeight:
+    """Host image of a quantised weight: what fastnn's pass stores in the constant's bytes
+    plus QuantizedWeightMeta (src/backend/mod.rs:42-58)."""
+    dtype: int
+    rows: int                      # N (or OC)
+    inner: int                     # K (or IC/g*KH*KW)
+    words: np.ndarray              # uint32
+    scales: np.ndarray             # float32
+    zeros: np.ndarray              # float32 (empty for I4CB)
+    qblock: int = 0
+    codebook: Optional[np.ndarray] = None
+
+    @property
+    def bit_width(self) -> int:
+        return 8 if self.dtype in (DT_I8, DT_U8, DT_F8, DT_F8R) else 4
+
+    def packed_bytes(self) -> int:
+        items = 32 // self.bit_width
+        return self.rows * (-(-self.inner // items)) * 4
+
+
+def quantize_weights(dtype: int, w_nk: np.ndarray, qblock: int = 32) -> PackedWeight:
+    """Quantise a transposed [N,K] f32 matrix with fastnn's packer for `dtype` (host, no GPU)."""
+    l = load_library()
+    w = np.ascontiguousarray(w_nk, dtype=np.float32)
+    if w.ndim != 2:
+        raise FnnError(4, "quantize_weights expects a 2-D [N,K] matrix")
+    rows, inner = w.shape
+    words = np.zeros(l.fnn_packed_words(dtype, rows, inner), np.uint32)
+    if dtype == DT_I4CB:
+        bpr = -(-inner // qblock)
+        scales = np.zeros(rows * bpr, np.float32)
+        zeros = np.zeros(0, np.float32)
+        cb = np.zeros(16, np.float32)
+    else:
+        scales = np.zeros(rows, np.float32)
+        zeros = np.zeros(rows, np.float32)
+        cb = None
+    rc = l.fnn_quantize_weights(dtype, _np_ptr(w), rows, inner, qblock if dtype == DT_I4CB else 0,
+                                _np_ptr(words), _np_ptr(scales), _np_ptr(zeros) if zeros.size else None,
+                                _np_ptr(cb))
+    if rc:
+        raise FnnError(rc, f"fnn_quantize_weights failed for dtype {dtype} (NaN in a codebook weight?)")
+    return PackedWeight(dtype, rows, inner, words, scales, zeros, qblock if dtype == DT_I4CB else 0, cb)
+
+
+def quantize_weights_kn(dtype: int, w_kn: np.ndarray, qblock: int = 32) -> PackedWeight:
+    """Logical [K,N] weight (as a graph holds it) -> transposed -> packed [N,K]."""
+    l = load_library()
+    w = np.ascontiguousarray(w_kn, dtype=np.float32)
+    k, n = w.shape
+    t = np.empty((n, k), np.float32)
+    l.fnn_transpose_kn_to_nk(_np_ptr(w), k, n, _np_ptr(t))
+    return quantize_weights(dtype, t, qblock)
+
+
+class DeviceBuffer:
+    """A device allocation owned by a HipContext."""
+
+    def __init__(self, ctx: "HipContext", nbytes: int):
+        self.ctx = ctx
+        self.nbytes = nbytes
+        p = _vp()
+        ctx._check(ctx.lib.fnn_hip_malloc(ctx.handle, nbytes, C.byref(p)))
+        self.ptr = p.value
+
+    def upload(self, arr: np.ndarray, offset: int = 0):
+        a = np.ascontiguousarray(arr)
+        assert offset + a.nbytes <= self.nbytes
+        self.ctx._check(self.ctx.lib.fnn_hip_upload(self.ctx.handle, _vp(self.ptr + offset), _np_ptr(a), a.nbytes))
+        return self
+
+    def download(self, dtype, count: int, offset: int = 0) -> np.ndarray:
+        out = np.empty(count, dtype=dtype)
+        assert offset + out.nbytes <= self.nbytes
+        self.ctx._check(self.ctx.lib.fnn_hip_download(self.ctx.handle, _np_ptr(out), _vp(self.ptr + offset), out.nbytes))
+        return out
+
+    def free(self):
+        if self.ptr:
+            self.ctx.lib.fnn_hip_free(self.ctx.handle, _vp(self.ptr))
+            self.ptr = 0
+
+
+class HipContext:
+    """One device + one HIP stream (fnn_hip_ctx)."""
+
+    def __init__(self, device: int = 0):
+        self.lib = load_library()
+        h = _vp()
+        rc = self.lib.fnn_hip_create(device, C.byref(h))
+        if rc:
+            raise FnnError(rc, self.lib.fnn_hip_last_error(None).decode())
+        self.handle = h
+        self._next_key = 1
+
+    def close(self):
+        if self.handle:
+            self.lib.fnn_hip_destroy(self.handle)
+            self.handle = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *a):
+        self.close()
+
+    def _check(self, rc: int):
+        if rc:
+            raise FnnError(rc, self.lib.fnn_hip_last_error(self.handle).decode())
+
+    def sync(self):
+        self._check(self.lib.fnn_hip_sync(self.handle))
+
+    def alloc(self, nbytes: int) -> DeviceBuffer:
+        return DeviceBuffer(self, nbytes)
+
+    def to_device(self, arr: np.ndarray) -> DeviceBuffer:
+        a = np.ascontiguousarray(arr)
+        return DeviceBuffer(self, max(a.nbytes, 16)).upload(a)
+
+    # ---- weights ----
+    def register(self, pw: PackedWeight, key: Optional[int] = None):
+        if key is None:
+            key = self._next_key
+            self._next_key += 1
+        h = _vp()
+        self._check(self.lib.fnn_hip_weight_register(
+            self.handle, key, pw.dtype, _np_ptr(pw.words), pw.words.size, pw.rows, pw.inner,
+            _np_ptr(pw.scales) if pw.scales.size else None, pw.scales.size,
+            _np_ptr(pw.zeros) if pw.zeros.size else None, pw.zeros.size, pw.qblock,
+            _np_ptr(pw.codebook) if pw.codebook is not None else None, C.byref(h)))
+        return h
+
+    def release(self, wh):
+        self._check(self.lib.fnn_hip_weight_release(self.handle, wh))
+
+    def dequant(self, wh, rows: int, inner: int) -> np.ndarray:
+        out = np.empty((rows, inner), np.float32)
+        self._check(self.lib.fnn_hip_dequant(self.handle, wh, _np_ptr(out), 0))
+        return out
+
+    # ---- MatMul ----
+    def qmatmul(self, wh, a: np.ndarray, n: int, bias: Optional[np.ndarray] = None, act: int = ACT_NONE,
+                flags: int = 0) -> np.ndarray:
+        """Host-pointer call: copies in, runs, copies out, synchronises."""
+        a = np.ascontiguousarray(a, dtype=np.float32)
+        m = a.shape[0]
+        out = np.empty((m, n), np.float32)
+        b = None if bias is None else np.ascontiguousarray(bias, dtype=np.float32)
+        self._check(self.lib.fnn_hip_qmatmul(self.handle, wh, _np_ptr(a), m, _np_ptr(b), act, _np_ptr(out), flags))
+        return out
+
+    def qmatmul_dev(self, wh, a_ptr: int, m: int, out_ptr: int, bias_ptr: int = 0, act: int = ACT_NONE,
+                    flags: int = 0):
+        """Device-pointer call: only enqueues on the context's stream."""
+        self._check(self.lib.fnn_hip_qmatmul(self.handle, wh, _vp(a_ptr), m, _vp(bias_ptr) if bias_ptr else None, act,
+                                             _vp(out_ptr), flags | FLAG_DEVICE_PTRS))
+
+    def quantize_activations(self, x: np.ndarray, scale: float = 0.0, zp: float = 0.0) -> np.ndarray:
+        x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1)
+        payload = np.zeros(8 + x.size, np.uint8)
+        self._check(self.lib.fnn_hip_quantize_activations(self.handle, _np_ptr(x), x.size, scale, zp,
+                                                          _np_ptr(payload), 0))
+        return payload
+
+    def qmatmul_i8act(self, wh, payload: np.ndarray, m: int, n: int, want_acc: bool = False, flags: int = 0):
+        payload = np.ascontiguousarray(payload, dtype=np.uint8)
+        out = np.empty((m, n), np.float32)
+        acc = np.zeros((m, n), np.int32) if want_acc else None
+        self._check(self.lib.fnn_hip_qmatmul_i8act(self.handle, wh, _np_ptr(payload), m, _np_ptr(out), _np_ptr(acc),
+                                                   flags))
+        return (out, acc) if want_acc else out
+
+    def qconv2d(self, wh, x: np.ndarray, oc: int, kh: int, kw: int, stride: int, pad: int, dil: int, groups: int,
+                bias: Optional[np.ndarray] = None, act: int = ACT_NONE, want_acc: bool = False):
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        b, c, h, w = x.shape
+
+        def osz(i, k):
+            dk = (k - 1) * dil + 1
+            return (i + 2 * pad - dk) // stride + 1 if i + 2 * pad >= dk else 0
+        ho, wo = osz(h, kh), osz(w, kw)
+        y = np.zeros((b, oc, ho, wo), np.float32)
+        acc = np.zeros((b, oc, ho, wo), np.int32) if want_acc else None
+        bb = None if bias is None else np.ascontiguousarray(bias, dtype=np.float32)
+        self._check(self.lib.fnn_hip_qconv2d(self.handle, wh, _np_ptr(x), b, c, h, w, kh, kw, stride, pad, dil, groups,
+                                             _np_ptr(bb), act, _np_ptr(y), _np_ptr(acc), 0))
+        return (y, acc) if want_acc else y
+
+    # ---- timing / graphs ----
+    def timer_start(self):
+        self._check(self.lib.fnn_hip_timer_start(self.handle))
+
+    def timer_stop(self) -> float:
+        ms = C.c_float()
+        self._check(self.lib.fnn_hip_timer_stop(self.handle, C.byref(ms)))
+        return ms.value
+
+    def graph_begin(self):
+        self._check(self.lib.fnn_hip_graph_begin(self.handle))
+
+    def graph_end(self):
+        g = _vp()
+        self._check(self.lib.fnn_hip_graph_end(self.handle, C.byref(g)))
+        return g
+
+    def graph_launch(self, g):
+        self._check(self.lib.fnn_hip_graph_launch(self.handle, g))
+
+    def graph_destroy(self, g):
+        self.lib.fnn_hip_graph_destroy(self.handle, g)

@@ -1,0 +1,166 @@
+/*
+ * fastnn_hip.h -- C ABI of libfastnn_hip.so: fastnn's weight-quantised MatMul
+ * path (fused dequant GEMV/GEMM, I8-activation GEMM, quantised Conv2d) as
+ * hand-written HIP kernels for gfx950 (MI355X).
+ *
+ * These are the entry points a `HipBackend: Backend` in fastnn binds through
+ * FFI.  Each declaration names the fastnn interface it replaces (paths are
+ * relative to the fastnn source tree).
+ *
+ * Conventions
+ *   - every function returns an fnn_status; nothing throws or aborts across
+ *     the boundary; the message of the last failure on a context is returned
+ *     by fnn_hip_last_error();
+ *   - one context = one device + one HIP stream; a context is not re-entrant,
+ *     matching the single-threaded dispatch contract of
+ *     src/backend/cpu/mod.rs:176-188;
+ *   - pointers are host pointers unless FNN_FLAG_DEVICE_PTRS is given; with
+ *     host pointers a call copies in, runs, copies out and synchronises; with
+ *     device pointers a call only enqueues work on the context's stream.
+ */
+#ifndef FASTNN_HIP_H
+#define FASTNN_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* BackendError variants of src/backend/mod.rs:6-12. */
+typedef enum {
+    FNN_OK = 0,
+    FNN_ERR_DISPATCH = 1,
+    FNN_ERR_MEMORY = 2,
+    FNN_ERR_UNSUPPORTED_OP = 3,
+    FNN_ERR_COMPILATION = 4
+} fnn_status;
+
+/* PackedWord types of src/dtypes/mod.rs:11-19; I4CB is I4x8 with a codebook
+ * (QuantizedWeightMeta.codebooks non-empty, src/backend/mod.rs:42-58). */
+typedef enum {
+    FNN_DT_I8 = 0,
+    FNN_DT_I4 = 1,
+    FNN_DT_U8 = 2,
+    FNN_DT_U4 = 3,
+    FNN_DT_F8 = 4,
+    FNN_DT_F8R = 5,
+    FNN_DT_F4 = 6,
+    FNN_DT_I4CB = 7
+} fnn_dtype;
+
+/* activation_type of src/backend/cpu/mod.rs:408-413 */
+typedef enum { FNN_ACT_NONE = 0, FNN_ACT_RELU = 1, FNN_ACT_GELU = 2, FNN_ACT_SILU = 3 } fnn_act;
+
+enum {
+    FNN_FLAG_DEVICE_PTRS = 1 << 0,    /* activations / outputs / bias live in device memory      */
+    FNN_FLAG_I4CB_AS_WRITTEN = 1 << 1,/* codebook MatMul multiplies by reshape(deq,[K,N]) the way */
+                                      /* src/backend/cpu/matmul.rs:206-212 does (K == N only)     */
+    FNN_FLAG_ACT_F16_SINGLE = 1 << 2, /* MFMA path: round activations to f16 once (default keeps  */
+                                      /* a second f16 residual term, i.e. ~22 mantissa bits)      */
+    FNN_FLAG_FORCE_GENERIC = 1 << 3   /* take the shape-agnostic kernel (testing aid)             */
+};
+
+typedef struct fnn_hip_ctx fnn_hip_ctx;
+typedef struct fnn_hip_weight fnn_hip_weight;
+typedef struct fnn_hip_graph fnn_hip_graph;
+
+/* ---- context: Backend::name / allocate_arena, src/backend/mod.rs:152-158 ---- */
+int fnn_hip_device_count(void);
+int fnn_hip_create(int device, fnn_hip_ctx **out);
+void fnn_hip_destroy(fnn_hip_ctx *ctx);
+/* message of the last failing call on ctx (ctx may be NULL for create failures) */
+const char *fnn_hip_last_error(fnn_hip_ctx *ctx);
+int fnn_hip_sync(fnn_hip_ctx *ctx);
+
+/* device arena: Backend::allocate_arena / write_arena / read_arena,
+ * src/backend/mod.rs:157,245-253 */
+int fnn_hip_malloc(fnn_hip_ctx *ctx, size_t bytes, void **dptr);
+int fnn_hip_free(fnn_hip_ctx *ctx, void *dptr);
+int fnn_hip_upload(fnn_hip_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes);
+int fnn_hip_download(fnn_hip_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes);
+
+/* ---- weights: get_or_cache_packed + packed_tensor_from_meta,
+ * src/backend/cpu/mod.rs:62-89, src/backend/cpu/matmul.rs:81-152.
+ * Uploads the packed words once; `key` identifies the weight the way the CPU
+ * cache keys (offset,size).  words: rows*ceil(inner/ITEMS) u32 (a trailing
+ * 16-word margin may be present and is ignored).  shape is [rows, inner] =
+ * [N, K] for MatMul, [OC, IC/g*KH*KW] for Conv2d.  n_zeros may be 0 (zeros
+ * are then 0.0).  codebook16 non-NULL selects the codebook type. */
+int fnn_hip_weight_register(fnn_hip_ctx *ctx, uint64_t key, int dtype, const uint32_t *words,
+                            size_t n_words, int64_t rows, int64_t inner, const float *scales,
+                            size_t n_scales, const float *zeros, size_t n_zeros,
+                            int quant_block_size, const float *codebook16, fnn_hip_weight **out);
+int fnn_hip_weight_lookup(fnn_hip_ctx *ctx, uint64_t key, fnn_hip_weight **out);
+int fnn_hip_weight_release(fnn_hip_ctx *ctx, fnn_hip_weight *w);
+
+/* PackedTensor::get_or_init_f32_weights, src/packed_tensor.rs:469-521:
+ * out[rows*inner] = unpack*scale + zero, or scales[blk]*codebook[nibble]. */
+int fnn_hip_dequant(fnn_hip_ctx *ctx, const fnn_hip_weight *w, float *out, int flags);
+
+/* ---- quantised MatMul with f32 activations:
+ * dispatch arms "matmul_i8|i4|u8|u4|f8|f8r|f4" (src/backend/cpu/mod.rs:3192-3315)
+ * -> quantized_matmul_dispatch (src/backend/cpu/matmul.rs:165-225)
+ * -> gemm_batch_packed_simd (src/backend/cpu/microkernels/gemm.rs:1982-2088);
+ * fused with the bias add and ReLU/GELU/SiLU that the MatMulAdd{Relu,Gelu,Silu}
+ * and Op{Relu,Gelu,Silu} fusions stand for
+ * (src/compiler/passes/fusion/matmul_add_relu.rs:92-110).
+ *   out[m,n] = act( (sum_k A[m,k]*u(W[n,k]))*scale[n] + zero[n]*sum_k A[m,k] + bias[n] )
+ * A: [M,K] f32 row-major; out: [M,N] f32 row-major; bias: [N] or NULL. */
+int fnn_hip_qmatmul(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *a, int64_t m,
+                    const float *bias, int act, float *out, int flags);
+
+/* ---- I8 activations: kernel "quantize_activations"
+ * (src/backend/cpu/mod.rs:6928-7008): payload = [scale f32][zp f32][numel x i8].
+ * scale <= 0 selects the dynamic mode (scale = max|x|/127, zp = 0). */
+int fnn_hip_quantize_activations(fnn_hip_ctx *ctx, const float *x, int64_t numel, float scale,
+                                 float zp, uint8_t *payload, int flags);
+
+/* "matmul_i8_i8" / "matmul_i4_i8": gemm_cpu_flat_i8_i8x4 / gemm_cpu_flat_i8_i4x8
+ * (src/backend/cpu/microkernels/gemm.rs:1641-1975).  acc_out (nullable, [M,N]
+ * i32) receives the exact integer accumulators sum q_w*q_a when zp_a == 0. */
+int fnn_hip_qmatmul_i8act(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const uint8_t *payload,
+                          int64_t m, float *out, int32_t *acc_out, int flags);
+
+/* ---- quantised Conv2d, I8 weights, f32 NCHW activations:
+ * conv2d_packed_i8x4 (src/backend/cpu/packed_conv.rs:1118-1196) =
+ * im2col + per-(image,group) dynamic int8 activation quantisation
+ * (packed_conv.rs:125-232) + gemm_packed_i8x4_fused_raw (packed_conv.rs:444-625).
+ * acc_out (nullable, same shape as y) receives the i32 accumulators incl. bias_q. */
+int fnn_hip_qconv2d(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *x, int64_t b,
+                    int64_t c, int64_t h, int64_t wd, int kh, int kw, int stride, int pad,
+                    int dil, int groups, const float *bias, int act, float *y, int32_t *acc_out,
+                    int flags);
+
+/* ---- stream timing (Backend::dispatch_profile, src/backend/mod.rs:178-211):
+ * HIP events recorded on the context's stream. */
+int fnn_hip_timer_start(fnn_hip_ctx *ctx);
+int fnn_hip_timer_stop(fnn_hip_ctx *ctx, float *elapsed_ms);
+
+/* ---- HIP graphs over device-pointer calls: capture a dispatch sequence once,
+ * replay it with one launch (a static-shape plan, src/backend/executor.rs:639-667). */
+int fnn_hip_graph_begin(fnn_hip_ctx *ctx);
+int fnn_hip_graph_end(fnn_hip_ctx *ctx, fnn_hip_graph **out);
+int fnn_hip_graph_launch(fnn_hip_ctx *ctx, fnn_hip_graph *g);
+int fnn_hip_graph_destroy(fnn_hip_ctx *ctx, fnn_hip_graph *g);
+
+/* ---- host-side weight quantisers (no GPU needed): the packers the
+ * quantisation pass calls (src/compiler/passes/quantization.rs:170-260,
+ * 281-495): from_f32_per_channel_asymmetric (I8/I4/U8/U4/F4,
+ * src/packed_tensor.rs:834-1049), from_f32_per_channel (F8/F8R, :661-742),
+ * from_f32_per_block_codebook (I4CB, :1209-1313).  w_nk is the transposed
+ * [N,K] matrix; words must hold fnn_packed_words() entries. */
+size_t fnn_packed_words(int dtype, int64_t rows, int64_t inner);
+int fnn_quantize_weights(int dtype, const float *w_nk, int64_t rows, int64_t inner,
+                         int quant_block_size, uint32_t *words, float *scales, float *zeros,
+                         float *codebook16);
+/* [K,N] -> [N,K] (quantization.rs:144-156) */
+void fnn_transpose_kn_to_nk(const float *w_kn, int64_t k, int64_t n, float *w_nk);
+
+const char *fnn_hip_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FASTNN_HIP_H */

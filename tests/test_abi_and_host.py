@@ -1,0 +1,115 @@
+"""CPU-only checks of the product: the C-ABI library loads and exports every symbol the
+public header declares, and the host-side weight packers are bit-identical to the oracle."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+import fastnn_amd
+from fastnn_amd import lib as flib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    l = fastnn_amd.load_library()
+    header = open(os.path.join(ROOT, "include", "fastnn_hip.h")).read()
+    declared = set(re.findall(r"\b(fnn_[a-z0-9_]+)\s*\(", header))
+    declared -= {"fnn_status", "fnn_dtype", "fnn_act"}
+    assert declared, "no declarations parsed"
+    for name in sorted(declared):
+        assert hasattr(l, name), f"{name} declared in fastnn_hip.h but not exported"
+    assert declared == set(flib.EXPORTED_SYMBOLS)
+    assert b"gfx950" in l.fnn_hip_version()
+
+
+def test_backend_header_symbols_exported():
+    path = os.path.join(ROOT, "include", "fastnn_hip_backend.h")
+    if not os.path.exists(path):
+        pytest.skip("backend header not present")
+    l = fastnn_amd.load_library()
+    declared = set(re.findall(r"\b(fnn_backend_[a-z0-9_]+|fnn_plan_[a-z0-9_]+)\s*\(", open(path).read()))
+    for name in sorted(declared):
+        assert hasattr(l, name), name
+
+
+def test_missing_library_fails_loudly(tmp_path):
+    with pytest.raises(FileNotFoundError):
+        flib.load_library(str(tmp_path / "nope.so"))
+
+
+def test_no_product_file_touches_the_oracle():
+    """The shipped package must not import, link or call anything under oracle/."""
+    pkg = os.path.join(ROOT, "fastnn_amd")
+    for dirpath, _, files in os.walk(pkg):
+        if os.path.basename(dirpath) == "build":
+            continue
+        for f in files:
+            if f.endswith((".py", ".cpp", ".hip", ".h")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "fnn_oracle" not in text and "import oracle" not in text and "from oracle" not in text, f
+
+
+DTS = [flib.DT_I8, flib.DT_I4, flib.DT_U8, flib.DT_U4, flib.DT_F8, flib.DT_F8R, flib.DT_F4, flib.DT_I4CB]
+
+
+@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("shape", [(16, 64), (7, 37), (3, 5), (64, 512)])
+def test_host_packers_bit_identical_to_oracle(orc, dt, shape):
+    rng = np.random.default_rng(1000 + dt)
+    w = (rng.standard_normal(shape) * 0.02).astype(np.float32)
+    mask = rng.random(shape) < 0.01
+    w[mask] *= 8
+    if shape[0] > 2:
+        w[1] = 0.0            # all-zero row
+        w[2] = 0.015          # constant row (zero range)
+    pw = fastnn_amd.quantize_weights(dt, w)
+    po = orc.quantize(dt, w)
+    assert np.array_equal(pw.words, po.words)
+    assert pw.scales.tobytes() == po.scales.tobytes()
+    assert pw.zeros.tobytes() == po.zeros.tobytes()
+    if dt == flib.DT_I4CB:
+        assert pw.codebook.tobytes() == po.codebook.tobytes()
+        assert pw.qblock == 32
+
+
+def test_host_packers_special_values(orc):
+    vals = np.array([[0.0, -0.0, 1e-9, -1e-9, 300.0, -300.0, 0.0146, 0.0147, 0.99999994, 1.0000001,
+                      239.9, 240.1, 2.0 ** -9, 2.0 ** -10, 1.5 * 2.0 ** -9, 57344.0, 65536.0, 3e-5, 1.6e-5, 447.0]],
+                    np.float32)
+    for dt in (flib.DT_F8, flib.DT_F8R, flib.DT_F4, flib.DT_I8, flib.DT_I4):
+        pw = fastnn_amd.quantize_weights(dt, vals)
+        po = orc.quantize(dt, vals)
+        assert np.array_equal(pw.words, po.words), dt
+        assert pw.scales.tobytes() == po.scales.tobytes()
+    # direct lane encoders through a unit-scale row: scale == 1 when max|row| == MAX_REPRESENTABLE
+    row = np.concatenate([vals[0][np.abs(vals[0]) <= 240], [240.0]]).astype(np.float32)[None, :]
+    pw = fastnn_amd.quantize_weights(flib.DT_F8, row)
+    po = orc.quantize(orc.F8, row)
+    assert pw.scales[0] == 1.0 and np.array_equal(pw.words, po.words)
+
+
+def test_codebook_packer_large_matches_oracle(orc):
+    rng = np.random.default_rng(5)
+    w = np.where(rng.random((96, 256)) < 0.9, rng.laplace(0, 0.02, (96, 256)), rng.laplace(0, 0.1, (96, 256)))
+    w = w.astype(np.float32)
+    pw = fastnn_amd.quantize_weights(flib.DT_I4CB, w)
+    po = orc.quantize(orc.I4CB, w)
+    assert np.array_equal(pw.words, po.words)
+    assert pw.codebook.tobytes() == po.codebook.tobytes()
+    assert pw.scales.tobytes() == po.scales.tobytes()
+    with pytest.raises(fastnn_amd.FnnError):
+        bad = w.copy()
+        bad[0, 0] = np.nan
+        fastnn_amd.quantize_weights(flib.DT_I4CB, bad)
+
+
+def test_transpose_kn(orc):
+    rng = np.random.default_rng(6)
+    w = rng.standard_normal((70, 45)).astype(np.float32)
+    pw = fastnn_amd.quantize_weights_kn(flib.DT_I8, w)
+    po = orc.quantize_kn(orc.I8, w)
+    assert pw.rows == 45 and pw.inner == 70
+    assert np.array_equal(pw.words, po.words)

@@ -1,0 +1,338 @@
+"""GPU parity tests: the HIP path, called through the C ABI, against the CPU oracle on the
+same seeded inputs.  Bit-exact for packing, unpacking, codebook lookup, integer
+accumulators and quantised activations; float outputs within the tolerance stated at each
+test (max |d| / max |ref| and element-wise |d| <= tol*|ref| + tol*max|ref|)."""
+import numpy as np
+import pytest
+
+import fastnn_amd
+from fastnn_amd import lib as flib
+from gpu_common import NAMES, assert_close, rel_err, slice_rows, to_oracle
+
+pytestmark = pytest.mark.gpu
+
+ALL_DT = list(range(8))
+# f32-accumulate kernels (FMA GEMV, generic): stated tolerance 2e-5 of max|ref| vs the f64 oracle
+TOL_F32 = 2e-5
+# north-star bound for every f32-accumulate path
+TOL_NORTH_STAR = 1e-3
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = fastnn_amd.HipContext(0)
+    yield c
+    c.close()
+
+
+def _weights(rng, n, k, dist="normal"):
+    if dist == "laplace":
+        w = np.where(rng.random((n, k)) < 0.9, rng.laplace(0, 0.02, (n, k)), rng.laplace(0, 0.1, (n, k)))
+    else:
+        w = rng.standard_normal((n, k)) * 0.02
+        w[rng.random((n, k)) < 0.001] *= 8
+    return w.astype(np.float32)
+
+
+# --------------------------------------------------------------------------- decode
+def test_fp8_fp4_decode_tables_bit_exact(ctx, orc):
+    """Every F8/F8R byte and F4 nibble at every lane position decodes to the reference value
+    (NaN for all exponent-15 E4M3 bytes, +0.0 for FP4 nibble 0x8)."""
+    for dt, bits in ((flib.DT_F8, 8), (flib.DT_F8R, 8), (flib.DT_F4, 4)):
+        items = 32 // bits
+        ncodes = 1 << bits
+        # row r: code (r + lane) mod ncodes at every lane -> all codes at all positions
+        words = np.zeros(ncodes + 16, np.uint32)
+        for r in range(ncodes):
+            w = 0
+            for i in range(items):
+                w |= ((r + i) % ncodes) << (bits * i)
+            words[r] = w
+        pw = fastnn_amd.PackedWeight(dt, ncodes, items, words, np.ones(ncodes, np.float32),
+                                     np.zeros(ncodes, np.float32))
+        h = ctx.register(pw)
+        got = ctx.dequant(h, ncodes, items)
+        want = orc.dequant(to_oracle(orc, pw))
+        assert np.array_equal(np.isnan(got), np.isnan(want)), NAMES[dt]
+        ok = ~np.isnan(want)
+        assert np.array_equal(got[ok].view(np.uint32), want[ok].view(np.uint32)), NAMES[dt]
+        ctx.release(h)
+
+
+@pytest.mark.parametrize("dt", ALL_DT)
+@pytest.mark.parametrize("shape", [(64, 128), (33, 77), (5, 3), (256, 4096)])
+def test_dequant_bit_exact(ctx, orc, dt, shape):
+    """unpack*scale+zero (one multiply, one add) and scales[blk]*codebook[nibble] are bit-exact."""
+    rng = np.random.default_rng(2000 + dt)
+    n, k = shape
+    pw = fastnn_amd.quantize_weights(dt, _weights(rng, n, k, "laplace" if dt == 7 else "normal"))
+    h = ctx.register(pw)
+    got = ctx.dequant(h, n, k)
+    want = orc.dequant(to_oracle(orc, pw))
+    assert got.tobytes() == want.tobytes()
+    ctx.release(h)
+    if dt != flib.DT_I4CB:  # raw random words: every code incl. NaN bytes, random scales/zeros
+        items = 32 // pw.bit_width
+        kp = -(-k // items)
+        words = rng.integers(0, 2 ** 32, n * kp + 16, dtype=np.uint64).astype(np.uint32)
+        pr = fastnn_amd.PackedWeight(dt, n, k, words, rng.uniform(0.01, 2, n).astype(np.float32),
+                                     rng.uniform(-1, 1, n).astype(np.float32))
+        h = ctx.register(pr)
+        got = ctx.dequant(h, n, k)
+        want = orc.dequant(to_oracle(orc, pr))
+        assert np.array_equal(np.isnan(got), np.isnan(want))
+        ok = ~np.isnan(want)
+        assert np.array_equal(got[ok].view(np.uint32), want[ok].view(np.uint32))
+        ctx.release(h)
+
+
+def test_grouped_and_scalar_scales(ctx, orc):
+    rng = np.random.default_rng(3)
+    n, k = 12, 40
+    words = rng.integers(0, 2 ** 32, n * 10 + 16, dtype=np.uint64).astype(np.uint32)
+    for ns in (1, 3, 12):
+        pw = fastnn_amd.PackedWeight(flib.DT_I8, n, k, words, rng.uniform(0.5, 1.5, ns).astype(np.float32),
+                                     rng.uniform(-1, 1, ns).astype(np.float32))
+        h = ctx.register(pw)
+        assert ctx.dequant(h, n, k).tobytes() == orc.dequant(to_oracle(orc, pw)).tobytes()
+        a = rng.standard_normal((2, k)).astype(np.float32)
+        assert_close(ctx.qmatmul(h, a, n), orc.qmatmul(to_oracle(orc, pw), a), TOL_F32)
+        ctx.release(h)
+    # zero_points omitted (FP8 metadata): treated as zeros
+    pw = fastnn_amd.PackedWeight(flib.DT_F8, n, k, words & np.uint32(0x77777777),
+                                 rng.uniform(0.5, 1.5, n).astype(np.float32), np.zeros(0, np.float32))
+    h = ctx.register(pw)
+    po = orc.Packed(orc.F8, n, k, pw.words, pw.scales, np.zeros(n, np.float32))
+    assert ctx.dequant(h, n, k).tobytes() == orc.dequant(po).tobytes()
+    ctx.release(h)
+
+
+# --------------------------------------------------------------------------- f32-activation MatMul
+GEMV_SHAPES = [(1, 256, 64), (1, 1024, 100), (2, 512, 48), (3, 2048, 33), (4, 4096, 128), (1, 8192, 16)]
+RAGGED_SHAPES = [(1, 7, 5), (3, 9, 4), (2, 100, 17), (5, 61, 130), (9, 333, 20), (17, 4100, 12), (1, 48, 8)]
+
+
+@pytest.mark.parametrize("dt", ALL_DT)
+@pytest.mark.parametrize("m,k,n", GEMV_SHAPES + RAGGED_SHAPES)
+def test_qmatmul_matches_oracle(ctx, orc, dt, m, k, n):
+    rng = np.random.default_rng(3000 + dt * 17 + k)
+    pw = fastnn_amd.quantize_weights(dt, _weights(rng, n, k, "laplace" if dt == 7 else "normal"))
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    h = ctx.register(pw)
+    want = orc.qmatmul(to_oracle(orc, pw), a, order=2)
+    got = ctx.qmatmul(h, a, n)
+    assert_close(got, want, TOL_F32, f"{NAMES[dt]} {m}x{k}x{n}")
+    gen = ctx.qmatmul(h, a, n, flags=flib.FLAG_FORCE_GENERIC)
+    assert_close(gen, want, TOL_F32, f"generic {NAMES[dt]} {m}x{k}x{n}")
+    # the reference's own f32 summation orders sit inside the same band
+    assert rel_err(orc.qmatmul(to_oracle(orc, pw), a, order=1), want) <= TOL_F32 * 5
+    ctx.release(h)
+
+
+@pytest.mark.parametrize("dt", [0, 1, 4, 6, 7])
+@pytest.mark.parametrize("act", [0, 1, 2, 3])
+@pytest.mark.parametrize("m,k,n", [(1, 512, 96), (3, 130, 50)])
+def test_fused_bias_activation(ctx, orc, dt, act, m, k, n):
+    """act(matmul + bias) equals the unfused chain matmul_q -> add -> act."""
+    rng = np.random.default_rng(4000 + dt + act)
+    pw = fastnn_amd.quantize_weights(dt, _weights(rng, n, k, "laplace" if dt == 7 else "normal"))
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    bias = (rng.standard_normal(n) * 0.01).astype(np.float32)
+    h = ctx.register(pw)
+    want = orc.qmatmul(to_oracle(orc, pw), a, order=2, bias=bias, act=act)
+    assert_close(ctx.qmatmul(h, a, n, bias=bias, act=act), want, TOL_F32)
+    want_nb = orc.qmatmul(to_oracle(orc, pw), a, order=2, act=act)
+    assert_close(ctx.qmatmul(h, a, n, act=act), want_nb, TOL_F32)
+    ctx.release(h)
+
+
+def test_reference_literal_cases_on_gpu(ctx, orc, golden):
+    g = golden["gemm_f32act"]["asymmetric_zero_is_per_input_sum"]
+    po = orc.from_f32_slice(orc.I8, g["weights_f32"], g["n"], g["k"], g["w_scale"], g["w_zero"])
+    pw = fastnn_amd.PackedWeight(flib.DT_I8, g["n"], g["k"], po.words, po.scales, po.zeros)
+    h = ctx.register(pw)
+    a = np.array(g["input"], np.float32).reshape(g["m"], g["k"])
+    assert np.allclose(ctx.qmatmul(h, a, g["n"]).reshape(-1), g["expected"], atol=g["abs_tol"])
+    ctx.release(h)
+    dts = {"i4": 1, "i8": 0, "f8": 4, "f8r": 5}
+    for c in golden["seeded_end_to_end"]["cases"]:
+        if c["quantize"] not in dts:
+            continue
+        m, k, n = c["m"], c["k"], c["n"]
+        a = orc.seeded_values(c["seed"], m * k).reshape(m, k)
+        w = orc.seeded_values(c["seed"] + 1, k * n).reshape(k, n)
+        pw = fastnn_amd.quantize_weights_kn(dts[c["quantize"]], w)
+        h = ctx.register(pw)
+        got = ctx.qmatmul(h, a, n)
+        expected = (a.astype(np.float64) @ w.astype(np.float64))
+        allowed = np.maximum(c["abs_tol"], np.abs(expected) * c["rel_tol"])
+        assert np.all(np.abs(got - expected) <= allowed), c
+        ctx.release(h)
+
+
+def test_i4cb_as_written_variant(ctx, orc):
+    rng = np.random.default_rng(8)
+    n = k = 64
+    pw = fastnn_amd.quantize_weights(flib.DT_I4CB, _weights(rng, n, k, "laplace"))
+    a = rng.standard_normal((3, k)).astype(np.float32)
+    h = ctx.register(pw)
+    want = orc.qmatmul(to_oracle(orc, pw), a, order=2, i4cb_as_written=True)
+    assert_close(ctx.qmatmul(h, a, n, flags=flib.FLAG_I4CB_AS_WRITTEN), want, TOL_F32)
+    ctx.release(h)
+
+
+def test_device_pointer_calls_and_graph_replay(ctx, orc):
+    rng = np.random.default_rng(9)
+    n, k, m = 256, 1024, 1
+    pw = fastnn_amd.quantize_weights(flib.DT_I4, _weights(rng, n, k))
+    h = ctx.register(pw)
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    bias = (rng.standard_normal(n) * 0.01).astype(np.float32)
+    da, db, dout = ctx.to_device(a), ctx.to_device(bias), ctx.alloc(m * n * 4)
+    want = orc.qmatmul(to_oracle(orc, pw), a, order=2, bias=bias, act=3)
+    ctx.qmatmul_dev(h, da.ptr, m, dout.ptr, db.ptr, act=3)
+    ctx.sync()
+    eager = dout.download(np.float32, m * n).reshape(m, n)
+    assert_close(eager, want, TOL_F32)
+    ctx.graph_begin()
+    ctx.qmatmul_dev(h, da.ptr, m, dout.ptr, db.ptr, act=3)
+    g = ctx.graph_end()
+    for rep in range(3):  # every replay, with eager work and syncs in between, equals the eager result
+        dout.upload(np.zeros(m * n, np.float32))
+        ctx.graph_launch(g)
+        ctx.sync()
+        assert dout.download(np.float32, m * n).tobytes() == eager.tobytes(), rep
+        a2 = rng.standard_normal((m, k)).astype(np.float32)
+        ctx.qmatmul(h, a2, n)
+    ctx.graph_destroy(g)
+    for b in (da, db, dout):
+        b.free()
+    ctx.release(h)
+
+
+# --------------------------------------------------------------------------- I8 activations
+@pytest.mark.parametrize("numel", [1, 7, 256, 4099, 100000])
+def test_quantize_activations_bit_exact(ctx, orc, numel):
+    rng = np.random.default_rng(10 + numel)
+    x = (rng.standard_normal(numel) * 3).astype(np.float32)
+    assert ctx.quantize_activations(x).tobytes() == orc.quantize_activations(x).tobytes()
+    assert ctx.quantize_activations(x, 0.05, 0.25).tobytes() == orc.quantize_activations(x, 0.05, 0.25).tobytes()
+    z = np.zeros(numel, np.float32)
+    assert ctx.quantize_activations(z).tobytes() == orc.quantize_activations(z).tobytes()
+
+
+@pytest.mark.parametrize("dt", [0, 1])
+@pytest.mark.parametrize("m,k,n", [(1, 64, 32), (3, 61, 10), (16, 256, 64), (40, 1000, 72), (128, 512, 256)])
+@pytest.mark.parametrize("zp", [0.0, 0.375])
+def test_i8act_matmul_integer_exact(ctx, orc, dt, m, k, n, zp):
+    rng = np.random.default_rng(5000 + dt + k)
+    pw = fastnn_amd.quantize_weights(dt, _weights(rng, n, k))
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    payload = orc.quantize_activations(x) if zp == 0.0 else orc.quantize_activations(x, 0.03, zp)
+    h = ctx.register(pw)
+    want, want_acc = orc.qmatmul_i8act(to_oracle(orc, pw), payload, m, want_acc=True)
+    for flags in (0, flib.FLAG_FORCE_GENERIC):
+        got, acc = ctx.qmatmul_i8act(h, payload, m, n, want_acc=True, flags=flags)
+        if zp == 0.0:
+            assert np.array_equal(acc, want_acc)          # i32 accumulators bit-exact
+            assert_close(got, want, 1e-6)                  # same f32 formula on identical integers
+        else:
+            assert_close(got, want, TOL_F32)               # per-lane f32 path, summation order differs
+    ctx.release(h)
+
+
+def test_i8act_literals_on_gpu(ctx, orc, golden):
+    dts = {"i8": 0, "i4": 1}
+    for c in golden["gemm_i8act"]["cases"]:
+        po = orc.from_f32_slice(dts[c["dt"]], c["weights_f32"], c["n"], c["k"], c["w_scale"], c["w_zero"])
+        pw = fastnn_amd.PackedWeight(dts[c["dt"]], c["n"], c["k"], po.words, po.scales, po.zeros)
+        h = ctx.register(pw)
+        payload = orc.make_payload(c["act_scale"], c["act_zp"], c["act_i8"])
+        got = ctx.qmatmul_i8act(h, payload, c["m"], c["n"]).reshape(-1)
+        want = np.array(c["expected"]) if "expected" in c else orc.qmatmul_i8act(po, payload, c["m"]).reshape(-1)
+        assert np.allclose(got, want, atol=c["abs_tol"]), c["name"]
+        ctx.release(h)
+
+
+# --------------------------------------------------------------------------- quantised Conv2d
+CONVS = [
+    dict(b=2, c=3, h=20, w=24, oc=16, kh=3, kw=3, stride=2, pad=1, dil=1, groups=1),
+    dict(b=1, c=16, h=12, w=12, oc=32, kh=1, kw=1, stride=1, pad=0, dil=1, groups=1),
+    dict(b=1, c=8, h=10, w=7, oc=6, kh=3, kw=2, stride=1, pad=2, dil=2, groups=2),
+    dict(b=3, c=5, h=9, w=9, oc=7, kh=3, kw=3, stride=1, pad=1, dil=1, groups=1),
+    dict(b=1, c=32, h=16, w=16, oc=64, kh=3, kw=3, stride=1, pad=1, dil=1, groups=1),
+]
+
+
+@pytest.mark.parametrize("cfg", CONVS)
+@pytest.mark.parametrize("act", [0, 1, 3, 2])
+def test_qconv2d_i8(ctx, orc, cfg, act):
+    rng = np.random.default_rng(6000 + cfg["c"])
+    kk = cfg["c"] // cfg["groups"] * cfg["kh"] * cfg["kw"]
+    x = rng.uniform(0, 1, (cfg["b"], cfg["c"], cfg["h"], cfg["w"])).astype(np.float32)
+    wt = (rng.standard_normal((cfg["oc"], kk)) * np.sqrt(2.0 / kk)).astype(np.float32)
+    bias = (rng.standard_normal(cfg["oc"]) * 0.05).astype(np.float32)
+    pw = fastnn_amd.quantize_weights(flib.DT_I8, wt)
+    h = ctx.register(pw)
+    args = (cfg["kh"], cfg["kw"], cfg["stride"], cfg["pad"], cfg["dil"], cfg["groups"])
+    want, want_acc, _, _ = orc.qconv2d_i8(x, to_oracle(orc, pw), *args, bias=bias, act=act, want_acc=True)
+    got, acc = ctx.qconv2d(h, x, cfg["oc"], *args, bias=bias, act=act, want_acc=True)
+    assert np.array_equal(acc, want_acc)   # i32 accumulators (incl. bias_q) bit-exact
+    assert_close(got, want, 1e-5)          # same f32 formula; expf/tanhf differ in the last ulp
+    got_nb = ctx.qconv2d(h, x, cfg["oc"], *args, act=act)
+    assert_close(got_nb, orc.qconv2d_i8(x, to_oracle(orc, pw), *args, act=act), 1e-5)
+    ctx.release(h)
+
+
+def test_qconv2d_constant_and_empty(ctx, orc):
+    x = np.full((1, 2, 4, 4), 0.5, np.float32)
+    pw = fastnn_amd.quantize_weights(flib.DT_I8, np.array([[-0.2, 0.1], [0.1, 0.1]], np.float32))
+    h = ctx.register(pw)
+    got = ctx.qconv2d(h, x, 2, 1, 1, 1, 0, 1, 1)
+    assert_close(got, orc.qconv2d_i8(x, to_oracle(orc, pw), 1, 1, 1, 0, 1, 1), 1e-6)
+    # kernel larger than the padded input: empty output, no launch
+    y = ctx.qconv2d(h, np.zeros((1, 2, 1, 1), np.float32)[:, :, :1, :1], 2, 1, 1, 1, 0, 1, 1)
+    assert y.shape == (1, 2, 1, 1)
+    ctx.release(h)
+
+
+# --------------------------------------------------------------------------- error behaviour
+def test_error_paths_mirror_reference_messages(ctx):
+    rng = np.random.default_rng(11)
+    pw = fastnn_amd.quantize_weights(flib.DT_I8, rng.standard_normal((8, 16)).astype(np.float32))
+    bad = fastnn_amd.PackedWeight(pw.dtype, 8, 16, pw.words, np.zeros(0, np.float32), pw.zeros)
+    with pytest.raises(fastnn_amd.FnnError) as e:
+        ctx.register(bad)
+    assert e.value.kind == "Dispatch" and "scale" in e.value.message  # public_error_paths.rs:42-118
+    bad = fastnn_amd.PackedWeight(pw.dtype, 8, 16, pw.words, pw.scales[:3].copy(), pw.zeros[:3].copy())
+    with pytest.raises(fastnn_amd.FnnError) as e:
+        ctx.register(bad)
+    assert "incompatible with shape" in e.value.message
+    bad = fastnn_amd.PackedWeight(pw.dtype, 8, 16, pw.words[:10].copy(), pw.scales, pw.zeros)
+    with pytest.raises(fastnn_amd.FnnError) as e:
+        ctx.register(bad)
+    assert "payload too short" in e.value.message
+    bad = fastnn_amd.PackedWeight(pw.dtype, 8, 16, pw.words, pw.scales, pw.zeros[:4].copy())
+    with pytest.raises(fastnn_amd.FnnError) as e:
+        ctx.register(bad)
+    assert "length mismatch" in e.value.message
+    with pytest.raises(fastnn_amd.FnnError) as e:
+        ctx.register(fastnn_amd.PackedWeight(42, 8, 16, pw.words, pw.scales, pw.zeros))
+    assert e.value.kind == "UnsupportedOp"
+    h = ctx.register(pw, key=777)
+    with pytest.raises(fastnn_amd.FnnError):
+        ctx.register(pw, key=777)
+    with pytest.raises(fastnn_amd.FnnError) as e:
+        ctx.qmatmul(h, np.zeros((1, 16), np.float32), 8, act=9)
+    assert e.value.kind == "UnsupportedOp"
+    f8 = ctx.register(fastnn_amd.quantize_weights(flib.DT_F8, rng.standard_normal((8, 16)).astype(np.float32)))
+    with pytest.raises(fastnn_amd.FnnError) as e:
+        ctx.qmatmul_i8act(f8, np.zeros(8 + 16, np.uint8), 1, 8)
+    assert e.value.kind == "UnsupportedOp"
+    with pytest.raises(fastnn_amd.FnnError) as e:
+        ctx.qconv2d(h, np.zeros((1, 4, 4, 4), np.float32), 8, 2, 2, 1, 0, 1, 0)
+    assert "groups" in e.value.message
+    out = ctx.qmatmul(h, np.zeros((0, 16), np.float32), 8)   # empty batch is a no-op
+    assert out.shape == (0, 8)
+    ctx.release(h)
+    ctx.release(f8)
