@@ -1,0 +1,261 @@
+#!/usr/bin/env python3
+"""Benchmark of the weight-quantised MatMul hot path on one MI355X.
+
+A step is one fused dequant-MatMul call (bias + SiLU epilogue) over one batch of synthetic
+activations, with every operand already resident in HBM.  The default workload is the
+I4 GEMM of BASELINE.json's configs[1] (K=4096, N=11008) at M=1 (bandwidth-bound GEMV);
+`--m 256` selects the matrix-core regime of the same configuration.  Consecutive steps
+walk over a ring of distinct weight copies larger than the 256 MB Infinity Cache, so the
+reported GB/s is HBM traffic, not cache replay (`--ring 1` gives the warm number).
+
+Prints ONE JSON line (metric/value/... plus `roofline` and `cpu_baseline`).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "i8": 5000.0, "fp8": 5000.0}
+
+WORKLOADS = {
+    # name: (dtype name, K, N, bias, act)
+    "c1_i8": ("i8", 4096, 4096, False, "none"),
+    "c2_i4": ("i4", 4096, 11008, True, "silu"),
+    "c3_i4cb": ("i4cb", 4096, 4096, False, "none"),
+    "c4_f8_up": ("f8", 2048, 8192, False, "gelu"),
+    "c4_f4_up": ("f4", 2048, 8192, False, "gelu"),
+}
+
+
+def synth_weight(name: str, k: int, n: int, rng) -> np.ndarray:
+    """[N,K] f32 weights with the distribution the configuration names (seed 0)."""
+    if name == "c3_i4cb":
+        w = np.where(rng.random((n, k)) < 0.9, rng.laplace(0, 0.02, (n, k)), rng.laplace(0, 0.10, (n, k)))
+    elif name.startswith("c4"):
+        w = rng.standard_normal((n, k)) / np.sqrt(k)
+    else:
+        w = rng.standard_normal((n, k)) * 0.02
+        if name == "c2_i4":
+            idx = rng.choice(n * k, size=(n * k) // 1000, replace=False)
+            w.reshape(-1)[idx] *= 8
+    return w.astype(np.float32)
+
+
+def algorithmic_bytes(dt: str, m: int, k: int, n: int, bias: bool) -> int:
+    """Every operand read once + output written once; packed weights without the margin."""
+    bits = 8 if dt in ("i8", "u8", "f8", "f8r") else 4
+    wbytes = n * k * bits // 8
+    if dt == "i4cb":
+        side = 4 * n * (k // 32) + 64
+    elif dt in ("f8", "f8r"):
+        side = 4 * n
+    else:
+        side = 8 * n
+    if bias:
+        side += 4 * n
+    return wbytes + side + 4 * m * k + 4 * m * n
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=480)
+    ap.add_argument("--warmup", type=int, default=48)
+    ap.add_argument("--workload", default="c2_i4", choices=sorted(WORKLOADS))
+    ap.add_argument("--m", type=int, default=1)
+    ap.add_argument("--ring", type=int, default=0, help="distinct weight copies (0: enough for > 512 MB)")
+    ap.add_argument("--mode", default="graph", choices=["graph", "eager"])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--fast-act16", action="store_true", help="single f16 rounding of activations on the MFMA path")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (the path shards over N without changing the "
+              "per-GPU kernel); run with --gpus 1", file=sys.stderr)
+        return 2
+
+    import fastnn_amd
+    from fastnn_amd import lib as flib
+
+    dtn, k, n, has_bias, actn = WORKLOADS[args.workload]
+    dt = {"i8": flib.DT_I8, "i4": flib.DT_I4, "i4cb": flib.DT_I4CB, "f8": flib.DT_F8, "f4": flib.DT_F4}[dtn]
+    act = {"none": 0, "relu": 1, "gelu": 2, "silu": 3}[actn]
+    m = args.m
+    rng = np.random.default_rng(0)
+    w = synth_weight(args.workload, k, n, rng)
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    bias = (rng.standard_normal(n) * 0.01).astype(np.float32) if has_bias else None
+    t0 = time.time()
+    pw = fastnn_amd.quantize_weights(dt, w)
+    t_quant = time.time() - t0
+    del w
+
+    wbytes = pw.packed_bytes()
+    ring = args.ring if args.ring > 0 else max(2, int(np.ceil(544e6 / wbytes)))
+    flags = flib.FLAG_ACT_F16_SINGLE if args.fast_act16 else 0
+
+    ctx = fastnn_amd.HipContext(0)
+    handles = []
+    items = 32 // pw.bit_width
+    kp = -(-k // items)
+    base_words = pw.words[: n * kp].reshape(n, kp)
+    for i in range(ring):
+        # distinct HBM buffers: the same matrix with its rows rotated by i
+        if i == 0:
+            pwi = pw
+        else:
+            words = np.concatenate([np.roll(base_words, i, axis=0).reshape(-1), np.zeros(16, np.uint32)])
+            if dt == flib.DT_I4CB:
+                bpr = k // 32
+                sc = np.roll(pw.scales.reshape(n, bpr), i, axis=0).reshape(-1).copy()
+                zr = pw.zeros
+            else:
+                sc, zr = np.roll(pw.scales, i).copy(), np.roll(pw.zeros, i).copy()
+            pwi = fastnn_amd.PackedWeight(dt, n, k, words, sc, zr, pw.qblock, pw.codebook)
+        handles.append(ctx.register(pwi))
+    da = ctx.to_device(a)
+    dbias = ctx.to_device(bias) if has_bias else None
+    dout = ctx.alloc(m * n * 4)
+
+    def step(i: int):
+        ctx.qmatmul_dev(handles[i % ring], da.ptr, m, dout.ptr, dbias.ptr if dbias else 0, act, flags)
+
+    # untimed warmup (also sizes internal workspaces before any capture)
+    for i in range(args.warmup):
+        step(i)
+    ctx.sync()
+
+    steps = args.steps
+    graph = None
+    if args.mode == "graph":
+        # one graph = one trip round the ring; replayed steps/ring times
+        reps = max(1, steps // ring)
+        steps = reps * ring
+        ctx.graph_begin()
+        for i in range(ring):
+            step(i)
+        graph = ctx.graph_end()
+        ctx.graph_launch(graph)
+        ctx.sync()
+
+    ctx.sync()
+    t_start = time.perf_counter()
+    ctx.timer_start()
+    if graph is not None:
+        for _ in range(steps // ring):
+            ctx.graph_launch(graph)
+    else:
+        for i in range(steps):
+            step(i)
+    ev_ms = ctx.timer_stop()
+    ctx.sync()
+    wall_s = time.perf_counter() - t_start
+
+    ms_per_step = wall_s * 1e3 / steps
+    kernel_ms = ev_ms / steps            # HIP events on the launch stream over the timed region
+    abytes = algorithmic_bytes(dtn, m, k, n, has_bias)
+    flops = 2.0 * m * k * n
+    gbs = abytes / (ms_per_step * 1e-3) / 1e9
+    tops = flops / (ms_per_step * 1e-3) / 1e12
+
+    # what was timed is checked against a second, independent kernel (the shape-agnostic one)
+    # on the weight copy the last step used
+    got = dout.download(np.float32, m * n).reshape(m, n)
+    chk = ctx.qmatmul(handles[(steps - 1) % ring], a, n, bias=bias, act=act,
+                      flags=flags | flib.FLAG_FORCE_GENERIC)
+    self_check = float(np.abs(got - chk).max() / (np.abs(chk).max() + 1e-30))
+
+    bandwidth_bound = m <= 32
+    if bandwidth_bound:
+        achieved = abytes / (kernel_ms * 1e-3) / 1e9
+        roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                    "kernel_us": round(kernel_ms * 1e3, 3), "algorithmic_bytes": abytes}
+        metric, value, unit = f"qGEMM GB/s at M={m} ({dtn} K={k} N={n})", gbs, "GB/s"
+    else:
+        peak = MFMA_PEAK_TFLOPS["f16"]
+        achieved = flops / (kernel_ms * 1e-3) / 1e12
+        roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
+                    "frac": round(achieved / peak, 4), "traffic": None,
+                    "kernel_us": round(kernel_ms * 1e3, 3), "algorithmic_flops": flops}
+        metric, value, unit = f"qGEMM TOPS at M={m} ({dtn} K={k} N={n})", tops, "TFLOP/s"
+
+    cpu = None
+    if not args.no_cpu:
+        cpu = cpu_baseline(pw, a, bias, act, abytes, flops, bandwidth_bound, args.cpu_seconds)
+
+    out = {
+        "metric": metric, "value": round(value, 2), "unit": unit, "n_gpus": 1, "steps": steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 6), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: {dtn} weights [N={n},K={k}] per-channel, f32 activations "
+                               f"[M={m},K={k}] ~N(0,1), bias={has_bias}, act={actn}, seed 0",
+                   "m": m, "k": k, "n": n, "weight_ring": ring, "ring_bytes": ring * wbytes,
+                   "launch": args.mode, "act_rounding": "f16x1" if args.fast_act16 else "default"},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "gb_per_s": round(gbs, 1), "tflop_per_s": round(tops, 3),
+        "event_ms_total": round(ev_ms, 4), "wall_ms_total": round(wall_s * 1e3, 4),
+        "quantize_host_s": round(t_quant, 3), "self_check_max_rel": self_check,
+    }
+    print(json.dumps(out))
+    if graph is not None:
+        ctx.graph_destroy(graph)
+    ctx.close()
+    return 0
+
+
+def cpu_baseline(pw, a, bias, act, abytes, flops, bandwidth_bound, budget_s):
+    """The oracle's restatement of fastnn's CPU algorithm (gemm_batch_packed_simd: scalar
+    unpack per row, AVX2 dot per batch row, single thread below `cores` batch rows), timed on
+    this host on a bounded sample of the same workload."""
+    from oracle import oracle
+    po = oracle.Packed(pw.dtype, pw.rows, pw.inner, pw.words, pw.scales, pw.zeros, pw.qblock, pw.codebook)
+    m = a.shape[0]
+    n = pw.rows
+    # bound the sample: full N at small M, a row slice of the weight at large M
+    rows = n
+    est = 2e-9 * m * pw.inner * n + 4e-9 * pw.inner * n   # rough seconds per call
+    if est > budget_s / 4:
+        rows = max(64, int(n * (budget_s / 4) / est))
+    if rows < n:
+        items = 32 // pw.bit_width
+        kp = -(-pw.inner // items)
+        words = np.concatenate([pw.words[: rows * kp], np.zeros(16, np.uint32)])
+        if pw.dtype == 7:
+            bpr = pw.inner // pw.qblock
+            po = oracle.Packed(pw.dtype, rows, pw.inner, words, pw.scales[: rows * bpr], pw.zeros, pw.qblock, pw.codebook)
+        else:
+            po = oracle.Packed(pw.dtype, rows, pw.inner, words, pw.scales[:rows], pw.zeros[:rows])
+        bias = None if bias is None else bias[:rows]
+    frac = rows / n
+    times = []
+    t_end = time.perf_counter() + budget_s
+    oracle.qmatmul(po, a, order=1, bias=bias, act=act)  # warm-up
+    while time.perf_counter() < t_end and len(times) < 200:
+        t0 = time.perf_counter()
+        oracle.qmatmul(po, a, order=1, bias=bias, act=act)
+        times.append(time.perf_counter() - t0)
+    med = float(np.median(times))
+    if bandwidth_bound:
+        value, unit = abytes * frac / med / 1e9, "GB/s"
+    else:
+        value, unit = flops * frac / med / 1e12, "TFLOP/s"
+    return {"value": round(value, 4), "unit": unit, "cores": 1, "kind": "port",
+            "sample": f"{len(times)} calls of the C restatement of gemm_batch_packed_simd (AVX2 dot order, "
+                      f"-O2, one thread as the reference runs below `cores` batch rows) on {rows}/{n} weight rows, "
+                      f"M={m}; median {med * 1e3:.2f} ms per call; host nproc={os.cpu_count()}"}
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -408,13 +408,18 @@ int fnn_hip_qmatmul(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *a, i
     p.m = m; p.n = n; p.k = k; p.kp = w->kp; p.bpr = w->bpr; p.qblock = w->qblock; p.act = act;
     p.as_written = (flags & FNN_FLAG_I4CB_AS_WRITTEN) ? 1 : 0;
 
+    // kernel choice: matrix-core kernel for every M (bandwidth-bound at small M); the FMA GEMV
+    // serves the codebook type at M <= 4 and any weight when FNN_FLAG_PREFER_FMA asks for it;
+    // the shape-agnostic kernel takes what is left (ragged rows, unaligned pointers).
     bool handled = false;
     if (!(flags & FNN_FLAG_FORCE_GENERIC)) {
-        HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qgemv(w->dtype, p, ctx->stream, &handled));
+        const bool fma_first = (flags & FNN_FLAG_PREFER_FMA) || w->dtype == FNN_DT_I4CB;
+        if (fma_first) HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qgemv(w->dtype, p, ctx->stream, &handled));
         if (!handled) {
             int rc = fnn_mfma_qmatmul(ctx, ctx->stream, w, p, flags, &handled);
             if (rc) return rc;
         }
+        if (!handled && !fma_first) HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qgemv(w->dtype, p, ctx->stream, &handled));
     }
     if (!handled) HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qgemm_generic(w->dtype, p, ctx->stream));
     if (!dev) {

@@ -21,6 +21,7 @@ FLAG_DEVICE_PTRS = 1
 FLAG_I4CB_AS_WRITTEN = 2
 FLAG_ACT_F16_SINGLE = 4
 FLAG_FORCE_GENERIC = 8
+FLAG_PREFER_FMA = 16
 
 STATUS_NAMES = {0: "Ok", 1: "Dispatch", 2: "Memory", 3: "UnsupportedOp", 4: "Compilation"}
 

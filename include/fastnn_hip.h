@@ -59,7 +59,8 @@ enum {
                                       /* src/backend/cpu/matmul.rs:206-212 does (K == N only)     */
     FNN_FLAG_ACT_F16_SINGLE = 1 << 2, /* MFMA path: round activations to f16 once (default keeps  */
                                       /* a second f16 residual term, i.e. ~22 mantissa bits)      */
-    FNN_FLAG_FORCE_GENERIC = 1 << 3   /* take the shape-agnostic kernel (testing aid)             */
+    FNN_FLAG_FORCE_GENERIC = 1 << 3,  /* take the shape-agnostic kernel (testing aid)             */
+    FNN_FLAG_PREFER_FMA = 1 << 4      /* M <= 4: take the f32 FMA GEMV instead of the MFMA kernel */
 };
 
 typedef struct fnn_hip_ctx fnn_hip_ctx;

@@ -109,11 +109,14 @@ def test_grouped_and_scalar_scales(ctx, orc):
 
 # --------------------------------------------------------------------------- f32-activation MatMul
 GEMV_SHAPES = [(1, 256, 64), (1, 1024, 100), (2, 512, 48), (3, 2048, 33), (4, 4096, 128), (1, 8192, 16)]
+# matrix-core shapes: every M-tile count, several K-chunks, ragged N, K not a multiple of the tile
+MFMA_SHAPES = [(5, 512, 64), (16, 4096, 48), (17, 1024, 100), (33, 2048, 40), (64, 8192, 32), (100, 640, 72),
+               (256, 1024, 130), (8, 96, 16), (12, 12288, 24)]
 RAGGED_SHAPES = [(1, 7, 5), (3, 9, 4), (2, 100, 17), (5, 61, 130), (9, 333, 20), (17, 4100, 12), (1, 48, 8)]
 
 
 @pytest.mark.parametrize("dt", ALL_DT)
-@pytest.mark.parametrize("m,k,n", GEMV_SHAPES + RAGGED_SHAPES)
+@pytest.mark.parametrize("m,k,n", GEMV_SHAPES + RAGGED_SHAPES + MFMA_SHAPES)
 def test_qmatmul_matches_oracle(ctx, orc, dt, m, k, n):
     rng = np.random.default_rng(3000 + dt * 17 + k)
     pw = fastnn_amd.quantize_weights(dt, _weights(rng, n, k, "laplace" if dt == 7 else "normal"))
@@ -124,6 +127,8 @@ def test_qmatmul_matches_oracle(ctx, orc, dt, m, k, n):
     assert_close(got, want, TOL_F32, f"{NAMES[dt]} {m}x{k}x{n}")
     gen = ctx.qmatmul(h, a, n, flags=flib.FLAG_FORCE_GENERIC)
     assert_close(gen, want, TOL_F32, f"generic {NAMES[dt]} {m}x{k}x{n}")
+    fma = ctx.qmatmul(h, a, n, flags=flib.FLAG_PREFER_FMA)
+    assert_close(fma, want, TOL_F32, f"fma {NAMES[dt]} {m}x{k}x{n}")
     # the reference's own f32 summation orders sit inside the same band
     assert rel_err(orc.qmatmul(to_oracle(orc, pw), a, order=1), want) <= TOL_F32 * 5
     ctx.release(h)
@@ -336,3 +341,62 @@ def test_error_paths_mirror_reference_messages(ctx):
     assert out.shape == (0, 8)
     ctx.release(h)
     ctx.release(f8)
+
+
+# --------------------------------------------------------------------------- matrix-core specifics
+@pytest.mark.parametrize("dt", [0, 1, 4, 6])
+@pytest.mark.parametrize("mag", [1e-30, 1e-6, 1.0, 3e4, 1e9, 1e30])
+def test_mfma_activation_range_is_f32(ctx, orc, dt, mag):
+    """Activations far outside f16 range: the per-row power-of-two scaling keeps f32 accuracy."""
+    rng = np.random.default_rng(7000 + dt)
+    m, k, n = 6, 2048, 48
+    pw = fastnn_amd.quantize_weights(dt, _weights(rng, n, k))
+    a = (rng.standard_normal((m, k)) * mag).astype(np.float32)
+    a[1] *= 1e-3          # rows of very different magnitude
+    a[2, :100] *= 1e3     # and a wide spread inside one row
+    h = ctx.register(pw)
+    want = orc.qmatmul(to_oracle(orc, pw), a, order=2)
+    got = ctx.qmatmul(h, a, n)
+    for r in range(m):    # row-wise: each row is held to the tolerance on its own scale
+        assert_close(got[r], want[r], TOL_F32, f"row {r} mag {mag}")
+    ctx.release(h)
+
+
+@pytest.mark.parametrize("dt", [0, 1, 4, 6])
+def test_mfma_single_f16_rounding_meets_north_star_tolerance(ctx, orc, dt):
+    """FNN_FLAG_ACT_F16_SINGLE rounds activations to f16 once: stated tolerance 1e-3 of max|ref|."""
+    rng = np.random.default_rng(7100 + dt)
+    m, k, n = 64, 4096, 96
+    pw = fastnn_amd.quantize_weights(dt, _weights(rng, n, k))
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    h = ctx.register(pw)
+    want = orc.qmatmul(to_oracle(orc, pw), a, order=2)
+    got = ctx.qmatmul(h, a, n, flags=flib.FLAG_ACT_F16_SINGLE)
+    assert rel_err(got, want) <= TOL_NORTH_STAR
+    assert_close(ctx.qmatmul(h, a, n), want, TOL_F32)
+    ctx.release(h)
+
+
+@pytest.mark.parametrize("name,dt,k,n,ms", [("c1", 0, 4096, 4096, (1, 32)), ("c2", 1, 4096, 11008, (1, 16, 128, 256)),
+                                           ("c4_f8", 4, 2048, 8192, (64,)), ("c4_f4", 6, 8192, 2048, (64,))])
+def test_full_size_configs_on_row_sample(ctx, orc, name, dt, k, n, ms):
+    """BASELINE shapes at full size; the oracle checks a random sample of output columns
+    (weight rows are independent), plus linearity in the activations as a whole-tensor property."""
+    rng = np.random.default_rng(8000 + dt)
+    w = _weights(rng, n, k) if name in ("c1", "c2") else (rng.standard_normal((n, k)) / np.sqrt(k)).astype(np.float32)
+    pw = fastnn_amd.quantize_weights(dt, w)
+    bias = (rng.standard_normal(n) * 0.01).astype(np.float32)
+    h = ctx.register(pw)
+    rows = np.sort(rng.choice(n, 48, replace=False))
+    sub = to_oracle(orc, slice_rows(pw, rows))
+    for m in ms:
+        a = rng.standard_normal((m, k)).astype(np.float32)
+        got = ctx.qmatmul(h, a, n, bias=bias, act=flib.ACT_SILU)
+        want = orc.qmatmul(sub, a, order=2, bias=bias[rows], act=orc.ACT_SILU)
+        assert_close(got[:, rows], want, TOL_F32, f"{name} M={m}")
+        # linearity without epilogue: f(a1 + a2) == f(a1) + f(a2) up to rounding
+        a2 = rng.standard_normal((m, k)).astype(np.float32)
+        lhs = ctx.qmatmul(h, a + a2, n)
+        rhs = ctx.qmatmul(h, a, n).astype(np.float64) + ctx.qmatmul(h, a2, n).astype(np.float64)
+        assert rel_err(lhs, rhs) <= 1e-5
+    ctx.release(h)
