@@ -416,6 +416,10 @@ int fnn_hip_qmatmul(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *a, i
         const bool fma_first = (flags & FNN_FLAG_PREFER_FMA) || w->dtype == FNN_DT_I4CB;
         if (fma_first) HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qgemv(w->dtype, p, ctx->stream, &handled));
         if (!handled) {
+            int rc = fnn_mfma_qgemv(ctx, ctx->stream, w, p, flags, &handled);
+            if (rc) return rc;
+        }
+        if (!handled) {
             int rc = fnn_mfma_qmatmul(ctx, ctx->stream, w, p, flags, &handled);
             if (rc) return rc;
         }

@@ -84,12 +84,22 @@ __device__ __forceinline__ int wave_sum_i32(int v)
 }
 __device__ __forceinline__ float wave_min(float v)
 {
-    for (int o = 1; o < 64; o <<= 1) v = fminf(v, __shfl_xor(v, o, 64));
+    v = fminf(v, dpp_f32<0xB1>(v));
+    v = fminf(v, dpp_f32<0x4E>(v));
+    v = fminf(v, dpp_f32<0x141>(v));
+    v = fminf(v, dpp_f32<0x140>(v));
+    v = fminf(v, __shfl_xor(v, 16, 64));
+    v = fminf(v, __shfl_xor(v, 32, 64));
     return v;
 }
 __device__ __forceinline__ float wave_max(float v)
 {
-    for (int o = 1; o < 64; o <<= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    v = fmaxf(v, dpp_f32<0xB1>(v));
+    v = fmaxf(v, dpp_f32<0x4E>(v));
+    v = fmaxf(v, dpp_f32<0x141>(v));
+    v = fmaxf(v, dpp_f32<0x140>(v));
+    v = fmaxf(v, __shfl_xor(v, 16, 64));
+    v = fmaxf(v, __shfl_xor(v, 32, 64));
     return v;
 }
 

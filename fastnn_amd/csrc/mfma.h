@@ -11,6 +11,9 @@ int fnn_ctx_fail(fnn_hip_ctx *ctx, int code, const char *msg);
 // is left to the generic kernel.
 int fnn_mfma_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &p,
                      int flags, bool *handled);
+// M <= 4: bandwidth-bound GEMV on the matrix cores (weights requested before anything else).
+int fnn_mfma_qgemv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &p,
+                   int flags, bool *handled);
 // I8 activations x I8/I4 weights on int8 MFMA tiles with i32 accumulators.
 int fnn_mfma_qmatmul_i8act(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w,
                            const I8ActArgs &p, bool *handled);

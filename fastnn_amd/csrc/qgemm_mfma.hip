@@ -16,127 +16,13 @@
 // reduced through LDS in a fixed order and the affine/bias/activation epilogue is fused.
 // Up to M = 16*MTL activation rows per launch; bandwidth-bound while M is small.
 #include "mfma.h"
+#include "dech.h"
 
 #include <cstdlib>
 
 namespace {
 
-__device__ __forceinline__ f16x2 as_h2(uint32_t u) { return __builtin_bit_cast(f16x2, u); }
-__device__ __forceinline__ uint32_t as_u(f16x2 h) { return __builtin_bit_cast(uint32_t, h); }
-__device__ __forceinline__ f16x2 h2(float v) { return f16x2{(_Float16)v, (_Float16)v}; }
-
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ f16x8 pack8(uint32_t a, uint32_t b, uint32_t c, uint32_t d)
-{
-    return __builtin_bit_cast(f16x8, u32x4{a, b, c, d});
-}
-
-// Decoders: one MFMA step = 8 k-values of one weight row as f16x8.  `w` points at the
-// lane's packed words for the step (1 word for 4-bit types, 2 for 8-bit types).
-// PERM tells in which order the 8 k-values land in the operand (the activation fragments
-// are stored in LDS in the same order).
-template <int DT>
-struct DecH;
-
-// 1024 + v is exact in f16 for 0 <= v < 1024: OR-ing a small integer into the mantissa of
-// 0x6400 builds it without a convert; 1024 + 16 v likewise for the upper nibble of a byte.
-template <>
-struct DecH<FNN_DT_I4> {
-    static constexpr int WPS = 1;
-    static constexpr bool INTERLEAVED = true;  // operand order k = 0,4,1,5,2,6,3,7
-    __device__ static __forceinline__ f16x8 step(const uint32_t *w)
-    {
-        const uint32_t u = w[0] ^ 0x88888888u;  // nibble q -> q + 8
-        const uint32_t v = u >> 8;
-        f16x2 r0 = as_h2((u & 0x000F000Fu) | 0x64006400u) + h2(-1032.0f);
-        f16x2 r1 = __builtin_elementwise_fma(as_h2((u & 0x00F000F0u) | 0x64006400u), h2(0.0625f), h2(-72.0f));
-        f16x2 r2 = as_h2((v & 0x000F000Fu) | 0x64006400u) + h2(-1032.0f);
-        f16x2 r3 = __builtin_elementwise_fma(as_h2((v & 0x00F000F0u) | 0x64006400u), h2(0.0625f), h2(-72.0f));
-        return pack8(as_u(r0), as_u(r1), as_u(r2), as_u(r3));
-    }
-};
-template <>
-struct DecH<FNN_DT_U4> {
-    static constexpr int WPS = 1;
-    static constexpr bool INTERLEAVED = true;
-    __device__ static __forceinline__ f16x8 step(const uint32_t *w)
-    {
-        const uint32_t u = w[0];
-        const uint32_t v = u >> 8;
-        f16x2 r0 = as_h2((u & 0x000F000Fu) | 0x64006400u) + h2(-1024.0f);
-        f16x2 r1 = __builtin_elementwise_fma(as_h2((u & 0x00F000F0u) | 0x64006400u), h2(0.0625f), h2(-64.0f));
-        f16x2 r2 = as_h2((v & 0x000F000Fu) | 0x64006400u) + h2(-1024.0f);
-        f16x2 r3 = __builtin_elementwise_fma(as_h2((v & 0x00F000F0u) | 0x64006400u), h2(0.0625f), h2(-64.0f));
-        return pack8(as_u(r0), as_u(r1), as_u(r2), as_u(r3));
-    }
-};
-template <>
-struct DecH<FNN_DT_I8> {
-    static constexpr int WPS = 2;
-    static constexpr bool INTERLEAVED = false;
-    __device__ static __forceinline__ f16x8 step(const uint32_t *w)
-    {
-        const uint32_t u0 = w[0] ^ 0x80808080u, u1 = w[1] ^ 0x80808080u;  // byte q -> q + 128
-        f16x2 r0 = as_h2(__builtin_amdgcn_perm(0x64646464u, u0, 0x04010400u)) + h2(-1152.0f);
-        f16x2 r1 = as_h2(__builtin_amdgcn_perm(0x64646464u, u0, 0x04030402u)) + h2(-1152.0f);
-        f16x2 r2 = as_h2(__builtin_amdgcn_perm(0x64646464u, u1, 0x04010400u)) + h2(-1152.0f);
-        f16x2 r3 = as_h2(__builtin_amdgcn_perm(0x64646464u, u1, 0x04030402u)) + h2(-1152.0f);
-        return pack8(as_u(r0), as_u(r1), as_u(r2), as_u(r3));
-    }
-};
-template <>
-struct DecH<FNN_DT_U8> {
-    static constexpr int WPS = 2;
-    static constexpr bool INTERLEAVED = false;
-    __device__ static __forceinline__ f16x8 step(const uint32_t *w)
-    {
-        f16x2 r0 = as_h2(__builtin_amdgcn_perm(0x64646464u, w[0], 0x04010400u)) + h2(-1024.0f);
-        f16x2 r1 = as_h2(__builtin_amdgcn_perm(0x64646464u, w[0], 0x04030402u)) + h2(-1024.0f);
-        f16x2 r2 = as_h2(__builtin_amdgcn_perm(0x64646464u, w[1], 0x04010400u)) + h2(-1024.0f);
-        f16x2 r3 = as_h2(__builtin_amdgcn_perm(0x64646464u, w[1], 0x04030402u)) + h2(-1024.0f);
-        return pack8(as_u(r0), as_u(r1), as_u(r2), as_u(r3));
-    }
-};
-template <>
-struct DecH<FNN_DT_F8> {
-    static constexpr int WPS = 2;
-    static constexpr bool INTERLEAVED = false;
-    __device__ static __forceinline__ f16x8 step(const uint32_t *w)
-    {
-        f16x2 r0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w[0], 1.0f, false);
-        f16x2 r1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w[0], 1.0f, true);
-        f16x2 r2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w[1], 1.0f, false);
-        f16x2 r3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w[1], 1.0f, true);
-        return pack8(as_u(r0), as_u(r1), as_u(r2), as_u(r3));
-    }
-};
-template <>
-struct DecH<FNN_DT_F8R> {
-    static constexpr int WPS = 2;
-    static constexpr bool INTERLEAVED = false;
-    // an E5M2 byte is the upper byte of the f16 with the same value (incl. inf/NaN)
-    __device__ static __forceinline__ f16x8 step(const uint32_t *w)
-    {
-        uint32_t r0 = __builtin_amdgcn_perm(0u, w[0], 0x010C000Cu);
-        uint32_t r1 = __builtin_amdgcn_perm(0u, w[0], 0x030C020Cu);
-        uint32_t r2 = __builtin_amdgcn_perm(0u, w[1], 0x010C000Cu);
-        uint32_t r3 = __builtin_amdgcn_perm(0u, w[1], 0x030C020Cu);
-        return pack8(r0, r1, r2, r3);
-    }
-};
-template <>
-struct DecH<FNN_DT_F4> {
-    static constexpr int WPS = 1;
-    static constexpr bool INTERLEAVED = false;
-    __device__ static __forceinline__ f16x8 step(const uint32_t *w)
-    {
-        f16x2 r0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w[0], 1.0f, 0);
-        f16x2 r1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w[0], 1.0f, 1);
-        f16x2 r2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w[0], 1.0f, 2);
-        f16x2 r3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w[0], 1.0f, 3);
-        return pack8(as_u(r0), as_u(r1), as_u(r2), as_u(r3));
-    }
-};
+using namespace dech;
 
 struct MfmaArgs {
     const uint32_t *words;
