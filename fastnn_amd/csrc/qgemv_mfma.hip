@@ -11,13 +11,17 @@
 //
 // One workgroup = RT*16 weight rows x all of K, 8 waves.  Wave w owns the K slice
 // [w*512, (w+1)*512) of every round of 4096 k-values:
-//   1. it requests all of its packed bytes first (lane (n,g): row n, 16 bytes per tile);
-//   2. while they are in flight it converts its own slice of the activations: one group of
-//      8 floats per lane and row, scaled by a power of two taken from the slice maximum,
-//      split into hi + lo f16 and written to the wave's LDS area in operand order;
-//   3. MFMA steps, scale the slice partial back in f32;
-//   4. partial 16x16 tiles and activation sums of the 8 waves are added in a fixed order
-//      through LDS and the affine / bias / activation epilogue is applied.
+//   0. it requests its slice of the activations, then
+//   1. all of its packed bytes (lane (n,g): row n, 16 bytes per tile);
+//   2. while they are in flight it converts the activations: one group of 8 floats per lane
+//      and row, scaled by a power of two taken from the slice maximum and split into hi + lo
+//      f16 terms.  hi and lo occupy DIFFERENT ROWS of the 16-row MFMA operand (rows 0..M-1
+//      and M..2M-1), so one MFMA per step yields both partial products;
+//   3. MFMA steps; the slice partial is scaled back in f32;
+//   4. partial tiles and activation sums of the 8 waves are added in a fixed order through
+//      LDS (hi row + lo row), and the affine / bias / activation epilogue is applied.
+// Operand rows >= 2M are never read back, so their lanes load a clamped (valid) row
+// instead of zeros and no lane masking is needed in the inner loop.
 // Algorithmic bytes per launch: N*K*bits/8 + side tables + 4*M*(K+N).
 #include "dech.h"
 #include "mfma.h"
@@ -33,15 +37,15 @@ struct GemvArgs {
     const float *scales, *zeros, *a, *bias;
     float *out;
     int64_t m, n, k, kp;
-    int act, single;
+    int act;
 };
 
 constexpr int GV_NW = 8;        // waves per workgroup
 constexpr int GV_SLICE = 512;   // k-values per wave and round (64 groups of 8: one per lane)
 constexpr int GV_MMAX = 4;
 
-template <int DT, int RT, int MM>
-__global__ void __launch_bounds__(GV_NW * 64) qgemv_mfma_kernel(GemvArgs p)
+template <int DT, int RT, int MM, bool SINGLE, int NW>
+__global__ void __launch_bounds__(NW * 64) qgemv_mfma_kernel(GemvArgs p)
 {
     using D = DecH<DT>;
     constexpr int WPS = D::WPS;
@@ -49,24 +53,23 @@ __global__ void __launch_bounds__(GV_NW * 64) qgemv_mfma_kernel(GemvArgs p)
     constexpr int KT = 4 * SPT * 8;         // k-values per tile (128 / 64)
     constexpr int TPW = GV_SLICE / KT;      // tiles per wave and round (4 / 8)
     constexpr int NSTEP = TPW * SPT;        // MFMA steps per wave and round (16)
+    constexpr int ROWS = SINGLE ? MM : 2 * MM;  // operand rows in use: hi rows, then lo rows
 
-    // dynamic LDS: per wave [NSTEP][M][4 g] 16-byte fragments (hi plane, then lo plane)
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    const int frag_per_wave = NSTEP * MM * 4;
-    uint4 *a_hi_w = reinterpret_cast<uint4 *>(smem) + (size_t)(threadIdx.x >> 6) * frag_per_wave;
-    uint4 *a_lo_w = a_hi_w + (size_t)GV_NW * frag_per_wave;
-    __shared__ float red[GV_NW][RT][64];
+    // per wave: [NSTEP][ROWS][4 g] 16-byte operand fragments
+    extern __shared__ __attribute__((aligned(16))) uint4 frag_dyn[];  // GV_NW * NSTEP * ROWS * 4
+    __shared__ float red[GV_NW][RT][8][16];
     __shared__ float xred[GV_NW][GV_MMAX];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wv = tid >> 6;
+    constexpr int nw = NW;                  // waves in this workgroup (compile time: 8, or 4 for K <= 2048)
     const int ln = lane & 15;
     const int g = lane >> 4;
     const int64_t K = p.k, N = p.n, kp = p.kp;
-    constexpr int M = MM;  // activation rows of this instantiation (1, 2 or 4; p.m <= MM)
-    const int mreal = (int)p.m;
+    const int mreal = (int)p.m;             // <= MM
     const int64_t n0 = (int64_t)blockIdx.x * (RT * 16);
+    uint4 *fw = frag_dyn + wv * (NSTEP * ROWS * 4);
 
     const uint32_t *wrow[RT];
 #pragma unroll
@@ -76,30 +79,47 @@ __global__ void __launch_bounds__(GV_NW * 64) qgemv_mfma_kernel(GemvArgs p)
         wrow[r] = p.words + row * kp;
     }
 
+    // epilogue operands of the output this thread will finish (idx = tid): requested now,
+    // used after the last barrier, so their latency is off the critical path
+    const int e_r = (tid / (MM * 16)) % RT, e_m = (tid % (MM * 16)) >> 4, e_c = tid & 15;
+    int64_t e_n = n0 + e_r * 16 + e_c;
+    const bool e_ok = tid < RT * MM * 16 && e_m < mreal && e_n < N;
+    if (e_n > N - 1) e_n = N - 1;
+    const float e_scale = p.scales[e_n], e_zero = p.zeros[e_n];
+    const float e_bias = p.bias ? p.bias[e_n] : 0.0f;
+
     f32x4 tot[RT];
 #pragma unroll
     for (int r = 0; r < RT; r++) tot[r] = f32x4{0.f, 0.f, 0.f, 0.f};
-    float xsum[GV_MMAX] = {0.f, 0.f, 0.f, 0.f};
+    float xsum[MM];
+#pragma unroll
+    for (int m = 0; m < MM; m++) xsum[m] = 0.0f;
 
-    const int64_t round_k = (int64_t)GV_NW * GV_SLICE;
+    // operand fragment this lane reads at step s: row min(ln, ROWS-1), group g
+    const int rsel = ln < ROWS ? ln : ROWS - 1;
+    const uint4 *frd = fw + rsel * 4 + g;
+
+    const int64_t round_k = (int64_t)nw * GV_SLICE;
     for (int64_t k0 = 0; k0 < K; k0 += round_k) {
         const int64_t ks = k0 + (int64_t)wv * GV_SLICE;  // first k of this wave's slice
-        // ---- 0. this lane's group of 8 activations per row: requested ahead of the weight
-        //         stream so that it does not queue behind it
+        // ---- 0. this lane's group of 8 activations per row, ahead of the weight stream
         const int64_t kk = ks + (int64_t)lane * 8;
+        // (loads go to clamped, always valid addresses and are masked afterwards: no branch sits
+        //  between a load and the next one, so all of them are in flight together)
         float xr[MM][8];
+        const int64_t kkc = kk < K ? kk : K - 8;  // K % 8 == 0
 #pragma unroll
         for (int m = 0; m < MM; m++) {
-#pragma unroll
-            for (int j = 0; j < 8; j++) xr[m][j] = 0.0f;
-            if (m < mreal && kk < K) {  // K % 8 == 0
-                const float4 x0 = *reinterpret_cast<const float4 *>(p.a + (int64_t)m * K + kk);
-                const float4 x1 = *reinterpret_cast<const float4 *>(p.a + (int64_t)m * K + kk + 4);
-                xr[m][0] = x0.x; xr[m][1] = x0.y; xr[m][2] = x0.z; xr[m][3] = x0.w;
-                xr[m][4] = x1.x; xr[m][5] = x1.y; xr[m][6] = x1.z; xr[m][7] = x1.w;
-            }
+            const int64_t mrow = m < mreal ? m : mreal - 1;
+            const uint32_t keep = (m < mreal && kk < K) ? 0xffffffffu : 0u;
+            const uint4 x0 = *reinterpret_cast<const uint4 *>(p.a + mrow * K + kkc);
+            const uint4 x1 = *reinterpret_cast<const uint4 *>(p.a + mrow * K + kkc + 4);
+            xr[m][0] = __uint_as_float(x0.x & keep); xr[m][1] = __uint_as_float(x0.y & keep);
+            xr[m][2] = __uint_as_float(x0.z & keep); xr[m][3] = __uint_as_float(x0.w & keep);
+            xr[m][4] = __uint_as_float(x1.x & keep); xr[m][5] = __uint_as_float(x1.y & keep);
+            xr[m][6] = __uint_as_float(x1.z & keep); xr[m][7] = __uint_as_float(x1.w & keep);
         }
-        // ---- 1. request the packed bytes: tile t, lane (n,g): words [ (ks + t*KT)/EPW + g*4, +4 )
+        // ---- 1. the packed bytes: tile t, lane (n,g): words [slice + t*16 + g*4, +4) of row n
         uint32_t wq[RT][TPW * 4];
         const int64_t wbase = ks * 4 / (8 * SPT);         // word offset of the slice (ks * bits / 32)
 #pragma unroll
@@ -107,26 +127,28 @@ __global__ void __launch_bounds__(GV_NW * 64) qgemv_mfma_kernel(GemvArgs p)
 #pragma unroll
             for (int t = 0; t < TPW; t++) {
                 const int64_t woff = wbase + t * 16 + g * 4;
-                uint4 v = make_uint4(0, 0, 0, 0);
-                if (woff + 4 <= kp) v = *reinterpret_cast<const uint4 *>(wrow[r] + woff);
-                wq[r][t * 4 + 0] = v.x; wq[r][t * 4 + 1] = v.y; wq[r][t * 4 + 2] = v.z; wq[r][t * 4 + 3] = v.w;
+                const bool ok = woff + 4 <= kp;           // kp % 4 == 0, kp >= 4
+                const uint32_t keep = ok ? 0xffffffffu : 0u;
+                const uint4 v = *reinterpret_cast<const uint4 *>(wrow[r] + (ok ? woff : kp - 4));
+                wq[r][t * 4 + 0] = v.x & keep; wq[r][t * 4 + 1] = v.y & keep;
+                wq[r][t * 4 + 2] = v.z & keep; wq[r][t * 4 + 3] = v.w & keep;
             }
 
-        // ---- 2. this wave's activation slice -> f16 hi/lo fragments in its LDS area
-        float csc[GV_MMAX] = {1.f, 1.f, 1.f, 1.f};
+        // ---- 2. activation slice -> f16 hi/lo operand rows in this wave's LDS area
+        float csc[MM];
         {
-            // group -> (tile, g, step) and fragment slot (step*M + m)*4 + g
+            // this lane's group -> (tile, g, step); fragment slot (step*ROWS + row)*4 + g
             const int kl = lane * 8;
             const int t = kl / KT, rr = kl % KT;
             const int gg = rr / (SPT * 8), st = (rr % (SPT * 8)) / 8;
+            const int slot = (t * SPT + st) * ROWS * 4 + gg;
 #pragma unroll
             for (int m = 0; m < MM; m++) {
                 const float *x = xr[m];
                 float mx = fmaxf(fmaxf(fmaxf(fabsf(x[0]), fabsf(x[1])), fmaxf(fabsf(x[2]), fabsf(x[3]))),
                                  fmaxf(fmaxf(fabsf(x[4]), fabsf(x[5])), fmaxf(fabsf(x[6]), fabsf(x[7]))));
                 mx = wave_max(mx);
-                const float s = wave_sum(((x[0] + x[1]) + (x[2] + x[3])) + ((x[4] + x[5]) + (x[6] + x[7])));
-                xsum[m] += s;
+                xsum[m] += wave_sum(((x[0] + x[1]) + (x[2] + x[3])) + ((x[4] + x[5]) + (x[6] + x[7])));
                 // power of two e with max*2^-e in [2^14, 2^15), clamped so that 2^-e is finite
                 int ex = (int)((__float_as_uint(mx) >> 23) & 0xff) - 127 - 14;
                 if (mx == 0.0f) ex = 0;
@@ -141,90 +163,92 @@ __global__ void __launch_bounds__(GV_NW * 64) qgemv_mfma_kernel(GemvArgs p)
                     hi[j] = (_Float16)v;
                     lo[j] = (_Float16)(v - (float)hi[j]);
                 }
-                const int dst = ((t * SPT + st) * M + m) * 4 + gg;
-                a_hi_w[dst] = __builtin_bit_cast(uint4, f16x8{hi[0], hi[1], hi[2], hi[3], hi[4], hi[5], hi[6], hi[7]});
-                if (!p.single)
-                    a_lo_w[dst] = __builtin_bit_cast(uint4, f16x8{lo[0], lo[1], lo[2], lo[3], lo[4], lo[5], lo[6], lo[7]});
+                fw[slot + m * 4] = __builtin_bit_cast(uint4, f16x8{hi[0], hi[1], hi[2], hi[3], hi[4], hi[5], hi[6], hi[7]});
+                if (!SINGLE)
+                    fw[slot + (MM + m) * 4] =
+                        __builtin_bit_cast(uint4, f16x8{lo[0], lo[1], lo[2], lo[3], lo[4], lo[5], lo[6], lo[7]});
             }
         }
         __syncthreads();
 
-        // ---- 3. MFMA over the slice
-        f32x4 acc[RT], acl[RT];  // hi and lo terms keep separate dependency chains
+        // ---- 3. MFMA over the slice: straight-line, one MFMA per step and row tile
+        f32x4 acc[RT];
 #pragma unroll
-        for (int r = 0; r < RT; r++) acc[r] = acl[r] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int r = 0; r < RT; r++) acc[r] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int t = 0; t < TPW; t++)
+        for (int s = 0; s < NSTEP; s++) {
+            const f16x8 av = __builtin_bit_cast(f16x8, frd[s * ROWS * 4]);
 #pragma unroll
-            for (int st = 0; st < SPT; st++) {
-                uint4 vh = make_uint4(0, 0, 0, 0), vl = make_uint4(0, 0, 0, 0);
-                if (ln < M) {
-                    const int src = ((t * SPT + st) * M + ln) * 4 + g;
-                    vh = a_hi_w[src];
-                    if (!p.single) vl = a_lo_w[src];
-                }
-                const f16x8 ah = __builtin_bit_cast(f16x8, vh);
-                const f16x8 al = __builtin_bit_cast(f16x8, vl);
-#pragma unroll
-                for (int r = 0; r < RT; r++) {
-                    const f16x8 b = D::step(&wq[r][t * 4 + st * WPS]);
-                    acc[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah, b, acc[r], 0, 0, 0);
-                    if (!p.single) acl[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(al, b, acl[r], 0, 0, 0);
-                }
+            for (int r = 0; r < RT; r++) {
+                const f16x8 b = D::step(&wq[r][s * WPS]);   // tile t = s / SPT, step s % SPT
+                acc[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, b, acc[r], 0, 0, 0);
             }
-        // acc[i] is activation row g*4 + i: only g == 0 carries rows < 4
+        }
+        // acc[i] is operand row g*4 + i, i.e. activation row (g*4 + i) % MM (hi or lo part)
 #pragma unroll
         for (int r = 0; r < RT; r++)
 #pragma unroll
-            for (int i = 0; i < 4; i++) tot[r][i] = fmaf(acc[r][i] + acl[r][i], csc[i], tot[r][i]);
+            for (int i = 0; i < 4; i++) tot[r][i] = fmaf(acc[r][i], csc[i % MM], tot[r][i]);
         __syncthreads();  // the wave areas are rewritten by the next round
     }
 
-    // ---- 4. fixed-order reduction over the waves, fused epilogue
-    if (g == 0) {
+    // ---- 4. fixed-order reduction over the waves (hi row + lo row), fused epilogue
+    if (g < 2) {
 #pragma unroll
         for (int r = 0; r < RT; r++)
 #pragma unroll
-            for (int i = 0; i < 4; i++) red[wv][r][i * 16 + ln] = tot[r][i];
+            for (int i = 0; i < 4; i++) red[wv][r][g * 4 + i][ln] = tot[r][i];
     }
     if (lane == 0) {
 #pragma unroll
-        for (int m = 0; m < GV_MMAX; m++) xred[wv][m] = xsum[m];
+        for (int m = 0; m < GV_MMAX; m++) xred[wv][m] = m < MM ? xsum[m < MM ? m : 0] : 0.0f;
     }
     __syncthreads();
-    for (int idx = tid; idx < RT * 64; idx += GV_NW * 64) {
-        const int r = idx >> 6, e = idx & 63;
-        const int m = e >> 4;
-        const int64_t n = n0 + r * 16 + (e & 15);
-        if (m >= mreal || n >= N) continue;
+    if (e_ok) {  // RT*MM*16 <= 128 outputs: one per thread
         float dot = 0.0f, xs = 0.0f;
 #pragma unroll
-        for (int w = 0; w < GV_NW; w++) {
-            dot += red[w][r][e];
-            xs += xred[w][m];
+        for (int w = 0; w < GV_NW; w++) {   // all reads issued together; absent waves add 0
+            const int ws = w < nw ? w : 0;
+            float v = red[ws][e_r][e_m][e_c];
+            if (!SINGLE) v += red[ws][e_r][MM + e_m][e_c];
+            dot += w < nw ? v : 0.0f;
+            xs += w < nw ? xred[ws][e_m] : 0.0f;
         }
-        p.out[(int64_t)m * N + n] = fnn_epilogue(dot, p.scales[n], p.zeros[n], xs, p.bias, n, p.act);
+        const float v = dot * e_scale + e_zero * xs + e_bias;   // fnn_epilogue with preloaded operands
+        p.out[(int64_t)e_m * N + e_n] = fnn_activation(p.bias ? v : dot * e_scale + e_zero * xs, p.act);
+    }
+}
+
+template <int DT, bool SINGLE, int NW>
+void launch_mm(const GemvArgs &p, hipStream_t s)
+{
+    constexpr int RT = 1;
+    const dim3 grid((unsigned)((p.n + RT * 16 - 1) / (RT * 16))), blk(NW * 64);
+    // operand fragments: waves x 16 steps x rows x 4 groups x 16 bytes
+    const int mm = p.m <= 1 ? 1 : (p.m <= 2 ? 2 : 4);
+    const size_t lds = (size_t)NW * 16 * (SINGLE ? mm : 2 * mm) * 4 * 16;
+    if (mm == 1) hipLaunchKernelGGL((qgemv_mfma_kernel<DT, RT, 1, SINGLE, NW>), grid, blk, lds, s, p);
+    else if (mm == 2) hipLaunchKernelGGL((qgemv_mfma_kernel<DT, RT, 2, SINGLE, NW>), grid, blk, lds, s, p);
+    else {
+        auto kern = qgemv_mfma_kernel<DT, RT, 4, SINGLE, NW>;
+        static bool attr_set = false;   // up to 64 KiB of dynamic LDS plus the static reduction buffers
+        if (!attr_set) {
+            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+            attr_set = true;
+        }
+        hipLaunchKernelGGL(kern, grid, blk, lds, s, p);
     }
 }
 
 template <int DT>
-hipError_t launch_gemv(const GemvArgs &p, hipStream_t s)
+hipError_t launch_gemv(const GemvArgs &p, bool single, hipStream_t s)
 {
-    static const int env_rt = []() { const char *e = getenv("FNN_GEMV_MFMA_RT"); return (e && *e) ? atoi(e) : 0; }();
-    int rt = (p.n >= 16384) ? 2 : 1;
-    if (env_rt > 0) rt = env_rt;
-    // hi (+ lo) fragment planes: 8 waves x 16 steps x M rows x 4 groups x 16 bytes
-    const int mm = p.m <= 1 ? 1 : (p.m <= 2 ? 2 : 4);
-    const size_t lds = (size_t)GV_NW * 16 * (size_t)mm * 4 * 16 * (p.single ? 1 : 2);
-    const dim3 g1((unsigned)((p.n + 15) / 16)), g2((unsigned)((p.n + 31) / 32)), blk(GV_NW * 64);
-    if (rt == 2) {
-        if (mm == 1) hipLaunchKernelGGL((qgemv_mfma_kernel<DT, 2, 1>), g2, blk, lds, s, p);
-        else if (mm == 2) hipLaunchKernelGGL((qgemv_mfma_kernel<DT, 2, 2>), g2, blk, lds, s, p);
-        else hipLaunchKernelGGL((qgemv_mfma_kernel<DT, 2, 4>), g2, blk, lds, s, p);
+    // 8 waves split K in slices of 512; short K (<= 2048) runs 4-wave workgroups so that no wave idles
+    if (p.k <= 4 * GV_SLICE) {
+        if (single) launch_mm<DT, true, 4>(p, s); else launch_mm<DT, false, 4>(p, s);
     } else {
-        if (mm == 1) hipLaunchKernelGGL((qgemv_mfma_kernel<DT, 1, 1>), g1, blk, lds, s, p);
-        else if (mm == 2) hipLaunchKernelGGL((qgemv_mfma_kernel<DT, 1, 2>), g1, blk, lds, s, p);
-        else hipLaunchKernelGGL((qgemv_mfma_kernel<DT, 1, 4>), g1, blk, lds, s, p);
+        if (single) launch_mm<DT, true, 8>(p, s); else launch_mm<DT, false, 8>(p, s);
     }
     return hipGetLastError();
 }
@@ -241,16 +265,16 @@ int fnn_mfma_qgemv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, con
     GemvArgs p;
     p.words = q.words; p.scales = q.scales; p.zeros = q.zeros; p.a = q.a; p.bias = q.bias; p.out = q.out;
     p.m = q.m; p.n = q.n; p.k = q.k; p.kp = q.kp; p.act = q.act;
-    p.single = (flags & FNN_FLAG_ACT_F16_SINGLE) ? 1 : 0;
+    const bool single = (flags & FNN_FLAG_ACT_F16_SINGLE) != 0;
     hipError_t e;
     switch (w->dtype) {
-    case FNN_DT_I8: e = launch_gemv<FNN_DT_I8>(p, s); break;
-    case FNN_DT_I4: e = launch_gemv<FNN_DT_I4>(p, s); break;
-    case FNN_DT_U8: e = launch_gemv<FNN_DT_U8>(p, s); break;
-    case FNN_DT_U4: e = launch_gemv<FNN_DT_U4>(p, s); break;
-    case FNN_DT_F8: e = launch_gemv<FNN_DT_F8>(p, s); break;
-    case FNN_DT_F8R: e = launch_gemv<FNN_DT_F8R>(p, s); break;
-    case FNN_DT_F4: e = launch_gemv<FNN_DT_F4>(p, s); break;
+    case FNN_DT_I8: e = launch_gemv<FNN_DT_I8>(p, single, s); break;
+    case FNN_DT_I4: e = launch_gemv<FNN_DT_I4>(p, single, s); break;
+    case FNN_DT_U8: e = launch_gemv<FNN_DT_U8>(p, single, s); break;
+    case FNN_DT_U4: e = launch_gemv<FNN_DT_U4>(p, single, s); break;
+    case FNN_DT_F8: e = launch_gemv<FNN_DT_F8>(p, single, s); break;
+    case FNN_DT_F8R: e = launch_gemv<FNN_DT_F8R>(p, single, s); break;
+    case FNN_DT_F4: e = launch_gemv<FNN_DT_F4>(p, single, s); break;
     default: return FNN_OK;
     }
     if (e != hipSuccess) return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, hipGetErrorString(e));
