@@ -78,6 +78,11 @@ def main() -> int:
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--fast-act16", action="store_true", help="single f16 rounding of activations on the MFMA path")
+    ap.add_argument("--probe", default="", choices=["", "read", "copy"],
+                    help="instead of the MatMul, time a plain streaming read / copy of the same number of bytes "
+                         "per launch over the same ring (device ceiling; calibration kernel for byte counters)")
+    ap.add_argument("--traffic-json", default="", help="JSON file {\"fetch_bytes\": .., \"write_bytes\": ..} with "
+                    "counter-derived HBM bytes per launch (see profiles/); copied into roofline.traffic")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path shards over N without changing the "
@@ -127,8 +132,17 @@ def main() -> int:
     dbias = ctx.to_device(bias) if has_bias else None
     dout = ctx.alloc(m * n * 4)
 
+    probe_src, probe_dst = [], None
+    if args.probe:
+        # same launch count, same ring size, same bytes per launch as the MatMul's packed weights
+        probe_src = [ctx.alloc(wbytes).ptr for _ in range(ring)]
+        probe_dst = ctx.alloc(wbytes).ptr if args.probe == "copy" else 0
+
     def step(i: int):
-        ctx.qmatmul_dev(handles[i % ring], da.ptr, m, dout.ptr, dbias.ptr if dbias else 0, act, flags)
+        if args.probe:
+            ctx.probe_stream(probe_src[i % ring], probe_dst, wbytes)
+        else:
+            ctx.qmatmul_dev(handles[i % ring], da.ptr, m, dout.ptr, dbias.ptr if dbias else 0, act, flags)
 
     # untimed warmup (also sizes internal workspaces before any capture)
     for i in range(args.warmup):
@@ -174,6 +188,10 @@ def main() -> int:
     chk = ctx.qmatmul(handles[(steps - 1) % ring], a, n, bias=bias, act=act,
                       flags=flags | flib.FLAG_FORCE_GENERIC)
     self_check = float(np.abs(got - chk).max() / (np.abs(chk).max() + 1e-30))
+    if args.probe:
+        self_check = None
+        abytes = wbytes * (2 if args.probe == "copy" else 1)
+        gbs = abytes / (ms_per_step * 1e-3) / 1e9
 
     bandwidth_bound = m <= 32
     if bandwidth_bound:
@@ -182,6 +200,8 @@ def main() -> int:
                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
                     "kernel_us": round(kernel_ms * 1e3, 3), "algorithmic_bytes": abytes}
         metric, value, unit = f"qGEMM GB/s at M={m} ({dtn} K={k} N={n})", gbs, "GB/s"
+        if args.probe:
+            metric = f"plain {args.probe} of {wbytes} bytes per launch"
     else:
         peak = MFMA_PEAK_TFLOPS["f16"]
         achieved = flops / (kernel_ms * 1e-3) / 1e12
@@ -189,6 +209,29 @@ def main() -> int:
                     "frac": round(achieved / peak, 4), "traffic": None,
                     "kernel_us": round(kernel_ms * 1e3, 3), "algorithmic_flops": flops}
         metric, value, unit = f"qGEMM TOPS at M={m} ({dtn} K={k} N={n})", tops, "TFLOP/s"
+
+    # device ceiling for one launch of this size: a plain streaming read of the packed bytes
+    # over the same ring of buffers, timed the same way
+    src_ptrs = probe_src if probe_src else [ctx.alloc(wbytes).ptr for _ in range(ring)]
+    for ptr in src_ptrs:
+        ctx.probe_stream(ptr, 0, wbytes)
+    ctx.sync()
+    nprobe = max(len(src_ptrs) * 4, 64)
+    ctx.timer_start()
+    for i in range(nprobe):
+        ctx.probe_stream(src_ptrs[i % len(src_ptrs)], 0, wbytes)
+    probe_ms = ctx.timer_stop() / nprobe
+    stream_read_gbs = wbytes / (probe_ms * 1e-3) / 1e9
+    roofline["device_stream_read"] = {"gb_per_s": round(stream_read_gbs, 1), "us": round(probe_ms * 1e3, 3),
+                                      "bytes": wbytes,
+                                      "note": "plain read of the same packed bytes per launch, same ring, same timing"}
+    # counter-derived HBM bytes per launch, recorded under profiles/ for the measured configurations
+    tj = args.traffic_json or os.path.join(ROOT, "profiles", f"traffic_{args.workload}_m{m}.json")
+    if not args.probe and os.path.exists(tj):
+        with open(tj) as f:
+            td = json.load(f)
+        roofline["traffic"] = td.get("bytes")
+        roofline["traffic_detail"] = td
 
     cpu = None
     if not args.no_cpu:

@@ -17,6 +17,8 @@
 #include "i8act.h"
 #include "mfma.h"
 
+hipError_t launch_probe(const void *src, void *dst, size_t bytes, uint32_t *sink, hipStream_t s);
+
 struct fnn_hip_graph {
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
@@ -572,6 +574,15 @@ int fnn_hip_qconv2d(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *x, i
         if (acc_out) HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(acc_out, dacc, yout, hipMemcpyDeviceToHost, ctx->stream));
         HIP_TRY(ctx, FNN_ERR_DISPATCH, hipStreamSynchronize(ctx->stream));
     }
+    return FNN_OK;
+}
+
+int fnn_hip_probe_stream(fnn_hip_ctx *ctx, const void *src_dev, void *dst_dev, size_t bytes)
+{
+    if (!ctx || !src_dev) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_probe_stream: NULL argument");
+    if ((reinterpret_cast<uintptr_t>(src_dev) & 15) || (reinterpret_cast<uintptr_t>(dst_dev) & 15))
+        return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_probe_stream: pointers must be 16-byte aligned");
+    HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_probe(src_dev, dst_dev, bytes, reinterpret_cast<uint32_t *>(ctx->scratch), ctx->stream));
     return FNN_OK;
 }
 

@@ -31,7 +31,7 @@ EXPORTED_SYMBOLS = [
     "fnn_hip_malloc", "fnn_hip_free", "fnn_hip_upload", "fnn_hip_download",
     "fnn_hip_weight_register", "fnn_hip_weight_lookup", "fnn_hip_weight_release", "fnn_hip_dequant",
     "fnn_hip_qmatmul", "fnn_hip_quantize_activations", "fnn_hip_qmatmul_i8act", "fnn_hip_qconv2d",
-    "fnn_hip_timer_start", "fnn_hip_timer_stop",
+    "fnn_hip_timer_start", "fnn_hip_timer_stop", "fnn_hip_probe_stream",
     "fnn_hip_graph_begin", "fnn_hip_graph_end", "fnn_hip_graph_launch", "fnn_hip_graph_destroy",
     "fnn_packed_words", "fnn_quantize_weights", "fnn_transpose_kn_to_nk", "fnn_hip_version",
 ]
@@ -94,6 +94,7 @@ def _prototype(l):
     l.fnn_hip_qmatmul_i8act.argtypes = [_vp, _vp, _vp, _i64, _vp, _vp, C.c_int]
     l.fnn_hip_qconv2d.argtypes = [_vp, _vp, _vp, _i64, _i64, _i64, _i64, C.c_int, C.c_int, C.c_int, C.c_int,
                                   C.c_int, C.c_int, _vp, C.c_int, _vp, _vp, C.c_int]
+    l.fnn_hip_probe_stream.argtypes = [_vp, _vp, _vp, _sz]
     l.fnn_hip_timer_start.argtypes = [_vp]
     l.fnn_hip_timer_stop.argtypes = [_vp, C.POINTER(C.c_float)]
     l.fnn_hip_graph_begin.argtypes = [_vp]
@@ -313,6 +314,9 @@ class HipContext:
         return (y, acc) if want_acc else y
 
     # ---- timing / graphs ----
+    def probe_stream(self, src_ptr: int, dst_ptr: int, nbytes: int):
+        self._check(self.lib.fnn_hip_probe_stream(self.handle, _vp(src_ptr), _vp(dst_ptr) if dst_ptr else None, nbytes))
+
     def timer_start(self):
         self._check(self.lib.fnn_hip_timer_start(self.handle))
 

@@ -139,6 +139,12 @@ int fnn_hip_qconv2d(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *x, i
 int fnn_hip_timer_start(fnn_hip_ctx *ctx);
 int fnn_hip_timer_stop(fnn_hip_ctx *ctx, float *elapsed_ms);
 
+/* Memory-system probe (no counterpart in fastnn; measurement aid): one launch that streams
+ * `bytes` from src_dev (16-byte aligned device pointers); dst_dev == NULL reads only,
+ * otherwise copies.  Gives the bandwidth a single launch of that size reaches on the
+ * device and a kernel of known traffic to calibrate hardware byte counters with. */
+int fnn_hip_probe_stream(fnn_hip_ctx *ctx, const void *src_dev, void *dst_dev, size_t bytes);
+
 /* ---- HIP graphs over device-pointer calls: capture a dispatch sequence once,
  * replay it with one launch (a static-shape plan, src/backend/executor.rs:639-667). */
 int fnn_hip_graph_begin(fnn_hip_ctx *ctx);
