@@ -1,0 +1,150 @@
+"""Python view of the host-side HipBackend (include/fastnn_hip_backend.h).
+
+Mirrors fastnn's ``Backend`` trait surface for the quantised-MatMul path
+(src/backend/mod.rs:133-255): ``ExecutablePlan`` holds ``Instruction``s over one byte
+arena, ``HipBackend.dispatch`` runs them on the GPU.  Instruction and argument meaning
+follow CpuBackend::dispatch (src/backend/cpu/mod.rs:2644-2683); a kernel without a GPU
+implementation raises ``FnnError`` of kind ``UnsupportedOp`` whose message is the kernel
+name.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional, Sequence
+
+import numpy as np
+
+from . import lib as _l
+from .lib import FnnError, Slice, WeightMeta
+
+BITS_OF = {_l.DT_I8: 8, _l.DT_I4: 4, _l.DT_U8: 8, _l.DT_U4: 4, _l.DT_F8: 8, _l.DT_F8R: 8, _l.DT_F4: 4, _l.DT_I4CB: 4}
+KERNEL_OF = {_l.DT_I8: "matmul_i8", _l.DT_I4: "matmul_i4", _l.DT_U8: "matmul_u8", _l.DT_U4: "matmul_u4",
+             _l.DT_F8: "matmul_f8", _l.DT_F8R: "matmul_f8r", _l.DT_F4: "matmul_f4", _l.DT_I4CB: "matmul_i4"}
+
+
+def meta_of(pw: "_l.PackedWeight", shape: Optional[Sequence[int]] = None):
+    """QuantizedWeightMeta of a packed weight (src/backend/mod.rs:40-58) as plain fields."""
+    return dict(bit_width=BITS_OF[pw.dtype], scales=np.ascontiguousarray(pw.scales, np.float32),
+                zero_points=np.ascontiguousarray(pw.zeros, np.float32),
+                shape=list(shape) if shape is not None else [pw.rows, pw.inner],
+                quant_block_size=pw.qblock if pw.dtype == _l.DT_I4CB else 0,
+                codebook=None if pw.codebook is None else np.ascontiguousarray(pw.codebook, np.float32))
+
+
+class ExecutablePlan:
+    """ExecutablePlan {instructions, arena_size} (src/backend/mod.rs:109-131)."""
+
+    def __init__(self, arena_size: int):
+        self.lib = _l.load_library()
+        h = C.c_void_p()
+        rc = self.lib.fnn_plan_create(arena_size, C.byref(h))
+        if rc:
+            raise FnnError(rc, "fnn_plan_create failed")
+        self.handle = h
+        self.arena_size = arena_size
+
+    def __len__(self):
+        return int(self.lib.fnn_plan_len(self.handle))
+
+    def _ok(self, rc, what):
+        if rc:
+            raise FnnError(rc, f"{what}: malformed instruction")
+
+    def write_const(self, offset: int, data) -> "ExecutablePlan":
+        buf = np.ascontiguousarray(data).view(np.uint8).reshape(-1)
+        self._ok(self.lib.fnn_plan_add_write_const(self.handle, Slice(offset, buf.nbytes), buf.ctypes.data_as(C.c_void_p),
+                                                   buf.nbytes), "WriteConst")
+        return self
+
+    def fill(self, offset: int, size: int, value: float) -> "ExecutablePlan":
+        self._ok(self.lib.fnn_plan_add_fill(self.handle, Slice(offset, size), value), "Fill")
+        return self
+
+    def memcopy(self, dst, src) -> "ExecutablePlan":
+        self._ok(self.lib.fnn_plan_add_memcopy(self.handle, Slice(*dst), Slice(*src)), "MemCopy")
+        return self
+
+    def call_kernel(self, kernel_name: str, inputs, output, params=(), meta: Optional[dict] = None) -> "ExecutablePlan":
+        ins = (Slice * max(len(inputs), 1))(*[Slice(o, s) for o, s in inputs])
+        par = (C.c_uint64 * max(len(params), 1))(*[int(p) for p in params])
+        mp = None
+        keep = []
+        if meta is not None:
+            sc = np.ascontiguousarray(meta["scales"], np.float32)
+            zp = np.ascontiguousarray(meta["zero_points"], np.float32)
+            sh = np.ascontiguousarray(meta["shape"], np.uint64)
+            cb = meta.get("codebook")
+            cb = None if cb is None else np.ascontiguousarray(cb, np.float32)
+            keep = [sc, zp, sh, cb]
+            m = WeightMeta(int(meta["bit_width"]), sc.ctypes.data_as(C.c_void_p), sc.size,
+                           zp.ctypes.data_as(C.c_void_p), zp.size, sh.ctypes.data_as(C.c_void_p), sh.size,
+                           int(meta.get("quant_block_size", 0)), None if cb is None else cb.ctypes.data_as(C.c_void_p))
+            mp = C.byref(m)
+        self._ok(self.lib.fnn_plan_add_call_kernel(self.handle, kernel_name.encode(), ins, len(inputs), Slice(*output),
+                                                   par, len(params), mp), kernel_name)
+        del keep
+        return self
+
+    def close(self):
+        if self.handle:
+            self.lib.fnn_plan_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class HipBackend:
+    """Backend (src/backend/mod.rs:133-255): name / allocate_arena / write_arena / read_arena / dispatch."""
+
+    def __init__(self, device: int = 0):
+        self.lib = _l.load_library()
+        h = C.c_void_p()
+        rc = self.lib.fnn_backend_create(device, C.byref(h))
+        if rc:
+            msg = self.lib.fnn_hip_last_error(None)
+            raise FnnError(rc, msg.decode() if msg else "fnn_backend_create failed")
+        self.handle = h
+
+    def _check(self, rc):
+        if rc:
+            raise FnnError(rc, self.lib.fnn_backend_last_error(self.handle).decode())
+
+    @property
+    def name(self) -> str:
+        return self.lib.fnn_backend_name(self.handle).decode()
+
+    def allocate_arena(self, total_bytes: int):
+        self._check(self.lib.fnn_backend_allocate_arena(self.handle, total_bytes))
+
+    def write_arena(self, offset: int, data):
+        buf = np.ascontiguousarray(data).view(np.uint8).reshape(-1)
+        self._check(self.lib.fnn_backend_write_arena(self.handle, offset, buf.ctypes.data_as(C.c_void_p), buf.nbytes))
+
+    def read_arena(self, offset: int, size: int, dtype=np.uint8) -> np.ndarray:
+        out = np.empty(size, np.uint8)
+        self._check(self.lib.fnn_backend_read_arena(self.handle, offset, out.ctypes.data_as(C.c_void_p), size))
+        return out.view(dtype)
+
+    def dispatch(self, plan: ExecutablePlan):
+        self._check(self.lib.fnn_backend_dispatch(self.handle, plan.handle))
+
+    def dispatch_profile(self, plan: ExecutablePlan):
+        n = len(plan)
+        t = (C.c_uint64 * max(n, 1))()
+        self._check(self.lib.fnn_backend_dispatch_profile(self.handle, plan.handle, t, n))
+        return [int(t[i]) for i in range(n)]
+
+    def close(self):
+        if self.handle:
+            self.lib.fnn_backend_destroy(self.handle)
+            self.handle = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *a):
+        self.close()

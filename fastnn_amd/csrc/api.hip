@@ -16,8 +16,11 @@
 
 #include "i8act.h"
 #include "mfma.h"
+#include "../../include/fastnn_hip_backend.h"
 
 hipError_t launch_probe(const void *src, void *dst, size_t bytes, uint32_t *sink, hipStream_t s);
+hipError_t launch_fill(float *dst, uint64_t n, float value, hipStream_t s);
+hipError_t launch_eltwise(int op, const float *a, const float *b, uint64_t nb, float *out, uint64_t n, hipStream_t s);
 
 struct fnn_hip_graph {
     hipGraph_t graph = nullptr;
@@ -583,6 +586,30 @@ int fnn_hip_probe_stream(fnn_hip_ctx *ctx, const void *src_dev, void *dst_dev, s
     if ((reinterpret_cast<uintptr_t>(src_dev) & 15) || (reinterpret_cast<uintptr_t>(dst_dev) & 15))
         return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_probe_stream: pointers must be 16-byte aligned");
     HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_probe(src_dev, dst_dev, bytes, reinterpret_cast<uint32_t *>(ctx->scratch), ctx->stream));
+    return FNN_OK;
+}
+
+int fnn_hip_elementwise(fnn_hip_ctx *ctx, int op, const float *a, const float *b, uint64_t nb, float *out, uint64_t n)
+{
+    if (!ctx || !a || !out) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_elementwise: NULL argument");
+    if (op < 0 || op > 3) return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "fnn_hip_elementwise: unknown op %d", op);
+    if (op == 0 && (!b || nb == 0)) return fail(ctx, FNN_ERR_DISPATCH, "add_f32: missing second operand");
+    HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_eltwise(op, a, b, nb, out, n, ctx->stream));
+    return FNN_OK;
+}
+
+int fnn_hip_fill_f32(fnn_hip_ctx *ctx, float *dst, uint64_t n, float value)
+{
+    if (!ctx || (!dst && n)) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_fill_f32: NULL argument");
+    HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_fill(dst, n, value, ctx->stream));
+    return FNN_OK;
+}
+
+int fnn_hip_copy(fnn_hip_ctx *ctx, void *dst_dev, const void *src_dev, uint64_t bytes)
+{
+    if (!ctx || ((!dst_dev || !src_dev) && bytes)) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_copy: NULL argument");
+    if (bytes == 0) return FNN_OK;
+    HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(dst_dev, src_dev, bytes, hipMemcpyDeviceToDevice, ctx->stream));
     return FNN_OK;
 }
 

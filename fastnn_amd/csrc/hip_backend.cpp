@@ -1,0 +1,552 @@
+// Host-side HipBackend: walks fastnn's instruction stream (src/backend/mod.rs:60-131)
+// over a device-resident arena and routes the quantised MatMul / Conv2d kernels to
+// libfastnn_hip's C ABI.  Plain C++ on top of that ABI: no HIP types appear here.
+//
+// Follows CpuBackend::dispatch (src/backend/cpu/mod.rs:2644-2683) for instruction order
+// and slice handling, quantized_matmul_dispatch (src/backend/cpu/matmul.rs:165-225) for
+// the [activation, weight] / [M,K,N] convention, and the conv2d arm
+// (src/backend/cpu/mod.rs:4106-4260) for the nine Conv2d params.  A kernel name that has
+// no GPU implementation yields FNN_ERR_UNSUPPORTED_OP naming the kernel, so that a
+// caller can run that one instruction elsewhere (src/backend/wgpu/mod.rs:162-239).
+#include <chrono>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <string>
+#include <vector>
+
+#include "../../include/fastnn_hip_backend.h"
+
+namespace {
+
+enum InstrKind { K_WRITE_CONST, K_CALL, K_FILL, K_MEMCOPY };
+
+struct Meta {
+    bool present = false;
+    uint64_t bit_width = 0;
+    std::vector<float> scales, zeros, codebook;
+    std::vector<uint64_t> shape;
+    uint64_t qblock = 0;
+};
+
+struct Instr {
+    InstrKind kind;
+    fnn_slice dst{0, 0}, src{0, 0};
+    std::vector<uint8_t> data;
+    float value = 0.0f;
+    std::string kernel;
+    std::vector<fnn_slice> inputs;
+    std::vector<uint64_t> params;
+    Meta meta;
+    bool clobbered = false;  // WriteConst only: another instruction of the plan writes into dst
+};
+
+bool overlaps(const fnn_slice &a, const fnn_slice &b)
+{
+    return a.size && b.size && a.offset < b.offset + b.size && b.offset < a.offset + a.size;
+}
+
+struct KernelName {
+    std::string base;
+    int act = FNN_ACT_NONE;
+};
+
+// "matmul_i4_silu" -> {"matmul_i4", SILU}; names without an epilogue tag pass through.
+KernelName split_activation(const std::string &name)
+{
+    KernelName r{name, FNN_ACT_NONE};
+    static const struct { const char *suffix; int act; } tags[] = {
+        {"_relu", FNN_ACT_RELU}, {"_gelu", FNN_ACT_GELU}, {"_silu", FNN_ACT_SILU}};
+    for (const auto &t : tags) {
+        size_t n = strlen(t.suffix);
+        if (name.size() > n && name.compare(name.size() - n, n, t.suffix) == 0) {
+            r.base = name.substr(0, name.size() - n);
+            r.act = t.act;
+            return r;
+        }
+    }
+    return r;
+}
+
+int matmul_dtype(const std::string &base)
+{
+    if (base == "matmul_i8") return FNN_DT_I8;
+    if (base == "matmul_i4") return FNN_DT_I4;
+    if (base == "matmul_u8") return FNN_DT_U8;
+    if (base == "matmul_u4") return FNN_DT_U4;
+    if (base == "matmul_f8") return FNN_DT_F8;
+    if (base == "matmul_f8r") return FNN_DT_F8R;
+    if (base == "matmul_f4") return FNN_DT_F4;
+    return -1;
+}
+
+}  // namespace
+
+struct fnn_plan {
+    uint64_t arena_size = 0;
+    std::vector<Instr> instrs;
+    bool analysed = false;
+    // WriteConst payloads stay valid in the arena of this backend at this generation
+    const fnn_backend *resident_on = nullptr;
+    uint64_t resident_generation = 0;
+};
+
+struct fnn_backend {
+    fnn_hip_ctx *ctx = nullptr;
+    uint8_t *arena = nullptr;
+    uint64_t arena_bytes = 0;
+    uint64_t generation = 1;  // bumped whenever the host rewrites the arena
+    std::string err;
+    std::map<std::pair<uint64_t, uint64_t>, fnn_hip_weight *> weights;  // (offset,size) like get_or_cache_packed
+    std::vector<uint8_t> stage;
+};
+
+namespace {
+
+int fail(fnn_backend *b, int code, const char *fmt, ...)
+{
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    if (b) b->err = buf;
+    return code;
+}
+
+int lift(fnn_backend *b, int st)
+{
+    if (st != FNN_OK) {
+        const char *m = fnn_hip_last_error(b->ctx);
+        b->err = m ? m : "libfastnn_hip call failed";
+    }
+    return st;
+}
+
+bool in_arena(const fnn_backend *b, const fnn_slice &s)
+{
+    return s.offset <= b->arena_bytes && s.size <= b->arena_bytes - s.offset;
+}
+
+void drop_weights(fnn_backend *b)
+{
+    for (auto &kv : b->weights) fnn_hip_weight_release(b->ctx, kv.second);
+    b->weights.clear();
+}
+
+void drop_weights_overlapping(fnn_backend *b, const fnn_slice &s)
+{
+    for (auto it = b->weights.begin(); it != b->weights.end();) {
+        fnn_slice w{it->first.first, it->first.second};
+        if (overlaps(w, s)) {
+            fnn_hip_weight_release(b->ctx, it->second);
+            it = b->weights.erase(it);
+        } else {
+            ++it;
+        }
+    }
+}
+
+// get_or_cache_packed + packed_tensor_from_meta: the packed words are taken from the
+// arena bytes of w_slice once and kept as a registered device weight.
+int weight_for(fnn_backend *b, const fnn_slice &ws, int dtype, const Meta &meta, uint64_t rows,
+               uint64_t inner, const char *kernel, fnn_hip_weight **out)
+{
+    auto key = std::make_pair(ws.offset, ws.size);
+    auto it = b->weights.find(key);
+    if (it != b->weights.end()) {
+        *out = it->second;
+        return FNN_OK;
+    }
+    if (ws.size % 4) return fail(b, FNN_ERR_DISPATCH, "%s: weight slice of %llu bytes is not whole u32 words", kernel, (unsigned long long)ws.size);
+    b->stage.resize(ws.size);
+    int st = lift(b, fnn_hip_download(b->ctx, b->stage.data(), b->arena + ws.offset, ws.size));
+    if (st) return st;
+    static const float one = 1.0f, zero = 0.0f;
+    const float *sc = &one, *zp = &zero;
+    size_t nsc = 1, nzp = 1;
+    int qb = 0;
+    const float *cb = nullptr;
+    if (meta.present) {
+        sc = meta.scales.data(); nsc = meta.scales.size();
+        zp = meta.zeros.data(); nzp = meta.zeros.size();
+        qb = (int)meta.qblock;
+        if (!meta.codebook.empty()) cb = meta.codebook.data();
+    }
+    fnn_hip_weight *w = nullptr;
+    uint64_t id = ws.offset * 0x9E3779B97F4A7C15ull ^ ws.size;
+    st = lift(b, fnn_hip_weight_register(b->ctx, id, dtype, (const uint32_t *)b->stage.data(), ws.size / 4,
+                                         (int64_t)rows, (int64_t)inner, sc, nsc, zp, nzp, qb, cb, &w));
+    if (st) return st;
+    b->weights[key] = w;
+    *out = w;
+    return FNN_OK;
+}
+
+int run_matmul(fnn_backend *b, const Instr &in, const KernelName &kn, int dtype)
+{
+    const char *name = in.kernel.c_str();
+    if (in.inputs.size() < 2) return FNN_OK;  // the CPU arm ignores a malformed slice list
+    if (in.params.size() < 3) return fail(b, FNN_ERR_DISPATCH, "%s: expected params [M,K,N]", name);
+    uint64_t m = in.params[0], k = in.params[1], n = in.params[2];
+    const fnn_slice &as = in.inputs[0], &ws = in.inputs[1];
+    if (as.size < m * k * 4) return fail(b, FNN_ERR_DISPATCH, "%s: activation slice holds %llu bytes, M*K*4 = %llu", name, (unsigned long long)as.size, (unsigned long long)(m * k * 4));
+    if (in.dst.size < m * n * 4) return fail(b, FNN_ERR_DISPATCH, "%s: output slice holds %llu bytes, M*N*4 = %llu", name, (unsigned long long)in.dst.size, (unsigned long long)(m * n * 4));
+    if (in.meta.present && !in.meta.codebook.empty()) {
+        if (dtype != FNN_DT_I4) return fail(b, FNN_ERR_DISPATCH, "%s: a codebook needs 4-bit indices", name);
+        dtype = FNN_DT_I4CB;
+    }
+    const float *bias = nullptr;
+    if (in.inputs.size() >= 3 && in.inputs[2].size) {
+        if (in.inputs[2].size < n * 4) return fail(b, FNN_ERR_DISPATCH, "%s: bias slice holds %llu bytes, N*4 = %llu", name, (unsigned long long)in.inputs[2].size, (unsigned long long)(n * 4));
+        bias = (const float *)(b->arena + in.inputs[2].offset);
+    }
+    fnn_hip_weight *w = nullptr;
+    int st = weight_for(b, ws, dtype, in.meta, n, k, name, &w);
+    if (st) return st;
+    if (m == 0 || n == 0) return FNN_OK;
+    return lift(b, fnn_hip_qmatmul(b->ctx, w, (const float *)(b->arena + as.offset), (int64_t)m, bias, kn.act,
+                                   (float *)(b->arena + in.dst.offset), FNN_FLAG_DEVICE_PTRS));
+}
+
+int run_matmul_i8act(fnn_backend *b, const Instr &in, int dtype)
+{
+    const char *name = in.kernel.c_str();
+    if (in.inputs.size() != 2) return FNN_OK;
+    if (in.params.size() < 3) return fail(b, FNN_ERR_DISPATCH, "%s: expected params [M,K,N]", name);
+    uint64_t m = in.params[0], k = in.params[1], n = in.params[2];
+    const fnn_slice &as = in.inputs[0], &ws = in.inputs[1];
+    if (as.size < 8 + m * k) return fail(b, FNN_ERR_DISPATCH, "%s: activation payload holds %llu bytes, 8+M*K = %llu", name, (unsigned long long)as.size, (unsigned long long)(8 + m * k));
+    if (in.dst.size < m * n * 4) return fail(b, FNN_ERR_DISPATCH, "%s: output slice holds %llu bytes, M*N*4 = %llu", name, (unsigned long long)in.dst.size, (unsigned long long)(m * n * 4));
+    fnn_hip_weight *w = nullptr;
+    int st = weight_for(b, ws, dtype, in.meta, n, k, name, &w);
+    if (st) return st;
+    if (m == 0 || n == 0) return FNN_OK;
+    return lift(b, fnn_hip_qmatmul_i8act(b->ctx, w, b->arena + as.offset, (int64_t)m, (float *)(b->arena + in.dst.offset),
+                                         nullptr, FNN_FLAG_DEVICE_PTRS));
+}
+
+int run_quantize_activations(fnn_backend *b, const Instr &in)
+{
+    uint64_t numel = in.params.empty() ? 0 : in.params[0];
+    bool per_channel = in.params.size() > 1 && in.params[1] == 1 && in.params.size() > 2 && in.params[2] > 0;
+    if (per_channel) return fail(b, FNN_ERR_UNSUPPORTED_OP, "quantize_activations: per-channel payloads are not implemented on the GPU");
+    if (in.inputs.empty()) return FNN_OK;
+    const fnn_slice &xs = in.inputs[0];
+    if (in.dst.size < 8) return fail(b, FNN_ERR_DISPATCH, "quantize_activations: output slice has no room for the header");
+    uint64_t cap = in.dst.size - 8;
+    if (numel > cap) numel = cap;  // min(out_bytes.len() - header, numel)
+    if (xs.size < numel * 4) return fail(b, FNN_ERR_DISPATCH, "quantize_activations: input slice holds %llu bytes, numel*4 = %llu", (unsigned long long)xs.size, (unsigned long long)(numel * 4));
+    float scale = 0.0f, zp = 0.0f;  // scale <= 0: dynamic max|x|/127
+    if (in.params.size() >= 5) {
+        uint32_t sb = (uint32_t)in.params[3], zb = (uint32_t)in.params[4];
+        memcpy(&scale, &sb, 4);
+        memcpy(&zp, &zb, 4);
+        if (!(scale > 0.0f)) return fail(b, FNN_ERR_UNSUPPORTED_OP, "quantize_activations: calibrated scale %g is not positive", (double)scale);
+    }
+    return lift(b, fnn_hip_quantize_activations(b->ctx, (const float *)(b->arena + xs.offset), (int64_t)numel, scale, zp,
+                                                b->arena + in.dst.offset, FNN_FLAG_DEVICE_PTRS));
+}
+
+int run_conv2d_i8(fnn_backend *b, const Instr &in, const KernelName &kn)
+{
+    const char *name = in.kernel.c_str();
+    if (in.inputs.size() < 2) return FNN_OK;
+    if (in.params.size() < 9)
+        return fail(b, FNN_ERR_DISPATCH, "%s: expected at least 9 params [stride, padding, dilation, groups, input_c, input_h, input_w, kernel_h, kernel_w]", name);
+    const uint64_t *p = in.params.data();
+    uint64_t stride = p[0], pad = p[1], dil = p[2], groups = p[3], c = p[4], h = p[5], wd = p[6], kh = p[7], kw = p[8];
+    if (groups == 0) return fail(b, FNN_ERR_DISPATCH, "%s: groups=0", name);
+    if (!in.meta.present) return fail(b, FNN_ERR_DISPATCH, "%s: missing weight_meta", name);
+    if (in.meta.shape.empty()) return fail(b, FNN_ERR_DISPATCH, "%s: weight_meta has no shape", name);
+    uint64_t oc = in.meta.shape[0], inner = 1;
+    for (size_t i = 1; i < in.meta.shape.size(); i++) inner *= in.meta.shape[i];
+    uint64_t chw = c * h * wd;
+    uint64_t batch = (in.inputs[0].size / 4) / (chw ? chw : 1);
+    const float *bias = nullptr;
+    if (in.inputs.size() >= 3 && in.inputs[2].size) {
+        if (in.inputs[2].size < oc * 4) return fail(b, FNN_ERR_DISPATCH, "%s: bias slice holds %llu bytes, OC*4 = %llu", name, (unsigned long long)in.inputs[2].size, (unsigned long long)(oc * 4));
+        bias = (const float *)(b->arena + in.inputs[2].offset);
+    }
+    if (stride == 0 || dil == 0) return fail(b, FNN_ERR_DISPATCH, "%s: stride and dilation must be positive", name);
+    uint64_t eh = dil * (kh - 1) + 1, ew = dil * (kw - 1) + 1;
+    if (h + 2 * pad < eh || wd + 2 * pad < ew) return fail(b, FNN_ERR_DISPATCH, "%s: kernel larger than padded input", name);
+    uint64_t oh = (h + 2 * pad - eh) / stride + 1, ow = (wd + 2 * pad - ew) / stride + 1;
+    if (in.dst.size < batch * oc * oh * ow * 4) return fail(b, FNN_ERR_DISPATCH, "%s: output slice holds %llu bytes, needs %llu", name, (unsigned long long)in.dst.size, (unsigned long long)(batch * oc * oh * ow * 4));
+    fnn_hip_weight *w = nullptr;
+    int st = weight_for(b, in.inputs[1], FNN_DT_I8, in.meta, oc, inner, name, &w);
+    if (st) return st;
+    if (batch == 0) return FNN_OK;
+    return lift(b, fnn_hip_qconv2d(b->ctx, w, (const float *)(b->arena + in.inputs[0].offset), (int64_t)batch, (int64_t)c,
+                                   (int64_t)h, (int64_t)wd, (int)kh, (int)kw, (int)stride, (int)pad, (int)dil, (int)groups,
+                                   bias, kn.act, (float *)(b->arena + in.dst.offset), nullptr, FNN_FLAG_DEVICE_PTRS));
+}
+
+int run_elementwise(fnn_backend *b, const Instr &in, int op)
+{
+    const char *name = in.kernel.c_str();
+    if (in.inputs.empty()) return FNN_OK;
+    uint64_t n = in.dst.size / 4;
+    const fnn_slice &a = in.inputs[0];
+    if (a.size / 4 < n) n = a.size / 4;
+    const float *bp = nullptr;
+    uint64_t nb = 0;
+    if (op == 0) {
+        if (in.inputs.size() < 2 || in.inputs[1].size < 4) return fail(b, FNN_ERR_DISPATCH, "%s: expected two inputs", name);
+        bp = (const float *)(b->arena + in.inputs[1].offset);
+        nb = in.inputs[1].size / 4;
+    }
+    return lift(b, fnn_hip_elementwise(b->ctx, op, (const float *)(b->arena + a.offset), bp, nb,
+                                       (float *)(b->arena + in.dst.offset), n));
+}
+
+int run_call(fnn_backend *b, const Instr &in)
+{
+    for (const auto &s : in.inputs)
+        if (!in_arena(b, s)) return fail(b, FNN_ERR_DISPATCH, "%s: input slice [%llu,+%llu) outside the arena of %llu bytes", in.kernel.c_str(), (unsigned long long)s.offset, (unsigned long long)s.size, (unsigned long long)b->arena_bytes);
+    if (!in_arena(b, in.dst)) return fail(b, FNN_ERR_DISPATCH, "%s: output slice [%llu,+%llu) outside the arena of %llu bytes", in.kernel.c_str(), (unsigned long long)in.dst.offset, (unsigned long long)in.dst.size, (unsigned long long)b->arena_bytes);
+    const std::string &name = in.kernel;
+    if (name == "quantize_activations") return run_quantize_activations(b, in);
+    if (name == "matmul_i8_i8") return run_matmul_i8act(b, in, FNN_DT_I8);
+    if (name == "matmul_i4_i8") return run_matmul_i8act(b, in, FNN_DT_I4);
+    if (name == "add_f32") return run_elementwise(b, in, 0);
+    if (name == "relu_f32") return run_elementwise(b, in, 1);
+    if (name == "gelu_f32") return run_elementwise(b, in, 2);
+    if (name == "silu_f32") return run_elementwise(b, in, 3);
+    KernelName kn = split_activation(name);
+    int dt = matmul_dtype(kn.base);
+    if (dt >= 0) return run_matmul(b, in, kn, dt);
+    if (kn.base == "conv2d_i8") return run_conv2d_i8(b, in, kn);
+    return fail(b, FNN_ERR_UNSUPPORTED_OP, "%s", name.c_str());
+}
+
+void analyse(fnn_plan *p)
+{
+    for (auto &c : p->instrs) {
+        if (c.kind != K_WRITE_CONST) continue;
+        c.clobbered = false;
+        for (const auto &o : p->instrs) {
+            if (&o == &c) continue;
+            if (overlaps(o.dst, c.dst)) { c.clobbered = true; break; }
+        }
+    }
+    p->analysed = true;
+}
+
+int run_instr(fnn_backend *b, fnn_plan *p, Instr &in, bool consts_resident)
+{
+    switch (in.kind) {
+    case K_WRITE_CONST: {
+        fnn_slice d{in.dst.offset, in.data.size()};
+        if (!in_arena(b, d)) return fail(b, FNN_ERR_MEMORY, "WriteConst: %llu bytes at %llu outside the arena of %llu bytes", (unsigned long long)d.size, (unsigned long long)d.offset, (unsigned long long)b->arena_bytes);
+        if (consts_resident && !in.clobbered) return FNN_OK;  // bytes already in place and never overwritten
+        if (d.size == 0) return FNN_OK;
+        drop_weights_overlapping(b, d);
+        return lift(b, fnn_hip_upload(b->ctx, b->arena + d.offset, in.data.data(), d.size));
+    }
+    case K_FILL:
+        if (!in_arena(b, in.dst)) return fail(b, FNN_ERR_MEMORY, "Fill: slice outside the arena");
+        return lift(b, fnn_hip_fill_f32(b->ctx, (float *)(b->arena + in.dst.offset), in.dst.size / 4, in.value));
+    case K_MEMCOPY: {
+        if (!in_arena(b, in.dst) || !in_arena(b, in.src)) return fail(b, FNN_ERR_MEMORY, "MemCopy: slice outside the arena");
+        uint64_t n = in.dst.size < in.src.size ? in.dst.size : in.src.size;
+        if (n == 0 || in.dst.offset == in.src.offset) return FNN_OK;
+        fnn_slice d{in.dst.offset, n}, s{in.src.offset, n};
+        if (overlaps(d, s)) return fail(b, FNN_ERR_DISPATCH, "MemCopy: source and destination overlap");
+        return lift(b, fnn_hip_copy(b->ctx, b->arena + d.offset, b->arena + s.offset, n));
+    }
+    case K_CALL:
+        return run_call(b, in);
+    }
+    (void)p;
+    return FNN_OK;
+}
+
+int dispatch_impl(fnn_backend *b, fnn_plan *p, uint64_t *elapsed_ns, uint64_t n_elapsed)
+{
+    if (!b || !p) return fail(b, FNN_ERR_DISPATCH, "dispatch: NULL argument");
+    if (!b->arena) return fail(b, FNN_ERR_MEMORY, "dispatch: no arena allocated");
+    if (p->arena_size > b->arena_bytes) return fail(b, FNN_ERR_MEMORY, "dispatch: plan needs an arena of %llu bytes, backend holds %llu", (unsigned long long)p->arena_size, (unsigned long long)b->arena_bytes);
+    if (elapsed_ns && n_elapsed < p->instrs.size()) return fail(b, FNN_ERR_DISPATCH, "dispatch_profile: room for %llu timings, plan has %llu instructions", (unsigned long long)n_elapsed, (unsigned long long)p->instrs.size());
+    if (!p->analysed) analyse(p);
+    bool resident = p->resident_on == b && p->resident_generation == b->generation;
+    for (size_t i = 0; i < p->instrs.size(); i++) {
+        auto t0 = std::chrono::steady_clock::now();
+        int st = run_instr(b, p, p->instrs[i], resident);
+        if (st == FNN_OK && elapsed_ns) st = lift(b, fnn_hip_sync(b->ctx));
+        if (st != FNN_OK) {
+            fnn_hip_sync(b->ctx);
+            return st;
+        }
+        if (elapsed_ns) elapsed_ns[i] = (uint64_t)std::chrono::duration_cast<std::chrono::nanoseconds>(std::chrono::steady_clock::now() - t0).count();
+    }
+    int st = lift(b, fnn_hip_sync(b->ctx));
+    if (st == FNN_OK) {
+        p->resident_on = b;
+        p->resident_generation = b->generation;
+    }
+    return st;
+}
+
+}  // namespace
+
+extern "C" {
+
+int fnn_backend_create(int device, fnn_backend **out)
+{
+    if (!out) return FNN_ERR_DISPATCH;
+    *out = nullptr;
+    fnn_hip_ctx *ctx = nullptr;
+    int st = fnn_hip_create(device, &ctx);
+    if (st) return st;
+    fnn_backend *b = new fnn_backend();
+    b->ctx = ctx;
+    *out = b;
+    return FNN_OK;
+}
+
+void fnn_backend_destroy(fnn_backend *b)
+{
+    if (!b) return;
+    drop_weights(b);
+    if (b->arena) fnn_hip_free(b->ctx, b->arena);
+    fnn_hip_destroy(b->ctx);
+    delete b;
+}
+
+const char *fnn_backend_name(const fnn_backend *) { return "hip"; }
+
+const char *fnn_backend_last_error(const fnn_backend *b) { return b ? b->err.c_str() : "no backend"; }
+
+int fnn_backend_allocate_arena(fnn_backend *b, uint64_t total_bytes)
+{
+    if (!b) return FNN_ERR_DISPATCH;
+    drop_weights(b);
+    if (b->arena) {
+        fnn_hip_free(b->ctx, b->arena);
+        b->arena = nullptr;
+        b->arena_bytes = 0;
+    }
+    b->generation++;
+    // CpuBuffer::new zero-fills; keep 64 bytes of slack so that vector loads at the end stay inside
+    void *d = nullptr;
+    uint64_t padded = ((total_bytes + 63) / 64) * 64 + 64;
+    int st = lift(b, fnn_hip_malloc(b->ctx, padded, &d));
+    if (st) return st;
+    b->arena = (uint8_t *)d;
+    b->arena_bytes = total_bytes;
+    st = lift(b, fnn_hip_fill_f32(b->ctx, (float *)d, padded / 4, 0.0f));
+    if (st) return st;
+    return lift(b, fnn_hip_sync(b->ctx));
+}
+
+int fnn_backend_write_arena(fnn_backend *b, uint64_t offset, const void *data, uint64_t size)
+{
+    if (!b) return FNN_ERR_DISPATCH;
+    fnn_slice s{offset, size};
+    if (!b->arena || !in_arena(b, s)) return fail(b, FNN_ERR_MEMORY, "write_arena: %llu bytes at %llu outside the arena of %llu bytes", (unsigned long long)size, (unsigned long long)offset, (unsigned long long)b->arena_bytes);
+    if (size == 0) return FNN_OK;
+    if (!data) return fail(b, FNN_ERR_DISPATCH, "write_arena: NULL data");
+    drop_weights_overlapping(b, s);
+    b->generation++;
+    return lift(b, fnn_hip_upload(b->ctx, b->arena + offset, data, size));
+}
+
+int fnn_backend_read_arena(fnn_backend *b, uint64_t offset, void *out, uint64_t size)
+{
+    if (!b) return FNN_ERR_DISPATCH;
+    fnn_slice s{offset, size};
+    if (!b->arena || !in_arena(b, s)) return fail(b, FNN_ERR_MEMORY, "read_arena: %llu bytes at %llu outside the arena of %llu bytes", (unsigned long long)size, (unsigned long long)offset, (unsigned long long)b->arena_bytes);
+    if (size == 0) return FNN_OK;
+    if (!out) return fail(b, FNN_ERR_DISPATCH, "read_arena: NULL destination");
+    return lift(b, fnn_hip_download(b->ctx, out, b->arena + offset, size));
+}
+
+int fnn_plan_create(uint64_t arena_size, fnn_plan **out)
+{
+    if (!out) return FNN_ERR_DISPATCH;
+    *out = new fnn_plan();
+    (*out)->arena_size = arena_size;
+    return FNN_OK;
+}
+
+void fnn_plan_destroy(fnn_plan *p) { delete p; }
+
+uint64_t fnn_plan_len(const fnn_plan *p) { return p ? p->instrs.size() : 0; }
+
+static void touched(fnn_plan *p)
+{
+    p->analysed = false;
+    p->resident_on = nullptr;
+}
+
+int fnn_plan_add_write_const(fnn_plan *p, fnn_slice dst, const void *data, uint64_t len)
+{
+    if (!p || (!data && len)) return FNN_ERR_DISPATCH;
+    Instr in;
+    in.kind = K_WRITE_CONST;
+    in.dst = fnn_slice{dst.offset, len};
+    in.data.assign((const uint8_t *)data, (const uint8_t *)data + len);
+    p->instrs.push_back(std::move(in));
+    touched(p);
+    return FNN_OK;
+}
+
+int fnn_plan_add_fill(fnn_plan *p, fnn_slice dst, float value)
+{
+    if (!p) return FNN_ERR_DISPATCH;
+    Instr in;
+    in.kind = K_FILL;
+    in.dst = dst;
+    in.value = value;
+    p->instrs.push_back(std::move(in));
+    touched(p);
+    return FNN_OK;
+}
+
+int fnn_plan_add_memcopy(fnn_plan *p, fnn_slice dst, fnn_slice src)
+{
+    if (!p) return FNN_ERR_DISPATCH;
+    Instr in;
+    in.kind = K_MEMCOPY;
+    in.dst = dst;
+    in.src = src;
+    p->instrs.push_back(std::move(in));
+    touched(p);
+    return FNN_OK;
+}
+
+int fnn_plan_add_call_kernel(fnn_plan *p, const char *kernel_name, const fnn_slice *inputs, uint64_t n_inputs,
+                             fnn_slice output, const uint64_t *params, uint64_t n_params, const fnn_weight_meta *meta)
+{
+    if (!p || !kernel_name || (!inputs && n_inputs) || (!params && n_params)) return FNN_ERR_DISPATCH;
+    Instr in;
+    in.kind = K_CALL;
+    in.kernel = kernel_name;
+    in.inputs.assign(inputs, inputs + n_inputs);
+    in.dst = output;
+    in.params.assign(params, params + n_params);
+    if (meta) {
+        in.meta.present = true;
+        in.meta.bit_width = meta->bit_width;
+        if (meta->scales) in.meta.scales.assign(meta->scales, meta->scales + meta->n_scales);
+        if (meta->zero_points) in.meta.zeros.assign(meta->zero_points, meta->zero_points + meta->n_zero_points);
+        if (meta->shape) in.meta.shape.assign(meta->shape, meta->shape + meta->n_shape);
+        in.meta.qblock = meta->quant_block_size;
+        if (meta->codebook16) in.meta.codebook.assign(meta->codebook16, meta->codebook16 + 16);
+    }
+    p->instrs.push_back(std::move(in));
+    touched(p);
+    return FNN_OK;
+}
+
+int fnn_backend_dispatch(fnn_backend *b, fnn_plan *p) { return dispatch_impl(b, p, nullptr, 0); }
+
+int fnn_backend_dispatch_profile(fnn_backend *b, fnn_plan *p, uint64_t *elapsed_ns, uint64_t n)
+{
+    if (!elapsed_ns) return fail(b, FNN_ERR_DISPATCH, "dispatch_profile: NULL timings");
+    return dispatch_impl(b, p, elapsed_ns, n);
+}
+
+}  // extern "C"

@@ -35,6 +35,15 @@ EXPORTED_SYMBOLS = [
     "fnn_hip_graph_begin", "fnn_hip_graph_end", "fnn_hip_graph_launch", "fnn_hip_graph_destroy",
     "fnn_packed_words", "fnn_quantize_weights", "fnn_transpose_kn_to_nk", "fnn_hip_version",
 ]
+# every symbol include/fastnn_hip_backend.h declares
+BACKEND_SYMBOLS = [
+    "fnn_backend_create", "fnn_backend_destroy", "fnn_backend_name", "fnn_backend_last_error",
+    "fnn_backend_allocate_arena", "fnn_backend_write_arena", "fnn_backend_read_arena",
+    "fnn_plan_create", "fnn_plan_destroy", "fnn_plan_add_write_const", "fnn_plan_add_fill",
+    "fnn_plan_add_memcopy", "fnn_plan_add_call_kernel", "fnn_plan_len",
+    "fnn_backend_dispatch", "fnn_backend_dispatch_profile",
+    "fnn_hip_elementwise", "fnn_hip_fill_f32", "fnn_hip_copy",
+]
 
 
 class FnnError(RuntimeError):
@@ -69,7 +78,20 @@ def load_library(path: Optional[str] = None):
 
 _vp = C.c_void_p
 _i64 = C.c_int64
+_u64 = C.c_uint64
 _sz = C.c_size_t
+
+
+class Slice(C.Structure):
+    """fnn_slice: BufferSlice {offset, size} in bytes."""
+    _fields_ = [("offset", C.c_uint64), ("size", C.c_uint64)]
+
+
+class WeightMeta(C.Structure):
+    """fnn_weight_meta: QuantizedWeightMeta."""
+    _fields_ = [("bit_width", C.c_uint64), ("scales", _vp), ("n_scales", C.c_uint64),
+                ("zero_points", _vp), ("n_zero_points", C.c_uint64), ("shape", _vp), ("n_shape", C.c_uint64),
+                ("quant_block_size", C.c_uint64), ("codebook16", _vp)]
 
 
 def _prototype(l):
@@ -107,6 +129,31 @@ def _prototype(l):
     l.fnn_transpose_kn_to_nk.argtypes = [_vp, _i64, _i64, _vp]
     l.fnn_transpose_kn_to_nk.restype = None
     l.fnn_hip_version.restype = C.c_char_p
+    l.fnn_backend_create.argtypes = [C.c_int, C.POINTER(_vp)]
+    l.fnn_backend_destroy.argtypes = [_vp]
+    l.fnn_backend_destroy.restype = None
+    l.fnn_backend_name.argtypes = [_vp]
+    l.fnn_backend_name.restype = C.c_char_p
+    l.fnn_backend_last_error.argtypes = [_vp]
+    l.fnn_backend_last_error.restype = C.c_char_p
+    l.fnn_backend_allocate_arena.argtypes = [_vp, _u64]
+    l.fnn_backend_write_arena.argtypes = [_vp, _u64, _vp, _u64]
+    l.fnn_backend_read_arena.argtypes = [_vp, _u64, _vp, _u64]
+    l.fnn_plan_create.argtypes = [_u64, C.POINTER(_vp)]
+    l.fnn_plan_destroy.argtypes = [_vp]
+    l.fnn_plan_destroy.restype = None
+    l.fnn_plan_add_write_const.argtypes = [_vp, Slice, _vp, _u64]
+    l.fnn_plan_add_fill.argtypes = [_vp, Slice, C.c_float]
+    l.fnn_plan_add_memcopy.argtypes = [_vp, Slice, Slice]
+    l.fnn_plan_add_call_kernel.argtypes = [_vp, C.c_char_p, C.POINTER(Slice), _u64, Slice, C.POINTER(_u64), _u64,
+                                           C.POINTER(WeightMeta)]
+    l.fnn_plan_len.argtypes = [_vp]
+    l.fnn_plan_len.restype = _u64
+    l.fnn_backend_dispatch.argtypes = [_vp, _vp]
+    l.fnn_backend_dispatch_profile.argtypes = [_vp, _vp, C.POINTER(_u64), _u64]
+    l.fnn_hip_elementwise.argtypes = [_vp, C.c_int, _vp, _vp, _u64, _vp, _u64]
+    l.fnn_hip_fill_f32.argtypes = [_vp, _vp, _u64, C.c_float]
+    l.fnn_hip_copy.argtypes = [_vp, _vp, _vp, _u64]
 
 
 def _np_ptr(a: Optional[np.ndarray]):

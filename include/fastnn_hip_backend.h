@@ -1,0 +1,85 @@
+/*
+ * fastnn_hip_backend.h -- C view of the host-side HipBackend: the instruction-level
+ * contract fastnn's executor hands a backend (src/backend/mod.rs:27-131), consumed here
+ * without Rust.  A plan is a list of WriteConst / CallKernel / Fill / MemCopy
+ * instructions over one byte arena; fnn_backend_dispatch() walks it sequentially the way
+ * CpuBackend::dispatch does (src/backend/cpu/mod.rs:2644-2683), running the quantised
+ * MatMul / Conv2d kernels (and the few f32 elementwise kernels found between them) on
+ * the GPU against a device-resident arena.  A kernel name it does not implement returns
+ * FNN_ERR_UNSUPPORTED_OP, which a Rust HipBackend answers by running that single
+ * instruction on CpuBackend (as WgpuBackend does, src/backend/wgpu/mod.rs:162-239).
+ */
+#ifndef FASTNN_HIP_BACKEND_H
+#define FASTNN_HIP_BACKEND_H
+
+#include "fastnn_hip.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct fnn_backend fnn_backend;
+typedef struct fnn_plan fnn_plan;
+
+/* BufferSlice, src/backend/mod.rs:27-38 */
+typedef struct {
+    uint64_t offset;
+    uint64_t size;
+} fnn_slice;
+
+/* QuantizedWeightMeta, src/backend/mod.rs:40-58 (codebook16 == NULL: no codebook) */
+typedef struct {
+    uint64_t bit_width;
+    const float *scales;
+    uint64_t n_scales;
+    const float *zero_points;
+    uint64_t n_zero_points;
+    const uint64_t *shape;
+    uint64_t n_shape;
+    uint64_t quant_block_size;
+    const float *codebook16;
+} fnn_weight_meta;
+
+/* Backend::name / allocate_arena / write_arena / read_arena, src/backend/mod.rs:152-254 */
+int fnn_backend_create(int device, fnn_backend **out);
+void fnn_backend_destroy(fnn_backend *b);
+const char *fnn_backend_name(const fnn_backend *b);
+const char *fnn_backend_last_error(const fnn_backend *b);
+int fnn_backend_allocate_arena(fnn_backend *b, uint64_t total_bytes);
+int fnn_backend_write_arena(fnn_backend *b, uint64_t offset, const void *data, uint64_t size);
+int fnn_backend_read_arena(fnn_backend *b, uint64_t offset, void *out, uint64_t size);
+
+/* ExecutablePlan / Instruction, src/backend/mod.rs:60-107 */
+int fnn_plan_create(uint64_t arena_size, fnn_plan **out);
+void fnn_plan_destroy(fnn_plan *p);
+int fnn_plan_add_write_const(fnn_plan *p, fnn_slice dst, const void *data, uint64_t len);
+int fnn_plan_add_fill(fnn_plan *p, fnn_slice dst, float value);
+int fnn_plan_add_memcopy(fnn_plan *p, fnn_slice dst, fnn_slice src);
+/* kernel_name as CpuBackend::compile emits it (src/backend/cpu/mod.rs:415-495, 815-865);
+ * a quantised MatMul may carry the epilogue the fusion pass attached as a suffix
+ * "_relu" | "_gelu" | "_silu" and a third input slice for the bias. */
+int fnn_plan_add_call_kernel(fnn_plan *p, const char *kernel_name, const fnn_slice *inputs,
+                             uint64_t n_inputs, fnn_slice output, const uint64_t *params,
+                             uint64_t n_params, const fnn_weight_meta *meta);
+uint64_t fnn_plan_len(const fnn_plan *p);
+
+/* Backend::dispatch, src/backend/mod.rs:167-176.  Synchronises before returning. */
+int fnn_backend_dispatch(fnn_backend *b, fnn_plan *p);
+/* Backend::dispatch_profile, src/backend/mod.rs:178-211: elapsed_ns[i] per instruction */
+int fnn_backend_dispatch_profile(fnn_backend *b, fnn_plan *p, uint64_t *elapsed_ns, uint64_t n);
+
+/* f32 elementwise kernels found between quantised layers ("add_f32" with the second operand
+ * broadcast by index modulo its length, "relu_f32", "gelu_f32", "silu_f32";
+ * src/backend/cpu/mod.rs:2699-2751).  op: 0 add, 1 relu, 2 gelu, 3 silu.  Device pointers. */
+int fnn_hip_elementwise(fnn_hip_ctx *ctx, int op, const float *a, const float *b, uint64_t nb,
+                        float *out, uint64_t n);
+
+/* Instruction::Fill (f32 elements) and Instruction::MemCopy on device memory
+ * (src/backend/mod.rs:92-106); both only enqueue on the context's stream. */
+int fnn_hip_fill_f32(fnn_hip_ctx *ctx, float *dst, uint64_t n, float value);
+int fnn_hip_copy(fnn_hip_ctx *ctx, void *dst_dev, const void *src_dev, uint64_t bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

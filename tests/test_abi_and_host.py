@@ -27,12 +27,34 @@ def test_library_exports_every_declared_symbol():
 
 def test_backend_header_symbols_exported():
     path = os.path.join(ROOT, "include", "fastnn_hip_backend.h")
-    if not os.path.exists(path):
-        pytest.skip("backend header not present")
     l = fastnn_amd.load_library()
-    declared = set(re.findall(r"\b(fnn_backend_[a-z0-9_]+|fnn_plan_[a-z0-9_]+)\s*\(", open(path).read()))
+    declared = set(re.findall(r"\b(fnn_[a-z0-9_]+)\s*\(", open(path).read()))
+    assert len(declared) >= 16
     for name in sorted(declared):
-        assert hasattr(l, name), name
+        assert hasattr(l, name), f"{name} declared in fastnn_hip_backend.h but not exported"
+    assert declared == set(flib.BACKEND_SYMBOLS)
+
+
+def test_plan_builds_without_a_gpu():
+    """Plans are host objects: building one needs no device; malformed instructions are refused."""
+    from fastnn_amd.backend import ExecutablePlan
+    p = ExecutablePlan(4096)
+    p.write_const(0, np.arange(16, dtype=np.float32)).fill(64, 64, 1.5).memcopy((128, 64), (0, 64))
+    p.call_kernel("matmul_i8_relu", [(0, 64), (256, 64)], (512, 64), [1, 16, 16],
+                  dict(bit_width=8, scales=[1.0], zero_points=[0.0], shape=[16, 16]))
+    assert len(p) == 4
+    l = fastnn_amd.load_library()
+    assert l.fnn_plan_add_call_kernel(p.handle, None, None, 0, flib.Slice(0, 0), None, 0, None) != 0
+    p.close()
+
+
+def test_backend_create_without_gpu_reports_an_error():
+    l = fastnn_amd.load_library()
+    if l.fnn_hip_device_count() > 0:
+        pytest.skip("a GPU is present")
+    from fastnn_amd.backend import HipBackend
+    with pytest.raises(flib.FnnError):
+        HipBackend(0)
 
 
 def test_missing_library_fails_loudly(tmp_path):

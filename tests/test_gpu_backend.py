@@ -1,0 +1,231 @@
+"""GPU tests of the host-side HipBackend: plans of WriteConst / CallKernel / Fill / MemCopy
+instructions dispatched against a device arena, checked with the CPU oracle.  The plans are
+laid out the way fastnn's compile step emits them for a quantised model: constants first,
+then one CallKernel per layer, kernel names carrying the fused epilogue as a suffix."""
+import numpy as np
+import pytest
+
+import fastnn_amd
+from fastnn_amd import lib as flib
+from fastnn_amd.backend import ExecutablePlan, HipBackend, KERNEL_OF, meta_of
+from gpu_common import assert_close, to_oracle
+
+pytestmark = pytest.mark.gpu
+
+
+class Arena:
+    """Bump allocator for byte offsets, 64-byte aligned like fastnn's memory planner slots."""
+
+    def __init__(self):
+        self.top = 0
+
+    def take(self, nbytes):
+        off = self.top
+        self.top += (nbytes + 63) // 64 * 64
+        return (off, nbytes)
+
+
+@pytest.fixture(scope="module")
+def be():
+    b = HipBackend(0)
+    yield b
+    b.close()
+
+
+def _w(rng, n, k):
+    return (rng.standard_normal((n, k)) * 0.05).astype(np.float32)
+
+
+def test_name_and_arena_roundtrip(be):
+    assert be.name == "hip"
+    be.allocate_arena(1000)
+    assert not be.read_arena(0, 1000).any()          # a fresh arena is zero-filled
+    data = np.arange(250, dtype=np.float32)
+    be.write_arena(0, data)
+    assert np.array_equal(be.read_arena(0, 1000, np.float32), data)
+    be.write_arena(996, np.float32([7.0]))
+    assert be.read_arena(996, 4, np.float32)[0] == 7.0
+    with pytest.raises(flib.FnnError) as e:
+        be.write_arena(998, np.float32([1.0]))
+    assert e.value.kind == "Memory"
+    with pytest.raises(flib.FnnError):
+        be.read_arena(1, 1000)
+
+
+@pytest.mark.parametrize("m", [1, 8, 64])
+def test_mlp_block_plan_fp8_up_fp4_down(be, orc, m):
+    """x -> FP8 up-projection + bias + GELU (fused suffix) -> FP4 down-projection -> residual add."""
+    rng = np.random.default_rng(90 + m)
+    d, f = 256, 1024
+    x = rng.standard_normal((m, d)).astype(np.float32)
+    up = fastnn_amd.quantize_weights(flib.DT_F8, _w(rng, f, d))
+    down = fastnn_amd.quantize_weights(flib.DT_F4, _w(rng, d, f))
+    b_up = (rng.standard_normal(f) * 0.1).astype(np.float32)
+    a = Arena()
+    s_x, s_up, s_bup, s_down = a.take(x.nbytes), a.take(up.words.nbytes), a.take(b_up.nbytes), a.take(down.words.nbytes)
+    s_h, s_y, s_out = a.take(m * f * 4), a.take(m * d * 4), a.take(m * d * 4)
+    plan = ExecutablePlan(a.top)
+    plan.write_const(s_up[0], up.words).write_const(s_bup[0], b_up).write_const(s_down[0], down.words)
+    plan.call_kernel("matmul_f8_gelu", [s_x, s_up, s_bup], s_h, [m, d, f], meta_of(up))
+    plan.call_kernel("matmul_f4", [s_h, s_down], s_y, [m, f, d], meta_of(down))
+    plan.call_kernel("add_f32", [s_y, s_x], s_out, [m * d])
+    be.allocate_arena(a.top)
+    be.write_arena(s_x[0], x)
+    be.dispatch(plan)
+    h_ref = orc.qmatmul(to_oracle(orc, up), x, bias=b_up, act=flib.ACT_GELU)
+    y_ref = orc.qmatmul(to_oracle(orc, down), h_ref) + x
+    got_h = be.read_arena(*s_h, np.float32).reshape(m, f)
+    got = be.read_arena(*s_out, np.float32).reshape(m, d)
+    assert_close(got_h, h_ref, 2e-5, "hidden")
+    assert_close(got, y_ref, 1e-4, "block output")       # the second layer sees got_h, not h_ref
+    # second dispatch with a new input: constants stay resident, result follows the input
+    x2 = rng.standard_normal((m, d)).astype(np.float32)
+    be.write_arena(s_x[0], x2)
+    be.dispatch(plan)
+    h2 = orc.qmatmul(to_oracle(orc, up), x2, bias=b_up, act=flib.ACT_GELU)
+    y2 = orc.qmatmul(to_oracle(orc, down), h2) + x2
+    assert_close(be.read_arena(*s_out, np.float32).reshape(m, d), y2, 1e-4, "second dispatch")
+    times = be.dispatch_profile(plan)
+    assert len(times) == len(plan) and all(t > 0 for t in times[3:])
+
+
+@pytest.mark.parametrize("dt", list(range(8)))
+@pytest.mark.parametrize("act", ["", "_relu", "_silu"])
+def test_every_matmul_kernel_name(be, orc, dt, act):
+    rng = np.random.default_rng(300 + dt)
+    m, k, n = 3, 160, 72
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    pw = fastnn_amd.quantize_weights(dt, _w(rng, n, k))
+    a = Arena()
+    s_x, s_w, s_o = a.take(x.nbytes), a.take(pw.words.nbytes), a.take(m * n * 4)
+    plan = ExecutablePlan(a.top).write_const(s_x[0], x).write_const(s_w[0], pw.words)
+    plan.call_kernel(KERNEL_OF[dt] + act, [s_x, s_w], s_o, [m, k, n], meta_of(pw))
+    be.allocate_arena(a.top)
+    be.dispatch(plan)
+    code = {"": 0, "_relu": 1, "_silu": 3}[act]
+    want = orc.qmatmul(to_oracle(orc, pw), x, act=code)
+    assert_close(be.read_arena(*s_o, np.float32).reshape(m, n), want, 2e-5, KERNEL_OF[dt] + act)
+
+
+@pytest.mark.parametrize("dt,name", [(flib.DT_I8, "matmul_i8_i8"), (flib.DT_I4, "matmul_i4_i8")])
+@pytest.mark.parametrize("calibrated", [False, True])
+def test_i8_activation_chain(be, orc, dt, name, calibrated):
+    """quantize_activations -> matmul_*_i8: payload bytes bit-exact, output equal to the oracle's."""
+    rng = np.random.default_rng(17)
+    m, k, n = 6, 200, 40
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    pw = fastnn_amd.quantize_weights(dt, _w(rng, n, k))
+    a = Arena()
+    s_x, s_w, s_q, s_o = a.take(x.nbytes), a.take(pw.words.nbytes), a.take(8 + m * k), a.take(m * n * 4)
+    params = [m * k, 0, 0]
+    scale, zp = np.float32(0.03), np.float32(0.25)
+    if calibrated:
+        params += [int(scale.view(np.uint32)), int(zp.view(np.uint32))]
+    plan = ExecutablePlan(a.top).write_const(s_w[0], pw.words)
+    plan.call_kernel("quantize_activations", [s_x], s_q, params)
+    plan.call_kernel(name, [s_q, s_w], s_o, [m, k, n], meta_of(pw))
+    be.allocate_arena(a.top)
+    be.write_arena(s_x[0], x)
+    be.dispatch(plan)
+    payload = orc.quantize_activations(x, float(scale), float(zp)) if calibrated else orc.quantize_activations(x)
+    assert np.array_equal(be.read_arena(*s_q), payload)
+    want = orc.qmatmul_i8act(to_oracle(orc, pw), payload, m)
+    assert_close(be.read_arena(*s_o, np.float32).reshape(m, n), want, 1e-6, name)
+
+
+@pytest.mark.parametrize("act,code", [("", 0), ("_relu", 1), ("_silu", 3)])
+def test_conv2d_i8_plan(be, orc, act, code):
+    rng = np.random.default_rng(41)
+    b, c, h, w, oc, kh, kw, stride, pad, dil, groups = 2, 8, 14, 11, 12, 3, 3, 2, 1, 1, 2
+    kk = c // groups * kh * kw
+    x = rng.uniform(0, 1, (b, c, h, w)).astype(np.float32)
+    pw = fastnn_amd.quantize_weights(flib.DT_I8, (rng.standard_normal((oc, kk)) * 0.1).astype(np.float32))
+    bias = (rng.standard_normal(oc) * 0.05).astype(np.float32)
+    want = orc.qconv2d_i8(x, to_oracle(orc, pw), kh, kw, stride, pad, dil, groups, bias=bias, act=code)
+    a = Arena()
+    s_x, s_w, s_b, s_y = a.take(x.nbytes), a.take(pw.words.nbytes), a.take(bias.nbytes), a.take(want.nbytes)
+    plan = ExecutablePlan(a.top).write_const(s_w[0], pw.words).write_const(s_b[0], bias)
+    plan.call_kernel("conv2d_i8" + act, [s_x, s_w, s_b], s_y, [stride, pad, dil, groups, c, h, w, kh, kw],
+                     meta_of(pw, [oc, c // groups, kh, kw]))
+    be.allocate_arena(a.top)
+    be.write_arena(s_x[0], x)
+    be.dispatch(plan)
+    assert_close(be.read_arena(*s_y, np.float32).reshape(want.shape), want, 1e-5, "conv2d_i8" + act)
+
+
+def test_fill_memcopy_and_elementwise(be, orc):
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal(1000).astype(np.float32)
+    a = Arena()
+    s_x, s_f, s_c, s_r, s_g, s_s, s_a = (a.take(4000) for _ in range(7))
+    s_row = a.take(40)
+    plan = ExecutablePlan(a.top).write_const(s_x[0], x).write_const(s_row[0], x[:10])
+    plan.fill(s_f[0], s_f[1], -2.5).memcopy(s_c, s_x)
+    plan.call_kernel("relu_f32", [s_x], s_r, [1000]).call_kernel("gelu_f32", [s_x], s_g, [1000])
+    plan.call_kernel("silu_f32", [s_x], s_s, [1000]).call_kernel("add_f32", [s_x, s_row], s_a, [1000])
+    be.allocate_arena(a.top)
+    be.dispatch(plan)
+    rd = lambda s: be.read_arena(*s, np.float32)
+    assert np.all(rd(s_f) == np.float32(-2.5))
+    assert np.array_equal(rd(s_c), x)
+    assert np.array_equal(rd(s_r), np.maximum(x, 0))
+    assert_close(rd(s_g), orc.act_fn(x, flib.ACT_GELU), 1e-6)
+    assert_close(rd(s_s), orc.act_fn(x, flib.ACT_SILU), 1e-6)
+    assert np.array_equal(rd(s_a), x + np.tile(x[:10], 100))      # second operand broadcast modulo its length
+
+
+def test_unsupported_and_malformed_instructions(be):
+    be.allocate_arena(4096)
+    p = ExecutablePlan(4096).call_kernel("softmax_f32", [(0, 64)], (64, 64), [16])
+    with pytest.raises(flib.FnnError) as e:
+        be.dispatch(p)
+    assert e.value.kind == "UnsupportedOp" and e.value.message == "softmax_f32"
+    p = ExecutablePlan(4096).call_kernel("conv2d_i4", [(0, 64), (64, 64)], (128, 64), [1] * 9)
+    with pytest.raises(flib.FnnError) as e:
+        be.dispatch(p)
+    assert e.value.kind == "UnsupportedOp"
+    p = ExecutablePlan(4096).call_kernel("matmul_i8", [(0, 64), (64, 64)], (128, 64), [4, 4])
+    with pytest.raises(flib.FnnError) as e:
+        be.dispatch(p)
+    assert e.value.kind == "Dispatch" and "expected params [M,K,N]" in e.value.message
+    p = ExecutablePlan(4096).call_kernel("conv2d_i8", [(0, 64), (64, 64)], (128, 64), [1, 0, 1, 0, 1, 4, 4, 1, 1],
+                                         dict(bit_width=8, scales=[1.0], zero_points=[0.0], shape=[1, 1]))
+    with pytest.raises(flib.FnnError) as e:
+        be.dispatch(p)
+    assert "groups=0" in e.value.message
+    p = ExecutablePlan(4096).call_kernel("conv2d_i8", [(0, 64), (64, 64)], (128, 64), [1, 0, 1, 1, 1, 4, 4, 1, 1])
+    with pytest.raises(flib.FnnError) as e:
+        be.dispatch(p)
+    assert "missing weight_meta" in e.value.message
+    p = ExecutablePlan(4096).call_kernel("matmul_i8", [(0, 64), (4090, 64)], (128, 64), [1, 16, 4])
+    with pytest.raises(flib.FnnError) as e:
+        be.dispatch(p)
+    assert "outside the arena" in e.value.message
+    p = ExecutablePlan(8192)
+    with pytest.raises(flib.FnnError) as e:
+        be.dispatch(p)
+    assert e.value.kind == "Memory"
+    # weight slice shorter than rows*kp words: packed_tensor_from_meta's length check
+    p = ExecutablePlan(4096).call_kernel("matmul_i8", [(0, 64), (64, 16)], (128, 64), [1, 16, 4],
+                                         dict(bit_width=8, scales=[1.0], zero_points=[0.0], shape=[4, 16]))
+    with pytest.raises(flib.FnnError) as e:
+        be.dispatch(p)
+    assert e.value.kind == "Dispatch"
+
+
+def test_rewritten_weights_are_re_registered(be, orc):
+    """write_arena over a weight slice drops the cached device weight (the CPU cache would go stale)."""
+    rng = np.random.default_rng(77)
+    m, k, n = 2, 64, 16
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    pw1 = fastnn_amd.quantize_weights(flib.DT_I8, _w(rng, n, k))
+    pw2 = fastnn_amd.quantize_weights(flib.DT_I8, _w(rng, n, k))
+    a = Arena()
+    s_x, s_w, s_o = a.take(x.nbytes), a.take(pw1.words.nbytes), a.take(m * n * 4)
+    be.allocate_arena(a.top)
+    be.write_arena(s_x[0], x)
+    for pw in (pw1, pw2):
+        be.write_arena(s_w[0], pw.words)
+        plan = ExecutablePlan(a.top).call_kernel("matmul_i8", [s_x, s_w], s_o, [m, k, n], meta_of(pw))
+        be.dispatch(plan)
+        assert_close(be.read_arena(*s_o, np.float32).reshape(m, n), orc.qmatmul(to_oracle(orc, pw), x), 2e-5)
