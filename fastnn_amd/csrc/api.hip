@@ -38,7 +38,7 @@ struct fnn_hip_ctx {
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     std::string err;
     std::unordered_map<uint64_t, fnn_hip_weight *> weights;
-    Staging st_a, st_out, st_bias, st_acc, st_tmp, st_tmp2;
+    Staging st_a, st_out, st_bias, st_acc, st_tmp, st_tmp2, st_cnt;
     float *scratch = nullptr;  // small reduction scratch (partials)
     bool capturing = false;
 };
@@ -113,6 +113,7 @@ void free_weight(fnn_hip_weight *w)
     if (w->zeros) (void)hipFree(w->zeros);
     if (w->codebook) (void)hipFree(w->codebook);
     if (w->row_qsum) (void)hipFree(w->row_qsum);
+    if (w->umean) (void)hipFree(w->umean);
     delete w;
 }
 
@@ -161,7 +162,7 @@ void fnn_hip_destroy(fnn_hip_ctx *ctx)
     (void)hipSetDevice(ctx->device);
     if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
     for (auto &kv : ctx->weights) free_weight(kv.second);
-    for (Staging *s : {&ctx->st_a, &ctx->st_out, &ctx->st_bias, &ctx->st_acc, &ctx->st_tmp, &ctx->st_tmp2})
+    for (Staging *s : {&ctx->st_a, &ctx->st_out, &ctx->st_bias, &ctx->st_acc, &ctx->st_tmp, &ctx->st_tmp2, &ctx->st_cnt})
         if (s->ptr) (void)hipFree(s->ptr);
     if (ctx->scratch) (void)hipFree(ctx->scratch);
     if (ctx->ev0) (void)hipEventDestroy(ctx->ev0);
@@ -425,6 +426,10 @@ int fnn_hip_qmatmul(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *a, i
             if (rc) return rc;
         }
         if (!handled) {
+            int rc = fnn_tiled_qmatmul(ctx, ctx->stream, w, p, flags, &handled);
+            if (rc) return rc;
+        }
+        if (!handled) {
             int rc = fnn_mfma_qmatmul(ctx, ctx->stream, w, p, flags, &handled);
             if (rc) return rc;
         }
@@ -678,11 +683,16 @@ int fnn_hip_graph_destroy(fnn_hip_ctx *ctx, fnn_hip_graph *g)
 // staging access for the MFMA translation unit
 int fnn_ctx_ensure_tmp(fnn_hip_ctx *ctx, int which, size_t bytes, void **ptr)
 {
-    Staging &s = which == 0 ? ctx->st_tmp : ctx->st_tmp2;
+    Staging &s = which == 0 ? ctx->st_tmp : (which == 1 ? ctx->st_tmp2 : ctx->st_cnt);
+    const void *before = s.ptr;
     int rc = ensure(ctx, s, bytes);
     if (rc) return rc;
+    // which == 2: arrival counters, zero whenever (re)allocated; kernels leave them at zero
+    if (which == 2 && s.ptr != before) HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemsetAsync(s.ptr, 0, s.cap, ctx->stream));
     *ptr = s.ptr;
     return FNN_OK;
 }
+
+bool fnn_ctx_capturing(fnn_hip_ctx *ctx) { return ctx->capturing; }
 
 int fnn_ctx_fail(fnn_hip_ctx *ctx, int code, const char *msg) { return fail(ctx, code, "%s", msg); }

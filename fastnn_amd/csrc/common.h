@@ -29,6 +29,7 @@ struct fnn_hip_weight {
     float *zeros;       // device; [rows]
     float *codebook;    // device; 16 floats (I4CB) or nullptr
     int32_t *row_qsum;  // device; [rows] sum of integer lanes per row (I8/I4), for the conv epilogue
+    float *umean;       // device; [rows] mean lane value per row, built on first single-pass GEMM use
     int qblock;         // I4CB block length along inner
     int64_t bpr;        // blocks per row
     struct fnn_hip_ctx *ctx;

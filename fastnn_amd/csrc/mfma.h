@@ -6,6 +6,12 @@
 // context services implemented beside the C ABI
 int fnn_ctx_ensure_tmp(fnn_hip_ctx *ctx, int which, size_t bytes, void **ptr);
 int fnn_ctx_fail(fnn_hip_ctx *ctx, int code, const char *msg);
+bool fnn_ctx_capturing(fnn_hip_ctx *ctx);
+
+// M >= 5: activations prepared once as f16 operands, 4-wave output tiles with the
+// activations staged through LDS and optional split of K (deterministic reduction).
+int fnn_tiled_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &p,
+                      int flags, bool *handled);
 
 // f32 activations x packed weights on f16 MFMA tiles; *handled = false when the shape
 // is left to the generic kernel.

@@ -1,0 +1,498 @@
+// Tiled matrix-core quantised MatMul for gfx950, M >= 5 activation rows.
+//
+//   out[m,n] = act((sum_k A[m,k]*u(W[n,k]))*scale[n] + zero[n]*sum_k A[m,k] + bias[n])
+//   (gemm_batch_packed_simd + apply_affine_dot, src/backend/cpu/microkernels/gemm.rs:1982-2088,
+//    src/backend/cpu/microkernels/mod.rs:283-295)
+//
+// Two launches:
+//  1. act_prep_kernel turns the f32 activations into f16 MFMA operands once per call (not
+//     once per workgroup): each row is scaled by a power of two so that max|x| lands in
+//     [2^14, 2^15) and written as hi = f16(x') and, in the default mode, lo = f16((x'-hi)*2^11),
+//     so that hi + lo*2^-11 carries ~22 mantissa bits.  hi and lo rows sit in neighbouring
+//     32-row blocks and go through the same MFMAs as different operand rows.  Row sums
+//     (for the zero-point term) are accumulated in f32 in a fixed order.
+//  2. qgemm_tile_kernel: a workgroup of 4 waves owns a BM x BN output tile and a K range;
+//     the f16 activations are staged through LDS (double buffered), the packed weights go
+//     from HBM straight into registers in MFMA operand order (lane = weight row, 16 bytes
+//     of a row per load), are decoded to f16 there (integer lanes, E4M3/E5M2/E2M1 values
+//     are exact in f16) and multiplied with v_mfma_f32_32x32x16_f16.  With K split over
+//     several workgroups the partial tiles meet in a workspace and the last workgroup to
+//     arrive adds them in split order, so results do not depend on scheduling.
+//
+// FNN_FLAG_ACT_F16_SINGLE keeps hi only and removes the first-order effect of the rounding
+// on rows with a non-zero mean lane value: dot -= mean_k(u[n,k]) * sum_k (hi - x').
+#include "mfma.h"
+#include "dech.h"
+
+#include <cstdlib>
+
+namespace {
+
+using namespace dech;
+
+constexpr int BK = 64;          // k-values per main-loop iteration
+constexpr int LDS_ROW = 144;    // bytes per activation row in LDS: 128 + 16 of padding (bank spread)
+constexpr float LO_UP = 2048.0f, LO_DOWN = 1.0f / 2048.0f;
+
+struct PrepArgs {
+    const float *a;
+    _Float16 *ap;     // [rows_pad][kpad]
+    int *rexp;        // [m_pad] power-of-two exponent applied to the row
+    float *xsum;      // [m_pad] sum_k A[m,k]
+    float *esum;      // [m_pad] sum_k (hi - x') (single mode)
+    int64_t m, k, kpad;
+    int precise, interleaved;
+};
+
+// effective operand row of activation row m: blocks of 32 rows; hi blocks even, lo blocks odd
+__device__ __host__ inline int64_t eff_row(int64_t m, int precise, int lo)
+{
+    if (!precise) return m;
+    return (m / 32) * 64 + lo * 32 + m % 32;
+}
+
+__global__ void __launch_bounds__(256) act_prep_kernel(PrepArgs p)
+{
+    __shared__ float red[3][4];
+    const int64_t m = blockIdx.x;
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const int64_t K = p.k, ngroups = p.kpad / 8;
+    _Float16 *hi_row = p.ap + eff_row(m, p.precise, 0) * p.kpad;
+    _Float16 *lo_row = p.precise ? p.ap + eff_row(m, 1, 1) * p.kpad : nullptr;
+    if (m >= p.m) {  // padding rows of the last tile: zero operands
+        const uint4 z = make_uint4(0, 0, 0, 0);
+        for (int64_t g = tid; g < ngroups; g += 256) {
+            reinterpret_cast<uint4 *>(hi_row)[g] = z;
+            if (lo_row) reinterpret_cast<uint4 *>(lo_row)[g] = z;
+        }
+        if (tid == 0) { p.rexp[m] = 0; p.xsum[m] = 0.0f; p.esum[m] = 0.0f; }
+        return;
+    }
+    const float *x = p.a + m * K;
+    const bool vec = (K % 4 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0);
+    float mx = 0.0f, sum = 0.0f;
+    if (vec) {
+        for (int64_t i = tid; i < K / 4; i += 256) {
+            const float4 v = reinterpret_cast<const float4 *>(x)[i];
+            mx = fmaxf(mx, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+            sum += (v.x + v.y) + (v.z + v.w);
+        }
+    } else {
+        for (int64_t i = tid; i < K; i += 256) {
+            mx = fmaxf(mx, fabsf(x[i]));
+            sum += x[i];
+        }
+    }
+    mx = wave_max(mx);
+    sum = wave_sum(sum);
+    if (lane == 0) { red[0][wv] = mx; red[1][wv] = sum; }
+    __syncthreads();
+    mx = fmaxf(fmaxf(red[0][0], red[0][1]), fmaxf(red[0][2], red[0][3]));
+    sum = (red[1][0] + red[1][1]) + (red[1][2] + red[1][3]);
+    int e = 0;
+    if (mx > 0.0f && mx < __builtin_huge_valf()) {
+        int ex;
+        (void)frexpf(mx, &ex);  // mx = f * 2^ex, f in [0.5, 1)
+        e = 15 - ex;            // mx * 2^e in [2^14, 2^15)
+    }
+    float err = 0.0f;
+    for (int64_t g = tid; g < ngroups; g += 256) {
+        float v[8];
+        const int64_t k0 = g * 8;
+        if (vec && k0 + 8 <= K) {
+            const float4 a0 = *reinterpret_cast<const float4 *>(x + k0);
+            const float4 a1 = *reinterpret_cast<const float4 *>(x + k0 + 4);
+            v[0] = a0.x; v[1] = a0.y; v[2] = a0.z; v[3] = a0.w;
+            v[4] = a1.x; v[5] = a1.y; v[6] = a1.z; v[7] = a1.w;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; j++) v[j] = (k0 + j < K) ? x[k0 + j] : 0.0f;
+        }
+        f16x8 h, l;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            // operand slot j holds k = 0,4,1,5,2,6,3,7 for the nibble decoders
+            const int src = p.interleaved ? ((j & 1) * 4 + (j >> 1)) : j;
+            const float xs = ldexpf(v[src], e);
+            const _Float16 hh = (_Float16)xs;
+            h[j] = hh;
+            const float r = xs - (float)hh;
+            l[j] = (_Float16)(r * LO_UP);
+            err -= r;
+        }
+        *reinterpret_cast<f16x8 *>(hi_row + k0) = h;
+        if (lo_row) *reinterpret_cast<f16x8 *>(lo_row + k0) = l;
+    }
+    err = wave_sum(err);
+    if (lane == 0) red[2][wv] = err;
+    __syncthreads();
+    if (tid == 0) {
+        p.rexp[m] = e;
+        p.xsum[m] = sum;
+        p.esum[m] = (red[2][0] + red[2][1]) + (red[2][2] + red[2][3]);
+    }
+}
+
+// mean lane value per weight row (single mode compensation); one wave per row
+template <int DT>
+__global__ void __launch_bounds__(64) row_umean_kernel(const uint32_t *words, int64_t rows, int64_t kp, int64_t k, float *umean)
+{
+    const int64_t r = blockIdx.x;
+    if (r >= rows) return;
+    constexpr int EPW = Codec<DT>::EPW;
+    float s = 0.0f;
+    for (int64_t i = threadIdx.x; i < kp; i += 64) {
+        float v[EPW];
+        Codec<DT>::decode(words[r * kp + i], v);
+#pragma unroll
+        for (int j = 0; j < EPW; j++)
+            if (i * EPW + j < k) s += v[j];
+    }
+    s = wave_sum(s);
+    if (threadIdx.x == 0) umean[r] = s / (float)k;
+}
+
+struct TileArgs {
+    const uint32_t *words;
+    const float *scales, *zeros, *umean, *bias;
+    const _Float16 *ap;
+    const int *rexp;
+    const float *xsum, *esum;
+    float *out, *part;
+    unsigned *counters;
+    int64_t m, n, kp, kpad;
+    int act, splits, iters, ips, mtiles, ntiles;
+};
+
+template <int DT, int WGM, int WGN, int TM, int TN, bool PRECISE>
+__global__ void __launch_bounds__(256) qgemm_tile_kernel(TileArgs p)
+{
+    using D = DecH<DT>;
+    constexpr int WPS = D::WPS;          // words per 8 k-values
+    constexpr int WPL = 4 * WPS;         // words per lane, column block and iteration
+    constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
+    constexpr int ACH = BM * 8 / 256;    // 16-byte activation chunks per thread and iteration
+    static_assert(WGM * WGN == 4, "4 waves");
+    static_assert(!PRECISE || TM % 2 == 0, "hi/lo block pairs stay in one wave");
+    static_assert(BM * 8 % 256 == 0, "whole chunks per thread");
+
+    __shared__ __attribute__((aligned(16))) unsigned char a_lds[2][BM * LDS_ROW];
+    __shared__ unsigned arrival;
+
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const int wm = wv / WGN, wn = wv % WGN;
+    const int lr = lane & 31, h = lane >> 5;
+
+    // workgroup id -> tile: ids that share a weight column tile land on the same XCD (ids
+    // are dealt round-robin over the 8 XCDs, each with its own L2)
+    const unsigned total = gridDim.x;
+    unsigned L = blockIdx.x;
+    {
+        const unsigned xcd = L & 7, slot = L >> 3, q = total >> 3, r = total & 7;
+        L = xcd * q + (xcd < r ? xcd : r) + slot;
+    }
+    const int mt = L % p.mtiles;
+    const unsigned rest = L / p.mtiles;
+    const int z = rest % p.splits;
+    const int nt = rest / p.splits;
+    const int64_t n0 = (int64_t)nt * BN;
+    const int it0 = z * p.ips;
+    const int it1 = (it0 + p.ips < p.iters) ? it0 + p.ips : p.iters;
+
+    // weight row pointers of this lane (clamped: lanes past N repeat the last row)
+    const uint32_t *wrow[TN];
+#pragma unroll
+    for (int tn = 0; tn < TN; tn++) {
+        int64_t row = n0 + (wn * TN + tn) * 32 + lr;
+        if (row > p.n - 1) row = p.n - 1;
+        wrow[tn] = p.words + row * p.kp + h * WPL;
+    }
+    // activation chunks of this thread: chunk c = tid + 256*j -> row c/8, 16-byte column c%8
+    // (chunk j of a thread is 32 rows below chunk j-1)
+    const _Float16 *asrc = p.ap + ((int64_t)mt * BM + tid / 8) * p.kpad + (tid % 8) * 8;
+    const int64_t astep = 32 * p.kpad;
+    const int adst = (tid / 8) * LDS_ROW + (tid % 8) * 16;
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int tm = 0; tm < TM; tm++)
+#pragma unroll
+        for (int tn = 0; tn < TN; tn++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) acc[tm][tn][i] = 0.0f;
+
+    uint32_t wcur[TN][WPL], wnext[TN][WPL];
+    u32x4 areg[ACH];
+
+    auto load_w = [&](int it, uint32_t(&wq)[TN][WPL]) {
+        const int64_t off = (int64_t)it * (2 * WPL);   // words of the row before this iteration
+#pragma unroll
+        for (int tn = 0; tn < TN; tn++)
+#pragma unroll
+            for (int q = 0; q < WPL / 4; q++) {
+                const int64_t wo = off + h * WPL + q * 4;   // word index inside the row
+                const bool ok = wo + 4 <= p.kp;
+                const uint4 t = *reinterpret_cast<const uint4 *>(wrow[tn] + (ok ? off + q * 4 : 0));
+                const uint32_t msk = ok ? 0xffffffffu : 0u;
+                wq[tn][q * 4 + 0] = t.x & msk; wq[tn][q * 4 + 1] = t.y & msk;
+                wq[tn][q * 4 + 2] = t.z & msk; wq[tn][q * 4 + 3] = t.w & msk;
+            }
+    };
+#define FNN_LOAD_A(IT)                                                                                   \
+    _Pragma("unroll") for (int j = 0; j < ACH; j++)                                                      \
+        areg[j] = *reinterpret_cast<const u32x4 *>(asrc + j * astep + (int64_t)(IT) * BK)
+#define FNN_STORE_A(BUF)                                                                                 \
+    _Pragma("unroll") for (int j = 0; j < ACH; j++)                                                      \
+        *reinterpret_cast<u32x4 *>(&a_lds[BUF][adst + j * 32 * LDS_ROW]) = areg[j]
+
+    if (it0 < it1) {
+        load_w(it0, wcur);
+        FNN_LOAD_A(it0);
+        FNN_STORE_A(0);
+    }
+    __syncthreads();
+    int buf = 0;
+    for (int it = it0; it < it1; it++) {
+        const bool more = it + 1 < it1;
+        if (more) {
+            load_w(it + 1, wnext);
+            FNN_LOAD_A(it + 1);
+        }
+        const unsigned char *abase = &a_lds[buf][(wm * TM * 32 + lr) * LDS_ROW + h * 64];
+#pragma unroll
+        for (int s = 0; s < 4; s++) {
+            f16x8 af[TM], bf[TN];
+#pragma unroll
+            for (int tm = 0; tm < TM; tm++)
+                af[tm] = *reinterpret_cast<const f16x8 *>(abase + tm * 32 * LDS_ROW + s * 16);
+#pragma unroll
+            for (int tn = 0; tn < TN; tn++) bf[tn] = D::step(&wcur[tn][s * WPS]);
+#pragma unroll
+            for (int tm = 0; tm < TM; tm++)
+#pragma unroll
+                for (int tn = 0; tn < TN; tn++)
+                    acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[tm], bf[tn], acc[tm][tn], 0, 0, 0);
+        }
+        if (more) { FNN_STORE_A(buf ^ 1); }
+        __syncthreads();
+        if (more) {
+#pragma unroll
+            for (int tn = 0; tn < TN; tn++)
+#pragma unroll
+                for (int q = 0; q < WPL; q++) wcur[tn][q] = wnext[tn][q];
+        }
+        buf ^= 1;
+    }
+
+#undef FNN_LOAD_A
+#undef FNN_STORE_A
+
+    // ---- epilogue.  acc[i] of a 32x32 block: row (i/4)*8 + h*4 + i%4, column lr.
+    constexpr int TMO = PRECISE ? TM / 2 : TM;       // output row blocks per wave
+    const int64_t mrow0 = ((int64_t)mt * BM / (PRECISE ? 64 : 32) + wm * TMO) * 32;
+    auto row_of = [&](int to, int i) -> int64_t { return mrow0 + to * 32 + (i / 4) * 8 + h * 4 + (i % 4); };
+    auto col_of = [&](int tn) -> int64_t { return n0 + (wn * TN + tn) * 32 + lr; };
+    // this workgroup's share of sum_k A[m,k]*u(W[n,k]), scaled back to the row's magnitude
+    auto dot_of = [&](int to, int tn, int i, int e) -> float {
+        float v;
+        if constexpr (PRECISE) v = acc[2 * to][tn][i] + acc[2 * to + 1][tn][i] * LO_DOWN;
+        else v = acc[to][tn][i];
+        return ldexpf(v, -e);
+    };
+
+    const bool split = p.splits > 1;
+    if (split) {
+        // partial tiles: part[z][m][n]; the last workgroup of the tile to arrive adds them in z order
+#pragma unroll
+        for (int to = 0; to < TMO; to++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const int64_t m = row_of(to, i);
+                if (m >= p.m) continue;
+                const int e = p.rexp[m];
+#pragma unroll
+                for (int tn = 0; tn < TN; tn++) {
+                    const int64_t n = col_of(tn);
+                    if (n < p.n) p.part[((int64_t)z * p.m + m) * p.n + n] = dot_of(to, tn, i, e);
+                }
+            }
+        __threadfence();
+        __syncthreads();
+        if (tid == 0) arrival = atomicAdd(&p.counters[nt * p.mtiles + mt], 1u);
+        __syncthreads();
+        if (arrival != (unsigned)(p.splits - 1)) return;
+        __threadfence();
+        if (tid == 0) p.counters[nt * p.mtiles + mt] = 0;   // ready for the next launch
+    }
+
+    float sc[TN], zp[TN], bi[TN], um[TN];
+#pragma unroll
+    for (int tn = 0; tn < TN; tn++) {
+        const int64_t n = col_of(tn);
+        const bool ok = n < p.n;
+        sc[tn] = ok ? p.scales[n] : 0.0f;
+        zp[tn] = ok ? p.zeros[n] : 0.0f;
+        bi[tn] = (ok && p.bias) ? p.bias[n] : 0.0f;
+        um[tn] = (!PRECISE && ok && p.umean) ? p.umean[n] : 0.0f;
+    }
+#pragma unroll
+    for (int to = 0; to < TMO; to++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const int64_t m = row_of(to, i);
+            if (m >= p.m) continue;
+            const int e = p.rexp[m];
+            const float xs = p.xsum[m];
+            float corr = 0.0f;
+            if constexpr (!PRECISE) corr = ldexpf(p.esum[m], -e);
+#pragma unroll
+            for (int tn = 0; tn < TN; tn++) {
+                const int64_t n = col_of(tn);
+                if (n >= p.n) continue;
+                float d;
+                if (split) {
+                    d = 0.0f;
+                    for (int zz = 0; zz < p.splits; zz++)
+                        d += __builtin_nontemporal_load(&p.part[((int64_t)zz * p.m + m) * p.n + n]);
+                } else {
+                    d = dot_of(to, tn, i, e);
+                }
+                if constexpr (!PRECISE) d = d - um[tn] * corr;
+                float v = d * sc[tn] + zp[tn] * xs;
+                if (p.bias) v = v + bi[tn];
+                p.out[m * p.n + n] = fnn_activation(v, p.act);
+            }
+        }
+}
+
+int env_int(const char *name, int dflt)
+{
+    const char *s = getenv(name);
+    return s ? atoi(s) : dflt;
+}
+
+template <int DT, int WGM, int WGN, int TM, int TN, bool PRECISE>
+hipError_t launch_tile(const TileArgs &p, hipStream_t s)
+{
+    const unsigned total = (unsigned)p.mtiles * p.ntiles * p.splits;
+    hipLaunchKernelGGL((qgemm_tile_kernel<DT, WGM, WGN, TM, TN, PRECISE>), dim3(total), dim3(256), 0, s, p);
+    return hipGetLastError();
+}
+
+template <int DT>
+hipError_t launch_umean(const fnn_hip_weight *w, float *umean, hipStream_t s)
+{
+    hipLaunchKernelGGL(row_umean_kernel<DT>, dim3((unsigned)w->rows), dim3(64), 0, s, w->words, w->rows, w->kp, w->inner, umean);
+    return hipGetLastError();
+}
+
+template <int DT>
+int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &q, int flags)
+{
+    const bool precise = !(flags & FNN_FLAG_ACT_F16_SINGLE);
+    const int64_t M = q.m, N = q.n, K = q.k;
+    const int64_t kpad = (K + BK - 1) / BK * BK;
+    const int64_t mp32 = (M + 31) / 32 * 32;
+    const int64_t meff = precise ? 2 * mp32 : mp32;
+    // tile shape by effective row count
+    int cfg;            // 0: 128x128 (2x2 waves of 64x64), 1: 64x128 (1x4 waves of 64x32), 2: 32x128 (1x4 waves of 32x32)
+    if (meff > 64) cfg = 0;
+    else if (meff == 64) cfg = 1;
+    else cfg = 2;
+    static const int env_cfg = env_int("FNN_TILE_CFG", -1);
+    if (env_cfg >= 0 && env_cfg <= 2 && !(env_cfg == 2 && precise)) cfg = env_cfg;
+    const int bm = cfg == 0 ? 128 : (cfg == 1 ? 64 : 32);
+    const int bn = 128;
+    const int mtiles = (int)((meff + bm - 1) / bm);
+    const int ntiles = (int)((N + bn - 1) / bn);
+    const int64_t rows_pad = (int64_t)mtiles * bm;
+    const int64_t m_pad = precise ? rows_pad / 2 : rows_pad;
+    const int iters = (int)(kpad / BK);
+    // split K until about two workgroups per CU are in flight
+    static const int env_split = env_int("FNN_TILE_SPLIT", 0);
+    static const int env_target = env_int("FNN_TILE_TARGET", 0);
+    int splits = 1;
+    const int base = mtiles * ntiles;
+    if (base < env_target) splits = (env_target + base - 1) / base;
+    if (splits > 16) splits = 16;
+    if (env_split > 0) splits = env_split;
+    if (splits > iters / 2) splits = iters / 2 > 0 ? iters / 2 : 1;
+    int ips = (iters + splits - 1) / splits;
+    splits = (iters + ips - 1) / ips;   // no empty split
+
+    // workspace: operands + row tables; partial tiles; arrival counters
+    const size_t ap_bytes = (size_t)rows_pad * kpad * 2;
+    const size_t meta_off = (ap_bytes + 255) / 256 * 256;
+    void *ws0 = nullptr, *ws1 = nullptr, *ws2 = nullptr;
+    int rc;
+    if ((rc = fnn_ctx_ensure_tmp(ctx, 0, meta_off + (size_t)m_pad * 12 + 256, &ws0))) return rc;
+    if (splits > 1 && (rc = fnn_ctx_ensure_tmp(ctx, 1, (size_t)splits * M * N * 4, &ws1))) return rc;
+    if ((rc = fnn_ctx_ensure_tmp(ctx, 2, (size_t)base * 4, &ws2))) return rc;
+
+    fnn_hip_weight *wm = const_cast<fnn_hip_weight *>(w);
+    const bool want_umean = !precise && (DT == FNN_DT_I8 || DT == FNN_DT_I4 || DT == FNN_DT_U8 || DT == FNN_DT_U4 || DT == FNN_DT_F4);
+    if (want_umean && !wm->umean) {
+        if (fnn_ctx_capturing(ctx)) return fnn_ctx_fail(ctx, FNN_ERR_MEMORY, "first single-pass use of a weight during graph capture");
+        if (hipMalloc((void **)&wm->umean, (size_t)w->rows * 4 + 64) != hipSuccess)
+            return fnn_ctx_fail(ctx, FNN_ERR_MEMORY, "out of device memory (row means)");
+        hipError_t e = launch_umean<DT>(w, wm->umean, s);
+        if (e != hipSuccess) return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, hipGetErrorString(e));
+    }
+
+    PrepArgs pa;
+    pa.a = q.a;
+    pa.ap = (_Float16 *)ws0;
+    pa.rexp = (int *)((char *)ws0 + meta_off);
+    pa.xsum = (float *)(pa.rexp + m_pad);
+    pa.esum = pa.xsum + m_pad;
+    pa.m = M; pa.k = K; pa.kpad = kpad;
+    pa.precise = precise ? 1 : 0;
+    pa.interleaved = DecH<DT>::INTERLEAVED ? 1 : 0;
+    hipLaunchKernelGGL(act_prep_kernel, dim3((unsigned)m_pad), dim3(256), 0, s, pa);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, hipGetErrorString(e));
+
+    TileArgs t;
+    t.words = q.words; t.scales = q.scales; t.zeros = q.zeros; t.umean = want_umean ? wm->umean : nullptr; t.bias = q.bias;
+    t.ap = pa.ap; t.rexp = pa.rexp; t.xsum = pa.xsum; t.esum = pa.esum;
+    t.out = q.out; t.part = (float *)ws1; t.counters = (unsigned *)ws2;
+    t.m = M; t.n = N; t.kp = q.kp; t.kpad = kpad;
+    t.act = q.act; t.splits = splits; t.iters = iters; t.ips = ips; t.mtiles = mtiles; t.ntiles = ntiles;
+    if (precise) {
+        if (cfg == 0) e = launch_tile<DT, 2, 2, 2, 2, true>(t, s);
+        else e = launch_tile<DT, 1, 4, 2, 1, true>(t, s);
+    } else {
+        if (cfg == 0) e = launch_tile<DT, 2, 2, 2, 2, false>(t, s);
+        else if (cfg == 1) e = launch_tile<DT, 1, 4, 2, 1, false>(t, s);
+        else e = launch_tile<DT, 1, 4, 1, 1, false>(t, s);
+    }
+    if (e != hipSuccess) return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, hipGetErrorString(e));
+    return FNN_OK;
+}
+
+}  // namespace
+
+int fnn_tiled_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &q, int flags, bool *handled)
+{
+    *handled = false;
+    static const int min_m = env_int("FNN_TILE_MIN_M", 65);
+    if (q.m < min_m) return FNN_OK;                             // few rows: the slab kernel is faster
+    if (w->dtype == FNN_DT_I4CB) return FNN_OK;                 // codebook type: other kernels
+    if (q.kp % 4 != 0) return FNN_OK;                           // 16-byte pieces of a weight row
+    if (reinterpret_cast<uintptr_t>(q.words) & 15) return FNN_OK;
+    if (q.m > (1 << 22) || q.n > (1 << 24)) return FNN_OK;      // 32-bit tile counts
+    int rc;
+    switch (w->dtype) {
+    case FNN_DT_I8: rc = run_tiled<FNN_DT_I8>(ctx, s, w, q, flags); break;
+    case FNN_DT_I4: rc = run_tiled<FNN_DT_I4>(ctx, s, w, q, flags); break;
+    case FNN_DT_U8: rc = run_tiled<FNN_DT_U8>(ctx, s, w, q, flags); break;
+    case FNN_DT_U4: rc = run_tiled<FNN_DT_U4>(ctx, s, w, q, flags); break;
+    case FNN_DT_F8: rc = run_tiled<FNN_DT_F8>(ctx, s, w, q, flags); break;
+    case FNN_DT_F8R: rc = run_tiled<FNN_DT_F8R>(ctx, s, w, q, flags); break;
+    case FNN_DT_F4: rc = run_tiled<FNN_DT_F4>(ctx, s, w, q, flags); break;
+    default: return FNN_OK;
+    }
+    if (rc) return rc;
+    *handled = true;
+    return FNN_OK;
+}
