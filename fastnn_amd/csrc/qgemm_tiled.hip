@@ -11,13 +11,16 @@
 //     so that hi + lo*2^-11 carries ~22 mantissa bits.  hi and lo rows sit in neighbouring
 //     32-row blocks and go through the same MFMAs as different operand rows.  Row sums
 //     (for the zero-point term) are accumulated in f32 in a fixed order.
-//  2. qgemm_tile_kernel: a workgroup of 4 waves owns a BM x BN output tile and a K range;
-//     the f16 activations are staged through LDS (double buffered), the packed weights go
-//     from HBM straight into registers in MFMA operand order (lane = weight row, 16 bytes
-//     of a row per load), are decoded to f16 there (integer lanes, E4M3/E5M2/E2M1 values
-//     are exact in f16) and multiplied with v_mfma_f32_32x32x16_f16.  With K split over
-//     several workgroups the partial tiles meet in a workspace and the last workgroup to
-//     arrive adds them in split order, so results do not depend on scheduling.
+//  2. qgemm_tile_kernel: a workgroup of 4 waves owns a BM x BN output tile and a K range.
+//     Both operands travel HBM -> LDS with global_load_lds_dwordx4 (no registers in between)
+//     through a ring of NS stages of 64 k-values, so several stages are in flight while one
+//     is consumed; 16-byte chunks are placed with an XOR swizzle that keeps the 128-bit LDS
+//     reads of the MFMA operands free of bank conflicts.  The packed weights are decoded to
+//     f16 in registers (integer lanes, E4M3/E5M2/E2M1 values are exact in f16) and multiplied
+//     with v_mfma_f32_32x32x16_f16.
+//  3. With K split over several workgroups (few activation rows: not enough tiles to fill
+//     the chip) the partial tiles go to a workspace and splitk_epilogue_kernel adds them in
+//     split order, so results do not depend on scheduling.
 //
 // FNN_FLAG_ACT_F16_SINGLE keeps hi only and removes the first-order effect of the rounding
 // on rows with a non-zero mean lane value: dot -= mean_k(u[n,k]) * sum_k (hi - x').
@@ -31,7 +34,6 @@ namespace {
 using namespace dech;
 
 constexpr int BK = 64;          // k-values per main-loop iteration
-constexpr int LDS_ROW = 144;    // bytes per activation row in LDS: 128 + 16 of padding (bank spread)
 constexpr float LO_UP = 2048.0f, LO_DOWN = 1.0f / 2048.0f;
 
 struct PrepArgs {
@@ -154,30 +156,45 @@ __global__ void __launch_bounds__(64) row_umean_kernel(const uint32_t *words, in
 
 struct TileArgs {
     const uint32_t *words;
+    const uint32_t *zero_chunk;   // 16 zero bytes: source of weight chunks past the end of a row
     const float *scales, *zeros, *umean, *bias;
     const _Float16 *ap;
     const int *rexp;
     const float *xsum, *esum;
     float *out, *part;
-    unsigned *counters;
     int64_t m, n, kp, kpad;
     int act, splits, iters, ips, mtiles, ntiles;
 };
 
-template <int DT, int WGM, int WGN, int TM, int TN, bool PRECISE>
+// HBM -> LDS without passing registers: lane i of the wave stores its 16 bytes at
+// LDS address m0 + 16*i.  The compiler does not see these loads: waits are placed by hand.
+__device__ __forceinline__ void load_to_lds16(const void *gptr, unsigned lds_wave_base)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_wave_base), "v"(gptr) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void wait_loads_but()
+{
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+template <int DT, int WGM, int WGN, int TM, int TN, bool PRECISE, int NS>
 __global__ void __launch_bounds__(256) qgemm_tile_kernel(TileArgs p)
 {
     using D = DecH<DT>;
     constexpr int WPS = D::WPS;          // words per 8 k-values
-    constexpr int WPL = 4 * WPS;         // words per lane, column block and iteration
+    constexpr int WC = 2 * WPS;          // 16-byte weight chunks per row and stage (32 or 64 bytes)
     constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
-    constexpr int ACH = BM * 8 / 256;    // 16-byte activation chunks per thread and iteration
+    constexpr int A_BYTES = BM * 128, W_BYTES = BN * WC * 16, STAGE = A_BYTES + W_BYTES;
+    constexpr int A_LPW = BM / 32;             // activation load instructions per wave and stage
+    constexpr int W_LPW = BN * WC / 256;       // weight load instructions per wave and stage
+    constexpr int LPS = A_LPW + W_LPW;
     static_assert(WGM * WGN == 4, "4 waves");
     static_assert(!PRECISE || TM % 2 == 0, "hi/lo block pairs stay in one wave");
-    static_assert(BM * 8 % 256 == 0, "whole chunks per thread");
+    static_assert(BN * WC % 256 == 0 && NS >= 2 && NS <= 8, "stage shape");
 
-    __shared__ __attribute__((aligned(16))) unsigned char a_lds[2][BM * LDS_ROW];
-    __shared__ unsigned arrival;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char *)smem;
 
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const int wm = wv / WGN, wn = wv % WGN;
@@ -199,19 +216,44 @@ __global__ void __launch_bounds__(256) qgemm_tile_kernel(TileArgs p)
     const int it0 = z * p.ips;
     const int it1 = (it0 + p.ips < p.iters) ? it0 + p.ips : p.iters;
 
-    // weight row pointers of this lane (clamped: lanes past N repeat the last row)
-    const uint32_t *wrow[TN];
+    // ---- what this lane fetches per stage.  LDS slot s of a region = 16-byte chunk s.
+    // activations: chunk (row, g) lives at slot row*8 + (g ^ (row & 7))
+    const _Float16 *a_src[A_LPW];
 #pragma unroll
-    for (int tn = 0; tn < TN; tn++) {
-        int64_t row = n0 + (wn * TN + tn) * 32 + lr;
-        if (row > p.n - 1) row = p.n - 1;
-        wrow[tn] = p.words + row * p.kp + h * WPL;
+    for (int j = 0; j < A_LPW; j++) {
+        const int slot = (wv * A_LPW + j) * 64 + lane;
+        const int row = slot >> 3, g = (slot & 7) ^ (row & 7);
+        a_src[j] = p.ap + ((int64_t)mt * BM + row) * p.kpad + g * 8;
     }
-    // activation chunks of this thread: chunk c = tid + 256*j -> row c/8, 16-byte column c%8
-    // (chunk j of a thread is 32 rows below chunk j-1)
-    const _Float16 *asrc = p.ap + ((int64_t)mt * BM + tid / 8) * p.kpad + (tid % 8) * 8;
-    const int64_t astep = 32 * p.kpad;
-    const int adst = (tid / 8) * LDS_ROW + (tid % 8) * 16;
+    // weights: chunk (row, c) lives at slot row*WC + (c ^ swz(row)); rows past N repeat the last row
+    const uint32_t *w_src[W_LPW];
+    int w_chunk[W_LPW];
+#pragma unroll
+    for (int j = 0; j < W_LPW; j++) {
+        const int slot = (wv * W_LPW + j) * 64 + lane;
+        const int row = slot / WC;
+        const int sw = (WC == 2) ? ((row >> 2) & 1) : ((row >> 1) & 3);
+        const int c = (slot % WC) ^ sw;
+        int64_t grow = n0 + row;
+        if (grow > p.n - 1) grow = p.n - 1;
+        w_src[j] = p.words + grow * p.kp + c * 4;
+        w_chunk[j] = c * 4;
+    }
+    const unsigned a_dst = __builtin_amdgcn_readfirstlane(lds0 + wv * A_LPW * 1024);
+    const unsigned w_dst = __builtin_amdgcn_readfirstlane(lds0 + A_BYTES + wv * W_LPW * 1024);
+
+    auto issue = [&](int it, int buf) {
+        const int itc = it < it1 ? it : it1 - 1;   // past the end: a harmless repeat keeps the load count fixed
+        const unsigned sb = buf * STAGE;
+#pragma unroll
+        for (int j = 0; j < W_LPW; j++) {
+            const int64_t wo = (int64_t)itc * (WC * 4);
+            const bool ok = wo + w_chunk[j] + 4 <= p.kp;
+            load_to_lds16(ok ? w_src[j] + wo : p.zero_chunk, w_dst + sb + j * 1024);
+        }
+#pragma unroll
+        for (int j = 0; j < A_LPW; j++) load_to_lds16(a_src[j] + (int64_t)itc * BK, a_dst + sb + j * 1024);
+    };
 
     f32x16 acc[TM][TN];
 #pragma unroll
@@ -221,115 +263,74 @@ __global__ void __launch_bounds__(256) qgemm_tile_kernel(TileArgs p)
 #pragma unroll
             for (int i = 0; i < 16; i++) acc[tm][tn][i] = 0.0f;
 
-    uint32_t wcur[TN][WPL], wnext[TN][WPL];
-    u32x4 areg[ACH];
-
-    auto load_w = [&](int it, uint32_t(&wq)[TN][WPL]) {
-        const int64_t off = (int64_t)it * (2 * WPL);   // words of the row before this iteration
+    // operand read offsets inside a stage
+    int a_off[TM], w_off[TN];
 #pragma unroll
-        for (int tn = 0; tn < TN; tn++)
+    for (int tm = 0; tm < TM; tm++) a_off[tm] = ((wm * TM + tm) * 32 + lr) * 128;
 #pragma unroll
-            for (int q = 0; q < WPL / 4; q++) {
-                const int64_t wo = off + h * WPL + q * 4;   // word index inside the row
-                const bool ok = wo + 4 <= p.kp;
-                const uint4 t = *reinterpret_cast<const uint4 *>(wrow[tn] + (ok ? off + q * 4 : 0));
-                const uint32_t msk = ok ? 0xffffffffu : 0u;
-                wq[tn][q * 4 + 0] = t.x & msk; wq[tn][q * 4 + 1] = t.y & msk;
-                wq[tn][q * 4 + 2] = t.z & msk; wq[tn][q * 4 + 3] = t.w & msk;
-            }
-    };
-#define FNN_LOAD_A(IT)                                                                                   \
-    _Pragma("unroll") for (int j = 0; j < ACH; j++)                                                      \
-        areg[j] = *reinterpret_cast<const u32x4 *>(asrc + j * astep + (int64_t)(IT) * BK)
-#define FNN_STORE_A(BUF)                                                                                 \
-    _Pragma("unroll") for (int j = 0; j < ACH; j++)                                                      \
-        *reinterpret_cast<u32x4 *>(&a_lds[BUF][adst + j * 32 * LDS_ROW]) = areg[j]
+    for (int tn = 0; tn < TN; tn++) {
+        const int row = (wn * TN + tn) * 32 + lr;
+        if constexpr (WC == 2) w_off[tn] = A_BYTES + (row * 2 + (h ^ ((row >> 2) & 1))) * 16;
+        else w_off[tn] = A_BYTES + row * 64;   // chunk index added per read
+    }
+    const int asw = lr & 7;   // row & 7 of every activation row this lane reads
 
     if (it0 < it1) {
-        load_w(it0, wcur);
-        FNN_LOAD_A(it0);
-        FNN_STORE_A(0);
+#pragma unroll
+        for (int st = 0; st < NS - 1; st++) issue(it0 + st, st);
+        int buf = 0;
+        for (int it = it0; it < it1; it++) {
+            wait_loads_but<(NS - 2) * LPS>();   // this wave's part of stage `buf` has landed
+            __syncthreads();                    // ... and everybody else's; stage buf-1 is free again
+            {
+                int nb = buf + NS - 1;
+                if (nb >= NS) nb -= NS;
+                issue(it + NS - 1, nb);
+            }
+            const unsigned char *sbase = smem + buf * STAGE;
+            uint32_t wq[TN][4 * WPS];
+#pragma unroll
+            for (int tn = 0; tn < TN; tn++) {
+                if constexpr (WC == 2) {
+                    const u32x4 t = *reinterpret_cast<const u32x4 *>(sbase + w_off[tn]);
+                    wq[tn][0] = t[0]; wq[tn][1] = t[1]; wq[tn][2] = t[2]; wq[tn][3] = t[3];
+                } else {
+                    const int row = (wn * TN + tn) * 32 + lr;
+                    const int sw = (row >> 1) & 3;
+                    const u32x4 t0 = *reinterpret_cast<const u32x4 *>(sbase + w_off[tn] + (((2 * h) ^ sw) * 16));
+                    const u32x4 t1 = *reinterpret_cast<const u32x4 *>(sbase + w_off[tn] + (((2 * h + 1) ^ sw) * 16));
+                    wq[tn][0] = t0[0]; wq[tn][1] = t0[1]; wq[tn][2] = t0[2]; wq[tn][3] = t0[3];
+                    wq[tn][4] = t1[0]; wq[tn][5] = t1[1]; wq[tn][6] = t1[2]; wq[tn][7] = t1[3];
+                }
+            }
+#pragma unroll
+            for (int s = 0; s < 4; s++) {
+                f16x8 af[TM], bf[TN];
+#pragma unroll
+                for (int tm = 0; tm < TM; tm++)
+                    af[tm] = *reinterpret_cast<const f16x8 *>(sbase + a_off[tm] + (((4 * h + s) ^ asw) * 16));
+#pragma unroll
+                for (int tn = 0; tn < TN; tn++) bf[tn] = D::step(&wq[tn][s * WPS]);
+#pragma unroll
+                for (int tm = 0; tm < TM; tm++)
+#pragma unroll
+                    for (int tn = 0; tn < TN; tn++)
+                        acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[tm], bf[tn], acc[tm][tn], 0, 0, 0);
+            }
+            buf = (buf + 1 == NS) ? 0 : buf + 1;
+        }
+        wait_loads_but<0>();   // nothing may still be writing LDS when the workgroup retires
     }
-    __syncthreads();
-    int buf = 0;
-    for (int it = it0; it < it1; it++) {
-        const bool more = it + 1 < it1;
-        if (more) {
-            load_w(it + 1, wnext);
-            FNN_LOAD_A(it + 1);
-        }
-        const unsigned char *abase = &a_lds[buf][(wm * TM * 32 + lr) * LDS_ROW + h * 64];
-#pragma unroll
-        for (int s = 0; s < 4; s++) {
-            f16x8 af[TM], bf[TN];
-#pragma unroll
-            for (int tm = 0; tm < TM; tm++)
-                af[tm] = *reinterpret_cast<const f16x8 *>(abase + tm * 32 * LDS_ROW + s * 16);
-#pragma unroll
-            for (int tn = 0; tn < TN; tn++) bf[tn] = D::step(&wcur[tn][s * WPS]);
-#pragma unroll
-            for (int tm = 0; tm < TM; tm++)
-#pragma unroll
-                for (int tn = 0; tn < TN; tn++)
-                    acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[tm], bf[tn], acc[tm][tn], 0, 0, 0);
-        }
-        if (more) { FNN_STORE_A(buf ^ 1); }
-        __syncthreads();
-        if (more) {
-#pragma unroll
-            for (int tn = 0; tn < TN; tn++)
-#pragma unroll
-                for (int q = 0; q < WPL; q++) wcur[tn][q] = wnext[tn][q];
-        }
-        buf ^= 1;
-    }
-
-#undef FNN_LOAD_A
-#undef FNN_STORE_A
 
     // ---- epilogue.  acc[i] of a 32x32 block: row (i/4)*8 + h*4 + i%4, column lr.
     constexpr int TMO = PRECISE ? TM / 2 : TM;       // output row blocks per wave
     const int64_t mrow0 = ((int64_t)mt * BM / (PRECISE ? 64 : 32) + wm * TMO) * 32;
-    auto row_of = [&](int to, int i) -> int64_t { return mrow0 + to * 32 + (i / 4) * 8 + h * 4 + (i % 4); };
-    auto col_of = [&](int tn) -> int64_t { return n0 + (wn * TN + tn) * 32 + lr; };
-    // this workgroup's share of sum_k A[m,k]*u(W[n,k]), scaled back to the row's magnitude
-    auto dot_of = [&](int to, int tn, int i, int e) -> float {
-        float v;
-        if constexpr (PRECISE) v = acc[2 * to][tn][i] + acc[2 * to + 1][tn][i] * LO_DOWN;
-        else v = acc[to][tn][i];
-        return ldexpf(v, -e);
-    };
-
-    const bool split = p.splits > 1;
-    if (split) {
-        // partial tiles: part[z][m][n]; the last workgroup of the tile to arrive adds them in z order
-#pragma unroll
-        for (int to = 0; to < TMO; to++)
-#pragma unroll
-            for (int i = 0; i < 16; i++) {
-                const int64_t m = row_of(to, i);
-                if (m >= p.m) continue;
-                const int e = p.rexp[m];
-#pragma unroll
-                for (int tn = 0; tn < TN; tn++) {
-                    const int64_t n = col_of(tn);
-                    if (n < p.n) p.part[((int64_t)z * p.m + m) * p.n + n] = dot_of(to, tn, i, e);
-                }
-            }
-        __threadfence();
-        __syncthreads();
-        if (tid == 0) arrival = atomicAdd(&p.counters[nt * p.mtiles + mt], 1u);
-        __syncthreads();
-        if (arrival != (unsigned)(p.splits - 1)) return;
-        __threadfence();
-        if (tid == 0) p.counters[nt * p.mtiles + mt] = 0;   // ready for the next launch
-    }
-
     float sc[TN], zp[TN], bi[TN], um[TN];
+    const bool split = p.splits > 1;
 #pragma unroll
     for (int tn = 0; tn < TN; tn++) {
-        const int64_t n = col_of(tn);
-        const bool ok = n < p.n;
+        const int64_t n = n0 + (wn * TN + tn) * 32 + lr;
+        const bool ok = n < p.n && !split;
         sc[tn] = ok ? p.scales[n] : 0.0f;
         zp[tn] = ok ? p.zeros[n] : 0.0f;
         bi[tn] = (ok && p.bias) ? p.bias[n] : 0.0f;
@@ -339,7 +340,7 @@ __global__ void __launch_bounds__(256) qgemm_tile_kernel(TileArgs p)
     for (int to = 0; to < TMO; to++)
 #pragma unroll
         for (int i = 0; i < 16; i++) {
-            const int64_t m = row_of(to, i);
+            const int64_t m = mrow0 + to * 32 + (i / 4) * 8 + h * 4 + (i % 4);
             if (m >= p.m) continue;
             const int e = p.rexp[m];
             const float xs = p.xsum[m];
@@ -347,22 +348,37 @@ __global__ void __launch_bounds__(256) qgemm_tile_kernel(TileArgs p)
             if constexpr (!PRECISE) corr = ldexpf(p.esum[m], -e);
 #pragma unroll
             for (int tn = 0; tn < TN; tn++) {
-                const int64_t n = col_of(tn);
+                const int64_t n = n0 + (wn * TN + tn) * 32 + lr;
                 if (n >= p.n) continue;
-                float d;
+                float v;
+                if constexpr (PRECISE) v = acc[2 * to][tn][i] + acc[2 * to + 1][tn][i] * LO_DOWN;
+                else v = acc[to][tn][i];
+                float d = ldexpf(v, -e);   // this workgroup's share of sum_k A[m,k]*u(W[n,k])
                 if (split) {
-                    d = 0.0f;
-                    for (int zz = 0; zz < p.splits; zz++)
-                        d += __builtin_nontemporal_load(&p.part[((int64_t)zz * p.m + m) * p.n + n]);
+                    p.part[((int64_t)z * p.m + m) * p.n + n] = d;
                 } else {
-                    d = dot_of(to, tn, i, e);
+                    if constexpr (!PRECISE) d = d - um[tn] * corr;
+                    float o = d * sc[tn] + zp[tn] * xs;
+                    if (p.bias) o = o + bi[tn];
+                    p.out[m * p.n + n] = fnn_activation(o, p.act);
                 }
-                if constexpr (!PRECISE) d = d - um[tn] * corr;
-                float v = d * sc[tn] + zp[tn] * xs;
-                if (p.bias) v = v + bi[tn];
-                p.out[m * p.n + n] = fnn_activation(v, p.act);
             }
         }
+}
+
+// sum of the K-split partial tiles in split order + affine / bias / activation epilogue
+__global__ void __launch_bounds__(256) splitk_epilogue_kernel(TileArgs p, int single)
+{
+    const int64_t total = p.m * p.n;
+    for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * 256) {
+        const int64_t m = idx / p.n, n = idx % p.n;
+        float d = 0.0f;
+        for (int zz = 0; zz < p.splits; zz++) d += p.part[(int64_t)zz * total + idx];
+        if (single && p.umean) d = d - p.umean[n] * ldexpf(p.esum[m], -p.rexp[m]);
+        float o = d * p.scales[n] + p.zeros[n] * p.xsum[m];
+        if (p.bias) o = o + p.bias[n];
+        p.out[idx] = fnn_activation(o, p.act);
+    }
 }
 
 int env_int(const char *name, int dflt)
@@ -371,11 +387,21 @@ int env_int(const char *name, int dflt)
     return s ? atoi(s) : dflt;
 }
 
-template <int DT, int WGM, int WGN, int TM, int TN, bool PRECISE>
+template <int DT, int WGM, int WGN, int TM, int TN, bool PRECISE, int NS>
 hipError_t launch_tile(const TileArgs &p, hipStream_t s)
 {
+    constexpr int WC = 2 * DecH<DT>::WPS;
+    constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
+    constexpr size_t lds = (size_t)NS * (BM * 128 + BN * WC * 16);
+    auto kern = qgemm_tile_kernel<DT, WGM, WGN, TM, TN, PRECISE, NS>;
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
     const unsigned total = (unsigned)p.mtiles * p.ntiles * p.splits;
-    hipLaunchKernelGGL((qgemm_tile_kernel<DT, WGM, WGN, TM, TN, PRECISE>), dim3(total), dim3(256), 0, s, p);
+    hipLaunchKernelGGL(kern, dim3(total), dim3(256), lds, s, p);
     return hipGetLastError();
 }
 
@@ -408,26 +434,25 @@ int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QM
     const int64_t rows_pad = (int64_t)mtiles * bm;
     const int64_t m_pad = precise ? rows_pad / 2 : rows_pad;
     const int iters = (int)(kpad / BK);
-    // split K until about two workgroups per CU are in flight
+    // few tiles: split K until about two workgroups per CU are in flight
     static const int env_split = env_int("FNN_TILE_SPLIT", 0);
-    static const int env_target = env_int("FNN_TILE_TARGET", 0);
+    static const int env_target = env_int("FNN_TILE_TARGET", 512);
     int splits = 1;
     const int base = mtiles * ntiles;
-    if (base < env_target) splits = (env_target + base - 1) / base;
-    if (splits > 16) splits = 16;
+    if (base < 256) splits = (env_target + base - 1) / base;
+    if (splits > 32) splits = 32;
     if (env_split > 0) splits = env_split;
-    if (splits > iters / 2) splits = iters / 2 > 0 ? iters / 2 : 1;
+    if (splits > iters / 4) splits = iters / 4 > 0 ? iters / 4 : 1;
     int ips = (iters + splits - 1) / splits;
     splits = (iters + ips - 1) / ips;   // no empty split
 
-    // workspace: operands + row tables; partial tiles; arrival counters
+    // workspace: operands + row tables; partial tiles
     const size_t ap_bytes = (size_t)rows_pad * kpad * 2;
     const size_t meta_off = (ap_bytes + 255) / 256 * 256;
-    void *ws0 = nullptr, *ws1 = nullptr, *ws2 = nullptr;
+    void *ws0 = nullptr, *ws1 = nullptr;
     int rc;
     if ((rc = fnn_ctx_ensure_tmp(ctx, 0, meta_off + (size_t)m_pad * 12 + 256, &ws0))) return rc;
     if (splits > 1 && (rc = fnn_ctx_ensure_tmp(ctx, 1, (size_t)splits * M * N * 4, &ws1))) return rc;
-    if ((rc = fnn_ctx_ensure_tmp(ctx, 2, (size_t)base * 4, &ws2))) return rc;
 
     fnn_hip_weight *wm = const_cast<fnn_hip_weight *>(w);
     const bool want_umean = !precise && (DT == FNN_DT_I8 || DT == FNN_DT_I4 || DT == FNN_DT_U8 || DT == FNN_DT_U4 || DT == FNN_DT_F4);
@@ -453,20 +478,29 @@ int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QM
     if (e != hipSuccess) return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, hipGetErrorString(e));
 
     TileArgs t;
-    t.words = q.words; t.scales = q.scales; t.zeros = q.zeros; t.umean = want_umean ? wm->umean : nullptr; t.bias = q.bias;
+    t.words = q.words;
+    t.zero_chunk = q.words + w->rows * w->kp;   // the zeroed margin behind the last row
+    t.scales = q.scales; t.zeros = q.zeros; t.umean = want_umean ? wm->umean : nullptr; t.bias = q.bias;
     t.ap = pa.ap; t.rexp = pa.rexp; t.xsum = pa.xsum; t.esum = pa.esum;
-    t.out = q.out; t.part = (float *)ws1; t.counters = (unsigned *)ws2;
+    t.out = q.out; t.part = (float *)ws1;
     t.m = M; t.n = N; t.kp = q.kp; t.kpad = kpad;
     t.act = q.act; t.splits = splits; t.iters = iters; t.ips = ips; t.mtiles = mtiles; t.ntiles = ntiles;
     if (precise) {
-        if (cfg == 0) e = launch_tile<DT, 2, 2, 2, 2, true>(t, s);
-        else e = launch_tile<DT, 1, 4, 2, 1, true>(t, s);
+        if (cfg == 0) e = launch_tile<DT, 2, 2, 2, 2, true, 3>(t, s);
+        else e = launch_tile<DT, 1, 4, 2, 1, true, 4>(t, s);
     } else {
-        if (cfg == 0) e = launch_tile<DT, 2, 2, 2, 2, false>(t, s);
-        else if (cfg == 1) e = launch_tile<DT, 1, 4, 2, 1, false>(t, s);
-        else e = launch_tile<DT, 1, 4, 1, 1, false>(t, s);
+        if (cfg == 0) e = launch_tile<DT, 2, 2, 2, 2, false, 3>(t, s);
+        else if (cfg == 1) e = launch_tile<DT, 1, 4, 2, 1, false, 4>(t, s);
+        else e = launch_tile<DT, 1, 4, 1, 1, false, 6>(t, s);
     }
     if (e != hipSuccess) return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, hipGetErrorString(e));
+    if (splits > 1) {
+        int64_t blocks = (M * N + 255) / 256;
+        if (blocks > 2048) blocks = 2048;
+        hipLaunchKernelGGL(splitk_epilogue_kernel, dim3((unsigned)blocks), dim3(256), 0, s, t, precise ? 0 : 1);
+        e = hipGetLastError();
+        if (e != hipSuccess) return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, hipGetErrorString(e));
+    }
     return FNN_OK;
 }
 
@@ -475,8 +509,8 @@ int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QM
 int fnn_tiled_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &q, int flags, bool *handled)
 {
     *handled = false;
-    static const int min_m = env_int("FNN_TILE_MIN_M", 65);
-    if (q.m < min_m) return FNN_OK;                             // few rows: the slab kernel is faster
+    static const int min_m = env_int("FNN_TILE_MIN_M", 5);
+    if (q.m < min_m) return FNN_OK;
     if (w->dtype == FNN_DT_I4CB) return FNN_OK;                 // codebook type: other kernels
     if (q.kp % 4 != 0) return FNN_OK;                           // 16-byte pieces of a weight row
     if (reinterpret_cast<uintptr_t>(q.words) & 15) return FNN_OK;
