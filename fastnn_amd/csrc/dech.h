@@ -23,18 +23,24 @@ struct DecH;
 
 // 1024 + v is exact in f16 for 0 <= v < 1024: OR-ing a small integer into the mantissa of
 // 0x6400 builds it without a convert; 1024 + 16 v likewise for the upper nibble of a byte.
+// (u & mask) ^ bits in one v_bitop3_b32 (truth table of (s0 & s1) ^ s2)
+__device__ __forceinline__ uint32_t and_xor(uint32_t u, uint32_t mask, uint32_t bits)
+{
+    return __builtin_amdgcn_bitop3_b32(u, mask, bits, 0x6A);
+}
 template <>
 struct DecH<FNN_DT_I4> {
     static constexpr int WPS = 1;
     static constexpr bool INTERLEAVED = true;  // operand order k = 0,4,1,5,2,6,3,7
     __device__ static __forceinline__ f16x8 step(const uint32_t *w)
     {
-        const uint32_t u = w[0] ^ 0x88888888u;  // nibble q -> q + 8
+        // nibble q -> q + 8 (flip its top bit) inside the mantissa of 1024.0: one logic op per pair
+        const uint32_t u = w[0];
         const uint32_t v = u >> 8;
-        f16x2 r0 = as_h2((u & 0x000F000Fu) | 0x64006400u) + h2(-1032.0f);
-        f16x2 r1 = __builtin_elementwise_fma(as_h2((u & 0x00F000F0u) | 0x64006400u), h2(0.0625f), h2(-72.0f));
-        f16x2 r2 = as_h2((v & 0x000F000Fu) | 0x64006400u) + h2(-1032.0f);
-        f16x2 r3 = __builtin_elementwise_fma(as_h2((v & 0x00F000F0u) | 0x64006400u), h2(0.0625f), h2(-72.0f));
+        f16x2 r0 = as_h2(and_xor(u, 0x000F000Fu, 0x64086408u)) + h2(-1032.0f);
+        f16x2 r1 = __builtin_elementwise_fma(as_h2(and_xor(u, 0x00F000F0u, 0x64806480u)), h2(0.0625f), h2(-72.0f));
+        f16x2 r2 = as_h2(and_xor(v, 0x000F000Fu, 0x64086408u)) + h2(-1032.0f);
+        f16x2 r3 = __builtin_elementwise_fma(as_h2(and_xor(v, 0x00F000F0u, 0x64806480u)), h2(0.0625f), h2(-72.0f));
         return pack8(as_u(r0), as_u(r1), as_u(r2), as_u(r3));
     }
 };
@@ -46,10 +52,10 @@ struct DecH<FNN_DT_U4> {
     {
         const uint32_t u = w[0];
         const uint32_t v = u >> 8;
-        f16x2 r0 = as_h2((u & 0x000F000Fu) | 0x64006400u) + h2(-1024.0f);
-        f16x2 r1 = __builtin_elementwise_fma(as_h2((u & 0x00F000F0u) | 0x64006400u), h2(0.0625f), h2(-64.0f));
-        f16x2 r2 = as_h2((v & 0x000F000Fu) | 0x64006400u) + h2(-1024.0f);
-        f16x2 r3 = __builtin_elementwise_fma(as_h2((v & 0x00F000F0u) | 0x64006400u), h2(0.0625f), h2(-64.0f));
+        f16x2 r0 = as_h2(and_xor(u, 0x000F000Fu, 0x64006400u)) + h2(-1024.0f);
+        f16x2 r1 = __builtin_elementwise_fma(as_h2(and_xor(u, 0x00F000F0u, 0x64006400u)), h2(0.0625f), h2(-64.0f));
+        f16x2 r2 = as_h2(and_xor(v, 0x000F000Fu, 0x64006400u)) + h2(-1024.0f);
+        f16x2 r3 = __builtin_elementwise_fma(as_h2(and_xor(v, 0x00F000F0u, 0x64006400u)), h2(0.0625f), h2(-64.0f));
         return pack8(as_u(r0), as_u(r1), as_u(r2), as_u(r3));
     }
 };

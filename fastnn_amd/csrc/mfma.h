@@ -1,4 +1,4 @@
-// MFMA GEMM entry points (matrix-core path for M >= 5 activation rows).
+// Matrix-core kernel entry points.
 #pragma once
 #include "common.h"
 #include "i8act.h"
@@ -13,13 +13,6 @@ bool fnn_ctx_capturing(fnn_hip_ctx *ctx);
 int fnn_tiled_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &p,
                       int flags, bool *handled);
 
-// f32 activations x packed weights on f16 MFMA tiles; *handled = false when the shape
-// is left to the generic kernel.
-int fnn_mfma_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &p,
-                     int flags, bool *handled);
 // M <= 4: bandwidth-bound GEMV on the matrix cores (weights requested before anything else).
 int fnn_mfma_qgemv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &p,
                    int flags, bool *handled);
-// I8 activations x I8/I4 weights on int8 MFMA tiles with i32 accumulators.
-int fnn_mfma_qmatmul_i8act(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w,
-                           const I8ActArgs &p, bool *handled);

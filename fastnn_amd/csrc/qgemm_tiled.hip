@@ -8,8 +8,8 @@
 //  1. act_prep_kernel turns the f32 activations into f16 MFMA operands once per call (not
 //     once per workgroup): each row is scaled by a power of two so that max|x| lands in
 //     [2^14, 2^15) and written as hi = f16(x') and, in the default mode, lo = f16((x'-hi)*2^11),
-//     so that hi + lo*2^-11 carries ~22 mantissa bits.  hi and lo rows sit in neighbouring
-//     32-row blocks and go through the same MFMAs as different operand rows.  Row sums
+//     so that hi + lo*2^-11 carries ~22 mantissa bits.  The 16 hi rows and the 16 lo rows of
+//     16 activation rows form one 32-row MFMA block: same MFMAs, different operand rows.  Row sums
 //     (for the zero-point term) are accumulated in f32 in a fixed order.
 //  2. qgemm_tile_kernel: a workgroup of 4 waves owns a BM x BN output tile and a K range.
 //     Both operands travel HBM -> LDS with global_load_lds_dwordx4 (no registers in between)
@@ -38,7 +38,8 @@ constexpr float LO_UP = 2048.0f, LO_DOWN = 1.0f / 2048.0f;
 
 struct PrepArgs {
     const float *a;
-    _Float16 *ap;     // [rows_pad][kpad]
+    _Float16 *ap;     // [kpad/64][rows_pad][64]: the rows of one 64-wide k block are contiguous
+    int64_t rows_pad;
     int *rexp;        // [m_pad] power-of-two exponent applied to the row
     float *xsum;      // [m_pad] sum_k A[m,k]
     float *esum;      // [m_pad] sum_k (hi - x') (single mode)
@@ -46,11 +47,11 @@ struct PrepArgs {
     int precise, interleaved;
 };
 
-// effective operand row of activation row m: blocks of 32 rows; hi blocks even, lo blocks odd
+// effective operand row of activation row m: a 32-row MFMA block holds 16 hi rows, then their 16 lo rows
 __device__ __host__ inline int64_t eff_row(int64_t m, int precise, int lo)
 {
     if (!precise) return m;
-    return (m / 32) * 64 + lo * 32 + m % 32;
+    return (m / 16) * 32 + lo * 16 + m % 16;
 }
 
 __global__ void __launch_bounds__(256) act_prep_kernel(PrepArgs p)
@@ -59,21 +60,46 @@ __global__ void __launch_bounds__(256) act_prep_kernel(PrepArgs p)
     const int64_t m = blockIdx.x;
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const int64_t K = p.k, ngroups = p.kpad / 8;
-    _Float16 *hi_row = p.ap + eff_row(m, p.precise, 0) * p.kpad;
-    _Float16 *lo_row = p.precise ? p.ap + eff_row(m, 1, 1) * p.kpad : nullptr;
+    // 16-byte group g of a row: k block g/8, position g%8 inside the block's 128-byte row
+    _Float16 *hi_row = p.ap + eff_row(m, p.precise, 0) * 64;
+    _Float16 *lo_row = p.precise ? p.ap + eff_row(m, 1, 1) * 64 : nullptr;
+    const int64_t kb_stride = p.rows_pad * 64;
+    auto group_at = [&](_Float16 *row, int64_t g) { return row + (g >> 3) * kb_stride + (g & 7) * 8; };
     if (m >= p.m) {  // padding rows of the last tile: zero operands
         const uint4 z = make_uint4(0, 0, 0, 0);
         for (int64_t g = tid; g < ngroups; g += 256) {
-            reinterpret_cast<uint4 *>(hi_row)[g] = z;
-            if (lo_row) reinterpret_cast<uint4 *>(lo_row)[g] = z;
+            *reinterpret_cast<uint4 *>(group_at(hi_row, g)) = z;
+            if (lo_row) *reinterpret_cast<uint4 *>(group_at(lo_row, g)) = z;
         }
         if (tid == 0) { p.rexp[m] = 0; p.xsum[m] = 0.0f; p.esum[m] = 0.0f; }
         return;
     }
     const float *x = p.a + m * K;
-    const bool vec = (K % 4 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0);
+    const bool vec = (K % 8 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0);
+    constexpr int RG = 4;                       // 8-value groups a thread can keep in registers
+    const bool in_regs = vec && ngroups <= 256 * RG && p.kpad == K;
+    float4 keep[RG][2];
     float mx = 0.0f, sum = 0.0f;
-    if (vec) {
+    if (in_regs) {
+        // one trip to memory: the row stays in registers between the statistics and the conversion
+#pragma unroll
+        for (int r = 0; r < RG; r++) {
+            const int64_t g = tid + 256 * r;
+            keep[r][0] = keep[r][1] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (g < ngroups) {
+                keep[r][0] = *reinterpret_cast<const float4 *>(x + g * 8);
+                keep[r][1] = *reinterpret_cast<const float4 *>(x + g * 8 + 4);
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < RG; r++)
+#pragma unroll
+            for (int q = 0; q < 2; q++) {
+                const float4 v = keep[r][q];
+                mx = fmaxf(mx, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+                sum += (v.x + v.y) + (v.z + v.w);
+            }
+    } else if (vec) {
         for (int64_t i = tid; i < K / 4; i += 256) {
             const float4 v = reinterpret_cast<const float4 *>(x)[i];
             mx = fmaxf(mx, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
@@ -98,18 +124,7 @@ __global__ void __launch_bounds__(256) act_prep_kernel(PrepArgs p)
         e = 15 - ex;            // mx * 2^e in [2^14, 2^15)
     }
     float err = 0.0f;
-    for (int64_t g = tid; g < ngroups; g += 256) {
-        float v[8];
-        const int64_t k0 = g * 8;
-        if (vec && k0 + 8 <= K) {
-            const float4 a0 = *reinterpret_cast<const float4 *>(x + k0);
-            const float4 a1 = *reinterpret_cast<const float4 *>(x + k0 + 4);
-            v[0] = a0.x; v[1] = a0.y; v[2] = a0.z; v[3] = a0.w;
-            v[4] = a1.x; v[5] = a1.y; v[6] = a1.z; v[7] = a1.w;
-        } else {
-#pragma unroll
-            for (int j = 0; j < 8; j++) v[j] = (k0 + j < K) ? x[k0 + j] : 0.0f;
-        }
+    auto convert = [&](int64_t g, const float(&v)[8]) {
         f16x8 h, l;
 #pragma unroll
         for (int j = 0; j < 8; j++) {
@@ -122,8 +137,34 @@ __global__ void __launch_bounds__(256) act_prep_kernel(PrepArgs p)
             l[j] = (_Float16)(r * LO_UP);
             err -= r;
         }
-        *reinterpret_cast<f16x8 *>(hi_row + k0) = h;
-        if (lo_row) *reinterpret_cast<f16x8 *>(lo_row + k0) = l;
+        *reinterpret_cast<f16x8 *>(group_at(hi_row, g)) = h;
+        if (lo_row) *reinterpret_cast<f16x8 *>(group_at(lo_row, g)) = l;
+    };
+    if (in_regs) {
+#pragma unroll
+        for (int r = 0; r < RG; r++) {
+            const int64_t g = tid + 256 * r;
+            if (g < ngroups) {
+                const float v[8] = {keep[r][0].x, keep[r][0].y, keep[r][0].z, keep[r][0].w,
+                                    keep[r][1].x, keep[r][1].y, keep[r][1].z, keep[r][1].w};
+                convert(g, v);
+            }
+        }
+    } else {
+        for (int64_t g = tid; g < ngroups; g += 256) {
+            float v[8];
+            const int64_t k0 = g * 8;
+            if (vec && k0 + 8 <= K) {
+                const float4 a0 = *reinterpret_cast<const float4 *>(x + k0);
+                const float4 a1 = *reinterpret_cast<const float4 *>(x + k0 + 4);
+                v[0] = a0.x; v[1] = a0.y; v[2] = a0.z; v[3] = a0.w;
+                v[4] = a1.x; v[5] = a1.y; v[6] = a1.z; v[7] = a1.w;
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; j++) v[j] = (k0 + j < K) ? x[k0 + j] : 0.0f;
+            }
+            convert(g, v);
+        }
     }
     err = wave_sum(err);
     if (lane == 0) red[2][wv] = err;
@@ -162,7 +203,7 @@ struct TileArgs {
     const int *rexp;
     const float *xsum, *esum;
     float *out, *part;
-    int64_t m, n, kp, kpad;
+    int64_t m, n, kp, kpad, rows_pad;
     int act, splits, iters, ips, mtiles, ntiles;
 };
 
@@ -190,8 +231,7 @@ __global__ void __launch_bounds__(256) qgemm_tile_kernel(TileArgs p)
     constexpr int W_LPW = BN * WC / 256;       // weight load instructions per wave and stage
     constexpr int LPS = A_LPW + W_LPW;
     static_assert(WGM * WGN == 4, "4 waves");
-    static_assert(!PRECISE || TM % 2 == 0, "hi/lo block pairs stay in one wave");
-    static_assert(BN * WC % 256 == 0 && NS >= 2 && NS <= 8, "stage shape");
+    static_assert(BN * WC % 256 == 0 && NS >= 3 && NS <= 8, "stage shape");
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char *)smem;
@@ -200,14 +240,10 @@ __global__ void __launch_bounds__(256) qgemm_tile_kernel(TileArgs p)
     const int wm = wv / WGN, wn = wv % WGN;
     const int lr = lane & 31, h = lane >> 5;
 
-    // workgroup id -> tile: ids that share a weight column tile land on the same XCD (ids
-    // are dealt round-robin over the 8 XCDs, each with its own L2)
-    const unsigned total = gridDim.x;
-    unsigned L = blockIdx.x;
-    {
-        const unsigned xcd = L & 7, slot = L >> 3, q = total >> 3, r = total & 7;
-        L = xcd * q + (xcd < r ? xcd : r) + slot;
-    }
+    // workgroup id -> tile, row tile fastest.  Ids are dealt round-robin over the 8 XCDs (each with
+    // its own L2), so an XCD keeps meeting the same few row tiles of the activations, the operand
+    // with the most bytes per MAC, while the packed weights stream through.
+    const unsigned L = blockIdx.x;
     const int mt = L % p.mtiles;
     const unsigned rest = L / p.mtiles;
     const int z = rest % p.splits;
@@ -217,13 +253,15 @@ __global__ void __launch_bounds__(256) qgemm_tile_kernel(TileArgs p)
     const int it1 = (it0 + p.ips < p.iters) ? it0 + p.ips : p.iters;
 
     // ---- what this lane fetches per stage.  LDS slot s of a region = 16-byte chunk s.
-    // activations: chunk (row, g) lives at slot row*8 + (g ^ (row & 7))
+    // The LDS has 64 banks of 4 bytes: a 128-bit read is conflict-free when every 16 lanes cover
+    // all sixteen 16-byte slots of a 256-byte window, hence the row-dependent XOR of the chunk index.
+    // activations: chunk (row, g) lives at slot row*8 + (g ^ ((row >> 1) & 7))
     const _Float16 *a_src[A_LPW];
 #pragma unroll
     for (int j = 0; j < A_LPW; j++) {
         const int slot = (wv * A_LPW + j) * 64 + lane;
-        const int row = slot >> 3, g = (slot & 7) ^ (row & 7);
-        a_src[j] = p.ap + ((int64_t)mt * BM + row) * p.kpad + g * 8;
+        const int row = slot >> 3, g = (slot & 7) ^ ((row >> 1) & 7);
+        a_src[j] = p.ap + ((int64_t)mt * BM + row) * 64 + g * 8;
     }
     // weights: chunk (row, c) lives at slot row*WC + (c ^ swz(row)); rows past N repeat the last row
     const uint32_t *w_src[W_LPW];
@@ -232,27 +270,45 @@ __global__ void __launch_bounds__(256) qgemm_tile_kernel(TileArgs p)
     for (int j = 0; j < W_LPW; j++) {
         const int slot = (wv * W_LPW + j) * 64 + lane;
         const int row = slot / WC;
-        const int sw = (WC == 2) ? ((row >> 2) & 1) : ((row >> 1) & 3);
+        const int sw = (WC == 2) ? ((row >> 3) & 1) : ((row >> 2) & 3);
         const int c = (slot % WC) ^ sw;
         int64_t grow = n0 + row;
         if (grow > p.n - 1) grow = p.n - 1;
         w_src[j] = p.words + grow * p.kp + c * 4;
         w_chunk[j] = c * 4;
     }
+    const int64_t a_step = p.rows_pad * 64;   // elements between consecutive k blocks
     const unsigned a_dst = __builtin_amdgcn_readfirstlane(lds0 + wv * A_LPW * 1024);
     const unsigned w_dst = __builtin_amdgcn_readfirstlane(lds0 + A_BYTES + wv * W_LPW * 1024);
 
-    auto issue = [&](int it, int buf) {
-        const int itc = it < it1 ? it : it1 - 1;   // past the end: a harmless repeat keeps the load count fixed
-        const unsigned sb = buf * STAGE;
+    // running source pointers: advanced after every stage, frozen once the K range is exhausted
+    // (the extra requests of the last iterations re-read the final stage and are never consumed)
 #pragma unroll
-        for (int j = 0; j < W_LPW; j++) {
-            const int64_t wo = (int64_t)itc * (WC * 4);
-            const bool ok = wo + w_chunk[j] + 4 <= p.kp;
-            load_to_lds16(ok ? w_src[j] + wo : p.zero_chunk, w_dst + sb + j * 1024);
+    for (int j = 0; j < A_LPW; j++) a_src[j] += (int64_t)it0 * a_step;
+#pragma unroll
+    for (int j = 0; j < W_LPW; j++) w_src[j] += (int64_t)it0 * (WC * 4);
+    const bool ragged = (p.kp % (WC * 4)) != 0;   // the last stage of a row is partly past its end
+    auto issue = [&](int it, int buf) {
+        const unsigned sb = buf * STAGE;
+        if (ragged && it >= p.iters - 1) {
+#pragma unroll
+            for (int j = 0; j < W_LPW; j++) {
+                const bool ok = (int64_t)(p.iters - 1) * (WC * 4) + w_chunk[j] + 4 <= p.kp;
+                load_to_lds16(ok ? w_src[j] : p.zero_chunk, w_dst + sb + j * 1024);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < W_LPW; j++) load_to_lds16(w_src[j], w_dst + sb + j * 1024);
         }
 #pragma unroll
-        for (int j = 0; j < A_LPW; j++) load_to_lds16(a_src[j] + (int64_t)itc * BK, a_dst + sb + j * 1024);
+        for (int j = 0; j < A_LPW; j++) load_to_lds16(a_src[j], a_dst + sb + j * 1024);
+        const bool more = it + 1 < it1;           // wave-uniform
+        const int64_t astep = more ? a_step : 0;
+        const int wstep = more ? WC * 4 : 0;
+#pragma unroll
+        for (int j = 0; j < A_LPW; j++) a_src[j] += astep;
+#pragma unroll
+        for (int j = 0; j < W_LPW; j++) w_src[j] += wstep;
     };
 
     f32x16 acc[TM][TN];
@@ -270,25 +326,19 @@ __global__ void __launch_bounds__(256) qgemm_tile_kernel(TileArgs p)
 #pragma unroll
     for (int tn = 0; tn < TN; tn++) {
         const int row = (wn * TN + tn) * 32 + lr;
-        if constexpr (WC == 2) w_off[tn] = A_BYTES + (row * 2 + (h ^ ((row >> 2) & 1))) * 16;
+        if constexpr (WC == 2) w_off[tn] = A_BYTES + (row * 2 + (h ^ ((row >> 3) & 1))) * 16;
         else w_off[tn] = A_BYTES + row * 64;   // chunk index added per read
     }
-    const int asw = lr & 7;   // row & 7 of every activation row this lane reads
+    const int asw = (lr >> 1) & 7;   // (row >> 1) & 7 of every activation row this lane reads
 
     if (it0 < it1) {
-#pragma unroll
-        for (int st = 0; st < NS - 1; st++) issue(it0 + st, st);
-        int buf = 0;
-        for (int it = it0; it < it1; it++) {
-            wait_loads_but<(NS - 2) * LPS>();   // this wave's part of stage `buf` has landed
-            __syncthreads();                    // ... and everybody else's; stage buf-1 is free again
-            {
-                int nb = buf + NS - 1;
-                if (nb >= NS) nb -= NS;
-                issue(it + NS - 1, nb);
-            }
-            const unsigned char *sbase = smem + buf * STAGE;
-            uint32_t wq[TN][4 * WPS];
+        // ---- main loop: a flat software pipeline over the MFMA steps (4 per stage).
+        //  - activation fragments are requested from LDS two steps ahead (ring of 4 register sets),
+        //  - weight words are decoded one step ahead,
+        //  - the stage hand-over (wait for the next stage, barrier, request of a further stage)
+        //    sits between steps 1 and 2; steps 2 and 3 already read the next stage's operands,
+        // so the matrix cores never wait for a whole LDS round trip.
+        auto read_w = [&](const unsigned char *sbase, uint32_t(&wq)[TN][4 * WPS]) {
 #pragma unroll
             for (int tn = 0; tn < TN; tn++) {
                 if constexpr (WC == 2) {
@@ -296,35 +346,90 @@ __global__ void __launch_bounds__(256) qgemm_tile_kernel(TileArgs p)
                     wq[tn][0] = t[0]; wq[tn][1] = t[1]; wq[tn][2] = t[2]; wq[tn][3] = t[3];
                 } else {
                     const int row = (wn * TN + tn) * 32 + lr;
-                    const int sw = (row >> 1) & 3;
+                    const int sw = (row >> 2) & 3;
                     const u32x4 t0 = *reinterpret_cast<const u32x4 *>(sbase + w_off[tn] + (((2 * h) ^ sw) * 16));
                     const u32x4 t1 = *reinterpret_cast<const u32x4 *>(sbase + w_off[tn] + (((2 * h + 1) ^ sw) * 16));
                     wq[tn][0] = t0[0]; wq[tn][1] = t0[1]; wq[tn][2] = t0[2]; wq[tn][3] = t0[3];
                     wq[tn][4] = t1[0]; wq[tn][5] = t1[1]; wq[tn][6] = t1[2]; wq[tn][7] = t1[3];
                 }
             }
+        };
+        auto read_a = [&](const unsigned char *sbase, int s, f16x8(&af)[TM]) {
 #pragma unroll
-            for (int s = 0; s < 4; s++) {
-                f16x8 af[TM], bf[TN];
+            for (int tm = 0; tm < TM; tm++)
+                af[tm] = *reinterpret_cast<const f16x8 *>(sbase + a_off[tm] + (((4 * h + s) ^ asw) * 16));
+        };
+        auto decode = [&](const uint32_t(&wq)[TN][4 * WPS], int s, f16x8(&bf)[TN]) {
 #pragma unroll
-                for (int tm = 0; tm < TM; tm++)
-                    af[tm] = *reinterpret_cast<const f16x8 *>(sbase + a_off[tm] + (((4 * h + s) ^ asw) * 16));
+            for (int tn = 0; tn < TN; tn++) bf[tn] = D::step(&wq[tn][s * WPS]);
+        };
+        auto mfmas = [&](const f16x8(&af)[TM], const f16x8(&bf)[TN]) {
 #pragma unroll
-                for (int tn = 0; tn < TN; tn++) bf[tn] = D::step(&wq[tn][s * WPS]);
+            for (int tm = 0; tm < TM; tm++)
 #pragma unroll
-                for (int tm = 0; tm < TM; tm++)
+                for (int tn = 0; tn < TN; tn++)
+                    acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[tm], bf[tn], acc[tm][tn], 0, 0, 0);
+        };
+
 #pragma unroll
-                    for (int tn = 0; tn < TN; tn++)
-                        acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[tm], bf[tn], acc[tm][tn], 0, 0, 0);
+        for (int st = 0; st < NS - 1; st++) issue(it0 + st, st);
+        uint32_t wq[TN][4 * WPS], wqn[TN][4 * WPS];
+        f16x8 af[4][TM], bfr[2][TN];
+        wait_loads_but<(NS - 2) * LPS>();   // first stage: this wave's part has landed
+        __syncthreads();                    // ... and everybody else's
+        read_w(smem, wq);
+        read_a(smem, 0, af[0]);
+        read_a(smem, 1, af[1]);
+        decode(wq, 0, bfr[0]);
+        int buf = 0;
+        for (int it = it0; it < it1; it++) {
+            const unsigned char *sbase = smem + buf * STAGE;
+            const int nbuf = (buf + 1 == NS) ? 0 : buf + 1;
+            const unsigned char *nbase = smem + nbuf * STAGE;
+            const bool more = it + 1 < it1;
+            // step 0
+            read_a(sbase, 2, af[2]);
+            decode(wq, 1, bfr[1]);
+            mfmas(af[0], bfr[0]);
+            // step 1
+            read_a(sbase, 3, af[3]);
+            decode(wq, 2, bfr[0]);
+            mfmas(af[1], bfr[1]);
+            // hand-over
+            if (more) {
+                wait_loads_but<(NS - 3) * LPS>();   // this wave's part of the next stage has landed
+                __syncthreads();                    // everybody's; the stage before the current one is free
+                int fb = buf + NS - 1;
+                if (fb >= NS) fb -= NS;
+                issue(it + NS - 1, fb);
+                // step 2, with the first reads of the next stage
+                read_w(nbase, wqn);
+                read_a(nbase, 0, af[0]);
             }
-            buf = (buf + 1 == NS) ? 0 : buf + 1;
+            decode(wq, 3, bfr[1]);
+            mfmas(af[2], bfr[0]);
+            // step 3
+            if (more) {
+                read_a(nbase, 1, af[1]);
+                decode(wqn, 0, bfr[0]);
+            }
+            mfmas(af[3], bfr[1]);
+#pragma unroll
+            for (int tn = 0; tn < TN; tn++)
+#pragma unroll
+                for (int q = 0; q < 4 * WPS; q++) wq[tn][q] = wqn[tn][q];
+            buf = nbuf;
         }
         wait_loads_but<0>();   // nothing may still be writing LDS when the workgroup retires
     }
 
-    // ---- epilogue.  acc[i] of a 32x32 block: row (i/4)*8 + h*4 + i%4, column lr.
-    constexpr int TMO = PRECISE ? TM / 2 : TM;       // output row blocks per wave
-    const int64_t mrow0 = ((int64_t)mt * BM / (PRECISE ? 64 : 32) + wm * TMO) * 32;
+
+
+    // ---- epilogue.  acc[i] of a 32x32 block: row (i/4)*8 + h*4 + i%4, column lr.  With hi/lo
+    // operands a block holds 16 output rows: hi in rows 0..15 (i < 8), lo in rows 16..31 (i + 8).
+    constexpr int RPB = PRECISE ? 16 : 32;           // output rows per block
+    constexpr int NI = PRECISE ? 8 : 16;
+    const int64_t mrow0 = ((int64_t)mt * (BM / 32) + wm * TM) * RPB;
     float sc[TN], zp[TN], bi[TN], um[TN];
     const bool split = p.splits > 1;
 #pragma unroll
@@ -337,10 +442,10 @@ __global__ void __launch_bounds__(256) qgemm_tile_kernel(TileArgs p)
         um[tn] = (!PRECISE && ok && p.umean) ? p.umean[n] : 0.0f;
     }
 #pragma unroll
-    for (int to = 0; to < TMO; to++)
+    for (int tm = 0; tm < TM; tm++)
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-            const int64_t m = mrow0 + to * 32 + (i / 4) * 8 + h * 4 + (i % 4);
+        for (int i = 0; i < NI; i++) {
+            const int64_t m = mrow0 + tm * RPB + (i / 4) * 8 + h * 4 + (i % 4);
             if (m >= p.m) continue;
             const int e = p.rexp[m];
             const float xs = p.xsum[m];
@@ -351,8 +456,8 @@ __global__ void __launch_bounds__(256) qgemm_tile_kernel(TileArgs p)
                 const int64_t n = n0 + (wn * TN + tn) * 32 + lr;
                 if (n >= p.n) continue;
                 float v;
-                if constexpr (PRECISE) v = acc[2 * to][tn][i] + acc[2 * to + 1][tn][i] * LO_DOWN;
-                else v = acc[to][tn][i];
+                if constexpr (PRECISE) v = acc[tm][tn][i] + acc[tm][tn][i + 8] * LO_DOWN;
+                else v = acc[tm][tn][i];
                 float d = ldexpf(v, -e);   // this workgroup's share of sum_k A[m,k]*u(W[n,k])
                 if (split) {
                     p.part[((int64_t)z * p.m + m) * p.n + n] = d;
@@ -418,15 +523,15 @@ int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QM
     const bool precise = !(flags & FNN_FLAG_ACT_F16_SINGLE);
     const int64_t M = q.m, N = q.n, K = q.k;
     const int64_t kpad = (K + BK - 1) / BK * BK;
-    const int64_t mp32 = (M + 31) / 32 * 32;
-    const int64_t meff = precise ? 2 * mp32 : mp32;
+    const int64_t meff = precise ? (M + 15) / 16 * 32 : (M + 31) / 32 * 32;
     // tile shape by effective row count
-    int cfg;            // 0: 128x128 (2x2 waves of 64x64), 1: 64x128 (1x4 waves of 64x32), 2: 32x128 (1x4 waves of 32x32)
+    // 0: 128x128 (2x2 waves of 64x64), 1: 64x128 (4 waves of 64x32), 2: 32x128 (4 waves of 32x32)
+    int cfg;
     if (meff > 64) cfg = 0;
     else if (meff == 64) cfg = 1;
     else cfg = 2;
     static const int env_cfg = env_int("FNN_TILE_CFG", -1);
-    if (env_cfg >= 0 && env_cfg <= 2 && !(env_cfg == 2 && precise)) cfg = env_cfg;
+    if (env_cfg >= 0 && env_cfg <= 2) cfg = env_cfg;
     const int bm = cfg == 0 ? 128 : (cfg == 1 ? 64 : 32);
     const int bn = 128;
     const int mtiles = (int)((meff + bm - 1) / bm);
@@ -470,7 +575,7 @@ int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QM
     pa.rexp = (int *)((char *)ws0 + meta_off);
     pa.xsum = (float *)(pa.rexp + m_pad);
     pa.esum = pa.xsum + m_pad;
-    pa.m = M; pa.k = K; pa.kpad = kpad;
+    pa.m = M; pa.k = K; pa.kpad = kpad; pa.rows_pad = rows_pad;
     pa.precise = precise ? 1 : 0;
     pa.interleaved = DecH<DT>::INTERLEAVED ? 1 : 0;
     hipLaunchKernelGGL(act_prep_kernel, dim3((unsigned)m_pad), dim3(256), 0, s, pa);
@@ -483,11 +588,12 @@ int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QM
     t.scales = q.scales; t.zeros = q.zeros; t.umean = want_umean ? wm->umean : nullptr; t.bias = q.bias;
     t.ap = pa.ap; t.rexp = pa.rexp; t.xsum = pa.xsum; t.esum = pa.esum;
     t.out = q.out; t.part = (float *)ws1;
-    t.m = M; t.n = N; t.kp = q.kp; t.kpad = kpad;
+    t.m = M; t.n = N; t.kp = q.kp; t.kpad = kpad; t.rows_pad = rows_pad;
     t.act = q.act; t.splits = splits; t.iters = iters; t.ips = ips; t.mtiles = mtiles; t.ntiles = ntiles;
     if (precise) {
         if (cfg == 0) e = launch_tile<DT, 2, 2, 2, 2, true, 3>(t, s);
-        else e = launch_tile<DT, 1, 4, 2, 1, true, 4>(t, s);
+        else if (cfg == 1) e = launch_tile<DT, 1, 4, 2, 1, true, 4>(t, s);
+        else e = launch_tile<DT, 1, 4, 1, 1, true, 6>(t, s);
     } else {
         if (cfg == 0) e = launch_tile<DT, 2, 2, 2, 2, false, 3>(t, s);
         else if (cfg == 1) e = launch_tile<DT, 1, 4, 2, 1, false, 4>(t, s);
