@@ -38,7 +38,7 @@ struct fnn_hip_ctx {
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     std::string err;
     std::unordered_map<uint64_t, fnn_hip_weight *> weights;
-    Staging st_a, st_out, st_bias, st_acc, st_tmp, st_tmp2, st_cnt;
+    Staging st_a, st_out, st_bias, st_acc, st_tmp, st_tmp2, st_tmp3, st_cnt;
     float *scratch = nullptr;  // small reduction scratch (partials)
     bool capturing = false;
 };
@@ -162,7 +162,7 @@ void fnn_hip_destroy(fnn_hip_ctx *ctx)
     (void)hipSetDevice(ctx->device);
     if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
     for (auto &kv : ctx->weights) free_weight(kv.second);
-    for (Staging *s : {&ctx->st_a, &ctx->st_out, &ctx->st_bias, &ctx->st_acc, &ctx->st_tmp, &ctx->st_tmp2, &ctx->st_cnt})
+    for (Staging *s : {&ctx->st_a, &ctx->st_out, &ctx->st_bias, &ctx->st_acc, &ctx->st_tmp, &ctx->st_tmp2, &ctx->st_tmp3, &ctx->st_cnt})
         if (s->ptr) (void)hipFree(s->ptr);
     if (ctx->scratch) (void)hipFree(ctx->scratch);
     if (ctx->ev0) (void)hipEventDestroy(ctx->ev0);
@@ -678,7 +678,7 @@ int fnn_hip_graph_destroy(fnn_hip_ctx *ctx, fnn_hip_graph *g)
 // staging access for the MFMA translation unit
 int fnn_ctx_ensure_tmp(fnn_hip_ctx *ctx, int which, size_t bytes, void **ptr)
 {
-    Staging &s = which == 0 ? ctx->st_tmp : (which == 1 ? ctx->st_tmp2 : ctx->st_cnt);
+    Staging &s = which == 0 ? ctx->st_tmp : (which == 1 ? ctx->st_tmp2 : (which == 2 ? ctx->st_cnt : ctx->st_tmp3));
     const void *before = s.ptr;
     int rc = ensure(ctx, s, bytes);
     if (rc) return rc;

@@ -33,6 +33,18 @@ namespace {
 
 using namespace dech;
 
+// internal operand type: weights already expanded to f16 (8 k-values = 4 words), no decode
+constexpr int DT_F16_DENSE = 64;
+}  // namespace
+namespace dech {
+template <>
+struct DecH<64> {
+    static constexpr int WPS = 4;
+    static constexpr bool INTERLEAVED = false;
+    __device__ static __forceinline__ f16x8 step(const uint32_t *w) { return pack8(w[0], w[1], w[2], w[3]); }
+};
+}  // namespace dech
+namespace {
 constexpr int BK = 64;          // k-values per main-loop iteration
 constexpr float LO_UP = 2048.0f, LO_DOWN = 1.0f / 2048.0f;
 
@@ -205,6 +217,7 @@ struct TileArgs {
     float *out, *part;
     int64_t m, n, kp, kpad, rows_pad;
     int act, splits, iters, ips, mtiles, ntiles;
+    int a_wrap;   // > 0: the activation operand has a_wrap k blocks and is swept again after them (weights = [hi | lo])
 };
 
 // HBM -> LDS without passing registers: lane i of the wave stores its 16 bytes at
@@ -224,7 +237,7 @@ __global__ void __launch_bounds__(256) qgemm_tile_kernel(TileArgs p)
 {
     using D = DecH<DT>;
     constexpr int WPS = D::WPS;          // words per 8 k-values
-    constexpr int WC = 2 * WPS;          // 16-byte weight chunks per row and stage (32 or 64 bytes)
+    constexpr int WC = 2 * WPS;          // 16-byte weight chunks per row and stage (32, 64 or 128 bytes)
     constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
     constexpr int A_BYTES = BM * 128, W_BYTES = BN * WC * 16, STAGE = A_BYTES + W_BYTES;
     constexpr int A_LPW = BM / 32;             // activation load instructions per wave and stage
@@ -270,7 +283,7 @@ __global__ void __launch_bounds__(256) qgemm_tile_kernel(TileArgs p)
     for (int j = 0; j < W_LPW; j++) {
         const int slot = (wv * W_LPW + j) * 64 + lane;
         const int row = slot / WC;
-        const int sw = (WC == 2) ? ((row >> 3) & 1) : ((row >> 2) & 3);
+        const int sw = (WC == 2) ? ((row >> 3) & 1) : (WC == 4 ? ((row >> 2) & 3) : ((row >> 1) & 7));
         const int c = (slot % WC) ^ sw;
         int64_t grow = n0 + row;
         if (grow > p.n - 1) grow = p.n - 1;
@@ -284,7 +297,7 @@ __global__ void __launch_bounds__(256) qgemm_tile_kernel(TileArgs p)
     // running source pointers: advanced after every stage, frozen once the K range is exhausted
     // (the extra requests of the last iterations re-read the final stage and are never consumed)
 #pragma unroll
-    for (int j = 0; j < A_LPW; j++) a_src[j] += (int64_t)it0 * a_step;
+    for (int j = 0; j < A_LPW; j++) a_src[j] += (int64_t)(p.a_wrap ? it0 % p.a_wrap : it0) * a_step;
 #pragma unroll
     for (int j = 0; j < W_LPW; j++) w_src[j] += (int64_t)it0 * (WC * 4);
     const bool ragged = (p.kp % (WC * 4)) != 0;   // the last stage of a row is partly past its end
@@ -303,7 +316,8 @@ __global__ void __launch_bounds__(256) qgemm_tile_kernel(TileArgs p)
 #pragma unroll
         for (int j = 0; j < A_LPW; j++) load_to_lds16(a_src[j], a_dst + sb + j * 1024);
         const bool more = it + 1 < it1;           // wave-uniform
-        const int64_t astep = more ? a_step : 0;
+        int64_t astep = more ? a_step : 0;
+        if (p.a_wrap && more && (it + 1) % p.a_wrap == 0) astep = -(int64_t)(p.a_wrap - 1) * a_step;
         const int wstep = more ? WC * 4 : 0;
 #pragma unroll
         for (int j = 0; j < A_LPW; j++) a_src[j] += astep;
@@ -327,7 +341,7 @@ __global__ void __launch_bounds__(256) qgemm_tile_kernel(TileArgs p)
     for (int tn = 0; tn < TN; tn++) {
         const int row = (wn * TN + tn) * 32 + lr;
         if constexpr (WC == 2) w_off[tn] = A_BYTES + (row * 2 + (h ^ ((row >> 3) & 1))) * 16;
-        else w_off[tn] = A_BYTES + row * 64;   // chunk index added per read
+        else w_off[tn] = A_BYTES + row * (WC * 16);   // chunk index added per read
     }
     const int asw = (lr >> 1) & 7;   // (row >> 1) & 7 of every activation row this lane reads
 
@@ -345,12 +359,14 @@ __global__ void __launch_bounds__(256) qgemm_tile_kernel(TileArgs p)
                     const u32x4 t = *reinterpret_cast<const u32x4 *>(sbase + w_off[tn]);
                     wq[tn][0] = t[0]; wq[tn][1] = t[1]; wq[tn][2] = t[2]; wq[tn][3] = t[3];
                 } else {
+                    constexpr int CPH = WC / 2;   // chunks per lane half: 2 (8-bit types) or 4 (f16)
                     const int row = (wn * TN + tn) * 32 + lr;
-                    const int sw = (row >> 2) & 3;
-                    const u32x4 t0 = *reinterpret_cast<const u32x4 *>(sbase + w_off[tn] + (((2 * h) ^ sw) * 16));
-                    const u32x4 t1 = *reinterpret_cast<const u32x4 *>(sbase + w_off[tn] + (((2 * h + 1) ^ sw) * 16));
-                    wq[tn][0] = t0[0]; wq[tn][1] = t0[1]; wq[tn][2] = t0[2]; wq[tn][3] = t0[3];
-                    wq[tn][4] = t1[0]; wq[tn][5] = t1[1]; wq[tn][6] = t1[2]; wq[tn][7] = t1[3];
+                    const int sw = (WC == 4) ? ((row >> 2) & 3) : ((row >> 1) & 7);
+#pragma unroll
+                    for (int c = 0; c < CPH; c++) {
+                        const u32x4 t = *reinterpret_cast<const u32x4 *>(sbase + w_off[tn] + (((CPH * h + c) ^ sw) * 16));
+                        wq[tn][4 * c + 0] = t[0]; wq[tn][4 * c + 1] = t[1]; wq[tn][4 * c + 2] = t[2]; wq[tn][4 * c + 3] = t[3];
+                    }
                 }
             }
         };
@@ -517,8 +533,15 @@ hipError_t launch_umean(const fnn_hip_weight *w, float *umean, hipStream_t s)
     return hipGetLastError();
 }
 
+// weights expanded beforehand to f16 [N][2*kpad] = [hi | lo] (codebook type): replaces the packed operand
+struct DenseOperand {
+    const uint32_t *words;
+    const float *row_scale, *row_zero;
+};
+
 template <int DT>
-int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &q, int flags)
+int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &q, int flags,
+              const DenseOperand *dense = nullptr)
 {
     const bool precise = !(flags & FNN_FLAG_ACT_F16_SINGLE);
     const int64_t M = q.m, N = q.n, K = q.k;
@@ -538,7 +561,8 @@ int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QM
     const int ntiles = (int)((N + bn - 1) / bn);
     const int64_t rows_pad = (int64_t)mtiles * bm;
     const int64_t m_pad = precise ? rows_pad / 2 : rows_pad;
-    const int iters = (int)(kpad / BK);
+    const int passes = dense ? 2 : 1;
+    const int iters = (int)(kpad / BK) * passes;
     // few tiles: split K until about two workgroups per CU are in flight
     static const int env_split = env_int("FNN_TILE_SPLIT", 0);
     static const int env_target = env_int("FNN_TILE_TARGET", 512);
@@ -560,8 +584,8 @@ int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QM
     if (splits > 1 && (rc = fnn_ctx_ensure_tmp(ctx, 1, (size_t)splits * M * N * 4, &ws1))) return rc;
 
     fnn_hip_weight *wm = const_cast<fnn_hip_weight *>(w);
-    const bool want_umean = !precise && (DT == FNN_DT_I8 || DT == FNN_DT_I4 || DT == FNN_DT_U8 || DT == FNN_DT_U4 || DT == FNN_DT_F4);
-    if (want_umean && !wm->umean) {
+    const bool want_umean = !precise && !dense && (DT == FNN_DT_I8 || DT == FNN_DT_I4 || DT == FNN_DT_U8 || DT == FNN_DT_U4 || DT == FNN_DT_F4);
+    if constexpr (DT != DT_F16_DENSE) if (want_umean && !wm->umean) {
         if (fnn_ctx_capturing(ctx)) return fnn_ctx_fail(ctx, FNN_ERR_MEMORY, "first single-pass use of a weight during graph capture");
         if (hipMalloc((void **)&wm->umean, (size_t)w->rows * 4 + 64) != hipSuccess)
             return fnn_ctx_fail(ctx, FNN_ERR_MEMORY, "out of device memory (row means)");
@@ -589,6 +613,13 @@ int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QM
     t.ap = pa.ap; t.rexp = pa.rexp; t.xsum = pa.xsum; t.esum = pa.esum;
     t.out = q.out; t.part = (float *)ws1;
     t.m = M; t.n = N; t.kp = q.kp; t.kpad = kpad; t.rows_pad = rows_pad;
+    t.a_wrap = 0;
+    if (dense) {
+        t.words = dense->words; t.zero_chunk = dense->words;
+        t.scales = dense->row_scale; t.zeros = dense->row_zero;
+        t.kp = kpad;                      // words per row: 2*kpad f16
+        t.a_wrap = (int)(kpad / BK);
+    }
     t.act = q.act; t.splits = splits; t.iters = iters; t.ips = ips; t.mtiles = mtiles; t.ntiles = ntiles;
     if (precise) {
         if (cfg == 0) e = launch_tile<DT, 2, 2, 2, 2, true, 3>(t, s);
@@ -610,6 +641,77 @@ int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QM
     return FNN_OK;
 }
 
+// Codebook type: w[n,k] = scales[n, k/qblock] * codebook[nibble]  (to_f32_vec_codebook,
+// src/packed_tensor.rs:469-521).  Expanded per call into a transient f16 operand: the row is scaled
+// by a power of two (max |w| of the row into [2^14, 2^15)) and each value written as hi = f16(w'),
+// lo = f16(w' - hi); hi and lo follow each other along K and the GEMM runs over both with the same
+// activations, so the product keeps ~22 mantissa bits of the f32 weight.
+__global__ void __launch_bounds__(256) expand_codebook_kernel(const uint32_t *words, const float *scales, const float *codebook,
+                                                              int64_t rows, int64_t inner, int64_t kp, int64_t bpr, int qblock,
+                                                              int64_t kpad, _Float16 *out, float *row_scale, float *row_zero)
+{
+    __shared__ float cb[16];
+    __shared__ float red[4];
+    const int64_t r = blockIdx.x;
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    if (tid < 16) cb[tid] = codebook[tid];
+    __syncthreads();
+    float cbmax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; i++) cbmax = fmaxf(cbmax, fabsf(cb[i]));
+    float smax = 0.0f;
+    for (int64_t b = tid; b < bpr; b += 256) smax = fmaxf(smax, fabsf(scales[r * bpr + b]));
+    smax = wave_max(smax);
+    if (lane == 0) red[wv] = smax;
+    __syncthreads();
+    const float mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3])) * cbmax;   // bound of |w| on the row
+    int e = 0;
+    if (mx > 0.0f && mx < __builtin_huge_valf()) {
+        int ex;
+        (void)frexpf(mx, &ex);
+        e = 15 - ex;
+    }
+    _Float16 *hi = out + r * 2 * kpad, *lo = hi + kpad;
+    for (int64_t g = tid; g < kpad / 8; g += 256) {
+        f16x8 h8, l8;
+        const uint32_t wd = g < kp ? words[r * kp + g] : 0u;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int64_t k = g * 8 + j;
+            float v = 0.0f;
+            if (k < inner) v = scales[r * bpr + k / qblock] * cb[(wd >> (4 * j)) & 0xf];
+            const float vs = ldexpf(v, e);
+            const _Float16 hh = (_Float16)vs;
+            h8[j] = hh;
+            l8[j] = (_Float16)(vs - (float)hh);
+        }
+        *reinterpret_cast<f16x8 *>(hi + g * 8) = h8;
+        *reinterpret_cast<f16x8 *>(lo + g * 8) = l8;
+    }
+    if (tid == 0) {
+        row_scale[r] = ldexpf(1.0f, -e);
+        row_zero[r] = 0.0f;
+    }
+}
+
+int run_tiled_codebook(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &q, int flags)
+{
+    const int64_t kpad = (q.k + BK - 1) / BK * BK;
+    const size_t op_bytes = (size_t)q.n * 2 * kpad * 2;
+    const size_t tab_off = (op_bytes + 255) / 256 * 256;
+    void *ws = nullptr;
+    int rc = fnn_ctx_ensure_tmp(ctx, 3, tab_off + (size_t)q.n * 8 + 256, &ws);
+    if (rc) return rc;
+    _Float16 *op = (_Float16 *)ws;
+    float *row_scale = (float *)((char *)ws + tab_off), *row_zero = row_scale + q.n;
+    hipLaunchKernelGGL(expand_codebook_kernel, dim3((unsigned)q.n), dim3(256), 0, s, q.words, q.scales, q.codebook, q.n, q.k,
+                       q.kp, q.bpr, q.qblock, kpad, op, row_scale, row_zero);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, hipGetErrorString(e));
+    DenseOperand d{(const uint32_t *)op, row_scale, row_zero};
+    return run_tiled<DT_F16_DENSE>(ctx, s, w, q, flags, &d);
+}
+
 }  // namespace
 
 int fnn_tiled_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &q, int flags, bool *handled)
@@ -617,7 +719,13 @@ int fnn_tiled_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, 
     *handled = false;
     static const int min_m = env_int("FNN_TILE_MIN_M", 5);
     if (q.m < min_m) return FNN_OK;
-    if (w->dtype == FNN_DT_I4CB) return FNN_OK;                 // codebook type: other kernels
+    if (w->dtype == FNN_DT_I4CB) {
+        if (q.as_written || q.qblock <= 0 || q.n > (1 << 24) || q.m > (1 << 22)) return FNN_OK;
+        int rc = run_tiled_codebook(ctx, s, w, q, flags);
+        if (rc) return rc;
+        *handled = true;
+        return FNN_OK;
+    }
     if (q.kp % 4 != 0) return FNN_OK;                           // 16-byte pieces of a weight row
     if (reinterpret_cast<uintptr_t>(q.words) & 15) return FNN_OK;
     if (q.m > (1 << 22) || q.n > (1 << 24)) return FNN_OK;      // 32-bit tile counts
