@@ -78,6 +78,7 @@ def main() -> int:
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--fast-act16", action="store_true", help="single f16 rounding of activations on the MFMA path")
+    ap.add_argument("--no-m256", action="store_true", help="skip the extra M=256 leg (TOPS and fraction of MFMA peak)")
     ap.add_argument("--probe", default="", choices=["", "read", "copy"],
                     help="instead of the MatMul, time a plain streaming read / copy of the same number of bytes "
                          "per launch over the same ring (device ceiling; calibration kernel for byte counters)")
@@ -236,6 +237,11 @@ def main() -> int:
         roofline["traffic"] = td.get("bytes")
         roofline["traffic_detail"] = td
 
+    # second half of the metric: the same weights at M=256 (GEMM regime), TOPS against the dense f16 MFMA peak
+    m256 = None
+    if not args.probe and not args.no_m256 and m != 256:
+        m256 = gemm_leg(ctx, flib, handles, ring, k, n, dbias, act, a_seed=1, m2=256)
+
     cpu = None
     if not args.no_cpu:
         cpu = cpu_baseline(pw, a, bias, act, abytes, flops, bandwidth_bound, args.cpu_seconds)
@@ -250,6 +256,7 @@ def main() -> int:
                    "launch": args.mode, "act_rounding": "f16x1" if args.fast_act16 else "default"},
         "roofline": roofline,
         "cpu_baseline": cpu,
+        "gemm_m256": m256,
         "gb_per_s": round(gbs, 1), "tflop_per_s": round(tops, 3),
         "event_ms_total": round(ev_ms, 4), "wall_ms_total": round(wall_s * 1e3, 4),
         "quantize_host_s": round(t_quant, 3), "self_check_max_rel": self_check,
@@ -259,6 +266,41 @@ def main() -> int:
         ctx.graph_destroy(graph)
     ctx.close()
     return 0
+
+
+def gemm_leg(ctx, flib, handles, ring, k, n, dbias, act, a_seed, m2):
+    """Eager launches of the same MatMul at M=m2 over the same ring of weight copies, timed with HIP
+    events on the launch stream; both activation modes; checked against the shape-agnostic kernel."""
+    a2 = np.random.default_rng(a_seed).standard_normal((m2, k)).astype(np.float32)
+    da2 = ctx.to_device(a2)
+    dout2 = ctx.alloc(m2 * n * 4)
+    flops = 2.0 * m2 * k * n
+    peak = MFMA_PEAK_TFLOPS["f16"]
+    res = {"m": m2, "peak": peak, "unit": "TFLOP/s", "flops": flops}
+    for name, fl in (("default", 0), ("f16x1", flib.FLAG_ACT_F16_SINGLE)):
+        f = fl | flib.FLAG_DEVICE_PTRS
+        for i in range(ring):
+            ctx.qmatmul_dev(handles[i], da2.ptr, m2, dout2.ptr, dbias.ptr if dbias else 0, act, f)
+        ctx.sync()
+        reps = max(ring, 40)
+        ctx.timer_start()
+        for i in range(reps):
+            ctx.qmatmul_dev(handles[i % ring], da2.ptr, m2, dout2.ptr, dbias.ptr if dbias else 0, act, f)
+        ms = ctx.timer_stop() / reps
+        got = dout2.download(np.float32, m2 * n).reshape(m2, n)
+        ctx.qmatmul_dev(handles[(reps - 1) % ring], da2.ptr, m2, dout2.ptr, dbias.ptr if dbias else 0, act,
+                        flib.FLAG_DEVICE_PTRS | flib.FLAG_FORCE_GENERIC)
+        ctx.sync()
+        chk = dout2.download(np.float32, m2 * n).reshape(m2, n)
+        t = flops / (ms * 1e-3) / 1e12
+        res[name] = {"us": round(ms * 1e3, 2), "tflop_per_s": round(t, 1), "frac": round(t / peak, 4),
+                     "self_check_max_rel": float(np.abs(got - chk).max() / (np.abs(chk).max() + 1e-30))}
+    res["note"] = ("algorithmic flops 2*M*K*N over the whole call (activation preparation + GEMM kernels); "
+                   "'default' keeps f32-accurate activations as f16 hi+lo operand rows (twice the MFMA work), "
+                   "'f16x1' rounds them to f16 once")
+    da2.free()
+    dout2.free()
+    return res
 
 
 def cpu_baseline(pw, a, bias, act, abytes, flops, bandwidth_bound, budget_s):
