@@ -114,6 +114,7 @@ void free_weight(fnn_hip_weight *w)
     if (w->codebook) (void)hipFree(w->codebook);
     if (w->row_qsum) (void)hipFree(w->row_qsum);
     if (w->umean) (void)hipFree(w->umean);
+    if (w->words4) (void)hipFree(w->words4);
     delete w;
 }
 
@@ -496,7 +497,8 @@ int fnn_hip_qmatmul_i8act(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const uint8
     p.acc_out = dacc; p.m = m; p.n = n; p.k = k; p.kp = w->kp;
     bool handled = false;
     if (!(flags & FNN_FLAG_FORCE_GENERIC)) {
-        (void)handled;   // integer matrix-core kernel: not built yet, the generic kernel serves every shape
+        int rc = fnn_i8_tiled_matmul(ctx, ctx->stream, w, p, &handled);
+        if (rc) return rc;
     }
     if (!handled) HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qgemm_i8act_generic(w->dtype, p, ctx->stream));
     if (!dev) {
@@ -571,7 +573,17 @@ int fnn_hip_qconv2d(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *x, i
     p.actq = p.minmax_partial + (size_t)(b * groups) * QCONV_NPART * 2;
     p.b = b; p.c = c; p.h = h; p.w = wd; p.oc = oc; p.ho = ho; p.wo = wo; p.kp = w->kp;
     p.kh = kh; p.kw = kw; p.stride = stride; p.pad = pad; p.dil = dil; p.groups = groups; p.act = act;
-    HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qconv2d_i8(p, ctx->stream));
+    if (flags & FNN_FLAG_FORCE_GENERIC) {
+        HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qconv2d_i8(p, ctx->stream, 0));
+    } else {
+        HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qconv2d_i8(p, ctx->stream, 1));
+        bool handled = false;
+        if (b * groups > 0 && ho * wo > 0) {
+            int rc2 = fnn_i8_tiled_conv(ctx, ctx->stream, w, p, &handled);
+            if (rc2) return rc2;
+        }
+        if (!handled) HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qconv2d_i8(p, ctx->stream, 2));
+    }
     if (!dev) {
         HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(y, dy, yout, hipMemcpyDeviceToHost, ctx->stream));
         if (acc_out) HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(acc_out, dacc, yout, hipMemcpyDeviceToHost, ctx->stream));

@@ -30,6 +30,8 @@ struct fnn_hip_weight {
     float *codebook;    // device; 16 floats (I4CB) or nullptr
     int32_t *row_qsum;  // device; [rows] sum of integer lanes per row (I8/I4), for the conv epilogue
     float *umean;       // device; [rows] mean lane value per row, built on first single-pass GEMM use
+    uint32_t *words4;   // device; rows re-strided to kp4 = ceil4(kp) words (+16 zero words) when kp % 4 != 0,
+    int64_t kp4;        //         built on first use by a kernel that fetches 16-byte pieces of a row
     int qblock;         // I4CB block length along inner
     int64_t bpr;        // blocks per row
     struct fnn_hip_ctx *ctx;

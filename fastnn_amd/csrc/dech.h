@@ -127,4 +127,26 @@ struct DecH<FNN_DT_F4> {
     }
 };
 
+// ---- int8 operands for v_mfma_i32_32x32x32_i8: one MFMA step = 16 k-values of a weight row (4 words).
+template <int DT>
+struct DecI;
+template <>
+struct DecI<FNN_DT_I8> {
+    static constexpr int WPS = 4;              // words per step
+    static constexpr bool INTERLEAVED = false;
+    __device__ static __forceinline__ f16x8 step(const uint32_t *w) { return pack8(w[0], w[1], w[2], w[3]); }
+};
+// 4-bit lanes become 16*q: the nibble moved to (or left in) the high half of a byte is the signed
+// byte 16*q.  Low nibbles (even k) and high nibbles (odd k) of a word form two operand words, so the
+// operand order inside 8 k-values is 0,2,4,6,1,3,5,7; the activations are stored in the same order.
+template <>
+struct DecI<FNN_DT_I4> {
+    static constexpr int WPS = 2;
+    static constexpr bool INTERLEAVED = true;
+    __device__ static __forceinline__ f16x8 step(const uint32_t *w)
+    {
+        return pack8((w[0] << 4) & 0xF0F0F0F0u, w[0] & 0xF0F0F0F0u, (w[1] << 4) & 0xF0F0F0F0u, w[1] & 0xF0F0F0F0u);
+    }
+};
+
 }  // namespace dech

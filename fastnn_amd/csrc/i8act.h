@@ -32,4 +32,4 @@ hipError_t launch_quantize_activations(const float *x, int64_t numel, float scal
                                        uint8_t *payload, float *scratch_partial, hipStream_t s);
 hipError_t launch_qgemm_i8act_generic(int dtype, const I8ActArgs &p, hipStream_t s);
 hipError_t launch_row_qsum(const fnn_hip_weight *w, int32_t *out, hipStream_t s);
-hipError_t launch_qconv2d_i8(const QConvArgs &p, hipStream_t s);
+hipError_t launch_qconv2d_i8(const QConvArgs &p, hipStream_t s, int phase);

@@ -16,3 +16,8 @@ int fnn_tiled_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, 
 // M <= 4: bandwidth-bound GEMV on the matrix cores (weights requested before anything else).
 int fnn_mfma_qgemv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &p,
                    int flags, bool *handled);
+
+// I8 activations x I8/I4 weights and the quantised Conv2d on int8 MFMA tiles with i32 accumulators.
+int fnn_i8_tiled_matmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const I8ActArgs &p, bool *handled);
+// p.actq must already hold the (image, group) activation scales.
+int fnn_i8_tiled_conv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QConvArgs &p, bool *handled);

@@ -60,6 +60,54 @@ __global__ void __launch_bounds__(256) conv_minmax_kernel(QConvArgs a)
     }
 }
 
+// The same min/max without walking the im2col matrix: an input pixel (ih, iw) appears in it iff some
+// tap reaches it, which factorises into a row condition and a column condition; the zero of the
+// padding takes part iff some tap falls outside.  min/max do not depend on order or multiplicity,
+// so the result is identical to the scan above.
+__global__ void __launch_bounds__(256) conv_minmax_cover_kernel(QConvArgs a, int pad_touched)
+{
+    extern __shared__ unsigned char cov[];   // [h] rows reached, then [w] columns reached
+    __shared__ float smn[4], smx[4];
+    unsigned char *cov_h = cov, *cov_w = cov + a.h;
+    for (int64_t t = threadIdx.x; t < a.h + a.w; t += blockDim.x) {
+        const bool is_h = t < a.h;
+        const int64_t pos = is_h ? t : t - a.h;
+        const int taps = is_h ? a.kh : a.kw;
+        const int64_t outs = is_h ? a.ho : a.wo;
+        unsigned char hit = 0;
+        for (int i = 0; i < taps; i++) {
+            const int64_t num = pos + a.pad - (int64_t)i * a.dil;   // = o * stride
+            if (num >= 0 && num % a.stride == 0 && num / a.stride < outs) hit = 1;
+        }
+        cov[t] = hit;
+    }
+    __syncthreads();
+    const int bg = blockIdx.y;
+    const int64_t nn = bg / a.groups, g = bg % a.groups;
+    const int64_t cg = a.c / a.groups;
+    const float *xg = a.x + (nn * a.c + g * cg) * a.h * a.w;
+    const int64_t hw = a.h * a.w, total = cg * hw;
+    float mn = pad_touched ? 0.0f : INFINITY, mx = pad_touched ? 0.0f : -INFINITY;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t rem = idx % hw;
+        const int64_t ih = rem / a.w, iw = rem % a.w;
+        if (cov_h[ih] && cov_w[iw]) {
+            const float v = xg[idx];
+            mn = fminf(mn, v);
+            mx = fmaxf(mx, v);
+        }
+    }
+    mn = wave_min(mn);
+    mx = wave_max(mx);
+    if ((threadIdx.x & 63) == 0) { smn[threadIdx.x >> 6] = mn; smx[threadIdx.x >> 6] = mx; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float *dst = a.minmax_partial + ((int64_t)bg * QCONV_NPART + blockIdx.x) * 2;
+        dst[0] = fminf(fminf(smn[0], smn[1]), fminf(smn[2], smn[3]));
+        dst[1] = fmaxf(fmaxf(smx[0], smx[1]), fmaxf(smx[2], smx[3]));
+    }
+}
+
 // scale = range/255 (1 if range <= 0), zero = mn + 128*scale (0 if range <= 0), inv = 1/scale
 // (src/backend/cpu/packed_conv.rs:149-156)
 __global__ void __launch_bounds__(64) conv_actq_kernel(QConvArgs a, int nparts)
@@ -182,7 +230,8 @@ hipError_t launch_row_qsum(const fnn_hip_weight *w, int32_t *out, hipStream_t s)
     return hipGetLastError();
 }
 
-hipError_t launch_qconv2d_i8(const QConvArgs &p, hipStream_t s)
+// phase 0: everything; 1: the (image, group) activation scales only; 2: the direct kernel only (scales present)
+hipError_t launch_qconv2d_i8(const QConvArgs &p, hipStream_t s, int phase)
 {
     const int64_t bg = p.b * p.groups;
     const int64_t cg = p.c / p.groups, ocg = p.oc / p.groups;
@@ -192,8 +241,30 @@ hipError_t launch_qconv2d_i8(const QConvArgs &p, hipStream_t s)
     int64_t nparts = (total + 256 * 16 - 1) / (256 * 16);
     if (nparts > QCONV_NPART) nparts = QCONV_NPART;
     if (nparts < 1) nparts = 1;
-    hipLaunchKernelGGL(conv_minmax_kernel, dim3((unsigned)nparts, (unsigned)bg), dim3(256), 0, s, p);
-    hipLaunchKernelGGL(conv_actq_kernel, dim3((unsigned)bg), dim3(64), 0, s, p, (int)nparts);
+    if (phase != 2) {
+        if (p.h + p.w <= 32768 && cg > 0) {
+            // does any tap fall into the padding?  (rows and columns separately)
+            int pad_touched = 0;
+            for (int64_t o = 0; o < p.ho && !pad_touched; o++)
+                for (int i = 0; i < p.kh; i++) {
+                    const int64_t ih = o * p.stride + (int64_t)i * p.dil - p.pad;
+                    if (ih < 0 || ih >= p.h) { pad_touched = 1; break; }
+                }
+            for (int64_t o = 0; o < p.wo && !pad_touched; o++)
+                for (int i = 0; i < p.kw; i++) {
+                    const int64_t iw = o * p.stride + (int64_t)i * p.dil - p.pad;
+                    if (iw < 0 || iw >= p.w) { pad_touched = 1; break; }
+                }
+            const int64_t elems = cg * p.h * p.w;
+            nparts = (elems + 256 * 16 - 1) / (256 * 16);
+            if (nparts > QCONV_NPART) nparts = QCONV_NPART;
+            if (nparts < 1) nparts = 1;
+            hipLaunchKernelGGL(conv_minmax_cover_kernel, dim3((unsigned)nparts, (unsigned)bg), dim3(256), (size_t)(p.h + p.w), s, p, pad_touched);
+        } else
+            hipLaunchKernelGGL(conv_minmax_kernel, dim3((unsigned)nparts, (unsigned)bg), dim3(256), 0, s, p);
+        hipLaunchKernelGGL(conv_actq_kernel, dim3((unsigned)bg), dim3(64), 0, s, p, (int)nparts);
+    }
+    if (phase == 1) return hipGetLastError();
     dim3 grid((unsigned)((np + 255) / 256), (unsigned)((ocg + CONV_OCT - 1) / CONV_OCT), (unsigned)bg);
     hipLaunchKernelGGL(conv_i8_kernel, grid, dim3(256), 0, s, p);
     return hipGetLastError();

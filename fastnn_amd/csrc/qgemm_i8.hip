@@ -1,0 +1,366 @@
+// Integer matrix-core path for gfx950: I8 activations x I8/I4 weights with exact i32 accumulators
+// on v_mfma_i32_32x32x32_i8, serving
+//   - "matmul_i8_i8" / "matmul_i4_i8" (gemm_cpu_flat_i8_i8x4 / gemm_cpu_flat_i8_i4x8,
+//     src/backend/cpu/microkernels/gemm.rs:1641-1975), and
+//   - the quantised Conv2d lowering conv2d_packed_i8x4 (im2col + per-(image,group) int8 activation
+//     quantisation + integer GEMM + 4-term dequantise, src/backend/cpu/packed_conv.rs:125-232,444-625).
+// Three launches per call: an operand kernel writes the int8 activation matrix in the tile-major
+// layout of the GEMM kernel (for conv it evaluates im2col and the quantisation on the fly and also
+// leaves sum_k q_a per row), the shared tiled GEMM kernel produces raw i32 accumulators, and an
+// epilogue kernel applies the reference's float formula (and scatters conv outputs to NCHW).
+#include "mfma.h"
+#include "dech.h"
+
+#include <type_traits>
+
+namespace {
+
+using namespace dech;
+
+constexpr float LO_UP = 2048.0f, LO_DOWN = 1.0f / 2048.0f;   // f16 mode of the shared kernel (unused here)
+#include "tile_kernel.h"
+
+constexpr int KB = 128;   // k-values (= bytes) per stage and activation row
+
+// position of k inside its group of 8 in the operand: identity, or 0,2,4,6,1,3,5,7 for nibble weights
+__device__ __forceinline__ int slot_of(int j, int interleaved) { return interleaved ? ((j & 1) * 4 + (j >> 1)) : j; }
+
+// ---- I8-activation MatMul operand: payload rows -> tile-major int8 [kpad/128][rows_pad][128] + sum q_a per row
+__global__ void __launch_bounds__(256) i8_rows_operand_kernel(const int8_t *qa, int64_t m, int64_t k, int64_t kpad,
+                                                              int64_t rows_pad, int interleaved, int8_t *a8, int32_t *qsum)
+{
+    __shared__ int red[4];
+    const int64_t r = blockIdx.x;
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    int s = 0;
+    for (int64_t c = tid; c < kpad / 16; c += 256) {   // 16-byte chunk c of the row
+        uint32_t out[4] = {0, 0, 0, 0};
+        if (r < m) {
+#pragma unroll
+            for (int g8 = 0; g8 < 2; g8++)
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    const int64_t kk = c * 16 + g8 * 8 + j;
+                    const int q = kk < k ? (int)qa[r * k + kk] : 0;
+                    s += q;
+                    const int pos = g8 * 8 + slot_of(j, interleaved);
+                    out[pos >> 2] |= (uint32_t)(uint8_t)q << (8 * (pos & 3));
+                }
+        }
+        const int64_t kb = c >> 3, cc = c & 7;
+        *reinterpret_cast<uint4 *>(a8 + (kb * rows_pad + r) * KB + cc * 16) = make_uint4(out[0], out[1], out[2], out[3]);
+    }
+    s = wave_sum_i32(s);
+    if (lane == 0) red[wv] = s;
+    __syncthreads();
+    if (tid == 0) qsum[r] = (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+// res = dot*sw + zw*input_sum with dot = acc*sa, input_sum = sum(q_a)*sa + K*za
+// (gemm.rs:1641-1975).  With za != 0 the reference multiplies per lane in f32; the same quantity is
+// formed here from the integer sums: sum (q_a*sa + za)*q_w = sa*acc + za*sum_k q_w.
+__global__ void __launch_bounds__(256) i8_matmul_epilogue_kernel(const int32_t *c, const uint8_t *payload, const int32_t *qsum,
+                                                                 const int32_t *wsum, const float *scales, const float *zeros,
+                                                                 int64_t m, int64_t n, int64_t k, float *out, int32_t *acc_out)
+{
+    const float sa = reinterpret_cast<const float *>(payload)[0];
+    const float za = reinterpret_cast<const float *>(payload)[1];
+    const int64_t total = m * n;
+    for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * 256) {
+        const int64_t r = idx / n, col = idx % n;
+        const int acc = c[idx];
+        const float sw = scales[col], zw = zeros[col];
+        float res;
+        if (za != 0.0f) {
+            const float d = (float)acc * sa + za * (float)wsum[col];
+            const float s = (float)qsum[r] * sa + (float)k * za;
+            res = d * sw + zw * s;
+        } else {
+            const float dot = (float)acc * sa;
+            const float input_sum = (float)qsum[r] * sa + (float)k * za;
+            res = dot * sw + zw * input_sum;
+        }
+        out[idx] = res;
+        if (acc_out) acc_out[idx] = (za != 0.0f) ? 0 : acc;
+    }
+}
+
+// ---- conv operand: im2col row (image nn, pixel p) of group g, quantised with the (image, group) scale:
+// q = clamp(round((v - za) * inv), -128, 127)  (packed_conv.rs:149-232).
+// A workgroup owns 64 consecutive rows; thread (row, slot) walks the 16-value chunks slot, slot+4, ...
+// that hold data (neighbouring lanes = neighbouring pixels: the NCHW reads coalesce), the (ic, i, j)
+// tap of a chunk is advanced by carries instead of divisions; all-zero chunks are written in a second sweep.
+constexpr int CONV_CPB = 8;   // 16-value chunks of a row per workgroup
+
+__global__ void __launch_bounds__(256) conv_operand_kernel(QConvArgs a, int g, int kk, int64_t kpad, int64_t rows_pad,
+                                                           int8_t *a8, int32_t *qsum)
+{
+    __shared__ int part[4][64];
+    const int tid = threadIdx.x, rr = tid & 63, slot = tid >> 6;
+    const int64_t np = a.ho * a.wo;
+    const int64_t r = (int64_t)blockIdx.x * 64 + rr;
+    const int64_t rows = a.b * np;
+    const int64_t cg = a.c / a.groups;
+    const int live_chunks = (kk + 15) / 16, all_chunks = (int)(kpad / 16);
+    const bool live = r < rows;
+    int s = 0;
+    if (r < rows_pad) {
+        const int64_t nn = live ? r / np : 0, p = live ? r % np : 0;
+        const int bg = (int)(nn * a.groups + g);
+        const float za = a.actq[bg * 4 + 1], inv = a.actq[bg * 4 + 2];
+        const float *xg = a.x + (nn * a.c + g * cg) * a.h * a.w;
+        const int khw = a.kh * a.kw;
+        const int64_t ih0 = (p / a.wo) * a.stride - a.pad, iw0 = (p % a.wo) * a.stride - a.pad;
+        const int c_end = (int)(blockIdx.y + 1) * CONV_CPB < live_chunks ? (int)(blockIdx.y + 1) * CONV_CPB : live_chunks;
+        for (int c = (int)blockIdx.y * CONV_CPB + slot; c < c_end; c += 4) {
+            uint32_t out[4] = {0, 0, 0, 0};
+            if (live) {
+                int e = c * 16;
+                int ic = e / khw, rem = e % khw;
+                int i = rem / a.kw, j = rem % a.kw;
+#pragma unroll
+                for (int t = 0; t < 16; t++) {
+                    if (e < kk) {
+                        const int64_t ih = ih0 + (int64_t)i * a.dil, iw = iw0 + (int64_t)j * a.dil;
+                        float v = 0.0f;
+                        if (ih >= 0 && ih < a.h && iw >= 0 && iw < a.w) v = xg[((int64_t)ic * a.h + ih) * a.w + iw];
+                        const float q = roundf((v - za) * inv);
+                        const int qi = (q != q) ? 0 : (int)fminf(fmaxf(q, -128.0f), 127.0f);
+                        s += qi;
+                        out[t >> 2] |= (uint32_t)(uint8_t)qi << (8 * (t & 3));
+                    }
+                    e++;
+                    if (++j == a.kw) { j = 0; if (++i == a.kh) { i = 0; ic++; } }
+                }
+            }
+            *reinterpret_cast<uint4 *>(a8 + ((int64_t)(c >> 3) * rows_pad + r) * KB + (c & 7) * 16) = make_uint4(out[0], out[1], out[2], out[3]);
+        }
+    }
+    part[slot][rr] = s;
+    // chunks past the data: zeros, written with consecutive lanes on consecutive 16-byte pieces of a row
+    const int zc = all_chunks - live_chunks;
+    if (zc > 0 && blockIdx.y == 0) {
+        const int64_t row0 = (int64_t)blockIdx.x * 64;
+        for (int64_t idx = tid; idx < (int64_t)64 * zc; idx += 256) {
+            const int64_t row = row0 + idx / zc;
+            const int c = live_chunks + (int)(idx % zc);
+            if (row < rows_pad)
+                *reinterpret_cast<uint4 *>(a8 + ((int64_t)(c >> 3) * rows_pad + row) * KB + (c & 7) * 16) = make_uint4(0, 0, 0, 0);
+        }
+    }
+    __syncthreads();
+    // one partial sum per chunk group; the epilogue adds them
+    if (tid < 64 && r < rows_pad) qsum[(int64_t)blockIdx.y * rows_pad + r] = (part[0][tid] + part[1][tid]) + (part[2][tid] + part[3][tid]);
+}
+
+// acc = bias_q + sum q_a*q_w; val = acc*sab + zw*(sa*sum q_a) + za*(sw*sum q_w) + (za*zw)*K, left to right,
+// then the activation (packed_conv.rs:469-505,571,604-606).  A workgroup takes 64 rows of C (read along the
+// channels, as stored), turns the tile in LDS and writes NCHW with consecutive lanes on consecutive pixels.
+__global__ void __launch_bounds__(256) conv_epilogue_kernel(QConvArgs a, int g, int kk, const int32_t *c, int ocg,
+                                                            const int32_t *qsum, int nq, int64_t rows_pad)
+{
+    __shared__ float tile[64 * 65];   // [channel of the block][row], padded
+    __shared__ int itile[64 * 65];    // accumulators incl. bias_q, same shape
+    const int64_t np = a.ho * a.wo, rows = a.b * np;
+    const int64_t row0 = (int64_t)blockIdx.x * 64;
+    const int f0 = blockIdx.y * 64;
+    const int fb = ocg - f0 < 64 ? ocg - f0 : 64;   // channels of this block
+    const int tid = threadIdx.x;
+    for (int idx = tid; idx < 64 * fb; idx += 256) {
+        const int rr = idx / fb, fl = idx % fb, f = f0 + fl;
+        const int64_t r = row0 + rr;
+        if (r >= rows) continue;
+        const int64_t nn = r / np;
+        const int64_t ch = (int64_t)g * ocg + f;
+        const int bg = (int)(nn * a.groups + g);
+        const float sa = a.actq[bg * 4 + 0], za = a.actq[bg * 4 + 1];
+        const float sw = a.scales[ch], zw = a.zeros[ch];
+        const float sab = sa * sw;
+        int bias_q = 0;
+        if (a.bias) {
+            const float bq = roundf(a.bias[ch] / sab);
+            bias_q = (bq != bq) ? 0 : (bq >= 2147483648.0f ? 2147483647 : (bq <= -2147483648.0f ? (-2147483647 - 1) : (int)bq));
+        }
+        const int accv = c[r * ocg + f] + bias_q;
+        int qs = 0;
+        for (int y = 0; y < nq; y++) qs += qsum[(int64_t)y * rows_pad + r];
+        const float rsum = sa * (float)qs;
+        const float w_term = sw * (float)a.row_qsum[ch];
+        const float zp_prod = za * zw;
+        float val = (float)accv * sab;
+        val = val + zw * rsum;
+        val = val + za * w_term;
+        val = val + zp_prod * (float)kk;
+        if (a.act == FNN_ACT_RELU) val = fmaxf(val, 0.0f);
+        else if (a.act == FNN_ACT_SILU) val = val / (1.0f + expf(-val));
+        else if (a.act == FNN_ACT_GELU) val = val * 0.5f * (1.0f + tanhf(val * 0.7978846f * (1.0f + 0.044715f * val * val)));
+        tile[fl * 65 + rr] = val;
+        itile[fl * 65 + rr] = accv;
+    }
+    __syncthreads();
+    for (int idx = tid; idx < 64 * fb; idx += 256) {
+        const int fl = idx / 64, rr = idx % 64;
+        const int64_t r = row0 + rr;
+        if (r >= rows) continue;
+        const int64_t nn = r / np, p = r % np;
+        const int64_t o = (nn * a.oc + (int64_t)g * ocg + f0 + fl) * np + p;
+        a.y[o] = tile[fl * 65 + rr];
+        if (a.acc_out) a.acc_out[o] = itile[fl * 65 + rr];
+    }
+}
+
+template <int DT, int WGM, int WGN, int TM, int TN, int NS>
+hipError_t launch_i8_tile(const TileArgs &p, hipStream_t s)
+{
+    constexpr int WC = 2 * DecI<DT>::WPS;
+    constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
+    constexpr size_t lds = (size_t)NS * (BM * 128 + BN * WC * 16);
+    auto kern = qgemm_tile_kernel<DT, WGM, WGN, TM, TN, false, NS, true>;
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)p.mtiles * p.ntiles), dim3(256), lds, s, p);
+    return hipGetLastError();
+}
+
+__global__ void __launch_bounds__(256) restride_rows_kernel(const uint32_t *src, int64_t rows, int64_t kp, int64_t kp4, uint32_t *dst)
+{
+    const int64_t total = rows * kp4 + 16;   // + zero margin
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+        const int64_t r = i / kp4, c = i % kp4;
+        dst[i] = (r < rows && c < kp) ? src[r * kp + c] : 0u;
+    }
+}
+
+// weight rows as 16-byte addressable pieces: the registered words, or a re-strided copy when kp % 4 != 0
+int aligned_rows(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const uint32_t **words, int64_t *kp)
+{
+    if (w->kp % 4 == 0) { *words = w->words; *kp = w->kp; return FNN_OK; }
+    fnn_hip_weight *wm = const_cast<fnn_hip_weight *>(w);
+    if (!wm->words4) {
+        if (fnn_ctx_capturing(ctx)) return fnn_ctx_fail(ctx, FNN_ERR_MEMORY, "first integer use of a weight during graph capture");
+        const int64_t kp4 = (w->kp + 3) / 4 * 4;
+        if (hipMalloc((void **)&wm->words4, (size_t)(w->rows * kp4 + 16) * 4) != hipSuccess)
+            return fnn_ctx_fail(ctx, FNN_ERR_MEMORY, "out of device memory (re-strided weight rows)");
+        wm->kp4 = kp4;
+        int64_t blocks = (w->rows * kp4 + 16 + 255) / 256;
+        if (blocks > 2048) blocks = 2048;
+        hipLaunchKernelGGL(restride_rows_kernel, dim3((unsigned)blocks), dim3(256), 0, s, w->words, w->rows, w->kp, kp4, wm->words4);
+        if (hipGetLastError() != hipSuccess) return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, "re-striding weight rows failed");
+    }
+    *words = wm->words4; *kp = wm->kp4;
+    return FNN_OK;
+}
+
+// C[m][n] = sum_k A8[m][k] * q_w[n0 + n][k] for `n` weight rows starting at row n0 (rows of kp words, 16-byte aligned)
+template <int DT>
+hipError_t run_i8_gemm(const uint32_t *words, int64_t kp, int64_t rows_total, int64_t n0, int64_t n, const int8_t *a8, int64_t m,
+                       int64_t rows_pad, int64_t kpad, int32_t *c, int64_t ldc, hipStream_t s)
+{
+    TileArgs t = {};
+    t.words = words + n0 * kp;
+    t.zero_chunk = words + rows_total * kp;   // the zeroed margin behind the last row
+    t.ap = reinterpret_cast<const _Float16 *>(a8);
+    t.c_i32 = c; t.ldc = ldc;
+    t.m = m; t.n = n; t.kp = kp; t.kpad = kpad; t.rows_pad = rows_pad;
+    t.splits = 1; t.iters = (int)(kpad / KB); t.ips = t.iters; t.mtiles = (int)(rows_pad / 128); t.a_wrap = 0;
+    if (n <= 64) {   // narrow outputs (early conv layers): 128 x 64 tiles, four waves stacked along M
+        t.ntiles = (int)((n + 63) / 64);
+        return launch_i8_tile<DT, 4, 1, 1, 2, 3>(t, s);
+    }
+    t.ntiles = (int)((n + 127) / 128);
+    return launch_i8_tile<DT, 2, 2, 2, 2, 3>(t, s);
+}
+
+}  // namespace
+
+int fnn_i8_tiled_matmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const I8ActArgs &p, bool *handled)
+{
+    *handled = false;
+    if (w->dtype != FNN_DT_I8 && w->dtype != FNN_DT_I4) return FNN_OK;
+    if (reinterpret_cast<uintptr_t>(p.words) & 15) return FNN_OK;
+    if (p.m < 1 || p.m > (1 << 22) || p.n > (1 << 24) || p.k > (1 << 20)) return FNN_OK;
+    const int64_t kpad = (p.k + KB - 1) / KB * KB;
+    const int64_t rows_pad = (p.m + 127) / 128 * 128;
+    const size_t a_bytes = (size_t)rows_pad * kpad;
+    const size_t q_off = (a_bytes + 255) / 256 * 256;
+    void *ws0 = nullptr, *ws1 = nullptr;
+    int rc;
+    if ((rc = fnn_ctx_ensure_tmp(ctx, 0, q_off + (size_t)rows_pad * 4 + 256, &ws0))) return rc;
+    if ((rc = fnn_ctx_ensure_tmp(ctx, 1, (size_t)p.m * p.n * 4 + 256, &ws1))) return rc;
+    fnn_hip_weight *wm = const_cast<fnn_hip_weight *>(w);
+    if (!wm->row_qsum) {
+        if (fnn_ctx_capturing(ctx)) return fnn_ctx_fail(ctx, FNN_ERR_MEMORY, "first integer use of a weight during graph capture");
+        if (hipMalloc((void **)&wm->row_qsum, (size_t)w->rows * 4 + 64) != hipSuccess)
+            return fnn_ctx_fail(ctx, FNN_ERR_MEMORY, "out of device memory (row sums)");
+        hipError_t e = launch_row_qsum(w, wm->row_qsum, s);
+        if (e != hipSuccess) return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, hipGetErrorString(e));
+    }
+    const uint32_t *words;
+    int64_t kp;
+    if ((rc = aligned_rows(ctx, s, w, &words, &kp))) return rc;
+    int8_t *a8 = (int8_t *)ws0;
+    int32_t *qsum = (int32_t *)((char *)ws0 + q_off);
+    int32_t *c = (int32_t *)ws1;
+    const int interleaved = w->dtype == FNN_DT_I4 ? 1 : 0;
+    hipLaunchKernelGGL(i8_rows_operand_kernel, dim3((unsigned)rows_pad), dim3(256), 0, s,
+                       reinterpret_cast<const int8_t *>(p.payload + 8), p.m, p.k, kpad, rows_pad, interleaved, a8, qsum);
+    hipError_t e = hipGetLastError();
+    if (e == hipSuccess)
+        e = w->dtype == FNN_DT_I8 ? run_i8_gemm<FNN_DT_I8>(words, kp, w->rows, 0, p.n, a8, p.m, rows_pad, kpad, c, p.n, s)
+                                  : run_i8_gemm<FNN_DT_I4>(words, kp, w->rows, 0, p.n, a8, p.m, rows_pad, kpad, c, p.n, s);
+    if (e == hipSuccess) {
+        int64_t blocks = (p.m * p.n + 255) / 256;
+        if (blocks > 4096) blocks = 4096;
+        hipLaunchKernelGGL(i8_matmul_epilogue_kernel, dim3((unsigned)blocks), dim3(256), 0, s, c, p.payload, qsum, wm->row_qsum,
+                           p.scales, p.zeros, p.m, p.n, p.k, p.out, p.acc_out);
+        e = hipGetLastError();
+    }
+    if (e != hipSuccess) return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, hipGetErrorString(e));
+    *handled = true;
+    return FNN_OK;
+}
+
+// after the (image, group) activation scales are known (p.actq): operand, integer GEMM and epilogue per group
+int fnn_i8_tiled_conv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QConvArgs &p, bool *handled)
+{
+    *handled = false;
+    if (w->dtype != FNN_DT_I8 || (reinterpret_cast<uintptr_t>(p.words) & 15)) return FNN_OK;
+    const int64_t np = p.ho * p.wo, rows = p.b * np;
+    const int64_t cg = p.c / p.groups, ocg = p.oc / p.groups, kk = cg * p.kh * p.kw;
+    if (rows < 1 || rows > (1ll << 28) || kk > (1 << 20) || ocg < 1) return FNN_OK;
+    const int64_t kpad = (kk + KB - 1) / KB * KB;
+    const int64_t rows_pad = (rows + 127) / 128 * 128;
+    const size_t a_bytes = (size_t)rows_pad * kpad;
+    const size_t q_off = (a_bytes + 255) / 256 * 256;
+    void *ws1 = nullptr, *ws3 = nullptr;
+    int rc;
+    const int nq = (int)(((kk + 15) / 16 + CONV_CPB - 1) / CONV_CPB);   // partial row sums per row
+    if (nq > 65535) return FNN_OK;
+    if ((rc = fnn_ctx_ensure_tmp(ctx, 3, q_off + (size_t)rows_pad * 4 * nq + 256, &ws3))) return rc;   // 0 holds the scales
+    if ((rc = fnn_ctx_ensure_tmp(ctx, 1, (size_t)rows * ocg * 4 + 256, &ws1))) return rc;
+    const uint32_t *words;
+    int64_t kp;
+    if ((rc = aligned_rows(ctx, s, w, &words, &kp))) return rc;
+    int8_t *a8 = (int8_t *)ws3;
+    int32_t *qsum = (int32_t *)((char *)ws3 + q_off);
+    int32_t *c = (int32_t *)ws1;
+    if (ocg > 65535 * 64) return FNN_OK;
+    for (int g = 0; g < p.groups; g++) {
+        const dim3 grid((unsigned)(rows_pad / 64), (unsigned)nq);
+        hipLaunchKernelGGL(conv_operand_kernel, grid, dim3(256), 0, s, p, g, (int)kk, kpad, rows_pad, a8, qsum);
+        hipError_t e = hipGetLastError();
+        if (e == hipSuccess) e = run_i8_gemm<FNN_DT_I8>(words, kp, w->rows, g * ocg, ocg, a8, rows, rows_pad, kpad, c, ocg, s);
+        if (e == hipSuccess) {
+            hipLaunchKernelGGL(conv_epilogue_kernel, dim3((unsigned)((rows + 63) / 64), (unsigned)((ocg + 63) / 64)), dim3(256), 0, s, p, g,
+                               (int)kk, c, (int)ocg, qsum, nq, rows_pad);
+            e = hipGetLastError();
+        }
+        if (e != hipSuccess) return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, hipGetErrorString(e));
+    }
+    *handled = true;
+    return FNN_OK;
+}

@@ -28,6 +28,7 @@
 #include "dech.h"
 
 #include <cstdlib>
+#include <type_traits>
 
 namespace {
 
@@ -45,8 +46,9 @@ struct DecH<64> {
 };
 }  // namespace dech
 namespace {
-constexpr int BK = 64;          // k-values per main-loop iteration
+// the lo activation term is stored scaled by 2^11 so that it stays in the normal f16 range
 constexpr float LO_UP = 2048.0f, LO_DOWN = 1.0f / 2048.0f;
+constexpr int BK = 64;          // k-values per main-loop iteration
 
 struct PrepArgs {
     const float *a;
@@ -207,285 +209,7 @@ __global__ void __launch_bounds__(64) row_umean_kernel(const uint32_t *words, in
     if (threadIdx.x == 0) umean[r] = s / (float)k;
 }
 
-struct TileArgs {
-    const uint32_t *words;
-    const uint32_t *zero_chunk;   // 16 zero bytes: source of weight chunks past the end of a row
-    const float *scales, *zeros, *umean, *bias;
-    const _Float16 *ap;
-    const int *rexp;
-    const float *xsum, *esum;
-    float *out, *part;
-    int64_t m, n, kp, kpad, rows_pad;
-    int act, splits, iters, ips, mtiles, ntiles;
-    int a_wrap;   // > 0: the activation operand has a_wrap k blocks and is swept again after them (weights = [hi | lo])
-};
-
-// HBM -> LDS without passing registers: lane i of the wave stores its 16 bytes at
-// LDS address m0 + 16*i.  The compiler does not see these loads: waits are placed by hand.
-__device__ __forceinline__ void load_to_lds16(const void *gptr, unsigned lds_wave_base)
-{
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_wave_base), "v"(gptr) : "memory");
-}
-template <int N>
-__device__ __forceinline__ void wait_loads_but()
-{
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-}
-
-template <int DT, int WGM, int WGN, int TM, int TN, bool PRECISE, int NS>
-__global__ void __launch_bounds__(256) qgemm_tile_kernel(TileArgs p)
-{
-    using D = DecH<DT>;
-    constexpr int WPS = D::WPS;          // words per 8 k-values
-    constexpr int WC = 2 * WPS;          // 16-byte weight chunks per row and stage (32, 64 or 128 bytes)
-    constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
-    constexpr int A_BYTES = BM * 128, W_BYTES = BN * WC * 16, STAGE = A_BYTES + W_BYTES;
-    constexpr int A_LPW = BM / 32;             // activation load instructions per wave and stage
-    constexpr int W_LPW = BN * WC / 256;       // weight load instructions per wave and stage
-    constexpr int LPS = A_LPW + W_LPW;
-    static_assert(WGM * WGN == 4, "4 waves");
-    static_assert(BN * WC % 256 == 0 && NS >= 3 && NS <= 8, "stage shape");
-
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char *)smem;
-
-    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
-    const int wm = wv / WGN, wn = wv % WGN;
-    const int lr = lane & 31, h = lane >> 5;
-
-    // workgroup id -> tile, row tile fastest.  Ids are dealt round-robin over the 8 XCDs (each with
-    // its own L2), so an XCD keeps meeting the same few row tiles of the activations, the operand
-    // with the most bytes per MAC, while the packed weights stream through.
-    const unsigned L = blockIdx.x;
-    const int mt = L % p.mtiles;
-    const unsigned rest = L / p.mtiles;
-    const int z = rest % p.splits;
-    const int nt = rest / p.splits;
-    const int64_t n0 = (int64_t)nt * BN;
-    const int it0 = z * p.ips;
-    const int it1 = (it0 + p.ips < p.iters) ? it0 + p.ips : p.iters;
-
-    // ---- what this lane fetches per stage.  LDS slot s of a region = 16-byte chunk s.
-    // The LDS has 64 banks of 4 bytes: a 128-bit read is conflict-free when every 16 lanes cover
-    // all sixteen 16-byte slots of a 256-byte window, hence the row-dependent XOR of the chunk index.
-    // activations: chunk (row, g) lives at slot row*8 + (g ^ ((row >> 1) & 7))
-    const _Float16 *a_src[A_LPW];
-#pragma unroll
-    for (int j = 0; j < A_LPW; j++) {
-        const int slot = (wv * A_LPW + j) * 64 + lane;
-        const int row = slot >> 3, g = (slot & 7) ^ ((row >> 1) & 7);
-        a_src[j] = p.ap + ((int64_t)mt * BM + row) * 64 + g * 8;
-    }
-    // weights: chunk (row, c) lives at slot row*WC + (c ^ swz(row)); rows past N repeat the last row
-    const uint32_t *w_src[W_LPW];
-    int w_chunk[W_LPW];
-#pragma unroll
-    for (int j = 0; j < W_LPW; j++) {
-        const int slot = (wv * W_LPW + j) * 64 + lane;
-        const int row = slot / WC;
-        const int sw = (WC == 2) ? ((row >> 3) & 1) : (WC == 4 ? ((row >> 2) & 3) : ((row >> 1) & 7));
-        const int c = (slot % WC) ^ sw;
-        int64_t grow = n0 + row;
-        if (grow > p.n - 1) grow = p.n - 1;
-        w_src[j] = p.words + grow * p.kp + c * 4;
-        w_chunk[j] = c * 4;
-    }
-    const int64_t a_step = p.rows_pad * 64;   // elements between consecutive k blocks
-    const unsigned a_dst = __builtin_amdgcn_readfirstlane(lds0 + wv * A_LPW * 1024);
-    const unsigned w_dst = __builtin_amdgcn_readfirstlane(lds0 + A_BYTES + wv * W_LPW * 1024);
-
-    // running source pointers: advanced after every stage, frozen once the K range is exhausted
-    // (the extra requests of the last iterations re-read the final stage and are never consumed)
-#pragma unroll
-    for (int j = 0; j < A_LPW; j++) a_src[j] += (int64_t)(p.a_wrap ? it0 % p.a_wrap : it0) * a_step;
-#pragma unroll
-    for (int j = 0; j < W_LPW; j++) w_src[j] += (int64_t)it0 * (WC * 4);
-    const bool ragged = (p.kp % (WC * 4)) != 0;   // the last stage of a row is partly past its end
-    auto issue = [&](int it, int buf) {
-        const unsigned sb = buf * STAGE;
-        if (ragged && it >= p.iters - 1) {
-#pragma unroll
-            for (int j = 0; j < W_LPW; j++) {
-                const bool ok = (int64_t)(p.iters - 1) * (WC * 4) + w_chunk[j] + 4 <= p.kp;
-                load_to_lds16(ok ? w_src[j] : p.zero_chunk, w_dst + sb + j * 1024);
-            }
-        } else {
-#pragma unroll
-            for (int j = 0; j < W_LPW; j++) load_to_lds16(w_src[j], w_dst + sb + j * 1024);
-        }
-#pragma unroll
-        for (int j = 0; j < A_LPW; j++) load_to_lds16(a_src[j], a_dst + sb + j * 1024);
-        const bool more = it + 1 < it1;           // wave-uniform
-        int64_t astep = more ? a_step : 0;
-        if (p.a_wrap && more && (it + 1) % p.a_wrap == 0) astep = -(int64_t)(p.a_wrap - 1) * a_step;
-        const int wstep = more ? WC * 4 : 0;
-#pragma unroll
-        for (int j = 0; j < A_LPW; j++) a_src[j] += astep;
-#pragma unroll
-        for (int j = 0; j < W_LPW; j++) w_src[j] += wstep;
-    };
-
-    f32x16 acc[TM][TN];
-#pragma unroll
-    for (int tm = 0; tm < TM; tm++)
-#pragma unroll
-        for (int tn = 0; tn < TN; tn++)
-#pragma unroll
-            for (int i = 0; i < 16; i++) acc[tm][tn][i] = 0.0f;
-
-    // operand read offsets inside a stage
-    int a_off[TM], w_off[TN];
-#pragma unroll
-    for (int tm = 0; tm < TM; tm++) a_off[tm] = ((wm * TM + tm) * 32 + lr) * 128;
-#pragma unroll
-    for (int tn = 0; tn < TN; tn++) {
-        const int row = (wn * TN + tn) * 32 + lr;
-        if constexpr (WC == 2) w_off[tn] = A_BYTES + (row * 2 + (h ^ ((row >> 3) & 1))) * 16;
-        else w_off[tn] = A_BYTES + row * (WC * 16);   // chunk index added per read
-    }
-    const int asw = (lr >> 1) & 7;   // (row >> 1) & 7 of every activation row this lane reads
-
-    if (it0 < it1) {
-        // ---- main loop: a flat software pipeline over the MFMA steps (4 per stage).
-        //  - activation fragments are requested from LDS two steps ahead (ring of 4 register sets),
-        //  - weight words are decoded one step ahead,
-        //  - the stage hand-over (wait for the next stage, barrier, request of a further stage)
-        //    sits between steps 1 and 2; steps 2 and 3 already read the next stage's operands,
-        // so the matrix cores never wait for a whole LDS round trip.
-        auto read_w = [&](const unsigned char *sbase, uint32_t(&wq)[TN][4 * WPS]) {
-#pragma unroll
-            for (int tn = 0; tn < TN; tn++) {
-                if constexpr (WC == 2) {
-                    const u32x4 t = *reinterpret_cast<const u32x4 *>(sbase + w_off[tn]);
-                    wq[tn][0] = t[0]; wq[tn][1] = t[1]; wq[tn][2] = t[2]; wq[tn][3] = t[3];
-                } else {
-                    constexpr int CPH = WC / 2;   // chunks per lane half: 2 (8-bit types) or 4 (f16)
-                    const int row = (wn * TN + tn) * 32 + lr;
-                    const int sw = (WC == 4) ? ((row >> 2) & 3) : ((row >> 1) & 7);
-#pragma unroll
-                    for (int c = 0; c < CPH; c++) {
-                        const u32x4 t = *reinterpret_cast<const u32x4 *>(sbase + w_off[tn] + (((CPH * h + c) ^ sw) * 16));
-                        wq[tn][4 * c + 0] = t[0]; wq[tn][4 * c + 1] = t[1]; wq[tn][4 * c + 2] = t[2]; wq[tn][4 * c + 3] = t[3];
-                    }
-                }
-            }
-        };
-        auto read_a = [&](const unsigned char *sbase, int s, f16x8(&af)[TM]) {
-#pragma unroll
-            for (int tm = 0; tm < TM; tm++)
-                af[tm] = *reinterpret_cast<const f16x8 *>(sbase + a_off[tm] + (((4 * h + s) ^ asw) * 16));
-        };
-        auto decode = [&](const uint32_t(&wq)[TN][4 * WPS], int s, f16x8(&bf)[TN]) {
-#pragma unroll
-            for (int tn = 0; tn < TN; tn++) bf[tn] = D::step(&wq[tn][s * WPS]);
-        };
-        auto mfmas = [&](const f16x8(&af)[TM], const f16x8(&bf)[TN]) {
-#pragma unroll
-            for (int tm = 0; tm < TM; tm++)
-#pragma unroll
-                for (int tn = 0; tn < TN; tn++)
-                    acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[tm], bf[tn], acc[tm][tn], 0, 0, 0);
-        };
-
-#pragma unroll
-        for (int st = 0; st < NS - 1; st++) issue(it0 + st, st);
-        uint32_t wq[TN][4 * WPS], wqn[TN][4 * WPS];
-        f16x8 af[4][TM], bfr[2][TN];
-        wait_loads_but<(NS - 2) * LPS>();   // first stage: this wave's part has landed
-        __syncthreads();                    // ... and everybody else's
-        read_w(smem, wq);
-        read_a(smem, 0, af[0]);
-        read_a(smem, 1, af[1]);
-        decode(wq, 0, bfr[0]);
-        int buf = 0;
-        for (int it = it0; it < it1; it++) {
-            const unsigned char *sbase = smem + buf * STAGE;
-            const int nbuf = (buf + 1 == NS) ? 0 : buf + 1;
-            const unsigned char *nbase = smem + nbuf * STAGE;
-            const bool more = it + 1 < it1;
-            // step 0
-            read_a(sbase, 2, af[2]);
-            decode(wq, 1, bfr[1]);
-            mfmas(af[0], bfr[0]);
-            // step 1
-            read_a(sbase, 3, af[3]);
-            decode(wq, 2, bfr[0]);
-            mfmas(af[1], bfr[1]);
-            // hand-over
-            if (more) {
-                wait_loads_but<(NS - 3) * LPS>();   // this wave's part of the next stage has landed
-                __syncthreads();                    // everybody's; the stage before the current one is free
-                int fb = buf + NS - 1;
-                if (fb >= NS) fb -= NS;
-                issue(it + NS - 1, fb);
-                // step 2, with the first reads of the next stage
-                read_w(nbase, wqn);
-                read_a(nbase, 0, af[0]);
-            }
-            decode(wq, 3, bfr[1]);
-            mfmas(af[2], bfr[0]);
-            // step 3
-            if (more) {
-                read_a(nbase, 1, af[1]);
-                decode(wqn, 0, bfr[0]);
-            }
-            mfmas(af[3], bfr[1]);
-#pragma unroll
-            for (int tn = 0; tn < TN; tn++)
-#pragma unroll
-                for (int q = 0; q < 4 * WPS; q++) wq[tn][q] = wqn[tn][q];
-            buf = nbuf;
-        }
-        wait_loads_but<0>();   // nothing may still be writing LDS when the workgroup retires
-    }
-
-
-
-    // ---- epilogue.  acc[i] of a 32x32 block: row (i/4)*8 + h*4 + i%4, column lr.  With hi/lo
-    // operands a block holds 16 output rows: hi in rows 0..15 (i < 8), lo in rows 16..31 (i + 8).
-    constexpr int RPB = PRECISE ? 16 : 32;           // output rows per block
-    constexpr int NI = PRECISE ? 8 : 16;
-    const int64_t mrow0 = ((int64_t)mt * (BM / 32) + wm * TM) * RPB;
-    float sc[TN], zp[TN], bi[TN], um[TN];
-    const bool split = p.splits > 1;
-#pragma unroll
-    for (int tn = 0; tn < TN; tn++) {
-        const int64_t n = n0 + (wn * TN + tn) * 32 + lr;
-        const bool ok = n < p.n && !split;
-        sc[tn] = ok ? p.scales[n] : 0.0f;
-        zp[tn] = ok ? p.zeros[n] : 0.0f;
-        bi[tn] = (ok && p.bias) ? p.bias[n] : 0.0f;
-        um[tn] = (!PRECISE && ok && p.umean) ? p.umean[n] : 0.0f;
-    }
-#pragma unroll
-    for (int tm = 0; tm < TM; tm++)
-#pragma unroll
-        for (int i = 0; i < NI; i++) {
-            const int64_t m = mrow0 + tm * RPB + (i / 4) * 8 + h * 4 + (i % 4);
-            if (m >= p.m) continue;
-            const int e = p.rexp[m];
-            const float xs = p.xsum[m];
-            float corr = 0.0f;
-            if constexpr (!PRECISE) corr = ldexpf(p.esum[m], -e);
-#pragma unroll
-            for (int tn = 0; tn < TN; tn++) {
-                const int64_t n = n0 + (wn * TN + tn) * 32 + lr;
-                if (n >= p.n) continue;
-                float v;
-                if constexpr (PRECISE) v = acc[tm][tn][i] + acc[tm][tn][i + 8] * LO_DOWN;
-                else v = acc[tm][tn][i];
-                float d = ldexpf(v, -e);   // this workgroup's share of sum_k A[m,k]*u(W[n,k])
-                if (split) {
-                    p.part[((int64_t)z * p.m + m) * p.n + n] = d;
-                } else {
-                    if constexpr (!PRECISE) d = d - um[tn] * corr;
-                    float o = d * sc[tn] + zp[tn] * xs;
-                    if (p.bias) o = o + bi[tn];
-                    p.out[m * p.n + n] = fnn_activation(o, p.act);
-                }
-            }
-        }
-}
+#include "tile_kernel.h"
 
 // sum of the K-split partial tiles in split order + affine / bias / activation epilogue
 __global__ void __launch_bounds__(256) splitk_epilogue_kernel(TileArgs p, int single)
