@@ -26,7 +26,7 @@ struct QConvArgs {
     int64_t b, c, h, w, oc, ho, wo, kp;
     int kh, kw, stride, pad, dil, groups, act;
 };
-constexpr int QCONV_NPART = 64;
+constexpr int QCONV_NPART = 512;
 
 hipError_t launch_quantize_activations(const float *x, int64_t numel, float scale, float zp,
                                        uint8_t *payload, float *scratch_partial, hipStream_t s);

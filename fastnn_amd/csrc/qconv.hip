@@ -88,13 +88,26 @@ __global__ void __launch_bounds__(256) conv_minmax_cover_kernel(QConvArgs a, int
     const float *xg = a.x + (nn * a.c + g * cg) * a.h * a.w;
     const int64_t hw = a.h * a.w, total = cg * hw;
     float mn = pad_touched ? 0.0f : INFINITY, mx = pad_touched ? 0.0f : -INFINITY;
-    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * blockDim.x) {
-        const int64_t rem = idx % hw;
-        const int64_t ih = rem / a.w, iw = rem % a.w;
-        if (cov_h[ih] && cov_w[iw]) {
-            const float v = xg[idx];
-            mn = fminf(mn, v);
-            mx = fmaxf(mx, v);
+    if (total < (1ll << 31)) {   // 32-bit index arithmetic
+        const unsigned hw32 = (unsigned)hw, w32 = (unsigned)a.w, tot32 = (unsigned)total, stride = gridDim.x * blockDim.x;
+        for (unsigned idx = blockIdx.x * blockDim.x + threadIdx.x; idx < tot32; idx += stride) {
+            const unsigned rem = idx % hw32;
+            const unsigned ih = rem / w32, iw = rem - ih * w32;
+            if (cov_h[ih] && cov_w[iw]) {
+                const float v = xg[idx];
+                mn = fminf(mn, v);
+                mx = fmaxf(mx, v);
+            }
+        }
+    } else {
+        for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * blockDim.x) {
+            const int64_t rem = idx % hw;
+            const int64_t ih = rem / a.w, iw = rem % a.w;
+            if (cov_h[ih] && cov_w[iw]) {
+                const float v = xg[idx];
+                mn = fminf(mn, v);
+                mx = fmaxf(mx, v);
+            }
         }
     }
     mn = wave_min(mn);
@@ -256,7 +269,7 @@ hipError_t launch_qconv2d_i8(const QConvArgs &p, hipStream_t s, int phase)
                     if (iw < 0 || iw >= p.w) { pad_touched = 1; break; }
                 }
             const int64_t elems = cg * p.h * p.w;
-            nparts = (elems + 256 * 16 - 1) / (256 * 16);
+            nparts = (elems + 256 * 4 - 1) / (256 * 4);
             if (nparts > QCONV_NPART) nparts = QCONV_NPART;
             if (nparts < 1) nparts = 1;
             hipLaunchKernelGGL(conv_minmax_cover_kernel, dim3((unsigned)nparts, (unsigned)bg), dim3(256), (size_t)(p.h + p.w), s, p, pad_touched);

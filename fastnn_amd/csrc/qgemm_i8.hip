@@ -90,7 +90,7 @@ __global__ void __launch_bounds__(256) i8_matmul_epilogue_kernel(const int32_t *
 // A workgroup owns 64 consecutive rows; thread (row, slot) walks the 16-value chunks slot, slot+4, ...
 // that hold data (neighbouring lanes = neighbouring pixels: the NCHW reads coalesce), the (ic, i, j)
 // tap of a chunk is advanced by carries instead of divisions; all-zero chunks are written in a second sweep.
-constexpr int CONV_CPB = 8;   // 16-value chunks of a row per workgroup
+constexpr int CONV_CPB = 4;   // 16-value chunks of a row per workgroup (one per thread slot)
 
 __global__ void __launch_bounds__(256) conv_operand_kernel(QConvArgs a, int g, int kk, int64_t kpad, int64_t rows_pad,
                                                            int8_t *a8, int32_t *qsum)
@@ -156,40 +156,58 @@ __global__ void __launch_bounds__(256) conv_operand_kernel(QConvArgs a, int g, i
 // acc = bias_q + sum q_a*q_w; val = acc*sab + zw*(sa*sum q_a) + za*(sw*sum q_w) + (za*zw)*K, left to right,
 // then the activation (packed_conv.rs:469-505,571,604-606).  A workgroup takes 64 rows of C (read along the
 // channels, as stored), turns the tile in LDS and writes NCHW with consecutive lanes on consecutive pixels.
+constexpr int EPI_CH = 32;   // channels per epilogue workgroup
+
 __global__ void __launch_bounds__(256) conv_epilogue_kernel(QConvArgs a, int g, int kk, const int32_t *c, int ocg,
                                                             const int32_t *qsum, int nq, int64_t rows_pad)
 {
-    __shared__ float tile[64 * 65];   // [channel of the block][row], padded
-    __shared__ int itile[64 * 65];    // accumulators incl. bias_q, same shape
+    __shared__ float tile[EPI_CH * 65];   // [channel of the block][row], padded
+    __shared__ int itile[EPI_CH * 65];    // accumulators incl. bias_q, same shape
+    __shared__ float r_sa[64], r_za[64], r_sum[64];          // per row: activation scale / zero of its image, sa * sum q_a
+    __shared__ float c_sw[EPI_CH], c_zw[EPI_CH], c_wt[EPI_CH], c_bias[EPI_CH];   // per channel
     const int64_t np = a.ho * a.wo, rows = a.b * np;
     const int64_t row0 = (int64_t)blockIdx.x * 64;
-    const int f0 = blockIdx.y * 64;
-    const int fb = ocg - f0 < 64 ? ocg - f0 : 64;   // channels of this block
+    const int f0 = blockIdx.y * EPI_CH;
+    const int fb = ocg - f0 < EPI_CH ? ocg - f0 : EPI_CH;   // channels of this block
     const int tid = threadIdx.x;
+    if (tid < 64) {
+        const int64_t r = row0 + tid;
+        if (r < rows) {
+            const int bg = (int)((r / np) * a.groups + g);
+            const float sa = a.actq[bg * 4 + 0];
+            int qs = 0;
+            for (int y = 0; y < nq; y++) qs += qsum[(int64_t)y * rows_pad + r];
+            r_sa[tid] = sa;
+            r_za[tid] = a.actq[bg * 4 + 1];
+            r_sum[tid] = sa * (float)qs;
+        }
+    } else if (tid < 64 + fb) {
+        const int fl = tid - 64;
+        const int64_t ch = (int64_t)g * ocg + f0 + fl;
+        const float sw = a.scales[ch];
+        c_sw[fl] = sw;
+        c_zw[fl] = a.zeros[ch];
+        c_wt[fl] = sw * (float)a.row_qsum[ch];
+        c_bias[fl] = a.bias ? a.bias[ch] : 0.0f;
+    }
+    __syncthreads();
     for (int idx = tid; idx < 64 * fb; idx += 256) {
-        const int rr = idx / fb, fl = idx % fb, f = f0 + fl;
+        const int rr = idx / fb, fl = idx - rr * fb;
         const int64_t r = row0 + rr;
         if (r >= rows) continue;
-        const int64_t nn = r / np;
-        const int64_t ch = (int64_t)g * ocg + f;
-        const int bg = (int)(nn * a.groups + g);
-        const float sa = a.actq[bg * 4 + 0], za = a.actq[bg * 4 + 1];
-        const float sw = a.scales[ch], zw = a.zeros[ch];
+        const float sa = r_sa[rr], za = r_za[rr];
+        const float sw = c_sw[fl], zw = c_zw[fl];
         const float sab = sa * sw;
         int bias_q = 0;
         if (a.bias) {
-            const float bq = roundf(a.bias[ch] / sab);
+            const float bq = roundf(c_bias[fl] / sab);
             bias_q = (bq != bq) ? 0 : (bq >= 2147483648.0f ? 2147483647 : (bq <= -2147483648.0f ? (-2147483647 - 1) : (int)bq));
         }
-        const int accv = c[r * ocg + f] + bias_q;
-        int qs = 0;
-        for (int y = 0; y < nq; y++) qs += qsum[(int64_t)y * rows_pad + r];
-        const float rsum = sa * (float)qs;
-        const float w_term = sw * (float)a.row_qsum[ch];
+        const int accv = c[r * ocg + f0 + fl] + bias_q;
         const float zp_prod = za * zw;
         float val = (float)accv * sab;
-        val = val + zw * rsum;
-        val = val + za * w_term;
+        val = val + zw * r_sum[rr];
+        val = val + za * c_wt[fl];
         val = val + zp_prod * (float)kk;
         if (a.act == FNN_ACT_RELU) val = fmaxf(val, 0.0f);
         else if (a.act == FNN_ACT_SILU) val = val / (1.0f + expf(-val));
@@ -198,14 +216,17 @@ __global__ void __launch_bounds__(256) conv_epilogue_kernel(QConvArgs a, int g, 
         itile[fl * 65 + rr] = accv;
     }
     __syncthreads();
-    for (int idx = tid; idx < 64 * fb; idx += 256) {
-        const int fl = idx / 64, rr = idx % 64;
-        const int64_t r = row0 + rr;
-        if (r >= rows) continue;
-        const int64_t nn = r / np, p = r % np;
-        const int64_t o = (nn * a.oc + (int64_t)g * ocg + f0 + fl) * np + p;
-        a.y[o] = tile[fl * 65 + rr];
-        if (a.acc_out) a.acc_out[o] = itile[fl * 65 + rr];
+    // NCHW stores: consecutive lanes on consecutive pixels
+    const int rr = tid & 63;
+    const int64_t r = row0 + rr;
+    if (r < rows) {
+        const int64_t nn = (rows < (1ll << 31)) ? (int64_t)((unsigned)r / (unsigned)np) : r / np;
+        const int64_t p = r - nn * np;
+        for (int fl = tid >> 6; fl < fb; fl += 4) {
+            const int64_t o = (nn * a.oc + (int64_t)g * ocg + f0 + fl) * np + p;
+            a.y[o] = tile[fl * 65 + rr];
+            if (a.acc_out) a.acc_out[o] = itile[fl * 65 + rr];
+        }
     }
 }
 
@@ -348,14 +369,14 @@ int fnn_i8_tiled_conv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, 
     int8_t *a8 = (int8_t *)ws3;
     int32_t *qsum = (int32_t *)((char *)ws3 + q_off);
     int32_t *c = (int32_t *)ws1;
-    if (ocg > 65535 * 64) return FNN_OK;
+    if (ocg > 65535 * EPI_CH) return FNN_OK;
     for (int g = 0; g < p.groups; g++) {
         const dim3 grid((unsigned)(rows_pad / 64), (unsigned)nq);
         hipLaunchKernelGGL(conv_operand_kernel, grid, dim3(256), 0, s, p, g, (int)kk, kpad, rows_pad, a8, qsum);
         hipError_t e = hipGetLastError();
         if (e == hipSuccess) e = run_i8_gemm<FNN_DT_I8>(words, kp, w->rows, g * ocg, ocg, a8, rows, rows_pad, kpad, c, ocg, s);
         if (e == hipSuccess) {
-            hipLaunchKernelGGL(conv_epilogue_kernel, dim3((unsigned)((rows + 63) / 64), (unsigned)((ocg + 63) / 64)), dim3(256), 0, s, p, g,
+            hipLaunchKernelGGL(conv_epilogue_kernel, dim3((unsigned)((rows + 63) / 64), (unsigned)((ocg + EPI_CH - 1) / EPI_CH)), dim3(256), 0, s, p, g,
                                (int)kk, c, (int)ocg, qsum, nq, rows_pad);
             e = hipGetLastError();
         }
