@@ -104,24 +104,24 @@ __global__ void __launch_bounds__(256) qgemm_tile_kernel(TileArgs p)
     for (int j = 0; j < A_LPW; j++) a_src[j] += (int64_t)(p.a_wrap ? it0 % p.a_wrap : it0) * a_step;
 #pragma unroll
     for (int j = 0; j < W_LPW; j++) w_src[j] += (int64_t)it0 * (WC * 4);
+    int a_pos = p.a_wrap ? it0 % p.a_wrap : 0;    // position inside the activation sweep
     const bool ragged = (p.kp % (WC * 4)) != 0;   // the last stage of a row is partly past its end
     auto issue = [&](int it, int buf) {
         const unsigned sb = buf * STAGE;
-        if (ragged && it >= p.iters - 1) {
+        const bool last_ragged = ragged && it >= p.iters - 1;   // wave-uniform; folded into selects, no branch
 #pragma unroll
-            for (int j = 0; j < W_LPW; j++) {
-                const bool ok = (int64_t)(p.iters - 1) * (WC * 4) + w_chunk[j] + 4 <= p.kp;
-                load_to_lds16(ok ? w_src[j] : p.zero_chunk, w_dst + sb + j * 1024);
-            }
-        } else {
-#pragma unroll
-            for (int j = 0; j < W_LPW; j++) load_to_lds16(w_src[j], w_dst + sb + j * 1024);
+        for (int j = 0; j < W_LPW; j++) {
+            const bool past = last_ragged && ((int64_t)(p.iters - 1) * (WC * 4) + w_chunk[j] + 4 > p.kp);
+            load_to_lds16(past ? p.zero_chunk : w_src[j], w_dst + sb + j * 1024);
         }
 #pragma unroll
         for (int j = 0; j < A_LPW; j++) load_to_lds16(a_src[j], a_dst + sb + j * 1024);
         const bool more = it + 1 < it1;           // wave-uniform
         int64_t astep = more ? a_step : 0;
-        if (p.a_wrap && more && (it + 1) % p.a_wrap == 0) astep = -(int64_t)(p.a_wrap - 1) * a_step;
+        if (p.a_wrap && more && ++a_pos == p.a_wrap) {   // second sweep over the activations
+            a_pos = 0;
+            astep = -(int64_t)(p.a_wrap - 1) * a_step;
+        }
         const int wstep = more ? WC * 4 : 0;
 #pragma unroll
         for (int j = 0; j < A_LPW; j++) a_src[j] += astep;
@@ -206,12 +206,14 @@ __global__ void __launch_bounds__(256) qgemm_tile_kernel(TileArgs p)
         read_a(smem, 0, af[0]);
         read_a(smem, 1, af[1]);
         decode(wq, 0, bfr[0]);
+        // The loop body is one straight-line block (no branches), so the compiler can interleave LDS
+        // reads, decode and MFMAs across the whole stage; the last stage, which has no successor to
+        // hand over to, is peeled off.
         int buf = 0;
-        for (int it = it0; it < it1; it++) {
+        for (int it = it0; it < it1 - 1; it++) {
             const unsigned char *sbase = smem + buf * STAGE;
             const int nbuf = (buf + 1 == NS) ? 0 : buf + 1;
             const unsigned char *nbase = smem + nbuf * STAGE;
-            const bool more = it + 1 < it1;
             // step 0
             read_a(sbase, 2, af[2]);
             decode(wq, 1, bfr[1]);
@@ -221,29 +223,37 @@ __global__ void __launch_bounds__(256) qgemm_tile_kernel(TileArgs p)
             decode(wq, 2, bfr[0]);
             mfmas(af[1], bfr[1]);
             // hand-over
-            if (more) {
-                wait_loads_but<(NS - 3) * LPS>();   // this wave's part of the next stage has landed
-                __syncthreads();                    // everybody's; the stage before the current one is free
-                int fb = buf + NS - 1;
-                if (fb >= NS) fb -= NS;
-                issue(it + NS - 1, fb);
-                // step 2, with the first reads of the next stage
-                read_w(nbase, wqn);
-                read_a(nbase, 0, af[0]);
-            }
+            wait_loads_but<(NS - 3) * LPS>();   // this wave's part of the next stage has landed
+            __syncthreads();                    // everybody's; the stage before the current one is free
+            int fb = buf + NS - 1;
+            if (fb >= NS) fb -= NS;
+            issue(it + NS - 1, fb);
+            // step 2, with the first reads of the next stage
+            read_w(nbase, wqn);
+            read_a(nbase, 0, af[0]);
             decode(wq, 3, bfr[1]);
             mfmas(af[2], bfr[0]);
             // step 3
-            if (more) {
-                read_a(nbase, 1, af[1]);
-                decode(wqn, 0, bfr[0]);
-            }
+            read_a(nbase, 1, af[1]);
+            decode(wqn, 0, bfr[0]);
             mfmas(af[3], bfr[1]);
 #pragma unroll
             for (int tn = 0; tn < TN; tn++)
 #pragma unroll
                 for (int q = 0; q < 4 * WPS; q++) wq[tn][q] = wqn[tn][q];
             buf = nbuf;
+        }
+        {   // last stage
+            const unsigned char *sbase = smem + buf * STAGE;
+            read_a(sbase, 2, af[2]);
+            decode(wq, 1, bfr[1]);
+            mfmas(af[0], bfr[0]);
+            read_a(sbase, 3, af[3]);
+            decode(wq, 2, bfr[0]);
+            mfmas(af[1], bfr[1]);
+            decode(wq, 3, bfr[1]);
+            mfmas(af[2], bfr[0]);
+            mfmas(af[3], bfr[1]);
         }
         wait_loads_but<0>();   // nothing may still be writing LDS when the workgroup retires
     }
