@@ -287,13 +287,25 @@ int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QM
     const int64_t m_pad = precise ? rows_pad / 2 : rows_pad;
     const int passes = dense ? 2 : 1;
     const int iters = (int)(kpad / BK) * passes;
-    // few tiles: split K until about two workgroups per CU are in flight
+    // Split K over workgroups when the tiles alone do not fill the 256 CUs.  The factor minimises a
+    // small cost model in microseconds, fitted to sweeps over the split factor on the benchmark shapes:
+    // stages per workgroup x time a CU needs per stage x workgroups per CU (a CU gets through
+    // stages at the same rate with one or several workgroups resident, but a lone workgroup cannot
+    // hide its load latency: factor 1.5), plus, for s > 1, the write + read of s partial [M,N] tiles.
     static const int env_split = env_int("FNN_TILE_SPLIT", 0);
-    static const int env_target = env_int("FNN_TILE_TARGET", 512);
-    int splits = 1;
     const int base = mtiles * ntiles;
-    if (base < 256) splits = (env_target + base - 1) / base;
-    if (splits > 32) splits = 32;
+    const double t_bits = DecH<DT>::WPS == 1 ? 0.4 : (DecH<DT>::WPS == 2 ? 0.7 : 1.0);
+    const double t_stage = t_bits * (cfg == 0 ? 1.0 : (cfg == 1 ? 0.5 : 0.25));
+    const double part_us = (double)M * (double)N * 8.0 / 3.0e6;
+    int splits = 1;
+    double best = 1e30;
+    for (int sp = 1; sp <= 32 && sp <= (iters / 4 > 0 ? iters / 4 : 1); sp++) {
+        const int per = (iters + sp - 1) / sp;
+        const double r = (double)base * sp / 256.0;
+        const double wgs = r <= 1.0 ? 1.5 : (double)(int64_t)(r + 0.95);
+        const double cost = per * t_stage * wgs + (sp > 1 ? 2.0 * sp * part_us : 0.0);
+        if (cost < best - 1e-9) { best = cost; splits = sp; }
+    }
     if (env_split > 0) splits = env_split;
     if (splits > iters / 4) splits = iters / 4 > 0 ? iters / 4 : 1;
     int ips = (iters + splits - 1) / splits;
@@ -345,7 +357,10 @@ int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QM
         t.a_wrap = (int)(kpad / BK);
     }
     t.act = q.act; t.splits = splits; t.iters = iters; t.ips = ips; t.mtiles = mtiles; t.ntiles = ntiles;
-    if (precise) {
+    static const int env_ns = env_int("FNN_TILE_NS", 0);
+    const bool deep = cfg == 0 && (env_ns == 5 || (env_ns == 0 && base * splits <= 256));
+    if (deep) e = precise ? launch_tile<DT, 2, 2, 2, 2, true, 5>(t, s) : launch_tile<DT, 2, 2, 2, 2, false, 5>(t, s);
+    else if (precise) {
         if (cfg == 0) e = launch_tile<DT, 2, 2, 2, 2, true, 3>(t, s);
         else if (cfg == 1) e = launch_tile<DT, 1, 4, 2, 1, true, 4>(t, s);
         else e = launch_tile<DT, 1, 4, 1, 1, true, 6>(t, s);

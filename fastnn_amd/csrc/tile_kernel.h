@@ -98,27 +98,37 @@ __global__ void __launch_bounds__(256) qgemm_tile_kernel(TileArgs p)
     const unsigned a_dst = __builtin_amdgcn_readfirstlane(lds0 + wv * A_LPW * 1024);
     const unsigned w_dst = __builtin_amdgcn_readfirstlane(lds0 + A_BYTES + wv * W_LPW * 1024);
 
+    // dense f16 weights ([hi | lo] halves): rows are whole stages long and the activations are swept twice;
+    // packed weights: one sweep, and the last stage of a row may be partly past its end
+    constexpr bool DENSE = !INT8 && D::WPS == 4;
     // running source pointers: advanced after every stage, frozen once the K range is exhausted
     // (the extra requests of the last iterations re-read the final stage and are never consumed)
 #pragma unroll
-    for (int j = 0; j < A_LPW; j++) a_src[j] += (int64_t)(p.a_wrap ? it0 % p.a_wrap : it0) * a_step;
+    for (int j = 0; j < A_LPW; j++) a_src[j] += (int64_t)(DENSE ? it0 % p.a_wrap : it0) * a_step;
 #pragma unroll
     for (int j = 0; j < W_LPW; j++) w_src[j] += (int64_t)it0 * (WC * 4);
-    int a_pos = p.a_wrap ? it0 % p.a_wrap : 0;    // position inside the activation sweep
-    const bool ragged = (p.kp % (WC * 4)) != 0;   // the last stage of a row is partly past its end
+    int a_pos = DENSE ? it0 % p.a_wrap : 0;       // position inside the activation sweep
+    const bool ragged = !DENSE && (p.kp % (WC * 4)) != 0;
+    bool w_past[W_LPW];   // this lane's chunk of the last stage lies behind the end of the row
+#pragma unroll
+    for (int j = 0; j < W_LPW; j++) w_past[j] = (int64_t)(p.iters - 1) * (WC * 4) + w_chunk[j] + 4 > p.kp;
     auto issue = [&](int it, int buf) {
         const unsigned sb = buf * STAGE;
         const bool last_ragged = ragged && it >= p.iters - 1;   // wave-uniform; folded into selects, no branch
 #pragma unroll
         for (int j = 0; j < W_LPW; j++) {
-            const bool past = last_ragged && ((int64_t)(p.iters - 1) * (WC * 4) + w_chunk[j] + 4 > p.kp);
-            load_to_lds16(past ? p.zero_chunk : w_src[j], w_dst + sb + j * 1024);
+            // both addresses are read into values first: a select between the memory locations
+            // would keep the pointer array in scratch memory
+            const uint64_t wa = reinterpret_cast<uint64_t>(w_src[j]);
+            const uint64_t za = reinterpret_cast<uint64_t>(p.zero_chunk);
+            const uint64_t mask = (last_ragged && w_past[j]) ? ~0ull : 0ull;
+            load_to_lds16(reinterpret_cast<const void *>((wa & ~mask) | (za & mask)), w_dst + sb + j * 1024);
         }
 #pragma unroll
         for (int j = 0; j < A_LPW; j++) load_to_lds16(a_src[j], a_dst + sb + j * 1024);
         const bool more = it + 1 < it1;           // wave-uniform
         int64_t astep = more ? a_step : 0;
-        if (p.a_wrap && more && ++a_pos == p.a_wrap) {   // second sweep over the activations
+        if (DENSE && more && ++a_pos == p.a_wrap) {   // second sweep over the activations
             a_pos = 0;
             astep = -(int64_t)(p.a_wrap - 1) * a_step;
         }
@@ -296,16 +306,30 @@ __global__ void __launch_bounds__(256) qgemm_tile_kernel(TileArgs p)
         bi[tn] = (ok && p.bias) ? p.bias[n] : 0.0f;
         um[tn] = (!PRECISE && ok && p.umean) ? p.umean[n] : 0.0f;
     }
+    // row constants of every output row this lane holds, requested together (clamped rows, masked
+    // later) so that their latencies overlap instead of chaining behind the stores
+    int rexp[TM][NI];
+    float rxs[TM][NI], rcorr[TM][NI];
+#pragma unroll
+    for (int tm = 0; tm < TM; tm++)
+#pragma unroll
+        for (int i = 0; i < NI; i++) {
+            int64_t m = mrow0 + tm * RPB + (i / 4) * 8 + h * 4 + (i % 4);
+            if (m > p.m - 1) m = p.m - 1;
+            rexp[tm][i] = p.rexp[m];
+            rxs[tm][i] = split ? 0.0f : p.xsum[m];
+            rcorr[tm][i] = (!PRECISE && !split) ? p.esum[m] : 0.0f;
+        }
 #pragma unroll
     for (int tm = 0; tm < TM; tm++)
 #pragma unroll
         for (int i = 0; i < NI; i++) {
             const int64_t m = mrow0 + tm * RPB + (i / 4) * 8 + h * 4 + (i % 4);
             if (m >= p.m) continue;
-            const int e = p.rexp[m];
-            const float xs = p.xsum[m];
+            const int e = rexp[tm][i];
+            const float xs = rxs[tm][i];
             float corr = 0.0f;
-            if constexpr (!PRECISE) corr = ldexpf(p.esum[m], -e);
+            if constexpr (!PRECISE) corr = ldexpf(rcorr[tm][i], -e);
 #pragma unroll
             for (int tn = 0; tn < TN; tn++) {
                 const int64_t n = n0 + (wn * TN + tn) * 32 + lr;
@@ -325,4 +349,3 @@ __global__ void __launch_bounds__(256) qgemm_tile_kernel(TileArgs p)
             }
         }
 }
-
