@@ -46,6 +46,11 @@ class ExecutablePlan:
     def __len__(self):
         return int(self.lib.fnn_plan_len(self.handle))
 
+    @property
+    def replayed(self) -> bool:
+        """True when the last dispatch of this plan ran as a HIP-graph replay."""
+        return bool(self.lib.fnn_plan_replayed(self.handle))
+
     def _ok(self, rc, what):
         if rc:
             raise FnnError(rc, f"{what}: malformed instruction")

@@ -41,6 +41,7 @@ struct fnn_hip_ctx {
     Staging st_a, st_out, st_bias, st_acc, st_tmp, st_tmp2, st_tmp3, st_cnt;
     float *scratch = nullptr;  // small reduction scratch (partials)
     bool capturing = false;
+    uint64_t ws_epoch = 0;     // bumped whenever a staging buffer is re-allocated (captured graphs go stale)
 };
 
 namespace {
@@ -78,6 +79,7 @@ int ensure(fnn_hip_ctx *ctx, Staging &s, size_t bytes)
     size_t cap = bytes < 4096 ? 4096 : bytes;
     HIP_TRY(ctx, FNN_ERR_MEMORY, hipMalloc(&s.ptr, cap));
     s.cap = cap;
+    ctx->ws_epoch++;
     return FNN_OK;
 }
 
@@ -674,6 +676,8 @@ int fnn_hip_graph_launch(fnn_hip_ctx *ctx, fnn_hip_graph *g)
     HIP_TRY(ctx, FNN_ERR_DISPATCH, hipGraphLaunch(g->exec, ctx->stream));
     return FNN_OK;
 }
+
+uint64_t fnn_hip_workspace_epoch(const fnn_hip_ctx *ctx) { return ctx ? ctx->ws_epoch : 0; }
 
 int fnn_hip_graph_destroy(fnn_hip_ctx *ctx, fnn_hip_graph *g)
 {

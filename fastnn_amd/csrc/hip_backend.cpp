@@ -8,9 +8,11 @@
 // (src/backend/cpu/mod.rs:4106-4260) for the nine Conv2d params.  A kernel name that has
 // no GPU implementation yields FNN_ERR_UNSUPPORTED_OP naming the kernel, so that a
 // caller can run that one instruction elsewhere (src/backend/wgpu/mod.rs:162-239).
+#include <atomic>
 #include <chrono>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <map>
 #include <string>
@@ -87,16 +89,31 @@ struct fnn_plan {
     uint64_t arena_size = 0;
     std::vector<Instr> instrs;
     bool analysed = false;
-    // WriteConst payloads stay valid in the arena of this backend at this generation
-    const fnn_backend *resident_on = nullptr;
+    bool uploads_every_run = false;   // some WriteConst target is overwritten by the plan itself
+    // WriteConst payloads stay valid in the arena of this backend (by unique id) at this generation
+    uint64_t resident_uid = 0;
     uint64_t resident_generation = 0;
+    uint64_t resident_seq = 0;        // host writes up to this sequence number are accounted for
+    // HIP graph of the instruction stream, captured on a dispatch that found everything resident;
+    // valid while the backend, its arena, its cached weights and the context's workspaces are the same
+    fnn_hip_graph *graph = nullptr;
+    uint64_t graph_uid = 0, graph_generation = 0, graph_weights_epoch = 0, graph_ws_epoch = 0;
+    int graph_failures = 0;           // captures that did not go through; after two the plan stays eager
+    bool last_replayed = false;
 };
 
 struct fnn_backend {
     fnn_hip_ctx *ctx = nullptr;
     uint8_t *arena = nullptr;
     uint64_t arena_bytes = 0;
-    uint64_t generation = 1;  // bumped whenever the host rewrites the arena
+    uint64_t uid = 0;         // never reused within the process
+    uint64_t generation = 1;  // bumped when the arena is re-allocated or the write log overflows
+    // host writes into the arena since the backend was created: (sequence number, byte range).
+    // A plan's constants stay resident across a write that touches none of them (the usual
+    // "write the input, dispatch, read the output" cycle uploads the weights only once).
+    uint64_t write_seq = 0;
+    std::vector<std::pair<uint64_t, fnn_slice>> host_writes;
+    uint64_t weights_epoch = 0;  // bumped whenever a cached device weight is created or released
     std::string err;
     std::map<std::pair<uint64_t, uint64_t>, fnn_hip_weight *> weights;  // (offset,size) like get_or_cache_packed
     std::vector<uint8_t> stage;
@@ -133,6 +150,7 @@ void drop_weights(fnn_backend *b)
 {
     for (auto &kv : b->weights) fnn_hip_weight_release(b->ctx, kv.second);
     b->weights.clear();
+    b->weights_epoch++;
 }
 
 void drop_weights_overlapping(fnn_backend *b, const fnn_slice &s)
@@ -142,6 +160,7 @@ void drop_weights_overlapping(fnn_backend *b, const fnn_slice &s)
         if (overlaps(w, s)) {
             fnn_hip_weight_release(b->ctx, it->second);
             it = b->weights.erase(it);
+            b->weights_epoch++;
         } else {
             ++it;
         }
@@ -180,6 +199,7 @@ int weight_for(fnn_backend *b, const fnn_slice &ws, int dtype, const Meta &meta,
                                          (int64_t)rows, (int64_t)inner, sc, nsc, zp, nzp, qb, cb, &w));
     if (st) return st;
     b->weights[key] = w;
+    b->weights_epoch++;
     *out = w;
     return FNN_OK;
 }
@@ -330,6 +350,7 @@ void analyse(fnn_plan *p)
             if (&o == &c) continue;
             if (overlaps(o.dst, c.dst)) { c.clobbered = true; break; }
         }
+        if (c.clobbered && !c.data.empty()) p->uploads_every_run = true;
     }
     p->analysed = true;
 }
@@ -370,7 +391,57 @@ int dispatch_impl(fnn_backend *b, fnn_plan *p, uint64_t *elapsed_ns, uint64_t n_
     if (p->arena_size > b->arena_bytes) return fail(b, FNN_ERR_MEMORY, "dispatch: plan needs an arena of %llu bytes, backend holds %llu", (unsigned long long)p->arena_size, (unsigned long long)b->arena_bytes);
     if (elapsed_ns && n_elapsed < p->instrs.size()) return fail(b, FNN_ERR_DISPATCH, "dispatch_profile: room for %llu timings, plan has %llu instructions", (unsigned long long)n_elapsed, (unsigned long long)p->instrs.size());
     if (!p->analysed) analyse(p);
-    bool resident = p->resident_on == b && p->resident_generation == b->generation;
+    bool resident = p->resident_uid == b->uid && p->resident_generation == b->generation;
+    if (resident && p->resident_seq != b->write_seq) {
+        // the host wrote into the arena since: still resident unless a constant was hit
+        for (const auto &hw : b->host_writes) {
+            if (hw.first <= p->resident_seq) continue;
+            for (const auto &c : p->instrs)
+                if (c.kind == K_WRITE_CONST && overlaps(c.dst, hw.second)) { resident = false; break; }
+            if (!resident) break;
+        }
+        if (resident) p->resident_seq = b->write_seq;
+    }
+
+    // Replay: a plan whose constants are in place, whose weights are all cached and whose
+    // workspaces have their final size launches as one HIP graph (the executor's static-shape
+    // plan, src/backend/executor.rs:639-667).  Profiling, re-uploaded constants and anything
+    // that fails under capture keep the instruction-by-instruction path.
+    static const bool graphs_on = [] { const char *e = getenv("FNN_PLAN_GRAPH"); return !(e && e[0] == '0'); }();
+    const bool may_replay = graphs_on && !elapsed_ns && resident && !p->uploads_every_run && p->graph_failures < 2;
+    if (p->graph && !(may_replay && p->graph_uid == b->uid && p->graph_generation == b->generation &&
+                      p->graph_weights_epoch == b->weights_epoch && p->graph_ws_epoch == fnn_hip_workspace_epoch(b->ctx))) {
+        fnn_hip_graph_destroy(p->graph_uid == b->uid ? b->ctx : nullptr, p->graph);
+        p->graph = nullptr;
+    }
+    if (may_replay && !p->graph) {
+        const uint64_t w0 = b->weights_epoch, s0 = fnn_hip_workspace_epoch(b->ctx);
+        if (fnn_hip_graph_begin(b->ctx) == FNN_OK) {
+            int st = FNN_OK;
+            for (size_t i = 0; i < p->instrs.size() && st == FNN_OK; i++) st = run_instr(b, p, p->instrs[i], true);
+            fnn_hip_graph *g = nullptr;
+            int en = fnn_hip_graph_end(b->ctx, &g);
+            if (st == FNN_OK && en == FNN_OK && g && w0 == b->weights_epoch && s0 == fnn_hip_workspace_epoch(b->ctx)) {
+                p->graph = g;
+                p->graph_uid = b->uid; p->graph_generation = b->generation;
+                p->graph_weights_epoch = w0; p->graph_ws_epoch = s0;
+            } else {
+                if (g) fnn_hip_graph_destroy(b->ctx, g);
+                p->graph_failures++;
+                b->err.clear();
+            }
+        } else {
+            p->graph_failures++;
+        }
+    }
+    p->last_replayed = false;
+    if (p->graph) {
+        int st = lift(b, fnn_hip_graph_launch(b->ctx, p->graph));
+        if (st == FNN_OK) st = lift(b, fnn_hip_sync(b->ctx));
+        p->last_replayed = st == FNN_OK;
+        return st;
+    }
+
     for (size_t i = 0; i < p->instrs.size(); i++) {
         auto t0 = std::chrono::steady_clock::now();
         int st = run_instr(b, p, p->instrs[i], resident);
@@ -383,8 +454,9 @@ int dispatch_impl(fnn_backend *b, fnn_plan *p, uint64_t *elapsed_ns, uint64_t n_
     }
     int st = lift(b, fnn_hip_sync(b->ctx));
     if (st == FNN_OK) {
-        p->resident_on = b;
+        p->resident_uid = b->uid;
         p->resident_generation = b->generation;
+        p->resident_seq = b->write_seq;
     }
     return st;
 }
@@ -400,7 +472,9 @@ int fnn_backend_create(int device, fnn_backend **out)
     fnn_hip_ctx *ctx = nullptr;
     int st = fnn_hip_create(device, &ctx);
     if (st) return st;
+    static std::atomic<uint64_t> next_uid{1};
     fnn_backend *b = new fnn_backend();
+    b->uid = next_uid++;
     b->ctx = ctx;
     *out = b;
     return FNN_OK;
@@ -449,7 +523,13 @@ int fnn_backend_write_arena(fnn_backend *b, uint64_t offset, const void *data, u
     if (size == 0) return FNN_OK;
     if (!data) return fail(b, FNN_ERR_DISPATCH, "write_arena: NULL data");
     drop_weights_overlapping(b, s);
-    b->generation++;
+    b->write_seq++;
+    if (b->host_writes.size() >= 256) {   // forget the log: every plan uploads its constants again
+        b->host_writes.clear();
+        b->generation++;
+    } else {
+        b->host_writes.emplace_back(b->write_seq, s);
+    }
     return lift(b, fnn_hip_upload(b->ctx, b->arena + offset, data, size));
 }
 
@@ -471,14 +551,26 @@ int fnn_plan_create(uint64_t arena_size, fnn_plan **out)
     return FNN_OK;
 }
 
-void fnn_plan_destroy(fnn_plan *p) { delete p; }
+void fnn_plan_destroy(fnn_plan *p)
+{
+    if (!p) return;
+    if (p->graph) fnn_hip_graph_destroy(nullptr, p->graph);   // every dispatch ends with a sync: nothing in flight
+    delete p;
+}
 
 uint64_t fnn_plan_len(const fnn_plan *p) { return p ? p->instrs.size() : 0; }
+
+int fnn_plan_replayed(const fnn_plan *p) { return p && p->last_replayed ? 1 : 0; }
 
 static void touched(fnn_plan *p)
 {
     p->analysed = false;
-    p->resident_on = nullptr;
+    p->uploads_every_run = false;
+    p->resident_uid = 0;
+    if (p->graph) {
+        fnn_hip_graph_destroy(nullptr, p->graph);
+        p->graph = nullptr;
+    }
 }
 
 int fnn_plan_add_write_const(fnn_plan *p, fnn_slice dst, const void *data, uint64_t len)

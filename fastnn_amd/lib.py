@@ -33,6 +33,7 @@ EXPORTED_SYMBOLS = [
     "fnn_hip_qmatmul", "fnn_hip_quantize_activations", "fnn_hip_qmatmul_i8act", "fnn_hip_qconv2d",
     "fnn_hip_timer_start", "fnn_hip_timer_stop", "fnn_hip_probe_stream",
     "fnn_hip_graph_begin", "fnn_hip_graph_end", "fnn_hip_graph_launch", "fnn_hip_graph_destroy",
+    "fnn_hip_workspace_epoch",
     "fnn_packed_words", "fnn_quantize_weights", "fnn_transpose_kn_to_nk", "fnn_hip_version",
 ]
 # every symbol include/fastnn_hip_backend.h declares
@@ -40,7 +41,7 @@ BACKEND_SYMBOLS = [
     "fnn_backend_create", "fnn_backend_destroy", "fnn_backend_name", "fnn_backend_last_error",
     "fnn_backend_allocate_arena", "fnn_backend_write_arena", "fnn_backend_read_arena",
     "fnn_plan_create", "fnn_plan_destroy", "fnn_plan_add_write_const", "fnn_plan_add_fill",
-    "fnn_plan_add_memcopy", "fnn_plan_add_call_kernel", "fnn_plan_len",
+    "fnn_plan_add_memcopy", "fnn_plan_add_call_kernel", "fnn_plan_len", "fnn_plan_replayed",
     "fnn_backend_dispatch", "fnn_backend_dispatch_profile",
     "fnn_hip_elementwise", "fnn_hip_fill_f32", "fnn_hip_copy",
 ]
@@ -123,6 +124,8 @@ def _prototype(l):
     l.fnn_hip_graph_end.argtypes = [_vp, C.POINTER(_vp)]
     l.fnn_hip_graph_launch.argtypes = [_vp, _vp]
     l.fnn_hip_graph_destroy.argtypes = [_vp, _vp]
+    l.fnn_hip_workspace_epoch.argtypes = [_vp]
+    l.fnn_hip_workspace_epoch.restype = _u64
     l.fnn_packed_words.argtypes = [C.c_int, _i64, _i64]
     l.fnn_packed_words.restype = _sz
     l.fnn_quantize_weights.argtypes = [C.c_int, _vp, _i64, _i64, C.c_int, _vp, _vp, _vp, _vp]
@@ -149,6 +152,8 @@ def _prototype(l):
                                            C.POINTER(WeightMeta)]
     l.fnn_plan_len.argtypes = [_vp]
     l.fnn_plan_len.restype = _u64
+    l.fnn_plan_replayed.argtypes = [_vp]
+    l.fnn_plan_replayed.restype = C.c_int
     l.fnn_backend_dispatch.argtypes = [_vp, _vp]
     l.fnn_backend_dispatch_profile.argtypes = [_vp, _vp, C.POINTER(_u64), _u64]
     l.fnn_hip_elementwise.argtypes = [_vp, C.c_int, _vp, _vp, _u64, _vp, _u64]

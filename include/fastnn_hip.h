@@ -151,6 +151,10 @@ int fnn_hip_graph_begin(fnn_hip_ctx *ctx);
 int fnn_hip_graph_end(fnn_hip_ctx *ctx, fnn_hip_graph **out);
 int fnn_hip_graph_launch(fnn_hip_ctx *ctx, fnn_hip_graph *g);
 int fnn_hip_graph_destroy(fnn_hip_ctx *ctx, fnn_hip_graph *g);
+/* Counts how often the context re-allocated one of its internal workspaces (no counterpart in
+ * fastnn).  A captured graph holds the workspace addresses of its capture: when the count has
+ * changed since, the graph is stale and must be captured again instead of launched. */
+uint64_t fnn_hip_workspace_epoch(const fnn_hip_ctx *ctx);
 
 /* ---- host-side weight quantisers (no GPU needed): the packers the
  * quantisation pass calls (src/compiler/passes/quantization.rs:170-260,

@@ -63,8 +63,16 @@ int fnn_plan_add_call_kernel(fnn_plan *p, const char *kernel_name, const fnn_sli
                              uint64_t n_params, const fnn_weight_meta *meta);
 uint64_t fnn_plan_len(const fnn_plan *p);
 
-/* Backend::dispatch, src/backend/mod.rs:167-176.  Synchronises before returning. */
+/* Backend::dispatch, src/backend/mod.rs:167-176.  Synchronises before returning.
+ * The first dispatch of a plan uploads its WriteConst payloads and runs instruction by
+ * instruction; while the constants stay in place (fnn_backend_write_arena elsewhere in the arena
+ * does not disturb them) later dispatches skip the uploads and replay the instruction stream as
+ * one HIP graph, the static-shape plan reuse of src/backend/executor.rs:639-667.
+ * FNN_PLAN_GRAPH=0 in the environment keeps every dispatch instruction by instruction. */
 int fnn_backend_dispatch(fnn_backend *b, fnn_plan *p);
+/* 1 when the last dispatch of the plan ran as a graph replay, else 0 (no counterpart in fastnn:
+ * lets tests and tools see which path ran). */
+int fnn_plan_replayed(const fnn_plan *p);
 /* Backend::dispatch_profile, src/backend/mod.rs:178-211: elapsed_ns[i] per instruction */
 int fnn_backend_dispatch_profile(fnn_backend *b, fnn_plan *p, uint64_t *elapsed_ns, uint64_t n);
 

@@ -229,3 +229,69 @@ def test_rewritten_weights_are_re_registered(be, orc):
         plan = ExecutablePlan(a.top).call_kernel("matmul_i8", [s_x, s_w], s_o, [m, k, n], meta_of(pw))
         be.dispatch(plan)
         assert_close(be.read_arena(*s_o, np.float32).reshape(m, n), orc.qmatmul(to_oracle(orc, pw), x), 2e-5)
+
+
+def test_resident_plan_replays_as_graph(be, orc):
+    """From the second dispatch on a plan whose constants are in place runs as one HIP-graph replay.
+    Every replay is checked against the instruction-by-instruction path (dispatch_profile never replays)
+    and the oracle, with host writes, reads and eager dispatches between the replays."""
+    rng = np.random.default_rng(4242)
+    m, d, f = 24, 256, 768
+    up = fastnn_amd.quantize_weights(flib.DT_I4, _w(rng, f, d))
+    down = fastnn_amd.quantize_weights(flib.DT_F8, _w(rng, d, f))
+    b_up = (rng.standard_normal(f) * 0.1).astype(np.float32)
+    a = Arena()
+    s_x, s_up, s_bup, s_down = a.take(m * d * 4), a.take(up.words.nbytes), a.take(b_up.nbytes), a.take(down.words.nbytes)
+    s_h, s_y, s_out, s_cp = a.take(m * f * 4), a.take(m * d * 4), a.take(m * d * 4), a.take(m * d * 4)
+    plan = ExecutablePlan(a.top)
+    plan.write_const(s_up[0], up.words).write_const(s_bup[0], b_up).write_const(s_down[0], down.words)
+    plan.fill(s_y[0], s_y[1], 0.0)
+    plan.call_kernel("matmul_i4_silu", [s_x, s_up, s_bup], s_h, [m, d, f], meta_of(up))
+    plan.call_kernel("matmul_f8", [s_h, s_down], s_y, [m, f, d], meta_of(down))
+    plan.call_kernel("add_f32", [s_y, s_x], s_out, [m * d])
+    plan.memcopy(s_cp, s_out)
+    be.allocate_arena(a.top)
+    replays = 0
+    for it in range(6):
+        x = rng.standard_normal((m, d)).astype(np.float32)
+        be.write_arena(s_x[0], x)                      # touches no constant: the plan stays resident
+        be.dispatch(plan)
+        replays += plan.replayed
+        assert plan.replayed == (it >= 1), f"dispatch {it}"
+        got = be.read_arena(*s_cp, np.float32).copy()
+        h_ref = orc.qmatmul(to_oracle(orc, up), x, bias=b_up, act=flib.ACT_SILU)
+        want = orc.qmatmul(to_oracle(orc, down), h_ref) + x
+        assert_close(got.reshape(m, d), want, 1e-4, f"dispatch {it}")
+        be.write_arena(s_cp[0], np.zeros(m * d, np.float32))
+        be.dispatch_profile(plan)                      # same instructions, one by one
+        assert not plan.replayed
+        assert np.array_equal(be.read_arena(*s_cp, np.float32), got), f"replay {it} differs from the eager path"
+    assert replays == 5
+    # rewriting a constant from the host ends residency: the next dispatch uploads and runs eagerly,
+    # and its result follows the plan's own payload again
+    be.write_arena(s_bup[0], np.zeros_like(b_up))
+    be.dispatch(plan)
+    assert not plan.replayed
+    assert_close(be.read_arena(*s_cp, np.float32).reshape(m, d), want, 1e-4, "after a constant was overwritten")
+    be.dispatch(plan)
+    assert plan.replayed
+    assert_close(be.read_arena(*s_cp, np.float32).reshape(m, d), want, 1e-4, "replay after re-upload")
+
+
+def test_plan_that_rewrites_its_constants_never_replays(be, orc):
+    """A WriteConst target that another instruction overwrites is uploaded on every dispatch (eager path)."""
+    rng = np.random.default_rng(5)
+    m, k, n = 4, 64, 32
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    pw = fastnn_amd.quantize_weights(flib.DT_I8, _w(rng, n, k))
+    a = Arena()
+    s_x, s_w, s_o = a.take(x.nbytes), a.take(pw.words.nbytes), a.take(m * n * 4)
+    plan = ExecutablePlan(a.top).write_const(s_x[0], x).write_const(s_w[0], pw.words)
+    plan.call_kernel("matmul_i8", [s_x, s_w], s_o, [m, k, n], meta_of(pw))
+    plan.call_kernel("relu_f32", [s_x], s_x, [m * k])      # clobbers the constant input
+    be.allocate_arena(a.top)
+    want = orc.qmatmul(to_oracle(orc, pw), x)
+    for _ in range(3):
+        be.dispatch(plan)
+        assert not plan.replayed
+        assert_close(be.read_arena(*s_o, np.float32).reshape(m, n), want, 2e-5, "clobbered constant")
