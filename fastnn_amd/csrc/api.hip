@@ -518,8 +518,8 @@ int fnn_hip_qconv2d(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *x, i
 {
     if (!ctx) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_hip_qconv2d: NULL context");
     if (!w) return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8: missing weight_meta for quantized weight");
-    if (w->dtype != FNN_DT_I8)
-        return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "conv2d: only I8 weights have an integer conv kernel (dtype %d)", w->dtype);
+    if (w->dtype != FNN_DT_I8 && w->dtype != FNN_DT_I4)
+        return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "conv2d: only I8 and I4 weights have an integer conv kernel (dtype %d)", w->dtype);
     if (groups <= 0) return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8: groups must be > 0");
     if (b < 0 || c <= 0 || h <= 0 || wd <= 0 || kh <= 0 || kw <= 0 || stride <= 0 || dil <= 0 || pad < 0)
         return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8: invalid geometry");
@@ -575,6 +575,7 @@ int fnn_hip_qconv2d(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *x, i
     p.actq = p.minmax_partial + (size_t)(b * groups) * QCONV_NPART * 2;
     p.b = b; p.c = c; p.h = h; p.w = wd; p.oc = oc; p.ho = ho; p.wo = wo; p.kp = w->kp;
     p.kh = kh; p.kw = kw; p.stride = stride; p.pad = pad; p.dil = dil; p.groups = groups; p.act = act;
+    p.wbits = w->dtype == FNN_DT_I4 ? 4 : 8;
     if (flags & FNN_FLAG_FORCE_GENERIC) {
         HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qconv2d_i8(p, ctx->stream, 0));
     } else {

@@ -294,8 +294,12 @@ int run_conv2d_i8(fnn_backend *b, const Instr &in, const KernelName &kn)
     if (h + 2 * pad < eh || wd + 2 * pad < ew) return fail(b, FNN_ERR_DISPATCH, "%s: kernel larger than padded input", name);
     uint64_t oh = (h + 2 * pad - eh) / stride + 1, ow = (wd + 2 * pad - ew) / stride + 1;
     if (in.dst.size < batch * oc * oh * ow * 4) return fail(b, FNN_ERR_DISPATCH, "%s: output slice holds %llu bytes, needs %llu", name, (unsigned long long)in.dst.size, (unsigned long long)(batch * oc * oh * ow * 4));
+    // the CPU arm picks the integer kernel by bit width, not by name (src/backend/cpu/mod.rs:4258-4264)
+    const int dtype = in.meta.bit_width == 4 ? FNN_DT_I4 : FNN_DT_I8;
+    if (dtype == FNN_DT_I4 && !in.meta.codebook.empty())
+        return fail(b, FNN_ERR_UNSUPPORTED_OP, "%s: codebook weights have no GPU conv kernel", name);
     fnn_hip_weight *w = nullptr;
-    int st = weight_for(b, in.inputs[1], FNN_DT_I8, in.meta, oc, inner, name, &w);
+    int st = weight_for(b, in.inputs[1], dtype, in.meta, oc, inner, name, &w);
     if (st) return st;
     if (batch == 0) return FNN_OK;
     return lift(b, fnn_hip_qconv2d(b->ctx, w, (const float *)(b->arena + in.inputs[0].offset), (int64_t)batch, (int64_t)c,
@@ -337,7 +341,7 @@ int run_call(fnn_backend *b, const Instr &in)
     KernelName kn = split_activation(name);
     int dt = matmul_dtype(kn.base);
     if (dt >= 0) return run_matmul(b, in, kn, dt);
-    if (kn.base == "conv2d_i8") return run_conv2d_i8(b, in, kn);
+    if (kn.base == "conv2d_i8" || kn.base == "conv2d_i4") return run_conv2d_i8(b, in, kn);
     return fail(b, FNN_ERR_UNSUPPORTED_OP, "%s", name.c_str());
 }
 

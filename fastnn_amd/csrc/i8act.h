@@ -13,7 +13,7 @@ struct I8ActArgs {
 };
 
 struct QConvArgs {
-    const uint32_t *words;   // [OC, kp] I8 words
+    const uint32_t *words;   // [OC, kp] I8 or I4 words
     const float *scales;     // [OC]
     const float *zeros;      // [OC]
     const int32_t *row_qsum; // [OC] sum of q_w per output channel
@@ -25,6 +25,7 @@ struct QConvArgs {
     float *actq;             // [B*G][4]: sa, za, inv, unused
     int64_t b, c, h, w, oc, ho, wo, kp;
     int kh, kw, stride, pad, dil, groups, act;
+    int wbits;               // 8: I8 weights, activations quantised to 256 levels; 4: I4 weights, 16 levels
 };
 constexpr int QCONV_NPART = 512;
 

@@ -1,7 +1,9 @@
-// Quantised Conv2d (I8 weights, f32 NCHW activations) for gfx950:
+// Quantised Conv2d (I8 or I4 weights, f32 NCHW activations) for gfx950:
 // conv2d_packed_i8x4 = im2col + per-(image,group) dynamic int8 activation quantisation +
 // integer GEMM with the fused 4-term dequantise, bias and activation
-// (src/backend/cpu/packed_conv.rs:125-232,444-625,1118-1196).
+// (src/backend/cpu/packed_conv.rs:125-232,444-625,1118-1196);
+// conv2d_packed_i4x8 = the same with 4-bit weights and activations quantised to 16 levels
+// (packed_conv.rs:236-283,659-841,1202-1280).
 //
 // The im2col matrix is never materialised: its (min,max) scan and the activation
 // quantisation are evaluated from the NCHW input through the index formula
@@ -121,8 +123,9 @@ __global__ void __launch_bounds__(256) conv_minmax_cover_kernel(QConvArgs a, int
     }
 }
 
-// scale = range/255 (1 if range <= 0), zero = mn + 128*scale (0 if range <= 0), inv = 1/scale
-// (src/backend/cpu/packed_conv.rs:149-156)
+// 8-bit: scale = range/255 (1 if range <= 0), zero = mn + 128*scale (0 if range <= 0), inv = 1/scale
+// (src/backend/cpu/packed_conv.rs:149-156); 4-bit: scale = range/15 (1 if range <= 0),
+// zero = mn + 8*scale in either case (packed_conv.rs:260-263)
 __global__ void __launch_bounds__(64) conv_actq_kernel(QConvArgs a, int nparts)
 {
     const int bg = blockIdx.x;
@@ -135,8 +138,14 @@ __global__ void __launch_bounds__(64) conv_actq_kernel(QConvArgs a, int nparts)
     mx = wave_max(mx);
     if (threadIdx.x == 0) {
         const float range = mx - mn;
-        const float scale = (range > 0.0f) ? range / 255.0f : 1.0f;
-        const float zero = (range > 0.0f) ? mn + 128.0f * scale : 0.0f;
+        float scale, zero;
+        if (a.wbits == 4) {
+            scale = (range > 0.0f) ? range / 15.0f : 1.0f;
+            zero = mn + 8.0f * scale;
+        } else {
+            scale = (range > 0.0f) ? range / 255.0f : 1.0f;
+            zero = (range > 0.0f) ? mn + 128.0f * scale : 0.0f;
+        }
         const float inv = (scale != 0.0f) ? 1.0f / scale : 0.0f;
         a.actq[bg * 4 + 0] = scale;
         a.actq[bg * 4 + 1] = zero;
@@ -168,15 +177,20 @@ __global__ void __launch_bounds__(256) conv_i8_kernel(QConvArgs a)
     for (int t = 0; t < CONV_OCT; t++) acc[t] = 0;
     int qasum = 0;
     const int8_t *wb = reinterpret_cast<const int8_t *>(a.words);
+    const float qlo = a.wbits == 4 ? -8.0f : -128.0f, qhi = a.wbits == 4 ? 7.0f : 127.0f;
     for (int64_t e = 0; e < kk; e++) {
         const float v = col_value(xg, a.h, a.w, a.kh, a.kw, a.stride, a.pad, a.dil, a.wo, p, e);
         const float t = roundf((v - za) * inv);
-        const int q = (t != t) ? 0 : (int)fminf(fmaxf(t, -128.0f), 127.0f);
+        const int q = (t != t) ? 0 : (int)fminf(fmaxf(t, qlo), qhi);
         qasum += q;
 #pragma unroll
         for (int t2 = 0; t2 < CONV_OCT; t2++) {
             const int64_t f = f0 + t2;
-            if (f < ocg) acc[t2] += q * (int)wb[((g * ocg + f) * a.kp) * 4 + e];
+            if (f >= ocg) continue;
+            int qw;
+            if (a.wbits == 4) qw = ((int)(a.words[(g * ocg + f) * a.kp + e / 8] << (28 - 4 * (int)(e % 8)))) >> 28;
+            else qw = (int)wb[((g * ocg + f) * a.kp) * 4 + e];
+            acc[t2] += q * qw;
         }
     }
     const float r = sa * (float)qasum;

@@ -110,6 +110,8 @@ __global__ void __launch_bounds__(256) conv_operand_kernel(QConvArgs a, int g, i
         const float za = a.actq[bg * 4 + 1], inv = a.actq[bg * 4 + 2];
         const float *xg = a.x + (nn * a.c + g * cg) * a.h * a.w;
         const int khw = a.kh * a.kw;
+        const float qlo = a.wbits == 4 ? -8.0f : -128.0f, qhi = a.wbits == 4 ? 7.0f : 127.0f;
+        const int interleaved = a.wbits == 4;   // the 4-bit weight decoder delivers k = 0,2,4,6,1,3,5,7 of each 8
         const int64_t ih0 = (p / a.wo) * a.stride - a.pad, iw0 = (p % a.wo) * a.stride - a.pad;
         const int c_end = (int)(blockIdx.y + 1) * CONV_CPB < live_chunks ? (int)(blockIdx.y + 1) * CONV_CPB : live_chunks;
         for (int c = (int)blockIdx.y * CONV_CPB + slot; c < c_end; c += 4) {
@@ -125,9 +127,10 @@ __global__ void __launch_bounds__(256) conv_operand_kernel(QConvArgs a, int g, i
                         float v = 0.0f;
                         if (ih >= 0 && ih < a.h && iw >= 0 && iw < a.w) v = xg[((int64_t)ic * a.h + ih) * a.w + iw];
                         const float q = roundf((v - za) * inv);
-                        const int qi = (q != q) ? 0 : (int)fminf(fmaxf(q, -128.0f), 127.0f);
+                        const int qi = (q != q) ? 0 : (int)fminf(fmaxf(q, qlo), qhi);
                         s += qi;
-                        out[t >> 2] |= (uint32_t)(uint8_t)qi << (8 * (t & 3));
+                        const int pos = (t & 8) + slot_of(t & 7, interleaved);
+                        out[pos >> 2] |= (uint32_t)(uint8_t)qi << (8 * (pos & 3));
                     }
                     e++;
                     if (++j == a.kw) { j = 0; if (++i == a.kh) { i = 0; ic++; } }
@@ -349,7 +352,7 @@ int fnn_i8_tiled_matmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w
 int fnn_i8_tiled_conv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QConvArgs &p, bool *handled)
 {
     *handled = false;
-    if (w->dtype != FNN_DT_I8 || (reinterpret_cast<uintptr_t>(p.words) & 15)) return FNN_OK;
+    if ((w->dtype != FNN_DT_I8 && w->dtype != FNN_DT_I4) || (reinterpret_cast<uintptr_t>(p.words) & 15)) return FNN_OK;
     const int64_t np = p.ho * p.wo, rows = p.b * np;
     const int64_t cg = p.c / p.groups, ocg = p.oc / p.groups, kk = cg * p.kh * p.kw;
     if (rows < 1 || rows > (1ll << 28) || kk > (1 << 20) || ocg < 1) return FNN_OK;
@@ -374,7 +377,9 @@ int fnn_i8_tiled_conv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, 
         const dim3 grid((unsigned)(rows_pad / 64), (unsigned)nq);
         hipLaunchKernelGGL(conv_operand_kernel, grid, dim3(256), 0, s, p, g, (int)kk, kpad, rows_pad, a8, qsum);
         hipError_t e = hipGetLastError();
-        if (e == hipSuccess) e = run_i8_gemm<FNN_DT_I8>(words, kp, w->rows, g * ocg, ocg, a8, rows, rows_pad, kpad, c, ocg, s);
+        if (e == hipSuccess)
+            e = w->dtype == FNN_DT_I8 ? run_i8_gemm<FNN_DT_I8>(words, kp, w->rows, g * ocg, ocg, a8, rows, rows_pad, kpad, c, ocg, s)
+                                      : run_i8_gemm<FNN_DT_I4>(words, kp, w->rows, g * ocg, ocg, a8, rows, rows_pad, kpad, c, ocg, s);
         if (e == hipSuccess) {
             hipLaunchKernelGGL(conv_epilogue_kernel, dim3((unsigned)((rows + 63) / 64), (unsigned)((ocg + EPI_CH - 1) / EPI_CH)), dim3(256), 0, s, p, g,
                                (int)kk, c, (int)ocg, qsum, nq, rows_pad);

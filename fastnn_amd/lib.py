@@ -350,7 +350,7 @@ class HipContext:
         return (out, acc) if want_acc else out
 
     def qconv2d(self, wh, x: np.ndarray, oc: int, kh: int, kw: int, stride: int, pad: int, dil: int, groups: int,
-                bias: Optional[np.ndarray] = None, act: int = ACT_NONE, want_acc: bool = False):
+                bias: Optional[np.ndarray] = None, act: int = ACT_NONE, want_acc: bool = False, flags: int = 0):
         x = np.ascontiguousarray(x, dtype=np.float32)
         b, c, h, w = x.shape
 
@@ -362,7 +362,7 @@ class HipContext:
         acc = np.zeros((b, oc, ho, wo), np.int32) if want_acc else None
         bb = None if bias is None else np.ascontiguousarray(bias, dtype=np.float32)
         self._check(self.lib.fnn_hip_qconv2d(self.handle, wh, _np_ptr(x), b, c, h, w, kh, kw, stride, pad, dil, groups,
-                                             _np_ptr(bb), act, _np_ptr(y), _np_ptr(acc), 0))
+                                             _np_ptr(bb), act, _np_ptr(y), _np_ptr(acc), flags))
         return (y, acc) if want_acc else y
 
     # ---- timing / graphs ----

@@ -997,19 +997,20 @@ size_t fnn_or_conv_out_size(size_t input, size_t kernel, size_t stride, size_t p
  *     val = acc*sab + zw*r + za*w_term + zp_prod*K, left to right in f32;
  *   activation (:571,604-606: SiLU x/(1+exp(-x)); GELU val*0.5*(1+tanh(val*0.7978846*(1+0.044715*val*val))));
  *   y[b, oc, p] = val                                          (:1176-1188). */
-int fnn_or_qconv2d_i8(const float *x, size_t b, size_t c, size_t h, size_t w,
-                      const uint32_t *words, size_t oc, const float *scales, size_t n_scales,
-                      const float *zeros, size_t n_zeros, const float *bias, size_t kh, size_t kw,
-                      size_t stride, size_t pad, size_t dil, size_t groups, int act, float *y,
-                      int32_t *acc_out, float *act_scale_out, float *act_zero_out)
+static int qconv2d_int(int bits, const float *x, size_t b, size_t c, size_t h, size_t w,
+                       const uint32_t *words, size_t oc, const float *scales, size_t n_scales,
+                       const float *zeros, size_t n_zeros, const float *bias, size_t kh, size_t kw,
+                       size_t stride, size_t pad, size_t dil, size_t groups, int act, float *y,
+                       int32_t *acc_out, float *act_scale_out, float *act_zero_out)
 {
+    const size_t items = (bits == 4) ? 8 : 4;
     if (groups == 0 || c % groups || oc % groups) return -1;
     size_t cg = c / groups, ocg = oc / groups;
     size_t ho = fnn_or_conv_out_size(h, kh, stride, pad, dil);
     size_t wo = fnn_or_conv_out_size(w, kw, stride, pad, dil);
     size_t np = ho * wo;
     size_t kk = cg * kh * kw;
-    size_t kp = ceil_div(kk, 4);
+    size_t kp = ceil_div(kk, items);
     float *col = (float *)malloc((np * kk + 1) * sizeof(float));
     int8_t *qa = (int8_t *)malloc(np * kk + 1);
     if (!col || !qa) { free(col); free(qa); return -2; }
@@ -1035,19 +1036,27 @@ int fnn_or_qconv2d_i8(const float *x, size_t b, size_t c, size_t h, size_t w,
                 mx = fmaxf(mx, col[i]);
             }
             float range = mx - mn;
-            float sa = (range > 0.0f) ? range / 255.0f : 1.0f;
-            float za = (range > 0.0f) ? mn + 128.0f * sa : 0.0f;
+            float sa, za;
+            if (bits == 4) { /* packed_conv.rs:260-263: the zero point is formed in either case */
+                sa = (range > 0.0f) ? range / 15.0f : 1.0f;
+                za = mn + 8.0f * sa;
+            } else {
+                sa = (range > 0.0f) ? range / 255.0f : 1.0f;
+                za = (range > 0.0f) ? mn + 128.0f * sa : 0.0f;
+            }
+            const float qlo = (bits == 4) ? -8.0f : -128.0f, qhi = (bits == 4) ? 7.0f : 127.0f;
             float inv = (sa != 0.0f) ? 1.0f / sa : 0.0f;
             if (act_scale_out) act_scale_out[nn * groups + g] = sa;
             if (act_zero_out) act_zero_out[nn * groups + g] = za;
             for (size_t i = 0; i < np * kk; i++)
-                qa[i] = (int8_t)sat_i32(clampf(roundf((col[i] - za) * inv), -128.0f, 127.0f), -128,
-                                        127);
+                qa[i] = (int8_t)sat_i32(clampf(roundf((col[i] - za) * inv), qlo, qhi), (int32_t)qlo,
+                                        (int32_t)qhi);
             for (size_t f = 0; f < ocg; f++) {
                 size_t ch = g * ocg + f;
                 const uint32_t *wrow = words + ch * kp;
                 int32_t qb = 0;
-                for (size_t p = 0; p < kp; p++) qb += fnn_or_i8x4_sum(wrow[p]);
+                for (size_t p = 0; p < kp; p++)
+                    qb += (bits == 4) ? fnn_or_i4x8_sum(wrow[p]) : fnn_or_i8x4_sum(wrow[p]);
                 float sw = (n_scales > 1) ? scales[ch] : scales[0];
                 float zw = (n_zeros > 1) ? zeros[ch] : (n_zeros ? zeros[0] : 0.0f);
                 float sab = sa * sw;
@@ -1060,7 +1069,8 @@ int fnn_or_qconv2d_i8(const float *x, size_t b, size_t c, size_t h, size_t w,
                     int32_t qasum = 0;
                     int32_t acc = bias_q;
                     for (size_t e = 0; e < kk; e++) {
-                        int32_t qw = (int32_t)(int8_t)(wrow[e / 4] >> (8 * (e % 4)));
+                        int32_t qw = (bits == 4) ? nib_s(wrow[e / 8], (int)(e % 8))
+                                                 : (int32_t)(int8_t)(wrow[e / 4] >> (8 * (e % 4)));
                         qasum += arow[e];
                         acc += arow[e] * qw;
                     }
@@ -1084,6 +1094,31 @@ int fnn_or_qconv2d_i8(const float *x, size_t b, size_t c, size_t h, size_t w,
     free(col);
     free(qa);
     return 0;
+}
+
+int fnn_or_qconv2d_i8(const float *x, size_t b, size_t c, size_t h, size_t w,
+                      const uint32_t *words, size_t oc, const float *scales, size_t n_scales,
+                      const float *zeros, size_t n_zeros, const float *bias, size_t kh, size_t kw,
+                      size_t stride, size_t pad, size_t dil, size_t groups, int act, float *y,
+                      int32_t *acc_out, float *act_scale_out, float *act_zero_out)
+{
+    return qconv2d_int(8, x, b, c, h, w, words, oc, scales, n_scales, zeros, n_zeros, bias, kh, kw,
+                       stride, pad, dil, groups, act, y, acc_out, act_scale_out, act_zero_out);
+}
+
+/* conv2d_packed_i4x8 (packed_conv.rs:1202-1280): the same lowering with I4x8 weights and the
+ * im2col matrix quantised to 16 levels, sa = range/15 (1 if range <= 0), za = mn + 8*sa,
+ * q_a = clamp(round((x - za)*(1/sa)), -8, 7) (im2col_pack_i4x8, :236-283, which fills its
+ * words in place, so the as-written and the intended algorithm coincide); per channel and per
+ * pixel exactly the four-term formula of the 8-bit kernel (gemm_packed_i4x8_fused_raw, :659-841). */
+int fnn_or_qconv2d_i4(const float *x, size_t b, size_t c, size_t h, size_t w,
+                      const uint32_t *words, size_t oc, const float *scales, size_t n_scales,
+                      const float *zeros, size_t n_zeros, const float *bias, size_t kh, size_t kw,
+                      size_t stride, size_t pad, size_t dil, size_t groups, int act, float *y,
+                      int32_t *acc_out, float *act_scale_out, float *act_zero_out)
+{
+    return qconv2d_int(4, x, b, c, h, w, words, oc, scales, n_scales, zeros, n_zeros, bias, kh, kw,
+                       stride, pad, dil, groups, act, y, acc_out, act_scale_out, act_zero_out);
 }
 
 /* ------------------------------------------------------------------------ */

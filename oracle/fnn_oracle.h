@@ -102,6 +102,14 @@ int fnn_or_qconv2d_i8(const float *x, size_t b, size_t c, size_t h, size_t w,
                       int act, float *y, int32_t *acc_out, float *act_scale_out,
                       float *act_zero_out);
 
+/* I4x8 weights, activations quantised to 16 levels (packed_conv.rs:236-283,659-841,1202-1280) */
+int fnn_or_qconv2d_i4(const float *x, size_t b, size_t c, size_t h, size_t w,
+                      const uint32_t *words, size_t oc, const float *scales, size_t n_scales,
+                      const float *zeros, size_t n_zeros, const float *bias,
+                      size_t kh, size_t kw, size_t stride, size_t pad, size_t dil, size_t groups,
+                      int act, float *y, int32_t *acc_out, float *act_scale_out,
+                      float *act_zero_out);
+
 /* ---- generators used by the reference's own tests ------------------------ */
 void fnn_or_seeded_values(uint64_t seed, size_t len, float *out);
 

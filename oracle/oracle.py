@@ -96,6 +96,7 @@ def _proto(l):
     l.fnn_or_qconv2d_i8.argtypes = [_f32p, _sz, _sz, _sz, _sz, _u32p, _sz, C.c_void_p, _sz,
                                     C.c_void_p, _sz, C.c_void_p, _sz, _sz, _sz, _sz, _sz, _sz,
                                     C.c_int, _f32p, C.c_void_p, C.c_void_p, C.c_void_p]
+    l.fnn_or_qconv2d_i4.argtypes = l.fnn_or_qconv2d_i8.argtypes
     l.fnn_or_seeded_values.argtypes = [C.c_uint64, _sz, _f32p]
 
 
@@ -272,7 +273,7 @@ def conv_out_size(inp, kernel, stride, pad, dil) -> int:
 
 def qconv2d_i8(x, p: Packed, kh: int, kw: int, stride: int, pad: int, dil: int, groups: int,
                bias=None, act: int = ACT_NONE, want_acc: bool = False):
-    """x NCHW f32; p packed [OC, C/g*KH*KW] I8 weights."""
+    """x NCHW f32; p packed [OC, C/g*KH*KW] I8 weights (or I4 weights: the 16-level variant)."""
     x = _f32(x)
     b, c, h, w = x.shape
     oc = p.rows
@@ -282,10 +283,10 @@ def qconv2d_i8(x, p: Packed, kh: int, kw: int, stride: int, pad: int, dil: int, 
     sa = np.zeros(b * groups, np.float32)
     za = np.zeros(b * groups, np.float32)
     bb = None if bias is None else _f32(bias)
-    rc = lib().fnn_or_qconv2d_i8(x.reshape(-1), b, c, h, w, p.words, oc, _ptr(p.scales),
-                                 p.scales.size, _ptr(p.zeros), p.zeros.size, _ptr(bb), kh, kw,
-                                 stride, pad, dil, groups, act, y.reshape(-1), _ptr(acc),
-                                 _ptr(sa), _ptr(za))
+    fn = lib().fnn_or_qconv2d_i4 if p.dt == I4 else lib().fnn_or_qconv2d_i8
+    rc = fn(x.reshape(-1), b, c, h, w, p.words, oc, _ptr(p.scales),
+            p.scales.size, _ptr(p.zeros), p.zeros.size, _ptr(bb), kh, kw,
+            stride, pad, dil, groups, act, y.reshape(-1), _ptr(acc), _ptr(sa), _ptr(za))
     if rc:
         raise ValueError(f"qconv2d_i8 rc={rc}")
     if want_acc:

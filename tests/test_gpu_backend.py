@@ -134,23 +134,25 @@ def test_i8_activation_chain(be, orc, dt, name, calibrated):
 
 
 @pytest.mark.parametrize("act,code", [("", 0), ("_relu", 1), ("_silu", 3)])
-def test_conv2d_i8_plan(be, orc, act, code):
+@pytest.mark.parametrize("wdt,kname", [(flib.DT_I8, "conv2d_i8"), (flib.DT_I4, "conv2d_i4")])
+def test_conv2d_i8_plan(be, orc, act, code, wdt, kname):
+    """conv2d_i8 / conv2d_i4: the integer kernel is picked by the bit width of the weight metadata."""
     rng = np.random.default_rng(41)
     b, c, h, w, oc, kh, kw, stride, pad, dil, groups = 2, 8, 14, 11, 12, 3, 3, 2, 1, 1, 2
     kk = c // groups * kh * kw
     x = rng.uniform(0, 1, (b, c, h, w)).astype(np.float32)
-    pw = fastnn_amd.quantize_weights(flib.DT_I8, (rng.standard_normal((oc, kk)) * 0.1).astype(np.float32))
+    pw = fastnn_amd.quantize_weights(wdt, (rng.standard_normal((oc, kk)) * 0.1).astype(np.float32))
     bias = (rng.standard_normal(oc) * 0.05).astype(np.float32)
     want = orc.qconv2d_i8(x, to_oracle(orc, pw), kh, kw, stride, pad, dil, groups, bias=bias, act=code)
     a = Arena()
     s_x, s_w, s_b, s_y = a.take(x.nbytes), a.take(pw.words.nbytes), a.take(bias.nbytes), a.take(want.nbytes)
     plan = ExecutablePlan(a.top).write_const(s_w[0], pw.words).write_const(s_b[0], bias)
-    plan.call_kernel("conv2d_i8" + act, [s_x, s_w, s_b], s_y, [stride, pad, dil, groups, c, h, w, kh, kw],
+    plan.call_kernel(kname + act, [s_x, s_w, s_b], s_y, [stride, pad, dil, groups, c, h, w, kh, kw],
                      meta_of(pw, [oc, c // groups, kh, kw]))
     be.allocate_arena(a.top)
     be.write_arena(s_x[0], x)
     be.dispatch(plan)
-    assert_close(be.read_arena(*s_y, np.float32).reshape(want.shape), want, 1e-5, "conv2d_i8" + act)
+    assert_close(be.read_arena(*s_y, np.float32).reshape(want.shape), want, 1e-5, kname + act)
 
 
 def test_fill_memcopy_and_elementwise(be, orc):

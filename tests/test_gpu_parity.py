@@ -271,13 +271,15 @@ CONVS = [
 
 @pytest.mark.parametrize("cfg", CONVS)
 @pytest.mark.parametrize("act", [0, 1, 3, 2])
-def test_qconv2d_i8(ctx, orc, cfg, act):
+@pytest.mark.parametrize("wdt", [flib.DT_I8, flib.DT_I4])
+def test_qconv2d_i8(ctx, orc, cfg, act, wdt):
+    """I8 weights: conv2d_packed_i8x4; I4 weights: conv2d_packed_i4x8 (activations quantised to 16 levels)."""
     rng = np.random.default_rng(6000 + cfg["c"])
     kk = cfg["c"] // cfg["groups"] * cfg["kh"] * cfg["kw"]
     x = rng.uniform(0, 1, (cfg["b"], cfg["c"], cfg["h"], cfg["w"])).astype(np.float32)
     wt = (rng.standard_normal((cfg["oc"], kk)) * np.sqrt(2.0 / kk)).astype(np.float32)
     bias = (rng.standard_normal(cfg["oc"]) * 0.05).astype(np.float32)
-    pw = fastnn_amd.quantize_weights(flib.DT_I8, wt)
+    pw = fastnn_amd.quantize_weights(wdt, wt)
     h = ctx.register(pw)
     args = (cfg["kh"], cfg["kw"], cfg["stride"], cfg["pad"], cfg["dil"], cfg["groups"])
     want, want_acc, _, _ = orc.qconv2d_i8(x, to_oracle(orc, pw), *args, bias=bias, act=act, want_acc=True)
@@ -286,12 +288,17 @@ def test_qconv2d_i8(ctx, orc, cfg, act):
     assert_close(got, want, 1e-5)          # same f32 formula; expf/tanhf differ in the last ulp
     got_nb = ctx.qconv2d(h, x, cfg["oc"], *args, act=act)
     assert_close(got_nb, orc.qconv2d_i8(x, to_oracle(orc, pw), *args, act=act), 1e-5)
+    # the direct kernel (no im2col operand, no matrix cores) gives the same accumulators
+    got_d, acc_d = ctx.qconv2d(h, x, cfg["oc"], *args, bias=bias, act=act, want_acc=True, flags=flib.FLAG_FORCE_GENERIC)
+    assert np.array_equal(acc_d, want_acc)
+    assert_close(got_d, want, 1e-5)
     ctx.release(h)
 
 
-def test_qconv2d_constant_and_empty(ctx, orc):
+@pytest.mark.parametrize("wdt", [flib.DT_I8, flib.DT_I4])
+def test_qconv2d_constant_and_empty(ctx, orc, wdt):
     x = np.full((1, 2, 4, 4), 0.5, np.float32)
-    pw = fastnn_amd.quantize_weights(flib.DT_I8, np.array([[-0.2, 0.1], [0.1, 0.1]], np.float32))
+    pw = fastnn_amd.quantize_weights(wdt, np.array([[-0.2, 0.1], [0.1, 0.1]], np.float32))
     h = ctx.register(pw)
     got = ctx.qconv2d(h, x, 2, 1, 1, 1, 0, 1, 1)
     assert_close(got, orc.qconv2d_i8(x, to_oracle(orc, pw), 1, 1, 1, 0, 1, 1), 1e-6)

@@ -7,7 +7,13 @@ import torch
 import torch.nn.functional as F
 
 
-def _qw(p, k):
+def _qw(p, k, bits=8):
+    if bits == 4:
+        kp = -(-k // 8)
+        words = p.words[: p.rows * kp].reshape(p.rows, kp)
+        nib = (words[:, :, None] >> (4 * np.arange(8, dtype=np.uint32))) & 0xF
+        nib = nib.astype(np.int64).reshape(p.rows, kp * 8)[:, :k]
+        return np.where(nib >= 8, nib - 16, nib)
     kp = -(-k // 4)
     w = p.words[: p.rows * kp].view(np.int8).reshape(p.rows, kp * 4)[:, :k]
     return w.astype(np.int64)
@@ -20,8 +26,11 @@ def _qw(p, k):
     dict(b=1, c=5, h=6, w=6, oc=3, kh=3, kw=3, stride=1, pad=1, dil=1, groups=1),
 ])
 @pytest.mark.parametrize("act", [0, 1, 3])
-def test_conv_matches_float_conv_of_dequantised(orc, cfg, act):
+@pytest.mark.parametrize("bits", [8, 4])
+def test_conv_matches_float_conv_of_dequantised(orc, cfg, act, bits):
+    """bits=8: conv2d_packed_i8x4; bits=4: conv2d_packed_i4x8 (16 activation levels, 4-bit weights)."""
     rng = np.random.default_rng(300)
+    levels, half, qlo, qhi = (255.0, 128.0, -128, 127) if bits == 8 else (15.0, 8.0, -8, 7)
     b, c, h, w, oc, kh, kw = (cfg[x] for x in ("b", "c", "h", "w", "oc", "kh", "kw"))
     stride, pad, dil, groups = cfg["stride"], cfg["pad"], cfg["dil"], cfg["groups"]
     cg = c // groups
@@ -29,9 +38,9 @@ def test_conv_matches_float_conv_of_dequantised(orc, cfg, act):
     x = rng.uniform(0, 1, (b, c, h, w)).astype(np.float32)
     wt = (rng.standard_normal((oc, kk)) * 0.1).astype(np.float32)
     bias = (rng.standard_normal(oc) * 0.05).astype(np.float32)
-    p = orc.quantize(orc.I8, wt)
+    p = orc.quantize(orc.I8 if bits == 8 else orc.I4, wt)
     y, acc, sa, za = orc.qconv2d_i8(x, p, kh, kw, stride, pad, dil, groups, bias=bias, act=act, want_acc=True)
-    qw = _qw(p, kk)
+    qw = _qw(p, kk, bits)
     ocg = oc // groups
     for n in range(b):
         for g in range(groups):
@@ -40,11 +49,11 @@ def test_conv_matches_float_conv_of_dequantised(orc, cfg, act):
             mn, mx = np.float32(col.min()), np.float32(col.max())
             s = sa[n * groups + g]
             z = za[n * groups + g]
-            assert s == np.float32(mx - mn) / np.float32(255.0)
-            assert z == np.float32(mn + np.float32(128.0) * s)
+            assert s == np.float32(mx - mn) / np.float32(levels)
+            assert z == np.float32(mn + np.float32(half) * s)
             inv = np.float32(1.0) / s
             t = (col.astype(np.float32) - z) * inv
-            qa = np.clip(np.sign(t) * np.floor(np.abs(t) + np.float32(0.5)), -128, 127).astype(np.int64)
+            qa = np.clip(np.sign(t) * np.floor(np.abs(t) + np.float32(0.5)), qlo, qhi).astype(np.int64)
             for f in range(ocg):
                 ch = g * ocg + f
                 sab = np.float32(s * p.scales[ch])
@@ -79,3 +88,19 @@ def test_conv_constant_input_has_unit_scale(orc):
     assert sa[0] == 1.0 and za[0] == 0.0  # zero range -> scale 1, zero 0; 0.5 rounds to 1
     deq = orc.dequant(p)
     assert np.allclose(y[0, :, 0, 0], deq.sum(axis=1), atol=1e-5)
+
+
+def test_conv_i4_constant_input_keeps_its_zero_point(orc):
+    """The 4-bit activation quantiser forms zero = min + 8*scale also for a flat input
+    (packed_conv.rs:260-263): 0.5 everywhere -> scale 1, zero 8.5, q = clamp(round(-8), -8, 7) = -8,
+    dequantised back to exactly 0.5."""
+    x = np.full((1, 2, 4, 4), 0.5, np.float32)
+    wt = np.ones((2, 2), np.float32) * 0.1
+    wt[0, 0] = -0.2
+    p = orc.quantize(orc.I4, wt)
+    y, acc, sa, za = orc.qconv2d_i8(x, p, 1, 1, 1, 0, 1, 1, want_acc=True)
+    assert sa[0] == 1.0 and za[0] == 8.5
+    qw = _qw(p, 2, 4)
+    assert np.array_equal(acc[0, :, 0, 0], -8 * qw.sum(axis=1))
+    deq = orc.dequant(p)
+    assert np.allclose(y[0, :, 0, 0], 0.5 * deq.sum(axis=1), atol=1e-5)
