@@ -19,6 +19,9 @@
 #include "../../include/fastnn_hip_backend.h"
 
 hipError_t launch_probe(const void *src, void *dst, size_t bytes, uint32_t *sink, hipStream_t s);
+hipError_t launch_im2col_f32(const float *x, float *col, int64_t b, int64_t c, int groups, int g, int64_t h, int64_t w,
+                             int64_t ho, int64_t wo, int kh, int kw, int stride, int pad, int dil, hipStream_t s);
+hipError_t launch_rows_to_nchw(const float *src, float *y, int64_t b, int64_t np, int64_t oc, int64_t ch0, int64_t ocg, hipStream_t s);
 hipError_t launch_fill(float *dst, uint64_t n, float value, hipStream_t s);
 hipError_t launch_eltwise(int op, const float *a, const float *b, uint64_t nb, float *out, uint64_t n, hipStream_t s);
 
@@ -38,7 +41,7 @@ struct fnn_hip_ctx {
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     std::string err;
     std::unordered_map<uint64_t, fnn_hip_weight *> weights;
-    Staging st_a, st_out, st_bias, st_acc, st_tmp, st_tmp2, st_tmp3, st_cnt;
+    Staging st_a, st_out, st_bias, st_acc, st_tmp, st_tmp2, st_tmp3, st_cnt, st_col, st_rows;
     float *scratch = nullptr;  // small reduction scratch (partials)
     bool capturing = false;
     uint64_t ws_epoch = 0;     // bumped whenever a staging buffer is re-allocated (captured graphs go stale)
@@ -165,7 +168,7 @@ void fnn_hip_destroy(fnn_hip_ctx *ctx)
     (void)hipSetDevice(ctx->device);
     if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
     for (auto &kv : ctx->weights) free_weight(kv.second);
-    for (Staging *s : {&ctx->st_a, &ctx->st_out, &ctx->st_bias, &ctx->st_acc, &ctx->st_tmp, &ctx->st_tmp2, &ctx->st_tmp3, &ctx->st_cnt})
+    for (Staging *s : {&ctx->st_a, &ctx->st_out, &ctx->st_bias, &ctx->st_acc, &ctx->st_tmp, &ctx->st_tmp2, &ctx->st_tmp3, &ctx->st_cnt, &ctx->st_col, &ctx->st_rows})
         if (s->ptr) (void)hipFree(s->ptr);
     if (ctx->scratch) (void)hipFree(ctx->scratch);
     if (ctx->ev0) (void)hipEventDestroy(ctx->ev0);
@@ -518,8 +521,9 @@ int fnn_hip_qconv2d(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *x, i
 {
     if (!ctx) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_hip_qconv2d: NULL context");
     if (!w) return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8: missing weight_meta for quantized weight");
-    if (w->dtype != FNN_DT_I8 && w->dtype != FNN_DT_I4)
-        return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "conv2d: only I8 and I4 weights have an integer conv kernel (dtype %d)", w->dtype);
+    const bool integer_kernel = w->dtype == FNN_DT_I8 || w->dtype == FNN_DT_I4;
+    if (!integer_kernel && acc_out)
+        return fail(ctx, FNN_ERR_DISPATCH, "conv2d: weight type %d runs as an f32 convolution and has no i32 accumulators", w->dtype);
     if (groups <= 0) return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8: groups must be > 0");
     if (b < 0 || c <= 0 || h <= 0 || wd <= 0 || kh <= 0 || kw <= 0 || stride <= 0 || dil <= 0 || pad < 0)
         return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8: invalid geometry");
@@ -541,7 +545,7 @@ int fnn_hip_qconv2d(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *x, i
     if (b * groups > 65535) return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "conv2d_i8: batch*groups > 65535");
     const bool dev = (flags & FNN_FLAG_DEVICE_PTRS) != 0;
     fnn_hip_weight *wm = const_cast<fnn_hip_weight *>(w);
-    if (!wm->row_qsum) {
+    if (integer_kernel && !wm->row_qsum) {
         if (ctx->capturing) return fail(ctx, FNN_ERR_MEMORY, "conv2d_i8: first use of a weight during graph capture");
         HIP_TRY(ctx, FNN_ERR_MEMORY, hipMalloc((void **)&wm->row_qsum, (size_t)oc * 4 + 64));
         HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_row_qsum(w, wm->row_qsum, ctx->stream));
@@ -566,6 +570,38 @@ int fnn_hip_qconv2d(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *x, i
             if ((rc = ensure(ctx, ctx->st_acc, yout))) return rc;
             dacc = (int32_t *)ctx->st_acc.ptr;
         }
+    }
+    if (!integer_kernel) {
+        // f32 convolution with dequantised weights (src/backend/cpu/mod.rs:4204-4257): im2col rows,
+        // fused-dequant MatMul per group (bias and activation in its epilogue), [pixel, channel] -> NCHW
+        const int64_t cg = c / groups, ocg = oc / groups, kk = cg * kh * kw, np = ho * wo, rows = b * np;
+        if (rows > (1ll << 31) || b > 65535) return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "conv2d: %lld output pixels exceed the f32 path's limit", (long long)rows);
+        if ((rc = ensure(ctx, ctx->st_col, (size_t)rows * kk * 4 + 256))) return rc;
+        if ((rc = ensure(ctx, ctx->st_rows, (size_t)rows * ocg * 4 + 256))) return rc;
+        float *col = (float *)ctx->st_col.ptr, *rows_out = (float *)ctx->st_rows.ptr;
+        for (int g = 0; g < groups; g++) {
+            HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_im2col_f32(dx, col, b, c, groups, g, h, wd, ho, wo, kh, kw, stride, pad, dil, ctx->stream));
+            if (groups == 1) {
+                if ((rc = fnn_hip_qmatmul(ctx, w, col, rows, dbias, act, rows_out, FNN_FLAG_DEVICE_PTRS | (flags & FNN_FLAG_FORCE_GENERIC)))) return rc;
+            } else {
+                // a slice of the weight rows: the shape-agnostic kernel takes the offset pointers as they are
+                QMatmulArgs q;
+                q.words = w->words + (size_t)g * ocg * w->kp;
+                q.scales = w->dtype == FNN_DT_I4CB ? w->scales + (size_t)g * ocg * w->bpr : w->scales + (size_t)g * ocg;
+                q.zeros = w->zeros ? w->zeros + (size_t)g * ocg : nullptr;
+                q.codebook = w->codebook;
+                q.a = col; q.bias = dbias ? dbias + (size_t)g * ocg : nullptr; q.out = rows_out;
+                q.m = rows; q.n = ocg; q.k = kk; q.kp = w->kp; q.bpr = w->bpr; q.qblock = w->qblock; q.act = act;
+                q.as_written = 0;
+                HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qgemm_generic(w->dtype, q, ctx->stream));
+            }
+            HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_rows_to_nchw(rows_out, dy, b, np, oc, (int64_t)g * ocg, ocg, ctx->stream));
+        }
+        if (!dev) {
+            HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(y, dy, yout, hipMemcpyDeviceToHost, ctx->stream));
+            HIP_TRY(ctx, FNN_ERR_DISPATCH, hipStreamSynchronize(ctx->stream));
+        }
+        return FNN_OK;
     }
     if ((rc = ensure(ctx, ctx->st_tmp, (size_t)(b * groups) * (QCONV_NPART * 2 + 4) * 4))) return rc;
     QConvArgs p;

@@ -294,10 +294,16 @@ int run_conv2d_i8(fnn_backend *b, const Instr &in, const KernelName &kn)
     if (h + 2 * pad < eh || wd + 2 * pad < ew) return fail(b, FNN_ERR_DISPATCH, "%s: kernel larger than padded input", name);
     uint64_t oh = (h + 2 * pad - eh) / stride + 1, ow = (wd + 2 * pad - ew) / stride + 1;
     if (in.dst.size < batch * oc * oh * ow * 4) return fail(b, FNN_ERR_DISPATCH, "%s: output slice holds %llu bytes, needs %llu", name, (unsigned long long)in.dst.size, (unsigned long long)(batch * oc * oh * ow * 4));
-    // the CPU arm picks the integer kernel by bit width, not by name (src/backend/cpu/mod.rs:4258-4264)
-    const int dtype = in.meta.bit_width == 4 ? FNN_DT_I4 : FNN_DT_I8;
-    if (dtype == FNN_DT_I4 && !in.meta.codebook.empty())
-        return fail(b, FNN_ERR_UNSUPPORTED_OP, "%s: codebook weights have no GPU conv kernel", name);
+    // weight type as the CPU arm decides it (src/backend/cpu/mod.rs:4248-4264): by name for the types that run
+    // as an f32 convolution with dequantised weights, else by bit width (codebook weights: f32 path as well)
+    int dtype;
+    if (kn.base == "conv2d_u4") dtype = FNN_DT_U4;
+    else if (kn.base == "conv2d_u8") dtype = FNN_DT_U8;
+    else if (kn.base == "conv2d_f4") dtype = FNN_DT_F4;
+    else if (kn.base == "conv2d_f8r") dtype = FNN_DT_F8R;
+    else if (kn.base == "conv2d_f8") dtype = FNN_DT_F8;
+    else if (in.meta.bit_width == 4) dtype = in.meta.codebook.empty() ? FNN_DT_I4 : FNN_DT_I4CB;
+    else dtype = FNN_DT_I8;
     fnn_hip_weight *w = nullptr;
     int st = weight_for(b, in.inputs[1], dtype, in.meta, oc, inner, name, &w);
     if (st) return st;
@@ -341,7 +347,9 @@ int run_call(fnn_backend *b, const Instr &in)
     KernelName kn = split_activation(name);
     int dt = matmul_dtype(kn.base);
     if (dt >= 0) return run_matmul(b, in, kn, dt);
-    if (kn.base == "conv2d_i8" || kn.base == "conv2d_i4") return run_conv2d_i8(b, in, kn);
+    if (kn.base == "conv2d_i8" || kn.base == "conv2d_i4" || kn.base == "conv2d_u8" || kn.base == "conv2d_u4" ||
+        kn.base == "conv2d_f8" || kn.base == "conv2d_f8r" || kn.base == "conv2d_f4")
+        return run_conv2d_i8(b, in, kn);
     return fail(b, FNN_ERR_UNSUPPORTED_OP, "%s", name.c_str());
 }
 

@@ -124,11 +124,16 @@ int fnn_hip_quantize_activations(fnn_hip_ctx *ctx, const float *x, int64_t numel
 int fnn_hip_qmatmul_i8act(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const uint8_t *payload,
                           int64_t m, float *out, int32_t *acc_out, int flags);
 
-/* ---- quantised Conv2d, I8 weights, f32 NCHW activations:
- * conv2d_packed_i8x4 (src/backend/cpu/packed_conv.rs:1118-1196) =
- * im2col + per-(image,group) dynamic int8 activation quantisation
- * (packed_conv.rs:125-232) + gemm_packed_i8x4_fused_raw (packed_conv.rs:444-625).
- * acc_out (nullable, same shape as y) receives the i32 accumulators incl. bias_q. */
+/* ---- quantised Conv2d, f32 NCHW activations, the "conv2d_*" arm of CpuBackend::dispatch
+ * (src/backend/cpu/mod.rs:4100-4266), selected by the type of the registered weight:
+ *  I8: conv2d_packed_i8x4 (src/backend/cpu/packed_conv.rs:1118-1196) = im2col + per-(image,group)
+ *      dynamic int8 activation quantisation (packed_conv.rs:125-232) + gemm_packed_i8x4_fused_raw
+ *      (packed_conv.rs:444-625);
+ *  I4: conv2d_packed_i4x8 (packed_conv.rs:1202-1280): the same with 4-bit weights and activations
+ *      quantised to 16 levels (packed_conv.rs:236-283, 659-841);
+ *  U8, U4, F8, F8R, F4, I4CB: weights dequantised, f32 convolution conv2d_f32_im2col_gemm
+ *      (src/backend/cpu/mod.rs:4204-4257, src/backend/cpu/microkernels/conv.rs:509-660).
+ * acc_out (nullable, same shape as y; I8 and I4 only) receives the i32 accumulators incl. bias_q. */
 int fnn_hip_qconv2d(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *x, int64_t b,
                     int64_t c, int64_t h, int64_t wd, int kh, int kw, int stride, int pad,
                     int dil, int groups, const float *bias, int act, float *y, int32_t *acc_out,

@@ -1121,6 +1121,59 @@ int fnn_or_qconv2d_i4(const float *x, size_t b, size_t c, size_t h, size_t w,
                        stride, pad, dil, groups, act, y, acc_out, act_scale_out, act_zero_out);
 }
 
+/* Conv2d for the weight types without an integer kernel (U8, U4, F8, F8R, F4 and 4-bit codebook
+ * weights; backend/cpu/mod.rs:4204-4257): the weights are dequantised to f32 once
+ * (get_or_init_f32_weights, packed_tensor.rs:469-521) and conv2d_f32_im2col_gemm
+ * (microkernels/conv.rs:509-660) runs an ordinary f32 convolution:
+ *   y[b, oc, p] = act( sum_e W[oc, e] * col[p, e] + bias[oc] ),
+ * col as in the integer lowering (im2col.rs:32-52), bias and activation applied after the GEMM
+ * (conv_gemm.rs:26-47,154-235; GELU in its tanh form with the cubic term, :121-143).
+ * The GEMM is a third-party SGEMM (crate gemm 0.19 / matrixmultiply): its summation order is not
+ * part of the contract, so the sum is taken in double here and results are compared by tolerance. */
+int fnn_or_qconv2d_float(int dt, const float *x, size_t b, size_t c, size_t h, size_t w,
+                         const uint32_t *words, size_t oc, const float *scales, size_t n_scales,
+                         const float *zeros, size_t n_zeros, size_t qblock, const float *codebook,
+                         const float *bias, size_t kh, size_t kw, size_t stride, size_t pad,
+                         size_t dil, size_t groups, int act, float *y)
+{
+    if (groups == 0 || c % groups || oc % groups) return -1;
+    size_t cg = c / groups, ocg = oc / groups;
+    size_t ho = fnn_or_conv_out_size(h, kh, stride, pad, dil);
+    size_t wo = fnn_or_conv_out_size(w, kw, stride, pad, dil);
+    size_t np = ho * wo;
+    size_t kk = cg * kh * kw;
+    float *wf = (float *)malloc((oc * kk + 1) * sizeof(float));
+    if (!wf) return -2;
+    int rc = fnn_or_dequant(dt, words, oc, kk, scales, n_scales, zeros, n_zeros, qblock, codebook, wf);
+    if (rc) { free(wf); return rc; }
+    for (size_t nn = 0; nn < b; nn++)
+        for (size_t g = 0; g < groups; g++) {
+            const float *xin = x + nn * c * h * w + g * cg * h * w;
+            for (size_t f = 0; f < ocg; f++) {
+                size_t ch = g * ocg + f;
+                const float *wrow = wf + ch * kk;
+                for (size_t oh = 0; oh < ho; oh++)
+                    for (size_t ow = 0; ow < wo; ow++) {
+                        double acc = 0.0;
+                        for (size_t ic = 0; ic < cg; ic++)
+                            for (size_t i = 0; i < kh; i++)
+                                for (size_t j = 0; j < kw; j++) {
+                                    size_t ih = oh * stride + i * dil - pad; /* wraps when < 0 */
+                                    size_t iw = ow * stride + j * dil - pad;
+                                    if (ih < h && iw < w)
+                                        acc += (double)wrow[(ic * kh + i) * kw + j] *
+                                               (double)xin[(ic * h + ih) * w + iw];
+                                }
+                        float v = (float)acc;
+                        if (bias) v = v + bias[ch];
+                        y[(nn * oc + ch) * np + oh * wo + ow] = fnn_or_act(v, act);
+                    }
+            }
+        }
+    free(wf);
+    return 0;
+}
+
 /* ------------------------------------------------------------------------ */
 /* generators                                                                 */
 /* ------------------------------------------------------------------------ */

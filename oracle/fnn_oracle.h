@@ -110,6 +110,14 @@ int fnn_or_qconv2d_i4(const float *x, size_t b, size_t c, size_t h, size_t w,
                       int act, float *y, int32_t *acc_out, float *act_scale_out,
                       float *act_zero_out);
 
+/* weight types without an integer kernel: dequantise once, f32 convolution
+ * (backend/cpu/mod.rs:4204-4257, microkernels/conv.rs:509-660) */
+int fnn_or_qconv2d_float(int dt, const float *x, size_t b, size_t c, size_t h, size_t w,
+                         const uint32_t *words, size_t oc, const float *scales, size_t n_scales,
+                         const float *zeros, size_t n_zeros, size_t qblock, const float *codebook,
+                         const float *bias, size_t kh, size_t kw, size_t stride, size_t pad,
+                         size_t dil, size_t groups, int act, float *y);
+
 /* ---- generators used by the reference's own tests ------------------------ */
 void fnn_or_seeded_values(uint64_t seed, size_t len, float *out);
 

@@ -97,6 +97,9 @@ def _proto(l):
                                     C.c_void_p, _sz, C.c_void_p, _sz, _sz, _sz, _sz, _sz, _sz,
                                     C.c_int, _f32p, C.c_void_p, C.c_void_p, C.c_void_p]
     l.fnn_or_qconv2d_i4.argtypes = l.fnn_or_qconv2d_i8.argtypes
+    l.fnn_or_qconv2d_float.argtypes = [C.c_int, _f32p, _sz, _sz, _sz, _sz, _u32p, _sz, C.c_void_p, _sz,
+                                       C.c_void_p, _sz, _sz, C.c_void_p, C.c_void_p, _sz, _sz, _sz, _sz,
+                                       _sz, _sz, C.c_int, _f32p]
     l.fnn_or_seeded_values.argtypes = [C.c_uint64, _sz, _f32p]
 
 
@@ -291,4 +294,22 @@ def qconv2d_i8(x, p: Packed, kh: int, kw: int, stride: int, pad: int, dil: int, 
         raise ValueError(f"qconv2d_i8 rc={rc}")
     if want_acc:
         return y, acc, sa, za
+    return y
+
+
+def qconv2d_float(x, p: Packed, kh: int, kw: int, stride: int, pad: int, dil: int, groups: int,
+                  bias=None, act: int = ACT_NONE) -> np.ndarray:
+    """Conv2d of the weight types without an integer kernel: f32 convolution with dequantised weights."""
+    x = _f32(x)
+    b, c, h, w = x.shape
+    oc = p.rows
+    ho, wo = conv_out_size(h, kh, stride, pad, dil), conv_out_size(w, kw, stride, pad, dil)
+    y = np.zeros((b, oc, ho, wo), np.float32)
+    bb = None if bias is None else _f32(bias)
+    rc = lib().fnn_or_qconv2d_float(p.dt, x.reshape(-1), b, c, h, w, p.words, oc, _ptr(p.scales), p.scales.size,
+                                    _ptr(p.zeros) if p.zeros.size else None, p.zeros.size, p.qblock,
+                                    _ptr(p.codebook), _ptr(bb), kh, kw, stride, pad, dil, groups, act,
+                                    y.reshape(-1))
+    if rc:
+        raise ValueError(f"qconv2d_float rc={rc}")
     return y

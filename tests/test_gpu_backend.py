@@ -297,3 +297,30 @@ def test_plan_that_rewrites_its_constants_never_replays(be, orc):
         be.dispatch(plan)
         assert not plan.replayed
         assert_close(be.read_arena(*s_o, np.float32).reshape(m, n), want, 2e-5, "clobbered constant")
+
+
+@pytest.mark.parametrize("wdt,kname", [(flib.DT_U8, "conv2d_u8"), (flib.DT_U4, "conv2d_u4"), (flib.DT_F8, "conv2d_f8"),
+                                       (flib.DT_F8R, "conv2d_f8r"), (flib.DT_F4, "conv2d_f4"), (flib.DT_I4CB, "conv2d_i4")])
+def test_conv2d_float_weight_plans(be, orc, wdt, kname):
+    """conv2d_{u8,u4,f8,f8r,f4} and conv2d_i4 with a codebook: f32 convolution with dequantised weights."""
+    rng = np.random.default_rng(43 + wdt)
+    b, c, h, w, oc, kh, kw, stride, pad, dil, groups = 2, 32, 10, 9, 24, 1, 1, 1, 0, 1, 1
+    kk = c // groups * kh * kw
+    x = rng.standard_normal((b, c, h, w)).astype(np.float32)
+    pw = fastnn_amd.quantize_weights(wdt, (rng.standard_normal((oc, kk)) * 0.2).astype(np.float32))
+    bias = (rng.standard_normal(oc) * 0.05).astype(np.float32)
+    want = orc.qconv2d_float(x, to_oracle(orc, pw), kh, kw, stride, pad, dil, groups, bias=bias, act=flib.ACT_SILU)
+    a = Arena()
+    s_x, s_w, s_b, s_y = a.take(x.nbytes), a.take(pw.words.nbytes), a.take(bias.nbytes), a.take(want.nbytes)
+    plan = ExecutablePlan(a.top).write_const(s_w[0], pw.words).write_const(s_b[0], bias)
+    plan.call_kernel(kname + "_silu", [s_x, s_w, s_b], s_y, [stride, pad, dil, groups, c, h, w, kh, kw],
+                     meta_of(pw, [oc, c // groups, kh, kw]))
+    be.allocate_arena(a.top)
+    be.write_arena(s_x[0], x)
+    be.dispatch(plan)
+    assert_close(be.read_arena(*s_y, np.float32).reshape(want.shape), want, 2e-5, kname)
+    be.write_arena(s_x[0], x * 0.5)                     # resident plan: graph replay of the three launches
+    be.dispatch(plan)
+    assert plan.replayed
+    want2 = orc.qconv2d_float(x * 0.5, to_oracle(orc, pw), kh, kw, stride, pad, dil, groups, bias=bias, act=flib.ACT_SILU)
+    assert_close(be.read_arena(*s_y, np.float32).reshape(want.shape), want2, 2e-5, kname + " replay")

@@ -308,6 +308,42 @@ def test_qconv2d_constant_and_empty(ctx, orc, wdt):
     ctx.release(h)
 
 
+FLOAT_CONVS = [
+    dict(b=2, c=4, h=20, w=24, oc=16, kh=3, kw=3, stride=2, pad=1, dil=1, groups=1),
+    dict(b=1, c=32, h=12, w=12, oc=48, kh=1, kw=1, stride=1, pad=0, dil=1, groups=1),
+    dict(b=1, c=8, h=10, w=7, oc=6, kh=3, kw=2, stride=1, pad=2, dil=2, groups=2),
+    dict(b=3, c=32, h=9, w=9, oc=40, kh=3, kw=3, stride=1, pad=1, dil=1, groups=1),
+]
+
+
+@pytest.mark.parametrize("cfg", FLOAT_CONVS)
+@pytest.mark.parametrize("wdt", [flib.DT_U8, flib.DT_U4, flib.DT_F8, flib.DT_F8R, flib.DT_F4, flib.DT_I4CB])
+def test_qconv2d_float_weight_types(ctx, orc, cfg, wdt):
+    """Weight types without an integer conv kernel: f32 convolution with the dequantised weights
+    (im2col rows + fused-dequant MatMul + NCHW turn on the GPU); f32 accumulation, stated bound 2e-5."""
+    rng = np.random.default_rng(6100 + cfg["c"] + wdt)
+    kk = cfg["c"] // cfg["groups"] * cfg["kh"] * cfg["kw"]
+    if wdt == flib.DT_I4CB and kk % 32:
+        pytest.skip("codebook blocks of 32 values")
+    x = rng.standard_normal((cfg["b"], cfg["c"], cfg["h"], cfg["w"])).astype(np.float32)
+    wt = (rng.standard_normal((cfg["oc"], kk)) * np.sqrt(2.0 / kk)).astype(np.float32)
+    bias = (rng.standard_normal(cfg["oc"]) * 0.05).astype(np.float32)
+    pw = fastnn_amd.quantize_weights(wdt, wt)
+    h = ctx.register(pw)
+    args = (cfg["kh"], cfg["kw"], cfg["stride"], cfg["pad"], cfg["dil"], cfg["groups"])
+    for act in (0, 1, 2, 3):
+        want = orc.qconv2d_float(x, to_oracle(orc, pw), *args, bias=bias, act=act)
+        got = ctx.qconv2d(h, x, cfg["oc"], *args, bias=bias, act=act)
+        assert_close(got, want, 2e-5, f"act {act}")
+    assert_close(ctx.qconv2d(h, x, cfg["oc"], *args), orc.qconv2d_float(x, to_oracle(orc, pw), *args), 2e-5, "no bias")
+    got_g = ctx.qconv2d(h, x, cfg["oc"], *args, bias=bias, act=3, flags=flib.FLAG_FORCE_GENERIC)
+    assert_close(got_g, orc.qconv2d_float(x, to_oracle(orc, pw), *args, bias=bias, act=3), 2e-5, "shape-agnostic kernel")
+    with pytest.raises(fastnn_amd.FnnError) as e:      # no integer accumulators on this path
+        ctx.qconv2d(h, x, cfg["oc"], *args, want_acc=True)
+    assert e.value.kind == "Dispatch"
+    ctx.release(h)
+
+
 # --------------------------------------------------------------------------- error behaviour
 def test_error_paths_mirror_reference_messages(ctx):
     rng = np.random.default_rng(11)

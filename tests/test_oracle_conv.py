@@ -104,3 +104,46 @@ def test_conv_i4_constant_input_keeps_its_zero_point(orc):
     assert np.array_equal(acc[0, :, 0, 0], -8 * qw.sum(axis=1))
     deq = orc.dequant(p)
     assert np.allclose(y[0, :, 0, 0], 0.5 * deq.sum(axis=1), atol=1e-5)
+
+
+@pytest.mark.parametrize("dt", ["U8", "U4", "F8", "F8R", "F4", "I4CB"])
+@pytest.mark.parametrize("cfg", [
+    dict(b=2, c=4, h=9, w=11, oc=6, kh=3, kw=3, stride=2, pad=1, dil=1, groups=1),
+    dict(b=1, c=8, h=10, w=7, oc=4, kh=3, kw=2, stride=1, pad=2, dil=2, groups=2),
+    dict(b=1, c=32, h=5, w=5, oc=8, kh=1, kw=1, stride=1, pad=0, dil=1, groups=1),
+])
+def test_float_conv_equals_torch_conv_of_dequantised_weights(orc, dt, cfg):
+    """The weight types without an integer conv kernel: an ordinary convolution with the dequantised
+    weights, bias added after the sum, then the activation (checked against torch.nn.functional.conv2d
+    in float64, an independent implementation)."""
+    rng = np.random.default_rng(77)
+    b, c, h, w, oc, kh, kw = (cfg[x] for x in ("b", "c", "h", "w", "oc", "kh", "kw"))
+    stride, pad, dil, groups = cfg["stride"], cfg["pad"], cfg["dil"], cfg["groups"]
+    kk = c // groups * kh * kw
+    x = rng.standard_normal((b, c, h, w)).astype(np.float32)
+    wt = (rng.standard_normal((oc, kk)) * 0.2).astype(np.float32)
+    bias = (rng.standard_normal(oc) * 0.1).astype(np.float32)
+    code = getattr(orc, dt)
+    if dt == "I4CB":
+        if kk % 32:
+            pytest.skip("codebook blocks of 32")
+        p = orc.quantize(code, wt, qblock=32)
+    else:
+        p = orc.quantize(code, wt)
+    deq = orc.dequant(p).astype(np.float64).reshape(oc, c // groups, kh, kw)
+    for act in (0, 1, 2, 3):
+        got = orc.qconv2d_float(x, p, kh, kw, stride, pad, dil, groups, bias=bias, act=act)
+        ref = F.conv2d(torch.from_numpy(x.astype(np.float64)), torch.from_numpy(deq), torch.from_numpy(bias.astype(np.float64)),
+                       stride=stride, padding=pad, dilation=dil, groups=groups).numpy()
+        if act == 1:
+            ref = np.maximum(ref, 0)
+        elif act == 2:
+            ref = 0.5 * ref * (1 + np.tanh(0.7978846 * (ref + 0.044715 * ref ** 3)))
+        elif act == 3:
+            ref = ref / (1 + np.exp(-ref))
+        assert got.shape == ref.shape
+        assert np.abs(got - ref).max() <= 2e-6 * (np.abs(ref).max() + 1), (dt, cfg, act)
+    nb = orc.qconv2d_float(x, p, kh, kw, stride, pad, dil, groups)
+    ref = F.conv2d(torch.from_numpy(x.astype(np.float64)), torch.from_numpy(deq), None, stride=stride, padding=pad,
+                   dilation=dil, groups=groups).numpy()
+    assert np.abs(nb - ref).max() <= 2e-6 * (np.abs(ref).max() + 1)
