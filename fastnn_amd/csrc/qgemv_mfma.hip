@@ -169,8 +169,9 @@ __global__ void __launch_bounds__(NW * 64) qgemv_mfma_kernel(GemvArgs p)
                         __builtin_bit_cast(uint4, f16x8{lo[0], lo[1], lo[2], lo[3], lo[4], lo[5], lo[6], lo[7]});
             }
         }
-        // (the fragments are written and read by this wave only: LDS operations of one wave complete in
-        //  order, so no workgroup barrier is needed here or before the next round rewrites the area)
+        // (only this wave reads these fragments, but the workgroup barrier stays: with the waves kept in
+        //  step the weight stream measures 5-8 % faster for the 8-bit types than without it)
+        __syncthreads();
 
         // ---- 3. MFMA over the slice: straight-line, one MFMA per step and row tile
         f32x4 acc[RT];
@@ -190,6 +191,7 @@ __global__ void __launch_bounds__(NW * 64) qgemv_mfma_kernel(GemvArgs p)
         for (int r = 0; r < RT; r++)
 #pragma unroll
             for (int i = 0; i < 4; i++) tot[r][i] = fmaf(acc[r][i], csc[i % MM], tot[r][i]);
+        __syncthreads();  // the wave areas are rewritten by the next round
     }
 
     // ---- 4. fixed-order reduction over the waves (hi row + lo row), fused epilogue

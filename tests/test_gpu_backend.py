@@ -182,10 +182,14 @@ def test_unsupported_and_malformed_instructions(be):
     with pytest.raises(flib.FnnError) as e:
         be.dispatch(p)
     assert e.value.kind == "UnsupportedOp" and e.value.message == "softmax_f32"
+    p = ExecutablePlan(4096).call_kernel("conv2d_i4_i8", [(0, 64), (64, 64)], (128, 64), [1] * 9)
+    with pytest.raises(flib.FnnError) as e:      # the I8-payload conv variants are not implemented
+        be.dispatch(p)
+    assert e.value.kind == "UnsupportedOp" and e.value.message == "conv2d_i4_i8"
     p = ExecutablePlan(4096).call_kernel("conv2d_i4", [(0, 64), (64, 64)], (128, 64), [1] * 9)
     with pytest.raises(flib.FnnError) as e:
         be.dispatch(p)
-    assert e.value.kind == "UnsupportedOp"
+    assert e.value.kind == "Dispatch" and "missing weight_meta" in e.value.message
     p = ExecutablePlan(4096).call_kernel("matmul_i8", [(0, 64), (64, 64)], (128, 64), [4, 4])
     with pytest.raises(flib.FnnError) as e:
         be.dispatch(p)
