@@ -24,6 +24,11 @@ hipError_t launch_im2col_f32(const float *x, float *col, int64_t b, int64_t c, i
 hipError_t launch_rows_to_nchw(const float *src, float *y, int64_t b, int64_t np, int64_t oc, int64_t ch0, int64_t ocg, hipStream_t s);
 hipError_t launch_fill(float *dst, uint64_t n, float value, hipStream_t s);
 hipError_t launch_eltwise(int op, const float *a, const float *b, uint64_t nb, float *out, uint64_t n, hipStream_t s);
+hipError_t launch_copy2d(float *dst, uint64_t dst_pitch, uint64_t dst_len, const float *src, uint64_t src_pitch, uint64_t src_len,
+                         uint64_t width, uint64_t height, hipStream_t s);
+hipError_t launch_maxpool2d(const float *x, uint64_t in_len, float *y, uint64_t out_len, uint64_t c, uint64_t h, uint64_t w,
+                            uint64_t ho, uint64_t wo, int kernel, int stride, int pad, hipStream_t s);
+hipError_t launch_upsample_nearest2d(const float *x, float *y, uint64_t nc, uint64_t h, uint64_t w, int sh, int sw, hipStream_t s);
 
 struct fnn_hip_graph {
     hipGraph_t graph = nullptr;
@@ -661,6 +666,35 @@ int fnn_hip_copy(fnn_hip_ctx *ctx, void *dst_dev, const void *src_dev, uint64_t 
     if (!ctx || ((!dst_dev || !src_dev) && bytes)) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_copy: NULL argument");
     if (bytes == 0) return FNN_OK;
     HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(dst_dev, src_dev, bytes, hipMemcpyDeviceToDevice, ctx->stream));
+    return FNN_OK;
+}
+
+int fnn_hip_copy2d_f32(fnn_hip_ctx *ctx, float *dst, uint64_t dst_pitch, uint64_t dst_len, const float *src, uint64_t src_pitch,
+                       uint64_t src_len, uint64_t width, uint64_t height)
+{
+    if (!ctx || ((!dst || !src) && width && height)) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_copy2d_f32: NULL argument");
+    HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_copy2d(dst, dst_pitch, dst_len, src, src_pitch, src_len, width, height, ctx->stream));
+    return FNN_OK;
+}
+
+int fnn_hip_maxpool2d_f32(fnn_hip_ctx *ctx, const float *x, uint64_t in_len, float *y, uint64_t out_len, uint64_t n, uint64_t c,
+                          uint64_t h, uint64_t w, uint64_t kernel, uint64_t stride, uint64_t pad)
+{
+    if (!ctx || !x || !y) return fail(ctx, FNN_ERR_DISPATCH, "pool_f32: NULL argument");
+    if (kernel == 0 || stride == 0 || kernel > 1024 || pad > 1024) return fail(ctx, FNN_ERR_DISPATCH, "pool_f32: invalid kernel, stride or padding");
+    const uint64_t hp = h + 2 * pad, wp = w + 2 * pad;
+    const uint64_t ho = (hp > kernel ? hp - kernel : 0) / stride + 1, wo = (wp > kernel ? wp - kernel : 0) / stride + 1;
+    uint64_t total = n * c * ho * wo;
+    if (total > out_len) total = out_len;   // writes past the output slice are dropped (ops.rs:147-149)
+    HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_maxpool2d(x, in_len, y, total, c, h, w, ho, wo, (int)kernel, (int)stride, (int)pad, ctx->stream));
+    return FNN_OK;
+}
+
+int fnn_hip_upsample_nearest2d_f32(fnn_hip_ctx *ctx, const float *x, float *y, uint64_t nc, uint64_t h, uint64_t w, uint64_t sh, uint64_t sw)
+{
+    if (!ctx || !x || !y) return fail(ctx, FNN_ERR_DISPATCH, "upsample_nearest2d: NULL argument");
+    if (sh > 1024 || sw > 1024) return fail(ctx, FNN_ERR_DISPATCH, "upsample_nearest2d: scale too large");
+    HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_upsample_nearest2d(x, y, nc, h, w, (int)sh, (int)sw, ctx->stream));
     return FNN_OK;
 }
 

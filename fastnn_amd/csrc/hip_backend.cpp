@@ -97,7 +97,7 @@ struct fnn_plan {
     // HIP graph of the instruction stream, captured on a dispatch that found everything resident;
     // valid while the backend, its arena, its cached weights and the context's workspaces are the same
     fnn_hip_graph *graph = nullptr;
-    uint64_t graph_uid = 0, graph_generation = 0, graph_weights_epoch = 0, graph_ws_epoch = 0;
+    uint64_t graph_uid = 0, graph_generation = 0, graph_weights_epoch = 0, graph_ws_epoch = 0, graph_scratch_epoch = 0;
     int graph_failures = 0;           // captures that did not go through; after two the plan stays eager
     bool last_replayed = false;
 };
@@ -117,6 +117,8 @@ struct fnn_backend {
     std::string err;
     std::map<std::pair<uint64_t, uint64_t>, fnn_hip_weight *> weights;  // (offset,size) like get_or_cache_packed
     std::vector<uint8_t> stage;
+    uint8_t *scratch = nullptr;   // device copy of an input that overlaps its output
+    uint64_t scratch_bytes = 0, scratch_epoch = 0;
 };
 
 namespace {
@@ -331,6 +333,116 @@ int run_elementwise(fnn_backend *b, const Instr &in, int op)
                                        (float *)(b->arena + in.dst.offset), n));
 }
 
+// An f32 op that reads `in` and writes `out` elementwise-unrelated positions must not alias: the CPU arms copy
+// the input first when the slices overlap (src/backend/cpu/arena.rs:14-60).  Here: one device copy into the
+// backend's scratch buffer.
+int staged_input(fnn_backend *b, const fnn_slice &in, const fnn_slice &out, const float **src)
+{
+    *src = (const float *)(b->arena + in.offset);
+    if (!overlaps(in, out)) return FNN_OK;
+    if (b->scratch_bytes < in.size) {
+        if (b->scratch) fnn_hip_free(b->ctx, b->scratch);
+        b->scratch = nullptr;
+        b->scratch_bytes = 0;
+        void *d = nullptr;
+        int st = lift(b, fnn_hip_malloc(b->ctx, in.size + 64, &d));
+        if (st) return st;
+        b->scratch = (uint8_t *)d;
+        b->scratch_bytes = in.size;
+        b->scratch_epoch++;
+    }
+    int st = lift(b, fnn_hip_copy(b->ctx, b->scratch, b->arena + in.offset, in.size));
+    *src = (const float *)b->scratch;
+    return st;
+}
+
+// "concat": params [axis, inner_stride, outer_count] (src/backend/cpu/mod.rs:4267-4324)
+int run_concat(fnn_backend *b, const Instr &in)
+{
+    if (in.inputs.empty()) return FNN_OK;
+    const uint64_t out_len = in.dst.size / 4;
+    float *out = (float *)(b->arena + in.dst.offset);
+    for (const auto &s : in.inputs)
+        if (overlaps(s, in.dst)) return fail(b, FNN_ERR_DISPATCH, "concat: an input overlaps the output");
+    if (in.params.size() >= 3) {
+        const uint64_t outer = in.params[2] ? in.params[2] : 1;
+        uint64_t pitch = 0;
+        for (const auto &s : in.inputs) pitch += (s.size / 4) / outer;
+        uint64_t off = 0;
+        for (const auto &s : in.inputs) {
+            const uint64_t len = s.size / 4, bs = len / outer;
+            if (len % outer) return fail(b, FNN_ERR_DISPATCH, "concat: input of %llu elements does not split into %llu outer positions", (unsigned long long)len, (unsigned long long)outer);
+            if (off < out_len) {
+                int st = lift(b, fnn_hip_copy2d_f32(b->ctx, out + off, pitch, out_len - off, (const float *)(b->arena + s.offset), bs, len, bs, in.params[2]));
+                if (st) return st;
+            }
+            off += bs;
+        }
+        return FNN_OK;
+    }
+    uint64_t off = 0;   // legacy form without axis information: inputs one after the other
+    for (const auto &s : in.inputs) {
+        const uint64_t len = s.size / 4;
+        if (off < out_len) {
+            int st = lift(b, fnn_hip_copy2d_f32(b->ctx, out + off, len, out_len - off, (const float *)(b->arena + s.offset), len, len, len, 1));
+            if (st) return st;
+        }
+        off += len;
+    }
+    return FNN_OK;
+}
+
+// "slice_f32": params [dim, start, end, stride] (src/backend/cpu/mod.rs:4721-4760)
+int run_slice(fnn_backend *b, const Instr &in)
+{
+    if (in.inputs.empty()) return FNN_OK;
+    if (in.params.size() != 4) return fail(b, FNN_ERR_DISPATCH, "slice_f32: expected params [dim, start, end, stride]");
+    const uint64_t start = in.params[1], end = in.params[2], stride = in.params[3];
+    const uint64_t in_len = in.inputs[0].size / 4, out_len = in.dst.size / 4;
+    uint64_t range_len = end > start ? end - start : 0;
+    if (range_len < 1) range_len = 1;
+    const uint64_t dim_size = out_len ? (in_len * range_len) / out_len : 0;
+    const uint64_t outer = (dim_size > 0 && stride > 0) ? in_len / dim_size / stride : 1;
+    const uint64_t slice_elems = range_len * stride;
+    const uint64_t first = start * stride;
+    if (first >= in_len || slice_elems == 0) return FNN_OK;
+    const float *src = nullptr;
+    int st = staged_input(b, in.inputs[0], in.dst, &src);
+    if (st) return st;
+    return lift(b, fnn_hip_copy2d_f32(b->ctx, (float *)(b->arena + in.dst.offset), slice_elems, out_len, src + first, dim_size * stride,
+                                      in_len - first, slice_elems, outer));
+}
+
+// "pool_f32": params [kernel, stride, padding, is_max, N, C, H, W] (src/backend/cpu/mod.rs:4362-4397)
+int run_pool(fnn_backend *b, const Instr &in)
+{
+    if (in.inputs.empty()) return FNN_OK;
+    if (in.params.size() != 8) return fail(b, FNN_ERR_DISPATCH, "pool_f32: expected params [kernel, stride, padding, is_max, N, C, H, W]");
+    const uint64_t *p = in.params.data();
+    if (p[3] != 1) return fail(b, FNN_ERR_UNSUPPORTED_OP, "pool_f32: average pooling is not implemented on the GPU");
+    const float *src = nullptr;
+    int st = staged_input(b, in.inputs[0], in.dst, &src);
+    if (st) return st;
+    return lift(b, fnn_hip_maxpool2d_f32(b->ctx, src, in.inputs[0].size / 4, (float *)(b->arena + in.dst.offset), in.dst.size / 4, p[4], p[5],
+                                         p[6], p[7], p[0], p[1], p[2]));
+}
+
+// "upsample_nearest2d": params [scale_h, scale_w, h_in, w_in], defaults 2, 2, 1, 1 (src/backend/cpu/mod.rs:5496-5535)
+int run_upsample(fnn_backend *b, const Instr &in)
+{
+    if (in.inputs.empty()) return FNN_OK;
+    const uint64_t sh = in.params.size() > 0 ? in.params[0] : 2, sw = in.params.size() > 1 ? in.params[1] : 2;
+    const uint64_t h = in.params.size() > 2 ? in.params[2] : 1, w = in.params.size() > 3 ? in.params[3] : 1;
+    const uint64_t hw = h * w, in_len = in.inputs[0].size / 4;
+    if (!(sh > 0 && sw > 0 && hw > 0 && in_len > 0 && in_len % hw == 0)) return FNN_OK;   // the CPU arm does nothing either
+    const uint64_t nc = in_len / hw;
+    if (in.dst.size / 4 < nc * hw * sh * sw) return fail(b, FNN_ERR_DISPATCH, "upsample_nearest2d: output slice holds %llu values, needs %llu", (unsigned long long)(in.dst.size / 4), (unsigned long long)(nc * hw * sh * sw));
+    const float *src = nullptr;
+    int st = staged_input(b, in.inputs[0], in.dst, &src);
+    if (st) return st;
+    return lift(b, fnn_hip_upsample_nearest2d_f32(b->ctx, src, (float *)(b->arena + in.dst.offset), nc, h, w, sh, sw));
+}
+
 int run_call(fnn_backend *b, const Instr &in)
 {
     for (const auto &s : in.inputs)
@@ -344,6 +456,10 @@ int run_call(fnn_backend *b, const Instr &in)
     if (name == "relu_f32") return run_elementwise(b, in, 1);
     if (name == "gelu_f32") return run_elementwise(b, in, 2);
     if (name == "silu_f32") return run_elementwise(b, in, 3);
+    if (name == "concat") return run_concat(b, in);
+    if (name == "slice_f32") return run_slice(b, in);
+    if (name == "pool_f32") return run_pool(b, in);
+    if (name == "upsample_nearest2d") return run_upsample(b, in);
     KernelName kn = split_activation(name);
     int dt = matmul_dtype(kn.base);
     if (dt >= 0) return run_matmul(b, in, kn, dt);
@@ -422,21 +538,22 @@ int dispatch_impl(fnn_backend *b, fnn_plan *p, uint64_t *elapsed_ns, uint64_t n_
     static const bool graphs_on = [] { const char *e = getenv("FNN_PLAN_GRAPH"); return !(e && e[0] == '0'); }();
     const bool may_replay = graphs_on && !elapsed_ns && resident && !p->uploads_every_run && p->graph_failures < 2;
     if (p->graph && !(may_replay && p->graph_uid == b->uid && p->graph_generation == b->generation &&
-                      p->graph_weights_epoch == b->weights_epoch && p->graph_ws_epoch == fnn_hip_workspace_epoch(b->ctx))) {
+                      p->graph_weights_epoch == b->weights_epoch && p->graph_ws_epoch == fnn_hip_workspace_epoch(b->ctx) &&
+                      p->graph_scratch_epoch == b->scratch_epoch)) {
         fnn_hip_graph_destroy(p->graph_uid == b->uid ? b->ctx : nullptr, p->graph);
         p->graph = nullptr;
     }
     if (may_replay && !p->graph) {
-        const uint64_t w0 = b->weights_epoch, s0 = fnn_hip_workspace_epoch(b->ctx);
+        const uint64_t w0 = b->weights_epoch, s0 = fnn_hip_workspace_epoch(b->ctx), c0 = b->scratch_epoch;
         if (fnn_hip_graph_begin(b->ctx) == FNN_OK) {
             int st = FNN_OK;
             for (size_t i = 0; i < p->instrs.size() && st == FNN_OK; i++) st = run_instr(b, p, p->instrs[i], true);
             fnn_hip_graph *g = nullptr;
             int en = fnn_hip_graph_end(b->ctx, &g);
-            if (st == FNN_OK && en == FNN_OK && g && w0 == b->weights_epoch && s0 == fnn_hip_workspace_epoch(b->ctx)) {
+            if (st == FNN_OK && en == FNN_OK && g && w0 == b->weights_epoch && s0 == fnn_hip_workspace_epoch(b->ctx) && c0 == b->scratch_epoch) {
                 p->graph = g;
                 p->graph_uid = b->uid; p->graph_generation = b->generation;
-                p->graph_weights_epoch = w0; p->graph_ws_epoch = s0;
+                p->graph_weights_epoch = w0; p->graph_ws_epoch = s0; p->graph_scratch_epoch = c0;
             } else {
                 if (g) fnn_hip_graph_destroy(b->ctx, g);
                 p->graph_failures++;
@@ -497,6 +614,7 @@ void fnn_backend_destroy(fnn_backend *b)
     if (!b) return;
     drop_weights(b);
     if (b->arena) fnn_hip_free(b->ctx, b->arena);
+    if (b->scratch) fnn_hip_free(b->ctx, b->scratch);
     fnn_hip_destroy(b->ctx);
     delete b;
 }

@@ -82,6 +82,21 @@ int fnn_backend_dispatch_profile(fnn_backend *b, fnn_plan *p, uint64_t *elapsed_
 int fnn_hip_elementwise(fnn_hip_ctx *ctx, int op, const float *a, const float *b, uint64_t nb,
                         float *out, uint64_t n);
 
+/* f32 data movement between quantised convolutions, device pointers, lengths in elements:
+ *  copy2d: `height` rows of `width` values, dst[r*dst_pitch + c] = src[r*src_pitch + c], dropped where either
+ *    index leaves its buffer: the block copies of "concat" (src/backend/cpu/mod.rs:4267-4324) and "slice_f32"
+ *    (:4721-4760);
+ *  maxpool2d: "pool_f32" with is_max = 1 (:4362-4397, src/backend/cpu/microkernels/ops.rs:104-158), output
+ *    Ho = sat_sub(H + 2*pad, kernel)/stride + 1, writes past out_len dropped;
+ *  upsample_nearest2d: "upsample_nearest2d" (:5496-5535, src/backend/cpu/microkernels/misc.rs:338-364). */
+int fnn_hip_copy2d_f32(fnn_hip_ctx *ctx, float *dst, uint64_t dst_pitch, uint64_t dst_len, const float *src,
+                       uint64_t src_pitch, uint64_t src_len, uint64_t width, uint64_t height);
+int fnn_hip_maxpool2d_f32(fnn_hip_ctx *ctx, const float *x, uint64_t in_len, float *y, uint64_t out_len,
+                          uint64_t n, uint64_t c, uint64_t h, uint64_t w, uint64_t kernel, uint64_t stride,
+                          uint64_t pad);
+int fnn_hip_upsample_nearest2d_f32(fnn_hip_ctx *ctx, const float *x, float *y, uint64_t nc, uint64_t h,
+                                   uint64_t w, uint64_t sh, uint64_t sw);
+
 /* Instruction::Fill (f32 elements) and Instruction::MemCopy on device memory
  * (src/backend/mod.rs:92-106); both only enqueue on the context's stream. */
 int fnn_hip_fill_f32(fnn_hip_ctx *ctx, float *dst, uint64_t n, float value);

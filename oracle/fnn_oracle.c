@@ -1175,6 +1175,99 @@ int fnn_or_qconv2d_float(int dt, const float *x, size_t b, size_t c, size_t h, s
 }
 
 /* ------------------------------------------------------------------------ */
+/* f32 data-movement ops found between quantised convolutions                 */
+/* ------------------------------------------------------------------------ */
+
+/* "concat" (backend/cpu/mod.rs:4267-4324): params [axis, inner_stride, outer_count]; every input
+ * contributes blocks of elems/max(outer_count,1) values; for each outer position the blocks of
+ * all inputs follow each other in the output.  Copies are clamped to the input and output lengths
+ * and the output position advances by the (input-clamped) length.  Returns values written. */
+size_t fnn_or_concat(const float *const *inputs, const size_t *lens, size_t n_inputs,
+                     size_t outer_count, float *out, size_t out_len)
+{
+    size_t off = 0;
+    for (size_t o = 0; o < outer_count; o++)
+        for (size_t si = 0; si < n_inputs; si++) {
+            size_t bs = lens[si] / (outer_count ? outer_count : 1);
+            size_t src = o * bs;
+            size_t end = src + bs < lens[si] ? src + bs : lens[si];
+            size_t copy_len = end > src ? end - src : 0;
+            size_t dst_end = off + copy_len < out_len ? off + copy_len : out_len;
+            size_t actual = dst_end > off ? dst_end - off : 0;
+            memcpy(out + off, inputs[si] + src, actual * sizeof(float));
+            off += copy_len;
+        }
+    return off;
+}
+
+/* "slice_f32" (backend/cpu/mod.rs:4721-4760): params [dim, start, end, stride] where stride is the
+ * number of elements per index of the sliced dimension; dim_size = in_len*range/out_len,
+ * outer = in_len/dim_size/stride, each outer position copies range*stride values from
+ * i*dim_size*stride + start*stride. */
+void fnn_or_slice(const float *in, size_t in_len, size_t start, size_t end, size_t stride,
+                  float *out, size_t out_len)
+{
+    size_t range_len = end > start ? end - start : 0;
+    if (range_len < 1) range_len = 1;
+    size_t dim_size = out_len ? (in_len * range_len) / out_len : 0;
+    size_t outer = (dim_size > 0 && stride > 0) ? in_len / dim_size / stride : 1;
+    size_t slice_elems = range_len * stride;
+    for (size_t i = 0; i < outer; i++) {
+        size_t src = i * dim_size * stride + start * stride;
+        size_t dst = i * slice_elems;
+        size_t room = in_len > src ? in_len - src : 0;
+        size_t copy_len = slice_elems < room ? slice_elems : room;
+        if (copy_len > 0) memcpy(out + dst, in + src, copy_len * sizeof(float));
+    }
+}
+
+/* "pool_f32" with is_max = 1 (backend/cpu/mod.rs:4362-4397, microkernels/ops.rs:104-158):
+ * params [kernel, stride, padding, is_max, N, C, H, W]; Ho = sat_sub(H + 2p, kernel)/stride + 1;
+ * the window maximum starts at -inf and is replaced on a strict `>`; taps in the padding are skipped. */
+void fnn_or_maxpool2d(const float *in, size_t in_len, size_t n, size_t c, size_t h, size_t w,
+                      size_t kernel, size_t stride, size_t pad, float *out, size_t out_len)
+{
+    size_t hp = h + 2 * pad, wp = w + 2 * pad;
+    size_t ho = (hp > kernel ? hp - kernel : 0) / stride + 1;
+    size_t wo = (wp > kernel ? wp - kernel : 0) / stride + 1;
+    for (size_t nn = 0; nn < n; nn++)
+        for (size_t cc = 0; cc < c; cc++)
+            for (size_t hh = 0; hh < ho; hh++)
+                for (size_t ww = 0; ww < wo; ww++) {
+                    float val = -INFINITY;
+                    for (size_t kh = 0; kh < kernel; kh++)
+                        for (size_t kw = 0; kw < kernel; kw++) {
+                            size_t hi = hh * stride + kh, wi = ww * stride + kw;
+                            if (hi < pad || wi < pad) continue;
+                            hi -= pad;
+                            wi -= pad;
+                            if (hi >= h || wi >= w) continue;
+                            size_t idx = nn * (c * h * w) + cc * (h * w) + hi * w + wi;
+                            if (idx < in_len && in[idx] > val) val = in[idx];
+                        }
+                    size_t o = nn * (c * ho * wo) + cc * (ho * wo) + hh * wo + ww;
+                    if (o < out_len) out[o] = val;
+                }
+}
+
+/* "upsample_nearest2d" (backend/cpu/mod.rs:5496-5535, microkernels/misc.rs:338-364):
+ * params [scale_h, scale_w, h_in, w_in]; nc = in_len/(h_in*w_in); every input value fills a
+ * scale_h x scale_w block of the output. */
+void fnn_or_upsample_nearest2d(const float *in, size_t nc, size_t h, size_t w, size_t sh, size_t sw,
+                               float *out)
+{
+    size_t hw = h * w, orow = w * sw;
+    for (size_t i = 0; i < nc; i++)
+        for (size_t hi = 0; hi < h; hi++)
+            for (size_t wi = 0; wi < w; wi++) {
+                float v = in[i * hw + hi * w + wi];
+                for (size_t a = 0; a < sh; a++)
+                    for (size_t b = 0; b < sw; b++)
+                        out[i * hw * sh * sw + (hi * sh + a) * orow + wi * sw + b] = v;
+            }
+}
+
+/* ------------------------------------------------------------------------ */
 /* generators                                                                 */
 /* ------------------------------------------------------------------------ */
 

@@ -118,6 +118,16 @@ int fnn_or_qconv2d_float(int dt, const float *x, size_t b, size_t c, size_t h, s
                          const float *bias, size_t kh, size_t kw, size_t stride, size_t pad,
                          size_t dil, size_t groups, int act, float *y);
 
+/* ---- f32 data-movement ops between quantised convolutions ---------------- */
+size_t fnn_or_concat(const float *const *inputs, const size_t *lens, size_t n_inputs,
+                     size_t outer_count, float *out, size_t out_len);
+void fnn_or_slice(const float *in, size_t in_len, size_t start, size_t end, size_t stride,
+                  float *out, size_t out_len);
+void fnn_or_maxpool2d(const float *in, size_t in_len, size_t n, size_t c, size_t h, size_t w,
+                      size_t kernel, size_t stride, size_t pad, float *out, size_t out_len);
+void fnn_or_upsample_nearest2d(const float *in, size_t nc, size_t h, size_t w, size_t sh, size_t sw,
+                               float *out);
+
 /* ---- generators used by the reference's own tests ------------------------ */
 void fnn_or_seeded_values(uint64_t seed, size_t len, float *out);
 

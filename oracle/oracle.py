@@ -100,6 +100,11 @@ def _proto(l):
     l.fnn_or_qconv2d_float.argtypes = [C.c_int, _f32p, _sz, _sz, _sz, _sz, _u32p, _sz, C.c_void_p, _sz,
                                        C.c_void_p, _sz, _sz, C.c_void_p, C.c_void_p, _sz, _sz, _sz, _sz,
                                        _sz, _sz, C.c_int, _f32p]
+    l.fnn_or_concat.argtypes = [C.c_void_p, C.c_void_p, _sz, _sz, _f32p, _sz]
+    l.fnn_or_concat.restype = _sz
+    l.fnn_or_slice.argtypes = [_f32p, _sz, _sz, _sz, _sz, _f32p, _sz]
+    l.fnn_or_maxpool2d.argtypes = [_f32p, _sz, _sz, _sz, _sz, _sz, _sz, _sz, _sz, _f32p, _sz]
+    l.fnn_or_upsample_nearest2d.argtypes = [_f32p, _sz, _sz, _sz, _sz, _sz, _f32p]
     l.fnn_or_seeded_values.argtypes = [C.c_uint64, _sz, _f32p]
 
 
@@ -313,3 +318,39 @@ def qconv2d_float(x, p: Packed, kh: int, kw: int, stride: int, pad: int, dil: in
     if rc:
         raise ValueError(f"qconv2d_float rc={rc}")
     return y
+
+
+def concat(inputs, outer_count: int, out_len: int) -> np.ndarray:
+    """The "concat" kernel: params [axis, inner_stride, outer_count]; inputs are flat f32 arrays."""
+    arrs = [_f32(a).reshape(-1) for a in inputs]
+    ptrs = (C.c_void_p * len(arrs))(*[a.ctypes.data for a in arrs])
+    lens = (C.c_size_t * len(arrs))(*[a.size for a in arrs])
+    out = np.zeros(out_len, np.float32)
+    lib().fnn_or_concat(ptrs, lens, len(arrs), outer_count, out, out_len)
+    return out
+
+
+def slice_f32(x, start: int, end: int, stride: int, out_len: int) -> np.ndarray:
+    """The "slice_f32" kernel: params [dim, start, end, stride = elements per index of the sliced dim]."""
+    x = _f32(x).reshape(-1)
+    out = np.zeros(out_len, np.float32)
+    lib().fnn_or_slice(x, x.size, start, end, stride, out, out_len)
+    return out
+
+
+def maxpool2d(x, kernel: int, stride: int, pad: int) -> np.ndarray:
+    x = _f32(x)
+    n, c, h, w = x.shape
+    ho = max(h + 2 * pad - kernel, 0) // stride + 1
+    wo = max(w + 2 * pad - kernel, 0) // stride + 1
+    out = np.zeros((n, c, ho, wo), np.float32)
+    lib().fnn_or_maxpool2d(x.reshape(-1), x.size, n, c, h, w, kernel, stride, pad, out.reshape(-1), out.size)
+    return out
+
+
+def upsample_nearest2d(x, sh: int, sw: int) -> np.ndarray:
+    x = _f32(x)
+    n, c, h, w = x.shape
+    out = np.zeros((n, c, h * sh, w * sw), np.float32)
+    lib().fnn_or_upsample_nearest2d(x.reshape(-1), n * c, h, w, sh, sw, out.reshape(-1))
+    return out

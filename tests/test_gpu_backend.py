@@ -328,3 +328,116 @@ def test_conv2d_float_weight_plans(be, orc, wdt, kname):
     assert plan.replayed
     want2 = orc.qconv2d_float(x * 0.5, to_oracle(orc, pw), kh, kw, stride, pad, dil, groups, bias=bias, act=flib.ACT_SILU)
     assert_close(be.read_arena(*s_y, np.float32).reshape(want.shape), want2, 2e-5, kname + " replay")
+
+
+def test_data_movement_kernels(be, orc):
+    """concat / slice_f32 / pool_f32 (max) / upsample_nearest2d: bit-identical to the oracle (pure data movement)."""
+    rng = np.random.default_rng(8)
+    n, c, h, w = 2, 6, 8, 10
+    x = rng.standard_normal((n, c, h, w)).astype(np.float32)
+    x2 = rng.standard_normal((n, 3, h, w)).astype(np.float32)
+    a = Arena()
+    s_x, s_x2 = a.take(x.nbytes), a.take(x2.nbytes)
+    s_cat = a.take((x.size + x2.size) * 4)
+    s_lo, s_hi = a.take(n * 2 * h * w * 4), a.take(n * 4 * h * w * 4)
+    s_pool = a.take(x.nbytes)
+    s_pool2 = a.take(n * c * (h // 2) * (w // 2) * 4)
+    s_up = a.take(x.size * 4 * 4)
+    s_flat = a.take((x.size + x2.size) * 4)
+    plan = ExecutablePlan(a.top).write_const(s_x[0], x).write_const(s_x2[0], x2)
+    plan.call_kernel("concat", [s_x, s_x2], s_cat, [1, h * w, n])                 # channel axis: outer = N
+    plan.call_kernel("slice_f32", [s_x], s_lo, [1, 0, 2, h * w])                  # channels [0,2)
+    plan.call_kernel("slice_f32", [s_x], s_hi, [1, 2, 6, h * w])                  # channels [2,6)
+    plan.call_kernel("pool_f32", [s_x], s_pool, [5, 1, 2, 1, n, c, h, w])         # the SPPF pooling
+    plan.call_kernel("pool_f32", [s_x], s_pool2, [2, 2, 0, 1, n, c, h, w])
+    plan.call_kernel("upsample_nearest2d", [s_x], s_up, [2, 2, h, w])
+    plan.call_kernel("concat", [s_x, s_x2], s_flat, [])                           # legacy form: one after the other
+    be.allocate_arena(a.top)
+    for it in range(2):                                                           # second pass: graph replay
+        be.dispatch(plan)
+        assert plan.replayed == (it == 1)
+        rd = lambda s: be.read_arena(*s, np.float32)
+        assert np.array_equal(rd(s_cat), np.concatenate([x, x2], axis=1).reshape(-1))
+        assert np.array_equal(rd(s_cat), orc.concat([x, x2], n, x.size + x2.size))
+        assert np.array_equal(rd(s_lo), x[:, 0:2].reshape(-1))
+        assert np.array_equal(rd(s_hi), orc.slice_f32(x, 2, 6, h * w, n * 4 * h * w))
+        assert np.array_equal(rd(s_pool), orc.maxpool2d(x, 5, 1, 2).reshape(-1))
+        assert np.array_equal(rd(s_pool2), orc.maxpool2d(x, 2, 2, 0).reshape(-1))
+        assert np.array_equal(rd(s_up), orc.upsample_nearest2d(x, 2, 2).reshape(-1))
+        assert np.array_equal(rd(s_flat), np.concatenate([x.reshape(-1), x2.reshape(-1)]))
+    # in-place pooling (input slot reused as output): the input is staged first, as the CPU arm does
+    p2 = ExecutablePlan(a.top).write_const(s_x[0], x).call_kernel("pool_f32", [s_x], s_x, [3, 1, 1, 1, n, c, h, w])
+    be.dispatch(p2)
+    assert np.array_equal(be.read_arena(*s_x, np.float32), orc.maxpool2d(x, 3, 1, 1).reshape(-1))
+    with pytest.raises(flib.FnnError) as e:
+        be.dispatch(ExecutablePlan(a.top).call_kernel("pool_f32", [s_x], s_pool, [2, 2, 0, 0, n, c, h, w]))
+    assert e.value.kind == "UnsupportedOp"
+    with pytest.raises(flib.FnnError) as e:
+        be.dispatch(ExecutablePlan(a.top).call_kernel("slice_f32", [s_x], s_lo, [1, 0, 2]))
+    assert "expected params [dim, start, end, stride]" in e.value.message
+
+
+def test_c2f_sppf_neck_fragment_as_one_plan(be, orc):
+    """A YOLO-style fragment through the plan dispatcher: C2f (1x1 conv, channel split, two 3x3 convs with a
+    residual add, concat, 1x1 conv), an SPPF pooling pyramid and an upsample + concat, I8 convolutions with
+    bias + SiLU; compared with the same chain of oracle calls."""
+    rng = np.random.default_rng(21)
+    n, c, h, w = 1, 16, 12, 12
+    hw = h * w
+    x = rng.uniform(0, 1, (n, c, h, w)).astype(np.float32)
+    def conv_w(oc, ic, k):
+        kk = ic * k * k
+        pw = fastnn_amd.quantize_weights(flib.DT_I8, (rng.standard_normal((oc, kk)) * np.sqrt(2.0 / kk)).astype(np.float32))
+        return pw, (rng.standard_normal(oc) * 0.05).astype(np.float32)
+    cv1, m1, m2, cv2 = conv_w(16, 16, 1), conv_w(8, 8, 3), conv_w(8, 8, 3), conv_w(16, 24, 1)
+    a = Arena()
+    f4 = lambda ch, hh=h, ww=w: a.take(n * ch * hh * ww * 4)
+    s_x, s_y, s_a, s_b, s_t, s_u, s_r, s_cat, s_out = f4(16), f4(16), f4(8), f4(8), f4(8), f4(8), f4(8), f4(24), f4(16)
+    s_p1, s_p2, s_p3, s_sp = f4(16), f4(16), f4(16), f4(64)
+    s_up, s_neck = f4(64, 2 * h, 2 * w), f4(64 + 16, 2 * h, 2 * w)
+    skip = rng.uniform(0, 1, (n, 16, 2 * h, 2 * w)).astype(np.float32)
+    s_skip = f4(16, 2 * h, 2 * w)
+    plan = ExecutablePlan(0)
+    slots = {}
+    for name, (pw, bias) in dict(cv1=cv1, m1=m1, m2=m2, cv2=cv2).items():
+        slots[name] = (a.take(pw.words.nbytes), a.take(bias.nbytes))
+    plan = ExecutablePlan(a.top).write_const(s_skip[0], skip)
+    for name, (pw, bias) in dict(cv1=cv1, m1=m1, m2=m2, cv2=cv2).items():
+        plan.write_const(slots[name][0][0], pw.words).write_const(slots[name][1][0], bias)
+    def conv(name, pw, src, dst, ic, k):
+        plan.call_kernel("conv2d_i8_silu", [src, slots[name][0], slots[name][1]], dst, [1, k // 2, 1, 1, ic, h, w, k, k],
+                         meta_of(pw, [pw.rows, ic, k, k]))
+    conv("cv1", cv1[0], s_x, s_y, 16, 1)
+    plan.call_kernel("slice_f32", [s_y], s_a, [1, 0, 8, hw]).call_kernel("slice_f32", [s_y], s_b, [1, 8, 16, hw])
+    conv("m1", m1[0], s_b, s_t, 8, 3)
+    conv("m2", m2[0], s_t, s_u, 8, 3)
+    plan.call_kernel("add_f32", [s_b, s_u], s_r, [n * 8 * hw])
+    plan.call_kernel("concat", [s_a, s_b, s_r], s_cat, [1, hw, n])
+    conv("cv2", cv2[0], s_cat, s_out, 24, 1)
+    plan.call_kernel("pool_f32", [s_out], s_p1, [5, 1, 2, 1, n, 16, h, w])
+    plan.call_kernel("pool_f32", [s_p1], s_p2, [5, 1, 2, 1, n, 16, h, w])
+    plan.call_kernel("pool_f32", [s_p2], s_p3, [5, 1, 2, 1, n, 16, h, w])
+    plan.call_kernel("concat", [s_out, s_p1, s_p2, s_p3], s_sp, [1, hw, n])
+    plan.call_kernel("upsample_nearest2d", [s_sp], s_up, [2, 2, h, w])
+    plan.call_kernel("concat", [s_up, s_skip], s_neck, [1, 4 * hw, n])
+    be.allocate_arena(a.top)
+
+    def reference(xin):
+        q = lambda pwb, t, k: orc.qconv2d_i8(t, to_oracle(orc, pwb[0]), k, k, 1, k // 2, 1, 1, bias=pwb[1], act=flib.ACT_SILU)
+        y = q(cv1, xin, 1)
+        ya, yb = y[:, :8], y[:, 8:]
+        r = yb + q(m2, q(m1, yb, 3), 3)
+        out = q(cv2, np.concatenate([ya, yb, r], axis=1), 1)
+        p1 = orc.maxpool2d(out, 5, 1, 2); p2 = orc.maxpool2d(p1, 5, 1, 2); p3 = orc.maxpool2d(p2, 5, 1, 2)
+        sp = np.concatenate([out, p1, p2, p3], axis=1)
+        return np.concatenate([orc.upsample_nearest2d(sp, 2, 2), skip], axis=1)
+
+    for it in range(3):
+        xin = x if it == 0 else rng.uniform(0, 1, x.shape).astype(np.float32)
+        be.write_arena(s_x[0], xin)
+        be.dispatch(plan)
+        assert plan.replayed == (it >= 1)
+        got = be.read_arena(*s_neck, np.float32).reshape(n, 80, 2 * h, 2 * w)
+        # each conv re-quantises its input from the previous result: differences of one rounding step can
+        # propagate, so the chain is compared at 2e-3 of the output range (single convs: 1e-5)
+        assert_close(got, reference(xin), 2e-3, f"fragment, dispatch {it}")

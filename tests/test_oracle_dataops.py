@@ -1,0 +1,64 @@
+"""Pins the oracle's restatement of the f32 data-movement kernels that sit between quantised
+convolutions (concat, slice_f32, pool_f32 max, upsample_nearest2d) against numpy / torch."""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+
+@pytest.mark.parametrize("axis", [0, 1, 2, 3])
+def test_concat_is_numpy_concatenate(orc, axis):
+    rng = np.random.default_rng(1)
+    shapes = [[2, 3, 4, 5], [2, 3, 4, 5], [2, 3, 4, 5]]
+    shapes[1][axis] += 2
+    shapes[2][axis] = 1
+    xs = [rng.standard_normal(s).astype(np.float32) for s in shapes]
+    want = np.concatenate(xs, axis=axis)
+    outer = int(np.prod(shapes[0][:axis]))          # params[2] = product of the dims before the axis
+    got = orc.concat(xs, outer, want.size)
+    assert np.array_equal(got, want.reshape(-1))
+
+
+def test_concat_clamps_to_the_output(orc):
+    a, b = np.arange(6, dtype=np.float32), np.arange(10, 14, dtype=np.float32)
+    got = orc.concat([a, b], 1, 8)                  # room for 8 of the 10 values
+    assert np.array_equal(got, np.concatenate([a, b])[:8])
+
+
+@pytest.mark.parametrize("dim,start,end", [(1, 0, 4), (1, 4, 8), (2, 1, 3), (3, 2, 5), (0, 1, 2)])
+def test_slice_is_numpy_slicing(orc, dim, start, end):
+    rng = np.random.default_rng(2)
+    x = rng.standard_normal((2, 8, 4, 6)).astype(np.float32)
+    idx = [slice(None)] * 4
+    idx[dim] = slice(start, end)
+    want = x[tuple(idx)]
+    stride = int(np.prod(x.shape[dim + 1:]))        # elements per index of the sliced dimension
+    got = orc.slice_f32(x, start, end, stride, want.size)
+    assert np.array_equal(got, want.reshape(-1))
+
+
+@pytest.mark.parametrize("k,s,p", [(5, 1, 2), (2, 2, 0), (3, 2, 1), (3, 1, 0)])
+def test_maxpool_is_torch_max_pool2d(orc, k, s, p):
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((2, 3, 11, 9)).astype(np.float32)
+    want = F.max_pool2d(torch.from_numpy(x), k, s, p).numpy()
+    got = orc.maxpool2d(x, k, s, p)
+    assert got.shape == want.shape and np.array_equal(got, want)
+
+
+def test_maxpool_window_in_the_padding_only_is_minus_inf(orc):
+    x = np.ones((1, 1, 2, 2), np.float32)
+    got = orc.maxpool2d(x, 1, 1, 1)                 # 4x4 output, the border windows see padding only
+    assert got.shape == (1, 1, 4, 4)
+    assert np.all(np.isneginf(got[0, 0, 0])) and got[0, 0, 1, 1] == 1.0
+
+
+@pytest.mark.parametrize("sh,sw", [(2, 2), (1, 3), (3, 1)])
+def test_upsample_is_numpy_repeat(orc, sh, sw):
+    rng = np.random.default_rng(4)
+    x = rng.standard_normal((2, 3, 5, 4)).astype(np.float32)
+    want = np.repeat(np.repeat(x, sh, axis=2), sw, axis=3)
+    assert np.array_equal(orc.upsample_nearest2d(x, sh, sw), want)
+    if sh == sw:
+        t = F.interpolate(torch.from_numpy(x), scale_factor=sh, mode="nearest").numpy()
+        assert np.array_equal(want, t)
