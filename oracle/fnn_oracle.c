@@ -22,8 +22,12 @@
  *   f32 MatMul ............. closed-form literals microkernels/tests.rs:369-763,
  *                            seeded end-to-end bounds tests/cpu_reference_oracle.rs
  *   I8-activation MatMul ... exact integers; literals microkernels/tests.rs:369-678
- *   conv lowering .......... equals float conv of dequantised operands; integer
- *                            accumulators exact; brute-force direct convolution
+ *   conv lowering .......... (I8 and I4 weights) equals float conv of dequantised operands; integer
+ *                            accumulators exact; brute-force direct convolution; activation
+ *                            quantiser re-derived in f32; flat-input special cases
+ *   conv, other types ...... torch.nn.functional.conv2d in f64 on the dequantised weights
+ *   concat / slice / max pool / nearest upsample ... numpy concatenate, slicing, repeat and
+ *                            torch max_pool2d / interpolate (bit-identical data movement)
  *   What only an execution of the Rust crate could pin tighter: the last-bit
  *   value of its AVX/Rayon f32 summation order (tolerance-only by design).
  */
