@@ -21,3 +21,7 @@ int fnn_mfma_qgemv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, con
 int fnn_i8_tiled_matmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const I8ActArgs &p, bool *handled);
 // p.actq must already hold the (image, group) activation scales.
 int fnn_i8_tiled_conv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QConvArgs &p, bool *handled);
+
+// Weight rows as 16-byte addressable pieces: the registered words, or (when kp % 4 != 0) a copy with the
+// rows re-strided to a multiple of four words, zero-filled, made on first use and kept with the weight.
+int fnn_aligned_rows(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const uint32_t **words, int64_t *kp);

@@ -259,13 +259,15 @@ __global__ void __launch_bounds__(256) restride_rows_kernel(const uint32_t *src,
     }
 }
 
+}  // namespace
+
 // weight rows as 16-byte addressable pieces: the registered words, or a re-strided copy when kp % 4 != 0
-int aligned_rows(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const uint32_t **words, int64_t *kp)
+int fnn_aligned_rows(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const uint32_t **words, int64_t *kp)
 {
     if (w->kp % 4 == 0) { *words = w->words; *kp = w->kp; return FNN_OK; }
     fnn_hip_weight *wm = const_cast<fnn_hip_weight *>(w);
     if (!wm->words4) {
-        if (fnn_ctx_capturing(ctx)) return fnn_ctx_fail(ctx, FNN_ERR_MEMORY, "first integer use of a weight during graph capture");
+        if (fnn_ctx_capturing(ctx)) return fnn_ctx_fail(ctx, FNN_ERR_MEMORY, "first use of re-strided weight rows during graph capture");
         const int64_t kp4 = (w->kp + 3) / 4 * 4;
         if (hipMalloc((void **)&wm->words4, (size_t)(w->rows * kp4 + 16) * 4) != hipSuccess)
             return fnn_ctx_fail(ctx, FNN_ERR_MEMORY, "out of device memory (re-strided weight rows)");
@@ -278,6 +280,8 @@ int aligned_rows(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const
     *words = wm->words4; *kp = wm->kp4;
     return FNN_OK;
 }
+
+namespace {
 
 // C[m][n] = sum_k A8[m][k] * q_w[n0 + n][k] for `n` weight rows starting at row n0 (rows of kp words, 16-byte aligned)
 template <int DT>
@@ -317,7 +321,7 @@ int fnn_i8_tiled_matmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w
     if ((rc = fnn_ctx_ensure_tmp(ctx, 1, (size_t)p.m * p.n * 4 + 256, &ws1))) return rc;
     fnn_hip_weight *wm = const_cast<fnn_hip_weight *>(w);
     if (!wm->row_qsum) {
-        if (fnn_ctx_capturing(ctx)) return fnn_ctx_fail(ctx, FNN_ERR_MEMORY, "first integer use of a weight during graph capture");
+        if (fnn_ctx_capturing(ctx)) return fnn_ctx_fail(ctx, FNN_ERR_MEMORY, "first use of re-strided weight rows during graph capture");
         if (hipMalloc((void **)&wm->row_qsum, (size_t)w->rows * 4 + 64) != hipSuccess)
             return fnn_ctx_fail(ctx, FNN_ERR_MEMORY, "out of device memory (row sums)");
         hipError_t e = launch_row_qsum(w, wm->row_qsum, s);
@@ -325,7 +329,7 @@ int fnn_i8_tiled_matmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w
     }
     const uint32_t *words;
     int64_t kp;
-    if ((rc = aligned_rows(ctx, s, w, &words, &kp))) return rc;
+    if ((rc = fnn_aligned_rows(ctx, s, w, &words, &kp))) return rc;
     int8_t *a8 = (int8_t *)ws0;
     int32_t *qsum = (int32_t *)((char *)ws0 + q_off);
     int32_t *c = (int32_t *)ws1;
@@ -368,7 +372,7 @@ int fnn_i8_tiled_conv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, 
     if ((rc = fnn_ctx_ensure_tmp(ctx, 1, (size_t)rows * ocg * 4 + 256, &ws1))) return rc;
     const uint32_t *words;
     int64_t kp;
-    if ((rc = aligned_rows(ctx, s, w, &words, &kp))) return rc;
+    if ((rc = fnn_aligned_rows(ctx, s, w, &words, &kp))) return rc;
     int8_t *a8 = (int8_t *)ws3;
     int32_t *qsum = (int32_t *)((char *)ws3 + q_off);
     int32_t *c = (int32_t *)ws1;

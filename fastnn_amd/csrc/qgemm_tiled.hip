@@ -344,7 +344,7 @@ int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QM
 
     TileArgs t;
     t.words = q.words;
-    t.zero_chunk = q.words + w->rows * w->kp;   // the zeroed margin behind the last row
+    t.zero_chunk = q.words + w->rows * q.kp;    // the zeroed margin behind the last row
     t.scales = q.scales; t.zeros = q.zeros; t.umean = want_umean ? wm->umean : nullptr; t.bias = q.bias;
     t.ap = pa.ap; t.rexp = pa.rexp; t.xsum = pa.xsum; t.esum = pa.esum;
     t.out = q.out; t.part = (float *)ws1;
@@ -465,18 +465,22 @@ int fnn_tiled_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, 
         *handled = true;
         return FNN_OK;
     }
-    if (q.kp % 4 != 0) return FNN_OK;                           // 16-byte pieces of a weight row
-    if (reinterpret_cast<uintptr_t>(q.words) & 15) return FNN_OK;
+    if (w->dtype < FNN_DT_I8 || w->dtype > FNN_DT_F4) return FNN_OK;
     if (q.m > (1 << 22) || q.n > (1 << 24)) return FNN_OK;      // 32-bit tile counts
+    // the kernel fetches 16-byte pieces of a weight row: rows whose length is not a multiple of four words
+    // are read from a re-strided copy (made once per weight)
+    QMatmulArgs qa = q;
     int rc;
+    if (q.words == w->words && (rc = fnn_aligned_rows(ctx, s, w, &qa.words, &qa.kp))) return rc;
+    if (qa.kp % 4 != 0 || (reinterpret_cast<uintptr_t>(qa.words) & 15)) return FNN_OK;
     switch (w->dtype) {
-    case FNN_DT_I8: rc = run_tiled<FNN_DT_I8>(ctx, s, w, q, flags); break;
-    case FNN_DT_I4: rc = run_tiled<FNN_DT_I4>(ctx, s, w, q, flags); break;
-    case FNN_DT_U8: rc = run_tiled<FNN_DT_U8>(ctx, s, w, q, flags); break;
-    case FNN_DT_U4: rc = run_tiled<FNN_DT_U4>(ctx, s, w, q, flags); break;
-    case FNN_DT_F8: rc = run_tiled<FNN_DT_F8>(ctx, s, w, q, flags); break;
-    case FNN_DT_F8R: rc = run_tiled<FNN_DT_F8R>(ctx, s, w, q, flags); break;
-    case FNN_DT_F4: rc = run_tiled<FNN_DT_F4>(ctx, s, w, q, flags); break;
+    case FNN_DT_I8: rc = run_tiled<FNN_DT_I8>(ctx, s, w, qa, flags); break;
+    case FNN_DT_I4: rc = run_tiled<FNN_DT_I4>(ctx, s, w, qa, flags); break;
+    case FNN_DT_U8: rc = run_tiled<FNN_DT_U8>(ctx, s, w, qa, flags); break;
+    case FNN_DT_U4: rc = run_tiled<FNN_DT_U4>(ctx, s, w, qa, flags); break;
+    case FNN_DT_F8: rc = run_tiled<FNN_DT_F8>(ctx, s, w, qa, flags); break;
+    case FNN_DT_F8R: rc = run_tiled<FNN_DT_F8R>(ctx, s, w, qa, flags); break;
+    case FNN_DT_F4: rc = run_tiled<FNN_DT_F4>(ctx, s, w, qa, flags); break;
     default: return FNN_OK;
     }
     if (rc) return rc;
