@@ -134,6 +134,10 @@ class HipBackend:
         self._check(self.lib.fnn_backend_read_arena(self.handle, offset, out.ctypes.data_as(C.c_void_p), size))
         return out.view(dtype)
 
+    def set_kernel_flags(self, flags: int):
+        """Extra FNN_FLAG_* bits for every MatMul / Conv2d call (e.g. lib.FLAG_ACT_F16_SINGLE)."""
+        self._check(self.lib.fnn_backend_set_kernel_flags(self.handle, flags))
+
     def dispatch(self, plan: ExecutablePlan):
         self._check(self.lib.fnn_backend_dispatch(self.handle, plan.handle))
 

@@ -587,7 +587,7 @@ int fnn_hip_qconv2d(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *x, i
         for (int g = 0; g < groups; g++) {
             HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_im2col_f32(dx, col, b, c, groups, g, h, wd, ho, wo, kh, kw, stride, pad, dil, ctx->stream));
             if (groups == 1) {
-                if ((rc = fnn_hip_qmatmul(ctx, w, col, rows, dbias, act, rows_out, FNN_FLAG_DEVICE_PTRS | (flags & FNN_FLAG_FORCE_GENERIC)))) return rc;
+                if ((rc = fnn_hip_qmatmul(ctx, w, col, rows, dbias, act, rows_out, FNN_FLAG_DEVICE_PTRS | (flags & (FNN_FLAG_FORCE_GENERIC | FNN_FLAG_ACT_F16_SINGLE))))) return rc;
             } else {
                 // a slice of the weight rows: the shape-agnostic kernel takes the offset pointers as they are
                 QMatmulArgs q;

@@ -114,6 +114,7 @@ struct fnn_backend {
     uint64_t write_seq = 0;
     std::vector<std::pair<uint64_t, fnn_slice>> host_writes;
     uint64_t weights_epoch = 0;  // bumped whenever a cached device weight is created or released
+    int kernel_flags = 0;        // extra FNN_FLAG_* bits for every MatMul / Conv2d call
     std::string err;
     std::map<std::pair<uint64_t, uint64_t>, fnn_hip_weight *> weights;  // (offset,size) like get_or_cache_packed
     std::vector<uint8_t> stage;
@@ -229,7 +230,7 @@ int run_matmul(fnn_backend *b, const Instr &in, const KernelName &kn, int dtype)
     if (st) return st;
     if (m == 0 || n == 0) return FNN_OK;
     return lift(b, fnn_hip_qmatmul(b->ctx, w, (const float *)(b->arena + as.offset), (int64_t)m, bias, kn.act,
-                                   (float *)(b->arena + in.dst.offset), FNN_FLAG_DEVICE_PTRS));
+                                   (float *)(b->arena + in.dst.offset), FNN_FLAG_DEVICE_PTRS | b->kernel_flags));
 }
 
 int run_matmul_i8act(fnn_backend *b, const Instr &in, int dtype)
@@ -312,7 +313,7 @@ int run_conv2d_i8(fnn_backend *b, const Instr &in, const KernelName &kn)
     if (batch == 0) return FNN_OK;
     return lift(b, fnn_hip_qconv2d(b->ctx, w, (const float *)(b->arena + in.inputs[0].offset), (int64_t)batch, (int64_t)c,
                                    (int64_t)h, (int64_t)wd, (int)kh, (int)kw, (int)stride, (int)pad, (int)dil, (int)groups,
-                                   bias, kn.act, (float *)(b->arena + in.dst.offset), nullptr, FNN_FLAG_DEVICE_PTRS));
+                                   bias, kn.act, (float *)(b->arena + in.dst.offset), nullptr, FNN_FLAG_DEVICE_PTRS | b->kernel_flags));
 }
 
 int run_elementwise(fnn_backend *b, const Instr &in, int op)
@@ -620,6 +621,16 @@ void fnn_backend_destroy(fnn_backend *b)
 }
 
 const char *fnn_backend_name(const fnn_backend *) { return "hip"; }
+
+int fnn_backend_set_kernel_flags(fnn_backend *b, int flags)
+{
+    if (!b) return FNN_ERR_DISPATCH;
+    if (flags & ~(FNN_FLAG_ACT_F16_SINGLE | FNN_FLAG_FORCE_GENERIC | FNN_FLAG_PREFER_FMA))
+        return fail(b, FNN_ERR_DISPATCH, "set_kernel_flags: only ACT_F16_SINGLE, FORCE_GENERIC and PREFER_FMA can be set per backend");
+    if (flags != b->kernel_flags) b->weights_epoch++;   // captured graphs hold the old kernel choice
+    b->kernel_flags = flags;
+    return FNN_OK;
+}
 
 const char *fnn_backend_last_error(const fnn_backend *b) { return b ? b->err.c_str() : "no backend"; }
 

@@ -39,6 +39,7 @@ EXPORTED_SYMBOLS = [
 # every symbol include/fastnn_hip_backend.h declares
 BACKEND_SYMBOLS = [
     "fnn_backend_create", "fnn_backend_destroy", "fnn_backend_name", "fnn_backend_last_error",
+    "fnn_backend_set_kernel_flags",
     "fnn_backend_allocate_arena", "fnn_backend_write_arena", "fnn_backend_read_arena",
     "fnn_plan_create", "fnn_plan_destroy", "fnn_plan_add_write_const", "fnn_plan_add_fill",
     "fnn_plan_add_memcopy", "fnn_plan_add_call_kernel", "fnn_plan_len", "fnn_plan_replayed",
@@ -138,6 +139,7 @@ def _prototype(l):
     l.fnn_backend_destroy.restype = None
     l.fnn_backend_name.argtypes = [_vp]
     l.fnn_backend_name.restype = C.c_char_p
+    l.fnn_backend_set_kernel_flags.argtypes = [_vp, C.c_int]
     l.fnn_backend_last_error.argtypes = [_vp]
     l.fnn_backend_last_error.restype = C.c_char_p
     l.fnn_backend_allocate_arena.argtypes = [_vp, _u64]

@@ -44,6 +44,11 @@ typedef struct {
 int fnn_backend_create(int device, fnn_backend **out);
 void fnn_backend_destroy(fnn_backend *b);
 const char *fnn_backend_name(const fnn_backend *b);
+/* FNN_FLAG_* bits OR-ed into every quantised MatMul / Conv2d call the backend makes from now on (no
+ * counterpart in fastnn): FNN_FLAG_ACT_F16_SINGLE trades the default 2e-5 agreement for 1e-3 and about a third
+ * less time at M >= 64; FNN_FLAG_FORCE_GENERIC / FNN_FLAG_PREFER_FMA select kernels for testing.  Other bits
+ * are refused.  Plans captured before the change are captured again. */
+int fnn_backend_set_kernel_flags(fnn_backend *b, int flags);
 const char *fnn_backend_last_error(const fnn_backend *b);
 int fnn_backend_allocate_arena(fnn_backend *b, uint64_t total_bytes);
 int fnn_backend_write_arena(fnn_backend *b, uint64_t offset, const void *data, uint64_t size);

@@ -441,3 +441,40 @@ def test_c2f_sppf_neck_fragment_as_one_plan(be, orc):
         # each conv re-quantises its input from the previous result: differences of one rounding step can
         # propagate, so the chain is compared at 2e-3 of the output range (single convs: 1e-5)
         assert_close(got, reference(xin), 2e-3, f"fragment, dispatch {it}")
+
+
+def test_backend_kernel_flags_single_f16_activations(be, orc):
+    """FNN_FLAG_ACT_F16_SINGLE per backend: the MLP block at 64 tokens agrees to 1e-3 (default: 2e-5), a plan
+    captured under the old flags is captured again, and unknown bits are refused."""
+    rng = np.random.default_rng(64)
+    m, d, f = 64, 256, 1024
+    x = rng.standard_normal((m, d)).astype(np.float32)
+    up = fastnn_amd.quantize_weights(flib.DT_I4, _w(rng, f, d))
+    down = fastnn_amd.quantize_weights(flib.DT_I8, _w(rng, d, f))
+    a = Arena()
+    s_x, s_up, s_down, s_h, s_y = a.take(x.nbytes), a.take(up.words.nbytes), a.take(down.words.nbytes), a.take(m * f * 4), a.take(m * d * 4)
+    plan = ExecutablePlan(a.top).write_const(s_up[0], up.words).write_const(s_down[0], down.words)
+    plan.call_kernel("matmul_i4_relu", [s_x, s_up], s_h, [m, d, f], meta_of(up))
+    plan.call_kernel("matmul_i8", [s_h, s_down], s_y, [m, f, d], meta_of(down))
+    be.allocate_arena(a.top)
+    be.write_arena(s_x[0], x)
+    h_ref = orc.qmatmul(to_oracle(orc, up), x, act=flib.ACT_RELU)
+    want = orc.qmatmul(to_oracle(orc, down), h_ref)
+    try:
+        be.dispatch(plan); be.dispatch(plan)
+        assert plan.replayed
+        precise = be.read_arena(*s_y, np.float32).reshape(m, d).copy()
+        assert_close(precise, want, 1e-4, "default flags")
+        be.set_kernel_flags(flib.FLAG_ACT_F16_SINGLE)
+        be.dispatch(plan)
+        assert not plan.replayed                      # the old capture is stale
+        fast = be.read_arena(*s_y, np.float32).reshape(m, d).copy()
+        assert_close(fast, want, 1e-3, "single f16 activations")
+        assert not np.array_equal(fast, precise)      # it really is the other kernel variant
+        be.dispatch(plan)
+        assert plan.replayed
+        assert np.array_equal(be.read_arena(*s_y, np.float32).reshape(m, d), fast)
+        with pytest.raises(flib.FnnError):
+            be.set_kernel_flags(flib.FLAG_DEVICE_PTRS)
+    finally:
+        be.set_kernel_flags(0)
