@@ -88,25 +88,36 @@ __global__ void __launch_bounds__(256) conv_minmax_cover_kernel(QConvArgs a, int
     const int64_t nn = bg / a.groups, g = bg % a.groups;
     const int64_t cg = a.c / a.groups;
     const float *xg = a.x + (nn * a.c + g * cg) * a.h * a.w;
-    const int64_t hw = a.h * a.w, total = cg * hw;
     float mn = pad_touched ? 0.0f : INFINITY, mx = pad_touched ? 0.0f : -INFINITY;
-    if (total < (1ll << 31)) {   // 32-bit index arithmetic
-        const unsigned hw32 = (unsigned)hw, w32 = (unsigned)a.w, tot32 = (unsigned)total, stride = gridDim.x * blockDim.x;
-        for (unsigned idx = blockIdx.x * blockDim.x + threadIdx.x; idx < tot32; idx += stride) {
-            const unsigned rem = idx % hw32;
-            const unsigned ih = rem / w32, iw = rem - ih * w32;
-            if (cov_h[ih] && cov_w[iw]) {
-                const float v = xg[idx];
-                mn = fminf(mn, v);
-                mx = fmaxf(mx, v);
-            }
-        }
-    } else {
-        for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * blockDim.x) {
-            const int64_t rem = idx % hw;
-            const int64_t ih = rem / a.w, iw = rem % a.w;
-            if (cov_h[ih] && cov_w[iw]) {
-                const float v = xg[idx];
+    // A wave takes a chunk of whole image rows (channel, ih) at a time, consecutive lanes on consecutive
+    // elements (16 bytes per lane when the row length allows): rows and columns no tap reaches are skipped by
+    // two table lookups, and the index arithmetic is per 16 bytes, not per element.
+    const int64_t nrows = cg * a.h;
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6), nwaves = (int64_t)gridDim.x * 4;
+    const bool vec4 = (a.w % 4 == 0) && ((reinterpret_cast<uintptr_t>(xg) & 15) == 0);
+    const int per_lane = vec4 ? 4 : 1;
+    const int64_t span = 64 * per_lane;                              // elements a wave covers per step
+    const int64_t rows_per_chunk = a.w >= span ? 1 : span / a.w;     // whole rows per chunk
+    const int64_t steps = a.w >= span ? (a.w + span - 1) / span : 1; // steps per chunk (long rows)
+    const int64_t chunks = (nrows + rows_per_chunk - 1) / rows_per_chunk;
+    for (int64_t ch = wave; ch < chunks; ch += nwaves) {
+        const int64_t row0 = ch * rows_per_chunk;
+        for (int64_t st = 0; st < steps; st++) {
+            const int64_t e = st * span + (int64_t)lane * per_lane;   // element inside the chunk
+            const int64_t sub = e / a.w, iw = e - sub * a.w;
+            const int64_t row = row0 + sub;
+            if (sub >= rows_per_chunk || row >= nrows || iw >= a.w) continue;
+            if (!cov_h[row % a.h]) continue;
+            const float *src = xg + row * a.w + iw;
+            if (vec4) {
+                const float4 v = *reinterpret_cast<const float4 *>(src);
+                if (cov_w[iw + 0]) { mn = fminf(mn, v.x); mx = fmaxf(mx, v.x); }
+                if (cov_w[iw + 1]) { mn = fminf(mn, v.y); mx = fmaxf(mx, v.y); }
+                if (cov_w[iw + 2]) { mn = fminf(mn, v.z); mx = fmaxf(mx, v.z); }
+                if (cov_w[iw + 3]) { mn = fminf(mn, v.w); mx = fmaxf(mx, v.w); }
+            } else if (cov_w[iw]) {
+                const float v = *src;
                 mn = fminf(mn, v);
                 mx = fmaxf(mx, v);
             }
@@ -284,6 +295,8 @@ hipError_t launch_qconv2d_i8(const QConvArgs &p, hipStream_t s, int phase)
                 }
             const int64_t elems = cg * p.h * p.w;
             nparts = (elems + 256 * 4 - 1) / (256 * 4);
+            const int64_t cap = 4096 / bg > 32 ? 4096 / bg : 32;   // about 4096 workgroups over all images
+            if (nparts > cap) nparts = cap;
             if (nparts > QCONV_NPART) nparts = QCONV_NPART;
             if (nparts < 1) nparts = 1;
             hipLaunchKernelGGL(conv_minmax_cover_kernel, dim3((unsigned)nparts, (unsigned)bg), dim3(256), (size_t)(p.h + p.w), s, p, pad_touched);
