@@ -5,3 +5,4 @@ from .lib import (  # noqa: F401
     FLAG_ACT_F16_SINGLE, FLAG_DEVICE_PTRS, FLAG_FORCE_GENERIC, FLAG_I4CB_AS_WRITTEN, FLAG_PREFER_FMA,
     FnnError, HipContext, PackedWeight, load_library, quantize_weights, quantize_weights_kn,
 )
+from .aot import AotExecutor, weight_dtype_of  # noqa: F401,E402

@@ -1,0 +1,137 @@
+"""The host-side mirror of fastnn.AotExecutor(nodes, params, input_names, output_names, input_shapes, quantize):
+argument handling and lowering need no GPU; forward() is checked against the oracle on the GPU."""
+import numpy as np
+import pytest
+
+import fastnn_amd
+from fastnn_amd import lib as flib
+from fastnn_amd.aot import AotExecutor, weight_dtype_of
+
+
+def mlp_nodes():
+    """x -> MatMul(w1) -> Add(b1) -> Gelu -> MatMul(w2) -> Add(x) (residual), all values strings as the
+    reference's Python side passes them (fastnn/io/graph_builder.py)."""
+    return [
+        {"name": "fc1", "op_type": "MatMul", "inputs": "[x, w1]", "outputs": "[h0]"},
+        {"name": "b1", "op_type": "Add", "inputs": "[h0, b1]", "outputs": "[h1]"},
+        {"name": "act", "op_type": "Gelu", "inputs": "[h1]", "outputs": "[h2]"},
+        {"name": "fc2", "op_type": "MatMul", "inputs": "[h2, w2]", "outputs": "[y0]"},
+        {"name": "res", "op_type": "Add", "inputs": "[y0, x]", "outputs": "[y]"},
+    ]
+
+
+def mlp_params(rng, d=64, f=160):
+    return {"w1": (rng.standard_normal((d, f)) * 0.1).astype(np.float32), "b1": (rng.standard_normal(f) * 0.1).astype(np.float32),
+            "w2": (rng.standard_normal((f, d)) * 0.1).astype(np.float32)}
+
+
+def test_quantize_argument_mapping_and_errors():
+    """src/python/nn.rs:1320-1358."""
+    assert weight_dtype_of(None) is None and weight_dtype_of("f32") is None
+    assert weight_dtype_of(4) == flib.DT_I4 and weight_dtype_of(8) == flib.DT_I8
+    for s, dt in dict(i4=flib.DT_I4, i8=flib.DT_I8, u4=flib.DT_U4, u8=flib.DT_U8, f8=flib.DT_F8, f8r=flib.DT_F8R,
+                      f4=flib.DT_F4, i4cb=flib.DT_I4CB).items():
+        assert weight_dtype_of(s) == dt
+    with pytest.raises(ValueError, match=r"unsupported quantize value for integer: 5 \(expected 4 or 8\)"):
+        weight_dtype_of(5)
+    with pytest.raises(ValueError, match="unsupported quantize string: 'int8'"):
+        weight_dtype_of("int8")
+    with pytest.raises(TypeError, match="quantize must be int"):
+        weight_dtype_of(4.0)
+
+
+def test_lowering_needs_no_gpu_and_fuses_bias_and_activation():
+    rng = np.random.default_rng(0)
+    ex = AotExecutor(mlp_nodes(), mlp_params(rng), ["x"], ["y"], {"x": [3, 64]}, quantize="f8")
+    assert [i[0] for i in ex.instructions] == ["matmul_f8_gelu", "matmul_f8", "add_f32"]
+    assert ex.instructions[0][3] == [3, 64, 160] and ex.instructions[1][3] == [3, 160, 64]
+    assert ex.instructions[0][1] == ["x", "w1", "bias"]          # the Add(b1) went into the epilogue
+    assert ex.arena_size % 64 == 0
+    # the hidden value is also a graph output: nothing may be folded away behind it
+    ex2 = AotExecutor(mlp_nodes(), mlp_params(rng), ["x"], ["y", "h0"], {"x": [3, 64]}, quantize=8)
+    assert [i[0] for i in ex2.instructions] == ["matmul_i8", "add_f32", "gelu_f32", "matmul_i8", "add_f32"]
+
+
+def test_lowering_errors():
+    rng = np.random.default_rng(0)
+    p = mlp_params(rng)
+    with pytest.raises(flib.FnnError) as e:
+        AotExecutor(mlp_nodes() + [{"name": "s", "op_type": "Softmax", "inputs": "[y]", "outputs": "[z]"}], p, ["x"], ["z"],
+                    {"x": [3, 64]}, quantize=4)
+    assert e.value.kind == "UnsupportedOp" and e.value.message == "Softmax"
+    with pytest.raises(flib.FnnError) as e:
+        AotExecutor(mlp_nodes(), p, ["x"], ["y"], {"x": [3, 64]}, quantize=None)
+    assert e.value.kind == "UnsupportedOp"
+    with pytest.raises(flib.FnnError):
+        AotExecutor(mlp_nodes(), p, ["x"], ["y"], {"x": [-1, 64]}, quantize=4)     # symbolic batch
+    with pytest.raises(flib.FnnError):
+        AotExecutor(mlp_nodes(), p, ["x"], ["nope"], {"x": [3, 64]}, quantize=4)
+    with pytest.raises(flib.FnnError):
+        AotExecutor(mlp_nodes(), p, ["x"], ["y"], {"x": [3, 65]}, quantize=4)      # K mismatch
+
+
+def test_conv_lowering():
+    rng = np.random.default_rng(1)
+    nodes = [
+        {"name": "c1", "op_type": "Conv", "inputs": "[x, w, b]", "outputs": "[c]", "strides": "2", "pads": "1", "group": "1"},
+        {"name": "a1", "op_type": "Silu", "inputs": "[c]", "outputs": "[s]"},
+        {"name": "p", "op_type": "MaxPool", "inputs": "[s]", "outputs": "[m]", "kernel_shape": "5", "strides": "1", "pads": "2"},
+        {"name": "cat", "op_type": "Concat", "inputs": "[s, m]", "outputs": "[k]", "axis": "1"},
+        {"name": "up", "op_type": "Resize", "inputs": "[k]", "outputs": "[y]", "mode": "nearest", "scale_h": "2", "scale_w": "2"},
+    ]
+    params = {"w": rng.standard_normal((8, 3, 3, 3)).astype(np.float32), "b": np.zeros(8, np.float32)}
+    ex = AotExecutor(nodes, params, ["x"], ["y"], {"x": [1, 3, 16, 16]}, quantize="i8")
+    assert [i[0] for i in ex.instructions] == ["conv2d_i8_silu", "pool_f32", "concat", "upsample_nearest2d"]
+    assert ex.instructions[0][3] == [2, 1, 1, 1, 3, 16, 16, 3, 3]
+    assert ex.instructions[1][3] == [5, 1, 2, 1, 1, 8, 8, 8]
+    assert ex.instructions[2][3] == [1, 64, 1]
+    assert ex.instructions[3][3] == [2, 2, 8, 8]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("quantize", [4, 8, "i4", "i8", "u4", "u8", "f8", "f8r", "f4", "i4cb"])
+def test_forward_matches_oracle(orc, quantize):
+    from gpu_common import assert_close, to_oracle
+    rng = np.random.default_rng(7)
+    params = mlp_params(rng)
+    ex = AotExecutor(mlp_nodes(), params, ["x"], ["y"], {"x": [5, 64]}, quantize=quantize)
+    dt = weight_dtype_of(quantize)
+    p1 = to_oracle(orc, fastnn_amd.quantize_weights_kn(dt, params["w1"]))
+    p2 = to_oracle(orc, fastnn_amd.quantize_weights_kn(dt, params["w2"]))
+    try:
+        for it in range(3):
+            x = rng.standard_normal((5, 64)).astype(np.float32)
+            got = ex.forward({"x": x})["y"]
+            h = orc.qmatmul(p1, x, bias=params["b1"], act=flib.ACT_GELU)
+            want = orc.qmatmul(p2, h) + x
+            assert got.shape == (5, 64)
+            assert_close(got, want, 1e-4, f"quantize={quantize} call {it}")
+            assert ex.replayed == (it >= 1)
+    finally:
+        ex.close()
+
+
+@pytest.mark.gpu
+def test_forward_conv_graph(orc):
+    from gpu_common import assert_close, to_oracle
+    rng = np.random.default_rng(9)
+    nodes = [
+        {"name": "c1", "op_type": "Conv", "inputs": "[x, w, b]", "outputs": "[c]", "strides": "2", "pads": "1"},
+        {"name": "a1", "op_type": "Silu", "inputs": "[c]", "outputs": "[s]"},
+        {"name": "p", "op_type": "MaxPool", "inputs": "[s]", "outputs": "[m]", "kernel_shape": "5", "strides": "1", "pads": "2"},
+        {"name": "cat", "op_type": "Concat", "inputs": "[s, m]", "outputs": "[k]", "axis": "1"},
+        {"name": "up", "op_type": "Resize", "inputs": "[k]", "outputs": "[y]", "mode": "nearest", "scale_h": "2", "scale_w": "2"},
+    ]
+    w = (rng.standard_normal((8, 3, 3, 3)) * 0.3).astype(np.float32)
+    b = (rng.standard_normal(8) * 0.05).astype(np.float32)
+    x = rng.uniform(0, 1, (2, 3, 16, 16)).astype(np.float32)
+    ex = AotExecutor(nodes, {"w": w, "b": b}, ["x"], ["y"], {"x": list(x.shape)}, quantize=8)
+    try:
+        got = ex.forward({"x": x})["y"]
+        pw = to_oracle(orc, fastnn_amd.quantize_weights(flib.DT_I8, w.reshape(8, 27)))
+        s = orc.qconv2d_i8(x, pw, 3, 3, 2, 1, 1, 1, bias=b, act=flib.ACT_SILU)
+        want = orc.upsample_nearest2d(np.concatenate([s, orc.maxpool2d(s, 5, 1, 2)], axis=1), 2, 2)
+        assert got.shape == want.shape == (2, 16, 16, 16)
+        assert_close(got, want, 1e-5, "conv graph")
+    finally:
+        ex.close()
