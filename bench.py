@@ -41,6 +41,7 @@ WORKLOADS = {
 COMPOSITE = {
     "c4_mlp_f8": ("mlp", "f8"), "c4_mlp_f4": ("mlp", "f4"),
     "c5_yolo_b1": ("yolo", 1), "c5_yolo_b16": ("yolo", 16),
+    "c5_yolo_graph_b1": ("yolo_graph", 1), "c5_yolo_graph_b16": ("yolo_graph", 16),
 }
 
 # YOLOv8n-shaped conv list (width 0.25, depth 0.33, 640x640 input, Detect head excluded): (C_in, H_in, C_out, k, stride);
@@ -61,6 +62,77 @@ def yolo_convs():
     conv(64, 80, 64, 3, 2); c2f(192, 128, 1, 40)
     conv(128, 40, 128, 3, 2); c2f(384, 256, 1, 20)
     return L
+
+
+def yolo_graph(batch, rng, size=640):
+    """The same network as a graph in the reference's node-dict form (backbone layers 0-9, neck layers 10-21, Detect
+    head excluded): Conv + SiLU, C2f with channel Split / residual Add / Concat, SPPF max-pool pyramid, nearest
+    2x Resize.  Returns (nodes, params, input shape, output names)."""
+    nodes, params = [], {}
+    cnt = [0]
+
+    def uid(p):
+        cnt[0] += 1
+        return f"{p}{cnt[0]}"
+
+    def conv(x, c, oc, k, s):
+        w, b, y0, y = uid("w"), uid("b"), uid("c"), uid("s")
+        kk = c * k * k
+        params[w] = (rng.standard_normal((oc, c, k, k)) * np.sqrt(2.0 / kk)).astype(np.float32)
+        params[b] = (rng.standard_normal(oc) * 0.05).astype(np.float32)
+        nodes.append({"name": y0, "op_type": "Conv", "inputs": f"[{x}, {w}, {b}]", "outputs": f"[{y0}]", "strides": str(s),
+                      "pads": str(k // 2), "group": "1"})
+        nodes.append({"name": y, "op_type": "Silu", "inputs": f"[{y0}]", "outputs": f"[{y}]"})
+        return y
+
+    def c2f(x, c1, c2, n, shortcut):
+        y = conv(x, c1, c2, 1, 1)
+        a, b = uid("h"), uid("h")
+        nodes.append({"name": a, "op_type": "Split", "inputs": f"[{y}]", "outputs": f"[{a}, {b}]", "axis": "1"})
+        parts, last = [a, b], b
+        for _ in range(n):
+            t = conv(conv(last, c2 // 2, c2 // 2, 3, 1), c2 // 2, c2 // 2, 3, 1)
+            if shortcut:
+                r = uid("r")
+                nodes.append({"name": r, "op_type": "Add", "inputs": f"[{last}, {t}]", "outputs": f"[{r}]"})
+                t = r
+            parts.append(t)
+            last = t
+        cat = uid("k")
+        nodes.append({"name": cat, "op_type": "Concat", "inputs": "[" + ", ".join(parts) + "]", "outputs": f"[{cat}]", "axis": "1"})
+        return conv(cat, (2 + n) * c2 // 2, c2, 1, 1)
+
+    def concat(xs):
+        cat = uid("k")
+        nodes.append({"name": cat, "op_type": "Concat", "inputs": "[" + ", ".join(xs) + "]", "outputs": f"[{cat}]", "axis": "1"})
+        return cat
+
+    def up(x):
+        u = uid("u")
+        nodes.append({"name": u, "op_type": "Resize", "inputs": f"[{x}]", "outputs": f"[{u}]", "mode": "nearest", "scale_h": "2", "scale_w": "2"})
+        return u
+
+    x = conv("x", 3, 16, 3, 2)
+    x = conv(x, 16, 32, 3, 2)
+    x = c2f(x, 32, 32, 1, True)
+    x = conv(x, 32, 64, 3, 2)
+    p3 = c2f(x, 64, 64, 2, True)
+    x = conv(p3, 64, 128, 3, 2)
+    p4 = c2f(x, 128, 128, 2, True)
+    x = conv(p4, 128, 256, 3, 2)
+    x = c2f(x, 256, 256, 1, True)
+    s = conv(x, 256, 128, 1, 1)                                   # SPPF
+    pools = [s]
+    for _ in range(3):
+        m = uid("m")
+        nodes.append({"name": m, "op_type": "MaxPool", "inputs": f"[{pools[-1]}]", "outputs": f"[{m}]", "kernel_shape": "5", "strides": "1", "pads": "2"})
+        pools.append(m)
+    p5 = conv(concat(pools), 512, 256, 1, 1)
+    n4 = c2f(concat([up(p5), p4]), 384, 128, 1, False)
+    n3 = c2f(concat([up(n4), p3]), 192, 64, 1, False)
+    n4b = c2f(concat([conv(n3, 64, 64, 3, 2), n4]), 192, 128, 1, False)
+    n5 = c2f(concat([conv(n4b, 128, 128, 3, 2), p5]), 384, 256, 1, False)
+    return nodes, params, [batch, 3, size, size], [n3, n4b, n5]
 
 
 def composite(args) -> int:
@@ -124,6 +196,35 @@ def composite(args) -> int:
                          "max_rel_vs_default": float(np.abs(y1 - y).max() / (np.abs(y).max() + 1e-30))}}
         print(json.dumps(out))
         be.close()
+        return 0
+    if kind == "yolo_graph":
+        from fastnn_amd.aot import AotExecutor
+        batch = par
+        nodes, params, shape, outs = yolo_graph(batch, rng)
+        t0 = time.perf_counter()
+        ex = AotExecutor(nodes, params, ["x"], outs, {"x": shape}, quantize=8)
+        build_s = time.perf_counter() - t0
+        ex.write_inputs({"x": rng.uniform(0, 1, shape).astype(np.float32)})
+        for _ in range(2 + warm):
+            ex.dispatch()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            ex.dispatch()
+        ms = (time.perf_counter() - t0) * 1e3 / steps
+        flops = sum(2.0 * batch * ((h + 2 * (k // 2) - k) // s + 1) ** 2 * c * k * k * oc for (c, h, oc, k, s) in yolo_convs())
+        y = [ex.read_output(o) for o in outs]
+        kinds = {}
+        for ins in ex.instructions:
+            kinds[ins[0]] = kinds.get(ins[0], 0) + 1
+        out = {"metric": f"C5 YOLOv8n-shaped I8 graph forward (backbone + neck as one plan, B={batch})",
+               "value": round(batch / (ms * 1e-3), 1), "unit": "images/s", "n_gpus": 1, "steps": steps, "warmup": warm,
+               "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "i8/i32",
+               "data": "synthetic", "config": {"workload": args.workload, "launch": "AotExecutor plan, HIP-graph replay + sync per step",
+                                               "instructions": kinds, "arena_bytes": ex.arena_size},
+               "tops": round(flops / (ms * 1e-3) / 1e12, 2), "replayed": ex.replayed, "lowering_s": round(build_s, 2),
+               "outputs": [list(t.shape) for t in y], "finite_output": bool(all(np.isfinite(t).all() for t in y))}
+        print(json.dumps(out))
+        ex.close()
         return 0
     batch = par
     ctx = fastnn_amd.HipContext(0)

@@ -192,6 +192,28 @@ class AotExecutor:
                 inner = int(np.prod(shape[axis + 1:], dtype=np.int64))
                 outer = int(np.prod(shape[:axis], dtype=np.int64))
                 self._emit("concat", ins, outs[0], [v.slot for v in vals], out.slot, [axis, inner, outer])
+            elif op == "Split":
+                # one slice_f32 per output (src/onnx/converter.rs:549-612): explicit `split` sizes, else equal
+                # parts with the remainder in the last one
+                a = self._val(ins[0])
+                rank = len(a.shape)
+                axis = _attr_int(nd, "axis", default=0)
+                axis = axis + rank if axis < 0 else axis
+                axis = min(max(axis, 0), rank - 1)
+                sizes = [int(v) for v in nd.get("split", "").split(",") if v.strip()]
+                if not (len(sizes) == len(outs) and all(v > 0 for v in sizes)):
+                    part = a.shape[axis] // max(len(outs), 1)
+                    if part < 1:
+                        raise FnnError(4, f"Split: {a.shape[axis]} values along axis {axis} into {len(outs)} outputs")
+                    sizes = [part] * (len(outs) - 1) + [a.shape[axis] - part * (len(outs) - 1)]
+                inner = int(np.prod(a.shape[axis + 1:], dtype=np.int64))
+                start = 0
+                for o, sz in zip(outs, sizes):
+                    shape = list(a.shape)
+                    shape[axis] = sz
+                    out = self._new_value(o, shape)
+                    self._emit("slice_f32", ins, o, [a.slot], out.slot, [axis, start, start + sz, inner])
+                    start += sz
             elif op == "Resize":
                 a = self._val(ins[0])
                 if nd.get("mode", "nearest") != "nearest":
@@ -355,6 +377,25 @@ class AotExecutor:
             v = self._values[name]
             out[name] = self._backend.read_arena(*v.slot, np.float32).reshape(v.shape).copy()
         return out
+
+    def write_inputs(self, inputs: Dict[str, np.ndarray]):
+        """Copies the inputs into their arena slots (what forward() does first)."""
+        self._ensure_plan()
+        for name in self.input_names:
+            v = self._values[name]
+            x = np.ascontiguousarray(inputs[name], dtype=np.float32)
+            if x.shape != v.shape:
+                raise FnnError(1, f"input '{name}' has shape {x.shape}, compiled for {v.shape}")
+            self._backend.write_arena(v.slot[0], x)
+
+    def dispatch(self):
+        """Runs the plan on whatever the input slots hold (inputs resident on the device) and synchronises."""
+        self._ensure_plan()
+        self._backend.dispatch(self._plan)
+
+    def read_output(self, name: str) -> np.ndarray:
+        v = self._values[name]
+        return self._backend.read_arena(*v.slot, np.float32).reshape(v.shape).copy()
 
     @property
     def replayed(self) -> bool:
