@@ -125,6 +125,7 @@ void free_weight(fnn_hip_weight *w)
     if (w->row_qsum) (void)hipFree(w->row_qsum);
     if (w->umean) (void)hipFree(w->umean);
     if (w->words4) (void)hipFree(w->words4);
+    if (w->dense16) (void)hipFree(w->dense16);
     delete w;
 }
 

@@ -438,15 +438,31 @@ int run_tiled_codebook(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w,
     const int64_t kpad = (q.k + BK - 1) / BK * BK;
     const size_t op_bytes = (size_t)q.n * 2 * kpad * 2;
     const size_t tab_off = (op_bytes + 255) / 256 * 256;
-    void *ws = nullptr;
-    int rc = fnn_ctx_ensure_tmp(ctx, 3, tab_off + (size_t)q.n * 8 + 256, &ws);
-    if (rc) return rc;
+    const size_t total = tab_off + (size_t)q.n * 8 + 256;
+    // The expansion is kept with the weight (eight times the packed bytes, what the CPU path spends on its
+    // cached f32 copy); FNN_CODEBOOK_CACHE=0 expands into a workspace on every call instead.
+    static const bool keep = env_int("FNN_CODEBOOK_CACHE", 1) != 0;
+    fnn_hip_weight *wm = const_cast<fnn_hip_weight *>(w);
+    void *ws = keep && q.words == w->words ? wm->dense16 : nullptr;
+    bool expand = true;
+    if (ws) {
+        expand = false;
+    } else if (keep && q.words == w->words && !fnn_ctx_capturing(ctx)) {
+        if (hipMalloc(&wm->dense16, total) != hipSuccess)
+            return fnn_ctx_fail(ctx, FNN_ERR_MEMORY, "out of device memory (expanded codebook weight)");
+        ws = wm->dense16;
+    } else {
+        int rc = fnn_ctx_ensure_tmp(ctx, 3, total, &ws);
+        if (rc) return rc;
+    }
     _Float16 *op = (_Float16 *)ws;
     float *row_scale = (float *)((char *)ws + tab_off), *row_zero = row_scale + q.n;
-    hipLaunchKernelGGL(expand_codebook_kernel, dim3((unsigned)q.n), dim3(256), 0, s, q.words, q.scales, q.codebook, q.n, q.k,
-                       q.kp, q.bpr, q.qblock, kpad, op, row_scale, row_zero);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, hipGetErrorString(e));
+    if (expand) {
+        hipLaunchKernelGGL(expand_codebook_kernel, dim3((unsigned)q.n), dim3(256), 0, s, q.words, q.scales, q.codebook, q.n, q.k,
+                           q.kp, q.bpr, q.qblock, kpad, op, row_scale, row_zero);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, hipGetErrorString(e));
+    }
     DenseOperand d{(const uint32_t *)op, row_scale, row_zero};
     return run_tiled<DT_F16_DENSE>(ctx, s, w, q, flags, &d);
 }
