@@ -618,6 +618,7 @@ int fnn_hip_qconv2d(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *x, i
     p.b = b; p.c = c; p.h = h; p.w = wd; p.oc = oc; p.ho = ho; p.wo = wo; p.kp = w->kp;
     p.kh = kh; p.kw = kw; p.stride = stride; p.pad = pad; p.dil = dil; p.groups = groups; p.act = act;
     p.wbits = w->dtype == FNN_DT_I4 ? 4 : 8;
+    p.x8 = nullptr; p.payload_i4 = 0;
     if (flags & FNN_FLAG_FORCE_GENERIC) {
         HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qconv2d_i8(p, ctx->stream, 0));
     } else {
@@ -632,6 +633,81 @@ int fnn_hip_qconv2d(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *x, i
     if (!dev) {
         HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(y, dy, yout, hipMemcpyDeviceToHost, ctx->stream));
         if (acc_out) HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(acc_out, dacc, yout, hipMemcpyDeviceToHost, ctx->stream));
+        HIP_TRY(ctx, FNN_ERR_DISPATCH, hipStreamSynchronize(ctx->stream));
+    }
+    return FNN_OK;
+}
+
+int fnn_hip_qconv2d_i8act(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const uint8_t *payload, int64_t b, int64_t c,
+                          int64_t h, int64_t wd, int kh, int kw, int stride, int pad, int dil, int groups,
+                          const float *bias, int act, float *y, int flags)
+{
+    if (!ctx) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_hip_qconv2d_i8act: NULL context");
+    if (!w) return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8_i8: missing weight_meta for quantized weight");
+    if (w->dtype != FNN_DT_I8 && w->dtype != FNN_DT_I4)
+        return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "conv2d_i8_i8: weight type %d has no I8-activation kernel", w->dtype);
+    if (groups <= 0) return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8_i8: groups must be > 0");
+    if (b < 0 || c <= 0 || h <= 0 || wd <= 0 || kh <= 0 || kw <= 0 || stride <= 0 || dil <= 0 || pad < 0)
+        return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8_i8: invalid geometry");
+    if (c % groups || w->rows % groups)
+        return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8_i8: channels (%lld in, %lld out) not divisible by groups %d",
+                    (long long)c, (long long)w->rows, groups);
+    if (w->inner != (c / groups) * kh * kw)
+        return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8_i8: weight inner dim %lld != C/g*KH*KW = %lld", (long long)w->inner,
+                    (long long)((c / groups) * kh * kw));
+    if (act < FNN_ACT_NONE || act > FNN_ACT_SILU) return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "conv2d_i8_i8: unknown activation %d", act);
+    auto osz = [](int64_t in, int k, int s, int p, int d) -> int64_t {
+        int64_t dk = (int64_t)(k - 1) * d + 1;
+        return (in + 2 * p >= dk) ? (in + 2 * p - dk) / s + 1 : 0;
+    };
+    const int64_t ho = osz(h, kh, stride, pad, dil), wo = osz(wd, kw, stride, pad, dil);
+    const int64_t oc = w->rows;
+    if (b == 0 || ho == 0 || wo == 0) return FNN_OK;
+    if (!payload || !y) return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8_i8: NULL input or output pointer");
+    if (b * groups > 65535) return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "conv2d_i8_i8: batch*groups > 65535");
+    const bool dev = (flags & FNN_FLAG_DEVICE_PTRS) != 0;
+    if (dev && (reinterpret_cast<uintptr_t>(payload) & 3))
+        return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8_i8: activation payload must be 4-byte aligned");
+    fnn_hip_weight *wm = const_cast<fnn_hip_weight *>(w);
+    if (!wm->row_qsum) {
+        if (ctx->capturing) return fail(ctx, FNN_ERR_MEMORY, "conv2d_i8_i8: first use of a weight during graph capture");
+        HIP_TRY(ctx, FNN_ERR_MEMORY, hipMalloc((void **)&wm->row_qsum, (size_t)oc * 4 + 64));
+        HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_row_qsum(w, wm->row_qsum, ctx->stream));
+    }
+    const size_t xin = (size_t)(b * c * h * wd) + 8, yout = (size_t)(b * oc * ho * wo) * 4;
+    const uint8_t *dp = payload;
+    const float *dbias = bias;
+    float *dy = y;
+    int rc;
+    if (!dev) {
+        if ((rc = ensure(ctx, ctx->st_a, xin))) return rc;
+        if ((rc = ensure(ctx, ctx->st_out, yout))) return rc;
+        HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(ctx->st_a.ptr, payload, xin, hipMemcpyHostToDevice, ctx->stream));
+        dp = (const uint8_t *)ctx->st_a.ptr;
+        dy = (float *)ctx->st_out.ptr;
+        if (bias) {
+            if ((rc = ensure(ctx, ctx->st_bias, (size_t)oc * 4))) return rc;
+            HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(ctx->st_bias.ptr, bias, (size_t)oc * 4, hipMemcpyHostToDevice, ctx->stream));
+            dbias = (const float *)ctx->st_bias.ptr;
+        }
+    }
+    if ((rc = ensure(ctx, ctx->st_tmp, (size_t)(b * groups) * (QCONV_NPART * 2 + 4) * 4))) return rc;
+    QConvArgs p;
+    p.words = w->words; p.scales = w->scales; p.zeros = w->zeros; p.row_qsum = wm->row_qsum;
+    p.x = nullptr; p.bias = dbias; p.y = dy; p.acc_out = nullptr;
+    p.minmax_partial = (float *)ctx->st_tmp.ptr;
+    p.actq = p.minmax_partial + (size_t)(b * groups) * QCONV_NPART * 2;
+    p.b = b; p.c = c; p.h = h; p.w = wd; p.oc = oc; p.ho = ho; p.wo = wo; p.kp = w->kp;
+    p.kh = kh; p.kw = kw; p.stride = stride; p.pad = pad; p.dil = dil; p.groups = groups; p.act = act;
+    p.wbits = w->dtype == FNN_DT_I4 ? 4 : 8;
+    p.x8 = reinterpret_cast<const int8_t *>(dp + 8);
+    p.payload_i4 = w->dtype == FNN_DT_I4;
+    HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_conv_actq_from_payload(dp, p.actq, (int)(b * groups), ctx->stream));
+    bool handled = false;
+    if ((rc = fnn_i8_tiled_conv(ctx, ctx->stream, w, p, &handled))) return rc;
+    if (!handled) return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "conv2d_i8_i8: shape outside the integer GEMM's limits");
+    if (!dev) {
+        HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(y, dy, yout, hipMemcpyDeviceToHost, ctx->stream));
         HIP_TRY(ctx, FNN_ERR_DISPATCH, hipStreamSynchronize(ctx->stream));
     }
     return FNN_OK;

@@ -316,6 +316,47 @@ int run_conv2d_i8(fnn_backend *b, const Instr &in, const KernelName &kn)
                                    bias, kn.act, (float *)(b->arena + in.dst.offset), nullptr, FNN_FLAG_DEVICE_PTRS | b->kernel_flags));
 }
 
+// "conv2d_i8_i8" / "conv2d_i4_i8" (src/backend/cpu/mod.rs:3848-4098): input 0 is an activation payload
+// [scale][zero][i8 NCHW]; the weight kernel is picked by weight_meta.bit_width
+int run_conv2d_i8act(fnn_backend *b, const Instr &in, const KernelName &kn)
+{
+    const char *name = in.kernel.c_str();
+    if (in.inputs.size() < 2) return FNN_OK;
+    if (in.params.size() < 9)
+        return fail(b, FNN_ERR_DISPATCH, "%s: expected at least 9 params [stride, padding, dilation, groups, input_c, input_h, input_w, kernel_h, kernel_w]", name);
+    const uint64_t *p = in.params.data();
+    uint64_t stride = p[0], pad = p[1], dil = p[2], groups = p[3], c = p[4], h = p[5], wd = p[6], kh = p[7], kw = p[8];
+    if (groups == 0) return fail(b, FNN_ERR_DISPATCH, "%s: groups=0", name);
+    if (!in.meta.present) return fail(b, FNN_ERR_DISPATCH, "%s: missing weight_meta", name);
+    if (in.meta.shape.empty()) return fail(b, FNN_ERR_DISPATCH, "%s: weight_meta has no shape", name);
+    if (in.inputs[0].size < 8) return fail(b, FNN_ERR_DISPATCH, "%s: activation payload holds %llu bytes, the header alone is 8", name, (unsigned long long)in.inputs[0].size);
+    if (in.inputs[0].offset & 3) return fail(b, FNN_ERR_DISPATCH, "%s: activation payload must be 4-byte aligned", name);
+    uint64_t oc = in.meta.shape[0], inner = 1;
+    for (size_t i = 1; i < in.meta.shape.size(); i++) inner *= in.meta.shape[i];
+    uint64_t chw = c * h * wd;
+    uint64_t batch = (in.inputs[0].size - 8) / (chw ? chw : 1);
+    const float *bias = nullptr;
+    if (in.inputs.size() >= 3 && in.inputs[2].size) {
+        if (in.inputs[2].size < oc * 4) return fail(b, FNN_ERR_DISPATCH, "%s: bias slice holds %llu bytes, OC*4 = %llu", name, (unsigned long long)in.inputs[2].size, (unsigned long long)(oc * 4));
+        bias = (const float *)(b->arena + in.inputs[2].offset);
+    }
+    if (stride == 0 || dil == 0) return fail(b, FNN_ERR_DISPATCH, "%s: stride and dilation must be positive", name);
+    uint64_t eh = dil * (kh - 1) + 1, ew = dil * (kw - 1) + 1;
+    if (h + 2 * pad < eh || wd + 2 * pad < ew) return fail(b, FNN_ERR_DISPATCH, "%s: kernel larger than padded input", name);
+    uint64_t oh = (h + 2 * pad - eh) / stride + 1, ow = (wd + 2 * pad - ew) / stride + 1;
+    if (in.dst.size < batch * oc * oh * ow * 4) return fail(b, FNN_ERR_DISPATCH, "%s: output slice holds %llu bytes, needs %llu", name, (unsigned long long)in.dst.size, (unsigned long long)(batch * oc * oh * ow * 4));
+    if (in.meta.bit_width == 4 && !in.meta.codebook.empty())
+        return fail(b, FNN_ERR_UNSUPPORTED_OP, "%s: codebook weights have no I8-activation kernel", name);
+    const int dtype = in.meta.bit_width == 4 ? FNN_DT_I4 : FNN_DT_I8;
+    fnn_hip_weight *w = nullptr;
+    int st = weight_for(b, in.inputs[1], dtype, in.meta, oc, inner, name, &w);
+    if (st) return st;
+    if (batch == 0) return FNN_OK;
+    return lift(b, fnn_hip_qconv2d_i8act(b->ctx, w, b->arena + in.inputs[0].offset, (int64_t)batch, (int64_t)c, (int64_t)h, (int64_t)wd,
+                                         (int)kh, (int)kw, (int)stride, (int)pad, (int)dil, (int)groups, bias, kn.act,
+                                         (float *)(b->arena + in.dst.offset), FNN_FLAG_DEVICE_PTRS | b->kernel_flags));
+}
+
 int run_elementwise(fnn_backend *b, const Instr &in, int op)
 {
     const char *name = in.kernel.c_str();
@@ -467,6 +508,7 @@ int run_call(fnn_backend *b, const Instr &in)
     if (kn.base == "conv2d_i8" || kn.base == "conv2d_i4" || kn.base == "conv2d_u8" || kn.base == "conv2d_u4" ||
         kn.base == "conv2d_f8" || kn.base == "conv2d_f8r" || kn.base == "conv2d_f4")
         return run_conv2d_i8(b, in, kn);
+    if (kn.base == "conv2d_i8_i8" || kn.base == "conv2d_i4_i8") return run_conv2d_i8act(b, in, kn);
     return fail(b, FNN_ERR_UNSUPPORTED_OP, "%s", name.c_str());
 }
 

@@ -26,6 +26,9 @@ struct QConvArgs {
     int64_t b, c, h, w, oc, ho, wo, kp;
     int kh, kw, stride, pad, dil, groups, act;
     int wbits;               // 8: I8 weights, activations quantised to 256 levels; 4: I4 weights, 16 levels
+    const int8_t *x8;        // non-null: the input is already int8 [B,C,H,W] (an activation payload's data)
+                             // with one (scale, zero) for the whole tensor in actq; padding taps are the integer 0
+    int payload_i4;          // with x8 and I4 weights: the matmul_i4_i8 formula and a float bias
 };
 constexpr int QCONV_NPART = 512;
 
@@ -34,3 +37,5 @@ hipError_t launch_quantize_activations(const float *x, int64_t numel, float scal
 hipError_t launch_qgemm_i8act_generic(int dtype, const I8ActArgs &p, hipStream_t s);
 hipError_t launch_row_qsum(const fnn_hip_weight *w, int32_t *out, hipStream_t s);
 hipError_t launch_qconv2d_i8(const QConvArgs &p, hipStream_t s, int phase);
+// actq[i] = (scale, zero, 0, 0) of an activation payload's header, for i < nbg
+hipError_t launch_conv_actq_from_payload(const uint8_t *payload, float *actq, int nbg, hipStream_t s);

@@ -268,6 +268,23 @@ hipError_t launch_row_qsum(const fnn_hip_weight *w, int32_t *out, hipStream_t s)
     return hipGetLastError();
 }
 
+__global__ void __launch_bounds__(256) conv_actq_from_payload_kernel(const uint8_t *payload, float *actq, int nbg)
+{
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= nbg) return;
+    const float *hdr = reinterpret_cast<const float *>(payload);
+    actq[i * 4 + 0] = hdr[0];
+    actq[i * 4 + 1] = hdr[1];
+    actq[i * 4 + 2] = 0.0f;
+    actq[i * 4 + 3] = 0.0f;
+}
+
+hipError_t launch_conv_actq_from_payload(const uint8_t *payload, float *actq, int nbg, hipStream_t s)
+{
+    hipLaunchKernelGGL(conv_actq_from_payload_kernel, dim3((unsigned)((nbg + 255) / 256)), dim3(256), 0, s, payload, actq, nbg);
+    return hipGetLastError();
+}
+
 // phase 0: everything; 1: the (image, group) activation scales only; 2: the direct kernel only (scales present)
 hipError_t launch_qconv2d_i8(const QConvArgs &p, hipStream_t s, int phase)
 {

@@ -108,7 +108,9 @@ __global__ void __launch_bounds__(256) conv_operand_kernel(QConvArgs a, int g, i
         const int64_t nn = live ? r / np : 0, p = live ? r % np : 0;
         const int bg = (int)(nn * a.groups + g);
         const float za = a.actq[bg * 4 + 1], inv = a.actq[bg * 4 + 2];
-        const float *xg = a.x + (nn * a.c + g * cg) * a.h * a.w;
+        const int64_t x_off = (nn * a.c + g * cg) * a.h * a.w;
+        const float *xg = a.x + x_off;
+        const int8_t *xq = a.x8 ? a.x8 + x_off : nullptr;
         const int khw = a.kh * a.kw;
         const float qlo = a.wbits == 4 ? -8.0f : -128.0f, qhi = a.wbits == 4 ? 7.0f : 127.0f;
         const int interleaved = a.wbits == 4;   // the 4-bit weight decoder delivers k = 0,2,4,6,1,3,5,7 of each 8
@@ -124,10 +126,15 @@ __global__ void __launch_bounds__(256) conv_operand_kernel(QConvArgs a, int g, i
                 for (int t = 0; t < 16; t++) {
                     if (e < kk) {
                         const int64_t ih = ih0 + (int64_t)i * a.dil, iw = iw0 + (int64_t)j * a.dil;
-                        float v = 0.0f;
-                        if (ih >= 0 && ih < a.h && iw >= 0 && iw < a.w) v = xg[((int64_t)ic * a.h + ih) * a.w + iw];
-                        const float q = roundf((v - za) * inv);
-                        const int qi = (q != q) ? 0 : (int)fminf(fmaxf(q, qlo), qhi);
+                        const bool inside = ih >= 0 && ih < a.h && iw >= 0 && iw < a.w;
+                        int qi;
+                        if (xq) {   // already quantised (mod.rs:3878-3905 + im2col_i8, packed_conv.rs:69-115)
+                            qi = inside ? xq[((int64_t)ic * a.h + ih) * a.w + iw] : 0;
+                        } else {
+                            const float v = inside ? xg[((int64_t)ic * a.h + ih) * a.w + iw] : 0.0f;
+                            const float q = roundf((v - za) * inv);
+                            qi = (q != q) ? 0 : (int)fminf(fmaxf(q, qlo), qhi);
+                        }
                         s += qi;
                         const int pos = (t & 8) + slot_of(t & 7, interleaved);
                         out[pos >> 2] |= (uint32_t)(uint8_t)qi << (8 * (pos & 3));
@@ -202,16 +209,28 @@ __global__ void __launch_bounds__(256) conv_epilogue_kernel(QConvArgs a, int g, 
         const float sw = c_sw[fl], zw = c_zw[fl];
         const float sab = sa * sw;
         int bias_q = 0;
-        if (a.bias) {
+        if (a.bias && !a.payload_i4) {
             const float bq = roundf(c_bias[fl] / sab);
             bias_q = (bq != bq) ? 0 : (bq >= 2147483648.0f ? 2147483647 : (bq <= -2147483648.0f ? (-2147483647 - 1) : (int)bq));
         }
-        const int accv = c[r * ocg + f0 + fl] + bias_q;
-        const float zp_prod = za * zw;
-        float val = (float)accv * sab;
-        val = val + zw * r_sum[rr];
-        val = val + za * c_wt[fl];
-        val = val + zp_prod * (float)kk;
+        int accv;
+        float val;
+        if (a.payload_i4) {
+            // gemm_cpu_flat_i8_i4x8 on the gathered rows, then `+ bias` in f32 (mod.rs:3975-4032);
+            // for za != 0 the dot of the dequantised activations is formed from the integer sums
+            accv = c[r * ocg + f0 + fl];
+            const float dot = (za != 0.0f) ? (float)accv * sa + za * (float)a.row_qsum[(int64_t)g * ocg + f0 + fl] : (float)accv * sa;
+            const float input_sum = r_sum[rr] + (float)kk * za;
+            val = dot * sw + zw * input_sum;
+            if (a.bias) val += c_bias[fl];
+        } else {
+            accv = c[r * ocg + f0 + fl] + bias_q;
+            const float zp_prod = za * zw;
+            val = (float)accv * sab;
+            val = val + zw * r_sum[rr];
+            val = val + za * c_wt[fl];
+            val = val + zp_prod * (float)kk;
+        }
         if (a.act == FNN_ACT_RELU) val = fmaxf(val, 0.0f);
         else if (a.act == FNN_ACT_SILU) val = val / (1.0f + expf(-val));
         else if (a.act == FNN_ACT_GELU) val = val * 0.5f * (1.0f + tanhf(val * 0.7978846f * (1.0f + 0.044715f * val * val)));

@@ -30,7 +30,7 @@ EXPORTED_SYMBOLS = [
     "fnn_hip_device_count", "fnn_hip_create", "fnn_hip_destroy", "fnn_hip_last_error", "fnn_hip_sync",
     "fnn_hip_malloc", "fnn_hip_free", "fnn_hip_upload", "fnn_hip_download",
     "fnn_hip_weight_register", "fnn_hip_weight_lookup", "fnn_hip_weight_release", "fnn_hip_dequant",
-    "fnn_hip_qmatmul", "fnn_hip_quantize_activations", "fnn_hip_qmatmul_i8act", "fnn_hip_qconv2d",
+    "fnn_hip_qmatmul", "fnn_hip_quantize_activations", "fnn_hip_qmatmul_i8act", "fnn_hip_qconv2d", "fnn_hip_qconv2d_i8act",
     "fnn_hip_timer_start", "fnn_hip_timer_stop", "fnn_hip_probe_stream",
     "fnn_hip_graph_begin", "fnn_hip_graph_end", "fnn_hip_graph_launch", "fnn_hip_graph_destroy",
     "fnn_hip_workspace_epoch",
@@ -119,6 +119,8 @@ def _prototype(l):
     l.fnn_hip_qmatmul_i8act.argtypes = [_vp, _vp, _vp, _i64, _vp, _vp, C.c_int]
     l.fnn_hip_qconv2d.argtypes = [_vp, _vp, _vp, _i64, _i64, _i64, _i64, C.c_int, C.c_int, C.c_int, C.c_int,
                                   C.c_int, C.c_int, _vp, C.c_int, _vp, _vp, C.c_int]
+    l.fnn_hip_qconv2d_i8act.argtypes = [_vp, _vp, _vp, _i64, _i64, _i64, _i64, C.c_int, C.c_int, C.c_int, C.c_int,
+                                        C.c_int, C.c_int, _vp, C.c_int, _vp, C.c_int]
     l.fnn_hip_probe_stream.argtypes = [_vp, _vp, _vp, _sz]
     l.fnn_hip_timer_start.argtypes = [_vp]
     l.fnn_hip_timer_stop.argtypes = [_vp, C.POINTER(C.c_float)]
@@ -367,6 +369,23 @@ class HipContext:
         self._check(self.lib.fnn_hip_qconv2d(self.handle, wh, _np_ptr(x), b, c, h, w, kh, kw, stride, pad, dil, groups,
                                              _np_ptr(bb), act, _np_ptr(y), _np_ptr(acc), flags))
         return (y, acc) if want_acc else y
+
+    def qconv2d_i8act(self, wh, payload: np.ndarray, shape, oc: int, kh: int, kw: int, stride: int, pad: int, dil: int,
+                      groups: int, bias: Optional[np.ndarray] = None, act: int = ACT_NONE, flags: int = 0):
+        """conv2d_i8_i8 / conv2d_i4_i8: `payload` = [scale][zero][int8 NCHW of `shape`]."""
+        payload = np.ascontiguousarray(payload, dtype=np.uint8)
+        b, c, h, w = shape
+        if payload.size != 8 + b * c * h * w:
+            raise ValueError(f"payload holds {payload.size} bytes, 8 + B*C*H*W = {8 + b * c * h * w}")
+
+        def osz(i, k):
+            dk = (k - 1) * dil + 1
+            return (i + 2 * pad - dk) // stride + 1 if i + 2 * pad >= dk else 0
+        y = np.zeros((b, oc, osz(h, kh), osz(w, kw)), np.float32)
+        bb = None if bias is None else np.ascontiguousarray(bias, dtype=np.float32)
+        self._check(self.lib.fnn_hip_qconv2d_i8act(self.handle, wh, _np_ptr(payload), b, c, h, w, kh, kw, stride, pad,
+                                                   dil, groups, _np_ptr(bb), act, _np_ptr(y), flags))
+        return y
 
     # ---- timing / graphs ----
     def probe_stream(self, src_ptr: int, dst_ptr: int, nbytes: int):

@@ -139,6 +139,20 @@ int fnn_hip_qconv2d(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *x, i
                     int dil, int groups, const float *bias, int act, float *y, int32_t *acc_out,
                     int flags);
 
+/* "conv2d_i8_i8[_act]" / "conv2d_i4_i8[_act]" (src/backend/cpu/mod.rs:3848-4098): the input is an
+ * I8 activation payload [scale f32][zero f32][B*C*H*W x i8] (NCHW) as fnn_hip_quantize_activations
+ * writes it; the int8 values are gathered with im2col_i8 (src/backend/cpu/packed_conv.rs:69-115,
+ * padding taps are the integer 0), then
+ *  I8 weights: gemm_packed_i8x4_fused_raw with the payload's (scale, zero)
+ *      (packed_conv.rs:444-625, bias rounded to the accumulator grid);
+ *  I4 weights: gemm_cpu_flat_i8_i4x8 (src/backend/cpu/microkernels/gemm.rs:1795-1975), then the bias
+ *      added in f32 and the activation (mod.rs:4002-4032).
+ * y is f32 NCHW.  A device payload pointer must be 4-byte aligned. */
+int fnn_hip_qconv2d_i8act(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const uint8_t *payload,
+                          int64_t b, int64_t c, int64_t h, int64_t wd, int kh, int kw, int stride,
+                          int pad, int dil, int groups, const float *bias, int act, float *y,
+                          int flags);
+
 /* ---- stream timing (Backend::dispatch_profile, src/backend/mod.rs:178-211):
  * HIP events recorded on the context's stream. */
 int fnn_hip_timer_start(fnn_hip_ctx *ctx);

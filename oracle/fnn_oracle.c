@@ -25,6 +25,9 @@
  *   conv lowering .......... (I8 and I4 weights) equals float conv of dequantised operands; integer
  *                            accumulators exact; brute-force direct convolution; activation
  *                            quantiser re-derived in f32; flat-input special cases
+ *   conv on I8 payloads .... f64 convolution of the dequantised int8 activations (torch unfold on the
+ *                            exact integers, padding taps = integer 0) with the dequantised weights;
+ *                            bias on the accumulator grid (8-bit) or in f32 (4-bit); zero = 0 and != 0
  *   conv, other types ...... torch.nn.functional.conv2d in f64 on the dequantised weights
  *   concat / slice / max pool / nearest upsample ... numpy concatenate, slicing, repeat and
  *                            torch max_pool2d / interpolate (bit-identical data movement)
@@ -1123,6 +1126,104 @@ int fnn_or_qconv2d_i4(const float *x, size_t b, size_t c, size_t h, size_t w,
 {
     return qconv2d_int(4, x, b, c, h, w, words, oc, scales, n_scales, zeros, n_zeros, bias, kh, kw,
                        stride, pad, dil, groups, act, y, acc_out, act_scale_out, act_zero_out);
+}
+
+/* "conv2d_i8_i8" / "conv2d_i4_i8" (backend/cpu/mod.rs:3848-4098): the activation arrives as an I8 payload
+ * [scale f32][zero f32][B*C*H*W x i8] (quantize_activations); per image and group the int8 values
+ * are gathered with im2col_i8 (packed_conv.rs:69-115, padding taps are the integer 0), then
+ *   I8 weights: gemm_packed_i8x4_fused_raw with (sa, za) of the payload, i.e. the four-term
+ *     formula of conv2d_packed_i8x4 incl. the integer bias (packed_conv.rs:444-625);
+ *   I4 weights: gemm_cpu_flat_i8_i4x8 (microkernels/gemm.rs:1795-1975) on [sa][za][col],
+ *     then `+ bias` in f32 and the activation (mod.rs:4002-4032);
+ * results go to NCHW. */
+int fnn_or_qconv2d_i8payload(int dt, const uint8_t *payload, size_t payload_len, size_t c, size_t h,
+                             size_t w, const uint32_t *words, size_t oc, const float *scales,
+                             size_t n_scales, const float *zeros, size_t n_zeros, const float *bias,
+                             size_t kh, size_t kw, size_t stride, size_t pad, size_t dil,
+                             size_t groups, int act, float *y)
+{
+    if (dt != FNN_OR_I8 && dt != FNN_OR_I4) return -1;
+    if (groups == 0 || c % groups || oc % groups || payload_len < 8) return -1;
+    float sa, za;
+    memcpy(&sa, payload, 4);
+    memcpy(&za, payload + 4, 4);
+    const int8_t *x8 = (const int8_t *)(payload + 8);
+    size_t chw = c * h * w;
+    size_t b = chw ? (payload_len - 8) / chw : 0;
+    size_t cg = c / groups, ocg = oc / groups;
+    size_t ho = fnn_or_conv_out_size(h, kh, stride, pad, dil);
+    size_t wo = fnn_or_conv_out_size(w, kw, stride, pad, dil);
+    size_t np = ho * wo, kk = cg * kh * kw;
+    size_t items = (dt == FNN_OR_I4) ? 8 : 4, kp = ceil_div(kk, items);
+    uint8_t *pl = (uint8_t *)malloc(8 + np * kk + 1);
+    float *tmp = (float *)malloc((np * ocg + 1) * sizeof(float));
+    if (!pl || !tmp) { free(pl); free(tmp); return -2; }
+    memcpy(pl, payload, 8);
+    int8_t *col = (int8_t *)(pl + 8);
+    for (size_t nn = 0; nn < b; nn++)
+        for (size_t g = 0; g < groups; g++) {
+            const int8_t *xin = x8 + nn * chw + g * cg * h * w;
+            for (size_t oh = 0; oh < ho; oh++)
+                for (size_t ow = 0; ow < wo; ow++)
+                    for (size_t ic = 0; ic < cg; ic++)
+                        for (size_t i = 0; i < kh; i++)
+                            for (size_t j = 0; j < kw; j++) {
+                                size_t ih = oh * stride + i * dil, iw = ow * stride + j * dil;
+                                int8_t v = 0;
+                                if (ih < h + pad && iw < w + pad && ih >= pad && iw >= pad)
+                                    v = xin[(ic * h + (ih - pad)) * w + (iw - pad)];
+                                col[(oh * wo + ow) * kk + ic * kh * kw + i * kw + j] = v;
+                            }
+            const uint32_t *wg = words + g * ocg * kp;
+            const float *sg = (n_scales > 1) ? scales + g * ocg : scales;
+            const float *zg = (n_zeros > 1) ? zeros + g * ocg : zeros;
+            if (dt == FNN_OR_I4) {
+                int rc = fnn_or_qmatmul_i8act(dt, wg, ocg, kk, sg, n_scales > 1 ? ocg : n_scales, zg,
+                                              n_zeros > 1 ? ocg : n_zeros, pl, 8 + np * kk, np, tmp, NULL);
+                if (rc) { free(pl); free(tmp); return rc; }
+                for (size_t p = 0; p < np; p++)
+                    for (size_t f = 0; f < ocg; f++) {
+                        float val = tmp[p * ocg + f];
+                        if (bias) val += bias[g * ocg + f];
+                        if (act == FNN_OR_ACT_RELU) val = fmaxf(val, 0.0f);
+                        else if (act == FNN_OR_ACT_SILU) val = val / (1.0f + expf(-val));
+                        else if (act == FNN_OR_ACT_GELU)
+                            val = val * 0.5f * (1.0f + tanhf(val * 0.7978846f * (1.0f + 0.044715f * val * val)));
+                        y[(nn * oc + g * ocg + f) * np + p] = val;
+                    }
+                continue;
+            }
+            for (size_t f = 0; f < ocg; f++) {
+                size_t ch = g * ocg + f;
+                const uint32_t *wrow = wg + f * kp;
+                int32_t qb = 0;
+                for (size_t p = 0; p < kp; p++) qb += fnn_or_i8x4_sum(wrow[p]);
+                float sw = (n_scales > 1) ? sg[f] : sg[0];
+                float zw = (n_zeros > 1) ? zg[f] : (n_zeros ? zg[0] : 0.0f);
+                float sab = sa * sw;
+                int32_t bias_q = 0;
+                if (bias) bias_q = sat_i32(roundf(bias[ch] / sab), -2147483647 - 1, 2147483647);
+                float w_term = sw * (float)qb, zp_prod = za * zw;
+                for (size_t p = 0; p < np; p++) {
+                    const int8_t *arow = col + p * kk;
+                    int32_t qasum = 0, acc = bias_q;
+                    for (size_t e = 0; e < kk; e++) {
+                        qasum += arow[e];
+                        acc += arow[e] * (int32_t)(int8_t)(wrow[e / 4] >> (8 * (e % 4)));
+                    }
+                    float r = sa * (float)qasum;
+                    float val = (float)acc * sab + zw * r + za * w_term + zp_prod * (float)kk;
+                    if (act == FNN_OR_ACT_RELU) val = fmaxf(val, 0.0f);
+                    else if (act == FNN_OR_ACT_SILU) val = val / (1.0f + expf(-val));
+                    else if (act == FNN_OR_ACT_GELU)
+                        val = val * 0.5f * (1.0f + tanhf(val * 0.7978846f * (1.0f + 0.044715f * val * val)));
+                    y[(nn * oc + ch) * np + p] = val;
+                }
+            }
+        }
+    free(pl);
+    free(tmp);
+    return 0;
 }
 
 /* Conv2d for the weight types without an integer kernel (U8, U4, F8, F8R, F4 and 4-bit codebook

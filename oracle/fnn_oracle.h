@@ -110,6 +110,13 @@ int fnn_or_qconv2d_i4(const float *x, size_t b, size_t c, size_t h, size_t w,
                       int act, float *y, int32_t *acc_out, float *act_scale_out,
                       float *act_zero_out);
 
+/* "conv2d_i8_i8" / "conv2d_i4_i8": I8 activation payload, integer im2col (backend/cpu/mod.rs:3848-4098) */
+int fnn_or_qconv2d_i8payload(int dt, const uint8_t *payload, size_t payload_len, size_t c, size_t h,
+                             size_t w, const uint32_t *words, size_t oc, const float *scales,
+                             size_t n_scales, const float *zeros, size_t n_zeros, const float *bias,
+                             size_t kh, size_t kw, size_t stride, size_t pad, size_t dil,
+                             size_t groups, int act, float *y);
+
 /* weight types without an integer kernel: dequantise once, f32 convolution
  * (backend/cpu/mod.rs:4204-4257, microkernels/conv.rs:509-660) */
 int fnn_or_qconv2d_float(int dt, const float *x, size_t b, size_t c, size_t h, size_t w,

@@ -97,6 +97,8 @@ def _proto(l):
                                     C.c_void_p, _sz, C.c_void_p, _sz, _sz, _sz, _sz, _sz, _sz,
                                     C.c_int, _f32p, C.c_void_p, C.c_void_p, C.c_void_p]
     l.fnn_or_qconv2d_i4.argtypes = l.fnn_or_qconv2d_i8.argtypes
+    l.fnn_or_qconv2d_i8payload.argtypes = [C.c_int, _u8p, _sz, _sz, _sz, _sz, _u32p, _sz, C.c_void_p, _sz, C.c_void_p,
+                                           _sz, C.c_void_p, _sz, _sz, _sz, _sz, _sz, _sz, C.c_int, _f32p]
     l.fnn_or_qconv2d_float.argtypes = [C.c_int, _f32p, _sz, _sz, _sz, _sz, _u32p, _sz, C.c_void_p, _sz,
                                        C.c_void_p, _sz, _sz, C.c_void_p, C.c_void_p, _sz, _sz, _sz, _sz,
                                        _sz, _sz, C.c_int, _f32p]
@@ -354,3 +356,20 @@ def upsample_nearest2d(x, sh: int, sw: int) -> np.ndarray:
     out = np.zeros((n, c, h * sh, w * sw), np.float32)
     lib().fnn_or_upsample_nearest2d(x.reshape(-1), n * c, h, w, sh, sw, out.reshape(-1))
     return out
+
+
+def qconv2d_i8payload(payload, shape, p: Packed, kh: int, kw: int, stride: int, pad: int, dil: int, groups: int,
+                      bias=None, act: int = ACT_NONE) -> np.ndarray:
+    """conv2d_i8_i8 / conv2d_i4_i8: `payload` = [scale][zero][B*C*H*W int8] of an NCHW tensor of `shape`."""
+    payload = np.ascontiguousarray(payload, np.uint8)
+    b, c, h, w = shape
+    oc = p.rows
+    ho, wo = conv_out_size(h, kh, stride, pad, dil), conv_out_size(w, kw, stride, pad, dil)
+    y = np.zeros((b, oc, ho, wo), np.float32)
+    bb = None if bias is None else _f32(bias)
+    rc = lib().fnn_or_qconv2d_i8payload(p.dt, payload, payload.size, c, h, w, p.words, oc, _ptr(p.scales), p.scales.size,
+                                        _ptr(p.zeros), p.zeros.size, _ptr(bb), kh, kw, stride, pad, dil, groups, act,
+                                        y.reshape(-1))
+    if rc:
+        raise ValueError(f"qconv2d_i8payload rc={rc}")
+    return y

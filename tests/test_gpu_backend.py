@@ -155,6 +155,39 @@ def test_conv2d_i8_plan(be, orc, act, code, wdt, kname):
     assert_close(be.read_arena(*s_y, np.float32).reshape(want.shape), want, 1e-5, kname + act)
 
 
+@pytest.mark.parametrize("act,code", [("", 0), ("_relu", 1), ("_gelu", 2), ("_silu", 3)])
+@pytest.mark.parametrize("wdt,kname", [(flib.DT_I8, "conv2d_i8_i8"), (flib.DT_I4, "conv2d_i4_i8")])
+@pytest.mark.parametrize("calibrated", [False, True])
+def test_conv2d_on_i8_payload_plan(be, orc, act, code, wdt, kname, calibrated):
+    """quantize_activations -> conv2d_{i8,i4}_i8: the conv reads the int8 payload (no second
+    quantisation); the weight kernel is picked by the bit width of the weight metadata.
+    Calibrated: scale/zero given as f32 bit patterns, zero != 0 (the dequantised-lane form)."""
+    rng = np.random.default_rng(43)
+    b, c, h, w, oc, kh, kw, stride, pad, dil, groups = 2, 8, 14, 11, 12, 3, 3, 2, 1, 1, 2
+    kk = c // groups * kh * kw
+    x = rng.uniform(-1, 1, (b, c, h, w)).astype(np.float32)
+    pw = fastnn_amd.quantize_weights(wdt, (rng.standard_normal((oc, kk)) * 0.1).astype(np.float32))
+    bias = (rng.standard_normal(oc) * 0.05).astype(np.float32)
+    scale, zp = np.float32(0.009), np.float32(0.11)
+    payload = orc.quantize_activations(x.reshape(-1), float(scale), float(zp)) if calibrated else orc.quantize_activations(x.reshape(-1))
+    want = orc.qconv2d_i8payload(payload, x.shape, to_oracle(orc, pw), kh, kw, stride, pad, dil, groups, bias=bias, act=code)
+    a = Arena()
+    s_x, s_q, s_w, s_b, s_y = a.take(x.nbytes), a.take(8 + x.size), a.take(pw.words.nbytes), a.take(bias.nbytes), a.take(want.nbytes)
+    plan = ExecutablePlan(a.top).write_const(s_w[0], pw.words).write_const(s_b[0], bias)
+    qparams = [x.size, 0, 0]
+    if calibrated:
+        qparams += [int(scale.view(np.uint32)), int(zp.view(np.uint32))]
+    plan.call_kernel("quantize_activations", [s_x], s_q, qparams)
+    plan.call_kernel(kname + act, [s_q, s_w, s_b], s_y, [stride, pad, dil, groups, c, h, w, kh, kw],
+                     meta_of(pw, [oc, c // groups, kh, kw]))
+    be.allocate_arena(a.top)
+    be.write_arena(s_x[0], x)
+    be.dispatch(plan)
+    assert np.array_equal(be.read_arena(*s_q), payload)
+    tol = 1e-5 if not calibrated else 2e-5      # zero != 0: integer-sum form vs the reference's per-lane f32 sums
+    assert_close(be.read_arena(*s_y, np.float32).reshape(want.shape), want, tol, kname + act)
+
+
 def test_fill_memcopy_and_elementwise(be, orc):
     rng = np.random.default_rng(5)
     x = rng.standard_normal(1000).astype(np.float32)
@@ -183,9 +216,13 @@ def test_unsupported_and_malformed_instructions(be):
         be.dispatch(p)
     assert e.value.kind == "UnsupportedOp" and e.value.message == "softmax_f32"
     p = ExecutablePlan(4096).call_kernel("conv2d_i4_i8", [(0, 64), (64, 64)], (128, 64), [1] * 9)
-    with pytest.raises(flib.FnnError) as e:      # the I8-payload conv variants are not implemented
+    with pytest.raises(flib.FnnError) as e:
         be.dispatch(p)
-    assert e.value.kind == "UnsupportedOp" and e.value.message == "conv2d_i4_i8"
+    assert e.value.kind == "Dispatch" and "missing weight_meta" in e.value.message
+    p = ExecutablePlan(4096).call_kernel("conv2d_u8_i8", [(0, 64), (64, 64)], (128, 64), [1] * 9)
+    with pytest.raises(flib.FnnError) as e:      # no such name in the reference's dispatch either
+        be.dispatch(p)
+    assert e.value.kind == "UnsupportedOp" and e.value.message == "conv2d_u8_i8"
     p = ExecutablePlan(4096).call_kernel("conv2d_i4", [(0, 64), (64, 64)], (128, 64), [1] * 9)
     with pytest.raises(flib.FnnError) as e:
         be.dispatch(p)

@@ -308,6 +308,43 @@ def test_qconv2d_constant_and_empty(ctx, orc, wdt):
     ctx.release(h)
 
 
+@pytest.mark.parametrize("cfg", CONVS)
+@pytest.mark.parametrize("wdt", [flib.DT_I8, flib.DT_I4])
+@pytest.mark.parametrize("za", [0.0, 0.37])
+def test_qconv2d_on_i8_payload(ctx, orc, cfg, wdt, za):
+    """conv2d_i8_i8 / conv2d_i4_i8: int8 NCHW payload in, im2col on the integers (padding = 0),
+    integer GEMM, then the 4-term formula with integer bias (I8) or the matmul_i4_i8 formula with
+    an f32 bias (I4).  With za == 0 and no bias/activation the result is an exact function of
+    the integer accumulators, so it must match the oracle to the last f32 operation (1e-6)."""
+    rng = np.random.default_rng(6200 + cfg["c"])
+    kk = cfg["c"] // cfg["groups"] * cfg["kh"] * cfg["kw"]
+    shape = (cfg["b"], cfg["c"], cfg["h"], cfg["w"])
+    q = rng.integers(-128, 128, shape).astype(np.int8)
+    payload = orc.make_payload(0.0123, za, q.reshape(-1))
+    wt = (rng.standard_normal((cfg["oc"], kk)) * np.sqrt(2.0 / kk)).astype(np.float32)
+    bias = (rng.standard_normal(cfg["oc"]) * 0.05).astype(np.float32)
+    pw = fastnn_amd.quantize_weights(wdt, wt)
+    h = ctx.register(pw)
+    args = (cfg["kh"], cfg["kw"], cfg["stride"], cfg["pad"], cfg["dil"], cfg["groups"])
+    tol = 1e-6 if za == 0.0 else 2e-5
+    assert_close(ctx.qconv2d_i8act(h, payload, shape, cfg["oc"], *args),
+                 orc.qconv2d_i8payload(payload, shape, to_oracle(orc, pw), *args), tol, "plain")
+    for act in (0, 1, 2, 3):
+        want = orc.qconv2d_i8payload(payload, shape, to_oracle(orc, pw), *args, bias=bias, act=act)
+        got = ctx.qconv2d_i8act(h, payload, shape, cfg["oc"], *args, bias=bias, act=act)
+        assert_close(got, want, max(tol, 1e-5), f"act {act}")
+    ctx.release(h)
+
+
+def test_qconv2d_on_i8_payload_rejects_other_weight_types(ctx):
+    pw = fastnn_amd.quantize_weights(flib.DT_U8, np.ones((2, 2), np.float32))
+    h = ctx.register(pw)
+    with pytest.raises(fastnn_amd.FnnError) as e:
+        ctx.qconv2d_i8act(h, np.zeros(8 + 2 * 16, np.uint8), (1, 2, 4, 4), 2, 1, 1, 1, 0, 1, 1)
+    assert e.value.kind == "UnsupportedOp"
+    ctx.release(h)
+
+
 FLOAT_CONVS = [
     dict(b=2, c=4, h=20, w=24, oc=16, kh=3, kw=3, stride=2, pad=1, dil=1, groups=1),
     dict(b=1, c=32, h=12, w=12, oc=48, kh=1, kw=1, stride=1, pad=0, dil=1, groups=1),

@@ -147,3 +147,54 @@ def test_float_conv_equals_torch_conv_of_dequantised_weights(orc, dt, cfg):
     ref = F.conv2d(torch.from_numpy(x.astype(np.float64)), torch.from_numpy(deq), None, stride=stride, padding=pad,
                    dilation=dil, groups=groups).numpy()
     assert np.abs(nb - ref).max() <= 2e-6 * (np.abs(ref).max() + 1)
+
+
+@pytest.mark.parametrize("cfg", [
+    dict(b=2, c=3, h=9, w=11, oc=4, kh=3, kw=3, stride=2, pad=1, dil=1, groups=1),
+    dict(b=1, c=4, h=10, w=7, oc=4, kh=3, kw=2, stride=1, pad=2, dil=2, groups=2),
+    dict(b=1, c=8, h=6, w=6, oc=3, kh=1, kw=1, stride=1, pad=0, dil=1, groups=1),
+])
+@pytest.mark.parametrize("act", [0, 1, 2, 3])
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("zero_act", [True, False])
+def test_conv_on_i8_payload_matches_float_conv(orc, cfg, act, bits, zero_act):
+    """conv2d_i8_i8 / conv2d_i4_i8: the float meaning is a convolution of the dequantised int8
+    activations (padding taps are the integer 0, i.e. the value `za`) with the dequantised
+    weights; the 8-bit form adds the bias rounded to the accumulator grid, the 4-bit form
+    adds it in f32."""
+    rng = np.random.default_rng(310)
+    b, c, h, w, oc, kh, kw = (cfg[x] for x in ("b", "c", "h", "w", "oc", "kh", "kw"))
+    stride, pad, dil, groups = cfg["stride"], cfg["pad"], cfg["dil"], cfg["groups"]
+    cg, ocg = c // groups, oc // groups
+    kk = cg * kh * kw
+    q = rng.integers(-128, 128, (b, c, h, w)).astype(np.int8)
+    sa, za = np.float32(0.0123), np.float32(0.0 if zero_act else 0.37)
+    payload = np.concatenate([np.array([sa, za], np.float32).view(np.uint8), q.view(np.uint8).reshape(-1)])
+    wt = (rng.standard_normal((oc, kk)) * 0.1).astype(np.float32)
+    bias = (rng.standard_normal(oc) * 0.05).astype(np.float32)
+    p = orc.quantize(orc.I8 if bits == 8 else orc.I4, wt)
+    y = orc.qconv2d_i8payload(payload, (b, c, h, w), p, kh, kw, stride, pad, dil, groups, bias=bias, act=act)
+    qw = _qw(p, kk, bits)
+    for n in range(b):
+        for g in range(groups):
+            xs = torch.from_numpy(q[n:n + 1, g * cg:(g + 1) * cg].astype(np.float64))
+            col = F.unfold(xs, (kh, kw), dilation=dil, padding=pad, stride=stride)[0].numpy().T  # exact ints
+            da = col * float(sa) + float(za)
+            for f in range(ocg):
+                ch = g * ocg + f
+                dw = qw[ch] * float(p.scales[ch]) + float(p.zeros[ch])
+                if bits == 8:
+                    sab = np.float32(sa * p.scales[ch])
+                    r = np.float32(bias[ch] / sab)
+                    bq = int(np.sign(r) * np.floor(abs(r) + np.float32(0.5)))
+                    val = da @ dw + bq * float(sab)
+                else:
+                    val = da @ dw + float(bias[ch])
+                if act == 1:
+                    val = np.maximum(val, 0)
+                elif act == 2:
+                    val = 0.5 * val * (1 + np.tanh(0.7978845608 * (val + 0.044715 * val ** 3)))
+                elif act == 3:
+                    val = val / (1 + np.exp(-val))
+                got = y[n, ch].reshape(-1)
+                assert np.abs(got - val).max() <= 2e-5 * (np.abs(val).max() + 1), (cfg, ch)
