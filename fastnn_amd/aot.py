@@ -171,7 +171,7 @@ class AotExecutor:
                 a = self._val(ins[0])
                 out = self._new_value(outs[0], a.shape)
                 self._emit(_ACT_KERNEL[op], ins, outs[0], [a.slot], out.slot, [int(np.prod(a.shape))])
-            elif op == "MaxPool":
+            elif op in ("MaxPool", "AvgPool"):
                 a = self._val(ins[0])
                 k = _attr_int(nd, "kernel_size", "kernel_shape", default=2)
                 s = _attr_int(nd, "stride", "strides", default=k)
@@ -179,7 +179,7 @@ class AotExecutor:
                 n, c, h, w = a.shape
                 ho, wo = max(h + 2 * p - k, 0) // s + 1, max(w + 2 * p - k, 0) // s + 1
                 out = self._new_value(outs[0], (n, c, ho, wo))
-                self._emit("pool_f32", ins, outs[0], [a.slot], out.slot, [k, s, p, 1, n, c, h, w])
+                self._emit("pool_f32", ins, outs[0], [a.slot], out.slot, [k, s, p, 1 if op == "MaxPool" else 0, n, c, h, w])
             elif op == "Concat":
                 vals = [self._val(i) for i in ins]
                 rank = len(vals[0].shape)

@@ -26,6 +26,8 @@ hipError_t launch_fill(float *dst, uint64_t n, float value, hipStream_t s);
 hipError_t launch_eltwise(int op, const float *a, const float *b, uint64_t nb, float *out, uint64_t n, hipStream_t s);
 hipError_t launch_copy2d(float *dst, uint64_t dst_pitch, uint64_t dst_len, const float *src, uint64_t src_pitch, uint64_t src_len,
                          uint64_t width, uint64_t height, hipStream_t s);
+hipError_t launch_avgpool2d(const float *x, uint64_t in_len, float *y, uint64_t out_len, uint64_t h, uint64_t w,
+                            uint64_t ho, uint64_t wo, int kernel, int stride, int pad, hipStream_t s);
 hipError_t launch_maxpool2d(const float *x, uint64_t in_len, float *y, uint64_t out_len, uint64_t c, uint64_t h, uint64_t w,
                             uint64_t ho, uint64_t wo, int kernel, int stride, int pad, hipStream_t s);
 hipError_t launch_upsample_nearest2d(const float *x, float *y, uint64_t nc, uint64_t h, uint64_t w, int sh, int sw, hipStream_t s);
@@ -764,6 +766,19 @@ int fnn_hip_maxpool2d_f32(fnn_hip_ctx *ctx, const float *x, uint64_t in_len, flo
     uint64_t total = n * c * ho * wo;
     if (total > out_len) total = out_len;   // writes past the output slice are dropped (ops.rs:147-149)
     HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_maxpool2d(x, in_len, y, total, c, h, w, ho, wo, (int)kernel, (int)stride, (int)pad, ctx->stream));
+    return FNN_OK;
+}
+
+int fnn_hip_avgpool2d_f32(fnn_hip_ctx *ctx, const float *x, uint64_t in_len, float *y, uint64_t out_len, uint64_t n, uint64_t c,
+                          uint64_t h, uint64_t w, uint64_t kernel, uint64_t stride, uint64_t pad)
+{
+    if (!ctx || !x || !y) return fail(ctx, FNN_ERR_DISPATCH, "pool_f32: NULL argument");
+    if (kernel == 0 || stride == 0 || kernel > 1024 || pad > 1024) return fail(ctx, FNN_ERR_DISPATCH, "pool_f32: invalid kernel, stride or padding");
+    const uint64_t hp = h + 2 * pad, wp = w + 2 * pad;
+    const uint64_t ho = (hp > kernel ? hp - kernel : 0) / stride + 1, wo = (wp > kernel ? wp - kernel : 0) / stride + 1;
+    uint64_t total = n * c * ho * wo;
+    if (total > out_len) total = out_len;   // writes past the output slice are dropped (ops.rs:203-205)
+    HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_avgpool2d(x, in_len, y, total, h, w, ho, wo, (int)kernel, (int)stride, (int)pad, ctx->stream));
     return FNN_OK;
 }
 

@@ -58,6 +58,32 @@ __global__ void __launch_bounds__(256) maxpool2d_kernel(const float *x, uint64_t
     (void)c;
 }
 
+// window mean over the taps inside the image (padding taps neither add nor count), summed in (kh, kw) order
+__global__ void __launch_bounds__(256) avgpool2d_kernel(const float *x, uint64_t in_len, float *y, uint64_t out_len,
+                                                        uint64_t h, uint64_t w, uint64_t ho, uint64_t wo, int kernel, int stride, int pad)
+{
+    for (uint64_t o = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; o < out_len; o += (uint64_t)gridDim.x * blockDim.x) {
+        const uint64_t ww = o % wo, t = o / wo, hh = t % ho, nc = t / ho;
+        float val = 0.0f;
+        int count = 0;
+        for (int kh = 0; kh < kernel; kh++) {
+            const int64_t hi = (int64_t)(hh * stride) + kh - pad;
+            if (hi < 0 || hi >= (int64_t)h) continue;
+            for (int kw = 0; kw < kernel; kw++) {
+                const int64_t wi = (int64_t)(ww * stride) + kw - pad;
+                if (wi < 0 || wi >= (int64_t)w) continue;
+                const uint64_t idx = (nc * h + (uint64_t)hi) * w + (uint64_t)wi;
+                if (idx < in_len) {
+                    val += x[idx];
+                    count++;
+                }
+            }
+        }
+        if (count > 0) val /= (float)count;
+        y[o] = val;
+    }
+}
+
 __global__ void __launch_bounds__(256) upsample_nearest2d_kernel(const float *x, float *y, uint64_t total, uint64_t h, uint64_t w, int sh, int sw)
 {
     const uint64_t wo = w * sw, ho = h * sh;
@@ -87,6 +113,14 @@ hipError_t launch_maxpool2d(const float *x, uint64_t in_len, float *y, uint64_t 
 {
     if (out_len == 0) return hipSuccess;
     hipLaunchKernelGGL(maxpool2d_kernel, dim3(grid_for(out_len)), dim3(256), 0, s, x, in_len, y, out_len, c, h, w, ho, wo, kernel, stride, pad);
+    return hipGetLastError();
+}
+
+hipError_t launch_avgpool2d(const float *x, uint64_t in_len, float *y, uint64_t out_len, uint64_t h, uint64_t w,
+                            uint64_t ho, uint64_t wo, int kernel, int stride, int pad, hipStream_t s)
+{
+    if (out_len == 0) return hipSuccess;
+    hipLaunchKernelGGL(avgpool2d_kernel, dim3(grid_for(out_len)), dim3(256), 0, s, x, in_len, y, out_len, h, w, ho, wo, kernel, stride, pad);
     return hipGetLastError();
 }
 

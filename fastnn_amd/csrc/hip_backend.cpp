@@ -455,16 +455,18 @@ int run_slice(fnn_backend *b, const Instr &in)
                                       in_len - first, slice_elems, outer));
 }
 
-// "pool_f32": params [kernel, stride, padding, is_max, N, C, H, W] (src/backend/cpu/mod.rs:4362-4397)
+// "pool_f32": params [kernel, stride, padding, is_max, N, C, H, W] (src/backend/cpu/mod.rs:4362-4470)
 int run_pool(fnn_backend *b, const Instr &in)
 {
     if (in.inputs.empty()) return FNN_OK;
     if (in.params.size() != 8) return fail(b, FNN_ERR_DISPATCH, "pool_f32: expected params [kernel, stride, padding, is_max, N, C, H, W]");
     const uint64_t *p = in.params.data();
-    if (p[3] != 1) return fail(b, FNN_ERR_UNSUPPORTED_OP, "pool_f32: average pooling is not implemented on the GPU");
     const float *src = nullptr;
     int st = staged_input(b, in.inputs[0], in.dst, &src);
     if (st) return st;
+    if (p[3] != 1)   // pool_avg_f32_scalar (src/backend/cpu/microkernels/ops.rs:162-210)
+        return lift(b, fnn_hip_avgpool2d_f32(b->ctx, src, in.inputs[0].size / 4, (float *)(b->arena + in.dst.offset), in.dst.size / 4, p[4],
+                                             p[5], p[6], p[7], p[0], p[1], p[2]));
     return lift(b, fnn_hip_maxpool2d_f32(b->ctx, src, in.inputs[0].size / 4, (float *)(b->arena + in.dst.offset), in.dst.size / 4, p[4], p[5],
                                          p[6], p[7], p[0], p[1], p[2]));
 }

@@ -45,7 +45,7 @@ BACKEND_SYMBOLS = [
     "fnn_plan_add_memcopy", "fnn_plan_add_call_kernel", "fnn_plan_len", "fnn_plan_replayed",
     "fnn_backend_dispatch", "fnn_backend_dispatch_profile",
     "fnn_hip_elementwise", "fnn_hip_fill_f32", "fnn_hip_copy",
-    "fnn_hip_copy2d_f32", "fnn_hip_maxpool2d_f32", "fnn_hip_upsample_nearest2d_f32",
+    "fnn_hip_copy2d_f32", "fnn_hip_maxpool2d_f32", "fnn_hip_avgpool2d_f32", "fnn_hip_upsample_nearest2d_f32",
 ]
 
 

@@ -93,10 +93,15 @@ int fnn_hip_elementwise(fnn_hip_ctx *ctx, int op, const float *a, const float *b
  *    (:4721-4760);
  *  maxpool2d: "pool_f32" with is_max = 1 (:4362-4397, src/backend/cpu/microkernels/ops.rs:104-158), output
  *    Ho = sat_sub(H + 2*pad, kernel)/stride + 1, writes past out_len dropped;
+ *  avgpool2d: "pool_f32" with is_max != 1 (:4398-4470, ops.rs:162-210): the mean over the taps inside the image
+ *    (padding taps are not counted), summed in (kh, kw) order;
  *  upsample_nearest2d: "upsample_nearest2d" (:5496-5535, src/backend/cpu/microkernels/misc.rs:338-364). */
 int fnn_hip_copy2d_f32(fnn_hip_ctx *ctx, float *dst, uint64_t dst_pitch, uint64_t dst_len, const float *src,
                        uint64_t src_pitch, uint64_t src_len, uint64_t width, uint64_t height);
 int fnn_hip_maxpool2d_f32(fnn_hip_ctx *ctx, const float *x, uint64_t in_len, float *y, uint64_t out_len,
+                          uint64_t n, uint64_t c, uint64_t h, uint64_t w, uint64_t kernel, uint64_t stride,
+                          uint64_t pad);
+int fnn_hip_avgpool2d_f32(fnn_hip_ctx *ctx, const float *x, uint64_t in_len, float *y, uint64_t out_len,
                           uint64_t n, uint64_t c, uint64_t h, uint64_t w, uint64_t kernel, uint64_t stride,
                           uint64_t pad);
 int fnn_hip_upsample_nearest2d_f32(fnn_hip_ctx *ctx, const float *x, float *y, uint64_t nc, uint64_t h,

@@ -1355,6 +1355,37 @@ void fnn_or_maxpool2d(const float *in, size_t in_len, size_t n, size_t c, size_t
                 }
 }
 
+/* "pool_f32" with is_max != 1 (backend/cpu/mod.rs:4398-4470, microkernels/ops.rs:162-210; the AVX2
+ * form ops.rs:425-560 sums interior windows in the same (kh, kw) order and divides by kernel^2, which
+ * is the tap count there): mean over the taps inside the image, padding taps are not counted. */
+void fnn_or_avgpool2d(const float *in, size_t in_len, size_t n, size_t c, size_t h, size_t w,
+                      size_t kernel, size_t stride, size_t pad, float *out, size_t out_len)
+{
+    size_t hp = h + 2 * pad, wp = w + 2 * pad;
+    size_t ho = (hp > kernel ? hp - kernel : 0) / stride + 1;
+    size_t wo = (wp > kernel ? wp - kernel : 0) / stride + 1;
+    for (size_t nn = 0; nn < n; nn++)
+        for (size_t cc = 0; cc < c; cc++)
+            for (size_t hh = 0; hh < ho; hh++)
+                for (size_t ww = 0; ww < wo; ww++) {
+                    float val = 0.0f;
+                    size_t count = 0;
+                    for (size_t kh = 0; kh < kernel; kh++)
+                        for (size_t kw = 0; kw < kernel; kw++) {
+                            size_t hi = hh * stride + kh, wi = ww * stride + kw;
+                            if (hi < pad || wi < pad) continue;
+                            hi -= pad;
+                            wi -= pad;
+                            if (hi >= h || wi >= w) continue;
+                            size_t idx = nn * (c * h * w) + cc * (h * w) + hi * w + wi;
+                            if (idx < in_len) { val += in[idx]; count++; }
+                        }
+                    if (count > 0) val /= (float)count;
+                    size_t o = nn * (c * ho * wo) + cc * (ho * wo) + hh * wo + ww;
+                    if (o < out_len) out[o] = val;
+                }
+}
+
 /* "upsample_nearest2d" (backend/cpu/mod.rs:5496-5535, microkernels/misc.rs:338-364):
  * params [scale_h, scale_w, h_in, w_in]; nc = in_len/(h_in*w_in); every input value fills a
  * scale_h x scale_w block of the output. */

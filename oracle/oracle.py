@@ -106,6 +106,7 @@ def _proto(l):
     l.fnn_or_concat.restype = _sz
     l.fnn_or_slice.argtypes = [_f32p, _sz, _sz, _sz, _sz, _f32p, _sz]
     l.fnn_or_maxpool2d.argtypes = [_f32p, _sz, _sz, _sz, _sz, _sz, _sz, _sz, _sz, _f32p, _sz]
+    l.fnn_or_avgpool2d.argtypes = [_f32p, _sz, _sz, _sz, _sz, _sz, _sz, _sz, _sz, _f32p, _sz]
     l.fnn_or_upsample_nearest2d.argtypes = [_f32p, _sz, _sz, _sz, _sz, _sz, _f32p]
     l.fnn_or_seeded_values.argtypes = [C.c_uint64, _sz, _f32p]
 
@@ -347,6 +348,16 @@ def maxpool2d(x, kernel: int, stride: int, pad: int) -> np.ndarray:
     wo = max(w + 2 * pad - kernel, 0) // stride + 1
     out = np.zeros((n, c, ho, wo), np.float32)
     lib().fnn_or_maxpool2d(x.reshape(-1), x.size, n, c, h, w, kernel, stride, pad, out.reshape(-1), out.size)
+    return out
+
+
+def avgpool2d(x, kernel: int, stride: int, pad: int) -> np.ndarray:
+    x = _f32(x)
+    n, c, h, w = x.shape
+    ho = max(h + 2 * pad - kernel, 0) // stride + 1
+    wo = max(w + 2 * pad - kernel, 0) // stride + 1
+    out = np.zeros((n, c, ho, wo), np.float32)
+    lib().fnn_or_avgpool2d(x.reshape(-1), x.size, n, c, h, w, kernel, stride, pad, out.reshape(-1), out.size)
     return out
 
 

@@ -406,9 +406,12 @@ def test_data_movement_kernels(be, orc):
     p2 = ExecutablePlan(a.top).write_const(s_x[0], x).call_kernel("pool_f32", [s_x], s_x, [3, 1, 1, 1, n, c, h, w])
     be.dispatch(p2)
     assert np.array_equal(be.read_arena(*s_x, np.float32), orc.maxpool2d(x, 3, 1, 1).reshape(-1))
-    with pytest.raises(flib.FnnError) as e:
-        be.dispatch(ExecutablePlan(a.top).call_kernel("pool_f32", [s_x], s_pool, [2, 2, 0, 0, n, c, h, w]))
-    assert e.value.kind == "UnsupportedOp"
+    # average pooling (is_max = 0): same summation order as the CPU kernel, so bit-identical too
+    be.write_arena(s_x[0], x)
+    for (k, s, p) in [(5, 1, 2), (2, 2, 0), (3, 2, 1)]:
+        want = orc.avgpool2d(x, k, s, p)
+        be.dispatch(ExecutablePlan(a.top).call_kernel("pool_f32", [s_x], (s_pool[0], want.nbytes), [k, s, p, 0, n, c, h, w]))
+        assert np.array_equal(be.read_arena(s_pool[0], want.nbytes, np.float32), want.reshape(-1)), (k, s, p)
     with pytest.raises(flib.FnnError) as e:
         be.dispatch(ExecutablePlan(a.top).call_kernel("slice_f32", [s_x], s_lo, [1, 0, 2]))
     assert "expected params [dim, start, end, stride]" in e.value.message

@@ -1,5 +1,5 @@
 """Pins the oracle's restatement of the f32 data-movement kernels that sit between quantised
-convolutions (concat, slice_f32, pool_f32 max, upsample_nearest2d) against numpy / torch."""
+convolutions (concat, slice_f32, pool_f32 max and average, upsample_nearest2d) against numpy / torch."""
 import numpy as np
 import pytest
 import torch
@@ -51,6 +51,27 @@ def test_maxpool_window_in_the_padding_only_is_minus_inf(orc):
     got = orc.maxpool2d(x, 1, 1, 1)                 # 4x4 output, the border windows see padding only
     assert got.shape == (1, 1, 4, 4)
     assert np.all(np.isneginf(got[0, 0, 0])) and got[0, 0, 1, 1] == 1.0
+
+
+@pytest.mark.parametrize("k,s,p", [(5, 1, 2), (2, 2, 0), (3, 2, 1), (3, 1, 0)])
+def test_avgpool_is_torch_avg_pool2d_without_padding_in_the_count(orc, k, s, p):
+    """Mean over the taps inside the image: torch's avg_pool2d(count_include_pad=False), evaluated in
+    f64 (the f32 window sum is within 1e-6 of it); on integer-valued input with a power-of-two tap
+    count the result is exact."""
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((2, 3, 11, 9)).astype(np.float32)
+    want = F.avg_pool2d(torch.from_numpy(x).double(), k, s, p, count_include_pad=False).numpy()
+    got = orc.avgpool2d(x, k, s, p)
+    assert got.shape == want.shape and np.abs(got - want).max() <= 1e-6
+    xi = rng.integers(-50, 50, (1, 2, 8, 8)).astype(np.float32)
+    want = F.avg_pool2d(torch.from_numpy(xi).double(), 2, 2, 0).numpy()
+    assert np.array_equal(orc.avgpool2d(xi, 2, 2, 0), want.astype(np.float32))
+
+
+def test_avgpool_window_in_the_padding_only_is_zero(orc):
+    x = np.ones((1, 1, 2, 2), np.float32)
+    got = orc.avgpool2d(x, 1, 1, 1)
+    assert got.shape == (1, 1, 4, 4) and np.all(got[0, 0, 0] == 0.0) and got[0, 0, 1, 1] == 1.0
 
 
 @pytest.mark.parametrize("sh,sw", [(2, 2), (1, 3), (3, 1)])
