@@ -478,6 +478,14 @@ int fnn_hip_quantize_activations(fnn_hip_ctx *ctx, const float *x, int64_t numel
     return FNN_OK;
 }
 
+int fnn_hip_dequantize_activations(fnn_hip_ctx *ctx, const uint8_t *payload, uint64_t payload_len, float *out, uint64_t n)
+{
+    if (!ctx || ((!payload || !out) && n)) return fail(ctx, FNN_ERR_DISPATCH, "dequantize_activations: NULL argument");
+    if (reinterpret_cast<uintptr_t>(payload) & 3) return fail(ctx, FNN_ERR_DISPATCH, "dequantize_activations: payload must be 4-byte aligned");
+    HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_dequantize_activations(payload, payload_len, out, n, ctx->stream));
+    return FNN_OK;
+}
+
 int fnn_hip_qmatmul_i8act(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const uint8_t *payload,
                           int64_t m, float *out, int32_t *acc_out, int flags)
 {

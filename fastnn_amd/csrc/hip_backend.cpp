@@ -272,6 +272,19 @@ int run_quantize_activations(fnn_backend *b, const Instr &in)
                                                 b->arena + in.dst.offset, FNN_FLAG_DEVICE_PTRS));
 }
 
+// "dequantize_activations": params [numel, is_per_channel, num_channels] (src/backend/cpu/mod.rs:7009-7088)
+int run_dequantize_activations(fnn_backend *b, const Instr &in)
+{
+    uint64_t numel = in.params.empty() ? 0 : in.params[0];
+    bool per_channel = in.params.size() > 2 && in.params[1] == 1 && in.params[2] > 0;
+    if (per_channel) return fail(b, FNN_ERR_UNSUPPORTED_OP, "dequantize_activations: per-channel payloads are not implemented on the GPU");
+    if (in.inputs.empty()) return FNN_OK;
+    const uint64_t out_len = in.dst.size / 4;
+    if (numel > out_len) numel = out_len;   // out_f32.len().min(numel)
+    return lift(b, fnn_hip_dequantize_activations(b->ctx, b->arena + in.inputs[0].offset, in.inputs[0].size,
+                                                  (float *)(b->arena + in.dst.offset), numel));
+}
+
 int run_conv2d_i8(fnn_backend *b, const Instr &in, const KernelName &kn)
 {
     const char *name = in.kernel.c_str();
@@ -494,6 +507,7 @@ int run_call(fnn_backend *b, const Instr &in)
     if (!in_arena(b, in.dst)) return fail(b, FNN_ERR_DISPATCH, "%s: output slice [%llu,+%llu) outside the arena of %llu bytes", in.kernel.c_str(), (unsigned long long)in.dst.offset, (unsigned long long)in.dst.size, (unsigned long long)b->arena_bytes);
     const std::string &name = in.kernel;
     if (name == "quantize_activations") return run_quantize_activations(b, in);
+    if (name == "dequantize_activations") return run_dequantize_activations(b, in);
     if (name == "matmul_i8_i8") return run_matmul_i8act(b, in, FNN_DT_I8);
     if (name == "matmul_i4_i8") return run_matmul_i8act(b, in, FNN_DT_I4);
     if (name == "add_f32") return run_elementwise(b, in, 0);

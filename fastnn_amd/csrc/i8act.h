@@ -34,6 +34,7 @@ constexpr int QCONV_NPART = 512;
 
 hipError_t launch_quantize_activations(const float *x, int64_t numel, float scale, float zp,
                                        uint8_t *payload, float *scratch_partial, hipStream_t s);
+hipError_t launch_dequantize_activations(const uint8_t *payload, uint64_t payload_len, float *out, uint64_t n, hipStream_t s);
 hipError_t launch_qgemm_i8act_generic(int dtype, const I8ActArgs &p, hipStream_t s);
 hipError_t launch_row_qsum(const fnn_hip_weight *w, int32_t *out, hipStream_t s);
 hipError_t launch_qconv2d_i8(const QConvArgs &p, hipStream_t s, int phase);

@@ -134,7 +134,28 @@ __global__ void __launch_bounds__(256) qgemm_i8act_generic_kernel(I8ActArgs p)
     }
 }
 
+// out[i] = q[i]*scale + zp, two roundings as the CPU loop has them (no contraction);
+// values past the payload read as q = 0
+__global__ void __launch_bounds__(256) dequantize_act_kernel(const uint8_t *payload, uint64_t payload_len, float *out, uint64_t n)
+{
+    const float scale = payload_len >= 4 ? reinterpret_cast<const float *>(payload)[0] : 1.0f;
+    const float zp = payload_len >= 8 ? reinterpret_cast<const float *>(payload)[1] : 0.0f;
+    for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (uint64_t)gridDim.x * 256) {
+        const int q = (8 + i < payload_len) ? (int)(int8_t)payload[8 + i] : 0;
+        out[i] = __fadd_rn(__fmul_rn((float)q, scale), zp);
+    }
+}
+
 }  // namespace
+
+hipError_t launch_dequantize_activations(const uint8_t *payload, uint64_t payload_len, float *out, uint64_t n, hipStream_t s)
+{
+    if (n == 0) return hipSuccess;
+    uint64_t blocks = (n + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(dequantize_act_kernel, dim3((unsigned)blocks), dim3(256), 0, s, payload, payload_len, out, n);
+    return hipGetLastError();
+}
 
 hipError_t launch_quantize_activations(const float *x, int64_t numel, float scale, float zp,
                                        uint8_t *payload, float *scratch_partial, hipStream_t s)

@@ -30,7 +30,7 @@ EXPORTED_SYMBOLS = [
     "fnn_hip_device_count", "fnn_hip_create", "fnn_hip_destroy", "fnn_hip_last_error", "fnn_hip_sync",
     "fnn_hip_malloc", "fnn_hip_free", "fnn_hip_upload", "fnn_hip_download",
     "fnn_hip_weight_register", "fnn_hip_weight_lookup", "fnn_hip_weight_release", "fnn_hip_dequant",
-    "fnn_hip_qmatmul", "fnn_hip_quantize_activations", "fnn_hip_qmatmul_i8act", "fnn_hip_qconv2d", "fnn_hip_qconv2d_i8act",
+    "fnn_hip_qmatmul", "fnn_hip_quantize_activations", "fnn_hip_dequantize_activations", "fnn_hip_qmatmul_i8act", "fnn_hip_qconv2d", "fnn_hip_qconv2d_i8act",
     "fnn_hip_timer_start", "fnn_hip_timer_stop", "fnn_hip_probe_stream",
     "fnn_hip_graph_begin", "fnn_hip_graph_end", "fnn_hip_graph_launch", "fnn_hip_graph_destroy",
     "fnn_hip_workspace_epoch",

@@ -118,6 +118,12 @@ int fnn_hip_qmatmul(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *a, i
 int fnn_hip_quantize_activations(fnn_hip_ctx *ctx, const float *x, int64_t numel, float scale,
                                  float zp, uint8_t *payload, int flags);
 
+/* kernel "dequantize_activations", per-tensor form (src/backend/cpu/mod.rs:7009-7088):
+ * out[i] = q[i]*scale + zero for i < n, q = 0 where the payload ends early.  Device pointers;
+ * the call is queued on the context's stream. */
+int fnn_hip_dequantize_activations(fnn_hip_ctx *ctx, const uint8_t *payload, uint64_t payload_len,
+                                   float *out, uint64_t n);
+
 /* "matmul_i8_i8" / "matmul_i4_i8": gemm_cpu_flat_i8_i8x4 / gemm_cpu_flat_i8_i4x8
  * (src/backend/cpu/microkernels/gemm.rs:1641-1975).  acc_out (nullable, [M,N]
  * i32) receives the exact integer accumulators sum q_w*q_a when zp_a == 0. */

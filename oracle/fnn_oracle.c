@@ -896,6 +896,20 @@ void fnn_or_bias_act(float *out, size_t m, size_t n, const float *bias, int act)
 /* I8-activation MatMul                                                       */
 /* ------------------------------------------------------------------------ */
 
+/* "dequantize_activations", per-tensor form (backend/cpu/mod.rs:7063-7086): header scale
+ * (1.0 if absent) and zero (0.0 if absent), out[i] = (q as f32)*scale + zp, q = 0 past the data. */
+void fnn_or_dequantize_activations(const uint8_t *payload, size_t payload_len, float *out, size_t n)
+{
+    float scale = 1.0f, zp = 0.0f;
+    if (payload_len >= 4) memcpy(&scale, payload, 4);
+    if (payload_len >= 8) memcpy(&zp, payload + 4, 4);
+    for (size_t i = 0; i < n; i++) {
+        int8_t q = (8 + i < payload_len) ? (int8_t)payload[8 + i] : 0;
+        volatile float prod = (float)q * scale;   /* two roundings, no contraction */
+        out[i] = prod + zp;
+    }
+}
+
 /* backend/cpu/mod.rs:6987-7007 -- dynamic per-tensor mode: scale = max|x|/127
  * (1 when all zero), zp = 0, q = clamp(round((x - zp)/scale), -128, 127);
  * payload = [scale f32 LE][zp f32 LE][numel x i8]. */

@@ -85,6 +85,8 @@ float fnn_or_act(float x, int act);
 
 /* ---- I8-activation MatMul ------------------------------------------------ */
 void fnn_or_quantize_activations(const float *x, size_t numel, uint8_t *payload);
+/* "dequantize_activations", per-tensor form (backend/cpu/mod.rs:7063-7086) */
+void fnn_or_dequantize_activations(const uint8_t *payload, size_t payload_len, float *out, size_t n);
 void fnn_or_quantize_activations_calibrated(const float *x, size_t numel, float scale, float zp,
                                             uint8_t *payload);
 int  fnn_or_qmatmul_i8act(int dt, const uint32_t *words, size_t n, size_t k,

@@ -88,6 +88,7 @@ def _proto(l):
     l.fnn_or_act.argtypes = [C.c_float, C.c_int]
     l.fnn_or_act.restype = C.c_float
     l.fnn_or_quantize_activations.argtypes = [_f32p, _sz, _u8p]
+    l.fnn_or_dequantize_activations.argtypes = [_u8p, _sz, _f32p, _sz]
     l.fnn_or_quantize_activations_calibrated.argtypes = [_f32p, _sz, C.c_float, C.c_float, _u8p]
     l.fnn_or_qmatmul_i8act.argtypes = [C.c_int, _u32p, _sz, _sz, C.c_void_p, _sz, C.c_void_p, _sz,
                                        _u8p, _sz, _sz, _f32p, C.c_void_p]
@@ -256,6 +257,13 @@ def quantize_activations(x, scale: Optional[float] = None, zp: float = 0.0) -> n
     else:
         lib().fnn_or_quantize_activations_calibrated(x, x.size, scale, zp, payload)
     return payload
+
+
+def dequantize_activations(payload, n: int) -> np.ndarray:
+    payload = np.ascontiguousarray(payload, np.uint8)
+    out = np.zeros(n, np.float32)
+    lib().fnn_or_dequantize_activations(payload, payload.size, out, n)
+    return out
 
 
 def make_payload(scale: float, zp: float, q_i8) -> np.ndarray:

@@ -133,6 +133,36 @@ def test_i8_activation_chain(be, orc, dt, name, calibrated):
     assert_close(be.read_arena(*s_o, np.float32).reshape(m, n), want, 1e-6, name)
 
 
+@pytest.mark.parametrize("calibrated", [False, True])
+def test_quantize_then_dequantize_activations(be, orc, calibrated):
+    """quantize_activations -> dequantize_activations (per-tensor): payload and the f32 values
+    q*scale + zero are bit-identical to the oracle's; an output slice shorter than numel is filled
+    as far as it goes."""
+    rng = np.random.default_rng(19)
+    x = rng.standard_normal(1000).astype(np.float32)
+    a = Arena()
+    s_x, s_q, s_y, s_short = a.take(x.nbytes), a.take(8 + x.size), a.take(x.nbytes), a.take(400)
+    params = [x.size, 0, 0]
+    scale, zp = np.float32(0.021), np.float32(-0.3)
+    if calibrated:
+        params += [int(scale.view(np.uint32)), int(zp.view(np.uint32))]
+    plan = ExecutablePlan(a.top)
+    plan.call_kernel("quantize_activations", [s_x], s_q, params)
+    plan.call_kernel("dequantize_activations", [s_q], s_y, [x.size, 0, 0])
+    plan.call_kernel("dequantize_activations", [s_q], s_short, [x.size, 0, 0])
+    be.allocate_arena(a.top)
+    be.write_arena(s_x[0], x)
+    be.dispatch(plan)
+    payload = orc.quantize_activations(x, float(scale), float(zp)) if calibrated else orc.quantize_activations(x)
+    assert np.array_equal(be.read_arena(*s_q), payload)
+    want = orc.dequantize_activations(payload, x.size)
+    assert np.array_equal(be.read_arena(*s_y, np.float32), want)
+    assert np.array_equal(be.read_arena(*s_short, np.float32), want[:100])
+    with pytest.raises(flib.FnnError) as e:
+        be.dispatch(ExecutablePlan(a.top).call_kernel("dequantize_activations", [s_q], s_y, [x.size, 1, 4]))
+    assert e.value.kind == "UnsupportedOp"
+
+
 @pytest.mark.parametrize("act,code", [("", 0), ("_relu", 1), ("_silu", 3)])
 @pytest.mark.parametrize("wdt,kname", [(flib.DT_I8, "conv2d_i8"), (flib.DT_I4, "conv2d_i4")])
 def test_conv2d_i8_plan(be, orc, act, code, wdt, kname):

@@ -83,3 +83,20 @@ def test_upsample_is_numpy_repeat(orc, sh, sw):
     if sh == sw:
         t = F.interpolate(torch.from_numpy(x), scale_factor=sh, mode="nearest").numpy()
         assert np.array_equal(want, t)
+
+
+def test_dequantize_activations_inverts_the_payload(orc):
+    """q*scale + zp with two f32 roundings (numpy does the same two operations); a quantise ->
+    dequantise round trip stays within half a step; a payload that ends early reads as q = 0."""
+    rng = np.random.default_rng(9)
+    q = rng.integers(-128, 128, 300).astype(np.int8)
+    scale, zp = np.float32(0.0371), np.float32(-0.42)
+    payload = orc.make_payload(scale, zp, q)
+    got = orc.dequantize_activations(payload, 300)
+    assert np.array_equal(got, q.astype(np.float32) * scale + zp)
+    x = rng.standard_normal(500).astype(np.float32)
+    pl = orc.quantize_activations(x)
+    s = pl[:4].view(np.float32)[0]
+    assert np.abs(orc.dequantize_activations(pl, 500) - x).max() <= 0.5 * s * (1 + 1e-6)
+    short = orc.dequantize_activations(payload[:8 + 100], 120)
+    assert np.array_equal(short[:100], got[:100]) and np.all(short[100:] == zp)
