@@ -86,76 +86,90 @@ __global__ void __launch_bounds__(256) i8_matmul_epilogue_kernel(const int32_t *
 }
 
 // ---- conv operand: im2col row (image nn, pixel p) of group g, quantised with the (image, group) scale:
-// q = clamp(round((v - za) * inv), -128, 127)  (packed_conv.rs:149-232).
-// A workgroup owns 64 consecutive rows; thread (row, slot) walks the 16-value chunks slot, slot+4, ...
-// that hold data (neighbouring lanes = neighbouring pixels: the NCHW reads coalesce), the (ic, i, j)
-// tap of a chunk is advanced by carries instead of divisions; all-zero chunks are written in a second sweep.
-constexpr int CONV_CPB = 4;   // 16-value chunks of a row per workgroup (one per thread slot)
+// q = clamp(round((v - za) * inv), -128, 127)  (packed_conv.rs:149-232); for an input that is already int8
+// (X8) the values are taken as they are and padding taps are the integer 0 (packed_conv.rs:69-115).
+// A workgroup owns 64 consecutive rows and CONV_CPB 16-value chunks of them: wave `slot` takes one chunk, so the
+// (channel, tap) geometry of a chunk is the same for the whole wave and neighbouring lanes = neighbouring pixels
+// (the NCHW reads coalesce).  The 16 loads of a chunk go to clamped, always valid addresses and are masked
+// afterwards: no branch sits between them, so all of them are in flight together.
+constexpr int CONV_CPB = 4;   // 16-value chunks of a row per workgroup (one per wave)
 
+template <bool X8>
 __global__ void __launch_bounds__(256) conv_operand_kernel(QConvArgs a, int g, int kk, int64_t kpad, int64_t rows_pad,
                                                            int8_t *a8, int32_t *qsum)
 {
     __shared__ int part[4][64];
     const int tid = threadIdx.x, rr = tid & 63, slot = tid >> 6;
-    const int64_t np = a.ho * a.wo;
+    const uint32_t np = (uint32_t)(a.ho * a.wo), wo = (uint32_t)a.wo;
     const int64_t r = (int64_t)blockIdx.x * 64 + rr;
-    const int64_t rows = a.b * np;
-    const int64_t cg = a.c / a.groups;
+    const int64_t rows = a.b * (int64_t)np;   // < 2^31 (checked on the host)
+    const int cg = (int)(a.c / a.groups);
     const int live_chunks = (kk + 15) / 16, all_chunks = (int)(kpad / 16);
     const bool live = r < rows;
+    const int c = (int)blockIdx.y * CONV_CPB + slot;
     int s = 0;
-    if (r < rows_pad) {
-        const int64_t nn = live ? r / np : 0, p = live ? r % np : 0;
-        const int bg = (int)(nn * a.groups + g);
+    if (r < rows_pad && c < live_chunks) {
+        const uint32_t ru = live ? (uint32_t)r : 0u;
+        const uint32_t nn = ru / np, p = ru - nn * np;
+        const uint32_t oh = p / wo, ow = p - oh * wo;
+        const int bg = (int)nn * a.groups + g;
         const float za = a.actq[bg * 4 + 1], inv = a.actq[bg * 4 + 2];
-        const int64_t x_off = (nn * a.c + g * cg) * a.h * a.w;
+        const int64_t x_off = ((int64_t)nn * a.c + (int64_t)g * cg) * a.h * a.w;
         const float *xg = a.x + x_off;
-        const int8_t *xq = a.x8 ? a.x8 + x_off : nullptr;
-        const int khw = a.kh * a.kw;
+        const int8_t *xq = a.x8 + x_off;
+        const int khw = a.kh * a.kw, hh = (int)a.h, ww = (int)a.w;
         const float qlo = a.wbits == 4 ? -8.0f : -128.0f, qhi = a.wbits == 4 ? 7.0f : 127.0f;
         const int interleaved = a.wbits == 4;   // the 4-bit weight decoder delivers k = 0,2,4,6,1,3,5,7 of each 8
-        const int64_t ih0 = (p / a.wo) * a.stride - a.pad, iw0 = (p % a.wo) * a.stride - a.pad;
-        const int c_end = (int)(blockIdx.y + 1) * CONV_CPB < live_chunks ? (int)(blockIdx.y + 1) * CONV_CPB : live_chunks;
-        for (int c = (int)blockIdx.y * CONV_CPB + slot; c < c_end; c += 4) {
-            uint32_t out[4] = {0, 0, 0, 0};
-            if (live) {
-                int e = c * 16;
-                int ic = e / khw, rem = e % khw;
-                int i = rem / a.kw, j = rem % a.kw;
+        const int ih0 = (int)oh * a.stride - a.pad, iw0 = (int)ow * a.stride - a.pad;
+        // tap geometry of the chunk (the same for every lane of the wave), advanced by carries
+        const int e0 = c * 16;
+        int ic = e0 / khw, rem = e0 - ic * khw;
+        int i = rem / a.kw, j = rem - i * a.kw;
+        int off[16];
+        uint32_t inside = 0;
 #pragma unroll
-                for (int t = 0; t < 16; t++) {
-                    if (e < kk) {
-                        const int64_t ih = ih0 + (int64_t)i * a.dil, iw = iw0 + (int64_t)j * a.dil;
-                        const bool inside = ih >= 0 && ih < a.h && iw >= 0 && iw < a.w;
-                        int qi;
-                        if (xq) {   // already quantised (mod.rs:3878-3905 + im2col_i8, packed_conv.rs:69-115)
-                            qi = inside ? xq[((int64_t)ic * a.h + ih) * a.w + iw] : 0;
-                        } else {
-                            const float v = inside ? xg[((int64_t)ic * a.h + ih) * a.w + iw] : 0.0f;
-                            const float q = roundf((v - za) * inv);
-                            qi = (q != q) ? 0 : (int)fminf(fmaxf(q, qlo), qhi);
-                        }
-                        s += qi;
-                        const int pos = (t & 8) + slot_of(t & 7, interleaved);
-                        out[pos >> 2] |= (uint32_t)(uint8_t)qi << (8 * (pos & 3));
-                    }
-                    e++;
-                    if (++j == a.kw) { j = 0; if (++i == a.kh) { i = 0; ic++; } }
-                }
-            }
-            *reinterpret_cast<uint4 *>(a8 + ((int64_t)(c >> 3) * rows_pad + r) * KB + (c & 7) * 16) = make_uint4(out[0], out[1], out[2], out[3]);
+        for (int t = 0; t < 16; t++) {
+            const int ih = ih0 + i * a.dil, iw = iw0 + j * a.dil;
+            const bool in = live && e0 + t < kk && ih >= 0 && ih < hh && iw >= 0 && iw < ww;
+            off[t] = in ? (ic * hh + ih) * ww + iw : 0;   // < 2^31 (checked on the host)
+            inside |= in ? (1u << t) : 0u;
+            if (++j == a.kw) { j = 0; if (++i == a.kh) { i = 0; ic++; } }
         }
+        float v[16];
+        int v8[16];
+#pragma unroll
+        for (int t = 0; t < 16; t++) {
+            if (X8) v8[t] = xq[off[t]];
+            else v[t] = xg[off[t]];
+        }
+        uint32_t out[4] = {0, 0, 0, 0};
+#pragma unroll
+        for (int t = 0; t < 16; t++) {
+            const bool in = (inside >> t) & 1u;
+            int qi;
+            if (X8) {
+                qi = in ? v8[t] : 0;
+            } else {
+                const float q = roundf(((in ? v[t] : 0.0f) - za) * inv);
+                qi = (q != q) ? 0 : (int)fminf(fmaxf(q, qlo), qhi);
+            }
+            if (!(live && e0 + t < kk)) qi = 0;   // past K, or a padding row of the operand
+            s += qi;
+            const int pos = (t & 8) + slot_of(t & 7, interleaved);
+            out[pos >> 2] |= (uint32_t)(uint8_t)qi << (8 * (pos & 3));
+        }
+        *reinterpret_cast<uint4 *>(a8 + ((int64_t)(c >> 3) * rows_pad + r) * KB + (c & 7) * 16) = make_uint4(out[0], out[1], out[2], out[3]);
     }
     part[slot][rr] = s;
     // chunks past the data: zeros, written with consecutive lanes on consecutive 16-byte pieces of a row
     const int zc = all_chunks - live_chunks;
     if (zc > 0 && blockIdx.y == 0) {
         const int64_t row0 = (int64_t)blockIdx.x * 64;
-        for (int64_t idx = tid; idx < (int64_t)64 * zc; idx += 256) {
+        for (int idx = tid; idx < 64 * zc; idx += 256) {
             const int64_t row = row0 + idx / zc;
-            const int c = live_chunks + (int)(idx % zc);
+            const int cz = live_chunks + idx % zc;
             if (row < rows_pad)
-                *reinterpret_cast<uint4 *>(a8 + ((int64_t)(c >> 3) * rows_pad + row) * KB + (c & 7) * 16) = make_uint4(0, 0, 0, 0);
+                *reinterpret_cast<uint4 *>(a8 + ((int64_t)(cz >> 3) * rows_pad + row) * KB + (cz & 7) * 16) = make_uint4(0, 0, 0, 0);
         }
     }
     __syncthreads();
@@ -379,6 +393,7 @@ int fnn_i8_tiled_conv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, 
     const int64_t np = p.ho * p.wo, rows = p.b * np;
     const int64_t cg = p.c / p.groups, ocg = p.oc / p.groups, kk = cg * p.kh * p.kw;
     if (rows < 1 || rows > (1ll << 28) || kk > (1 << 20) || ocg < 1) return FNN_OK;
+    if (cg * p.h * p.w >= (1ll << 31) || p.ho * p.wo >= (1ll << 31)) return FNN_OK;   // 32-bit offsets inside an image slab
     const int64_t kpad = (kk + KB - 1) / KB * KB;
     const int64_t rows_pad = (rows + 127) / 128 * 128;
     const size_t a_bytes = (size_t)rows_pad * kpad;
@@ -398,7 +413,8 @@ int fnn_i8_tiled_conv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, 
     if (ocg > 65535 * EPI_CH) return FNN_OK;
     for (int g = 0; g < p.groups; g++) {
         const dim3 grid((unsigned)(rows_pad / 64), (unsigned)nq);
-        hipLaunchKernelGGL(conv_operand_kernel, grid, dim3(256), 0, s, p, g, (int)kk, kpad, rows_pad, a8, qsum);
+        if (p.x8) hipLaunchKernelGGL(conv_operand_kernel<true>, grid, dim3(256), 0, s, p, g, (int)kk, kpad, rows_pad, a8, qsum);
+        else hipLaunchKernelGGL(conv_operand_kernel<false>, grid, dim3(256), 0, s, p, g, (int)kk, kpad, rows_pad, a8, qsum);
         hipError_t e = hipGetLastError();
         if (e == hipSuccess)
             e = w->dtype == FNN_DT_I8 ? run_i8_gemm<FNN_DT_I8>(words, kp, w->rows, g * ocg, ocg, a8, rows, rows_pad, kpad, c, ocg, s)
