@@ -94,17 +94,18 @@ __global__ void __launch_bounds__(256) i8_matmul_epilogue_kernel(const int32_t *
 // afterwards: no branch sits between them, so all of them are in flight together.
 constexpr int CONV_CPB = 4;   // 16-value chunks of a row per workgroup (one per wave)
 
-template <bool X8>
+template <bool X8, bool W4>   // X8: int8 input; W4: 4-bit weights (16 activation levels unless X8, interleaved operand)
 __global__ void __launch_bounds__(256) conv_operand_kernel(QConvArgs a, int g, int kk, int64_t kpad, int64_t rows_pad,
                                                            int8_t *a8, int32_t *qsum)
 {
     __shared__ int part[4][64];
-    const int tid = threadIdx.x, rr = tid & 63, slot = tid >> 6;
+    const int tid = threadIdx.x, rr = tid & 63;
+    const int slot = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave index: the chunk geometry stays in scalar registers
     const uint32_t np = (uint32_t)(a.ho * a.wo), wo = (uint32_t)a.wo;
     const int64_t r = (int64_t)blockIdx.x * 64 + rr;
     const int64_t rows = a.b * (int64_t)np;   // < 2^31 (checked on the host)
-    const int cg = (int)(a.c / a.groups);
-    const int live_chunks = (kk + 15) / 16, all_chunks = (int)(kpad / 16);
+    const int cg = (int)a.c / a.groups;
+    const int live_chunks = (kk + 15) / 16;
     const bool live = r < rows;
     const int c = (int)blockIdx.y * CONV_CPB + slot;
     int s = 0;
@@ -118,10 +119,12 @@ __global__ void __launch_bounds__(256) conv_operand_kernel(QConvArgs a, int g, i
         const float *xg = a.x + x_off;
         const int8_t *xq = a.x8 + x_off;
         const int khw = a.kh * a.kw, hh = (int)a.h, ww = (int)a.w;
-        const float qlo = a.wbits == 4 ? -8.0f : -128.0f, qhi = a.wbits == 4 ? 7.0f : 127.0f;
-        const int interleaved = a.wbits == 4;   // the 4-bit weight decoder delivers k = 0,2,4,6,1,3,5,7 of each 8
+        constexpr int qlo = W4 ? -8 : -128, qhi = W4 ? 7 : 127;
+        constexpr int interleaved = W4;   // the 4-bit weight decoder delivers k = 0,2,4,6,1,3,5,7 of each 8
         const int ih0 = (int)oh * a.stride - a.pad, iw0 = (int)ow * a.stride - a.pad;
-        // tap geometry of the chunk (the same for every lane of the wave), advanced by carries
+        // tap geometry of the chunk (the same for every lane of the wave), advanced by carries.
+        // Rows past the last one (r >= rows) compute pixel 0 of image 0: their bytes only reach accumulator
+        // rows and row sums that nothing reads.
         const int e0 = c * 16;
         int ic = e0 / khw, rem = e0 - ic * khw;
         int i = rem / a.kw, j = rem - i * a.kw;
@@ -130,7 +133,7 @@ __global__ void __launch_bounds__(256) conv_operand_kernel(QConvArgs a, int g, i
 #pragma unroll
         for (int t = 0; t < 16; t++) {
             const int ih = ih0 + i * a.dil, iw = iw0 + j * a.dil;
-            const bool in = live && e0 + t < kk && ih >= 0 && ih < hh && iw >= 0 && iw < ww;
+            const bool in = e0 + t < kk && (unsigned)ih < (unsigned)hh && (unsigned)iw < (unsigned)ww;
             off[t] = in ? (ic * hh + ih) * ww + iw : 0;   // < 2^31 (checked on the host)
             inside |= in ? (1u << t) : 0u;
             if (++j == a.kw) { j = 0; if (++i == a.kh) { i = 0; ic++; } }
@@ -150,10 +153,13 @@ __global__ void __launch_bounds__(256) conv_operand_kernel(QConvArgs a, int g, i
             if (X8) {
                 qi = in ? v8[t] : 0;
             } else {
-                const float q = roundf(((in ? v[t] : 0.0f) - za) * inv);
-                qi = (q != q) ? 0 : (int)fminf(fmaxf(q, qlo), qhi);
+                // round half away from zero, then clamp: trunc(x + copysign(0.49999997, x)) equals roundf(x)
+                // after the clamp for every float (the conversion truncates, saturates and maps NaN to 0)
+                const float x = ((in ? v[t] : 0.0f) - za) * inv;
+                qi = (int)(x + __builtin_copysignf(0.49999997f, x));
+                qi = max(qlo, min(qi, qhi));
+                if (!(e0 + t < kk)) qi = 0;   // past K
             }
-            if (!(live && e0 + t < kk)) qi = 0;   // past K, or a padding row of the operand
             s += qi;
             const int pos = (t & 8) + slot_of(t & 7, interleaved);
             out[pos >> 2] |= (uint32_t)(uint8_t)qi << (8 * (pos & 3));
@@ -161,20 +167,13 @@ __global__ void __launch_bounds__(256) conv_operand_kernel(QConvArgs a, int g, i
         *reinterpret_cast<uint4 *>(a8 + ((int64_t)(c >> 3) * rows_pad + r) * KB + (c & 7) * 16) = make_uint4(out[0], out[1], out[2], out[3]);
     }
     part[slot][rr] = s;
-    // chunks past the data: zeros, written with consecutive lanes on consecutive 16-byte pieces of a row
-    const int zc = all_chunks - live_chunks;
-    if (zc > 0 && blockIdx.y == 0) {
-        const int64_t row0 = (int64_t)blockIdx.x * 64;
-        for (int idx = tid; idx < 64 * zc; idx += 256) {
-            const int64_t row = row0 + idx / zc;
-            const int cz = live_chunks + idx % zc;
-            if (row < rows_pad)
-                *reinterpret_cast<uint4 *>(a8 + ((int64_t)(cz >> 3) * rows_pad + row) * KB + (cz & 7) * 16) = make_uint4(0, 0, 0, 0);
-        }
-    }
+    // Chunks past the data (k >= K rounded up to 16) are not written: the weight operand is zero there
+    // (rows end in zero lanes and reads past a row go to the zero chunk), and an int8 product with zero is
+    // zero whatever the activation byte holds.
     __syncthreads();
     // one partial sum per chunk group; the epilogue adds them
-    if (tid < 64 && r < rows_pad) qsum[(int64_t)blockIdx.y * rows_pad + r] = (part[0][tid] + part[1][tid]) + (part[2][tid] + part[3][tid]);
+    const int64_t qrow = (int64_t)blockIdx.x * 64 + tid;
+    if (tid < 64 && qrow < rows_pad) qsum[(int64_t)blockIdx.y * rows_pad + qrow] = (part[0][tid] + part[1][tid]) + (part[2][tid] + part[3][tid]);
 }
 
 // acc = bias_q + sum q_a*q_w; val = acc*sab + zw*(sa*sum q_a) + za*(sw*sum q_w) + (za*zw)*K, left to right,
@@ -413,8 +412,11 @@ int fnn_i8_tiled_conv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, 
     if (ocg > 65535 * EPI_CH) return FNN_OK;
     for (int g = 0; g < p.groups; g++) {
         const dim3 grid((unsigned)(rows_pad / 64), (unsigned)nq);
-        if (p.x8) hipLaunchKernelGGL(conv_operand_kernel<true>, grid, dim3(256), 0, s, p, g, (int)kk, kpad, rows_pad, a8, qsum);
-        else hipLaunchKernelGGL(conv_operand_kernel<false>, grid, dim3(256), 0, s, p, g, (int)kk, kpad, rows_pad, a8, qsum);
+        const bool w4 = p.wbits == 4;
+        if (p.x8 && w4) hipLaunchKernelGGL((conv_operand_kernel<true, true>), grid, dim3(256), 0, s, p, g, (int)kk, kpad, rows_pad, a8, qsum);
+        else if (p.x8) hipLaunchKernelGGL((conv_operand_kernel<true, false>), grid, dim3(256), 0, s, p, g, (int)kk, kpad, rows_pad, a8, qsum);
+        else if (w4) hipLaunchKernelGGL((conv_operand_kernel<false, true>), grid, dim3(256), 0, s, p, g, (int)kk, kpad, rows_pad, a8, qsum);
+        else hipLaunchKernelGGL((conv_operand_kernel<false, false>), grid, dim3(256), 0, s, p, g, (int)kk, kpad, rows_pad, a8, qsum);
         hipError_t e = hipGetLastError();
         if (e == hipSuccess)
             e = w->dtype == FNN_DT_I8 ? run_i8_gemm<FNN_DT_I8>(words, kp, w->rows, g * ocg, ocg, a8, rows, rows_pad, kpad, c, ocg, s)
