@@ -186,58 +186,73 @@ __global__ void __launch_bounds__(256) conv_epilogue_kernel(QConvArgs a, int g, 
 {
     __shared__ float tile[EPI_CH * 65];   // [channel of the block][row], padded
     __shared__ int itile[EPI_CH * 65];    // accumulators incl. bias_q, same shape
+    __shared__ int r_part[4][64];                            // partial sums of q_a per row
     __shared__ float r_sa[64], r_za[64], r_sum[64];          // per row: activation scale / zero of its image, sa * sum q_a
     __shared__ float c_sw[EPI_CH], c_zw[EPI_CH], c_wt[EPI_CH], c_bias[EPI_CH];   // per channel
-    const int64_t np = a.ho * a.wo, rows = a.b * np;
+    const uint32_t np = (uint32_t)(a.ho * a.wo);
+    const int64_t rows = a.b * (int64_t)np;
     const int64_t row0 = (int64_t)blockIdx.x * 64;
     const int f0 = blockIdx.y * EPI_CH;
     const int fb = ocg - f0 < EPI_CH ? ocg - f0 : EPI_CH;   // channels of this block
     const int tid = threadIdx.x;
-    if (tid < 64) {
-        const int64_t r = row0 + tid;
+    {
+        // sum q_a of a row: its nq partial sums are split over the four waves and read four at a time
+        const int part = tid >> 6, rr = tid & 63;
+        const int64_t r = row0 + rr;
+        int qs = 0;
         if (r < rows) {
-            const int bg = (int)((r / np) * a.groups + g);
-            const float sa = a.actq[bg * 4 + 0];
-            int qs = 0;
-            for (int y = 0; y < nq; y++) qs += qsum[(int64_t)y * rows_pad + r];
-            r_sa[tid] = sa;
-            r_za[tid] = a.actq[bg * 4 + 1];
-            r_sum[tid] = sa * (float)qs;
+            const int32_t *q = qsum + r;
+            int y = part;
+            for (; y + 12 < nq; y += 16) {
+                const int q0 = q[(int64_t)y * rows_pad], q1 = q[(int64_t)(y + 4) * rows_pad];
+                const int q2 = q[(int64_t)(y + 8) * rows_pad], q3 = q[(int64_t)(y + 12) * rows_pad];
+                qs += (q0 + q1) + (q2 + q3);
+            }
+            for (; y < nq; y += 4) qs += q[(int64_t)y * rows_pad];
         }
-    } else if (tid < 64 + fb) {
-        const int fl = tid - 64;
-        const int64_t ch = (int64_t)g * ocg + f0 + fl;
-        const float sw = a.scales[ch];
-        c_sw[fl] = sw;
-        c_zw[fl] = a.zeros[ch];
-        c_wt[fl] = sw * (float)a.row_qsum[ch];
-        c_bias[fl] = a.bias ? a.bias[ch] : 0.0f;
+        r_part[part][rr] = qs;
+        if (tid < 64) {
+            if (r < rows) {
+                const int bg = (int)((uint32_t)r / np) * a.groups + g;
+                r_sa[tid] = a.actq[bg * 4 + 0];
+                r_za[tid] = a.actq[bg * 4 + 1];
+            }
+        } else if (tid < 64 + fb) {
+            const int fl = tid - 64;
+            const int64_t ch = (int64_t)g * ocg + f0 + fl;
+            const float sw = a.scales[ch];
+            c_sw[fl] = sw;
+            c_zw[fl] = a.zeros[ch];
+            c_wt[fl] = sw * (float)a.row_qsum[ch];
+            c_bias[fl] = a.bias ? a.bias[ch] : 0.0f;
+        }
     }
     __syncthreads();
-    for (int idx = tid; idx < 64 * fb; idx += 256) {
-        const int rr = idx / fb, fl = idx - rr * fb;
-        const int64_t r = row0 + rr;
-        if (r >= rows) continue;
+    if (tid < 64) r_sum[tid] = r_sa[tid] * (float)((r_part[0][tid] + r_part[1][tid]) + (r_part[2][tid] + r_part[3][tid]));
+    __syncthreads();
+    auto element = [&](int rr, int fl, int acc_in) {
         const float sa = r_sa[rr], za = r_za[rr];
         const float sw = c_sw[fl], zw = c_zw[fl];
         const float sab = sa * sw;
-        int bias_q = 0;
-        if (a.bias && !a.payload_i4) {
-            const float bq = roundf(c_bias[fl] / sab);
-            bias_q = (bq != bq) ? 0 : (bq >= 2147483648.0f ? 2147483647 : (bq <= -2147483648.0f ? (-2147483647 - 1) : (int)bq));
-        }
         int accv;
         float val;
         if (a.payload_i4) {
             // gemm_cpu_flat_i8_i4x8 on the gathered rows, then `+ bias` in f32 (mod.rs:3975-4032);
             // for za != 0 the dot of the dequantised activations is formed from the integer sums
-            accv = c[r * ocg + f0 + fl];
+            accv = acc_in;
             const float dot = (za != 0.0f) ? (float)accv * sa + za * (float)a.row_qsum[(int64_t)g * ocg + f0 + fl] : (float)accv * sa;
             const float input_sum = r_sum[rr] + (float)kk * za;
             val = dot * sw + zw * input_sum;
             if (a.bias) val += c_bias[fl];
         } else {
-            accv = c[r * ocg + f0 + fl] + bias_q;
+            int bias_q = 0;
+            if (a.bias) {
+                // round half away from zero and saturate: trunc(x + copysign(0.49999997, x)) equals roundf(x)
+                // wherever the result fits an i32, and the conversion saturates and maps NaN to 0
+                const float x = c_bias[fl] / sab;
+                bias_q = (int)(x + __builtin_copysignf(0.49999997f, x));
+            }
+            accv = acc_in + bias_q;
             const float zp_prod = za * zw;
             val = (float)accv * sab;
             val = val + zw * r_sum[rr];
@@ -249,16 +264,38 @@ __global__ void __launch_bounds__(256) conv_epilogue_kernel(QConvArgs a, int g, 
         else if (a.act == FNN_ACT_GELU) val = val * 0.5f * (1.0f + tanhf(val * 0.7978846f * (1.0f + 0.044715f * val * val)));
         tile[fl * 65 + rr] = val;
         itile[fl * 65 + rr] = accv;
+    };
+    // consecutive threads on consecutive channels of a row of C (as stored); for the usual block widths the
+    // (row, channel) of a thread comes from shifts and all of its accumulators are requested together
+    if (fb == 32 || fb == 16) {
+        const int sh = fb == 32 ? 5 : 4;
+        const int fl = tid & (fb - 1), rbase = tid >> sh, rstep = 256 >> sh, n_it = 64 / rstep;   // 8 or 4 rows per thread
+        int accs[8];
+#pragma unroll
+        for (int it = 0; it < 8; it++) {
+            const int64_t r = row0 + rbase + it * rstep;
+            accs[it] = (it < n_it && r < rows) ? c[r * ocg + f0 + fl] : 0;
+        }
+#pragma unroll
+        for (int it = 0; it < 8; it++) {
+            const int rr = rbase + it * rstep;
+            if (it < n_it && row0 + rr < rows) element(rr, fl, accs[it]);
+        }
+    } else {
+        for (int idx = tid; idx < 64 * fb; idx += 256) {
+            const int rr = idx / fb, fl = idx - rr * fb;
+            const int64_t r = row0 + rr;
+            if (r < rows) element(rr, fl, c[r * ocg + f0 + fl]);
+        }
     }
     __syncthreads();
     // NCHW stores: consecutive lanes on consecutive pixels
     const int rr = tid & 63;
     const int64_t r = row0 + rr;
     if (r < rows) {
-        const int64_t nn = (rows < (1ll << 31)) ? (int64_t)((unsigned)r / (unsigned)np) : r / np;
-        const int64_t p = r - nn * np;
+        const uint32_t nn = (uint32_t)r / np, p = (uint32_t)r - nn * np;
         for (int fl = tid >> 6; fl < fb; fl += 4) {
-            const int64_t o = (nn * a.oc + (int64_t)g * ocg + f0 + fl) * np + p;
+            const int64_t o = ((int64_t)nn * a.oc + (int64_t)g * ocg + f0 + fl) * np + p;
             a.y[o] = tile[fl * 65 + rr];
             if (a.acc_out) a.acc_out[o] = itile[fl * 65 + rr];
         }
