@@ -134,6 +134,42 @@ __global__ void __launch_bounds__(256) conv_minmax_cover_kernel(QConvArgs a, int
     }
 }
 
+// Every input row and column is reached by some tap (the usual case: stride <= kernel extent) and the slab of the
+// (image, group) is 16-byte aligned: a plain min/max over the contiguous slab, four 16-byte loads in flight per lane.
+__global__ void __launch_bounds__(256) conv_minmax_flat_kernel(QConvArgs a, int pad_touched)
+{
+    __shared__ float smn[4], smx[4];
+    const int bg = blockIdx.y;
+    const int64_t nn = bg / a.groups, g = bg % a.groups;
+    const int64_t cg = a.c / a.groups;
+    const float4 *x4 = reinterpret_cast<const float4 *>(a.x + (nn * a.c + g * cg) * a.h * a.w);
+    const int64_t n4 = (cg * a.h * a.w) >> 2;
+    float mn = pad_touched ? 0.0f : INFINITY, mx = pad_touched ? 0.0f : -INFINITY;
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    for (; i + 3 * stride < n4; i += 4 * stride) {
+        const float4 v0 = x4[i], v1 = x4[i + stride], v2 = x4[i + 2 * stride], v3 = x4[i + 3 * stride];
+        mn = fminf(fminf(fminf(mn, fminf(v0.x, v0.y)), fminf(fminf(v0.z, v0.w), fminf(v1.x, v1.y))),
+                   fminf(fminf(fminf(v1.z, v1.w), fminf(v2.x, v2.y)), fminf(fminf(v2.z, v2.w), fminf(fminf(v3.x, v3.y), fminf(v3.z, v3.w)))));
+        mx = fmaxf(fmaxf(fmaxf(mx, fmaxf(v0.x, v0.y)), fmaxf(fmaxf(v0.z, v0.w), fmaxf(v1.x, v1.y))),
+                   fmaxf(fmaxf(fmaxf(v1.z, v1.w), fmaxf(v2.x, v2.y)), fmaxf(fmaxf(v2.z, v2.w), fmaxf(fmaxf(v3.x, v3.y), fmaxf(v3.z, v3.w)))));
+    }
+    for (; i < n4; i += stride) {
+        const float4 v = x4[i];
+        mn = fminf(fminf(mn, fminf(v.x, v.y)), fminf(v.z, v.w));
+        mx = fmaxf(fmaxf(mx, fmaxf(v.x, v.y)), fmaxf(v.z, v.w));
+    }
+    mn = wave_min(mn);
+    mx = wave_max(mx);
+    if ((threadIdx.x & 63) == 0) { smn[threadIdx.x >> 6] = mn; smx[threadIdx.x >> 6] = mx; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float *dst = a.minmax_partial + ((int64_t)bg * QCONV_NPART + blockIdx.x) * 2;
+        dst[0] = fminf(fminf(smn[0], smn[1]), fminf(smn[2], smn[3]));
+        dst[1] = fmaxf(fmaxf(smx[0], smx[1]), fmaxf(smx[2], smx[3]));
+    }
+}
+
 // 8-bit: scale = range/255 (1 if range <= 0), zero = mn + 128*scale (0 if range <= 0), inv = 1/scale
 // (src/backend/cpu/packed_conv.rs:149-156); 4-bit: scale = range/15 (1 if range <= 0),
 // zero = mn + 8*scale in either case (packed_conv.rs:260-263)
@@ -310,13 +346,28 @@ hipError_t launch_qconv2d_i8(const QConvArgs &p, hipStream_t s, int phase)
                     const int64_t iw = o * p.stride + (int64_t)i * p.dil - p.pad;
                     if (iw < 0 || iw >= p.w) { pad_touched = 1; break; }
                 }
+            // is every input row / column reached by some tap?
+            auto all_reached = [&](int64_t len, int taps, int64_t outs) {
+                for (int64_t pos = 0; pos < len; pos++) {
+                    bool hit = false;
+                    for (int i = 0; i < taps && !hit; i++) {
+                        const int64_t num = pos + p.pad - (int64_t)i * p.dil;
+                        hit = num >= 0 && num % p.stride == 0 && num / p.stride < outs;
+                    }
+                    if (!hit) return false;
+                }
+                return true;
+            };
             const int64_t elems = cg * p.h * p.w;
+            const bool flat = elems % 4 == 0 && (reinterpret_cast<uintptr_t>(p.x) & 15) == 0 &&
+                              all_reached(p.h, p.kh, p.ho) && all_reached(p.w, p.kw, p.wo);
             nparts = (elems + 256 * 4 - 1) / (256 * 4);
             const int64_t cap = 4096 / bg > 32 ? 4096 / bg : 32;   // about 4096 workgroups over all images
             if (nparts > cap) nparts = cap;
             if (nparts > QCONV_NPART) nparts = QCONV_NPART;
             if (nparts < 1) nparts = 1;
-            hipLaunchKernelGGL(conv_minmax_cover_kernel, dim3((unsigned)nparts, (unsigned)bg), dim3(256), (size_t)(p.h + p.w), s, p, pad_touched);
+            if (flat) hipLaunchKernelGGL(conv_minmax_flat_kernel, dim3((unsigned)nparts, (unsigned)bg), dim3(256), 0, s, p, pad_touched);
+            else hipLaunchKernelGGL(conv_minmax_cover_kernel, dim3((unsigned)nparts, (unsigned)bg), dim3(256), (size_t)(p.h + p.w), s, p, pad_touched);
         } else
             hipLaunchKernelGGL(conv_minmax_kernel, dim3((unsigned)nparts, (unsigned)bg), dim3(256), 0, s, p);
         hipLaunchKernelGGL(conv_actq_kernel, dim3((unsigned)bg), dim3(64), 0, s, p, (int)nparts);
