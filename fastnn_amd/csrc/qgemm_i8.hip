@@ -25,27 +25,46 @@ constexpr int KB = 128;   // k-values (= bytes) per stage and activation row
 // position of k inside its group of 8 in the operand: identity, or 0,2,4,6,1,3,5,7 for nibble weights
 __device__ __forceinline__ int slot_of(int j, int interleaved) { return interleaved ? ((j & 1) * 4 + (j >> 1)) : j; }
 
-// ---- I8-activation MatMul operand: payload rows -> tile-major int8 [kpad/128][rows_pad][128] + sum q_a per row
+// ---- I8-activation MatMul operand: payload rows -> tile-major int8 [kpad/128][rows_pad][128] + sum q_a per row.
+// Whole 16-byte chunks of 8-byte aligned rows are moved as two 8-byte loads (a byte permutation for the
+// interleaved operand of the nibble decoders, a 4-way dot with ones for the row sum); ragged ends byte by byte.
+template <bool IL>
 __global__ void __launch_bounds__(256) i8_rows_operand_kernel(const int8_t *qa, int64_t m, int64_t k, int64_t kpad,
-                                                              int64_t rows_pad, int interleaved, int8_t *a8, int32_t *qsum)
+                                                              int64_t rows_pad, int8_t *a8, int32_t *qsum)
 {
     __shared__ int red[4];
     const int64_t r = blockIdx.x;
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const bool rows_aligned = (k % 8 == 0) && ((reinterpret_cast<uintptr_t>(qa) & 7) == 0);
     int s = 0;
     for (int64_t c = tid; c < kpad / 16; c += 256) {   // 16-byte chunk c of the row
         uint32_t out[4] = {0, 0, 0, 0};
         if (r < m) {
-#pragma unroll
-            for (int g8 = 0; g8 < 2; g8++)
-#pragma unroll
-                for (int j = 0; j < 8; j++) {
-                    const int64_t kk = c * 16 + g8 * 8 + j;
-                    const int q = kk < k ? (int)qa[r * k + kk] : 0;
-                    s += q;
-                    const int pos = g8 * 8 + slot_of(j, interleaved);
-                    out[pos >> 2] |= (uint32_t)(uint8_t)q << (8 * (pos & 3));
+            if (rows_aligned && c * 16 + 16 <= k) {
+                const uint2 lo = *reinterpret_cast<const uint2 *>(qa + r * k + c * 16);
+                const uint2 hi = *reinterpret_cast<const uint2 *>(qa + r * k + c * 16 + 8);
+                s += __builtin_amdgcn_sdot4((int)lo.x, 0x01010101, 0, false) + __builtin_amdgcn_sdot4((int)lo.y, 0x01010101, 0, false) +
+                     __builtin_amdgcn_sdot4((int)hi.x, 0x01010101, 0, false) + __builtin_amdgcn_sdot4((int)hi.y, 0x01010101, 0, false);
+                if (IL) {   // operand slot order k = 0,2,4,6,1,3,5,7 of each 8
+                    out[0] = __builtin_amdgcn_perm(lo.y, lo.x, 0x06040200u);
+                    out[1] = __builtin_amdgcn_perm(lo.y, lo.x, 0x07050301u);
+                    out[2] = __builtin_amdgcn_perm(hi.y, hi.x, 0x06040200u);
+                    out[3] = __builtin_amdgcn_perm(hi.y, hi.x, 0x07050301u);
+                } else {
+                    out[0] = lo.x; out[1] = lo.y; out[2] = hi.x; out[3] = hi.y;
                 }
+            } else {
+#pragma unroll
+                for (int g8 = 0; g8 < 2; g8++)
+#pragma unroll
+                    for (int j = 0; j < 8; j++) {
+                        const int64_t kk = c * 16 + g8 * 8 + j;
+                        const int q = kk < k ? (int)qa[r * k + kk] : 0;
+                        s += q;
+                        const int pos = g8 * 8 + slot_of(j, IL);
+                        out[pos >> 2] |= (uint32_t)(uint8_t)q << (8 * (pos & 3));
+                    }
+            }
         }
         const int64_t kb = c >> 3, cc = c & 7;
         *reinterpret_cast<uint4 *>(a8 + (kb * rows_pad + r) * KB + cc * 16) = make_uint4(out[0], out[1], out[2], out[3]);
@@ -63,24 +82,20 @@ __global__ void __launch_bounds__(256) i8_matmul_epilogue_kernel(const int32_t *
                                                                  const int32_t *wsum, const float *scales, const float *zeros,
                                                                  int64_t m, int64_t n, int64_t k, float *out, int32_t *acc_out)
 {
+    // a thread owns one output column (its weight constants stay in registers) and walks rows blockIdx.y, +gridDim.y, ...
     const float sa = reinterpret_cast<const float *>(payload)[0];
     const float za = reinterpret_cast<const float *>(payload)[1];
-    const int64_t total = m * n;
-    for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * 256) {
-        const int64_t r = idx / n, col = idx % n;
+    const int64_t col = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (col >= n) return;
+    const float sw = scales[col], zw = zeros[col];
+    const float zwsum = za * (float)wsum[col];
+    const float kza = (float)k * za;
+    for (int64_t r = blockIdx.y; r < m; r += gridDim.y) {
+        const int64_t idx = r * n + col;
         const int acc = c[idx];
-        const float sw = scales[col], zw = zeros[col];
-        float res;
-        if (za != 0.0f) {
-            const float d = (float)acc * sa + za * (float)wsum[col];
-            const float s = (float)qsum[r] * sa + (float)k * za;
-            res = d * sw + zw * s;
-        } else {
-            const float dot = (float)acc * sa;
-            const float input_sum = (float)qsum[r] * sa + (float)k * za;
-            res = dot * sw + zw * input_sum;
-        }
-        out[idx] = res;
+        const float input_sum = (float)qsum[r] * sa + kza;
+        const float dot = (za != 0.0f) ? (float)acc * sa + zwsum : (float)acc * sa;
+        out[idx] = dot * sw + zw * input_sum;
         if (acc_out) acc_out[idx] = (za != 0.0f) ? 0 : acc;
     }
 }
@@ -403,16 +418,22 @@ int fnn_i8_tiled_matmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w
     int32_t *qsum = (int32_t *)((char *)ws0 + q_off);
     int32_t *c = (int32_t *)ws1;
     const int interleaved = w->dtype == FNN_DT_I4 ? 1 : 0;
-    hipLaunchKernelGGL(i8_rows_operand_kernel, dim3((unsigned)rows_pad), dim3(256), 0, s,
-                       reinterpret_cast<const int8_t *>(p.payload + 8), p.m, p.k, kpad, rows_pad, interleaved, a8, qsum);
+    if (interleaved)
+        hipLaunchKernelGGL(i8_rows_operand_kernel<true>, dim3((unsigned)rows_pad), dim3(256), 0, s,
+                           reinterpret_cast<const int8_t *>(p.payload + 8), p.m, p.k, kpad, rows_pad, a8, qsum);
+    else
+        hipLaunchKernelGGL(i8_rows_operand_kernel<false>, dim3((unsigned)rows_pad), dim3(256), 0, s,
+                           reinterpret_cast<const int8_t *>(p.payload + 8), p.m, p.k, kpad, rows_pad, a8, qsum);
     hipError_t e = hipGetLastError();
     if (e == hipSuccess)
         e = w->dtype == FNN_DT_I8 ? run_i8_gemm<FNN_DT_I8>(words, kp, w->rows, 0, p.n, a8, p.m, rows_pad, kpad, c, p.n, s)
                                   : run_i8_gemm<FNN_DT_I4>(words, kp, w->rows, 0, p.n, a8, p.m, rows_pad, kpad, c, p.n, s);
     if (e == hipSuccess) {
-        int64_t blocks = (p.m * p.n + 255) / 256;
-        if (blocks > 4096) blocks = 4096;
-        hipLaunchKernelGGL(i8_matmul_epilogue_kernel, dim3((unsigned)blocks), dim3(256), 0, s, c, p.payload, qsum, wm->row_qsum,
+        const int64_t colb = (p.n + 255) / 256;
+        int64_t rowb = (4096 + colb - 1) / colb;   // about 4096 workgroups
+        if (rowb > p.m) rowb = p.m;
+        if (rowb > 65535) rowb = 65535;
+        hipLaunchKernelGGL(i8_matmul_epilogue_kernel, dim3((unsigned)colb, (unsigned)rowb), dim3(256), 0, s, c, p.payload, qsum, wm->row_qsum,
                            p.scales, p.zeros, p.m, p.n, p.k, p.out, p.acc_out);
         e = hipGetLastError();
     }
