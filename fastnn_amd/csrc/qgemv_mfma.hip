@@ -9,10 +9,11 @@
 // element and v_mfma_f32_16x16x32_f16 does the multiply-accumulate, so the kernel runs at
 // the speed the weights arrive from HBM.
 //
-// One workgroup = RT*16 weight rows x all of K, 8 waves.  Wave w owns the K slice
+// One workgroup = RT*16 weight rows (RT = 1..3, chosen per shape) x all of K, 8 waves.  Wave w owns the K slice
 // [w*512, (w+1)*512) of every round of 4096 k-values:
 //   0. it requests its slice of the activations, then
-//   1. all of its packed bytes (lane (n,g): row n, 16 bytes per tile);
+//   1. all of its packed bytes (lane (n,g): row n, 16 bytes per tile); scheduling barriers pin this order
+//      (left alone, the compiler sinks most of these requests below step 2 and puts step 3's waits into it);
 //   2. while they are in flight it converts the activations: one group of 8 floats per lane
 //      and row, scaled by a power of two taken from the slice maximum and split into hi + lo
 //      f16 terms.  hi and lo occupy DIFFERENT ROWS of the 16-row MFMA operand (rows 0..M-1
@@ -120,6 +121,8 @@ __global__ void __launch_bounds__(NW * 64) qgemv_mfma_kernel(GemvArgs p)
             xr[m][6] = __uint_as_float(x1.z & keep); xr[m][7] = __uint_as_float(x1.w & keep);
         }
         // ---- 1. the packed bytes: tile t, lane (n,g): words [slice + t*16 + g*4, +4) of row n
+        // (a chunk past the end of the row re-reads the row's last chunk instead: it only meets activations
+        //  that are masked to zero, and the bytes belong to the same output row)
         uint32_t wq[RT][TPW * 4];
         const int64_t wbase = ks * 4 / (8 * SPT);         // word offset of the slice (ks * bits / 32)
 #pragma unroll
@@ -128,11 +131,12 @@ __global__ void __launch_bounds__(NW * 64) qgemv_mfma_kernel(GemvArgs p)
             for (int t = 0; t < TPW; t++) {
                 const int64_t woff = wbase + t * 16 + g * 4;
                 const bool ok = woff + 4 <= kp;           // kp % 4 == 0, kp >= 4
-                const uint32_t keep = ok ? 0xffffffffu : 0u;
                 const uint4 v = *reinterpret_cast<const uint4 *>(wrow[r] + (ok ? woff : kp - 4));
-                wq[r][t * 4 + 0] = v.x & keep; wq[r][t * 4 + 1] = v.y & keep;
-                wq[r][t * 4 + 2] = v.z & keep; wq[r][t * 4 + 3] = v.w & keep;
+                wq[r][t * 4 + 0] = v.x; wq[r][t * 4 + 1] = v.y; wq[r][t * 4 + 2] = v.z; wq[r][t * 4 + 3] = v.w;
             }
+        // every request of the round is issued before anything waits: the activations (oldest requests) are
+        // converted while the packed bytes are still on their way
+        __builtin_amdgcn_sched_barrier(0);
 
         // ---- 2. activation slice -> f16 hi/lo operand rows in this wave's LDS area
         float csc[MM];
@@ -169,9 +173,10 @@ __global__ void __launch_bounds__(NW * 64) qgemv_mfma_kernel(GemvArgs p)
                         __builtin_bit_cast(uint4, f16x8{lo[0], lo[1], lo[2], lo[3], lo[4], lo[5], lo[6], lo[7]});
             }
         }
-        // (only this wave reads these fragments, but the workgroup barrier stays: with the waves kept in
-        //  step the weight stream measures 5-8 % faster for the 8-bit types than without it)
-        __syncthreads();
+        // only this wave reads these fragments, and the LDS serves a wave's requests in order: no workgroup
+        // barrier, just a point the compiler moves no memory operation across
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_sched_barrier(0);   // nothing of step 3 (it waits for the packed bytes) moves up into step 2
 
         // ---- 3. MFMA over the slice: straight-line, one MFMA per step and row tile
         f32x4 acc[RT];
@@ -191,7 +196,7 @@ __global__ void __launch_bounds__(NW * 64) qgemv_mfma_kernel(GemvArgs p)
         for (int r = 0; r < RT; r++)
 #pragma unroll
             for (int i = 0; i < 4; i++) tot[r][i] = fmaf(acc[r][i], csc[i % MM], tot[r][i]);
-        __syncthreads();  // the wave areas are rewritten by the next round
+        __builtin_amdgcn_wave_barrier();  // the wave's own area is rewritten by its next round
     }
 
     // ---- 4. fixed-order reduction over the waves (hi row + lo row), fused epilogue
@@ -221,10 +226,9 @@ __global__ void __launch_bounds__(NW * 64) qgemv_mfma_kernel(GemvArgs p)
     }
 }
 
-template <int DT, bool SINGLE, int NW>
-void launch_mm(const GemvArgs &p, hipStream_t s)
+template <int DT, int RT, bool SINGLE, int NW>
+void launch_rt(const GemvArgs &p, hipStream_t s)
 {
-    constexpr int RT = 1;
     const dim3 grid((unsigned)((p.n + RT * 16 - 1) / (RT * 16))), blk(NW * 64);
     // operand fragments: waves x 16 steps x rows x 4 groups x 16 bytes
     const int mm = p.m <= 1 ? 1 : (p.m <= 2 ? 2 : 4);
@@ -240,6 +244,37 @@ void launch_mm(const GemvArgs &p, hipStream_t s)
             attr_set = true;
         }
         hipLaunchKernelGGL(kern, grid, blk, lds, s, p);
+    }
+}
+
+// Row tiles (of 16 weight rows) per workgroup.  A workgroup converts its activation slice once for all of its
+// row tiles, so more tiles mean less repeated work (the larger M, the more it weighs), but the workgroups
+// should still come in whole rounds over the 256 CUs: cost ~ rounds * (conversion + tiles).
+// C2 (N = 11008): M=2 9.2 -> 8.2 us, M=4 12.3 -> 9.4 us with three tiles; at M=1 one tile is as fast or faster.
+inline int gemv_row_tiles(int64_t n, int64_t m)
+{
+    static const int forced = [] { const char *e = getenv("FNN_GEMV_RT"); return e ? atoi(e) : 0; }();
+    if (forced >= 1 && forced <= 3) return forced;
+    if (m <= 1) return 1;   // one activation row: the conversion is cheap and more workgroups in flight win (measured)
+    const int mm = m <= 2 ? 2 : 4;
+    const double conv = 0.6 + 0.6 * mm;
+    int best = 1;
+    double best_cost = 1e30;
+    for (int rt = 1; rt <= 3; rt++) {
+        const int64_t wgs = (n + rt * 16 - 1) / (rt * 16);
+        const double cost = (double)((wgs + 255) / 256) * (conv + rt);
+        if (cost < best_cost - 1e-9) { best_cost = cost; best = rt; }
+    }
+    return best;
+}
+
+template <int DT, bool SINGLE, int NW>
+void launch_mm(const GemvArgs &p, hipStream_t s)
+{
+    switch (gemv_row_tiles(p.n, p.m)) {
+    case 3: launch_rt<DT, 3, SINGLE, NW>(p, s); break;
+    case 2: launch_rt<DT, 2, SINGLE, NW>(p, s); break;
+    default: launch_rt<DT, 1, SINGLE, NW>(p, s); break;
     }
 }
 
