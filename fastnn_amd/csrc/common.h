@@ -108,6 +108,28 @@ __device__ __forceinline__ float wave_max(float v)
     return v;
 }
 
+// The same reductions with a wave-uniform result (scalar registers): rows of 16 lanes by DPP, then the four row
+// results are read with v_readlane instead of two round trips through the LDS permute path.
+__device__ __forceinline__ float wave_max_uniform(float v)
+{
+    v = fmaxf(v, dpp_f32<0xB1>(v));
+    v = fmaxf(v, dpp_f32<0x4E>(v));
+    v = fmaxf(v, dpp_f32<0x141>(v));
+    v = fmaxf(v, dpp_f32<0x140>(v));
+    const int b = __float_as_int(v);
+    const float r0 = __int_as_float(__builtin_amdgcn_readlane(b, 0)), r1 = __int_as_float(__builtin_amdgcn_readlane(b, 16));
+    const float r2 = __int_as_float(__builtin_amdgcn_readlane(b, 32)), r3 = __int_as_float(__builtin_amdgcn_readlane(b, 48));
+    return fmaxf(fmaxf(r0, r1), fmaxf(r2, r3));
+}
+__device__ __forceinline__ float wave_sum_uniform(float v)
+{
+    v = row16_sum(v);
+    const int b = __float_as_int(v);
+    const float r0 = __int_as_float(__builtin_amdgcn_readlane(b, 0)), r1 = __int_as_float(__builtin_amdgcn_readlane(b, 16));
+    const float r2 = __int_as_float(__builtin_amdgcn_readlane(b, 32)), r3 = __int_as_float(__builtin_amdgcn_readlane(b, 48));
+    return (r0 + r1) + (r2 + r3);
+}
+
 // ---------------------------------------------------------------------------
 // word codecs: raw lane value u(w) as f32, before scale/zero
 // (src/dtypes/{i8x4,i4x8,u8x4,u4x8,f8x4,f8x4r,f4x8}.rs unpack_to_f32).

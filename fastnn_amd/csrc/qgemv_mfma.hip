@@ -151,8 +151,8 @@ __global__ void __launch_bounds__(NW * 64) qgemv_mfma_kernel(GemvArgs p)
                 const float *x = xr[m];
                 float mx = fmaxf(fmaxf(fmaxf(fabsf(x[0]), fabsf(x[1])), fmaxf(fabsf(x[2]), fabsf(x[3]))),
                                  fmaxf(fmaxf(fabsf(x[4]), fabsf(x[5])), fmaxf(fabsf(x[6]), fabsf(x[7]))));
-                mx = wave_max(mx);
-                xsum[m] += wave_sum(((x[0] + x[1]) + (x[2] + x[3])) + ((x[4] + x[5]) + (x[6] + x[7])));
+                mx = wave_max_uniform(mx);
+                xsum[m] += wave_sum_uniform(((x[0] + x[1]) + (x[2] + x[3])) + ((x[4] + x[5]) + (x[6] + x[7])));
                 // power of two e with max*2^-e in [2^14, 2^15), clamped so that 2^-e is finite
                 int ex = (int)((__float_as_uint(mx) >> 23) & 0xff) - 127 - 14;
                 if (mx == 0.0f) ex = 0;
