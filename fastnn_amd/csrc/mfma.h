@@ -13,7 +13,7 @@ bool fnn_ctx_capturing(fnn_hip_ctx *ctx);
 int fnn_tiled_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &p,
                       int flags, bool *handled);
 
-// M <= 4: bandwidth-bound GEMV on the matrix cores (weights requested before anything else).
+// M <= 8: bandwidth-bound GEMV on the matrix cores (weights requested before anything else).
 int fnn_mfma_qgemv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &p,
                    int flags, bool *handled);
 

@@ -1,4 +1,4 @@
-// Bandwidth-bound quantised GEMV on the matrix cores (M <= 4 activation rows) for gfx950.
+// Bandwidth-bound quantised GEMV on the matrix cores (M <= 8 activation rows) for gfx950.
 //
 //   out[m,n] = act((sum_k A[m,k]*u(W[n,k]))*scale[n] + zero[n]*sum_k A[m,k] + bias[n])
 //   (gemm_batch_packed_simd + apply_affine_dot, src/backend/cpu/microkernels/gemm.rs:1982-2088,
@@ -43,7 +43,7 @@ struct GemvArgs {
 
 constexpr int GV_NW = 8;        // waves per workgroup
 constexpr int GV_SLICE = 512;   // k-values per wave and round (64 groups of 8: one per lane)
-constexpr int GV_MMAX = 4;
+constexpr int GV_MMAX = 8;
 
 template <int DT, int RT, int MM, bool SINGLE, int NW>
 __global__ void __launch_bounds__(NW * 64) qgemv_mfma_kernel(GemvArgs p)
@@ -58,7 +58,8 @@ __global__ void __launch_bounds__(NW * 64) qgemv_mfma_kernel(GemvArgs p)
 
     // per wave: [NSTEP][ROWS][4 g] 16-byte operand fragments
     extern __shared__ __attribute__((aligned(16))) uint4 frag_dyn[];  // GV_NW * NSTEP * ROWS * 4
-    __shared__ float red[GV_NW][RT][8][16];
+    constexpr int RROWS = ROWS > 8 ? 16 : 8;   // operand rows kept for the reduction
+    __shared__ float red[GV_NW][RT][RROWS][16];
     __shared__ float xred[GV_NW][GV_MMAX];
 
     const int tid = threadIdx.x;
@@ -195,12 +196,16 @@ __global__ void __launch_bounds__(NW * 64) qgemv_mfma_kernel(GemvArgs p)
 #pragma unroll
         for (int r = 0; r < RT; r++)
 #pragma unroll
-            for (int i = 0; i < 4; i++) tot[r][i] = fmaf(acc[r][i], csc[i % MM], tot[r][i]);
+            for (int i = 0; i < 4; i++) {
+                // eight activation rows: operand row g*4 + i belongs to activation row (g & 1)*4 + i
+                const float cs = MM == 8 ? ((g & 1) ? csc[(4 + i) % MM] : csc[i % MM]) : csc[i % MM];
+                tot[r][i] = fmaf(acc[r][i], cs, tot[r][i]);
+            }
         __builtin_amdgcn_wave_barrier();  // the wave's own area is rewritten by its next round
     }
 
     // ---- 4. fixed-order reduction over the waves (hi row + lo row), fused epilogue
-    if (g < 2) {
+    if (g * 4 < RROWS) {
 #pragma unroll
         for (int r = 0; r < RT; r++)
 #pragma unroll
@@ -231,16 +236,25 @@ void launch_rt(const GemvArgs &p, hipStream_t s)
 {
     const dim3 grid((unsigned)((p.n + RT * 16 - 1) / (RT * 16))), blk(NW * 64);
     // operand fragments: waves x 16 steps x rows x 4 groups x 16 bytes
-    const int mm = p.m <= 1 ? 1 : (p.m <= 2 ? 2 : 4);
+    const int mm = p.m <= 1 ? 1 : (p.m <= 2 ? 2 : (p.m <= 4 ? 4 : 8));
     const size_t lds = (size_t)NW * 16 * (SINGLE ? mm : 2 * mm) * 4 * 16;
     if (mm == 1) hipLaunchKernelGGL((qgemv_mfma_kernel<DT, RT, 1, SINGLE, NW>), grid, blk, lds, s, p);
     else if (mm == 2) hipLaunchKernelGGL((qgemv_mfma_kernel<DT, RT, 2, SINGLE, NW>), grid, blk, lds, s, p);
-    else {
+    else if (mm == 4) {
         auto kern = qgemv_mfma_kernel<DT, RT, 4, SINGLE, NW>;
         static bool attr_set = false;   // up to 64 KiB of dynamic LDS plus the static reduction buffers
         if (!attr_set) {
             (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+            attr_set = true;
+        }
+        hipLaunchKernelGGL(kern, grid, blk, lds, s, p);
+    } else {
+        auto kern = qgemv_mfma_kernel<DT, RT, 8, SINGLE, NW>;
+        static bool attr_set = false;   // up to 128 KiB of dynamic LDS: one workgroup per CU
+        if (!attr_set) {
+            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
             attr_set = true;
         }
         hipLaunchKernelGGL(kern, grid, blk, lds, s, p);
@@ -251,16 +265,17 @@ void launch_rt(const GemvArgs &p, hipStream_t s)
 // row tiles, so more tiles mean less repeated work (the larger M, the more it weighs), but the workgroups
 // should still come in whole rounds over the 256 CUs: cost ~ rounds * (conversion + tiles).
 // C2 (N = 11008): M=2 9.2 -> 8.2 us, M=4 12.3 -> 9.4 us with three tiles; at M=1 one tile is as fast or faster.
-inline int gemv_row_tiles(int64_t n, int64_t m)
+inline int gemv_row_tiles(int64_t n, int64_t m, int nw)
 {
     static const int forced = [] { const char *e = getenv("FNN_GEMV_RT"); return e ? atoi(e) : 0; }();
-    if (forced >= 1 && forced <= 3) return forced;
     if (m <= 1) return 1;   // one activation row: the conversion is cheap and more workgroups in flight win (measured)
-    const int mm = m <= 2 ? 2 : 4;
+    const int mm = m <= 2 ? 2 : (m <= 4 ? 4 : 8);
+    if (forced >= 1 && forced <= 3 && forced * mm * 16 <= nw * 64) return forced;
     const double conv = 0.6 + 0.6 * mm;
     int best = 1;
     double best_cost = 1e30;
     for (int rt = 1; rt <= 3; rt++) {
+        if (rt * mm * 16 > nw * 64) break;   // one output per thread in the epilogue
         const int64_t wgs = (n + rt * 16 - 1) / (rt * 16);
         const double cost = (double)((wgs + 255) / 256) * (conv + rt);
         if (cost < best_cost - 1e-9) { best_cost = cost; best = rt; }
@@ -271,7 +286,7 @@ inline int gemv_row_tiles(int64_t n, int64_t m)
 template <int DT, bool SINGLE, int NW>
 void launch_mm(const GemvArgs &p, hipStream_t s)
 {
-    switch (gemv_row_tiles(p.n, p.m)) {
+    switch (gemv_row_tiles(p.n, p.m, NW)) {
     case 3: launch_rt<DT, 3, SINGLE, NW>(p, s); break;
     case 2: launch_rt<DT, 2, SINGLE, NW>(p, s); break;
     default: launch_rt<DT, 1, SINGLE, NW>(p, s); break;
