@@ -17,7 +17,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libfastnn_hip.so")
 
-HIP_SOURCES = ["api.hip", "qgemv.hip", "qgemm_generic.hip", "qgemm_tiled.hip", "qgemm_i8.hip", "qgemv_mfma.hip", "i8act.hip", "qconv.hip", "qconv_float.hip", "probe.hip", "eltwise.hip"]
+HIP_SOURCES = ["api.hip", "qgemv.hip", "qgemm_generic.hip", "qgemm_tiled.hip", "qgemm_i8.hip", "qgemv_mfma.hip", "qgemv_rows16.hip", "i8act.hip", "qconv.hip", "qconv_float.hip", "probe.hip", "eltwise.hip"]
 HOST_SOURCES = ["quantize_host.cpp", "hip_backend.cpp"]
 
 # -ffp-contract=off: the integer/quantisation formulas must evaluate exactly as written;

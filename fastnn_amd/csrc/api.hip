@@ -440,6 +440,10 @@ int fnn_hip_qmatmul(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *a, i
             if (rc) return rc;
         }
         if (!handled) {
+            int rc = fnn_mfma_rows16(ctx, ctx->stream, w, p, flags, &handled);
+            if (rc) return rc;
+        }
+        if (!handled) {
             int rc = fnn_tiled_qmatmul(ctx, ctx->stream, w, p, flags, &handled);
             if (rc) return rc;
         }

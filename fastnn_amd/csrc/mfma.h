@@ -17,6 +17,11 @@ int fnn_tiled_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, 
 int fnn_mfma_qgemv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &p,
                    int flags, bool *handled);
 
+// 9 <= M <= 16: the same organisation with the 16 activation rows as the MFMA operand rows, loaded straight
+// into registers (no preparation or reduction launch).
+int fnn_mfma_rows16(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &p,
+                    int flags, bool *handled);
+
 // I8 activations x I8/I4 weights and the quantised Conv2d on int8 MFMA tiles with i32 accumulators.
 int fnn_i8_tiled_matmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const I8ActArgs &p, bool *handled);
 // p.actq must already hold the (image, group) activation scales.
