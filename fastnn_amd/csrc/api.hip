@@ -632,17 +632,27 @@ int fnn_hip_qconv2d(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *x, i
     p.b = b; p.c = c; p.h = h; p.w = wd; p.oc = oc; p.ho = ho; p.wo = wo; p.kp = w->kp;
     p.kh = kh; p.kw = kw; p.stride = stride; p.pad = pad; p.dil = dil; p.groups = groups; p.act = act;
     p.wbits = w->dtype == FNN_DT_I4 ? 4 : 8;
-    p.x8 = nullptr; p.payload_i4 = 0;
+    p.x8 = nullptr; p.payload_i4 = 0; p.nparts = 0;
     if (flags & FNN_FLAG_FORCE_GENERIC) {
-        HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qconv2d_i8(p, ctx->stream, 0));
+        HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qconv2d_i8(p, ctx->stream, 0, nullptr));
     } else {
-        HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qconv2d_i8(p, ctx->stream, 1));
+        // range scan; the scales are then formed by the operand kernel itself (one launch less) when a workgroup's
+        // 64 rows touch at most two images, else by the small kernel of their own
+        int nparts = 0;
+        HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qconv2d_i8(p, ctx->stream, 3, &nparts));
+        const int64_t kk_g = (c / groups) * kh * kw;
+        const int64_t operand_wgs = ((b * ho * wo + 63) / 64) * (((kk_g + 15) / 16 + 3) / 4);
+        const bool fused_scales = ho * wo >= 64 && nparts <= QCONV_NPART && operand_wgs <= 8192;   // many workgroups: cheaper once
+        if (fused_scales) p.nparts = nparts;
+        else HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qconv2d_i8(p, ctx->stream, 4, &nparts));
         bool handled = false;
-        if (b * groups > 0 && ho * wo > 0) {
-            int rc2 = fnn_i8_tiled_conv(ctx, ctx->stream, w, p, &handled);
-            if (rc2) return rc2;
+        int rc2 = fnn_i8_tiled_conv(ctx, ctx->stream, w, p, &handled);
+        if (rc2) return rc2;
+        if (!handled) {
+            if (fused_scales) HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qconv2d_i8(p, ctx->stream, 4, &nparts));
+            p.nparts = 0;
+            HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qconv2d_i8(p, ctx->stream, 2, nullptr));
         }
-        if (!handled) HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qconv2d_i8(p, ctx->stream, 2));
     }
     if (!dev) {
         HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(y, dy, yout, hipMemcpyDeviceToHost, ctx->stream));
@@ -715,7 +725,7 @@ int fnn_hip_qconv2d_i8act(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const uint8
     p.kh = kh; p.kw = kw; p.stride = stride; p.pad = pad; p.dil = dil; p.groups = groups; p.act = act;
     p.wbits = w->dtype == FNN_DT_I4 ? 4 : 8;
     p.x8 = reinterpret_cast<const int8_t *>(dp + 8);
-    p.payload_i4 = w->dtype == FNN_DT_I4;
+    p.payload_i4 = w->dtype == FNN_DT_I4; p.nparts = 0;
     HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_conv_actq_from_payload(dp, p.actq, (int)(b * groups), ctx->stream));
     bool handled = false;
     if ((rc = fnn_i8_tiled_conv(ctx, ctx->stream, w, p, &handled))) return rc;

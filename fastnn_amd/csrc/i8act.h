@@ -29,6 +29,8 @@ struct QConvArgs {
     const int8_t *x8;        // non-null: the input is already int8 [B,C,H,W] (an activation payload's data)
                              // with one (scale, zero) for the whole tensor in actq; padding taps are the integer 0
     int payload_i4;          // with x8 and I4 weights: the matmul_i4_i8 formula and a float bias
+    int nparts;              // > 0: actq is not filled yet; the operand kernel reduces the nparts partial ranges of
+                             // its images itself (and stores actq for the epilogue); 0: actq holds the scales
 };
 constexpr int QCONV_NPART = 512;
 
@@ -37,6 +39,8 @@ hipError_t launch_quantize_activations(const float *x, int64_t numel, float scal
 hipError_t launch_dequantize_activations(const uint8_t *payload, uint64_t payload_len, float *out, uint64_t n, hipStream_t s);
 hipError_t launch_qgemm_i8act_generic(int dtype, const I8ActArgs &p, hipStream_t s);
 hipError_t launch_row_qsum(const fnn_hip_weight *w, int32_t *out, hipStream_t s);
-hipError_t launch_qconv2d_i8(const QConvArgs &p, hipStream_t s, int phase);
+// phase 0: everything with the direct kernel; 1: range scan + scales; 2: the direct kernel only (scales present);
+// 3: range scan only (*nparts = partial ranges per image and group); 4: scales from *nparts partial ranges
+hipError_t launch_qconv2d_i8(const QConvArgs &p, hipStream_t s, int phase, int *nparts);
 // actq[i] = (scale, zero, 0, 0) of an activation payload's header, for i < nbg
 hipError_t launch_conv_actq_from_payload(const uint8_t *payload, float *actq, int nbg, hipStream_t s);

@@ -321,8 +321,7 @@ hipError_t launch_conv_actq_from_payload(const uint8_t *payload, float *actq, in
     return hipGetLastError();
 }
 
-// phase 0: everything; 1: the (image, group) activation scales only; 2: the direct kernel only (scales present)
-hipError_t launch_qconv2d_i8(const QConvArgs &p, hipStream_t s, int phase)
+hipError_t launch_qconv2d_i8(const QConvArgs &p, hipStream_t s, int phase, int *nparts_io)
 {
     const int64_t bg = p.b * p.groups;
     const int64_t cg = p.c / p.groups, ocg = p.oc / p.groups;
@@ -332,6 +331,10 @@ hipError_t launch_qconv2d_i8(const QConvArgs &p, hipStream_t s, int phase)
     int64_t nparts = (total + 256 * 16 - 1) / (256 * 16);
     if (nparts > QCONV_NPART) nparts = QCONV_NPART;
     if (nparts < 1) nparts = 1;
+    if (phase == 4) {
+        hipLaunchKernelGGL(conv_actq_kernel, dim3((unsigned)bg), dim3(64), 0, s, p, nparts_io ? *nparts_io : 1);
+        return hipGetLastError();
+    }
     if (phase != 2) {
         if (p.h + p.w <= 32768 && cg > 0) {
             // does any tap fall into the padding?  (rows and columns separately)
@@ -370,9 +373,10 @@ hipError_t launch_qconv2d_i8(const QConvArgs &p, hipStream_t s, int phase)
             else hipLaunchKernelGGL(conv_minmax_cover_kernel, dim3((unsigned)nparts, (unsigned)bg), dim3(256), (size_t)(p.h + p.w), s, p, pad_touched);
         } else
             hipLaunchKernelGGL(conv_minmax_kernel, dim3((unsigned)nparts, (unsigned)bg), dim3(256), 0, s, p);
-        hipLaunchKernelGGL(conv_actq_kernel, dim3((unsigned)bg), dim3(64), 0, s, p, (int)nparts);
+        if (nparts_io) *nparts_io = (int)nparts;
+        if (phase != 3) hipLaunchKernelGGL(conv_actq_kernel, dim3((unsigned)bg), dim3(64), 0, s, p, (int)nparts);
     }
-    if (phase == 1) return hipGetLastError();
+    if (phase == 1 || phase == 3) return hipGetLastError();
     dim3 grid((unsigned)((np + 255) / 256), (unsigned)((ocg + CONV_OCT - 1) / CONV_OCT), (unsigned)bg);
     hipLaunchKernelGGL(conv_i8_kernel, grid, dim3(256), 0, s, p);
     return hipGetLastError();

@@ -123,13 +123,65 @@ __global__ void __launch_bounds__(256) conv_operand_kernel(QConvArgs a, int g, i
     const int live_chunks = (kk + 15) / 16;
     const bool live = r < rows;
     const int c = (int)blockIdx.y * CONV_CPB + slot;
+    // Scales not formed yet (a.nparts > 0): every workgroup reduces the partial ranges of the (at most two) images
+    // its 64 rows belong to and derives scale, zero and 1/scale exactly as conv_actq_kernel does; the workgroups of
+    // the first chunk group also store them for the epilogue.
+    __shared__ float s_mm[2][2][4];
+    __shared__ float s_q[2][3];
+    const int64_t r_first = (int64_t)blockIdx.x * 64;
+    const bool own_scales = !X8 && a.nparts > 0 && r_first < rows;
+    int bg_a = 0;
+    if (own_scales) {
+        const int64_t r_last = r_first + 63 < rows ? r_first + 63 : rows - 1;
+        bg_a = (int)((uint32_t)r_first / np) * a.groups + g;
+        const int bg_b = (int)((uint32_t)r_last / np) * a.groups + g;
+        const int nimg = bg_b != bg_a ? 2 : 1;
+        for (int w = 0; w < nimg; w++) {
+            const float *part = a.minmax_partial + (int64_t)(w ? bg_b : bg_a) * QCONV_NPART * 2;
+            float mn = INFINITY, mx = -INFINITY;
+            for (int i = tid; i < a.nparts; i += 256) {
+                mn = fminf(mn, part[i * 2]);
+                mx = fmaxf(mx, part[i * 2 + 1]);
+            }
+            mn = wave_min(mn);
+            mx = wave_max(mx);
+            if (rr == 0) { s_mm[w][0][tid >> 6] = mn; s_mm[w][1][tid >> 6] = mx; }
+        }
+        __syncthreads();
+        if (tid < nimg) {
+            const float mn = fminf(fminf(s_mm[tid][0][0], s_mm[tid][0][1]), fminf(s_mm[tid][0][2], s_mm[tid][0][3]));
+            const float mx = fmaxf(fmaxf(s_mm[tid][1][0], s_mm[tid][1][1]), fmaxf(s_mm[tid][1][2], s_mm[tid][1][3]));
+            const float range = mx - mn;
+            float scale, zero;
+            if (W4) {
+                scale = (range > 0.0f) ? range / 15.0f : 1.0f;
+                zero = mn + 8.0f * scale;
+            } else {
+                scale = (range > 0.0f) ? range / 255.0f : 1.0f;
+                zero = (range > 0.0f) ? mn + 128.0f * scale : 0.0f;
+            }
+            const float inv = (scale != 0.0f) ? 1.0f / scale : 0.0f;
+            s_q[tid][0] = scale; s_q[tid][1] = zero; s_q[tid][2] = inv;
+            if (blockIdx.y == 0) {
+                float *dst = a.actq + (tid ? bg_b : bg_a) * 4;
+                dst[0] = scale; dst[1] = zero; dst[2] = inv; dst[3] = 0.0f;
+            }
+        }
+        __syncthreads();
+    }
     int s = 0;
     if (r < rows_pad && c < live_chunks) {
         const uint32_t ru = live ? (uint32_t)r : 0u;
         const uint32_t nn = ru / np, p = ru - nn * np;
         const uint32_t oh = p / wo, ow = p - oh * wo;
         const int bg = (int)nn * a.groups + g;
-        const float za = a.actq[bg * 4 + 1], inv = a.actq[bg * 4 + 2];
+        float za, inv;
+        if (X8 || a.nparts <= 0) {
+            za = a.actq[bg * 4 + 1]; inv = a.actq[bg * 4 + 2];
+        } else {
+            const int w = (own_scales && bg != bg_a) ? 1 : 0;
+            za = own_scales ? s_q[w][1] : 0.0f; inv = own_scales ? s_q[w][2] : 0.0f;
+        }
         const int64_t x_off = ((int64_t)nn * a.c + (int64_t)g * cg) * a.h * a.w;
         const float *xg = a.x + x_off;
         const int8_t *xq = a.x8 + x_off;
