@@ -288,8 +288,11 @@ int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QM
     const int64_t meff = precise ? (M + 15) / 16 * 32 : (M + 31) / 32 * 32;
     // tile shape by effective row count
     // 0: 128x128 (2x2 waves of 64x64), 1: 64x128 (4 waves of 64x32), 2: 32x128 (4 waves of 32x32)
+    // (measured: with at most 128 tiles of 128x128 the 64-row tiles win, they need a smaller K split or none:
+    //  C1 M=64 24.1 -> 20.6 us, M=256 39.2 -> 36.7 us, FP8 2048->8192 M=64 23.5 -> 19.9 us; the dense codebook
+    //  operand, swept twice, is the exception)
     int cfg;
-    if (meff > 64) cfg = 0;
+    if (meff > 64) cfg = (!dense && ((meff + 127) / 128) * ((N + 127) / 128) <= 128) ? 1 : 0;
     else if (meff == 64) cfg = 1;
     else cfg = 2;
     static const int env_cfg = env_int("FNN_TILE_CFG", -1);
@@ -319,7 +322,7 @@ int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QM
         const double r = (double)base * sp / 256.0;
         const double wgs = r <= 1.0 ? 1.5 : (double)(int64_t)(r + 0.95);
         const double cost = per * t_stage * wgs + (sp > 1 ? 2.0 * sp * part_us : 0.0);
-        if (cost < best - 1e-9) { best = cost; splits = sp; }
+        if (cost < best * 0.995) { best = cost; splits = sp; }   // on a tie the coarser split wins
     }
     if (env_split > 0) splits = env_split;
     if (splits > iters / 4) splits = iters / 4 > 0 ? iters / 4 : 1;
