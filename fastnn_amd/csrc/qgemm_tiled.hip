@@ -320,7 +320,9 @@ int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QM
     for (int sp = 1; sp <= 32 && sp <= (iters / 4 > 0 ? iters / 4 : 1); sp++) {
         const int per = (iters + sp - 1) / sp;
         const double r = (double)base * sp / 256.0;
-        const double wgs = r <= 1.0 ? 1.5 : (double)(int64_t)(r + 0.95);
+        // (the dense operand's 128x128 stages take 96 KB of LDS: one workgroup per CU, rounds do not overlap)
+        const double wgs = (dense && cfg == 0) ? 1.5 * (double)(int64_t)(r + 0.999)
+                                               : (r <= 1.0 ? 1.5 : (double)(int64_t)(r + 0.95));
         const double cost = per * t_stage * wgs + (sp > 1 ? 2.0 * sp * part_us : 0.0);
         if (cost < best * 0.995) { best = cost; splits = sp; }   // on a tie the coarser split wins
     }
