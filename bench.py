@@ -526,7 +526,7 @@ def gemm_leg(ctx, flib, handles, ring, k, n, dbias, act, a_seed, m2):
         for i in range(ring):
             ctx.qmatmul_dev(handles[i], da2.ptr, m2, dout2.ptr, dbias.ptr if dbias else 0, act, f)
         ctx.sync()
-        reps = max(ring, 40)
+        reps = max(ring, 200)
         ctx.timer_start()
         for i in range(reps):
             ctx.qmatmul_dev(handles[i % ring], da2.ptr, m2, dout2.ptr, dbias.ptr if dbias else 0, act, f)
