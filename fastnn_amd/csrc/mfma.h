@@ -13,6 +13,9 @@ bool fnn_ctx_capturing(fnn_hip_ctx *ctx);
 int fnn_tiled_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &p,
                       int flags, bool *handled);
 
+// single-f16 activation mode: mean lane value per weight row (null for types whose lanes have zero mean)
+int fnn_row_means(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const float **umean);
+
 // M <= 8: bandwidth-bound GEMV on the matrix cores (weights requested before anything else).
 int fnn_mfma_qgemv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &p,
                    int flags, bool *handled);

@@ -491,6 +491,32 @@ int run_tiled_codebook(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w,
 
 }  // namespace
 
+// Mean lane value per weight row, built on the first single-f16 use of a weight whose lanes have a non-zero mean
+// (asymmetric integer types, FP4): *umean stays null for the other types.
+int fnn_row_means(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const float **umean)
+{
+    *umean = nullptr;
+    const int dt = w->dtype;
+    if (dt != FNN_DT_I8 && dt != FNN_DT_I4 && dt != FNN_DT_U8 && dt != FNN_DT_U4 && dt != FNN_DT_F4) return FNN_OK;
+    fnn_hip_weight *wm = const_cast<fnn_hip_weight *>(w);
+    if (!wm->umean) {
+        if (fnn_ctx_capturing(ctx)) return fnn_ctx_fail(ctx, FNN_ERR_MEMORY, "first single-pass use of a weight during graph capture");
+        if (hipMalloc((void **)&wm->umean, (size_t)w->rows * 4 + 64) != hipSuccess)
+            return fnn_ctx_fail(ctx, FNN_ERR_MEMORY, "out of device memory (row means)");
+        hipError_t e;
+        switch (dt) {
+        case FNN_DT_I8: e = launch_umean<FNN_DT_I8>(w, wm->umean, s); break;
+        case FNN_DT_I4: e = launch_umean<FNN_DT_I4>(w, wm->umean, s); break;
+        case FNN_DT_U8: e = launch_umean<FNN_DT_U8>(w, wm->umean, s); break;
+        case FNN_DT_U4: e = launch_umean<FNN_DT_U4>(w, wm->umean, s); break;
+        default: e = launch_umean<FNN_DT_F4>(w, wm->umean, s); break;
+        }
+        if (e != hipSuccess) return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, hipGetErrorString(e));
+    }
+    *umean = wm->umean;
+    return FNN_OK;
+}
+
 int fnn_tiled_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &q, int flags, bool *handled)
 {
     *handled = false;

@@ -36,6 +36,7 @@ using namespace dech;
 struct GemvArgs {
     const uint32_t *words;
     const float *scales, *zeros, *a, *bias;
+    const float *umean;   // single-f16 mode: mean lane value per weight row, or null
     float *out;
     int64_t m, n, k, kp;
     int act;
@@ -61,6 +62,7 @@ __global__ void __launch_bounds__(NW * 64) qgemv_mfma_kernel(GemvArgs p)
     constexpr int RROWS = ROWS > 8 ? 16 : 8;   // operand rows kept for the reduction
     __shared__ float red[GV_NW][RT][RROWS][16];
     __shared__ float xred[GV_NW][GV_MMAX];
+    __shared__ float ered[GV_NW][GV_MMAX];   // single-f16 mode: sum_k (hi - x) per activation row
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -89,13 +91,14 @@ __global__ void __launch_bounds__(NW * 64) qgemv_mfma_kernel(GemvArgs p)
     if (e_n > N - 1) e_n = N - 1;
     const float e_scale = p.scales[e_n], e_zero = p.zeros[e_n];
     const float e_bias = p.bias ? p.bias[e_n] : 0.0f;
+    const float e_umean = (SINGLE && p.umean) ? p.umean[e_n] : 0.0f;
 
     f32x4 tot[RT];
 #pragma unroll
     for (int r = 0; r < RT; r++) tot[r] = f32x4{0.f, 0.f, 0.f, 0.f};
-    float xsum[MM];
+    float xsum[MM], xerr[MM];
 #pragma unroll
-    for (int m = 0; m < MM; m++) xsum[m] = 0.0f;
+    for (int m = 0; m < MM; m++) xsum[m] = xerr[m] = 0.0f;
 
     // operand fragment this lane reads at step s: row min(ln, ROWS-1), group g
     const int rsel = ln < ROWS ? ln : ROWS - 1;
@@ -161,13 +164,18 @@ __global__ void __launch_bounds__(NW * 64) qgemv_mfma_kernel(GemvArgs p)
                 const float inv = __uint_as_float((uint32_t)(127 - ex) << 23);
                 csc[m] = __uint_as_float((uint32_t)(127 + ex) << 23);
                 _Float16 hi[8], lo[8];
+                float rerr = 0.0f;
 #pragma unroll
                 for (int j = 0; j < 8; j++) {
                     const int src = D::INTERLEAVED ? ((j >> 1) + 4 * (j & 1)) : j;
                     const float v = x[src] * inv;
                     hi[j] = (_Float16)v;
                     lo[j] = (_Float16)(v - (float)hi[j]);
+                    if (SINGLE) rerr += (float)hi[j] - v;
                 }
+                // single-f16 mode: the rounding of the row, in the units of x, for the first-order correction
+                // dot -= mean_k u[n,k] * sum_k (hi - x)
+                if (SINGLE) xerr[m] += csc[m] * wave_sum_uniform(rerr);
                 fw[slot + m * 4] = __builtin_bit_cast(uint4, f16x8{hi[0], hi[1], hi[2], hi[3], hi[4], hi[5], hi[6], hi[7]});
                 if (!SINGLE)
                     fw[slot + (MM + m) * 4] =
@@ -213,11 +221,14 @@ __global__ void __launch_bounds__(NW * 64) qgemv_mfma_kernel(GemvArgs p)
     }
     if (lane == 0) {
 #pragma unroll
-        for (int m = 0; m < GV_MMAX; m++) xred[wv][m] = m < MM ? xsum[m < MM ? m : 0] : 0.0f;
+        for (int m = 0; m < GV_MMAX; m++) {
+            xred[wv][m] = m < MM ? xsum[m < MM ? m : 0] : 0.0f;
+            ered[wv][m] = m < MM ? xerr[m < MM ? m : 0] : 0.0f;
+        }
     }
     __syncthreads();
     if (e_ok) {  // RT*MM*16 <= 128 outputs: one per thread
-        float dot = 0.0f, xs = 0.0f;
+        float dot = 0.0f, xs = 0.0f, es = 0.0f;
 #pragma unroll
         for (int w = 0; w < GV_NW; w++) {   // all reads issued together; absent waves add 0
             const int ws = w < nw ? w : 0;
@@ -225,7 +236,9 @@ __global__ void __launch_bounds__(NW * 64) qgemv_mfma_kernel(GemvArgs p)
             if (!SINGLE) v += red[ws][e_r][MM + e_m][e_c];
             dot += w < nw ? v : 0.0f;
             xs += w < nw ? xred[ws][e_m] : 0.0f;
+            if (SINGLE) es += w < nw ? ered[ws][e_m] : 0.0f;
         }
+        if (SINGLE) dot = dot - e_umean * es;
         const float v = dot * e_scale + e_zero * xs + e_bias;   // fnn_epilogue with preloaded operands
         p.out[(int64_t)e_m * N + e_n] = fnn_activation(p.bias ? v : dot * e_scale + e_zero * xs, p.act);
     }
@@ -318,6 +331,11 @@ int fnn_mfma_qgemv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, con
     p.words = q.words; p.scales = q.scales; p.zeros = q.zeros; p.a = q.a; p.bias = q.bias; p.out = q.out;
     p.m = q.m; p.n = q.n; p.k = q.k; p.kp = q.kp; p.act = q.act;
     const bool single = (flags & FNN_FLAG_ACT_F16_SINGLE) != 0;
+    p.umean = nullptr;
+    if (single) {
+        int rc = fnn_row_means(ctx, s, w, &p.umean);
+        if (rc) return rc;
+    }
     hipError_t e;
     switch (w->dtype) {
     case FNN_DT_I8: e = launch_gemv<FNN_DT_I8>(p, single, s); break;

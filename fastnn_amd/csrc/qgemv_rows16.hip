@@ -32,6 +32,7 @@ using namespace dech;
 struct Rows16Args {
     const uint32_t *words;
     const float *scales, *zeros, *a, *bias;
+    const float *umean;   // single-f16 mode: mean lane value per weight row, or null
     float *out;
     int64_t m, n, k, kp;
     int act;
@@ -57,6 +58,7 @@ __global__ void __launch_bounds__(NW * 64) qgemv_rows16_kernel(Rows16Args p)
     __shared__ float red[NW][RT][16][16];
     __shared__ float xred[NW][16];
     __shared__ float cscs[NW][16];
+    __shared__ float ered[NW][16];   // single-f16 mode: sum_k (hi - x) per activation row
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -94,9 +96,9 @@ __global__ void __launch_bounds__(NW * 64) qgemv_rows16_kernel(Rows16Args p)
     f32x4 tot[RT];
 #pragma unroll
     for (int r = 0; r < RT; r++) tot[r] = f32x4{0.f, 0.f, 0.f, 0.f};
-    float xsum[PPT];
+    float xsum[PPT], xerr[PPT];
 #pragma unroll
-    for (int j = 0; j < PPT; j++) xsum[j] = 0.0f;
+    for (int j = 0; j < PPT; j++) xsum[j] = xerr[j] = 0.0f;
 
     const int64_t round_k = (int64_t)NW * R16_SLICE;
     for (int64_t k0 = 0; k0 < K; k0 += round_k) {
@@ -131,7 +133,7 @@ __global__ void __launch_bounds__(NW * 64) qgemv_rows16_kernel(Rows16Args p)
         __builtin_amdgcn_sched_barrier(0);   // every request of the round is out before anything waits
 
         // ---- 2. row statistics of the slice
-        float inv[PPT];
+        float inv[PPT], csc[PPT];
 #pragma unroll
         for (int j = 0; j < PPT; j++) {
             float mx = 0.0f, sum = 0.0f;
@@ -157,7 +159,8 @@ __global__ void __launch_bounds__(NW * 64) qgemv_rows16_kernel(Rows16Args p)
             if (mx == 0.0f) ex = 0;
             ex = ex < -100 ? -100 : (ex > 120 ? 120 : ex);
             inv[j] = __uint_as_float((uint32_t)(127 - ex) << 23);
-            if (grp == 0) cscs[wv][j * RPP + lrow] = __uint_as_float((uint32_t)(127 + ex) << 23);
+            csc[j] = __uint_as_float((uint32_t)(127 + ex) << 23);
+            if (grp == 0) cscs[wv][j * RPP + lrow] = csc[j];
         }
 
         // ---- 3. tile by tile: operand fragments through the wave's LDS buffer, then the MFMA steps
@@ -171,6 +174,7 @@ __global__ void __launch_bounds__(NW * 64) qgemv_rows16_kernel(Rows16Args p)
                 const float x[8] = {__uint_as_float(xa[t][j].x), __uint_as_float(xa[t][j].y), __uint_as_float(xa[t][j].z), __uint_as_float(xa[t][j].w),
                                     __uint_as_float(xb[t][j].x), __uint_as_float(xb[t][j].y), __uint_as_float(xb[t][j].z), __uint_as_float(xb[t][j].w)};
                 f16x8 hi, lo;
+                float rerr = 0.0f;
 #pragma unroll
                 for (int e = 0; e < 8; e++) {
                     const int src = D::INTERLEAVED ? ((e >> 1) + 4 * (e & 1)) : e;
@@ -178,7 +182,9 @@ __global__ void __launch_bounds__(NW * 64) qgemv_rows16_kernel(Rows16Args p)
                     const _Float16 h = (_Float16)v;
                     hi[e] = h;
                     lo[e] = (_Float16)(v - (float)h);
+                    if (SINGLE) rerr += (float)h - v;
                 }
+                if (SINGLE) xerr[j] += csc[j] * rerr;   // this lane's share; summed over the row's lanes at the end
                 *reinterpret_cast<f16x8 *>(fwr + wr_off[j]) = hi;
                 if (!SINGLE) *reinterpret_cast<f16x8 *>(fwr + wr_off[j] + 16 * 64) = lo;
             }
@@ -213,21 +219,38 @@ __global__ void __launch_bounds__(NW * 64) qgemv_rows16_kernel(Rows16Args p)
     for (int r = 0; r < RT; r++)
 #pragma unroll
         for (int i = 0; i < 4; i++) red[wv][r][g * 4 + i][ln] = tot[r][i];
+    if (SINGLE) {
+#pragma unroll
+        for (int j = 0; j < PPT; j++) {   // over the LPR neighbouring lanes that hold the same row
+            float v = xerr[j];
+            v += dpp_f32<0xB1>(v);
+            v += dpp_f32<0x4E>(v);
+            v += dpp_f32<0x141>(v);
+            if (LPR == 16) v += dpp_f32<0x140>(v);
+            xerr[j] = v;
+        }
+    }
     if (grp == 0) {
 #pragma unroll
-        for (int j = 0; j < PPT; j++) xred[wv][j * RPP + lrow] = xsum[j];
+        for (int j = 0; j < PPT; j++) {
+            xred[wv][j * RPP + lrow] = xsum[j];
+            ered[wv][j * RPP + lrow] = xerr[j];
+        }
     }
     __syncthreads();
     for (int o = tid; o < RT * 256; o += NW * 64) {
         const int r = o >> 8, m = (o >> 4) & 15, c = o & 15;
         const int64_t n = n0 + r * 16 + c;
         if (m >= mreal || n >= N) continue;
-        float dot = 0.0f, xs = 0.0f;
+        float dot = 0.0f, xs = 0.0f, es = 0.0f;
 #pragma unroll
         for (int w = 0; w < NW; w++) {
             dot += red[w][r][m][c];
             xs += xred[w][m];
+            if (SINGLE) es += ered[w][m];
         }
+        // single-f16 mode, first-order correction of the rounding: dot -= mean_k u[n,k] * sum_k (hi - x)
+        if (SINGLE && p.umean) dot = dot - p.umean[n] * es;
         p.out[(int64_t)m * N + n] = fnn_epilogue(dot, p.scales[n], p.zeros[n], xs, p.bias, n, p.act);
     }
 }
@@ -294,6 +317,11 @@ int fnn_mfma_rows16(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, co
     p.words = q.words; p.scales = q.scales; p.zeros = q.zeros; p.a = q.a; p.bias = q.bias; p.out = q.out;
     p.m = q.m; p.n = q.n; p.k = q.k; p.kp = q.kp; p.act = q.act;
     const bool single = (flags & FNN_FLAG_ACT_F16_SINGLE) != 0;
+    p.umean = nullptr;
+    if (single) {
+        int rc = fnn_row_means(ctx, s, w, &p.umean);
+        if (rc) return rc;
+    }
     hipError_t e;
     switch (w->dtype) {
     case FNN_DT_I8: e = launch_rows16<FNN_DT_I8>(p, single, s); break;

@@ -113,6 +113,10 @@ GEMV_SHAPES = [(1, 256, 64), (1, 1024, 100), (2, 512, 48), (3, 2048, 33), (4, 40
 MFMA_SHAPES = [(5, 512, 64), (16, 4096, 48), (17, 1024, 100), (33, 2048, 40), (64, 8192, 32), (100, 640, 72),
                (256, 1024, 130), (8, 96, 16), (12, 12288, 24)]
 RAGGED_SHAPES = [(1, 7, 5), (3, 9, 4), (2, 100, 17), (5, 61, 130), (9, 333, 20), (17, 4100, 12), (1, 48, 8)]
+# one-launch kernels for 2..16 rows: several row tiles per workgroup (wide N), 4- and 8-wave workgroups (K <= 2048 or
+# more), K with a partial last slice and more than one round of 4096
+ROW_TILE_SHAPES = [(2, 1024, 8500), (4, 4096, 8500), (7, 1024, 8500), (8, 2048, 4400), (6, 8200, 40), (13, 4096, 8500),
+                   (16, 1024, 4400), (9, 520, 40), (11, 8200, 24), (16, 4096, 16)]
 
 
 @pytest.mark.parametrize("dt", ALL_DT)
@@ -131,6 +135,23 @@ def test_qmatmul_matches_oracle(ctx, orc, dt, m, k, n):
     assert_close(fma, want, TOL_F32, f"fma {NAMES[dt]} {m}x{k}x{n}")
     # the reference's own f32 summation orders sit inside the same band
     assert rel_err(orc.qmatmul(to_oracle(orc, pw), a, order=1), want) <= TOL_F32 * 5
+    ctx.release(h)
+
+
+@pytest.mark.parametrize("dt", [0, 1, 2, 3, 4, 5, 6])
+@pytest.mark.parametrize("m,k,n", ROW_TILE_SHAPES)
+def test_qmatmul_row_tile_kernels(ctx, orc, dt, m, k, n):
+    """M <= 8 (hi / lo operand rows of one MFMA) and 9 <= M <= 16 (activation rows = operand rows), with bias and
+    activation, both activation modes; f32 accumulation, stated bounds 2e-5 / 1e-3 of max|ref|."""
+    rng = np.random.default_rng(3500 + dt * 31 + m)
+    pw = fastnn_amd.quantize_weights(dt, _weights(rng, n, k))
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    bias = (rng.standard_normal(n) * 0.01).astype(np.float32)
+    h = ctx.register(pw)
+    want = orc.qmatmul(to_oracle(orc, pw), a, order=2, bias=bias, act=3)
+    assert_close(ctx.qmatmul(h, a, n, bias=bias, act=3), want, TOL_F32, f"{NAMES[dt]} {m}x{k}x{n}")
+    assert_close(ctx.qmatmul(h, a, n, bias=bias, act=3, flags=flib.FLAG_ACT_F16_SINGLE), want, TOL_NORTH_STAR,
+                 f"f16x1 {NAMES[dt]} {m}x{k}x{n}")
     ctx.release(h)
 
 
