@@ -207,12 +207,19 @@ class AotExecutor:
                         raise FnnError(4, f"Split: {a.shape[axis]} values along axis {axis} into {len(outs)} outputs")
                     sizes = [part] * (len(outs) - 1) + [a.shape[axis] - part * (len(outs) - 1)]
                 inner = int(np.prod(a.shape[axis + 1:], dtype=np.int64))
+                outer = int(np.prod(a.shape[:axis], dtype=np.int64))
                 start = 0
                 for o, sz in zip(outs, sizes):
                     shape = list(a.shape)
                     shape[axis] = sz
-                    out = self._new_value(o, shape)
-                    self._emit("slice_f32", ins, o, [a.slot], out.slot, [axis, start, start + sz, inner])
+                    byte0 = start * inner * 4
+                    if outer == 1 and byte0 % 64 == 0:
+                        # one outer block: the part is a contiguous, aligned range of the input's slot; values are
+                        # never overwritten (one slot per value), so it needs no copy
+                        self._values[o] = _Value(shape, (a.slot[0] + byte0, sz * inner * 4))
+                    else:
+                        out = self._new_value(o, shape)
+                        self._emit("slice_f32", ins, o, [a.slot], out.slot, [axis, start, start + sz, inner])
                     start += sz
             elif op == "Resize":
                 a = self._val(ins[0])
