@@ -381,8 +381,6 @@ def test_qconv2d_float_weight_types(ctx, orc, cfg, wdt):
     (im2col rows + fused-dequant MatMul + NCHW turn on the GPU); f32 accumulation, stated bound 2e-5."""
     rng = np.random.default_rng(6100 + cfg["c"] + wdt)
     kk = cfg["c"] // cfg["groups"] * cfg["kh"] * cfg["kw"]
-    if wdt == flib.DT_I4CB and kk % 32:
-        pytest.skip("codebook blocks of 32 values")
     x = rng.standard_normal((cfg["b"], cfg["c"], cfg["h"], cfg["w"])).astype(np.float32)
     wt = (rng.standard_normal((cfg["oc"], kk)) * np.sqrt(2.0 / kk)).astype(np.float32)
     bias = (rng.standard_normal(cfg["oc"]) * 0.05).astype(np.float32)
@@ -482,15 +480,25 @@ def test_mfma_single_f16_rounding_meets_north_star_tolerance(ctx, orc, dt):
 
 
 @pytest.mark.parametrize("name,dt,k,n,ms", [("c1", 0, 4096, 4096, (1, 32)), ("c2", 1, 4096, 11008, (1, 16, 128, 256)),
-                                           ("c4_f8", 4, 2048, 8192, (64,)), ("c4_f4", 6, 8192, 2048, (64,))])
+                                           ("c3", 7, 4096, 4096, (1, 64, 256)),
+                                           ("c4_f8_up", 4, 2048, 8192, (64,)), ("c4_f8_down", 4, 8192, 2048, (64,)),
+                                           ("c4_f4_up", 6, 2048, 8192, (64,)), ("c4_f4_down", 6, 8192, 2048, (64,))])
 def test_full_size_configs_on_row_sample(ctx, orc, name, dt, k, n, ms):
     """BASELINE shapes at full size; the oracle checks a random sample of output columns
-    (weight rows are independent), plus linearity in the activations as a whole-tensor property."""
-    rng = np.random.default_rng(8000 + dt)
-    w = _weights(rng, n, k) if name in ("c1", "c2") else (rng.standard_normal((n, k)) / np.sqrt(k)).astype(np.float32)
+    (weight rows are independent), plus linearity in the activations as a whole-tensor property.
+    The codebook weight is also dequantised whole, bit for bit."""
+    rng = np.random.default_rng(8000 + dt + k // 1024)
+    if name in ("c1", "c2"):
+        w = _weights(rng, n, k)
+    elif name == "c3":
+        w = _weights(rng, n, k, "laplace")
+    else:
+        w = (rng.standard_normal((n, k)) / np.sqrt(k)).astype(np.float32)
     pw = fastnn_amd.quantize_weights(dt, w)
     bias = (rng.standard_normal(n) * 0.01).astype(np.float32)
     h = ctx.register(pw)
+    if name == "c3":
+        assert ctx.dequant(h, n, k).tobytes() == orc.dequant(to_oracle(orc, pw)).tobytes()
     rows = np.sort(rng.choice(n, 48, replace=False))
     sub = to_oracle(orc, slice_rows(pw, rows))
     for m in ms:

@@ -125,8 +125,6 @@ def test_float_conv_equals_torch_conv_of_dequantised_weights(orc, dt, cfg):
     bias = (rng.standard_normal(oc) * 0.1).astype(np.float32)
     code = getattr(orc, dt)
     if dt == "I4CB":
-        if kk % 32:
-            pytest.skip("codebook blocks of 32")
         p = orc.quantize(code, wt, qblock=32)
     else:
         p = orc.quantize(code, wt)

@@ -204,3 +204,33 @@ def test_dequant_is_one_multiply_add(orc, dt):
     w1 = (raw * scales[0] + zeros[0]).astype(np.float32)
     g1 = orc.dequant(p1)
     assert np.array_equal(g1[~np.isnan(g1)], w1[~np.isnan(w1)])
+
+
+def test_kmeans16_f32_sums_run_in_data_order(orc):
+    """The Lloyd step adds each cluster's members into an f32 sum in data order (packed_tensor.rs:49-63);
+    that order decides the last bit of the codebook.  Independent re-derivation: assignment by argmin
+    (lowest index on ties), per-cluster running f32 sum via cumsum (sequential in numpy), one f32 divide.
+    The case is order-sensitive: the same iteration with f64 means gives a different codebook."""
+    rng = np.random.default_rng(77)
+    data = np.concatenate([rng.uniform(-1, 1, 30000), rng.uniform(-1e-3, 1e-3, 10000)]).astype(np.float32)
+    rng.shuffle(data)
+    n = data.size
+    srt = np.sort(data)
+    c = np.array([srt[min(int(np.float32((np.float32(i) + np.float32(0.5)) / np.float32(16)) * np.float32(n)), n - 1)]
+                  for i in range(16)], np.float32)
+    c64 = c.copy()
+    iters = 4
+    for _ in range(iters):
+        a = np.argmin(np.abs(data[:, None] - c[None, :]), axis=1)
+        for ci in range(16):
+            mem = data[a == ci]
+            if mem.size:
+                c[ci] = np.cumsum(mem, dtype=np.float32)[-1] / np.float32(mem.size)
+        a64 = np.argmin(np.abs(data[:, None] - c64[None, :]), axis=1)
+        for ci in range(16):
+            mem = data[a64 == ci]
+            if mem.size:
+                c64[ci] = np.float32(mem.astype(np.float64).sum() / mem.size)
+    got = orc.kmeans16(data, iters=iters)
+    assert np.array_equal(got, np.sort(c))
+    assert not np.array_equal(got, np.sort(c64))     # a pairwise / f64 sum would not pass the line above
