@@ -28,7 +28,7 @@ def meta_of(pw: "_l.PackedWeight", shape: Optional[Sequence[int]] = None):
                 zero_points=np.ascontiguousarray(pw.zeros, np.float32),
                 shape=list(shape) if shape is not None else [pw.rows, pw.inner],
                 quant_block_size=pw.qblock if pw.dtype == _l.DT_I4CB else 0,
-                codebook=None if pw.codebook is None else np.ascontiguousarray(pw.codebook, np.float32))
+                codebooks=None if pw.codebook is None else np.ascontiguousarray(pw.codebook, np.float32).reshape(1, 16))
 
 
 class ExecutablePlan:
@@ -53,7 +53,8 @@ class ExecutablePlan:
 
     def _ok(self, rc, what):
         if rc:
-            raise FnnError(rc, f"{what}: malformed instruction")
+            msg = self.lib.fnn_backend_last_error(None)
+            raise FnnError(rc, f"{what}: {msg.decode() if msg else 'malformed instruction'}")
 
     def write_const(self, offset: int, data) -> "ExecutablePlan":
         buf = np.ascontiguousarray(data).view(np.uint8).reshape(-1)
@@ -69,7 +70,10 @@ class ExecutablePlan:
         self._ok(self.lib.fnn_plan_add_memcopy(self.handle, Slice(*dst), Slice(*src)), "MemCopy")
         return self
 
-    def call_kernel(self, kernel_name: str, inputs, output, params=(), meta: Optional[dict] = None) -> "ExecutablePlan":
+    def call_kernel(self, kernel_name: str, inputs, output, params=(), meta: Optional[dict] = None,
+                    secondary_output=None) -> "ExecutablePlan":
+        """Instruction::CallKernel.  meta["codebooks"]: [n, 16] f32 (QuantizedWeightMeta.codebooks) or None;
+        secondary_output: (offset, size) of CallKernel.secondary_output_slice or None."""
         ins = (Slice * max(len(inputs), 1))(*[Slice(o, s) for o, s in inputs])
         par = (C.c_uint64 * max(len(params), 1))(*[int(p) for p in params])
         mp = None
@@ -78,14 +82,16 @@ class ExecutablePlan:
             sc = np.ascontiguousarray(meta["scales"], np.float32)
             zp = np.ascontiguousarray(meta["zero_points"], np.float32)
             sh = np.ascontiguousarray(meta["shape"], np.uint64)
-            cb = meta.get("codebook")
-            cb = None if cb is None else np.ascontiguousarray(cb, np.float32)
+            cb = meta.get("codebooks")
+            cb = None if cb is None else np.ascontiguousarray(cb, np.float32).reshape(-1, 16)
             keep = [sc, zp, sh, cb]
             m = WeightMeta(int(meta["bit_width"]), sc.ctypes.data_as(C.c_void_p), sc.size,
                            zp.ctypes.data_as(C.c_void_p), zp.size, sh.ctypes.data_as(C.c_void_p), sh.size,
-                           int(meta.get("quant_block_size", 0)), None if cb is None else cb.ctypes.data_as(C.c_void_p))
+                           int(meta.get("quant_block_size", 0)), None if cb is None else cb.ctypes.data_as(C.c_void_p),
+                           0 if cb is None else cb.shape[0])
             mp = C.byref(m)
-        self._ok(self.lib.fnn_plan_add_call_kernel(self.handle, kernel_name.encode(), ins, len(inputs), Slice(*output),
+        sec = None if secondary_output is None else C.byref(Slice(*secondary_output))
+        self._ok(self.lib.fnn_plan_add_call_kernel(self.handle, kernel_name.encode(), ins, len(inputs), Slice(*output), sec,
                                                    par, len(params), mp), kernel_name)
         del keep
         return self
@@ -110,7 +116,7 @@ class HipBackend:
         h = C.c_void_p()
         rc = self.lib.fnn_backend_create(device, C.byref(h))
         if rc:
-            msg = self.lib.fnn_hip_last_error(None)
+            msg = self.lib.fnn_backend_last_error(None)
             raise FnnError(rc, msg.decode() if msg else "fnn_backend_create failed")
         self.handle = h
 
@@ -137,6 +143,14 @@ class HipBackend:
     def set_kernel_flags(self, flags: int):
         """Extra FNN_FLAG_* bits for every MatMul / Conv2d call (e.g. lib.FLAG_ACT_F16_SINGLE)."""
         self._check(self.lib.fnn_backend_set_kernel_flags(self.handle, flags))
+
+    def set_graph_replay(self, enabled: bool):
+        """Resident plans replay as one HIP graph (default) or run instruction by instruction."""
+        self._check(self.lib.fnn_backend_set_graph_replay(self.handle, 1 if enabled else 0))
+
+    def set_option(self, option: int, value: int):
+        """fnn_hip_set_option on the backend's context (lib.OPT_* constants)."""
+        self._check(self.lib.fnn_backend_set_option(self.handle, option, value))
 
     def dispatch(self, plan: ExecutablePlan):
         self._check(self.lib.fnn_backend_dispatch(self.handle, plan.handle))

@@ -18,7 +18,6 @@
 #include "mfma.h"
 #include "../../include/fastnn_hip_backend.h"
 
-hipError_t launch_probe(const void *src, void *dst, size_t bytes, uint32_t *sink, hipStream_t s);
 hipError_t launch_im2col_f32(const float *x, float *col, int64_t b, int64_t c, int groups, int g, int64_t h, int64_t w,
                              int64_t ho, int64_t wo, int kh, int kw, int stride, int pad, int dil, hipStream_t s);
 hipError_t launch_rows_to_nchw(const float *src, float *y, int64_t b, int64_t np, int64_t oc, int64_t ch0, int64_t ocg, hipStream_t s);
@@ -29,7 +28,7 @@ hipError_t launch_copy2d(float *dst, uint64_t dst_pitch, uint64_t dst_len, const
 hipError_t launch_avgpool2d(const float *x, uint64_t in_len, float *y, uint64_t out_len, uint64_t h, uint64_t w,
                             uint64_t ho, uint64_t wo, int kernel, int stride, int pad, hipStream_t s);
 hipError_t launch_maxpool2d(const float *x, uint64_t in_len, float *y, uint64_t out_len, uint64_t c, uint64_t h, uint64_t w,
-                            uint64_t ho, uint64_t wo, int kernel, int stride, int pad, hipStream_t s);
+                            uint64_t ho, uint64_t wo, int kernel, int stride, int pad, int64_t *indices, uint64_t idx_len, hipStream_t s);
 hipError_t launch_upsample_nearest2d(const float *x, float *y, uint64_t nc, uint64_t h, uint64_t w, int sh, int sw, hipStream_t s);
 
 struct fnn_hip_graph {
@@ -46,9 +45,10 @@ struct fnn_hip_ctx {
     int device = 0;
     hipStream_t stream = nullptr;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
-    std::string err;
+    char err[1024] = {0};      // fixed storage: recording a failure never allocates
     std::unordered_map<uint64_t, fnn_hip_weight *> weights;
-    Staging st_a, st_out, st_bias, st_acc, st_tmp, st_tmp2, st_tmp3, st_cnt, st_col, st_rows;
+    Staging st_a, st_out, st_bias, st_acc, st_tmp, st_tmp2, st_tmp3, st_col, st_rows;
+    int64_t options[FNN_OPT_COUNT];
     float *scratch = nullptr;  // small reduction scratch (partials)
     bool capturing = false;
     uint64_t ws_epoch = 0;     // bumped whenever a staging buffer is re-allocated (captured graphs go stale)
@@ -56,18 +56,47 @@ struct fnn_hip_ctx {
 
 namespace {
 
-thread_local std::string g_err;  // failures without a context
+thread_local char g_err[1024] = {0};  // failures without a context
 
-int fail(fnn_hip_ctx *ctx, int code, const char *fmt, ...)
+int fail(fnn_hip_ctx *ctx, int code, const char *fmt, ...) noexcept
 {
-    char buf[1024];
+    char *buf = ctx ? ctx->err : g_err;
     va_list ap;
     va_start(ap, fmt);
-    vsnprintf(buf, sizeof(buf), fmt, ap);
+    vsnprintf(buf, 1024, fmt, ap);
     va_end(ap);
-    if (ctx) ctx->err = buf; else g_err = buf;
     return code;
 }
+
+// Every extern "C" body runs inside this: a C++ exception (std::bad_alloc from a container, std::length_error, ...)
+// becomes a status code and a message instead of unwinding into the caller's language.
+template <class F>
+int guarded(fnn_hip_ctx *ctx, const char *fn, F &&body) noexcept
+{
+    try {
+        return body();
+    } catch (const std::bad_alloc &) {
+        return fail(ctx, FNN_ERR_MEMORY, "%s: out of host memory", fn);
+    } catch (const std::exception &e) {
+        return fail(ctx, FNN_ERR_DISPATCH, "%s: %s", fn, e.what());
+    } catch (...) {
+        return fail(ctx, FNN_ERR_DISPATCH, "%s: unknown C++ exception", fn);
+    }
+}
+
+// option defaults, and the range fnn_hip_set_option accepts
+struct OptionSpec { int64_t dflt, lo, hi; };
+const OptionSpec kOptions[FNN_OPT_COUNT] = {
+    {0, 0, 0},        // (unused index 0)
+    {1, 0, 1},        // FNN_OPT_CODEBOOK_CACHE
+    {0, 0, 3},        // FNN_OPT_GEMV_ROW_TILES
+    {0, 0, 3},        // FNN_OPT_ROWS16_ROW_TILES
+    {9, 1, 17},       // FNN_OPT_ROWS16_MIN_M
+    {-1, -1, 2},      // FNN_OPT_TILE_SHAPE
+    {0, 0, 32},       // FNN_OPT_TILE_SPLIT
+    {0, 0, 6},        // FNN_OPT_TILE_STAGES
+    {5, 1, 1 << 20},  // FNN_OPT_TILE_MIN_M
+};
 
 #define HIP_TRY(ctx, code, expr)                                                              \
     do {                                                                                      \
@@ -146,28 +175,31 @@ int fnn_hip_device_count(void)
 
 int fnn_hip_create(int device, fnn_hip_ctx **out)
 {
-    if (!out) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_hip_create: out is NULL");
-    *out = nullptr;
-    int n = 0;
-    hipError_t e = hipGetDeviceCount(&n);
-    if (e != hipSuccess || n <= 0)
-        return fail(nullptr, FNN_ERR_MEMORY, "fnn_hip_create: no HIP device (%s)",
-                    e == hipSuccess ? "count 0" : hipGetErrorString(e));
-    if (device < 0 || device >= n)
-        return fail(nullptr, FNN_ERR_DISPATCH, "fnn_hip_create: device %d out of range [0,%d)", device, n);
-    fnn_hip_ctx *ctx = new (std::nothrow) fnn_hip_ctx();
-    if (!ctx) return fail(nullptr, FNN_ERR_MEMORY, "fnn_hip_create: out of host memory");
-    ctx->device = device;
-    if ((e = hipSetDevice(device)) != hipSuccess ||
-        (e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking)) != hipSuccess ||
-        (e = hipEventCreate(&ctx->ev0)) != hipSuccess || (e = hipEventCreate(&ctx->ev1)) != hipSuccess ||
-        (e = hipMalloc((void **)&ctx->scratch, 64 * 1024)) != hipSuccess) {
-        int rc = fail(nullptr, FNN_ERR_MEMORY, "fnn_hip_create: %s", hipGetErrorString(e));
-        fnn_hip_destroy(ctx);
-        return rc;
-    }
-    *out = ctx;
-    return FNN_OK;
+    return guarded(nullptr, "fnn_hip_create", [&]() -> int {
+        if (!out) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_hip_create: out is NULL");
+        *out = nullptr;
+        int n = 0;
+        hipError_t e = hipGetDeviceCount(&n);
+        if (e != hipSuccess || n <= 0)
+            return fail(nullptr, FNN_ERR_MEMORY, "fnn_hip_create: no HIP device (%s)",
+                        e == hipSuccess ? "count 0" : hipGetErrorString(e));
+        if (device < 0 || device >= n)
+            return fail(nullptr, FNN_ERR_DISPATCH, "fnn_hip_create: device %d out of range [0,%d)", device, n);
+        fnn_hip_ctx *ctx = new (std::nothrow) fnn_hip_ctx();
+        if (!ctx) return fail(nullptr, FNN_ERR_MEMORY, "fnn_hip_create: out of host memory");
+        ctx->device = device;
+        for (int i = 0; i < FNN_OPT_COUNT; i++) ctx->options[i] = kOptions[i].dflt;
+        if ((e = hipSetDevice(device)) != hipSuccess ||
+            (e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking)) != hipSuccess ||
+            (e = hipEventCreate(&ctx->ev0)) != hipSuccess || (e = hipEventCreate(&ctx->ev1)) != hipSuccess ||
+            (e = hipMalloc((void **)&ctx->scratch, 64 * 1024)) != hipSuccess) {
+            int rc = fail(nullptr, FNN_ERR_MEMORY, "fnn_hip_create: %s", hipGetErrorString(e));
+            fnn_hip_destroy(ctx);
+            return rc;
+        }
+        *out = ctx;
+        return FNN_OK;
+    });
 }
 
 void fnn_hip_destroy(fnn_hip_ctx *ctx)
@@ -176,7 +208,7 @@ void fnn_hip_destroy(fnn_hip_ctx *ctx)
     (void)hipSetDevice(ctx->device);
     if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
     for (auto &kv : ctx->weights) free_weight(kv.second);
-    for (Staging *s : {&ctx->st_a, &ctx->st_out, &ctx->st_bias, &ctx->st_acc, &ctx->st_tmp, &ctx->st_tmp2, &ctx->st_tmp3, &ctx->st_cnt, &ctx->st_col, &ctx->st_rows})
+    for (Staging *s : {&ctx->st_a, &ctx->st_out, &ctx->st_bias, &ctx->st_acc, &ctx->st_tmp, &ctx->st_tmp2, &ctx->st_tmp3, &ctx->st_col, &ctx->st_rows})
         if (s->ptr) (void)hipFree(s->ptr);
     if (ctx->scratch) (void)hipFree(ctx->scratch);
     if (ctx->ev0) (void)hipEventDestroy(ctx->ev0);
@@ -185,49 +217,86 @@ void fnn_hip_destroy(fnn_hip_ctx *ctx)
     delete ctx;
 }
 
-const char *fnn_hip_last_error(fnn_hip_ctx *ctx) { return ctx ? ctx->err.c_str() : g_err.c_str(); }
+const char *fnn_hip_last_error(fnn_hip_ctx *ctx) { return ctx ? ctx->err : g_err; }
 
 int fnn_hip_sync(fnn_hip_ctx *ctx)
 {
-    if (!ctx) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_hip_sync: NULL context");
-    HIP_TRY(ctx, FNN_ERR_DISPATCH, hipStreamSynchronize(ctx->stream));
-    return FNN_OK;
+    return guarded(ctx, "fnn_hip_sync", [&]() -> int {
+        if (!ctx) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_hip_sync: NULL context");
+        HIP_TRY(ctx, FNN_ERR_DISPATCH, hipStreamSynchronize(ctx->stream));
+        return FNN_OK;
+    });
 }
+
+int fnn_hip_set_option(fnn_hip_ctx *ctx, int option, int64_t value)
+{
+    return guarded(ctx, "fnn_hip_set_option", [&]() -> int {
+        if (!ctx) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_hip_set_option: NULL context");
+        if (option <= 0 || option >= FNN_OPT_COUNT) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_set_option: unknown option %d", option);
+        const OptionSpec &o = kOptions[option];
+        if (value < o.lo || value > o.hi)
+            return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_set_option: value %lld of option %d outside [%lld, %lld]", (long long)value,
+                        option, (long long)o.lo, (long long)o.hi);
+        if (ctx->capturing) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_set_option: graph capture active");
+        ctx->options[option] = value;
+        return FNN_OK;
+    });
+}
+
+int fnn_hip_get_option(fnn_hip_ctx *ctx, int option, int64_t *value)
+{
+    return guarded(ctx, "fnn_hip_get_option", [&]() -> int {
+        if (!ctx || !value) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_get_option: NULL argument");
+        if (option <= 0 || option >= FNN_OPT_COUNT) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_get_option: unknown option %d", option);
+        *value = ctx->options[option];
+        return FNN_OK;
+    });
+}
+
+void *fnn_hip_stream(fnn_hip_ctx *ctx) { return ctx ? (void *)ctx->stream : nullptr; }
 
 int fnn_hip_malloc(fnn_hip_ctx *ctx, size_t bytes, void **dptr)
 {
-    if (!ctx || !dptr) return fail(ctx, FNN_ERR_MEMORY, "fnn_hip_malloc: NULL argument");
-    *dptr = nullptr;
-    HIP_TRY(ctx, FNN_ERR_MEMORY, hipSetDevice(ctx->device));
-    HIP_TRY(ctx, FNN_ERR_MEMORY, hipMalloc(dptr, bytes ? bytes : 1));
-    return FNN_OK;
+    return guarded(ctx, "fnn_hip_malloc", [&]() -> int {
+        if (!ctx || !dptr) return fail(ctx, FNN_ERR_MEMORY, "fnn_hip_malloc: NULL argument");
+        *dptr = nullptr;
+        HIP_TRY(ctx, FNN_ERR_MEMORY, hipSetDevice(ctx->device));
+        HIP_TRY(ctx, FNN_ERR_MEMORY, hipMalloc(dptr, bytes ? bytes : 1));
+        return FNN_OK;
+    });
 }
 
 int fnn_hip_free(fnn_hip_ctx *ctx, void *dptr)
 {
-    if (!ctx) return fail(nullptr, FNN_ERR_MEMORY, "fnn_hip_free: NULL context");
-    if (!dptr) return FNN_OK;
-    HIP_TRY(ctx, FNN_ERR_MEMORY, hipStreamSynchronize(ctx->stream));
-    HIP_TRY(ctx, FNN_ERR_MEMORY, hipFree(dptr));
-    return FNN_OK;
+    return guarded(ctx, "fnn_hip_free", [&]() -> int {
+        if (!ctx) return fail(nullptr, FNN_ERR_MEMORY, "fnn_hip_free: NULL context");
+        if (!dptr) return FNN_OK;
+        HIP_TRY(ctx, FNN_ERR_MEMORY, hipStreamSynchronize(ctx->stream));
+        HIP_TRY(ctx, FNN_ERR_MEMORY, hipFree(dptr));
+        return FNN_OK;
+    });
 }
 
 int fnn_hip_upload(fnn_hip_ctx *ctx, void *dst, const void *src, size_t bytes)
 {
-    if (!ctx || (bytes && (!dst || !src))) return fail(ctx, FNN_ERR_MEMORY, "fnn_hip_upload: NULL argument");
-    if (!bytes) return FNN_OK;
-    HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx->stream));
-    HIP_TRY(ctx, FNN_ERR_MEMORY, hipStreamSynchronize(ctx->stream));
-    return FNN_OK;
+    return guarded(ctx, "fnn_hip_upload", [&]() -> int {
+        if (!ctx || (bytes && (!dst || !src))) return fail(ctx, FNN_ERR_MEMORY, "fnn_hip_upload: NULL argument");
+        if (!bytes) return FNN_OK;
+        HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx->stream));
+        HIP_TRY(ctx, FNN_ERR_MEMORY, hipStreamSynchronize(ctx->stream));
+        return FNN_OK;
+    });
 }
 
 int fnn_hip_download(fnn_hip_ctx *ctx, void *dst, const void *src, size_t bytes)
 {
-    if (!ctx || (bytes && (!dst || !src))) return fail(ctx, FNN_ERR_MEMORY, "fnn_hip_download: NULL argument");
-    if (!bytes) return FNN_OK;
-    HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx->stream));
-    HIP_TRY(ctx, FNN_ERR_MEMORY, hipStreamSynchronize(ctx->stream));
-    return FNN_OK;
+    return guarded(ctx, "fnn_hip_download", [&]() -> int {
+        if (!ctx || (bytes && (!dst || !src))) return fail(ctx, FNN_ERR_MEMORY, "fnn_hip_download: NULL argument");
+        if (!bytes) return FNN_OK;
+        HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx->stream));
+        HIP_TRY(ctx, FNN_ERR_MEMORY, hipStreamSynchronize(ctx->stream));
+        return FNN_OK;
+    });
 }
 
 // Validation mirrors packed_tensor_from_meta (src/backend/cpu/matmul.rs:81-152).
@@ -236,655 +305,698 @@ int fnn_hip_weight_register(fnn_hip_ctx *ctx, uint64_t key, int dtype, const uin
                             size_t n_scales, const float *zeros, size_t n_zeros,
                             int quant_block_size, const float *codebook16, fnn_hip_weight **out)
 {
-    if (!ctx) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_hip_weight_register: NULL context");
-    if (out) *out = nullptr;
-    if (codebook16 && dtype == FNN_DT_I4) dtype = FNN_DT_I4CB;
-    const int items = items_of(dtype);
-    const char *kn = kernel_name_of(dtype);
-    if (!items) return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "unsupported packed dtype %d", dtype);
-    if (rows <= 0 || inner <= 0)
-        return fail(ctx, FNN_ERR_DISPATCH, "%s: invalid weight shape [%lld, %lld]", kn, (long long)rows, (long long)inner);
-    if (!scales || n_scales == 0)
-        return fail(ctx, FNN_ERR_DISPATCH, "%s: quantized weight metadata missing scales", kn);
-    if (n_zeros != 0 && n_zeros != n_scales && dtype != FNN_DT_I4CB)
-        return fail(ctx, FNN_ERR_DISPATCH,
-                    "%s: quantized weight metadata length mismatch: %zu scales vs %zu zero_points", kn,
-                    n_scales, n_zeros);
-    if (n_zeros != 0 && !zeros)
-        return fail(ctx, FNN_ERR_DISPATCH, "%s: zero_points pointer is NULL", kn);
-    const size_t urows = (size_t)rows;
-    const bool valid_len = n_scales == 1 || n_scales == urows ||
-                           (n_scales > 1 && urows > n_scales && urows % n_scales == 0) ||
-                           (quant_block_size > 0 && n_scales > urows && n_scales % urows == 0);
-    if (!valid_len)
-        return fail(ctx, FNN_ERR_DISPATCH,
-                    "%s: quantized weight metadata length %zu incompatible with shape [%lld, %lld] "
-                    "(expected 1, %lld, or a divisor of %lld)",
-                    kn, n_scales, (long long)rows, (long long)inner, (long long)rows, (long long)rows);
-    const int64_t kp = (inner + items - 1) / items;
-    const size_t expected = (size_t)(rows * kp);
-    if (!words || n_words < expected)
-        return fail(ctx, FNN_ERR_DISPATCH,
-                    "%s: quantized weight payload too short: got %zu packed words for shape [%lld, %lld], "
-                    "expected at least %zu",
-                    kn, words ? n_words : (size_t)0, (long long)rows, (long long)inner, expected);
-    int64_t bpr = 0;
-    if (dtype == FNN_DT_I4CB) {
-        if (!codebook16) return fail(ctx, FNN_ERR_DISPATCH, "%s: codebook weight without codebook", kn);
-        if (quant_block_size <= 0)
-            return fail(ctx, FNN_ERR_DISPATCH, "%s: codebook weight needs quant_block_size > 0", kn);
-        bpr = (inner + quant_block_size - 1) / quant_block_size;
-        if (n_scales < (size_t)(rows * bpr))
-            return fail(ctx, FNN_ERR_DISPATCH, "%s: codebook weight needs %lld block scales, got %zu", kn,
-                        (long long)(rows * bpr), n_scales);
-    } else if (quant_block_size > 0 && n_scales > urows) {
-        return fail(ctx, FNN_ERR_UNSUPPORTED_OP,
-                    "%s: per-block scales without a codebook are not produced by the quantisation pass", kn);
-    }
-    if (ctx->weights.count(key))
-        return fail(ctx, FNN_ERR_DISPATCH, "weight key %llu already registered", (unsigned long long)key);
-
-    HIP_TRY(ctx, FNN_ERR_MEMORY, hipSetDevice(ctx->device));
-    fnn_hip_weight *w = new (std::nothrow) fnn_hip_weight();
-    if (!w) return fail(ctx, FNN_ERR_MEMORY, "out of host memory");
-    memset(w, 0, sizeof(*w));
-    w->key = key; w->dtype = dtype; w->rows = rows; w->inner = inner; w->items = items; w->kp = kp;
-    w->qblock = (dtype == FNN_DT_I4CB) ? quant_block_size : 0;
-    w->bpr = bpr; w->ctx = ctx;
-
-    // device copy of the words, with the two value-preserving canonicalisations that let
-    // the hardware converts stand for the reference's decode tables:
-    //   F8: every exponent-15 byte decodes to NaN (src/dtypes/f8x4.rs:36) -> OCP NaN 0x7F/0xFF;
-    //   F4: nibble 0x8 decodes to +0.0 (src/dtypes/f4x8.rs:31-35) -> 0x0.
-    std::vector<uint32_t> host(expected);
-    memcpy(host.data(), words, expected * sizeof(uint32_t));
-    if (dtype == FNN_DT_F8) {
-        for (auto &x : host)
-            for (int i = 0; i < 4; i++)
-                if (((x >> (8 * i)) & 0x78u) == 0x78u) x |= (0x7Fu << (8 * i));
-    } else if (dtype == FNN_DT_F4) {
-        for (auto &x : host)
-            for (int i = 0; i < 8; i++)
-                if (((x >> (4 * i)) & 0xFu) == 0x8u) x &= ~(0xFu << (4 * i));
-    }
-    const size_t pad = 256;
-    hipError_t e;
-    auto bail = [&](const char *what) {
-        int rc = fail(ctx, FNN_ERR_MEMORY, "%s: %s", what, hipGetErrorString(e));
-        free_weight(w);
-        return rc;
-    };
-    if ((e = hipMalloc((void **)&w->words, expected * 4 + pad)) != hipSuccess) return bail("hipMalloc(words)");
-    if ((e = hipMemsetAsync(w->words, 0, expected * 4 + pad, ctx->stream)) != hipSuccess) return bail("hipMemset(words)");
-    if ((e = hipMemcpyAsync(w->words, host.data(), expected * 4, hipMemcpyHostToDevice, ctx->stream)) != hipSuccess)
-        return bail("hipMemcpy(words)");
-
-    // scales / zeros expanded to one entry per row (scale_for_row / zero_for_row,
-    // src/packed_tensor.rs:438-462; group rule src/backend/cpu/matmul.rs:147-149)
-    std::vector<float> sc, zr;
-    if (dtype == FNN_DT_I4CB) {
-        sc.assign(scales, scales + rows * bpr);
-        zr.assign((size_t)rows, 0.0f);
-    } else {
-        sc.resize((size_t)rows);
-        zr.resize((size_t)rows);
-        const size_t group = (n_scales > 1 && urows > n_scales) ? urows / n_scales : 1;
-        for (size_t r = 0; r < urows; r++) {
-            const size_t idx = (n_scales == 1) ? 0 : r / group;
-            sc[r] = scales[idx];
-            zr[r] = n_zeros ? zeros[idx] : 0.0f;
+    return guarded(ctx, "fnn_hip_weight_register", [&]() -> int {
+        if (!ctx) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_hip_weight_register: NULL context");
+        if (out) *out = nullptr;
+        if (codebook16 && dtype == FNN_DT_I4) dtype = FNN_DT_I4CB;
+        const int items = items_of(dtype);
+        const char *kn = kernel_name_of(dtype);
+        if (!items) return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "unsupported packed dtype %d", dtype);
+        if (rows <= 0 || inner <= 0)
+            return fail(ctx, FNN_ERR_DISPATCH, "%s: invalid weight shape [%lld, %lld]", kn, (long long)rows, (long long)inner);
+        if (!scales || n_scales == 0)
+            return fail(ctx, FNN_ERR_DISPATCH, "%s: quantized weight metadata missing scales", kn);
+        if (n_zeros != 0 && n_zeros != n_scales && dtype != FNN_DT_I4CB)
+            return fail(ctx, FNN_ERR_DISPATCH,
+                        "%s: quantized weight metadata length mismatch: %zu scales vs %zu zero_points", kn,
+                        n_scales, n_zeros);
+        if (n_zeros != 0 && !zeros)
+            return fail(ctx, FNN_ERR_DISPATCH, "%s: zero_points pointer is NULL", kn);
+        const size_t urows = (size_t)rows;
+        const bool valid_len = n_scales == 1 || n_scales == urows ||
+                               (n_scales > 1 && urows > n_scales && urows % n_scales == 0) ||
+                               (quant_block_size > 0 && n_scales > urows && n_scales % urows == 0);
+        if (!valid_len)
+            return fail(ctx, FNN_ERR_DISPATCH,
+                        "%s: quantized weight metadata length %zu incompatible with shape [%lld, %lld] "
+                        "(expected 1, %lld, or a divisor of %lld)",
+                        kn, n_scales, (long long)rows, (long long)inner, (long long)rows, (long long)rows);
+        const int64_t kp = (inner + items - 1) / items;
+        const size_t expected = (size_t)(rows * kp);
+        if (!words || n_words < expected)
+            return fail(ctx, FNN_ERR_DISPATCH,
+                        "%s: quantized weight payload too short: got %zu packed words for shape [%lld, %lld], "
+                        "expected at least %zu",
+                        kn, words ? n_words : (size_t)0, (long long)rows, (long long)inner, expected);
+        int64_t bpr = 0;
+        if (dtype == FNN_DT_I4CB) {
+            if (!codebook16) return fail(ctx, FNN_ERR_DISPATCH, "%s: codebook weight without codebook", kn);
+            if (quant_block_size <= 0)
+                return fail(ctx, FNN_ERR_DISPATCH, "%s: codebook weight needs quant_block_size > 0", kn);
+            bpr = (inner + quant_block_size - 1) / quant_block_size;
+            if (n_scales < (size_t)(rows * bpr))
+                return fail(ctx, FNN_ERR_DISPATCH, "%s: codebook weight needs %lld block scales, got %zu", kn,
+                            (long long)(rows * bpr), n_scales);
+        } else if (quant_block_size > 0 && n_scales > urows) {
+            return fail(ctx, FNN_ERR_UNSUPPORTED_OP,
+                        "%s: per-block scales without a codebook are not produced by the quantisation pass", kn);
         }
-    }
-    if ((e = hipMalloc((void **)&w->scales, sc.size() * 4 + 64)) != hipSuccess) return bail("hipMalloc(scales)");
-    if ((e = hipMalloc((void **)&w->zeros, zr.size() * 4 + 64)) != hipSuccess) return bail("hipMalloc(zeros)");
-    if ((e = hipMemcpyAsync(w->scales, sc.data(), sc.size() * 4, hipMemcpyHostToDevice, ctx->stream)) != hipSuccess)
-        return bail("hipMemcpy(scales)");
-    if ((e = hipMemcpyAsync(w->zeros, zr.data(), zr.size() * 4, hipMemcpyHostToDevice, ctx->stream)) != hipSuccess)
-        return bail("hipMemcpy(zeros)");
-    if (dtype == FNN_DT_I4CB) {
-        if ((e = hipMalloc((void **)&w->codebook, 64)) != hipSuccess) return bail("hipMalloc(codebook)");
-        if ((e = hipMemcpyAsync(w->codebook, codebook16, 64, hipMemcpyHostToDevice, ctx->stream)) != hipSuccess)
-            return bail("hipMemcpy(codebook)");
-    }
-    if ((e = hipStreamSynchronize(ctx->stream)) != hipSuccess) return bail("hipStreamSynchronize");
-    ctx->weights[key] = w;
-    if (out) *out = w;
-    return FNN_OK;
+        if (ctx->weights.count(key))
+            return fail(ctx, FNN_ERR_DISPATCH, "weight key %llu already registered", (unsigned long long)key);
+
+        HIP_TRY(ctx, FNN_ERR_MEMORY, hipSetDevice(ctx->device));
+        fnn_hip_weight *w = new (std::nothrow) fnn_hip_weight();
+        if (!w) return fail(ctx, FNN_ERR_MEMORY, "out of host memory");
+        memset(w, 0, sizeof(*w));
+        w->key = key; w->dtype = dtype; w->rows = rows; w->inner = inner; w->items = items; w->kp = kp;
+        w->qblock = (dtype == FNN_DT_I4CB) ? quant_block_size : 0;
+        w->bpr = bpr; w->ctx = ctx;
+
+        // device copy of the words, with the two value-preserving canonicalisations that let
+        // the hardware converts stand for the reference's decode tables:
+        //   F8: every exponent-15 byte decodes to NaN (src/dtypes/f8x4.rs:36) -> OCP NaN 0x7F/0xFF;
+        //   F4: nibble 0x8 decodes to +0.0 (src/dtypes/f4x8.rs:31-35) -> 0x0.
+        std::vector<uint32_t> host(expected);
+        memcpy(host.data(), words, expected * sizeof(uint32_t));
+        if (dtype == FNN_DT_F8) {
+            for (auto &x : host)
+                for (int i = 0; i < 4; i++)
+                    if (((x >> (8 * i)) & 0x78u) == 0x78u) x |= (0x7Fu << (8 * i));
+        } else if (dtype == FNN_DT_F4) {
+            for (auto &x : host)
+                for (int i = 0; i < 8; i++)
+                    if (((x >> (4 * i)) & 0xFu) == 0x8u) x &= ~(0xFu << (4 * i));
+        }
+        const size_t pad = 256;
+        hipError_t e;
+        auto bail = [&](const char *what) {
+            int rc = fail(ctx, FNN_ERR_MEMORY, "%s: %s", what, hipGetErrorString(e));
+            free_weight(w);
+            return rc;
+        };
+        if ((e = hipMalloc((void **)&w->words, expected * 4 + pad)) != hipSuccess) return bail("hipMalloc(words)");
+        if ((e = hipMemsetAsync(w->words, 0, expected * 4 + pad, ctx->stream)) != hipSuccess) return bail("hipMemset(words)");
+        if ((e = hipMemcpyAsync(w->words, host.data(), expected * 4, hipMemcpyHostToDevice, ctx->stream)) != hipSuccess)
+            return bail("hipMemcpy(words)");
+
+        // scales / zeros expanded to one entry per row (scale_for_row / zero_for_row,
+        // src/packed_tensor.rs:438-462; group rule src/backend/cpu/matmul.rs:147-149)
+        std::vector<float> sc, zr;
+        if (dtype == FNN_DT_I4CB) {
+            sc.assign(scales, scales + rows * bpr);
+            zr.assign((size_t)rows, 0.0f);
+        } else {
+            sc.resize((size_t)rows);
+            zr.resize((size_t)rows);
+            const size_t group = (n_scales > 1 && urows > n_scales) ? urows / n_scales : 1;
+            for (size_t r = 0; r < urows; r++) {
+                const size_t idx = (n_scales == 1) ? 0 : r / group;
+                sc[r] = scales[idx];
+                zr[r] = n_zeros ? zeros[idx] : 0.0f;
+            }
+        }
+        if ((e = hipMalloc((void **)&w->scales, sc.size() * 4 + 64)) != hipSuccess) return bail("hipMalloc(scales)");
+        if ((e = hipMalloc((void **)&w->zeros, zr.size() * 4 + 64)) != hipSuccess) return bail("hipMalloc(zeros)");
+        if ((e = hipMemcpyAsync(w->scales, sc.data(), sc.size() * 4, hipMemcpyHostToDevice, ctx->stream)) != hipSuccess)
+            return bail("hipMemcpy(scales)");
+        if ((e = hipMemcpyAsync(w->zeros, zr.data(), zr.size() * 4, hipMemcpyHostToDevice, ctx->stream)) != hipSuccess)
+            return bail("hipMemcpy(zeros)");
+        if (dtype == FNN_DT_I4CB) {
+            if ((e = hipMalloc((void **)&w->codebook, 64)) != hipSuccess) return bail("hipMalloc(codebook)");
+            if ((e = hipMemcpyAsync(w->codebook, codebook16, 64, hipMemcpyHostToDevice, ctx->stream)) != hipSuccess)
+                return bail("hipMemcpy(codebook)");
+        }
+        if ((e = hipStreamSynchronize(ctx->stream)) != hipSuccess) return bail("hipStreamSynchronize");
+        ctx->weights[key] = w;
+        if (out) *out = w;
+        return FNN_OK;
+    });
 }
 
 int fnn_hip_weight_lookup(fnn_hip_ctx *ctx, uint64_t key, fnn_hip_weight **out)
 {
-    if (!ctx || !out) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_weight_lookup: NULL argument");
-    auto it = ctx->weights.find(key);
-    *out = (it == ctx->weights.end()) ? nullptr : it->second;
-    if (!*out) return fail(ctx, FNN_ERR_DISPATCH, "weight key %llu not registered", (unsigned long long)key);
-    return FNN_OK;
+    return guarded(ctx, "fnn_hip_weight_lookup", [&]() -> int {
+        if (!ctx || !out) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_weight_lookup: NULL argument");
+        auto it = ctx->weights.find(key);
+        *out = (it == ctx->weights.end()) ? nullptr : it->second;
+        if (!*out) return fail(ctx, FNN_ERR_DISPATCH, "weight key %llu not registered", (unsigned long long)key);
+        return FNN_OK;
+    });
 }
 
 int fnn_hip_weight_release(fnn_hip_ctx *ctx, fnn_hip_weight *w)
 {
-    if (!ctx || !w) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_weight_release: NULL argument");
-    auto it = ctx->weights.find(w->key);
-    if (it == ctx->weights.end() || it->second != w)
-        return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_weight_release: weight does not belong to this context");
-    HIP_TRY(ctx, FNN_ERR_DISPATCH, hipStreamSynchronize(ctx->stream));
-    ctx->weights.erase(it);
-    free_weight(w);
-    return FNN_OK;
+    return guarded(ctx, "fnn_hip_weight_release", [&]() -> int {
+        if (!ctx || !w) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_weight_release: NULL argument");
+        auto it = ctx->weights.find(w->key);
+        if (it == ctx->weights.end() || it->second != w)
+            return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_weight_release: weight does not belong to this context");
+        HIP_TRY(ctx, FNN_ERR_DISPATCH, hipStreamSynchronize(ctx->stream));
+        ctx->weights.erase(it);
+        free_weight(w);
+        return FNN_OK;
+    });
 }
 
 int fnn_hip_dequant(fnn_hip_ctx *ctx, const fnn_hip_weight *w, float *out, int flags)
 {
-    if (!ctx || !w || !out) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_dequant: NULL argument");
-    const size_t bytes = (size_t)(w->rows * w->inner) * 4;
-    float *dout = out;
-    if (!(flags & FNN_FLAG_DEVICE_PTRS)) {
-        int rc = ensure(ctx, ctx->st_out, bytes);
-        if (rc) return rc;
-        dout = (float *)ctx->st_out.ptr;
-    }
-    HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_dequant(w, dout, ctx->stream));
-    if (!(flags & FNN_FLAG_DEVICE_PTRS)) {
-        HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(out, dout, bytes, hipMemcpyDeviceToHost, ctx->stream));
-        HIP_TRY(ctx, FNN_ERR_DISPATCH, hipStreamSynchronize(ctx->stream));
-    }
-    return FNN_OK;
+    return guarded(ctx, "fnn_hip_dequant", [&]() -> int {
+        if (!ctx || !w || !out) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_dequant: NULL argument");
+        const size_t bytes = (size_t)(w->rows * w->inner) * 4;
+        float *dout = out;
+        if (!(flags & FNN_FLAG_DEVICE_PTRS)) {
+            int rc = ensure(ctx, ctx->st_out, bytes);
+            if (rc) return rc;
+            dout = (float *)ctx->st_out.ptr;
+        }
+        HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_dequant(w, dout, ctx->stream));
+        if (!(flags & FNN_FLAG_DEVICE_PTRS)) {
+            HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(out, dout, bytes, hipMemcpyDeviceToHost, ctx->stream));
+            HIP_TRY(ctx, FNN_ERR_DISPATCH, hipStreamSynchronize(ctx->stream));
+        }
+        return FNN_OK;
+    });
 }
 
 int fnn_hip_qmatmul(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *a, int64_t m,
                     const float *bias, int act, float *out, int flags)
 {
-    if (!ctx || !w) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_qmatmul: NULL context or weight");
-    const char *kn = kernel_name_of(w->dtype);
-    if (m < 0) return fail(ctx, FNN_ERR_DISPATCH, "%s: expected params [M,K,N], got M=%lld", kn, (long long)m);
-    if (m == 0) return FNN_OK;
-    if (!a || !out) return fail(ctx, FNN_ERR_DISPATCH, "%s: NULL activation or output pointer", kn);
-    if (act < FNN_ACT_NONE || act > FNN_ACT_SILU)
-        return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "%s: unknown activation %d", kn, act);
-    if ((flags & FNN_FLAG_I4CB_AS_WRITTEN) && w->dtype != FNN_DT_I4CB)
-        return fail(ctx, FNN_ERR_DISPATCH, "%s: as-written mode applies to codebook weights only", kn);
-    const int64_t n = w->rows, k = w->inner;
-    const bool dev = (flags & FNN_FLAG_DEVICE_PTRS) != 0;
-    const float *da = a, *dbias = bias;
-    float *dout = out;
-    if (!dev) {
-        int rc;
-        if ((rc = ensure(ctx, ctx->st_a, (size_t)(m * k) * 4))) return rc;
-        if ((rc = ensure(ctx, ctx->st_out, (size_t)(m * n) * 4))) return rc;
-        HIP_TRY(ctx, FNN_ERR_MEMORY,
-                hipMemcpyAsync(ctx->st_a.ptr, a, (size_t)(m * k) * 4, hipMemcpyHostToDevice, ctx->stream));
-        da = (const float *)ctx->st_a.ptr;
-        dout = (float *)ctx->st_out.ptr;
-        if (bias) {
-            if ((rc = ensure(ctx, ctx->st_bias, (size_t)n * 4))) return rc;
+    return guarded(ctx, "fnn_hip_qmatmul", [&]() -> int {
+        if (!ctx || !w) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_qmatmul: NULL context or weight");
+        const char *kn = kernel_name_of(w->dtype);
+        if (m < 0) return fail(ctx, FNN_ERR_DISPATCH, "%s: expected params [M,K,N], got M=%lld", kn, (long long)m);
+        if (m == 0) return FNN_OK;
+        if (!a || !out) return fail(ctx, FNN_ERR_DISPATCH, "%s: NULL activation or output pointer", kn);
+        if (act < FNN_ACT_NONE || act > FNN_ACT_SILU)
+            return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "%s: unknown activation %d", kn, act);
+        if ((flags & FNN_FLAG_I4CB_AS_WRITTEN) && w->dtype != FNN_DT_I4CB)
+            return fail(ctx, FNN_ERR_DISPATCH, "%s: as-written mode applies to codebook weights only", kn);
+        const int64_t n = w->rows, k = w->inner;
+        const bool dev = (flags & FNN_FLAG_DEVICE_PTRS) != 0;
+        const float *da = a, *dbias = bias;
+        float *dout = out;
+        if (!dev) {
+            int rc;
+            if ((rc = ensure(ctx, ctx->st_a, (size_t)(m * k) * 4))) return rc;
+            if ((rc = ensure(ctx, ctx->st_out, (size_t)(m * n) * 4))) return rc;
             HIP_TRY(ctx, FNN_ERR_MEMORY,
-                    hipMemcpyAsync(ctx->st_bias.ptr, bias, (size_t)n * 4, hipMemcpyHostToDevice, ctx->stream));
-            dbias = (const float *)ctx->st_bias.ptr;
+                    hipMemcpyAsync(ctx->st_a.ptr, a, (size_t)(m * k) * 4, hipMemcpyHostToDevice, ctx->stream));
+            da = (const float *)ctx->st_a.ptr;
+            dout = (float *)ctx->st_out.ptr;
+            if (bias) {
+                if ((rc = ensure(ctx, ctx->st_bias, (size_t)n * 4))) return rc;
+                HIP_TRY(ctx, FNN_ERR_MEMORY,
+                        hipMemcpyAsync(ctx->st_bias.ptr, bias, (size_t)n * 4, hipMemcpyHostToDevice, ctx->stream));
+                dbias = (const float *)ctx->st_bias.ptr;
+            }
         }
-    }
-    QMatmulArgs p;
-    p.words = w->words; p.scales = w->scales; p.zeros = w->zeros; p.codebook = w->codebook;
-    p.a = da; p.bias = dbias; p.out = dout;
-    p.m = m; p.n = n; p.k = k; p.kp = w->kp; p.bpr = w->bpr; p.qblock = w->qblock; p.act = act;
-    p.as_written = (flags & FNN_FLAG_I4CB_AS_WRITTEN) ? 1 : 0;
+        QMatmulArgs p;
+        p.words = w->words; p.scales = w->scales; p.zeros = w->zeros; p.codebook = w->codebook;
+        p.a = da; p.bias = dbias; p.out = dout;
+        p.m = m; p.n = n; p.k = k; p.kp = w->kp; p.bpr = w->bpr; p.qblock = w->qblock; p.act = act;
+        p.as_written = (flags & FNN_FLAG_I4CB_AS_WRITTEN) ? 1 : 0;
 
-    // kernel choice: matrix-core kernel for every M (bandwidth-bound at small M); the FMA GEMV
-    // serves the codebook type at M <= 4 and any weight when FNN_FLAG_PREFER_FMA asks for it;
-    // the shape-agnostic kernel takes what is left (ragged rows, unaligned pointers).
-    bool handled = false;
-    if (!(flags & FNN_FLAG_FORCE_GENERIC)) {
-        const bool fma_first = (flags & FNN_FLAG_PREFER_FMA) || w->dtype == FNN_DT_I4CB;
-        if (fma_first) HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qgemv(w->dtype, p, ctx->stream, &handled));
-        if (!handled) {
-            int rc = fnn_mfma_qgemv(ctx, ctx->stream, w, p, flags, &handled);
-            if (rc) return rc;
+        // kernel choice: matrix-core kernel for every M (bandwidth-bound at small M); the FMA GEMV
+        // serves the codebook type at M <= 4 and any weight when FNN_FLAG_PREFER_FMA asks for it;
+        // the shape-agnostic kernel takes what is left (ragged rows, unaligned pointers).
+        bool handled = false;
+        if (!(flags & FNN_FLAG_FORCE_GENERIC)) {
+            const bool fma_first = (flags & FNN_FLAG_PREFER_FMA) || w->dtype == FNN_DT_I4CB;
+            if (fma_first) HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qgemv(w->dtype, p, ctx->stream, &handled));
+            if (!handled) {
+                int rc = fnn_mfma_qgemv(ctx, ctx->stream, w, p, flags, &handled);
+                if (rc) return rc;
+            }
+            if (!handled) {
+                int rc = fnn_mfma_rows16(ctx, ctx->stream, w, p, flags, &handled);
+                if (rc) return rc;
+            }
+            if (!handled) {
+                int rc = fnn_tiled_qmatmul(ctx, ctx->stream, w, p, flags, &handled);
+                if (rc) return rc;
+            }
+            if (!handled && !fma_first) HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qgemv(w->dtype, p, ctx->stream, &handled));
         }
-        if (!handled) {
-            int rc = fnn_mfma_rows16(ctx, ctx->stream, w, p, flags, &handled);
-            if (rc) return rc;
+        if (!handled) HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qgemm_generic(w->dtype, p, ctx->stream));
+        if (!dev) {
+            HIP_TRY(ctx, FNN_ERR_MEMORY,
+                    hipMemcpyAsync(out, dout, (size_t)(m * n) * 4, hipMemcpyDeviceToHost, ctx->stream));
+            HIP_TRY(ctx, FNN_ERR_DISPATCH, hipStreamSynchronize(ctx->stream));
         }
-        if (!handled) {
-            int rc = fnn_tiled_qmatmul(ctx, ctx->stream, w, p, flags, &handled);
-            if (rc) return rc;
-        }
-        if (!handled && !fma_first) HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qgemv(w->dtype, p, ctx->stream, &handled));
-    }
-    if (!handled) HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qgemm_generic(w->dtype, p, ctx->stream));
-    if (!dev) {
-        HIP_TRY(ctx, FNN_ERR_MEMORY,
-                hipMemcpyAsync(out, dout, (size_t)(m * n) * 4, hipMemcpyDeviceToHost, ctx->stream));
-        HIP_TRY(ctx, FNN_ERR_DISPATCH, hipStreamSynchronize(ctx->stream));
-    }
-    return FNN_OK;
+        return FNN_OK;
+    });
 }
 
 int fnn_hip_quantize_activations(fnn_hip_ctx *ctx, const float *x, int64_t numel, float scale,
                                  float zp, uint8_t *payload, int flags)
 {
-    if (!ctx || !x || !payload || numel < 0)
-        return fail(ctx, FNN_ERR_DISPATCH, "quantize_activations: NULL or invalid argument");
-    const bool dev = (flags & FNN_FLAG_DEVICE_PTRS) != 0;
-    const float *dx = x;
-    uint8_t *dp = payload;
-    if (!dev) {
-        int rc;
-        if ((rc = ensure(ctx, ctx->st_a, (size_t)numel * 4 + 16))) return rc;
-        if ((rc = ensure(ctx, ctx->st_out, (size_t)numel + 16))) return rc;
-        HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(ctx->st_a.ptr, x, (size_t)numel * 4, hipMemcpyHostToDevice, ctx->stream));
-        dx = (const float *)ctx->st_a.ptr;
-        dp = (uint8_t *)ctx->st_out.ptr;
-    }
-    HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_quantize_activations(dx, numel, scale, zp, dp, ctx->scratch, ctx->stream));
-    if (!dev) {
-        HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(payload, dp, (size_t)numel + 8, hipMemcpyDeviceToHost, ctx->stream));
-        HIP_TRY(ctx, FNN_ERR_DISPATCH, hipStreamSynchronize(ctx->stream));
-    }
-    return FNN_OK;
+    return guarded(ctx, "fnn_hip_quantize_activations", [&]() -> int {
+        if (!ctx || !x || !payload || numel < 0)
+            return fail(ctx, FNN_ERR_DISPATCH, "quantize_activations: NULL or invalid argument");
+        const bool dev = (flags & FNN_FLAG_DEVICE_PTRS) != 0;
+        const float *dx = x;
+        uint8_t *dp = payload;
+        if (!dev) {
+            int rc;
+            if ((rc = ensure(ctx, ctx->st_a, (size_t)numel * 4 + 16))) return rc;
+            if ((rc = ensure(ctx, ctx->st_out, (size_t)numel + 16))) return rc;
+            HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(ctx->st_a.ptr, x, (size_t)numel * 4, hipMemcpyHostToDevice, ctx->stream));
+            dx = (const float *)ctx->st_a.ptr;
+            dp = (uint8_t *)ctx->st_out.ptr;
+        }
+        HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_quantize_activations(dx, numel, scale, zp, dp, ctx->scratch, ctx->stream));
+        if (!dev) {
+            HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(payload, dp, (size_t)numel + 8, hipMemcpyDeviceToHost, ctx->stream));
+            HIP_TRY(ctx, FNN_ERR_DISPATCH, hipStreamSynchronize(ctx->stream));
+        }
+        return FNN_OK;
+    });
 }
 
 int fnn_hip_dequantize_activations(fnn_hip_ctx *ctx, const uint8_t *payload, uint64_t payload_len, float *out, uint64_t n)
 {
-    if (!ctx || ((!payload || !out) && n)) return fail(ctx, FNN_ERR_DISPATCH, "dequantize_activations: NULL argument");
-    if (reinterpret_cast<uintptr_t>(payload) & 3) return fail(ctx, FNN_ERR_DISPATCH, "dequantize_activations: payload must be 4-byte aligned");
-    HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_dequantize_activations(payload, payload_len, out, n, ctx->stream));
-    return FNN_OK;
+    return guarded(ctx, "fnn_hip_dequantize_activations", [&]() -> int {
+        if (!ctx || ((!payload || !out) && n)) return fail(ctx, FNN_ERR_DISPATCH, "dequantize_activations: NULL argument");
+        if (reinterpret_cast<uintptr_t>(payload) & 3) return fail(ctx, FNN_ERR_DISPATCH, "dequantize_activations: payload must be 4-byte aligned");
+        HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_dequantize_activations(payload, payload_len, out, n, ctx->stream));
+        return FNN_OK;
+    });
 }
 
 int fnn_hip_qmatmul_i8act(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const uint8_t *payload,
                           int64_t m, float *out, int32_t *acc_out, int flags)
 {
-    if (!ctx || !w) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_qmatmul_i8act: NULL context or weight");
-    if (w->dtype != FNN_DT_I8 && w->dtype != FNN_DT_I4)
-        return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "matmul_*_i8: weight dtype %d has no I8-activation kernel", w->dtype);
-    const char *kn = (w->dtype == FNN_DT_I8) ? "matmul_i8_i8" : "matmul_i4_i8";
-    if (m < 0) return fail(ctx, FNN_ERR_DISPATCH, "%s: expected params [M,K,N]", kn);
-    if (m == 0) return FNN_OK;
-    if (!payload || !out) return fail(ctx, FNN_ERR_DISPATCH, "%s: NULL payload or output pointer", kn);
-    const int64_t n = w->rows, k = w->inner;
-    const bool dev = (flags & FNN_FLAG_DEVICE_PTRS) != 0;
-    const uint8_t *dp = payload;
-    float *dout = out;
-    int32_t *dacc = acc_out;
-    if (!dev) {
-        int rc;
-        if ((rc = ensure(ctx, ctx->st_a, (size_t)(m * k) + 8 + 16))) return rc;
-        if ((rc = ensure(ctx, ctx->st_out, (size_t)(m * n) * 4))) return rc;
-        HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(ctx->st_a.ptr, payload, (size_t)(m * k) + 8, hipMemcpyHostToDevice, ctx->stream));
-        dp = (const uint8_t *)ctx->st_a.ptr;
-        dout = (float *)ctx->st_out.ptr;
-        if (acc_out) {
-            if ((rc = ensure(ctx, ctx->st_acc, (size_t)(m * n) * 4))) return rc;
-            dacc = (int32_t *)ctx->st_acc.ptr;
+    return guarded(ctx, "fnn_hip_qmatmul_i8act", [&]() -> int {
+        if (!ctx || !w) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_qmatmul_i8act: NULL context or weight");
+        if (w->dtype != FNN_DT_I8 && w->dtype != FNN_DT_I4)
+            return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "matmul_*_i8: weight dtype %d has no I8-activation kernel", w->dtype);
+        const char *kn = (w->dtype == FNN_DT_I8) ? "matmul_i8_i8" : "matmul_i4_i8";
+        if (m < 0) return fail(ctx, FNN_ERR_DISPATCH, "%s: expected params [M,K,N]", kn);
+        if (m == 0) return FNN_OK;
+        if (!payload || !out) return fail(ctx, FNN_ERR_DISPATCH, "%s: NULL payload or output pointer", kn);
+        const int64_t n = w->rows, k = w->inner;
+        const bool dev = (flags & FNN_FLAG_DEVICE_PTRS) != 0;
+        const uint8_t *dp = payload;
+        float *dout = out;
+        int32_t *dacc = acc_out;
+        if (!dev) {
+            int rc;
+            if ((rc = ensure(ctx, ctx->st_a, (size_t)(m * k) + 8 + 16))) return rc;
+            if ((rc = ensure(ctx, ctx->st_out, (size_t)(m * n) * 4))) return rc;
+            HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(ctx->st_a.ptr, payload, (size_t)(m * k) + 8, hipMemcpyHostToDevice, ctx->stream));
+            dp = (const uint8_t *)ctx->st_a.ptr;
+            dout = (float *)ctx->st_out.ptr;
+            if (acc_out) {
+                if ((rc = ensure(ctx, ctx->st_acc, (size_t)(m * n) * 4))) return rc;
+                dacc = (int32_t *)ctx->st_acc.ptr;
+            }
         }
-    }
-    I8ActArgs p;
-    p.words = w->words; p.scales = w->scales; p.zeros = w->zeros; p.payload = dp; p.out = dout;
-    p.acc_out = dacc; p.m = m; p.n = n; p.k = k; p.kp = w->kp;
-    bool handled = false;
-    if (!(flags & FNN_FLAG_FORCE_GENERIC)) {
-        int rc = fnn_i8_tiled_matmul(ctx, ctx->stream, w, p, &handled);
-        if (rc) return rc;
-    }
-    if (!handled) HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qgemm_i8act_generic(w->dtype, p, ctx->stream));
-    if (!dev) {
-        HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(out, dout, (size_t)(m * n) * 4, hipMemcpyDeviceToHost, ctx->stream));
-        if (acc_out)
-            HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(acc_out, dacc, (size_t)(m * n) * 4, hipMemcpyDeviceToHost, ctx->stream));
-        HIP_TRY(ctx, FNN_ERR_DISPATCH, hipStreamSynchronize(ctx->stream));
-    }
-    return FNN_OK;
+        I8ActArgs p;
+        p.words = w->words; p.scales = w->scales; p.zeros = w->zeros; p.payload = dp; p.out = dout;
+        p.acc_out = dacc; p.m = m; p.n = n; p.k = k; p.kp = w->kp;
+        bool handled = false;
+        if (!(flags & FNN_FLAG_FORCE_GENERIC)) {
+            int rc = fnn_i8_tiled_matmul(ctx, ctx->stream, w, p, &handled);
+            if (rc) return rc;
+        }
+        if (!handled) HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qgemm_i8act_generic(w->dtype, p, ctx->stream));
+        if (!dev) {
+            HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(out, dout, (size_t)(m * n) * 4, hipMemcpyDeviceToHost, ctx->stream));
+            if (acc_out)
+                HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(acc_out, dacc, (size_t)(m * n) * 4, hipMemcpyDeviceToHost, ctx->stream));
+            HIP_TRY(ctx, FNN_ERR_DISPATCH, hipStreamSynchronize(ctx->stream));
+        }
+        return FNN_OK;
+    });
 }
 
 int fnn_hip_qconv2d(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *x, int64_t b, int64_t c,
                     int64_t h, int64_t wd, int kh, int kw, int stride, int pad, int dil, int groups,
                     const float *bias, int act, float *y, int32_t *acc_out, int flags)
 {
-    if (!ctx) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_hip_qconv2d: NULL context");
-    if (!w) return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8: missing weight_meta for quantized weight");
-    const bool integer_kernel = w->dtype == FNN_DT_I8 || w->dtype == FNN_DT_I4;
-    if (!integer_kernel && acc_out)
-        return fail(ctx, FNN_ERR_DISPATCH, "conv2d: weight type %d runs as an f32 convolution and has no i32 accumulators", w->dtype);
-    if (groups <= 0) return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8: groups must be > 0");
-    if (b < 0 || c <= 0 || h <= 0 || wd <= 0 || kh <= 0 || kw <= 0 || stride <= 0 || dil <= 0 || pad < 0)
-        return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8: invalid geometry");
-    if (c % groups || w->rows % groups)
-        return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8: channels (%lld in, %lld out) not divisible by groups %d",
-                    (long long)c, (long long)w->rows, groups);
-    if (w->inner != (c / groups) * kh * kw)
-        return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8: weight inner dim %lld != C/g*KH*KW = %lld", (long long)w->inner,
-                    (long long)((c / groups) * kh * kw));
-    if (act < FNN_ACT_NONE || act > FNN_ACT_SILU) return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "conv2d_i8: unknown activation %d", act);
-    auto osz = [](int64_t in, int k, int s, int p, int d) -> int64_t {
-        int64_t dk = (int64_t)(k - 1) * d + 1;
-        return (in + 2 * p >= dk) ? (in + 2 * p - dk) / s + 1 : 0;
-    };
-    const int64_t ho = osz(h, kh, stride, pad, dil), wo = osz(wd, kw, stride, pad, dil);
-    const int64_t oc = w->rows;
-    if (b == 0 || ho == 0 || wo == 0) return FNN_OK;
-    if (!x || !y) return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8: NULL input or output pointer");
-    if (b * groups > 65535) return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "conv2d_i8: batch*groups > 65535");
-    const bool dev = (flags & FNN_FLAG_DEVICE_PTRS) != 0;
-    fnn_hip_weight *wm = const_cast<fnn_hip_weight *>(w);
-    if (integer_kernel && !wm->row_qsum) {
-        if (ctx->capturing) return fail(ctx, FNN_ERR_MEMORY, "conv2d_i8: first use of a weight during graph capture");
-        HIP_TRY(ctx, FNN_ERR_MEMORY, hipMalloc((void **)&wm->row_qsum, (size_t)oc * 4 + 64));
-        HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_row_qsum(w, wm->row_qsum, ctx->stream));
-    }
-    const size_t xin = (size_t)(b * c * h * wd) * 4, yout = (size_t)(b * oc * ho * wo) * 4;
-    const float *dx = x, *dbias = bias;
-    float *dy = y;
-    int32_t *dacc = acc_out;
-    int rc;
-    if (!dev) {
-        if ((rc = ensure(ctx, ctx->st_a, xin))) return rc;
-        if ((rc = ensure(ctx, ctx->st_out, yout))) return rc;
-        HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(ctx->st_a.ptr, x, xin, hipMemcpyHostToDevice, ctx->stream));
-        dx = (const float *)ctx->st_a.ptr;
-        dy = (float *)ctx->st_out.ptr;
-        if (bias) {
-            if ((rc = ensure(ctx, ctx->st_bias, (size_t)oc * 4))) return rc;
-            HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(ctx->st_bias.ptr, bias, (size_t)oc * 4, hipMemcpyHostToDevice, ctx->stream));
-            dbias = (const float *)ctx->st_bias.ptr;
+    return guarded(ctx, "fnn_hip_qconv2d", [&]() -> int {
+        if (!ctx) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_hip_qconv2d: NULL context");
+        if (!w) return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8: missing weight_meta for quantized weight");
+        const bool integer_kernel = w->dtype == FNN_DT_I8 || w->dtype == FNN_DT_I4;
+        if (!integer_kernel && acc_out)
+            return fail(ctx, FNN_ERR_DISPATCH, "conv2d: weight type %d runs as an f32 convolution and has no i32 accumulators", w->dtype);
+        if (groups <= 0) return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8: groups must be > 0");
+        if (b < 0 || c <= 0 || h <= 0 || wd <= 0 || kh <= 0 || kw <= 0 || stride <= 0 || dil <= 0 || pad < 0)
+            return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8: invalid geometry");
+        if (c % groups || w->rows % groups)
+            return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8: channels (%lld in, %lld out) not divisible by groups %d",
+                        (long long)c, (long long)w->rows, groups);
+        if (w->inner != (c / groups) * kh * kw)
+            return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8: weight inner dim %lld != C/g*KH*KW = %lld", (long long)w->inner,
+                        (long long)((c / groups) * kh * kw));
+        if (act < FNN_ACT_NONE || act > FNN_ACT_SILU) return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "conv2d_i8: unknown activation %d", act);
+        auto osz = [](int64_t in, int k, int s, int p, int d) -> int64_t {
+            int64_t dk = (int64_t)(k - 1) * d + 1;
+            return (in + 2 * p >= dk) ? (in + 2 * p - dk) / s + 1 : 0;
+        };
+        const int64_t ho = osz(h, kh, stride, pad, dil), wo = osz(wd, kw, stride, pad, dil);
+        const int64_t oc = w->rows;
+        if (b == 0 || ho == 0 || wo == 0) return FNN_OK;
+        if (!x || !y) return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8: NULL input or output pointer");
+        if (b * groups > 65535) return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "conv2d_i8: batch*groups > 65535");
+        const bool dev = (flags & FNN_FLAG_DEVICE_PTRS) != 0;
+        fnn_hip_weight *wm = const_cast<fnn_hip_weight *>(w);
+        if (integer_kernel && !wm->row_qsum) {
+            if (ctx->capturing) return fail(ctx, FNN_ERR_MEMORY, "conv2d_i8: first use of a weight during graph capture");
+            HIP_TRY(ctx, FNN_ERR_MEMORY, hipMalloc((void **)&wm->row_qsum, (size_t)oc * 4 + 64));
+            HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_row_qsum(w, wm->row_qsum, ctx->stream));
         }
-        if (acc_out) {
-            if ((rc = ensure(ctx, ctx->st_acc, yout))) return rc;
-            dacc = (int32_t *)ctx->st_acc.ptr;
-        }
-    }
-    if (!integer_kernel) {
-        // f32 convolution with dequantised weights (src/backend/cpu/mod.rs:4204-4257): im2col rows,
-        // fused-dequant MatMul per group (bias and activation in its epilogue), [pixel, channel] -> NCHW
-        const int64_t cg = c / groups, ocg = oc / groups, kk = cg * kh * kw, np = ho * wo, rows = b * np;
-        if (rows > (1ll << 31) || b > 65535) return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "conv2d: %lld output pixels exceed the f32 path's limit", (long long)rows);
-        if ((rc = ensure(ctx, ctx->st_col, (size_t)rows * kk * 4 + 256))) return rc;
-        if ((rc = ensure(ctx, ctx->st_rows, (size_t)rows * ocg * 4 + 256))) return rc;
-        float *col = (float *)ctx->st_col.ptr, *rows_out = (float *)ctx->st_rows.ptr;
-        for (int g = 0; g < groups; g++) {
-            HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_im2col_f32(dx, col, b, c, groups, g, h, wd, ho, wo, kh, kw, stride, pad, dil, ctx->stream));
-            if (groups == 1) {
-                if ((rc = fnn_hip_qmatmul(ctx, w, col, rows, dbias, act, rows_out, FNN_FLAG_DEVICE_PTRS | (flags & (FNN_FLAG_FORCE_GENERIC | FNN_FLAG_ACT_F16_SINGLE))))) return rc;
-            } else {
-                // a slice of the weight rows: the shape-agnostic kernel takes the offset pointers as they are
-                QMatmulArgs q;
-                q.words = w->words + (size_t)g * ocg * w->kp;
-                q.scales = w->dtype == FNN_DT_I4CB ? w->scales + (size_t)g * ocg * w->bpr : w->scales + (size_t)g * ocg;
-                q.zeros = w->zeros ? w->zeros + (size_t)g * ocg : nullptr;
-                q.codebook = w->codebook;
-                q.a = col; q.bias = dbias ? dbias + (size_t)g * ocg : nullptr; q.out = rows_out;
-                q.m = rows; q.n = ocg; q.k = kk; q.kp = w->kp; q.bpr = w->bpr; q.qblock = w->qblock; q.act = act;
-                q.as_written = 0;
-                HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qgemm_generic(w->dtype, q, ctx->stream));
+        const size_t xin = (size_t)(b * c * h * wd) * 4, yout = (size_t)(b * oc * ho * wo) * 4;
+        const float *dx = x, *dbias = bias;
+        float *dy = y;
+        int32_t *dacc = acc_out;
+        int rc;
+        if (!dev) {
+            if ((rc = ensure(ctx, ctx->st_a, xin))) return rc;
+            if ((rc = ensure(ctx, ctx->st_out, yout))) return rc;
+            HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(ctx->st_a.ptr, x, xin, hipMemcpyHostToDevice, ctx->stream));
+            dx = (const float *)ctx->st_a.ptr;
+            dy = (float *)ctx->st_out.ptr;
+            if (bias) {
+                if ((rc = ensure(ctx, ctx->st_bias, (size_t)oc * 4))) return rc;
+                HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(ctx->st_bias.ptr, bias, (size_t)oc * 4, hipMemcpyHostToDevice, ctx->stream));
+                dbias = (const float *)ctx->st_bias.ptr;
             }
-            HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_rows_to_nchw(rows_out, dy, b, np, oc, (int64_t)g * ocg, ocg, ctx->stream));
+            if (acc_out) {
+                if ((rc = ensure(ctx, ctx->st_acc, yout))) return rc;
+                dacc = (int32_t *)ctx->st_acc.ptr;
+            }
+        }
+        if (!integer_kernel) {
+            // f32 convolution with dequantised weights (src/backend/cpu/mod.rs:4204-4257): im2col rows,
+            // fused-dequant MatMul per group (bias and activation in its epilogue), [pixel, channel] -> NCHW
+            const int64_t cg = c / groups, ocg = oc / groups, kk = cg * kh * kw, np = ho * wo, rows = b * np;
+            if (rows > (1ll << 31) || b > 65535) return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "conv2d: %lld output pixels exceed the f32 path's limit", (long long)rows);
+            if ((rc = ensure(ctx, ctx->st_col, (size_t)rows * kk * 4 + 256))) return rc;
+            if ((rc = ensure(ctx, ctx->st_rows, (size_t)rows * ocg * 4 + 256))) return rc;
+            float *col = (float *)ctx->st_col.ptr, *rows_out = (float *)ctx->st_rows.ptr;
+            for (int g = 0; g < groups; g++) {
+                HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_im2col_f32(dx, col, b, c, groups, g, h, wd, ho, wo, kh, kw, stride, pad, dil, ctx->stream));
+                if (groups == 1) {
+                    if ((rc = fnn_hip_qmatmul(ctx, w, col, rows, dbias, act, rows_out, FNN_FLAG_DEVICE_PTRS | (flags & (FNN_FLAG_FORCE_GENERIC | FNN_FLAG_ACT_F16_SINGLE))))) return rc;
+                } else {
+                    // a slice of the weight rows: the shape-agnostic kernel takes the offset pointers as they are
+                    QMatmulArgs q;
+                    q.words = w->words + (size_t)g * ocg * w->kp;
+                    q.scales = w->dtype == FNN_DT_I4CB ? w->scales + (size_t)g * ocg * w->bpr : w->scales + (size_t)g * ocg;
+                    q.zeros = w->zeros ? w->zeros + (size_t)g * ocg : nullptr;
+                    q.codebook = w->codebook;
+                    q.a = col; q.bias = dbias ? dbias + (size_t)g * ocg : nullptr; q.out = rows_out;
+                    q.m = rows; q.n = ocg; q.k = kk; q.kp = w->kp; q.bpr = w->bpr; q.qblock = w->qblock; q.act = act;
+                    q.as_written = 0;
+                    HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qgemm_generic(w->dtype, q, ctx->stream));
+                }
+                HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_rows_to_nchw(rows_out, dy, b, np, oc, (int64_t)g * ocg, ocg, ctx->stream));
+            }
+            if (!dev) {
+                HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(y, dy, yout, hipMemcpyDeviceToHost, ctx->stream));
+                HIP_TRY(ctx, FNN_ERR_DISPATCH, hipStreamSynchronize(ctx->stream));
+            }
+            return FNN_OK;
+        }
+        if ((rc = ensure(ctx, ctx->st_tmp, (size_t)(b * groups) * (QCONV_NPART * 2 + 4) * 4))) return rc;
+        QConvArgs p;
+        p.words = w->words; p.scales = w->scales; p.zeros = w->zeros; p.row_qsum = wm->row_qsum;
+        p.x = dx; p.bias = dbias; p.y = dy; p.acc_out = dacc;
+        p.minmax_partial = (float *)ctx->st_tmp.ptr;
+        p.actq = p.minmax_partial + (size_t)(b * groups) * QCONV_NPART * 2;
+        p.b = b; p.c = c; p.h = h; p.w = wd; p.oc = oc; p.ho = ho; p.wo = wo; p.kp = w->kp;
+        p.kh = kh; p.kw = kw; p.stride = stride; p.pad = pad; p.dil = dil; p.groups = groups; p.act = act;
+        p.wbits = w->dtype == FNN_DT_I4 ? 4 : 8;
+        p.x8 = nullptr; p.payload_i4 = 0; p.nparts = 0;
+        if (flags & FNN_FLAG_FORCE_GENERIC) {
+            HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qconv2d_i8(p, ctx->stream, 0, nullptr));
+        } else {
+            // range scan; the scales are then formed by the operand kernel itself (one launch less) when a workgroup's
+            // 64 rows touch at most two images, else by the small kernel of their own
+            int nparts = 0;
+            HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qconv2d_i8(p, ctx->stream, 3, &nparts));
+            const int64_t kk_g = (c / groups) * kh * kw;
+            const int64_t operand_wgs = ((b * ho * wo + 63) / 64) * (((kk_g + 15) / 16 + 3) / 4);
+            const bool fused_scales = ho * wo >= 64 && nparts <= QCONV_NPART && operand_wgs <= 8192;   // many workgroups: cheaper once
+            if (fused_scales) p.nparts = nparts;
+            else HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qconv2d_i8(p, ctx->stream, 4, &nparts));
+            bool handled = false;
+            int rc2 = fnn_i8_tiled_conv(ctx, ctx->stream, w, p, &handled);
+            if (rc2) return rc2;
+            if (!handled) {
+                if (fused_scales) HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qconv2d_i8(p, ctx->stream, 4, &nparts));
+                p.nparts = 0;
+                HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qconv2d_i8(p, ctx->stream, 2, nullptr));
+            }
         }
         if (!dev) {
             HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(y, dy, yout, hipMemcpyDeviceToHost, ctx->stream));
+            if (acc_out) HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(acc_out, dacc, yout, hipMemcpyDeviceToHost, ctx->stream));
             HIP_TRY(ctx, FNN_ERR_DISPATCH, hipStreamSynchronize(ctx->stream));
         }
         return FNN_OK;
-    }
-    if ((rc = ensure(ctx, ctx->st_tmp, (size_t)(b * groups) * (QCONV_NPART * 2 + 4) * 4))) return rc;
-    QConvArgs p;
-    p.words = w->words; p.scales = w->scales; p.zeros = w->zeros; p.row_qsum = wm->row_qsum;
-    p.x = dx; p.bias = dbias; p.y = dy; p.acc_out = dacc;
-    p.minmax_partial = (float *)ctx->st_tmp.ptr;
-    p.actq = p.minmax_partial + (size_t)(b * groups) * QCONV_NPART * 2;
-    p.b = b; p.c = c; p.h = h; p.w = wd; p.oc = oc; p.ho = ho; p.wo = wo; p.kp = w->kp;
-    p.kh = kh; p.kw = kw; p.stride = stride; p.pad = pad; p.dil = dil; p.groups = groups; p.act = act;
-    p.wbits = w->dtype == FNN_DT_I4 ? 4 : 8;
-    p.x8 = nullptr; p.payload_i4 = 0; p.nparts = 0;
-    if (flags & FNN_FLAG_FORCE_GENERIC) {
-        HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qconv2d_i8(p, ctx->stream, 0, nullptr));
-    } else {
-        // range scan; the scales are then formed by the operand kernel itself (one launch less) when a workgroup's
-        // 64 rows touch at most two images, else by the small kernel of their own
-        int nparts = 0;
-        HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qconv2d_i8(p, ctx->stream, 3, &nparts));
-        const int64_t kk_g = (c / groups) * kh * kw;
-        const int64_t operand_wgs = ((b * ho * wo + 63) / 64) * (((kk_g + 15) / 16 + 3) / 4);
-        const bool fused_scales = ho * wo >= 64 && nparts <= QCONV_NPART && operand_wgs <= 8192;   // many workgroups: cheaper once
-        if (fused_scales) p.nparts = nparts;
-        else HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qconv2d_i8(p, ctx->stream, 4, &nparts));
-        bool handled = false;
-        int rc2 = fnn_i8_tiled_conv(ctx, ctx->stream, w, p, &handled);
-        if (rc2) return rc2;
-        if (!handled) {
-            if (fused_scales) HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qconv2d_i8(p, ctx->stream, 4, &nparts));
-            p.nparts = 0;
-            HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qconv2d_i8(p, ctx->stream, 2, nullptr));
-        }
-    }
-    if (!dev) {
-        HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(y, dy, yout, hipMemcpyDeviceToHost, ctx->stream));
-        if (acc_out) HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(acc_out, dacc, yout, hipMemcpyDeviceToHost, ctx->stream));
-        HIP_TRY(ctx, FNN_ERR_DISPATCH, hipStreamSynchronize(ctx->stream));
-    }
-    return FNN_OK;
+    });
 }
 
 int fnn_hip_qconv2d_i8act(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const uint8_t *payload, int64_t b, int64_t c,
                           int64_t h, int64_t wd, int kh, int kw, int stride, int pad, int dil, int groups,
                           const float *bias, int act, float *y, int flags)
 {
-    if (!ctx) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_hip_qconv2d_i8act: NULL context");
-    if (!w) return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8_i8: missing weight_meta for quantized weight");
-    if (w->dtype != FNN_DT_I8 && w->dtype != FNN_DT_I4)
-        return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "conv2d_i8_i8: weight type %d has no I8-activation kernel", w->dtype);
-    if (groups <= 0) return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8_i8: groups must be > 0");
-    if (b < 0 || c <= 0 || h <= 0 || wd <= 0 || kh <= 0 || kw <= 0 || stride <= 0 || dil <= 0 || pad < 0)
-        return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8_i8: invalid geometry");
-    if (c % groups || w->rows % groups)
-        return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8_i8: channels (%lld in, %lld out) not divisible by groups %d",
-                    (long long)c, (long long)w->rows, groups);
-    if (w->inner != (c / groups) * kh * kw)
-        return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8_i8: weight inner dim %lld != C/g*KH*KW = %lld", (long long)w->inner,
-                    (long long)((c / groups) * kh * kw));
-    if (act < FNN_ACT_NONE || act > FNN_ACT_SILU) return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "conv2d_i8_i8: unknown activation %d", act);
-    auto osz = [](int64_t in, int k, int s, int p, int d) -> int64_t {
-        int64_t dk = (int64_t)(k - 1) * d + 1;
-        return (in + 2 * p >= dk) ? (in + 2 * p - dk) / s + 1 : 0;
-    };
-    const int64_t ho = osz(h, kh, stride, pad, dil), wo = osz(wd, kw, stride, pad, dil);
-    const int64_t oc = w->rows;
-    if (b == 0 || ho == 0 || wo == 0) return FNN_OK;
-    if (!payload || !y) return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8_i8: NULL input or output pointer");
-    if (b * groups > 65535) return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "conv2d_i8_i8: batch*groups > 65535");
-    const bool dev = (flags & FNN_FLAG_DEVICE_PTRS) != 0;
-    if (dev && (reinterpret_cast<uintptr_t>(payload) & 3))
-        return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8_i8: activation payload must be 4-byte aligned");
-    fnn_hip_weight *wm = const_cast<fnn_hip_weight *>(w);
-    if (!wm->row_qsum) {
-        if (ctx->capturing) return fail(ctx, FNN_ERR_MEMORY, "conv2d_i8_i8: first use of a weight during graph capture");
-        HIP_TRY(ctx, FNN_ERR_MEMORY, hipMalloc((void **)&wm->row_qsum, (size_t)oc * 4 + 64));
-        HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_row_qsum(w, wm->row_qsum, ctx->stream));
-    }
-    const size_t xin = (size_t)(b * c * h * wd) + 8, yout = (size_t)(b * oc * ho * wo) * 4;
-    const uint8_t *dp = payload;
-    const float *dbias = bias;
-    float *dy = y;
-    int rc;
-    if (!dev) {
-        if ((rc = ensure(ctx, ctx->st_a, xin))) return rc;
-        if ((rc = ensure(ctx, ctx->st_out, yout))) return rc;
-        HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(ctx->st_a.ptr, payload, xin, hipMemcpyHostToDevice, ctx->stream));
-        dp = (const uint8_t *)ctx->st_a.ptr;
-        dy = (float *)ctx->st_out.ptr;
-        if (bias) {
-            if ((rc = ensure(ctx, ctx->st_bias, (size_t)oc * 4))) return rc;
-            HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(ctx->st_bias.ptr, bias, (size_t)oc * 4, hipMemcpyHostToDevice, ctx->stream));
-            dbias = (const float *)ctx->st_bias.ptr;
+    return guarded(ctx, "fnn_hip_qconv2d_i8act", [&]() -> int {
+        if (!ctx) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_hip_qconv2d_i8act: NULL context");
+        if (!w) return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8_i8: missing weight_meta for quantized weight");
+        if (w->dtype != FNN_DT_I8 && w->dtype != FNN_DT_I4)
+            return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "conv2d_i8_i8: weight type %d has no I8-activation kernel", w->dtype);
+        if (groups <= 0) return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8_i8: groups must be > 0");
+        if (b < 0 || c <= 0 || h <= 0 || wd <= 0 || kh <= 0 || kw <= 0 || stride <= 0 || dil <= 0 || pad < 0)
+            return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8_i8: invalid geometry");
+        if (c % groups || w->rows % groups)
+            return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8_i8: channels (%lld in, %lld out) not divisible by groups %d",
+                        (long long)c, (long long)w->rows, groups);
+        if (w->inner != (c / groups) * kh * kw)
+            return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8_i8: weight inner dim %lld != C/g*KH*KW = %lld", (long long)w->inner,
+                        (long long)((c / groups) * kh * kw));
+        if (act < FNN_ACT_NONE || act > FNN_ACT_SILU) return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "conv2d_i8_i8: unknown activation %d", act);
+        auto osz = [](int64_t in, int k, int s, int p, int d) -> int64_t {
+            int64_t dk = (int64_t)(k - 1) * d + 1;
+            return (in + 2 * p >= dk) ? (in + 2 * p - dk) / s + 1 : 0;
+        };
+        const int64_t ho = osz(h, kh, stride, pad, dil), wo = osz(wd, kw, stride, pad, dil);
+        const int64_t oc = w->rows;
+        if (b == 0 || ho == 0 || wo == 0) return FNN_OK;
+        if (!payload || !y) return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8_i8: NULL input or output pointer");
+        if (b * groups > 65535) return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "conv2d_i8_i8: batch*groups > 65535");
+        const bool dev = (flags & FNN_FLAG_DEVICE_PTRS) != 0;
+        if (dev && (reinterpret_cast<uintptr_t>(payload) & 3))
+            return fail(ctx, FNN_ERR_DISPATCH, "conv2d_i8_i8: activation payload must be 4-byte aligned");
+        fnn_hip_weight *wm = const_cast<fnn_hip_weight *>(w);
+        if (!wm->row_qsum) {
+            if (ctx->capturing) return fail(ctx, FNN_ERR_MEMORY, "conv2d_i8_i8: first use of a weight during graph capture");
+            HIP_TRY(ctx, FNN_ERR_MEMORY, hipMalloc((void **)&wm->row_qsum, (size_t)oc * 4 + 64));
+            HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_row_qsum(w, wm->row_qsum, ctx->stream));
         }
-    }
-    if ((rc = ensure(ctx, ctx->st_tmp, (size_t)(b * groups) * (QCONV_NPART * 2 + 4) * 4))) return rc;
-    QConvArgs p;
-    p.words = w->words; p.scales = w->scales; p.zeros = w->zeros; p.row_qsum = wm->row_qsum;
-    p.x = nullptr; p.bias = dbias; p.y = dy; p.acc_out = nullptr;
-    p.minmax_partial = (float *)ctx->st_tmp.ptr;
-    p.actq = p.minmax_partial + (size_t)(b * groups) * QCONV_NPART * 2;
-    p.b = b; p.c = c; p.h = h; p.w = wd; p.oc = oc; p.ho = ho; p.wo = wo; p.kp = w->kp;
-    p.kh = kh; p.kw = kw; p.stride = stride; p.pad = pad; p.dil = dil; p.groups = groups; p.act = act;
-    p.wbits = w->dtype == FNN_DT_I4 ? 4 : 8;
-    p.x8 = reinterpret_cast<const int8_t *>(dp + 8);
-    p.payload_i4 = w->dtype == FNN_DT_I4; p.nparts = 0;
-    HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_conv_actq_from_payload(dp, p.actq, (int)(b * groups), ctx->stream));
-    bool handled = false;
-    if ((rc = fnn_i8_tiled_conv(ctx, ctx->stream, w, p, &handled))) return rc;
-    if (!handled) return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "conv2d_i8_i8: shape outside the integer GEMM's limits");
-    if (!dev) {
-        HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(y, dy, yout, hipMemcpyDeviceToHost, ctx->stream));
-        HIP_TRY(ctx, FNN_ERR_DISPATCH, hipStreamSynchronize(ctx->stream));
-    }
-    return FNN_OK;
-}
-
-int fnn_hip_probe_stream(fnn_hip_ctx *ctx, const void *src_dev, void *dst_dev, size_t bytes)
-{
-    if (!ctx || !src_dev) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_probe_stream: NULL argument");
-    if ((reinterpret_cast<uintptr_t>(src_dev) & 15) || (reinterpret_cast<uintptr_t>(dst_dev) & 15))
-        return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_probe_stream: pointers must be 16-byte aligned");
-    HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_probe(src_dev, dst_dev, bytes, reinterpret_cast<uint32_t *>(ctx->scratch), ctx->stream));
-    return FNN_OK;
+        const size_t xin = (size_t)(b * c * h * wd) + 8, yout = (size_t)(b * oc * ho * wo) * 4;
+        const uint8_t *dp = payload;
+        const float *dbias = bias;
+        float *dy = y;
+        int rc;
+        if (!dev) {
+            if ((rc = ensure(ctx, ctx->st_a, xin))) return rc;
+            if ((rc = ensure(ctx, ctx->st_out, yout))) return rc;
+            HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(ctx->st_a.ptr, payload, xin, hipMemcpyHostToDevice, ctx->stream));
+            dp = (const uint8_t *)ctx->st_a.ptr;
+            dy = (float *)ctx->st_out.ptr;
+            if (bias) {
+                if ((rc = ensure(ctx, ctx->st_bias, (size_t)oc * 4))) return rc;
+                HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(ctx->st_bias.ptr, bias, (size_t)oc * 4, hipMemcpyHostToDevice, ctx->stream));
+                dbias = (const float *)ctx->st_bias.ptr;
+            }
+        }
+        if ((rc = ensure(ctx, ctx->st_tmp, (size_t)(b * groups) * (QCONV_NPART * 2 + 4) * 4))) return rc;
+        QConvArgs p;
+        p.words = w->words; p.scales = w->scales; p.zeros = w->zeros; p.row_qsum = wm->row_qsum;
+        p.x = nullptr; p.bias = dbias; p.y = dy; p.acc_out = nullptr;
+        p.minmax_partial = (float *)ctx->st_tmp.ptr;
+        p.actq = p.minmax_partial + (size_t)(b * groups) * QCONV_NPART * 2;
+        p.b = b; p.c = c; p.h = h; p.w = wd; p.oc = oc; p.ho = ho; p.wo = wo; p.kp = w->kp;
+        p.kh = kh; p.kw = kw; p.stride = stride; p.pad = pad; p.dil = dil; p.groups = groups; p.act = act;
+        p.wbits = w->dtype == FNN_DT_I4 ? 4 : 8;
+        p.x8 = reinterpret_cast<const int8_t *>(dp + 8);
+        p.payload_i4 = w->dtype == FNN_DT_I4; p.nparts = 0;
+        HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_conv_actq_from_payload(dp, p.actq, (int)(b * groups), ctx->stream));
+        bool handled = false;
+        if ((rc = fnn_i8_tiled_conv(ctx, ctx->stream, w, p, &handled))) return rc;
+        if (!handled) return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "conv2d_i8_i8: shape outside the integer GEMM's limits");
+        if (!dev) {
+            HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(y, dy, yout, hipMemcpyDeviceToHost, ctx->stream));
+            HIP_TRY(ctx, FNN_ERR_DISPATCH, hipStreamSynchronize(ctx->stream));
+        }
+        return FNN_OK;
+    });
 }
 
 int fnn_hip_elementwise(fnn_hip_ctx *ctx, int op, const float *a, const float *b, uint64_t nb, float *out, uint64_t n)
 {
-    if (!ctx || !a || !out) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_elementwise: NULL argument");
-    if (op < 0 || op > 3) return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "fnn_hip_elementwise: unknown op %d", op);
-    if (op == 0 && (!b || nb == 0)) return fail(ctx, FNN_ERR_DISPATCH, "add_f32: missing second operand");
-    HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_eltwise(op, a, b, nb, out, n, ctx->stream));
-    return FNN_OK;
+    return guarded(ctx, "fnn_hip_elementwise", [&]() -> int {
+        if (!ctx || !a || !out) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_elementwise: NULL argument");
+        if (op < 0 || op > 3) return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "fnn_hip_elementwise: unknown op %d", op);
+        if (op == 0 && (!b || nb == 0)) return fail(ctx, FNN_ERR_DISPATCH, "add_f32: missing second operand");
+        HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_eltwise(op, a, b, nb, out, n, ctx->stream));
+        return FNN_OK;
+    });
 }
 
 int fnn_hip_fill_f32(fnn_hip_ctx *ctx, float *dst, uint64_t n, float value)
 {
-    if (!ctx || (!dst && n)) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_fill_f32: NULL argument");
-    HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_fill(dst, n, value, ctx->stream));
-    return FNN_OK;
+    return guarded(ctx, "fnn_hip_fill_f32", [&]() -> int {
+        if (!ctx || (!dst && n)) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_fill_f32: NULL argument");
+        HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_fill(dst, n, value, ctx->stream));
+        return FNN_OK;
+    });
 }
 
 int fnn_hip_copy(fnn_hip_ctx *ctx, void *dst_dev, const void *src_dev, uint64_t bytes)
 {
-    if (!ctx || ((!dst_dev || !src_dev) && bytes)) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_copy: NULL argument");
-    if (bytes == 0) return FNN_OK;
-    HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(dst_dev, src_dev, bytes, hipMemcpyDeviceToDevice, ctx->stream));
-    return FNN_OK;
+    return guarded(ctx, "fnn_hip_copy", [&]() -> int {
+        if (!ctx || ((!dst_dev || !src_dev) && bytes)) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_copy: NULL argument");
+        if (bytes == 0) return FNN_OK;
+        HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(dst_dev, src_dev, bytes, hipMemcpyDeviceToDevice, ctx->stream));
+        return FNN_OK;
+    });
 }
 
 int fnn_hip_copy2d_f32(fnn_hip_ctx *ctx, float *dst, uint64_t dst_pitch, uint64_t dst_len, const float *src, uint64_t src_pitch,
                        uint64_t src_len, uint64_t width, uint64_t height)
 {
-    if (!ctx || ((!dst || !src) && width && height)) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_copy2d_f32: NULL argument");
-    HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_copy2d(dst, dst_pitch, dst_len, src, src_pitch, src_len, width, height, ctx->stream));
-    return FNN_OK;
+    return guarded(ctx, "fnn_hip_copy2d_f32", [&]() -> int {
+        if (!ctx || ((!dst || !src) && width && height)) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_copy2d_f32: NULL argument");
+        HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_copy2d(dst, dst_pitch, dst_len, src, src_pitch, src_len, width, height, ctx->stream));
+        return FNN_OK;
+    });
 }
 
 int fnn_hip_maxpool2d_f32(fnn_hip_ctx *ctx, const float *x, uint64_t in_len, float *y, uint64_t out_len, uint64_t n, uint64_t c,
-                          uint64_t h, uint64_t w, uint64_t kernel, uint64_t stride, uint64_t pad)
+                          uint64_t h, uint64_t w, uint64_t kernel, uint64_t stride, uint64_t pad, int64_t *indices, uint64_t idx_len)
 {
-    if (!ctx || !x || !y) return fail(ctx, FNN_ERR_DISPATCH, "pool_f32: NULL argument");
-    if (kernel == 0 || stride == 0 || kernel > 1024 || pad > 1024) return fail(ctx, FNN_ERR_DISPATCH, "pool_f32: invalid kernel, stride or padding");
-    const uint64_t hp = h + 2 * pad, wp = w + 2 * pad;
-    const uint64_t ho = (hp > kernel ? hp - kernel : 0) / stride + 1, wo = (wp > kernel ? wp - kernel : 0) / stride + 1;
-    uint64_t total = n * c * ho * wo;
-    if (total > out_len) total = out_len;   // writes past the output slice are dropped (ops.rs:147-149)
-    HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_maxpool2d(x, in_len, y, total, c, h, w, ho, wo, (int)kernel, (int)stride, (int)pad, ctx->stream));
-    return FNN_OK;
+    return guarded(ctx, "fnn_hip_maxpool2d_f32", [&]() -> int {
+        if (!ctx || !x || !y) return fail(ctx, FNN_ERR_DISPATCH, "pool_f32: NULL argument");
+        if (kernel == 0 || stride == 0 || kernel > 1024 || pad > 1024) return fail(ctx, FNN_ERR_DISPATCH, "pool_f32: invalid kernel, stride or padding");
+        const uint64_t hp = h + 2 * pad, wp = w + 2 * pad;
+        const uint64_t ho = (hp > kernel ? hp - kernel : 0) / stride + 1, wo = (wp > kernel ? wp - kernel : 0) / stride + 1;
+        uint64_t total = n * c * ho * wo;
+        if (total > out_len) total = out_len;   // writes past the output slice are dropped (ops.rs:147-149)
+        HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_maxpool2d(x, in_len, y, total, c, h, w, ho, wo, (int)kernel, (int)stride, (int)pad, indices,
+                                                         indices ? (idx_len < n * c * ho * wo ? idx_len : n * c * ho * wo) : 0, ctx->stream));
+        return FNN_OK;
+    });
 }
 
 int fnn_hip_avgpool2d_f32(fnn_hip_ctx *ctx, const float *x, uint64_t in_len, float *y, uint64_t out_len, uint64_t n, uint64_t c,
                           uint64_t h, uint64_t w, uint64_t kernel, uint64_t stride, uint64_t pad)
 {
-    if (!ctx || !x || !y) return fail(ctx, FNN_ERR_DISPATCH, "pool_f32: NULL argument");
-    if (kernel == 0 || stride == 0 || kernel > 1024 || pad > 1024) return fail(ctx, FNN_ERR_DISPATCH, "pool_f32: invalid kernel, stride or padding");
-    const uint64_t hp = h + 2 * pad, wp = w + 2 * pad;
-    const uint64_t ho = (hp > kernel ? hp - kernel : 0) / stride + 1, wo = (wp > kernel ? wp - kernel : 0) / stride + 1;
-    uint64_t total = n * c * ho * wo;
-    if (total > out_len) total = out_len;   // writes past the output slice are dropped (ops.rs:203-205)
-    HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_avgpool2d(x, in_len, y, total, h, w, ho, wo, (int)kernel, (int)stride, (int)pad, ctx->stream));
-    return FNN_OK;
+    return guarded(ctx, "fnn_hip_avgpool2d_f32", [&]() -> int {
+        if (!ctx || !x || !y) return fail(ctx, FNN_ERR_DISPATCH, "pool_f32: NULL argument");
+        if (kernel == 0 || stride == 0 || kernel > 1024 || pad > 1024) return fail(ctx, FNN_ERR_DISPATCH, "pool_f32: invalid kernel, stride or padding");
+        const uint64_t hp = h + 2 * pad, wp = w + 2 * pad;
+        const uint64_t ho = (hp > kernel ? hp - kernel : 0) / stride + 1, wo = (wp > kernel ? wp - kernel : 0) / stride + 1;
+        uint64_t total = n * c * ho * wo;
+        if (total > out_len) total = out_len;   // writes past the output slice are dropped (ops.rs:203-205)
+        HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_avgpool2d(x, in_len, y, total, h, w, ho, wo, (int)kernel, (int)stride, (int)pad, ctx->stream));
+        return FNN_OK;
+    });
 }
 
 int fnn_hip_upsample_nearest2d_f32(fnn_hip_ctx *ctx, const float *x, float *y, uint64_t nc, uint64_t h, uint64_t w, uint64_t sh, uint64_t sw)
 {
-    if (!ctx || !x || !y) return fail(ctx, FNN_ERR_DISPATCH, "upsample_nearest2d: NULL argument");
-    if (sh > 1024 || sw > 1024) return fail(ctx, FNN_ERR_DISPATCH, "upsample_nearest2d: scale too large");
-    HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_upsample_nearest2d(x, y, nc, h, w, (int)sh, (int)sw, ctx->stream));
-    return FNN_OK;
+    return guarded(ctx, "fnn_hip_upsample_nearest2d_f32", [&]() -> int {
+        if (!ctx || !x || !y) return fail(ctx, FNN_ERR_DISPATCH, "upsample_nearest2d: NULL argument");
+        if (sh > 1024 || sw > 1024) return fail(ctx, FNN_ERR_DISPATCH, "upsample_nearest2d: scale too large");
+        HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_upsample_nearest2d(x, y, nc, h, w, (int)sh, (int)sw, ctx->stream));
+        return FNN_OK;
+    });
 }
 
 int fnn_hip_timer_start(fnn_hip_ctx *ctx)
 {
-    if (!ctx) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_hip_timer_start: NULL context");
-    HIP_TRY(ctx, FNN_ERR_DISPATCH, hipEventRecord(ctx->ev0, ctx->stream));
-    return FNN_OK;
+    return guarded(ctx, "fnn_hip_timer_start", [&]() -> int {
+        if (!ctx) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_hip_timer_start: NULL context");
+        HIP_TRY(ctx, FNN_ERR_DISPATCH, hipEventRecord(ctx->ev0, ctx->stream));
+        return FNN_OK;
+    });
 }
 
 int fnn_hip_timer_stop(fnn_hip_ctx *ctx, float *ms)
 {
-    if (!ctx || !ms) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_timer_stop: NULL argument");
-    HIP_TRY(ctx, FNN_ERR_DISPATCH, hipEventRecord(ctx->ev1, ctx->stream));
-    HIP_TRY(ctx, FNN_ERR_DISPATCH, hipEventSynchronize(ctx->ev1));
-    HIP_TRY(ctx, FNN_ERR_DISPATCH, hipEventElapsedTime(ms, ctx->ev0, ctx->ev1));
-    return FNN_OK;
+    return guarded(ctx, "fnn_hip_timer_stop", [&]() -> int {
+        if (!ctx || !ms) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_timer_stop: NULL argument");
+        HIP_TRY(ctx, FNN_ERR_DISPATCH, hipEventRecord(ctx->ev1, ctx->stream));
+        HIP_TRY(ctx, FNN_ERR_DISPATCH, hipEventSynchronize(ctx->ev1));
+        HIP_TRY(ctx, FNN_ERR_DISPATCH, hipEventElapsedTime(ms, ctx->ev0, ctx->ev1));
+        return FNN_OK;
+    });
 }
 
 int fnn_hip_graph_begin(fnn_hip_ctx *ctx)
 {
-    if (!ctx) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_hip_graph_begin: NULL context");
-    if (ctx->capturing) return fail(ctx, FNN_ERR_DISPATCH, "graph capture already active");
-    HIP_TRY(ctx, FNN_ERR_DISPATCH, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
-    ctx->capturing = true;
-    return FNN_OK;
+    return guarded(ctx, "fnn_hip_graph_begin", [&]() -> int {
+        if (!ctx) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_hip_graph_begin: NULL context");
+        if (ctx->capturing) return fail(ctx, FNN_ERR_DISPATCH, "graph capture already active");
+        HIP_TRY(ctx, FNN_ERR_DISPATCH, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
+        ctx->capturing = true;
+        return FNN_OK;
+    });
 }
 
 int fnn_hip_graph_end(fnn_hip_ctx *ctx, fnn_hip_graph **out)
 {
-    if (!ctx || !out) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_graph_end: NULL argument");
-    if (!ctx->capturing) return fail(ctx, FNN_ERR_DISPATCH, "no graph capture active");
-    ctx->capturing = false;
-    fnn_hip_graph *g = new (std::nothrow) fnn_hip_graph();
-    if (!g) return fail(ctx, FNN_ERR_MEMORY, "out of host memory");
-    hipError_t e = hipStreamEndCapture(ctx->stream, &g->graph);
-    if (e == hipSuccess) e = hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0);
-    if (e != hipSuccess) {
-        if (g->graph) (void)hipGraphDestroy(g->graph);
-        delete g;
-        return fail(ctx, FNN_ERR_DISPATCH, "graph capture failed: %s", hipGetErrorString(e));
-    }
-    *out = g;
-    return FNN_OK;
+    return guarded(ctx, "fnn_hip_graph_end", [&]() -> int {
+        if (!ctx || !out) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_graph_end: NULL argument");
+        if (!ctx->capturing) return fail(ctx, FNN_ERR_DISPATCH, "no graph capture active");
+        *out = nullptr;
+        // the stream leaves capture mode first, whatever fails afterwards
+        hipGraph_t graph = nullptr;
+        hipError_t e = hipStreamEndCapture(ctx->stream, &graph);
+        ctx->capturing = false;
+        if (e != hipSuccess) return fail(ctx, FNN_ERR_DISPATCH, "graph capture failed: %s", hipGetErrorString(e));
+        fnn_hip_graph *g = new (std::nothrow) fnn_hip_graph();
+        if (!g) {
+            (void)hipGraphDestroy(graph);
+            return fail(ctx, FNN_ERR_MEMORY, "out of host memory");
+        }
+        g->graph = graph;
+        e = hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0);
+        if (e != hipSuccess) {
+            (void)hipGraphDestroy(g->graph);
+            delete g;
+            return fail(ctx, FNN_ERR_DISPATCH, "graph instantiation failed: %s", hipGetErrorString(e));
+        }
+        *out = g;
+        return FNN_OK;
+    });
 }
 
 int fnn_hip_graph_launch(fnn_hip_ctx *ctx, fnn_hip_graph *g)
 {
-    if (!ctx || !g) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_graph_launch: NULL argument");
-    HIP_TRY(ctx, FNN_ERR_DISPATCH, hipGraphLaunch(g->exec, ctx->stream));
-    return FNN_OK;
+    return guarded(ctx, "fnn_hip_graph_launch", [&]() -> int {
+        if (!ctx || !g) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_graph_launch: NULL argument");
+        HIP_TRY(ctx, FNN_ERR_DISPATCH, hipGraphLaunch(g->exec, ctx->stream));
+        return FNN_OK;
+    });
 }
 
 uint64_t fnn_hip_workspace_epoch(const fnn_hip_ctx *ctx) { return ctx ? ctx->ws_epoch : 0; }
 
 int fnn_hip_graph_destroy(fnn_hip_ctx *ctx, fnn_hip_graph *g)
 {
-    if (!g) return FNN_OK;
-    if (ctx && ctx->stream) (void)hipStreamSynchronize(ctx->stream);
-    if (g->exec) (void)hipGraphExecDestroy(g->exec);
-    if (g->graph) (void)hipGraphDestroy(g->graph);
-    delete g;
-    return FNN_OK;
+    return guarded(ctx, "fnn_hip_graph_destroy", [&]() -> int {
+        if (!g) return FNN_OK;
+        if (ctx && ctx->stream) (void)hipStreamSynchronize(ctx->stream);
+        if (g->exec) (void)hipGraphExecDestroy(g->exec);
+        if (g->graph) (void)hipGraphDestroy(g->graph);
+        delete g;
+        return FNN_OK;
+    });
 }
 
 }  // extern "C"
 
-// staging access for the MFMA translation unit
+// staging access for the matrix-core translation units
 int fnn_ctx_ensure_tmp(fnn_hip_ctx *ctx, int which, size_t bytes, void **ptr)
 {
-    Staging &s = which == 0 ? ctx->st_tmp : (which == 1 ? ctx->st_tmp2 : (which == 2 ? ctx->st_cnt : ctx->st_tmp3));
-    const void *before = s.ptr;
+    Staging &s = which == 0 ? ctx->st_tmp : (which == 1 ? ctx->st_tmp2 : ctx->st_tmp3);
     int rc = ensure(ctx, s, bytes);
     if (rc) return rc;
-    // which == 2: arrival counters, zero whenever (re)allocated; kernels leave them at zero
-    if (which == 2 && s.ptr != before) HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemsetAsync(s.ptr, 0, s.cap, ctx->stream));
     *ptr = s.ptr;
     return FNN_OK;
 }
@@ -892,3 +1004,5 @@ int fnn_ctx_ensure_tmp(fnn_hip_ctx *ctx, int which, size_t bytes, void **ptr)
 bool fnn_ctx_capturing(fnn_hip_ctx *ctx) { return ctx->capturing; }
 
 int fnn_ctx_fail(fnn_hip_ctx *ctx, int code, const char *msg) { return fail(ctx, code, "%s", msg); }
+
+int64_t fnn_ctx_option(const fnn_hip_ctx *ctx, int option) { return ctx->options[option]; }

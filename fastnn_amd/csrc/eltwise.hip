@@ -34,12 +34,17 @@ __global__ void __launch_bounds__(256) copy2d_kernel(float *dst, uint64_t dst_pi
 }
 
 // window maximum from -inf with a strict `>` (a NaN never wins), taps in the padding skipped
+// indices (nullable): window position kh*kernel + kw of the first strict maximum in (kh, kw) order, 0 when no tap
+// lies inside the image; an output position is visited when it lies inside the value slice or the index slice
 __global__ void __launch_bounds__(256) maxpool2d_kernel(const float *x, uint64_t in_len, float *y, uint64_t out_len, uint64_t c,
-                                                        uint64_t h, uint64_t w, uint64_t ho, uint64_t wo, int kernel, int stride, int pad)
+                                                        uint64_t h, uint64_t w, uint64_t ho, uint64_t wo, int kernel, int stride, int pad,
+                                                        int64_t *indices, uint64_t idx_len)
 {
-    for (uint64_t o = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; o < out_len; o += (uint64_t)gridDim.x * blockDim.x) {
+    const uint64_t total = out_len > idx_len ? out_len : idx_len;
+    for (uint64_t o = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; o < total; o += (uint64_t)gridDim.x * blockDim.x) {
         const uint64_t ww = o % wo, t = o / wo, hh = t % ho, nc = t / ho;   // nc = n*c + channel
         float val = -INFINITY;
+        int best = 0;
         for (int kh = 0; kh < kernel; kh++) {
             const int64_t hi = (int64_t)(hh * stride) + kh - pad;
             if (hi < 0 || hi >= (int64_t)h) continue;
@@ -49,11 +54,12 @@ __global__ void __launch_bounds__(256) maxpool2d_kernel(const float *x, uint64_t
                 const uint64_t idx = (nc * h + (uint64_t)hi) * w + (uint64_t)wi;
                 if (idx < in_len) {
                     const float v = x[idx];
-                    if (v > val) val = v;
+                    if (v > val) { val = v; best = kh * kernel + kw; }
                 }
             }
         }
-        y[o] = val;
+        if (o < out_len) y[o] = val;
+        if (o < idx_len) indices[o] = best;
     }
     (void)c;
 }
@@ -109,10 +115,13 @@ hipError_t launch_copy2d(float *dst, uint64_t dst_pitch, uint64_t dst_len, const
 }
 
 hipError_t launch_maxpool2d(const float *x, uint64_t in_len, float *y, uint64_t out_len, uint64_t c, uint64_t h, uint64_t w,
-                            uint64_t ho, uint64_t wo, int kernel, int stride, int pad, hipStream_t s)
+                            uint64_t ho, uint64_t wo, int kernel, int stride, int pad, int64_t *indices, uint64_t idx_len, hipStream_t s)
 {
-    if (out_len == 0) return hipSuccess;
-    hipLaunchKernelGGL(maxpool2d_kernel, dim3(grid_for(out_len)), dim3(256), 0, s, x, in_len, y, out_len, c, h, w, ho, wo, kernel, stride, pad);
+    if (!indices) idx_len = 0;
+    const uint64_t total = out_len > idx_len ? out_len : idx_len;
+    if (total == 0) return hipSuccess;
+    hipLaunchKernelGGL(maxpool2d_kernel, dim3(grid_for(total)), dim3(256), 0, s, x, in_len, y, out_len, c, h, w, ho, wo, kernel, stride, pad,
+                       indices, idx_len);
     return hipGetLastError();
 }
 

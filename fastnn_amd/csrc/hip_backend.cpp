@@ -14,7 +14,10 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <algorithm>
+#include <exception>
 #include <map>
+#include <new>
 #include <string>
 #include <vector>
 
@@ -38,6 +41,8 @@ struct Instr {
     std::vector<uint8_t> data;
     float value = 0.0f;
     std::string kernel;
+    bool has_secondary = false;   // CallKernel.secondary_output_slice (MaxPool indices)
+    fnn_slice secondary{0, 0};
     std::vector<fnn_slice> inputs;
     std::vector<uint64_t> params;
     Meta meta;
@@ -88,7 +93,10 @@ int matmul_dtype(const std::string &base)
 struct fnn_plan {
     uint64_t arena_size = 0;
     std::vector<Instr> instrs;
+    uint64_t uid = 0;                 // never reused within the process
+    uint64_t revision = 0;            // bumped whenever an instruction is added
     bool analysed = false;
+    std::vector<fnn_slice> writes;    // union of every byte range the plan writes, as disjoint sorted intervals
     bool uploads_every_run = false;   // some WriteConst target is overwritten by the plan itself
     // WriteConst payloads stay valid in the arena of this backend (by unique id) at this generation
     uint64_t resident_uid = 0;
@@ -108,14 +116,17 @@ struct fnn_backend {
     uint64_t arena_bytes = 0;
     uint64_t uid = 0;         // never reused within the process
     uint64_t generation = 1;  // bumped when the arena is re-allocated or the write log overflows
-    // host writes into the arena since the backend was created: (sequence number, byte range).
-    // A plan's constants stay resident across a write that touches none of them (the usual
-    // "write the input, dispatch, read the output" cycle uploads the weights only once).
+    // Writes into the arena that a plan cannot know of: host writes (write_arena) and everything another plan's
+    // dispatch wrote.  One entry per distinct byte range, with the sequence number of the latest write to it, so the
+    // usual cycle (same input ranges every forward, the same few plans taking turns) keeps the log at a fixed size.
+    // A plan's constants stay resident across writes that touch none of them.
     uint64_t write_seq = 0;
     std::vector<std::pair<uint64_t, fnn_slice>> host_writes;
+    uint64_t last_plan_uid = 0, last_plan_revision = 0;   // the plan whose write set was logged last
+    bool graph_replay = true;    // resident plans replay as one HIP graph (fnn_backend_set_graph_replay)
     uint64_t weights_epoch = 0;  // bumped whenever a cached device weight is created or released
     int kernel_flags = 0;        // extra FNN_FLAG_* bits for every MatMul / Conv2d call
-    std::string err;
+    char err[1024] = {0};        // fixed storage: recording a failure never allocates
     std::map<std::pair<uint64_t, uint64_t>, fnn_hip_weight *> weights;  // (offset,size) like get_or_cache_packed
     std::vector<uint8_t> stage;
     uint8_t *scratch = nullptr;   // device copy of an input that overlaps its output
@@ -124,24 +135,56 @@ struct fnn_backend {
 
 namespace {
 
-int fail(fnn_backend *b, int code, const char *fmt, ...)
+thread_local char g_err[1024] = {0};   // failures without a backend (create, plan building)
+
+int fail(fnn_backend *b, int code, const char *fmt, ...) noexcept
 {
-    char buf[512];
+    char *buf = b ? b->err : g_err;
     va_list ap;
     va_start(ap, fmt);
-    vsnprintf(buf, sizeof buf, fmt, ap);
+    vsnprintf(buf, 1024, fmt, ap);
     va_end(ap);
-    if (b) b->err = buf;
     return code;
 }
 
-int lift(fnn_backend *b, int st)
+int lift(fnn_backend *b, int st) noexcept
 {
     if (st != FNN_OK) {
         const char *m = fnn_hip_last_error(b->ctx);
-        b->err = m ? m : "libfastnn_hip call failed";
+        snprintf(b->err, sizeof b->err, "%s", m && *m ? m : "libfastnn_hip call failed");
     }
     return st;
+}
+
+// Every extern "C" body runs inside this: a C++ exception (std::bad_alloc from a container that copies a weight
+// payload, std::length_error, ...) becomes a status code and a message instead of unwinding into the caller.
+template <class F>
+int guarded(fnn_backend *b, const char *fn, F &&body) noexcept
+{
+    try {
+        return body();
+    } catch (const std::bad_alloc &) {
+        return fail(b, FNN_ERR_MEMORY, "%s: out of host memory", fn);
+    } catch (const std::exception &e) {
+        return fail(b, FNN_ERR_DISPATCH, "%s: %s", fn, e.what());
+    } catch (...) {
+        return fail(b, FNN_ERR_DISPATCH, "%s: unknown C++ exception", fn);
+    }
+}
+
+// One more write to `s` that plans must notice: the entry of the same range takes the new sequence number, a new
+// range is appended.  Past 4096 distinct ranges the log is dropped and every plan uploads its constants again.
+void log_write(fnn_backend *b, const fnn_slice &s)
+{
+    if (s.size == 0) return;
+    for (auto &e : b->host_writes)
+        if (e.second.offset == s.offset && e.second.size == s.size) { e.first = b->write_seq; return; }
+    if (b->host_writes.size() >= 4096) {
+        b->host_writes.clear();
+        b->generation++;
+        return;
+    }
+    b->host_writes.emplace_back(b->write_seq, s);
 }
 
 bool in_arena(const fnn_backend *b, const fnn_slice &s)
@@ -480,8 +523,17 @@ int run_pool(fnn_backend *b, const Instr &in)
     if (p[3] != 1)   // pool_avg_f32_scalar (src/backend/cpu/microkernels/ops.rs:162-210)
         return lift(b, fnn_hip_avgpool2d_f32(b->ctx, src, in.inputs[0].size / 4, (float *)(b->arena + in.dst.offset), in.dst.size / 4, p[4],
                                              p[5], p[6], p[7], p[0], p[1], p[2]));
+    // secondary output: i64 window position kh*kernel + kw of the maximum (MaxPool indices)
+    int64_t *indices = nullptr;
+    uint64_t idx_len = 0;
+    if (in.has_secondary && in.secondary.size >= 8) {
+        if (in.secondary.offset & 7) return fail(b, FNN_ERR_DISPATCH, "pool_f32: secondary output slice must be 8-byte aligned");
+        if (overlaps(in.secondary, in.dst) || overlaps(in.secondary, in.inputs[0])) return fail(b, FNN_ERR_DISPATCH, "pool_f32: secondary output overlaps another slice");
+        indices = (int64_t *)(b->arena + in.secondary.offset);
+        idx_len = in.secondary.size / 8;
+    }
     return lift(b, fnn_hip_maxpool2d_f32(b->ctx, src, in.inputs[0].size / 4, (float *)(b->arena + in.dst.offset), in.dst.size / 4, p[4], p[5],
-                                         p[6], p[7], p[0], p[1], p[2]));
+                                         p[6], p[7], p[0], p[1], p[2], indices, idx_len));
 }
 
 // "upsample_nearest2d": params [scale_h, scale_w, h_in, w_in], defaults 2, 2, 1, 1 (src/backend/cpu/mod.rs:5496-5535)
@@ -505,6 +557,7 @@ int run_call(fnn_backend *b, const Instr &in)
     for (const auto &s : in.inputs)
         if (!in_arena(b, s)) return fail(b, FNN_ERR_DISPATCH, "%s: input slice [%llu,+%llu) outside the arena of %llu bytes", in.kernel.c_str(), (unsigned long long)s.offset, (unsigned long long)s.size, (unsigned long long)b->arena_bytes);
     if (!in_arena(b, in.dst)) return fail(b, FNN_ERR_DISPATCH, "%s: output slice [%llu,+%llu) outside the arena of %llu bytes", in.kernel.c_str(), (unsigned long long)in.dst.offset, (unsigned long long)in.dst.size, (unsigned long long)b->arena_bytes);
+    if (in.has_secondary && !in_arena(b, in.secondary)) return fail(b, FNN_ERR_DISPATCH, "%s: secondary output slice [%llu,+%llu) outside the arena of %llu bytes", in.kernel.c_str(), (unsigned long long)in.secondary.offset, (unsigned long long)in.secondary.size, (unsigned long long)b->arena_bytes);
     const std::string &name = in.kernel;
     if (name == "quantize_activations") return run_quantize_activations(b, in);
     if (name == "dequantize_activations") return run_dequantize_activations(b, in);
@@ -535,11 +588,42 @@ void analyse(fnn_plan *p)
         c.clobbered = false;
         for (const auto &o : p->instrs) {
             if (&o == &c) continue;
-            if (overlaps(o.dst, c.dst)) { c.clobbered = true; break; }
+            if (overlaps(o.dst, c.dst) || (o.has_secondary && overlaps(o.secondary, c.dst))) { c.clobbered = true; break; }
         }
         if (c.clobbered && !c.data.empty()) p->uploads_every_run = true;
     }
+    // the plan's write set as disjoint intervals (touching ranges are joined, gaps are never bridged)
+    std::vector<fnn_slice> w;
+    for (const auto &o : p->instrs) {
+        if (o.dst.size) w.push_back(o.dst);
+        if (o.has_secondary && o.secondary.size) w.push_back(o.secondary);
+    }
+    std::sort(w.begin(), w.end(), [](const fnn_slice &a, const fnn_slice &b) { return a.offset < b.offset; });
+    p->writes.clear();
+    for (const auto &r : w) {
+        if (!p->writes.empty() && r.offset <= p->writes.back().offset + p->writes.back().size) {
+            const uint64_t end = std::max(p->writes.back().offset + p->writes.back().size, r.offset + r.size);
+            p->writes.back().size = end - p->writes.back().offset;
+        } else {
+            p->writes.push_back(r);
+        }
+    }
     p->analysed = true;
+}
+
+// After a dispatch of `p`: what it wrote is news to every other plan of this backend.  Logged when the plan (or its
+// instruction list) differs from the one logged last; repeated dispatches of one plan add nothing.
+void note_dispatched(fnn_backend *b, fnn_plan *p)
+{
+    if (b->last_plan_uid != p->uid || b->last_plan_revision != p->revision) {
+        b->write_seq++;
+        for (const auto &r : p->writes) log_write(b, r);
+        b->last_plan_uid = p->uid;
+        b->last_plan_revision = p->revision;
+    }
+    p->resident_uid = b->uid;
+    p->resident_generation = b->generation;
+    p->resident_seq = b->write_seq;
 }
 
 int run_instr(fnn_backend *b, fnn_plan *p, Instr &in, bool consts_resident)
@@ -594,8 +678,7 @@ int dispatch_impl(fnn_backend *b, fnn_plan *p, uint64_t *elapsed_ns, uint64_t n_
     // workspaces have their final size launches as one HIP graph (the executor's static-shape
     // plan, src/backend/executor.rs:639-667).  Profiling, re-uploaded constants and anything
     // that fails under capture keep the instruction-by-instruction path.
-    static const bool graphs_on = [] { const char *e = getenv("FNN_PLAN_GRAPH"); return !(e && e[0] == '0'); }();
-    const bool may_replay = graphs_on && !elapsed_ns && resident && !p->uploads_every_run && p->graph_failures < 2;
+    const bool may_replay = b->graph_replay && !elapsed_ns && resident && !p->uploads_every_run && p->graph_failures < 2;
     if (p->graph && !(may_replay && p->graph_uid == b->uid && p->graph_generation == b->generation &&
                       p->graph_weights_epoch == b->weights_epoch && p->graph_ws_epoch == fnn_hip_workspace_epoch(b->ctx) &&
                       p->graph_scratch_epoch == b->scratch_epoch)) {
@@ -616,7 +699,7 @@ int dispatch_impl(fnn_backend *b, fnn_plan *p, uint64_t *elapsed_ns, uint64_t n_
             } else {
                 if (g) fnn_hip_graph_destroy(b->ctx, g);
                 p->graph_failures++;
-                b->err.clear();
+                b->err[0] = 0;
             }
         } else {
             p->graph_failures++;
@@ -627,6 +710,7 @@ int dispatch_impl(fnn_backend *b, fnn_plan *p, uint64_t *elapsed_ns, uint64_t n_
         int st = lift(b, fnn_hip_graph_launch(b->ctx, p->graph));
         if (st == FNN_OK) st = lift(b, fnn_hip_sync(b->ctx));
         p->last_replayed = st == FNN_OK;
+        if (st == FNN_OK) note_dispatched(b, p);
         return st;
     }
 
@@ -636,16 +720,17 @@ int dispatch_impl(fnn_backend *b, fnn_plan *p, uint64_t *elapsed_ns, uint64_t n_
         if (st == FNN_OK && elapsed_ns) st = lift(b, fnn_hip_sync(b->ctx));
         if (st != FNN_OK) {
             fnn_hip_sync(b->ctx);
+            // what ran before the failure has written: other plans must see it
+            b->write_seq++;
+            for (const auto &r : p->writes) log_write(b, r);
+            b->last_plan_uid = 0;
+            p->resident_uid = 0;
             return st;
         }
         if (elapsed_ns) elapsed_ns[i] = (uint64_t)std::chrono::duration_cast<std::chrono::nanoseconds>(std::chrono::steady_clock::now() - t0).count();
     }
     int st = lift(b, fnn_hip_sync(b->ctx));
-    if (st == FNN_OK) {
-        p->resident_uid = b->uid;
-        p->resident_generation = b->generation;
-        p->resident_seq = b->write_seq;
-    }
+    if (st == FNN_OK) note_dispatched(b, p);
     return st;
 }
 
@@ -655,17 +740,26 @@ extern "C" {
 
 int fnn_backend_create(int device, fnn_backend **out)
 {
-    if (!out) return FNN_ERR_DISPATCH;
-    *out = nullptr;
-    fnn_hip_ctx *ctx = nullptr;
-    int st = fnn_hip_create(device, &ctx);
-    if (st) return st;
-    static std::atomic<uint64_t> next_uid{1};
-    fnn_backend *b = new fnn_backend();
-    b->uid = next_uid++;
-    b->ctx = ctx;
-    *out = b;
-    return FNN_OK;
+    return guarded(nullptr, "fnn_backend_create", [&]() -> int {
+        if (!out) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_backend_create: out is NULL");
+        *out = nullptr;
+        fnn_hip_ctx *ctx = nullptr;
+        int st = fnn_hip_create(device, &ctx);
+        if (st) {
+            snprintf(g_err, sizeof g_err, "%s", fnn_hip_last_error(nullptr));
+            return st;
+        }
+        static std::atomic<uint64_t> next_uid{1};
+        fnn_backend *b = new (std::nothrow) fnn_backend();
+        if (!b) {
+            fnn_hip_destroy(ctx);
+            return fail(nullptr, FNN_ERR_MEMORY, "fnn_backend_create: out of host memory");
+        }
+        b->uid = next_uid++;
+        b->ctx = ctx;
+        *out = b;
+        return FNN_OK;
+    });
 }
 
 void fnn_backend_destroy(fnn_backend *b)
@@ -682,7 +776,7 @@ const char *fnn_backend_name(const fnn_backend *) { return "hip"; }
 
 int fnn_backend_set_kernel_flags(fnn_backend *b, int flags)
 {
-    if (!b) return FNN_ERR_DISPATCH;
+    if (!b) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_backend_set_kernel_flags: NULL backend");
     if (flags & ~(FNN_FLAG_ACT_F16_SINGLE | FNN_FLAG_FORCE_GENERIC | FNN_FLAG_PREFER_FMA))
         return fail(b, FNN_ERR_DISPATCH, "set_kernel_flags: only ACT_F16_SINGLE, FORCE_GENERIC and PREFER_FMA can be set per backend");
     if (flags != b->kernel_flags) b->weights_epoch++;   // captured graphs hold the old kernel choice
@@ -690,64 +784,85 @@ int fnn_backend_set_kernel_flags(fnn_backend *b, int flags)
     return FNN_OK;
 }
 
-const char *fnn_backend_last_error(const fnn_backend *b) { return b ? b->err.c_str() : "no backend"; }
+int fnn_backend_set_graph_replay(fnn_backend *b, int enabled)
+{
+    if (!b) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_backend_set_graph_replay: NULL backend");
+    b->graph_replay = enabled != 0;
+    return FNN_OK;
+}
+
+int fnn_backend_set_option(fnn_backend *b, int option, int64_t value)
+{
+    if (!b) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_backend_set_option: NULL backend");
+    int st = lift(b, fnn_hip_set_option(b->ctx, option, value));
+    if (st == FNN_OK) b->weights_epoch++;   // captured graphs hold the old kernel choice
+    return st;
+}
+
+const char *fnn_backend_last_error(const fnn_backend *b) { return b ? b->err : g_err; }
 
 int fnn_backend_allocate_arena(fnn_backend *b, uint64_t total_bytes)
 {
-    if (!b) return FNN_ERR_DISPATCH;
-    drop_weights(b);
-    if (b->arena) {
-        fnn_hip_free(b->ctx, b->arena);
-        b->arena = nullptr;
-        b->arena_bytes = 0;
-    }
-    b->generation++;
-    // CpuBuffer::new zero-fills; keep 64 bytes of slack so that vector loads at the end stay inside
-    void *d = nullptr;
-    uint64_t padded = ((total_bytes + 63) / 64) * 64 + 64;
-    int st = lift(b, fnn_hip_malloc(b->ctx, padded, &d));
-    if (st) return st;
-    b->arena = (uint8_t *)d;
-    b->arena_bytes = total_bytes;
-    st = lift(b, fnn_hip_fill_f32(b->ctx, (float *)d, padded / 4, 0.0f));
-    if (st) return st;
-    return lift(b, fnn_hip_sync(b->ctx));
+    return guarded(b, "fnn_backend_allocate_arena", [&]() -> int {
+        if (!b) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_backend_allocate_arena: NULL backend");
+        drop_weights(b);
+        if (b->arena) {
+            fnn_hip_free(b->ctx, b->arena);
+            b->arena = nullptr;
+            b->arena_bytes = 0;
+        }
+        b->generation++;
+        b->host_writes.clear();
+        // CpuBuffer::new zero-fills; keep 64 bytes of slack so that vector loads at the end stay inside
+        void *d = nullptr;
+        uint64_t padded = ((total_bytes + 63) / 64) * 64 + 64;
+        int st = lift(b, fnn_hip_malloc(b->ctx, padded, &d));
+        if (st) return st;
+        b->arena = (uint8_t *)d;
+        b->arena_bytes = total_bytes;
+        st = lift(b, fnn_hip_fill_f32(b->ctx, (float *)d, padded / 4, 0.0f));
+        if (st) return st;
+        return lift(b, fnn_hip_sync(b->ctx));
+    });
 }
 
 int fnn_backend_write_arena(fnn_backend *b, uint64_t offset, const void *data, uint64_t size)
 {
-    if (!b) return FNN_ERR_DISPATCH;
-    fnn_slice s{offset, size};
-    if (!b->arena || !in_arena(b, s)) return fail(b, FNN_ERR_MEMORY, "write_arena: %llu bytes at %llu outside the arena of %llu bytes", (unsigned long long)size, (unsigned long long)offset, (unsigned long long)b->arena_bytes);
-    if (size == 0) return FNN_OK;
-    if (!data) return fail(b, FNN_ERR_DISPATCH, "write_arena: NULL data");
-    drop_weights_overlapping(b, s);
-    b->write_seq++;
-    if (b->host_writes.size() >= 256) {   // forget the log: every plan uploads its constants again
-        b->host_writes.clear();
-        b->generation++;
-    } else {
-        b->host_writes.emplace_back(b->write_seq, s);
-    }
-    return lift(b, fnn_hip_upload(b->ctx, b->arena + offset, data, size));
+    return guarded(b, "fnn_backend_write_arena", [&]() -> int {
+        if (!b) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_backend_write_arena: NULL backend");
+        fnn_slice s{offset, size};
+        if (!b->arena || !in_arena(b, s)) return fail(b, FNN_ERR_MEMORY, "write_arena: %llu bytes at %llu outside the arena of %llu bytes", (unsigned long long)size, (unsigned long long)offset, (unsigned long long)b->arena_bytes);
+        if (size == 0) return FNN_OK;
+        if (!data) return fail(b, FNN_ERR_DISPATCH, "write_arena: NULL data");
+        drop_weights_overlapping(b, s);
+        b->write_seq++;
+        log_write(b, s);
+        return lift(b, fnn_hip_upload(b->ctx, b->arena + offset, data, size));
+    });
 }
 
 int fnn_backend_read_arena(fnn_backend *b, uint64_t offset, void *out, uint64_t size)
 {
-    if (!b) return FNN_ERR_DISPATCH;
-    fnn_slice s{offset, size};
-    if (!b->arena || !in_arena(b, s)) return fail(b, FNN_ERR_MEMORY, "read_arena: %llu bytes at %llu outside the arena of %llu bytes", (unsigned long long)size, (unsigned long long)offset, (unsigned long long)b->arena_bytes);
-    if (size == 0) return FNN_OK;
-    if (!out) return fail(b, FNN_ERR_DISPATCH, "read_arena: NULL destination");
-    return lift(b, fnn_hip_download(b->ctx, out, b->arena + offset, size));
+    return guarded(b, "fnn_backend_read_arena", [&]() -> int {
+        if (!b) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_backend_read_arena: NULL backend");
+        fnn_slice s{offset, size};
+        if (!b->arena || !in_arena(b, s)) return fail(b, FNN_ERR_MEMORY, "read_arena: %llu bytes at %llu outside the arena of %llu bytes", (unsigned long long)size, (unsigned long long)offset, (unsigned long long)b->arena_bytes);
+        if (size == 0) return FNN_OK;
+        if (!out) return fail(b, FNN_ERR_DISPATCH, "read_arena: NULL destination");
+        return lift(b, fnn_hip_download(b->ctx, out, b->arena + offset, size));
+    });
 }
 
 int fnn_plan_create(uint64_t arena_size, fnn_plan **out)
 {
-    if (!out) return FNN_ERR_DISPATCH;
-    *out = new fnn_plan();
-    (*out)->arena_size = arena_size;
-    return FNN_OK;
+    return guarded(nullptr, "fnn_plan_create", [&]() -> int {
+        if (!out) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_plan_create: out is NULL");
+        static std::atomic<uint64_t> next_uid{1};
+        *out = new fnn_plan();
+        (*out)->arena_size = arena_size;
+        (*out)->uid = next_uid++;
+        return FNN_OK;
+    });
 }
 
 void fnn_plan_destroy(fnn_plan *p)
@@ -766,6 +881,7 @@ static void touched(fnn_plan *p)
     p->analysed = false;
     p->uploads_every_run = false;
     p->resident_uid = 0;
+    p->revision++;
     if (p->graph) {
         fnn_hip_graph_destroy(nullptr, p->graph);
         p->graph = nullptr;
@@ -774,70 +890,95 @@ static void touched(fnn_plan *p)
 
 int fnn_plan_add_write_const(fnn_plan *p, fnn_slice dst, const void *data, uint64_t len)
 {
-    if (!p || (!data && len)) return FNN_ERR_DISPATCH;
-    Instr in;
-    in.kind = K_WRITE_CONST;
-    in.dst = fnn_slice{dst.offset, len};
-    in.data.assign((const uint8_t *)data, (const uint8_t *)data + len);
-    p->instrs.push_back(std::move(in));
-    touched(p);
-    return FNN_OK;
+    return guarded(nullptr, "fnn_plan_add_write_const", [&]() -> int {
+        if (!p || (!data && len)) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_plan_add_write_const: NULL argument");
+        Instr in;
+        in.kind = K_WRITE_CONST;
+        in.dst = fnn_slice{dst.offset, len};
+        in.data.assign((const uint8_t *)data, (const uint8_t *)data + len);
+        p->instrs.push_back(std::move(in));
+        touched(p);
+        return FNN_OK;
+    });
 }
 
 int fnn_plan_add_fill(fnn_plan *p, fnn_slice dst, float value)
 {
-    if (!p) return FNN_ERR_DISPATCH;
-    Instr in;
-    in.kind = K_FILL;
-    in.dst = dst;
-    in.value = value;
-    p->instrs.push_back(std::move(in));
-    touched(p);
-    return FNN_OK;
+    return guarded(nullptr, "fnn_plan_add_fill", [&]() -> int {
+        if (!p) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_plan_add_fill: NULL plan");
+        Instr in;
+        in.kind = K_FILL;
+        in.dst = dst;
+        in.value = value;
+        p->instrs.push_back(std::move(in));
+        touched(p);
+        return FNN_OK;
+    });
 }
 
 int fnn_plan_add_memcopy(fnn_plan *p, fnn_slice dst, fnn_slice src)
 {
-    if (!p) return FNN_ERR_DISPATCH;
-    Instr in;
-    in.kind = K_MEMCOPY;
-    in.dst = dst;
-    in.src = src;
-    p->instrs.push_back(std::move(in));
-    touched(p);
-    return FNN_OK;
+    return guarded(nullptr, "fnn_plan_add_memcopy", [&]() -> int {
+        if (!p) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_plan_add_memcopy: NULL plan");
+        Instr in;
+        in.kind = K_MEMCOPY;
+        in.dst = dst;
+        in.src = src;
+        p->instrs.push_back(std::move(in));
+        touched(p);
+        return FNN_OK;
+    });
 }
 
 int fnn_plan_add_call_kernel(fnn_plan *p, const char *kernel_name, const fnn_slice *inputs, uint64_t n_inputs,
-                             fnn_slice output, const uint64_t *params, uint64_t n_params, const fnn_weight_meta *meta)
+                             fnn_slice output, const fnn_slice *secondary_output, const uint64_t *params,
+                             uint64_t n_params, const fnn_weight_meta *meta)
 {
-    if (!p || !kernel_name || (!inputs && n_inputs) || (!params && n_params)) return FNN_ERR_DISPATCH;
-    Instr in;
-    in.kind = K_CALL;
-    in.kernel = kernel_name;
-    in.inputs.assign(inputs, inputs + n_inputs);
-    in.dst = output;
-    in.params.assign(params, params + n_params);
-    if (meta) {
-        in.meta.present = true;
-        in.meta.bit_width = meta->bit_width;
-        if (meta->scales) in.meta.scales.assign(meta->scales, meta->scales + meta->n_scales);
-        if (meta->zero_points) in.meta.zeros.assign(meta->zero_points, meta->zero_points + meta->n_zero_points);
-        if (meta->shape) in.meta.shape.assign(meta->shape, meta->shape + meta->n_shape);
-        in.meta.qblock = meta->quant_block_size;
-        if (meta->codebook16) in.meta.codebook.assign(meta->codebook16, meta->codebook16 + 16);
-    }
-    p->instrs.push_back(std::move(in));
-    touched(p);
-    return FNN_OK;
+    return guarded(nullptr, "fnn_plan_add_call_kernel", [&]() -> int {
+        if (!p || !kernel_name || (!inputs && n_inputs) || (!params && n_params))
+            return fail(nullptr, FNN_ERR_DISPATCH, "fnn_plan_add_call_kernel: NULL argument");
+        Instr in;
+        in.kind = K_CALL;
+        in.kernel = kernel_name;
+        in.inputs.assign(inputs, inputs + n_inputs);
+        in.dst = output;
+        if (secondary_output) {
+            in.has_secondary = true;
+            in.secondary = *secondary_output;
+        }
+        in.params.assign(params, params + n_params);
+        if (meta) {
+            // QuantizedWeightMeta.codebooks is a Vec<[f32; 16]>.  The quantisation pass emits one codebook per weight
+            // (src/packed_tensor.rs:1310) and every decode of the reference reads codebooks[0] only
+            // (src/packed_tensor.rs:398, 489, 586), whatever the vector's length: so does this backend.
+            if (meta->n_codebooks >= 1 && !meta->codebooks)
+                return fail(nullptr, FNN_ERR_DISPATCH, "%s: weight_meta.n_codebooks = %llu with a NULL codebooks pointer", kernel_name,
+                            (unsigned long long)meta->n_codebooks);
+            in.meta.present = true;
+            in.meta.bit_width = meta->bit_width;
+            if (meta->scales) in.meta.scales.assign(meta->scales, meta->scales + meta->n_scales);
+            if (meta->zero_points) in.meta.zeros.assign(meta->zero_points, meta->zero_points + meta->n_zero_points);
+            if (meta->shape) in.meta.shape.assign(meta->shape, meta->shape + meta->n_shape);
+            in.meta.qblock = meta->quant_block_size;
+            if (meta->n_codebooks >= 1) in.meta.codebook.assign(meta->codebooks, meta->codebooks + 16);
+        }
+        p->instrs.push_back(std::move(in));
+        touched(p);
+        return FNN_OK;
+    });
 }
 
-int fnn_backend_dispatch(fnn_backend *b, fnn_plan *p) { return dispatch_impl(b, p, nullptr, 0); }
+int fnn_backend_dispatch(fnn_backend *b, fnn_plan *p)
+{
+    return guarded(b, "fnn_backend_dispatch", [&]() -> int { return dispatch_impl(b, p, nullptr, 0); });
+}
 
 int fnn_backend_dispatch_profile(fnn_backend *b, fnn_plan *p, uint64_t *elapsed_ns, uint64_t n)
 {
-    if (!elapsed_ns) return fail(b, FNN_ERR_DISPATCH, "dispatch_profile: NULL timings");
-    return dispatch_impl(b, p, elapsed_ns, n);
+    return guarded(b, "fnn_backend_dispatch_profile", [&]() -> int {
+        if (!elapsed_ns) return fail(b, FNN_ERR_DISPATCH, "dispatch_profile: NULL timings");
+        return dispatch_impl(b, p, elapsed_ns, n);
+    });
 }
 
 }  // extern "C"

@@ -1,5 +1,7 @@
 // Matrix-core kernel entry points.
 #pragma once
+#include <atomic>
+
 #include "common.h"
 #include "i8act.h"
 
@@ -7,6 +9,22 @@
 int fnn_ctx_ensure_tmp(fnn_hip_ctx *ctx, int which, size_t bytes, void **ptr);
 int fnn_ctx_fail(fnn_hip_ctx *ctx, int code, const char *msg);
 bool fnn_ctx_capturing(fnn_hip_ctx *ctx);
+// value of a per-context option (FNN_OPT_*, set through fnn_hip_set_option)
+int64_t fnn_ctx_option(const fnn_hip_ctx *ctx, int option);
+
+// Raises a kernel's dynamic LDS limit once per device.  `done` is a bit mask of devices (one static per kernel
+// instantiation); safe from several threads, and a second device gets its own call.
+inline hipError_t fnn_raise_lds_limit(std::atomic<uint64_t> &done, const void *kernel, int bytes)
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    const uint64_t bit = 1ull << (dev & 63);
+    if (done.load(std::memory_order_acquire) & bit) return hipSuccess;
+    e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e == hipSuccess) done.fetch_or(bit, std::memory_order_release);
+    return e;
+}
 
 // M >= 5: activations prepared once as f16 operands, 4-wave output tiles with the
 // activations staged through LDS and optional split of K (deterministic reduction).

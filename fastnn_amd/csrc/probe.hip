@@ -1,43 +1,89 @@
-// Memory-system probes: a plain streaming read and a plain copy of a known number of bytes.
-// They give (a) the bandwidth one launch of a given size can reach on this device, the
-// ceiling a bandwidth-bound kernel of that size is judged against, and (b) a reference
-// kernel of known traffic to scale hardware byte counters with.
-#include "common.h"
+// Memory-system probes, built as a library of their own (libfnn_probe.so): not part of the product ABI.
+// A plain streaming read and a plain copy of a known number of bytes give (a) the bandwidth one launch of a
+// given size can reach on this device, the ceiling a bandwidth-bound kernel of that size is judged against,
+// and (b) a kernel of known traffic to scale hardware byte counters with.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
 
 namespace {
 
-__global__ void __launch_bounds__(512) probe_read_kernel(const uint4 *__restrict__ src, size_t n16, uint32_t *sink)
+// A workgroup of 256 lanes walks chunks of 256*U consecutive 16-byte pieces; a lane has U independent loads
+// in flight (addresses past the end are clamped to the last piece and their values masked).
+template <int U>
+__global__ void __launch_bounds__(256) probe_read_kernel(const uint4 *__restrict__ src, size_t n16, uint32_t *sink)
 {
-    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    const size_t nchunks = (n16 + 256 * U - 1) / (256 * U);
     uint32_t acc = 0;
-    for (; i < n16; i += stride) {
-        const uint4 v = src[i];
-        acc += v.x ^ v.y ^ v.z ^ v.w;
+    for (size_t chunk = blockIdx.x; chunk < nchunks; chunk += gridDim.x) {
+        const size_t base = chunk * 256 * U + threadIdx.x;
+        uint4 v[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const size_t i = base + (size_t)u * 256;
+            v[u] = src[i < n16 ? i : n16 - 1];
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) acc += v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
     }
     if (acc == 0x9e3779b9u) sink[0] = acc;  // practically never true: keeps the loads alive
 }
 
-__global__ void __launch_bounds__(512) probe_copy_kernel(const uint4 *__restrict__ src, uint4 *__restrict__ dst, size_t n16)
+template <int U>
+__global__ void __launch_bounds__(256) probe_copy_kernel(const uint4 *__restrict__ src, uint4 *__restrict__ dst, size_t n16)
 {
-    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const size_t stride = (size_t)gridDim.x * blockDim.x;
-    for (; i < n16; i += stride) dst[i] = src[i];
+    const size_t nchunks = (n16 + 256 * U - 1) / (256 * U);
+    for (size_t chunk = blockIdx.x; chunk < nchunks; chunk += gridDim.x) {
+        const size_t base = chunk * 256 * U + threadIdx.x;
+        uint4 v[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const size_t i = base + (size_t)u * 256;
+            v[u] = src[i < n16 ? i : n16 - 1];
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const size_t i = base + (size_t)u * 256;
+            if (i < n16) dst[i] = v[u];
+        }
+    }
+}
+
+template <int U>
+hipError_t launch(const void *src, void *dst, size_t n16, unsigned grid, uint32_t *sink, hipStream_t s)
+{
+    if (dst)
+        hipLaunchKernelGGL(probe_copy_kernel<U>, dim3(grid), dim3(256), 0, s, reinterpret_cast<const uint4 *>(src),
+                           reinterpret_cast<uint4 *>(dst), n16);
+    else
+        hipLaunchKernelGGL(probe_read_kernel<U>, dim3(grid), dim3(256), 0, s, reinterpret_cast<const uint4 *>(src), n16, sink);
+    return hipGetLastError();
 }
 
 }  // namespace
 
-hipError_t launch_probe(const void *src, void *dst, size_t bytes, uint32_t *sink, hipStream_t s)
+// One launch on `stream` (a hipStream_t) that reads `bytes` from src_dev, and writes them to dst_dev unless that
+// is NULL.  loads_per_lane: 1, 2, 4 or 8 independent 16-byte loads per lane and trip; workgroups: 0 = one per
+// chunk (everything requested at once), else a fixed grid walking the chunks.  sink_dev: 4 writable bytes.
+// Returns 0 or the hipError_t value.
+extern "C" int fnn_probe_stream(void *stream, const void *src_dev, void *dst_dev, size_t bytes, int loads_per_lane,
+                                int workgroups, void *sink_dev)
 {
+    if (!src_dev || !sink_dev) return (int)hipErrorInvalidValue;
+    if ((reinterpret_cast<uintptr_t>(src_dev) & 15) || (reinterpret_cast<uintptr_t>(dst_dev) & 15)) return (int)hipErrorInvalidValue;
     const size_t n16 = bytes / 16;
-    if (n16 == 0) return hipSuccess;
-    size_t blocks = (n16 + 511) / 512;
-    if (blocks > 2048) blocks = 2048;
-    if (dst)
-        hipLaunchKernelGGL(probe_copy_kernel, dim3((unsigned)blocks), dim3(512), 0, s,
-                           reinterpret_cast<const uint4 *>(src), reinterpret_cast<uint4 *>(dst), n16);
-    else
-        hipLaunchKernelGGL(probe_read_kernel, dim3((unsigned)blocks), dim3(512), 0, s,
-                           reinterpret_cast<const uint4 *>(src), n16, sink);
-    return hipGetLastError();
+    if (n16 == 0) return 0;
+    const int u = loads_per_lane;
+    if (u != 1 && u != 2 && u != 4 && u != 8) return (int)hipErrorInvalidValue;
+    const size_t nchunks = (n16 + 256 * (size_t)u - 1) / (256 * (size_t)u);
+    size_t grid = workgroups > 0 ? (size_t)workgroups : nchunks;
+    if (grid > nchunks) grid = nchunks;
+    if (grid > 0x7fffffffu) grid = 0x7fffffffu;
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    uint32_t *sink = reinterpret_cast<uint32_t *>(sink_dev);
+    switch (u) {
+    case 1: return (int)launch<1>(src_dev, dst_dev, n16, (unsigned)grid, sink, s);
+    case 2: return (int)launch<2>(src_dev, dst_dev, n16, (unsigned)grid, sink, s);
+    case 4: return (int)launch<4>(src_dev, dst_dev, n16, (unsigned)grid, sink, s);
+    default: return (int)launch<8>(src_dev, dst_dev, n16, (unsigned)grid, sink, s);
+    }
 }

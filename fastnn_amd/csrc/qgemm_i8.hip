@@ -376,12 +376,9 @@ hipError_t launch_i8_tile(const TileArgs &p, hipStream_t s)
     constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
     constexpr size_t lds = (size_t)NS * (BM * 128 + BN * WC * 16);
     auto kern = qgemm_tile_kernel<DT, WGM, WGN, TM, TN, false, NS, true>;
-    static bool attr_set = false;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return e;
-        attr_set = true;
-    }
+    static std::atomic<uint64_t> lds_raised{0};
+    hipError_t e = fnn_raise_lds_limit(lds_raised, reinterpret_cast<const void *>(kern), (int)lds);
+    if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, dim3((unsigned)p.mtiles * p.ntiles), dim3(256), lds, s, p);
     return hipGetLastError();
 }

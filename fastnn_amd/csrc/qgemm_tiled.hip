@@ -241,12 +241,6 @@ __global__ void __launch_bounds__(256) splitk_epilogue_kernel(TileArgs p, int si
     }
 }
 
-int env_int(const char *name, int dflt)
-{
-    const char *s = getenv(name);
-    return s ? atoi(s) : dflt;
-}
-
 template <int DT, int WGM, int WGN, int TM, int TN, bool PRECISE, int NS>
 hipError_t launch_tile(const TileArgs &p, hipStream_t s)
 {
@@ -254,12 +248,9 @@ hipError_t launch_tile(const TileArgs &p, hipStream_t s)
     constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
     constexpr size_t lds = (size_t)NS * (BM * 128 + BN * WC * 16);
     auto kern = qgemm_tile_kernel<DT, WGM, WGN, TM, TN, PRECISE, NS>;
-    static bool attr_set = false;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return e;
-        attr_set = true;
-    }
+    static std::atomic<uint64_t> lds_raised{0};
+    hipError_t e = fnn_raise_lds_limit(lds_raised, reinterpret_cast<const void *>(kern), (int)lds);
+    if (e != hipSuccess) return e;
     const unsigned total = (unsigned)p.mtiles * p.ntiles * p.splits;
     hipLaunchKernelGGL(kern, dim3(total), dim3(256), lds, s, p);
     return hipGetLastError();
@@ -295,8 +286,8 @@ int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QM
     if (meff > 64) cfg = (!dense && ((meff + 127) / 128) * ((N + 127) / 128) <= 128) ? 1 : 0;
     else if (meff == 64) cfg = 1;
     else cfg = 2;
-    static const int env_cfg = env_int("FNN_TILE_CFG", -1);
-    if (env_cfg >= 0 && env_cfg <= 2) cfg = env_cfg;
+    const int64_t opt_cfg = fnn_ctx_option(ctx, FNN_OPT_TILE_SHAPE);
+    if (opt_cfg >= 0 && opt_cfg <= 2) cfg = (int)opt_cfg;
     const int bm = cfg == 0 ? 128 : (cfg == 1 ? 64 : 32);
     const int bn = 128;
     const int mtiles = (int)((meff + bm - 1) / bm);
@@ -310,7 +301,7 @@ int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QM
     // stages per workgroup x time a CU needs per stage x workgroups per CU (a CU gets through
     // stages at the same rate with one or several workgroups resident, but a lone workgroup cannot
     // hide its load latency: factor 1.5), plus, for s > 1, the write + read of s partial [M,N] tiles.
-    static const int env_split = env_int("FNN_TILE_SPLIT", 0);
+    const int env_split = (int)fnn_ctx_option(ctx, FNN_OPT_TILE_SPLIT);
     const int base = mtiles * ntiles;
     const double t_bits = DecH<DT>::WPS == 1 ? 0.4 : (DecH<DT>::WPS == 2 ? 0.7 : 1.0);
     const double t_stage = t_bits * (cfg == 0 ? 1.0 : (cfg == 1 ? 0.5 : 0.25));
@@ -377,7 +368,7 @@ int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QM
         t.a_wrap = (int)(kpad / BK);
     }
     t.act = q.act; t.splits = splits; t.iters = iters; t.ips = ips; t.mtiles = mtiles; t.ntiles = ntiles;
-    static const int env_ns = env_int("FNN_TILE_NS", 0);
+    const int env_ns = (int)fnn_ctx_option(ctx, FNN_OPT_TILE_STAGES);
     const bool deep = cfg == 0 && (env_ns == 5 || (env_ns == 0 && base * splits <= 256));
     if (deep) e = precise ? launch_tile<DT, 2, 2, 2, 2, true, 5>(t, s) : launch_tile<DT, 2, 2, 2, 2, false, 5>(t, s);
     else if (precise) {
@@ -462,8 +453,8 @@ int run_tiled_codebook(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w,
     const size_t tab_off = (op_bytes + 255) / 256 * 256;
     const size_t total = tab_off + (size_t)q.n * 8 + 256;
     // The expansion is kept with the weight (eight times the packed bytes, what the CPU path spends on its
-    // cached f32 copy); FNN_CODEBOOK_CACHE=0 expands into a workspace on every call instead.
-    static const bool keep = env_int("FNN_CODEBOOK_CACHE", 1) != 0;
+    // cached f32 copy); with FNN_OPT_CODEBOOK_CACHE = 0 a call expands into a workspace instead.
+    const bool keep = fnn_ctx_option(ctx, FNN_OPT_CODEBOOK_CACHE) != 0;
     fnn_hip_weight *wm = const_cast<fnn_hip_weight *>(w);
     void *ws = keep && q.words == w->words ? wm->dense16 : nullptr;
     bool expand = true;
@@ -520,7 +511,7 @@ int fnn_row_means(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, cons
 int fnn_tiled_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &q, int flags, bool *handled)
 {
     *handled = false;
-    static const int min_m = env_int("FNN_TILE_MIN_M", 5);
+    const int64_t min_m = fnn_ctx_option(ctx, FNN_OPT_TILE_MIN_M);
     if (q.m < min_m) return FNN_OK;
     if (w->dtype == FNN_DT_I4CB) {
         if (q.as_written || q.qblock <= 0 || q.n > (1 << 24) || q.m > (1 << 22)) return FNN_OK;

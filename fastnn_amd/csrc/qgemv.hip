@@ -156,13 +156,6 @@ __global__ void __launch_bounds__(MAXT) qgemv_kernel(QMatmulArgs p)
     }
 }
 
-int env_int(const char *name, int dflt)
-{
-    const char *s = getenv(name);
-    if (!s || !*s) return dflt;
-    return atoi(s);
-}
-
 template <int DT, int MT, int RG, int MAXT>
 hipError_t launch_one(const QMatmulArgs &p, int nw, hipStream_t s)
 {
@@ -186,12 +179,6 @@ hipError_t launch_rg(const QMatmulArgs &p, hipStream_t s)
     // rows per workgroup: enough workgroups to give every CU (256) a few.
     int rg = (p.n >= 16384) ? 8 : 4;
     if (p.n <= 1024) rg = 2;
-    static const int env_nw = env_int("FNN_GEMV_NW", 0);  // tuning overrides, read once
-    static const int env_rg = env_int("FNN_GEMV_RG", 0);
-    if (env_nw > 0) nw = env_nw;
-    if (env_rg > 0) rg = env_rg;
-    if (nw < 1) nw = 1;
-    if (nw > MAXT / 64) nw = MAXT / 64;
     switch (rg) {
     case 2: return launch_one<DT, MT, 2, MAXT>(p, nw, s);
     case 8: return launch_one<DT, MT, 8, MAXT>(p, nw, s);

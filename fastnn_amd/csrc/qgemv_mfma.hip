@@ -255,21 +255,13 @@ void launch_rt(const GemvArgs &p, hipStream_t s)
     else if (mm == 2) hipLaunchKernelGGL((qgemv_mfma_kernel<DT, RT, 2, SINGLE, NW>), grid, blk, lds, s, p);
     else if (mm == 4) {
         auto kern = qgemv_mfma_kernel<DT, RT, 4, SINGLE, NW>;
-        static bool attr_set = false;   // up to 64 KiB of dynamic LDS plus the static reduction buffers
-        if (!attr_set) {
-            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
-            attr_set = true;
-        }
+        static std::atomic<uint64_t> lds_raised{0};   // up to 64 KiB of dynamic LDS plus the static reduction buffers
+        (void)fnn_raise_lds_limit(lds_raised, reinterpret_cast<const void *>(kern), 96 * 1024);
         hipLaunchKernelGGL(kern, grid, blk, lds, s, p);
     } else {
         auto kern = qgemv_mfma_kernel<DT, RT, 8, SINGLE, NW>;
-        static bool attr_set = false;   // up to 128 KiB of dynamic LDS: one workgroup per CU
-        if (!attr_set) {
-            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
-            attr_set = true;
-        }
+        static std::atomic<uint64_t> lds_raised{0};   // up to 128 KiB of dynamic LDS: one workgroup per CU
+        (void)fnn_raise_lds_limit(lds_raised, reinterpret_cast<const void *>(kern), 128 * 1024);
         hipLaunchKernelGGL(kern, grid, blk, lds, s, p);
     }
 }
@@ -278,9 +270,8 @@ void launch_rt(const GemvArgs &p, hipStream_t s)
 // row tiles, so more tiles mean less repeated work (the larger M, the more it weighs), but the workgroups
 // should still come in whole rounds over the 256 CUs: cost ~ rounds * (conversion + tiles).
 // C2 (N = 11008): M=2 9.2 -> 8.2 us, M=4 12.3 -> 9.4 us with three tiles; at M=1 one tile is as fast or faster.
-inline int gemv_row_tiles(int64_t n, int64_t m, int nw)
+inline int gemv_row_tiles(int64_t n, int64_t m, int nw, int forced)
 {
-    static const int forced = [] { const char *e = getenv("FNN_GEMV_RT"); return e ? atoi(e) : 0; }();
     if (m <= 1) return 1;   // one activation row: the conversion is cheap and more workgroups in flight win (measured)
     const int mm = m <= 2 ? 2 : (m <= 4 ? 4 : 8);
     if (forced >= 1 && forced <= 3 && forced * mm * 16 <= nw * 64) return forced;
@@ -297,9 +288,9 @@ inline int gemv_row_tiles(int64_t n, int64_t m, int nw)
 }
 
 template <int DT, bool SINGLE, int NW>
-void launch_mm(const GemvArgs &p, hipStream_t s)
+void launch_mm(const GemvArgs &p, int forced_rt, hipStream_t s)
 {
-    switch (gemv_row_tiles(p.n, p.m, NW)) {
+    switch (gemv_row_tiles(p.n, p.m, NW, forced_rt)) {
     case 3: launch_rt<DT, 3, SINGLE, NW>(p, s); break;
     case 2: launch_rt<DT, 2, SINGLE, NW>(p, s); break;
     default: launch_rt<DT, 1, SINGLE, NW>(p, s); break;
@@ -307,13 +298,13 @@ void launch_mm(const GemvArgs &p, hipStream_t s)
 }
 
 template <int DT>
-hipError_t launch_gemv(const GemvArgs &p, bool single, hipStream_t s)
+hipError_t launch_gemv(const GemvArgs &p, bool single, int forced_rt, hipStream_t s)
 {
     // 8 waves split K in slices of 512; short K (<= 2048) runs 4-wave workgroups so that no wave idles
     if (p.k <= 4 * GV_SLICE) {
-        if (single) launch_mm<DT, true, 4>(p, s); else launch_mm<DT, false, 4>(p, s);
+        if (single) launch_mm<DT, true, 4>(p, forced_rt, s); else launch_mm<DT, false, 4>(p, forced_rt, s);
     } else {
-        if (single) launch_mm<DT, true, 8>(p, s); else launch_mm<DT, false, 8>(p, s);
+        if (single) launch_mm<DT, true, 8>(p, forced_rt, s); else launch_mm<DT, false, 8>(p, forced_rt, s);
     }
     return hipGetLastError();
 }
@@ -336,15 +327,16 @@ int fnn_mfma_qgemv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, con
         int rc = fnn_row_means(ctx, s, w, &p.umean);
         if (rc) return rc;
     }
+    const int rt = (int)fnn_ctx_option(ctx, FNN_OPT_GEMV_ROW_TILES);   // 0: by the cost model
     hipError_t e;
     switch (w->dtype) {
-    case FNN_DT_I8: e = launch_gemv<FNN_DT_I8>(p, single, s); break;
-    case FNN_DT_I4: e = launch_gemv<FNN_DT_I4>(p, single, s); break;
-    case FNN_DT_U8: e = launch_gemv<FNN_DT_U8>(p, single, s); break;
-    case FNN_DT_U4: e = launch_gemv<FNN_DT_U4>(p, single, s); break;
-    case FNN_DT_F8: e = launch_gemv<FNN_DT_F8>(p, single, s); break;
-    case FNN_DT_F8R: e = launch_gemv<FNN_DT_F8R>(p, single, s); break;
-    case FNN_DT_F4: e = launch_gemv<FNN_DT_F4>(p, single, s); break;
+    case FNN_DT_I8: e = launch_gemv<FNN_DT_I8>(p, single, rt, s); break;
+    case FNN_DT_I4: e = launch_gemv<FNN_DT_I4>(p, single, rt, s); break;
+    case FNN_DT_U8: e = launch_gemv<FNN_DT_U8>(p, single, rt, s); break;
+    case FNN_DT_U4: e = launch_gemv<FNN_DT_U4>(p, single, rt, s); break;
+    case FNN_DT_F8: e = launch_gemv<FNN_DT_F8>(p, single, rt, s); break;
+    case FNN_DT_F8R: e = launch_gemv<FNN_DT_F8R>(p, single, rt, s); break;
+    case FNN_DT_F4: e = launch_gemv<FNN_DT_F4>(p, single, rt, s); break;
     default: return FNN_OK;
     }
     if (e != hipSuccess) return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, hipGetErrorString(e));

@@ -258,9 +258,8 @@ __global__ void __launch_bounds__(NW * 64) qgemv_rows16_kernel(Rows16Args p)
 // row tiles per workgroup: the activation block is converted once per workgroup, so as many as the registers
 // allow while the workgroups still cover the CUs
 template <int DT>
-inline int rows16_tiles(int64_t n)
+inline int rows16_tiles(int64_t n, int forced)
 {
-    static const int forced = [] { const char *e = getenv("FNN_ROWS16_RT"); return e ? atoi(e) : 0; }();
     constexpr int max_rt = DecH<DT>::WPS == 1 ? 3 : 2;   // 8-bit types hold twice the packed words per tile
     if (forced >= 1 && forced <= max_rt) return forced;
     int best = 1;
@@ -281,9 +280,9 @@ void launch_rt(const Rows16Args &p, hipStream_t s)
 }
 
 template <int DT, bool SINGLE, int NW>
-void launch_nw(const Rows16Args &p, hipStream_t s)
+void launch_nw(const Rows16Args &p, int forced_rt, hipStream_t s)
 {
-    const int rt = rows16_tiles<DT>(p.n);
+    const int rt = rows16_tiles<DT>(p.n, forced_rt);
     if constexpr (DecH<DT>::WPS == 1) {
         if (rt == 3) { launch_rt<DT, 3, SINGLE, NW>(p, s); return; }
     }
@@ -292,13 +291,13 @@ void launch_nw(const Rows16Args &p, hipStream_t s)
 }
 
 template <int DT>
-hipError_t launch_rows16(const Rows16Args &p, bool single, hipStream_t s)
+hipError_t launch_rows16(const Rows16Args &p, bool single, int forced_rt, hipStream_t s)
 {
     // 8 waves split K in slices of 512; short K (<= 2048) runs 4-wave workgroups so that no wave idles
     if (p.k <= 4 * R16_SLICE) {
-        if (single) launch_nw<DT, true, 4>(p, s); else launch_nw<DT, false, 4>(p, s);
+        if (single) launch_nw<DT, true, 4>(p, forced_rt, s); else launch_nw<DT, false, 4>(p, forced_rt, s);
     } else {
-        if (single) launch_nw<DT, true, 8>(p, s); else launch_nw<DT, false, 8>(p, s);
+        if (single) launch_nw<DT, true, 8>(p, forced_rt, s); else launch_nw<DT, false, 8>(p, forced_rt, s);
     }
     return hipGetLastError();
 }
@@ -309,7 +308,7 @@ int fnn_mfma_rows16(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, co
                     int flags, bool *handled)
 {
     *handled = false;
-    static const int min_m = [] { const char *e = getenv("FNN_ROWS16_MIN_M"); return e ? atoi(e) : 9; }();
+    const int64_t min_m = fnn_ctx_option(ctx, FNN_OPT_ROWS16_MIN_M);
     if (q.m < min_m || q.m > 16 || w->dtype == FNN_DT_I4CB) return FNN_OK;
     if (q.kp % 4 != 0 || q.k % 8 != 0) return FNN_OK;
     if ((reinterpret_cast<uintptr_t>(q.a) & 15) || (reinterpret_cast<uintptr_t>(q.words) & 15)) return FNN_OK;
@@ -322,15 +321,16 @@ int fnn_mfma_rows16(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, co
         int rc = fnn_row_means(ctx, s, w, &p.umean);
         if (rc) return rc;
     }
+    const int rt = (int)fnn_ctx_option(ctx, FNN_OPT_ROWS16_ROW_TILES);   // 0: by the cost model
     hipError_t e;
     switch (w->dtype) {
-    case FNN_DT_I8: e = launch_rows16<FNN_DT_I8>(p, single, s); break;
-    case FNN_DT_I4: e = launch_rows16<FNN_DT_I4>(p, single, s); break;
-    case FNN_DT_U8: e = launch_rows16<FNN_DT_U8>(p, single, s); break;
-    case FNN_DT_U4: e = launch_rows16<FNN_DT_U4>(p, single, s); break;
-    case FNN_DT_F8: e = launch_rows16<FNN_DT_F8>(p, single, s); break;
-    case FNN_DT_F8R: e = launch_rows16<FNN_DT_F8R>(p, single, s); break;
-    case FNN_DT_F4: e = launch_rows16<FNN_DT_F4>(p, single, s); break;
+    case FNN_DT_I8: e = launch_rows16<FNN_DT_I8>(p, single, rt, s); break;
+    case FNN_DT_I4: e = launch_rows16<FNN_DT_I4>(p, single, rt, s); break;
+    case FNN_DT_U8: e = launch_rows16<FNN_DT_U8>(p, single, rt, s); break;
+    case FNN_DT_U4: e = launch_rows16<FNN_DT_U4>(p, single, rt, s); break;
+    case FNN_DT_F8: e = launch_rows16<FNN_DT_F8>(p, single, rt, s); break;
+    case FNN_DT_F8R: e = launch_rows16<FNN_DT_F8R>(p, single, rt, s); break;
+    case FNN_DT_F4: e = launch_rows16<FNN_DT_F4>(p, single, rt, s); break;
     default: return FNN_OK;
     }
     if (e != hipSuccess) return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, hipGetErrorString(e));

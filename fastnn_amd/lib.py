@@ -22,16 +22,24 @@ FLAG_I4CB_AS_WRITTEN = 2
 FLAG_ACT_F16_SINGLE = 4
 FLAG_FORCE_GENERIC = 8
 FLAG_PREFER_FMA = 16
+OPT_CODEBOOK_CACHE = 1
+OPT_GEMV_ROW_TILES = 2
+OPT_ROWS16_ROW_TILES = 3
+OPT_ROWS16_MIN_M = 4
+OPT_TILE_SHAPE = 5
+OPT_TILE_SPLIT = 6
+OPT_TILE_STAGES = 7
+OPT_TILE_MIN_M = 8
 
 STATUS_NAMES = {0: "Ok", 1: "Dispatch", 2: "Memory", 3: "UnsupportedOp", 4: "Compilation"}
 
 # every symbol include/fastnn_hip.h declares
 EXPORTED_SYMBOLS = [
-    "fnn_hip_device_count", "fnn_hip_create", "fnn_hip_destroy", "fnn_hip_last_error", "fnn_hip_sync",
+    "fnn_hip_device_count", "fnn_hip_create", "fnn_hip_destroy", "fnn_hip_last_error", "fnn_hip_sync", "fnn_hip_set_option", "fnn_hip_get_option", "fnn_hip_stream",
     "fnn_hip_malloc", "fnn_hip_free", "fnn_hip_upload", "fnn_hip_download",
     "fnn_hip_weight_register", "fnn_hip_weight_lookup", "fnn_hip_weight_release", "fnn_hip_dequant",
     "fnn_hip_qmatmul", "fnn_hip_quantize_activations", "fnn_hip_dequantize_activations", "fnn_hip_qmatmul_i8act", "fnn_hip_qconv2d", "fnn_hip_qconv2d_i8act",
-    "fnn_hip_timer_start", "fnn_hip_timer_stop", "fnn_hip_probe_stream",
+    "fnn_hip_timer_start", "fnn_hip_timer_stop",
     "fnn_hip_graph_begin", "fnn_hip_graph_end", "fnn_hip_graph_launch", "fnn_hip_graph_destroy",
     "fnn_hip_workspace_epoch",
     "fnn_packed_words", "fnn_quantize_weights", "fnn_transpose_kn_to_nk", "fnn_hip_version",
@@ -39,7 +47,7 @@ EXPORTED_SYMBOLS = [
 # every symbol include/fastnn_hip_backend.h declares
 BACKEND_SYMBOLS = [
     "fnn_backend_create", "fnn_backend_destroy", "fnn_backend_name", "fnn_backend_last_error",
-    "fnn_backend_set_kernel_flags",
+    "fnn_backend_set_kernel_flags", "fnn_backend_set_graph_replay", "fnn_backend_set_option",
     "fnn_backend_allocate_arena", "fnn_backend_write_arena", "fnn_backend_read_arena",
     "fnn_plan_create", "fnn_plan_destroy", "fnn_plan_add_write_const", "fnn_plan_add_fill",
     "fnn_plan_add_memcopy", "fnn_plan_add_call_kernel", "fnn_plan_len", "fnn_plan_replayed",
@@ -94,7 +102,7 @@ class WeightMeta(C.Structure):
     """fnn_weight_meta: QuantizedWeightMeta."""
     _fields_ = [("bit_width", C.c_uint64), ("scales", _vp), ("n_scales", C.c_uint64),
                 ("zero_points", _vp), ("n_zero_points", C.c_uint64), ("shape", _vp), ("n_shape", C.c_uint64),
-                ("quant_block_size", C.c_uint64), ("codebook16", _vp)]
+                ("quant_block_size", C.c_uint64), ("codebooks", _vp), ("n_codebooks", C.c_uint64)]
 
 
 def _prototype(l):
@@ -105,6 +113,10 @@ def _prototype(l):
     l.fnn_hip_last_error.argtypes = [_vp]
     l.fnn_hip_last_error.restype = C.c_char_p
     l.fnn_hip_sync.argtypes = [_vp]
+    l.fnn_hip_set_option.argtypes = [_vp, C.c_int, _i64]
+    l.fnn_hip_get_option.argtypes = [_vp, C.c_int, C.POINTER(_i64)]
+    l.fnn_hip_stream.argtypes = [_vp]
+    l.fnn_hip_stream.restype = _vp
     l.fnn_hip_malloc.argtypes = [_vp, _sz, C.POINTER(_vp)]
     l.fnn_hip_free.argtypes = [_vp, _vp]
     l.fnn_hip_upload.argtypes = [_vp, _vp, _vp, _sz]
@@ -121,7 +133,6 @@ def _prototype(l):
                                   C.c_int, C.c_int, _vp, C.c_int, _vp, _vp, C.c_int]
     l.fnn_hip_qconv2d_i8act.argtypes = [_vp, _vp, _vp, _i64, _i64, _i64, _i64, C.c_int, C.c_int, C.c_int, C.c_int,
                                         C.c_int, C.c_int, _vp, C.c_int, _vp, C.c_int]
-    l.fnn_hip_probe_stream.argtypes = [_vp, _vp, _vp, _sz]
     l.fnn_hip_timer_start.argtypes = [_vp]
     l.fnn_hip_timer_stop.argtypes = [_vp, C.POINTER(C.c_float)]
     l.fnn_hip_graph_begin.argtypes = [_vp]
@@ -142,6 +153,8 @@ def _prototype(l):
     l.fnn_backend_name.argtypes = [_vp]
     l.fnn_backend_name.restype = C.c_char_p
     l.fnn_backend_set_kernel_flags.argtypes = [_vp, C.c_int]
+    l.fnn_backend_set_graph_replay.argtypes = [_vp, C.c_int]
+    l.fnn_backend_set_option.argtypes = [_vp, C.c_int, _i64]
     l.fnn_backend_last_error.argtypes = [_vp]
     l.fnn_backend_last_error.restype = C.c_char_p
     l.fnn_backend_allocate_arena.argtypes = [_vp, _u64]
@@ -153,8 +166,8 @@ def _prototype(l):
     l.fnn_plan_add_write_const.argtypes = [_vp, Slice, _vp, _u64]
     l.fnn_plan_add_fill.argtypes = [_vp, Slice, C.c_float]
     l.fnn_plan_add_memcopy.argtypes = [_vp, Slice, Slice]
-    l.fnn_plan_add_call_kernel.argtypes = [_vp, C.c_char_p, C.POINTER(Slice), _u64, Slice, C.POINTER(_u64), _u64,
-                                           C.POINTER(WeightMeta)]
+    l.fnn_plan_add_call_kernel.argtypes = [_vp, C.c_char_p, C.POINTER(Slice), _u64, Slice, C.POINTER(Slice),
+                                           C.POINTER(_u64), _u64, C.POINTER(WeightMeta)]
     l.fnn_plan_len.argtypes = [_vp]
     l.fnn_plan_len.restype = _u64
     l.fnn_plan_replayed.argtypes = [_vp]
@@ -164,6 +177,10 @@ def _prototype(l):
     l.fnn_hip_elementwise.argtypes = [_vp, C.c_int, _vp, _vp, _u64, _vp, _u64]
     l.fnn_hip_fill_f32.argtypes = [_vp, _vp, _u64, C.c_float]
     l.fnn_hip_copy.argtypes = [_vp, _vp, _vp, _u64]
+    l.fnn_hip_copy2d_f32.argtypes = [_vp, _vp, _u64, _u64, _vp, _u64, _u64, _u64, _u64]
+    l.fnn_hip_maxpool2d_f32.argtypes = [_vp, _vp, _u64, _vp, _u64, _u64, _u64, _u64, _u64, _u64, _u64, _u64, _vp, _u64]
+    l.fnn_hip_avgpool2d_f32.argtypes = [_vp, _vp, _u64, _vp, _u64, _u64, _u64, _u64, _u64, _u64, _u64, _u64]
+    l.fnn_hip_upsample_nearest2d_f32.argtypes = [_vp, _vp, _vp, _u64, _u64, _u64, _u64, _u64]
 
 
 def _np_ptr(a: Optional[np.ndarray]):
@@ -294,6 +311,15 @@ class HipContext:
     def sync(self):
         self._check(self.lib.fnn_hip_sync(self.handle))
 
+    def set_option(self, option: int, value: int):
+        """fnn_hip_set_option: per-context kernel selection (OPT_* constants)."""
+        self._check(self.lib.fnn_hip_set_option(self.handle, option, value))
+
+    def get_option(self, option: int) -> int:
+        v = _i64()
+        self._check(self.lib.fnn_hip_get_option(self.handle, option, C.byref(v)))
+        return v.value
+
     def alloc(self, nbytes: int) -> DeviceBuffer:
         return DeviceBuffer(self, nbytes)
 
@@ -388,8 +414,9 @@ class HipContext:
         return y
 
     # ---- timing / graphs ----
-    def probe_stream(self, src_ptr: int, dst_ptr: int, nbytes: int):
-        self._check(self.lib.fnn_hip_probe_stream(self.handle, _vp(src_ptr), _vp(dst_ptr) if dst_ptr else None, nbytes))
+    def stream(self) -> int:
+        """The context's hipStream_t as an integer (fnn_hip_stream)."""
+        return self.lib.fnn_hip_stream(self.handle) or 0
 
     def timer_start(self):
         self._check(self.lib.fnn_hip_timer_start(self.handle))

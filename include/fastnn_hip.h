@@ -9,8 +9,9 @@
  *
  * Conventions
  *   - every function returns an fnn_status; nothing throws or aborts across
- *     the boundary; the message of the last failure on a context is returned
- *     by fnn_hip_last_error();
+ *     the boundary (every entry point catches C++ exceptions: std::bad_alloc
+ *     becomes FNN_ERR_MEMORY, anything else FNN_ERR_DISPATCH); the message of
+ *     the last failure on a context is returned by fnn_hip_last_error();
  *   - one context = one device + one HIP stream; a context is not re-entrant,
  *     matching the single-threaded dispatch contract of
  *     src/backend/cpu/mod.rs:176-188;
@@ -81,6 +82,27 @@ int fnn_hip_malloc(fnn_hip_ctx *ctx, size_t bytes, void **dptr);
 int fnn_hip_free(fnn_hip_ctx *ctx, void *dptr);
 int fnn_hip_upload(fnn_hip_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes);
 int fnn_hip_download(fnn_hip_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes);
+
+/* Per-context options (no counterpart in fastnn, whose CPU kernels read tuning values from the environment once per
+ * process): kernel selection for measurements and tests.  Defaults give the automatic choice.  Unknown options and
+ * values out of range are refused with FNN_ERR_DISPATCH; graphs captured earlier keep the choice of their capture. */
+enum {
+    FNN_OPT_CODEBOOK_CACHE = 1,   /* 1 (default): a codebook weight keeps its f16 expansion (8x the packed bytes)   */
+                                  /* after its first MatMul with M >= 5; 0: a call expands into a workspace         */
+    FNN_OPT_GEMV_ROW_TILES = 2,   /* M <= 8 kernel: 16-row tiles per workgroup, 1..3; 0 (default) = cost model      */
+    FNN_OPT_ROWS16_ROW_TILES = 3, /* 9 <= M <= 16 kernel: the same                                                  */
+    FNN_OPT_ROWS16_MIN_M = 4,     /* smallest M the 16-row kernel takes (default 9; 17 switches it off)             */
+    FNN_OPT_TILE_SHAPE = 5,       /* tiled GEMM: 0 = 128x128, 1 = 64x128, 2 = 32x128; -1 (default) = by shape       */
+    FNN_OPT_TILE_SPLIT = 6,       /* tiled GEMM: K split over this many workgroups; 0 (default) = cost model        */
+    FNN_OPT_TILE_STAGES = 7,      /* tiled GEMM, 128x128 tiles: 5 = deep ring, 3 = shallow; 0 (default) = by shape  */
+    FNN_OPT_TILE_MIN_M = 8,       /* smallest M the tiled GEMM takes (default 5)                                    */
+    FNN_OPT_COUNT = 9
+};
+int fnn_hip_set_option(fnn_hip_ctx *ctx, int option, int64_t value);
+int fnn_hip_get_option(fnn_hip_ctx *ctx, int option, int64_t *value);
+/* The context's hipStream_t as an opaque pointer, for callers that enqueue work of their own in order with the
+ * library's (no counterpart in fastnn). */
+void *fnn_hip_stream(fnn_hip_ctx *ctx);
 
 /* ---- weights: get_or_cache_packed + packed_tensor_from_meta,
  * src/backend/cpu/mod.rs:62-89, src/backend/cpu/matmul.rs:81-152.
@@ -163,12 +185,6 @@ int fnn_hip_qconv2d_i8act(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const uint8
  * HIP events recorded on the context's stream. */
 int fnn_hip_timer_start(fnn_hip_ctx *ctx);
 int fnn_hip_timer_stop(fnn_hip_ctx *ctx, float *elapsed_ms);
-
-/* Memory-system probe (no counterpart in fastnn; measurement aid): one launch that streams
- * `bytes` from src_dev (16-byte aligned device pointers); dst_dev == NULL reads only,
- * otherwise copies.  Gives the bandwidth a single launch of that size reaches on the
- * device and a kernel of known traffic to calibrate hardware byte counters with. */
-int fnn_hip_probe_stream(fnn_hip_ctx *ctx, const void *src_dev, void *dst_dev, size_t bytes);
 
 /* ---- HIP graphs over device-pointer calls: capture a dispatch sequence once,
  * replay it with one launch (a static-shape plan, src/backend/executor.rs:639-667). */

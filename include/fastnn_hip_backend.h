@@ -27,7 +27,9 @@ typedef struct {
     uint64_t size;
 } fnn_slice;
 
-/* QuantizedWeightMeta, src/backend/mod.rs:40-58 (codebook16 == NULL: no codebook) */
+/* QuantizedWeightMeta, src/backend/mod.rs:40-58.  codebooks: n_codebooks x 16 floats (Vec<[f32; 16]>), 0 = no
+ * codebook.  Like every decode of the reference (src/packed_tensor.rs:398, 489, 586) the kernels read
+ * codebooks[0] only, whatever n_codebooks is. */
 typedef struct {
     uint64_t bit_width;
     const float *scales;
@@ -37,7 +39,8 @@ typedef struct {
     const uint64_t *shape;
     uint64_t n_shape;
     uint64_t quant_block_size;
-    const float *codebook16;
+    const float *codebooks;
+    uint64_t n_codebooks;
 } fnn_weight_meta;
 
 /* Backend::name / allocate_arena / write_arena / read_arena, src/backend/mod.rs:152-254 */
@@ -49,6 +52,11 @@ const char *fnn_backend_name(const fnn_backend *b);
  * less time at M >= 64; FNN_FLAG_FORCE_GENERIC / FNN_FLAG_PREFER_FMA select kernels for testing.  Other bits
  * are refused.  Plans captured before the change are captured again. */
 int fnn_backend_set_kernel_flags(fnn_backend *b, int flags);
+/* Resident plans replay as one HIP graph (default, enabled != 0) or run instruction by instruction on every
+ * dispatch (enabled == 0); no counterpart in fastnn. */
+int fnn_backend_set_graph_replay(fnn_backend *b, int enabled);
+/* fnn_hip_set_option on the backend's context (FNN_OPT_*); plans captured before the change are captured again. */
+int fnn_backend_set_option(fnn_backend *b, int option, int64_t value);
 const char *fnn_backend_last_error(const fnn_backend *b);
 int fnn_backend_allocate_arena(fnn_backend *b, uint64_t total_bytes);
 int fnn_backend_write_arena(fnn_backend *b, uint64_t offset, const void *data, uint64_t size);
@@ -62,18 +70,23 @@ int fnn_plan_add_fill(fnn_plan *p, fnn_slice dst, float value);
 int fnn_plan_add_memcopy(fnn_plan *p, fnn_slice dst, fnn_slice src);
 /* kernel_name as CpuBackend::compile emits it (src/backend/cpu/mod.rs:415-495, 815-865);
  * a quantised MatMul may carry the epilogue the fusion pass attached as a suffix
- * "_relu" | "_gelu" | "_silu" and a third input slice for the bias. */
+ * "_relu" | "_gelu" | "_silu" and a third input slice for the bias.
+ * secondary_output: CallKernel.secondary_output_slice (src/backend/mod.rs:66-67), NULL for None; "pool_f32" with
+ * is_max = 1 writes the i64 window position kh*kernel + kw of each maximum there
+ * (src/backend/cpu/mod.rs:4402-4410, src/backend/cpu/microkernels/ops.rs:150-155); other kernels ignore it.
+ * params are resolved values: a caller with symbolic dims (param_dims + ShapeEnv,
+ * src/backend/cpu/params.rs:11-39) resolves them before building the plan. */
 int fnn_plan_add_call_kernel(fnn_plan *p, const char *kernel_name, const fnn_slice *inputs,
-                             uint64_t n_inputs, fnn_slice output, const uint64_t *params,
-                             uint64_t n_params, const fnn_weight_meta *meta);
+                             uint64_t n_inputs, fnn_slice output, const fnn_slice *secondary_output,
+                             const uint64_t *params, uint64_t n_params, const fnn_weight_meta *meta);
 uint64_t fnn_plan_len(const fnn_plan *p);
 
 /* Backend::dispatch, src/backend/mod.rs:167-176.  Synchronises before returning.
  * The first dispatch of a plan uploads its WriteConst payloads and runs instruction by
  * instruction; while the constants stay in place (fnn_backend_write_arena elsewhere in the arena
- * does not disturb them) later dispatches skip the uploads and replay the instruction stream as
- * one HIP graph, the static-shape plan reuse of src/backend/executor.rs:639-667.
- * FNN_PLAN_GRAPH=0 in the environment keeps every dispatch instruction by instruction. */
+ * does not disturb them, and neither does what another plan dispatched on this backend wrote) later
+ * dispatches skip the uploads and replay the instruction stream as one HIP graph, the static-shape plan
+ * reuse of src/backend/executor.rs:639-667 (see fnn_backend_set_graph_replay). */
 int fnn_backend_dispatch(fnn_backend *b, fnn_plan *p);
 /* 1 when the last dispatch of the plan ran as a graph replay, else 0 (no counterpart in fastnn:
  * lets tests and tools see which path ran). */
@@ -92,7 +105,8 @@ int fnn_hip_elementwise(fnn_hip_ctx *ctx, int op, const float *a, const float *b
  *    index leaves its buffer: the block copies of "concat" (src/backend/cpu/mod.rs:4267-4324) and "slice_f32"
  *    (:4721-4760);
  *  maxpool2d: "pool_f32" with is_max = 1 (:4362-4397, src/backend/cpu/microkernels/ops.rs:104-158), output
- *    Ho = sat_sub(H + 2*pad, kernel)/stride + 1, writes past out_len dropped;
+ *    Ho = sat_sub(H + 2*pad, kernel)/stride + 1, writes past out_len dropped; indices (nullable, idx_len i64
+ *    entries) receives kh*kernel + kw of the first strict maximum in (kh, kw) order, 0 for an empty window;
  *  avgpool2d: "pool_f32" with is_max != 1 (:4398-4470, ops.rs:162-210): the mean over the taps inside the image
  *    (padding taps are not counted), summed in (kh, kw) order;
  *  upsample_nearest2d: "upsample_nearest2d" (:5496-5535, src/backend/cpu/microkernels/misc.rs:338-364). */
@@ -100,7 +114,7 @@ int fnn_hip_copy2d_f32(fnn_hip_ctx *ctx, float *dst, uint64_t dst_pitch, uint64_
                        uint64_t src_pitch, uint64_t src_len, uint64_t width, uint64_t height);
 int fnn_hip_maxpool2d_f32(fnn_hip_ctx *ctx, const float *x, uint64_t in_len, float *y, uint64_t out_len,
                           uint64_t n, uint64_t c, uint64_t h, uint64_t w, uint64_t kernel, uint64_t stride,
-                          uint64_t pad);
+                          uint64_t pad, int64_t *indices, uint64_t idx_len);
 int fnn_hip_avgpool2d_f32(fnn_hip_ctx *ctx, const float *x, uint64_t in_len, float *y, uint64_t out_len,
                           uint64_t n, uint64_t c, uint64_t h, uint64_t w, uint64_t kernel, uint64_t stride,
                           uint64_t pad);

@@ -1342,9 +1342,12 @@ void fnn_or_slice(const float *in, size_t in_len, size_t start, size_t end, size
 
 /* "pool_f32" with is_max = 1 (backend/cpu/mod.rs:4362-4397, microkernels/ops.rs:104-158):
  * params [kernel, stride, padding, is_max, N, C, H, W]; Ho = sat_sub(H + 2p, kernel)/stride + 1;
- * the window maximum starts at -inf and is replaced on a strict `>`; taps in the padding are skipped. */
+ * the window maximum starts at -inf and is replaced on a strict `>`; taps in the padding are skipped.
+ * indices (nullable, the CallKernel's secondary output; ops.rs:110-155): best_kh*kernel + best_kw of the
+ * tap that last replaced the maximum, (0, 0) when none did. */
 void fnn_or_maxpool2d(const float *in, size_t in_len, size_t n, size_t c, size_t h, size_t w,
-                      size_t kernel, size_t stride, size_t pad, float *out, size_t out_len)
+                      size_t kernel, size_t stride, size_t pad, float *out, size_t out_len,
+                      int64_t *indices, size_t idx_len)
 {
     size_t hp = h + 2 * pad, wp = w + 2 * pad;
     size_t ho = (hp > kernel ? hp - kernel : 0) / stride + 1;
@@ -1354,6 +1357,7 @@ void fnn_or_maxpool2d(const float *in, size_t in_len, size_t n, size_t c, size_t
             for (size_t hh = 0; hh < ho; hh++)
                 for (size_t ww = 0; ww < wo; ww++) {
                     float val = -INFINITY;
+                    size_t best_kh = 0, best_kw = 0;
                     for (size_t kh = 0; kh < kernel; kh++)
                         for (size_t kw = 0; kw < kernel; kw++) {
                             size_t hi = hh * stride + kh, wi = ww * stride + kw;
@@ -1362,10 +1366,15 @@ void fnn_or_maxpool2d(const float *in, size_t in_len, size_t n, size_t c, size_t
                             wi -= pad;
                             if (hi >= h || wi >= w) continue;
                             size_t idx = nn * (c * h * w) + cc * (h * w) + hi * w + wi;
-                            if (idx < in_len && in[idx] > val) val = in[idx];
+                            if (idx < in_len && in[idx] > val) {
+                                val = in[idx];
+                                best_kh = kh;
+                                best_kw = kw;
+                            }
                         }
                     size_t o = nn * (c * ho * wo) + cc * (ho * wo) + hh * wo + ww;
                     if (o < out_len) out[o] = val;
+                    if (indices && o < idx_len) indices[o] = (int64_t)(best_kh * kernel + best_kw);
                 }
 }
 

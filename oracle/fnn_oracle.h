@@ -135,7 +135,8 @@ void fnn_or_slice(const float *in, size_t in_len, size_t start, size_t end, size
 void fnn_or_avgpool2d(const float *in, size_t in_len, size_t n, size_t c, size_t h, size_t w,
                       size_t kernel, size_t stride, size_t pad, float *out, size_t out_len);
 void fnn_or_maxpool2d(const float *in, size_t in_len, size_t n, size_t c, size_t h, size_t w,
-                      size_t kernel, size_t stride, size_t pad, float *out, size_t out_len);
+                      size_t kernel, size_t stride, size_t pad, float *out, size_t out_len,
+                      int64_t *indices, size_t idx_len);
 void fnn_or_upsample_nearest2d(const float *in, size_t nc, size_t h, size_t w, size_t sh, size_t sw,
                                float *out);
 

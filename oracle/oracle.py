@@ -106,7 +106,7 @@ def _proto(l):
     l.fnn_or_concat.argtypes = [C.c_void_p, C.c_void_p, _sz, _sz, _f32p, _sz]
     l.fnn_or_concat.restype = _sz
     l.fnn_or_slice.argtypes = [_f32p, _sz, _sz, _sz, _sz, _f32p, _sz]
-    l.fnn_or_maxpool2d.argtypes = [_f32p, _sz, _sz, _sz, _sz, _sz, _sz, _sz, _sz, _f32p, _sz]
+    l.fnn_or_maxpool2d.argtypes = [_f32p, _sz, _sz, _sz, _sz, _sz, _sz, _sz, _sz, _f32p, _sz, C.c_void_p, _sz]
     l.fnn_or_avgpool2d.argtypes = [_f32p, _sz, _sz, _sz, _sz, _sz, _sz, _sz, _sz, _f32p, _sz]
     l.fnn_or_upsample_nearest2d.argtypes = [_f32p, _sz, _sz, _sz, _sz, _sz, _f32p]
     l.fnn_or_seeded_values.argtypes = [C.c_uint64, _sz, _f32p]
@@ -349,14 +349,17 @@ def slice_f32(x, start: int, end: int, stride: int, out_len: int) -> np.ndarray:
     return out
 
 
-def maxpool2d(x, kernel: int, stride: int, pad: int) -> np.ndarray:
+def maxpool2d(x, kernel: int, stride: int, pad: int, return_indices: bool = False):
+    """"pool_f32" with is_max = 1; with return_indices also the i64 secondary output (kh*kernel + kw per window)."""
     x = _f32(x)
     n, c, h, w = x.shape
     ho = max(h + 2 * pad - kernel, 0) // stride + 1
     wo = max(w + 2 * pad - kernel, 0) // stride + 1
     out = np.zeros((n, c, ho, wo), np.float32)
-    lib().fnn_or_maxpool2d(x.reshape(-1), x.size, n, c, h, w, kernel, stride, pad, out.reshape(-1), out.size)
-    return out
+    idx = np.zeros((n, c, ho, wo), np.int64) if return_indices else None
+    lib().fnn_or_maxpool2d(x.reshape(-1), x.size, n, c, h, w, kernel, stride, pad, out.reshape(-1), out.size,
+                           None if idx is None else idx.ctypes.data_as(C.c_void_p), 0 if idx is None else idx.size)
+    return (out, idx) if return_indices else out
 
 
 def avgpool2d(x, kernel: int, stride: int, pad: int) -> np.ndarray:

@@ -44,8 +44,26 @@ def test_plan_builds_without_a_gpu():
                   dict(bit_width=8, scales=[1.0], zero_points=[0.0], shape=[16, 16]))
     assert len(p) == 4
     l = fastnn_amd.load_library()
-    assert l.fnn_plan_add_call_kernel(p.handle, None, None, 0, flib.Slice(0, 0), None, 0, None) != 0
+    assert l.fnn_plan_add_call_kernel(p.handle, None, None, 0, flib.Slice(0, 0), None, None, 0, None) != 0
+    assert b"NULL argument" in l.fnn_backend_last_error(None)
+    # CallKernel.secondary_output_slice and a meta with several codebooks (the kernels read codebooks[0])
+    p.call_kernel("pool_f32", [(0, 64)], (512, 64), [2, 2, 0, 1, 1, 1, 4, 4], secondary_output=(1024, 128))
+    p.call_kernel("matmul_i4", [(0, 64), (256, 64)], (512, 64), [1, 32, 4],
+                  dict(bit_width=4, scales=[1.0] * 4, zero_points=[], shape=[4, 32], quant_block_size=32,
+                       codebooks=np.zeros((2, 16), np.float32)))
+    assert len(p) == 6
     p.close()
+
+
+def test_entry_points_refuse_null_handles_with_a_message():
+    """No entry point dereferences a NULL handle: each returns a status and leaves a message."""
+    l = fastnn_amd.load_library()
+    assert l.fnn_hip_set_option(None, flib.OPT_TILE_SPLIT, 2) == 1
+    assert b"NULL context" in l.fnn_hip_last_error(None)
+    assert l.fnn_hip_sync(None) == 1
+    assert l.fnn_backend_set_graph_replay(None, 0) == 1
+    assert l.fnn_backend_dispatch(None, None) == 1
+    assert l.fnn_hip_stream(None) is None
 
 
 def test_backend_create_without_gpu_reports_an_error():

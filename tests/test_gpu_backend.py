@@ -548,3 +548,156 @@ def test_backend_kernel_flags_single_f16_activations(be, orc):
             be.set_kernel_flags(flib.FLAG_DEVICE_PTRS)
     finally:
         be.set_kernel_flags(0)
+
+
+def test_two_plans_sharing_an_arena_do_not_trust_stale_constants(be, orc):
+    """Plan A and plan B lay their constants over the same bytes of one backend's arena.  Each dispatch of one
+    overwrites the other's constants (uploads, kernel outputs): the other plan must notice, upload again and
+    run eagerly, and both must keep agreeing with the oracle however they alternate.  Two plans whose byte
+    ranges are disjoint keep their residency (and their graph replays) across each other's dispatches."""
+    rng = np.random.default_rng(77)
+    m, k, n = 4, 256, 128
+    xa, xb = rng.standard_normal((m, k)).astype(np.float32), rng.standard_normal((m, k)).astype(np.float32)
+    wa = fastnn_amd.quantize_weights(flib.DT_I8, _w(rng, n, k))
+    wb = fastnn_amd.quantize_weights(flib.DT_I4, _w(rng, n, k))
+    ba = (rng.standard_normal(n) * 0.1).astype(np.float32)
+    a = Arena()
+    s_x, s_w, s_b, s_o = a.take(xa.nbytes), a.take(wa.words.nbytes), a.take(ba.nbytes), a.take(m * n * 4)
+    # A: weight at s_w, bias at s_b, output at s_o.  B: its (shorter) weight at the same offset, and its output lands
+    # on A's bias.
+    pa = ExecutablePlan(a.top).write_const(s_x[0], xa).write_const(s_w[0], wa.words).write_const(s_b[0], ba)
+    pa.call_kernel("matmul_i8_relu", [s_x, s_w, s_b], s_o, [m, k, n], meta_of(wa))
+    s_wb = (s_w[0], wb.words.nbytes)
+    pb = ExecutablePlan(a.top).write_const(s_x[0], xb).write_const(s_wb[0], wb.words)
+    pb.call_kernel("matmul_i4", [s_x, s_wb], (s_b[0], m * n * 4), [m, k, n], meta_of(wb))
+    want_a = orc.qmatmul(to_oracle(orc, wa), xa, bias=ba, act=flib.ACT_RELU)
+    want_b = orc.qmatmul(to_oracle(orc, wb), xb)
+    be.allocate_arena(a.top + m * n * 4)
+    for which in "aabbabbaab":
+        if which == "a":
+            be.dispatch(pa)
+            assert_close(be.read_arena(*s_o, np.float32).reshape(m, n), want_a, 2e-5, "plan A after " + which)
+        else:
+            be.dispatch(pb)
+            assert_close(be.read_arena(s_b[0], m * n * 4, np.float32).reshape(m, n), want_b, 2e-5, "plan B")
+    # a replay only ever follows a dispatch of the same plan
+    be.dispatch(pa); be.dispatch(pa)
+    assert pa.replayed
+    be.dispatch(pb)
+    assert not pb.replayed
+    be.dispatch(pa)
+    assert not pa.replayed
+    assert_close(be.read_arena(*s_o, np.float32).reshape(m, n), want_a, 2e-5, "plan A at the end")
+    # disjoint plans: residency and replays survive the other plan's dispatches
+    a2 = Arena()
+    t_x, t_w, t_o = a2.take(xa.nbytes), a2.take(wa.words.nbytes), a2.take(m * n * 4)
+    u_x, u_w, u_o = a2.take(xb.nbytes), a2.take(wb.words.nbytes), a2.take(m * n * 4)
+    pc = ExecutablePlan(a2.top).write_const(t_x[0], xa).write_const(t_w[0], wa.words)
+    pc.call_kernel("matmul_i8", [t_x, t_w], t_o, [m, k, n], meta_of(wa))
+    pd = ExecutablePlan(a2.top).write_const(u_x[0], xb).write_const(u_w[0], wb.words)
+    pd.call_kernel("matmul_i4", [u_x, u_w], u_o, [m, k, n], meta_of(wb))
+    be.allocate_arena(a2.top)
+    want_c = orc.qmatmul(to_oracle(orc, wa), xa)
+    for it in range(4):
+        be.dispatch(pc); be.dispatch(pd)
+        assert pc.replayed == (it >= 1) and pd.replayed == (it >= 1), it
+        assert_close(be.read_arena(*t_o, np.float32).reshape(m, n), want_c, 2e-5, "disjoint plan C")
+        assert_close(be.read_arena(*u_o, np.float32).reshape(m, n), want_b, 2e-5, "disjoint plan D")
+
+
+def test_many_forwards_keep_the_plan_resident(be, orc):
+    """The write log holds one entry per distinct byte range: a thousand write-input / dispatch cycles neither
+    overflow it nor end the plan's residency (every dispatch after the first is a graph replay)."""
+    rng = np.random.default_rng(78)
+    m, k, n = 2, 128, 64
+    pw = fastnn_amd.quantize_weights(flib.DT_I8, _w(rng, n, k))
+    a = Arena()
+    s_x, s_w, s_o = a.take(m * k * 4), a.take(pw.words.nbytes), a.take(m * n * 4)
+    plan = ExecutablePlan(a.top).write_const(s_w[0], pw.words).call_kernel("matmul_i8", [s_x, s_w], s_o, [m, k, n], meta_of(pw))
+    be.allocate_arena(a.top)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    replays = 0
+    for it in range(1000):
+        be.write_arena(s_x[0], x)
+        be.dispatch(plan)
+        replays += plan.replayed
+    assert replays == 999
+    assert_close(be.read_arena(*s_o, np.float32).reshape(m, n), orc.qmatmul(to_oracle(orc, pw), x), 2e-5, "after 1000 forwards")
+
+
+def test_maxpool_secondary_output_holds_the_window_positions(be, orc):
+    """CallKernel.secondary_output_slice of "pool_f32" (is_max = 1): i64 kh*kernel + kw of each maximum, bit-identical to
+    the oracle, eager and replayed; an index slice shorter than the output takes the leading entries only."""
+    rng = np.random.default_rng(79)
+    n, c, h, w = 2, 5, 9, 7
+    x = rng.permutation(n * c * h * w).astype(np.float32).reshape(n, c, h, w)
+    x[0, 0, :3, :3] = 1000.0                                   # ties: the first tap in (kh, kw) order stays
+    for (k, s, p) in [(5, 1, 2), (2, 2, 0), (3, 2, 1)]:
+        want_v, want_i = orc.maxpool2d(x, k, s, p, return_indices=True)
+        a = Arena()
+        s_x, s_v, s_i = a.take(x.nbytes), a.take(want_v.nbytes), a.take(want_i.nbytes)
+        s_short = a.take(8 * 10)
+        plan = ExecutablePlan(a.top).write_const(s_x[0], x)
+        plan.call_kernel("pool_f32", [s_x], s_v, [k, s, p, 1, n, c, h, w], secondary_output=s_i)
+        plan.call_kernel("pool_f32", [s_x], s_v, [k, s, p, 1, n, c, h, w], secondary_output=s_short)
+        be.allocate_arena(a.top)
+        for it in range(2):
+            be.dispatch(plan)
+            assert plan.replayed == (it == 1)
+            assert np.array_equal(be.read_arena(*s_v, np.float32), want_v.reshape(-1)), (k, s, p)
+            assert np.array_equal(be.read_arena(*s_i, np.int64), want_i.reshape(-1)), (k, s, p)
+            assert np.array_equal(be.read_arena(*s_short, np.int64), want_i.reshape(-1)[:10]), (k, s, p)
+    with pytest.raises(flib.FnnError):
+        be.dispatch(ExecutablePlan(a.top).call_kernel("pool_f32", [s_x], s_v, [k, s, p, 1, n, c, h, w], secondary_output=(s_i[0] + 4, 64)))
+
+
+def test_meta_with_several_codebooks_reads_the_first(be, orc):
+    """QuantizedWeightMeta.codebooks is a vector; every decode of the reference reads entry 0."""
+    rng = np.random.default_rng(80)
+    m, k, n = 3, 128, 48
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    pw = fastnn_amd.quantize_weights(flib.DT_I4CB, _w(rng, n, k))
+    meta = meta_of(pw)
+    meta["codebooks"] = np.concatenate([meta["codebooks"], rng.standard_normal((3, 16)).astype(np.float32)])
+    a = Arena()
+    s_x, s_w, s_o = a.take(x.nbytes), a.take(pw.words.nbytes), a.take(m * n * 4)
+    plan = ExecutablePlan(a.top).write_const(s_x[0], x).write_const(s_w[0], pw.words)
+    plan.call_kernel("matmul_i4", [s_x, s_w], s_o, [m, k, n], meta)
+    be.allocate_arena(a.top)
+    be.dispatch(plan)
+    assert_close(be.read_arena(*s_o, np.float32).reshape(m, n), orc.qmatmul(to_oracle(orc, pw), x), 2e-5, "codebooks[0]")
+
+
+def test_graph_replay_switch_and_context_options(be, orc):
+    """fnn_backend_set_graph_replay(0) keeps every dispatch instruction by instruction; per-context options select
+    kernel variants without changing results beyond the stated tolerance, and refuse values out of range."""
+    rng = np.random.default_rng(81)
+    m, k, n = 64, 512, 256
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    pw = fastnn_amd.quantize_weights(flib.DT_I4, _w(rng, n, k))
+    a = Arena()
+    s_x, s_w, s_o = a.take(x.nbytes), a.take(pw.words.nbytes), a.take(m * n * 4)
+    plan = ExecutablePlan(a.top).write_const(s_x[0], x).write_const(s_w[0], pw.words)
+    plan.call_kernel("matmul_i4", [s_x, s_w], s_o, [m, k, n], meta_of(pw))
+    want = orc.qmatmul(to_oracle(orc, pw), x)
+    be.allocate_arena(a.top)
+    try:
+        be.set_graph_replay(False)
+        for _ in range(3):
+            be.dispatch(plan)
+            assert not plan.replayed
+        be.set_graph_replay(True)
+        be.dispatch(plan)
+        assert plan.replayed
+        for opt, val in [(flib.OPT_TILE_SHAPE, 0), (flib.OPT_TILE_SHAPE, 2), (flib.OPT_TILE_SPLIT, 2), (flib.OPT_TILE_SPLIT, 0)]:
+            be.set_option(opt, val)
+            be.dispatch(plan)                              # the graph is captured again with the new choice
+            assert_close(be.read_arena(*s_o, np.float32).reshape(m, n), want, 2e-5, f"option {opt}={val}")
+        with pytest.raises(flib.FnnError):
+            be.set_option(flib.OPT_TILE_SHAPE, 7)
+        with pytest.raises(flib.FnnError):
+            be.set_option(99, 0)
+    finally:
+        be.set_graph_replay(True)
+        be.set_option(flib.OPT_TILE_SHAPE, -1)
+        be.set_option(flib.OPT_TILE_SPLIT, 0)

@@ -46,6 +46,35 @@ def test_maxpool_is_torch_max_pool2d(orc, k, s, p):
     assert got.shape == want.shape and np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("k,s,p", [(5, 1, 2), (2, 2, 0), (3, 2, 1), (3, 1, 0)])
+def test_maxpool_indices_are_window_positions_of_torchs_argmax(orc, k, s, p):
+    """The secondary output holds kh*kernel + kw of the maximum inside its window.  torch returns the flat position
+    in the input plane instead: converted here (distinct random values, so the argmax is unique)."""
+    rng = np.random.default_rng(4)
+    x = rng.permutation(2 * 3 * 11 * 9).astype(np.float32).reshape(2, 3, 11, 9)
+    want_v, flat = F.max_pool2d(torch.from_numpy(x), k, s, p, return_indices=True)
+    got_v, got_i = orc.maxpool2d(x, k, s, p, return_indices=True)
+    assert np.array_equal(got_v, want_v.numpy())
+    flat = flat.numpy()
+    hh = np.arange(flat.shape[2]).reshape(1, 1, -1, 1)
+    ww = np.arange(flat.shape[3]).reshape(1, 1, 1, -1)
+    kh = flat // 9 - (hh * s - p)
+    kw = flat % 9 - (ww * s - p)
+    assert got_i.dtype == np.int64 and np.array_equal(got_i, kh * k + kw)
+
+
+def test_maxpool_indices_on_ties_and_empty_windows(orc):
+    """Strict `>`: among equal values the first tap in (kh, kw) order stays; a window that sees only padding
+    reports position 0."""
+    x = np.zeros((1, 1, 4, 4), np.float32)
+    x[0, 0, 1, 1] = x[0, 0, 1, 2] = x[0, 0, 2, 1] = 5.0
+    v, i = orc.maxpool2d(x, 3, 1, 0, return_indices=True)        # 2x2 windows over the 4x4 plane
+    assert np.array_equal(v, np.full((1, 1, 2, 2), 5.0, np.float32))
+    assert i[0, 0].tolist() == [[1 * 3 + 1, 1 * 3 + 0], [0 * 3 + 1, 0 * 3 + 0]]
+    v, i = orc.maxpool2d(np.ones((1, 1, 2, 2), np.float32), 1, 1, 1, return_indices=True)
+    assert np.isneginf(v[0, 0, 0, 0]) and i[0, 0, 0, 0] == 0 and i[0, 0, 1, 1] == 0
+
+
 def test_maxpool_window_in_the_padding_only_is_minus_inf(orc):
     x = np.ones((1, 1, 2, 2), np.float32)
     got = orc.maxpool2d(x, 1, 1, 1)                 # 4x4 output, the border windows see padding only
