@@ -52,11 +52,38 @@ struct fnn_hip_ctx {
     float *scratch = nullptr;  // small reduction scratch (partials)
     bool capturing = false;
     uint64_t ws_epoch = 0;     // bumped whenever a staging buffer is re-allocated (captured graphs go stale)
+    unsigned char *static_ws = nullptr;   // this device's copy of the library's static workspace
+    bool static_mode = false;             // inside fnn_hip_qmatmul_static: workspaces come from static_ws, nothing allocates
 };
+
+// Workspace of fnn_hip_qmatmul_static, part of the library's device image: every GPU the library runs on holds one
+// copy (32 MiB) until the process ends.  Region 0: prepared activation operands + row tables; region 1: split-K
+// partial tiles.  Host code never passes the array's name to a kernel: the device address of each GPU's copy is
+// looked up once per device (static_workspace_of) and kept.
+constexpr size_t kStaticOperandBytes = 8u << 20;
+constexpr size_t kStaticPartialBytes = 24u << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticOperandBytes + kStaticPartialBytes];
 
 namespace {
 
 thread_local char g_err[1024] = {0};  // failures without a context
+
+// device address of `scratch` on the current device; looked up on the first context of each device
+hipError_t static_workspace_of(int device, unsigned char **out)
+{
+    static std::mutex mu;
+    static unsigned char *ptrs[64] = {nullptr};
+    std::lock_guard<std::mutex> lock(mu);
+    unsigned char *&slot = ptrs[device & 63];
+    if (!slot) {
+        void *p = nullptr;
+        hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        slot = static_cast<unsigned char *>(p);
+    }
+    *out = slot;
+    return hipSuccess;
+}
 
 int fail(fnn_hip_ctx *ctx, int code, const char *fmt, ...) noexcept
 {
@@ -109,6 +136,7 @@ int ensure(fnn_hip_ctx *ctx, Staging &s, size_t bytes)
 {
     if (bytes <= s.cap && s.ptr) return FNN_OK;
     if (ctx->capturing) return fail(ctx, FNN_ERR_MEMORY, "staging growth during graph capture");
+    if (ctx->static_mode) return fail(ctx, FNN_ERR_MEMORY, "fnn_hip_qmatmul_static: this call would allocate %zu bytes of staging", bytes);
     if (s.ptr) {
         HIP_TRY(ctx, FNN_ERR_MEMORY, hipStreamSynchronize(ctx->stream));
         HIP_TRY(ctx, FNN_ERR_MEMORY, hipFree(s.ptr));
@@ -192,7 +220,8 @@ int fnn_hip_create(int device, fnn_hip_ctx **out)
         if ((e = hipSetDevice(device)) != hipSuccess ||
             (e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking)) != hipSuccess ||
             (e = hipEventCreate(&ctx->ev0)) != hipSuccess || (e = hipEventCreate(&ctx->ev1)) != hipSuccess ||
-            (e = hipMalloc((void **)&ctx->scratch, 64 * 1024)) != hipSuccess) {
+            (e = hipMalloc((void **)&ctx->scratch, 64 * 1024)) != hipSuccess ||
+        (e = static_workspace_of(device, &ctx->static_ws)) != hipSuccess) {
             int rc = fail(nullptr, FNN_ERR_MEMORY, "fnn_hip_create: %s", hipGetErrorString(e));
             fnn_hip_destroy(ctx);
             return rc;
@@ -535,6 +564,25 @@ int fnn_hip_qmatmul(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *a, i
         }
         return FNN_OK;
     });
+}
+
+int fnn_hip_qmatmul_static(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *a_dev, int64_t m,
+                           const float *bias_dev, int act, float *out_dev, int flags)
+{
+    if (!ctx || !w) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_qmatmul_static: NULL context or weight");
+    if (m > FNN_STATIC_MAX_M)
+        return fail(ctx, FNN_ERR_MEMORY, "fnn_hip_qmatmul_static: M = %lld exceeds the limit of %d rows: use fnn_hip_qmatmul",
+                    (long long)m, FNN_STATIC_MAX_M);
+    if (flags & ~(FNN_FLAG_DEVICE_PTRS | FNN_FLAG_ACT_F16_SINGLE | FNN_FLAG_FORCE_GENERIC | FNN_FLAG_PREFER_FMA))
+        return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_qmatmul_static: flag not available here");
+    // device pointers only (host pointers would need staging buffers); workspaces come from the static array for the
+    // duration of the call, and everything that would allocate fails instead
+    struct Mode {
+        fnn_hip_ctx *c;
+        explicit Mode(fnn_hip_ctx *c_) : c(c_) { c->static_mode = true; }
+        ~Mode() { c->static_mode = false; }
+    } mode(ctx);
+    return fnn_hip_qmatmul(ctx, w, a_dev, m, bias_dev, act, out_dev, flags | FNN_FLAG_DEVICE_PTRS);
 }
 
 int fnn_hip_quantize_activations(fnn_hip_ctx *ctx, const float *x, int64_t numel, float scale,
@@ -994,6 +1042,17 @@ int fnn_hip_graph_destroy(fnn_hip_ctx *ctx, fnn_hip_graph *g)
 // staging access for the matrix-core translation units
 int fnn_ctx_ensure_tmp(fnn_hip_ctx *ctx, int which, size_t bytes, void **ptr)
 {
+    if (ctx->static_mode) {
+        // fnn_hip_qmatmul_static: fixed regions of the static workspace, nothing grows
+        const size_t off = which == 0 ? 0 : kStaticOperandBytes;
+        const size_t cap = which == 0 ? kStaticOperandBytes : (which == 1 ? kStaticPartialBytes : 0);
+        if (bytes > cap)
+            return fail(ctx, FNN_ERR_MEMORY,
+                        "fnn_hip_qmatmul_static: this shape needs %zu bytes of %s workspace, the static buffer holds %zu: use fnn_hip_qmatmul",
+                        bytes, which == 0 ? "operand" : (which == 1 ? "split-K" : "weight expansion"), cap);
+        *ptr = ctx->static_ws + off;
+        return FNN_OK;
+    }
     Staging &s = which == 0 ? ctx->st_tmp : (which == 1 ? ctx->st_tmp2 : ctx->st_tmp3);
     int rc = ensure(ctx, s, bytes);
     if (rc) return rc;
@@ -1002,6 +1061,8 @@ int fnn_ctx_ensure_tmp(fnn_hip_ctx *ctx, int which, size_t bytes, void **ptr)
 }
 
 bool fnn_ctx_capturing(fnn_hip_ctx *ctx) { return ctx->capturing; }
+
+bool fnn_ctx_no_alloc(fnn_hip_ctx *ctx) { return ctx->capturing || ctx->static_mode; }
 
 int fnn_ctx_fail(fnn_hip_ctx *ctx, int code, const char *msg) { return fail(ctx, code, "%s", msg); }
 

@@ -9,6 +9,8 @@
 int fnn_ctx_ensure_tmp(fnn_hip_ctx *ctx, int which, size_t bytes, void **ptr);
 int fnn_ctx_fail(fnn_hip_ctx *ctx, int code, const char *msg);
 bool fnn_ctx_capturing(fnn_hip_ctx *ctx);
+// true while device memory must not be allocated: graph capture, or a call through fnn_hip_qmatmul_static
+bool fnn_ctx_no_alloc(fnn_hip_ctx *ctx);
 // value of a per-context option (FNN_OPT_*, set through fnn_hip_set_option)
 int64_t fnn_ctx_option(const fnn_hip_ctx *ctx, int option);
 

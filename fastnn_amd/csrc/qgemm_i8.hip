@@ -400,7 +400,7 @@ int fnn_aligned_rows(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, c
     if (w->kp % 4 == 0) { *words = w->words; *kp = w->kp; return FNN_OK; }
     fnn_hip_weight *wm = const_cast<fnn_hip_weight *>(w);
     if (!wm->words4) {
-        if (fnn_ctx_capturing(ctx)) return fnn_ctx_fail(ctx, FNN_ERR_MEMORY, "first use of re-strided weight rows during graph capture");
+        if (fnn_ctx_no_alloc(ctx)) return fnn_ctx_fail(ctx, FNN_ERR_MEMORY, "first use of re-strided weight rows while allocation is not allowed (graph capture, fnn_hip_qmatmul_static)");
         const int64_t kp4 = (w->kp + 3) / 4 * 4;
         if (hipMalloc((void **)&wm->words4, (size_t)(w->rows * kp4 + 16) * 4) != hipSuccess)
             return fnn_ctx_fail(ctx, FNN_ERR_MEMORY, "out of device memory (re-strided weight rows)");
@@ -454,7 +454,7 @@ int fnn_i8_tiled_matmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w
     if ((rc = fnn_ctx_ensure_tmp(ctx, 1, (size_t)p.m * p.n * 4 + 256, &ws1))) return rc;
     fnn_hip_weight *wm = const_cast<fnn_hip_weight *>(w);
     if (!wm->row_qsum) {
-        if (fnn_ctx_capturing(ctx)) return fnn_ctx_fail(ctx, FNN_ERR_MEMORY, "first use of re-strided weight rows during graph capture");
+        if (fnn_ctx_no_alloc(ctx)) return fnn_ctx_fail(ctx, FNN_ERR_MEMORY, "first use of re-strided weight rows while allocation is not allowed (graph capture, fnn_hip_qmatmul_static)");
         if (hipMalloc((void **)&wm->row_qsum, (size_t)w->rows * 4 + 64) != hipSuccess)
             return fnn_ctx_fail(ctx, FNN_ERR_MEMORY, "out of device memory (row sums)");
         hipError_t e = launch_row_qsum(w, wm->row_qsum, s);

@@ -333,7 +333,7 @@ int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QM
     fnn_hip_weight *wm = const_cast<fnn_hip_weight *>(w);
     const bool want_umean = !precise && !dense && (DT == FNN_DT_I8 || DT == FNN_DT_I4 || DT == FNN_DT_U8 || DT == FNN_DT_U4 || DT == FNN_DT_F4);
     if constexpr (DT != DT_F16_DENSE) if (want_umean && !wm->umean) {
-        if (fnn_ctx_capturing(ctx)) return fnn_ctx_fail(ctx, FNN_ERR_MEMORY, "first single-pass use of a weight during graph capture");
+        if (fnn_ctx_no_alloc(ctx)) return fnn_ctx_fail(ctx, FNN_ERR_MEMORY, "first single-pass use of a weight while allocation is not allowed (graph capture, fnn_hip_qmatmul_static)");
         if (hipMalloc((void **)&wm->umean, (size_t)w->rows * 4 + 64) != hipSuccess)
             return fnn_ctx_fail(ctx, FNN_ERR_MEMORY, "out of device memory (row means)");
         hipError_t e = launch_umean<DT>(w, wm->umean, s);
@@ -460,7 +460,7 @@ int run_tiled_codebook(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w,
     bool expand = true;
     if (ws) {
         expand = false;
-    } else if (keep && q.words == w->words && !fnn_ctx_capturing(ctx)) {
+    } else if (keep && q.words == w->words && !fnn_ctx_no_alloc(ctx)) {
         if (hipMalloc(&wm->dense16, total) != hipSuccess)
             return fnn_ctx_fail(ctx, FNN_ERR_MEMORY, "out of device memory (expanded codebook weight)");
         ws = wm->dense16;
@@ -491,7 +491,7 @@ int fnn_row_means(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, cons
     if (dt != FNN_DT_I8 && dt != FNN_DT_I4 && dt != FNN_DT_U8 && dt != FNN_DT_U4 && dt != FNN_DT_F4) return FNN_OK;
     fnn_hip_weight *wm = const_cast<fnn_hip_weight *>(w);
     if (!wm->umean) {
-        if (fnn_ctx_capturing(ctx)) return fnn_ctx_fail(ctx, FNN_ERR_MEMORY, "first single-pass use of a weight during graph capture");
+        if (fnn_ctx_no_alloc(ctx)) return fnn_ctx_fail(ctx, FNN_ERR_MEMORY, "first single-pass use of a weight while allocation is not allowed (graph capture, fnn_hip_qmatmul_static)");
         if (hipMalloc((void **)&wm->umean, (size_t)w->rows * 4 + 64) != hipSuccess)
             return fnn_ctx_fail(ctx, FNN_ERR_MEMORY, "out of device memory (row means)");
         hipError_t e;

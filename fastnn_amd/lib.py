@@ -38,7 +38,7 @@ EXPORTED_SYMBOLS = [
     "fnn_hip_device_count", "fnn_hip_create", "fnn_hip_destroy", "fnn_hip_last_error", "fnn_hip_sync", "fnn_hip_set_option", "fnn_hip_get_option", "fnn_hip_stream",
     "fnn_hip_malloc", "fnn_hip_free", "fnn_hip_upload", "fnn_hip_download",
     "fnn_hip_weight_register", "fnn_hip_weight_lookup", "fnn_hip_weight_release", "fnn_hip_dequant",
-    "fnn_hip_qmatmul", "fnn_hip_quantize_activations", "fnn_hip_dequantize_activations", "fnn_hip_qmatmul_i8act", "fnn_hip_qconv2d", "fnn_hip_qconv2d_i8act",
+    "fnn_hip_qmatmul", "fnn_hip_qmatmul_static", "fnn_hip_quantize_activations", "fnn_hip_dequantize_activations", "fnn_hip_qmatmul_i8act", "fnn_hip_qconv2d", "fnn_hip_qconv2d_i8act",
     "fnn_hip_timer_start", "fnn_hip_timer_stop",
     "fnn_hip_graph_begin", "fnn_hip_graph_end", "fnn_hip_graph_launch", "fnn_hip_graph_destroy",
     "fnn_hip_workspace_epoch",
@@ -127,6 +127,7 @@ def _prototype(l):
     l.fnn_hip_weight_release.argtypes = [_vp, _vp]
     l.fnn_hip_dequant.argtypes = [_vp, _vp, _vp, C.c_int]
     l.fnn_hip_qmatmul.argtypes = [_vp, _vp, _vp, _i64, _vp, C.c_int, _vp, C.c_int]
+    l.fnn_hip_qmatmul_static.argtypes = [_vp, _vp, _vp, _i64, _vp, C.c_int, _vp, C.c_int]
     l.fnn_hip_quantize_activations.argtypes = [_vp, _vp, _i64, C.c_float, C.c_float, _vp, C.c_int]
     l.fnn_hip_qmatmul_i8act.argtypes = [_vp, _vp, _vp, _i64, _vp, _vp, C.c_int]
     l.fnn_hip_qconv2d.argtypes = [_vp, _vp, _vp, _i64, _i64, _i64, _i64, C.c_int, C.c_int, C.c_int, C.c_int,
@@ -364,6 +365,12 @@ class HipContext:
         """Device-pointer call: only enqueues on the context's stream."""
         self._check(self.lib.fnn_hip_qmatmul(self.handle, wh, _vp(a_ptr), m, _vp(bias_ptr) if bias_ptr else None, act,
                                              _vp(out_ptr), flags | FLAG_DEVICE_PTRS))
+
+    def qmatmul_static(self, wh, a_ptr: int, m: int, out_ptr: int, bias_ptr: int = 0, act: int = ACT_NONE,
+                       flags: int = 0):
+        """fnn_hip_qmatmul_static: the device-pointer MatMul that allocates nothing (static workspace)."""
+        self._check(self.lib.fnn_hip_qmatmul_static(self.handle, wh, _vp(a_ptr), m, _vp(bias_ptr) if bias_ptr else None,
+                                                    act, _vp(out_ptr), flags))
 
     def quantize_activations(self, x: np.ndarray, scale: float = 0.0, zp: float = 0.0) -> np.ndarray:
         x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1)

@@ -134,6 +134,25 @@ int fnn_hip_dequant(fnn_hip_ctx *ctx, const fnn_hip_weight *w, float *out, int f
 int fnn_hip_qmatmul(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *a, int64_t m,
                     const float *bias, int act, float *out, int flags);
 
+/* fnn_hip_qmatmul for callers that cannot allocate device memory: code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc.  No counterpart in fastnn.  Same kernels and the same result as
+ * fnn_hip_qmatmul with FNN_FLAG_DEVICE_PTRS (a, bias, out are device pointers; the call only enqueues work on the
+ * context's stream), but the workspaces of the M >= 17 path (prepared activation operands, split-K partial tiles)
+ * come from a 32 MiB array inside the library's device image instead of hipMalloc, and the call makes no
+ * allocation of any kind.  Limits, refused with FNN_ERR_MEMORY and a message that names them:
+ *   - M <= FNN_STATIC_MAX_M;
+ *   - operand workspace 2*ceil16(M)*ceil64(K)*2 + 12*M bytes <= 8 MiB (M = 256 at K = 4096 uses 4 MiB; half of
+ *     that with FNN_FLAG_ACT_F16_SINGLE), split-K partials splits*M*N*4 bytes <= 24 MiB;
+ *   - per-weight side tables that fnn_hip_qmatmul builds on first use (the f16 expansion of a codebook weight at
+ *     M >= 5, row means for FNN_FLAG_ACT_F16_SINGLE, re-strided rows when ceil(K/ITEMS) % 4 != 0) must exist
+ *     already: call fnn_hip_qmatmul once per weight and flag combination beforehand.
+ * Every GPU the library runs on holds its copy of the array until the process ends, and every call on a GPU, from
+ * any context, uses that one copy: calls that overlap in time on one GPU (two contexts, two threads) race; calls
+ * on one context are ordered by its stream.  Nothing in the array needs to start at zero. */
+#define FNN_STATIC_MAX_M 4096
+int fnn_hip_qmatmul_static(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *a_dev, int64_t m,
+                           const float *bias_dev, int act, float *out_dev, int flags);
+
 /* ---- I8 activations: kernel "quantize_activations"
  * (src/backend/cpu/mod.rs:6928-7008): payload = [scale f32][zp f32][numel x i8].
  * scale <= 0 selects the dynamic mode (scale = max|x|/127, zp = 0). */
