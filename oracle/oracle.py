@@ -23,13 +23,42 @@ DT_NAMES = {I8: "i8", I4: "i4", U8: "u8", U4: "u4", F8: "f8", F8R: "f8r", F4: "f
 MARGIN = 16
 
 
+_BASE_SO = os.path.join(_HERE, "libfnn_cpu_baseline.so")
+
+
 def build(force: bool = False) -> str:
-    """Compile the oracle with gcc (strict IEEE flags live in the Makefile)."""
-    src = os.path.join(_HERE, "fnn_oracle.c")
-    if force or not os.path.exists(_SO) or os.path.getmtime(_SO) < os.path.getmtime(src):
-        subprocess.run(["make", "-C", _HERE, "-B", "libfnn_oracle.so"], check=True,
-                       stdout=subprocess.DEVNULL)
+    """Compile the oracle and the tuned CPU baseline with gcc (flags live in the Makefile)."""
+    for so, src in ((_SO, "fnn_oracle.c"), (_BASE_SO, "fnn_cpu_baseline.c")):
+        if force or not os.path.exists(so) or os.path.getmtime(so) < os.path.getmtime(os.path.join(_HERE, src)):
+            subprocess.run(["make", "-C", _HERE, "-B", os.path.basename(so)], check=True, stdout=subprocess.DEVNULL)
     return _SO
+
+
+_base_lib = None
+
+
+def cpu_qgemm(p: "Packed", a, bias=None, act: int = 0, threads: int = 1) -> np.ndarray:
+    """The tuned CPU baseline (fnn_cpu_baseline.c): AVX2 unpack + FMA dots, weight rows over `threads` threads.
+    I8 and I4 per-channel weights only; raises for other types or on a CPU without AVX2/FMA."""
+    global _base_lib
+    if _base_lib is None:
+        if not os.path.exists(_BASE_SO):
+            build()
+        _base_lib = C.CDLL(_BASE_SO)
+        _base_lib.fnn_cpu_qgemm.argtypes = [C.c_int, C.c_void_p, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p,
+                                            C.c_int64, C.c_void_p, C.c_int, C.c_void_p, C.c_int]
+    a = _f32(a)
+    m, k = a.shape
+    assert k == p.inner
+    out = np.zeros((m, p.rows), np.float32)
+    b = None if bias is None else _f32(bias)
+    zeros = p.zeros if p.zeros.size == p.rows else None
+    rc = _base_lib.fnn_cpu_qgemm(p.dt, p.words.ctypes.data_as(C.c_void_p), p.rows, k, p.scales.ctypes.data_as(C.c_void_p),
+                                 None if zeros is None else zeros.ctypes.data_as(C.c_void_p), a.ctypes.data_as(C.c_void_p), m,
+                                 None if b is None else b.ctypes.data_as(C.c_void_p), act, out.ctypes.data_as(C.c_void_p), threads)
+    if rc:
+        raise ValueError(f"fnn_cpu_qgemm rc={rc}")
+    return out
 
 
 _lib = None

@@ -164,3 +164,24 @@ def test_quantize_activations_formula(orc):
     assert s == np.float32(1.0) and pl[4:8].view(np.float32)[0] == 0.0
     assert list(pl[8:].view(np.int8)) == [0, 1, -2, 0, 1, 127, -127, 64]
     assert orc.quantize_activations(np.zeros(4, np.float32))[:4].view(np.float32)[0] == 1.0
+
+
+@pytest.mark.parametrize("dt", [0, 1])
+@pytest.mark.parametrize("m,threads", [(1, 1), (1, 4), (5, 3)])
+def test_tuned_cpu_baseline_agrees_with_the_restatement(orc, dt, m, threads):
+    """bench.py's cpu_baseline (AVX2 unpack + FMA dots, weight rows over threads) computes the same MatMul as the
+    oracle's restatement; its summation order differs, so the comparison is at 1e-5 of max|out| (f64-accumulated
+    reference), with ragged K and N and every epilogue."""
+    import fastnn_amd
+    rng = np.random.default_rng(50 + dt)
+    n, k = 203, 1000 if dt == 0 else 1000 // 8 * 8 + 8
+    pw = fastnn_amd.quantize_weights(dt, (rng.standard_normal((n, k)) * 0.05).astype(np.float32))
+    po = orc.Packed(pw.dtype, pw.rows, pw.inner, pw.words, pw.scales, pw.zeros, pw.qblock, pw.codebook)
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    bias = (rng.standard_normal(n) * 0.1).astype(np.float32)
+    for act in range(4):
+        want = orc.qmatmul(po, a, order=2, bias=bias, act=act)
+        got = orc.cpu_qgemm(po, a, bias=bias, act=act, threads=threads)
+        assert np.abs(got - want).max() <= 1e-5 * np.abs(want).max(), (dt, act)
+    with pytest.raises(ValueError):
+        orc.cpu_qgemm(orc.Packed(4, pw.rows, pw.inner, pw.words, pw.scales, pw.zeros), a)
