@@ -15,7 +15,9 @@ from typing import Optional, Sequence
 import numpy as np
 
 from . import lib as _l
-from .lib import FnnError, Slice, WeightMeta
+import json
+
+from .lib import DimExpr, FnnError, Slice, WeightMeta
 
 BITS_OF = {_l.DT_I8: 8, _l.DT_I4: 4, _l.DT_U8: 8, _l.DT_U4: 4, _l.DT_F8: 8, _l.DT_F8R: 8, _l.DT_F4: 4, _l.DT_I4CB: 4}
 KERNEL_OF = {_l.DT_I8: "matmul_i8", _l.DT_I4: "matmul_i4", _l.DT_U8: "matmul_u8", _l.DT_U4: "matmul_u4",
@@ -34,14 +36,60 @@ def meta_of(pw: "_l.PackedWeight", shape: Optional[Sequence[int]] = None):
 class ExecutablePlan:
     """ExecutablePlan {instructions, arena_size} (src/backend/mod.rs:109-131)."""
 
-    def __init__(self, arena_size: int):
+    def __init__(self, arena_size: int, _handle=None):
         self.lib = _l.load_library()
-        h = C.c_void_p()
-        rc = self.lib.fnn_plan_create(arena_size, C.byref(h))
-        if rc:
-            raise FnnError(rc, "fnn_plan_create failed")
-        self.handle = h
+        if _handle is None:
+            h = C.c_void_p()
+            rc = self.lib.fnn_plan_create(arena_size, C.byref(h))
+            if rc:
+                raise FnnError(rc, "fnn_plan_create failed")
+            _handle = h
+        self.handle = _handle
         self.arena_size = arena_size
+
+    @classmethod
+    def load(cls, path_or_bytes) -> "ExecutablePlan":
+        """ExecutablePlan::load (src/backend/mod.rs:124-130): a plan saved by fastnn with bincode."""
+        data = path_or_bytes if isinstance(path_or_bytes, (bytes, bytearray)) else open(path_or_bytes, "rb").read()
+        lib = _l.load_library()
+        h = C.c_void_p()
+        buf = (C.c_uint8 * max(len(data), 1)).from_buffer_copy(bytes(data) if data else b"\0")
+        rc = lib.fnn_plan_from_bincode(buf, len(data), C.byref(h))
+        if rc:
+            msg = lib.fnn_backend_last_error(None)
+            raise FnnError(rc, msg.decode() if msg else "fnn_plan_from_bincode failed")
+        return cls(int(lib.fnn_plan_arena_size(h)), _handle=h)
+
+    def to_bytes(self) -> bytes:
+        """ExecutablePlan::save (src/backend/mod.rs:117-122) into memory."""
+        need = C.c_uint64()
+        self._ok(self.lib.fnn_plan_to_bincode(self.handle, None, 0, C.byref(need)), "save")
+        buf = (C.c_uint8 * max(need.value, 1))()
+        self._ok(self.lib.fnn_plan_to_bincode(self.handle, buf, need.value, C.byref(need)), "save")
+        return bytes(buf[: need.value])
+
+    def save(self, path: str):
+        with open(path, "wb") as f:
+            f.write(self.to_bytes())
+
+    def describe(self, index: int) -> dict:
+        """One instruction as a dict (fnn_plan_describe)."""
+        buf = C.create_string_buffer(1 << 16)
+        self._ok(self.lib.fnn_plan_describe(self.handle, index, buf, len(buf)), "describe")
+        return json.loads(buf.value.decode())
+
+    def set_param_dims(self, index: int, dims) -> "ExecutablePlan":
+        """CallKernel.param_dims of instruction `index`: ints (Known), str (Symbol) or (str, max) (Bounded)."""
+        arr = (DimExpr * max(len(dims), 1))()
+        for i, d in enumerate(dims):
+            if isinstance(d, str):
+                arr[i] = DimExpr(1, 0, d.encode())
+            elif isinstance(d, tuple):
+                arr[i] = DimExpr(2, int(d[1]), d[0].encode())
+            else:
+                arr[i] = DimExpr(0, int(d), None)
+        self._ok(self.lib.fnn_plan_set_param_dims(self.handle, index, arr, len(dims)), "param_dims")
+        return self
 
     def __len__(self):
         return int(self.lib.fnn_plan_len(self.handle))
@@ -152,8 +200,14 @@ class HipBackend:
         """fnn_hip_set_option on the backend's context (lib.OPT_* constants)."""
         self._check(self.lib.fnn_backend_set_option(self.handle, option, value))
 
-    def dispatch(self, plan: ExecutablePlan):
-        self._check(self.lib.fnn_backend_dispatch(self.handle, plan.handle))
+    def dispatch(self, plan: ExecutablePlan, shape_env: Optional[dict] = None):
+        """Backend::dispatch; shape_env = {symbol: value} is the call's ShapeEnv (empty when omitted)."""
+        if not shape_env:
+            self._check(self.lib.fnn_backend_dispatch(self.handle, plan.handle))
+            return
+        names = (C.c_char_p * len(shape_env))(*[k.encode() for k in shape_env])
+        values = (C.c_uint64 * len(shape_env))(*[int(v) for v in shape_env.values()])
+        self._check(self.lib.fnn_backend_dispatch_env(self.handle, plan.handle, names, values, len(shape_env)))
 
     def dispatch_profile(self, plan: ExecutablePlan):
         n = len(plan)

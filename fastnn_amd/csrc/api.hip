@@ -123,6 +123,8 @@ const OptionSpec kOptions[FNN_OPT_COUNT] = {
     {0, 0, 32},       // FNN_OPT_TILE_SPLIT
     {0, 0, 6},        // FNN_OPT_TILE_STAGES
     {5, 1, 1 << 20},  // FNN_OPT_TILE_MIN_M
+    {0, 0, 1},        // FNN_OPT_GEMV_INT8
+    {0, 0, 65535},    // FNN_OPT_GEMV_GRID
 };
 
 #define HIP_TRY(ctx, code, expr)                                                              \
@@ -542,6 +544,10 @@ int fnn_hip_qmatmul(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *a, i
         if (!(flags & FNN_FLAG_FORCE_GENERIC)) {
             const bool fma_first = (flags & FNN_FLAG_PREFER_FMA) || w->dtype == FNN_DT_I4CB;
             if (fma_first) HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qgemv(w->dtype, p, ctx->stream, &handled));
+            if (!handled && !(flags & FNN_FLAG_ACT_F16_SINGLE)) {
+                int rc = fnn_i8dot_qgemv(ctx, ctx->stream, w, p, &handled);
+                if (rc) return rc;
+            }
             if (!handled) {
                 int rc = fnn_mfma_qgemv(ctx, ctx->stream, w, p, flags, &handled);
                 if (rc) return rc;

@@ -45,6 +45,16 @@ struct Instr {
     fnn_slice secondary{0, 0};
     std::vector<fnn_slice> inputs;
     std::vector<uint64_t> params;
+    // CallKernel.param_dims (src/backend/mod.rs:72-78): symbolic forms of `params`, resolved at dispatch time
+    struct Dim {
+        uint32_t kind = 0;      // 0 Known(value), 1 Symbol(sym), 2 Bounded{sym, max: value}
+        uint64_t value = 0;
+        std::string sym;
+    };
+    bool has_param_dims = false;
+    std::vector<Dim> param_dims;
+    bool has_node_id = false;   // CallKernel.node_id: carried through load / save, not used by dispatch
+    uint64_t node_id = 0;
     Meta meta;
     bool clobbered = false;  // WriteConst only: another instruction of the plan writes into dst
 };
@@ -93,6 +103,8 @@ int matmul_dtype(const std::string &base)
 struct fnn_plan {
     uint64_t arena_size = 0;
     std::vector<Instr> instrs;
+    std::vector<uint64_t> levels;     // ExecutablePlan.levels: carried through load / save (dispatch is sequential)
+    std::string graph_env;            // shape environment the captured graph was recorded under
     uint64_t uid = 0;                 // never reused within the process
     uint64_t revision = 0;            // bumped whenever an instruction is added
     bool analysed = false;
@@ -126,6 +138,8 @@ struct fnn_backend {
     bool graph_replay = true;    // resident plans replay as one HIP graph (fnn_backend_set_graph_replay)
     uint64_t weights_epoch = 0;  // bumped whenever a cached device weight is created or released
     int kernel_flags = 0;        // extra FNN_FLAG_* bits for every MatMul / Conv2d call
+    std::vector<std::pair<std::string, uint64_t>> shape_env;   // ShapeEnv of the dispatch in progress
+    std::string shape_env_sig;   // the same as one string: graphs recorded under another environment are stale
     char err[1024] = {0};        // fixed storage: recording a failure never allocates
     std::map<std::pair<uint64_t, uint64_t>, fnn_hip_weight *> weights;  // (offset,size) like get_or_cache_packed
     std::vector<uint8_t> stage;
@@ -250,12 +264,46 @@ int weight_for(fnn_backend *b, const fnn_slice &ws, int dtype, const Meta &meta,
     return FNN_OK;
 }
 
+// resolve_params (src/backend/cpu/params.rs:11-39): with param_dims present the first `expected` parameters are the
+// dims evaluated in the dispatch's shape environment (DimExpr::evaluate_with_env, src/ir/node.rs:511-531), else the
+// stored params as they are.
+int resolve_params(fnn_backend *b, const Instr &in, size_t expected, std::vector<uint64_t> &out)
+{
+    if (!in.has_param_dims) {
+        out = in.params;
+        return FNN_OK;
+    }
+    if (in.param_dims.size() < expected)
+        return fail(b, FNN_ERR_DISPATCH, "resolve_params: param_dims has %zu elements but expected %zu", in.param_dims.size(), expected);
+    out.clear();
+    for (size_t i = 0; i < expected; i++) {
+        const Instr::Dim &d = in.param_dims[i];
+        if (d.kind == 0) { out.push_back(d.value); continue; }
+        const uint64_t *bound = nullptr;
+        for (const auto &kv : b->shape_env)
+            if (kv.first == d.sym) { bound = &kv.second; break; }
+        if (d.kind == 2) {
+            if (bound && *bound > d.value)
+                return fail(b, FNN_ERR_DISPATCH, "resolve_params: DimExpr::Bounded: symbol '%s' resolved to %llu, exceeds bound %llu",
+                            d.sym.c_str(), (unsigned long long)*bound, (unsigned long long)d.value);
+            out.push_back(bound ? *bound : d.value);
+        } else {
+            if (!bound) return fail(b, FNN_ERR_DISPATCH, "resolve_params: DimExpr::Symbol '%s' is not bound in the ShapeEnv", d.sym.c_str());
+            out.push_back(*bound);
+        }
+    }
+    return FNN_OK;
+}
+
 int run_matmul(fnn_backend *b, const Instr &in, const KernelName &kn, int dtype)
 {
     const char *name = in.kernel.c_str();
     if (in.inputs.size() < 2) return FNN_OK;  // the CPU arm ignores a malformed slice list
-    if (in.params.size() < 3) return fail(b, FNN_ERR_DISPATCH, "%s: expected params [M,K,N]", name);
-    uint64_t m = in.params[0], k = in.params[1], n = in.params[2];
+    std::vector<uint64_t> par;
+    int rs = resolve_params(b, in, 3, par);
+    if (rs) return rs;
+    if (par.size() < 3) return fail(b, FNN_ERR_DISPATCH, "%s: expected params [M,K,N]", name);
+    uint64_t m = par[0], k = par[1], n = par[2];
     const fnn_slice &as = in.inputs[0], &ws = in.inputs[1];
     if (as.size < m * k * 4) return fail(b, FNN_ERR_DISPATCH, "%s: activation slice holds %llu bytes, M*K*4 = %llu", name, (unsigned long long)as.size, (unsigned long long)(m * k * 4));
     if (in.dst.size < m * n * 4) return fail(b, FNN_ERR_DISPATCH, "%s: output slice holds %llu bytes, M*N*4 = %llu", name, (unsigned long long)in.dst.size, (unsigned long long)(m * n * 4));
@@ -280,8 +328,11 @@ int run_matmul_i8act(fnn_backend *b, const Instr &in, int dtype)
 {
     const char *name = in.kernel.c_str();
     if (in.inputs.size() != 2) return FNN_OK;
-    if (in.params.size() < 3) return fail(b, FNN_ERR_DISPATCH, "%s: expected params [M,K,N]", name);
-    uint64_t m = in.params[0], k = in.params[1], n = in.params[2];
+    std::vector<uint64_t> par;
+    int rs = resolve_params(b, in, 3, par);
+    if (rs) return rs;
+    if (par.size() < 3) return fail(b, FNN_ERR_DISPATCH, "%s: expected params [M,K,N]", name);
+    uint64_t m = par[0], k = par[1], n = par[2];
     const fnn_slice &as = in.inputs[0], &ws = in.inputs[1];
     if (as.size < 8 + m * k) return fail(b, FNN_ERR_DISPATCH, "%s: activation payload holds %llu bytes, 8+M*K = %llu", name, (unsigned long long)as.size, (unsigned long long)(8 + m * k));
     if (in.dst.size < m * n * 4) return fail(b, FNN_ERR_DISPATCH, "%s: output slice holds %llu bytes, M*N*4 = %llu", name, (unsigned long long)in.dst.size, (unsigned long long)(m * n * 4));
@@ -679,7 +730,7 @@ int dispatch_impl(fnn_backend *b, fnn_plan *p, uint64_t *elapsed_ns, uint64_t n_
     // plan, src/backend/executor.rs:639-667).  Profiling, re-uploaded constants and anything
     // that fails under capture keep the instruction-by-instruction path.
     const bool may_replay = b->graph_replay && !elapsed_ns && resident && !p->uploads_every_run && p->graph_failures < 2;
-    if (p->graph && !(may_replay && p->graph_uid == b->uid && p->graph_generation == b->generation &&
+    if (p->graph && !(may_replay && p->graph_env == b->shape_env_sig && p->graph_uid == b->uid && p->graph_generation == b->generation &&
                       p->graph_weights_epoch == b->weights_epoch && p->graph_ws_epoch == fnn_hip_workspace_epoch(b->ctx) &&
                       p->graph_scratch_epoch == b->scratch_epoch)) {
         fnn_hip_graph_destroy(p->graph_uid == b->uid ? b->ctx : nullptr, p->graph);
@@ -696,6 +747,7 @@ int dispatch_impl(fnn_backend *b, fnn_plan *p, uint64_t *elapsed_ns, uint64_t n_
                 p->graph = g;
                 p->graph_uid = b->uid; p->graph_generation = b->generation;
                 p->graph_weights_epoch = w0; p->graph_ws_epoch = s0; p->graph_scratch_epoch = c0;
+                p->graph_env = b->shape_env_sig;
             } else {
                 if (g) fnn_hip_graph_destroy(b->ctx, g);
                 p->graph_failures++;
@@ -960,7 +1012,7 @@ int fnn_plan_add_call_kernel(fnn_plan *p, const char *kernel_name, const fnn_sli
             if (meta->zero_points) in.meta.zeros.assign(meta->zero_points, meta->zero_points + meta->n_zero_points);
             if (meta->shape) in.meta.shape.assign(meta->shape, meta->shape + meta->n_shape);
             in.meta.qblock = meta->quant_block_size;
-            if (meta->n_codebooks >= 1) in.meta.codebook.assign(meta->codebooks, meta->codebooks + 16);
+            if (meta->n_codebooks >= 1) in.meta.codebook.assign(meta->codebooks, meta->codebooks + 16 * meta->n_codebooks);
         }
         p->instrs.push_back(std::move(in));
         touched(p);
@@ -968,9 +1020,341 @@ int fnn_plan_add_call_kernel(fnn_plan *p, const char *kernel_name, const fnn_sli
     });
 }
 
+int fnn_plan_set_param_dims(fnn_plan *p, uint64_t instruction, const fnn_dim_expr *dims, uint64_t n_dims)
+{
+    return guarded(nullptr, "fnn_plan_set_param_dims", [&]() -> int {
+        if (!p || (!dims && n_dims)) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_plan_set_param_dims: NULL argument");
+        if (instruction >= p->instrs.size() || p->instrs[instruction].kind != K_CALL)
+            return fail(nullptr, FNN_ERR_DISPATCH, "fnn_plan_set_param_dims: instruction %llu is not a CallKernel", (unsigned long long)instruction);
+        std::vector<Instr::Dim> v;
+        for (uint64_t i = 0; i < n_dims; i++) {
+            Instr::Dim d;
+            d.kind = dims[i].kind;
+            d.value = dims[i].value;
+            if (d.kind > 2) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_plan_set_param_dims: unknown DimExpr kind %u", d.kind);
+            if (d.kind != 0) {
+                if (!dims[i].symbol) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_plan_set_param_dims: symbolic dim without a name");
+                d.sym = dims[i].symbol;
+            }
+            v.push_back(std::move(d));
+        }
+        p->instrs[instruction].param_dims = std::move(v);
+        p->instrs[instruction].has_param_dims = true;
+        touched(p);
+        return FNN_OK;
+    });
+}
+
+static int set_shape_env(fnn_backend *b, const char *const *names, const uint64_t *values, uint64_t n)
+{
+    b->shape_env.clear();
+    b->shape_env_sig.clear();
+    for (uint64_t i = 0; i < n; i++) {
+        if (!names[i]) return fail(b, FNN_ERR_DISPATCH, "dispatch: NULL symbol name in the shape environment");
+        for (const auto &kv : b->shape_env)   // ShapeEnv::bind: one value per symbol
+            if (kv.first == names[i] && kv.second != values[i])
+                return fail(b, FNN_ERR_DISPATCH, "ShapeEnv: symbol '%s' bound to %llu then inconsistently to %llu", names[i],
+                            (unsigned long long)kv.second, (unsigned long long)values[i]);
+        b->shape_env.emplace_back(names[i], values[i]);
+        b->shape_env_sig += names[i];
+        b->shape_env_sig += '=';
+        b->shape_env_sig += std::to_string(values[i]);
+        b->shape_env_sig += ';';
+    }
+    return FNN_OK;
+}
+
 int fnn_backend_dispatch(fnn_backend *b, fnn_plan *p)
 {
-    return guarded(b, "fnn_backend_dispatch", [&]() -> int { return dispatch_impl(b, p, nullptr, 0); });
+    return guarded(b, "fnn_backend_dispatch", [&]() -> int {
+        if (b) { b->shape_env.clear(); b->shape_env_sig.clear(); }
+        return dispatch_impl(b, p, nullptr, 0);
+    });
+}
+
+int fnn_backend_dispatch_env(fnn_backend *b, fnn_plan *p, const char *const *names, const uint64_t *values, uint64_t n_symbols)
+{
+    return guarded(b, "fnn_backend_dispatch_env", [&]() -> int {
+        if (!b) return fail(nullptr, FNN_ERR_DISPATCH, "dispatch: NULL argument");
+        if ((!names || !values) && n_symbols) return fail(b, FNN_ERR_DISPATCH, "dispatch: NULL shape environment");
+        int st = set_shape_env(b, names, values, n_symbols);
+        if (st) return st;
+        return dispatch_impl(b, p, nullptr, 0);
+    });
+}
+
+// ---- ExecutablePlan::save / load (src/backend/mod.rs:117-131): bincode 1.3 with its default options, i.e. little
+// endian, fixed-width integers (usize and u64 as 8 bytes, enum variant index as u32), sequence and string lengths as
+// u64, Option as one tag byte, f32 as 4 bytes, fixed-size arrays without a length, Arc<T> as T.
+namespace {
+
+struct Reader {
+    const uint8_t *p;
+    uint64_t left;
+    bool ok = true;
+    bool take(void *dst, uint64_t n)
+    {
+        if (!ok || n > left) { ok = false; return false; }
+        memcpy(dst, p, n);
+        p += n;
+        left -= n;
+        return true;
+    }
+    uint64_t u64() { uint64_t v = 0; take(&v, 8); return v; }
+    uint32_t u32() { uint32_t v = 0; take(&v, 4); return v; }
+    uint8_t u8() { uint8_t v = 0; take(&v, 1); return v; }
+    float f32() { float v = 0; take(&v, 4); return v; }
+    // a length that the remaining bytes can hold at `elem` bytes per element (refuses absurd lengths before allocating)
+    uint64_t len(uint64_t elem)
+    {
+        const uint64_t n = u64();
+        if (ok && elem && n > left / elem) ok = false;
+        return ok ? n : 0;
+    }
+    std::string str()
+    {
+        const uint64_t n = len(1);
+        std::string s((size_t)n, '\0');
+        if (n) take(&s[0], n);
+        return s;
+    }
+    fnn_slice slice() { fnn_slice s; s.offset = u64(); s.size = u64(); return s; }
+};
+
+struct Writer {
+    std::vector<uint8_t> out;
+    void put(const void *src, size_t n) { const uint8_t *b = (const uint8_t *)src; out.insert(out.end(), b, b + n); }
+    void u64(uint64_t v) { put(&v, 8); }
+    void u32(uint32_t v) { put(&v, 4); }
+    void u8(uint8_t v) { put(&v, 1); }
+    void f32(float v) { put(&v, 4); }
+    void str(const std::string &s) { u64(s.size()); put(s.data(), s.size()); }
+    void slice(const fnn_slice &s) { u64(s.offset); u64(s.size); }
+};
+
+}  // namespace
+
+int fnn_plan_from_bincode(const void *bytes, uint64_t len, fnn_plan **out)
+{
+    return guarded(nullptr, "fnn_plan_from_bincode", [&]() -> int {
+        if (!out || (!bytes && len)) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_plan_from_bincode: NULL argument");
+        *out = nullptr;
+        Reader r{(const uint8_t *)bytes, len};
+        fnn_plan *p = nullptr;
+        int st = fnn_plan_create(0, &p);
+        if (st) return st;
+        auto bad = [&](const char *what, uint64_t index) {
+            const uint64_t at = len - r.left;
+            fnn_plan_destroy(p);
+            return fail(nullptr, FNN_ERR_COMPILATION, "fnn_plan_from_bincode: %s (instruction %llu, byte %llu of %llu)", what,
+                        (unsigned long long)index, (unsigned long long)at, (unsigned long long)len);
+        };
+        // ExecutablePlan { instructions: Vec<Instruction>, arena_size: usize, levels: Vec<usize> }
+        const uint64_t n_instr = r.len(4);
+        for (uint64_t i = 0; i < n_instr; i++) {
+            Instr in;
+            const uint32_t variant = r.u32();   // enum Instruction { CallKernel, MemCopy, Fill, WriteConst }
+            if (!r.ok) return bad("truncated", i);
+            switch (variant) {
+            case 0: {
+                in.kind = K_CALL;
+                in.kernel = r.str();                                  // kernel_name: String
+                const uint64_t n_in = r.len(16);                      // input_slices: Vec<BufferSlice>
+                for (uint64_t k = 0; k < n_in; k++) in.inputs.push_back(r.slice());
+                in.dst = r.slice();                                   // output_slice: BufferSlice
+                const uint8_t has_sec = r.u8();                       // secondary_output_slice: Option<BufferSlice>
+                if (has_sec > 1) return bad("Option tag is neither 0 nor 1 (secondary_output_slice)", i);
+                if (has_sec) { in.has_secondary = true; in.secondary = r.slice(); }
+                const uint64_t n_par = r.len(8);                      // params: Vec<usize>
+                for (uint64_t k = 0; k < n_par; k++) in.params.push_back(r.u64());
+                const uint8_t has_node = r.u8();                      // node_id: Option<NodeId = usize>
+                if (has_node > 1) return bad("Option tag is neither 0 nor 1 (node_id)", i);
+                if (has_node) { in.has_node_id = true; in.node_id = r.u64(); }
+                const uint8_t has_dims = r.u8();                      // param_dims: Option<Vec<DimExpr>>
+                if (has_dims > 1) return bad("Option tag is neither 0 nor 1 (param_dims)", i);
+                if (has_dims) {
+                    in.has_param_dims = true;
+                    const uint64_t n_d = r.len(4);
+                    for (uint64_t k = 0; k < n_d && r.ok; k++) {
+                        Instr::Dim d;
+                        d.kind = r.u32();                             // enum DimExpr { Known(u64), Symbol(String), Bounded { sym, max } }
+                        if (d.kind == 0) d.value = r.u64();
+                        else if (d.kind == 1) d.sym = r.str();
+                        else if (d.kind == 2) { d.sym = r.str(); d.value = r.u64(); }
+                        else return bad("unknown DimExpr variant", i);
+                        in.param_dims.push_back(std::move(d));
+                    }
+                }
+                const uint8_t has_meta = r.u8();                      // weight_meta: Option<Arc<QuantizedWeightMeta>>
+                if (has_meta > 1) return bad("Option tag is neither 0 nor 1 (weight_meta)", i);
+                if (has_meta) {
+                    in.meta.present = true;
+                    in.meta.bit_width = r.u64();                      // bit_width: usize
+                    const uint64_t n_sc = r.len(4);                   // scales: Vec<f32>
+                    for (uint64_t k = 0; k < n_sc; k++) in.meta.scales.push_back(r.f32());
+                    const uint64_t n_zp = r.len(4);                   // zero_points: Vec<f32>
+                    for (uint64_t k = 0; k < n_zp; k++) in.meta.zeros.push_back(r.f32());
+                    const uint64_t n_sh = r.len(8);                   // shape: Vec<usize>
+                    for (uint64_t k = 0; k < n_sh; k++) in.meta.shape.push_back(r.u64());
+                    in.meta.qblock = r.u64();                         // quant_block_size: usize
+                    const uint64_t n_cb = r.len(64);                  // codebooks: Vec<[f32; 16]>
+                    for (uint64_t k = 0; k < n_cb * 16; k++) in.meta.codebook.push_back(r.f32());
+                }
+                break;
+            }
+            case 1: in.kind = K_MEMCOPY; in.dst = r.slice(); in.src = r.slice(); break;    // MemCopy { dst, src }
+            case 2: in.kind = K_FILL; in.dst = r.slice(); in.value = r.f32(); break;        // Fill { dst, value: f32 }
+            case 3: {                                                                       // WriteConst { dst, data: Vec<u8> }
+                in.kind = K_WRITE_CONST;
+                in.dst = r.slice();
+                const uint64_t n = r.len(1);
+                in.data.resize((size_t)n);
+                if (n) r.take(in.data.data(), n);
+                in.dst.size = in.data.size();   // the dispatcher copies data.len() bytes to dst.offset (src/backend/cpu/mod.rs:7111-7121)
+                break;
+            }
+            default: return bad("unknown Instruction variant", i);
+            }
+            if (!r.ok) return bad("truncated", i);
+            p->instrs.push_back(std::move(in));
+        }
+        p->arena_size = r.u64();
+        const uint64_t n_lv = r.len(8);
+        for (uint64_t k = 0; k < n_lv; k++) p->levels.push_back(r.u64());
+        if (!r.ok) return bad("truncated after the instructions", n_instr);
+        if (r.left) return bad("trailing bytes", n_instr);
+        touched(p);
+        *out = p;
+        return FNN_OK;
+    });
+}
+
+int fnn_plan_to_bincode(const fnn_plan *p, void *buf, uint64_t cap, uint64_t *needed)
+{
+    return guarded(nullptr, "fnn_plan_to_bincode", [&]() -> int {
+        if (!p || !needed) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_plan_to_bincode: NULL argument");
+        Writer w;
+        w.u64(p->instrs.size());
+        for (const Instr &in : p->instrs) {
+            switch (in.kind) {
+            case K_CALL:
+                w.u32(0);
+                w.str(in.kernel);
+                w.u64(in.inputs.size());
+                for (const auto &s : in.inputs) w.slice(s);
+                w.slice(in.dst);
+                w.u8(in.has_secondary ? 1 : 0);
+                if (in.has_secondary) w.slice(in.secondary);
+                w.u64(in.params.size());
+                for (uint64_t v : in.params) w.u64(v);
+                w.u8(in.has_node_id ? 1 : 0);
+                if (in.has_node_id) w.u64(in.node_id);
+                w.u8(in.has_param_dims ? 1 : 0);
+                if (in.has_param_dims) {
+                    w.u64(in.param_dims.size());
+                    for (const auto &d : in.param_dims) {
+                        w.u32(d.kind);
+                        if (d.kind == 0) w.u64(d.value);
+                        else if (d.kind == 1) w.str(d.sym);
+                        else { w.str(d.sym); w.u64(d.value); }
+                    }
+                }
+                w.u8(in.meta.present ? 1 : 0);
+                if (in.meta.present) {
+                    w.u64(in.meta.bit_width);
+                    w.u64(in.meta.scales.size());
+                    for (float v : in.meta.scales) w.f32(v);
+                    w.u64(in.meta.zeros.size());
+                    for (float v : in.meta.zeros) w.f32(v);
+                    w.u64(in.meta.shape.size());
+                    for (uint64_t v : in.meta.shape) w.u64(v);
+                    w.u64(in.meta.qblock);
+                    w.u64(in.meta.codebook.size() / 16);
+                    for (float v : in.meta.codebook) w.f32(v);
+                }
+                break;
+            case K_MEMCOPY: w.u32(1); w.slice(in.dst); w.slice(in.src); break;
+            case K_FILL: w.u32(2); w.slice(in.dst); w.f32(in.value); break;
+            case K_WRITE_CONST:
+                w.u32(3);
+                w.slice(in.dst);
+                w.u64(in.data.size());
+                w.put(in.data.data(), in.data.size());
+                break;
+            }
+        }
+        w.u64(p->arena_size);
+        // levels: as loaded; a plan built through fnn_plan_add_* is sequential (level i for instruction i)
+        if (p->levels.size() == p->instrs.size()) {
+            w.u64(p->levels.size());
+            for (uint64_t v : p->levels) w.u64(v);
+        } else {
+            w.u64(p->instrs.size());
+            for (uint64_t i = 0; i < p->instrs.size(); i++) w.u64(i);
+        }
+        *needed = w.out.size();
+        if (buf && cap >= w.out.size()) memcpy(buf, w.out.data(), w.out.size());
+        else if (buf) return fail(nullptr, FNN_ERR_MEMORY, "fnn_plan_to_bincode: buffer of %llu bytes, plan needs %llu", (unsigned long long)cap, (unsigned long long)w.out.size());
+        return FNN_OK;
+    });
+}
+
+uint64_t fnn_plan_arena_size(const fnn_plan *p) { return p ? p->arena_size : 0; }
+
+int fnn_plan_describe(const fnn_plan *p, uint64_t instruction, char *buf, uint64_t cap)
+{
+    return guarded(nullptr, "fnn_plan_describe", [&]() -> int {
+        if (!p || !buf || cap == 0) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_plan_describe: NULL argument");
+        if (instruction >= p->instrs.size()) return fail(nullptr, FNN_ERR_DISPATCH, "fnn_plan_describe: instruction %llu of %zu", (unsigned long long)instruction, p->instrs.size());
+        const Instr &in = p->instrs[instruction];
+        std::string s;
+        auto sl = [](const fnn_slice &x) { return "[" + std::to_string(x.offset) + "," + std::to_string(x.size) + "]"; };
+        switch (in.kind) {
+        case K_WRITE_CONST: s = "{\"op\":\"WriteConst\",\"dst\":" + sl(in.dst) + ",\"len\":" + std::to_string(in.data.size()) + "}"; break;
+        case K_FILL: {
+            char v[64];
+            snprintf(v, sizeof v, "%.9g", (double)in.value);
+            s = "{\"op\":\"Fill\",\"dst\":" + sl(in.dst) + ",\"value\":" + v + "}";
+            break;
+        }
+        case K_MEMCOPY: s = "{\"op\":\"MemCopy\",\"dst\":" + sl(in.dst) + ",\"src\":" + sl(in.src) + "}"; break;
+        case K_CALL: {
+            s = "{\"op\":\"CallKernel\",\"kernel\":\"" + in.kernel + "\",\"inputs\":[";
+            for (size_t i = 0; i < in.inputs.size(); i++) s += (i ? "," : "") + sl(in.inputs[i]);
+            s += "],\"output\":" + sl(in.dst);
+            s += ",\"secondary\":" + (in.has_secondary ? sl(in.secondary) : std::string("null"));
+            s += ",\"params\":[";
+            for (size_t i = 0; i < in.params.size(); i++) s += (i ? "," : "") + std::to_string(in.params[i]);
+            s += "],\"node_id\":" + (in.has_node_id ? std::to_string(in.node_id) : std::string("null"));
+            s += ",\"param_dims\":";
+            if (!in.has_param_dims) s += "null";
+            else {
+                s += "[";
+                for (size_t i = 0; i < in.param_dims.size(); i++) {
+                    const auto &d = in.param_dims[i];
+                    s += i ? "," : "";
+                    if (d.kind == 0) s += std::to_string(d.value);
+                    else if (d.kind == 1) s += "\"" + d.sym + "\"";
+                    else s += "{\"sym\":\"" + d.sym + "\",\"max\":" + std::to_string(d.value) + "}";
+                }
+                s += "]";
+            }
+            s += ",\"meta\":";
+            if (!in.meta.present) s += "null";
+            else {
+                s += "{\"bit_width\":" + std::to_string(in.meta.bit_width) + ",\"n_scales\":" + std::to_string(in.meta.scales.size()) +
+                     ",\"n_zero_points\":" + std::to_string(in.meta.zeros.size()) + ",\"shape\":[";
+                for (size_t i = 0; i < in.meta.shape.size(); i++) s += (i ? "," : "") + std::to_string(in.meta.shape[i]);
+                s += "],\"quant_block_size\":" + std::to_string(in.meta.qblock) + ",\"n_codebooks\":" + std::to_string(in.meta.codebook.size() / 16) + "}";
+            }
+            s += "}";
+            break;
+        }
+        }
+        if (s.size() + 1 > cap) return fail(nullptr, FNN_ERR_MEMORY, "fnn_plan_describe: needs %zu bytes", s.size() + 1);
+        memcpy(buf, s.c_str(), s.size() + 1);
+        return FNN_OK;
+    });
 }
 
 int fnn_backend_dispatch_profile(fnn_backend *b, fnn_plan *p, uint64_t *elapsed_ns, uint64_t n)

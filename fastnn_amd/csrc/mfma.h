@@ -40,6 +40,10 @@ int fnn_row_means(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, cons
 int fnn_mfma_qgemv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &p,
                    int flags, bool *handled);
 
+// M <= 4, integer weights (I8, I4, U4): int8 matrix cores, activations as three exact base-256 digit rows, one
+// workgroup per CU walking the row tiles (no decode arithmetic, activations converted once per workgroup).
+int fnn_i8dot_qgemv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &p, bool *handled);
+
 // 9 <= M <= 16: the same organisation with the 16 activation rows as the MFMA operand rows, loaded straight
 // into registers (no preparation or reduction launch).
 int fnn_mfma_rows16(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &p,

@@ -30,6 +30,8 @@ OPT_TILE_SHAPE = 5
 OPT_TILE_SPLIT = 6
 OPT_TILE_STAGES = 7
 OPT_TILE_MIN_M = 8
+OPT_GEMV_INT8 = 9
+OPT_GEMV_GRID = 10
 
 STATUS_NAMES = {0: "Ok", 1: "Dispatch", 2: "Memory", 3: "UnsupportedOp", 4: "Compilation"}
 
@@ -50,8 +52,9 @@ BACKEND_SYMBOLS = [
     "fnn_backend_set_kernel_flags", "fnn_backend_set_graph_replay", "fnn_backend_set_option",
     "fnn_backend_allocate_arena", "fnn_backend_write_arena", "fnn_backend_read_arena",
     "fnn_plan_create", "fnn_plan_destroy", "fnn_plan_add_write_const", "fnn_plan_add_fill",
-    "fnn_plan_add_memcopy", "fnn_plan_add_call_kernel", "fnn_plan_len", "fnn_plan_replayed",
-    "fnn_backend_dispatch", "fnn_backend_dispatch_profile",
+    "fnn_plan_add_memcopy", "fnn_plan_add_call_kernel", "fnn_plan_len", "fnn_plan_replayed", "fnn_plan_arena_size",
+    "fnn_plan_set_param_dims", "fnn_plan_from_bincode", "fnn_plan_to_bincode", "fnn_plan_describe",
+    "fnn_backend_dispatch", "fnn_backend_dispatch_env", "fnn_backend_dispatch_profile",
     "fnn_hip_elementwise", "fnn_hip_fill_f32", "fnn_hip_copy",
     "fnn_hip_copy2d_f32", "fnn_hip_maxpool2d_f32", "fnn_hip_avgpool2d_f32", "fnn_hip_upsample_nearest2d_f32",
 ]
@@ -96,6 +99,11 @@ _sz = C.c_size_t
 class Slice(C.Structure):
     """fnn_slice: BufferSlice {offset, size} in bytes."""
     _fields_ = [("offset", C.c_uint64), ("size", C.c_uint64)]
+
+
+class DimExpr(C.Structure):
+    """fnn_dim_expr: kind 0 Known(value), 1 Symbol(symbol), 2 Bounded{sym: symbol, max: value}."""
+    _fields_ = [("kind", C.c_uint32), ("value", C.c_uint64), ("symbol", C.c_char_p)]
 
 
 class WeightMeta(C.Structure):
@@ -174,6 +182,13 @@ def _prototype(l):
     l.fnn_plan_replayed.argtypes = [_vp]
     l.fnn_plan_replayed.restype = C.c_int
     l.fnn_backend_dispatch.argtypes = [_vp, _vp]
+    l.fnn_backend_dispatch_env.argtypes = [_vp, _vp, C.POINTER(C.c_char_p), C.POINTER(_u64), _u64]
+    l.fnn_plan_arena_size.argtypes = [_vp]
+    l.fnn_plan_arena_size.restype = _u64
+    l.fnn_plan_set_param_dims.argtypes = [_vp, _u64, C.POINTER(DimExpr), _u64]
+    l.fnn_plan_from_bincode.argtypes = [_vp, _u64, C.POINTER(_vp)]
+    l.fnn_plan_to_bincode.argtypes = [_vp, _vp, _u64, C.POINTER(_u64)]
+    l.fnn_plan_describe.argtypes = [_vp, _u64, C.c_char_p, _u64]
     l.fnn_backend_dispatch_profile.argtypes = [_vp, _vp, C.POINTER(_u64), _u64]
     l.fnn_hip_elementwise.argtypes = [_vp, C.c_int, _vp, _vp, _u64, _vp, _u64]
     l.fnn_hip_fill_f32.argtypes = [_vp, _vp, _u64, C.c_float]

@@ -96,7 +96,11 @@ enum {
     FNN_OPT_TILE_SPLIT = 6,       /* tiled GEMM: K split over this many workgroups; 0 (default) = cost model        */
     FNN_OPT_TILE_STAGES = 7,      /* tiled GEMM, 128x128 tiles: 5 = deep ring, 3 = shallow; 0 (default) = by shape  */
     FNN_OPT_TILE_MIN_M = 8,       /* smallest M the tiled GEMM takes (default 5)                                    */
-    FNN_OPT_COUNT = 9
+    FNN_OPT_GEMV_INT8 = 9,        /* 1: M <= 4 with I8 / I4 / U4 weights runs on the int8 matrix cores (activations as  */
+                                  /* four exact base-256 digit rows, integer sums: agreement ~1e-6 instead of 2e-5);   */
+                                  /* 0 (default): the f16 GEMV kernel, which measures 0 to 15 % faster                 */
+    FNN_OPT_GEMV_GRID = 10,       /* workgroups of the int8 GEMV kernel; 0 (default) = one per CU                      */
+    FNN_OPT_COUNT = 11
 };
 int fnn_hip_set_option(fnn_hip_ctx *ctx, int option, int64_t value);
 int fnn_hip_get_option(fnn_hip_ctx *ctx, int option, int64_t *value);

@@ -80,6 +80,32 @@ int fnn_plan_add_call_kernel(fnn_plan *p, const char *kernel_name, const fnn_sli
                              uint64_t n_inputs, fnn_slice output, const fnn_slice *secondary_output,
                              const uint64_t *params, uint64_t n_params, const fnn_weight_meta *meta);
 uint64_t fnn_plan_len(const fnn_plan *p);
+uint64_t fnn_plan_arena_size(const fnn_plan *p);
+
+/* CallKernel.param_dims (src/backend/mod.rs:72-78): the symbolic form of `params`, one DimExpr
+ * (src/ir/node.rs:163-167) per parameter.  kind 0 = Known(value), 1 = Symbol(symbol), 2 = Bounded { sym: symbol,
+ * max: value }.  A quantised MatMul with param_dims takes [M, K, N] from them at dispatch time, evaluated in the
+ * dispatch's shape environment exactly as resolve_params does (src/backend/cpu/params.rs:11-39,
+ * DimExpr::evaluate_with_env, src/ir/node.rs:511-531): a Symbol must be bound, a Bounded dim falls back to its max
+ * and refuses a larger binding; error texts are the reference's.  The other kernels of this backend take their
+ * params as stored, like their CPU arms. */
+typedef struct {
+    uint32_t kind;
+    uint64_t value;
+    const char *symbol;   /* NULL for kind 0 */
+} fnn_dim_expr;
+int fnn_plan_set_param_dims(fnn_plan *p, uint64_t instruction, const fnn_dim_expr *dims, uint64_t n_dims);
+
+/* ExecutablePlan::load / save (src/backend/mod.rs:117-131): the serde layout of ExecutablePlan, Instruction,
+ * BufferSlice, QuantizedWeightMeta and DimExpr under bincode 1.3's default options (little endian, usize / u64 as 8
+ * bytes, enum variant index as u32, Vec / String length as u64, Option as one tag byte, [f32; 16] without a length,
+ * Arc<T> as T).  from_bincode refuses truncated input, trailing bytes, unknown variants and lengths the remaining
+ * bytes cannot hold (FNN_ERR_COMPILATION, message with the byte offset).  node_id and levels are kept and written
+ * back unchanged.  to_bincode: *needed receives the size; buf may be NULL to ask for it. */
+int fnn_plan_from_bincode(const void *bytes, uint64_t len, fnn_plan **out);
+int fnn_plan_to_bincode(const fnn_plan *p, void *buf, uint64_t cap, uint64_t *needed);
+/* One instruction as a line of JSON (no counterpart in fastnn: for tools and tests). */
+int fnn_plan_describe(const fnn_plan *p, uint64_t instruction, char *buf, uint64_t cap);
 
 /* Backend::dispatch, src/backend/mod.rs:167-176.  Synchronises before returning.
  * The first dispatch of a plan uploads its WriteConst payloads and runs instruction by
@@ -88,6 +114,12 @@ uint64_t fnn_plan_len(const fnn_plan *p);
  * dispatches skip the uploads and replay the instruction stream as one HIP graph, the static-shape plan
  * reuse of src/backend/executor.rs:639-667 (see fnn_backend_set_graph_replay). */
 int fnn_backend_dispatch(fnn_backend *b, fnn_plan *p);
+/* Backend::dispatch with its ShapeEnv argument (src/backend/mod.rs:167-176, src/ir/node.rs:347-391): n_symbols
+ * (name, value) bindings, valid for this dispatch; fnn_backend_dispatch is the same with an empty environment.  A
+ * name bound twice to different values is refused, as ShapeEnv::bind does.  A resident plan replays its graph only
+ * under the environment the graph was recorded with. */
+int fnn_backend_dispatch_env(fnn_backend *b, fnn_plan *p, const char *const *names, const uint64_t *values,
+                             uint64_t n_symbols);
 /* 1 when the last dispatch of the plan ran as a graph replay, else 0 (no counterpart in fastnn:
  * lets tests and tools see which path ran). */
 int fnn_plan_replayed(const fnn_plan *p);

@@ -701,3 +701,73 @@ def test_graph_replay_switch_and_context_options(be, orc):
         be.set_graph_replay(True)
         be.set_option(flib.OPT_TILE_SHAPE, -1)
         be.set_option(flib.OPT_TILE_SPLIT, 0)
+
+
+def test_loaded_plan_dispatches_with_a_shape_environment(be, orc):
+    """The hand-assembled saved plan (tests/golden/executable_plan.bin) runs on the device: constants from its
+    WriteConst payloads, [M, K, N] of both MatMuls resolved from param_dims under ShapeEnv {B: 2} (a Symbol and a
+    Bounded dim), results against the oracle on the fixture's own words and metadata."""
+    import os
+    import struct
+    from fastnn_amd.backend import ExecutablePlan as EP
+    here = os.path.dirname(os.path.abspath(__file__))
+    plan = EP.load(os.path.join(here, "golden", "executable_plan.bin"))
+    rows = [[1, -1, 2, -2, 3, -3, 4, -4], [5, 6, 7, 8, -5, -6, -7, -8], [127, -128, 0, 1, -1, 64, -64, 10], [0, 0, 0, 9, 0, 0, -9, 0]]
+    words = np.frombuffer(b"".join(struct.pack("<8b", *r) for r in rows), np.uint32)
+    w8 = orc.Packed(flib.DT_I8, 4, 8, np.concatenate([words, np.zeros(16, np.uint32)]), np.float32([0.5, 0.25, 1.0, 2.0]),
+                    np.float32([0.0, 0.5, -1.0, 0.0]))
+    idx = [[(3 * k + r) % 16 for k in range(32)] for r in range(2)]
+    cbw = np.array([sum(n << (4 * i) for i, n in enumerate(row[w * 8:(w + 1) * 8])) for row in idx for w in range(4)], np.uint32)
+    wcb = orc.Packed(flib.DT_I4CB, 2, 32, np.concatenate([cbw, np.zeros(16, np.uint32)]), np.float32([0.75, 1.5]), np.zeros(0, np.float32), 32,
+                     np.float32([-1.0 + 2.0 * i / 15.0 for i in range(16)]))
+    rng = np.random.default_rng(91)
+    x1 = rng.standard_normal((2, 8)).astype(np.float32)
+    x2 = rng.standard_normal((2, 32)).astype(np.float32)
+    be.allocate_arena(plan.arena_size)
+    for it in range(3):
+        be.write_arena(0, x1)
+        be.write_arena(576, x2)
+        be.dispatch(plan, {"B": 2})
+        assert plan.replayed == (it >= 1)
+        y1 = orc.qmatmul(w8, x1, bias=np.float32([0.5, -0.25, 1.0, 0.0]), act=flib.ACT_RELU)
+        assert_close(be.read_arena(256, 32, np.float32).reshape(2, 4), y1, 2e-5, "matmul_i8_relu of the loaded plan")
+        assert np.array_equal(be.read_arena(320, 32, np.float32), be.read_arena(256, 32, np.float32))          # MemCopy
+        pv, pi = orc.maxpool2d(be.read_arena(320, 32, np.float32).reshape(1, 2, 2, 2), 2, 2, 0, return_indices=True)
+        assert np.array_equal(be.read_arena(384, 8, np.float32), pv.reshape(-1))
+        assert np.array_equal(be.read_arena(392, 16, np.int64), pi.reshape(-1))
+        assert_close(be.read_arena(1152, 16, np.float32).reshape(2, 2), orc.qmatmul(wcb, x2), 2e-5, "codebook matmul of the loaded plan")
+    # another binding of the same plan: one row; the graph recorded under B = 2 is not replayed
+    be.dispatch(plan, {"B": 1})
+    assert_close(be.read_arena(1152, 8, np.float32).reshape(1, 2), orc.qmatmul(wcb, x2[:1]), 2e-5, "B = 1")
+    with pytest.raises(flib.FnnError) as e:
+        be.dispatch(plan)                              # empty environment
+    assert e.value.kind == "Dispatch" and "DimExpr::Symbol 'B' is not bound in the ShapeEnv" in e.value.message
+    plan.close()
+
+
+def test_bounded_dims_fall_back_to_their_maximum_and_refuse_larger_bindings(be, orc):
+    rng = np.random.default_rng(92)
+    k, n = 64, 24
+    pw = fastnn_amd.quantize_weights(flib.DT_F8, _w(rng, n, k))
+    x = rng.standard_normal((4, k)).astype(np.float32)
+    a = Arena()
+    s_x, s_w, s_o = a.take(x.nbytes), a.take(pw.words.nbytes), a.take(4 * n * 4)
+    plan = ExecutablePlan(a.top).write_const(s_x[0], x).write_const(s_w[0], pw.words)
+    plan.call_kernel("matmul_f8", [s_x, s_w], s_o, [1, k, n], meta_of(pw))       # stored params say M = 1
+    plan.set_param_dims(2, [("T", 4), k, n])
+    be.allocate_arena(a.top)
+    want = orc.qmatmul(to_oracle(orc, pw), x)
+    be.dispatch(plan)                                  # unbound Bounded dim: its max, 4 rows
+    assert_close(be.read_arena(*s_o, np.float32).reshape(4, n), want, 2e-5, "Bounded -> max")
+    be.write_arena(s_o[0], np.zeros(4 * n, np.float32))
+    be.dispatch(plan, {"T": 3})
+    got = be.read_arena(*s_o, np.float32).reshape(4, n)
+    assert_close(got[:3], want[:3], 2e-5, "T = 3")
+    assert not got[3].any()
+    with pytest.raises(flib.FnnError) as e:
+        be.dispatch(plan, {"T": 5})
+    assert "DimExpr::Bounded: symbol 'T' resolved to 5, exceeds bound 4" in e.value.message
+    plan.set_param_dims(2, [1, k])
+    with pytest.raises(flib.FnnError) as e:
+        be.dispatch(plan)
+    assert "param_dims has 2 elements but expected 3" in e.value.message
