@@ -209,6 +209,19 @@ class HipBackend:
         values = (C.c_uint64 * len(shape_env))(*[int(v) for v in shape_env.values()])
         self._check(self.lib.fnn_backend_dispatch_env(self.handle, plan.handle, names, values, len(shape_env)))
 
+    def dispatch_from(self, plan: ExecutablePlan, first: int = 0, shape_env: Optional[dict] = None):
+        """One segment of a dispatch (fnn_backend_dispatch_from): returns None when the end of the plan was reached,
+        else the index of the instruction whose kernel has no GPU implementation (run it elsewhere, resume behind it)."""
+        env = shape_env or {}
+        names = (C.c_char_p * max(len(env), 1))(*[k.encode() for k in env])
+        values = (C.c_uint64 * max(len(env), 1))(*[int(v) for v in env.values()])
+        stopped = C.c_uint64()
+        rc = self.lib.fnn_backend_dispatch_from(self.handle, plan.handle, names, values, len(env), first, C.byref(stopped))
+        if rc == 3:
+            return int(stopped.value)
+        self._check(rc)
+        return None
+
     def dispatch_profile(self, plan: ExecutablePlan):
         n = len(plan)
         t = (C.c_uint64 * max(n, 1))()

@@ -119,6 +119,8 @@ struct fnn_plan {
     fnn_hip_graph *graph = nullptr;
     uint64_t graph_uid = 0, graph_generation = 0, graph_weights_epoch = 0, graph_ws_epoch = 0, graph_scratch_epoch = 0;
     int graph_failures = 0;           // captures that did not go through; after two the plan stays eager
+    bool has_unsupported = false;     // a segmented dispatch stopped at a kernel without a GPU implementation
+    bool segment_resident = false;    // residency as the first segment of the pass in progress found it
     bool last_replayed = false;
 };
 
@@ -706,15 +708,20 @@ int run_instr(fnn_backend *b, fnn_plan *p, Instr &in, bool consts_resident)
     return FNN_OK;
 }
 
-int dispatch_impl(fnn_backend *b, fnn_plan *p, uint64_t *elapsed_ns, uint64_t n_elapsed)
+// first / stopped_at: a caller that runs unsupported kernels elsewhere dispatches in segments.  With stopped_at given,
+// an instruction that returns FNN_ERR_UNSUPPORTED_OP ends the segment (index in *stopped_at, nothing of it has run)
+// and the caller resumes at the next index; a plan that ever stopped this way is not replayed as a graph.
+int dispatch_impl(fnn_backend *b, fnn_plan *p, uint64_t *elapsed_ns, uint64_t n_elapsed, uint64_t first = 0, uint64_t *stopped_at = nullptr)
 {
     if (!b || !p) return fail(b, FNN_ERR_DISPATCH, "dispatch: NULL argument");
+    if (first > p->instrs.size()) return fail(b, FNN_ERR_DISPATCH, "dispatch: first instruction %llu of %zu", (unsigned long long)first, p->instrs.size());
     if (!b->arena) return fail(b, FNN_ERR_MEMORY, "dispatch: no arena allocated");
     if (p->arena_size > b->arena_bytes) return fail(b, FNN_ERR_MEMORY, "dispatch: plan needs an arena of %llu bytes, backend holds %llu", (unsigned long long)p->arena_size, (unsigned long long)b->arena_bytes);
     if (elapsed_ns && n_elapsed < p->instrs.size()) return fail(b, FNN_ERR_DISPATCH, "dispatch_profile: room for %llu timings, plan has %llu instructions", (unsigned long long)n_elapsed, (unsigned long long)p->instrs.size());
     if (!p->analysed) analyse(p);
     bool resident = p->resident_uid == b->uid && p->resident_generation == b->generation;
-    if (resident && p->resident_seq != b->write_seq) {
+    if (first > 0) resident = p->segment_resident;   // later segment of one pass: as the first segment found it
+    else if (resident && p->resident_seq != b->write_seq) {
         // the host wrote into the arena since: still resident unless a constant was hit
         for (const auto &hw : b->host_writes) {
             if (hw.first <= p->resident_seq) continue;
@@ -729,7 +736,8 @@ int dispatch_impl(fnn_backend *b, fnn_plan *p, uint64_t *elapsed_ns, uint64_t n_
     // workspaces have their final size launches as one HIP graph (the executor's static-shape
     // plan, src/backend/executor.rs:639-667).  Profiling, re-uploaded constants and anything
     // that fails under capture keep the instruction-by-instruction path.
-    const bool may_replay = b->graph_replay && !elapsed_ns && resident && !p->uploads_every_run && p->graph_failures < 2;
+    if (first == 0) p->segment_resident = resident;
+    const bool may_replay = b->graph_replay && !elapsed_ns && first == 0 && !p->has_unsupported && resident && !p->uploads_every_run && p->graph_failures < 2;
     if (p->graph && !(may_replay && p->graph_env == b->shape_env_sig && p->graph_uid == b->uid && p->graph_generation == b->generation &&
                       p->graph_weights_epoch == b->weights_epoch && p->graph_ws_epoch == fnn_hip_workspace_epoch(b->ctx) &&
                       p->graph_scratch_epoch == b->scratch_epoch)) {
@@ -766,10 +774,23 @@ int dispatch_impl(fnn_backend *b, fnn_plan *p, uint64_t *elapsed_ns, uint64_t n_
         return st;
     }
 
-    for (size_t i = 0; i < p->instrs.size(); i++) {
+    for (size_t i = (size_t)first; i < p->instrs.size(); i++) {
         auto t0 = std::chrono::steady_clock::now();
         int st = run_instr(b, p, p->instrs[i], resident);
         if (st == FNN_OK && elapsed_ns) st = lift(b, fnn_hip_sync(b->ctx));
+        if (st == FNN_ERR_UNSUPPORTED_OP && stopped_at) {
+            // the caller runs this instruction itself and comes back with first = i + 1
+            fnn_hip_sync(b->ctx);
+            *stopped_at = i;
+            p->has_unsupported = true;
+            if (b->last_plan_uid != p->uid || b->last_plan_revision != p->revision) {
+                b->write_seq++;
+                for (const auto &r : p->writes) log_write(b, r);
+                b->last_plan_uid = p->uid;
+                b->last_plan_revision = p->revision;
+            }
+            return st;
+        }
         if (st != FNN_OK) {
             fnn_hip_sync(b->ctx);
             // what ran before the failure has written: other plans must see it
@@ -931,6 +952,7 @@ int fnn_plan_replayed(const fnn_plan *p) { return p && p->last_replayed ? 1 : 0;
 static void touched(fnn_plan *p)
 {
     p->analysed = false;
+    p->has_unsupported = false;
     p->uploads_every_run = false;
     p->resident_uid = 0;
     p->revision++;
@@ -1069,6 +1091,19 @@ int fnn_backend_dispatch(fnn_backend *b, fnn_plan *p)
     return guarded(b, "fnn_backend_dispatch", [&]() -> int {
         if (b) { b->shape_env.clear(); b->shape_env_sig.clear(); }
         return dispatch_impl(b, p, nullptr, 0);
+    });
+}
+
+int fnn_backend_dispatch_from(fnn_backend *b, fnn_plan *p, const char *const *names, const uint64_t *values, uint64_t n_symbols,
+                              uint64_t first, uint64_t *stopped_at)
+{
+    return guarded(b, "fnn_backend_dispatch_from", [&]() -> int {
+        if (!b || !stopped_at) return fail(b, FNN_ERR_DISPATCH, "dispatch: NULL argument");
+        if ((!names || !values) && n_symbols) return fail(b, FNN_ERR_DISPATCH, "dispatch: NULL shape environment");
+        int st = set_shape_env(b, names, values, n_symbols);
+        if (st) return st;
+        *stopped_at = p ? p->instrs.size() : 0;
+        return dispatch_impl(b, p, nullptr, 0, first, stopped_at);
     });
 }
 

@@ -54,7 +54,7 @@ BACKEND_SYMBOLS = [
     "fnn_plan_create", "fnn_plan_destroy", "fnn_plan_add_write_const", "fnn_plan_add_fill",
     "fnn_plan_add_memcopy", "fnn_plan_add_call_kernel", "fnn_plan_len", "fnn_plan_replayed", "fnn_plan_arena_size",
     "fnn_plan_set_param_dims", "fnn_plan_from_bincode", "fnn_plan_to_bincode", "fnn_plan_describe",
-    "fnn_backend_dispatch", "fnn_backend_dispatch_env", "fnn_backend_dispatch_profile",
+    "fnn_backend_dispatch", "fnn_backend_dispatch_env", "fnn_backend_dispatch_from", "fnn_backend_dispatch_profile",
     "fnn_hip_elementwise", "fnn_hip_fill_f32", "fnn_hip_copy",
     "fnn_hip_copy2d_f32", "fnn_hip_maxpool2d_f32", "fnn_hip_avgpool2d_f32", "fnn_hip_upsample_nearest2d_f32",
 ]
@@ -183,6 +183,7 @@ def _prototype(l):
     l.fnn_plan_replayed.restype = C.c_int
     l.fnn_backend_dispatch.argtypes = [_vp, _vp]
     l.fnn_backend_dispatch_env.argtypes = [_vp, _vp, C.POINTER(C.c_char_p), C.POINTER(_u64), _u64]
+    l.fnn_backend_dispatch_from.argtypes = [_vp, _vp, C.POINTER(C.c_char_p), C.POINTER(_u64), _u64, _u64, C.POINTER(_u64)]
     l.fnn_plan_arena_size.argtypes = [_vp]
     l.fnn_plan_arena_size.restype = _u64
     l.fnn_plan_set_param_dims.argtypes = [_vp, _u64, C.POINTER(DimExpr), _u64]

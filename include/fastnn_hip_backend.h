@@ -120,6 +120,15 @@ int fnn_backend_dispatch(fnn_backend *b, fnn_plan *p);
  * under the environment the graph was recorded with. */
 int fnn_backend_dispatch_env(fnn_backend *b, fnn_plan *p, const char *const *names, const uint64_t *values,
                              uint64_t n_symbols);
+/* Dispatch in segments, for a caller that runs kernels this library does not implement somewhere else, one
+ * instruction at a time, the way WgpuBackend falls back to CpuBackend (src/backend/wgpu/mod.rs:162-239): runs the
+ * instructions from index `first` on.  An instruction that is FNN_ERR_UNSUPPORTED_OP ends the segment with that
+ * status, its index in *stopped_at and nothing of it executed (the message is the kernel name); the caller runs it
+ * (fnn_backend_read_arena / fnn_backend_write_arena) and calls again with first = *stopped_at + 1.  FNN_OK means the
+ * end of the plan was reached (*stopped_at = fnn_plan_len).  Such a plan is never replayed as a graph; its constants
+ * still stay resident between passes. */
+int fnn_backend_dispatch_from(fnn_backend *b, fnn_plan *p, const char *const *names, const uint64_t *values,
+                              uint64_t n_symbols, uint64_t first, uint64_t *stopped_at);
 /* 1 when the last dispatch of the plan ran as a graph replay, else 0 (no counterpart in fastnn:
  * lets tests and tools see which path ran). */
 int fnn_plan_replayed(const fnn_plan *p);

@@ -771,3 +771,40 @@ def test_bounded_dims_fall_back_to_their_maximum_and_refuse_larger_bindings(be, 
     with pytest.raises(flib.FnnError) as e:
         be.dispatch(plan)
     assert "param_dims has 2 elements but expected 3" in e.value.message
+
+
+def test_segmented_dispatch_hands_unsupported_kernels_to_the_caller(be, orc):
+    """A plan with a kernel this library does not implement ("sigmoid_f32") between two quantised MatMuls: the dispatch
+    stops at it with the kernel's index, the caller computes it on the host through read_arena / write_arena and
+    resumes behind it, as a Rust HipBackend does with CpuBackend.  The constants stay resident between passes."""
+    rng = np.random.default_rng(93)
+    m, d, f = 4, 64, 96
+    w1 = fastnn_amd.quantize_weights(flib.DT_I8, _w(rng, f, d))
+    w2 = fastnn_amd.quantize_weights(flib.DT_I4, _w(rng, d, f))
+    a = Arena()
+    s_x, s_w1, s_w2, s_h, s_g, s_y = a.take(m * d * 4), a.take(w1.words.nbytes), a.take(w2.words.nbytes), a.take(m * f * 4), a.take(m * f * 4), a.take(m * d * 4)
+    plan = ExecutablePlan(a.top).write_const(s_w1[0], w1.words).write_const(s_w2[0], w2.words)
+    plan.call_kernel("matmul_i8", [s_x, s_w1], s_h, [m, d, f], meta_of(w1))
+    plan.call_kernel("sigmoid_f32", [s_h], s_g, [m * f])
+    plan.call_kernel("matmul_i4", [s_g, s_w2], s_y, [m, f, d], meta_of(w2))
+    be.allocate_arena(a.top)
+    with pytest.raises(flib.FnnError) as e:
+        be.dispatch(plan)
+    assert e.value.kind == "UnsupportedOp" and e.value.message == "sigmoid_f32"
+    for it in range(3):
+        x = rng.standard_normal((m, d)).astype(np.float32)
+        be.write_arena(s_x[0], x)
+        first, stops = 0, []
+        while True:
+            stop = be.dispatch_from(plan, first)
+            if stop is None:
+                break
+            stops.append(stop)
+            assert plan.describe(stop)["kernel"] == "sigmoid_f32"
+            h = be.read_arena(*s_h, np.float32)
+            be.write_arena(s_g[0], (1.0 / (1.0 + np.exp(-h.astype(np.float64)))).astype(np.float32))
+            first = stop + 1
+        assert stops == [3] and not plan.replayed
+        h_ref = orc.qmatmul(to_oracle(orc, w1), x)
+        g_ref = (1.0 / (1.0 + np.exp(-h_ref.astype(np.float64)))).astype(np.float32)
+        assert_close(be.read_arena(*s_y, np.float32).reshape(m, d), orc.qmatmul(to_oracle(orc, w2), g_ref), 1e-4, f"pass {it}")
