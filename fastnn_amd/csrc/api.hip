@@ -123,8 +123,7 @@ const OptionSpec kOptions[FNN_OPT_COUNT] = {
     {0, 0, 32},       // FNN_OPT_TILE_SPLIT
     {0, 0, 6},        // FNN_OPT_TILE_STAGES
     {5, 1, 1 << 20},  // FNN_OPT_TILE_MIN_M
-    {0, 0, 1},        // FNN_OPT_GEMV_INT8
-    {0, 0, 65535},    // FNN_OPT_GEMV_GRID
+    {1, 0, 1},        // FNN_OPT_GEMV_INT8
 };
 
 #define HIP_TRY(ctx, code, expr)                                                              \

@@ -14,12 +14,12 @@
 // operand, which a GEMV leaves empty anyway, so one MFMA per step yields the four exact i32 partial sums and the
 // matrix core does twice the k-values per instruction of the f16 form, with no decode arithmetic on the vector ALU.
 //
-// Work split: a workgroup converts the activation rows ONCE into digit fragments in LDS and then walks row tiles of 16
-// weight rows (tile = blockIdx.x, += gridDim.x): the grid is one workgroup per CU.  Wave w owns the K slices
-// w, w + NW, ... of every tile; the packed bytes of a wave's next (tile, slice) are requested before it works on the
-// current one, so a wave always has three slices in flight.  Per tile the waves' partial sums meet in LDS in a fixed
-// order (double-buffered: one workgroup barrier per tile) and 16*M threads apply the affine / bias / activation
-// epilogue.  Algorithmic bytes per launch: N*K*bits/8 + side tables + 4*M*(K+N).
+// Work split (the organisation of the f16 GEMV kernel): one workgroup = 16 weight rows x all of K; wave w owns the K
+// slices w, w + NW, ...; it requests its activation slice and its packed bytes, converts the activations into digit
+// fragments in its own LDS area while the bytes are on their way, multiplies, and the waves' partial sums meet in LDS
+// in a fixed order for the fused affine / bias / activation epilogue.  All global reads are raw buffer loads: an
+// address past the end of the weight tile, of K or of the activation rows reads as zero, so no lane clamps or masks.
+// Algorithmic bytes per launch: N*K*bits/8 + side tables + 4*M*(K+N).
 #include "mfma.h"
 
 namespace {
@@ -31,7 +31,6 @@ struct DotArgs {
     int64_t m, n, k, kp;
     int act;
     int nslice;   // slices of 512 k-values covering K
-    int spw;      // slices per wave and tile = ceil(nslice / NW)
     int ntiles;   // row tiles of 16
 };
 
@@ -73,84 +72,92 @@ struct Int8Op<FNN_DT_U4> {
     }
 };
 
-template <int DT, int MM, int NW>
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// Raw buffer descriptor over [base, base + bytes): loads past the end return zero instead of faulting, so no lane
+// clamps or masks its address (rows past N, slices past K, activation rows past M).
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t raw_buffer(const void *base, uint64_t bytes)
+{
+    const uint32_t n = bytes > 0xffffffffull ? 0xffffffffu : (uint32_t)bytes;
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)n, 0x00020000);
+}
+
+template <int DT, int MM, int NW, int RT>
 __global__ void __launch_bounds__(NW * 64) qgemv_i8dot_kernel(DotArgs p)
 {
     using W = Int8Op<DT>;
     constexpr int LOADS = W::LOADS, PER = W::PER_LOAD;
-    constexpr int R4 = 4 * MM;               // digit rows kept in LDS per step: row m*4 + digit
+    constexpr int R4 = 4 * MM;               // digit rows per step: row m*4 + digit, digit 0 the most significant
     constexpr bool FOUR_BIT = PER == 2;
 
-    // [slice][step][R4 rows][4 groups] 16-byte operand fragments, then [slice][MM] slice scales
+    // per wave: [step][R4 rows][4 groups] 16-byte operand fragments of the slice it is working on
     extern __shared__ __attribute__((aligned(16))) uint4 lds_dyn[];
-    __shared__ float red[2][NW][MM][16];
+    __shared__ float red[NW][RT][MM][16];
     __shared__ float xred[NW][MM];
 
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const int ln = lane & 15, g = lane >> 4;
     const int64_t K = p.k, N = p.n, kp = p.kp;
     const int mreal = (int)p.m;
-    const int nslice = p.nslice, spw = p.spw;
-    uint4 *frag = lds_dyn;
-    float *cscale = reinterpret_cast<float *>(lds_dyn + (size_t)nslice * NSTEP * R4 * 4);
+    const int64_t n0 = (int64_t)blockIdx.x * (16 * RT);
+    uint4 *frag = lds_dyn + wv * (NSTEP * R4 * 4);
 
-    // units of work of this wave: (tile, slice) pairs, tile-major
-    const int my_tiles = ((int)blockIdx.x < p.ntiles) ? (p.ntiles - 1 - (int)blockIdx.x) / (int)gridDim.x + 1 : 0;
-    const int nunits = my_tiles * spw;
-
-    // this lane's group of 8 activations of every row for one slice (clamped address, masked afterwards)
-    auto load_slice = [&](int slice, float (&xr)[MM][8]) {
-        const int64_t kk = (int64_t)slice * SL + lane * 8;
-        const int64_t kkc = kk < K ? kk : K - 8;   // K % 8 == 0
+    // the tile's 16 weight rows (rows past N read as zero) and the activation rows (rows past M read as zero)
+    const __amdgpu_buffer_rsrc_t wbuf = raw_buffer(p.words + n0 * kp, (uint64_t)(N - n0) * (uint64_t)kp * 4);
+    __amdgpu_buffer_rsrc_t abuf[MM];
 #pragma unroll
-        for (int m = 0; m < MM; m++) {
-            const int64_t mrow = m < mreal ? m : mreal - 1;
-            const uint32_t keep = (m < mreal && kk < K) ? 0xffffffffu : 0u;
-            const uint4 x0 = *reinterpret_cast<const uint4 *>(p.a + mrow * K + kkc);
-            const uint4 x1 = *reinterpret_cast<const uint4 *>(p.a + mrow * K + kkc + 4);
-            xr[m][0] = __uint_as_float(x0.x & keep); xr[m][1] = __uint_as_float(x0.y & keep);
-            xr[m][2] = __uint_as_float(x0.z & keep); xr[m][3] = __uint_as_float(x0.w & keep);
-            xr[m][4] = __uint_as_float(x1.x & keep); xr[m][5] = __uint_as_float(x1.y & keep);
-            xr[m][6] = __uint_as_float(x1.z & keep); xr[m][7] = __uint_as_float(x1.w & keep);
-        }
-    };
-    // lane (n, g), load l of a slice: words [slice*SL*bits/32 + l*16 + g*4, +4) of row n; a chunk past the end of the
-    // row re-reads the row's last chunk (its activation digits are zero), a slice past K likewise
-    uint32_t wq0[LOADS][4], wq1[LOADS][4], wq2[LOADS][4];
-    auto request = [&](int unit, uint32_t (&dst)[LOADS][4]) {
-        const int it = unit / spw, j = unit - it * spw;
-        const int slice = wv + j * NW;
-        int64_t row = ((int64_t)blockIdx.x + (int64_t)it * gridDim.x) * 16 + ln;
-        if (row > N - 1) row = N - 1;
-        const uint32_t *wrow = p.words + row * kp;
-        const int64_t wbase = (int64_t)slice * (LOADS * 16);
+    for (int m = 0; m < MM; m++) abuf[m] = raw_buffer(p.a + (int64_t)m * K, m < mreal ? (uint64_t)K * 4 : 0);
+    const uint32_t wlane = (uint32_t)ln * (uint32_t)kp * 4 + (uint32_t)g * 16;   // 16 rows of kp words: below 4 GiB (checked on the host)
+
+    // the thread that finishes output (row tile r, m, column c): tid = (r*MM + m)*16 + c; its epilogue operands are
+    // requested first
+    const int e_r = tid / (MM * 16), e_m = (tid >> 4) % MM, e_c = tid & 15;
+    const int64_t e_n = n0 + e_r * 16 + e_c;
+    const bool finisher = tid < RT * MM * 16 && e_m < mreal && e_n < N;
+    float e_scale = 0.0f, e_zero = 0.0f, e_bias = 0.0f;
+    if (finisher) {
+        e_scale = p.scales[e_n];
+        e_zero = p.zeros[e_n];
+        e_bias = p.bias ? p.bias[e_n] : 0.0f;
+    }
+
+    // operand fragment this lane reads at a step: operand row ln = activation row ln / 4, digit ln % 4 (rows past M: row 0)
+    const uint4 *frd = frag + ((ln >> 2) < MM ? ln : 0) * 4 + g;
+
+    float tot[RT];         // lanes with g < MM: partial dot of (activation row g, weight row n0 + r*16 + ln)
 #pragma unroll
-        for (int l = 0; l < LOADS; l++) {
-            const int64_t woff = wbase + l * 16 + g * 4;
-            const uint4 v = *reinterpret_cast<const uint4 *>(wrow + (woff + 4 <= kp ? woff : kp - 4));   // kp % 4 == 0, kp >= 4
-            dst[l][0] = v.x; dst[l][1] = v.y; dst[l][2] = v.z; dst[l][3] = v.w;
-        }
-    };
-
-    // ---- requests first: the wave's first activation slice (oldest, so that its conversion does not wait for packed
-    // bytes), then the packed bytes of its first three units; everything is in flight while the activations are converted
-    float xr[MM][8];
-    load_slice(wv < nslice ? wv : nslice - 1, xr);
-    if (nunits > 0) request(0, wq0);
-    if (nunits > 1) request(1, wq1);
-    if (nunits > 2) request(2, wq2);
-    __builtin_amdgcn_sched_barrier(0);
-
-    // ---- activation rows -> digit fragments (wave w: slices w, w + NW, ..., the ones it multiplies with later, so no
-    // workgroup barrier separates the two)
+    for (int r = 0; r < RT; r++) tot[r] = 0.0f;
     float xsum[MM];
 #pragma unroll
     for (int m = 0; m < MM; m++) xsum[m] = 0.0f;
-    for (int slice = wv; slice < nslice; slice += NW) {
-        if (slice != wv) load_slice(slice, xr);
+
+    for (int slice = wv; slice < p.nslice; slice += NW) {
+        // ---- requests: this lane's 8 activations per row (oldest: their conversion does not wait for packed bytes),
+        // then the slice's packed bytes; lane (n, g), load l: words [slice*SL*bits/32 + l*16 + g*4, +4) of row n.
+        // Bytes past the end of a row belong to the next row or read as zero: their activation digits are zero.
+        u32x4 xa[MM][2];
+        const uint32_t aoff = ((uint32_t)slice * SL + (uint32_t)lane * 8) * 4;
 #pragma unroll
         for (int m = 0; m < MM; m++) {
-            const float *x = xr[m];
+            xa[m][0] = __builtin_amdgcn_raw_buffer_load_b128(abuf[m], aoff, 0, 0);
+            xa[m][1] = __builtin_amdgcn_raw_buffer_load_b128(abuf[m], aoff + 16, 0, 0);
+        }
+        u32x4 wq[RT][LOADS];
+        const uint32_t woff = wlane + (uint32_t)slice * (LOADS * 64);
+#pragma unroll
+        for (int r = 0; r < RT; r++)
+#pragma unroll
+            for (int l = 0; l < LOADS; l++)
+                wq[r][l] = __builtin_amdgcn_raw_buffer_load_b128(wbuf, woff + (uint32_t)r * 16 * (uint32_t)kp * 4 + l * 64, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+
+        // ---- activation slice -> four digit rows per activation row in this wave's LDS area
+        float cs[MM];
+#pragma unroll
+        for (int m = 0; m < MM; m++) {
+            float x[8];
+#pragma unroll
+            for (int j = 0; j < 4; j++) { x[j] = __uint_as_float(xa[m][0][j]); x[4 + j] = __uint_as_float(xa[m][1][j]); }
             float mx = fmaxf(fmaxf(fmaxf(fabsf(x[0]), fabsf(x[1])), fmaxf(fabsf(x[2]), fabsf(x[3]))),
                              fmaxf(fmaxf(fabsf(x[4]), fabsf(x[5])), fmaxf(fabsf(x[6]), fabsf(x[7]))));
             mx = wave_max_uniform(mx);
@@ -164,166 +171,126 @@ __global__ void __launch_bounds__(NW * 64) qgemv_i8dot_kernel(DotArgs p)
             // a NaN or an infinity among the slice's activations shows in their sum: the integer digits cannot carry
             // it, so the slice scale does (the row's outputs become NaN, as the float path's would be NaN or inf)
             const bool finite = fabsf(ssum) <= 3.4028234663852886e38f;
-            if (lane == 0) cscale[slice * MM + m] = finite ? __uint_as_float((uint32_t)(127 + ex) << 23) : __uint_as_float(0x7fc00000u);
-            // v = round(x * 2^-e), |v| < 2^30.  Its balanced base-256 digits (each in [-128, 127], v = sum d_j 256^j)
+            cs[m] = finite ? __uint_as_float((uint32_t)(127 + ex) << 23) : __uint_as_float(0x7fc00000u);
+            // v = trunc(x * 2^-e), |v| < 2^30.  Its balanced base-256 digits (each in [-128, 127], v = sum d_j 256^j)
             // are the bytes of (v + 0x80808080) ^ 0x80808080: adding 128 to every digit gives the plain unsigned
-            // base-256 form, flipping the top bit of every byte subtracts the 128 again.  Byte 3 is the top digit d0.
+            // base-256 form, flipping the top bit of every byte subtracts the 128 again.  Byte 3 is the top digit.
             uint32_t dg[8];
 #pragma unroll
-            for (int j = 0; j < 8; j++)
-                dg[j] = ((uint32_t)(int)rintf(x[j] * inv) + 0x80808080u) ^ 0x80808080u;
-            // digit rows: byte `dgt` of four activations side by side (4x4 byte transposes with v_perm_b32;
-            // selector bytes 0-3 pick from the second operand, 4-7 from the first)
+            for (int j = 0; j < 8; j++) dg[j] = ((uint32_t)(int)(x[j] * inv) + 0x80808080u) ^ 0x80808080u;
+            // digit rows: byte `d` of four activations side by side (4x4 byte transposes with v_perm_b32; selector
+            // bytes 0-3 pick from the second operand, 4-7 from the first)
             auto transpose4 = [](uint32_t a, uint32_t b, uint32_t c, uint32_t d, uint32_t (&o)[4]) {
                 const uint32_t ab_lo = __builtin_amdgcn_perm(b, a, 0x05010400u);   // a0 b0 a1 b1
                 const uint32_t ab_hi = __builtin_amdgcn_perm(b, a, 0x07030602u);   // a2 b2 a3 b3
                 const uint32_t cd_lo = __builtin_amdgcn_perm(d, c, 0x05010400u);
                 const uint32_t cd_hi = __builtin_amdgcn_perm(d, c, 0x07030602u);
-                o[0] = __builtin_amdgcn_perm(cd_lo, ab_lo, 0x05040100u);           // a0 b0 c0 d0: lowest digit d3
-                o[1] = __builtin_amdgcn_perm(cd_lo, ab_lo, 0x07060302u);           // a1 b1 c1 d1
+                o[0] = __builtin_amdgcn_perm(cd_lo, ab_lo, 0x05040100u);           // a0 b0 c0 d0: lowest digit
+                o[1] = __builtin_amdgcn_perm(cd_lo, ab_lo, 0x07060302u);
                 o[2] = __builtin_amdgcn_perm(cd_hi, ab_hi, 0x05040100u);
-                o[3] = __builtin_amdgcn_perm(cd_hi, ab_hi, 0x07060302u);           // a3 b3 c3 d3: top digit d0
+                o[3] = __builtin_amdgcn_perm(cd_hi, ab_hi, 0x07060302u);           // a3 b3 c3 d3: top digit
             };
-            uint32_t t0[4], t1[4];   // [byte of v]: t[3] = top digit row d0 ... t[0] = lowest digit row d3
-            // where this lane's 8 k-values sit in the operand fragments
+            uint32_t t0[4], t1[4];
             if constexpr (FOUR_BIT) {
-                // word `lane` of the slice: load l = lane / 16, group (lane / 4) % 4, word lane % 4 of the 16 bytes;
+                // word `lane` of the slice: load lane / 16, group (lane / 4) % 4, word lane % 4 of the lane's 16 bytes;
                 // even nibbles belong to step 2l, odd nibbles to step 2l + 1
                 transpose4(dg[0], dg[2], dg[4], dg[6], t0);
                 transpose4(dg[1], dg[3], dg[5], dg[7], t1);
-                const int l = lane >> 4, gg = (lane >> 2) & 3, jw = lane & 3;
                 uint32_t *f32w = reinterpret_cast<uint32_t *>(frag);
-                const int base_e = (((slice * NSTEP + 2 * l) * R4 + m * 4) * 4 + gg) * 4 + jw;   // in 4-byte words
-                const int base_o = base_e + R4 * 16;
+                const int base_e = ((2 * (lane >> 4) * R4 + m * 4) * 4 + ((lane >> 2) & 3)) * 4 + (lane & 3);   // 4-byte words
 #pragma unroll
                 for (int d = 0; d < 4; d++) {
                     f32w[base_e + d * 16] = t0[3 - d];
-                    f32w[base_o + d * 16] = t1[3 - d];
+                    f32w[base_e + R4 * 16 + d * 16] = t1[3 - d];
                 }
             } else {
                 // bytes [lane*8, +8) of the slice: step lane / 8, group (lane / 2) % 4, half lane % 2 of the 16 bytes
                 transpose4(dg[0], dg[1], dg[2], dg[3], t0);
                 transpose4(dg[4], dg[5], dg[6], dg[7], t1);
-                const int st = lane >> 3, gg = (lane >> 1) & 3, half = lane & 1;
                 uint2 *f64w = reinterpret_cast<uint2 *>(frag);
-                const int base = (((slice * NSTEP + st) * R4 + m * 4) * 4 + gg) * 2 + half;      // in 8-byte words
+                const int base = (((lane >> 3) * R4 + m * 4) * 4 + ((lane >> 1) & 3)) * 2 + (lane & 1);         // 8-byte words
 #pragma unroll
                 for (int d = 0; d < 4; d++) f64w[base + d * 8] = uint2{t0[3 - d], t1[3 - d]};
             }
         }
+        // only this wave reads the fragments it wrote, and the LDS serves a wave's requests in order
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+
+        // ---- integer MFMA over the slice
+        i32x4 acc[RT];
+#pragma unroll
+        for (int r = 0; r < RT; r++) acc[r] = i32x4{0, 0, 0, 0};
+#pragma unroll
+        for (int l = 0; l < LOADS; l++)
+#pragma unroll
+            for (int q = 0; q < PER; q++) {
+                const i32x4 av = __builtin_bit_cast(i32x4, frd[(l * PER + q) * R4 * 4]);
+#pragma unroll
+                for (int r = 0; r < RT; r++) {
+                    const uint32_t w4[4] = {wq[r][l][0], wq[r][l][1], wq[r][l][2], wq[r][l][3]};
+                    acc[r] = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, W::op(w4, q), acc[r], 0, 0, 0);
+                }
+            }
+        // acc[i] = operand row g*4 + i = digit i of activation row g
+        float csm = cs[0];
+#pragma unroll
+        for (int m = 1; m < MM; m++) csm = g == m ? cs[m] : csm;
+#pragma unroll
+        for (int r = 0; r < RT; r++) {
+            const float hi = fmaf((float)acc[r][0], 256.0f, (float)acc[r][1]), lo = fmaf((float)acc[r][2], 256.0f, (float)acc[r][3]);
+            tot[r] = fmaf(fmaf(hi, 65536.0f, lo), csm, tot[r]);
+        }
+        __builtin_amdgcn_wave_barrier();   // the wave's LDS area is rewritten by its next slice
+    }
+
+    // ---- the waves' partial sums in a fixed order, fused epilogue
+    if (g < MM) {
+#pragma unroll
+        for (int r = 0; r < RT; r++) red[wv][r][g][ln] = tot[r];
     }
     if (lane == 0) {
 #pragma unroll
         for (int m = 0; m < MM; m++) xred[wv][m] = xsum[m];
     }
-    // only this wave reads the fragments it wrote, and the LDS serves a wave's requests in order
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_sched_barrier(0);
-
-    // the thread that finishes output (m, column c) of every tile: tid = m*16 + c
-    const int e_m = tid >> 4, e_c = tid & 15;
-    const bool finisher = tid < MM * 16 && e_m < mreal;
-
-    // operand fragment this lane reads at a step: operand row ln = activation row ln / 4, digit ln % 4; rows past M
-    // re-read row 0
-    const uint4 *frd = frag + ((ln >> 2) < MM ? ln : 0) * 4 + g;
-    const float *csc = cscale + (g < MM ? g : 0);     // this lane's accumulators belong to activation row g
-
-    float tot = 0.0f;
-    float e_scale = 0.0f, e_zero = 0.0f, e_bias = 0.0f, e_xs = 0.0f;
-    int64_t e_n = 0;
-    auto work = [&](int unit, const uint32_t (&cur)[LOADS][4]) {
-        const int it = unit / spw, j = unit - it * spw;
-        const int slice = wv + j * NW;
-        const int64_t tile = (int64_t)blockIdx.x + (int64_t)it * gridDim.x;
-        if (j == 0 && finisher) {   // epilogue operands of this tile: requested now, used after the tile's barrier
-            e_n = tile * 16 + e_c;
-            const int64_t nn = e_n < N ? e_n : N - 1;
-            e_scale = p.scales[nn];
-            e_zero = p.zeros[nn];
-            e_bias = p.bias ? p.bias[nn] : 0.0f;
-        }
-        if (slice < nslice) {
-            i32x4 acc = i32x4{0, 0, 0, 0};
-            const uint4 *fs = frd + (size_t)slice * (NSTEP * R4 * 4);
+    __syncthreads();
+    if (finisher) {
+        float dot = 0.0f, xs = 0.0f;
 #pragma unroll
-            for (int l = 0; l < LOADS; l++)
-#pragma unroll
-                for (int q = 0; q < PER; q++) {
-                    const i32x4 av = __builtin_bit_cast(i32x4, fs[(l * PER + q) * R4 * 4]);
-                    acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, W::op(cur[l], q), acc, 0, 0, 0);
-                }
-            // acc[i] = operand row g*4 + i = digit i of activation row g
-            const float hi = fmaf((float)acc[0], 256.0f, (float)acc[1]), lo = fmaf((float)acc[2], 256.0f, (float)acc[3]);
-            tot = fmaf(fmaf(hi, 65536.0f, lo), csc[slice * MM], tot);
-        }
-        if (j == spw - 1) {
-            // the tile's partial sums of all waves meet in LDS (buffer it & 1); one barrier per tile
-            const int par = it & 1;
-            if (g < MM) red[par][wv][g][ln] = tot;
-            tot = 0.0f;
-            __syncthreads();
-            if (finisher) {
-                if (it == 0) {      // the waves' activation sums: written before the first tile's barrier
-#pragma unroll
-                    for (int w = 0; w < NW; w++) e_xs += xred[w][e_m];
-                }
-                if (e_n < N) {
-                    float dot = 0.0f;
-#pragma unroll
-                    for (int w = 0; w < NW; w++) dot += red[par][w][e_m][e_c];
-                    dot *= W::POST;
-                    const float v = dot * e_scale + e_zero * e_xs;
-                    p.out[(int64_t)e_m * N + e_n] = fnn_activation(p.bias ? v + e_bias : v, p.act);
-                }
-            }
-        }
-    };
-
-    // three units in flight per wave: a buffer is requested again as soon as its unit is done
-    for (int u = 0; u < nunits; u += 3) {
-        work(u, wq0);
-        if (u + 3 < nunits) request(u + 3, wq0);
-        if (u + 1 < nunits) {
-            work(u + 1, wq1);
-            if (u + 4 < nunits) request(u + 4, wq1);
-        }
-        if (u + 2 < nunits) {
-            work(u + 2, wq2);
-            if (u + 5 < nunits) request(u + 5, wq2);
-        }
+        for (int w = 0; w < NW; w++) { dot += red[w][e_r][e_m][e_c]; xs += xred[w][e_m]; }
+        dot *= W::POST;
+        const float v = dot * e_scale + e_zero * xs;
+        p.out[(int64_t)e_m * N + e_n] = fnn_activation(p.bias ? v + e_bias : v, p.act);
     }
 }
 
-template <int DT, int MM, int NW>
-hipError_t launch_nw(DotArgs p, int grid, hipStream_t s, bool *handled)
+template <int DT, int MM, int NW, int RT>
+hipError_t launch_rt(DotArgs p, hipStream_t s, bool *handled)
 {
     p.nslice = (int)((p.k + SL - 1) / SL);
-    p.spw = (p.nslice + NW - 1) / NW;
-    p.ntiles = (int)((p.n + 15) / 16);
-    const size_t lds = (size_t)p.nslice * NSTEP * 4 * MM * 4 * 16 + (size_t)p.nslice * MM * 4;
-    if (lds > 128 * 1024) return hipSuccess;   // long K with several rows: left to the f16 kernels
-    auto kern = qgemv_i8dot_kernel<DT, MM, NW>;
-    if (lds > 48 * 1024) {
-        static std::atomic<uint64_t> lds_raised{0};
-        hipError_t e = fnn_raise_lds_limit(lds_raised, reinterpret_cast<const void *>(kern), 132 * 1024);
-        if (e != hipSuccess) return e;
-    }
-    if (grid <= 0) grid = 256;                 // one workgroup per CU
-    if (grid > p.ntiles) grid = p.ntiles;
-    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NW * 64), lds, s, p);
+    p.ntiles = (int)((p.n + 16 * RT - 1) / (16 * RT));
+    const size_t lds = (size_t)NW * NSTEP * 4 * MM * 4 * 16;    // 2 KiB per wave and activation row
+    hipLaunchKernelGGL((qgemv_i8dot_kernel<DT, MM, NW, RT>), dim3((unsigned)p.ntiles), dim3(NW * 64), lds, s, p);
     *handled = true;
     return hipGetLastError();
 }
 
+template <int DT, int MM, int NW>
+hipError_t launch_nw(const DotArgs &p, int rt, hipStream_t s, bool *handled)
+{
+    if (rt == 3 && MM * 48 <= NW * 64) return launch_rt<DT, MM, NW, 3>(p, s, handled);
+    if (rt >= 2 && MM * 32 <= NW * 64) return launch_rt<DT, MM, NW, 2>(p, s, handled);
+    return launch_rt<DT, MM, NW, 1>(p, s, handled);
+}
+
 template <int DT>
-hipError_t launch_dt(const DotArgs &p, int grid, hipStream_t s, bool *handled)
+hipError_t launch_dt(const DotArgs &p, int rt, hipStream_t s, bool *handled)
 {
     const int mm = p.m <= 1 ? 1 : (p.m <= 2 ? 2 : 4);
     const bool shortk = p.k <= 4 * SL;   // K <= 2048: four waves, so that no wave idles
-    if (mm == 1) return shortk ? launch_nw<DT, 1, 4>(p, grid, s, handled) : launch_nw<DT, 1, 8>(p, grid, s, handled);
-    if (mm == 2) return shortk ? launch_nw<DT, 2, 4>(p, grid, s, handled) : launch_nw<DT, 2, 8>(p, grid, s, handled);
-    return shortk ? launch_nw<DT, 4, 4>(p, grid, s, handled) : launch_nw<DT, 4, 8>(p, grid, s, handled);
+    if (mm == 1) return shortk ? launch_nw<DT, 1, 4>(p, rt, s, handled) : launch_nw<DT, 1, 8>(p, rt, s, handled);
+    if (mm == 2) return shortk ? launch_nw<DT, 2, 4>(p, rt, s, handled) : launch_nw<DT, 2, 8>(p, rt, s, handled);
+    return shortk ? launch_nw<DT, 4, 4>(p, rt, s, handled) : launch_nw<DT, 4, 8>(p, rt, s, handled);
 }
 
 }  // namespace
@@ -336,17 +303,32 @@ int fnn_i8dot_qgemv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, co
     if (q.m < 1 || q.m > 4 || q.n < 1) return FNN_OK;
     if (q.kp % 4 != 0 || q.k % 8 != 0 || q.k < 8) return FNN_OK;
     if ((reinterpret_cast<uintptr_t>(q.a) & 15) || (reinterpret_cast<uintptr_t>(q.words) & 15)) return FNN_OK;
-    if (q.n > (int64_t)16 * 0x7fffffff / 2) return FNN_OK;
+    if (q.n > (int64_t)16 * 0x7fffffff / 2 || q.kp * 4 * 48 >= (int64_t)1 << 31 || q.k >= (int64_t)1 << 29) return FNN_OK;   // 32-bit buffer offsets
     DotArgs p;
     p.words = q.words; p.scales = q.scales; p.zeros = q.zeros; p.a = q.a; p.bias = q.bias; p.out = q.out;
     p.m = q.m; p.n = q.n; p.k = q.k; p.kp = q.kp; p.act = q.act;
-    p.nslice = p.spw = p.ntiles = 0;
-    const int grid = (int)fnn_ctx_option(ctx, FNN_OPT_GEMV_GRID);
+    p.nslice = p.ntiles = 0;
+    // Row tiles (of 16 weight rows) per workgroup: a workgroup converts the activation rows once for all of its tiles,
+    // and the workgroups should come in whole rounds over the 256 CUs: cost ~ rounds * (rows to convert + tiles).
+    // Measured on N = 11008, K = 4096 (I4): M = 1 6.8 / 7.7 / 6.8 us with 1 / 2 / 3 tiles, M = 2 8.0 / 8.3 / 6.8,
+    // M = 4 10.4 / 9.5 / 7.5; on N = 4096 one tile (256 workgroups) is best for every M.
+    int rt = (int)fnn_ctx_option(ctx, FNN_OPT_GEMV_ROW_TILES);
+    if (rt == 0) {
+        const int mm = q.m <= 1 ? 1 : (q.m <= 2 ? 2 : 4);
+        const int nw = q.k <= 4 * SL ? 4 : 8;
+        int64_t best = -1;
+        for (int c = 1; c <= 3; c++) {
+            if (mm * 16 * c > nw * 64) break;   // one output per thread in the epilogue
+            const int64_t wgs = (q.n + 16 * c - 1) / (16 * c);
+            const int64_t cost = ((wgs + 255) / 256) * (mm + c);
+            if (best < 0 || cost < best) { best = cost; rt = c; }
+        }
+    }
     hipError_t e;
     switch (w->dtype) {
-    case FNN_DT_I8: e = launch_dt<FNN_DT_I8>(p, grid, s, handled); break;
-    case FNN_DT_I4: e = launch_dt<FNN_DT_I4>(p, grid, s, handled); break;
-    default: e = launch_dt<FNN_DT_U4>(p, grid, s, handled); break;
+    case FNN_DT_I8: e = launch_dt<FNN_DT_I8>(p, rt, s, handled); break;
+    case FNN_DT_I4: e = launch_dt<FNN_DT_I4>(p, rt, s, handled); break;
+    default: e = launch_dt<FNN_DT_U4>(p, rt, s, handled); break;
     }
     if (e != hipSuccess) { *handled = false; return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, hipGetErrorString(e)); }
     return FNN_OK;

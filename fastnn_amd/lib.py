@@ -31,7 +31,6 @@ OPT_TILE_SPLIT = 6
 OPT_TILE_STAGES = 7
 OPT_TILE_MIN_M = 8
 OPT_GEMV_INT8 = 9
-OPT_GEMV_GRID = 10
 
 STATUS_NAMES = {0: "Ok", 1: "Dispatch", 2: "Memory", 3: "UnsupportedOp", 4: "Compilation"}
 

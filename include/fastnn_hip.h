@@ -89,18 +89,17 @@ int fnn_hip_download(fnn_hip_ctx *ctx, void *dst_host, const void *src_dev, size
 enum {
     FNN_OPT_CODEBOOK_CACHE = 1,   /* 1 (default): a codebook weight keeps its f16 expansion (8x the packed bytes)   */
                                   /* after its first MatMul with M >= 5; 0: a call expands into a workspace         */
-    FNN_OPT_GEMV_ROW_TILES = 2,   /* M <= 8 kernel: 16-row tiles per workgroup, 1..3; 0 (default) = cost model      */
+    FNN_OPT_GEMV_ROW_TILES = 2,   /* M <= 8 kernels: 16-row tiles per workgroup, 1..3; 0 (default) = cost model     */
     FNN_OPT_ROWS16_ROW_TILES = 3, /* 9 <= M <= 16 kernel: the same                                                  */
     FNN_OPT_ROWS16_MIN_M = 4,     /* smallest M the 16-row kernel takes (default 9; 17 switches it off)             */
     FNN_OPT_TILE_SHAPE = 5,       /* tiled GEMM: 0 = 128x128, 1 = 64x128, 2 = 32x128; -1 (default) = by shape       */
     FNN_OPT_TILE_SPLIT = 6,       /* tiled GEMM: K split over this many workgroups; 0 (default) = cost model        */
     FNN_OPT_TILE_STAGES = 7,      /* tiled GEMM, 128x128 tiles: 5 = deep ring, 3 = shallow; 0 (default) = by shape  */
     FNN_OPT_TILE_MIN_M = 8,       /* smallest M the tiled GEMM takes (default 5)                                    */
-    FNN_OPT_GEMV_INT8 = 9,        /* 1: M <= 4 with I8 / I4 / U4 weights runs on the int8 matrix cores (activations as  */
-                                  /* four exact base-256 digit rows, integer sums: agreement ~1e-6 instead of 2e-5);   */
-                                  /* 0 (default): the f16 GEMV kernel, which measures 0 to 15 % faster                 */
-    FNN_OPT_GEMV_GRID = 10,       /* workgroups of the int8 GEMV kernel; 0 (default) = one per CU                      */
-    FNN_OPT_COUNT = 11
+    FNN_OPT_GEMV_INT8 = 9,        /* 1 (default): M <= 4 with I8 / I4 / U4 weights runs on the int8 matrix cores        */
+                                  /* (activations as four exact base-256 digit rows, integer sums, no weight decode);  */
+                                  /* 0: the f16 GEMV kernel takes them too                                             */
+    FNN_OPT_COUNT = 10
 };
 int fnn_hip_set_option(fnn_hip_ctx *ctx, int option, int64_t value);
 int fnn_hip_get_option(fnn_hip_ctx *ctx, int option, int64_t *value);

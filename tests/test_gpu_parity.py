@@ -133,12 +133,12 @@ def test_qmatmul_matches_oracle(ctx, orc, dt, m, k, n):
     assert_close(gen, want, TOL_F32, f"generic {NAMES[dt]} {m}x{k}x{n}")
     fma = ctx.qmatmul(h, a, n, flags=flib.FLAG_PREFER_FMA)
     assert_close(fma, want, TOL_F32, f"fma {NAMES[dt]} {m}x{k}x{n}")
-    if dt in (0, 1, 3) and m <= 4:     # the int8 matrix-core GEMV takes these when asked
-        ctx.set_option(flib.OPT_GEMV_INT8, 1)
+    if dt in (0, 1, 3) and m <= 4:     # default route: int8 matrix cores; the f16 GEMV kernel takes them when asked
+        ctx.set_option(flib.OPT_GEMV_INT8, 0)
         try:
-            assert_close(ctx.qmatmul(h, a, n), want, TOL_F32, f"int8 gemv {NAMES[dt]} {m}x{k}x{n}")
+            assert_close(ctx.qmatmul(h, a, n), want, TOL_F32, f"f16 gemv {NAMES[dt]} {m}x{k}x{n}")
         finally:
-            ctx.set_option(flib.OPT_GEMV_INT8, 0)
+            ctx.set_option(flib.OPT_GEMV_INT8, 1)
     # the reference's own f32 summation orders sit inside the same band
     assert rel_err(orc.qmatmul(to_oracle(orc, pw), a, order=1), want) <= TOL_F32 * 5
     ctx.release(h)
@@ -161,8 +161,8 @@ def test_qmatmul_row_tile_kernels(ctx, orc, dt, m, k, n):
     ctx.release(h)
 
 
-# int8 GEMV: several row tiles per workgroup (more than 256 tiles), partial last slice, two slices per wave (K > 4096),
-# four-wave workgroups (K <= 2048), a single tile, every row count
+# int8 GEMV: wide N, partial last slice, two slices per wave (K > 4096), four-wave workgroups (K <= 2048), a single
+# tile, ragged N, every row count
 INT8_GEMV_SHAPES = [(1, 4096, 8500), (2, 1024, 8500), (3, 520, 4200), (4, 8200, 72), (1, 2048, 16), (4, 4096, 4400), (1, 11008, 4096),
                     (2, 64, 40)]
 
@@ -170,10 +170,10 @@ INT8_GEMV_SHAPES = [(1, 4096, 8500), (2, 1024, 8500), (3, 520, 4200), (4, 8200, 
 @pytest.mark.parametrize("dt", [0, 1, 3])
 @pytest.mark.parametrize("m,k,n", INT8_GEMV_SHAPES)
 def test_int8_gemv_kernel(ctx, orc, dt, m, k, n):
-    """M <= 4 with I8 / I4 / U4 weights on the int8 matrix cores (FNN_OPT_GEMV_INT8): the activations enter as four
+    """M <= 4 with I8 / I4 / U4 weights on the int8 matrix cores (the default for these weights): the activations enter as four
     exact base-256 digits (30 bits below the maximum of their 512 k-values) and the sums are exact integers, so the
     result sits well inside the 2e-5 MatMul bound (asserted: 4e-6 of max|ref|, measured 4e-8 .. 2e-6); bias + SiLU
-    epilogue; other grids walk the row tiles differently and must give the same bits."""
+    epilogue."""
     rng = np.random.default_rng(3700 + dt * 13 + m + k)
     pw = fastnn_amd.quantize_weights(dt, _weights(rng, n, k))
     a = rng.standard_normal((m, k)).astype(np.float32)
@@ -181,16 +181,15 @@ def test_int8_gemv_kernel(ctx, orc, dt, m, k, n):
     bias = (rng.standard_normal(n) * 0.01).astype(np.float32)
     h = ctx.register(pw)
     want = orc.qmatmul(to_oracle(orc, pw), a, order=2, bias=bias, act=3)
-    ctx.set_option(flib.OPT_GEMV_INT8, 1)
+    got = ctx.qmatmul(h, a, n, bias=bias, act=3)
+    assert_close(got, want, 4e-6, f"int8 gemv {NAMES[dt]} {m}x{k}x{n}")
     try:
-        got = ctx.qmatmul(h, a, n, bias=bias, act=3)
-        assert_close(got, want, 4e-6, f"int8 gemv {NAMES[dt]} {m}x{k}x{n}")
-        for grid in (7, 1000):
-            ctx.set_option(flib.OPT_GEMV_GRID, grid)
-            assert np.array_equal(ctx.qmatmul(h, a, n, bias=bias, act=3), got), f"grid {grid}"
+        for rt in (1, 2, 3):               # any number of row tiles per workgroup gives the same bits
+            ctx.set_option(flib.OPT_GEMV_ROW_TILES, rt)
+            assert np.array_equal(ctx.qmatmul(h, a, n, bias=bias, act=3), got), f"{rt} row tiles"
     finally:
-        ctx.set_option(flib.OPT_GEMV_GRID, 0)
-        ctx.set_option(flib.OPT_GEMV_INT8, 0)
+        ctx.set_option(flib.OPT_GEMV_ROW_TILES, 0)
+        ctx.set_option(flib.OPT_GEMV_INT8, 1)
     ctx.release(h)
 
 
@@ -202,14 +201,10 @@ def test_int8_gemv_propagates_non_finite_activations(ctx, orc):
     pw = fastnn_amd.quantize_weights(flib.DT_I8, _weights(rng, n, k))
     a = rng.standard_normal((m, k)).astype(np.float32)
     h = ctx.register(pw)
-    ctx.set_option(flib.OPT_GEMV_INT8, 1)
-    try:
-        clean = ctx.qmatmul(h, a, n)
-        a[0, 700] = np.nan
-        a[2, 3] = np.inf
-        got = ctx.qmatmul(h, a, n)
-    finally:
-        ctx.set_option(flib.OPT_GEMV_INT8, 0)
+    clean = ctx.qmatmul(h, a, n)
+    a[0, 700] = np.nan
+    a[2, 3] = np.inf
+    got = ctx.qmatmul(h, a, n)
     assert np.isnan(got[0]).all() and np.isnan(got[2]).all()
     assert np.array_equal(got[1], clean[1])
     ctx.release(h)
