@@ -494,6 +494,9 @@ def main() -> int:
     ap.add_argument("--fast-act16", action="store_true", help="single f16 rounding of activations on the MFMA path")
     ap.add_argument("--no-extra", "--no-m256", dest="no_extra", action="store_true",
                     help="skip the extra legs (K=N=4096 GEMVs, M=256 GEMMs)")
+    ap.add_argument("--opt", action="append", default=[], metavar="NAME=VALUE",
+                    help="kernel selection option of the context, e.g. gemv_int8=0 for the f16 matrix-core GEMV "
+                         "(names: the FNN_OPT_* of include/fastnn_hip.h, lower case without the prefix)")
     ap.add_argument("--probe", default="", choices=["", "read", "copy"],
                     help="instead of the MatMul, time a plain streaming read / copy of the same number of bytes "
                          "per launch over the same ring (device ceiling; calibration kernel for byte counters)")
@@ -514,6 +517,15 @@ def main() -> int:
     m = args.m
     flags = flib.FLAG_ACT_F16_SINGLE if args.fast_act16 else 0
     ctx = fastnn_amd.HipContext(0)
+    opts = {}
+    for item in args.opt:
+        name, _, value = item.partition("=")
+        ident = getattr(flib, "OPT_" + name.strip().upper(), None)
+        if ident is None or not value.strip().lstrip("-").isdigit():
+            print(f"bench.py: unknown option {item!r}", file=sys.stderr)
+            return 2
+        ctx.set_option(ident, int(value))
+        opts[name.strip().lower()] = int(value)
     probe = Probe(ctx)
     r = make_ring(ctx, fastnn_amd, flib, args.workload, args.ring)
     dtn, k, n, wbytes, ring = r["dtn"], r["k"], r["n"], r["wbytes"], r["ring"]
@@ -629,7 +641,8 @@ def main() -> int:
         "config": {"workload": f"{args.workload}: {dtn} weights [N={n},K={k}] per-channel, f32 activations "
                                f"[M={m},K={k}] ~N(0,1), bias={has_bias}, act={r['actn']}, seed 0",
                    "m": m, "k": k, "n": n, "weight_ring": ring, "ring_bytes": ring * wbytes, "trips": t["trips"],
-                   "launch": args.mode, "act_rounding": "f16x1" if args.fast_act16 else "default"},
+                   "launch": args.mode, "act_rounding": "f16x1" if args.fast_act16 else "default",
+                   **({"options": opts} if opts else {})},
         "roofline": roofline,
         "cpu_baseline": cpu,
         "gemv_4096": gemv_4096,
