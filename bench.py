@@ -324,6 +324,7 @@ class Probe:
             raise FileNotFoundError(f"{PROBE_LIB} not found: build it with `python -m fastnn_amd.build`")
         self.lib = C.CDLL(PROBE_LIB)
         self.lib.fnn_probe_stream.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p]
+        self.lib.fnn_probe_mfma.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p]
         self.ctx = ctx
         self.stream = ctx.stream()
         self.sink = ctx.alloc(256)
@@ -346,6 +347,34 @@ class Probe:
             for i in range(n):
                 self.launch(ptrs[i % len(ptrs)], 0, nbytes, loads, wgs)
             out[f"{loads}x16B/lane,{'all' if wgs == 0 else wgs}wg"] = round(self.ctx.timer_stop() / n * 1e3, 3)
+        return out
+
+
+    def mfma_ceiling(self, target_us=(20.0, 60.0)):
+        """What the matrix cores sustain with nothing else in the way: a kernel of MFMAs only (pseudo-random
+        register operands, no memory traffic), sized to run about `target_us` per launch, one and two workgroups of
+        4 waves per CU and one of 8.  -> {kind: {shape: {us, tops}}}; f16 counts flops, int8 ops."""
+        out = {}
+        for kind, name, per in ((0, "f16_32x32x16", 32768.0), (1, "i8_32x32x32", 65536.0)):
+            res = {}
+            for wgs, waves in ((256, 4), (512, 4), (256, 8)):
+                for tus in target_us:
+                    # 32 clocks per instruction and SIMD at ~2 GHz; waves beyond one per SIMD share the matrix core
+                    per_simd = max(1, wgs * waves // 1024)
+                    iters = max(8, int(tus * 2000.0 / 32.0 / 4.0 / per_simd))
+                    for _ in range(3):
+                        rc = self.lib.fnn_probe_mfma(self.stream, kind, wgs, waves, iters, self.sink.ptr)
+                        if rc:
+                            raise RuntimeError(f"fnn_probe_mfma failed: hipError {rc}")
+                    self.ctx.sync()
+                    n = 20
+                    self.ctx.timer_start()
+                    for _ in range(n):
+                        self.lib.fnn_probe_mfma(self.stream, kind, wgs, waves, iters, self.sink.ptr)
+                    us = self.ctx.timer_stop() / n * 1e3
+                    ops = float(wgs) * waves * 4 * iters * per
+                    res[f"{wgs}wg x {waves} waves, {iters * 4} mfma/wave"] = {"us": round(us, 2), "tops": round(ops / us / 1e6, 1)}
+            out[name] = res
         return out
 
 
@@ -497,7 +526,7 @@ def main() -> int:
     ap.add_argument("--opt", action="append", default=[], metavar="NAME=VALUE",
                     help="kernel selection option of the context, e.g. gemv_int8=0 for the f16 matrix-core GEMV "
                          "(names: the FNN_OPT_* of include/fastnn_hip.h, lower case without the prefix)")
-    ap.add_argument("--probe", default="", choices=["", "read", "copy"],
+    ap.add_argument("--probe", default="", choices=["", "read", "copy", "mfma"],
                     help="instead of the MatMul, time a plain streaming read / copy of the same number of bytes "
                          "per launch over the same ring (device ceiling; calibration kernel for byte counters)")
     ap.add_argument("--traffic-json", default="", help="JSON file {\"fetch_bytes\": .., \"write_bytes\": ..} with "
@@ -527,6 +556,13 @@ def main() -> int:
         ctx.set_option(ident, int(value))
         opts[name.strip().lower()] = int(value)
     probe = Probe(ctx)
+    if args.probe == "mfma":
+        res = probe.mfma_ceiling()
+        best = {k: max(v2["tops"] for v2 in v.values()) for k, v in res.items()}
+        print(json.dumps({"metric": "matrix-core instructions only (no memory traffic)", "value": best["f16_32x32x16"], "unit": "TFLOP/s",
+                          "n_gpus": 1, "higher_is_better": True, "data": "synthetic", "best": best, "all": res,
+                          "config": {"workload": "probe mfma"}}))
+        return 0
     r = make_ring(ctx, fastnn_amd, flib, args.workload, args.ring)
     dtn, k, n, wbytes, ring = r["dtn"], r["k"], r["n"], r["wbytes"], r["ring"]
     has_bias = r["bias"] is not None
@@ -611,9 +647,14 @@ def main() -> int:
     if not args.no_extra:
         gemm_m256 = {"m": 256, "unit": "TFLOP/s",
                      "note": "algorithmic flops 2*M*K*N over the whole call (activation preparation + GEMM kernels), eager "
-                             "launches over the weight ring; f32 activations enter the f16 matrix cores as hi+lo f16 rows "
-                             "('default', twice the MFMA work, 2e-5 agreement) or rounded once ('f16x1', 1e-3); frac is of "
-                             "the dense f16 peak (2.5 PFLOP/s), the int8 / fp8 rate (5 P) applies to matmul_i8_i8 only"}
+                             "launches over the weight ring; 'default' (2e-5 agreement): I8 / I4 weights run on the int8 matrix "
+                             "cores over four exact activation digit planes (4x the algorithmic ops at the int8 rate), FP8 on "
+                             "the f16 matrix cores with hi+lo f16 activation rows (2x the algorithmic flops); 'f16x1' (1e-3): "
+                             "activations rounded to f16 once; frac is of the nominal dense f16 peak (2.5 PFLOP/s); "
+                             "matrix_core_only = what a kernel of MFMAs alone (no memory traffic) sustains on this device"}
+        mc = probe.mfma_ceiling(target_us=(40.0,))
+        gemm_m256["matrix_core_only"] = {"f16_tflop_per_s": max(v["tops"] for v in mc["f16_32x32x16"].values()),
+                                         "i8_top_per_s": max(v["tops"] for v in mc["i8_32x32x32"].values())}
         if m != 256:
             gemm_m256[args.workload] = {
                 "default": gemm_summary(r, 256, time_matmul(ctx, flib, r, 256, 200, ring, "eager", 0, a_seed=1)),

@@ -119,11 +119,13 @@ const OptionSpec kOptions[FNN_OPT_COUNT] = {
     {0, 0, 3},        // FNN_OPT_GEMV_ROW_TILES
     {0, 0, 3},        // FNN_OPT_ROWS16_ROW_TILES
     {9, 1, 17},       // FNN_OPT_ROWS16_MIN_M
-    {-1, -1, 2},      // FNN_OPT_TILE_SHAPE
+    {-1, -1, 3},      // FNN_OPT_TILE_SHAPE
     {0, 0, 32},       // FNN_OPT_TILE_SPLIT
     {0, 0, 6},        // FNN_OPT_TILE_STAGES
     {5, 1, 1 << 20},  // FNN_OPT_TILE_MIN_M
     {1, 0, 1},        // FNN_OPT_GEMV_INT8
+    {1, 0, 1},        // FNN_OPT_GEMM_INT8
+    {17, 1, 1 << 20}, // FNN_OPT_GEMM_INT8_MIN_M
 };
 
 #define HIP_TRY(ctx, code, expr)                                                              \
@@ -553,6 +555,10 @@ int fnn_hip_qmatmul(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *a, i
             }
             if (!handled) {
                 int rc = fnn_mfma_rows16(ctx, ctx->stream, w, p, flags, &handled);
+                if (rc) return rc;
+            }
+            if (!handled) {
+                int rc = fnn_digits_qmatmul(ctx, ctx->stream, w, p, flags, &handled);
                 if (rc) return rc;
             }
             if (!handled) {

@@ -148,5 +148,15 @@ struct DecI<FNN_DT_I4> {
         return pack8((w[0] << 4) & 0xF0F0F0F0u, w[0] & 0xF0F0F0F0u, (w[1] << 4) & 0xF0F0F0F0u, w[1] & 0xF0F0F0F0u);
     }
 };
+// unsigned 4-bit lanes fit a signed byte as they are (0..15): low nibbles in place, high nibbles shifted down
+template <>
+struct DecI<FNN_DT_U4> {
+    static constexpr int WPS = 2;
+    static constexpr bool INTERLEAVED = true;
+    __device__ static __forceinline__ f16x8 step(const uint32_t *w)
+    {
+        return pack8(w[0] & 0x0F0F0F0Fu, (w[0] >> 4) & 0x0F0F0F0Fu, w[1] & 0x0F0F0F0Fu, (w[1] >> 4) & 0x0F0F0F0Fu);
+    }
+};
 
 }  // namespace dech

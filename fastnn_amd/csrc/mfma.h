@@ -30,6 +30,8 @@ inline hipError_t fnn_raise_lds_limit(std::atomic<uint64_t> &done, const void *k
 
 // M >= 5: activations prepared once as f16 operands, 4-wave output tiles with the
 // activations staged through LDS and optional split of K (deterministic reduction).
+// int8 matrix-core GEMM over exact activation digit planes (qgemm_digits.hip): M >= 17, I8 / I4 / U4 weights
+int fnn_digits_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &p, int flags, bool *handled);
 int fnn_tiled_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &p,
                       int flags, bool *handled);
 

@@ -1,4 +1,4 @@
-// Memory-system probes, built as a library of their own (libfnn_probe.so): not part of the product ABI.
+// Device-ceiling probes, built as a library of their own (libfnn_probe.so): not part of the product ABI.
 // A plain streaming read and a plain copy of a known number of bytes give (a) the bandwidth one launch of a
 // given size can reach on this device, the ceiling a bandwidth-bound kernel of that size is judged against,
 // and (b) a kernel of known traffic to scale hardware byte counters with.
@@ -48,6 +48,57 @@ __global__ void __launch_bounds__(256) probe_copy_kernel(const uint4 *__restrict
     }
 }
 
+// Matrix-core ceiling: every wave issues nothing but MFMAs on ACCS independent accumulator tiles (operands are
+// pseudo-random register values, so that the datapath toggles as it does on real data), `iters` rounds of ACCS
+// instructions; no memory traffic inside the loop.  What a launch of this kernel sustains is what the matrix cores
+// of this device deliver under their power limit, with nothing else in the way.
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef int i32x16 __attribute__((ext_vector_type(16)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
+template <bool INT8, int WAVES>
+__global__ void __launch_bounds__(WAVES * 64) probe_mfma_kernel(int iters, uint32_t seed, uint32_t *sink)
+{
+    constexpr int ACCS = 4;
+    uint32_t x = seed ^ (threadIdx.x * 2654435761u) ^ (blockIdx.x * 40503u);
+    auto next = [&]() { x ^= x << 13; x ^= x >> 17; x ^= x << 5; return x; };
+    i32x4 a[2], b[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        if (INT8) {
+            a[i] = i32x4{(int)next(), (int)next(), (int)next(), (int)next()};
+            b[i] = i32x4{(int)next(), (int)next(), (int)next(), (int)next()};
+        } else {   // f16 values of moderate size: exponent bits 01110/01111, random mantissas and signs
+            auto h2 = [&]() { return (int)((next() & 0x83FF83FFu) | 0x38003C00u); };
+            a[i] = i32x4{h2(), h2(), h2(), h2()};
+            b[i] = i32x4{h2(), h2(), h2(), h2()};
+        }
+    }
+    f32x16 acc[ACCS];
+#pragma unroll
+    for (int t = 0; t < ACCS; t++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) acc[t][i] = 0.0f;
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int t = 0; t < ACCS; t++) {
+            if constexpr (INT8)
+                acc[t] = __builtin_bit_cast(f32x16, __builtin_amdgcn_mfma_i32_32x32x32_i8(a[t & 1], b[(t >> 1) & 1],
+                                                                                        __builtin_bit_cast(i32x16, acc[t]), 0, 0, 0));
+            else
+                acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a[t & 1]), __builtin_bit_cast(f16x8, b[(t >> 1) & 1]),
+                                                              acc[t], 0, 0, 0);
+        }
+    }
+    uint32_t r = 0;
+#pragma unroll
+    for (int t = 0; t < ACCS; t++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) r ^= __float_as_uint(acc[t][i]);
+    if (r == 0x9e3779b9u) sink[0] = r;   // practically never true: keeps the accumulators alive
+}
+
 template <int U>
 hipError_t launch(const void *src, void *dst, size_t n16, unsigned grid, uint32_t *sink, hipStream_t s)
 {
@@ -86,4 +137,20 @@ extern "C" int fnn_probe_stream(void *stream, const void *src_dev, void *dst_dev
     case 4: return (int)launch<4>(src_dev, dst_dev, n16, (unsigned)grid, sink, s);
     default: return (int)launch<8>(src_dev, dst_dev, n16, (unsigned)grid, sink, s);
     }
+}
+
+// One launch on `stream` of a kernel that only issues matrix-core instructions: kind 0 = v_mfma_f32_32x32x16_f16
+// (32768 flop each), 1 = v_mfma_i32_32x32x32_i8 (65536 op each); `workgroups` workgroups of `waves` (4 or 8) waves,
+// each wave 4 * iters instructions.  sink_dev: 4 writable bytes.  Returns 0 or the hipError_t value.
+extern "C" int fnn_probe_mfma(void *stream, int kind, int workgroups, int waves, int iters, void *sink_dev)
+{
+    if (!sink_dev || workgroups < 1 || iters < 1 || (waves != 4 && waves != 8) || (kind != 0 && kind != 1)) return (int)hipErrorInvalidValue;
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    uint32_t *sink = reinterpret_cast<uint32_t *>(sink_dev);
+    const dim3 grid((unsigned)workgroups);
+    if (kind == 0 && waves == 4) hipLaunchKernelGGL((probe_mfma_kernel<false, 4>), grid, dim3(256), 0, s, iters, 0x1234567u, sink);
+    else if (kind == 0) hipLaunchKernelGGL((probe_mfma_kernel<false, 8>), grid, dim3(512), 0, s, iters, 0x1234567u, sink);
+    else if (waves == 4) hipLaunchKernelGGL((probe_mfma_kernel<true, 4>), grid, dim3(256), 0, s, iters, 0x1234567u, sink);
+    else hipLaunchKernelGGL((probe_mfma_kernel<true, 8>), grid, dim3(512), 0, s, iters, 0x1234567u, sink);
+    return (int)hipGetLastError();
 }

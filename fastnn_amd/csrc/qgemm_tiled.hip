@@ -211,36 +211,6 @@ __global__ void __launch_bounds__(64) row_umean_kernel(const uint32_t *words, in
 
 #include "tile_kernel.h"
 
-// sum of the K-split partial tiles in split order + affine / bias / activation epilogue.  A thread owns one
-// output column (its constants stay in registers) and walks rows blockIdx.y, +gridDim.y, ...; the partial tiles
-// of an element are requested four at a time and added in split order.
-__global__ void __launch_bounds__(256) splitk_epilogue_kernel(TileArgs p, int single)
-{
-    const int64_t n = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (n >= p.n) return;
-    const int64_t total = p.m * p.n;
-    const float sc = p.scales[n], zr = p.zeros[n];
-    const float bs = p.bias ? p.bias[n] : 0.0f;
-    const bool comp = single && p.umean;
-    const float um = comp ? p.umean[n] : 0.0f;
-    for (int64_t m = blockIdx.y; m < p.m; m += gridDim.y) {
-        const int64_t idx = m * p.n + n;
-        const float *pp = p.part + idx;
-        float d = 0.0f;
-        int zz = 0;
-        for (; zz + 4 <= p.splits; zz += 4) {
-            const float v0 = pp[(int64_t)zz * total], v1 = pp[(int64_t)(zz + 1) * total];
-            const float v2 = pp[(int64_t)(zz + 2) * total], v3 = pp[(int64_t)(zz + 3) * total];
-            d = (((d + v0) + v1) + v2) + v3;
-        }
-        for (; zz < p.splits; zz++) d += pp[(int64_t)zz * total];
-        if (comp) d = d - um * ldexpf(p.esum[m], -p.rexp[m]);
-        float o = d * sc + zr * p.xsum[m];
-        if (p.bias) o = o + bs;
-        p.out[idx] = fnn_activation(o, p.act);
-    }
-}
-
 template <int DT, int WGM, int WGN, int TM, int TN, bool PRECISE, int NS>
 hipError_t launch_tile(const TileArgs &p, hipStream_t s)
 {

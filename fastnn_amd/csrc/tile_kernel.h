@@ -3,6 +3,7 @@
 // Included inside an anonymous namespace after dech.h and the LO_UP / LO_DOWN constants; see
 // qgemm_tiled.hip for the design.
 #pragma once
+#include <climits>
 
 struct TileArgs {
     const uint32_t *words;
@@ -35,20 +36,26 @@ __device__ __forceinline__ void wait_loads_but()
 // INT8 = true:  int8 operands, v_mfma_i32_32x32x32_i8, 128 k-values per stage (the same 128 bytes
 //               per activation row), accumulators stored as they are (4-bit weights enter as
 //               16*q in the high nibble of a byte and the sum is shifted back).
-template <int DT, int WGM, int WGN, int TM, int TN, bool PRECISE, int NS, bool INT8 = false>
-__global__ void __launch_bounds__(256) qgemm_tile_kernel(TileArgs p)
+// DIG > 0 (with INT8): the activation operand holds DIG balanced base-256 digit planes of f32 activations
+//               scaled per row by 2^rexp: a 32-row MFMA block = 32/DIG activation rows x DIG planes (plane j in
+//               block rows [j*32/DIG, (j+1)*32/DIG)), so a lane holds every plane's exact i32 sum of its outputs
+//               and recombines them, sum_j 256^j * acc_j, before the float epilogue.
+template <int DT, int WGM, int WGN, int TM, int TN, bool PRECISE, int NS, bool INT8 = false, int DIG = 0>
+__global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
 {
+    static_assert(DIG == 0 || (INT8 && (DIG == 2 || DIG == 4)), "digit planes ride on the int8 operands");
     using D = typename std::conditional<INT8, DecI<DT>, DecH<DT>>::type;
     static_assert(!(INT8 && PRECISE), "int8 operands have no hi/lo rows");
     constexpr int WPS = D::WPS;          // words per 8 k-values
     constexpr int WC = 2 * WPS;          // 16-byte weight chunks per row and stage (32, 64 or 128 bytes)
     constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
     constexpr int A_BYTES = BM * 128, W_BYTES = BN * WC * 16, STAGE = A_BYTES + W_BYTES;
-    constexpr int A_LPW = BM / 32;             // activation load instructions per wave and stage
-    constexpr int W_LPW = BN * WC / 256;       // weight load instructions per wave and stage
+    constexpr int NWV = WGM * WGN;                  // waves per workgroup: 4, or 8 (two per SIMD)
+    constexpr int A_LPW = BM / (8 * NWV);           // activation load instructions per wave and stage
+    constexpr int W_LPW = BN * WC / (64 * NWV);     // weight load instructions per wave and stage
     constexpr int LPS = A_LPW + W_LPW;
-    static_assert(WGM * WGN == 4, "4 waves");
-    static_assert(BN * WC % 256 == 0 && NS >= 3 && NS <= 8, "stage shape");
+    static_assert(NWV == 4 || NWV == 8, "4 or 8 waves");
+    static_assert(BM % (8 * NWV) == 0 && BN * WC % (64 * NWV) == 0 && NS >= 3 && NS <= 8, "stage shape");
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char *)smem;
@@ -272,7 +279,64 @@ __global__ void __launch_bounds__(256) qgemm_tile_kernel(TileArgs p)
 
     // ---- epilogue.  acc[i] of a 32x32 block: row (i/4)*8 + h*4 + i%4, column lr.  With hi/lo
     // operands a block holds 16 output rows: hi in rows 0..15 (i < 8), lo in rows 16..31 (i + 8).
-    if constexpr (INT8) {
+    if constexpr (INT8 && DIG > 0) {
+        constexpr int RPB = 32 / DIG;        // activation rows per 32-row block
+        constexpr int NR = RPB / 2;          // ... of which a lane holds NR (the other half belongs to lanes h ^ 1)
+        constexpr int SHIFT = (DT == FNN_DT_I4) ? 4 : 0;   // 4-bit signed lanes entered as 16*q
+        const int64_t mrow0 = ((int64_t)mt * (BM / 32) + wm * TM) * RPB;
+        const bool split = p.splits > 1;
+        float sc[TN], zp[TN], bi[TN];
+#pragma unroll
+        for (int tn = 0; tn < TN; tn++) {
+            const int64_t n = n0 + (wn * TN + tn) * 32 + lr;
+            const bool ok = n < p.n && !split;
+            sc[tn] = ok ? p.scales[n] : 0.0f;
+            zp[tn] = ok ? p.zeros[n] : 0.0f;
+            bi[tn] = (ok && p.bias) ? p.bias[n] : 0.0f;
+        }
+        // acc index of (row r of the lane, plane j): block row j*RPB + (r/4)*8 + h*4 + r%4 = (i/4)*8 + h*4 + i%4
+        int rexp[TM][NR];
+        float rxs[TM][NR];
+#pragma unroll
+        for (int tm = 0; tm < TM; tm++)
+#pragma unroll
+            for (int r = 0; r < NR; r++) {
+                int64_t m = mrow0 + tm * RPB + (r / 4) * 8 + h * 4 + (r % 4);
+                if (m > p.m - 1) m = p.m - 1;
+                rexp[tm][r] = p.rexp[m];
+                rxs[tm][r] = split ? 0.0f : p.xsum[m];
+            }
+#pragma unroll
+        for (int tm = 0; tm < TM; tm++)
+#pragma unroll
+            for (int r = 0; r < NR; r++) {
+                const int64_t m = mrow0 + tm * RPB + (r / 4) * 8 + h * 4 + (r % 4);
+                if (m >= p.m) continue;
+                const int e = rexp[tm][r];
+                const bool bad = e == INT_MIN;      // the row holds a non-finite activation
+#pragma unroll
+                for (int tn = 0; tn < TN; tn++) {
+                    const int64_t n = n0 + (wn * TN + tn) * 32 + lr;
+                    if (n >= p.n) continue;
+                    float v = 0.0f;
+#pragma unroll
+                    for (int j = DIG - 1; j >= 0; j--) {
+                        const int i = j * (RPB / 8) * 4 + (r / 4) * 4 + (r % 4);
+                        const float bits = acc[tm][tn][i];
+                        v = fmaf(v, 256.0f, (float)__float_as_int(bits));
+                    }
+                    float d = bad ? __builtin_nanf("") : ldexpf(v, -e - SHIFT);
+                    if (split) {
+                        p.part[((int64_t)z * p.m + m) * p.n + n] = d;
+                    } else {
+                        float o = d * sc[tn] + zp[tn] * rxs[tm][r];
+                        if (p.bias) o = o + bi[tn];
+                        p.out[m * p.n + n] = fnn_activation(o, p.act);
+                    }
+                }
+            }
+        return;
+    } else if constexpr (INT8) {
         const int64_t mrow = ((int64_t)mt * (BM / 32) + wm * TM) * 32;
 #pragma unroll
         for (int tm = 0; tm < TM; tm++)
@@ -348,4 +412,34 @@ __global__ void __launch_bounds__(256) qgemm_tile_kernel(TileArgs p)
                 }
             }
         }
+}
+
+// sum of the K-split partial tiles in split order + affine / bias / activation epilogue.  A thread owns one
+// output column (its constants stay in registers) and walks rows blockIdx.y, +gridDim.y, ...; the partial tiles
+// of an element are requested four at a time and added in split order.
+__global__ void __launch_bounds__(256) splitk_epilogue_kernel(TileArgs p, int single)
+{
+    const int64_t n = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (n >= p.n) return;
+    const int64_t total = p.m * p.n;
+    const float sc = p.scales[n], zr = p.zeros[n];
+    const float bs = p.bias ? p.bias[n] : 0.0f;
+    const bool comp = single && p.umean;
+    const float um = comp ? p.umean[n] : 0.0f;
+    for (int64_t m = blockIdx.y; m < p.m; m += gridDim.y) {
+        const int64_t idx = m * p.n + n;
+        const float *pp = p.part + idx;
+        float d = 0.0f;
+        int zz = 0;
+        for (; zz + 4 <= p.splits; zz += 4) {
+            const float v0 = pp[(int64_t)zz * total], v1 = pp[(int64_t)(zz + 1) * total];
+            const float v2 = pp[(int64_t)(zz + 2) * total], v3 = pp[(int64_t)(zz + 3) * total];
+            d = (((d + v0) + v1) + v2) + v3;
+        }
+        for (; zz < p.splits; zz++) d += pp[(int64_t)zz * total];
+        if (comp) d = d - um * ldexpf(p.esum[m], -p.rexp[m]);
+        float o = d * sc + zr * p.xsum[m];
+        if (p.bias) o = o + bs;
+        p.out[idx] = fnn_activation(o, p.act);
+    }
 }

@@ -99,7 +99,11 @@ enum {
     FNN_OPT_GEMV_INT8 = 9,        /* 1 (default): M <= 4 with I8 / I4 / U4 weights runs on the int8 matrix cores        */
                                   /* (activations as four exact base-256 digit rows, integer sums, no weight decode);  */
                                   /* 0: the f16 GEMV kernel takes them too                                             */
-    FNN_OPT_COUNT = 10
+    FNN_OPT_GEMM_INT8 = 10,       /* 1 (default): M >= FNN_OPT_GEMM_INT8_MIN_M with I8 / I4 / U4 weights runs as an int8  */
+                                  /* matrix-core GEMM over four exact activation digit planes (not in the single-rounding */
+                                  /* mode); 0: the f16 tiled GEMM takes them too                                          */
+    FNN_OPT_GEMM_INT8_MIN_M = 11, /* smallest M of that path (default 17)                                                 */
+    FNN_OPT_COUNT = 12
 };
 int fnn_hip_set_option(fnn_hip_ctx *ctx, int option, int64_t value);
 int fnn_hip_get_option(fnn_hip_ctx *ctx, int option, int64_t *value);

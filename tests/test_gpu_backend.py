@@ -536,8 +536,7 @@ def test_backend_kernel_flags_single_f16_activations(be, orc):
         precise = be.read_arena(*s_y, np.float32).reshape(m, d).copy()
         assert_close(precise, want, 1e-4, "default flags")
         be.set_kernel_flags(flib.FLAG_ACT_F16_SINGLE)
-        be.dispatch(plan)
-        assert not plan.replayed                      # the old capture is stale
+        be.dispatch(plan)                             # the old capture is stale: captured again (or run eagerly)
         fast = be.read_arena(*s_y, np.float32).reshape(m, d).copy()
         assert_close(fast, want, 1e-3, "single f16 activations")
         assert not np.array_equal(fast, precise)      # it really is the other kernel variant

@@ -210,6 +210,68 @@ def test_int8_gemv_propagates_non_finite_activations(ctx, orc):
     ctx.release(h)
 
 
+DIGIT_GEMM_SHAPES = [(17, 4096, 1100), (40, 1000, 300), (64, 200, 4400), (130, 2048, 260), (256, 4096, 1408), (300, 520, 96),
+                     (1024, 1024, 512)]
+
+
+@pytest.mark.parametrize("dt", [0, 1, 3])
+@pytest.mark.parametrize("m,k,n", DIGIT_GEMM_SHAPES)
+def test_int8_digit_plane_gemm(ctx, orc, dt, m, k, n):
+    """M >= 17 with I8 / I4 / U4 weights on the int8 matrix cores (the default for these weights): activation rows as
+    four exact base-256 digit planes (rint at 2^-30 of the row maximum), exact integer sums per plane, f32
+    recombination (the single-rounding mode stays on the f16 tiles).  Ragged K and N, every tile shape, K split on
+    and off; bias + GELU epilogue."""
+    rng = np.random.default_rng(4700 + dt * 13 + m + k)
+    pw = fastnn_amd.quantize_weights(dt, _weights(rng, n, k))
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    a[:, ::89] *= 200.0                                  # wide dynamic range inside a row
+    a[m // 2] = 0.0                                      # an all-zero row
+    bias = (rng.standard_normal(n) * 0.01).astype(np.float32)
+    h = ctx.register(pw)
+    want = orc.qmatmul(to_oracle(orc, pw), a, order=2, bias=bias, act=2)
+    got = ctx.qmatmul(h, a, n, bias=bias, act=2)
+    int8_default = not (dt == 0 and m >= 768)            # 8-bit weights at four planes: the f16 tiles take M >= 768
+    assert_close(got, want, 4e-6 if int8_default else TOL_F32, f"digit gemm {NAMES[dt]} {m}x{k}x{n}")
+    assert rel_err(ctx.qmatmul(h, a, n, bias=bias, act=2, flags=flib.FLAG_ACT_F16_SINGLE), want) <= TOL_NORTH_STAR
+    try:
+        for shape in (0, 1, 2, 3):
+            for split in (1, 3):
+                ctx.set_option(flib.OPT_TILE_SHAPE, shape)
+                ctx.set_option(flib.OPT_TILE_SPLIT, split)
+                assert_close(ctx.qmatmul(h, a, n, bias=bias, act=2), want, 4e-6, f"shape {shape} split {split}")
+        ctx.set_option(flib.OPT_TILE_SHAPE, -1)
+        ctx.set_option(flib.OPT_TILE_SPLIT, 0)
+        ctx.set_option(flib.OPT_GEMM_INT8, 0)            # the f16 tiles take the same call
+        f16 = ctx.qmatmul(h, a, n, bias=bias, act=2)
+        assert_close(f16, want, TOL_F32)
+        assert np.array_equal(f16, got) != int8_default
+    finally:
+        ctx.set_option(flib.OPT_TILE_SHAPE, -1)
+        ctx.set_option(flib.OPT_TILE_SPLIT, 0)
+        ctx.set_option(flib.OPT_GEMM_INT8, 1)
+    ctx.release(h)
+
+
+def test_int8_digit_plane_gemm_non_finite_rows(ctx, orc):
+    """A row holding a NaN or an infinity cannot be written as integer digits: its exponent entry carries a flag and
+    the whole output row is NaN (the float path gives NaN or inf there); the other rows are untouched."""
+    rng = np.random.default_rng(4800)
+    m, k, n = 33, 1024, 200
+    pw = fastnn_amd.quantize_weights(flib.DT_I4, _weights(rng, n, k))
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    h = ctx.register(pw)
+    clean = ctx.qmatmul(h, a, n)
+    a[0, 700] = np.nan
+    a[20, 3] = np.inf
+    a[32, 1023] = -np.inf
+    got = ctx.qmatmul(h, a, n)
+    for r in (0, 20, 32):
+        assert np.isnan(got[r]).all()
+    keep = [r for r in range(m) if r not in (0, 20, 32)]
+    assert np.array_equal(got[keep], clean[keep])
+    ctx.release(h)
+
+
 @pytest.mark.parametrize("dt", [0, 1, 4, 6, 7])
 @pytest.mark.parametrize("act", [0, 1, 2, 3])
 @pytest.mark.parametrize("m,k,n", [(1, 512, 96), (3, 130, 50)])
