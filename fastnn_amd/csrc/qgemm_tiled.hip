@@ -222,7 +222,7 @@ hipError_t launch_tile(const TileArgs &p, hipStream_t s)
     hipError_t e = fnn_raise_lds_limit(lds_raised, reinterpret_cast<const void *>(kern), (int)lds);
     if (e != hipSuccess) return e;
     const unsigned total = (unsigned)p.mtiles * p.ntiles * p.splits;
-    hipLaunchKernelGGL(kern, dim3(total), dim3(256), lds, s, p);
+    hipLaunchKernelGGL(kern, dim3(total), dim3(WGM * WGN * 64), lds, s, p);
     return hipGetLastError();
 }
 
@@ -257,8 +257,17 @@ int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QM
     else if (meff == 64) cfg = 1;
     else cfg = 2;
     const int64_t opt_cfg = fnn_ctx_option(ctx, FNN_OPT_TILE_SHAPE);
-    if (opt_cfg >= 0 && opt_cfg <= 2) cfg = (int)opt_cfg;
-    const int bm = cfg == 0 ? 128 : (cfg == 1 ? 64 : 32);
+    // 3 (by option only): 256x128 with 8 waves of 64x64, two waves per SIMD.  Measured on FP8 4096 x 4096 and 2048 -> 8192
+    // at M = 128 ... 1024: 0-30 % slower than the automatic choice, except where it turns the tile count into one whole
+    // round (2048 -> 8192, M = 1024, single rounding: 84 -> 57 us).  Deeper rings (8 stages) for the 64- and 32-row
+    // tiles changed nothing either: a wave's HBM -> LDS loads complete at about 3.7 bytes per clock however many are
+    // in flight, so four waves deliver ~15 bytes per clock and CU, eight ~30, twelve ~41.
+    // For 17 <= M <= 128 neither helps: 64 x 256 and 128 x 256 tiles with eight waves side by side along N (every
+    // wave loading) measured 10-40 % slower than the 4-wave tiles at every K split; these calls are bound by their
+    // three dependent launches (activation preparation, tiles, split-K reduction), not by delivery.
+    if (opt_cfg >= 0 && opt_cfg <= 3) cfg = (int)opt_cfg;
+    if (cfg == 3 && (DecH<DT>::WPS < 2 || dense)) cfg = 0;  // (8-bit weights only: a stage of 4-bit rows has too few 16-byte chunks for 8 waves)
+    const int bm = cfg == 3 ? 256 : (cfg == 0 ? 128 : (cfg == 1 ? 64 : 32));
     const int bn = 128;
     const int mtiles = (int)((meff + bm - 1) / bm);
     const int ntiles = (int)((N + bn - 1) / bn);
@@ -274,7 +283,7 @@ int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QM
     const int env_split = (int)fnn_ctx_option(ctx, FNN_OPT_TILE_SPLIT);
     const int base = mtiles * ntiles;
     const double t_bits = DecH<DT>::WPS == 1 ? 0.4 : (DecH<DT>::WPS == 2 ? 0.7 : 1.0);
-    const double t_stage = t_bits * (cfg == 0 ? 1.0 : (cfg == 1 ? 0.5 : 0.25));
+    const double t_stage = t_bits * (cfg == 3 ? 2.0 : (cfg == 0 ? 1.0 : (cfg == 1 ? 0.5 : 0.25)));
     const double part_us = (double)M * (double)N * 8.0 / 3.0e6;
     int splits = 1;
     double best = 1e30;
@@ -340,7 +349,12 @@ int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QM
     t.act = q.act; t.splits = splits; t.iters = iters; t.ips = ips; t.mtiles = mtiles; t.ntiles = ntiles;
     const int env_ns = (int)fnn_ctx_option(ctx, FNN_OPT_TILE_STAGES);
     const bool deep = cfg == 0 && (env_ns == 5 || (env_ns == 0 && base * splits <= 256));
-    if (deep) e = precise ? launch_tile<DT, 2, 2, 2, 2, true, 5>(t, s) : launch_tile<DT, 2, 2, 2, 2, false, 5>(t, s);
+    constexpr int WCX = 2 * DecH<DT>::WPS;
+    if (cfg == 3) {
+        if constexpr (WCX >= 4 && 3 * (256 * 128 + 128 * WCX * 16) <= 160 * 1024)
+            e = precise ? launch_tile<DT, 4, 2, 2, 2, true, 3>(t, s) : launch_tile<DT, 4, 2, 2, 2, false, 3>(t, s);
+        else e = hipErrorInvalidValue;
+    } else if (deep) e = precise ? launch_tile<DT, 2, 2, 2, 2, true, 5>(t, s) : launch_tile<DT, 2, 2, 2, 2, false, 5>(t, s);
     else if (precise) {
         if (cfg == 0) e = launch_tile<DT, 2, 2, 2, 2, true, 3>(t, s);
         else if (cfg == 1) e = launch_tile<DT, 1, 4, 2, 1, true, 4>(t, s);

@@ -26,6 +26,25 @@ __device__ __forceinline__ void load_to_lds16(const void *gptr, unsigned lds_wav
 {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_wave_base), "v"(gptr) : "memory");
 }
+// Up to four such loads behind one M0 write: load i lands at m0 + 1024*i + 16*lane.  The instruction offset moves
+// the LDS address and the memory address alike, so the pointers passed in are biased by -1024*i bytes.
+template <int N>
+__device__ __forceinline__ void load_group_to_lds16(const void *g0, const void *g1, const void *g2, const void *g3, unsigned lds_wave_base)
+{
+    static_assert(N >= 1 && N <= 4, "1..4 loads per M0 value");
+    if constexpr (N == 1)
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_wave_base), "v"(g0) : "memory");
+    else if constexpr (N == 2)
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off\n\tglobal_load_lds_dwordx4 %2, off offset:1024"
+                     ::"s"(lds_wave_base), "v"(g0), "v"(g1) : "memory");
+    else if constexpr (N == 3)
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off\n\tglobal_load_lds_dwordx4 %2, off offset:1024\n\t"
+                     "global_load_lds_dwordx4 %3, off offset:2048" ::"s"(lds_wave_base), "v"(g0), "v"(g1), "v"(g2) : "memory");
+    else
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off\n\tglobal_load_lds_dwordx4 %2, off offset:1024\n\t"
+                     "global_load_lds_dwordx4 %3, off offset:2048\n\tglobal_load_lds_dwordx4 %4, off offset:3072"
+                     ::"s"(lds_wave_base), "v"(g0), "v"(g1), "v"(g2), "v"(g3) : "memory");
+}
 template <int N>
 __device__ __forceinline__ void wait_loads_but()
 {
@@ -85,7 +104,7 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
     for (int j = 0; j < A_LPW; j++) {
         const int slot = (wv * A_LPW + j) * 64 + lane;
         const int row = slot >> 3, g = (slot & 7) ^ ((row >> 1) & 7);
-        a_src[j] = p.ap + ((int64_t)mt * BM + row) * 64 + g * 8;
+        a_src[j] = p.ap + ((int64_t)mt * BM + row) * 64 + g * 8 - (j & 3) * 512;   // (biased: see load_group_to_lds16)
     }
     // weights: chunk (row, c) lives at slot row*WC + (c ^ swz(row)); rows past N repeat the last row
     const uint32_t *w_src[W_LPW];
@@ -98,7 +117,7 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
         const int c = (slot % WC) ^ sw;
         int64_t grow = n0 + row;
         if (grow > p.n - 1) grow = p.n - 1;
-        w_src[j] = p.words + grow * p.kp + c * 4;
+        w_src[j] = p.words + grow * p.kp + c * 4 - (j & 3) * 256;                  // (biased likewise)
         w_chunk[j] = c * 4;
     }
     const int64_t a_step = p.rows_pad * 64;   // elements between consecutive k blocks
@@ -122,17 +141,34 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
     auto issue = [&](int it, int buf) {
         const unsigned sb = buf * STAGE;
         const bool last_ragged = ragged && it >= p.iters - 1;   // wave-uniform; folded into selects, no branch
+        const void *wp[W_LPW];
 #pragma unroll
         for (int j = 0; j < W_LPW; j++) {
             // both addresses are read into values first: a select between the memory locations
             // would keep the pointer array in scratch memory
             const uint64_t wa = reinterpret_cast<uint64_t>(w_src[j]);
-            const uint64_t za = reinterpret_cast<uint64_t>(p.zero_chunk);
+            const uint64_t za = reinterpret_cast<uint64_t>(p.zero_chunk) - (uint64_t)((j & 3) * 1024);
             const uint64_t mask = (last_ragged && w_past[j]) ? ~0ull : 0ull;
-            load_to_lds16(reinterpret_cast<const void *>((wa & ~mask) | (za & mask)), w_dst + sb + j * 1024);
+            wp[j] = reinterpret_cast<const void *>((wa & ~mask) | (za & mask));
         }
 #pragma unroll
-        for (int j = 0; j < A_LPW; j++) load_to_lds16(a_src[j], a_dst + sb + j * 1024);
+        for (int g = 0; g < W_LPW; g += 4) {
+            const int n = W_LPW - g >= 4 ? 4 : W_LPW - g;
+            const unsigned base = w_dst + sb + g * 1024;
+            if (n == 4) load_group_to_lds16<4>(wp[g], wp[g + 1 < W_LPW ? g + 1 : g], wp[g + 2 < W_LPW ? g + 2 : g], wp[g + 3 < W_LPW ? g + 3 : g], base);
+            else if (n == 3) load_group_to_lds16<3>(wp[g], wp[g + 1 < W_LPW ? g + 1 : g], wp[g + 2 < W_LPW ? g + 2 : g], nullptr, base);
+            else if (n == 2) load_group_to_lds16<2>(wp[g], wp[g + 1 < W_LPW ? g + 1 : g], nullptr, nullptr, base);
+            else load_group_to_lds16<1>(wp[g], nullptr, nullptr, nullptr, base);
+        }
+#pragma unroll
+        for (int g = 0; g < A_LPW; g += 4) {
+            const int n = A_LPW - g >= 4 ? 4 : A_LPW - g;
+            const unsigned base = a_dst + sb + g * 1024;
+            if (n == 4) load_group_to_lds16<4>(a_src[g], a_src[g + 1 < A_LPW ? g + 1 : g], a_src[g + 2 < A_LPW ? g + 2 : g], a_src[g + 3 < A_LPW ? g + 3 : g], base);
+            else if (n == 3) load_group_to_lds16<3>(a_src[g], a_src[g + 1 < A_LPW ? g + 1 : g], a_src[g + 2 < A_LPW ? g + 2 : g], nullptr, base);
+            else if (n == 2) load_group_to_lds16<2>(a_src[g], a_src[g + 1 < A_LPW ? g + 1 : g], nullptr, nullptr, base);
+            else load_group_to_lds16<1>(a_src[g], nullptr, nullptr, nullptr, base);
+        }
         const bool more = it + 1 < it1;           // wave-uniform
         int64_t astep = more ? a_step : 0;
         if (DENSE && more && ++a_pos == p.a_wrap) {   // second sweep over the activations
