@@ -325,6 +325,8 @@ class Probe:
         self.lib = C.CDLL(PROBE_LIB)
         self.lib.fnn_probe_stream.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p]
         self.lib.fnn_probe_mfma.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p]
+        self.lib.fnn_probe_lds_delivery.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p,
+                                                    C.POINTER(C.c_double)]
         self.ctx = ctx
         self.stream = ctx.stream()
         self.sink = ctx.alloc(256)
@@ -349,6 +351,31 @@ class Probe:
             out[f"{loads}x16B/lane,{'all' if wgs == 0 else wgs}wg"] = round(self.ctx.timer_stop() / n * 1e3, 3)
         return out
 
+
+    def lds_delivery(self, iters=400):
+        """Bytes per microsecond that loops of `global_load_lds_dwordx4` stages deliver into the LDS, by waves per
+        CU: 256 / 512 / 768 workgroups of 4 waves, 256 of 8 and of 16; ring of 3 stages (and 6 for 4 and 8 waves)."""
+        import ctypes as C
+        src = self.ctx.alloc(8 << 20)
+        out = {}
+        for name, waves, stages, wgs in (("4 waves/CU", 4, 3, 256), ("4 waves/CU, 6 stages", 4, 6, 256), ("2x4 waves/CU", 4, 3, 512),
+                                         ("3x4 waves/CU", 4, 3, 768), ("8 waves/CU", 8, 3, 256), ("8 waves/CU, 6 stages", 8, 6, 256),
+                                         ("16 waves/CU", 16, 3, 256)):
+            nbytes = C.c_double(0.0)
+            for _ in range(2):
+                rc = self.lib.fnn_probe_lds_delivery(self.stream, src.ptr, waves, stages, wgs, iters, self.sink.ptr, C.byref(nbytes))
+                if rc:
+                    raise RuntimeError(f"fnn_probe_lds_delivery failed: hipError {rc}")
+            self.ctx.sync()
+            n = 5
+            self.ctx.timer_start()
+            for _ in range(n):
+                self.lib.fnn_probe_lds_delivery(self.stream, src.ptr, waves, stages, wgs, iters, self.sink.ptr, C.byref(nbytes))
+            us = self.ctx.timer_stop() / n * 1e3
+            out[name] = {"us": round(us, 1), "tb_per_s": round(nbytes.value / us / 1e6, 2),
+                         "bytes_per_us_and_cu": round(nbytes.value / us / 256.0, 0)}
+        src.free()
+        return out
 
     def mfma_ceiling(self, target_us=(20.0, 60.0)):
         """What the matrix cores sustain with nothing else in the way: a kernel of MFMAs only (pseudo-random
@@ -526,7 +553,7 @@ def main() -> int:
     ap.add_argument("--opt", action="append", default=[], metavar="NAME=VALUE",
                     help="kernel selection option of the context, e.g. gemv_int8=0 for the f16 matrix-core GEMV "
                          "(names: the FNN_OPT_* of include/fastnn_hip.h, lower case without the prefix)")
-    ap.add_argument("--probe", default="", choices=["", "read", "copy", "mfma"],
+    ap.add_argument("--probe", default="", choices=["", "read", "copy", "mfma", "lds"],
                     help="instead of the MatMul, time a plain streaming read / copy of the same number of bytes "
                          "per launch over the same ring (device ceiling; calibration kernel for byte counters)")
     ap.add_argument("--traffic-json", default="", help="JSON file {\"fetch_bytes\": .., \"write_bytes\": ..} with "
@@ -562,6 +589,12 @@ def main() -> int:
         print(json.dumps({"metric": "matrix-core instructions only (no memory traffic)", "value": best["f16_32x32x16"], "unit": "TFLOP/s",
                           "n_gpus": 1, "higher_is_better": True, "data": "synthetic", "best": best, "all": res,
                           "config": {"workload": "probe mfma"}}))
+        return 0
+    if args.probe == "lds":
+        res = probe.lds_delivery()
+        print(json.dumps({"metric": "HBM/L2 -> LDS delivery of global_load_lds loops (no other work)", "value": max(v["tb_per_s"] for v in res.values()),
+                          "unit": "TB/s", "n_gpus": 1, "higher_is_better": True, "data": "synthetic", "all": res,
+                          "config": {"workload": "probe lds"}}))
         return 0
     r = make_ring(ctx, fastnn_amd, flib, args.workload, args.ring)
     dtn, k, n, wbytes, ring = r["dtn"], r["k"], r["n"], r["wbytes"], r["ring"]

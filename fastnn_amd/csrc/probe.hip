@@ -99,6 +99,54 @@ __global__ void __launch_bounds__(WAVES * 64) probe_mfma_kernel(int iters, uint3
     if (r == 0x9e3779b9u) sink[0] = r;   // practically never true: keeps the accumulators alive
 }
 
+// HBM / L2 -> LDS delivery: every wave of a workgroup issues LPW `global_load_lds_dwordx4` (1 KB each) per stage into
+// a ring of NS stages, one workgroup barrier per stage, no other work.  The source is a small region re-read by all
+// workgroups (L2 hits), so the figure is what the load path into the LDS delivers per CU for a given number of waves.
+template <int WAVES, int LPW, int NS>
+__global__ void __launch_bounds__(WAVES * 64) probe_lds_kernel(const uint4 *src, size_t region16, int iters, uint32_t *sink)
+{
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char *)smem;
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    constexpr int STAGE = WAVES * LPW * 1024;
+    const uint4 *base = src + (size_t)(blockIdx.x % 64) * region16;
+    uint32_t acc = 0;
+    auto issue = [&](int it, int buf) {
+#pragma unroll
+        for (int j = 0; j < LPW; j++) {
+            const size_t idx = ((size_t)it * WAVES * LPW + wv * LPW + j) * 64 + lane;
+            const uint4 *g = base + (idx % region16);
+            const unsigned dst = __builtin_amdgcn_readfirstlane(lds0 + buf * STAGE + (wv * LPW + j) * 1024);
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(dst), "v"(g) : "memory");
+        }
+    };
+    for (int s = 0; s < NS - 1; s++) issue(s, s);
+    int buf = 0;
+    for (int it = 0; it < iters; it++) {
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NS - 2) * LPW) : "memory");
+        __syncthreads();
+        int fb = buf + NS - 1;
+        if (fb >= NS) fb -= NS;
+        issue(it + NS - 1, fb);
+        acc ^= reinterpret_cast<const uint32_t *>(smem + buf * STAGE)[tid * 4];
+        buf = buf + 1 == NS ? 0 : buf + 1;
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // nothing may still be writing LDS when the workgroup retires
+    __syncthreads();
+    if (acc == 0x9e3779b9u) sink[0] = acc;
+}
+
+template <int WAVES, int LPW, int NS>
+hipError_t launch_lds(const void *src, size_t region16, int workgroups, int iters, uint32_t *sink, hipStream_t s)
+{
+    constexpr size_t lds = (size_t)NS * WAVES * LPW * 1024;
+    auto kern = probe_lds_kernel<WAVES, LPW, NS>;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(kern, dim3((unsigned)workgroups), dim3(WAVES * 64), lds, s, reinterpret_cast<const uint4 *>(src), region16, iters, sink);
+    return hipGetLastError();
+}
+
 template <int U>
 hipError_t launch(const void *src, void *dst, size_t n16, unsigned grid, uint32_t *sink, hipStream_t s)
 {
@@ -153,4 +201,25 @@ extern "C" int fnn_probe_mfma(void *stream, int kind, int workgroups, int waves,
     else if (waves == 4) hipLaunchKernelGGL((probe_mfma_kernel<true, 4>), grid, dim3(256), 0, s, iters, 0x1234567u, sink);
     else hipLaunchKernelGGL((probe_mfma_kernel<true, 8>), grid, dim3(512), 0, s, iters, 0x1234567u, sink);
     return (int)hipGetLastError();
+}
+
+// One launch on `stream` of the LDS delivery loop: `workgroups` workgroups of `waves` waves (4, 8 or 16; 4 loads of
+// 1 KB per wave and stage for 4 and 8 waves, 2 for 16), ring of `stages` (3 or 6) stages, `iters` stages per workgroup;
+// src_dev: at least 8 MiB (64 regions of 128 KiB, re-read by all workgroups).  *bytes_out = bytes delivered into LDS by
+// the launch.  Returns 0 or the hipError_t value.
+extern "C" int fnn_probe_lds_delivery(void *stream, const void *src_dev, int waves, int stages, int workgroups, int iters,
+                                      void *sink_dev, double *bytes_out)
+{
+    if (!src_dev || !sink_dev || workgroups < 1 || iters < 1) return (int)hipErrorInvalidValue;
+    if ((waves != 4 && waves != 8 && waves != 16) || (stages != 3 && stages != 6) || (waves == 16 && stages == 6)) return (int)hipErrorInvalidValue;
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    uint32_t *sink = reinterpret_cast<uint32_t *>(sink_dev);
+    const size_t region16 = 8192;
+    const int lpw = (waves == 16 || (waves == 8 && stages == 6)) ? 2 : 4;
+    if (bytes_out) *bytes_out = (double)workgroups * (iters + stages - 1) * waves * lpw * 1024.0;
+    if (waves == 4 && stages == 3) return (int)launch_lds<4, 4, 3>(src_dev, region16, workgroups, iters, sink, s);
+    if (waves == 4) return (int)launch_lds<4, 4, 6>(src_dev, region16, workgroups, iters, sink, s);
+    if (waves == 8 && stages == 3) return (int)launch_lds<8, 4, 3>(src_dev, region16, workgroups, iters, sink, s);
+    if (waves == 8) return (int)launch_lds<8, 2, 6>(src_dev, region16, workgroups, iters, sink, s);
+    return (int)launch_lds<16, 2, 3>(src_dev, region16, workgroups, iters, sink, s);
 }
