@@ -119,7 +119,7 @@ const OptionSpec kOptions[FNN_OPT_COUNT] = {
     {0, 0, 3},        // FNN_OPT_GEMV_ROW_TILES
     {0, 0, 3},        // FNN_OPT_ROWS16_ROW_TILES
     {9, 1, 17},       // FNN_OPT_ROWS16_MIN_M
-    {-1, -1, 3},      // FNN_OPT_TILE_SHAPE
+    {-1, -1, 4},      // FNN_OPT_TILE_SHAPE
     {0, 0, 32},       // FNN_OPT_TILE_SPLIT
     {0, 0, 6},        // FNN_OPT_TILE_STAGES
     {5, 1, 1 << 20},  // FNN_OPT_TILE_MIN_M

@@ -195,6 +195,7 @@ int run_digits(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const Q
     // tile shapes (operand rows x weight rows):
     //   0 = 128 x 128, 4 waves of 64 x 64 (4-bit weights: two workgroups per CU)   1 = 256 x 128, 4 waves of 128 x 64
     //   2 = 256 x 128, 8 waves of 64 x 64 (two waves per SIMD)                      3 = 256 x 256, 8 waves of 128 x 64 (4-bit weights)
+    //   4 = 256 x 192, 8 waves of 64 x 96 (4-bit weights): for N where 256-wide tiles leave CUs idle
     // Shape and K split minimise a small cost model in microseconds: rounds of workgroups over the CU slots x
     // (stages per workgroup x time per stage + a fixed cost per workgroup; resident workgroups share the CU), plus
     // the write and read of the partial tiles and the extra launch.  The stage times are measured on 4096 x 11008
@@ -207,9 +208,9 @@ int run_digits(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const Q
         Plan pl;
         pl.cfg = cfg;
         pl.bm = cfg == 0 ? 128 : 256;
-        const int bn = cfg == 3 ? 256 : 128;
+        const int bn = cfg == 3 ? 256 : (cfg == 4 ? 192 : 128);
         const int per_cu = (cfg == 0 && W4) ? 2 : 1;    // resident workgroups per CU (LDS)
-        const double t_stage = cfg == 3 ? 1.9 : (cfg == 2 ? 1.35 : (cfg == 1 ? 1.2 : (W4 ? 0.55 : 0.8)));
+        const double t_stage = cfg == 4 ? 1.5 : (cfg == 3 ? 1.9 : (cfg == 2 ? 1.35 : (cfg == 1 ? 1.2 : (W4 ? 0.55 : 0.8))));
         pl.mtiles = (int)((meff + pl.bm - 1) / pl.bm);
         pl.ntiles = (int)((N + bn - 1) / bn);
         const int base = pl.mtiles * pl.ntiles;
@@ -227,9 +228,13 @@ int run_digits(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const Q
     {
         const Plan big = plan_for(W4 ? 3 : 2);
         if (big.cost < pl.cost) pl = big;
+        if (W4) {
+            const Plan mid = plan_for(4);
+            if (mid.cost < pl.cost) pl = mid;
+        }
     }
     const int64_t opt_cfg = fnn_ctx_option(ctx, FNN_OPT_TILE_SHAPE);
-    if (opt_cfg >= 0 && opt_cfg <= 3) pl = plan_for((opt_cfg == 3 && !W4) ? 2 : (int)opt_cfg);   // (256 x 256 stages of 8-bit weights do not fit the LDS)
+    if (opt_cfg >= 0 && opt_cfg <= 4) pl = plan_for((opt_cfg >= 3 && !W4) ? 2 : (int)opt_cfg);   // (wider stages of 8-bit weights do not fit the LDS)
     const int cfg = pl.cfg, mtiles = pl.mtiles, ntiles = pl.ntiles;
     int splits = pl.splits;
     const int64_t rows_pad = (int64_t)mtiles * pl.bm;
@@ -272,7 +277,10 @@ int run_digits(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const Q
     constexpr int NS0 = (160 * 1024) / (128 * 128 + 128 * WC * 16) >= 6 ? 6 : 5;   // 128 x 128 tiles: 6 (4-bit), 5 (8-bit)
     constexpr int NS1 = (160 * 1024) / (256 * 128 + 128 * WC * 16) >= 4 ? 4 : 3;   // 256 x 128 tiles: 4 (4-bit), 3 (8-bit)
     const int opt_ns = (int)fnn_ctx_option(ctx, FNN_OPT_TILE_STAGES);
-    if (cfg == 3) {
+    if (cfg == 4) {
+        if constexpr (W4) e = launch_digit_tile<DT, 4, 2, 2, 3, 3, DIG>(t, s);
+        else e = hipErrorInvalidValue;
+    } else if (cfg == 3) {
         if constexpr (W4) e = launch_digit_tile<DT, 2, 4, 4, 2, 3, DIG>(t, s);
         else e = hipErrorInvalidValue;
     } else if (cfg == 2) e = launch_digit_tile<DT, 4, 2, 2, 2, 3, DIG>(t, s);

@@ -71,10 +71,16 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
     constexpr int A_BYTES = BM * 128, W_BYTES = BN * WC * 16, STAGE = A_BYTES + W_BYTES;
     constexpr int NWV = WGM * WGN;                  // waves per workgroup: 4, or 8 (two per SIMD)
     constexpr int A_LPW = BM / (8 * NWV);           // activation load instructions per wave and stage
-    constexpr int W_LPW = BN * WC / (64 * NWV);     // weight load instructions per wave and stage
+    // weight load instructions per wave and stage.  When the stage's weight chunks do not divide evenly over the
+    // waves (W_WAVES < NWV), the first W_WAVES waves take W_LPW loads each and the others none: the waits below
+    // count per wave.
+    constexpr int W_LOADS = BN * WC / 64;
+    constexpr int W_LPW = (W_LOADS + NWV - 1) / NWV;
+    constexpr int W_WAVES = W_LOADS / W_LPW;
     constexpr int LPS = A_LPW + W_LPW;
     static_assert(NWV == 4 || NWV == 8, "4 or 8 waves");
-    static_assert(BM % (8 * NWV) == 0 && BN * WC % (64 * NWV) == 0 && NS >= 3 && NS <= 8, "stage shape");
+    static_assert(BM % (8 * NWV) == 0 && BN * WC % 64 == 0 && W_LOADS % W_LPW == 0 && NS >= 3 && NS <= 8, "stage shape");
+    const bool w_on = W_WAVES == NWV || (int)(threadIdx.x >> 6) < W_WAVES;   // wave-uniform
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char *)smem;
@@ -153,6 +159,7 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
         }
 #pragma unroll
         for (int g = 0; g < W_LPW; g += 4) {
+            if (!w_on) break;
             const int n = W_LPW - g >= 4 ? 4 : W_LPW - g;
             const unsigned base = w_dst + sb + g * 1024;
             if (n == 4) load_group_to_lds16<4>(wp[g], wp[g + 1 < W_LPW ? g + 1 : g], wp[g + 2 < W_LPW ? g + 2 : g], wp[g + 3 < W_LPW ? g + 3 : g], base);
@@ -253,7 +260,9 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
         for (int st = 0; st < NS - 1; st++) issue(it0 + st, st);
         uint32_t wq[TN][4 * WPS], wqn[TN][4 * WPS];
         f16x8 af[4][TM], bfr[2][TN];
-        wait_loads_but<(NS - 2) * LPS>();   // first stage: this wave's part has landed
+        // first stage: this wave's part has landed
+        if (w_on) wait_loads_but<(NS - 2) * LPS>();
+        else wait_loads_but<(NS - 2) * A_LPW>();
         __syncthreads();                    // ... and everybody else's
         read_w(smem, wq);
         read_a(smem, 0, af[0]);
@@ -276,7 +285,9 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
             decode(wq, 2, bfr[0]);
             mfmas(af[1], bfr[1]);
             // hand-over
-            wait_loads_but<(NS - 3) * LPS>();   // this wave's part of the next stage has landed
+            // this wave's part of the next stage has landed
+            if (w_on) wait_loads_but<(NS - 3) * LPS>();
+            else wait_loads_but<(NS - 3) * A_LPW>();
             __syncthreads();                    // everybody's; the stage before the current one is free
             int fb = buf + NS - 1;
             if (fb >= NS) fb -= NS;

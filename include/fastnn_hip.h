@@ -94,7 +94,7 @@ enum {
     FNN_OPT_ROWS16_MIN_M = 4,     /* smallest M the 16-row kernel takes (default 9; 17 switches it off)             */
     FNN_OPT_TILE_SHAPE = 5,       /* tiled GEMMs, tile shape; -1 (default) = by shape.  f16 tiles: 0 = 128x128, 1 = 64x128, */
                                   /* 2 = 32x128, 3 = 256x128 with 8 waves (8-bit weights); int8 digit-plane tiles:       */
-                                  /* 0 = 128x128, 1 = 256x128, 2 = 256x128 with 8 waves, 3 = 256x256 with 8 waves (4-bit) */
+                                  /* 0 = 128x128, 1 = 256x128, 2 = 256x128 / 8 waves, 3 = 256x256, 4 = 256x192 (8 waves, 4-bit) */
     FNN_OPT_TILE_SPLIT = 6,       /* tiled GEMM: K split over this many workgroups; 0 (default) = cost model        */
     FNN_OPT_TILE_STAGES = 7,      /* tiled GEMMs: LDS ring depth where the shape has variants (3..6); 0 (default) = by shape */
     FNN_OPT_TILE_MIN_M = 8,       /* smallest M the tiled GEMM takes (default 5)                                    */

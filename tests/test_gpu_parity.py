@@ -234,7 +234,7 @@ def test_int8_digit_plane_gemm(ctx, orc, dt, m, k, n):
     assert_close(got, want, 4e-6 if int8_default else TOL_F32, f"digit gemm {NAMES[dt]} {m}x{k}x{n}")
     assert rel_err(ctx.qmatmul(h, a, n, bias=bias, act=2, flags=flib.FLAG_ACT_F16_SINGLE), want) <= TOL_NORTH_STAR
     try:
-        for shape in (0, 1, 2, 3):
+        for shape in (0, 1, 2, 3, 4):
             for split in (1, 3):
                 ctx.set_option(flib.OPT_TILE_SHAPE, shape)
                 ctx.set_option(flib.OPT_TILE_SPLIT, split)
