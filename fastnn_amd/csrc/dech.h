@@ -127,6 +127,14 @@ struct DecH<FNN_DT_F4> {
     }
 };
 
+// codebook nibbles are looked up by the tile kernel itself (a table in LDS); only the word geometry is used
+template <>
+struct DecH<FNN_DT_I4CB> {
+    static constexpr int WPS = 1;
+    static constexpr bool INTERLEAVED = false;
+    __device__ static __forceinline__ f16x8 step(const uint32_t *w) { return pack8(w[0], w[0], w[0], w[0]); }
+};
+
 // ---- int8 operands for v_mfma_i32_32x32x32_i8: one MFMA step = 16 k-values of a weight row (4 words).
 template <int DT>
 struct DecI;

@@ -282,7 +282,8 @@ int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QM
     // hide its load latency: factor 1.5), plus, for s > 1, the write + read of s partial [M,N] tiles.
     const int env_split = (int)fnn_ctx_option(ctx, FNN_OPT_TILE_SPLIT);
     const int base = mtiles * ntiles;
-    const double t_bits = DecH<DT>::WPS == 1 ? 0.4 : (DecH<DT>::WPS == 2 ? 0.7 : 1.0);
+    // (codebook weights decoded in the kernel: two MFMAs per step and the table look-ups)
+    const double t_bits = DT == FNN_DT_I4CB ? 0.9 : (DecH<DT>::WPS == 1 ? 0.4 : (DecH<DT>::WPS == 2 ? 0.7 : 1.0));
     const double t_stage = t_bits * (cfg == 3 ? 2.0 : (cfg == 0 ? 1.0 : (cfg == 1 ? 0.5 : 0.25)));
     const double part_us = (double)M * (double)N * 8.0 / 3.0e6;
     int splits = 1;
@@ -311,7 +312,7 @@ int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QM
 
     fnn_hip_weight *wm = const_cast<fnn_hip_weight *>(w);
     const bool want_umean = !precise && !dense && (DT == FNN_DT_I8 || DT == FNN_DT_I4 || DT == FNN_DT_U8 || DT == FNN_DT_U4 || DT == FNN_DT_F4);
-    if constexpr (DT != DT_F16_DENSE) if (want_umean && !wm->umean) {
+    if constexpr (DT != DT_F16_DENSE && DT != FNN_DT_I4CB) if (want_umean && !wm->umean) {
         if (fnn_ctx_no_alloc(ctx)) return fnn_ctx_fail(ctx, FNN_ERR_MEMORY, "first single-pass use of a weight while allocation is not allowed (graph capture, fnn_hip_qmatmul_static)");
         if (hipMalloc((void **)&wm->umean, (size_t)w->rows * 4 + 64) != hipSuccess)
             return fnn_ctx_fail(ctx, FNN_ERR_MEMORY, "out of device memory (row means)");
@@ -340,6 +341,11 @@ int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QM
     t.out = q.out; t.part = (float *)ws1;
     t.m = M; t.n = N; t.kp = q.kp; t.kpad = kpad; t.rows_pad = rows_pad;
     t.a_wrap = 0;
+    t.bscales = nullptr; t.codebook = nullptr; t.bpr = 0;
+    if constexpr (DT == FNN_DT_I4CB) {
+        t.bscales = q.scales; t.codebook = q.codebook; t.bpr = q.bpr;
+        t.scales = nullptr; t.zeros = nullptr;
+    }
     if (dense) {
         t.words = dense->words; t.zero_chunk = dense->words;
         t.scales = dense->row_scale; t.zeros = dense->row_zero;
@@ -499,6 +505,27 @@ int fnn_tiled_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, 
     if (q.m < min_m) return FNN_OK;
     if (w->dtype == FNN_DT_I4CB) {
         if (q.as_written || q.qblock <= 0 || q.n > (1 << 24) || q.m > (1 << 22)) return FNN_OK;
+        // blocks of 32 values: nibbles decoded inside the tile kernel (4 bits per value cross the memory system instead
+        // of the 32 of the expanded f16 hi + lo operand, and no expansion is kept with the weight); other block
+        // sizes, or by option, the expanded operand.  Measured on 4096 x 4096 (us, in-kernel / expanded): M = 5 ... 16
+        // 19-20 / 23-26, M = 32 23.3 / 24.5, M = 64 30.5 / 31.5, M = 128 41.2 / 42.4, M = 256 65.8 / 58.4, M = 1024
+        // 191 / 207; single rounding: M <= 16 20 / 24-27, M = 64 30.1 / 27.2, M = 256 48.3 / 46.2, M = 1024 119 / 99
+        // (the per-block fold of the accumulator, 2 x 64 FMAs per wave and stage, and the look-ups make the loop
+        // vector-ALU bound; the expanded operand's loop is the plain f16 one).
+        const int64_t opt_exp = fnn_ctx_option(ctx, FNN_OPT_CODEBOOK_EXPANDED);
+        const bool precise = !(flags & FNN_FLAG_ACT_F16_SINGLE);
+        const bool in_kernel = opt_exp == 0 ? (precise ? (q.m < 192 || q.m >= 512) : q.m <= 16) : opt_exp == 2;
+        if (q.qblock == 32 && in_kernel) {
+            QMatmulArgs qa = q;
+            int rc;
+            if (q.words == w->words && (rc = fnn_aligned_rows(ctx, s, w, &qa.words, &qa.kp))) return rc;
+            if (qa.kp % 4 == 0 && !(reinterpret_cast<uintptr_t>(qa.words) & 15)) {
+                rc = run_tiled<FNN_DT_I4CB>(ctx, s, w, qa, flags);
+                if (rc) return rc;
+                *handled = true;
+                return FNN_OK;
+            }
+        }
         int rc = run_tiled_codebook(ctx, s, w, q, flags);
         if (rc) return rc;
         *handled = true;

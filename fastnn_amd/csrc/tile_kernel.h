@@ -18,7 +18,25 @@ struct TileArgs {
     int64_t m, n, kp, kpad, rows_pad;
     int act, splits, iters, ips, mtiles, ntiles;
     int a_wrap;   // > 0: the activation operand has a_wrap k blocks and is swept again after them (weights = [hi | lo])
+    // codebook weights decoded in the kernel (DT = FNN_DT_I4CB): block scales [n][bpr] (one per 32 k-values), the 16
+    // table values, and the power of two the table is scaled by before it is split into f16 hi + lo
+    const float *bscales;
+    const float *codebook;
+    int64_t bpr;
 };
+
+// power of two that brings the largest table magnitude into [2^14, 2^15): the f16 hi + lo split of the scaled table
+// then carries ~22 bits of every entry (every thread computes the same value from the 16 cached floats)
+__device__ __forceinline__ int codebook_exp(const float *cb)
+{
+    float mx = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; i++) mx = fmaxf(mx, fabsf(cb[i]));
+    if (!(mx > 0.0f) || !(mx < __builtin_huge_valf())) return 0;
+    int ex;
+    (void)frexpf(mx, &ex);
+    return 15 - ex;
+}
 
 // HBM -> LDS without passing registers: lane i of the wave stores its 16 bytes at
 // LDS address m0 + 16*i.  The compiler does not see these loads: waits are placed by hand.
@@ -63,10 +81,16 @@ template <int DT, int WGM, int WGN, int TM, int TN, bool PRECISE, int NS, bool I
 __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
 {
     static_assert(DIG == 0 || (INT8 && (DIG == 2 || DIG == 4)), "digit planes ride on the int8 operands");
+    // Codebook weights (w[n,k] = bscale[n, k/32] * table[nibble], src/packed_tensor.rs:469-521) are decoded here:
+    // the nibble looks up an (f16 hi, f16 lo) pair of the scaled table value in LDS, two MFMAs per step (hi, lo)
+    // add into a per-block accumulator, and after the two steps of a 32-value block the accumulator is folded into
+    // the running sum with the block's scale: sum_blk s_blk * sum_k table[q]*a, the reference's association.
+    constexpr bool CB = !INT8 && DT == FNN_DT_I4CB;
     using D = typename std::conditional<INT8, DecI<DT>, DecH<DT>>::type;
     static_assert(!(INT8 && PRECISE), "int8 operands have no hi/lo rows");
     constexpr int WPS = D::WPS;          // words per 8 k-values
     constexpr int WC = 2 * WPS;          // 16-byte weight chunks per row and stage (32, 64 or 128 bytes)
+    constexpr int WQW = CB ? 8 : 4 * WPS; // weight words a lane holds per stage and 32-row block
     constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
     constexpr int A_BYTES = BM * 128, W_BYTES = BN * WC * 16, STAGE = A_BYTES + W_BYTES;
     constexpr int NWV = WGM * WGN;                  // waves per workgroup: 4, or 8 (two per SIMD)
@@ -88,6 +112,18 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const int wm = wv / WGN, wn = wv % WGN;
     const int lr = lane & 31, h = lane >> 5;
+    __shared__ uint32_t cbt[16];   // codebook mode: (hi | lo << 16) per table entry
+    int cb_exp = 0;
+    if constexpr (CB) {
+        cb_exp = codebook_exp(p.codebook);
+        if (tid < 16) {
+            const float v = ldexpf(p.codebook[tid], cb_exp);
+            const _Float16 hi = (_Float16)v;
+            const _Float16 lo = (_Float16)(v - (float)hi);
+            cbt[tid] = (uint32_t)__builtin_bit_cast(uint16_t, hi) | ((uint32_t)__builtin_bit_cast(uint16_t, lo) << 16);
+        }
+        // (the barrier before the first operand read orders this store)
+    }
 
     // workgroup id -> tile, row tile fastest.  Ids are dealt round-robin over the 8 XCDs (each with
     // its own L2), so an XCD keeps meeting the same few row tiles of the activations, the operand
@@ -204,7 +240,8 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
 #pragma unroll
     for (int tn = 0; tn < TN; tn++) {
         const int row = (wn * TN + tn) * 32 + lr;
-        if constexpr (WC == 2) w_off[tn] = A_BYTES + (row * 2 + (h ^ ((row >> 3) & 1))) * 16;
+        if constexpr (CB) w_off[tn] = A_BYTES + row * 32;   // both chunks of the row are read
+        else if constexpr (WC == 2) w_off[tn] = A_BYTES + (row * 2 + (h ^ ((row >> 3) & 1))) * 16;
         else w_off[tn] = A_BYTES + row * (WC * 16);   // chunk index added per read
     }
     const int asw = (lr >> 1) & 7;   // (row >> 1) & 7 of every activation row this lane reads
@@ -216,10 +253,18 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
         //  - the stage hand-over (wait for the next stage, barrier, request of a further stage)
         //    sits between steps 1 and 2; steps 2 and 3 already read the next stage's operands,
         // so the matrix cores never wait for a whole LDS round trip.
-        auto read_w = [&](const unsigned char *sbase, uint32_t(&wq)[TN][4 * WPS]) {
+        auto read_w = [&](const unsigned char *sbase, uint32_t(&wq)[TN][WQW]) {
 #pragma unroll
             for (int tn = 0; tn < TN; tn++) {
-                if constexpr (WC == 2) {
+                if constexpr (CB) {
+                    // the 8 words (64 nibbles) of the row's stage; MFMA step s takes word 2s + h
+                    const int row = (wn * TN + tn) * 32 + lr;
+                    const int sw = (row >> 3) & 1;
+                    const u32x4 t0 = *reinterpret_cast<const u32x4 *>(sbase + w_off[tn] + (0 ^ sw) * 16);
+                    const u32x4 t1 = *reinterpret_cast<const u32x4 *>(sbase + w_off[tn] + (1 ^ sw) * 16);
+                    wq[tn][0] = t0[0]; wq[tn][1] = t0[1]; wq[tn][2] = t0[2]; wq[tn][3] = t0[3];
+                    wq[tn][4] = t1[0]; wq[tn][5] = t1[1]; wq[tn][6] = t1[2]; wq[tn][7] = t1[3];
+                } else if constexpr (WC == 2) {
                     const u32x4 t = *reinterpret_cast<const u32x4 *>(sbase + w_off[tn]);
                     wq[tn][0] = t[0]; wq[tn][1] = t[1]; wq[tn][2] = t[2]; wq[tn][3] = t[3];
                 } else {
@@ -237,29 +282,78 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
         auto read_a = [&](const unsigned char *sbase, int s, f16x8(&af)[TM]) {
 #pragma unroll
             for (int tm = 0; tm < TM; tm++)
-                af[tm] = *reinterpret_cast<const f16x8 *>(sbase + a_off[tm] + (((4 * h + s) ^ asw) * 16));
+                af[tm] = *reinterpret_cast<const f16x8 *>(sbase + a_off[tm] + (((CB ? 2 * s + h : 4 * h + s) ^ asw) * 16));
         };
-        auto decode = [&](const uint32_t(&wq)[TN][4 * WPS], int s, f16x8(&bf)[TN]) {
+        f32x16 accb[CB ? TM : 1][CB ? TN : 1];   // codebook mode: sum over the current 32-value block
+        float bs_cur[TN][2], bs_nxt[TN][2];         // ... and the block scales of this lane's columns (this / next stage)
+        auto load_bscales = [&](int it, float(&bs)[TN][2]) {
 #pragma unroll
-            for (int tn = 0; tn < TN; tn++) bf[tn] = D::step(&wq[tn][s * WPS]);
+            for (int tn = 0; tn < TN; tn++) {
+                int64_t n = n0 + (wn * TN + tn) * 32 + lr;
+                if (n > p.n - 1) n = p.n - 1;
+#pragma unroll
+                for (int b = 0; b < 2; b++) {
+                    int64_t blk = 2 * (int64_t)it + b;
+                    if (blk > p.bpr - 1) blk = p.bpr - 1;   // past K: the activations are zero there
+                    bs[tn][b] = p.bscales[n * p.bpr + blk];
+                }
+            }
         };
-        auto mfmas = [&](const f16x8(&af)[TM], const f16x8(&bf)[TN]) {
+        auto decode = [&](const uint32_t(&wq)[TN][WQW], int s, f16x8(&bf)[TN], f16x8(&bl)[CB ? TN : 1]) {
+#pragma unroll
+            for (int tn = 0; tn < TN; tn++) {
+                if constexpr (CB) {
+                    const uint32_t w = h ? wq[tn][2 * s + 1] : wq[tn][2 * s];
+                    uint32_t d[8];
+                    d[0] = cbt[w & 15u];
+#pragma unroll
+                    for (int j = 1; j < 8; j++) d[j] = cbt[(w >> (4 * j)) & 15u];
+                    uint32_t hi4[4], lo4[4];
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        hi4[j] = __builtin_amdgcn_perm(d[2 * j + 1], d[2 * j], 0x05040100u);   // low halves: hi parts
+                        lo4[j] = __builtin_amdgcn_perm(d[2 * j + 1], d[2 * j], 0x07060302u);   // high halves: lo parts
+                    }
+                    bf[tn] = pack8(hi4[0], hi4[1], hi4[2], hi4[3]);
+                    bl[tn] = pack8(lo4[0], lo4[1], lo4[2], lo4[3]);
+                } else {
+                    bf[tn] = D::step(&wq[tn][s * WPS]);
+                }
+            }
+        };
+        // s = step inside the stage (codebook mode: steps 0,1 are one block, steps 2,3 the next)
+        auto mfmas = [&](const f16x8(&af)[TM], const f16x8(&bf)[TN], const f16x8(&bl)[CB ? TN : 1], int s) {
 #pragma unroll
             for (int tm = 0; tm < TM; tm++)
 #pragma unroll
                 for (int tn = 0; tn < TN; tn++)
-                    if constexpr (INT8)
+                    if constexpr (INT8) {
                         acc[tm][tn] = __builtin_bit_cast(f32x16, __builtin_amdgcn_mfma_i32_32x32x32_i8(
                                                                      __builtin_bit_cast(i32x4, af[tm]), __builtin_bit_cast(i32x4, bf[tn]),
                                                                      __builtin_bit_cast(i32x16, acc[tm][tn]), 0, 0, 0));
-                    else
+                    } else if constexpr (CB) {
+                        f32x16 c0 = accb[tm][tn];
+                        if ((s & 1) == 0) {
+#pragma unroll
+                            for (int i = 0; i < 16; i++) c0[i] = 0.0f;
+                        }
+                        c0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[tm], bf[tn], c0, 0, 0, 0);
+                        accb[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[tm], bl[tn], c0, 0, 0, 0);
+                        if (s & 1) {
+                            const float sc = bs_cur[tn][s >> 1];
+#pragma unroll
+                            for (int i = 0; i < 16; i++) acc[tm][tn][i] = fmaf(sc, accb[tm][tn][i], acc[tm][tn][i]);
+                        }
+                    } else {
                         acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[tm], bf[tn], acc[tm][tn], 0, 0, 0);
+                    }
         };
 
 #pragma unroll
         for (int st = 0; st < NS - 1; st++) issue(it0 + st, st);
-        uint32_t wq[TN][4 * WPS], wqn[TN][4 * WPS];
-        f16x8 af[4][TM], bfr[2][TN];
+        uint32_t wq[TN][WQW], wqn[TN][WQW];
+        f16x8 af[4][TM], bfr[2][TN], bfl[2][CB ? TN : 1];
+        if constexpr (CB) load_bscales(it0, bs_cur);
         // first stage: this wave's part has landed
         if (w_on) wait_loads_but<(NS - 2) * LPS>();
         else wait_loads_but<(NS - 2) * A_LPW>();
@@ -267,7 +361,7 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
         read_w(smem, wq);
         read_a(smem, 0, af[0]);
         read_a(smem, 1, af[1]);
-        decode(wq, 0, bfr[0]);
+        decode(wq, 0, bfr[0], bfl[0]);
         // The loop body is one straight-line block (no branches), so the compiler can interleave LDS
         // reads, decode and MFMAs across the whole stage; the last stage, which has no successor to
         // hand over to, is peeled off.
@@ -276,14 +370,15 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
             const unsigned char *sbase = smem + buf * STAGE;
             const int nbuf = (buf + 1 == NS) ? 0 : buf + 1;
             const unsigned char *nbase = smem + nbuf * STAGE;
+            if constexpr (CB) load_bscales(it + 1, bs_nxt);
             // step 0
             read_a(sbase, 2, af[2]);
-            decode(wq, 1, bfr[1]);
-            mfmas(af[0], bfr[0]);
+            decode(wq, 1, bfr[1], bfl[1]);
+            mfmas(af[0], bfr[0], bfl[0], 0);
             // step 1
             read_a(sbase, 3, af[3]);
-            decode(wq, 2, bfr[0]);
-            mfmas(af[1], bfr[1]);
+            decode(wq, 2, bfr[0], bfl[0]);
+            mfmas(af[1], bfr[1], bfl[1], 1);
             // hand-over
             // this wave's part of the next stage has landed
             if (w_on) wait_loads_but<(NS - 3) * LPS>();
@@ -295,29 +390,33 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
             // step 2, with the first reads of the next stage
             read_w(nbase, wqn);
             read_a(nbase, 0, af[0]);
-            decode(wq, 3, bfr[1]);
-            mfmas(af[2], bfr[0]);
+            decode(wq, 3, bfr[1], bfl[1]);
+            mfmas(af[2], bfr[0], bfl[0], 2);
             // step 3
             read_a(nbase, 1, af[1]);
-            decode(wqn, 0, bfr[0]);
-            mfmas(af[3], bfr[1]);
+            decode(wqn, 0, bfr[0], bfl[0]);
+            mfmas(af[3], bfr[1], bfl[1], 3);
 #pragma unroll
             for (int tn = 0; tn < TN; tn++)
 #pragma unroll
-                for (int q = 0; q < 4 * WPS; q++) wq[tn][q] = wqn[tn][q];
+                for (int q = 0; q < WQW; q++) wq[tn][q] = wqn[tn][q];
+            if constexpr (CB) {
+#pragma unroll
+                for (int tn = 0; tn < TN; tn++) { bs_cur[tn][0] = bs_nxt[tn][0]; bs_cur[tn][1] = bs_nxt[tn][1]; }
+            }
             buf = nbuf;
         }
         {   // last stage
             const unsigned char *sbase = smem + buf * STAGE;
             read_a(sbase, 2, af[2]);
-            decode(wq, 1, bfr[1]);
-            mfmas(af[0], bfr[0]);
+            decode(wq, 1, bfr[1], bfl[1]);
+            mfmas(af[0], bfr[0], bfl[0], 0);
             read_a(sbase, 3, af[3]);
-            decode(wq, 2, bfr[0]);
-            mfmas(af[1], bfr[1]);
-            decode(wq, 3, bfr[1]);
-            mfmas(af[2], bfr[0]);
-            mfmas(af[3], bfr[1]);
+            decode(wq, 2, bfr[0], bfl[0]);
+            mfmas(af[1], bfr[1], bfl[1], 1);
+            decode(wq, 3, bfr[1], bfl[1]);
+            mfmas(af[2], bfr[0], bfl[0], 2);
+            mfmas(af[3], bfr[1], bfl[1], 3);
         }
         wait_loads_but<0>();   // nothing may still be writing LDS when the workgroup retires
     }
@@ -412,8 +511,13 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
     for (int tn = 0; tn < TN; tn++) {
         const int64_t n = n0 + (wn * TN + tn) * 32 + lr;
         const bool ok = n < p.n && !split;
-        sc[tn] = ok ? p.scales[n] : 0.0f;
-        zp[tn] = ok ? p.zeros[n] : 0.0f;
+        if constexpr (CB) {   // block scales are applied in the loop; what is left is the table's power of two
+            sc[tn] = ok ? ldexpf(1.0f, -cb_exp) : 0.0f;
+            zp[tn] = 0.0f;
+        } else {
+            sc[tn] = ok ? p.scales[n] : 0.0f;
+            zp[tn] = ok ? p.zeros[n] : 0.0f;
+        }
         bi[tn] = (ok && p.bias) ? p.bias[n] : 0.0f;
         um[tn] = (!PRECISE && ok && p.umean) ? p.umean[n] : 0.0f;
     }
@@ -469,7 +573,8 @@ __global__ void __launch_bounds__(256) splitk_epilogue_kernel(TileArgs p, int si
     const int64_t n = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (n >= p.n) return;
     const int64_t total = p.m * p.n;
-    const float sc = p.scales[n], zr = p.zeros[n];
+    const float sc = p.codebook ? ldexpf(1.0f, -codebook_exp(p.codebook)) : p.scales[n];   // (codebook weights decoded in the tile kernel)
+    const float zr = p.codebook ? 0.0f : p.zeros[n];
     const float bs = p.bias ? p.bias[n] : 0.0f;
     const bool comp = single && p.umean;
     const float um = comp ? p.umean[n] : 0.0f;

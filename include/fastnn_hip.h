@@ -105,7 +105,10 @@ enum {
                                   /* matrix-core GEMM over four exact activation digit planes (not in the single-rounding */
                                   /* mode); 0: the f16 tiled GEMM takes them too                                          */
     FNN_OPT_GEMM_INT8_MIN_M = 11, /* smallest M of that path (default 17)                                                 */
-    FNN_OPT_COUNT = 12
+    FNN_OPT_CODEBOOK_EXPANDED = 12, /* codebook weights with blocks of 32 at M >= 5: 0 (default) = by M (decoded inside the */
+                                  /* tiled GEMM where that measured faster), 1 = always through the expanded f16 hi + lo  */
+                                  /* operand (FNN_OPT_CODEBOOK_CACHE), 2 = always decoded inside the tiled GEMM           */
+    FNN_OPT_COUNT = 13
 };
 int fnn_hip_set_option(fnn_hip_ctx *ctx, int option, int64_t value);
 int fnn_hip_get_option(fnn_hip_ctx *ctx, int option, int64_t *value);

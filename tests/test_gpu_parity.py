@@ -313,6 +313,41 @@ def test_reference_literal_cases_on_gpu(ctx, orc, golden):
         ctx.release(h)
 
 
+@pytest.mark.parametrize("m,k,n", [(5, 4096, 520), (16, 1056, 300), (40, 2048, 260), (64, 200, 4400), (130, 992, 96), (256, 4096, 256),
+                                   (600, 1024, 384)])
+def test_codebook_gemm_decoded_in_kernel_and_expanded(ctx, orc, m, k, n):
+    """Codebook weights at M >= 5: nibbles looked up inside the tiled GEMM (per-block accumulators folded with the
+    block scale, the reference's association) and the expanded f16 hi + lo operand are both within the MatMul bound
+    of the oracle, in both activation modes; ragged K (blocks of 32 that do not fill a 64-value stage, rows that are
+    not a multiple of 16 bytes) and ragged N; bias + SiLU."""
+    rng = np.random.default_rng(5100 + m + k)
+    pw = fastnn_amd.quantize_weights(flib.DT_I4CB, _weights(rng, n, k, "laplace"))
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    a[:, ::61] *= 50.0
+    bias = (rng.standard_normal(n) * 0.01).astype(np.float32)
+    h = ctx.register(pw)
+    want = orc.qmatmul(to_oracle(orc, pw), a, order=2, bias=bias, act=3)
+    try:
+        outs = {}
+        for mode in (2, 1, 0):
+            ctx.set_option(flib.OPT_CODEBOOK_EXPANDED, mode)
+            outs[mode] = ctx.qmatmul(h, a, n, bias=bias, act=3)
+            assert_close(outs[mode], want, TOL_F32, f"codebook mode {mode} {m}x{k}x{n}")
+            assert rel_err(ctx.qmatmul(h, a, n, bias=bias, act=3, flags=flib.FLAG_ACT_F16_SINGLE), want) <= TOL_NORTH_STAR
+        assert not np.array_equal(outs[2], outs[1])      # two different kernels
+        for split in (1, 2, 5):
+            ctx.set_option(flib.OPT_CODEBOOK_EXPANDED, 2)
+            ctx.set_option(flib.OPT_TILE_SPLIT, split)
+            for shape in (0, 1, 2):
+                ctx.set_option(flib.OPT_TILE_SHAPE, shape)
+                assert_close(ctx.qmatmul(h, a, n, bias=bias, act=3), want, TOL_F32, f"split {split} shape {shape}")
+    finally:
+        ctx.set_option(flib.OPT_CODEBOOK_EXPANDED, 0)
+        ctx.set_option(flib.OPT_TILE_SPLIT, 0)
+        ctx.set_option(flib.OPT_TILE_SHAPE, -1)
+    ctx.release(h)
+
+
 def test_i4cb_as_written_variant(ctx, orc):
     rng = np.random.default_rng(8)
     n = k = 64

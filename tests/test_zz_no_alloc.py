@@ -57,8 +57,9 @@ def test_static_entry_point_matches_the_allocating_one(orc):
 
 
 def test_static_entry_point_reuses_side_tables_but_never_builds_them(orc):
-    """A codebook weight at M >= 5 needs its f16 expansion: built by fnn_hip_qmatmul on first use, refused with a
-    message by the static entry point before that, used by it afterwards."""
+    """A codebook weight at M >= 5 run through its expanded f16 operand (by option) needs the expansion: built by
+    fnn_hip_qmatmul on first use, refused with a message by the static entry point before that, used by it afterwards.
+    Decoded inside the tiled GEMM (the default at this M) it needs no side table and works at once."""
     rng = np.random.default_rng(14)
     n, k, m = 256, 512, 48
     pw = fastnn_amd.quantize_weights(flib.DT_I4CB, (rng.laplace(0, 0.02, (n, k))).astype(np.float32))
@@ -66,6 +67,13 @@ def test_static_entry_point_reuses_side_tables_but_never_builds_them(orc):
     with fastnn_amd.HipContext(0) as ctx:
         h = ctx.register(pw)
         da, d_ref, d_got = ctx.to_device(a), ctx.alloc(m * n * 4), ctx.alloc(m * n * 4)
+        ctx.qmatmul_static(h, da.ptr, m, d_got.ptr)          # decoded in the kernel: nothing to build
+        ctx.qmatmul_dev(h, da.ptr, m, d_ref.ptr)
+        ctx.sync()
+        first = d_got.download(np.float32, m * n).reshape(m, n)
+        assert np.array_equal(first, d_ref.download(np.float32, m * n).reshape(m, n))
+        assert_close(first, orc.qmatmul(to_oracle(orc, pw), a), 2e-5, "codebook weight decoded in the kernel, static entry point")
+        ctx.set_option(flib.OPT_CODEBOOK_EXPANDED, 1)
         with pytest.raises(flib.FnnError) as e:
             ctx.qmatmul_static(h, da.ptr, m, d_got.ptr)
         assert e.value.kind == "Memory" and "fnn_hip_qmatmul_static" in e.value.message
