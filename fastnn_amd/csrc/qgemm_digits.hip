@@ -312,9 +312,10 @@ int fnn_digits_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w,
     if (dt != FNN_DT_I8 && dt != FNN_DT_I4 && dt != FNN_DT_U4) return FNN_OK;
     // exact i32 sums: |digit| <= 128, |lane| <= 128 (16*q for 4-bit signed lanes) -> K * 2^14 < 2^31
     if (q.m > (1 << 22) || q.n > (1 << 24) || q.k > (1 << 16)) return FNN_OK;
+    if (q.words != w->words) return FNN_OK;   // (a row slice of a weight: the zero margin behind the last row is not behind the slice)
     QMatmulArgs qa = q;
     int rc;
-    if (q.words == w->words && (rc = fnn_aligned_rows(ctx, s, w, &qa.words, &qa.kp))) return rc;
+    if ((rc = fnn_aligned_rows(ctx, s, w, &qa.words, &qa.kp))) return rc;
     if (qa.kp % 4 != 0 || (reinterpret_cast<uintptr_t>(qa.words) & 15)) return FNN_OK;
     // The single-rounding mode stays with the f16 tiles: two digit planes (15 bits below the row maximum) were 15 %
     // faster than one f16 row but measured 1.9e-3 on rows with a few 200x outliers, where a float rounding per
