@@ -98,7 +98,7 @@ enum {
     FNN_OPT_TILE_SPLIT = 6,       /* tiled GEMM: K split over this many workgroups; 0 (default) = cost model        */
     FNN_OPT_TILE_STAGES = 7,      /* tiled GEMMs: LDS ring depth where the shape has variants (3..6); 0 (default) = by shape */
     FNN_OPT_TILE_MIN_M = 8,       /* smallest M the tiled GEMM takes (default 5)                                    */
-    FNN_OPT_GEMV_INT8 = 9,        /* 1 (default): M <= 4 with I8 / I4 / U4 weights runs on the int8 matrix cores        */
+    FNN_OPT_GEMV_INT8 = 9,        /* 1 (default): M <= 8 with I8 / I4 / U4 weights runs on the int8 matrix cores        */
                                   /* (activations as four exact base-256 digit rows, integer sums, no weight decode);  */
                                   /* 0: the f16 GEMV kernel takes them too                                             */
     FNN_OPT_GEMM_INT8 = 10,       /* 1 (default): M >= FNN_OPT_GEMM_INT8_MIN_M with I8 / I4 / U4 weights runs as an int8  */
@@ -108,7 +108,9 @@ enum {
     FNN_OPT_CODEBOOK_EXPANDED = 12, /* codebook weights with blocks of 32 at M >= 5: 0 (default) = by M (decoded inside the */
                                   /* tiled GEMM where that measured faster), 1 = always through the expanded f16 hi + lo  */
                                   /* operand (FNN_OPT_CODEBOOK_CACHE), 2 = always decoded inside the tiled GEMM           */
-    FNN_OPT_COUNT = 13
+    FNN_OPT_GEMV_INT8_MAX_M = 13, /* largest M the int8 GEMV kernel takes, 1..16 (default 8: beyond that the f16 16-row      */
+                                  /* kernel measured faster, the activation chunks being converted one after the other)   */
+    FNN_OPT_COUNT = 14
 };
 int fnn_hip_set_option(fnn_hip_ctx *ctx, int option, int64_t value);
 int fnn_hip_get_option(fnn_hip_ctx *ctx, int option, int64_t *value);

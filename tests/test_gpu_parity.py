@@ -164,13 +164,14 @@ def test_qmatmul_row_tile_kernels(ctx, orc, dt, m, k, n):
 # int8 GEMV: wide N, partial last slice, two slices per wave (K > 4096), four-wave workgroups (K <= 2048), a single
 # tile, ragged N, every row count
 INT8_GEMV_SHAPES = [(1, 4096, 8500), (2, 1024, 8500), (3, 520, 4200), (4, 8200, 72), (1, 2048, 16), (4, 4096, 4400), (1, 11008, 4096),
-                    (2, 64, 40)]
+                    (2, 64, 40), (5, 4096, 4400), (7, 520, 300), (8, 2048, 8500), (11, 1032, 200), (16, 4096, 1100)]
 
 
 @pytest.mark.parametrize("dt", [0, 1, 3])
 @pytest.mark.parametrize("m,k,n", INT8_GEMV_SHAPES)
 def test_int8_gemv_kernel(ctx, orc, dt, m, k, n):
-    """M <= 4 with I8 / I4 / U4 weights on the int8 matrix cores (the default for these weights): the activations enter as four
+    """M <= 16 with I8 / I4 / U4 weights on the int8 matrix cores (the default for these weights up to M = 8; chunks of
+    four activation rows against the same packed bytes beyond M = 4): the activations enter as four
     exact base-256 digits (30 bits below the maximum of their 512 k-values) and the sums are exact integers, so the
     result sits well inside the 2e-5 MatMul bound (asserted: 4e-6 of max|ref|, measured 4e-8 .. 2e-6); bias + SiLU
     epilogue."""
@@ -181,6 +182,7 @@ def test_int8_gemv_kernel(ctx, orc, dt, m, k, n):
     bias = (rng.standard_normal(n) * 0.01).astype(np.float32)
     h = ctx.register(pw)
     want = orc.qmatmul(to_oracle(orc, pw), a, order=2, bias=bias, act=3)
+    ctx.set_option(flib.OPT_GEMV_INT8_MAX_M, 16)
     got = ctx.qmatmul(h, a, n, bias=bias, act=3)
     assert_close(got, want, 4e-6, f"int8 gemv {NAMES[dt]} {m}x{k}x{n}")
     try:
@@ -190,23 +192,25 @@ def test_int8_gemv_kernel(ctx, orc, dt, m, k, n):
     finally:
         ctx.set_option(flib.OPT_GEMV_ROW_TILES, 0)
         ctx.set_option(flib.OPT_GEMV_INT8, 1)
+        ctx.set_option(flib.OPT_GEMV_INT8_MAX_M, 8)
     ctx.release(h)
 
 
-def test_int8_gemv_propagates_non_finite_activations(ctx, orc):
+@pytest.mark.parametrize("m", [3, 7])
+def test_int8_gemv_propagates_non_finite_activations(ctx, orc, m):
     """The integer digits cannot carry a NaN or an infinity: the slice scale does, so the affected output rows are NaN
     (the float path gives NaN or inf there) and the other rows are untouched."""
     rng = np.random.default_rng(3800)
-    m, k, n = 3, 1024, 64
+    k, n = 1024, 64
     pw = fastnn_amd.quantize_weights(flib.DT_I8, _weights(rng, n, k))
     a = rng.standard_normal((m, k)).astype(np.float32)
     h = ctx.register(pw)
     clean = ctx.qmatmul(h, a, n)
     a[0, 700] = np.nan
-    a[2, 3] = np.inf
+    a[m - 1, 3] = np.inf
     got = ctx.qmatmul(h, a, n)
-    assert np.isnan(got[0]).all() and np.isnan(got[2]).all()
-    assert np.array_equal(got[1], clean[1])
+    assert np.isnan(got[0]).all() and np.isnan(got[m - 1]).all()
+    assert np.array_equal(got[1:m - 1], clean[1:m - 1])
     ctx.release(h)
 
 
@@ -597,10 +601,12 @@ def test_error_paths_mirror_reference_messages(ctx):
 # --------------------------------------------------------------------------- matrix-core specifics
 @pytest.mark.parametrize("dt", [0, 1, 4, 6])
 @pytest.mark.parametrize("mag", [1e-30, 1e-6, 1.0, 3e4, 1e9, 1e30])
-def test_mfma_activation_range_is_f32(ctx, orc, dt, mag):
-    """Activations far outside f16 range: the per-row power-of-two scaling keeps f32 accuracy."""
+@pytest.mark.parametrize("m", [3, 6, 14, 40])
+def test_mfma_activation_range_is_f32(ctx, orc, dt, mag, m):
+    """Activations far outside f16 range: the power-of-two scaling (per row, or per row and K slice) keeps f32
+    accuracy in every kernel of the M range (GEMV kernels, 16-row kernel, tiled GEMMs)."""
     rng = np.random.default_rng(7000 + dt)
-    m, k, n = 6, 2048, 48
+    k, n = 2048, 48
     pw = fastnn_amd.quantize_weights(dt, _weights(rng, n, k))
     a = (rng.standard_normal((m, k)) * mag).astype(np.float32)
     a[1] *= 1e-3          # rows of very different magnitude
