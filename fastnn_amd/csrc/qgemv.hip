@@ -352,15 +352,10 @@ hipError_t launch_qgemv(int dtype, const QMatmulArgs &p, hipStream_t s, bool *ha
     case FNN_DT_F8R: return launch_dt<FNN_DT_F8R>(p, s);
     case FNN_DT_F4: return launch_dt<FNN_DT_F4>(p, s);
     case FNN_DT_I4CB: {
-        // two activation rows per pass (a lane keeps 32 activations per row in registers)
-        QMatmulArgs q = p;
-        for (int64_t m0 = 0; m0 < p.m; m0 += 2) {
-            q.a = p.a + m0 * p.k;
-            q.out = p.out + m0 * p.n;
-            q.m = p.m - m0 < 2 ? p.m - m0 : 2;
-            const hipError_t e = q.m == 1 ? launch_codebook<1>(q, s) : launch_codebook<2>(q, s);
-            if (e != hipSuccess) return e;
-        }
+        // up to four activation rows in one pass: the looked-up block values are used by every row (a lane keeps 32
+        // activations per row in registers: 128 at four rows)
+        const hipError_t e = p.m == 1 ? launch_codebook<1>(p, s) : (p.m == 2 ? launch_codebook<2>(p, s) : (p.m == 3 ? launch_codebook<3>(p, s) : launch_codebook<4>(p, s)));
+        if (e != hipSuccess) return e;
         return hipSuccess;
     }
     default: *handled = false; return hipSuccess;
