@@ -447,6 +447,32 @@ def free_ring(ctx, r):
         r["dbias"].free()
 
 
+def time_i8act(ctx, flib, r, m, calls=200):
+    """matmul_i8_i8 / matmul_i4_i8: I8 activation payload x packed weights (quantised once on the host, resident),
+    eager launches over the weight ring.  Integer ops 2*M*K*N against the nominal int8 peak."""
+    import ctypes as C
+    k, n, ring = r["k"], r["n"], r["ring"]
+    x = np.random.default_rng(2).standard_normal((m, k)).astype(np.float32)
+    payload = ctx.quantize_activations(x)
+    dp, dout = ctx.to_device(payload), ctx.alloc(m * n * 4)
+    vp = C.c_void_p
+
+    def call(i):
+        ctx._check(ctx.lib.fnn_hip_qmatmul_i8act(ctx.handle, r["handles"][i % ring], vp(dp.ptr), m, vp(dout.ptr), None, flib.FLAG_DEVICE_PTRS))
+
+    for i in range(ring):
+        call(i)
+    ctx.sync()
+    ctx.timer_start()
+    for i in range(calls):
+        call(i)
+    us = ctx.timer_stop() * 1e3 / calls
+    dp.free()
+    dout.free()
+    tops = 2.0 * m * k * n / us / 1e6
+    return {"us": round(us, 2), "top_per_s": round(tops, 1), "frac": round(tops / MFMA_PEAK_TFLOPS["i8"], 4), "peak": MFMA_PEAK_TFLOPS["i8"], "calls": calls}
+
+
 def time_matmul(ctx, flib, r, m, steps_min, warmup, mode, flags=0, a_seed=0):
     """`steps_min` or more MatMul calls at M = m over the ring, rounded up to whole trips and to at least 20 of them.
     graph mode: one HIP graph = one trip round the ring.  Returns the continuous figure (events around all trips:
@@ -706,6 +732,8 @@ def main() -> int:
                 gemm_m256[wl] = {
                     "default": gemm_summary(r2, 256, time_matmul(ctx, flib, r2, 256, 200, r2["ring"], "eager", 0, a_seed=1)),
                     "f16x1": gemm_summary(r2, 256, time_matmul(ctx, flib, r2, 256, 200, r2["ring"], "eager", flib.FLAG_ACT_F16_SINGLE, a_seed=1))}
+            if wl == "c1_i8":
+                gemm_m256["c1_i8_i8act"] = time_i8act(ctx, flib, r2, 256)
             free_ring(ctx, r2)
 
     out = {

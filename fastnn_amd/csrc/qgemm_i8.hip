@@ -80,7 +80,7 @@ __global__ void __launch_bounds__(256) i8_rows_operand_kernel(const int8_t *qa, 
 // formed here from the integer sums: sum (q_a*sa + za)*q_w = sa*acc + za*sum_k q_w.
 __global__ void __launch_bounds__(256) i8_matmul_epilogue_kernel(const int32_t *c, const uint8_t *payload, const int32_t *qsum,
                                                                  const int32_t *wsum, const float *scales, const float *zeros,
-                                                                 int64_t m, int64_t n, int64_t k, float *out, int32_t *acc_out)
+                                                                 int64_t m, int64_t n, int64_t k, float *out, int32_t *acc_out, int splits)
 {
     // a thread owns one output column (its weight constants stay in registers) and walks rows blockIdx.y, +gridDim.y, ...
     const float sa = reinterpret_cast<const float *>(payload)[0];
@@ -92,7 +92,8 @@ __global__ void __launch_bounds__(256) i8_matmul_epilogue_kernel(const int32_t *
     const float kza = (float)k * za;
     for (int64_t r = blockIdx.y; r < m; r += gridDim.y) {
         const int64_t idx = r * n + col;
-        const int acc = c[idx];
+        int acc = c[idx];
+        for (int z = 1; z < splits; z++) acc += c[(int64_t)z * m * n + idx];   // exact whatever the order
         const float input_sum = (float)qsum[r] * sa + kza;
         const float dot = (za != 0.0f) ? (float)acc * sa + zwsum : (float)acc * sa;
         out[idx] = dot * sw + zw * input_sum;
@@ -379,7 +380,7 @@ hipError_t launch_i8_tile(const TileArgs &p, hipStream_t s)
     static std::atomic<uint64_t> lds_raised{0};
     hipError_t e = fnn_raise_lds_limit(lds_raised, reinterpret_cast<const void *>(kern), (int)lds);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(kern, dim3((unsigned)p.mtiles * p.ntiles), dim3(256), lds, s, p);
+    hipLaunchKernelGGL(kern, dim3((unsigned)p.mtiles * p.ntiles * p.splits), dim3(256), lds, s, p);
     return hipGetLastError();
 }
 
@@ -419,7 +420,7 @@ namespace {
 // C[m][n] = sum_k A8[m][k] * q_w[n0 + n][k] for `n` weight rows starting at row n0 (rows of kp words, 16-byte aligned)
 template <int DT>
 hipError_t run_i8_gemm(const uint32_t *words, int64_t kp, int64_t rows_total, int64_t n0, int64_t n, const int8_t *a8, int64_t m,
-                       int64_t rows_pad, int64_t kpad, int32_t *c, int64_t ldc, hipStream_t s)
+                       int64_t rows_pad, int64_t kpad, int32_t *c, int64_t ldc, hipStream_t s, int splits = 1)
 {
     TileArgs t = {};
     t.words = words + n0 * kp;
@@ -427,7 +428,10 @@ hipError_t run_i8_gemm(const uint32_t *words, int64_t kp, int64_t rows_total, in
     t.ap = reinterpret_cast<const _Float16 *>(a8);
     t.c_i32 = c; t.ldc = ldc;
     t.m = m; t.n = n; t.kp = kp; t.kpad = kpad; t.rows_pad = rows_pad;
-    t.splits = 1; t.iters = (int)(kpad / KB); t.ips = t.iters; t.mtiles = (int)(rows_pad / 128); t.a_wrap = 0;
+    t.iters = (int)(kpad / KB);
+    t.ips = (t.iters + splits - 1) / splits;
+    t.splits = (t.iters + t.ips - 1) / t.ips;   // (no empty split; the caller sized c for `splits` partial matrices)
+    t.mtiles = (int)(rows_pad / 128); t.a_wrap = 0;
     if (n <= 64) {   // narrow outputs (early conv layers): 128 x 64 tiles, four waves stacked along M
         t.ntiles = (int)((n + 63) / 64);
         return launch_i8_tile<DT, 4, 1, 1, 2, 3>(t, s);
@@ -450,8 +454,16 @@ int fnn_i8_tiled_matmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w
     const size_t q_off = (a_bytes + 255) / 256 * 256;
     void *ws0 = nullptr, *ws1 = nullptr;
     int rc;
+    // K split over workgroups while the tiles alone leave CUs idle: the partial matrices are exact integers, so the
+    // epilogue adds them in any order (4096 x 4096 at M = 256: 64 tiles, 31 -> 24 us with four K ranges)
+    const int64_t tiles = (rows_pad / 128) * (p.n <= 64 ? (p.n + 63) / 64 : (p.n + 127) / 128);
+    const int iters = (int)(kpad / KB);
+    int splits = (int)(256 / (tiles > 0 ? tiles : 1));
+    if (splits > iters / 4) splits = iters / 4;
+    if (splits > 16) splits = 16;
+    if (splits < 1) splits = 1;
     if ((rc = fnn_ctx_ensure_tmp(ctx, 0, q_off + (size_t)rows_pad * 4 + 256, &ws0))) return rc;
-    if ((rc = fnn_ctx_ensure_tmp(ctx, 1, (size_t)p.m * p.n * 4 + 256, &ws1))) return rc;
+    if ((rc = fnn_ctx_ensure_tmp(ctx, 1, (size_t)splits * p.m * p.n * 4 + 256, &ws1))) return rc;
     fnn_hip_weight *wm = const_cast<fnn_hip_weight *>(w);
     if (!wm->row_qsum) {
         if (fnn_ctx_no_alloc(ctx)) return fnn_ctx_fail(ctx, FNN_ERR_MEMORY, "first use of re-strided weight rows while allocation is not allowed (graph capture, fnn_hip_qmatmul_static)");
@@ -475,15 +487,17 @@ int fnn_i8_tiled_matmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w
                            reinterpret_cast<const int8_t *>(p.payload + 8), p.m, p.k, kpad, rows_pad, a8, qsum);
     hipError_t e = hipGetLastError();
     if (e == hipSuccess)
-        e = w->dtype == FNN_DT_I8 ? run_i8_gemm<FNN_DT_I8>(words, kp, w->rows, 0, p.n, a8, p.m, rows_pad, kpad, c, p.n, s)
-                                  : run_i8_gemm<FNN_DT_I4>(words, kp, w->rows, 0, p.n, a8, p.m, rows_pad, kpad, c, p.n, s);
+        e = w->dtype == FNN_DT_I8 ? run_i8_gemm<FNN_DT_I8>(words, kp, w->rows, 0, p.n, a8, p.m, rows_pad, kpad, c, p.n, s, splits)
+                                  : run_i8_gemm<FNN_DT_I4>(words, kp, w->rows, 0, p.n, a8, p.m, rows_pad, kpad, c, p.n, s, splits);
     if (e == hipSuccess) {
+        const int ips = (iters + splits - 1) / splits;
+        splits = (iters + ips - 1) / ips;   // as run_i8_gemm rounds it
         const int64_t colb = (p.n + 255) / 256;
         int64_t rowb = (4096 + colb - 1) / colb;   // about 4096 workgroups
         if (rowb > p.m) rowb = p.m;
         if (rowb > 65535) rowb = 65535;
         hipLaunchKernelGGL(i8_matmul_epilogue_kernel, dim3((unsigned)colb, (unsigned)rowb), dim3(256), 0, s, c, p.payload, qsum, wm->row_qsum,
-                           p.scales, p.zeros, p.m, p.n, p.k, p.out, p.acc_out);
+                           p.scales, p.zeros, p.m, p.n, p.k, p.out, p.acc_out, splits);
         e = hipGetLastError();
     }
     if (e != hipSuccess) return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, hipGetErrorString(e));

@@ -497,7 +497,7 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
                     const float bits = acc[tm][tn][i];   // (bit_cast on a vector element would read element 0)
                     int v = __float_as_int(bits);
                     if constexpr (DT == FNN_DT_I4) v >>= 4;
-                    p.c_i32[m * p.ldc + n] = v;
+                    p.c_i32[((int64_t)z * p.m + m) * p.ldc + n] = v;   // (K split: one exact partial matrix per split)
                 }
             }
         return;
