@@ -43,6 +43,18 @@ WORKLOADS = {
 }
 
 
+def parsed_options(args, flib):
+    """--opt NAME=VALUE items as (name, OPT_* identifier, value)."""
+    out = []
+    for item in args.opt:
+        name, _, value = item.partition("=")
+        ident = getattr(flib, "OPT_" + name.strip().upper(), None)
+        if ident is None or not value.strip().lstrip("-").isdigit():
+            raise ValueError(f"unknown option {item!r}")
+        out.append((name.strip().lower(), ident, int(value)))
+    return out
+
+
 # composite configurations: (kind, parameter)
 COMPOSITE = {
     "c4_mlp_f8": ("mlp", "f8"), "c4_mlp_f4": ("mlp", "f4"),
@@ -210,6 +222,8 @@ def composite(args) -> int:
         t0 = time.perf_counter()
         ex = AotExecutor(nodes, params, ["x"], outs, {"x": shape}, quantize=8)
         build_s = time.perf_counter() - t0
+        for _, ident, value in parsed_options(args, flib):
+            ex.set_option(ident, value)
         ex.write_inputs({"x": rng.uniform(0, 1, shape).astype(np.float32)})
         for _ in range(2 + warm):
             ex.dispatch()
@@ -226,7 +240,8 @@ def composite(args) -> int:
                "value": round(batch / (ms * 1e-3), 1), "unit": "images/s", "n_gpus": 1, "steps": steps, "warmup": warm,
                "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "i8/i32",
                "data": "synthetic", "config": {"workload": args.workload, "launch": "AotExecutor plan, HIP-graph replay + sync per step",
-                                               "instructions": kinds, "arena_bytes": ex.arena_size},
+                                               "instructions": kinds, "arena_bytes": ex.arena_size,
+                                               "options": {n: v for n, _, v in parsed_options(args, flib)}},
                "tops": round(flops / (ms * 1e-3) / 1e12, 2), "replayed": ex.replayed, "lowering_s": round(build_s, 2),
                "outputs": [list(t.shape) for t in y], "finite_output": bool(all(np.isfinite(t).all() for t in y))}
         print(json.dumps(out))
@@ -234,6 +249,8 @@ def composite(args) -> int:
         return 0
     batch = par
     ctx = fastnn_amd.HipContext(0)
+    for _, ident, value in parsed_options(args, flib):
+        ctx.set_option(ident, value)
     layers_ = []
     flops = 0.0
     for (c, h, oc, k, s) in yolo_convs():
@@ -275,7 +292,8 @@ def composite(args) -> int:
     out = {"metric": f"C5 YOLOv8n-shaped I8 conv list forward ({len(layers_)} convs + bias + SiLU, B={batch})",
            "value": round(batch / (ms * 1e-3), 1), "unit": "images/s", "n_gpus": 1, "steps": steps, "warmup": warm,
            "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "i8/i32",
-           "data": "synthetic", "config": {"workload": args.workload, "launch": args.mode + ", each conv on its own resident input"},
+           "data": "synthetic", "config": {"workload": args.workload, "launch": args.mode + ", each conv on its own resident input",
+                                           "options": {n: v for n, _, v in parsed_options(args, flib)}},
            "event_ms_per_step": round(ev, 4), "gop_per_step": round(flops / 1e9, 2), "top_per_s": round(flops / (ms * 1e-3) / 1e12, 2)}
     print(json.dumps(out))
     ctx.close()
@@ -593,6 +611,11 @@ def main() -> int:
     import fastnn_amd
     from fastnn_amd import lib as flib
 
+    try:
+        parsed_options(args, flib)
+    except ValueError as e:
+        print(f"bench.py: {e}", file=sys.stderr)
+        return 2
     if args.workload in COMPOSITE:
         return composite(args)
 
@@ -600,14 +623,9 @@ def main() -> int:
     flags = flib.FLAG_ACT_F16_SINGLE if args.fast_act16 else 0
     ctx = fastnn_amd.HipContext(0)
     opts = {}
-    for item in args.opt:
-        name, _, value = item.partition("=")
-        ident = getattr(flib, "OPT_" + name.strip().upper(), None)
-        if ident is None or not value.strip().lstrip("-").isdigit():
-            print(f"bench.py: unknown option {item!r}", file=sys.stderr)
-            return 2
-        ctx.set_option(ident, int(value))
-        opts[name.strip().lower()] = int(value)
+    for name, ident, value in parsed_options(args, flib):
+        ctx.set_option(ident, value)
+        opts[name] = value
     probe = Probe(ctx)
     if args.probe == "mfma":
         res = probe.mfma_ceiling()

@@ -385,6 +385,11 @@ class AotExecutor:
             out[name] = self._backend.read_arena(*v.slot, np.float32).reshape(v.shape).copy()
         return out
 
+    def set_option(self, option: int, value: int):
+        """Kernel-selection option of the backend's context (lib.OPT_* constants)."""
+        self._ensure_plan()
+        self._backend.set_option(option, value)
+
     def write_inputs(self, inputs: Dict[str, np.ndarray]):
         """Copies the inputs into their arena slots (what forward() does first)."""
         self._ensure_plan()

@@ -128,6 +128,7 @@ const OptionSpec kOptions[FNN_OPT_COUNT] = {
     {17, 1, 1 << 20}, // FNN_OPT_GEMM_INT8_MIN_M
     {0, 0, 2},        // FNN_OPT_CODEBOOK_EXPANDED
     {8, 1, 16},       // FNN_OPT_GEMV_INT8_MAX_M
+    {0, 0, 3},        // FNN_OPT_CONV_EPILOGUE
 };
 
 #define HIP_TRY(ctx, code, expr)                                                              \

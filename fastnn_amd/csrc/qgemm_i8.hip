@@ -104,15 +104,35 @@ __global__ void __launch_bounds__(256) i8_matmul_epilogue_kernel(const int32_t *
 // ---- conv operand: im2col row (image nn, pixel p) of group g, quantised with the (image, group) scale:
 // q = clamp(round((v - za) * inv), -128, 127)  (packed_conv.rs:149-232); for an input that is already int8
 // (X8) the values are taken as they are and padding taps are the integer 0 (packed_conv.rs:69-115).
-// A workgroup owns 64 consecutive rows and CONV_CPB 16-value chunks of them: wave `slot` takes one chunk, so the
-// (channel, tap) geometry of a chunk is the same for the whole wave and neighbouring lanes = neighbouring pixels
-// (the NCHW reads coalesce).  The 16 loads of a chunk go to clamped, always valid addresses and are masked
-// afterwards: no branch sits between them, so all of them are in flight together.
-constexpr int CONV_CPB = 4;   // 16-value chunks of a row per workgroup (one per wave)
+// A workgroup owns 64 consecutive rows and CONV_CPB * NC 16-value chunks of them: wave `slot` takes NC consecutive
+// chunks, so the (channel, tap) geometry is the same for the whole wave and lives in scalar registers, neighbouring
+// lanes = neighbouring pixels (the NCHW reads coalesce), and what a lane works out about its pixel (image, position,
+// which kernel rows and columns fall inside the image) is paid once per NC * 16 taps.  All loads of a wave are
+// requested before the first value is used.
+constexpr int CONV_CPB = 4;   // waves per workgroup, each with its own chunks
 
-template <bool X8, bool W4>   // X8: int8 input; W4: 4-bit weights (16 activation levels unless X8, interleaved operand)
+// n / d for 0 <= n < 2^31 by one multiplication (d >= 1 fixed per launch): mul = ceil(2^(31 + ceil(log2 d)) / d)
+struct FastDiv {
+    uint32_t d, mul, shr;
+    __device__ __forceinline__ uint32_t div(uint32_t n) const { return d == 1 ? n : __umulhi(n, mul) >> shr; }
+};
+inline FastDiv fast_div(uint32_t d)
+{
+    FastDiv f = {d, 0, 0};
+    if (d <= 1) { f.d = 1; return f; }
+    uint32_t lg = 0;
+    while ((1ull << lg) < d) lg++;
+    const uint64_t p2 = 1ull << (31 + lg);
+    f.mul = (uint32_t)((p2 + d - 1) / d);
+    f.shr = lg - 1;
+    return f;
+}
+struct ConvDivs { FastDiv np, wo, khw, kw; };
+
+template <bool X8, bool W4, int NC>   // X8: int8 input; W4: 4-bit weights (16 activation levels unless X8, interleaved operand)
+                                      // NC <= 4: a wave's taps are worked out one per lane
 __global__ void __launch_bounds__(256) conv_operand_kernel(QConvArgs a, int g, int kk, int64_t kpad, int64_t rows_pad,
-                                                           int8_t *a8, int32_t *qsum)
+                                                           int8_t *a8, int32_t *qsum, ConvDivs dv)
 {
     __shared__ int part[4][64];
     const int tid = threadIdx.x, rr = tid & 63;
@@ -123,7 +143,7 @@ __global__ void __launch_bounds__(256) conv_operand_kernel(QConvArgs a, int g, i
     const int cg = (int)a.c / a.groups;
     const int live_chunks = (kk + 15) / 16;
     const bool live = r < rows;
-    const int c = (int)blockIdx.y * CONV_CPB + slot;
+    const int c0 = ((int)blockIdx.y * CONV_CPB + slot) * NC;   // this wave's first chunk
     // Scales not formed yet (a.nparts > 0): every workgroup reduces the partial ranges of the (at most two) images
     // its 64 rows belong to and derives scale, zero and 1/scale exactly as conv_actq_kernel does; the workgroups of
     // the first chunk group also store them for the epilogue.
@@ -131,11 +151,12 @@ __global__ void __launch_bounds__(256) conv_operand_kernel(QConvArgs a, int g, i
     __shared__ float s_q[2][3];
     const int64_t r_first = (int64_t)blockIdx.x * 64;
     const bool own_scales = !X8 && a.nparts > 0 && r_first < rows;
+    const uint32_t nn0 = dv.np.div((uint32_t)(r_first < rows ? r_first : 0));   // image of the workgroup's first row
     int bg_a = 0;
     if (own_scales) {
         const int64_t r_last = r_first + 63 < rows ? r_first + 63 : rows - 1;
-        bg_a = (int)((uint32_t)r_first / np) * a.groups + g;
-        const int bg_b = (int)((uint32_t)r_last / np) * a.groups + g;
+        bg_a = (int)nn0 * a.groups + g;
+        const int bg_b = (int)dv.np.div((uint32_t)r_last) * a.groups + g;
         const int nimg = bg_b != bg_a ? 2 : 1;
         for (int w = 0; w < nimg; w++) {
             const float *part = a.minmax_partial + (int64_t)(w ? bg_b : bg_a) * QCONV_NPART * 2;
@@ -171,10 +192,10 @@ __global__ void __launch_bounds__(256) conv_operand_kernel(QConvArgs a, int g, i
         __syncthreads();
     }
     int s = 0;
-    if (r < rows_pad && c < live_chunks) {
+    if (r < rows_pad && c0 < live_chunks) {
         const uint32_t ru = live ? (uint32_t)r : 0u;
-        const uint32_t nn = ru / np, p = ru - nn * np;
-        const uint32_t oh = p / wo, ow = p - oh * wo;
+        const uint32_t nn = dv.np.div(ru), p = ru - nn * np;
+        const uint32_t oh = dv.wo.div(p), ow = p - oh * wo;
         const int bg = (int)nn * a.groups + g;
         float za, inv;
         if (X8 || a.nparts <= 0) {
@@ -183,56 +204,98 @@ __global__ void __launch_bounds__(256) conv_operand_kernel(QConvArgs a, int g, i
             const int w = (own_scales && bg != bg_a) ? 1 : 0;
             za = own_scales ? s_q[w][1] : 0.0f; inv = own_scales ? s_q[w][2] : 0.0f;
         }
-        const int64_t x_off = ((int64_t)nn * a.c + (int64_t)g * cg) * a.h * a.w;
-        const float *xg = a.x + x_off;
-        const int8_t *xq = a.x8 + x_off;
-        const int khw = a.kh * a.kw, hh = (int)a.h, ww = (int)a.w;
+        // One buffer descriptor per wave, from the group's slab in the image of the workgroup's first row to the end
+        // of the tensor: a lane's byte offset is (images further on) * image size + pixel offset + tap offset, and a
+        // tap outside the image (or past K, or of a row past the last one) gets the offset ~0, which the buffer
+        // range check answers with zero: no branch, no select on the loaded value (the host checked that the offsets
+        // of one workgroup fit 32 bits).
+        constexpr uint32_t ESZ = X8 ? 1 : 4;
+        const int64_t img = a.c * a.h * a.w;
+        const int64_t slab0 = ((int64_t)nn0 * a.c + (int64_t)g * cg) * a.h * a.w;
+        const void *base = X8 ? (const void *)(a.x8 + slab0) : (const void *)(a.x + slab0);
+        const int64_t left = (a.b * img - slab0) * ESZ;   // bytes from there to the end of the tensor
+        const __amdgpu_buffer_rsrc_t xbuf = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<void *>(base), 0, (int)(uint32_t)(left > 0xfffffff0ll ? 0xfffffff0ll : left), 0x00020000);
+        const int hh = (int)a.h, ww = (int)a.w;
         constexpr int qlo = W4 ? -8 : -128, qhi = W4 ? 7 : 127;
         constexpr int interleaved = W4;   // the 4-bit weight decoder delivers k = 0,2,4,6,1,3,5,7 of each 8
         const int ih0 = (int)oh * a.stride - a.pad, iw0 = (int)ow * a.stride - a.pad;
-        // tap geometry of the chunk (the same for every lane of the wave), advanced by carries.
-        // Rows past the last one (r >= rows) compute pixel 0 of image 0: their bytes only reach accumulator
-        // rows and row sums that nothing reads.
-        const int e0 = c * 16;
-        int ic = e0 / khw, rem = e0 - ic * khw;
-        int i = rem / a.kw, j = rem - i * a.kw;
-        int off[16];
-        uint32_t inside = 0;
-#pragma unroll
-        for (int t = 0; t < 16; t++) {
-            const int ih = ih0 + i * a.dil, iw = iw0 + j * a.dil;
-            const bool in = e0 + t < kk && (unsigned)ih < (unsigned)hh && (unsigned)iw < (unsigned)ww;
-            off[t] = in ? (ic * hh + ih) * ww + iw : 0;   // < 2^31 (checked on the host)
-            inside |= in ? (1u << t) : 0u;
-            if (++j == a.kw) { j = 0; if (++i == a.kh) { i = 0; ic++; } }
+        // which kernel rows (bits 0..14) and columns (bits 16..30) land inside the image for this pixel; bit 31 stays
+        // clear: taps past K ask for it
+        uint32_t okbits = 0;
+        for (int i = 0; i < a.kh; i++) okbits |= ((unsigned)(ih0 + i * a.dil) < (unsigned)hh ? 1u : 0u) << i;
+        for (int j = 0; j < a.kw; j++) okbits |= ((unsigned)(iw0 + j * a.dil) < (unsigned)ww ? 0x10000u : 0u) << j;
+        if (!live) okbits = 0;
+        const uint32_t lane_base = ((uint32_t)(nn - nn0) * (uint32_t)img + (uint32_t)(ih0 * ww + iw0)) * ESZ;   // (mod 2^32)
+        // Tap geometry: lane t works out tap e0 + t of this wave (channel, kernel row, kernel column -> offset inside
+        // the slab and the two bits the tap needs), and the unrolled loop below reads each tap's pair into scalar
+        // registers: no per-tap index arithmetic on either unit.
+        const int e0 = c0 * 16;
+        uint32_t tap_off, tap_need;
+        {
+            const uint32_t e = (uint32_t)(e0 + rr);
+            const uint32_t ic = dv.khw.div(e), rem = e - ic * (uint32_t)(a.kh * a.kw);
+            const uint32_t i = dv.kw.div(rem), j = rem - i * (uint32_t)a.kw;
+            tap_off = ((ic * (uint32_t)hh + i * (uint32_t)a.dil) * (uint32_t)ww + j * (uint32_t)a.dil) * ESZ;
+            tap_need = (int)e < kk ? ((1u << i) | (0x10000u << j)) : 0x80000000u;
         }
-        float v[16];
-        int v8[16];
+        float v[NC][16];
+        int v8[NC][16];
 #pragma unroll
-        for (int t = 0; t < 16; t++) {
-            if (X8) v8[t] = xq[off[t]];
-            else v[t] = xg[off[t]];
-        }
-        uint32_t out[4] = {0, 0, 0, 0};
+        for (int cc = 0; cc < NC; cc++)
 #pragma unroll
-        for (int t = 0; t < 16; t++) {
-            const bool in = (inside >> t) & 1u;
-            int qi;
-            if (X8) {
-                qi = in ? v8[t] : 0;
-            } else {
-                // round half away from zero, then clamp: trunc(x + copysign(0.49999997, x)) equals roundf(x)
-                // after the clamp for every float (the conversion truncates, saturates and maps NaN to 0)
-                const float x = ((in ? v[t] : 0.0f) - za) * inv;
-                qi = (int)(x + __builtin_copysignf(0.49999997f, x));
-                qi = max(qlo, min(qi, qhi));
-                if (!(e0 + t < kk)) qi = 0;   // past K
+            for (int t = 0; t < 16; t++) {
+                const uint32_t soff = (uint32_t)__builtin_amdgcn_readlane((int)tap_off, cc * 16 + t);
+                const uint32_t need = (uint32_t)__builtin_amdgcn_readlane((int)tap_need, cc * 16 + t);
+                const uint32_t vo = (okbits & need) == need ? lane_base + soff : ~0u;
+                if (X8) v8[cc][t] = (int)(int8_t)__builtin_amdgcn_raw_buffer_load_b8(xbuf, vo, 0, 0);
+                else v[cc][t] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xbuf, vo, 0, 0));
             }
-            s += qi;
-            const int pos = (t & 8) + slot_of(t & 7, interleaved);
-            out[pos >> 2] |= (uint32_t)(uint8_t)qi << (8 * (pos & 3));
+#pragma unroll
+        for (int cc = 0; cc < NC; cc++) {
+            const int c = c0 + cc;
+            if (c >= live_chunks) break;   // (wave-uniform)
+            int q[16];
+#pragma unroll
+            for (int t = 0; t < 16; t++) {
+                if (X8) {
+                    q[t] = v8[cc][t];
+                } else {
+                    // round half away from zero, then clamp: trunc(x + copysign(0.49999997, x)) equals roundf(x)
+                    // after the clamp for every float (the conversion truncates, saturates and maps NaN to 0)
+                    const float x = (v[cc][t] - za) * inv;
+                    const int qi = (int)(x + __builtin_copysignf(0.49999997f, x));
+                    q[t] = max(qlo, min(qi, qhi));
+                }
+            }
+            // byte `pos` of the 16 holds tap (pos & 8) + k(pos & 7), k = the inverse of slot_of; the row sum is a
+            // 4-way dot with ones
+            uint32_t out[4];
+            int tp[16];
+#pragma unroll
+            for (int pos = 0; pos < 16; pos++) {
+                const int sl = pos & 7;
+                tp[pos] = (pos & 8) + (interleaved ? ((sl & 3) * 2 + (sl >> 2)) : sl);
+            }
+#pragma unroll
+            for (int wi = 0; wi < 4; wi++) {
+                const uint32_t lo = __builtin_amdgcn_perm((uint32_t)q[tp[wi * 4 + 1]], (uint32_t)q[tp[wi * 4 + 0]], 0x0c0c0400u);
+                const uint32_t hi = __builtin_amdgcn_perm((uint32_t)q[tp[wi * 4 + 3]], (uint32_t)q[tp[wi * 4 + 2]], 0x04000c0cu);
+                out[wi] = lo | hi;
+            }
+            if (c * 16 + 16 > kk) {   // (wave-uniform) the chunk K ends in: bytes of taps past K are cleared
+#pragma unroll
+                for (int wi = 0; wi < 4; wi++) {
+                    uint32_t keep = 0;
+#pragma unroll
+                    for (int bq = 0; bq < 4; bq++) keep |= (c * 16 + tp[wi * 4 + bq] < kk) ? (0xffu << (8 * bq)) : 0u;
+                    out[wi] &= keep;
+                }
+            }
+#pragma unroll
+            for (int wi = 0; wi < 4; wi++) s = __builtin_amdgcn_sdot4((int)out[wi], 0x01010101, s, false);
+            *reinterpret_cast<uint4 *>(a8 + ((int64_t)(c >> 3) * rows_pad + r) * KB + (c & 7) * 16) = make_uint4(out[0], out[1], out[2], out[3]);
         }
-        *reinterpret_cast<uint4 *>(a8 + ((int64_t)(c >> 3) * rows_pad + r) * KB + (c & 7) * 16) = make_uint4(out[0], out[1], out[2], out[3]);
     }
     part[slot][rr] = s;
     // Chunks past the data (k >= K rounded up to 16) are not written: the weight operand is zero there
@@ -301,7 +364,6 @@ __global__ void __launch_bounds__(256) conv_epilogue_kernel(QConvArgs a, int g, 
     auto element = [&](int rr, int fl, int acc_in) {
         const float sa = r_sa[rr], za = r_za[rr];
         const float sw = c_sw[fl], zw = c_zw[fl];
-        const float sab = sa * sw;
         int accv;
         float val;
         if (a.payload_i4) {
@@ -312,24 +374,12 @@ __global__ void __launch_bounds__(256) conv_epilogue_kernel(QConvArgs a, int g, 
             const float input_sum = r_sum[rr] + (float)kk * za;
             val = dot * sw + zw * input_sum;
             if (a.bias) val += c_bias[fl];
+            if (a.act == FNN_ACT_RELU) val = fmaxf(val, 0.0f);
+            else if (a.act == FNN_ACT_SILU) val = val / (1.0f + expf(-val));
+            else if (a.act == FNN_ACT_GELU) val = val * 0.5f * (1.0f + tanhf(val * 0.7978846f * (1.0f + 0.044715f * val * val)));
         } else {
-            int bias_q = 0;
-            if (a.bias) {
-                // round half away from zero and saturate: trunc(x + copysign(0.49999997, x)) equals roundf(x)
-                // wherever the result fits an i32, and the conversion saturates and maps NaN to 0
-                const float x = c_bias[fl] / sab;
-                bias_q = (int)(x + __builtin_copysignf(0.49999997f, x));
-            }
-            accv = acc_in + bias_q;
-            const float zp_prod = za * zw;
-            val = (float)accv * sab;
-            val = val + zw * r_sum[rr];
-            val = val + za * c_wt[fl];
-            val = val + zp_prod * (float)kk;
+            val = conv_dequant(acc_in, sa, za, r_sum[rr], sw, zw, c_wt[fl], a.bias ? conv_bias_q(c_bias[fl], sa, sw) : 0, kk, a.act, &accv);
         }
-        if (a.act == FNN_ACT_RELU) val = fmaxf(val, 0.0f);
-        else if (a.act == FNN_ACT_SILU) val = val / (1.0f + expf(-val));
-        else if (a.act == FNN_ACT_GELU) val = val * 0.5f * (1.0f + tanhf(val * 0.7978846f * (1.0f + 0.044715f * val * val)));
         tile[fl * 65 + rr] = val;
         itile[fl * 65 + rr] = accv;
     };
@@ -370,13 +420,13 @@ __global__ void __launch_bounds__(256) conv_epilogue_kernel(QConvArgs a, int g, 
     }
 }
 
-template <int DT, int WGM, int WGN, int TM, int TN, int NS>
+template <int DT, int WGM, int WGN, int TM, int TN, int NS, bool CONV = false>
 hipError_t launch_i8_tile(const TileArgs &p, hipStream_t s)
 {
     constexpr int WC = 2 * DecI<DT>::WPS;
     constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
     constexpr size_t lds = (size_t)NS * (BM * 128 + BN * WC * 16);
-    auto kern = qgemm_tile_kernel<DT, WGM, WGN, TM, TN, false, NS, true>;
+    auto kern = qgemm_tile_kernel<DT, WGM, WGN, TM, TN, false, NS, true, 0, CONV>;
     static std::atomic<uint64_t> lds_raised{0};
     hipError_t e = fnn_raise_lds_limit(lds_raised, reinterpret_cast<const void *>(kern), (int)lds);
     if (e != hipSuccess) return e;
@@ -418,11 +468,14 @@ int fnn_aligned_rows(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, c
 namespace {
 
 // C[m][n] = sum_k A8[m][k] * q_w[n0 + n][k] for `n` weight rows starting at row n0 (rows of kp words, 16-byte aligned)
+// `conv` (optional): the conv epilogue runs inside the kernel (scales / zeros / bias / act in it are the group's) and c is not written
 template <int DT>
 hipError_t run_i8_gemm(const uint32_t *words, int64_t kp, int64_t rows_total, int64_t n0, int64_t n, const int8_t *a8, int64_t m,
-                       int64_t rows_pad, int64_t kpad, int32_t *c, int64_t ldc, hipStream_t s, int splits = 1)
+                       int64_t rows_pad, int64_t kpad, int32_t *c, int64_t ldc, hipStream_t s, int splits = 1, const TileArgs *conv = nullptr,
+                       bool small_tiles = false)
 {
     TileArgs t = {};
+    if (conv) { t.cv = conv->cv; t.scales = conv->scales; t.zeros = conv->zeros; t.bias = conv->bias; t.act = conv->act; }
     t.words = words + n0 * kp;
     t.zero_chunk = words + rows_total * kp;   // the zeroed margin behind the last row
     t.ap = reinterpret_cast<const _Float16 *>(a8);
@@ -432,12 +485,17 @@ hipError_t run_i8_gemm(const uint32_t *words, int64_t kp, int64_t rows_total, in
     t.ips = (t.iters + splits - 1) / splits;
     t.splits = (t.iters + t.ips - 1) / t.ips;   // (no empty split; the caller sized c for `splits` partial matrices)
     t.mtiles = (int)(rows_pad / 128); t.a_wrap = 0;
+    if (conv && small_tiles) {   // few rows: 64 x 64 tiles put the epilogue's arithmetic on four times as many waves
+        t.mtiles = (int)(rows_pad / 64);
+        t.ntiles = (int)((n + 63) / 64);
+        return launch_i8_tile<DT, 2, 2, 1, 1, 3, true>(t, s);
+    }
     if (n <= 64) {   // narrow outputs (early conv layers): 128 x 64 tiles, four waves stacked along M
         t.ntiles = (int)((n + 63) / 64);
-        return launch_i8_tile<DT, 4, 1, 1, 2, 3>(t, s);
+        return conv ? launch_i8_tile<DT, 4, 1, 1, 2, 3, true>(t, s) : launch_i8_tile<DT, 4, 1, 1, 2, 3>(t, s);
     }
     t.ntiles = (int)((n + 127) / 128);
-    return launch_i8_tile<DT, 2, 2, 2, 2, 3>(t, s);
+    return conv ? launch_i8_tile<DT, 2, 2, 2, 2, 3, true>(t, s) : launch_i8_tile<DT, 2, 2, 2, 2, 3>(t, s);
 }
 
 }  // namespace
@@ -514,13 +572,25 @@ int fnn_i8_tiled_conv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, 
     const int64_t cg = p.c / p.groups, ocg = p.oc / p.groups, kk = cg * p.kh * p.kw;
     if (rows < 1 || rows > (1ll << 28) || kk > (1 << 20) || ocg < 1) return FNN_OK;
     if (cg * p.h * p.w >= (1ll << 31) || p.ho * p.wo >= (1ll << 31)) return FNN_OK;   // 32-bit offsets inside an image slab
+    // the operand kernel keeps one validity bit per kernel row / column (15 of each) and addresses the images a workgroup's 64
+    // rows touch with 32-bit byte offsets from the first of them
+    const int64_t span = p.b < 63 / np + 2 ? p.b : 63 / np + 2;
+    if (p.kh > 15 || p.kw > 15 || span * p.c * p.h * p.w * 4 > 0xfffffff0ll) return FNN_OK;
     const int64_t kpad = (kk + KB - 1) / KB * KB;
     const int64_t rows_pad = (rows + 127) / 128 * 128;
     const size_t a_bytes = (size_t)rows_pad * kpad;
     const size_t q_off = (a_bytes + 255) / 256 * 256;
     void *ws1 = nullptr, *ws3 = nullptr;
     int rc;
-    const int nq = (int)(((kk + 15) / 16 + CONV_CPB - 1) / CONV_CPB);   // partial row sums per row
+    // chunks per wave: more of them spread a lane's per-pixel set-up over more taps, fewer keep the launch wide
+    const int64_t chunks = (kk + 15) / 16;
+    const int64_t wg1 = (rows_pad / 64) * ((chunks + CONV_CPB - 1) / CONV_CPB);   // workgroups with one chunk per wave
+    int nc = 1;
+    if (wg1 >= 2048) {   // enough workgroups left: the fewest chunk groups of at most 4 chunks per wave, evenly filled
+        const int64_t groups_max = (chunks + CONV_CPB * 4 - 1) / (CONV_CPB * 4);
+        nc = (int)((chunks + CONV_CPB * groups_max - 1) / (CONV_CPB * groups_max));
+    }
+    const int nq = (int)((chunks + CONV_CPB * nc - 1) / (CONV_CPB * nc));   // partial row sums per row
     if (nq > 65535) return FNN_OK;
     if ((rc = fnn_ctx_ensure_tmp(ctx, 3, q_off + (size_t)rows_pad * 4 * nq + 256, &ws3))) return rc;   // 0 holds the scales
     if ((rc = fnn_ctx_ensure_tmp(ctx, 1, (size_t)rows * ocg * 4 + 256, &ws1))) return rc;
@@ -531,18 +601,42 @@ int fnn_i8_tiled_conv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, 
     int32_t *qsum = (int32_t *)((char *)ws3 + q_off);
     int32_t *c = (int32_t *)ws1;
     if (ocg > 65535 * EPI_CH) return FNN_OK;
+    // the epilogue inside the GEMM kernel (one launch and the accumulator matrix's trip through memory less) or as a
+    // kernel of its own; the matmul-form epilogue of 4-bit weights on an int8 payload exists only as a kernel
+    const int opt_fused = fnn_ctx_option(ctx, FNN_OPT_CONV_EPILOGUE);
+    const bool fused = !p.payload_i4 && opt_fused != 2;
+    const int64_t tiles128 = (rows_pad / 128) * (ocg <= 64 ? 1 : (ocg + 127) / 128);
+    const bool small_tiles = tiles128 <= 256 && opt_fused != 3;   // less than one 128-row tile per CU
+    const bool vec4 = np % 4 == 0 && (reinterpret_cast<uintptr_t>(p.y) & 15) == 0 && (!p.acc_out || (reinterpret_cast<uintptr_t>(p.acc_out) & 15) == 0);
     for (int g = 0; g < p.groups; g++) {
         const dim3 grid((unsigned)(rows_pad / 64), (unsigned)nq);
         const bool w4 = p.wbits == 4;
-        if (p.x8 && w4) hipLaunchKernelGGL((conv_operand_kernel<true, true>), grid, dim3(256), 0, s, p, g, (int)kk, kpad, rows_pad, a8, qsum);
-        else if (p.x8) hipLaunchKernelGGL((conv_operand_kernel<true, false>), grid, dim3(256), 0, s, p, g, (int)kk, kpad, rows_pad, a8, qsum);
-        else if (w4) hipLaunchKernelGGL((conv_operand_kernel<false, true>), grid, dim3(256), 0, s, p, g, (int)kk, kpad, rows_pad, a8, qsum);
-        else hipLaunchKernelGGL((conv_operand_kernel<false, false>), grid, dim3(256), 0, s, p, g, (int)kk, kpad, rows_pad, a8, qsum);
+        const ConvDivs dv = {fast_div((uint32_t)np), fast_div((uint32_t)p.wo), fast_div((uint32_t)(p.kh * p.kw)), fast_div((uint32_t)p.kw)};
+        auto launch = [&](auto kern) { hipLaunchKernelGGL(kern, grid, dim3(256), 0, s, p, g, (int)kk, kpad, rows_pad, a8, qsum, dv); };
+        auto pick = [&](auto x8c, auto w4c) {
+            constexpr bool X8 = decltype(x8c)::value, W4 = decltype(w4c)::value;
+            if (nc == 4) launch(conv_operand_kernel<X8, W4, 4>);
+            else if (nc == 3) launch(conv_operand_kernel<X8, W4, 3>);
+            else if (nc == 2) launch(conv_operand_kernel<X8, W4, 2>);
+            else launch(conv_operand_kernel<X8, W4, 1>);
+        };
+        if (p.x8 && w4) pick(std::true_type{}, std::true_type{});
+        else if (p.x8) pick(std::true_type{}, std::false_type{});
+        else if (w4) pick(std::false_type{}, std::true_type{});
+        else pick(std::false_type{}, std::false_type{});
         hipError_t e = hipGetLastError();
+        TileArgs cv = {};
+        if (fused) {
+            cv.scales = p.scales + g * ocg; cv.zeros = p.zeros + g * ocg; cv.bias = p.bias ? p.bias + g * ocg : nullptr; cv.act = p.act;
+            cv.cv.y = p.y + g * ocg * np; cv.cv.acc_out = p.acc_out ? p.acc_out + g * ocg * np : nullptr;
+            cv.cv.actq = p.actq; cv.cv.qsum = qsum; cv.cv.row_qsum = p.row_qsum + g * ocg;
+            cv.cv.oc = p.oc; cv.cv.np = (uint32_t)np; cv.cv.nq = nq; cv.cv.groups = p.groups; cv.cv.g = g; cv.cv.kk = (int)kk;
+            cv.cv.vec4 = vec4 ? 1 : 0;
+        }
         if (e == hipSuccess)
-            e = w->dtype == FNN_DT_I8 ? run_i8_gemm<FNN_DT_I8>(words, kp, w->rows, g * ocg, ocg, a8, rows, rows_pad, kpad, c, ocg, s)
-                                      : run_i8_gemm<FNN_DT_I4>(words, kp, w->rows, g * ocg, ocg, a8, rows, rows_pad, kpad, c, ocg, s);
-        if (e == hipSuccess) {
+            e = w->dtype == FNN_DT_I8 ? run_i8_gemm<FNN_DT_I8>(words, kp, w->rows, g * ocg, ocg, a8, rows, rows_pad, kpad, c, ocg, s, 1, fused ? &cv : nullptr, small_tiles)
+                                      : run_i8_gemm<FNN_DT_I4>(words, kp, w->rows, g * ocg, ocg, a8, rows, rows_pad, kpad, c, ocg, s, 1, fused ? &cv : nullptr, small_tiles);
+        if (e == hipSuccess && !fused) {
             hipLaunchKernelGGL(conv_epilogue_kernel, dim3((unsigned)((rows + 63) / 64), (unsigned)((ocg + EPI_CH - 1) / EPI_CH)), dim3(256), 0, s, p, g,
                                (int)kk, c, (int)ocg, qsum, nq, rows_pad);
             e = hipGetLastError();

@@ -23,7 +23,56 @@ struct TileArgs {
     const float *bscales;
     const float *codebook;
     int64_t bpr;
+    // quantised Conv2d epilogue inside the int8 kernel (CONV): scales / zeros / bias above are those of the group's
+    // channels; y and acc_out start at the group's first channel of image 0
+    struct Conv {
+        float *y;                  // [B, OC, np]
+        int32_t *acc_out;          // same shape, or null
+        const float *actq;         // [B*groups][4]: activation scale, zero, 1/scale, unused
+        const int32_t *qsum;       // [nq][rows_pad]: partial sums of q_a per im2col row
+        const int32_t *row_qsum;   // [channels of the group]: sum of q_w
+        int64_t oc;
+        uint32_t np;
+        int nq, groups, g, kk;
+        int vec4;                  // np % 4 == 0 and 16-byte aligned outputs: four pixels per store
+    } cv;
 };
+
+// One output of the quantised Conv2d: acc = acc_in + bias_q; val = acc*sab + zw*(sa*sum q_a) + za*(sw*sum q_w)
+// + (za*zw)*K, left to right, then the activation (src/backend/cpu/packed_conv.rs:469-505,571,604-606).
+// rsum = sa * sum q_a of the row, wt = sw * sum q_w of the channel.
+// bias_q = round(bias / (sa*sw)) half away from zero, saturated: trunc(x + copysign(0.49999997, x)) equals roundf(x)
+// wherever the result fits an i32, and the conversion saturates and maps NaN to 0
+__device__ __forceinline__ int conv_bias_q(float bias, float sa, float sw)
+{
+    const float x = bias / (sa * sw);
+    return (int)(x + __builtin_copysignf(0.49999997f, x));
+}
+// x / (1 + exp(-x)) on the hardware exponential and reciprocal (v_exp_f32 of -x*log2(e), v_rcp_f32, one ulp each; the
+// rounded product adds |x| * 6e-8 to the exponential's relative error, which reaches the result scaled by
+// e/(1+e)): a few ulp of the result for x > -4 and below 1e-8 in absolute terms for smaller x, where the result
+// itself vanishes; about 6 instructions against ~35 for expf and an IEEE division.
+__device__ __forceinline__ float conv_silu(float x)
+{
+    const float e = __builtin_amdgcn_exp2f(x * -1.44269504f);   // exp(-x); inf for x < -88.7, 0 for x > 103
+    return x * __builtin_amdgcn_rcpf(1.0f + e);                  // x * 0 = -0 where e = inf, as x / inf
+}
+__device__ __forceinline__ float conv_dequant(int acc_in, float sa, float za, float rsum, float sw, float zw, float wt,
+                                              int bias_q, int kk, int act, int *acc_out)
+{
+    const float sab = sa * sw;
+    const int accv = acc_in + bias_q;
+    const float zp_prod = za * zw;
+    float val = (float)accv * sab;
+    val = val + zw * rsum;
+    val = val + za * wt;
+    val = val + zp_prod * (float)kk;
+    if (act == FNN_ACT_RELU) val = fmaxf(val, 0.0f);
+    else if (act == FNN_ACT_SILU) val = conv_silu(val);
+    else if (act == FNN_ACT_GELU) val = val * 0.5f * (1.0f + tanhf(val * 0.7978846f * (1.0f + 0.044715f * val * val)));
+    *acc_out = accv;
+    return val;
+}
 
 // power of two that brings the largest table magnitude into [2^14, 2^15): the f16 hi + lo split of the scaled table
 // then carries ~22 bits of every entry (every thread computes the same value from the 16 cached floats)
@@ -77,10 +126,14 @@ __device__ __forceinline__ void wait_loads_but()
 //               scaled per row by 2^rexp: a 32-row MFMA block = 32/DIG activation rows x DIG planes (plane j in
 //               block rows [j*32/DIG, (j+1)*32/DIG)), so a lane holds every plane's exact i32 sum of its outputs
 //               and recombines them, sum_j 256^j * acc_j, before the float epilogue.
-template <int DT, int WGM, int WGN, int TM, int TN, bool PRECISE, int NS, bool INT8 = false, int DIG = 0>
+// CONV (with INT8, DIG = 0): the rows are im2col rows (image, pixel); the accumulators are turned into the
+//               convolution's outputs here (conv_dequant) and stored NCHW, four consecutive pixels of a channel
+//               per lane and store where the image size allows.
+template <int DT, int WGM, int WGN, int TM, int TN, bool PRECISE, int NS, bool INT8 = false, int DIG = 0, bool CONV = false>
 __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
 {
     static_assert(DIG == 0 || (INT8 && (DIG == 2 || DIG == 4)), "digit planes ride on the int8 operands");
+    static_assert(!CONV || (INT8 && DIG == 0), "the conv epilogue belongs to the plain int8 kernel");
     // Codebook weights (w[n,k] = bscale[n, k/32] * table[nibble], src/packed_tensor.rs:469-521) are decoded here:
     // the nibble looks up an (f16 hi, f16 lo) pair of the scaled table value in LDS, two MFMAs per step (hi, lo)
     // add into a per-block accumulator, and after the two steps of a 32-value block the accumulator is folded into
@@ -136,6 +189,48 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
     const int64_t n0 = (int64_t)nt * BN;
     const int it0 = z * p.ips;
     const int it1 = (it0 + p.ips < p.iters) ? it0 + p.ips : p.iters;
+
+    // conv epilogue: per-row constants of the tile (activation scale / zero of the row's image, sum of q_a, NCHW
+    // offset of the pixel), requested now so that their latency hides behind the K loop
+    constexpr int CV_PARTS = CONV ? (WGM * WGN * 64) / (WGM * TM * 32) : 1;
+    __shared__ float cv_sa[CONV ? WGM * TM * 32 : 1], cv_za[CONV ? WGM * TM * 32 : 1];
+    __shared__ int cv_qs[CV_PARTS > 0 ? CV_PARTS : 1][CONV ? WGM * TM * 32 : 1];
+    __shared__ int64_t cv_off[CONV ? WGM * TM * 32 : 1];
+    if constexpr (CONV) {
+        constexpr int BM_ = WGM * TM * 32;
+        static_assert((WGM * WGN * 64) % BM_ == 0 && CV_PARTS >= 1, "whole row groups per workgroup");
+        const int row = threadIdx.x % BM_, part = threadIdx.x / BM_;
+        const int64_t r = (int64_t)mt * BM_ + row;
+        int qs = 0;
+        if (r < p.m)
+            for (int y = part; y < p.cv.nq; y += CV_PARTS) qs += p.cv.qsum[(int64_t)y * p.rows_pad + r];
+        cv_qs[part][row] = qs;
+        if (part == 0) {
+            float sa = 0.0f, za = 0.0f;
+            int64_t off = 0;
+            if (r < p.m) {
+                const uint32_t nn = (uint32_t)r / p.cv.np, px = (uint32_t)r - nn * p.cv.np;
+                const int bg = (int)nn * p.cv.groups + p.cv.g;
+                sa = p.cv.actq[bg * 4 + 0];
+                za = p.cv.actq[bg * 4 + 1];
+                off = (int64_t)nn * p.cv.oc * p.cv.np + px;
+            }
+            cv_sa[row] = sa; cv_za[row] = za; cv_off[row] = off;
+        }
+    }
+    // ... and this lane's channel constants (scale, zero, scale * sum q_w, bias)
+    float cv_sw[CONV ? TN : 1], cv_zw[CONV ? TN : 1], cv_wt[CONV ? TN : 1], cv_bi[CONV ? TN : 1];
+    if constexpr (CONV) {
+#pragma unroll
+        for (int tn = 0; tn < TN; tn++) {
+            const int64_t n = (int64_t)nt * (WGN * TN * 32) + (((threadIdx.x >> 6) % WGN) * TN + tn) * 32 + (threadIdx.x & 31);
+            const bool ok = n < p.n;
+            cv_sw[tn] = ok ? p.scales[n] : 0.0f;
+            cv_zw[tn] = ok ? p.zeros[n] : 0.0f;
+            cv_wt[tn] = ok ? cv_sw[tn] * (float)p.cv.row_qsum[n] : 0.0f;
+            cv_bi[tn] = (ok && p.bias) ? p.bias[n] : 0.0f;
+        }
+    }
 
     // ---- what this lane fetches per stage.  LDS slot s of a region = 16-byte chunk s.
     // The LDS has 64 banks of 4 bytes: a 128-bit read is conflict-free when every 16 lanes cover
@@ -478,6 +573,62 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
                         float o = d * sc[tn] + zp[tn] * rxs[tm][r];
                         if (p.bias) o = o + bi[tn];
                         p.out[m * p.n + n] = fnn_activation(o, p.act);
+                    }
+                }
+            }
+        return;
+    } else if constexpr (INT8 && CONV) {
+        __syncthreads();   // the row tables
+        const float *sw = cv_sw, *zw = cv_zw, *wt = cv_wt, *bi = cv_bi;
+        const bool has_bias = p.bias != nullptr;
+        const int64_t np = p.cv.np;
+#pragma unroll
+        for (int tm = 0; tm < TM; tm++)
+#pragma unroll
+            for (int ig = 0; ig < 4; ig++) {
+                const int rr0 = (wm * TM + tm) * 32 + ig * 8 + h * 4;   // four consecutive rows of the tile
+                const int64_t r0 = (int64_t)mt * BM + rr0;
+                if (r0 >= p.m) continue;
+                float sa[4], za[4], rs[4];
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    int qs = 0;
+#pragma unroll
+                    for (int y = 0; y < CV_PARTS; y++) qs += cv_qs[y][rr0 + j];
+                    sa[j] = cv_sa[rr0 + j];
+                    za[j] = cv_za[rr0 + j];
+                    rs[j] = sa[j] * (float)qs;
+                }
+#pragma unroll
+                for (int tn = 0; tn < TN; tn++) {
+                    const int64_t n = n0 + (wn * TN + tn) * 32 + lr;
+                    if (n >= p.n) continue;
+                    float v[4];
+                    int av[4], bq[4];
+                    // the rounded bias depends on (image, channel) only: one division for the four rows when they
+                    // share an image
+                    bq[0] = has_bias ? conv_bias_q(bi[tn], sa[0], sw[tn]) : 0;
+#pragma unroll
+                    for (int j = 1; j < 4; j++) bq[j] = (p.cv.vec4 || !has_bias) ? bq[0] : conv_bias_q(bi[tn], sa[j], sw[tn]);
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        const float bits = acc[tm][tn][ig * 4 + j];
+                        int a = __float_as_int(bits);
+                        if constexpr (DT == FNN_DT_I4) a >>= 4;
+                        v[j] = conv_dequant(a, sa[j], za[j], rs[j], sw[tn], zw[tn], wt[tn], bq[j], p.cv.kk, p.act, &av[j]);
+                    }
+                    if (p.cv.vec4) {
+                        const int64_t o = cv_off[rr0] + n * np;
+                        *reinterpret_cast<float4 *>(p.cv.y + o) = make_float4(v[0], v[1], v[2], v[3]);
+                        if (p.cv.acc_out) *reinterpret_cast<int4 *>(p.cv.acc_out + o) = make_int4(av[0], av[1], av[2], av[3]);
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < 4; j++) {
+                            if (r0 + j >= p.m) continue;
+                            const int64_t o = cv_off[rr0 + j] + n * np;
+                            p.cv.y[o] = v[j];
+                            if (p.cv.acc_out) p.cv.acc_out[o] = av[j];
+                        }
                     }
                 }
             }

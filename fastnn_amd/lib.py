@@ -35,6 +35,7 @@ OPT_GEMM_INT8 = 10
 OPT_GEMM_INT8_MIN_M = 11
 OPT_CODEBOOK_EXPANDED = 12
 OPT_GEMV_INT8_MAX_M = 13
+OPT_CONV_EPILOGUE = 14
 
 STATUS_NAMES = {0: "Ok", 1: "Dispatch", 2: "Memory", 3: "UnsupportedOp", 4: "Compilation"}
 

@@ -110,7 +110,11 @@ enum {
                                   /* operand (FNN_OPT_CODEBOOK_CACHE), 2 = always decoded inside the tiled GEMM           */
     FNN_OPT_GEMV_INT8_MAX_M = 13, /* largest M the int8 GEMV kernel takes, 1..16 (default 8: beyond that the f16 16-row      */
                                   /* kernel measured faster, the activation chunks being converted one after the other)   */
-    FNN_OPT_COUNT = 14
+    FNN_OPT_CONV_EPILOGUE = 14,   /* quantised Conv2d (I8 / I4 weights) on the int8 matrix cores: 0 (default) = by size,      */
+                                  /* 1 = dequantise + bias + activation + NCHW stores inside the GEMM kernel, 2 = as a kernel */
+                                  /* of its own after it, 3 = as 1 on 128-row tiles whatever the size (1 takes 64 x 64 tiles */
+                                  /* while those leave CUs idle)                                                           */
+    FNN_OPT_COUNT = 15
 };
 int fnn_hip_set_option(fnn_hip_ctx *ctx, int option, int64_t value);
 int fnn_hip_get_option(fnn_hip_ctx *ctx, int option, int64_t *value);

@@ -443,13 +443,24 @@ CONVS = [
     dict(b=1, c=8, h=10, w=7, oc=6, kh=3, kw=2, stride=1, pad=2, dil=2, groups=2),
     dict(b=3, c=5, h=9, w=9, oc=7, kh=3, kw=3, stride=1, pad=1, dil=1, groups=1),
     dict(b=1, c=32, h=16, w=16, oc=64, kh=3, kw=3, stride=1, pad=1, dil=1, groups=1),
+    dict(b=2, c=12, h=13, w=14, oc=160, kh=3, kw=3, stride=1, pad=1, dil=1, groups=1),   # two column tiles, rows past a row tile
 ]
+
+
+@pytest.fixture
+def conv_epilogue(ctx, request):
+    """Where the conv epilogue runs: 0 = by size, 2 = a kernel of its own, 3 = inside the GEMM kernel on 128-row tiles
+    (0 takes the 64-row tiles at these sizes)."""
+    ctx.set_option(flib.OPT_CONV_EPILOGUE, request.param)
+    yield request.param
+    ctx.set_option(flib.OPT_CONV_EPILOGUE, 0)
 
 
 @pytest.mark.parametrize("cfg", CONVS)
 @pytest.mark.parametrize("act", [0, 1, 3, 2])
 @pytest.mark.parametrize("wdt", [flib.DT_I8, flib.DT_I4])
-def test_qconv2d_i8(ctx, orc, cfg, act, wdt):
+@pytest.mark.parametrize("conv_epilogue", [0, 2, 3], indirect=True)
+def test_qconv2d_i8(ctx, orc, cfg, act, wdt, conv_epilogue):
     """I8 weights: conv2d_packed_i8x4; I4 weights: conv2d_packed_i4x8 (activations quantised to 16 levels)."""
     rng = np.random.default_rng(6000 + cfg["c"])
     kk = cfg["c"] // cfg["groups"] * cfg["kh"] * cfg["kw"]
