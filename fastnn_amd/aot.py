@@ -413,6 +413,11 @@ class AotExecutor:
     def replayed(self) -> bool:
         return bool(self._plan is not None and self._plan.replayed)
 
+    @property
+    def ranges_used(self) -> int:
+        """Conv instructions of the plan that took their activation ranges from the instruction before them."""
+        return 0 if self._plan is None else self._plan.ranges_used
+
     def close(self):
         if self._plan is not None:
             self._plan.close()

@@ -99,6 +99,11 @@ class ExecutablePlan:
         """True when the last dispatch of this plan ran as a HIP-graph replay."""
         return bool(self.lib.fnn_plan_replayed(self.handle))
 
+    @property
+    def ranges_used(self) -> int:
+        """Quantised Conv2d instructions that took their activation ranges from the instruction before them."""
+        return int(self.lib.fnn_plan_ranges_used(self.handle))
+
     def _ok(self, rc, what):
         if rc:
             msg = self.lib.fnn_backend_last_error(None)

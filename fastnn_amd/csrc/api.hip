@@ -15,6 +15,7 @@
 #include <vector>
 
 #include "i8act.h"
+#include "range_io.h"
 #include "mfma.h"
 #include "../../include/fastnn_hip_backend.h"
 
@@ -22,14 +23,15 @@ hipError_t launch_im2col_f32(const float *x, float *col, int64_t b, int64_t c, i
                              int64_t ho, int64_t wo, int kh, int kw, int stride, int pad, int dil, hipStream_t s);
 hipError_t launch_rows_to_nchw(const float *src, float *y, int64_t b, int64_t np, int64_t oc, int64_t ch0, int64_t ocg, hipStream_t s);
 hipError_t launch_fill(float *dst, uint64_t n, float value, hipStream_t s);
-hipError_t launch_eltwise(int op, const float *a, const float *b, uint64_t nb, float *out, uint64_t n, hipStream_t s);
+hipError_t launch_eltwise(int op, const float *a, const float *b, uint64_t nb, float *out, uint64_t n, hipStream_t s, FnnRangeIo *rio);
 hipError_t launch_copy2d(float *dst, uint64_t dst_pitch, uint64_t dst_len, const float *src, uint64_t src_pitch, uint64_t src_len,
-                         uint64_t width, uint64_t height, hipStream_t s);
+                         uint64_t width, uint64_t height, hipStream_t s, FnnRangeIo *rio);
 hipError_t launch_avgpool2d(const float *x, uint64_t in_len, float *y, uint64_t out_len, uint64_t h, uint64_t w,
                             uint64_t ho, uint64_t wo, int kernel, int stride, int pad, hipStream_t s);
 hipError_t launch_maxpool2d(const float *x, uint64_t in_len, float *y, uint64_t out_len, uint64_t c, uint64_t h, uint64_t w,
-                            uint64_t ho, uint64_t wo, int kernel, int stride, int pad, int64_t *indices, uint64_t idx_len, hipStream_t s);
-hipError_t launch_upsample_nearest2d(const float *x, float *y, uint64_t nc, uint64_t h, uint64_t w, int sh, int sw, hipStream_t s);
+                            uint64_t ho, uint64_t wo, int kernel, int stride, int pad, int64_t *indices, uint64_t idx_len, hipStream_t s,
+                            FnnRangeIo *rio);
+hipError_t launch_upsample_nearest2d(const float *x, float *y, uint64_t nc, uint64_t h, uint64_t w, int sh, int sw, hipStream_t s, FnnRangeIo *rio);
 
 struct fnn_hip_graph {
     hipGraph_t graph = nullptr;
@@ -54,6 +56,7 @@ struct fnn_hip_ctx {
     uint64_t ws_epoch = 0;     // bumped whenever a staging buffer is re-allocated (captured graphs go stale)
     unsigned char *static_ws = nullptr;   // this device's copy of the library's static workspace
     bool static_mode = false;             // inside fnn_hip_qmatmul_static: workspaces come from static_ws, nothing allocates
+    FnnRangeIo range;                     // value ranges handed from one call to the next (range_io.h)
 };
 
 // Workspace of fnn_hip_qmatmul_static, part of the library's device image: every GPU the library runs on holds one
@@ -129,6 +132,7 @@ const OptionSpec kOptions[FNN_OPT_COUNT] = {
     {0, 0, 2},        // FNN_OPT_CODEBOOK_EXPANDED
     {8, 1, 16},       // FNN_OPT_GEMV_INT8_MAX_M
     {0, 0, 3},        // FNN_OPT_CONV_EPILOGUE
+    {1, 0, 1},        // FNN_OPT_CONV_RANGES
 };
 
 #define HIP_TRY(ctx, code, expr)                                                              \
@@ -781,16 +785,38 @@ int fnn_hip_qconv2d(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *x, i
         p.kh = kh; p.kw = kw; p.stride = stride; p.pad = pad; p.dil = dil; p.groups = groups; p.act = act;
         p.wbits = w->dtype == FNN_DT_I4 ? 4 : 8;
         p.x8 = nullptr; p.payload_i4 = 0; p.nparts = 0;
+        p.part_stride = QCONV_NPART; p.range_zero = 0; p.range_out = nullptr; p.range_out_stride = 0;
+        FnnRangeIo &rio = ctx->range;
+        rio.in_used = 0;
         if (flags & FNN_FLAG_FORCE_GENERIC) {
+            if (rio.out_table) rio.out_failed = 1;
             HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qconv2d_i8(p, ctx->stream, 0, nullptr));
         } else {
-            // range scan; the scales are then formed by the operand kernel itself (one launch less) when a workgroup's
-            // 64 rows touch at most two images, else by the small kernel of their own
+            // the caller asks for partial ranges of y (range_io.h): the epilogue inside the GEMM kernel leaves them
+            const bool want_out = rio.out_table && dev && rio.out_parts == 0;
+            if (want_out && rio.out_images == (uint64_t)b && rio.out_image_elems == (uint64_t)(oc * ho * wo)) {
+                p.range_out = rio.out_table; p.range_out_stride = rio.out_stride;
+            }
+            // Activation ranges: from the partial pairs the producer of x left (usable when the im2col matrix holds
+            // every input value, i.e. every input row and column is reached by some tap, and the group is the whole
+            // image; the zero of the padding joins them), else from a scan of x.  The scales are then formed by the
+            // operand kernel itself (one launch less) when a workgroup's 64 rows touch at most two images and the
+            // pairs are few, else by the small kernel of their own.
             int nparts = 0;
-            HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qconv2d_i8(p, ctx->stream, 3, &nparts));
+            int pad_touched = 0;
+            bool all_reached = false;
+            if (rio.in_table && dev && groups == 1 && rio.in_parts > 0) fnn_conv_coverage(p, &pad_touched, &all_reached);
+            if (all_reached) {
+                p.minmax_partial = const_cast<float *>(rio.in_table);
+                p.part_stride = rio.in_stride; p.range_zero = pad_touched;
+                nparts = rio.in_parts;
+                rio.in_used = 1;
+            } else {
+                HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qconv2d_i8(p, ctx->stream, 3, &nparts));
+            }
             const int64_t kk_g = (c / groups) * kh * kw;
             const int64_t operand_wgs = ((b * ho * wo + 63) / 64) * (((kk_g + 15) / 16 + 3) / 4);
-            const bool fused_scales = ho * wo >= 64 && nparts <= QCONV_NPART && operand_wgs <= 8192;   // many workgroups: cheaper once
+            const bool fused_scales = ho * wo >= 64 && nparts <= 4 * QCONV_NPART && operand_wgs <= 8192;   // many workgroups: cheaper once
             if (fused_scales) p.nparts = nparts;
             else HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qconv2d_i8(p, ctx->stream, 4, &nparts));
             bool handled = false;
@@ -801,6 +827,7 @@ int fnn_hip_qconv2d(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *x, i
                 p.nparts = 0;
                 HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qconv2d_i8(p, ctx->stream, 2, nullptr));
             }
+            if (want_out && rio.out_parts == 0) rio.out_failed = 1;   // y is written, its ranges are not
         }
         if (!dev) {
             HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(y, dy, yout, hipMemcpyDeviceToHost, ctx->stream));
@@ -876,6 +903,7 @@ int fnn_hip_qconv2d_i8act(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const uint8
         p.wbits = w->dtype == FNN_DT_I4 ? 4 : 8;
         p.x8 = reinterpret_cast<const int8_t *>(dp + 8);
         p.payload_i4 = w->dtype == FNN_DT_I4; p.nparts = 0;
+        p.part_stride = QCONV_NPART; p.range_zero = 0; p.range_out = nullptr; p.range_out_stride = 0;
         HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_conv_actq_from_payload(dp, p.actq, (int)(b * groups), ctx->stream));
         bool handled = false;
         if ((rc = fnn_i8_tiled_conv(ctx, ctx->stream, w, p, &handled))) return rc;
@@ -894,7 +922,7 @@ int fnn_hip_elementwise(fnn_hip_ctx *ctx, int op, const float *a, const float *b
         if (!ctx || !a || !out) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_elementwise: NULL argument");
         if (op < 0 || op > 3) return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "fnn_hip_elementwise: unknown op %d", op);
         if (op == 0 && (!b || nb == 0)) return fail(ctx, FNN_ERR_DISPATCH, "add_f32: missing second operand");
-        HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_eltwise(op, a, b, nb, out, n, ctx->stream));
+        HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_eltwise(op, a, b, nb, out, n, ctx->stream, &ctx->range));
         return FNN_OK;
     });
 }
@@ -923,7 +951,7 @@ int fnn_hip_copy2d_f32(fnn_hip_ctx *ctx, float *dst, uint64_t dst_pitch, uint64_
 {
     return guarded(ctx, "fnn_hip_copy2d_f32", [&]() -> int {
         if (!ctx || ((!dst || !src) && width && height)) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_copy2d_f32: NULL argument");
-        HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_copy2d(dst, dst_pitch, dst_len, src, src_pitch, src_len, width, height, ctx->stream));
+        HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_copy2d(dst, dst_pitch, dst_len, src, src_pitch, src_len, width, height, ctx->stream, &ctx->range));
         return FNN_OK;
     });
 }
@@ -939,7 +967,7 @@ int fnn_hip_maxpool2d_f32(fnn_hip_ctx *ctx, const float *x, uint64_t in_len, flo
         uint64_t total = n * c * ho * wo;
         if (total > out_len) total = out_len;   // writes past the output slice are dropped (ops.rs:147-149)
         HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_maxpool2d(x, in_len, y, total, c, h, w, ho, wo, (int)kernel, (int)stride, (int)pad, indices,
-                                                         indices ? (idx_len < n * c * ho * wo ? idx_len : n * c * ho * wo) : 0, ctx->stream));
+                                                         indices ? (idx_len < n * c * ho * wo ? idx_len : n * c * ho * wo) : 0, ctx->stream, &ctx->range));
         return FNN_OK;
     });
 }
@@ -964,7 +992,7 @@ int fnn_hip_upsample_nearest2d_f32(fnn_hip_ctx *ctx, const float *x, float *y, u
     return guarded(ctx, "fnn_hip_upsample_nearest2d_f32", [&]() -> int {
         if (!ctx || !x || !y) return fail(ctx, FNN_ERR_DISPATCH, "upsample_nearest2d: NULL argument");
         if (sh > 1024 || sw > 1024) return fail(ctx, FNN_ERR_DISPATCH, "upsample_nearest2d: scale too large");
-        HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_upsample_nearest2d(x, y, nc, h, w, (int)sh, (int)sw, ctx->stream));
+        HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_upsample_nearest2d(x, y, nc, h, w, (int)sh, (int)sw, ctx->stream, &ctx->range));
         return FNN_OK;
     });
 }
@@ -1081,3 +1109,4 @@ bool fnn_ctx_no_alloc(fnn_hip_ctx *ctx) { return ctx->capturing || ctx->static_m
 int fnn_ctx_fail(fnn_hip_ctx *ctx, int code, const char *msg) { return fail(ctx, code, "%s", msg); }
 
 int64_t fnn_ctx_option(const fnn_hip_ctx *ctx, int option) { return ctx->options[option]; }
+FnnRangeIo *fnn_ctx_range_io(fnn_hip_ctx *ctx) { return &ctx->range; }

@@ -3,10 +3,34 @@
 // ("concat" :4267-4324, "slice_f32" :4721-4760, "pool_f32" max :4362-4397 with
 // microkernels/ops.rs:104-158, "upsample_nearest2d" :5496-5535 with microkernels/misc.rs:338-364).
 #include "common.h"
+#include "range_io.h"
 
 #include "../../include/fastnn_hip_backend.h"
 
 namespace {
+// Partial value ranges of what a launch writes, for the quantised Conv2d that reads the tensor next (range_io.h): with
+// a table the grid is (blocks, images), block (x, y) walks the values of image y only and leaves their (min, max) in
+// pair slot0 + x of that image; without one the grid is (blocks, 1) and the whole output counts as one image.
+struct RangeEmit {
+    float *table;           // [images][stride][2], or null
+    uint64_t image_elems;   // output values per image
+    int stride, slot0;
+};
+
+__device__ __forceinline__ void emit_range(const RangeEmit &re, float mn, float mx)
+{
+    __shared__ float smn[4], smx[4];
+    mn = wave_min(mn);
+    mx = wave_max(mx);
+    if ((threadIdx.x & 63) == 0) { smn[threadIdx.x >> 6] = mn; smx[threadIdx.x >> 6] = mx; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float *d = re.table + ((uint64_t)blockIdx.y * re.stride + re.slot0 + blockIdx.x) * 2;
+        d[0] = fminf(fminf(smn[0], smn[1]), fminf(smn[2], smn[3]));
+        d[1] = fmaxf(fmaxf(smx[0], smx[1]), fmaxf(smx[2], smx[3]));
+    }
+}
+
 __global__ void __launch_bounds__(256) eltwise_kernel(int op, const float *a, const float *b, uint64_t nb, float *out, uint64_t n)
 {
     for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
@@ -16,12 +40,38 @@ __global__ void __launch_bounds__(256) eltwise_kernel(int op, const float *a, co
         out[i] = v;
     }
 }
+// The same with ranges: block (x, y) takes 1024 * U consecutive values of image y, every thread requests its 4 * U
+// operands before it uses the first one.
+template <int U>
+__global__ void __launch_bounds__(256) eltwise_ranges_kernel(int op, const float *a, const float *b, uint64_t nb, float *out, RangeEmit re)
+{
+    const uint64_t base = (uint64_t)blockIdx.y * re.image_elems, j0 = (uint64_t)blockIdx.x * (1024 * U) + threadIdx.x;
+    float va[4 * U], vb[4 * U];
+#pragma unroll
+    for (int k = 0; k < 4 * U; k++) {
+        const uint64_t j = j0 + (uint64_t)k * 256;
+        const bool in = j < re.image_elems;
+        va[k] = in ? a[base + j] : 0.0f;
+        vb[k] = (in && op == 0) ? b[(base + j) % nb] : 0.0f;
+    }
+    float mn = INFINITY, mx = -INFINITY;
+#pragma unroll
+    for (int k = 0; k < 4 * U; k++) {
+        const uint64_t j = j0 + (uint64_t)k * 256;
+        if (j >= re.image_elems) continue;
+        const float v = op == 0 ? va[k] + vb[k] : fnn_activation(va[k], op);
+        out[base + j] = v;
+        mn = fminf(mn, v);
+        mx = fmaxf(mx, v);
+    }
+    emit_range(re, mn, mx);
+}
 __global__ void __launch_bounds__(256) fill_kernel(float *dst, uint64_t n, float value)
 {
     for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) dst[i] = value;
 }
 // height rows of width values: dst[r*dst_pitch + c] = src[r*src_pitch + c], clamped to both lengths
-// (the block copies of "concat" and "slice_f32")
+// (the block copies of "concat" and "slice_f32").
 __global__ void __launch_bounds__(256) copy2d_kernel(float *dst, uint64_t dst_pitch, uint64_t dst_len, const float *src,
                                                      uint64_t src_pitch, uint64_t src_len, uint64_t width, uint64_t height)
 {
@@ -32,16 +82,45 @@ __global__ void __launch_bounds__(256) copy2d_kernel(float *dst, uint64_t dst_pi
         if (si < src_len && di < dst_len) dst[di] = src[si];
     }
 }
+// The same with ranges, one image per row, nothing clipped: block (x, y) takes 1024 * U consecutive values of row y,
+// every thread requests its 4 * U values before it stores the first one.
+template <int U>
+__global__ void __launch_bounds__(256) copy2d_ranges_kernel(float *dst, uint64_t dst_pitch, const float *src, uint64_t src_pitch, uint64_t width,
+                                                            RangeEmit re)
+{
+    const float *s = src + (uint64_t)blockIdx.y * src_pitch;
+    float *d = dst + (uint64_t)blockIdx.y * dst_pitch;
+    const uint64_t c0 = (uint64_t)blockIdx.x * (1024 * U) + threadIdx.x;
+    float v[4 * U];
+#pragma unroll
+    for (int k = 0; k < 4 * U; k++) {
+        const uint64_t c = c0 + (uint64_t)k * 256;
+        v[k] = c < width ? s[c] : 0.0f;
+    }
+    float mn = INFINITY, mx = -INFINITY;
+#pragma unroll
+    for (int k = 0; k < 4 * U; k++) {
+        const uint64_t c = c0 + (uint64_t)k * 256;
+        if (c >= width) continue;
+        d[c] = v[k];
+        mn = fminf(mn, v[k]);
+        mx = fmaxf(mx, v[k]);
+    }
+    emit_range(re, mn, mx);
+}
 
 // window maximum from -inf with a strict `>` (a NaN never wins), taps in the padding skipped
 // indices (nullable): window position kh*kernel + kw of the first strict maximum in (kh, kw) order, 0 when no tap
 // lies inside the image; an output position is visited when it lies inside the value slice or the index slice
 __global__ void __launch_bounds__(256) maxpool2d_kernel(const float *x, uint64_t in_len, float *y, uint64_t out_len, uint64_t c,
                                                         uint64_t h, uint64_t w, uint64_t ho, uint64_t wo, int kernel, int stride, int pad,
-                                                        int64_t *indices, uint64_t idx_len)
+                                                        int64_t *indices, uint64_t idx_len, RangeEmit re)
 {
     const uint64_t total = out_len > idx_len ? out_len : idx_len;
-    for (uint64_t o = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; o < total; o += (uint64_t)gridDim.x * blockDim.x) {
+    const uint64_t ie = re.table ? re.image_elems : total, base = (uint64_t)blockIdx.y * ie;
+    float mn = INFINITY, mx = -INFINITY;
+    for (uint64_t j = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; j < ie && base + j < total; j += (uint64_t)gridDim.x * blockDim.x) {
+        const uint64_t o = base + j;
         const uint64_t ww = o % wo, t = o / wo, hh = t % ho, nc = t / ho;   // nc = n*c + channel
         float val = -INFINITY;
         int best = 0;
@@ -58,9 +137,14 @@ __global__ void __launch_bounds__(256) maxpool2d_kernel(const float *x, uint64_t
                 }
             }
         }
-        if (o < out_len) y[o] = val;
+        if (o < out_len) {
+            y[o] = val;
+            mn = fminf(mn, val);
+            mx = fmaxf(mx, val);
+        }
         if (o < idx_len) indices[o] = best;
     }
+    if (re.table) emit_range(re, mn, mx);
     (void)c;
 }
 
@@ -90,13 +174,21 @@ __global__ void __launch_bounds__(256) avgpool2d_kernel(const float *x, uint64_t
     }
 }
 
-__global__ void __launch_bounds__(256) upsample_nearest2d_kernel(const float *x, float *y, uint64_t total, uint64_t h, uint64_t w, int sh, int sw)
+__global__ void __launch_bounds__(256) upsample_nearest2d_kernel(const float *x, float *y, uint64_t total, uint64_t h, uint64_t w, int sh, int sw,
+                                                                 RangeEmit re)
 {
     const uint64_t wo = w * sw, ho = h * sh;
-    for (uint64_t o = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; o < total; o += (uint64_t)gridDim.x * blockDim.x) {
+    const uint64_t ie = re.table ? re.image_elems : total, base = (uint64_t)blockIdx.y * ie;
+    float mn = INFINITY, mx = -INFINITY;
+    for (uint64_t j = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; j < ie && base + j < total; j += (uint64_t)gridDim.x * blockDim.x) {
+        const uint64_t o = base + j;
         const uint64_t ow = o % wo, t = o / wo, oh = t % ho, nc = t / ho;
-        y[o] = x[(nc * h + oh / sh) * w + ow / sw];
+        const float v = x[(nc * h + oh / sh) * w + ow / sw];
+        y[o] = v;
+        mn = fminf(mn, v);
+        mx = fmaxf(mx, v);
     }
+    if (re.table) emit_range(re, mn, mx);
 }
 }  // namespace
 
@@ -106,22 +198,98 @@ static unsigned grid_for(uint64_t n)
     return (unsigned)(blocks > 8192 ? 8192 : (blocks < 1 ? 1 : blocks));
 }
 
+// Launch shape and table slice for the next call's range request (range_io.h): `per_image` values per image in
+// `images` images.  Without a usable request: one image, as many blocks as `n` values want.
+struct RangePlan {
+    RangeEmit re;
+    dim3 grid;
+    int parts;
+};
+static RangePlan range_plan(FnnRangeIo *rio, uint64_t n, uint64_t per_image, uint64_t images, unsigned flat_blocks)
+{
+    RangePlan rp;
+    rp.re = RangeEmit{nullptr, 0, 0, 0};
+    rp.grid = dim3(flat_blocks);
+    rp.parts = 0;
+    if (!rio || !rio->out_table) return rp;
+    uint64_t blocks = (per_image + 2047) / 2048;
+    if (blocks > 512) blocks = 512;
+    if (blocks < 1) blocks = 1;
+    if (per_image == 0 || images == 0 || images > 65535 || rio->out_images != images || per_image * images != n ||
+        (uint64_t)rio->out_parts + blocks > (uint64_t)rio->out_stride) {   // (out_parts: pairs already in place)
+        rio->out_failed = 1;
+        return rp;
+    }
+    rp.re = RangeEmit{rio->out_table, per_image, rio->out_stride, rio->out_parts};
+    rp.grid = dim3((unsigned)blocks, (unsigned)images);
+    rp.parts = (int)blocks;
+    return rp;
+}
+
+// The same for the kernels that give a block 1024 * U consecutive values of an image: the smallest U in 1, 2, 4, 8
+// whose pairs fit the table.
+static RangePlan range_plan_chunks(FnnRangeIo *rio, uint64_t n, uint64_t per_image, uint64_t images, int *unroll)
+{
+    RangePlan rp;
+    rp.re = RangeEmit{nullptr, 0, 0, 0};
+    rp.grid = dim3(1);
+    rp.parts = 0;
+    *unroll = 1;
+    if (!rio || !rio->out_table) return rp;
+    uint64_t blocks = 0;
+    int u = 1;
+    for (; u <= 8; u *= 2) {
+        blocks = (per_image + 1024 * u - 1) / (1024 * u);
+        if ((uint64_t)rio->out_parts + blocks <= (uint64_t)rio->out_stride) break;
+    }
+    if (u > 8 || per_image == 0 || images == 0 || images > 65535 || rio->out_images != images || per_image * images != n) {
+        rio->out_failed = 1;
+        return rp;
+    }
+    rp.re = RangeEmit{rio->out_table, per_image, rio->out_stride, rio->out_parts};
+    rp.grid = dim3((unsigned)blocks, (unsigned)images);
+    rp.parts = (int)blocks;
+    *unroll = u;
+    return rp;
+}
+
 hipError_t launch_copy2d(float *dst, uint64_t dst_pitch, uint64_t dst_len, const float *src, uint64_t src_pitch, uint64_t src_len,
-                         uint64_t width, uint64_t height, hipStream_t s)
+                         uint64_t width, uint64_t height, hipStream_t s, FnnRangeIo *rio)
 {
     if (width == 0 || height == 0) return hipSuccess;
-    hipLaunchKernelGGL(copy2d_kernel, dim3(grid_for(width * height)), dim3(256), 0, s, dst, dst_pitch, dst_len, src, src_pitch, src_len, width, height);
+    // (one image per row: the caller asks for ranges only when a row of the destination is an image)
+    // (a copy clipped by either length leaves values of the destination it has not seen: no ranges then; nor when a
+    // row of the destination is not an image of the reader)
+    const bool whole = dst_len >= (height - 1) * dst_pitch + width && src_len >= (height - 1) * src_pitch + width &&
+                       rio && rio->out_image_elems == dst_pitch;
+    if (!whole && rio && rio->out_table) rio->out_failed = 1;
+    int u = 1;
+    RangePlan rp = range_plan_chunks(whole ? rio : nullptr, width * height, width, height, &u);
+    if (rp.re.table) {
+        if (u == 1) hipLaunchKernelGGL(copy2d_ranges_kernel<1>, rp.grid, dim3(256), 0, s, dst, dst_pitch, src, src_pitch, width, rp.re);
+        else if (u == 2) hipLaunchKernelGGL(copy2d_ranges_kernel<2>, rp.grid, dim3(256), 0, s, dst, dst_pitch, src, src_pitch, width, rp.re);
+        else if (u == 4) hipLaunchKernelGGL(copy2d_ranges_kernel<4>, rp.grid, dim3(256), 0, s, dst, dst_pitch, src, src_pitch, width, rp.re);
+        else hipLaunchKernelGGL(copy2d_ranges_kernel<8>, rp.grid, dim3(256), 0, s, dst, dst_pitch, src, src_pitch, width, rp.re);
+        rio->out_parts += rp.parts;
+    } else {
+        hipLaunchKernelGGL(copy2d_kernel, dim3(grid_for(width * height)), dim3(256), 0, s, dst, dst_pitch, dst_len, src, src_pitch, src_len, width, height);
+    }
     return hipGetLastError();
 }
 
 hipError_t launch_maxpool2d(const float *x, uint64_t in_len, float *y, uint64_t out_len, uint64_t c, uint64_t h, uint64_t w,
-                            uint64_t ho, uint64_t wo, int kernel, int stride, int pad, int64_t *indices, uint64_t idx_len, hipStream_t s)
+                            uint64_t ho, uint64_t wo, int kernel, int stride, int pad, int64_t *indices, uint64_t idx_len, hipStream_t s,
+                            FnnRangeIo *rio)
 {
     if (!indices) idx_len = 0;
     const uint64_t total = out_len > idx_len ? out_len : idx_len;
     if (total == 0) return hipSuccess;
-    hipLaunchKernelGGL(maxpool2d_kernel, dim3(grid_for(total)), dim3(256), 0, s, x, in_len, y, out_len, c, h, w, ho, wo, kernel, stride, pad,
-                       indices, idx_len);
+    const bool images_match = idx_len <= out_len && rio && rio->out_image_elems == c * ho * wo;
+    if (!images_match && rio && rio->out_table) rio->out_failed = 1;
+    RangePlan rp = range_plan(images_match ? rio : nullptr, out_len, c * ho * wo, c * ho * wo ? out_len / (c * ho * wo) : 0, grid_for(total));
+    hipLaunchKernelGGL(maxpool2d_kernel, rp.grid, dim3(256), 0, s, x, in_len, y, out_len, c, h, w, ho, wo, kernel, stride, pad,
+                       indices, idx_len, rp.re);
+    if (rio) rio->out_parts += rp.parts;
     return hipGetLastError();
 }
 
@@ -133,11 +301,14 @@ hipError_t launch_avgpool2d(const float *x, uint64_t in_len, float *y, uint64_t 
     return hipGetLastError();
 }
 
-hipError_t launch_upsample_nearest2d(const float *x, float *y, uint64_t nc, uint64_t h, uint64_t w, int sh, int sw, hipStream_t s)
+hipError_t launch_upsample_nearest2d(const float *x, float *y, uint64_t nc, uint64_t h, uint64_t w, int sh, int sw, hipStream_t s, FnnRangeIo *rio)
 {
     const uint64_t total = nc * h * sh * w * sw;
     if (total == 0) return hipSuccess;
-    hipLaunchKernelGGL(upsample_nearest2d_kernel, dim3(grid_for(total)), dim3(256), 0, s, x, y, total, h, w, sh, sw);
+    const uint64_t per_image = rio && rio->out_table ? rio->out_image_elems : 0;
+    RangePlan rp = range_plan(rio, total, per_image, per_image ? total / per_image : 0, grid_for(total));
+    hipLaunchKernelGGL(upsample_nearest2d_kernel, rp.grid, dim3(256), 0, s, x, y, total, h, w, sh, sw, rp.re);
+    if (rio) rio->out_parts += rp.parts;
     return hipGetLastError();
 }
 
@@ -150,9 +321,20 @@ hipError_t launch_fill(float *dst, uint64_t n, float value, hipStream_t s)
     return hipGetLastError();
 }
 
-hipError_t launch_eltwise(int op, const float *a, const float *b, uint64_t nb, float *out, uint64_t n, hipStream_t s)
+hipError_t launch_eltwise(int op, const float *a, const float *b, uint64_t nb, float *out, uint64_t n, hipStream_t s, FnnRangeIo *rio)
 {
     if (n == 0) return hipSuccess;
+    const uint64_t per_image = rio && rio->out_table ? rio->out_image_elems : 0;
+    int u = 1;
+    RangePlan rp = range_plan_chunks(rio, n, per_image, per_image ? n / per_image : 0, &u);
+    if (rp.re.table) {
+        if (u == 1) hipLaunchKernelGGL(eltwise_ranges_kernel<1>, rp.grid, dim3(256), 0, s, op, a, b, nb ? nb : 1, out, rp.re);
+        else if (u == 2) hipLaunchKernelGGL(eltwise_ranges_kernel<2>, rp.grid, dim3(256), 0, s, op, a, b, nb ? nb : 1, out, rp.re);
+        else if (u == 4) hipLaunchKernelGGL(eltwise_ranges_kernel<4>, rp.grid, dim3(256), 0, s, op, a, b, nb ? nb : 1, out, rp.re);
+        else hipLaunchKernelGGL(eltwise_ranges_kernel<8>, rp.grid, dim3(256), 0, s, op, a, b, nb ? nb : 1, out, rp.re);
+        rio->out_parts += rp.parts;
+        return hipGetLastError();
+    }
     uint64_t blocks = (n + 255) / 256;
     if (blocks > 4096) blocks = 4096;
     hipLaunchKernelGGL(eltwise_kernel, dim3((unsigned)blocks), dim3(256), 0, s, op, a, b, nb, out, n);

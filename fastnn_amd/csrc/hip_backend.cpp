@@ -22,6 +22,7 @@
 #include <vector>
 
 #include "../../include/fastnn_hip_backend.h"
+#include "range_io.h"
 
 namespace {
 
@@ -122,6 +123,7 @@ struct fnn_plan {
     bool has_unsupported = false;     // a segmented dispatch stopped at a kernel without a GPU implementation
     bool segment_resident = false;    // residency as the first segment of the pass in progress found it
     bool last_replayed = false;
+    uint64_t ranges_used = 0;         // convolutions of the last host-side pass that took their ranges from a table
 };
 
 struct fnn_backend {
@@ -147,7 +149,16 @@ struct fnn_backend {
     std::vector<uint8_t> stage;
     uint8_t *scratch = nullptr;   // device copy of an input that overlaps its output
     uint64_t scratch_bytes = 0, scratch_epoch = 0;
+    // Value ranges handed from the instruction that writes an f32 tensor to the quantised Conv2d that reads it
+    // (range_io.h).  Tables are device memory kept per (plan, instruction); a live entry says that the bytes of
+    // `slice` are exactly what the table describes, and lasts until something writes into the slice or the dispatch
+    // pass ends.
+    struct RangeTable { float *dev = nullptr; uint64_t images = 0; };
+    struct LiveRange { fnn_slice slice; const float *table; int parts; uint64_t image_elems, images; };
+    std::map<std::pair<uint64_t, uint64_t>, RangeTable> range_tables;
+    std::vector<LiveRange> live_ranges;
 };
+constexpr int kRangeStride = 2048;   // pairs per image a table has room for
 
 namespace {
 
@@ -634,6 +645,113 @@ int run_call(fnn_backend *b, const Instr &in)
     return fail(b, FNN_ERR_UNSUPPORTED_OP, "%s", name.c_str());
 }
 
+// ---- value ranges between instructions -------------------------------------------------------------------------
+// Geometry of a quantised Conv2d instruction that takes its activation ranges from a table: integer weights, one
+// group (the range of a group's channels is not that of the image).
+struct ConvInput { uint64_t image_elems, images; };
+bool ranged_conv_input(const Instr &in, ConvInput *g)
+{
+    if (in.kind != K_CALL || in.inputs.size() < 2 || in.params.size() < 9 || !in.meta.present) return false;
+    const KernelName kn = split_activation(in.kernel);
+    if (kn.base != "conv2d_i8" && kn.base != "conv2d_i4") return false;
+    if (!in.meta.codebook.empty() || in.params[3] != 1) return false;
+    const uint64_t chw = in.params[4] * in.params[5] * in.params[6];
+    if (chw == 0 || in.inputs[0].size % (chw * 4) != 0 || in.inputs[0].size == 0) return false;
+    g->image_elems = chw;
+    g->images = in.inputs[0].size / (chw * 4);
+    return true;
+}
+
+// can the kernel behind this instruction leave ranges of what it writes?
+bool leaves_ranges(const Instr &in)
+{
+    if (in.kind != K_CALL) return false;
+    const std::string &n = in.kernel;
+    if (n == "add_f32" || n == "relu_f32" || n == "gelu_f32" || n == "silu_f32" || n == "concat" || n == "slice_f32" ||
+        n == "upsample_nearest2d")
+        return true;
+    if (n == "pool_f32") return in.params.size() == 8 && in.params[3] == 1;
+    const KernelName kn = split_activation(n);
+    return (kn.base == "conv2d_i8" || kn.base == "conv2d_i4") && in.meta.present && in.meta.codebook.empty();
+}
+
+void drop_ranges_overlapping(fnn_backend *b, const fnn_slice &s)
+{
+    if (!s.size) return;
+    auto &v = b->live_ranges;
+    v.erase(std::remove_if(v.begin(), v.end(), [&](const fnn_backend::LiveRange &r) { return overlaps(r.slice, s); }), v.end());
+}
+
+// If a later convolution of the plan reads what instruction `idx` writes (from the first byte of its output slice,
+// before anything overwrites it), asks the next call on the context for the partial ranges that convolution
+// needs; *covered = the convolution's input slice.
+void request_ranges(fnn_backend *b, fnn_plan *p, size_t idx, fnn_slice *covered)
+{
+    const Instr &in = p->instrs[idx];
+    FnnRangeIo *rio = fnn_ctx_range_io(b->ctx);
+    if (!in.dst.size) return;
+    for (size_t j = idx + 1; j < p->instrs.size(); j++) {
+        const Instr &nx = p->instrs[j];
+        ConvInput cj;
+        if (ranged_conv_input(nx, &cj) && nx.inputs[0].offset == in.dst.offset && nx.inputs[0].size <= in.dst.size && cj.images <= 65535) {
+            auto &t = b->range_tables[{p->uid, idx}];
+            if (t.dev && t.images < cj.images && !fnn_ctx_capturing(b->ctx)) {
+                fnn_hip_free(b->ctx, t.dev);
+                t.dev = nullptr;
+                b->weights_epoch++;   // a captured graph may hold the old table
+            }
+            if (!t.dev && !fnn_ctx_capturing(b->ctx)) {
+                void *d = nullptr;
+                if (fnn_hip_malloc(b->ctx, (size_t)cj.images * kRangeStride * 8, &d) == FNN_OK) { t.dev = (float *)d; t.images = cj.images; }
+            }
+            if (t.dev && t.images >= cj.images) {
+                rio->out_table = t.dev; rio->out_stride = kRangeStride;
+                rio->out_image_elems = cj.image_elems; rio->out_images = cj.images;
+                *covered = nx.inputs[0];
+            }
+            return;
+        }
+        if (overlaps(nx.dst, in.dst) || (nx.has_secondary && overlaps(nx.secondary, in.dst))) return;
+    }
+}
+
+void note_ranges(fnn_backend *b, const fnn_slice &covered)
+{
+    FnnRangeIo *rio = fnn_ctx_range_io(b->ctx);
+    if (rio->out_table && rio->out_parts > 0 && !rio->out_failed)
+        b->live_ranges.push_back(fnn_backend::LiveRange{covered, rio->out_table, rio->out_parts, rio->out_image_elems, rio->out_images});
+}
+
+int run_call_with_ranges(fnn_backend *b, fnn_plan *p, size_t idx)
+{
+    Instr &in = p->instrs[idx];
+    FnnRangeIo *rio = fnn_ctx_range_io(b->ctx);
+    *rio = FnnRangeIo{};
+    int64_t enabled = 1;
+    fnn_hip_get_option(b->ctx, FNN_OPT_CONV_RANGES, &enabled);
+    if (!enabled) return run_call(b, in);
+    // consumer: a convolution whose input slice is described by a live table
+    ConvInput ci;
+    if (ranged_conv_input(in, &ci)) {
+        for (const auto &r : b->live_ranges)
+            if (r.slice.offset == in.inputs[0].offset && r.slice.size == in.inputs[0].size && r.image_elems == ci.image_elems &&
+                r.images == ci.images) {
+                rio->in_table = r.table; rio->in_stride = kRangeStride; rio->in_parts = r.parts;
+                break;
+            }
+    }
+    // producer: some later convolution reads exactly what this instruction writes, before anything overwrites it
+    fnn_slice covered{0, 0};
+    if (leaves_ranges(in)) request_ranges(b, p, idx, &covered);
+    drop_ranges_overlapping(b, in.dst);
+    if (in.has_secondary) drop_ranges_overlapping(b, in.secondary);
+    const int st = run_call(b, in);
+    if (st == FNN_OK && rio->in_used) p->ranges_used++;
+    if (st == FNN_OK) note_ranges(b, covered);
+    *rio = FnnRangeIo{};
+    return st;
+}
+
 void analyse(fnn_plan *p)
 {
     for (auto &c : p->instrs) {
@@ -679,8 +797,10 @@ void note_dispatched(fnn_backend *b, fnn_plan *p)
     p->resident_seq = b->write_seq;
 }
 
-int run_instr(fnn_backend *b, fnn_plan *p, Instr &in, bool consts_resident)
+int run_instr(fnn_backend *b, fnn_plan *p, size_t idx, bool consts_resident)
 {
+    Instr &in = p->instrs[idx];
+    if (in.kind != K_CALL) drop_ranges_overlapping(b, in.kind == K_WRITE_CONST ? fnn_slice{in.dst.offset, in.data.size()} : in.dst);
     switch (in.kind) {
     case K_WRITE_CONST: {
         fnn_slice d{in.dst.offset, in.data.size()};
@@ -699,12 +819,26 @@ int run_instr(fnn_backend *b, fnn_plan *p, Instr &in, bool consts_resident)
         if (n == 0 || in.dst.offset == in.src.offset) return FNN_OK;
         fnn_slice d{in.dst.offset, n}, s{in.src.offset, n};
         if (overlaps(d, s)) return fail(b, FNN_ERR_DISPATCH, "MemCopy: source and destination overlap");
+        // a copy that feeds a quantised Conv2d (a Split of a one-image batch) runs as a kernel that leaves the ranges
+        FnnRangeIo *rio = fnn_ctx_range_io(b->ctx);
+        *rio = FnnRangeIo{};
+        int64_t ranges_on = 1;
+        fnn_hip_get_option(b->ctx, FNN_OPT_CONV_RANGES, &ranges_on);
+        fnn_slice covered{0, 0};
+        if (ranges_on && n == in.dst.size && n % 4 == 0 && d.offset % 4 == 0 && s.offset % 4 == 0) request_ranges(b, p, idx, &covered);
+        if (rio->out_table && covered.size == n) {
+            const uint64_t per = rio->out_image_elems, imgs = rio->out_images;
+            int st = lift(b, fnn_hip_copy2d_f32(b->ctx, (float *)(b->arena + d.offset), per, n / 4, (const float *)(b->arena + s.offset), per, n / 4, per, imgs));
+            if (st == FNN_OK) note_ranges(b, covered);
+            *rio = FnnRangeIo{};
+            return st;
+        }
+        *rio = FnnRangeIo{};
         return lift(b, fnn_hip_copy(b->ctx, b->arena + d.offset, b->arena + s.offset, n));
     }
     case K_CALL:
-        return run_call(b, in);
+        return run_call_with_ranges(b, p, idx);
     }
-    (void)p;
     return FNN_OK;
 }
 
@@ -748,7 +882,10 @@ int dispatch_impl(fnn_backend *b, fnn_plan *p, uint64_t *elapsed_ns, uint64_t n_
         const uint64_t w0 = b->weights_epoch, s0 = fnn_hip_workspace_epoch(b->ctx), c0 = b->scratch_epoch;
         if (fnn_hip_graph_begin(b->ctx) == FNN_OK) {
             int st = FNN_OK;
-            for (size_t i = 0; i < p->instrs.size() && st == FNN_OK; i++) st = run_instr(b, p, p->instrs[i], true);
+            b->live_ranges.clear();
+            p->ranges_used = 0;
+            for (size_t i = 0; i < p->instrs.size() && st == FNN_OK; i++) st = run_instr(b, p, i, true);
+            b->live_ranges.clear();
             fnn_hip_graph *g = nullptr;
             int en = fnn_hip_graph_end(b->ctx, &g);
             if (st == FNN_OK && en == FNN_OK && g && w0 == b->weights_epoch && s0 == fnn_hip_workspace_epoch(b->ctx) && c0 == b->scratch_epoch) {
@@ -774,9 +911,11 @@ int dispatch_impl(fnn_backend *b, fnn_plan *p, uint64_t *elapsed_ns, uint64_t n_
         return st;
     }
 
+    b->live_ranges.clear();   // ranges never outlive a pass: between passes anyone may write into the arena
+    if (first == 0) p->ranges_used = 0;
     for (size_t i = (size_t)first; i < p->instrs.size(); i++) {
         auto t0 = std::chrono::steady_clock::now();
-        int st = run_instr(b, p, p->instrs[i], resident);
+        int st = run_instr(b, p, i, resident);
         if (st == FNN_OK && elapsed_ns) st = lift(b, fnn_hip_sync(b->ctx));
         if (st == FNN_ERR_UNSUPPORTED_OP && stopped_at) {
             // the caller runs this instruction itself and comes back with first = i + 1
@@ -841,6 +980,8 @@ void fnn_backend_destroy(fnn_backend *b)
     drop_weights(b);
     if (b->arena) fnn_hip_free(b->ctx, b->arena);
     if (b->scratch) fnn_hip_free(b->ctx, b->scratch);
+    for (auto &t : b->range_tables)
+        if (t.second.dev) fnn_hip_free(b->ctx, t.second.dev);
     fnn_hip_destroy(b->ctx);
     delete b;
 }
@@ -948,6 +1089,8 @@ void fnn_plan_destroy(fnn_plan *p)
 uint64_t fnn_plan_len(const fnn_plan *p) { return p ? p->instrs.size() : 0; }
 
 int fnn_plan_replayed(const fnn_plan *p) { return p && p->last_replayed ? 1 : 0; }
+
+uint64_t fnn_plan_ranges_used(const fnn_plan *p) { return p ? p->ranges_used : 0; }
 
 static void touched(fnn_plan *p)
 {

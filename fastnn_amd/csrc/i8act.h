@@ -31,6 +31,11 @@ struct QConvArgs {
     int payload_i4;          // with x8 and I4 weights: the matmul_i4_i8 formula and a float bias
     int nparts;              // > 0: actq is not filled yet; the operand kernel reduces the nparts partial ranges of
                              // its images itself (and stores actq for the epilogue); 0: actq holds the scales
+    int part_stride;         // pairs per (image, group) minmax_partial has room for
+    int range_zero;          // the partial ranges are those of the input tensor as its producer left them: the zero of
+                             // the padding still has to join them
+    float *range_out;        // non-null: partial (min, max) pairs of y per image go here, [B][range_out_stride][2]
+    int range_out_stride;
 };
 constexpr int QCONV_NPART = 512;
 
@@ -42,5 +47,6 @@ hipError_t launch_row_qsum(const fnn_hip_weight *w, int32_t *out, hipStream_t s)
 // phase 0: everything with the direct kernel; 1: range scan + scales; 2: the direct kernel only (scales present);
 // 3: range scan only (*nparts = partial ranges per image and group); 4: scales from *nparts partial ranges
 hipError_t launch_qconv2d_i8(const QConvArgs &p, hipStream_t s, int phase, int *nparts);
+void fnn_conv_coverage(const QConvArgs &p, int *pad_touched, bool *every_input_reached);
 // actq[i] = (scale, zero, 0, 0) of an activation payload's header, for i < nbg
 hipError_t launch_conv_actq_from_payload(const uint8_t *payload, float *actq, int nbg, hipStream_t s);

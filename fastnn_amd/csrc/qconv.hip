@@ -176,10 +176,10 @@ __global__ void __launch_bounds__(256) conv_minmax_flat_kernel(QConvArgs a, int 
 __global__ void __launch_bounds__(64) conv_actq_kernel(QConvArgs a, int nparts)
 {
     const int bg = blockIdx.x;
-    float mn = INFINITY, mx = -INFINITY;
+    float mn = a.range_zero ? 0.0f : INFINITY, mx = a.range_zero ? 0.0f : -INFINITY;
     for (int i = threadIdx.x; i < nparts; i += 64) {
-        mn = fminf(mn, a.minmax_partial[((int64_t)bg * QCONV_NPART + i) * 2]);
-        mx = fmaxf(mx, a.minmax_partial[((int64_t)bg * QCONV_NPART + i) * 2 + 1]);
+        mn = fminf(mn, a.minmax_partial[((int64_t)bg * a.part_stride + i) * 2]);
+        mx = fmaxf(mx, a.minmax_partial[((int64_t)bg * a.part_stride + i) * 2 + 1]);
     }
     mn = wave_min(mn);
     mx = wave_max(mx);
@@ -321,6 +321,36 @@ hipError_t launch_conv_actq_from_payload(const uint8_t *payload, float *actq, in
     return hipGetLastError();
 }
 
+// does any tap fall into the padding (rows and columns separately), and is every input row and column reached by
+// some tap?  With both known, min / max of the im2col matrix are those of the input slab, plus zero if padded.
+void fnn_conv_coverage(const QConvArgs &p, int *pad_touched_out, bool *every_input_reached)
+{
+    int pad_touched = 0;
+    for (int64_t o = 0; o < p.ho && !pad_touched; o++)
+        for (int i = 0; i < p.kh; i++) {
+            const int64_t ih = o * p.stride + (int64_t)i * p.dil - p.pad;
+            if (ih < 0 || ih >= p.h) { pad_touched = 1; break; }
+        }
+    for (int64_t o = 0; o < p.wo && !pad_touched; o++)
+        for (int i = 0; i < p.kw; i++) {
+            const int64_t iw = o * p.stride + (int64_t)i * p.dil - p.pad;
+            if (iw < 0 || iw >= p.w) { pad_touched = 1; break; }
+        }
+    auto all_reached = [&](int64_t len, int taps, int64_t outs) {
+        for (int64_t pos = 0; pos < len; pos++) {
+            bool hit = false;
+            for (int i = 0; i < taps && !hit; i++) {
+                const int64_t num = pos + p.pad - (int64_t)i * p.dil;
+                hit = num >= 0 && num % p.stride == 0 && num / p.stride < outs;
+            }
+            if (!hit) return false;
+        }
+        return true;
+    };
+    *pad_touched_out = pad_touched;
+    *every_input_reached = p.h + p.w <= 32768 && all_reached(p.h, p.kh, p.ho) && all_reached(p.w, p.kw, p.wo);
+}
+
 hipError_t launch_qconv2d_i8(const QConvArgs &p, hipStream_t s, int phase, int *nparts_io)
 {
     const int64_t bg = p.b * p.groups;
@@ -337,33 +367,11 @@ hipError_t launch_qconv2d_i8(const QConvArgs &p, hipStream_t s, int phase, int *
     }
     if (phase != 2) {
         if (p.h + p.w <= 32768 && cg > 0) {
-            // does any tap fall into the padding?  (rows and columns separately)
             int pad_touched = 0;
-            for (int64_t o = 0; o < p.ho && !pad_touched; o++)
-                for (int i = 0; i < p.kh; i++) {
-                    const int64_t ih = o * p.stride + (int64_t)i * p.dil - p.pad;
-                    if (ih < 0 || ih >= p.h) { pad_touched = 1; break; }
-                }
-            for (int64_t o = 0; o < p.wo && !pad_touched; o++)
-                for (int i = 0; i < p.kw; i++) {
-                    const int64_t iw = o * p.stride + (int64_t)i * p.dil - p.pad;
-                    if (iw < 0 || iw >= p.w) { pad_touched = 1; break; }
-                }
-            // is every input row / column reached by some tap?
-            auto all_reached = [&](int64_t len, int taps, int64_t outs) {
-                for (int64_t pos = 0; pos < len; pos++) {
-                    bool hit = false;
-                    for (int i = 0; i < taps && !hit; i++) {
-                        const int64_t num = pos + p.pad - (int64_t)i * p.dil;
-                        hit = num >= 0 && num % p.stride == 0 && num / p.stride < outs;
-                    }
-                    if (!hit) return false;
-                }
-                return true;
-            };
+            bool reached = false;
+            fnn_conv_coverage(p, &pad_touched, &reached);
             const int64_t elems = cg * p.h * p.w;
-            const bool flat = elems % 4 == 0 && (reinterpret_cast<uintptr_t>(p.x) & 15) == 0 &&
-                              all_reached(p.h, p.kh, p.ho) && all_reached(p.w, p.kw, p.wo);
+            const bool flat = elems % 4 == 0 && (reinterpret_cast<uintptr_t>(p.x) & 15) == 0 && reached;
             nparts = (elems + 256 * 4 - 1) / (256 * 4);
             const int64_t cap = 4096 / bg > 32 ? 4096 / bg : 32;   // about 4096 workgroups over all images
             if (nparts > cap) nparts = cap;

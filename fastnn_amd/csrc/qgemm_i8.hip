@@ -10,6 +10,7 @@
 // epilogue kernel applies the reference's float formula (and scatters conv outputs to NCHW).
 #include "mfma.h"
 #include "dech.h"
+#include "range_io.h"
 
 #include <type_traits>
 
@@ -159,8 +160,8 @@ __global__ void __launch_bounds__(256) conv_operand_kernel(QConvArgs a, int g, i
         const int bg_b = (int)dv.np.div((uint32_t)r_last) * a.groups + g;
         const int nimg = bg_b != bg_a ? 2 : 1;
         for (int w = 0; w < nimg; w++) {
-            const float *part = a.minmax_partial + (int64_t)(w ? bg_b : bg_a) * QCONV_NPART * 2;
-            float mn = INFINITY, mx = -INFINITY;
+            const float *part = a.minmax_partial + (int64_t)(w ? bg_b : bg_a) * a.part_stride * 2;
+            float mn = a.range_zero ? 0.0f : INFINITY, mx = a.range_zero ? 0.0f : -INFINITY;
             for (int i = tid; i < a.nparts; i += 256) {
                 mn = fminf(mn, part[i * 2]);
                 mx = fmaxf(mx, part[i * 2 + 1]);
@@ -420,13 +421,16 @@ __global__ void __launch_bounds__(256) conv_epilogue_kernel(QConvArgs a, int g, 
     }
 }
 
-template <int DT, int WGM, int WGN, int TM, int TN, int NS, bool CONV = false>
+template <int DT, int WGM, int WGN, int TM, int TN, int NS, bool CONV = false, bool CRNG = false>
 hipError_t launch_i8_tile(const TileArgs &p, hipStream_t s)
 {
+    if constexpr (CONV && !CRNG) {
+        if (p.cv.range_out) return launch_i8_tile<DT, WGM, WGN, TM, TN, NS, true, true>(p, s);
+    }
     constexpr int WC = 2 * DecI<DT>::WPS;
     constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
     constexpr size_t lds = (size_t)NS * (BM * 128 + BN * WC * 16);
-    auto kern = qgemm_tile_kernel<DT, WGM, WGN, TM, TN, false, NS, true, 0, CONV>;
+    auto kern = qgemm_tile_kernel<DT, WGM, WGN, TM, TN, false, NS, true, 0, CONV, CRNG>;
     static std::atomic<uint64_t> lds_raised{0};
     hipError_t e = fnn_raise_lds_limit(lds_raised, reinterpret_cast<const void *>(kern), (int)lds);
     if (e != hipSuccess) return e;
@@ -632,6 +636,14 @@ int fnn_i8_tiled_conv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, 
             cv.cv.actq = p.actq; cv.cv.qsum = qsum; cv.cv.row_qsum = p.row_qsum + g * ocg;
             cv.cv.oc = p.oc; cv.cv.np = (uint32_t)np; cv.cv.nq = nq; cv.cv.groups = p.groups; cv.cv.g = g; cv.cv.kk = (int)kk;
             cv.cv.vec4 = vec4 ? 1 : 0;
+            // partial ranges of y for the next convolution: one group, and tiles that meet at most two images
+            const int64_t bm = small_tiles ? 64 : 128;
+            const int64_t ntl = small_tiles ? (ocg + 63) / 64 : (ocg <= 64 ? 1 : (ocg + 127) / 128);
+            const int64_t parts = (np / bm + 2) * ntl;
+            if (p.range_out && p.groups == 1 && np >= bm && parts <= p.range_out_stride) {
+                cv.cv.range_out = p.range_out; cv.cv.range_stride = p.range_out_stride;
+                fnn_ctx_range_io(ctx)->out_parts = (int)parts;
+            }
         }
         if (e == hipSuccess)
             e = w->dtype == FNN_DT_I8 ? run_i8_gemm<FNN_DT_I8>(words, kp, w->rows, g * ocg, ocg, a8, rows, rows_pad, kpad, c, ocg, s, 1, fused ? &cv : nullptr, small_tiles)

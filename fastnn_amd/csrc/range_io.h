@@ -1,0 +1,30 @@
+// Value ranges that travel with an f32 tensor from the call that writes it to the quantised Conv2d that reads it:
+// the convolution's dynamic activation quantiser needs min / max of its input per image
+// (src/backend/cpu/im2col.rs:496-507), and a producer that has every value in registers anyway can leave partial
+// (min, max) pairs per image behind, which saves the consumer its scan of the tensor.
+//
+// A table is [images][stride][2] floats; a producer fills `parts` pairs per image (unused ones hold +inf, -inf).
+// The side channel below belongs to one context and to the NEXT call on it: the caller states what it wants
+// before the call and reads what happened after it.
+#pragma once
+#include <cstdint>
+
+struct fnn_hip_ctx;
+
+struct FnnRangeIo {
+    // request to the next call that writes an f32 tensor: leave partial ranges of the output, split in images of
+    // image_elems values, in out_table (room for out_stride pairs per image)
+    float *out_table = nullptr;
+    int out_stride = 0;
+    uint64_t out_image_elems = 0, out_images = 0;
+    int out_parts = 0;        // pairs per image in place: a call appends behind them (a tensor written by several calls,
+                              // e.g. the parts of a concat) and adds what it wrote; 0 after a single call: none
+    int out_failed = 0;       // answer: a call wrote values of the tensor without leaving their ranges
+    // offer to the next quantised Conv2d: partial ranges of its input, one image per batch entry
+    const float *in_table = nullptr;
+    int in_stride = 0, in_parts = 0;
+    int in_used = 0;          // answer: the convolution took them instead of scanning its input
+};
+
+FnnRangeIo *fnn_ctx_range_io(fnn_hip_ctx *ctx);
+bool fnn_ctx_capturing(fnn_hip_ctx *ctx);   // a HIP graph is being recorded on the context's stream: no allocation

@@ -35,6 +35,11 @@ struct TileArgs {
         uint32_t np;
         int nq, groups, g, kk;
         int vec4;                  // np % 4 == 0 and 16-byte aligned outputs: four pixels per store
+        // non-null (only with np >= rows of a tile, so that a tile meets at most two images): partial (min, max)
+        // pairs of the values this launch stores, [image][range_stride][2]; the tile (mt, nt) fills pair
+        // (mt - first tile of the image) * ntiles + nt of every image it meets, (np / BM + 2) * ntiles pairs per image
+        float *range_out;
+        int range_stride;
     } cv;
 };
 
@@ -129,11 +134,12 @@ __device__ __forceinline__ void wait_loads_but()
 // CONV (with INT8, DIG = 0): the rows are im2col rows (image, pixel); the accumulators are turned into the
 //               convolution's outputs here (conv_dequant) and stored NCHW, four consecutive pixels of a channel
 //               per lane and store where the image size allows.
-template <int DT, int WGM, int WGN, int TM, int TN, bool PRECISE, int NS, bool INT8 = false, int DIG = 0, bool CONV = false>
+template <int DT, int WGM, int WGN, int TM, int TN, bool PRECISE, int NS, bool INT8 = false, int DIG = 0, bool CONV = false, bool CRNG = false>
 __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
 {
     static_assert(DIG == 0 || (INT8 && (DIG == 2 || DIG == 4)), "digit planes ride on the int8 operands");
     static_assert(!CONV || (INT8 && DIG == 0), "the conv epilogue belongs to the plain int8 kernel");
+    static_assert(!CRNG || CONV, "output ranges come from the conv epilogue");   // CRNG: p.cv.range_out is set
     // Codebook weights (w[n,k] = bscale[n, k/32] * table[nibble], src/packed_tensor.rs:469-521) are decoded here:
     // the nibble looks up an (f16 hi, f16 lo) pair of the scaled table value in LDS, two MFMAs per step (hi, lo)
     // add into a per-block accumulator, and after the two steps of a 32-value block the accumulator is folded into
@@ -196,6 +202,8 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
     __shared__ float cv_sa[CONV ? WGM * TM * 32 : 1], cv_za[CONV ? WGM * TM * 32 : 1];
     __shared__ int cv_qs[CV_PARTS > 0 ? CV_PARTS : 1][CONV ? WGM * TM * 32 : 1];
     __shared__ int64_t cv_off[CONV ? WGM * TM * 32 : 1];
+    __shared__ unsigned char cv_img[CRNG ? WGM * TM * 32 : 1];   // 0: the image of the tile's first row, 1: the next one
+    __shared__ float cv_red[CRNG ? WGM * WGN : 1][4];
     if constexpr (CONV) {
         constexpr int BM_ = WGM * TM * 32;
         static_assert((WGM * WGN * 64) % BM_ == 0 && CV_PARTS >= 1, "whole row groups per workgroup");
@@ -208,14 +216,17 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
         if (part == 0) {
             float sa = 0.0f, za = 0.0f;
             int64_t off = 0;
+            unsigned char second = 0;
             if (r < p.m) {
                 const uint32_t nn = (uint32_t)r / p.cv.np, px = (uint32_t)r - nn * p.cv.np;
                 const int bg = (int)nn * p.cv.groups + p.cv.g;
                 sa = p.cv.actq[bg * 4 + 0];
                 za = p.cv.actq[bg * 4 + 1];
                 off = (int64_t)nn * p.cv.oc * p.cv.np + px;
+                if constexpr (CRNG) second = (r - row) / p.cv.np != nn;   // (r - row = the tile's first row)
             }
             cv_sa[row] = sa; cv_za[row] = za; cv_off[row] = off;
+            if constexpr (CRNG) cv_img[row] = second;
         }
     }
     // ... and this lane's channel constants (scale, zero, scale * sum q_w, bias)
@@ -582,6 +593,7 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
         const float *sw = cv_sw, *zw = cv_zw, *wt = cv_wt, *bi = cv_bi;
         const bool has_bias = p.bias != nullptr;
         const int64_t np = p.cv.np;
+        float mn0 = INFINITY, mx0 = -INFINITY, mn1 = INFINITY, mx1 = -INFINITY;   // of the stored values, per image
 #pragma unroll
         for (int tm = 0; tm < TM; tm++)
 #pragma unroll
@@ -590,8 +602,10 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
                 const int64_t r0 = (int64_t)mt * BM + rr0;
                 if (r0 >= p.m) continue;
                 float sa[4], za[4], rs[4];
+                bool second[4];
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
+                    second[j] = CRNG ? cv_img[rr0 + j] != 0 : false;
                     int qs = 0;
 #pragma unroll
                     for (int y = 0; y < CV_PARTS; y++) qs += cv_qs[y][rr0 + j];
@@ -617,6 +631,14 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
                         if constexpr (DT == FNN_DT_I4) a >>= 4;
                         v[j] = conv_dequant(a, sa[j], za[j], rs[j], sw[tn], zw[tn], wt[tn], bq[j], p.cv.kk, p.act, &av[j]);
                     }
+                    if constexpr (CRNG) {
+#pragma unroll
+                        for (int j = 0; j < 4; j++) {
+                            if (r0 + j >= p.m) continue;
+                            if (second[j]) { mn1 = fminf(mn1, v[j]); mx1 = fmaxf(mx1, v[j]); }
+                            else { mn0 = fminf(mn0, v[j]); mx0 = fmaxf(mx0, v[j]); }
+                        }
+                    }
                     if (p.cv.vec4) {
                         const int64_t o = cv_off[rr0] + n * np;
                         *reinterpret_cast<float4 *>(p.cv.y + o) = make_float4(v[0], v[1], v[2], v[3]);
@@ -632,6 +654,34 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
                     }
                 }
             }
+        if (CRNG && (int64_t)mt * BM < p.m) {   // (workgroup-uniform)
+            mn0 = wave_min(mn0); mx0 = wave_max(mx0); mn1 = wave_min(mn1); mx1 = wave_max(mx1);
+            if (lane == 0) { cv_red[wv][0] = mn0; cv_red[wv][1] = mx0; cv_red[wv][2] = mn1; cv_red[wv][3] = mx1; }
+            __syncthreads();
+            if (tid == 0) {
+#pragma unroll
+                for (int w2 = 1; w2 < NWV; w2++) {
+                    mn0 = fminf(mn0, cv_red[w2][0]); mx0 = fmaxf(mx0, cv_red[w2][1]);
+                    mn1 = fminf(mn1, cv_red[w2][2]); mx1 = fmaxf(mx1, cv_red[w2][3]);
+                }
+                const int64_t row_a = (int64_t)mt * BM;                                         // first row of the tile
+                const int64_t row_z = row_a + BM - 1 < p.m - 1 ? row_a + BM - 1 : p.m - 1;      // its last real row
+                const int64_t img_a = row_a / np, img_z = row_z / np;                           // (img_z <= img_a + 1)
+                const int per_m = (int)(np / BM) + 2;
+                float *dst = p.cv.range_out + ((img_a * p.cv.range_stride) + ((int64_t)mt - img_a * np / BM) * p.ntiles + nt) * 2;
+                dst[0] = mn0; dst[1] = mx0;
+                if (img_z != img_a) {   // the next image starts in this tile: its pair 0
+                    float *d1 = p.cv.range_out + ((img_z * p.cv.range_stride) + nt) * 2;
+                    d1[0] = mn1; d1[1] = mx1;
+                }
+                if (row_z >= (img_a + 1) * np - 1) {   // the image of the first row ends here: its unused pairs
+                    for (int64_t j = (int64_t)mt - img_a * np / BM + 1; j < per_m; j++) {
+                        float *d2 = p.cv.range_out + ((img_a * p.cv.range_stride) + j * p.ntiles + nt) * 2;
+                        d2[0] = INFINITY; d2[1] = -INFINITY;
+                    }
+                }
+            }
+        }
         return;
     } else if constexpr (INT8) {
         const int64_t mrow = ((int64_t)mt * (BM / 32) + wm * TM) * 32;

@@ -114,7 +114,10 @@ enum {
                                   /* 1 = dequantise + bias + activation + NCHW stores inside the GEMM kernel, 2 = as a kernel */
                                   /* of its own after it, 3 = as 1 on 128-row tiles whatever the size (1 takes 64 x 64 tiles */
                                   /* while those leave CUs idle)                                                           */
-    FNN_OPT_COUNT = 15
+    FNN_OPT_CONV_RANGES = 15,     /* plans: 1 (default) = the instruction that writes the input of a quantised Conv2d leaves   */
+                                  /* partial (min, max) pairs per image behind and the convolution does not scan its input; 0 = */
+                                  /* every convolution scans                                                               */
+    FNN_OPT_COUNT = 16
 };
 int fnn_hip_set_option(fnn_hip_ctx *ctx, int option, int64_t value);
 int fnn_hip_get_option(fnn_hip_ctx *ctx, int option, int64_t *value);

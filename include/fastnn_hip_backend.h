@@ -132,6 +132,10 @@ int fnn_backend_dispatch_from(fnn_backend *b, fnn_plan *p, const char *const *na
 /* 1 when the last dispatch of the plan ran as a graph replay, else 0 (no counterpart in fastnn:
  * lets tests and tools see which path ran). */
 int fnn_plan_replayed(const fnn_plan *p);
+/* Quantised Conv2d instructions of the plan that, on its last pass (or in its recorded graph), took the activation
+ * ranges the instruction before them left instead of scanning their input (FNN_OPT_CONV_RANGES; no counterpart in
+ * fastnn: lets tests and tools see which path ran). */
+uint64_t fnn_plan_ranges_used(const fnn_plan *p);
 /* Backend::dispatch_profile, src/backend/mod.rs:178-211: elapsed_ns[i] per instruction */
 int fnn_backend_dispatch_profile(fnn_backend *b, fnn_plan *p, uint64_t *elapsed_ns, uint64_t n);
 

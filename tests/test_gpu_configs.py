@@ -226,3 +226,37 @@ def test_yolo_graph_node_by_node_against_oracle(orc, batch, size):
         assert all(a <= 1e-1 and b <= 1e-2 for a, b in stats.values()), stats
     finally:
         ex.close()
+
+
+@pytest.mark.parametrize("batch,size", [(3, 160), (1, 224)])
+def test_conv_activation_ranges_from_the_producing_instruction(orc, batch, size):
+    """A quantised Conv2d in a plan takes min / max of its input from partial pairs the instruction before it left
+    (conv epilogue, Split / Concat copies, residual Add, MaxPool, Resize) instead of scanning the tensor.  min and
+    max do not depend on how the values are grouped, so every output must equal, bit for bit, what the plan gives
+    with every convolution scanning its own input; the sizes make output tiles straddle images (20 x 20 = 400 rows
+    per image against 64-row tiles) and fall below one tile (5 x 5), where the producer leaves nothing and the
+    consumer scans."""
+    rng = np.random.default_rng(11)
+    nodes, params, shape, outs = bench.yolo_graph(batch, rng, size=size)
+    x = rng.uniform(0, 1, shape).astype(np.float32)
+    results = {}
+    used = {}
+    for on in (1, 0):
+        ex = AotExecutor(nodes, params, ["x"], outs, {"x": shape}, quantize=8)
+        try:
+            ex.set_option(flib.OPT_CONV_RANGES, on)
+            first = ex.forward({"x": x})
+            again = ex.forward({"x": x})
+            assert ex.replayed
+            used[on] = ex.ranges_used
+            for name in outs:
+                assert np.array_equal(first[name], again[name]), name + ": replay differs from the first dispatch"
+            results[on] = again
+            if on:
+                assert _check_graph_against_oracle(orc, nodes, params, ex, x, f"ranges B={batch} {size}px") == 45
+        finally:
+            ex.close()
+    assert used[0] == 0
+    assert used[1] >= 30, used   # every conv but the first has a producer in the plan; the smallest maps fall back
+    for name in outs:
+        assert np.array_equal(results[1][name], results[0][name]), name
