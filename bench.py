@@ -224,6 +224,8 @@ def composite(args) -> int:
         build_s = time.perf_counter() - t0
         for _, ident, value in parsed_options(args, flib):
             ex.set_option(ident, value)
+        if args.mode == "eager":   # instruction by instruction instead of one HIP-graph replay (kernel traces)
+            ex.set_graph_replay(False)
         ex.write_inputs({"x": rng.uniform(0, 1, shape).astype(np.float32)})
         for _ in range(2 + warm):
             ex.dispatch()
@@ -239,10 +241,10 @@ def composite(args) -> int:
         out = {"metric": f"C5 YOLOv8n-shaped I8 graph forward (backbone + neck as one plan, B={batch})",
                "value": round(batch / (ms * 1e-3), 1), "unit": "images/s", "n_gpus": 1, "steps": steps, "warmup": warm,
                "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "i8/i32",
-               "data": "synthetic", "config": {"workload": args.workload, "launch": "AotExecutor plan, HIP-graph replay + sync per step",
+               "data": "synthetic", "config": {"workload": args.workload, "launch": "AotExecutor plan, " + ("HIP-graph replay" if args.mode == "graph" else "instruction by instruction") + " + sync per step",
                                                "instructions": kinds, "arena_bytes": ex.arena_size,
                                                "options": {n: v for n, _, v in parsed_options(args, flib)}},
-               "tops": round(flops / (ms * 1e-3) / 1e12, 2), "replayed": ex.replayed, "lowering_s": round(build_s, 2),
+               "tops": round(flops / (ms * 1e-3) / 1e12, 2), "replayed": ex.replayed, "convs_with_ranges_from_their_producer": ex.ranges_used, "lowering_s": round(build_s, 2),
                "outputs": [list(t.shape) for t in y], "finite_output": bool(all(np.isfinite(t).all() for t in y))}
         print(json.dumps(out))
         ex.close()

@@ -390,6 +390,11 @@ class AotExecutor:
         self._ensure_plan()
         self._backend.set_option(option, value)
 
+    def set_graph_replay(self, enabled: bool):
+        """Resident plan as one HIP-graph replay (default) or instruction by instruction."""
+        self._ensure_plan()
+        self._backend.set_graph_replay(enabled)
+
     def write_inputs(self, inputs: Dict[str, np.ndarray]):
         """Copies the inputs into their arena slots (what forward() does first)."""
         self._ensure_plan()

@@ -223,11 +223,28 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
                 sa = p.cv.actq[bg * 4 + 0];
                 za = p.cv.actq[bg * 4 + 1];
                 off = (int64_t)nn * p.cv.oc * p.cv.np + px;
-                if constexpr (CRNG) second = (r - row) / p.cv.np != nn;   // (r - row = the tile's first row)
+                if constexpr (CRNG) second = (uint32_t)(r - row) / p.cv.np != nn;   // (r - row = the tile's first row)
             }
             cv_sa[row] = sa; cv_za[row] = za; cv_off[row] = off;
             if constexpr (CRNG) cv_img[row] = second;
         }
+    }
+    // output ranges: which pair of which image this tile fills (32-bit arithmetic: rows < 2^31), worked out before the
+    // K loop.  Pair (tile - first tile of the image) * ntiles + nt; a tile that holds the last row of its first
+    // image also fills that image's unused pairs, up to np / BM + 2 per column tile.
+    uint32_t rng_img = 0;
+    int rng_slot = 0, rng_fill = 0, rng_per_m = 0;
+    bool rng_two = false;
+    if constexpr (CRNG) {
+        constexpr uint32_t BM_ = WGM * TM * 32;
+        const uint32_t np = p.cv.np, row_a = (uint32_t)mt * BM_;
+        const uint32_t last = (uint32_t)p.m - 1, row_z = row_a + BM_ - 1 < last ? row_a + BM_ - 1 : last;
+        rng_img = row_a / np;
+        const uint32_t img_end = (rng_img + 1) * np - 1;           // last row of that image
+        rng_slot = (int)((uint32_t)mt - (rng_img * np) / BM_);
+        rng_two = row_z > img_end;
+        rng_per_m = (int)(np / BM_) + 2;
+        rng_fill = row_z >= img_end ? rng_slot + 1 : rng_per_m;
     }
     // ... and this lane's channel constants (scale, zero, scale * sum q_w, bias)
     float cv_sw[CONV ? TN : 1], cv_zw[CONV ? TN : 1], cv_wt[CONV ? TN : 1], cv_bi[CONV ? TN : 1];
@@ -605,7 +622,7 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
                 bool second[4];
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
-                    second[j] = CRNG ? cv_img[rr0 + j] != 0 : false;
+                    second[j] = (CRNG && rng_two) ? cv_img[rr0 + j] != 0 : false;
                     int qs = 0;
 #pragma unroll
                     for (int y = 0; y < CV_PARTS; y++) qs += cv_qs[y][rr0 + j];
@@ -655,7 +672,8 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
                 }
             }
         if (CRNG && (int64_t)mt * BM < p.m) {   // (workgroup-uniform)
-            mn0 = wave_min(mn0); mx0 = wave_max(mx0); mn1 = wave_min(mn1); mx1 = wave_max(mx1);
+            mn0 = wave_min(mn0); mx0 = wave_max(mx0);
+            if (rng_two) { mn1 = wave_min(mn1); mx1 = wave_max(mx1); }
             if (lane == 0) { cv_red[wv][0] = mn0; cv_red[wv][1] = mx0; cv_red[wv][2] = mn1; cv_red[wv][3] = mx1; }
             __syncthreads();
             if (tid == 0) {
@@ -664,21 +682,16 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
                     mn0 = fminf(mn0, cv_red[w2][0]); mx0 = fmaxf(mx0, cv_red[w2][1]);
                     mn1 = fminf(mn1, cv_red[w2][2]); mx1 = fmaxf(mx1, cv_red[w2][3]);
                 }
-                const int64_t row_a = (int64_t)mt * BM;                                         // first row of the tile
-                const int64_t row_z = row_a + BM - 1 < p.m - 1 ? row_a + BM - 1 : p.m - 1;      // its last real row
-                const int64_t img_a = row_a / np, img_z = row_z / np;                           // (img_z <= img_a + 1)
-                const int per_m = (int)(np / BM) + 2;
-                float *dst = p.cv.range_out + ((img_a * p.cv.range_stride) + ((int64_t)mt - img_a * np / BM) * p.ntiles + nt) * 2;
+                float *row = p.cv.range_out + (int64_t)rng_img * p.cv.range_stride * 2;
+                float *dst = row + ((int64_t)rng_slot * p.ntiles + nt) * 2;
                 dst[0] = mn0; dst[1] = mx0;
-                if (img_z != img_a) {   // the next image starts in this tile: its pair 0
-                    float *d1 = p.cv.range_out + ((img_z * p.cv.range_stride) + nt) * 2;
+                if (rng_two) {   // the next image starts in this tile: its pair 0
+                    float *d1 = row + ((int64_t)p.cv.range_stride + nt) * 2;
                     d1[0] = mn1; d1[1] = mx1;
                 }
-                if (row_z >= (img_a + 1) * np - 1) {   // the image of the first row ends here: its unused pairs
-                    for (int64_t j = (int64_t)mt - img_a * np / BM + 1; j < per_m; j++) {
-                        float *d2 = p.cv.range_out + ((img_a * p.cv.range_stride) + j * p.ntiles + nt) * 2;
-                        d2[0] = INFINITY; d2[1] = -INFINITY;
-                    }
+                for (int j = rng_fill; j < rng_per_m; j++) {   // the image of the first row ends here: its unused pairs
+                    float *d2 = row + ((int64_t)j * p.ntiles + nt) * 2;
+                    d2[0] = INFINITY; d2[1] = -INFINITY;
                 }
             }
         }
