@@ -153,9 +153,9 @@ def yolo_graph(batch, rng, size=640):
     return nodes, params, [batch, 3, size, size], [n3, n4b, n5]
 
 
-def composite(args) -> int:
-    """C4 (FP8 / FP4 MLP stack, 64 tokens) through the plan dispatcher, or C5 (YOLOv8n-shaped I8 conv list)
-    through the conv entry point.  One step = one forward pass over resident inputs."""
+def composite_result(args) -> dict:
+    """C4 (FP8 / FP4 MLP stack, 64 tokens) through the plan dispatcher, or C5 (YOLOv8n-shaped I8 conv list / graph)
+    through the conv entry point / AotExecutor.  One step = one forward pass over resident inputs."""
     import fastnn_amd
     from fastnn_amd import lib as flib
     kind, par = COMPOSITE[args.workload]
@@ -212,9 +212,8 @@ def composite(args) -> int:
                "finite_output": bool(np.isfinite(y).all()),
                "f16x1": {"ms_per_step": round(ms1, 4), "tflop_per_s": round(flops / (ms1 * 1e-3) / 1e12, 2),
                          "max_rel_vs_default": float(np.abs(y1 - y).max() / (np.abs(y).max() + 1e-30))}}
-        print(json.dumps(out))
         be.close()
-        return 0
+        return out
     if kind == "yolo_graph":
         from fastnn_amd.aot import AotExecutor
         batch = par
@@ -246,9 +245,8 @@ def composite(args) -> int:
                                                "options": {n: v for n, _, v in parsed_options(args, flib)}},
                "tops": round(flops / (ms * 1e-3) / 1e12, 2), "replayed": ex.replayed, "convs_with_ranges_from_their_producer": ex.ranges_used, "lowering_s": round(build_s, 2),
                "outputs": [list(t.shape) for t in y], "finite_output": bool(all(np.isfinite(t).all() for t in y))}
-        print(json.dumps(out))
         ex.close()
-        return 0
+        return out
     batch = par
     ctx = fastnn_amd.HipContext(0)
     for _, ident, value in parsed_options(args, flib):
@@ -297,8 +295,12 @@ def composite(args) -> int:
            "data": "synthetic", "config": {"workload": args.workload, "launch": args.mode + ", each conv on its own resident input",
                                            "options": {n: v for n, _, v in parsed_options(args, flib)}},
            "event_ms_per_step": round(ev, 4), "gop_per_step": round(flops / 1e9, 2), "top_per_s": round(flops / (ms * 1e-3) / 1e12, 2)}
-    print(json.dumps(out))
     ctx.close()
+    return out
+
+
+def composite(args) -> int:
+    print(json.dumps(composite_result(args)))
     return 0
 
 
@@ -756,6 +758,22 @@ def main() -> int:
                 gemm_m256["c1_i8_i8act"] = time_i8act(ctx, flib, r2, 256)
             free_ring(ctx, r2)
 
+    # the composite configurations (conv list, conv plan, MLP stack), each its own short run: ms per forward
+    composites = None
+    if not args.no_extra:
+        import copy
+        composites = {}
+        ctx.close()
+        ctx = None
+        for wl in ("c5_yolo_b1", "c5_yolo_b16", "c5_yolo_graph_b1", "c5_yolo_graph_b16", "c4_mlp_f8", "c4_mlp_f4"):
+            a2 = copy.copy(args)
+            a2.workload, a2.steps, a2.warmup, a2.mode, a2.opt = wl, 30, 3, "graph", []
+            try:
+                res = composite_result(a2)
+                composites[wl] = {k2: res[k2] for k2 in ("metric", "ms_per_step", "value", "unit") if k2 in res}
+            except Exception as e:   # the headline stands on its own
+                composites[wl] = {"error": str(e)[:200]}
+
     out = {
         "metric": metric, "value": round(value, 2), "unit": unit, "n_gpus": 1, "steps": steps,
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 6), "higher_is_better": True,
@@ -769,12 +787,14 @@ def main() -> int:
         "cpu_baseline": cpu,
         "gemv_4096": gemv_4096,
         "gemm_m256": gemm_m256,
+        "composites": composites,
         "gb_per_s": round(gbs, 1), "tflop_per_s": round(tops, 3),
         "event_ms_total": round(t["event_ms_total"], 4), "wall_ms_total": round(t["wall_ms_total"], 4),
         "quantize_host_s": round(r["quantize_s"], 3), "self_check_max_rel": t["self_check_max_rel"],
     }
     print(json.dumps(out))
-    ctx.close()
+    if ctx is not None:
+        ctx.close()
     return 0
 
 
