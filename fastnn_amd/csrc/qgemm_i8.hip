@@ -4,10 +4,11 @@
 //     src/backend/cpu/microkernels/gemm.rs:1641-1975), and
 //   - the quantised Conv2d lowering conv2d_packed_i8x4 (im2col + per-(image,group) int8 activation
 //     quantisation + integer GEMM + 4-term dequantise, src/backend/cpu/packed_conv.rs:125-232,444-625).
-// Three launches per call: an operand kernel writes the int8 activation matrix in the tile-major
-// layout of the GEMM kernel (for conv it evaluates im2col and the quantisation on the fly and also
-// leaves sum_k q_a per row), the shared tiled GEMM kernel produces raw i32 accumulators, and an
-// epilogue kernel applies the reference's float formula (and scatters conv outputs to NCHW).
+// An operand kernel writes the int8 activation matrix in the tile-major layout of the GEMM kernel (for conv it
+// evaluates im2col and the quantisation on the fly) and leaves sum_k q_a per row; the shared tiled GEMM kernel
+// produces the i32 accumulators.  MatMul: an epilogue kernel applies the reference's float formula to them.
+// Conv: the same formula, the activation and the NCHW stores run inside the GEMM kernel (or, by option and for
+// the matmul-form epilogue of 4-bit weights on an int8 payload, as a kernel of their own).
 #include "mfma.h"
 #include "dech.h"
 #include "range_io.h"
@@ -434,7 +435,9 @@ hipError_t launch_i8_tile(const TileArgs &p, hipStream_t s)
     static std::atomic<uint64_t> lds_raised{0};
     hipError_t e = fnn_raise_lds_limit(lds_raised, reinterpret_cast<const void *>(kern), (int)lds);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(kern, dim3((unsigned)p.mtiles * p.ntiles * p.splits), dim3(256), lds, s, p);
+    // (a ring of three requests only the stages its K range has: one LDS buffer per stage, at most three)
+    const int bufs = (NS == 3 && p.ips < NS) ? p.ips : NS;
+    hipLaunchKernelGGL(kern, dim3((unsigned)p.mtiles * p.ntiles * p.splits), dim3(256), lds / NS * bufs, s, p);
     return hipGetLastError();
 }
 

@@ -472,13 +472,24 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
                     }
         };
 
+        // With a ring of three a hand-over waits for every outstanding load, so stages past the K range need not be
+        // requested to keep the wait counts right: a short K range (the first conv layers: one or two stages)
+        // then moves no byte twice and needs one LDS buffer per stage it has (the launcher sizes LDS to that).
+        // Deeper rings keep requesting (re-reads of the final stage that nothing consumes).
+        constexpr bool EXACT = NS == 3;
+        const bool one_stage = EXACT && it1 - it0 == 1;   // (workgroup-uniform)
+        if (one_stage) {
+            issue(it0, 0);
+        } else {
 #pragma unroll
-        for (int st = 0; st < NS - 1; st++) issue(it0 + st, st);
+            for (int st = 0; st < NS - 1; st++) issue(it0 + st, st);
+        }
         uint32_t wq[TN][WQW], wqn[TN][WQW];
         f16x8 af[4][TM], bfr[2][TN], bfl[2][CB ? TN : 1];
         if constexpr (CB) load_bscales(it0, bs_cur);
         // first stage: this wave's part has landed
-        if (w_on) wait_loads_but<(NS - 2) * LPS>();
+        if (one_stage) wait_loads_but<0>();
+        else if (w_on) wait_loads_but<(NS - 2) * LPS>();
         else wait_loads_but<(NS - 2) * A_LPW>();
         __syncthreads();                    // ... and everybody else's
         read_w(smem, wq);
@@ -509,7 +520,7 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
             __syncthreads();                    // everybody's; the stage before the current one is free
             int fb = buf + NS - 1;
             if (fb >= NS) fb -= NS;
-            issue(it + NS - 1, fb);
+            if (!EXACT || it + NS - 1 < it1) issue(it + NS - 1, fb);
             // step 2, with the first reads of the next stage
             read_w(nbase, wqn);
             read_a(nbase, 0, af[0]);
