@@ -248,6 +248,23 @@ __device__ __forceinline__ float fnn_epilogue(float dot, float scale, float zero
     return fnn_activation(v, act);
 }
 
+// n / d for 0 <= n < 2^31 by one multiplication (d >= 1 fixed per launch): mul = ceil(2^(31 + ceil(log2 d)) / d)
+struct FastDiv {
+    uint32_t d, mul, shr;
+    __device__ __forceinline__ uint32_t div(uint32_t n) const { return d == 1 ? n : __umulhi(n, mul) >> shr; }
+};
+static inline FastDiv fast_div(uint32_t d)
+{
+    FastDiv f = {d, 0, 0};
+    if (d <= 1) { f.d = 1; return f; }
+    uint32_t lg = 0;
+    while ((1ull << lg) < d) lg++;
+    const uint64_t p2 = 1ull << (31 + lg);
+    f.mul = (uint32_t)((p2 + d - 1) / d);
+    f.shr = lg - 1;
+    return f;
+}
+
 // ---------------------------------------------------------------------------
 // launch parameter blocks
 // ---------------------------------------------------------------------------

@@ -148,6 +148,44 @@ __global__ void __launch_bounds__(256) maxpool2d_kernel(const float *x, uint64_t
     (void)c;
 }
 
+// The same for tensors below 2^31 values: 32-bit index arithmetic, divisions by multiplication.
+__global__ void __launch_bounds__(256) maxpool2d_small_kernel(const float *x, uint32_t in_len, float *y, uint32_t out_len, uint32_t h, uint32_t w,
+                                                              FastDiv ho, FastDiv wo, int kernel, int stride, int pad, int64_t *indices,
+                                                              uint32_t idx_len, RangeEmit re)
+{
+    const uint32_t total = out_len > idx_len ? out_len : idx_len;
+    const uint32_t ie = re.table ? (uint32_t)re.image_elems : total, base = blockIdx.y * ie;
+    float mn = INFINITY, mx = -INFINITY;
+    for (uint32_t j = blockIdx.x * 256 + threadIdx.x; j < ie && base + j < total; j += gridDim.x * 256) {
+        const uint32_t o = base + j;
+        const uint32_t t = wo.div(o), ww = o - t * wo.d, nc = ho.div(t), hh = t - nc * ho.d;
+        const int h0 = (int)(hh * stride) - pad, w0 = (int)(ww * stride) - pad;
+        const uint64_t chan0 = (uint64_t)nc * h * w;   // this channel's first value
+        float val = -INFINITY;
+        int best = 0;
+        for (int kh = 0; kh < kernel; kh++) {
+            const int hi = h0 + kh;
+            if ((unsigned)hi >= h) continue;
+            for (int kw = 0; kw < kernel; kw++) {
+                const int wi = w0 + kw;
+                if ((unsigned)wi >= w) continue;
+                const uint64_t idx = chan0 + (uint32_t)hi * w + (uint32_t)wi;
+                if (idx < in_len) {
+                    const float v = x[idx];
+                    if (v > val) { val = v; best = kh * kernel + kw; }
+                }
+            }
+        }
+        if (o < out_len) {
+            y[o] = val;
+            mn = fminf(mn, val);
+            mx = fmaxf(mx, val);
+        }
+        if (o < idx_len) indices[o] = best;
+    }
+    if (re.table) emit_range(re, mn, mx);
+}
+
 // window mean over the taps inside the image (padding taps neither add nor count), summed in (kh, kw) order
 __global__ void __launch_bounds__(256) avgpool2d_kernel(const float *x, uint64_t in_len, float *y, uint64_t out_len,
                                                         uint64_t h, uint64_t w, uint64_t ho, uint64_t wo, int kernel, int stride, int pad)
@@ -184,6 +222,21 @@ __global__ void __launch_bounds__(256) upsample_nearest2d_kernel(const float *x,
         const uint64_t o = base + j;
         const uint64_t ow = o % wo, t = o / wo, oh = t % ho, nc = t / ho;
         const float v = x[(nc * h + oh / sh) * w + ow / sw];
+        y[o] = v;
+        mn = fminf(mn, v);
+        mx = fmaxf(mx, v);
+    }
+    if (re.table) emit_range(re, mn, mx);
+}
+__global__ void __launch_bounds__(256) upsample_nearest2d_small_kernel(const float *x, float *y, uint32_t total, uint32_t h, uint32_t w, FastDiv ho,
+                                                                       FastDiv wo, FastDiv sh, FastDiv sw, RangeEmit re)
+{
+    const uint32_t ie = re.table ? (uint32_t)re.image_elems : total, base = blockIdx.y * ie;
+    float mn = INFINITY, mx = -INFINITY;
+    for (uint32_t j = blockIdx.x * 256 + threadIdx.x; j < ie && base + j < total; j += gridDim.x * 256) {
+        const uint32_t o = base + j;
+        const uint32_t t = wo.div(o), ow = o - t * wo.d, nc = ho.div(t), oh = t - nc * ho.d;
+        const float v = x[((size_t)nc * h + sh.div(oh)) * w + sw.div(ow)];
         y[o] = v;
         mn = fminf(mn, v);
         mx = fmaxf(mx, v);
@@ -287,8 +340,12 @@ hipError_t launch_maxpool2d(const float *x, uint64_t in_len, float *y, uint64_t 
     const bool images_match = idx_len <= out_len && rio && rio->out_image_elems == c * ho * wo;
     if (!images_match && rio && rio->out_table) rio->out_failed = 1;
     RangePlan rp = range_plan(images_match ? rio : nullptr, out_len, c * ho * wo, c * ho * wo ? out_len / (c * ho * wo) : 0, grid_for(total));
-    hipLaunchKernelGGL(maxpool2d_kernel, rp.grid, dim3(256), 0, s, x, in_len, y, out_len, c, h, w, ho, wo, kernel, stride, pad,
-                       indices, idx_len, rp.re);
+    if (in_len < (1ull << 31) && total < (1ull << 31) && h * w < (1ull << 31))
+        hipLaunchKernelGGL(maxpool2d_small_kernel, rp.grid, dim3(256), 0, s, x, (uint32_t)in_len, y, (uint32_t)out_len, (uint32_t)h, (uint32_t)w,
+                           fast_div((uint32_t)ho), fast_div((uint32_t)wo), kernel, stride, pad, indices, (uint32_t)idx_len, rp.re);
+    else
+        hipLaunchKernelGGL(maxpool2d_kernel, rp.grid, dim3(256), 0, s, x, in_len, y, out_len, c, h, w, ho, wo, kernel, stride, pad,
+                           indices, idx_len, rp.re);
     if (rio) rio->out_parts += rp.parts;
     return hipGetLastError();
 }
@@ -307,7 +364,11 @@ hipError_t launch_upsample_nearest2d(const float *x, float *y, uint64_t nc, uint
     if (total == 0) return hipSuccess;
     const uint64_t per_image = rio && rio->out_table ? rio->out_image_elems : 0;
     RangePlan rp = range_plan(rio, total, per_image, per_image ? total / per_image : 0, grid_for(total));
-    hipLaunchKernelGGL(upsample_nearest2d_kernel, rp.grid, dim3(256), 0, s, x, y, total, h, w, sh, sw, rp.re);
+    if (total < (1ull << 31) && sh >= 1 && sw >= 1)
+        hipLaunchKernelGGL(upsample_nearest2d_small_kernel, rp.grid, dim3(256), 0, s, x, y, (uint32_t)total, (uint32_t)h, (uint32_t)w,
+                           fast_div((uint32_t)(h * sh)), fast_div((uint32_t)(w * sw)), fast_div((uint32_t)sh), fast_div((uint32_t)sw), rp.re);
+    else
+        hipLaunchKernelGGL(upsample_nearest2d_kernel, rp.grid, dim3(256), 0, s, x, y, total, h, w, sh, sw, rp.re);
     if (rio) rio->out_parts += rp.parts;
     return hipGetLastError();
 }
