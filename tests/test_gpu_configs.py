@@ -260,3 +260,71 @@ def test_conv_activation_ranges_from_the_producing_instruction(orc, batch, size)
     assert used[1] >= 30, used   # every conv but the first has a producer in the plan; the smallest maps fall back
     for name in outs:
         assert np.array_equal(results[1][name], results[0][name]), name
+
+
+def test_conv_activation_ranges_odd_shapes_and_every_producer(orc):
+    """Ranges handed over by every kind of producer (conv epilogue with unaligned image sizes, MaxPool, Resize, Add,
+    ReLU, Slice copies of a Split, Concat parts) and the cases that must fall back to a scan (a producer whose output
+    map is smaller than one tile; a strided 1x1 convolution that does not touch every input row): 13 x 11 maps (143
+    pixels per image: tiles straddle the three images, four pixels of a store group straddle them too), outputs equal
+    bit for bit with and without the hand-over."""
+    rng = np.random.default_rng(23)
+    nodes, params = [], {}
+    cnt = [0]
+
+    def uid(p):
+        cnt[0] += 1
+        return f"{p}{cnt[0]}"
+
+    def conv(x, c, oc, k, s, pad):
+        w, b, y0, y = uid("w"), uid("b"), uid("c"), uid("s")
+        kk = c * k * k
+        params[w] = (rng.standard_normal((oc, c, k, k)) * np.sqrt(2.0 / kk)).astype(np.float32)
+        params[b] = (rng.standard_normal(oc) * 0.05).astype(np.float32)
+        nodes.append({"name": y0, "op_type": "Conv", "inputs": f"[{x}, {w}, {b}]", "outputs": f"[{y0}]", "strides": str(s),
+                      "pads": str(pad), "group": "1"})
+        nodes.append({"name": y, "op_type": "Silu", "inputs": f"[{y0}]", "outputs": f"[{y}]"})
+        return y
+
+    c1 = conv("x", 5, 24, 3, 1, 1)                      # [3, 24, 13, 11]
+    c2 = conv(c1, 24, 40, 3, 2, 1)                      # [3, 40, 7, 6]: ranges from c1's epilogue; leaves none (42 pixels)
+    c3 = conv(c2, 40, 16, 1, 2, 0)                      # odd input rows / columns are never read: scans
+    nodes.append({"name": "m", "op_type": "MaxPool", "inputs": f"[{c1}]", "outputs": "[m]", "kernel_size": "3", "stride": "1",
+                  "padding": "1"})
+    c4 = conv("m", 24, 8, 3, 1, 1)
+    nodes.append({"name": "u", "op_type": "Resize", "inputs": f"[{c2}]", "outputs": "[u]", "mode": "nearest", "scale_h": "2",
+                  "scale_w": "2"})
+    c5 = conv("u", 40, 8, 3, 1, 1)
+    nodes.append({"name": "a", "op_type": "Add", "inputs": f"[{c1}, m]", "outputs": "[a]"})
+    c6 = conv("a", 24, 8, 1, 1, 0)
+    nodes.append({"name": "sp", "op_type": "Split", "inputs": f"[{c1}]", "outputs": "[h1, h2]", "axis": "1"})
+    c7 = conv("h2", 12, 8, 3, 1, 1)
+    nodes.append({"name": "k", "op_type": "Concat", "inputs": f"[{c4}, {c6}]", "outputs": "[k]", "axis": "1"})
+    c8 = conv("k", 16, 8, 1, 1, 0)
+    nodes.append({"name": "r", "op_type": "Relu", "inputs": "[m]", "outputs": "[r]"})
+    c9 = conv("r", 24, 8, 3, 1, 1)
+    outs = [c3, c5, c7, c8, c9]
+    shape = (3, 5, 13, 11)
+    x = rng.uniform(-1, 1, shape).astype(np.float32)
+    results, used = {}, {}
+    for on in (1, 0):
+        ex = AotExecutor(nodes, params, ["x"], outs, {"x": shape}, quantize=8)
+        try:
+            ex.set_option(flib.OPT_CONV_RANGES, on)
+            first = ex.forward({"x": x})
+            again = ex.forward({"x": x})
+            assert ex.replayed
+            for name in outs:
+                assert np.array_equal(first[name], again[name]), name
+            results[on], used[on] = again, ex.ranges_used
+            if on:   # the first convolution against the oracle: the scalar NCHW stores with ranges next to them
+                w = params["w1"]
+                pw = to_oracle(orc, fastnn_amd.quantize_weights(flib.DT_I8, w.reshape(24, 45)))
+                want = orc.qconv2d_i8(x, pw, 3, 3, 1, 1, 1, 1, bias=params["b2"], act=flib.ACT_SILU)
+                assert_close(ex.read_output(c1), want, 1e-5, "first convolution")
+        finally:
+            ex.close()
+    assert used[0] == 0
+    assert used[1] == 7, used   # c2, c4, c5, c6, c7, c8, c9; c3 and the first convolution scan
+    for name in outs:
+        assert np.array_equal(results[1][name], results[0][name]), name
