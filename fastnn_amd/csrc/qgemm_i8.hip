@@ -567,6 +567,7 @@ int fnn_i8_tiled_conv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, 
     // rows touch with 32-bit byte offsets from the first of them
     const int64_t span = p.b < 63 / np + 2 ? p.b : 63 / np + 2;
     if (p.kh > 15 || p.kw > 15 || span * p.c * p.h * p.w * 4 > 0xfffffff0ll) return FNN_OK;
+    if (p.pad > 32767 || p.dil > 32767 || p.stride > 32767) return FNN_OK;   // (its 32-bit pixel and tap offsets)
     const int64_t kpad = (kk + KB - 1) / KB * KB;
     const int64_t rows_pad = (rows + 127) / 128 * 128;
     const size_t a_bytes = (size_t)rows_pad * kpad;
