@@ -228,15 +228,26 @@ struct Codec<FNN_DT_I4CB> {
 // epilogue: apply_affine_dot (src/backend/cpu/microkernels/mod.rs:292-295)
 // then bias add and activation (src/backend/cpu/microkernels/activations.rs:557-593)
 // ---------------------------------------------------------------------------
+// x / (1 + exp(-x)) on the hardware exponential and reciprocal (v_exp_f32 of -x*log2(e), v_rcp_f32, one ulp each; the
+// rounded product adds |x| * 6e-8 to the exponential's relative error, which reaches the result scaled by
+// e/(1+e)): a few ulp of the result for x > -4 and below 1e-8 in absolute terms for smaller x, where the result
+// itself vanishes; about 6 instructions against ~35 for expf and an IEEE division.
+__device__ __forceinline__ float fnn_sigmoid_times(float x, float arg)   // x * sigmoid(arg)
+{
+    const float e = __builtin_amdgcn_exp2f(arg * -1.44269504f);   // exp(-arg); inf for arg < -88.7, 0 for arg > 103
+    return x * __builtin_amdgcn_rcpf(1.0f + e);                    // x * 0 where e = inf, as x / inf
+}
 __device__ __forceinline__ float fnn_activation(float v, int act)
 {
     if (act == FNN_ACT_RELU) return v > 0.0f ? v : 0.0f;
     if (act == FNN_ACT_GELU) {
+        // 0.5 * v * (1 + tanh(t)) = v * sigmoid(2t), t = 0.7978846 * (v + 0.044715 * v^3): the same function without
+        // the cancellation of 1 + tanh for negative v
         float x3 = v * v * v;
         float t = 0.7978846f * (v + 0.044715f * x3);
-        return 0.5f * v * (1.0f + tanhf(t));
+        return fnn_sigmoid_times(v, 2.0f * t);
     }
-    if (act == FNN_ACT_SILU) return v / (1.0f + expf(-v));
+    if (act == FNN_ACT_SILU) return fnn_sigmoid_times(v, v);
     return v;
 }
 

@@ -53,15 +53,6 @@ __device__ __forceinline__ int conv_bias_q(float bias, float sa, float sw)
     const float x = bias / (sa * sw);
     return (int)(x + __builtin_copysignf(0.49999997f, x));
 }
-// x / (1 + exp(-x)) on the hardware exponential and reciprocal (v_exp_f32 of -x*log2(e), v_rcp_f32, one ulp each; the
-// rounded product adds |x| * 6e-8 to the exponential's relative error, which reaches the result scaled by
-// e/(1+e)): a few ulp of the result for x > -4 and below 1e-8 in absolute terms for smaller x, where the result
-// itself vanishes; about 6 instructions against ~35 for expf and an IEEE division.
-__device__ __forceinline__ float conv_silu(float x)
-{
-    const float e = __builtin_amdgcn_exp2f(x * -1.44269504f);   // exp(-x); inf for x < -88.7, 0 for x > 103
-    return x * __builtin_amdgcn_rcpf(1.0f + e);                  // x * 0 = -0 where e = inf, as x / inf
-}
 __device__ __forceinline__ float conv_dequant(int acc_in, float sa, float za, float rsum, float sw, float zw, float wt,
                                               int bias_q, int kk, int act, int *acc_out)
 {
@@ -73,8 +64,8 @@ __device__ __forceinline__ float conv_dequant(int acc_in, float sa, float za, fl
     val = val + za * wt;
     val = val + zp_prod * (float)kk;
     if (act == FNN_ACT_RELU) val = fmaxf(val, 0.0f);
-    else if (act == FNN_ACT_SILU) val = conv_silu(val);
-    else if (act == FNN_ACT_GELU) val = val * 0.5f * (1.0f + tanhf(val * 0.7978846f * (1.0f + 0.044715f * val * val)));
+    else if (act == FNN_ACT_SILU) val = fnn_sigmoid_times(val, val);
+    else if (act == FNN_ACT_GELU) val = fnn_sigmoid_times(val, 2.0f * (val * 0.7978846f * (1.0f + 0.044715f * val * val)));   // = 0.5 v (1 + tanh(.))
     *acc_out = accv;
     return val;
 }
