@@ -807,3 +807,37 @@ def test_segmented_dispatch_hands_unsupported_kernels_to_the_caller(be, orc):
         h_ref = orc.qmatmul(to_oracle(orc, w1), x)
         g_ref = (1.0 / (1.0 + np.exp(-h_ref.astype(np.float64)))).astype(np.float32)
         assert_close(be.read_arena(*s_y, np.float32).reshape(m, d), orc.qmatmul(to_oracle(orc, w2), g_ref), 1e-4, f"pass {it}")
+
+
+@pytest.mark.parametrize("batch", [1, 3])
+def test_memcopy_and_fill_feeding_a_convolution(be, orc, batch):
+    """A MemCopy whose destination a quantised Conv2d reads runs as a copy kernel that leaves the activation ranges
+    (the convolution then does not scan); a Fill into the same slice afterwards must drop them again.  Both against
+    the oracle, and the plan's statistics say which path ran."""
+    rng = np.random.default_rng(61)
+    c, h, w, oc, k = 6, 17, 16, 10, 3
+    x = rng.uniform(-1, 1, (batch, c, h, w)).astype(np.float32)
+    pw = fastnn_amd.quantize_weights(flib.DT_I8, (rng.standard_normal((oc, c * k * k)) * 0.1).astype(np.float32))
+    bias = (rng.standard_normal(oc) * 0.05).astype(np.float32)
+    a = Arena()
+    s_in, s_x, s_w, s_b = a.take(x.nbytes), a.take(x.nbytes), a.take(pw.words.nbytes), a.take(bias.nbytes)
+    s_y = a.take(batch * oc * h * w * 4)
+    params, meta = [1, 1, 1, 1, c, h, w, k, k], meta_of(pw, [oc, c, k, k])
+    be.allocate_arena(a.top)
+    # copy, then convolution
+    plan = ExecutablePlan(a.top).write_const(s_w[0], pw.words).write_const(s_b[0], bias)
+    plan.memcopy(s_x, s_in).call_kernel("conv2d_i8_silu", [s_x, s_w, s_b], s_y, params, meta)
+    be.write_arena(s_in[0], x)
+    be.dispatch(plan)
+    want = orc.qconv2d_i8(x, to_oracle(orc, pw), k, k, 1, 1, 1, 1, bias=bias, act=flib.ACT_SILU)
+    assert_close(be.read_arena(*s_y, np.float32).reshape(want.shape), want, 1e-5, "copy -> conv")
+    assert plan.ranges_used == 1
+    be.dispatch(plan)   # (graph replay)
+    assert_close(be.read_arena(*s_y, np.float32).reshape(want.shape), want, 1e-5, "copy -> conv, replayed")
+    # copy, fill of the same slice, convolution: the copy's ranges no longer describe the slice
+    plan2 = ExecutablePlan(a.top).write_const(s_w[0], pw.words).write_const(s_b[0], bias)
+    plan2.memcopy(s_x, s_in).fill(s_x[0], s_x[1], 0.25).call_kernel("conv2d_i8_silu", [s_x, s_w, s_b], s_y, params, meta)
+    be.dispatch(plan2)
+    want2 = orc.qconv2d_i8(np.full_like(x, 0.25), to_oracle(orc, pw), k, k, 1, 1, 1, 1, bias=bias, act=flib.ACT_SILU)
+    assert_close(be.read_arena(*s_y, np.float32).reshape(want2.shape), want2, 1e-5, "copy -> fill -> conv")
+    assert plan2.ranges_used == 0
