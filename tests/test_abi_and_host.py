@@ -35,6 +35,27 @@ def test_backend_header_symbols_exported():
     assert declared == set(flib.BACKEND_SYMBOLS)
 
 
+def test_rust_glue_binds_only_declared_functions():
+    """integration/ffi.rs (the bindings a fastnn maintainer would add) names no function the headers do not declare,
+    and gives each the number of arguments its declaration has."""
+    def c_decls(text):
+        out = {}
+        for name, args in re.findall(r"\b(fnn_[a-z0-9_]+)\s*\(([^;{]*?)\)\s*;", text, re.S):
+            args = args.strip()
+            out[name] = 0 if args in ("", "void") else args.count(",") + 1
+        return out
+    headers = {}
+    for h in ("fastnn_hip.h", "fastnn_hip_backend.h"):
+        headers.update(c_decls(open(os.path.join(ROOT, "include", h)).read()))
+    rust = re.sub(r"//[^\n]*", "", open(os.path.join(ROOT, "integration", "ffi.rs")).read())
+    bound = re.findall(r"\bfn\s+(fnn_[a-z0-9_]+)\s*\(([^)]*)\)", rust, re.S)
+    assert len(bound) >= 20
+    for name, args in bound:
+        assert name in headers, f"ffi.rs binds {name}, which no header declares"
+        n_args = len([a for a in args.split(",") if a.strip()])
+        assert n_args == headers[name], f"{name}: {n_args} arguments in ffi.rs, {headers[name]} in the header"
+
+
 def test_plan_builds_without_a_gpu():
     """Plans are host objects: building one needs no device; malformed instructions are refused."""
     from fastnn_amd.backend import ExecutablePlan
