@@ -35,7 +35,7 @@ __global__ void __launch_bounds__(256) eltwise_kernel(int op, const float *a, co
 {
     for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
         float v = a[i];
-        if (op == 0) v = v + b[i % nb];
+        if (op == 0) v = v + b[nb >= n ? i : i % nb];   // (the usual residual add has operands of one length: no division)
         else v = fnn_activation(v, op);
         out[i] = v;
     }
@@ -43,7 +43,7 @@ __global__ void __launch_bounds__(256) eltwise_kernel(int op, const float *a, co
 // The same with ranges: block (x, y) takes 1024 * U consecutive values of image y, every thread requests its 4 * U
 // operands before it uses the first one.
 template <int U>
-__global__ void __launch_bounds__(256) eltwise_ranges_kernel(int op, const float *a, const float *b, uint64_t nb, float *out, RangeEmit re)
+__global__ void __launch_bounds__(256) eltwise_ranges_kernel(int op, const float *a, const float *b, uint64_t nb, float *out, uint64_t n, RangeEmit re)
 {
     const uint64_t base = (uint64_t)blockIdx.y * re.image_elems, j0 = (uint64_t)blockIdx.x * (1024 * U) + threadIdx.x;
     float va[4 * U], vb[4 * U];
@@ -52,7 +52,7 @@ __global__ void __launch_bounds__(256) eltwise_ranges_kernel(int op, const float
         const uint64_t j = j0 + (uint64_t)k * 256;
         const bool in = j < re.image_elems;
         va[k] = in ? a[base + j] : 0.0f;
-        vb[k] = (in && op == 0) ? b[(base + j) % nb] : 0.0f;
+        vb[k] = (in && op == 0) ? b[nb >= n ? base + j : (base + j) % nb] : 0.0f;
     }
     float mn = INFINITY, mx = -INFINITY;
 #pragma unroll
@@ -83,30 +83,49 @@ __global__ void __launch_bounds__(256) copy2d_kernel(float *dst, uint64_t dst_pi
     }
 }
 // The same with ranges, one image per row, nothing clipped: block (x, y) takes 1024 * U consecutive values of row y,
-// every thread requests its 4 * U values before it stores the first one.
-template <int U>
+// every thread requests its 4 * U values before it stores the first one (V4: as U 16-byte accesses, for rows that
+// start on 16-byte boundaries and hold a multiple of four values).
+template <int U, bool V4>
 __global__ void __launch_bounds__(256) copy2d_ranges_kernel(float *dst, uint64_t dst_pitch, const float *src, uint64_t src_pitch, uint64_t width,
                                                             RangeEmit re)
 {
     const float *s = src + (uint64_t)blockIdx.y * src_pitch;
     float *d = dst + (uint64_t)blockIdx.y * dst_pitch;
-    const uint64_t c0 = (uint64_t)blockIdx.x * (1024 * U) + threadIdx.x;
-    float v[4 * U];
-#pragma unroll
-    for (int k = 0; k < 4 * U; k++) {
-        const uint64_t c = c0 + (uint64_t)k * 256;
-        v[k] = c < width ? s[c] : 0.0f;
-    }
     float mn = INFINITY, mx = -INFINITY;
+    if constexpr (V4) {
+        const uint64_t c0 = ((uint64_t)blockIdx.x * (256 * U) + threadIdx.x) * 4;
+        float4 v[U];
 #pragma unroll
-    for (int k = 0; k < 4 * U; k++) {
-        const uint64_t c = c0 + (uint64_t)k * 256;
-        if (c >= width) continue;
-        d[c] = v[k];
-        mn = fminf(mn, v[k]);
-        mx = fmaxf(mx, v[k]);
+        for (int k = 0; k < U; k++) {
+            const uint64_t c = c0 + (uint64_t)k * 1024;
+            v[k] = c < width ? *reinterpret_cast<const float4 *>(s + c) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+#pragma unroll
+        for (int k = 0; k < U; k++) {
+            const uint64_t c = c0 + (uint64_t)k * 1024;
+            if (c >= width) continue;
+            *reinterpret_cast<float4 *>(d + c) = v[k];
+            mn = fminf(fminf(mn, fminf(v[k].x, v[k].y)), fminf(v[k].z, v[k].w));
+            mx = fmaxf(fmaxf(mx, fmaxf(v[k].x, v[k].y)), fmaxf(v[k].z, v[k].w));
+        }
+    } else {
+        const uint64_t c0 = (uint64_t)blockIdx.x * (1024 * U) + threadIdx.x;
+        float v[4 * U];
+#pragma unroll
+        for (int k = 0; k < 4 * U; k++) {
+            const uint64_t c = c0 + (uint64_t)k * 256;
+            v[k] = c < width ? s[c] : 0.0f;
+        }
+#pragma unroll
+        for (int k = 0; k < 4 * U; k++) {
+            const uint64_t c = c0 + (uint64_t)k * 256;
+            if (c >= width) continue;
+            d[c] = v[k];
+            mn = fminf(mn, v[k]);
+            mx = fmaxf(mx, v[k]);
+        }
     }
-    emit_range(re, mn, mx);
+    if (re.table) emit_range(re, mn, mx);
 }
 
 // window maximum from -inf with a strict `>` (a NaN never wins), taps in the padding skipped
@@ -310,23 +329,31 @@ hipError_t launch_copy2d(float *dst, uint64_t dst_pitch, uint64_t dst_len, const
                          uint64_t width, uint64_t height, hipStream_t s, FnnRangeIo *rio)
 {
     if (width == 0 || height == 0) return hipSuccess;
-    // (one image per row: the caller asks for ranges only when a row of the destination is an image)
-    // (a copy clipped by either length leaves values of the destination it has not seen: no ranges then; nor when a
-    // row of the destination is not an image of the reader)
-    const bool whole = dst_len >= (height - 1) * dst_pitch + width && src_len >= (height - 1) * src_pitch + width &&
-                       rio && rio->out_image_elems == dst_pitch;
-    if (!whole && rio && rio->out_table) rio->out_failed = 1;
-    int u = 1;
-    RangePlan rp = range_plan_chunks(whole ? rio : nullptr, width * height, width, height, &u);
-    if (rp.re.table) {
-        if (u == 1) hipLaunchKernelGGL(copy2d_ranges_kernel<1>, rp.grid, dim3(256), 0, s, dst, dst_pitch, src, src_pitch, width, rp.re);
-        else if (u == 2) hipLaunchKernelGGL(copy2d_ranges_kernel<2>, rp.grid, dim3(256), 0, s, dst, dst_pitch, src, src_pitch, width, rp.re);
-        else if (u == 4) hipLaunchKernelGGL(copy2d_ranges_kernel<4>, rp.grid, dim3(256), 0, s, dst, dst_pitch, src, src_pitch, width, rp.re);
-        else hipLaunchKernelGGL(copy2d_ranges_kernel<8>, rp.grid, dim3(256), 0, s, dst, dst_pitch, src, src_pitch, width, rp.re);
-        rio->out_parts += rp.parts;
-    } else {
+    // a copy clipped by either length keeps the kernel that checks every index (and leaves no ranges: it has not
+    // seen every value of the destination)
+    const bool whole = dst_len >= (height - 1) * dst_pitch + width && src_len >= (height - 1) * src_pitch + width;
+    // ranges: one image per row of the destination, so the rows must be the reader's images
+    const bool wanted = rio && rio->out_table;
+    const bool ranges = wanted && whole && rio->out_image_elems == dst_pitch;
+    if (wanted && !ranges) rio->out_failed = 1;
+    if (!whole || height > 65535) {
+        if (ranges) rio->out_failed = 1;
         hipLaunchKernelGGL(copy2d_kernel, dim3(grid_for(width * height)), dim3(256), 0, s, dst, dst_pitch, dst_len, src, src_pitch, src_len, width, height);
+        return hipGetLastError();
     }
+    int u = 1;
+    RangePlan rp = range_plan_chunks(ranges ? rio : nullptr, width * height, width, height, &u);
+    if (!rp.re.table) {   // no table (none wanted, or no room in it): the same kernel, one block per 1024 values of a row
+        u = 1;
+        rp.grid = dim3((unsigned)((width + 1023) / 1024), (unsigned)height);
+    }
+    const bool v4 = width % 4 == 0 && dst_pitch % 4 == 0 && src_pitch % 4 == 0 && ((reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src)) & 15) == 0;
+    auto go = [&](auto kern) { hipLaunchKernelGGL(kern, rp.grid, dim3(256), 0, s, dst, dst_pitch, src, src_pitch, width, rp.re); };
+    if (u == 1) v4 ? go(copy2d_ranges_kernel<1, true>) : go(copy2d_ranges_kernel<1, false>);
+    else if (u == 2) v4 ? go(copy2d_ranges_kernel<2, true>) : go(copy2d_ranges_kernel<2, false>);
+    else if (u == 4) v4 ? go(copy2d_ranges_kernel<4, true>) : go(copy2d_ranges_kernel<4, false>);
+    else v4 ? go(copy2d_ranges_kernel<8, true>) : go(copy2d_ranges_kernel<8, false>);
+    if (rp.re.table) rio->out_parts += rp.parts;
     return hipGetLastError();
 }
 
@@ -389,10 +416,10 @@ hipError_t launch_eltwise(int op, const float *a, const float *b, uint64_t nb, f
     int u = 1;
     RangePlan rp = range_plan_chunks(rio, n, per_image, per_image ? n / per_image : 0, &u);
     if (rp.re.table) {
-        if (u == 1) hipLaunchKernelGGL(eltwise_ranges_kernel<1>, rp.grid, dim3(256), 0, s, op, a, b, nb ? nb : 1, out, rp.re);
-        else if (u == 2) hipLaunchKernelGGL(eltwise_ranges_kernel<2>, rp.grid, dim3(256), 0, s, op, a, b, nb ? nb : 1, out, rp.re);
-        else if (u == 4) hipLaunchKernelGGL(eltwise_ranges_kernel<4>, rp.grid, dim3(256), 0, s, op, a, b, nb ? nb : 1, out, rp.re);
-        else hipLaunchKernelGGL(eltwise_ranges_kernel<8>, rp.grid, dim3(256), 0, s, op, a, b, nb ? nb : 1, out, rp.re);
+        if (u == 1) hipLaunchKernelGGL(eltwise_ranges_kernel<1>, rp.grid, dim3(256), 0, s, op, a, b, nb ? nb : 1, out, n, rp.re);
+        else if (u == 2) hipLaunchKernelGGL(eltwise_ranges_kernel<2>, rp.grid, dim3(256), 0, s, op, a, b, nb ? nb : 1, out, n, rp.re);
+        else if (u == 4) hipLaunchKernelGGL(eltwise_ranges_kernel<4>, rp.grid, dim3(256), 0, s, op, a, b, nb ? nb : 1, out, n, rp.re);
+        else hipLaunchKernelGGL(eltwise_ranges_kernel<8>, rp.grid, dim3(256), 0, s, op, a, b, nb ? nb : 1, out, n, rp.re);
         rio->out_parts += rp.parts;
         return hipGetLastError();
     }
