@@ -26,6 +26,8 @@ hipError_t launch_fill(float *dst, uint64_t n, float value, hipStream_t s);
 hipError_t launch_eltwise(int op, const float *a, const float *b, uint64_t nb, float *out, uint64_t n, hipStream_t s, FnnRangeIo *rio);
 hipError_t launch_copy2d(float *dst, uint64_t dst_pitch, uint64_t dst_len, const float *src, uint64_t src_pitch, uint64_t src_len,
                          uint64_t width, uint64_t height, hipStream_t s, FnnRangeIo *rio);
+hipError_t launch_concat(float *dst, uint64_t dst_pitch, int n_parts, const float *const *srcs, const uint64_t *widths, uint64_t height,
+                         hipStream_t s, FnnRangeIo *rio, bool *done);
 hipError_t launch_avgpool2d(const float *x, uint64_t in_len, float *y, uint64_t out_len, uint64_t h, uint64_t w,
                             uint64_t ho, uint64_t wo, int kernel, int stride, int pad, hipStream_t s);
 hipError_t launch_maxpool2d(const float *x, uint64_t in_len, float *y, uint64_t out_len, uint64_t c, uint64_t h, uint64_t w,
@@ -952,6 +954,27 @@ int fnn_hip_copy2d_f32(fnn_hip_ctx *ctx, float *dst, uint64_t dst_pitch, uint64_
     return guarded(ctx, "fnn_hip_copy2d_f32", [&]() -> int {
         if (!ctx || ((!dst || !src) && width && height)) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_copy2d_f32: NULL argument");
         HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_copy2d(dst, dst_pitch, dst_len, src, src_pitch, src_len, width, height, ctx->stream, &ctx->range));
+        return FNN_OK;
+    });
+}
+
+int fnn_hip_concat_f32(fnn_hip_ctx *ctx, float *dst, uint64_t dst_pitch, uint64_t dst_len, uint64_t n_parts, const float *const *srcs,
+                       const uint64_t *widths, const uint64_t *src_lens, uint64_t height)
+{
+    return guarded(ctx, "fnn_hip_concat_f32", [&]() -> int {
+        if (!ctx || !dst || (n_parts && (!srcs || !widths || !src_lens))) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_concat_f32: NULL argument");
+        // one launch when nothing is clipped and the parts are few; else part by part
+        bool whole = height > 0 && dst_len >= height * dst_pitch && n_parts <= 8;
+        for (uint64_t j = 0; j < n_parts && whole; j++) whole = srcs[j] && src_lens[j] >= height * widths[j] && widths[j] > 0;
+        bool done = false;
+        if (whole) HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_concat(dst, dst_pitch, (int)n_parts, srcs, widths, height, ctx->stream, &ctx->range, &done));
+        if (done) return FNN_OK;
+        uint64_t off = 0;
+        for (uint64_t j = 0; j < n_parts; j++) {
+            if (off < dst_len && widths[j] && srcs[j])
+                HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_copy2d(dst + off, dst_pitch, dst_len - off, srcs[j], widths[j], src_lens[j], widths[j], height, ctx->stream, &ctx->range));
+            off += widths[j];
+        }
         return FNN_OK;
     });
 }

@@ -128,6 +128,51 @@ __global__ void __launch_bounds__(256) copy2d_ranges_kernel(float *dst, uint64_t
     if (re.table) emit_range(re, mn, mx);
 }
 
+// "concat" along a middle axis in one launch: part j contributes `width[j]` values per outer position, stored at
+// offset off[j] of the destination's row; grid (blocks of 1024 values, outer positions, parts), blocks past a part's
+// width leave at once.  With ranges (one image per outer position) part j's pairs start at pair blk0[j].
+constexpr int CONCAT_MAX_PARTS = 8;
+struct ConcatArgs {
+    const float *src[CONCAT_MAX_PARTS];
+    uint64_t width[CONCAT_MAX_PARTS], off[CONCAT_MAX_PARTS];
+    uint32_t blk0[CONCAT_MAX_PARTS];
+};
+template <bool V4>
+__global__ void __launch_bounds__(256) concat_kernel(float *dst, uint64_t dst_pitch, ConcatArgs a, RangeEmit re)
+{
+    const int part = blockIdx.z;
+    const uint64_t width = a.width[part];
+    if ((uint64_t)blockIdx.x * 1024 >= width) return;   // (workgroup-uniform)
+    const float *s = a.src[part] + (uint64_t)blockIdx.y * width;
+    float *d = dst + (uint64_t)blockIdx.y * dst_pitch + a.off[part];
+    float mn = INFINITY, mx = -INFINITY;
+    if constexpr (V4) {
+        const uint64_t c = ((uint64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+        if (c < width) {
+            const float4 v = *reinterpret_cast<const float4 *>(s + c);
+            *reinterpret_cast<float4 *>(d + c) = v;
+            mn = fminf(fminf(v.x, v.y), fminf(v.z, v.w));
+            mx = fmaxf(fmaxf(v.x, v.y), fmaxf(v.z, v.w));
+        }
+    } else {
+        const uint64_t c0 = (uint64_t)blockIdx.x * 1024 + threadIdx.x;
+        float v[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) v[k] = c0 + k * 256 < width ? s[c0 + k * 256] : 0.0f;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            if (c0 + k * 256 >= width) continue;
+            d[c0 + k * 256] = v[k];
+            mn = fminf(mn, v[k]);
+            mx = fmaxf(mx, v[k]);
+        }
+    }
+    if (re.table) {
+        re.slot0 += (int)a.blk0[part];
+        emit_range(re, mn, mx);
+    }
+}
+
 // window maximum from -inf with a strict `>` (a NaN never wins), taps in the padding skipped
 // indices (nullable): window position kh*kernel + kw of the first strict maximum in (kh, kw) order, 0 when no tap
 // lies inside the image; an output position is visited when it lies inside the value slice or the index slice
@@ -354,6 +399,40 @@ hipError_t launch_copy2d(float *dst, uint64_t dst_pitch, uint64_t dst_len, const
     else if (u == 4) v4 ? go(copy2d_ranges_kernel<4, true>) : go(copy2d_ranges_kernel<4, false>);
     else v4 ? go(copy2d_ranges_kernel<8, true>) : go(copy2d_ranges_kernel<8, false>);
     if (rp.re.table) rio->out_parts += rp.parts;
+    return hipGetLastError();
+}
+
+// every part unclipped: dst holds height * dst_pitch values, part j holds height * width[j]
+hipError_t launch_concat(float *dst, uint64_t dst_pitch, int n_parts, const float *const *srcs, const uint64_t *widths, uint64_t height,
+                         hipStream_t s, FnnRangeIo *rio, bool *done)
+{
+    *done = false;
+    if (n_parts < 1 || n_parts > CONCAT_MAX_PARTS || height == 0 || height > 65535) return hipSuccess;
+    ConcatArgs a = {};
+    uint64_t off = 0, blocks = 0, max_blocks = 0;
+    bool v4 = dst_pitch % 4 == 0 && (reinterpret_cast<uintptr_t>(dst) & 15) == 0;
+    for (int j = 0; j < n_parts; j++) {
+        const uint64_t b = (widths[j] + 1023) / 1024;
+        a.src[j] = srcs[j]; a.width[j] = widths[j]; a.off[j] = off; a.blk0[j] = (uint32_t)blocks;
+        v4 = v4 && widths[j] % 4 == 0 && off % 4 == 0 && (reinterpret_cast<uintptr_t>(srcs[j]) & 15) == 0;
+        off += widths[j];
+        blocks += b;
+        if (b > max_blocks) max_blocks = b;
+    }
+    if (off > dst_pitch || max_blocks == 0 || max_blocks > (1u << 30)) return hipSuccess;
+    RangeEmit re{nullptr, 0, 0, 0};
+    if (rio && rio->out_table) {
+        if (rio->out_images == height && rio->out_image_elems == dst_pitch && off == dst_pitch &&
+            (uint64_t)rio->out_parts + blocks <= (uint64_t)rio->out_stride)
+            re = RangeEmit{rio->out_table, dst_pitch, rio->out_stride, rio->out_parts};
+        else
+            rio->out_failed = 1;
+    }
+    const dim3 grid((unsigned)max_blocks, (unsigned)height, (unsigned)n_parts);
+    if (v4) hipLaunchKernelGGL(concat_kernel<true>, grid, dim3(256), 0, s, dst, dst_pitch, a, re);
+    else hipLaunchKernelGGL(concat_kernel<false>, grid, dim3(256), 0, s, dst, dst_pitch, a, re);
+    if (re.table) rio->out_parts += (int)blocks;
+    *done = true;
     return hipGetLastError();
 }
 

@@ -530,17 +530,16 @@ int run_concat(fnn_backend *b, const Instr &in)
         const uint64_t outer = in.params[2] ? in.params[2] : 1;
         uint64_t pitch = 0;
         for (const auto &s : in.inputs) pitch += (s.size / 4) / outer;
-        uint64_t off = 0;
+        std::vector<const float *> srcs;
+        std::vector<uint64_t> widths, lens;
         for (const auto &s : in.inputs) {
-            const uint64_t len = s.size / 4, bs = len / outer;
+            const uint64_t len = s.size / 4;
             if (len % outer) return fail(b, FNN_ERR_DISPATCH, "concat: input of %llu elements does not split into %llu outer positions", (unsigned long long)len, (unsigned long long)outer);
-            if (off < out_len) {
-                int st = lift(b, fnn_hip_copy2d_f32(b->ctx, out + off, pitch, out_len - off, (const float *)(b->arena + s.offset), bs, len, bs, in.params[2]));
-                if (st) return st;
-            }
-            off += bs;
+            srcs.push_back((const float *)(b->arena + s.offset));
+            widths.push_back(len / outer);
+            lens.push_back(len);
         }
-        return FNN_OK;
+        return lift(b, fnn_hip_concat_f32(b->ctx, out, pitch, out_len, srcs.size(), srcs.data(), widths.data(), lens.data(), in.params[2]));
     }
     uint64_t off = 0;   // legacy form without axis information: inputs one after the other
     for (const auto &s : in.inputs) {

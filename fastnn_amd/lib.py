@@ -61,7 +61,7 @@ BACKEND_SYMBOLS = [
     "fnn_plan_set_param_dims", "fnn_plan_from_bincode", "fnn_plan_to_bincode", "fnn_plan_describe",
     "fnn_backend_dispatch", "fnn_backend_dispatch_env", "fnn_backend_dispatch_from", "fnn_backend_dispatch_profile",
     "fnn_hip_elementwise", "fnn_hip_fill_f32", "fnn_hip_copy",
-    "fnn_hip_copy2d_f32", "fnn_hip_maxpool2d_f32", "fnn_hip_avgpool2d_f32", "fnn_hip_upsample_nearest2d_f32",
+    "fnn_hip_copy2d_f32", "fnn_hip_concat_f32", "fnn_hip_maxpool2d_f32", "fnn_hip_avgpool2d_f32", "fnn_hip_upsample_nearest2d_f32",
 ]
 
 
@@ -202,6 +202,7 @@ def _prototype(l):
     l.fnn_hip_fill_f32.argtypes = [_vp, _vp, _u64, C.c_float]
     l.fnn_hip_copy.argtypes = [_vp, _vp, _vp, _u64]
     l.fnn_hip_copy2d_f32.argtypes = [_vp, _vp, _u64, _u64, _vp, _u64, _u64, _u64, _u64]
+    l.fnn_hip_concat_f32.argtypes = [_vp, _vp, _u64, _u64, _u64, _vp, _vp, _vp, _u64]
     l.fnn_hip_maxpool2d_f32.argtypes = [_vp, _vp, _u64, _vp, _u64, _u64, _u64, _u64, _u64, _u64, _u64, _u64, _vp, _u64]
     l.fnn_hip_avgpool2d_f32.argtypes = [_vp, _vp, _u64, _vp, _u64, _u64, _u64, _u64, _u64, _u64, _u64, _u64]
     l.fnn_hip_upsample_nearest2d_f32.argtypes = [_vp, _vp, _vp, _u64, _u64, _u64, _u64, _u64]

@@ -149,6 +149,9 @@ int fnn_hip_elementwise(fnn_hip_ctx *ctx, int op, const float *a, const float *b
  *  copy2d: `height` rows of `width` values, dst[r*dst_pitch + c] = src[r*src_pitch + c], dropped where either
  *    index leaves its buffer: the block copies of "concat" (src/backend/cpu/mod.rs:4267-4324) and "slice_f32"
  *    (:4721-4760);
+ *  concat: the parts of one "concat" (:4267-4324) in one call: part j holds `height` rows of widths[j] values
+ *    (src_lens[j] values in all) and lands at the sum of the widths before it in each row of dst (dst_pitch values
+ *    per row); one launch when nothing is clipped and there are at most 8 parts, else a copy2d per part;
  *  maxpool2d: "pool_f32" with is_max = 1 (:4362-4397, src/backend/cpu/microkernels/ops.rs:104-158), output
  *    Ho = sat_sub(H + 2*pad, kernel)/stride + 1, writes past out_len dropped; indices (nullable, idx_len i64
  *    entries) receives kh*kernel + kw of the first strict maximum in (kh, kw) order, 0 for an empty window;
@@ -157,6 +160,8 @@ int fnn_hip_elementwise(fnn_hip_ctx *ctx, int op, const float *a, const float *b
  *  upsample_nearest2d: "upsample_nearest2d" (:5496-5535, src/backend/cpu/microkernels/misc.rs:338-364). */
 int fnn_hip_copy2d_f32(fnn_hip_ctx *ctx, float *dst, uint64_t dst_pitch, uint64_t dst_len, const float *src,
                        uint64_t src_pitch, uint64_t src_len, uint64_t width, uint64_t height);
+int fnn_hip_concat_f32(fnn_hip_ctx *ctx, float *dst, uint64_t dst_pitch, uint64_t dst_len, uint64_t n_parts,
+                       const float *const *srcs, const uint64_t *widths, const uint64_t *src_lens, uint64_t height);
 int fnn_hip_maxpool2d_f32(fnn_hip_ctx *ctx, const float *x, uint64_t in_len, float *y, uint64_t out_len,
                           uint64_t n, uint64_t c, uint64_t h, uint64_t w, uint64_t kernel, uint64_t stride,
                           uint64_t pad, int64_t *indices, uint64_t idx_len);
