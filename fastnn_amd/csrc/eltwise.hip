@@ -64,7 +64,7 @@ __global__ void __launch_bounds__(256) eltwise_ranges_kernel(int op, const float
         mn = fminf(mn, v);
         mx = fmaxf(mx, v);
     }
-    emit_range(re, mn, mx);
+    if (re.table) emit_range(re, mn, mx);
 }
 __global__ void __launch_bounds__(256) fill_kernel(float *dst, uint64_t n, float value)
 {
@@ -307,6 +307,23 @@ __global__ void __launch_bounds__(256) upsample_nearest2d_small_kernel(const flo
     }
     if (re.table) emit_range(re, mn, mx);
 }
+// ... four consecutive outputs of a row per thread (output rows of a multiple of four values, 16-byte aligned y)
+__global__ void __launch_bounds__(256) upsample_nearest2d_v4_kernel(const float *x, float *y, uint32_t total, uint32_t h, uint32_t w, FastDiv ho,
+                                                                    FastDiv wo4, FastDiv sh, FastDiv sw, RangeEmit re)
+{
+    const uint32_t ie = (re.table ? (uint32_t)re.image_elems : total) / 4, base = blockIdx.y * ie;   // in groups of four
+    float mn = INFINITY, mx = -INFINITY;
+    for (uint32_t j = blockIdx.x * 256 + threadIdx.x; j < ie && base + j < total / 4; j += gridDim.x * 256) {
+        const uint32_t o4 = base + j;
+        const uint32_t t = wo4.div(o4), ow = (o4 - t * wo4.d) * 4, nc = ho.div(t), oh = t - nc * ho.d;
+        const float *row = x + ((size_t)nc * h + sh.div(oh)) * w;
+        const float4 v = make_float4(row[sw.div(ow)], row[sw.div(ow + 1)], row[sw.div(ow + 2)], row[sw.div(ow + 3)]);
+        *reinterpret_cast<float4 *>(y + (size_t)o4 * 4) = v;
+        mn = fminf(fminf(mn, fminf(v.x, v.y)), fminf(v.z, v.w));
+        mx = fmaxf(fmaxf(mx, fmaxf(v.x, v.y)), fmaxf(v.z, v.w));
+    }
+    if (re.table) emit_range(re, mn, mx);
+}
 }  // namespace
 
 static unsigned grid_for(uint64_t n)
@@ -470,7 +487,12 @@ hipError_t launch_upsample_nearest2d(const float *x, float *y, uint64_t nc, uint
     if (total == 0) return hipSuccess;
     const uint64_t per_image = rio && rio->out_table ? rio->out_image_elems : 0;
     RangePlan rp = range_plan(rio, total, per_image, per_image ? total / per_image : 0, grid_for(total));
-    if (total < (1ull << 31) && sh >= 1 && sw >= 1)
+    if (total < (1ull << 31) && sh >= 1 && sw >= 1 && (w * sw) % 4 == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0 &&
+        (!rp.re.table || rp.re.image_elems % 4 == 0)) {
+        const dim3 grid(rp.re.table ? rp.grid.x : grid_for(total / 4), rp.grid.y);
+        hipLaunchKernelGGL(upsample_nearest2d_v4_kernel, grid, dim3(256), 0, s, x, y, (uint32_t)total, (uint32_t)h, (uint32_t)w,
+                           fast_div((uint32_t)(h * sh)), fast_div((uint32_t)(w * sw / 4)), fast_div((uint32_t)sh), fast_div((uint32_t)sw), rp.re);
+    } else if (total < (1ull << 31) && sh >= 1 && sw >= 1)
         hipLaunchKernelGGL(upsample_nearest2d_small_kernel, rp.grid, dim3(256), 0, s, x, y, (uint32_t)total, (uint32_t)h, (uint32_t)w,
                            fast_div((uint32_t)(h * sh)), fast_div((uint32_t)(w * sw)), fast_div((uint32_t)sh), fast_div((uint32_t)sw), rp.re);
     else
@@ -500,6 +522,11 @@ hipError_t launch_eltwise(int op, const float *a, const float *b, uint64_t nb, f
         else if (u == 4) hipLaunchKernelGGL(eltwise_ranges_kernel<4>, rp.grid, dim3(256), 0, s, op, a, b, nb ? nb : 1, out, n, rp.re);
         else hipLaunchKernelGGL(eltwise_ranges_kernel<8>, rp.grid, dim3(256), 0, s, op, a, b, nb ? nb : 1, out, n, rp.re);
         rio->out_parts += rp.parts;
+        return hipGetLastError();
+    }
+    if (n <= (1ull << 40)) {   // no table: the same kernel over the whole tensor as one image (all operands of a thread requested first)
+        const RangeEmit none{nullptr, n, 0, 0};
+        hipLaunchKernelGGL(eltwise_ranges_kernel<1>, dim3((unsigned)((n + 1023) / 1024)), dim3(256), 0, s, op, a, b, nb ? nb : 1, out, n, none);
         return hipGetLastError();
     }
     uint64_t blocks = (n + 255) / 256;
