@@ -816,8 +816,7 @@ int fnn_hip_qconv2d(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *x, i
             } else {
                 HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qconv2d_i8(p, ctx->stream, 3, &nparts));
             }
-            const int64_t kk_g = (c / groups) * kh * kw;
-            const int64_t operand_wgs = ((b * ho * wo + 63) / 64) * (((kk_g + 15) / 16 + 3) / 4);
+            const int64_t operand_wgs = fnn_conv_operand_workgroups(p);
             const bool fused_scales = ho * wo >= 64 && nparts <= 4 * QCONV_NPART && operand_wgs <= 8192;   // many workgroups: cheaper once
             if (fused_scales) p.nparts = nparts;
             else HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qconv2d_i8(p, ctx->stream, 4, &nparts));

@@ -35,6 +35,8 @@ int fnn_digits_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w,
 int fnn_tiled_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &p,
                       int flags, bool *handled);
 
+int64_t fnn_conv_operand_workgroups(const QConvArgs &p);
+
 // single-f16 activation mode: mean lane value per weight row (null for types whose lanes have zero mean)
 int fnn_row_means(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const float **umean);
 

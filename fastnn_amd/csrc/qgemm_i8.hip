@@ -554,6 +554,29 @@ int fnn_i8_tiled_matmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w
     return FNN_OK;
 }
 
+namespace {
+// chunks per wave of the operand kernel: more of them spread a lane's per-pixel set-up over more taps, fewer keep the
+// launch wide
+int conv_chunks_per_wave(int64_t rows_pad, int64_t chunks)
+{
+    const int64_t wg1 = (rows_pad / 64) * ((chunks + CONV_CPB - 1) / CONV_CPB);   // workgroups with one chunk per wave
+    if (wg1 < 2048) return 1;
+    // enough workgroups left: the fewest chunk groups of at most 4 chunks per wave, evenly filled
+    const int64_t groups_max = (chunks + CONV_CPB * 4 - 1) / (CONV_CPB * 4);
+    return (int)((chunks + CONV_CPB * groups_max - 1) / (CONV_CPB * groups_max));
+}
+}  // namespace
+
+// workgroups the operand kernel of this convolution launches per group (each reduces the partial activation ranges of
+// its images itself when the scales are not formed yet)
+int64_t fnn_conv_operand_workgroups(const QConvArgs &p)
+{
+    const int64_t rows = p.b * p.ho * p.wo, rows_pad = (rows + 127) / 128 * 128;
+    const int64_t chunks = ((p.c / p.groups) * p.kh * p.kw + 15) / 16;
+    const int nc = conv_chunks_per_wave(rows_pad, chunks);
+    return (rows_pad / 64) * ((chunks + CONV_CPB * nc - 1) / (CONV_CPB * nc));
+}
+
 // after the (image, group) activation scales are known (p.actq): operand, integer GEMM and epilogue per group
 int fnn_i8_tiled_conv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QConvArgs &p, bool *handled)
 {
@@ -574,14 +597,8 @@ int fnn_i8_tiled_conv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, 
     const size_t q_off = (a_bytes + 255) / 256 * 256;
     void *ws1 = nullptr, *ws3 = nullptr;
     int rc;
-    // chunks per wave: more of them spread a lane's per-pixel set-up over more taps, fewer keep the launch wide
     const int64_t chunks = (kk + 15) / 16;
-    const int64_t wg1 = (rows_pad / 64) * ((chunks + CONV_CPB - 1) / CONV_CPB);   // workgroups with one chunk per wave
-    int nc = 1;
-    if (wg1 >= 2048) {   // enough workgroups left: the fewest chunk groups of at most 4 chunks per wave, evenly filled
-        const int64_t groups_max = (chunks + CONV_CPB * 4 - 1) / (CONV_CPB * 4);
-        nc = (int)((chunks + CONV_CPB * groups_max - 1) / (CONV_CPB * groups_max));
-    }
+    const int nc = conv_chunks_per_wave(rows_pad, chunks);
     const int nq = (int)((chunks + CONV_CPB * nc - 1) / (CONV_CPB * nc));   // partial row sums per row
     if (nq > 65535) return FNN_OK;
     if ((rc = fnn_ctx_ensure_tmp(ctx, 3, q_off + (size_t)rows_pad * 4 * nq + 256, &ws3))) return rc;   // 0 holds the scales
