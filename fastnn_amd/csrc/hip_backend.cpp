@@ -693,6 +693,16 @@ void request_ranges(fnn_backend *b, fnn_plan *p, size_t idx, fnn_slice *covered)
         const Instr &nx = p->instrs[j];
         ConvInput cj;
         if (ranged_conv_input(nx, &cj) && nx.inputs[0].offset == in.dst.offset && nx.inputs[0].size <= in.dst.size && cj.images <= 65535) {
+            if (b->range_tables.size() > 1024 && !fnn_ctx_capturing(b->ctx)) {
+                // plans come and go on a long-lived backend: the tables of the others are dropped (they get new
+                // ones on their next pass)
+                for (auto it = b->range_tables.begin(); it != b->range_tables.end();) {
+                    if (it->first.first == p->uid) { ++it; continue; }
+                    if (it->second.dev) fnn_hip_free(b->ctx, it->second.dev);
+                    it = b->range_tables.erase(it);
+                }
+                b->weights_epoch++;   // captured graphs may hold a dropped table
+            }
             auto &t = b->range_tables[{p->uid, idx}];
             if (t.dev && t.images < cj.images && !fnn_ctx_capturing(b->ctx)) {
                 fnn_hip_free(b->ctx, t.dev);
