@@ -20,7 +20,7 @@ LIB = os.path.join(HERE, "libfastnn_hip.so")
 PROBE_LIB = os.path.join(HERE, "libfnn_probe.so")
 PROBE_SOURCE = "probe.hip"
 
-HIP_SOURCES = ["api.hip", "qgemv.hip", "qgemm_generic.hip", "qgemm_tiled.hip", "qgemm_i8.hip", "qgemm_digits.hip", "qgemv_mfma.hip", "qgemv_i8dot.hip", "qgemv_rows16.hip", "i8act.hip", "qconv.hip", "qconv_float.hip", "eltwise.hip"]
+HIP_SOURCES = ["api.hip", "qgemv.hip", "qgemm_generic.hip", "qgemm_tiled.hip", "qgemm_i8.hip", "qgemm_digits.hip", "qgemv_mfma.hip", "qgemv_i8dot.hip", "qgemv_rows16.hip", "i8act.hip", "qconv.hip", "qconv_float.hip", "qconv_implicit.hip", "eltwise.hip"]
 HOST_SOURCES = ["quantize_host.cpp", "hip_backend.cpp"]
 
 # -ffp-contract=off: the integer/quantisation formulas must evaluate exactly as written;

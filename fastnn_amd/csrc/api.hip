@@ -135,6 +135,7 @@ const OptionSpec kOptions[FNN_OPT_COUNT] = {
     {8, 1, 16},       // FNN_OPT_GEMV_INT8_MAX_M
     {0, 0, 3},        // FNN_OPT_CONV_EPILOGUE
     {1, 0, 1},        // FNN_OPT_CONV_RANGES
+    {0, 0, 2},        // FNN_OPT_CONV_IMPLICIT
 };
 
 #define HIP_TRY(ctx, code, expr)                                                              \
@@ -801,9 +802,7 @@ int fnn_hip_qconv2d(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *x, i
             }
             // Activation ranges: from the partial pairs the producer of x left (usable when the im2col matrix holds
             // every input value, i.e. every input row and column is reached by some tap, and the group is the whole
-            // image; the zero of the padding joins them), else from a scan of x.  The scales are then formed by the
-            // operand kernel itself (one launch less) when a workgroup's 64 rows touch at most two images and the
-            // pairs are few, else by the small kernel of their own.
+            // image; the zero of the padding joins them), else from a scan of x.
             int nparts = 0;
             int pad_touched = 0;
             bool all_reached = false;
@@ -816,13 +815,20 @@ int fnn_hip_qconv2d(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *x, i
             } else {
                 HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qconv2d_i8(p, ctx->stream, 3, &nparts));
             }
-            const int64_t operand_wgs = fnn_conv_operand_workgroups(p);
-            const bool fused_scales = ho * wo >= 64 && nparts <= 4 * QCONV_NPART && operand_wgs <= 8192;   // many workgroups: cheaper once
+            // One implicit-GEMM kernel where it is ahead, else the operand kernel and the int8 GEMM.  Either forms
+            // the scales itself when its workgroups' rows touch at most two images and they are few enough for the
+            // repeated reduction to be cheaper than a launch.
+            int wg_rows = 64;
+            int64_t wgs = 0;
+            const bool implicit = fnn_implicit_conv_takes(w, p, ctx->options[FNN_OPT_CONV_IMPLICIT], &wg_rows, &wgs);
+            if (!implicit) { wg_rows = 64; wgs = fnn_conv_operand_workgroups(p); }
+            const bool fused_scales = ho * wo >= wg_rows && nparts <= 4 * QCONV_NPART && wgs <= 8192;
             if (fused_scales) p.nparts = nparts;
             else HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qconv2d_i8(p, ctx->stream, 4, &nparts));
             bool handled = false;
-            int rc2 = fnn_i8_tiled_conv(ctx, ctx->stream, w, p, &handled);
+            int rc2 = implicit ? fnn_i8_implicit_conv(ctx, ctx->stream, w, p, &handled) : fnn_i8_tiled_conv(ctx, ctx->stream, w, p, &handled);
             if (rc2) return rc2;
+            if (implicit && !handled) return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, "the implicit convolution kernel declined a shape it had accepted");
             if (!handled) {
                 if (fused_scales) HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qconv2d_i8(p, ctx->stream, 4, &nparts));
                 p.nparts = 0;

@@ -38,6 +38,35 @@ struct QConvArgs {
     int range_out_stride;
 };
 constexpr int QCONV_NPART = 512;
+// divisors of the im2col index arithmetic: pixels per image, output width, kernel area, kernel width
+struct ConvDivs { FastDiv np, wo, khw, kw; };
+
+// One output of the quantised Conv2d: acc = acc_in + bias_q; val = acc*sab + zw*(sa*sum q_a) + za*(sw*sum q_w)
+// + (za*zw)*K, left to right, then the activation (src/backend/cpu/packed_conv.rs:469-505,571,604-606).
+// rsum = sa * sum q_a of the row, wt = sw * sum q_w of the channel.
+// bias_q = round(bias / (sa*sw)) half away from zero, saturated: trunc(x + copysign(0.49999997, x)) equals roundf(x)
+// wherever the result fits an i32, and the conversion saturates and maps NaN to 0
+__device__ __forceinline__ int conv_bias_q(float bias, float sa, float sw)
+{
+    const float x = bias / (sa * sw);
+    return (int)(x + __builtin_copysignf(0.49999997f, x));
+}
+__device__ __forceinline__ float conv_dequant(int acc_in, float sa, float za, float rsum, float sw, float zw, float wt,
+                                              int bias_q, int kk, int act, int *acc_out)
+{
+    const float sab = sa * sw;
+    const int accv = acc_in + bias_q;
+    const float zp_prod = za * zw;
+    float val = (float)accv * sab;
+    val = val + zw * rsum;
+    val = val + za * wt;
+    val = val + zp_prod * (float)kk;
+    if (act == FNN_ACT_RELU) val = fmaxf(val, 0.0f);
+    else if (act == FNN_ACT_SILU) val = fnn_sigmoid_times(val, val);
+    else if (act == FNN_ACT_GELU) val = fnn_sigmoid_times(val, 2.0f * (val * 0.7978846f * (1.0f + 0.044715f * val * val)));   // = 0.5 v (1 + tanh(.))
+    *acc_out = accv;
+    return val;
+}
 
 hipError_t launch_quantize_activations(const float *x, int64_t numel, float scale, float zp,
                                        uint8_t *payload, float *scratch_partial, hipStream_t s);

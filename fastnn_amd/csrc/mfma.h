@@ -36,6 +36,9 @@ int fnn_tiled_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, 
                       int flags, bool *handled);
 
 int64_t fnn_conv_operand_workgroups(const QConvArgs &p);
+// the implicit-GEMM convolution (qconv_implicit.hip): rows of one of its workgroups for this shape, and the call
+bool fnn_implicit_conv_takes(const fnn_hip_weight *w, const QConvArgs &p, int option, int *wg_rows, int64_t *wgs);
+int fnn_i8_implicit_conv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QConvArgs &p, bool *handled);
 
 // single-f16 activation mode: mean lane value per weight row (null for types whose lanes have zero mean)
 int fnn_row_means(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const float **umean);

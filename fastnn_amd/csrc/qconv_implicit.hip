@@ -1,0 +1,476 @@
+// Quantised Conv2d (I8 or I4 weights, f32 NCHW activations) as one implicit GEMM on the int8 matrix cores:
+// conv2d_packed_i8x4 / conv2d_packed_i4x8 (src/backend/cpu/packed_conv.rs:125-283,444-841) without an im2col
+// operand in memory.  A wave owns 32 output pixels and TN x 32 output channels.  Per step of 32 k-values a lane
+// (pixel lane & 31, k half lane >> 5) fetches its 16 im2col taps straight from the NCHW input, quantises them with the
+// image's scale (q = clamp(round((v - za) * inv)), exactly the operand kernel's arithmetic) and packs them into the
+// A operand of v_mfma_i32_32x32x32_i8; the weight rows come as 16-byte loads in operand order.  KW waves of a
+// workgroup split the K range of the same pixels and add their exact i32 accumulators through LDS; the first of them
+// applies the reference's float formula (conv_dequant) and stores NCHW, four pixels of a channel per store.
+#include "mfma.h"
+#include "dech.h"
+#include "range_io.h"
+
+namespace {
+
+using namespace dech;
+
+struct ImplicitArgs {
+    QConvArgs a;
+    ConvDivs dv;
+    int g, kk, vec4;
+};
+
+template <int DT, int TN, int PW, int KW, bool RNG>
+__global__ void __launch_bounds__(64 * PW * KW) conv_implicit_kernel(ImplicitArgs p)
+{
+    constexpr int NW = PW * KW;
+    constexpr bool W4 = DT == FNN_DT_I4;
+    constexpr int WBYTES = W4 ? 8 : 16;          // packed bytes of 16 k-values of a weight row
+    const QConvArgs &a = p.a;
+    extern __shared__ int red[];                 // [PW][KW - 1][TN * 16 + 1][64]: accumulators and q sums of the other K slices
+    __shared__ float s_mm[2][2][NW];
+    __shared__ float s_q[2][3];
+    __shared__ float r_sa[PW][32], r_za[PW][32];
+    __shared__ int r_qs[PW][32];
+    __shared__ int64_t r_off[PW][32];
+    __shared__ float s_rng[PW][4];
+    __shared__ int r_img[PW][32];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6), pw = wv / KW, kw = wv % KW;
+    const int lr = lane & 31, hf = lane >> 5;
+    const int g = p.g, kk = p.kk;
+    const uint32_t np = (uint32_t)(a.ho * a.wo), wo = (uint32_t)a.wo;
+    const int64_t rows = a.b * (int64_t)np;
+    const int cg = (int)a.c / a.groups, ocg = (int)(a.oc / a.groups);
+    const int64_t r_first = (int64_t)blockIdx.x * (32 * PW);
+    const int64_t n0 = (int64_t)blockIdx.y * (TN * 32);
+    const uint32_t nn0 = p.dv.np.div((uint32_t)(r_first < rows ? r_first : 0));   // image of the workgroup's first row
+
+    // ---- activation scales: from the partial ranges (a.nparts > 0: the workgroup's rows meet at most two images) or
+    // from actq, as in the operand kernel of the explicit path
+    const bool own_scales = a.nparts > 0 && r_first < rows;
+    int bg_a = 0;
+    if (own_scales) {
+        const int64_t r_last = r_first + 32 * PW - 1 < rows ? r_first + 32 * PW - 1 : rows - 1;
+        bg_a = (int)nn0 * a.groups + g;
+        const int bg_b = (int)p.dv.np.div((uint32_t)r_last) * a.groups + g;
+        const int nimg = bg_b != bg_a ? 2 : 1;
+        for (int w = 0; w < nimg; w++) {
+            const float2 *part = reinterpret_cast<const float2 *>(a.minmax_partial) + (int64_t)(w ? bg_b : bg_a) * a.part_stride;
+            float mn = a.range_zero ? 0.0f : INFINITY, mx = a.range_zero ? 0.0f : -INFINITY;
+            for (int i = tid; i < a.nparts; i += 64 * NW) {
+                const float2 t = part[i];
+                mn = fminf(mn, t.x);
+                mx = fmaxf(mx, t.y);
+            }
+            mn = wave_min(mn);
+            mx = wave_max(mx);
+            if (lane == 0) { s_mm[w][0][wv] = mn; s_mm[w][1][wv] = mx; }
+        }
+        __syncthreads();
+        if (tid < nimg) {
+            float mn = s_mm[tid][0][0], mx = s_mm[tid][1][0];
+#pragma unroll
+            for (int w2 = 1; w2 < NW; w2++) { mn = fminf(mn, s_mm[tid][0][w2]); mx = fmaxf(mx, s_mm[tid][1][w2]); }
+            const float range = mx - mn;
+            float scale, zero;
+            if (W4) {
+                scale = (range > 0.0f) ? range / 15.0f : 1.0f;
+                zero = mn + 8.0f * scale;
+            } else {
+                scale = (range > 0.0f) ? range / 255.0f : 1.0f;
+                zero = (range > 0.0f) ? mn + 128.0f * scale : 0.0f;
+            }
+            const float inv = (scale != 0.0f) ? 1.0f / scale : 0.0f;
+            s_q[tid][0] = scale; s_q[tid][1] = zero; s_q[tid][2] = inv;
+        }
+        __syncthreads();
+    }
+
+    // ---- this lane's pixel
+    const int64_t r = r_first + pw * 32 + lr;
+    const bool live = r < rows;
+    const uint32_t ru = live ? (uint32_t)r : 0u;
+    const uint32_t nn = p.dv.np.div(ru), px = ru - nn * np;
+    const uint32_t oh = p.dv.wo.div(px), ow = px - oh * wo;
+    const int bg = (int)nn * a.groups + g;
+    float sa = 1.0f, za = 0.0f, inv = 0.0f;
+    if (a.nparts <= 0) {
+        sa = a.actq[bg * 4 + 0]; za = a.actq[bg * 4 + 1]; inv = a.actq[bg * 4 + 2];
+    } else if (own_scales) {
+        const int w = bg != bg_a ? 1 : 0;
+        sa = s_q[w][0]; za = s_q[w][1]; inv = s_q[w][2];
+    }
+    // one buffer descriptor per workgroup over the input from the group's slab of image nn0 on: a tap outside the
+    // image, past K or of a row past the last one gets the offset ~0, which the range check answers with zero
+    const int64_t img = a.c * a.h * a.w;
+    const int64_t slab0 = ((int64_t)nn0 * a.c + (int64_t)g * cg) * a.h * a.w;
+    const int64_t left = (a.b * img - slab0) * 4;
+    const __amdgpu_buffer_rsrc_t xbuf = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float *>(a.x + slab0), 0, (int)(uint32_t)(left > 0xfffffff0ll ? 0xfffffff0ll : left), 0x00020000);
+    const int hh = (int)a.h, ww = (int)a.w;
+    constexpr int qlo = W4 ? -8 : -128, qhi = W4 ? 7 : 127;
+    const int ih0 = (int)oh * a.stride - a.pad, iw0 = (int)ow * a.stride - a.pad;
+    uint32_t okbits = 0;   // kernel rows (bits 0..14) and columns (16..30) inside the image for this pixel
+    for (int i = 0; i < a.kh; i++) okbits |= ((unsigned)(ih0 + i * a.dil) < (unsigned)hh ? 1u : 0u) << i;
+    for (int j = 0; j < a.kw; j++) okbits |= ((unsigned)(iw0 + j * a.dil) < (unsigned)ww ? 0x10000u : 0u) << j;
+    if (!live) okbits = 0;
+    const uint32_t lane_base = ((uint32_t)(nn - nn0) * (uint32_t)img + (uint32_t)(ih0 * ww + iw0)) * 4;   // (mod 2^32)
+
+    // ---- weights: rows n0 + tn*32 + lr of the group, 16 k-values from byte (32*s + 16*hf) * bits / 8 of the row
+    const int64_t wrow0 = (int64_t)g * ocg + n0;
+    const int64_t wleft = ((int64_t)a.oc - wrow0) * a.kp * 4 + 256;   // (the zeroed margin behind the last row)
+    const __amdgpu_buffer_rsrc_t wbuf = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint32_t *>(a.words + wrow0 * a.kp), 0, (int)(uint32_t)(wleft > 0xfffffff0ll ? 0xfffffff0ll : wleft), 0x00020000);
+    uint32_t wlane[TN];
+#pragma unroll
+    for (int tn = 0; tn < TN; tn++) {
+        const int64_t n = n0 + tn * 32 + lr;
+        wlane[tn] = n < ocg ? (uint32_t)((tn * 32 + lr) * a.kp * 4 + hf * WBYTES) : ~0u;   // rows past the group: zero weights
+    }
+
+    const int nsteps = (kk + 31) / 32;
+    const uint32_t bperm = (uint32_t)(hf * 16) * 4;   // this lane's 16 taps sit in lanes 16*hf .. 16*hf + 15 of the geometry
+    i32x16 acc[TN];
+#pragma unroll
+    for (int tn = 0; tn < TN; tn++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) acc[tn][i] = 0;
+    int qs = 0;
+
+    // tap geometry of a step: lane l & 31 works out tap 32*s + (l & 31): offset inside the slab and the validity bits
+    // it needs (bit 31, never set in okbits, for taps past K)
+    auto geometry = [&](int s, uint32_t &tap_off, uint32_t &tap_need) {
+        const uint32_t e = (uint32_t)(32 * s + lr);
+        const uint32_t ic = p.dv.khw.div(e), rem = e - ic * (uint32_t)(a.kh * a.kw);
+        const uint32_t i = p.dv.kw.div(rem), j = rem - i * (uint32_t)a.kw;
+        tap_off = ((ic * (uint32_t)hh + i * (uint32_t)a.dil) * (uint32_t)ww + j * (uint32_t)a.dil) * 4;
+        tap_need = (int)e < kk ? ((1u << i) | (0x10000u << j)) : 0x80000000u;
+    };
+    auto fetch = [&](int s, float(&v)[16], u32x4(&wq)[TN]) {
+        uint32_t tap_off, tap_need;
+        geometry(s, tap_off, tap_need);
+#pragma unroll
+        for (int t = 0; t < 16; t++) {
+            const uint32_t soff = (uint32_t)__builtin_amdgcn_ds_bpermute((int)(bperm + 4 * t), (int)tap_off);
+            const uint32_t need = (uint32_t)__builtin_amdgcn_ds_bpermute((int)(bperm + 4 * t), (int)tap_need);
+            const uint32_t vo = (okbits & need) == need ? lane_base + soff : ~0u;
+            v[t] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xbuf, vo, 0, 0));
+        }
+#pragma unroll
+        for (int tn = 0; tn < TN; tn++) {
+            const uint32_t wo_ = wlane[tn] == ~0u ? ~0u : wlane[tn] + (uint32_t)s * (2 * WBYTES);
+            if (W4) {
+                const auto t2 = __builtin_amdgcn_raw_buffer_load_b64(wbuf, wo_, 0, 0);
+                wq[tn][0] = t2[0]; wq[tn][1] = t2[1]; wq[tn][2] = 0; wq[tn][3] = 0;
+            } else {
+                wq[tn] = __builtin_amdgcn_raw_buffer_load_b128(wbuf, wo_, 0, 0);
+            }
+        }
+    };
+    auto consume = [&](int s, const float(&v)[16], const u32x4(&wq)[TN]) {
+        int q[16];
+#pragma unroll
+        for (int t = 0; t < 16; t++) {
+            // round half away from zero, then clamp: trunc(x + copysign(0.49999997, x)) equals roundf(x) after the
+            // clamp for every float (the conversion truncates, saturates and maps NaN to 0)
+            const float x = (v[t] - za) * inv;
+            const int qi = (int)(x + __builtin_copysignf(0.49999997f, x));
+            q[t] = max(qlo, min(qi, qhi));
+        }
+        // operand byte `pos` holds tap (pos & 8) + k(pos & 7): the order the weight decoder delivers
+        i32x4 af;
+#pragma unroll
+        for (int wi = 0; wi < 4; wi++) {
+            int tp[4];
+#pragma unroll
+            for (int bq = 0; bq < 4; bq++) {
+                const int pos = wi * 4 + bq, sl = pos & 7;
+                tp[bq] = (pos & 8) + (W4 ? ((sl & 3) * 2 + (sl >> 2)) : sl);
+            }
+            const uint32_t lo = __builtin_amdgcn_perm((uint32_t)q[tp[1]], (uint32_t)q[tp[0]], 0x0c0c0400u);
+            const uint32_t hi = __builtin_amdgcn_perm((uint32_t)q[tp[3]], (uint32_t)q[tp[2]], 0x04000c0cu);
+            af[wi] = (int)(lo | hi);
+        }
+        const int past = 32 * s + 16 * hf + 16 - kk;   // taps of this lane past K: their bytes are cleared
+        if (past > 0) {
+#pragma unroll
+            for (int wi = 0; wi < 4; wi++) {
+                uint32_t keep = 0;
+#pragma unroll
+                for (int bq = 0; bq < 4; bq++) {
+                    const int pos = wi * 4 + bq, sl = pos & 7;
+                    const int tpp = (pos & 8) + (W4 ? ((sl & 3) * 2 + (sl >> 2)) : sl);
+                    keep |= (tpp < 16 - past) ? (0xffu << (8 * bq)) : 0u;
+                }
+                af[wi] &= (int)keep;
+            }
+        }
+#pragma unroll
+        for (int wi = 0; wi < 4; wi++) qs = __builtin_amdgcn_sdot4(af[wi], 0x01010101, qs, false);
+#pragma unroll
+        for (int tn = 0; tn < TN; tn++) {
+            const uint32_t w4[4] = {wq[tn][0], wq[tn][1], wq[tn][2], wq[tn][3]};
+            const f16x8 bf = DecI<DT>::step(w4);
+            acc[tn] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, __builtin_bit_cast(i32x4, bf), acc[tn], 0, 0, 0);
+        }
+    };
+
+    // ---- K loop of this wave: steps kw, kw + KW, ...; the next step's loads are requested before this one is used
+    {
+        float v0[16], v1[16];
+        u32x4 w0[TN], w1[TN];
+        int s = kw;
+        if (s < nsteps) fetch(s, v0, w0);
+        for (; s < nsteps; s += 2 * KW) {
+            if (s + KW < nsteps) fetch(s + KW, v1, w1);
+            consume(s, v0, w0);
+            if (s + KW < nsteps) {
+                if (s + 2 * KW < nsteps) fetch(s + 2 * KW, v0, w0);
+                consume(s + KW, v1, w1);
+            }
+        }
+    }
+
+    // ---- the K slices of a pixel block meet in LDS (exact integers: any order)
+    constexpr int SLOT = (TN * 16 + 1) * 64;
+    if (KW > 1) {
+        if (kw > 0) {
+            int *dst = red + (pw * (KW - 1) + (kw - 1)) * SLOT + lane;
+#pragma unroll
+            for (int tn = 0; tn < TN; tn++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) dst[(tn * 16 + i) * 64] = acc[tn][i];
+            dst[TN * 16 * 64] = qs;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k2 = 0; kw == 0 && k2 < KW - 1; k2++) {
+            const int *src = red + (pw * (KW - 1) + k2) * SLOT + lane;
+#pragma unroll
+            for (int tn = 0; tn < TN; tn++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) acc[tn][i] += src[(tn * 16 + i) * 64];
+            qs += src[TN * 16 * 64];
+        }
+    }
+    qs += __shfl_xor(qs, 32, 64);   // the two k halves of a pixel
+
+    // ---- epilogue: row constants through this wave's LDS rows, then acc[tn][i] = pixel (i/4)*8 + hf*4 + i%4 of the
+    // block, channel n0 + tn*32 + lr
+    // output ranges (RNG): the workgroup (block of 32 * PW pixels, column tile) fills pair
+    // (block - first block of the image) * column tiles + tile of every image it meets, (np / (32 * PW) + 2) * tiles
+    // pairs per image; the block that holds the last pixel of its first image also fills that image's unused pairs
+    float mn0 = INFINITY, mx0 = -INFINITY, mn1 = INFINITY, mx1 = -INFINITY;
+    bool rng_two = false;
+    if constexpr (RNG) {
+        const uint32_t row_z = (uint32_t)(r_first + 32 * PW - 1 < rows ? r_first + 32 * PW - 1 : rows - 1);
+        rng_two = r_first < rows && row_z > (nn0 + 1) * np - 1;
+    }
+    if (kw == 0) {
+        if (hf == 0) {
+            r_sa[pw][lr] = sa; r_za[pw][lr] = za; r_qs[pw][lr] = qs;
+            r_off[pw][lr] = (int64_t)nn * a.oc * np + px;
+            if (RNG) r_img[pw][lr] = nn != nn0;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        float sw[TN], zw[TN], bi[TN];
+        int wq_[TN];
+#pragma unroll
+        for (int tn = 0; tn < TN; tn++) {
+            const int64_t n = n0 + tn * 32 + lr;
+            const bool ok = n < ocg;
+            const int64_t ch = (int64_t)g * ocg + (ok ? n : 0);
+            sw[tn] = ok ? a.scales[ch] : 0.0f;
+            zw[tn] = ok ? a.zeros[ch] : 0.0f;
+            wq_[tn] = ok ? a.row_qsum[ch] : 0;
+            bi[tn] = (ok && a.bias) ? a.bias[ch] : 0.0f;
+        }
+        const bool has_bias = a.bias != nullptr;
+        float *y = a.y + (int64_t)g * ocg * np;
+        int32_t *acc_out = a.acc_out ? a.acc_out + (int64_t)g * ocg * np : nullptr;
+#pragma unroll
+        for (int ig = 0; ig < 4; ig++) {
+            const int rr0 = ig * 8 + hf * 4;
+            const int64_t r0 = r_first + pw * 32 + rr0;
+            if (r0 >= rows) continue;
+            float rsa[4], rza[4], rs[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                rsa[j] = r_sa[pw][rr0 + j];
+                rza[j] = r_za[pw][rr0 + j];
+                rs[j] = rsa[j] * (float)r_qs[pw][rr0 + j];
+            }
+#pragma unroll
+            for (int tn = 0; tn < TN; tn++) {
+                const int64_t n = n0 + tn * 32 + lr;
+                if (n >= ocg) continue;
+                float v[4];
+                int av[4], bq[4];
+                bq[0] = has_bias ? conv_bias_q(bi[tn], rsa[0], sw[tn]) : 0;
+#pragma unroll
+                for (int j = 1; j < 4; j++) bq[j] = (p.vec4 || !has_bias) ? bq[0] : conv_bias_q(bi[tn], rsa[j], sw[tn]);
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    int ai = acc[tn][ig * 4 + j];
+                    if (W4) ai >>= 4;
+                    v[j] = conv_dequant(ai, rsa[j], rza[j], rs[j], sw[tn], zw[tn], sw[tn] * (float)wq_[tn], bq[j], kk, a.act, &av[j]);
+                }
+                if constexpr (RNG) {
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        if (r0 + j >= rows) continue;
+                        if (rng_two && r_img[pw][rr0 + j]) { mn1 = fminf(mn1, v[j]); mx1 = fmaxf(mx1, v[j]); }
+                        else { mn0 = fminf(mn0, v[j]); mx0 = fmaxf(mx0, v[j]); }
+                    }
+                }
+                if (p.vec4) {
+                    const int64_t o = r_off[pw][rr0] + n * np;
+                    *reinterpret_cast<float4 *>(y + o) = make_float4(v[0], v[1], v[2], v[3]);
+                    if (acc_out) *reinterpret_cast<int4 *>(acc_out + o) = make_int4(av[0], av[1], av[2], av[3]);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        if (r0 + j >= rows) continue;
+                        const int64_t o = r_off[pw][rr0 + j] + n * np;
+                        y[o] = v[j];
+                        if (acc_out) acc_out[o] = av[j];
+                    }
+                }
+            }
+        }
+    }
+    if constexpr (RNG) {
+        if (r_first >= rows) return;   // (workgroup-uniform)
+        if (kw == 0) {
+            mn0 = wave_min(mn0); mx0 = wave_max(mx0);
+            if (rng_two) { mn1 = wave_min(mn1); mx1 = wave_max(mx1); }
+            if (lane == 0) { s_rng[pw][0] = mn0; s_rng[pw][1] = mx0; s_rng[pw][2] = mn1; s_rng[pw][3] = mx1; }
+        }
+        __syncthreads();
+        if (tid == 0) {
+#pragma unroll
+            for (int w2 = 1; w2 < PW; w2++) {
+                mn0 = fminf(mn0, s_rng[w2][0]); mx0 = fmaxf(mx0, s_rng[w2][1]);
+                mn1 = fminf(mn1, s_rng[w2][2]); mx1 = fmaxf(mx1, s_rng[w2][3]);
+            }
+            constexpr uint32_t BM = 32 * PW;
+            const uint32_t row_z = (uint32_t)(r_first + BM - 1 < rows ? r_first + BM - 1 : rows - 1);
+            const uint32_t img_end = (nn0 + 1) * np - 1;
+            const int nt = (int)blockIdx.y, ntiles = (int)gridDim.y;
+            const int slot = (int)(blockIdx.x - (nn0 * np) / BM), per_m = (int)(np / BM) + 2;
+            const int fill = row_z >= img_end ? slot + 1 : per_m;
+            float *row = a.range_out + (int64_t)nn0 * a.range_out_stride * 2;
+            float *dst = row + ((int64_t)slot * ntiles + nt) * 2;
+            dst[0] = mn0; dst[1] = mx0;
+            if (rng_two) {   // the next image starts in this block: its pair 0
+                float *d1 = row + ((int64_t)a.range_out_stride + nt) * 2;
+                d1[0] = mn1; d1[1] = mx1;
+            }
+            for (int j = fill; j < per_m; j++) {
+                float *d2 = row + ((int64_t)j * ntiles + nt) * 2;
+                d2[0] = INFINITY; d2[1] = -INFINITY;
+            }
+        }
+    }
+}
+
+template <int DT, int TN, int PW, int KW>
+hipError_t launch_implicit(const ImplicitArgs &p, int64_t rows, int64_t ocg, hipStream_t s)
+{
+    constexpr size_t lds = (size_t)PW * (KW - 1) * (TN * 16 + 1) * 64 * 4;
+    static_assert(lds <= 48 * 1024, "the K slices meet in the default LDS allowance");
+    const dim3 grid((unsigned)((rows + 32 * PW - 1) / (32 * PW)), (unsigned)((ocg + TN * 32 - 1) / (TN * 32)));
+    if (p.a.range_out) hipLaunchKernelGGL((conv_implicit_kernel<DT, TN, PW, KW, true>), grid, dim3(64 * PW * KW), lds, s, p);
+    else hipLaunchKernelGGL((conv_implicit_kernel<DT, TN, PW, KW, false>), grid, dim3(64 * PW * KW), lds, s, p);
+    return hipGetLastError();
+}
+
+template <int DT>
+hipError_t run_implicit(const ImplicitArgs &p, int64_t rows, int64_t ocg, int tn, int kw, hipStream_t s)
+{
+    if (tn == 2) {
+        if (kw == 4) return launch_implicit<DT, 2, 1, 4>(p, rows, ocg, s);
+        if (kw == 2) return launch_implicit<DT, 2, 2, 2>(p, rows, ocg, s);
+        return launch_implicit<DT, 2, 4, 1>(p, rows, ocg, s);
+    }
+    if (kw == 4) return launch_implicit<DT, 1, 1, 4>(p, rows, ocg, s);
+    if (kw == 2) return launch_implicit<DT, 1, 2, 2>(p, rows, ocg, s);
+    return launch_implicit<DT, 1, 4, 1>(p, rows, ocg, s);
+}
+
+// shape of the launch: channels per wave (tn * 32), K slices per pixel block, pixels of a workgroup
+void implicit_shape(const QConvArgs &p, int *tn_out, int *kw_out, int *wg_rows)
+{
+    const int64_t np = p.ho * p.wo, rows = p.b * np;
+    const int64_t ocg = p.oc / p.groups, kk = (p.c / p.groups) * p.kh * p.kw;
+    const int tn = ocg > 32 ? 2 : 1;
+    const int64_t ntn = (ocg + tn * 32 - 1) / (tn * 32);
+    const int64_t steps = (kk + 31) / 32;
+    // K slices per pixel block: more of them while the launch would leave CUs idle and a slice keeps a few steps
+    int kw = 1;
+    if (((rows + 127) / 128) * ntn < 512 && steps >= 4) kw = 2;
+    if (((rows + 63) / 64) * ntn < 256 && steps >= 8) kw = 4;
+    *tn_out = tn; *kw_out = kw; *wg_rows = 128 / kw;   // four waves: 4, 2 or 1 pixel blocks of 32
+}
+
+}  // namespace
+
+// Does the implicit kernel take this convolution?  option: FNN_OPT_CONV_IMPLICIT (0: where it measured faster than
+// the operand kernel + GEMM pair, 1: wherever it can run, 2: never).  *wg_rows = pixels of one of its workgroups,
+// *wgs = their number (the caller decides with them whether the kernel forms the activation scales itself: a
+// workgroup's rows must meet at most two images).
+bool fnn_implicit_conv_takes(const fnn_hip_weight *w, const QConvArgs &p, int option, int *wg_rows, int64_t *wgs)
+{
+    if (option == 2) return false;
+    if ((w->dtype != FNN_DT_I8 && w->dtype != FNN_DT_I4) || p.x8 || p.payload_i4) return false;
+    const int64_t np = p.ho * p.wo, rows = p.b * np;
+    const int64_t cg = p.c / p.groups, ocg = p.oc / p.groups, kk = cg * p.kh * p.kw;
+    if (rows < 1 || rows > (1ll << 28) || kk > (1 << 20) || ocg < 1) return false;
+    if (cg * p.h * p.w >= (1ll << 29) || np >= (1ll << 31)) return false;
+    int tn, kw, wr;
+    implicit_shape(p, &tn, &kw, &wr);
+    const int64_t span = p.b < (wr - 1) / np + 2 ? p.b : (wr - 1) / np + 2;   // images under one buffer descriptor
+    if (p.kh > 15 || p.kw > 15 || span * p.c * p.h * p.w * 4 > 0xfffffff0ll) return false;
+    if (p.pad > 32767 || p.dil > 32767 || p.stride > 32767) return false;
+    if (ocg * p.kp * 4 > 0x7fffffffll) return false;   // 32-bit byte offsets inside a tile's weight rows
+    if (option != 1) {
+        // one pass over the pixels per 32 * tn channels: ahead of the pair while the channels fit one or two MFMA
+        // columns and the launch has pixels enough to fill the chip
+        if (ocg > 64) return false;
+        if (rows < (tn == 1 ? 2048 : 65536)) return false;
+    }
+    if (wg_rows) *wg_rows = wr;
+    if (wgs) *wgs = ((rows + wr - 1) / wr) * ((ocg + tn * 32 - 1) / (tn * 32));
+    return true;
+}
+
+// p.range_out: the partial ranges of y are left when a workgroup meets at most two images and the pairs fit
+// (ctx's out_parts says so), as by the fused epilogue of the explicit path
+int fnn_i8_implicit_conv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QConvArgs &p, bool *handled)
+{
+    *handled = false;
+    if (!fnn_implicit_conv_takes(w, p, 1, nullptr, nullptr)) return FNN_OK;
+    const int64_t np = p.ho * p.wo, rows = p.b * np;
+    const int64_t cg = p.c / p.groups, ocg = p.oc / p.groups, kk = cg * p.kh * p.kw;
+    int tn, kw, wg_rows;
+    implicit_shape(p, &tn, &kw, &wg_rows);
+    ImplicitArgs ia;
+    ia.a = p;
+    ia.dv = ConvDivs{fast_div((uint32_t)np), fast_div((uint32_t)p.wo), fast_div((uint32_t)(p.kh * p.kw)), fast_div((uint32_t)p.kw)};
+    ia.kk = (int)kk;
+    ia.vec4 = (np % 4 == 0 && (reinterpret_cast<uintptr_t>(p.y) & 15) == 0 && (!p.acc_out || (reinterpret_cast<uintptr_t>(p.acc_out) & 15) == 0)) ? 1 : 0;
+    const int64_t parts = (np / wg_rows + 2) * ((ocg + tn * 32 - 1) / (tn * 32));
+    if (p.range_out && p.groups == 1 && np >= wg_rows && parts <= p.range_out_stride) fnn_ctx_range_io(ctx)->out_parts = (int)parts;
+    else ia.a.range_out = nullptr;
+    for (int g = 0; g < p.groups; g++) {
+        ia.g = g;
+        const hipError_t e = w->dtype == FNN_DT_I8 ? run_implicit<FNN_DT_I8>(ia, rows, ocg, tn, kw, s) : run_implicit<FNN_DT_I4>(ia, rows, ocg, tn, kw, s);
+        if (e != hipSuccess) return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, hipGetErrorString(e));
+    }
+    *handled = true;
+    return FNN_OK;
+}

@@ -113,7 +113,6 @@ __global__ void __launch_bounds__(256) i8_matmul_epilogue_kernel(const int32_t *
 // requested before the first value is used.
 constexpr int CONV_CPB = 4;   // waves per workgroup, each with its own chunks
 
-struct ConvDivs { FastDiv np, wo, khw, kw; };
 
 template <bool X8, bool W4, int NC>   // X8: int8 input; W4: 4-bit weights (16 activation levels unless X8, interleaved operand)
                                       // NC <= 4: a wave's taps are worked out one per lane

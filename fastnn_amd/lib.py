@@ -37,6 +37,7 @@ OPT_CODEBOOK_EXPANDED = 12
 OPT_GEMV_INT8_MAX_M = 13
 OPT_CONV_EPILOGUE = 14
 OPT_CONV_RANGES = 15
+OPT_CONV_IMPLICIT = 16
 
 STATUS_NAMES = {0: "Ok", 1: "Dispatch", 2: "Memory", 3: "UnsupportedOp", 4: "Compilation"}
 

@@ -117,7 +117,10 @@ enum {
     FNN_OPT_CONV_RANGES = 15,     /* plans: 1 (default) = the instruction that writes the input of a quantised Conv2d leaves   */
                                   /* partial (min, max) pairs per image behind and the convolution does not scan its input; 0 = */
                                   /* every convolution scans                                                               */
-    FNN_OPT_COUNT = 16
+    FNN_OPT_CONV_IMPLICIT = 16,   /* quantised Conv2d (I8 / I4 weights, f32 input): 1 = one implicit-GEMM kernel (im2col taps    */
+                                  /* fetched and quantised in the GEMM's operand registers, no int8 operand in memory), 2 = the */
+                                  /* operand kernel + GEMM pair, 0 (default) = by shape                                         */
+    FNN_OPT_COUNT = 17
 };
 int fnn_hip_set_option(fnn_hip_ctx *ctx, int option, int64_t value);
 int fnn_hip_get_option(fnn_hip_ctx *ctx, int option, int64_t *value);

@@ -228,14 +228,16 @@ def test_yolo_graph_node_by_node_against_oracle(orc, batch, size):
         ex.close()
 
 
+@pytest.mark.parametrize("implicit", [0, 1, 2])
 @pytest.mark.parametrize("batch,size", [(3, 160), (1, 224)])
-def test_conv_activation_ranges_from_the_producing_instruction(orc, batch, size):
+def test_conv_activation_ranges_from_the_producing_instruction(orc, batch, size, implicit):
     """A quantised Conv2d in a plan takes min / max of its input from partial pairs the instruction before it left
     (conv epilogue, Split / Concat copies, residual Add, MaxPool, Resize) instead of scanning the tensor.  min and
     max do not depend on how the values are grouped, so every output must equal, bit for bit, what the plan gives
     with every convolution scanning its own input; the sizes make output tiles straddle images (20 x 20 = 400 rows
     per image against 64-row tiles) and fall below one tile (5 x 5), where the producer leaves nothing and the
-    consumer scans."""
+    consumer scans.  implicit: which convolution kernel leaves and takes the pairs (0 = chosen by shape, 1 = the
+    implicit-GEMM kernel wherever it runs, 2 = the operand kernel + GEMM pair everywhere)."""
     rng = np.random.default_rng(11)
     nodes, params, shape, outs = bench.yolo_graph(batch, rng, size=size)
     x = rng.uniform(0, 1, shape).astype(np.float32)
@@ -245,6 +247,7 @@ def test_conv_activation_ranges_from_the_producing_instruction(orc, batch, size)
         ex = AotExecutor(nodes, params, ["x"], outs, {"x": shape}, quantize=8)
         try:
             ex.set_option(flib.OPT_CONV_RANGES, on)
+            ex.set_option(flib.OPT_CONV_IMPLICIT, implicit)
             first = ex.forward({"x": x})
             again = ex.forward({"x": x})
             assert ex.replayed

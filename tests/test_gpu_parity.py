@@ -483,6 +483,44 @@ def test_qconv2d_i8(ctx, orc, cfg, act, wdt, conv_epilogue):
     ctx.release(h)
 
 
+IMPLICIT_CONVS = CONVS + [
+    dict(b=2, c=8, h=40, w=40, oc=24, kh=3, kw=3, stride=1, pad=1, dil=1, groups=1),     # taken by shape; one k slice
+    dict(b=1, c=20, h=30, w=33, oc=40, kh=3, kw=3, stride=2, pad=1, dil=1, groups=1),    # two k slices, odd pixel count
+    dict(b=3, c=64, h=7, w=9, oc=70, kh=3, kw=3, stride=1, pad=1, dil=1, groups=1),      # four k slices, blocks over three images
+    dict(b=2, c=6, h=50, w=46, oc=12, kh=5, kw=5, stride=1, pad=2, dil=1, groups=2),     # groups, K past a step's end
+]
+
+
+@pytest.mark.parametrize("cfg", IMPLICIT_CONVS)
+@pytest.mark.parametrize("act", [0, 3])
+@pytest.mark.parametrize("wdt", [flib.DT_I8, flib.DT_I4])
+@pytest.mark.parametrize("mode", [0, 1])
+def test_qconv2d_implicit_gemm(ctx, orc, cfg, act, wdt, mode):
+    """The kernel that fetches and quantises the im2col taps in the MFMA operand registers (no int8 operand in
+    memory): the same accumulators as conv2d_packed_i8x4 / conv2d_packed_i4x8, bit for bit.  mode 1: wherever it can
+    run; mode 0: where the library picks it by shape (the larger of these cases)."""
+    ctx.set_option(flib.OPT_CONV_IMPLICIT, mode)
+    try:
+        rng = np.random.default_rng(6100 + cfg["c"])
+        kk = cfg["c"] // cfg["groups"] * cfg["kh"] * cfg["kw"]
+        x = rng.uniform(-0.3, 1, (cfg["b"], cfg["c"], cfg["h"], cfg["w"])).astype(np.float32)
+        x[1 % cfg["b"]] *= 3.0   # images with different ranges
+        wt = (rng.standard_normal((cfg["oc"], kk)) * np.sqrt(2.0 / kk)).astype(np.float32)
+        bias = (rng.standard_normal(cfg["oc"]) * 0.05).astype(np.float32)
+        pw = fastnn_amd.quantize_weights(wdt, wt)
+        h = ctx.register(pw)
+        args = (cfg["kh"], cfg["kw"], cfg["stride"], cfg["pad"], cfg["dil"], cfg["groups"])
+        want, want_acc, _, _ = orc.qconv2d_i8(x, to_oracle(orc, pw), *args, bias=bias, act=act, want_acc=True)
+        got, acc = ctx.qconv2d(h, x, cfg["oc"], *args, bias=bias, act=act, want_acc=True)
+        assert np.array_equal(acc, want_acc)
+        assert_close(got, want, 1e-5)
+        got_nb = ctx.qconv2d(h, x, cfg["oc"], *args, act=act)
+        assert_close(got_nb, orc.qconv2d_i8(x, to_oracle(orc, pw), *args, act=act), 1e-5)
+        ctx.release(h)
+    finally:
+        ctx.set_option(flib.OPT_CONV_IMPLICIT, 0)
+
+
 @pytest.mark.parametrize("wdt", [flib.DT_I8, flib.DT_I4])
 def test_qconv2d_constant_and_empty(ctx, orc, wdt):
     x = np.full((1, 2, 4, 4), 0.5, np.float32)
