@@ -68,6 +68,34 @@ __device__ __forceinline__ float conv_dequant(int acc_in, float sa, float za, fl
     return val;
 }
 
+// min / max over nparts (min, max) pairs at part (16-byte aligned) by the nthr threads of a workgroup, folded into
+// this thread's mn / mx: up to eight pairs per thread are requested before the first is used
+__device__ __forceinline__ void conv_fold_partial_ranges(const float *part, int nparts, int tid, int nthr, float &mn, float &mx)
+{
+    const float4 *p4 = reinterpret_cast<const float4 *>(part);
+    const int n4 = nparts >> 1;
+    float4 t[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const int i = tid + k * nthr;
+        t[k] = i < n4 ? p4[i] : make_float4(INFINITY, -INFINITY, INFINITY, -INFINITY);
+    }
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        mn = fminf(mn, fminf(t[k].x, t[k].z));
+        mx = fmaxf(mx, fmaxf(t[k].y, t[k].w));
+    }
+    for (int i = tid + 4 * nthr; i < n4; i += nthr) {
+        const float4 u = p4[i];
+        mn = fminf(mn, fminf(u.x, u.z));
+        mx = fmaxf(mx, fmaxf(u.y, u.w));
+    }
+    if ((nparts & 1) && tid == 0) {
+        mn = fminf(mn, part[(nparts - 1) * 2]);
+        mx = fmaxf(mx, part[(nparts - 1) * 2 + 1]);
+    }
+}
+
 hipError_t launch_quantize_activations(const float *x, int64_t numel, float scale, float zp,
                                        uint8_t *payload, float *scratch_partial, hipStream_t s);
 hipError_t launch_dequantize_activations(const uint8_t *payload, uint64_t payload_len, float *out, uint64_t n, hipStream_t s);

@@ -34,9 +34,14 @@ __global__ void __launch_bounds__(64 * PW * KW) conv_implicit_kernel(ImplicitArg
     __shared__ int r_qs[PW][32];
     __shared__ int64_t r_off[PW][32];
     __shared__ float s_rng[PW][4];
+    __shared__ int s_cnt;
     __shared__ int r_img[PW][32];
 
     const int tid = threadIdx.x, lane = tid & 63;
+    if constexpr (RNG) {
+        if (tid == 0) s_cnt = 0;
+        __syncthreads();
+    }
     const int wv = __builtin_amdgcn_readfirstlane(tid >> 6), pw = wv / KW, kw = wv % KW;
     const int lr = lane & 31, hf = lane >> 5;
     const int g = p.g, kk = p.kk;
@@ -57,13 +62,9 @@ __global__ void __launch_bounds__(64 * PW * KW) conv_implicit_kernel(ImplicitArg
         const int bg_b = (int)p.dv.np.div((uint32_t)r_last) * a.groups + g;
         const int nimg = bg_b != bg_a ? 2 : 1;
         for (int w = 0; w < nimg; w++) {
-            const float2 *part = reinterpret_cast<const float2 *>(a.minmax_partial) + (int64_t)(w ? bg_b : bg_a) * a.part_stride;
+            const float *part = a.minmax_partial + (int64_t)(w ? bg_b : bg_a) * a.part_stride * 2;
             float mn = a.range_zero ? 0.0f : INFINITY, mx = a.range_zero ? 0.0f : -INFINITY;
-            for (int i = tid; i < a.nparts; i += 64 * NW) {
-                const float2 t = part[i];
-                mn = fminf(mn, t.x);
-                mx = fmaxf(mx, t.y);
-            }
+            conv_fold_partial_ranges(part, a.nparts, tid, 64 * NW, mn, mx);
             mn = wave_min(mn);
             mx = wave_max(mx);
             if (lane == 0) { s_mm[w][0][wv] = mn; s_mm[w][1][wv] = mx; }
@@ -263,10 +264,11 @@ __global__ void __launch_bounds__(64 * PW * KW) conv_implicit_kernel(ImplicitArg
     // (block - first block of the image) * column tiles + tile of every image it meets, (np / (32 * PW) + 2) * tiles
     // pairs per image; the block that holds the last pixel of its first image also fills that image's unused pairs
     float mn0 = INFINITY, mx0 = -INFINITY, mn1 = INFINITY, mx1 = -INFINITY;
-    bool rng_two = false;
+    bool rng_two = false, rng_plain = false;
     if constexpr (RNG) {
         const uint32_t row_z = (uint32_t)(r_first + 32 * PW - 1 < rows ? r_first + 32 * PW - 1 : rows - 1);
         rng_two = r_first < rows && row_z > (nn0 + 1) * np - 1;
+        rng_plain = !rng_two && r_first + 32 * PW <= rows;
     }
     if (kw == 0) {
         if (hf == 0) {
@@ -320,11 +322,16 @@ __global__ void __launch_bounds__(64 * PW * KW) conv_implicit_kernel(ImplicitArg
                     v[j] = conv_dequant(ai, rsa[j], rza[j], rs[j], sw[tn], zw[tn], sw[tn] * (float)wq_[tn], bq[j], kk, a.act, &av[j]);
                 }
                 if constexpr (RNG) {
+                    if (rng_plain) {   // (workgroup-uniform) every pixel of the block exists and lies in one image
+                        mn0 = fminf(fminf(mn0, fminf(v[0], v[1])), fminf(v[2], v[3]));
+                        mx0 = fmaxf(fmaxf(mx0, fmaxf(v[0], v[1])), fmaxf(v[2], v[3]));
+                    } else {
 #pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        if (r0 + j >= rows) continue;
-                        if (rng_two && r_img[pw][rr0 + j]) { mn1 = fminf(mn1, v[j]); mx1 = fmaxf(mx1, v[j]); }
-                        else { mn0 = fminf(mn0, v[j]); mx0 = fmaxf(mx0, v[j]); }
+                        for (int j = 0; j < 4; j++) {
+                            if (r0 + j >= rows) continue;
+                            if (rng_two && r_img[pw][rr0 + j]) { mn1 = fminf(mn1, v[j]); mx1 = fmaxf(mx1, v[j]); }
+                            else { mn0 = fminf(mn0, v[j]); mx0 = fmaxf(mx0, v[j]); }
+                        }
                     }
                 }
                 if (p.vec4) {
@@ -345,13 +352,20 @@ __global__ void __launch_bounds__(64 * PW * KW) conv_implicit_kernel(ImplicitArg
     }
     if constexpr (RNG) {
         if (r_first >= rows) return;   // (workgroup-uniform)
-        if (kw == 0) {
-            mn0 = wave_min(mn0); mx0 = wave_max(mx0);
-            if (rng_two) { mn1 = wave_min(mn1); mx1 = wave_max(mx1); }
-            if (lane == 0) { s_rng[pw][0] = mn0; s_rng[pw][1] = mx0; s_rng[pw][2] = mn1; s_rng[pw][3] = mx1; }
+        if (kw != 0) return;
+        // the pixel blocks' waves leave their pairs in LDS and count themselves; the last to arrive combines them (no
+        // barrier: a wave that is done retires)
+        mn0 = wave_min(mn0); mx0 = wave_max(mx0);
+        if (rng_two) { mn1 = wave_min(mn1); mx1 = wave_max(mx1); }
+        int arrived = 0;
+        if (lane == 0) {
+            s_rng[pw][0] = mn0; s_rng[pw][1] = mx0; s_rng[pw][2] = mn1; s_rng[pw][3] = mx1;
+            __threadfence_block();
+            arrived = atomicAdd(&s_cnt, 1);
+            __threadfence_block();
         }
-        __syncthreads();
-        if (tid == 0) {
+        if (lane == 0 && arrived == PW - 1) {
+            mn0 = s_rng[0][0]; mx0 = s_rng[0][1]; mn1 = s_rng[0][2]; mx1 = s_rng[0][3];
 #pragma unroll
             for (int w2 = 1; w2 < PW; w2++) {
                 mn0 = fminf(mn0, s_rng[w2][0]); mx0 = fmaxf(mx0, s_rng[w2][1]);

@@ -146,10 +146,7 @@ __global__ void __launch_bounds__(256) conv_operand_kernel(QConvArgs a, int g, i
         for (int w = 0; w < nimg; w++) {
             const float *part = a.minmax_partial + (int64_t)(w ? bg_b : bg_a) * a.part_stride * 2;
             float mn = a.range_zero ? 0.0f : INFINITY, mx = a.range_zero ? 0.0f : -INFINITY;
-            for (int i = tid; i < a.nparts; i += 256) {
-                mn = fminf(mn, part[i * 2]);
-                mx = fmaxf(mx, part[i * 2 + 1]);
-            }
+            conv_fold_partial_ranges(part, a.nparts, tid, 256, mn, mx);
             mn = wave_min(mn);
             mx = wave_max(mx);
             if (rr == 0) { s_mm[w][0][tid >> 6] = mn; s_mm[w][1][tid >> 6] = mx; }

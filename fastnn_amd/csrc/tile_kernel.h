@@ -198,7 +198,7 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
     // image also fills that image's unused pairs, up to np / BM + 2 per column tile.
     uint32_t rng_img = 0;
     int rng_slot = 0, rng_fill = 0, rng_per_m = 0;
-    bool rng_two = false;
+    bool rng_two = false, rng_plain = false;
     if constexpr (CRNG) {
         constexpr uint32_t BM_ = WGM * TM * 32;
         const uint32_t np = p.cv.np, row_a = (uint32_t)mt * BM_;
@@ -209,6 +209,7 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
         rng_two = row_z > img_end;
         rng_per_m = (int)(np / BM_) + 2;
         rng_fill = row_z >= img_end ? rng_slot + 1 : rng_per_m;
+        rng_plain = !rng_two && row_a + BM_ - 1 <= last;
     }
     // ... and this lane's channel constants (scale, zero, scale * sum q_w, bias)
     float cv_sw[CONV ? TN : 1], cv_zw[CONV ? TN : 1], cv_wt[CONV ? TN : 1], cv_bi[CONV ? TN : 1];
@@ -624,11 +625,16 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
                         v[j] = conv_dequant(a, sa[j], za[j], rs[j], sw[tn], zw[tn], wt[tn], bq[j], p.cv.kk, p.act, &av[j]);
                     }
                     if constexpr (CRNG) {
+                        if (rng_plain) {   // (workgroup-uniform) every row of the tile exists and lies in one image
+                            mn0 = fminf(fminf(mn0, fminf(v[0], v[1])), fminf(v[2], v[3]));
+                            mx0 = fmaxf(fmaxf(mx0, fmaxf(v[0], v[1])), fmaxf(v[2], v[3]));
+                        } else {
 #pragma unroll
-                        for (int j = 0; j < 4; j++) {
-                            if (r0 + j >= p.m) continue;
-                            if (second[j]) { mn1 = fminf(mn1, v[j]); mx1 = fmaxf(mx1, v[j]); }
-                            else { mn0 = fminf(mn0, v[j]); mx0 = fmaxf(mx0, v[j]); }
+                            for (int j = 0; j < 4; j++) {
+                                if (r0 + j >= p.m) continue;
+                                if (second[j]) { mn1 = fminf(mn1, v[j]); mx1 = fmaxf(mx1, v[j]); }
+                                else { mn0 = fminf(mn0, v[j]); mx0 = fmaxf(mx0, v[j]); }
+                            }
                         }
                     }
                     if (p.cv.vec4) {
