@@ -183,6 +183,8 @@ def composite_result(args) -> dict:
             plan.call_kernel(KERNEL_OF[dt], [s_h, s2], s_y, [m, f, d], meta_of(w2))
             plan.call_kernel("add_f32", [s_y, s_x[i]], s_x[i + 1], [m * d])
         be = HipBackend(0)
+        for _, ident, value in parsed_options(args, flib):
+            be.set_option(ident, value)
         be.allocate_arena(top[0])
         be.write_arena(s_x[0][0], rng.standard_normal((m, d)).astype(np.float32))
         for _ in range(1 + warm):
@@ -207,7 +209,8 @@ def composite_result(args) -> dict:
         out = {"metric": f"C4 MLP stack forward ({par}, 4x[2048->8192 GELU, 8192->2048 + residual], 64 tokens)",
                "value": round(flops / (ms * 1e-3) / 1e12, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": steps, "warmup": warm,
                "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
-               "data": "synthetic", "config": {"workload": args.workload, "launch": "plan dispatch (12 instructions, HIP-graph replay) + sync per step"},
+               "data": "synthetic", "config": {"workload": args.workload, "launch": "plan dispatch (12 instructions, HIP-graph replay) + sync per step",
+                          "residual_adds_inside_the_matmul": plan.residuals_fused, "options": {n: v for n, _, v in parsed_options(args, flib)}},
                "weight_gb_per_s": round(wbytes / (ms * 1e-3) / 1e9, 1), "packed_weight_bytes": wbytes,
                "finite_output": bool(np.isfinite(y).all()),
                "f16x1": {"ms_per_step": round(ms1, 4), "tflop_per_s": round(flops / (ms1 * 1e-3) / 1e12, 2),

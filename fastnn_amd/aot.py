@@ -423,6 +423,11 @@ class AotExecutor:
         """Conv instructions of the plan that took their activation ranges from the instruction before them."""
         return 0 if self._plan is None else self._plan.ranges_used
 
+    @property
+    def residuals_fused(self) -> int:
+        """Add instructions of the plan whose sum the MatMul before them stored."""
+        return 0 if self._plan is None else self._plan.residuals_fused
+
     def close(self):
         if self._plan is not None:
             self._plan.close()

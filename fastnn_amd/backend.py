@@ -104,6 +104,11 @@ class ExecutablePlan:
         """Quantised Conv2d instructions that took their activation ranges from the instruction before them."""
         return int(self.lib.fnn_plan_ranges_used(self.handle))
 
+    @property
+    def residuals_fused(self) -> int:
+        """add_f32 instructions whose sum the MatMul before them stored (no launch of their own)."""
+        return int(self.lib.fnn_plan_residuals_fused(self.handle))
+
     def _ok(self, rc, what):
         if rc:
             msg = self.lib.fnn_backend_last_error(None)

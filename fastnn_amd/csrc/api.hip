@@ -59,6 +59,7 @@ struct fnn_hip_ctx {
     unsigned char *static_ws = nullptr;   // this device's copy of the library's static workspace
     bool static_mode = false;             // inside fnn_hip_qmatmul_static: workspaces come from static_ws, nothing allocates
     FnnRangeIo range;                     // value ranges handed from one call to the next (range_io.h)
+    FnnResidualIo residual;               // a residual addition handed to the next MatMul call (range_io.h)
 };
 
 // Workspace of fnn_hip_qmatmul_static, part of the library's device image: every GPU the library runs on holds one
@@ -136,6 +137,7 @@ const OptionSpec kOptions[FNN_OPT_COUNT] = {
     {0, 0, 3},        // FNN_OPT_CONV_EPILOGUE
     {1, 0, 1},        // FNN_OPT_CONV_RANGES
     {0, 0, 2},        // FNN_OPT_CONV_IMPLICIT
+    {1, 0, 1},        // FNN_OPT_FUSE_RESIDUAL
 };
 
 #define HIP_TRY(ctx, code, expr)                                                              \
@@ -1138,3 +1140,4 @@ int fnn_ctx_fail(fnn_hip_ctx *ctx, int code, const char *msg) { return fail(ctx,
 
 int64_t fnn_ctx_option(const fnn_hip_ctx *ctx, int option) { return ctx->options[option]; }
 FnnRangeIo *fnn_ctx_range_io(fnn_hip_ctx *ctx) { return &ctx->range; }
+FnnResidualIo *fnn_ctx_residual_io(fnn_hip_ctx *ctx) { return &ctx->residual; }

@@ -58,6 +58,8 @@ struct Instr {
     uint64_t node_id = 0;
     Meta meta;
     bool clobbered = false;  // WriteConst only: another instruction of the plan writes into dst
+    int add_operand = -1;    // MatMul whose output the next instruction (an add_f32) adds to a tensor: index (0 / 1) of that
+                             // tensor among the Add's inputs, found by analyse(); -1: nothing to fuse
 };
 
 bool overlaps(const fnn_slice &a, const fnn_slice &b)
@@ -124,6 +126,8 @@ struct fnn_plan {
     bool segment_resident = false;    // residency as the first segment of the pass in progress found it
     bool last_replayed = false;
     uint64_t ranges_used = 0;         // convolutions of the last host-side pass that took their ranges from a table
+    size_t add_done = (size_t)-1;     // index of an Add whose sum the MatMul before it has already stored
+    uint64_t residuals_fused = 0;     // such Adds in the last host-side pass
 };
 
 struct fnn_backend {
@@ -788,6 +792,33 @@ void analyse(fnn_plan *p)
             p->writes.push_back(r);
         }
     }
+    // MatMul followed by an Add of its whole output and another tensor of the same size: candidates for one call.
+    // Not when a quantised Conv2d reads the sum (the Add then leaves that convolution's activation ranges) and not
+    // when the sum overlaps the MatMul's own output or partly overlaps the other operand.
+    for (size_t i = 0; i + 1 < p->instrs.size(); i++) {
+        Instr &mm = p->instrs[i];
+        const Instr &ad = p->instrs[i + 1];
+        mm.add_operand = -1;
+        if (mm.kind != K_CALL || ad.kind != K_CALL || ad.kernel != "add_f32" || ad.inputs.size() != 2) continue;
+        const KernelName kn = split_activation(mm.kernel);
+        if (matmul_dtype(kn.base) < 0 || mm.has_param_dims || mm.params.size() < 3) continue;
+        const uint64_t bytes = mm.params[0] * mm.params[2] * 4;
+        if (bytes == 0 || mm.dst.size != bytes || ad.dst.size != bytes) continue;
+        int other = -1;
+        for (int k = 0; k < 2; k++)
+            if (ad.inputs[k].offset == mm.dst.offset && ad.inputs[k].size == bytes && ad.inputs[1 - k].size == bytes) other = 1 - k;
+        if (other < 0) continue;
+        const fnn_slice &res = ad.inputs[other];
+        if (overlaps(res, mm.dst) || overlaps(ad.dst, mm.dst)) continue;
+        if (overlaps(ad.dst, res) && ad.dst.offset != res.offset) continue;
+        if (ad.dst.offset % 4 || res.offset % 4) continue;
+        bool feeds_conv = false;
+        for (size_t j = i + 2; j < p->instrs.size() && !feeds_conv; j++) {
+            ConvInput cj;
+            feeds_conv = ranged_conv_input(p->instrs[j], &cj) && overlaps(p->instrs[j].inputs[0], ad.dst);
+        }
+        if (!feeds_conv) mm.add_operand = other;
+    }
     p->analysed = true;
 }
 
@@ -809,6 +840,12 @@ void note_dispatched(fnn_backend *b, fnn_plan *p)
 int run_instr(fnn_backend *b, fnn_plan *p, size_t idx, bool consts_resident)
 {
     Instr &in = p->instrs[idx];
+    if (idx == p->add_done) {   // the MatMul before this Add has stored the sum already
+        p->add_done = (size_t)-1;
+        drop_ranges_overlapping(b, in.dst);
+        return FNN_OK;
+    }
+    p->add_done = (size_t)-1;
     if (in.kind != K_CALL) drop_ranges_overlapping(b, in.kind == K_WRITE_CONST ? fnn_slice{in.dst.offset, in.data.size()} : in.dst);
     switch (in.kind) {
     case K_WRITE_CONST: {
@@ -845,8 +882,28 @@ int run_instr(fnn_backend *b, fnn_plan *p, size_t idx, bool consts_resident)
         *rio = FnnRangeIo{};
         return lift(b, fnn_hip_copy(b->ctx, b->arena + d.offset, b->arena + s.offset, n));
     }
-    case K_CALL:
-        return run_call_with_ranges(b, p, idx);
+    case K_CALL: {
+        int64_t fuse = 1;
+        fnn_hip_get_option(b->ctx, FNN_OPT_FUSE_RESIDUAL, &fuse);
+        if (in.add_operand < 0 || !fuse || idx + 1 >= p->instrs.size()) return run_call_with_ranges(b, p, idx);
+        // the Add behind this MatMul rides along: the MatMul's last kernel stores the sum too where it can
+        const Instr &ad = p->instrs[idx + 1];
+        const fnn_slice &other = ad.inputs[in.add_operand];
+        if (!in_arena(b, other) || !in_arena(b, ad.dst)) return run_call_with_ranges(b, p, idx);   // (the Add reports it)
+        FnnResidualIo *res = fnn_ctx_residual_io(b->ctx);
+        *res = FnnResidualIo{};
+        res->residual = (const float *)(b->arena + other.offset);
+        res->sum_out = (float *)(b->arena + ad.dst.offset);
+        res->of_out = (const float *)(b->arena + in.dst.offset);
+        res->elems = in.dst.size / 4;
+        const int st = run_call_with_ranges(b, p, idx);
+        if (st == FNN_OK && res->used) {
+            p->add_done = idx + 1;
+            p->residuals_fused++;
+        }
+        *res = FnnResidualIo{};
+        return st;
+    }
     }
     return FNN_OK;
 }
@@ -893,6 +950,8 @@ int dispatch_impl(fnn_backend *b, fnn_plan *p, uint64_t *elapsed_ns, uint64_t n_
             int st = FNN_OK;
             b->live_ranges.clear();
             p->ranges_used = 0;
+            p->residuals_fused = 0;
+            p->add_done = (size_t)-1;
             for (size_t i = 0; i < p->instrs.size() && st == FNN_OK; i++) st = run_instr(b, p, i, true);
             b->live_ranges.clear();
             fnn_hip_graph *g = nullptr;
@@ -921,7 +980,8 @@ int dispatch_impl(fnn_backend *b, fnn_plan *p, uint64_t *elapsed_ns, uint64_t n_
     }
 
     b->live_ranges.clear();   // ranges never outlive a pass: between passes anyone may write into the arena
-    if (first == 0) p->ranges_used = 0;
+    if (first == 0) { p->ranges_used = 0; p->residuals_fused = 0; }
+    p->add_done = (size_t)-1;
     for (size_t i = (size_t)first; i < p->instrs.size(); i++) {
         auto t0 = std::chrono::steady_clock::now();
         int st = run_instr(b, p, i, resident);
@@ -1100,6 +1160,7 @@ uint64_t fnn_plan_len(const fnn_plan *p) { return p ? p->instrs.size() : 0; }
 int fnn_plan_replayed(const fnn_plan *p) { return p && p->last_replayed ? 1 : 0; }
 
 uint64_t fnn_plan_ranges_used(const fnn_plan *p) { return p ? p->ranges_used : 0; }
+uint64_t fnn_plan_residuals_fused(const fnn_plan *p) { return p ? p->residuals_fused : 0; }
 
 static void touched(fnn_plan *p)
 {

@@ -20,6 +20,7 @@
 // depending on the weights' signs and zeros).
 #include "mfma.h"
 #include "dech.h"
+#include "range_io.h"
 
 #include <type_traits>
 
@@ -269,6 +270,10 @@ int run_digits(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const Q
     t.ap = reinterpret_cast<const _Float16 *>(d.planes);
     t.rexp = d.rexp; t.xsum = d.xsum;
     t.out = q.out; t.part = (float *)ws1;
+    if (FnnResidualIo *res = fnn_ctx_residual_io(ctx); splits > 1 && res->residual && res->of_out == q.out && res->elems == (uint64_t)(M * N)) {
+        t.residual = res->residual; t.sum_out = res->sum_out;
+        res->used = 1;
+    }
     t.m = M; t.n = N; t.kp = q.kp; t.kpad = kpad; t.rows_pad = rows_pad;
     t.act = q.act; t.splits = splits; t.iters = iters; t.ips = ips; t.mtiles = mtiles; t.ntiles = ntiles;
     // ring depth: a stage is requested NS - 2 stages before it is consumed, and what is in flight has to cover the

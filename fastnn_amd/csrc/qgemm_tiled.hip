@@ -26,6 +26,7 @@
 // on rows with a non-zero mean lane value: dot -= mean_k(u[n,k]) * sum_k (hi - x').
 #include "mfma.h"
 #include "dech.h"
+#include "range_io.h"
 
 #include <cstdlib>
 #include <type_traits>
@@ -339,6 +340,11 @@ int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QM
     t.scales = q.scales; t.zeros = q.zeros; t.umean = want_umean ? wm->umean : nullptr; t.bias = q.bias;
     t.ap = pa.ap; t.rexp = pa.rexp; t.xsum = pa.xsum; t.esum = pa.esum;
     t.out = q.out; t.part = (float *)ws1;
+    t.residual = nullptr; t.sum_out = nullptr;
+    if (FnnResidualIo *res = fnn_ctx_residual_io(ctx); splits > 1 && res->residual && res->of_out == q.out && res->elems == (uint64_t)(M * N)) {
+        t.residual = res->residual; t.sum_out = res->sum_out;
+        res->used = 1;
+    }
     t.m = M; t.n = N; t.kp = q.kp; t.kpad = kpad; t.rows_pad = rows_pad;
     t.a_wrap = 0;
     t.bscales = nullptr; t.codebook = nullptr; t.bpr = 0;

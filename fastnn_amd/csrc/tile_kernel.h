@@ -13,6 +13,8 @@ struct TileArgs {
     const int *rexp;
     const float *xsum, *esum;
     float *out, *part;
+    const float *residual;        // split-K reduction only: non-null = sum_out[m,n] = out[m,n] + residual[m,n] as well
+    float *sum_out;
     int32_t *c_i32;               // int8 mode: raw accumulators [m][ldc]
     int64_t ldc;
     int64_t m, n, kp, kpad, rows_pad;
@@ -787,6 +789,8 @@ __global__ void __launch_bounds__(256) splitk_epilogue_kernel(TileArgs p, int si
         if (comp) d = d - um * ldexpf(p.esum[m], -p.rexp[m]);
         float o = d * sc + zr * p.xsum[m];
         if (p.bias) o = o + bs;
-        p.out[idx] = fnn_activation(o, p.act);
+        o = fnn_activation(o, p.act);
+        p.out[idx] = o;
+        if (p.residual) p.sum_out[idx] = o + p.residual[idx];
     }
 }

@@ -136,6 +136,9 @@ int fnn_plan_replayed(const fnn_plan *p);
  * ranges the instruction before them left instead of scanning their input (FNN_OPT_CONV_RANGES; no counterpart in
  * fastnn: lets tests and tools see which path ran). */
 uint64_t fnn_plan_ranges_used(const fnn_plan *p);
+/* add_f32 instructions of the plan that, on its last pass (or in its recorded graph), did not run as a launch of
+ * their own because the MatMul before them stored the sum (FNN_OPT_FUSE_RESIDUAL; no counterpart in fastnn). */
+uint64_t fnn_plan_residuals_fused(const fnn_plan *p);
 /* Backend::dispatch_profile, src/backend/mod.rs:178-211: elapsed_ns[i] per instruction */
 int fnn_backend_dispatch_profile(fnn_backend *b, fnn_plan *p, uint64_t *elapsed_ns, uint64_t n);
 

@@ -841,3 +841,55 @@ def test_memcopy_and_fill_feeding_a_convolution(be, orc, batch):
     want2 = orc.qconv2d_i8(np.full_like(x, 0.25), to_oracle(orc, pw), k, k, 1, 1, 1, 1, bias=bias, act=flib.ACT_SILU)
     assert_close(be.read_arena(*s_y, np.float32).reshape(want2.shape), want2, 1e-5, "copy -> fill -> conv")
     assert plan2.ranges_used == 0
+
+
+@pytest.mark.parametrize("wdt,kname", [(flib.DT_F8, "matmul_f8"), (flib.DT_I4, "matmul_i4_relu"), (flib.DT_I4CB, "matmul_i4")])
+def test_matmul_followed_by_residual_add_runs_as_one_call(be, orc, wdt, kname):
+    """A MatMul whose output the next instruction adds to another tensor stores the sum from its own last kernel
+    (FNN_OPT_FUSE_RESIDUAL, the Add is skipped): every arrangement of the Add's operands gives, bit for bit, what
+    the two instructions give on their own, the MatMul's own output is still written, and the arrangements that
+    cannot ride along (the sum overwriting the MatMul's output, a convolution reading the sum) still run the Add."""
+    rng = np.random.default_rng(97 + wdt)
+    m, k, n = 64, 1024, 384
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    r = rng.standard_normal((m, n)).astype(np.float32)
+    pw = fastnn_amd.quantize_weights(wdt, _w(rng, n, k))
+    cw = fastnn_amd.quantize_weights(flib.DT_I8, _w(rng, 8, 6))
+    act = flib.ACT_RELU if kname.endswith("relu") else 0
+    want_y = orc.qmatmul(to_oracle(orc, pw), x, act=act)
+    a = Arena()
+    s_x, s_r, s_w, s_cw = a.take(x.nbytes), a.take(r.nbytes), a.take(pw.words.nbytes), a.take(cw.words.nbytes)
+    s_y = [a.take(m * n * 4) for _ in range(5)]
+    s_sum = [a.take(m * n * 4) for _ in range(5)]
+    s_r2, s_conv = a.take(r.nbytes), a.take(m * 8 * 8 * 8 * 4)
+    plan = ExecutablePlan(a.top).write_const(s_w[0], pw.words).write_const(s_cw[0], cw.words)
+    mm = lambda dst: plan.call_kernel(kname, [s_x, s_w], dst, [m, k, n], meta_of(pw))
+    mm(s_y[0]); plan.call_kernel("add_f32", [s_y[0], s_r], s_sum[0], [m * n])        # MatMul output first
+    mm(s_y[1]); plan.call_kernel("add_f32", [s_r, s_y[1]], s_sum[1], [m * n])        # ... second
+    plan.memcopy(s_r2, s_r)
+    mm(s_y[2]); plan.call_kernel("add_f32", [s_y[2], s_r2], s_r2, [m * n])           # the sum replaces the other operand
+    mm(s_y[3]); plan.call_kernel("add_f32", [s_y[3], s_r], s_y[3], [m * n])          # ... replaces the MatMul output: not fused
+    mm(s_y[4]); plan.call_kernel("add_f32", [s_y[4], s_r], s_sum[4], [m * n])        # a convolution reads the sum: not fused
+    plan.call_kernel("conv2d_i8", [s_sum[4], s_cw], s_conv, [1, 0, 1, 1, 6, 8, 8, 1, 1], meta_of(cw, shape=[8, 6, 1, 1]))
+    be.allocate_arena(a.top)
+    be.write_arena(s_x[0], x)
+    be.write_arena(s_r[0], r)
+    got = {}
+    try:
+        for fuse in (1, 0):
+            be.set_option(flib.OPT_FUSE_RESIDUAL, fuse)
+            be.dispatch(plan)
+            first = be.read_arena(0, a.top).copy()
+            be.dispatch(plan)
+            assert plan.replayed
+            got[fuse] = be.read_arena(0, a.top).copy()
+            assert np.array_equal(first, got[fuse]), "replay differs from the first dispatch"
+            assert plan.residuals_fused == (3 if fuse else 0)
+    finally:
+        be.set_option(flib.OPT_FUSE_RESIDUAL, 1)
+    assert np.array_equal(got[1], got[0])
+    view = lambda s: got[1][s[0]:s[0] + s[1]].view(np.float32).reshape(m, n)
+    for i in (0, 1, 2, 4):
+        assert_close(view(s_y[i]), want_y, 2e-5, f"MatMul output {i}")
+    for s in (s_sum[0], s_sum[1], s_r2, s_y[3], s_sum[4]):
+        assert np.array_equal(view(s), view(s_y[0]) + r)
