@@ -352,6 +352,7 @@ class Probe:
         self.lib.fnn_probe_mfma.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p]
         self.lib.fnn_probe_lds_delivery.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p,
                                                     C.POINTER(C.c_double)]
+        self.lib.fnn_probe_gemv_pattern.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_int, C.c_void_p]
         self.ctx = ctx
         self.stream = ctx.stream()
         self.sink = ctx.alloc(256)
@@ -376,6 +377,20 @@ class Probe:
             out[f"{loads}x16B/lane,{'all' if wgs == 0 else wgs}wg"] = round(self.ctx.timer_stop() / n * 1e3, 3)
         return out
 
+
+    def gemv_pattern(self, ptrs, rows, row_bytes, row_tiles=3):
+        """The int8 GEMV kernel's read pattern over rows x row_bytes packed bytes and nothing else (16 rows x 64
+        bytes per wave-load, a wave per 256-byte column segment, `row_tiles` * 16 rows per workgroup): microseconds."""
+        for p in ptrs:
+            self.lib.fnn_probe_gemv_pattern(self.stream, p, rows, row_bytes, row_tiles, self.sink.ptr)
+        self.ctx.sync()
+        n = max(len(ptrs) * 4, 64)
+        self.ctx.timer_start()
+        for i in range(n):
+            rc = self.lib.fnn_probe_gemv_pattern(self.stream, ptrs[i % len(ptrs)], rows, row_bytes, row_tiles, self.sink.ptr)
+            if rc:
+                raise RuntimeError(f"fnn_probe_gemv_pattern failed: hipError {rc}")
+        return round(self.ctx.timer_stop() / n * 1e3, 3)
 
     def lds_delivery(self, iters=400):
         """Bytes per microsecond that loops of `global_load_lds_dwordx4` stages deliver into the LDS, by waves per
@@ -713,6 +728,9 @@ def main() -> int:
                                       "frac_of_this_ceiling": round(ceil_us[best_cfg] / (kernel_ms * 1e3), 3),
                                       "note": "best plain read of the same packed bytes per launch over a ring of buffers of "
                                               "the same size, eager launches, events on the same stream"}
+    if bandwidth_bound and wbytes % n == 0 and (wbytes // n) % 2048 == 0:
+        # the same bytes read in the GEMV kernel's own order (16 rows x 64 bytes per wave-load) and nothing else
+        roofline["device_stream_read"]["gemv_pattern_us"] = {f"{rt}x16 rows/wg": probe.gemv_pattern(src_ptrs, n, wbytes // n, rt) for rt in (1, 2, 3)}
     # counter-derived HBM bytes per launch, recorded under profiles/ for the measured configurations
     tj = args.traffic_json or os.path.join(ROOT, "profiles", f"traffic_{args.workload}_m{m}.json")
     if os.path.exists(tj):

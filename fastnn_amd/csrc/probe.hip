@@ -28,6 +28,35 @@ __global__ void __launch_bounds__(256) probe_read_kernel(const uint4 *__restrict
     if (acc == 0x9e3779b9u) sink[0] = acc;  // practically never true: keeps the loads alive
 }
 
+// The read pattern of the int8 GEMV kernel and nothing else: a workgroup of 8 waves owns RT * 16 consecutive rows
+// of row_bytes bytes; wave w owns the byte columns [w * seg, (w + 1) * seg) of them (seg = 256: a slice of 512 4-bit
+// values); lane (row ln = lane & 15, group g = lane >> 4) requests bytes [l * 64 + g * 16, +16) of its segment in
+// every row tile, l = 0 .. seg / 64 - 1: RT * seg / 64 loads of 16 bytes per lane, each wave-load 16 rows x 64 bytes.
+template <int RT>
+__global__ void __launch_bounds__(512) probe_gemv_pattern_kernel(const unsigned char *__restrict__ src, size_t rows, size_t row_bytes,
+                                                                 uint32_t *sink)
+{
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, ln = lane & 15, g = lane >> 4;
+    const size_t n0 = (size_t)blockIdx.x * (16 * RT);
+    uint32_t acc = 0;
+    for (size_t seg0 = (size_t)wv * 256; seg0 < row_bytes; seg0 += 8 * 256) {
+        uint4 v[RT][4];
+#pragma unroll
+        for (int r = 0; r < RT; r++)
+#pragma unroll
+            for (int l = 0; l < 4; l++) {
+                size_t row = n0 + r * 16 + ln;
+                if (row >= rows) row = rows - 1;
+                v[r][l] = *reinterpret_cast<const uint4 *>(src + row * row_bytes + seg0 + l * 64 + g * 16);
+            }
+#pragma unroll
+        for (int r = 0; r < RT; r++)
+#pragma unroll
+            for (int l = 0; l < 4; l++) acc += v[r][l].x ^ v[r][l].y ^ v[r][l].z ^ v[r][l].w;
+    }
+    if (acc == 0x9e3779b9u) sink[0] = acc;
+}
+
 template <int U>
 __global__ void __launch_bounds__(256) probe_copy_kernel(const uint4 *__restrict__ src, uint4 *__restrict__ dst, size_t n16)
 {
@@ -185,6 +214,22 @@ extern "C" int fnn_probe_stream(void *stream, const void *src_dev, void *dst_dev
     case 4: return (int)launch<4>(src_dev, dst_dev, n16, (unsigned)grid, sink, s);
     default: return (int)launch<8>(src_dev, dst_dev, n16, (unsigned)grid, sink, s);
     }
+}
+
+// One launch on `stream` that reads rows x row_bytes bytes (row_bytes a multiple of 2048) in the int8 GEMV kernel's
+// order: workgroups of 8 waves over row_tiles * 16 rows (row_tiles 1, 2 or 3).  Returns 0 or the hipError_t value.
+extern "C" int fnn_probe_gemv_pattern(void *stream, const void *src_dev, size_t rows, size_t row_bytes, int row_tiles, void *sink_dev)
+{
+    if (!src_dev || !sink_dev || rows < 1 || row_bytes < 2048 || row_bytes % 2048 || row_tiles < 1 || row_tiles > 3) return (int)hipErrorInvalidValue;
+    if (reinterpret_cast<uintptr_t>(src_dev) & 15) return (int)hipErrorInvalidValue;
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    uint32_t *sink = reinterpret_cast<uint32_t *>(sink_dev);
+    const unsigned char *src = reinterpret_cast<const unsigned char *>(src_dev);
+    const dim3 grid((unsigned)((rows + 16 * row_tiles - 1) / (16 * row_tiles)));
+    if (row_tiles == 1) hipLaunchKernelGGL(probe_gemv_pattern_kernel<1>, grid, dim3(512), 0, s, src, rows, row_bytes, sink);
+    else if (row_tiles == 2) hipLaunchKernelGGL(probe_gemv_pattern_kernel<2>, grid, dim3(512), 0, s, src, rows, row_bytes, sink);
+    else hipLaunchKernelGGL(probe_gemv_pattern_kernel<3>, grid, dim3(512), 0, s, src, rows, row_bytes, sink);
+    return (int)hipGetLastError();
 }
 
 // One launch on `stream` of a kernel that only issues matrix-core instructions: kind 0 = v_mfma_f32_32x32x16_f16
