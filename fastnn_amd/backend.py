@@ -109,6 +109,11 @@ class ExecutablePlan:
         """add_f32 instructions whose sum the MatMul before them stored (no launch of their own)."""
         return int(self.lib.fnn_plan_residuals_fused(self.handle))
 
+    @property
+    def operands_handed(self) -> int:
+        """MatMul instructions whose activation operand the MatMul before them prepared."""
+        return int(self.lib.fnn_plan_operands_handed(self.handle))
+
     def _ok(self, rc, what):
         if rc:
             msg = self.lib.fnn_backend_last_error(None)

@@ -51,7 +51,7 @@ struct fnn_hip_ctx {
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     char err[1024] = {0};      // fixed storage: recording a failure never allocates
     std::unordered_map<uint64_t, fnn_hip_weight *> weights;
-    Staging st_a, st_out, st_bias, st_acc, st_tmp, st_tmp2, st_tmp3, st_col, st_rows;
+    Staging st_a, st_out, st_bias, st_acc, st_tmp, st_tmp2, st_tmp3, st_tmp4, st_col, st_rows;
     int64_t options[FNN_OPT_COUNT];
     float *scratch = nullptr;  // small reduction scratch (partials)
     bool capturing = false;
@@ -60,6 +60,8 @@ struct fnn_hip_ctx {
     bool static_mode = false;             // inside fnn_hip_qmatmul_static: workspaces come from static_ws, nothing allocates
     FnnRangeIo range;                     // value ranges handed from one call to the next (range_io.h)
     FnnResidualIo residual;               // a residual addition handed to the next MatMul call (range_io.h)
+    FnnPrepIo prep;                       // a prepared operand handed from one MatMul call to the next (range_io.h)
+    FnnPreparedOperand prepared;
 };
 
 // Workspace of fnn_hip_qmatmul_static, part of the library's device image: every GPU the library runs on holds one
@@ -138,6 +140,7 @@ const OptionSpec kOptions[FNN_OPT_COUNT] = {
     {1, 0, 1},        // FNN_OPT_CONV_RANGES
     {0, 0, 2},        // FNN_OPT_CONV_IMPLICIT
     {1, 0, 1},        // FNN_OPT_FUSE_RESIDUAL
+    {1, 0, 1},        // FNN_OPT_FUSE_PREP
 };
 
 #define HIP_TRY(ctx, code, expr)                                                              \
@@ -252,7 +255,7 @@ void fnn_hip_destroy(fnn_hip_ctx *ctx)
     (void)hipSetDevice(ctx->device);
     if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
     for (auto &kv : ctx->weights) free_weight(kv.second);
-    for (Staging *s : {&ctx->st_a, &ctx->st_out, &ctx->st_bias, &ctx->st_acc, &ctx->st_tmp, &ctx->st_tmp2, &ctx->st_tmp3, &ctx->st_col, &ctx->st_rows})
+    for (Staging *s : {&ctx->st_a, &ctx->st_out, &ctx->st_bias, &ctx->st_acc, &ctx->st_tmp, &ctx->st_tmp2, &ctx->st_tmp3, &ctx->st_tmp4, &ctx->st_col, &ctx->st_rows})
         if (s->ptr) (void)hipFree(s->ptr);
     if (ctx->scratch) (void)hipFree(ctx->scratch);
     if (ctx->ev0) (void)hipEventDestroy(ctx->ev0);
@@ -1125,7 +1128,7 @@ int fnn_ctx_ensure_tmp(fnn_hip_ctx *ctx, int which, size_t bytes, void **ptr)
         *ptr = ctx->static_ws + off;
         return FNN_OK;
     }
-    Staging &s = which == 0 ? ctx->st_tmp : (which == 1 ? ctx->st_tmp2 : ctx->st_tmp3);
+    Staging &s = which == 0 ? ctx->st_tmp : (which == 1 ? ctx->st_tmp2 : (which == 2 ? ctx->st_tmp3 : ctx->st_tmp4));
     int rc = ensure(ctx, s, bytes);
     if (rc) return rc;
     *ptr = s.ptr;
@@ -1141,3 +1144,6 @@ int fnn_ctx_fail(fnn_hip_ctx *ctx, int code, const char *msg) { return fail(ctx,
 int64_t fnn_ctx_option(const fnn_hip_ctx *ctx, int option) { return ctx->options[option]; }
 FnnRangeIo *fnn_ctx_range_io(fnn_hip_ctx *ctx) { return &ctx->range; }
 FnnResidualIo *fnn_ctx_residual_io(fnn_hip_ctx *ctx) { return &ctx->residual; }
+FnnPrepIo *fnn_ctx_prep_io(fnn_hip_ctx *ctx) { return &ctx->prep; }
+FnnPreparedOperand *fnn_ctx_prepared(fnn_hip_ctx *ctx) { return &ctx->prepared; }
+bool fnn_ctx_static_mode(fnn_hip_ctx *ctx) { return ctx->static_mode; }

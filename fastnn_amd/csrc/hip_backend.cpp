@@ -128,6 +128,8 @@ struct fnn_plan {
     uint64_t ranges_used = 0;         // convolutions of the last host-side pass that took their ranges from a table
     size_t add_done = (size_t)-1;     // index of an Add whose sum the MatMul before it has already stored
     uint64_t residuals_fused = 0;     // such Adds in the last host-side pass
+    size_t prep_ready = (size_t)-1;   // index of a MatMul whose operand the call before it has prepared
+    uint64_t operands_handed = 0;     // such MatMuls in the last host-side pass
 };
 
 struct fnn_backend {
@@ -846,6 +848,8 @@ int run_instr(fnn_backend *b, fnn_plan *p, size_t idx, bool consts_resident)
         return FNN_OK;
     }
     p->add_done = (size_t)-1;
+    const bool offered_here = p->prep_ready == idx;   // the call before this one prepared this MatMul's operand
+    p->prep_ready = (size_t)-1;
     if (in.kind != K_CALL) drop_ranges_overlapping(b, in.kind == K_WRITE_CONST ? fnn_slice{in.dst.offset, in.data.size()} : in.dst);
     switch (in.kind) {
     case K_WRITE_CONST: {
@@ -883,25 +887,62 @@ int run_instr(fnn_backend *b, fnn_plan *p, size_t idx, bool consts_resident)
         return lift(b, fnn_hip_copy(b->ctx, b->arena + d.offset, b->arena + s.offset, n));
     }
     case K_CALL: {
-        int64_t fuse = 1;
+        int64_t fuse = 1, hand = 1;
         fnn_hip_get_option(b->ctx, FNN_OPT_FUSE_RESIDUAL, &fuse);
-        if (in.add_operand < 0 || !fuse || idx + 1 >= p->instrs.size()) return run_call_with_ranges(b, p, idx);
+        fnn_hip_get_option(b->ctx, FNN_OPT_FUSE_PREP, &hand);
         // the Add behind this MatMul rides along: the MatMul's last kernel stores the sum too where it can
-        const Instr &ad = p->instrs[idx + 1];
-        const fnn_slice &other = ad.inputs[in.add_operand];
-        if (!in_arena(b, other) || !in_arena(b, ad.dst)) return run_call_with_ranges(b, p, idx);   // (the Add reports it)
+        bool with_res = in.add_operand >= 0 && fuse && idx + 1 < p->instrs.size();
+        if (with_res) {
+            const Instr &ad = p->instrs[idx + 1];
+            with_res = in_arena(b, ad.inputs[in.add_operand]) && in_arena(b, ad.dst);   // (else the Add reports it)
+        }
         FnnResidualIo *res = fnn_ctx_residual_io(b->ctx);
         *res = FnnResidualIo{};
-        res->residual = (const float *)(b->arena + other.offset);
-        res->sum_out = (float *)(b->arena + ad.dst.offset);
-        res->of_out = (const float *)(b->arena + in.dst.offset);
-        res->elems = in.dst.size / 4;
+        if (with_res) {
+            const Instr &ad = p->instrs[idx + 1];
+            res->residual = (const float *)(b->arena + ad.inputs[in.add_operand].offset);
+            res->sum_out = (float *)(b->arena + ad.dst.offset);
+            res->of_out = (const float *)(b->arena + in.dst.offset);
+            res->elems = in.dst.size / 4;
+        }
+        // ... and when the next call on the context is the MatMul that reads this one's result (or that sum), this
+        // call's reduction prepares its operand
+        FnnPrepIo *pio = fnn_ctx_prep_io(b->ctx);
+        *pio = FnnPrepIo{};
+        size_t consumer = (size_t)-1;
+        const KernelName kn = split_activation(in.kernel);
+        const bool plain_matmul = matmul_dtype(kn.base) >= 0 && !in.has_param_dims && in.params.size() >= 3 && in.meta.codebook.empty();
+        if (hand && plain_matmul) {
+            pio->offered = offered_here ? 1 : 0;
+            const size_t j = idx + (with_res ? 2 : 1);
+            const uint64_t m = in.params[0], n = in.params[2];
+            const fnn_slice &feeds = with_res ? p->instrs[idx + 1].dst : in.dst;
+            if (j < p->instrs.size() && in.dst.size == m * n * 4) {
+                const Instr &nx = p->instrs[j];
+                const KernelName kx = nx.kind == K_CALL ? split_activation(nx.kernel) : KernelName{};
+                const int dx = nx.kind == K_CALL ? matmul_dtype(kx.base) : -1;
+                if (dx >= 0 && !nx.has_param_dims && nx.params.size() >= 3 && nx.inputs.size() >= 2 && nx.meta.codebook.empty() &&
+                    nx.params[0] == m && nx.params[1] == n && nx.inputs[0].offset == feeds.offset && nx.inputs[0].size == m * n * 4 &&
+                    in_arena(b, nx.inputs[0]) && in_arena(b, nx.inputs[1])) {
+                    fnn_hip_weight *wn = nullptr;
+                    if (weight_for(b, nx.inputs[1], dx, nx.meta, nx.params[2], nx.params[1], nx.kernel.c_str(), &wn) == FNN_OK && wn) {
+                        pio->next_w = wn;
+                        pio->next_flags = FNN_FLAG_DEVICE_PTRS | b->kernel_flags;
+                        pio->next_a = (const float *)(b->arena + feeds.offset);
+                        consumer = j;
+                    }
+                }
+            }
+        }
         const int st = run_call_with_ranges(b, p, idx);
         if (st == FNN_OK && res->used) {
             p->add_done = idx + 1;
             p->residuals_fused++;
         }
+        if (st == FNN_OK && pio->consumed) p->operands_handed++;
+        if (st == FNN_OK && pio->produced && consumer != (size_t)-1 && (consumer == idx + 1 || p->add_done == idx + 1)) p->prep_ready = consumer;
         *res = FnnResidualIo{};
+        *pio = FnnPrepIo{};
         return st;
     }
     }
@@ -951,7 +992,9 @@ int dispatch_impl(fnn_backend *b, fnn_plan *p, uint64_t *elapsed_ns, uint64_t n_
             b->live_ranges.clear();
             p->ranges_used = 0;
             p->residuals_fused = 0;
+            p->operands_handed = 0;
             p->add_done = (size_t)-1;
+            p->prep_ready = (size_t)-1;
             for (size_t i = 0; i < p->instrs.size() && st == FNN_OK; i++) st = run_instr(b, p, i, true);
             b->live_ranges.clear();
             fnn_hip_graph *g = nullptr;
@@ -980,8 +1023,9 @@ int dispatch_impl(fnn_backend *b, fnn_plan *p, uint64_t *elapsed_ns, uint64_t n_
     }
 
     b->live_ranges.clear();   // ranges never outlive a pass: between passes anyone may write into the arena
-    if (first == 0) { p->ranges_used = 0; p->residuals_fused = 0; }
+    if (first == 0) { p->ranges_used = 0; p->residuals_fused = 0; p->operands_handed = 0; }
     p->add_done = (size_t)-1;
+    p->prep_ready = (size_t)-1;
     for (size_t i = (size_t)first; i < p->instrs.size(); i++) {
         auto t0 = std::chrono::steady_clock::now();
         int st = run_instr(b, p, i, resident);
@@ -1161,6 +1205,7 @@ int fnn_plan_replayed(const fnn_plan *p) { return p && p->last_replayed ? 1 : 0;
 
 uint64_t fnn_plan_ranges_used(const fnn_plan *p) { return p ? p->ranges_used : 0; }
 uint64_t fnn_plan_residuals_fused(const fnn_plan *p) { return p ? p->residuals_fused : 0; }
+uint64_t fnn_plan_operands_handed(const fnn_plan *p) { return p ? p->operands_handed : 0; }
 
 static void touched(fnn_plan *p)
 {

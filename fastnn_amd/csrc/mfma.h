@@ -11,6 +11,7 @@ int fnn_ctx_fail(fnn_hip_ctx *ctx, int code, const char *msg);
 bool fnn_ctx_capturing(fnn_hip_ctx *ctx);
 // true while device memory must not be allocated: graph capture, or a call through fnn_hip_qmatmul_static
 bool fnn_ctx_no_alloc(fnn_hip_ctx *ctx);
+bool fnn_ctx_static_mode(fnn_hip_ctx *ctx);
 // value of a per-context option (FNN_OPT_*, set through fnn_hip_set_option)
 int64_t fnn_ctx_option(const fnn_hip_ctx *ctx, int option);
 

@@ -69,36 +69,108 @@ __device__ __host__ inline int64_t eff_row(int64_t m, int precise, int lo)
     return (m / 16) * 32 + lo * 16 + m % 16;
 }
 
+constexpr int PREP_RG = 4;   // 8-value groups of a row a thread can keep in registers: rows of up to 8192 values
+
+// Statistics and conversion of activation row m held in registers: thread tid has the groups tid + 256 r (8 values
+// each, zeros past the row) in keep[r]; writes the hi (+ lo) operand rows, the row's exponent, sum and rounding sum.
+// Called by all 256 threads of a workgroup; red: shared scratch.
+__device__ __forceinline__ void prep_row_from_regs(const PrepArgs &p, int64_t m, const float4 (&keep)[PREP_RG][2], float (&red)[3][4])
+{
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const int64_t ngroups = p.kpad / 8;
+    _Float16 *hi_row = p.ap + eff_row(m, p.precise, 0) * 64;
+    _Float16 *lo_row = p.precise ? p.ap + eff_row(m, 1, 1) * 64 : nullptr;
+    const int64_t kb_stride = p.rows_pad * 64;
+    auto group_at = [&](_Float16 *row, int64_t g) { return row + (g >> 3) * kb_stride + (g & 7) * 8; };
+    float mx = 0.0f, sum = 0.0f;
+#pragma unroll
+    for (int r = 0; r < PREP_RG; r++)
+#pragma unroll
+        for (int q = 0; q < 2; q++) {
+            const float4 v = keep[r][q];
+            mx = fmaxf(mx, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+            sum += (v.x + v.y) + (v.z + v.w);
+        }
+    mx = wave_max(mx);
+    sum = wave_sum(sum);
+    if (lane == 0) { red[0][wv] = mx; red[1][wv] = sum; }
+    __syncthreads();
+    mx = fmaxf(fmaxf(red[0][0], red[0][1]), fmaxf(red[0][2], red[0][3]));
+    sum = (red[1][0] + red[1][1]) + (red[1][2] + red[1][3]);
+    int e = 0;
+    if (mx > 0.0f && mx < __builtin_huge_valf()) {
+        int ex;
+        (void)frexpf(mx, &ex);  // mx = f * 2^ex, f in [0.5, 1)
+        e = 15 - ex;            // mx * 2^e in [2^14, 2^15)
+    }
+    float err = 0.0f;
+#pragma unroll
+    for (int r = 0; r < PREP_RG; r++) {
+        const int64_t g = tid + 256 * r;
+        if (g < ngroups) {
+            const float v[8] = {keep[r][0].x, keep[r][0].y, keep[r][0].z, keep[r][0].w,
+                                keep[r][1].x, keep[r][1].y, keep[r][1].z, keep[r][1].w};
+            f16x8 h, l;
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                // operand slot j holds k = 0,4,1,5,2,6,3,7 for the nibble decoders
+                const int src = p.interleaved ? ((j & 1) * 4 + (j >> 1)) : j;
+                const float xs = ldexpf(v[src], e);
+                const _Float16 hh = (_Float16)xs;
+                h[j] = hh;
+                const float rr = xs - (float)hh;
+                l[j] = (_Float16)(rr * LO_UP);
+                err -= rr;
+            }
+            *reinterpret_cast<f16x8 *>(group_at(hi_row, g)) = h;
+            if (lo_row) *reinterpret_cast<f16x8 *>(group_at(lo_row, g)) = l;
+        }
+    }
+    err = wave_sum(err);
+    if (lane == 0) red[2][wv] = err;
+    __syncthreads();
+    if (tid == 0) {
+        p.rexp[m] = e;
+        p.xsum[m] = sum;
+        p.esum[m] = (red[2][0] + red[2][1]) + (red[2][2] + red[2][3]);
+    }
+}
+
+// zero operands for a padding row of the last tile
+__device__ __forceinline__ void prep_zero_row(const PrepArgs &p, int64_t m)
+{
+    const int tid = threadIdx.x;
+    const int64_t ngroups = p.kpad / 8;
+    _Float16 *hi_row = p.ap + eff_row(m, p.precise, 0) * 64;
+    _Float16 *lo_row = p.precise ? p.ap + eff_row(m, 1, 1) * 64 : nullptr;
+    const int64_t kb_stride = p.rows_pad * 64;
+    auto group_at = [&](_Float16 *row, int64_t g) { return row + (g >> 3) * kb_stride + (g & 7) * 8; };
+    const uint4 z = make_uint4(0, 0, 0, 0);
+    for (int64_t g = tid; g < ngroups; g += 256) {
+        *reinterpret_cast<uint4 *>(group_at(hi_row, g)) = z;
+        if (lo_row) *reinterpret_cast<uint4 *>(group_at(lo_row, g)) = z;
+    }
+    if (tid == 0) { p.rexp[m] = 0; p.xsum[m] = 0.0f; p.esum[m] = 0.0f; }
+}
+
 __global__ void __launch_bounds__(256) act_prep_kernel(PrepArgs p)
 {
     __shared__ float red[3][4];
     const int64_t m = blockIdx.x;
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const int64_t K = p.k, ngroups = p.kpad / 8;
-    // 16-byte group g of a row: k block g/8, position g%8 inside the block's 128-byte row
-    _Float16 *hi_row = p.ap + eff_row(m, p.precise, 0) * 64;
-    _Float16 *lo_row = p.precise ? p.ap + eff_row(m, 1, 1) * 64 : nullptr;
-    const int64_t kb_stride = p.rows_pad * 64;
-    auto group_at = [&](_Float16 *row, int64_t g) { return row + (g >> 3) * kb_stride + (g & 7) * 8; };
     if (m >= p.m) {  // padding rows of the last tile: zero operands
-        const uint4 z = make_uint4(0, 0, 0, 0);
-        for (int64_t g = tid; g < ngroups; g += 256) {
-            *reinterpret_cast<uint4 *>(group_at(hi_row, g)) = z;
-            if (lo_row) *reinterpret_cast<uint4 *>(group_at(lo_row, g)) = z;
-        }
-        if (tid == 0) { p.rexp[m] = 0; p.xsum[m] = 0.0f; p.esum[m] = 0.0f; }
+        prep_zero_row(p, m);
         return;
     }
     const float *x = p.a + m * K;
     const bool vec = (K % 8 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0);
-    constexpr int RG = 4;                       // 8-value groups a thread can keep in registers
-    const bool in_regs = vec && ngroups <= 256 * RG && p.kpad == K;
-    float4 keep[RG][2];
-    float mx = 0.0f, sum = 0.0f;
+    const bool in_regs = vec && ngroups <= 256 * PREP_RG && p.kpad == K;
     if (in_regs) {
         // one trip to memory: the row stays in registers between the statistics and the conversion
+        float4 keep[PREP_RG][2];
 #pragma unroll
-        for (int r = 0; r < RG; r++) {
+        for (int r = 0; r < PREP_RG; r++) {
             const int64_t g = tid + 256 * r;
             keep[r][0] = keep[r][1] = make_float4(0.f, 0.f, 0.f, 0.f);
             if (g < ngroups) {
@@ -106,15 +178,16 @@ __global__ void __launch_bounds__(256) act_prep_kernel(PrepArgs p)
                 keep[r][1] = *reinterpret_cast<const float4 *>(x + g * 8 + 4);
             }
         }
-#pragma unroll
-        for (int r = 0; r < RG; r++)
-#pragma unroll
-            for (int q = 0; q < 2; q++) {
-                const float4 v = keep[r][q];
-                mx = fmaxf(mx, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
-                sum += (v.x + v.y) + (v.z + v.w);
-            }
-    } else if (vec) {
+        prep_row_from_regs(p, m, keep, red);
+        return;
+    }
+    // 16-byte group g of a row: k block g/8, position g%8 inside the block's 128-byte row
+    _Float16 *hi_row = p.ap + eff_row(m, p.precise, 0) * 64;
+    _Float16 *lo_row = p.precise ? p.ap + eff_row(m, 1, 1) * 64 : nullptr;
+    const int64_t kb_stride = p.rows_pad * 64;
+    auto group_at = [&](_Float16 *row, int64_t g) { return row + (g >> 3) * kb_stride + (g & 7) * 8; };
+    float mx = 0.0f, sum = 0.0f;
+    if (vec) {
         for (int64_t i = tid; i < K / 4; i += 256) {
             const float4 v = reinterpret_cast<const float4 *>(x)[i];
             mx = fmaxf(mx, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
@@ -155,31 +228,19 @@ __global__ void __launch_bounds__(256) act_prep_kernel(PrepArgs p)
         *reinterpret_cast<f16x8 *>(group_at(hi_row, g)) = h;
         if (lo_row) *reinterpret_cast<f16x8 *>(group_at(lo_row, g)) = l;
     };
-    if (in_regs) {
+    for (int64_t g = tid; g < ngroups; g += 256) {
+        float v[8];
+        const int64_t k0 = g * 8;
+        if (vec && k0 + 8 <= K) {
+            const float4 a0 = *reinterpret_cast<const float4 *>(x + k0);
+            const float4 a1 = *reinterpret_cast<const float4 *>(x + k0 + 4);
+            v[0] = a0.x; v[1] = a0.y; v[2] = a0.z; v[3] = a0.w;
+            v[4] = a1.x; v[5] = a1.y; v[6] = a1.z; v[7] = a1.w;
+        } else {
 #pragma unroll
-        for (int r = 0; r < RG; r++) {
-            const int64_t g = tid + 256 * r;
-            if (g < ngroups) {
-                const float v[8] = {keep[r][0].x, keep[r][0].y, keep[r][0].z, keep[r][0].w,
-                                    keep[r][1].x, keep[r][1].y, keep[r][1].z, keep[r][1].w};
-                convert(g, v);
-            }
+            for (int j = 0; j < 8; j++) v[j] = (k0 + j < K) ? x[k0 + j] : 0.0f;
         }
-    } else {
-        for (int64_t g = tid; g < ngroups; g += 256) {
-            float v[8];
-            const int64_t k0 = g * 8;
-            if (vec && k0 + 8 <= K) {
-                const float4 a0 = *reinterpret_cast<const float4 *>(x + k0);
-                const float4 a1 = *reinterpret_cast<const float4 *>(x + k0 + 4);
-                v[0] = a0.x; v[1] = a0.y; v[2] = a0.z; v[3] = a0.w;
-                v[4] = a1.x; v[5] = a1.y; v[6] = a1.z; v[7] = a1.w;
-            } else {
-#pragma unroll
-                for (int j = 0; j < 8; j++) v[j] = (k0 + j < K) ? x[k0 + j] : 0.0f;
-            }
-            convert(g, v);
-        }
+        convert(g, v);
     }
     err = wave_sum(err);
     if (lane == 0) red[2][wv] = err;
@@ -212,6 +273,157 @@ __global__ void __launch_bounds__(64) row_umean_kernel(const uint32_t *words, in
 
 #include "tile_kernel.h"
 
+// Split-K reduction that also prepares the operand of the MatMul reading this one's result (a plan's next layer):
+// workgroup m owns output row m whole.  Thread (r, tid) of its RW * 256 threads owns the columns 8 * (tid + 256 r),
+// the group that thread tid of act_prep_kernel holds in keep[r]: it adds the partial tiles in split order and applies
+// the epilogue exactly as splitk_epilogue_kernel does, stores its eight values (and their sums with a residual), and
+// converts what the next MatMul reads, `use_sum` ? the sums : the values, as prep_row_from_regs would: the row
+// maximum is order-free, and the row sum and the rounding sum are formed by the threads r == 0 from the other
+// threads' terms in the order of act_prep_kernel's loops, so every word left behind equals what act_prep_kernel
+// writes for the same row.  n % 64 == 0, n <= 2048 * RW, no codebook scales; rows m >= p.m are the padding rows of
+// the next operand.
+template <int RW>
+__global__ void __launch_bounds__(256 * RW) splitk_prep_epilogue_kernel(TileArgs p, PrepArgs next, int single, int use_sum)
+{
+    constexpr int NWV = 4 * RW;
+    __shared__ float red_mx[NWV];
+    __shared__ float red[3][4];
+    __shared__ float s_sum[RW][2][256];
+    __shared__ float s_rr[RW][8][256];
+    const int64_t m = blockIdx.x;
+    const int t = threadIdx.x, tid = t & 255, r = t >> 8, lane = t & 63, wv = t >> 6;
+    const int64_t ngroups = p.n / 8;
+    _Float16 *hi_row = next.ap + eff_row(m, next.precise, 0) * 64;
+    _Float16 *lo_row = next.precise ? next.ap + eff_row(m, 1, 1) * 64 : nullptr;
+    const int64_t kb_stride = next.rows_pad * 64;
+    auto group_at = [&](_Float16 *row, int64_t g) { return row + (g >> 3) * kb_stride + (g & 7) * 8; };
+    if (m >= p.m) {
+        const uint4 z = make_uint4(0, 0, 0, 0);
+        for (int64_t g = t; g < ngroups; g += 256 * RW) {
+            *reinterpret_cast<uint4 *>(group_at(hi_row, g)) = z;
+            if (lo_row) *reinterpret_cast<uint4 *>(group_at(lo_row, g)) = z;
+        }
+        if (t == 0) { next.rexp[m] = 0; next.xsum[m] = 0.0f; next.esum[m] = 0.0f; }
+        return;
+    }
+    const int64_t total = p.m * p.n;
+    const bool comp = single && p.umean;
+    const int64_t g = tid + 256 * r;
+    const bool mine = g < ngroups;
+    float x[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};   // what the next MatMul reads in these columns
+    if (mine) {
+        const int64_t n0 = g * 8, idx = m * p.n + n0;
+        const float xs = p.xsum[m];
+        const float cterm = comp ? ldexpf(p.esum[m], -p.rexp[m]) : 0.0f;
+        float d[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        const float *pp = p.part + idx;
+        int zz = 0;
+        for (; zz + 4 <= p.splits; zz += 4) {
+            float4 v[4][2];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                v[u][0] = *reinterpret_cast<const float4 *>(pp + (int64_t)(zz + u) * total);
+                v[u][1] = *reinterpret_cast<const float4 *>(pp + (int64_t)(zz + u) * total + 4);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                d[0] += v[u][0].x; d[1] += v[u][0].y; d[2] += v[u][0].z; d[3] += v[u][0].w;
+                d[4] += v[u][1].x; d[5] += v[u][1].y; d[6] += v[u][1].z; d[7] += v[u][1].w;
+            }
+        }
+        for (; zz < p.splits; zz++) {
+            const float4 v0 = *reinterpret_cast<const float4 *>(pp + (int64_t)zz * total);
+            const float4 v1 = *reinterpret_cast<const float4 *>(pp + (int64_t)zz * total + 4);
+            d[0] += v0.x; d[1] += v0.y; d[2] += v0.z; d[3] += v0.w;
+            d[4] += v1.x; d[5] += v1.y; d[6] += v1.z; d[7] += v1.w;
+        }
+        float sc[8], zr[8];
+#pragma unroll
+        for (int q = 0; q < 2; q++) {
+            const float4 a = *reinterpret_cast<const float4 *>(p.scales + n0 + 4 * q);
+            const float4 b = *reinterpret_cast<const float4 *>(p.zeros + n0 + 4 * q);
+            sc[4 * q] = a.x; sc[4 * q + 1] = a.y; sc[4 * q + 2] = a.z; sc[4 * q + 3] = a.w;
+            zr[4 * q] = b.x; zr[4 * q + 1] = b.y; zr[4 * q + 2] = b.z; zr[4 * q + 3] = b.w;
+        }
+        float o[8], sm[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            float dj = d[j];
+            if (comp) dj = dj - p.umean[n0 + j] * cterm;
+            float v = dj * sc[j] + zr[j] * xs;
+            if (p.bias) v = v + p.bias[n0 + j];
+            o[j] = fnn_activation(v, p.act);
+            sm[j] = p.residual ? o[j] + p.residual[idx + j] : o[j];
+        }
+        *reinterpret_cast<float4 *>(p.out + idx) = make_float4(o[0], o[1], o[2], o[3]);
+        *reinterpret_cast<float4 *>(p.out + idx + 4) = make_float4(o[4], o[5], o[6], o[7]);
+        if (p.residual) {
+            *reinterpret_cast<float4 *>(p.sum_out + idx) = make_float4(sm[0], sm[1], sm[2], sm[3]);
+            *reinterpret_cast<float4 *>(p.sum_out + idx + 4) = make_float4(sm[4], sm[5], sm[6], sm[7]);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++) x[j] = use_sum ? sm[j] : o[j];
+    }
+    // ---- row statistics in act_prep_kernel's order
+    float mx = fmaxf(fmaxf(fmaxf(fabsf(x[0]), fabsf(x[1])), fmaxf(fabsf(x[2]), fabsf(x[3]))),
+                     fmaxf(fmaxf(fabsf(x[4]), fabsf(x[5])), fmaxf(fabsf(x[6]), fabsf(x[7]))));
+    mx = wave_max(mx);
+    if (lane == 0) red_mx[wv] = mx;
+    s_sum[r][0][tid] = (x[0] + x[1]) + (x[2] + x[3]);
+    s_sum[r][1][tid] = (x[4] + x[5]) + (x[6] + x[7]);
+    __syncthreads();
+    mx = red_mx[0];
+#pragma unroll
+    for (int w2 = 1; w2 < NWV; w2++) mx = fmaxf(mx, red_mx[w2]);
+    if (r == 0) {
+        float sum = 0.0f;
+#pragma unroll
+        for (int r2 = 0; r2 < RW; r2++) { sum += s_sum[r2][0][tid]; sum += s_sum[r2][1][tid]; }
+        sum = wave_sum(sum);
+        if (lane == 0) red[1][wv] = sum;
+    }
+    int e = 0;
+    if (mx > 0.0f && mx < __builtin_huge_valf()) {
+        int ex;
+        (void)frexpf(mx, &ex);
+        e = 15 - ex;
+    }
+    if (mine) {
+        f16x8 h, l;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int src = next.interleaved ? ((j & 1) * 4 + (j >> 1)) : j;
+            const float xs2 = ldexpf(x[src], e);
+            const _Float16 hh = (_Float16)xs2;
+            h[j] = hh;
+            const float rr = xs2 - (float)hh;
+            l[j] = (_Float16)(rr * LO_UP);
+            s_rr[r][j][tid] = rr;
+        }
+        *reinterpret_cast<f16x8 *>(group_at(hi_row, g)) = h;
+        if (lo_row) *reinterpret_cast<f16x8 *>(group_at(lo_row, g)) = l;
+    }
+    __syncthreads();
+    if (r == 0) {
+        float err = 0.0f;
+#pragma unroll
+        for (int r2 = 0; r2 < RW; r2++) {
+            if (tid + 256 * r2 < ngroups) {
+#pragma unroll
+                for (int j = 0; j < 8; j++) err -= s_rr[r2][j][tid];
+            }
+        }
+        err = wave_sum(err);
+        if (lane == 0) red[2][wv] = err;
+    }
+    __syncthreads();
+    if (t == 0) {
+        next.rexp[m] = e;
+        next.xsum[m] = (red[1][0] + red[1][1]) + (red[1][2] + red[1][3]);
+        next.esum[m] = (red[2][0] + red[2][1]) + (red[2][2] + red[2][3]);
+    }
+}
+
 template <int DT, int WGM, int WGN, int TM, int TN, bool PRECISE, int NS>
 hipError_t launch_tile(const TileArgs &p, hipStream_t s)
 {
@@ -240,12 +452,19 @@ struct DenseOperand {
     const float *row_scale, *row_zero;
 };
 
+// Shape of the prepared activation operand and of the tiles for an [M, K] x [N, K]^T product
+struct TileLayout {
+    bool precise;
+    int cfg, bm, mtiles, ntiles;
+    int64_t kpad, meff, rows_pad, m_pad;
+    size_t ap_bytes, meta_off, ws_bytes;
+};
+
 template <int DT>
-int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &q, int flags,
-              const DenseOperand *dense = nullptr)
+TileLayout tile_layout(fnn_hip_ctx *ctx, int64_t M, int64_t N, int64_t K, int flags, bool dense)
 {
+    TileLayout L;
     const bool precise = !(flags & FNN_FLAG_ACT_F16_SINGLE);
-    const int64_t M = q.m, N = q.n, K = q.k;
     const int64_t kpad = (K + BK - 1) / BK * BK;
     const int64_t meff = precise ? (M + 15) / 16 * 32 : (M + 31) / 32 * 32;
     // tile shape by effective row count
@@ -268,12 +487,41 @@ int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QM
     // three dependent launches (activation preparation, tiles, split-K reduction), not by delivery.
     if (opt_cfg >= 0 && opt_cfg <= 3) cfg = (int)opt_cfg;
     if (cfg == 3 && (DecH<DT>::WPS < 2 || dense)) cfg = 0;  // (8-bit weights only: a stage of 4-bit rows has too few 16-byte chunks for 8 waves)
-    const int bm = cfg == 3 ? 256 : (cfg == 0 ? 128 : (cfg == 1 ? 64 : 32));
-    const int bn = 128;
-    const int mtiles = (int)((meff + bm - 1) / bm);
-    const int ntiles = (int)((N + bn - 1) / bn);
-    const int64_t rows_pad = (int64_t)mtiles * bm;
-    const int64_t m_pad = precise ? rows_pad / 2 : rows_pad;
+    L.precise = precise; L.cfg = cfg;
+    L.bm = cfg == 3 ? 256 : (cfg == 0 ? 128 : (cfg == 1 ? 64 : 32));
+    L.mtiles = (int)((meff + L.bm - 1) / L.bm);
+    L.ntiles = (int)((N + 127) / 128);
+    L.kpad = kpad; L.meff = meff;
+    L.rows_pad = (int64_t)L.mtiles * L.bm;
+    L.m_pad = precise ? L.rows_pad / 2 : L.rows_pad;
+    L.ap_bytes = (size_t)L.rows_pad * kpad * 2;
+    L.meta_off = (L.ap_bytes + 255) / 256 * 256;
+    L.ws_bytes = L.meta_off + (size_t)L.m_pad * 12 + 256;
+    return L;
+}
+
+// the same for a weight whose type is known at run time; false: that type does not run through run_tiled's packed form
+bool tile_layout_of(fnn_hip_ctx *ctx, int dtype, int64_t M, int64_t N, int64_t K, int flags, TileLayout *L, int *interleaved)
+{
+    switch (dtype) {
+    case FNN_DT_U8: *L = tile_layout<FNN_DT_U8>(ctx, M, N, K, flags, false); *interleaved = DecH<FNN_DT_U8>::INTERLEAVED; return true;
+    case FNN_DT_F8: *L = tile_layout<FNN_DT_F8>(ctx, M, N, K, flags, false); *interleaved = DecH<FNN_DT_F8>::INTERLEAVED; return true;
+    case FNN_DT_F8R: *L = tile_layout<FNN_DT_F8R>(ctx, M, N, K, flags, false); *interleaved = DecH<FNN_DT_F8R>::INTERLEAVED; return true;
+    case FNN_DT_F4: *L = tile_layout<FNN_DT_F4>(ctx, M, N, K, flags, false); *interleaved = DecH<FNN_DT_F4>::INTERLEAVED; return true;
+    default: return false;
+    }
+}
+
+template <int DT>
+int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &q, int flags,
+              const DenseOperand *dense = nullptr)
+{
+    const int64_t M = q.m, N = q.n, K = q.k;
+    const TileLayout L = tile_layout<DT>(ctx, M, N, K, flags, dense != nullptr);
+    const bool precise = L.precise;
+    const int cfg = L.cfg;
+    const int64_t kpad = L.kpad, rows_pad = L.rows_pad, m_pad = L.m_pad;
+    const int mtiles = L.mtiles, ntiles = L.ntiles;
     const int passes = dense ? 2 : 1;
     const int iters = (int)(kpad / BK) * passes;
     // Split K over workgroups when the tiles alone do not fill the 256 CUs.  The factor minimises a
@@ -303,13 +551,21 @@ int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QM
     int ips = (iters + splits - 1) / splits;
     splits = (iters + ips - 1) / ips;   // no empty split
 
-    // workspace: operands + row tables; partial tiles
-    const size_t ap_bytes = (size_t)rows_pad * kpad * 2;
-    const size_t meta_off = (ap_bytes + 255) / 256 * 256;
-    void *ws0 = nullptr, *ws1 = nullptr;
+    // workspace: operands + row tables; partial tiles.  The operand may be in place already: the MatMul call before
+    // this one can have prepared it (FnnPrepIo), in which case nothing may touch that buffer before the tiles run.
+    const size_t meta_off = L.meta_off;
+    FnnPrepIo *pio = fnn_ctx_prep_io(ctx);
+    FnnPreparedOperand *have = fnn_ctx_prepared(ctx);
+    constexpr int kInterleaved = DecH<DT>::INTERLEAVED ? 1 : 0;
+    const bool handed = pio->offered && !dense && have->buffer && have->a == q.a && have->m == M && have->k == K && have->kpad == kpad &&
+                        have->rows_pad == rows_pad && have->precise == (precise ? 1 : 0) && have->interleaved == kInterleaved;
+    const int own_slot = handed ? have->slot : 0;
+    void *ws0 = handed ? have->buffer : nullptr, *ws1 = nullptr;
     int rc;
-    if ((rc = fnn_ctx_ensure_tmp(ctx, 0, meta_off + (size_t)m_pad * 12 + 256, &ws0))) return rc;
+    if (!handed && (rc = fnn_ctx_ensure_tmp(ctx, 0, L.ws_bytes, &ws0))) return rc;
     if (splits > 1 && (rc = fnn_ctx_ensure_tmp(ctx, 1, (size_t)splits * M * N * 4, &ws1))) return rc;
+    *have = FnnPreparedOperand{};   // (whatever was there is used by this call or stale)
+    pio->consumed = handed ? 1 : 0;
 
     fnn_hip_weight *wm = const_cast<fnn_hip_weight *>(w);
     const bool want_umean = !precise && !dense && (DT == FNN_DT_I8 || DT == FNN_DT_I4 || DT == FNN_DT_U8 || DT == FNN_DT_U4 || DT == FNN_DT_F4);
@@ -330,9 +586,12 @@ int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QM
     pa.m = M; pa.k = K; pa.kpad = kpad; pa.rows_pad = rows_pad;
     pa.precise = precise ? 1 : 0;
     pa.interleaved = DecH<DT>::INTERLEAVED ? 1 : 0;
-    hipLaunchKernelGGL(act_prep_kernel, dim3((unsigned)m_pad), dim3(256), 0, s, pa);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, hipGetErrorString(e));
+    hipError_t e = hipSuccess;
+    if (!handed) {
+        hipLaunchKernelGGL(act_prep_kernel, dim3((unsigned)m_pad), dim3(256), 0, s, pa);
+        e = hipGetLastError();
+        if (e != hipSuccess) return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, hipGetErrorString(e));
+    }
 
     TileArgs t;
     t.words = q.words;
@@ -378,6 +637,39 @@ int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QM
     }
     if (e != hipSuccess) return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, hipGetErrorString(e));
     if (splits > 1) {
+        // The reduction can leave the prepared operand of the MatMul that reads this result (a request in FnnPrepIo):
+        // whole rows per workgroup, in the other operand buffer than the one this call's own row tables live in.
+        TileLayout NL;
+        int n_il = 0;
+        const bool may_prepare = pio->next_w && !dense && !t.codebook && !fnn_ctx_static_mode(ctx) && M >= 17 && N % 64 == 0 && N <= 2048 * PREP_RG &&
+                                 (pio->next_a == q.out || (t.residual && pio->next_a == t.sum_out)) &&
+                                 pio->next_w->inner == N && tile_layout_of(ctx, pio->next_w->dtype, M, pio->next_w->rows, N, pio->next_flags, &NL, &n_il) &&
+                                 NL.kpad == N && !((reinterpret_cast<uintptr_t>(t.scales) | reinterpret_cast<uintptr_t>(t.zeros) | reinterpret_cast<uintptr_t>(t.out) |
+                                                    reinterpret_cast<uintptr_t>(t.sum_out) | reinterpret_cast<uintptr_t>(t.part)) & 15);
+        void *nb = nullptr;
+        const int next_slot = own_slot == 0 ? 3 : 0;
+        if (may_prepare && fnn_ctx_ensure_tmp(ctx, next_slot, NL.ws_bytes, &nb) == FNN_OK && nb) {
+            PrepArgs np;
+            np.a = nullptr;
+            np.ap = (_Float16 *)nb;
+            np.rexp = (int *)((char *)nb + NL.meta_off);
+            np.xsum = (float *)(np.rexp + NL.m_pad);
+            np.esum = np.xsum + NL.m_pad;
+            np.m = M; np.k = N; np.kpad = NL.kpad; np.rows_pad = NL.rows_pad;
+            np.precise = NL.precise ? 1 : 0;
+            np.interleaved = n_il;
+            const int use_sum = pio->next_a == q.out ? 0 : 1;
+            if (N > 4096) hipLaunchKernelGGL(splitk_prep_epilogue_kernel<4>, dim3((unsigned)NL.m_pad), dim3(1024), 0, s, t, np, precise ? 0 : 1, use_sum);
+            else if (N > 2048) hipLaunchKernelGGL(splitk_prep_epilogue_kernel<2>, dim3((unsigned)NL.m_pad), dim3(512), 0, s, t, np, precise ? 0 : 1, use_sum);
+            else hipLaunchKernelGGL(splitk_prep_epilogue_kernel<1>, dim3((unsigned)NL.m_pad), dim3(256), 0, s, t, np, precise ? 0 : 1, use_sum);
+            e = hipGetLastError();
+            if (e != hipSuccess) return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, hipGetErrorString(e));
+            have->a = pio->next_a; have->buffer = nb; have->slot = next_slot;
+            have->m = M; have->k = N; have->kpad = NL.kpad; have->rows_pad = NL.rows_pad;
+            have->precise = np.precise; have->interleaved = n_il;
+            pio->produced = 1;
+            return FNN_OK;
+        }
         const int64_t colb = (N + 255) / 256;
         int64_t rowb = (2048 + colb - 1) / colb;   // about 2048 workgroups
         if (rowb > M) rowb = M;

@@ -41,3 +41,31 @@ struct FnnResidualIo {
     int used = 0;
 };
 FnnResidualIo *fnn_ctx_residual_io(fnn_hip_ctx *ctx);
+
+// A prepared MatMul operand that travels from one MatMul call to the next: at 17 <= M the f16 matrix-core path
+// first turns its f32 activations into scaled f16 hi + lo operand rows (a launch of its own).  When the caller knows
+// that the next call on the context is the MatMul reading this one's result, the split-K reduction of this call can
+// leave that operand behind (it has the whole result row in registers), and the next call skips its preparation.
+// The conversion code is the same, so results are identical.
+struct fnn_hip_weight;
+struct FnnPrepIo {
+    // request to the next MatMul call: also prepare the operand of a MatMul with weight next_w and flags next_flags
+    // that reads next_a (this call's output, or the sum it stores for a residual)
+    const fnn_hip_weight *next_w = nullptr;
+    int next_flags = 0;
+    const float *next_a = nullptr;
+    int produced = 0;        // answer: done
+    // offer to the next MatMul call: no call has touched the context since the one that produced its operand
+    int offered = 0;
+    int consumed = 0;        // answer: the call used it
+};
+FnnPrepIo *fnn_ctx_prep_io(fnn_hip_ctx *ctx);
+// what a producing call left behind (library-private record, checked field by field by the consuming call)
+struct FnnPreparedOperand {
+    const float *a = nullptr;       // the f32 tensor the operand was made from
+    void *buffer = nullptr;         // operand rows + row tables
+    int slot = -1;                  // workspace slot of buffer
+    long long m = 0, k = 0, kpad = 0, rows_pad = 0;
+    int precise = 0, interleaved = 0;
+};
+FnnPreparedOperand *fnn_ctx_prepared(fnn_hip_ctx *ctx);

@@ -39,6 +39,7 @@ OPT_CONV_EPILOGUE = 14
 OPT_CONV_RANGES = 15
 OPT_CONV_IMPLICIT = 16
 OPT_FUSE_RESIDUAL = 17
+OPT_FUSE_PREP = 18
 
 STATUS_NAMES = {0: "Ok", 1: "Dispatch", 2: "Memory", 3: "UnsupportedOp", 4: "Compilation"}
 
@@ -59,7 +60,7 @@ BACKEND_SYMBOLS = [
     "fnn_backend_set_kernel_flags", "fnn_backend_set_graph_replay", "fnn_backend_set_option",
     "fnn_backend_allocate_arena", "fnn_backend_write_arena", "fnn_backend_read_arena",
     "fnn_plan_create", "fnn_plan_destroy", "fnn_plan_add_write_const", "fnn_plan_add_fill",
-    "fnn_plan_add_memcopy", "fnn_plan_add_call_kernel", "fnn_plan_len", "fnn_plan_replayed", "fnn_plan_ranges_used", "fnn_plan_residuals_fused", "fnn_plan_arena_size",
+    "fnn_plan_add_memcopy", "fnn_plan_add_call_kernel", "fnn_plan_len", "fnn_plan_replayed", "fnn_plan_ranges_used", "fnn_plan_residuals_fused", "fnn_plan_operands_handed", "fnn_plan_arena_size",
     "fnn_plan_set_param_dims", "fnn_plan_from_bincode", "fnn_plan_to_bincode", "fnn_plan_describe",
     "fnn_backend_dispatch", "fnn_backend_dispatch_env", "fnn_backend_dispatch_from", "fnn_backend_dispatch_profile",
     "fnn_hip_elementwise", "fnn_hip_fill_f32", "fnn_hip_copy",
@@ -192,6 +193,8 @@ def _prototype(l):
     l.fnn_plan_ranges_used.restype = C.c_uint64
     l.fnn_plan_residuals_fused.argtypes = [_vp]
     l.fnn_plan_residuals_fused.restype = C.c_uint64
+    l.fnn_plan_operands_handed.argtypes = [_vp]
+    l.fnn_plan_operands_handed.restype = C.c_uint64
     l.fnn_backend_dispatch.argtypes = [_vp, _vp]
     l.fnn_backend_dispatch_env.argtypes = [_vp, _vp, C.POINTER(C.c_char_p), C.POINTER(_u64), _u64]
     l.fnn_backend_dispatch_from.argtypes = [_vp, _vp, C.POINTER(C.c_char_p), C.POINTER(_u64), _u64, _u64, C.POINTER(_u64)]

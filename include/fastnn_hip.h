@@ -123,7 +123,10 @@ enum {
     FNN_OPT_FUSE_RESIDUAL = 17,   /* plans: 1 (default) = a MatMul whose output the next instruction adds to another tensor       */
                                   /* stores that sum from its own last kernel where it can (the Add instruction is then skipped; */
                                   /* same f32 addition, identical results), 0 = every Add runs as its own launch                 */
-    FNN_OPT_COUNT = 18
+    FNN_OPT_FUSE_PREP = 18,       /* plans: 1 (default) = a MatMul at 17 <= M whose result the next instruction multiplies (f16    */
+                                  /* matrix-core weight types) leaves that MatMul's prepared activation operand behind, which  */
+                                  /* then skips its own preparation launch (same conversion code, identical results); 0 = off  */
+    FNN_OPT_COUNT = 19
 };
 int fnn_hip_set_option(fnn_hip_ctx *ctx, int option, int64_t value);
 int fnn_hip_get_option(fnn_hip_ctx *ctx, int option, int64_t *value);

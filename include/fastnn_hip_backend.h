@@ -139,6 +139,9 @@ uint64_t fnn_plan_ranges_used(const fnn_plan *p);
 /* add_f32 instructions of the plan that, on its last pass (or in its recorded graph), did not run as a launch of
  * their own because the MatMul before them stored the sum (FNN_OPT_FUSE_RESIDUAL; no counterpart in fastnn). */
 uint64_t fnn_plan_residuals_fused(const fnn_plan *p);
+/* MatMul instructions of the plan that, on its last pass (or in its recorded graph), found their activation operand
+ * prepared by the split-K reduction of the MatMul before them (FNN_OPT_FUSE_PREP; no counterpart in fastnn). */
+uint64_t fnn_plan_operands_handed(const fnn_plan *p);
 /* Backend::dispatch_profile, src/backend/mod.rs:178-211: elapsed_ns[i] per instruction */
 int fnn_backend_dispatch_profile(fnn_backend *b, fnn_plan *p, uint64_t *elapsed_ns, uint64_t n);
 

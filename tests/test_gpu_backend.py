@@ -893,3 +893,63 @@ def test_matmul_followed_by_residual_add_runs_as_one_call(be, orc, wdt, kname):
         assert_close(view(s_y[i]), want_y, 2e-5, f"MatMul output {i}")
     for s in (s_sum[0], s_sum[1], s_r2, s_y[3], s_sum[4]):
         assert np.array_equal(view(s), view(s_y[0]) + r)
+
+
+@pytest.mark.parametrize("m", [64, 40])
+@pytest.mark.parametrize("single", [0, 1])
+def test_matmul_chain_hands_the_prepared_operand_on(be, orc, m, single):
+    """A MatMul whose result the next instruction multiplies leaves that MatMul's prepared activation operand behind
+    (FNN_OPT_FUSE_PREP): directly, and through the residual Add that rides in its reduction.  Same conversion code, so
+    every tensor of the chain equals, bit for bit, what the plan gives with every MatMul preparing its own operand;
+    an integer-weight MatMul (digit planes, another operand format) and a codebook one are not handed anything."""
+    rng = np.random.default_rng(131 + m + single)
+    d, f = 512, 2048
+    x = rng.standard_normal((m, d)).astype(np.float32)
+    w1 = fastnn_amd.quantize_weights(flib.DT_F8, _w(rng, f, d))
+    w2 = fastnn_amd.quantize_weights(flib.DT_F4, _w(rng, d, f))
+    w3 = fastnn_amd.quantize_weights(flib.DT_U8, _w(rng, f, d))
+    w4 = fastnn_amd.quantize_weights(flib.DT_I4, _w(rng, d, f))
+    b1 = (rng.standard_normal(f) * 0.1).astype(np.float32)
+    a = Arena()
+    s_x = a.take(x.nbytes)
+    s_w = [a.take(w.words.nbytes) for w in (w1, w2, w3, w4)]
+    s_b1 = a.take(b1.nbytes)
+    s_h, s_y, s_s, s_h2, s_y2 = a.take(m * f * 4), a.take(m * d * 4), a.take(m * d * 4), a.take(m * f * 4), a.take(m * d * 4)
+    plan = ExecutablePlan(a.top)
+    for s, w in zip(s_w, (w1, w2, w3, w4)):
+        plan.write_const(s[0], w.words)
+    plan.write_const(s_b1[0], b1)
+    plan.call_kernel("matmul_f8_gelu", [s_x, s_w[0], s_b1], s_h, [m, d, f], meta_of(w1))     # -> operand of the next
+    plan.call_kernel("matmul_f4", [s_h, s_w[1]], s_y, [m, f, d], meta_of(w2))                # handed; + Add -> operand of the next
+    plan.call_kernel("add_f32", [s_y, s_x], s_s, [m * d])
+    plan.call_kernel("matmul_u8_relu", [s_s, s_w[2]], s_h2, [m, d, f], meta_of(w3))          # handed; next has integer weights
+    plan.call_kernel("matmul_i4", [s_h2, s_w[3]], s_y2, [m, f, d], meta_of(w4))
+    be.allocate_arena(a.top)
+    be.write_arena(s_x[0], x)
+    got = {}
+    try:
+        be.set_kernel_flags(flib.FLAG_ACT_F16_SINGLE if single else 0)
+        for on in (1, 0):
+            be.set_option(flib.OPT_FUSE_PREP, on)
+            be.dispatch(plan)
+            first = be.read_arena(0, a.top).copy()
+            be.dispatch(plan)
+            assert plan.replayed
+            got[on] = be.read_arena(0, a.top).copy()
+            assert np.array_equal(first, got[on]), "replay differs from the first dispatch"
+            assert plan.operands_handed == (2 if on else 0)
+    finally:
+        be.set_option(flib.OPT_FUSE_PREP, 1)
+        be.set_kernel_flags(0)
+    assert np.array_equal(got[1], got[0])
+    view = lambda s, cols: got[1][s[0]:s[0] + s[1]].view(np.float32).reshape(m, cols)
+    tol = 1e-3 if single else 2e-5
+    h_ref = orc.qmatmul(to_oracle(orc, w1), x, bias=b1, act=flib.ACT_GELU)
+    assert_close(view(s_h, f), h_ref, tol, "first layer")
+    y_ref = orc.qmatmul(to_oracle(orc, w2), view(s_h, f))
+    assert_close(view(s_y, d), y_ref, tol, "second layer on the first layer's output")
+    assert np.array_equal(view(s_s, d), view(s_y, d) + x)
+    h2_ref = orc.qmatmul(to_oracle(orc, w3), view(s_s, d), act=flib.ACT_RELU)
+    assert_close(view(s_h2, f), h2_ref, tol, "third layer on the sum")
+    y2_ref = orc.qmatmul(to_oracle(orc, w4), view(s_h2, f))
+    assert_close(view(s_y2, d), y2_ref, tol, "fourth layer")
