@@ -250,6 +250,43 @@ __global__ void __launch_bounds__(256) maxpool2d_small_kernel(const float *x, ui
     if (re.table) emit_range(re, mn, mx);
 }
 
+// The same without indices for K x K windows that always meet the image (pad < K): the K * K taps are requested at once
+// from clamped coordinates.  A clamped tap repeats a value of the window, which leaves its maximum as it is; the
+// values meet in (kh, kw) order under the same comparison as above.
+template <int K>
+__global__ void __launch_bounds__(256) maxpool2d_window_kernel(const float *x, float *y, uint32_t out_len, uint32_t h, uint32_t w, FastDiv ho,
+                                                               FastDiv wo, int stride, int pad, RangeEmit re)
+{
+    const uint32_t ie = re.table ? (uint32_t)re.image_elems : out_len, base = blockIdx.y * ie;
+    float mn = INFINITY, mx = -INFINITY;
+    for (uint32_t j = blockIdx.x * 256 + threadIdx.x; j < ie && base + j < out_len; j += gridDim.x * 256) {
+        const uint32_t o = base + j;
+        const uint32_t t = wo.div(o), ww = o - t * wo.d, nc = ho.div(t), hh = t - nc * ho.d;
+        const int h0 = (int)(hh * stride) - pad, w0 = (int)(ww * stride) - pad;
+        const float *ch = x + (uint64_t)nc * h * w;
+        uint32_t ro[K], co[K];
+#pragma unroll
+        for (int k = 0; k < K; k++) {
+            ro[k] = (uint32_t)min(max(h0 + k, 0), (int)h - 1) * w;
+            co[k] = (uint32_t)min(max(w0 + k, 0), (int)w - 1);
+        }
+        float v[K][K];
+#pragma unroll
+        for (int kh = 0; kh < K; kh++)
+#pragma unroll
+            for (int kw = 0; kw < K; kw++) v[kh][kw] = ch[ro[kh] + co[kw]];
+        float val = -INFINITY;
+#pragma unroll
+        for (int kh = 0; kh < K; kh++)
+#pragma unroll
+            for (int kw = 0; kw < K; kw++) val = v[kh][kw] > val ? v[kh][kw] : val;
+        y[o] = val;
+        mn = fminf(mn, val);
+        mx = fmaxf(mx, val);
+    }
+    if (re.table) emit_range(re, mn, mx);
+}
+
 // window mean over the taps inside the image (padding taps neither add nor count), summed in (kh, kw) order
 __global__ void __launch_bounds__(256) avgpool2d_kernel(const float *x, uint64_t in_len, float *y, uint64_t out_len,
                                                         uint64_t h, uint64_t w, uint64_t ho, uint64_t wo, int kernel, int stride, int pad)
@@ -463,7 +500,16 @@ hipError_t launch_maxpool2d(const float *x, uint64_t in_len, float *y, uint64_t 
     const bool images_match = idx_len <= out_len && rio && rio->out_image_elems == c * ho * wo;
     if (!images_match && rio && rio->out_table) rio->out_failed = 1;
     RangePlan rp = range_plan(images_match ? rio : nullptr, out_len, c * ho * wo, c * ho * wo ? out_len / (c * ho * wo) : 0, grid_for(total));
-    if (in_len < (1ull << 31) && total < (1ull << 31) && h * w < (1ull << 31))
+    const uint64_t chans = ho * wo ? (out_len + ho * wo - 1) / (ho * wo) : 0;
+    const bool window = idx_len == 0 && (kernel == 2 || kernel == 3 || kernel == 5) && pad >= 0 && pad < kernel && stride >= 1 && h >= 1 && w >= 1 &&
+                        ho >= 1 && wo >= 1 && (int64_t)(ho - 1) * stride - pad <= (int64_t)h - 1 && (int64_t)(wo - 1) * stride - pad <= (int64_t)w - 1 &&
+                        chans * h * w <= in_len && in_len < (1ull << 31) && out_len < (1ull << 31);
+    if (window) {
+        const FastDiv dh = fast_div((uint32_t)ho), dw = fast_div((uint32_t)wo);
+        if (kernel == 2) hipLaunchKernelGGL(maxpool2d_window_kernel<2>, rp.grid, dim3(256), 0, s, x, y, (uint32_t)out_len, (uint32_t)h, (uint32_t)w, dh, dw, stride, pad, rp.re);
+        else if (kernel == 3) hipLaunchKernelGGL(maxpool2d_window_kernel<3>, rp.grid, dim3(256), 0, s, x, y, (uint32_t)out_len, (uint32_t)h, (uint32_t)w, dh, dw, stride, pad, rp.re);
+        else hipLaunchKernelGGL(maxpool2d_window_kernel<5>, rp.grid, dim3(256), 0, s, x, y, (uint32_t)out_len, (uint32_t)h, (uint32_t)w, dh, dw, stride, pad, rp.re);
+    } else if (in_len < (1ull << 31) && total < (1ull << 31) && h * w < (1ull << 31))
         hipLaunchKernelGGL(maxpool2d_small_kernel, rp.grid, dim3(256), 0, s, x, (uint32_t)in_len, y, (uint32_t)out_len, (uint32_t)h, (uint32_t)w,
                            fast_div((uint32_t)ho), fast_div((uint32_t)wo), kernel, stride, pad, indices, (uint32_t)idx_len, rp.re);
     else

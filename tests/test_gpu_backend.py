@@ -953,3 +953,27 @@ def test_matmul_chain_hands_the_prepared_operand_on(be, orc, m, single):
     assert_close(view(s_h2, f), h2_ref, tol, "third layer on the sum")
     y2_ref = orc.qmatmul(to_oracle(orc, w4), view(s_h2, f))
     assert_close(view(s_y2, d), y2_ref, tol, "fourth layer")
+
+
+@pytest.mark.parametrize("k,s,p", [(5, 1, 2), (3, 2, 2), (2, 1, 1), (5, 2, 4), (3, 1, 0), (4, 2, 1)])
+def test_maxpool_windows_with_special_values(be, orc, k, s, p):
+    """Max pooling with every tap requested at once from clamped coordinates (2 x 2, 3 x 3, 5 x 5 windows) and the
+    tap-by-tap kernel (4 x 4): the same bits as the CPU arm, also for signed zeros, infinities and NaN (never
+    selected: a window of NaN gives -inf), on odd map sizes and with the largest padding a window allows."""
+    rng = np.random.default_rng(1000 + 10 * k + p)
+    n, c, h, w = 2, 3, 7, 9
+    x = rng.standard_normal((n, c, h, w)).astype(np.float32)
+    x[rng.random(x.shape) < 0.15] = 0.0
+    x[rng.random(x.shape) < 0.10] = -0.0
+    x[rng.random(x.shape) < 0.05] = np.nan
+    x[rng.random(x.shape) < 0.03] = -np.inf
+    x[rng.random(x.shape) < 0.03] = np.inf
+    x[0, 0, :4, :5] = np.nan                      # whole windows of NaN
+    want = orc.maxpool2d(x, k, s, p)
+    a = Arena()
+    s_x, s_y = a.take(x.nbytes), a.take(want.nbytes)
+    plan = ExecutablePlan(a.top).write_const(s_x[0], x).call_kernel("pool_f32", [s_x], s_y, [k, s, p, 1, n, c, h, w])
+    be.allocate_arena(a.top)
+    be.dispatch(plan)
+    got = be.read_arena(*s_y, np.uint32)
+    assert np.array_equal(got, want.reshape(-1).view(np.uint32))
