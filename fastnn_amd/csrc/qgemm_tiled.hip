@@ -4,7 +4,7 @@
 //   (gemm_batch_packed_simd + apply_affine_dot, src/backend/cpu/microkernels/gemm.rs:1982-2088,
 //    src/backend/cpu/microkernels/mod.rs:283-295)
 //
-// Two launches:
+// Launches:
 //  1. act_prep_kernel turns the f32 activations into f16 MFMA operands once per call (not
 //     once per workgroup): each row is scaled by a power of two so that max|x| lands in
 //     [2^14, 2^15) and written as hi = f16(x') and, in the default mode, lo = f16((x'-hi)*2^11),
@@ -20,7 +20,10 @@
 //     with v_mfma_f32_32x32x16_f16.
 //  3. With K split over several workgroups (few activation rows: not enough tiles to fill
 //     the chip) the partial tiles go to a workspace and splitk_epilogue_kernel adds them in
-//     split order, so results do not depend on scheduling.
+//     split order, so results do not depend on scheduling.  Asked to (a plan whose next instruction is the MatMul
+//     that reads this result: FnnResidualIo / FnnPrepIo in range_io.h), that kernel also stores the sum with a
+//     residual, and splitk_prep_epilogue_kernel, one workgroup per output row, leaves the operand of step 1 for that
+//     next MatMul, which then starts at step 2.
 //
 // FNN_FLAG_ACT_F16_SINGLE keeps hi only and removes the first-order effect of the rounding
 // on rows with a non-zero mean lane value: dot -= mean_k(u[n,k]) * sum_k (hi - x').
