@@ -336,7 +336,12 @@ __global__ void __launch_bounds__(64 * PW * KW) conv_implicit_kernel(ImplicitArg
                 }
                 if (p.vec4) {
                     const int64_t o = r_off[pw][rr0] + n * np;
-                    *reinterpret_cast<float4 *>(y + o) = make_float4(v[0], v[1], v[2], v[3]);
+                    if constexpr (TN > 1) {   // stored below, channel by channel
+#pragma unroll
+                        for (int j = 0; j < 4; j++) acc[tn][ig * 4 + j] = __float_as_int(v[j]);
+                    } else {
+                        *reinterpret_cast<float4 *>(y + o) = make_float4(v[0], v[1], v[2], v[3]);
+                    }
                     if (acc_out) *reinterpret_cast<int4 *>(acc_out + o) = make_int4(av[0], av[1], av[2], av[3]);
                 } else {
 #pragma unroll
@@ -345,6 +350,24 @@ __global__ void __launch_bounds__(64 * PW * KW) conv_implicit_kernel(ImplicitArg
                         const int64_t o = r_off[pw][rr0 + j] + n * np;
                         y[o] = v[j];
                         if (acc_out) acc_out[o] = av[j];
+                    }
+                }
+            }
+        }
+        // several channel blocks per wave: the four stores that fill a channel's 128-byte line follow each other
+        if constexpr (TN > 1) {
+            if (p.vec4) {
+#pragma unroll
+                for (int tn = 0; tn < TN; tn++) {
+                    const int64_t n = n0 + tn * 32 + lr;
+                    if (n >= ocg) continue;
+#pragma unroll
+                    for (int ig = 0; ig < 4; ig++) {
+                        const int rr0 = ig * 8 + hf * 4;
+                        if (r_first + pw * 32 + rr0 >= rows) continue;
+                        const int64_t o = r_off[pw][rr0] + n * np;
+                        *reinterpret_cast<float4 *>(y + o) = make_float4(__int_as_float(acc[tn][ig * 4]), __int_as_float(acc[tn][ig * 4 + 1]),
+                                                                          __int_as_float(acc[tn][ig * 4 + 2]), __int_as_float(acc[tn][ig * 4 + 3]));
                     }
                 }
             }
