@@ -977,3 +977,71 @@ def test_maxpool_windows_with_special_values(be, orc, k, s, p):
     be.dispatch(plan)
     got = be.read_arena(*s_y, np.uint32)
     assert np.array_equal(got, want.reshape(-1).view(np.uint32))
+
+
+@pytest.mark.parametrize("seed", [3, 4])
+def test_random_matmul_chains_equal_with_and_without_plan_fusions(be, seed):
+    """Random chains of two to five MatMuls (mixed weight types, 17 <= M <= 200, optional bias and activation) with
+    residual Adds wherever an earlier tensor has the same width: the whole arena with FNN_OPT_FUSE_RESIDUAL and
+    FNN_OPT_FUSE_PREP on equals, byte for byte, the arena with both off, on the first dispatch and on the replay."""
+    rng = np.random.default_rng(seed)
+    engaged = 0
+    for case in range(8):
+        m = int(rng.choice([17, 24, 40, 64, 100, 128, 200]))
+        nl = int(rng.integers(2, 6))
+        dims = [int(rng.choice([64, 128, 192, 512, 1024, 2048, 4096, 512, 1024])) for _ in range(nl + 1)]
+        dts = [int(rng.choice([flib.DT_F8, flib.DT_F4, flib.DT_U8, flib.DT_F8R, flib.DT_F8, flib.DT_I4, flib.DT_I8])) for _ in range(nl)]
+        a = Arena()
+        x = rng.standard_normal((m, dims[0])).astype(np.float32)
+        s_x = a.take(x.nbytes)
+        ws = [fastnn_amd.quantize_weights(dts[i], (rng.standard_normal((dims[i + 1], dims[i])) / np.sqrt(dims[i])).astype(np.float32)) for i in range(nl)]
+        s_w = [a.take(w.words.nbytes) for w in ws]
+        plan_calls, consts = [], []
+        cur, same_width = s_x, {dims[0]: s_x}
+        for i in range(nl):
+            k, n = dims[i], dims[i + 1]
+            out = a.take(m * n * 4)
+            name = KERNEL_OF[dts[i]] + ["", "_relu", "_gelu", "_silu"][int(rng.integers(0, 4))]
+            inputs = [cur, s_w[i]]
+            if rng.random() < 0.5:
+                bias = (rng.standard_normal(n) * 0.1).astype(np.float32)
+                s_b = a.take(bias.nbytes)
+                consts.append((s_b, bias))
+                inputs.append(s_b)
+            plan_calls.append((name, inputs, out, [m, k, n], meta_of(ws[i])))
+            cur = out
+            if n in same_width and rng.random() < 0.7:
+                s_sum = a.take(m * n * 4)
+                pair = [cur, same_width[n]] if rng.random() < 0.5 else [same_width[n], cur]
+                plan_calls.append(("add_f32", pair, s_sum, [m * n], None))
+                cur = s_sum
+            same_width[n] = cur
+        plan = ExecutablePlan(a.top)
+        for s, w in zip(s_w, ws):
+            plan.write_const(s[0], w.words)
+        for s, v in consts:
+            plan.write_const(s[0], v)
+        for name, inputs, out, par, meta in plan_calls:
+            plan.call_kernel(name, inputs, out, par, meta)
+        be.allocate_arena(a.top)
+        be.write_arena(s_x[0], x)
+        got = {}
+        try:
+            for on in (1, 0):
+                be.set_option(flib.OPT_FUSE_PREP, on)
+                be.set_option(flib.OPT_FUSE_RESIDUAL, on)
+                be.dispatch(plan)
+                first = be.read_arena(0, a.top).copy()
+                be.dispatch(plan)
+                got[on] = be.read_arena(0, a.top).copy()
+                assert np.array_equal(first, got[on]), (case, on, "replay differs from the first dispatch")
+                if on:
+                    engaged += plan.residuals_fused + plan.operands_handed
+                else:
+                    assert plan.residuals_fused == 0 and plan.operands_handed == 0
+        finally:
+            be.set_option(flib.OPT_FUSE_PREP, 1)
+            be.set_option(flib.OPT_FUSE_RESIDUAL, 1)
+        assert np.array_equal(got[1], got[0]), (case, m, dims, dts)
+        plan.close()
+    assert engaged > 0
