@@ -234,6 +234,21 @@ __global__ void __launch_bounds__(64 * PW * KW) conv_implicit_kernel(ImplicitArg
         }
     }
 
+    // this lane's channel constants: requested when the K loop is done (not earlier: they would take registers the
+    // loop's loads in flight need), so that they travel while the K slices meet
+    float sw[TN], zw[TN], bi[TN];
+    int wq_[TN];
+#pragma unroll
+    for (int tn = 0; tn < TN; tn++) {
+        const int64_t n = n0 + tn * 32 + lr;
+        const bool ok = kw == 0 && n < ocg;
+        const int64_t ch = (int64_t)g * ocg + (ok ? n : 0);
+        sw[tn] = ok ? a.scales[ch] : 0.0f;
+        zw[tn] = ok ? a.zeros[ch] : 0.0f;
+        wq_[tn] = ok ? a.row_qsum[ch] : 0;
+        bi[tn] = (ok && a.bias) ? a.bias[ch] : 0.0f;
+    }
+
     // ---- the K slices of a pixel block meet in LDS (exact integers: any order)
     constexpr int SLOT = (TN * 16 + 1) * 64;
     if (KW > 1) {
@@ -279,18 +294,6 @@ __global__ void __launch_bounds__(64 * PW * KW) conv_implicit_kernel(ImplicitArg
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        float sw[TN], zw[TN], bi[TN];
-        int wq_[TN];
-#pragma unroll
-        for (int tn = 0; tn < TN; tn++) {
-            const int64_t n = n0 + tn * 32 + lr;
-            const bool ok = n < ocg;
-            const int64_t ch = (int64_t)g * ocg + (ok ? n : 0);
-            sw[tn] = ok ? a.scales[ch] : 0.0f;
-            zw[tn] = ok ? a.zeros[ch] : 0.0f;
-            wq_[tn] = ok ? a.row_qsum[ch] : 0;
-            bi[tn] = (ok && a.bias) ? a.bias[ch] : 0.0f;
-        }
         const bool has_bias = a.bias != nullptr;
         float *y = a.y + (int64_t)g * ocg * np;
         int32_t *acc_out = a.acc_out ? a.acc_out + (int64_t)g * ocg * np : nullptr;
