@@ -1128,7 +1128,9 @@ int fnn_ctx_ensure_tmp(fnn_hip_ctx *ctx, int which, size_t bytes, void **ptr)
         *ptr = ctx->static_ws + off;
         return FNN_OK;
     }
-    Staging &s = which == 0 ? ctx->st_tmp : (which == 1 ? ctx->st_tmp2 : (which == 2 ? ctx->st_tmp3 : ctx->st_tmp4));
+    // 0: prepared operands, 1: partial tiles / accumulators, 2 and 3: conv operand, transient weight expansion,
+    // 4: the prepared operand one MatMul call leaves for the next
+    Staging &s = which == 0 ? ctx->st_tmp : (which == 1 ? ctx->st_tmp2 : (which == 4 ? ctx->st_tmp4 : ctx->st_tmp3));
     int rc = ensure(ctx, s, bytes);
     if (rc) return rc;
     *ptr = s.ptr;

@@ -650,7 +650,7 @@ int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QM
                                  NL.kpad == N && !((reinterpret_cast<uintptr_t>(t.scales) | reinterpret_cast<uintptr_t>(t.zeros) | reinterpret_cast<uintptr_t>(t.out) |
                                                     reinterpret_cast<uintptr_t>(t.sum_out) | reinterpret_cast<uintptr_t>(t.part)) & 15);
         void *nb = nullptr;
-        const int next_slot = own_slot == 0 ? 3 : 0;
+        const int next_slot = own_slot == 0 ? 4 : 0;
         if (may_prepare && fnn_ctx_ensure_tmp(ctx, next_slot, NL.ws_bytes, &nb) == FNN_OK && nb) {
             PrepArgs np;
             np.a = nullptr;
