@@ -444,6 +444,8 @@ CONVS = [
     dict(b=3, c=5, h=9, w=9, oc=7, kh=3, kw=3, stride=1, pad=1, dil=1, groups=1),
     dict(b=1, c=32, h=16, w=16, oc=64, kh=3, kw=3, stride=1, pad=1, dil=1, groups=1),
     dict(b=2, c=12, h=13, w=14, oc=160, kh=3, kw=3, stride=1, pad=1, dil=1, groups=1),   # two column tiles, rows past a row tile
+    dict(b=2, c=32, h=11, w=12, oc=32, kh=3, kw=3, stride=1, pad=1, dil=1, groups=32),   # depthwise: every group in one launch of the direct kernel
+    dict(b=1, c=32, h=9, w=10, oc=48, kh=3, kw=3, stride=2, pad=1, dil=1, groups=16),
 ]
 
 
