@@ -331,3 +331,76 @@ def test_conv_activation_ranges_odd_shapes_and_every_producer(orc):
     assert used[1] == 7, used   # c2, c4, c5, c6, c7, c8, c9; c3 and the first convolution scan
     for name in outs:
         assert np.array_equal(results[1][name], results[0][name]), name
+
+
+@pytest.mark.parametrize("seed", [21, 22])
+def test_random_conv_graphs_equal_under_every_range_and_kernel_choice(seed):
+    """Random graphs of 3 x 3 / 1 x 1 / strided convolutions with MaxPool, Resize, residual Add, ReLU and Concat
+    between them (batch 1-3, maps of 9-40 pixels a side, 8-96 channels): the output of the plan is the same, bit for
+    bit, with the activation ranges handed over or scanned and with the implicit-GEMM kernel chosen by shape, forced
+    on or forced off, on the first dispatch and on the replay."""
+    rng = np.random.default_rng(seed)
+    for case in range(5):
+        b, c0 = int(rng.integers(1, 4)), int(rng.choice([3, 5, 8, 16]))
+        h, w = int(rng.integers(9, 41)), int(rng.integers(9, 41))
+        nodes, params, cnt = [], {}, [0]
+
+        def uid(p):
+            cnt[0] += 1
+            return f"{p}{cnt[0]}"
+
+        def conv(x, c, oc, k, s, pad):
+            wn, bn, y0, y = uid("w"), uid("b"), uid("c"), uid("s")
+            params[wn] = (rng.standard_normal((oc, c, k, k)) * np.sqrt(2.0 / (c * k * k))).astype(np.float32)
+            params[bn] = (rng.standard_normal(oc) * 0.05).astype(np.float32)
+            nodes.append({"name": y0, "op_type": "Conv", "inputs": f"[{x}, {wn}, {bn}]", "outputs": f"[{y0}]", "strides": str(s),
+                          "pads": str(pad), "group": "1"})
+            nodes.append({"name": y, "op_type": "Silu", "inputs": f"[{y0}]", "outputs": f"[{y}]"})
+            return y
+
+        cur, cc, ch, cw = "x", c0, h, w
+        for _ in range(int(rng.integers(3, 8))):
+            kind = rng.choice(["conv3", "conv1", "conv3s2", "pool", "up", "res", "relu", "cat"], p=[0.3, 0.2, 0.1, 0.08, 0.07, 0.1, 0.05, 0.1])
+            if kind in ("conv3", "conv1", "conv3s2"):
+                oc, k = int(rng.choice([8, 16, 24, 40, 64, 96])), (1 if kind == "conv1" else 3)
+                s = 2 if kind == "conv3s2" and min(ch, cw) >= 8 else 1
+                cur = conv(cur, cc, oc, k, s, k // 2)
+                cc, ch, cw = oc, (ch + 2 * (k // 2) - k) // s + 1, (cw + 2 * (k // 2) - k) // s + 1
+            elif kind == "pool":
+                y = uid("m")
+                nodes.append({"name": y, "op_type": "MaxPool", "inputs": f"[{cur}]", "outputs": f"[{y}]", "kernel_size": "5", "stride": "1", "padding": "2"})
+                cur = y
+            elif kind == "up" and ch * cw < 900:
+                y = uid("u")
+                nodes.append({"name": y, "op_type": "Resize", "inputs": f"[{cur}]", "outputs": f"[{y}]", "mode": "nearest", "scale_h": "2", "scale_w": "2"})
+                cur, ch, cw = y, ch * 2, cw * 2
+            elif kind == "res":
+                t, y = conv(cur, cc, cc, 3, 1, 1), uid("a")
+                nodes.append({"name": y, "op_type": "Add", "inputs": f"[{cur}, {t}]", "outputs": f"[{y}]"})
+                cur = y
+            elif kind == "relu":
+                y = uid("r")
+                nodes.append({"name": y, "op_type": "Relu", "inputs": f"[{cur}]", "outputs": f"[{y}]"})
+                cur = y
+            elif kind == "cat":
+                t, y = conv(cur, cc, 8, 1, 1, 0), uid("k")
+                nodes.append({"name": y, "op_type": "Concat", "inputs": f"[{cur}, {t}]", "outputs": f"[{y}]", "axis": "1"})
+                cur, cc = y, cc + 8
+        cur = conv(cur, cc, 8, 3, 1, 1)
+        shape = (b, c0, h, w)
+        x = rng.uniform(-1, 1, shape).astype(np.float32)
+        res = {}
+        for ranges, implicit in [(0, 0), (1, 0), (1, 1), (1, 2), (0, 1)]:
+            ex = AotExecutor(nodes, params, ["x"], [cur], {"x": shape}, quantize=8)
+            try:
+                ex.set_option(flib.OPT_CONV_RANGES, ranges)
+                ex.set_option(flib.OPT_CONV_IMPLICIT, implicit)
+                first = ex.forward({"x": x})[cur]
+                again = ex.forward({"x": x})[cur]
+                assert np.array_equal(first, again), (case, ranges, implicit, "replay differs from the first dispatch")
+                assert ranges or ex.ranges_used == 0
+                res[(ranges, implicit)] = again
+            finally:
+                ex.close()
+        for key, val in res.items():
+            assert np.array_equal(val, res[(0, 0)]), (case, key, shape, len(nodes))
