@@ -337,8 +337,9 @@ def test_conv_activation_ranges_odd_shapes_and_every_producer(orc):
 def test_random_conv_graphs_equal_under_every_range_and_kernel_choice(seed):
     """Random graphs of 3 x 3 / 1 x 1 / strided convolutions with MaxPool, Resize, residual Add, ReLU and Concat
     between them (batch 1-3, maps of 9-40 pixels a side, 8-96 channels): the output of the plan is the same, bit for
-    bit, with the activation ranges handed over or scanned and with the implicit-GEMM kernel chosen by shape, forced
-    on or forced off, on the first dispatch and on the replay."""
+    bit, with the activation ranges handed over or scanned, with the implicit-GEMM kernel chosen by shape, forced on or
+    forced off, and with the residual Adds inside the convolution before them or as launches of their own, on the first
+    dispatch and on the replay."""
     rng = np.random.default_rng(seed)
     for case in range(5):
         b, c0 = int(rng.integers(1, 4)), int(rng.choice([3, 5, 8, 16]))
@@ -390,17 +391,19 @@ def test_random_conv_graphs_equal_under_every_range_and_kernel_choice(seed):
         shape = (b, c0, h, w)
         x = rng.uniform(-1, 1, shape).astype(np.float32)
         res = {}
-        for ranges, implicit in [(0, 0), (1, 0), (1, 1), (1, 2), (0, 1)]:
+        for ranges, implicit, fuse in [(0, 0, 0), (1, 0, 1), (1, 1, 1), (1, 2, 1), (0, 1, 1), (1, 0, 0), (0, 2, 1)]:
             ex = AotExecutor(nodes, params, ["x"], [cur], {"x": shape}, quantize=8)
             try:
                 ex.set_option(flib.OPT_CONV_RANGES, ranges)
                 ex.set_option(flib.OPT_CONV_IMPLICIT, implicit)
+                ex.set_option(flib.OPT_FUSE_RESIDUAL, fuse)   # (the Add behind a convolution rides in its epilogue)
                 first = ex.forward({"x": x})[cur]
                 again = ex.forward({"x": x})[cur]
-                assert np.array_equal(first, again), (case, ranges, implicit, "replay differs from the first dispatch")
+                assert np.array_equal(first, again), (case, ranges, implicit, fuse, "replay differs from the first dispatch")
                 assert ranges or ex.ranges_used == 0
-                res[(ranges, implicit)] = again
+                assert fuse or ex.residuals_fused == 0
+                res[(ranges, implicit, fuse)] = again
             finally:
                 ex.close()
         for key, val in res.items():
-            assert np.array_equal(val, res[(0, 0)]), (case, key, shape, len(nodes))
+            assert np.array_equal(val, res[(0, 0, 0)]), (case, key, shape, len(nodes))
