@@ -336,17 +336,31 @@ def algorithmic_bytes(dt: str, m: int, k: int, n: int, bias: bool) -> int:
     return wbytes + side + 4 * m * k + 4 * m * n
 
 
-PROBE_LIB = os.path.join(ROOT, "fastnn_amd", "libfnn_probe.so")
+PROBE_SRC = os.path.join(ROOT, "bench_probe.hip")
+PROBE_LIB = os.path.join(ROOT, "libbench_probe.so")
+
+
+def build_probe(force: bool = False) -> str:
+    """Compiles bench_probe.hip (plain read / copy / matrix-core / LDS kernels that only this benchmark uses) into
+    libbench_probe.so beside it.  hipcc cross-compiles for gfx950 without a GPU."""
+    import subprocess
+    if force or not os.path.exists(PROBE_LIB) or os.path.getmtime(PROBE_LIB) < os.path.getmtime(PROBE_SRC):
+        cmd = ["/opt/rocm/bin/hipcc", "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
+               "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-shared", PROBE_SRC, "-o", PROBE_LIB]
+        r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        if r.returncode != 0:
+            raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), r.stdout))
+    return PROBE_LIB
 
 
 class Probe:
-    """The plain read / copy kernels of fastnn_amd/libfnn_probe.so (built beside the product library, not part of
-    it), launched on the context's stream so that the context's events time them."""
+    """The plain read / copy kernels of libbench_probe.so (this benchmark's own measurement aid, not part of the
+    product library), launched on the context's stream so that the context's events time them."""
 
     def __init__(self, ctx):
         import ctypes as C
         if not os.path.exists(PROBE_LIB):
-            raise FileNotFoundError(f"{PROBE_LIB} not found: build it with `python -m fastnn_amd.build`")
+            build_probe()
         self.lib = C.CDLL(PROBE_LIB)
         self.lib.fnn_probe_stream.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p]
         self.lib.fnn_probe_mfma.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p]

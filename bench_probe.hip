@@ -1,4 +1,4 @@
-// Device-ceiling probes, built as a library of their own (libfnn_probe.so): not part of the product ABI.
+// Device-ceiling probes, built by bench.py as a library of their own (libbench_probe.so): not part of the product ABI.
 // A plain streaming read and a plain copy of a known number of bytes give (a) the bandwidth one launch of a
 // given size can reach on this device, the ceiling a bandwidth-bound kernel of that size is judged against,
 // and (b) a kernel of known traffic to scale hardware byte counters with.

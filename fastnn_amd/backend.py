@@ -237,10 +237,16 @@ class HipBackend:
         self._check(rc)
         return None
 
-    def dispatch_profile(self, plan: ExecutablePlan):
+    def dispatch_profile(self, plan: ExecutablePlan, shape_env: Optional[dict] = None):
+        """Backend::dispatch_profile: nanoseconds per instruction, under the call's ShapeEnv (empty when omitted)."""
         n = len(plan)
         t = (C.c_uint64 * max(n, 1))()
-        self._check(self.lib.fnn_backend_dispatch_profile(self.handle, plan.handle, t, n))
+        if not shape_env:
+            self._check(self.lib.fnn_backend_dispatch_profile(self.handle, plan.handle, t, n))
+        else:
+            names = (C.c_char_p * len(shape_env))(*[k.encode() for k in shape_env])
+            values = (C.c_uint64 * len(shape_env))(*[int(v) for v in shape_env.values()])
+            self._check(self.lib.fnn_backend_dispatch_profile_env(self.handle, plan.handle, names, values, len(shape_env), t, n))
         return [int(t[i]) for i in range(n)]
 
     def close(self):

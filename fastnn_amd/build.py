@@ -16,9 +16,6 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libfastnn_hip.so")
-# measurement aid for bench.py (plain read / copy kernels), deliberately outside the product library
-PROBE_LIB = os.path.join(HERE, "libfnn_probe.so")
-PROBE_SOURCE = "probe.hip"
 
 HIP_SOURCES = ["api.hip", "qgemv.hip", "qgemm_generic.hip", "qgemm_tiled.hip", "qgemm_i8.hip", "qgemm_digits.hip", "qgemv_mfma.hip", "qgemv_i8dot.hip", "qgemv_rows16.hip", "i8act.hip", "qconv.hip", "qconv_float.hip", "qconv_implicit.hip", "eltwise.hip"]
 HOST_SOURCES = ["quantize_host.cpp", "hip_backend.cpp"]
@@ -81,9 +78,6 @@ def build(force: bool = False, verbose: bool = False) -> str:
                 print(out)
     if jobs or force or not os.path.exists(LIB):
         _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs + ["-lpthread"])
-    probe_src = os.path.join(CSRC, PROBE_SOURCE)
-    if force or _stale(PROBE_LIB, [probe_src]):
-        _run([hipcc] + HIP_FLAGS + ["-shared", probe_src, "-o", PROBE_LIB])
     return LIB
 
 

@@ -314,6 +314,25 @@ int resolve_params(fnn_backend *b, const Instr &in, size_t expected, std::vector
     return FNN_OK;
 }
 
+// M, K, N of a MatMul instruction when they do not depend on the dispatch's ShapeEnv: the stored params of an
+// instruction without param_dims, or param_dims whose first three entries are all DimExpr::Known, which is what
+// CpuBackend::compile emits for every MatMul of a static graph (src/backend/cpu/mod.rs:601-613) and what
+// resolve_params would return under any environment.
+bool static_mkn(const Instr &in, uint64_t *mkn)
+{
+    if (!in.has_param_dims) {
+        if (in.params.size() < 3) return false;
+        for (int i = 0; i < 3; i++) mkn[i] = in.params[i];
+        return true;
+    }
+    if (in.param_dims.size() < 3) return false;
+    for (int i = 0; i < 3; i++) {
+        if (in.param_dims[i].kind != 0) return false;
+        mkn[i] = in.param_dims[i].value;
+    }
+    return true;
+}
+
 int run_matmul(fnn_backend *b, const Instr &in, const KernelName &kn, int dtype)
 {
     const char *name = in.kernel.c_str();
@@ -803,8 +822,9 @@ void analyse(fnn_plan *p)
         mm.add_operand = -1;
         if (mm.kind != K_CALL || ad.kind != K_CALL || ad.kernel != "add_f32" || ad.inputs.size() != 2) continue;
         const KernelName kn = split_activation(mm.kernel);
-        if (matmul_dtype(kn.base) < 0 || mm.has_param_dims || mm.params.size() < 3) continue;
-        const uint64_t bytes = mm.params[0] * mm.params[2] * 4;
+        uint64_t mkn[3];
+        if (matmul_dtype(kn.base) < 0 || !static_mkn(mm, mkn)) continue;
+        const uint64_t bytes = mkn[0] * mkn[2] * 4;
         if (bytes == 0 || mm.dst.size != bytes || ad.dst.size != bytes) continue;
         int other = -1;
         for (int k = 0; k < 2; k++)
@@ -911,21 +931,22 @@ int run_instr(fnn_backend *b, fnn_plan *p, size_t idx, bool consts_resident)
         *pio = FnnPrepIo{};
         size_t consumer = (size_t)-1;
         const KernelName kn = split_activation(in.kernel);
-        const bool plain_matmul = matmul_dtype(kn.base) >= 0 && !in.has_param_dims && in.params.size() >= 3 && in.meta.codebook.empty();
+        uint64_t mkn[3] = {0, 0, 0}, nmkn[3] = {0, 0, 0};
+        const bool plain_matmul = matmul_dtype(kn.base) >= 0 && static_mkn(in, mkn) && in.meta.codebook.empty();
         if (hand && plain_matmul) {
             pio->offered = offered_here ? 1 : 0;
             const size_t j = idx + (with_res ? 2 : 1);
-            const uint64_t m = in.params[0], n = in.params[2];
+            const uint64_t m = mkn[0], n = mkn[2];
             const fnn_slice &feeds = with_res ? p->instrs[idx + 1].dst : in.dst;
             if (j < p->instrs.size() && in.dst.size == m * n * 4) {
                 const Instr &nx = p->instrs[j];
                 const KernelName kx = nx.kind == K_CALL ? split_activation(nx.kernel) : KernelName{};
                 const int dx = nx.kind == K_CALL ? matmul_dtype(kx.base) : -1;
-                if (dx >= 0 && !nx.has_param_dims && nx.params.size() >= 3 && nx.inputs.size() >= 2 && nx.meta.codebook.empty() &&
-                    nx.params[0] == m && nx.params[1] == n && nx.inputs[0].offset == feeds.offset && nx.inputs[0].size == m * n * 4 &&
+                if (dx >= 0 && static_mkn(nx, nmkn) && nx.inputs.size() >= 2 && nx.meta.codebook.empty() &&
+                    nmkn[0] == m && nmkn[1] == n && nx.inputs[0].offset == feeds.offset && nx.inputs[0].size == m * n * 4 &&
                     in_arena(b, nx.inputs[0]) && in_arena(b, nx.inputs[1])) {
                     fnn_hip_weight *wn = nullptr;
-                    if (weight_for(b, nx.inputs[1], dx, nx.meta, nx.params[2], nx.params[1], nx.kernel.c_str(), &wn) == FNN_OK && wn) {
+                    if (weight_for(b, nx.inputs[1], dx, nx.meta, nmkn[2], nmkn[1], nx.kernel.c_str(), &wn) == FNN_OK && wn) {
                         pio->next_w = wn;
                         pio->next_flags = FNN_FLAG_DEVICE_PTRS | b->kernel_flags;
                         pio->next_a = (const float *)(b->arena + feeds.offset);
@@ -1654,6 +1675,20 @@ int fnn_backend_dispatch_profile(fnn_backend *b, fnn_plan *p, uint64_t *elapsed_
 {
     return guarded(b, "fnn_backend_dispatch_profile", [&]() -> int {
         if (!elapsed_ns) return fail(b, FNN_ERR_DISPATCH, "dispatch_profile: NULL timings");
+        if (b) { b->shape_env.clear(); b->shape_env_sig.clear(); }   // an empty ShapeEnv, not the previous dispatch's
+        return dispatch_impl(b, p, elapsed_ns, n);
+    });
+}
+
+int fnn_backend_dispatch_profile_env(fnn_backend *b, fnn_plan *p, const char *const *names, const uint64_t *values, uint64_t n_symbols,
+                                     uint64_t *elapsed_ns, uint64_t n)
+{
+    return guarded(b, "fnn_backend_dispatch_profile_env", [&]() -> int {
+        if (!b) return fail(nullptr, FNN_ERR_DISPATCH, "dispatch_profile: NULL argument");
+        if (!elapsed_ns) return fail(b, FNN_ERR_DISPATCH, "dispatch_profile: NULL timings");
+        if ((!names || !values) && n_symbols) return fail(b, FNN_ERR_DISPATCH, "dispatch_profile: NULL shape environment");
+        int st = set_shape_env(b, names, values, n_symbols);
+        if (st) return st;
         return dispatch_impl(b, p, elapsed_ns, n);
     });
 }

@@ -63,6 +63,7 @@ BACKEND_SYMBOLS = [
     "fnn_plan_add_memcopy", "fnn_plan_add_call_kernel", "fnn_plan_len", "fnn_plan_replayed", "fnn_plan_ranges_used", "fnn_plan_residuals_fused", "fnn_plan_operands_handed", "fnn_plan_arena_size",
     "fnn_plan_set_param_dims", "fnn_plan_from_bincode", "fnn_plan_to_bincode", "fnn_plan_describe",
     "fnn_backend_dispatch", "fnn_backend_dispatch_env", "fnn_backend_dispatch_from", "fnn_backend_dispatch_profile",
+    "fnn_backend_dispatch_profile_env",
     "fnn_hip_elementwise", "fnn_hip_fill_f32", "fnn_hip_copy",
     "fnn_hip_copy2d_f32", "fnn_hip_concat_f32", "fnn_hip_maxpool2d_f32", "fnn_hip_avgpool2d_f32", "fnn_hip_upsample_nearest2d_f32",
 ]
@@ -205,6 +206,7 @@ def _prototype(l):
     l.fnn_plan_to_bincode.argtypes = [_vp, _vp, _u64, C.POINTER(_u64)]
     l.fnn_plan_describe.argtypes = [_vp, _u64, C.c_char_p, _u64]
     l.fnn_backend_dispatch_profile.argtypes = [_vp, _vp, C.POINTER(_u64), _u64]
+    l.fnn_backend_dispatch_profile_env.argtypes = [_vp, _vp, C.POINTER(C.c_char_p), C.POINTER(_u64), _u64, C.POINTER(_u64), _u64]
     l.fnn_hip_elementwise.argtypes = [_vp, C.c_int, _vp, _vp, _u64, _vp, _u64]
     l.fnn_hip_fill_f32.argtypes = [_vp, _vp, _u64, C.c_float]
     l.fnn_hip_copy.argtypes = [_vp, _vp, _vp, _u64]

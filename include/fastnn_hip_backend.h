@@ -144,6 +144,11 @@ uint64_t fnn_plan_residuals_fused(const fnn_plan *p);
 uint64_t fnn_plan_operands_handed(const fnn_plan *p);
 /* Backend::dispatch_profile, src/backend/mod.rs:178-211: elapsed_ns[i] per instruction */
 int fnn_backend_dispatch_profile(fnn_backend *b, fnn_plan *p, uint64_t *elapsed_ns, uint64_t n);
+/* The same under the ShapeEnv the trait method is handed (symbolic param_dims are resolved against it, as
+ * Backend::dispatch_profile's default does through dispatch, src/backend/mod.rs:178-211); the form without an
+ * environment runs under an empty one. */
+int fnn_backend_dispatch_profile_env(fnn_backend *b, fnn_plan *p, const char *const *names, const uint64_t *values,
+                                     uint64_t n_symbols, uint64_t *elapsed_ns, uint64_t n);
 
 /* f32 elementwise kernels found between quantised layers ("add_f32" with the second operand
  * broadcast by index modulo its length, "relu_f32", "gelu_f32", "silu_f32";

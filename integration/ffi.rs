@@ -111,4 +111,14 @@ extern "C" {
         stopped_at: *mut u64,
     ) -> c_int;
     pub fn fnn_backend_dispatch_profile(b: *mut fnn_backend, p: *mut fnn_plan, elapsed_ns: *mut u64, n: u64) -> c_int;
+    /// `fnn_backend_dispatch_profile` under the bindings of a `ShapeEnv`.
+    pub fn fnn_backend_dispatch_profile_env(
+        b: *mut fnn_backend,
+        p: *mut fnn_plan,
+        names: *const *const c_char,
+        values: *const u64,
+        n_symbols: u64,
+        elapsed_ns: *mut u64,
+        n: u64,
+    ) -> c_int;
 }

@@ -222,6 +222,35 @@ impl Drop for HipBackend {
     }
 }
 
+/// Kernel names of the weight-quantised MatMul with f32 activations (src/backend/cpu/mod.rs:459-495).  The
+/// I8-activation forms (`matmul_i8_i8`, `matmul_i4_i8`) have no fused epilogue on either backend.
+const QUANTISED_MATMULS: [&str; 7] =
+    ["matmul_i8", "matmul_i4", "matmul_u8", "matmul_u4", "matmul_f8", "matmul_f8r", "matmul_f4"];
+
+/// Suffix for a node's `fused_op`, with the mapping of `activation_type` in src/backend/cpu/mod.rs:408-413.
+fn epilogue_suffix(fused_op: Option<&str>) -> &'static str {
+    match fused_op {
+        Some("MatMulAddRelu") | Some("OpRelu") => "_relu",
+        Some("MatMulAddGelu") | Some("OpGelu") => "_gelu",
+        Some("MatMulAddSilu") | Some("OpSilu") => "_silu",
+        _ => "",
+    }
+}
+
+/// Appends `_relu` / `_gelu` / `_silu` to every quantised MatMul whose graph node carries a fused activation.
+/// Instructions without a `node_id`, nodes that are gone and every other kernel are left as they are.
+fn tag_matmul_epilogues(plan: &mut ExecutablePlan, graph: &ComputeGraph) {
+    for ins in plan.instructions.iter_mut() {
+        if let Instruction::CallKernel { kernel_name, node_id: Some(id), .. } = ins {
+            if !QUANTISED_MATMULS.contains(&kernel_name.as_str()) {
+                continue;
+            }
+            let fused = graph.get_node(*id).and_then(|n| n.attrs.get("fused_op")).map(|s| s.as_str());
+            kernel_name.push_str(epilogue_suffix(fused));
+        }
+    }
+}
+
 impl Backend for HipBackend {
     type Buffer = HipBuffer;
 
@@ -239,8 +268,18 @@ impl Backend for HipBackend {
         HipBuffer { bytes: total_bytes }
     }
 
+    /// `CpuBackend::compile`, then the fused epilogue of every quantised MatMul is carried in its kernel name.
+    ///
+    /// The CPU lowering works out `activation_type` from the node's `fused_op` attribute but names a quantised MatMul
+    /// `matmul_i8` / `matmul_i4` / ... without it (src/backend/cpu/mod.rs:406-413, 427-495), so the instruction
+    /// alone does not say that a ReLU / GELU / SiLU was folded into the node (`MatMulAdd{Relu,Gelu,Silu}`: the bias
+    /// is the third input slice; `Op{Relu,Gelu,Silu}`: no bias).  Conv2d names already carry the tag
+    /// (`conv2d_i8_silu`, src/backend/cpu/mod.rs:856-865); this gives MatMul the same form, which is what
+    /// libfastnn_hip reads: `matmul_<type>[_relu|_gelu|_silu]`, bias = third slice when present.
     fn compile(&self, graph: &ComputeGraph, memory_plan: &MemoryPlan) -> Result<ExecutablePlan, BackendError> {
-        CpuBackend.compile(graph, memory_plan)
+        let mut plan = CpuBackend.compile(graph, memory_plan)?;
+        tag_matmul_epilogues(&mut plan, graph);
+        Ok(plan)
     }
 
     fn dispatch(&self, plan: &ExecutablePlan, _arena: &HipBuffer, shape_env: &ShapeEnv) -> Result<(), BackendError> {
@@ -291,11 +330,31 @@ impl Backend for HipBackend {
         arena: &HipBuffer,
         shape_env: &ShapeEnv,
     ) -> Result<Vec<ProfileEntry>, BackendError> {
-        let (native, _, _) = self.lowered(plan)?;
+        let (native, symbol_ptrs, symbol_names) = self.lowered(plan)?;
         let n = plan.instructions.len();
         let mut ns = vec![0u64; n.max(1)];
-        // SAFETY: `ns` holds at least `n` entries.
-        let st = unsafe { ffi::fnn_backend_dispatch_profile(self.raw, native, ns.as_mut_ptr(), n as u64) };
+        // the same bindings `dispatch` passes: symbolic dims are profiled under this call's environment
+        let mut names: Vec<*const c_char> = Vec::new();
+        let mut values: Vec<u64> = Vec::new();
+        for (ptr, name) in symbol_ptrs.iter().zip(symbol_names.iter()) {
+            if let Some(v) = shape_env.resolve(name) {
+                names.push(*ptr);
+                values.push(v);
+            }
+        }
+        // SAFETY: `ns` holds at least `n` entries; `names` / `values` hold `names.len()` entries each and the
+        // CStrings behind `names` live in the plan cache entry that `native` belongs to.
+        let st = unsafe {
+            ffi::fnn_backend_dispatch_profile_env(
+                self.raw,
+                native,
+                names.as_ptr(),
+                values.as_ptr(),
+                names.len() as u64,
+                ns.as_mut_ptr(),
+                n as u64,
+            )
+        };
         if st == ffi::FNN_ERR_UNSUPPORTED_OP {
             return default_profile(self, plan, arena, shape_env);
         }

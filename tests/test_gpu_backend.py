@@ -1045,3 +1045,129 @@ def test_random_matmul_chains_equal_with_and_without_plan_fusions(be, seed):
         assert np.array_equal(got[1], got[0]), (case, m, dims, dts)
         plan.close()
     assert engaged > 0
+
+
+@pytest.mark.parametrize("dt", [flib.DT_I8, flib.DT_F4])
+def test_three_input_matmul_without_a_suffix_adds_the_bias_and_nothing_else(be, orc, dt):
+    """`matmul_<type>` with a third input slice: the slice is the bias, no activation is applied (the epilogue is
+    named by the suffix alone, as for conv2d_*); the same three slices under `_relu` apply max(x, 0) on top."""
+    rng = np.random.default_rng(410 + dt)
+    m, k, n = 5, 192, 80
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    pw = fastnn_amd.quantize_weights(dt, _w(rng, n, k))
+    bias = rng.standard_normal(n).astype(np.float32)
+    a = Arena()
+    s_x, s_w, s_b, s_o, s_r = a.take(x.nbytes), a.take(pw.words.nbytes), a.take(bias.nbytes), a.take(m * n * 4), a.take(m * n * 4)
+    plan = ExecutablePlan(a.top).write_const(s_x[0], x).write_const(s_w[0], pw.words).write_const(s_b[0], bias)
+    plan.call_kernel(KERNEL_OF[dt], [s_x, s_w, s_b], s_o, [m, k, n], meta_of(pw))
+    plan.call_kernel(KERNEL_OF[dt] + "_relu", [s_x, s_w, s_b], s_r, [m, k, n], meta_of(pw))
+    be.allocate_arena(a.top)
+    be.dispatch(plan)
+    want = orc.qmatmul(to_oracle(orc, pw), x, bias=bias)
+    assert (want < 0).any()
+    got = be.read_arena(*s_o, np.float32).reshape(m, n)
+    assert_close(got, want, 2e-5, "bias, no activation")
+    assert np.array_equal(be.read_arena(*s_r, np.float32).reshape(m, n), np.maximum(got, 0.0))
+
+
+@pytest.mark.parametrize("act,code", [("Relu", flib.ACT_RELU), ("Silu", flib.ACT_SILU)])
+def test_matmul_add_activation_nodes_reach_the_library_as_one_tagged_instruction(orc, act, code):
+    """MatMul -> Add(bias) -> Relu|Silu through AotExecutor(quantize=8): the native plan (what fnn_plan_add_call_kernel
+    received) holds one `matmul_i8_<act>` CallKernel with three input slices, and its result is act(xW + b)."""
+    from fastnn_amd.aot import AotExecutor
+    rng = np.random.default_rng(77)
+    d, f, m = 96, 160, 6
+    nodes = [{"name": "fc", "op_type": "MatMul", "inputs": "[x, w]", "outputs": "[h0]"},
+             {"name": "b", "op_type": "Add", "inputs": "[h0, bias]", "outputs": "[h1]"},
+             {"name": "a", "op_type": act, "inputs": "[h1]", "outputs": "[y]"}]
+    params = {"w": (rng.standard_normal((d, f)) * 0.1).astype(np.float32), "bias": rng.standard_normal(f).astype(np.float32)}
+    x = rng.standard_normal((m, d)).astype(np.float32)
+    ex = AotExecutor(nodes, params, ["x"], ["y"], {"x": [m, d]}, quantize=8)
+    try:
+        y = ex.forward({"x": x})["y"]
+        calls = [ex._plan.describe(i) for i in range(len(ex._plan))]
+        calls = [c for c in calls if c["op"] == "CallKernel"]
+        assert len(calls) == 1
+        assert calls[0]["kernel"] == "matmul_i8_" + act.lower()
+        assert len(calls[0]["inputs"]) == 3 and calls[0]["params"] == [m, d, f]
+    finally:
+        ex.close()
+    pw = fastnn_amd.quantize_weights(flib.DT_I8, np.ascontiguousarray(params["w"].T))
+    want = orc.qmatmul(to_oracle(orc, pw), x, bias=params["bias"], act=code)
+    assert_close(y, want, 2e-5, "act(xW + b)")
+
+
+def test_plan_fusions_engage_when_param_dims_are_all_known(be, orc):
+    """CpuBackend::compile gives every MatMul `param_dims: Some([m, k, n])`, all `Known` for a static graph
+    (src/backend/cpu/mod.rs:601-613): such a plan must fuse the residual Add and hand prepared operands on exactly
+    like the same plan without param_dims, with a byte-identical arena."""
+    rng = np.random.default_rng(141)
+    m, d, f = 64, 512, 2048
+    x = rng.standard_normal((m, d)).astype(np.float32)
+    w1 = fastnn_amd.quantize_weights(flib.DT_F8, _w(rng, f, d))
+    w2 = fastnn_amd.quantize_weights(flib.DT_F4, _w(rng, d, f))
+    w3 = fastnn_amd.quantize_weights(flib.DT_F8, _w(rng, f, d))
+    arenas = {}
+    for dims in (False, True):
+        a = Arena()
+        s_x = a.take(x.nbytes)
+        s_w = [a.take(w.words.nbytes) for w in (w1, w2, w3)]
+        s_h, s_y, s_s, s_h2 = a.take(m * f * 4), a.take(m * d * 4), a.take(m * d * 4), a.take(m * f * 4)
+        plan = ExecutablePlan(a.top)
+        for s, w in zip(s_w, (w1, w2, w3)):
+            plan.write_const(s[0], w.words)
+        plan.call_kernel("matmul_f8_gelu", [s_x, s_w[0]], s_h, [m, d, f], meta_of(w1))
+        plan.call_kernel("matmul_f4", [s_h, s_w[1]], s_y, [m, f, d], meta_of(w2))
+        plan.call_kernel("add_f32", [s_y, s_x], s_s, [m * d])
+        plan.call_kernel("matmul_f8", [s_s, s_w[2]], s_h2, [m, d, f], meta_of(w3))
+        if dims:
+            plan.set_param_dims(3, [m, d, f]).set_param_dims(4, [m, f, d]).set_param_dims(6, [m, d, f])
+        be.allocate_arena(a.top)
+        be.write_arena(s_x[0], x)
+        be.dispatch(plan)
+        be.dispatch(plan)
+        assert plan.residuals_fused == 1, dims
+        assert plan.operands_handed == 2, dims
+        arenas[dims] = be.read_arena(0, a.top).copy()
+    assert np.array_equal(arenas[False], arenas[True])
+    h = arenas[True][s_h[0]:s_h[0] + s_h[1]].view(np.float32).reshape(m, f)
+    assert_close(h, orc.qmatmul(to_oracle(orc, w1), x, act=flib.ACT_GELU), 2e-5, "first layer")
+    # a symbolic M keeps every instruction on its own
+    plan.set_param_dims(4, [("T", m), f, d])
+    be.dispatch(plan)
+    assert plan.residuals_fused == 0
+    assert np.array_equal(be.read_arena(0, a.top), arenas[True])
+
+
+def test_dispatch_profile_runs_under_the_shape_environment_it_is_given(be, orc):
+    """Backend::dispatch_profile resolves symbolic dims with the ShapeEnv of the call (src/backend/mod.rs:178-211), not
+    with whatever an earlier dispatch left behind; without bindings a Bounded dim takes its maximum."""
+    rng = np.random.default_rng(93)
+    k, n = 64, 24
+    pw = fastnn_amd.quantize_weights(flib.DT_F8, _w(rng, n, k))
+    x = rng.standard_normal((4, k)).astype(np.float32)
+    a = Arena()
+    s_x, s_w, s_o = a.take(x.nbytes), a.take(pw.words.nbytes), a.take(4 * n * 4)
+    plan = ExecutablePlan(a.top).write_const(s_x[0], x).write_const(s_w[0], pw.words)
+    plan.call_kernel("matmul_f8", [s_x, s_w], s_o, [1, k, n], meta_of(pw))
+    plan.set_param_dims(2, [("T", 4), k, n])
+    be.allocate_arena(a.top)
+    want = orc.qmatmul(to_oracle(orc, pw), x)
+    be.dispatch(plan, {"T": 2})
+    for rows in (3, 1):
+        be.write_arena(s_o[0], np.zeros(4 * n, np.float32))
+        times = be.dispatch_profile(plan, {"T": rows})
+        assert len(times) == 3 and times[2] > 0
+        got = be.read_arena(*s_o, np.float32).reshape(4, n)
+        assert_close(got[:rows], want[:rows], 2e-5, f"T = {rows}")
+        assert not got[rows:].any()
+    be.write_arena(s_o[0], np.zeros(4 * n, np.float32))
+    be.dispatch_profile(plan)                          # no environment: the bound, not the previous call's T = 1
+    assert_close(be.read_arena(*s_o, np.float32).reshape(4, n), want, 2e-5, "Bounded -> max")
+    sym = ExecutablePlan(a.top).write_const(s_x[0], x).write_const(s_w[0], pw.words)
+    sym.call_kernel("matmul_f8", [s_x, s_w], s_o, [1, k, n], meta_of(pw))
+    sym.set_param_dims(2, ["T", k, n])
+    be.dispatch(sym, {"T": 2})
+    with pytest.raises(flib.FnnError) as e:
+        be.dispatch_profile(sym)
+    assert "DimExpr::Symbol 'T' is not bound" in e.value.message

@@ -110,19 +110,30 @@ def test_every_yolo_layer_shape_at_batch_1(ctx, orc):
         _conv_case(ctx, orc, rng, 1, c, h, oc, k, s)
 
 
-@pytest.mark.parametrize("c,h,oc,k,s", [(3, 640, 16, 3, 2), (16, 320, 32, 3, 2), (64, 40, 64, 3, 1), (128, 40, 128, 3, 2),
-                                       (384, 20, 256, 1, 1)])
-def test_yolo_layer_shapes_at_batch_16(ctx, orc, c, h, oc, k, s):
-    """Batch 16 (every image has its own activation range): the first two layers (most rows), a 3x3 at K = 576,
-    the K = 1152 stride-2 layer and a C2f 1x1."""
-    _conv_case(ctx, orc, np.random.default_rng(51 + c), 16, c, h, oc, k, s)
+def _distinct_yolo_shapes():
+    seen, out = set(), []
+    for shp in bench.yolo_convs():
+        if shp not in seen:
+            seen.add(shp)
+            out.append(shp)
+    return out
 
 
-def _check_graph_against_oracle(orc, nodes, params, ex, x, tag):
+@pytest.mark.parametrize("c,h,oc,k,s", _distinct_yolo_shapes())
+def test_every_yolo_layer_shape_at_batch_16(ctx, orc, c, h, oc, k, s):
+    """Every distinct convolution shape of the 640x640 network at batch 16 (every image has its own activation
+    range; pixel tiles straddle images from the 40x40 maps down): i32 accumulators bit-exact for all 16 images,
+    outputs within 1e-5."""
+    _conv_case(ctx, orc, np.random.default_rng(51 + c + h + oc + k + s), 16, c, h, oc, k, s)
+
+
+def _check_graph_against_oracle(orc, nodes, params, ex, x, tag, images=None):
     """Every node of the graph against the oracle, each on the device's own value of its inputs (one arena slot
     per value, so every intermediate value can be read after the forward).  Convolutions: 1e-5; data movement
-    and the residual add: bit for bit."""
+    and the residual add: bit for bit.  images: the images of the batch the convolutions are checked on (every
+    node treats the images of a batch independently; None = all), the other nodes are always checked whole."""
     vals = {"x": x}
+    sel = slice(None) if images is None else list(images)
 
     def dev(name):
         if name not in vals:
@@ -143,9 +154,9 @@ def _check_graph_against_oracle(orc, nodes, params, ex, x, tag):
             assert nxt["op_type"] == "Silu" and _names(nxt["inputs"]) == o
             skip.add(i + 1)
             pw = to_oracle(orc, fastnn_amd.quantize_weights(flib.DT_I8, w.reshape(oc, ic * kh * kw)))
-            want = orc.qconv2d_i8(dev(ins[0]), pw, kh, kw, int(nd["strides"]), int(nd["pads"]), 1, 1, bias=params[ins[2]],
-                                  act=flib.ACT_SILU)
-            assert_close(dev(_names(nxt["outputs"])[0]), want, 1e-5, f"{tag}: conv node {nd['name']} {w.shape}")
+            want = orc.qconv2d_i8(np.ascontiguousarray(dev(ins[0])[sel]), pw, kh, kw, int(nd["strides"]), int(nd["pads"]), 1, 1,
+                                  bias=params[ins[2]], act=flib.ACT_SILU)
+            assert_close(dev(_names(nxt["outputs"])[0])[sel], want, 1e-5, f"{tag}: conv node {nd['name']} {w.shape}")
             n_conv += 1
         elif op == "Split":
             a = dev(ins[0])
@@ -165,21 +176,53 @@ def _check_graph_against_oracle(orc, nodes, params, ex, x, tag):
     return n_conv
 
 
-@pytest.mark.parametrize("batch,size", [(1, 640), (2, 96)])
+def _activation_codes(v, padded):
+    """int8 codes the quantised convolution gives its input, image by image: the range of the im2col matrix (the
+    tensor, plus 0 where a tap can fall into the padding), sa = range / 255 (1 when empty), za = min + 128 sa,
+    q = clamp(round((x - za) * (1 / sa)), -128, 127) with ties away from zero, all in f32
+    (src/backend/cpu/packed_conv.rs:149-156, 199-201; src/backend/cpu/im2col.rs:496-507)."""
+    v = np.asarray(v, np.float32)
+    out = np.empty(v.shape, np.int16)
+    for i in range(v.shape[0]):
+        mn, mx = np.float32(v[i].min()), np.float32(v[i].max())
+        if padded:
+            mn, mx = min(mn, np.float32(0)), max(mx, np.float32(0))
+        rng_ = np.float32(mx - mn)
+        sa = np.float32(rng_ / np.float32(255)) if rng_ > 0 else np.float32(1)
+        za = np.float32(mn + np.float32(128) * sa) if rng_ > 0 else np.float32(0)
+        t = ((v[i] - za) * np.float32(np.float32(1) / sa)).astype(np.float32)
+        q = np.sign(t) * np.floor(np.abs(t) + np.float32(0.5))
+        out[i] = np.clip(q, -128, 127).astype(np.int16)
+    return out
+
+
+@pytest.mark.parametrize("batch,size", [(1, 640), (2, 96), (16, 640)])
 def test_yolo_graph_node_by_node_against_oracle(orc, batch, size):
     """The backbone + neck as one resident plan (HIP-graph replay on the second forward) at the benchmark's
-    640x640, batch 1, and a small two-image case: every node against the oracle, then the three outputs against
-    the oracle chained from the input.  The node-by-node comparison (each conv against the oracle on the very
-    input the device saw, 1e-5) is the parity statement.  The chained comparison only guards against gross
-    divergence and carries a loose bound (max 1e-1, mean 1e-2 of max|ref|): a network of 8-bit activation
-    quantisers is not continuous in its input.  An activation within 1e-5 of a rounding boundary of the next
-    layer's quantiser may land on the other side, that moves the value by one quantisation step (0.8 % of the
-    layer's range), and downstream layers see a perturbation of that size, not of 1e-5; more than twenty quantised
-    layers follow one another, so the outputs of two correct implementations differ by the network's own
-    quantisation noise."""
+    640x640 with batch 1 and batch 16, and a small two-image case.  The batch-16 plan is another instruction stream
+    (Slice copies for Split, 44 convolutions taking their ranges from the producer, tiles holding pixels of two
+    images); there the convolutions are checked on images 0, 7 and 15 and every other node on the whole batch.
+
+    Parity statement: every node against the oracle on the very input the device saw (convolutions 1e-5, data
+    movement and Add bit for bit).
+
+    Chained statement: the oracle is also run from the input on its own, and for every convolution the int8 codes
+    that the activation quantiser gives the device's input tensor are compared with the codes it gives the
+    chained oracle's.  A network of 8-bit activation quantisers is not continuous: an activation within 1e-5 of
+    a rounding boundary may land on the other side, which moves that code by one step.  While such flips are the
+    only difference, codes differ by exactly one step in a few positions per hundred thousand: that is required of
+    the first six convolutions (every difference +-1, at most 0.2 % of a layer's codes).  Further down the flips
+    compound: a moved code moves the next layer's sums, a moved minimum or maximum moves that image's scale and
+    zero point and with them half of its codes by a step, and this random-weight network amplifies a perturbation
+    from layer to layer (measured at 640x640: 3e-5 of the codes after three layers, 2 % after ten, about half from
+    the fifteenth on, largest difference 5 steps of 255).  No implementation-independent bound tighter than a few
+    steps exists there, so the deep layers carry a guard against gross divergence only (at most 12 steps, outputs
+    within 1e-1 of max|ref| and 1e-2 on average); what pins them is the node-by-node statement above."""
     rng = np.random.default_rng(5)
     nodes, params, shape, outs = bench.yolo_graph(batch, rng, size=size)
     x = rng.uniform(0, 1, shape).astype(np.float32)
+    images = None if batch <= 2 else [0, 7, 15]
+    sel = slice(None) if images is None else images
     ex = AotExecutor(nodes, params, ["x"], outs, {"x": shape}, quantize=8)
     try:
         first = ex.forward({"x": x})
@@ -187,10 +230,11 @@ def test_yolo_graph_node_by_node_against_oracle(orc, batch, size):
         assert ex.replayed
         for name in outs:
             assert np.array_equal(first[name], got[name]), name + ": replay differs from the first dispatch"
-        assert _check_graph_against_oracle(orc, nodes, params, ex, x, f"B={batch} {size}px") == 45
-        # chained oracle from the input
-        vals = {"x": x}
+        assert _check_graph_against_oracle(orc, nodes, params, ex, x, f"B={batch} {size}px", images) == 45
+        # chained oracle from the input (on the sampled images: every node treats images independently)
+        vals = {"x": np.ascontiguousarray(x[sel])}
         skip = set()
+        worst_step, report = 0, []
         for i, nd in enumerate(nodes):
             if i in skip:
                 continue
@@ -200,6 +244,13 @@ def test_yolo_graph_node_by_node_against_oracle(orc, batch, size):
                 w = params[ins[1]]
                 oc, ic, kh, kw = w.shape
                 skip.add(i + 1)
+                dev_in = x if ins[0] == "x" else ex.read_output(ins[0])
+                qd = _activation_codes(dev_in[sel], int(nd["pads"]) > 0)
+                qo = _activation_codes(vals[ins[0]], int(nd["pads"]) > 0)
+                diff = np.abs(qd - qo)
+                share, step = float((diff != 0).mean()), int(diff.max())
+                report.append((nd["name"], round(share, 5), step))
+                worst_step = max(worst_step, step)
                 pw = to_oracle(orc, fastnn_amd.quantize_weights(flib.DT_I8, w.reshape(oc, ic * kh * kw)))
                 vals[_names(nodes[i + 1]["outputs"])[0]] = orc.qconv2d_i8(vals[ins[0]], pw, kh, kw, int(nd["strides"]),
                                                                            int(nd["pads"]), 1, 1, bias=params[ins[2]],
@@ -216,13 +267,16 @@ def test_yolo_graph_node_by_node_against_oracle(orc, batch, size):
                 vals[o[0]] = orc.maxpool2d(vals[ins[0]], 5, 1, 2)
             elif op == "Resize":
                 vals[o[0]] = orc.upsample_nearest2d(vals[ins[0]], 2, 2)
+        print("chained oracle, per convolution (name, share of differing input codes, largest difference):", report, flush=True)
+        assert all(step <= 1 and share <= 2e-3 for _, share, step in report[:6]), report
+        assert worst_step <= 12, report
         stats = {}
         for name in outs:
-            assert got[name].shape == vals[name].shape
-            d = np.abs(got[name].astype(np.float64) - vals[name])
+            assert got[name][sel].shape == vals[name].shape
+            d = np.abs(got[name][sel].astype(np.float64) - vals[name])
             mx = np.abs(vals[name]).max()
             stats[name] = (d.max() / mx, d.mean() / mx)
-        print("chained oracle, (max, mean) of |diff| / max|ref|:", stats, flush=True)
+        print("chained oracle, (max, mean) of |diff| / max|ref| of the outputs:", stats, flush=True)
         assert all(a <= 1e-1 and b <= 1e-2 for a, b in stats.values()), stats
     finally:
         ex.close()
