@@ -38,6 +38,8 @@ WORKLOADS = {
     "c3_i4cb": ("i4cb", 4096, 4096, False, "none"),
     "c4_f8_up": ("f8", 2048, 8192, False, "gelu"),
     "c4_f4_up": ("f4", 2048, 8192, False, "gelu"),
+    "c4_f8_down": ("f8", 8192, 2048, False, "none"),
+    "c4_f4_down": ("f4", 8192, 2048, False, "none"),
     "i4_4096": ("i4", 4096, 4096, False, "none"),
     "f8_4096": ("f8", 4096, 4096, False, "none"),
 }

@@ -54,6 +54,7 @@ struct fnn_hip_ctx {
     Staging st_a, st_out, st_bias, st_acc, st_tmp, st_tmp2, st_tmp3, st_tmp4, st_col, st_rows;
     int64_t options[FNN_OPT_COUNT];
     float *scratch = nullptr;  // small reduction scratch (partials)
+    uint32_t *stream_counters = nullptr;   // arrival counters of the streaming MatMul's column tiles (zero between launches)
     bool capturing = false;
     uint64_t ws_epoch = 0;     // bumped whenever a staging buffer is re-allocated (captured graphs go stale)
     unsigned char *static_ws = nullptr;   // this device's copy of the library's static workspace
@@ -141,6 +142,9 @@ const OptionSpec kOptions[FNN_OPT_COUNT] = {
     {0, 0, 2},        // FNN_OPT_CONV_IMPLICIT
     {1, 0, 1},        // FNN_OPT_FUSE_RESIDUAL
     {1, 0, 1},        // FNN_OPT_FUSE_PREP
+    {17, 1, 32},      // FNN_OPT_STREAM_MIN_M
+    {32, 0, 32},      // FNN_OPT_STREAM_MAX_M
+    {0, 0, 0xffff},   // FNN_OPT_STREAM_SHAPE
 };
 
 #define HIP_TRY(ctx, code, expr)                                                              \
@@ -239,6 +243,8 @@ int fnn_hip_create(int device, fnn_hip_ctx **out)
             (e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking)) != hipSuccess ||
             (e = hipEventCreate(&ctx->ev0)) != hipSuccess || (e = hipEventCreate(&ctx->ev1)) != hipSuccess ||
             (e = hipMalloc((void **)&ctx->scratch, 64 * 1024)) != hipSuccess ||
+            (e = hipMalloc((void **)&ctx->stream_counters, FNN_STREAM_COUNTERS * 4)) != hipSuccess ||
+            (e = hipMemsetAsync(ctx->stream_counters, 0, FNN_STREAM_COUNTERS * 4, ctx->stream)) != hipSuccess ||
         (e = static_workspace_of(device, &ctx->static_ws)) != hipSuccess) {
             int rc = fail(nullptr, FNN_ERR_MEMORY, "fnn_hip_create: %s", hipGetErrorString(e));
             fnn_hip_destroy(ctx);
@@ -258,6 +264,7 @@ void fnn_hip_destroy(fnn_hip_ctx *ctx)
     for (Staging *s : {&ctx->st_a, &ctx->st_out, &ctx->st_bias, &ctx->st_acc, &ctx->st_tmp, &ctx->st_tmp2, &ctx->st_tmp3, &ctx->st_tmp4, &ctx->st_col, &ctx->st_rows})
         if (s->ptr) (void)hipFree(s->ptr);
     if (ctx->scratch) (void)hipFree(ctx->scratch);
+    if (ctx->stream_counters) (void)hipFree(ctx->stream_counters);
     if (ctx->ev0) (void)hipEventDestroy(ctx->ev0);
     if (ctx->ev1) (void)hipEventDestroy(ctx->ev1);
     if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
@@ -570,6 +577,10 @@ int fnn_hip_qmatmul(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *a, i
             }
             if (!handled) {
                 int rc = fnn_mfma_rows16(ctx, ctx->stream, w, p, flags, &handled);
+                if (rc) return rc;
+            }
+            if (!handled) {
+                int rc = fnn_stream_qmatmul(ctx, ctx->stream, w, p, flags, &handled);
                 if (rc) return rc;
             }
             if (!handled) {
@@ -1148,6 +1159,7 @@ bool fnn_ctx_no_alloc(fnn_hip_ctx *ctx) { return ctx->capturing || ctx->static_m
 int fnn_ctx_fail(fnn_hip_ctx *ctx, int code, const char *msg) { return fail(ctx, code, "%s", msg); }
 
 int64_t fnn_ctx_option(const fnn_hip_ctx *ctx, int option) { return ctx->options[option]; }
+uint32_t *fnn_ctx_stream_counters(fnn_hip_ctx *ctx) { return ctx->stream_counters; }
 FnnRangeIo *fnn_ctx_range_io(fnn_hip_ctx *ctx) { return &ctx->range; }
 FnnResidualIo *fnn_ctx_residual_io(fnn_hip_ctx *ctx) { return &ctx->residual; }
 FnnPrepIo *fnn_ctx_prep_io(fnn_hip_ctx *ctx) { return &ctx->prep; }

@@ -31,6 +31,12 @@ inline hipError_t fnn_raise_lds_limit(std::atomic<uint64_t> &done, const void *k
 
 // M >= 5: activations prepared once as f16 operands, 4-wave output tiles with the
 // activations staged through LDS and optional split of K (deterministic reduction).
+// 17 <= M <= 32: one launch, weights streamed into the MFMA operand registers, activations converted in the kernel,
+// K split over workgroups and reduced by the last one to arrive (qgemm_stream.hip)
+int fnn_stream_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &p, int flags, bool *handled);
+// arrival counters of that kernel's column tiles: FNN_STREAM_COUNTERS words of device memory, zero between launches
+constexpr int FNN_STREAM_COUNTERS = 4096;
+uint32_t *fnn_ctx_stream_counters(fnn_hip_ctx *ctx);
 // int8 matrix-core GEMM over exact activation digit planes (qgemm_digits.hip): M >= 17, I8 / I4 / U4 weights
 int fnn_digits_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &p, int flags, bool *handled);
 int fnn_tiled_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &p,

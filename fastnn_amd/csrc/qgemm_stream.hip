@@ -1,0 +1,95 @@
+// Host side of the one-launch streaming MatMul for up to 32 activation rows (kernels: qgemm_stream_impl.h, one
+// translation unit per weight type): which calls it takes, the shape of the launch, the split-K workspace.
+#include "mfma.h"
+#include "qgemm_stream.h"
+#include "range_io.h"
+
+namespace {
+
+// RT, KR, splits and rounds from FNN_OPT_STREAM_SHAPE or by rule (MB follows from M).  The phases of a round (requests,
+// conversion, matrix cores) follow one another inside a workgroup, so a workgroup does one round where it can: one row
+// tile per wave, K / KR splits, and KR = 512 while that still gives the 256 CUs a workgroup each.
+bool plan_stream(int bits, bool int8, int64_t m, int64_t n, int64_t k, int64_t forced, StreamPlan *out)
+{
+    const int mb = (int)((m + 15) / 16);
+    if (mb < 1 || mb > 2) return false;   // (three and four blocks measured slower than the tiled path)
+    int rt = 1, kr = 512;
+    const int64_t nt1 = (n + FNN_STREAM_NW * 16 - 1) / (FNN_STREAM_NW * 16);
+    if (nt1 * ((k + 511) / 512) < 224) kr = 256;
+    int64_t splits = 0;
+    if (forced > 0) {
+        rt = (int)((forced >> 4) & 15);
+        kr = (int)(forced & 15) * 256;
+        splits = forced >> 8;
+        if (rt < 1 || rt > 2 || (kr != 256 && kr != 512)) return false;
+    }
+    if (mb * rt > (int8 ? 4 : 8)) return false;   // accumulator tiles that fit the registers
+    const int64_t kr_total = (k + kr - 1) / kr;   // rounds over all of K
+    if (splits == 0) splits = kr_total > 64 ? 64 : kr_total;
+    if (splits > kr_total || splits > 64) return false;
+    const int64_t rounds = (kr_total + splits - 1) / splits;
+    if ((splits - 1) * rounds >= kr_total) return false;   // an empty split
+    const int64_t ntiles = (n + FNN_STREAM_NW * rt * 16 - 1) / (FNN_STREAM_NW * rt * 16);
+    // By rule the kernel takes a call only where it measured faster than preparation + tiles + reduction as three
+    // launches: no more workgroups than the chip holds at once (a second wave of
+    // workgroups repeats every phase).  4096 x 4096 at M = 32: 14.4 against 17.9 us; 2048 -> 8192 FP8: 13.3 against 17.4;
+    // 4096 x 11008 (688 workgroups): 25.0 against 23.5; M = 64 on 4096 x 4096: 21.3 against 20.0.
+    if (forced == 0 && ntiles * splits > 320) return false;
+    *out = StreamPlan{mb, rt, kr, (int)splits, (int)rounds, (int)ntiles};
+    return true;
+}
+
+}  // namespace
+
+int fnn_stream_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &q, int flags, bool *handled)
+{
+    *handled = false;
+    const int64_t lo = fnn_ctx_option(ctx, FNN_OPT_STREAM_MIN_M), hi = fnn_ctx_option(ctx, FNN_OPT_STREAM_MAX_M);
+    if (q.m < lo || q.m > hi || q.m > 32 || q.n < 1) return FNN_OK;
+    if (flags & FNN_FLAG_ACT_F16_SINGLE) return FNN_OK;
+    const int dt = w->dtype;
+    const bool int_type = dt == FNN_DT_I8 || dt == FNN_DT_I4 || dt == FNN_DT_U4;
+    if (dt == FNN_DT_I4CB) return FNN_OK;
+    if (int_type && fnn_ctx_option(ctx, FNN_OPT_GEMM_INT8) == 0) return FNN_OK;
+    if (q.kp % 4 != 0 || q.k % 8 != 0 || q.k < 8) return FNN_OK;
+    // the f16 types multiply whatever bytes a lane load holds: every load must lie wholly inside or wholly past K
+    if (!int_type && q.k % (dt == FNN_DT_F4 ? 128 : 64) != 0) return FNN_OK;
+    if ((reinterpret_cast<uintptr_t>(q.a) & 15) || (reinterpret_cast<uintptr_t>(q.words) & 15)) return FNN_OK;
+    // 32-bit buffer offsets: a column tile of 256 rows, the activation block
+    if (q.kp * 4 * 256 >= (int64_t)1 << 31 || q.m * q.k * 4 >= (int64_t)0xFFFFFF00 || q.k >= (int64_t)1 << 28) return FNN_OK;
+    StreamPlan pl;
+    const int64_t forced = fnn_ctx_option(ctx, FNN_OPT_STREAM_SHAPE);
+    const int bits = (dt == FNN_DT_I4 || dt == FNN_DT_U4 || dt == FNN_DT_F4) ? 4 : 8;
+    if (!plan_stream(bits, int_type, q.m, q.n, q.k, forced, &pl)) return FNN_OK;
+    if (pl.ntiles > FNN_STREAM_COUNTERS) return FNN_OK;
+    StreamArgs p;
+    p.words = q.words; p.scales = q.scales; p.zeros = q.zeros; p.a = q.a; p.bias = q.bias; p.out = q.out;
+    p.residual = nullptr; p.sum_out = nullptr;
+    p.part = nullptr; p.count = fnn_ctx_stream_counters(ctx);
+    p.m = q.m; p.n = q.n; p.k = q.k; p.kp = q.kp;
+    p.act = q.act; p.splits = pl.splits; p.rounds = pl.rounds; p.ntiles = pl.ntiles;
+    if (pl.splits > 1) {
+        const size_t wgf = (size_t)pl.mb * pl.rt * 4 * FNN_STREAM_NW * 64 + 16 * pl.mb;
+        void *ws = nullptr;
+        int rc = fnn_ctx_ensure_tmp(ctx, 1, (size_t)pl.splits * pl.ntiles * wgf * 4, &ws);
+        if (rc) return rc;
+        p.part = (float *)ws;
+    }
+    if (FnnResidualIo *res = fnn_ctx_residual_io(ctx); res->residual && res->of_out == q.out && res->elems == (uint64_t)(q.m * q.n)) {
+        p.residual = res->residual; p.sum_out = res->sum_out;
+        res->used = 1;
+    }
+    hipError_t e;
+    switch (dt) {
+    case FNN_DT_I8: e = fnn_stream_launch_i8(pl, p, s); break;
+    case FNN_DT_I4: e = fnn_stream_launch_i4(pl, p, s); break;
+    case FNN_DT_U4: e = fnn_stream_launch_u4(pl, p, s); break;
+    case FNN_DT_U8: e = fnn_stream_launch_u8(pl, p, s); break;
+    case FNN_DT_F8: e = fnn_stream_launch_f8(pl, p, s); break;
+    case FNN_DT_F8R: e = fnn_stream_launch_f8r(pl, p, s); break;
+    default: e = fnn_stream_launch_f4(pl, p, s); break;
+    }
+    if (e != hipSuccess) return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, hipGetErrorString(e));
+    *handled = true;
+    return FNN_OK;
+}

@@ -1,0 +1,4 @@
+// One-launch streaming MatMul, I8 weights (kernels: qgemm_stream_impl.h).
+#include "qgemm_stream_impl.h"
+
+hipError_t fnn_stream_launch_i8(const StreamPlan &pl, const StreamArgs &p, hipStream_t s) { return launch_dt<FNN_DT_I8>(pl, p, s); }

@@ -40,6 +40,9 @@ OPT_CONV_RANGES = 15
 OPT_CONV_IMPLICIT = 16
 OPT_FUSE_RESIDUAL = 17
 OPT_FUSE_PREP = 18
+OPT_STREAM_MIN_M = 19
+OPT_STREAM_MAX_M = 20
+OPT_STREAM_SHAPE = 21
 
 STATUS_NAMES = {0: "Ok", 1: "Dispatch", 2: "Memory", 3: "UnsupportedOp", 4: "Compilation"}
 

@@ -126,7 +126,13 @@ enum {
     FNN_OPT_FUSE_PREP = 18,       /* plans: 1 (default) = a MatMul at 17 <= M whose result the next instruction multiplies (f16    */
                                   /* matrix-core weight types) leaves that MatMul's prepared activation operand behind, which  */
                                   /* then skips its own preparation launch (same conversion code, identical results); 0 = off  */
-    FNN_OPT_COUNT = 19
+    FNN_OPT_STREAM_MIN_M = 19,    /* smallest and largest M of the one-launch streaming MatMul (weights straight into the      */
+    FNN_OPT_STREAM_MAX_M = 20,    /* matrix-core operand registers, activations converted in the kernel, K split reduced by the  */
+                                  /* last workgroup to arrive): defaults 17 and 32, 1..32; MAX_M = 0 switches it off.  By rule   */
+                                  /* it declines shapes with more column tiles x K splits than the chip holds at once            */
+    FNN_OPT_STREAM_SHAPE = 21,    /* its launch shape: 0 (default) = by rule, else (splits << 8) | (row tiles per wave << 4) |   */
+                                  /* (k-values per round / 256), splits = 0 meaning one round per workgroup                      */
+    FNN_OPT_COUNT = 22
 };
 int fnn_hip_set_option(fnn_hip_ctx *ctx, int option, int64_t value);
 int fnn_hip_get_option(fnn_hip_ctx *ctx, int option, int64_t *value);

@@ -233,6 +233,7 @@ def test_int8_digit_plane_gemm(ctx, orc, dt, m, k, n):
     bias = (rng.standard_normal(n) * 0.01).astype(np.float32)
     h = ctx.register(pw)
     want = orc.qmatmul(to_oracle(orc, pw), a, order=2, bias=bias, act=2)
+    ctx.set_option(flib.OPT_STREAM_MAX_M, 0)             # (M <= 32 would go to the one-launch kernel, tested on its own)
     got = ctx.qmatmul(h, a, n, bias=bias, act=2)
     int8_default = not (dt == 0 and m >= 768)            # 8-bit weights at four planes: the f16 tiles take M >= 768
     assert_close(got, want, 4e-6 if int8_default else TOL_F32, f"digit gemm {NAMES[dt]} {m}x{k}x{n}")
@@ -253,7 +254,83 @@ def test_int8_digit_plane_gemm(ctx, orc, dt, m, k, n):
         ctx.set_option(flib.OPT_TILE_SHAPE, -1)
         ctx.set_option(flib.OPT_TILE_SPLIT, 0)
         ctx.set_option(flib.OPT_GEMM_INT8, 1)
+        ctx.set_option(flib.OPT_STREAM_MAX_M, 32)
     ctx.release(h)
+
+
+# one-launch streaming kernel: one and two activation blocks, ragged N and K (K % 512 != 0, K < 256), wide N (several
+# column tiles), long K (many splits), a single k chunk
+STREAM_SHAPES = [(17, 4096, 1100), (32, 2048, 4100), (24, 520, 300), (31, 8192, 136), (20, 64, 40), (32, 1160, 4096), (9, 4096, 520),
+                 (16, 2048, 2048)]
+# (splits << 8) | (row tiles per wave << 4) | (k per round / 256); 0 = by rule
+STREAM_FORMS = [0, 0x11, 0x12, 0x21, 0x22, 0x112, 0x211, 0x322, 0x512]
+
+
+@pytest.mark.parametrize("dt", [0, 1, 2, 3, 4, 5, 6])
+@pytest.mark.parametrize("m,k,n", STREAM_SHAPES)
+def test_streaming_matmul_kernel(ctx, orc, dt, m, k, n):
+    """17 <= M <= 32 (9 <= M by option) in one launch: weights straight into the matrix-core operand registers,
+    activations converted in the kernel (three exact digit planes of rint(x 2^-e), |v| < 2^22 per row and round, for
+    I8 / I4 / U4 weights; f16 hi + lo for U8 / F8 / F8R / F4), K split over workgroups and added in split order by the
+    last one to arrive.  Every launch form gives the oracle's result within 2e-5 of max|ref| (rows with a 200x dynamic
+    range, an all-zero row, bias + SiLU), a given form gives the same bits on every call, and a call that the rule
+    declines (K % 64 != 0 for the f16 types, too many workgroups) still comes out right through the other kernels."""
+    rng = np.random.default_rng(5100 + dt * 7 + m + k)
+    pw = fastnn_amd.quantize_weights(dt, _weights(rng, n, k))
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    a[:, ::89] *= 200.0
+    a[m // 2] = 0.0
+    bias = (rng.standard_normal(n) * 0.01).astype(np.float32)
+    h = ctx.register(pw)
+    want = orc.qmatmul(to_oracle(orc, pw), a, order=2, bias=bias, act=3)
+    try:
+        ctx.set_option(flib.OPT_STREAM_MIN_M, 9)
+        ctx.set_option(flib.OPT_ROWS16_MIN_M, 17)
+        for form in STREAM_FORMS:
+            ctx.set_option(flib.OPT_STREAM_SHAPE, form)
+            got = ctx.qmatmul(h, a, n, bias=bias, act=3)
+            assert_close(got, want, TOL_F32, f"stream {NAMES[dt]} {m}x{k}x{n} form {form:#x}")
+            again = ctx.qmatmul(h, a, n, bias=bias, act=3)
+            assert np.array_equal(got, again), f"form {form:#x}: two calls differ"
+    finally:
+        ctx.set_option(flib.OPT_STREAM_SHAPE, 0)
+        ctx.set_option(flib.OPT_STREAM_MIN_M, 17)
+        ctx.set_option(flib.OPT_ROWS16_MIN_M, 9)
+    ctx.release(h)
+
+
+def test_streaming_matmul_takes_the_default_route_and_propagates_non_finite_rows(ctx, orc):
+    """By default M = 17..32 on a shape the rule accepts runs in the streaming kernel: its result differs in the last
+    bits from the digit-plane / tiled path's (another summation), both within bounds.  A row holding a NaN or an
+    infinity gives a NaN row with integer weights (the digits cannot carry it; the float path gives NaN or inf) and
+    non-finite values with float weights; the other rows are untouched."""
+    rng = np.random.default_rng(5200)
+    m, k, n = 32, 2048, 1024
+    for dt in (flib.DT_I8, flib.DT_F8):
+        pw = fastnn_amd.quantize_weights(dt, _weights(rng, n, k))
+        a = rng.standard_normal((m, k)).astype(np.float32)
+        h = ctx.register(pw)
+        want = orc.qmatmul(to_oracle(orc, pw), a, order=2)
+        clean = ctx.qmatmul(h, a, n)
+        ctx.set_option(flib.OPT_STREAM_MAX_M, 0)
+        try:
+            other = ctx.qmatmul(h, a, n)
+        finally:
+            ctx.set_option(flib.OPT_STREAM_MAX_M, 32)
+        assert_close(clean, want, TOL_F32)
+        assert_close(other, want, TOL_F32)
+        assert not np.array_equal(clean, other)
+        a[0, 700] = np.nan
+        a[20, 3] = np.inf
+        a[31, 2047] = -np.inf
+        got = ctx.qmatmul(h, a, n)
+        for r in (0, 20, 31):
+            assert not np.isfinite(got[r]).any()
+            if dt == flib.DT_I8:
+                assert np.isnan(got[r]).all()
+        keep = [r for r in range(m) if r not in (0, 20, 31)]
+        assert np.array_equal(got[keep], clean[keep])
+        ctx.release(h)
 
 
 def test_int8_digit_plane_gemm_non_finite_rows(ctx, orc):
