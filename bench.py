@@ -607,6 +607,23 @@ def gemv_summary(r, m, t, probe_us=None):
     return out
 
 
+def matrix_entry(r, m, t):
+    """One (configuration, M) pair of the benchmark matrix: time per call, algorithmic bytes and flops, and the
+    fraction of the roof that applies (HBM for M <= 64: at most 128 flop per weight byte against a ridge of about 312;
+    the nominal dense f16 matrix-core peak above)."""
+    abytes = algorithmic_bytes(r["dtn"], m, r["k"], r["n"], r["bias"] is not None)
+    flops = 2.0 * m * r["k"] * r["n"]
+    sec = t["kernel_us"] * 1e-6
+    e = {"us": round(t["kernel_us"], 2), "us_median": round(t["per_trip_us_median"], 2), "us_min": round(t["per_trip_us_min"], 2),
+         "algorithmic_bytes": abytes, "flops": flops, "gb_per_s": round(abytes / sec / 1e9, 1),
+         "tflop_per_s": round(flops / sec / 1e12, 2), "self_check_max_rel": t["self_check_max_rel"]}
+    if m <= 64:
+        e["roof"], e["frac"] = "hbm", round(abytes / sec / 1e9 / HBM_PEAK_GBS, 4)
+    else:
+        e["roof"], e["frac"] = "mfma_f16", round(flops / sec / 1e12 / MFMA_PEAK_TFLOPS["f16"], 4)
+    return e
+
+
 def gemm_summary(r, m, t, peak_name="f16"):
     flops = 2.0 * m * r["k"] * r["n"]
     peak = MFMA_PEAK_TFLOPS[peak_name]
@@ -761,7 +778,7 @@ def main() -> int:
 
     # the other shapes the target is worded on, in the same line: the GEMV at K = N = 4096 (I8 and I4) and the
     # M = 256 GEMM for I4 (this configuration), I8 and FP8
-    gemv_4096, gemm_m256 = None, None
+    gemv_4096, gemm_m256, config_matrix = None, None, None
     if not args.no_extra:
         gemm_m256 = {"m": 256, "unit": "TFLOP/s",
                      "note": "algorithmic flops 2*M*K*N over the whole call (activation preparation + GEMM kernels), eager "
@@ -777,6 +794,20 @@ def main() -> int:
             gemm_m256[args.workload] = {
                 "default": gemm_summary(r, 256, time_matmul(ctx, flib, r, 256, 200, ring, "eager", 0, a_seed=1)),
                 "f16x1": gemm_summary(r, 256, time_matmul(ctx, flib, r, 256, 200, ring, "eager", flib.FLAG_ACT_F16_SINGLE, a_seed=1))}
+        # every (configuration, M) pair the benchmark configurations name, graph replay over the weight ring
+        config_matrix = {"note": "time per call (HIP events on the launch stream, graph replay of whole trips round a weight ring "
+                                 "larger than the Infinity Cache), algorithmic bytes / flops, fraction of the applicable roof: "
+                                 "8 TB/s HBM for M <= 64, nominal dense f16 matrix-core peak 2.5 PFLOP/s above"}
+        matrix_ms = {"c1_i8": (32,), "c2_i4": (16, 128, 256), "c3_i4cb": (1, 64, 256), "c4_f8_up": (64,), "c4_f8_down": (64,),
+                     "c4_f4_up": (64,), "c4_f4_down": (64,)}
+
+        def matrix_legs(rr):
+            for mm in matrix_ms.get(rr["workload"], ()):
+                tt = time_matmul(ctx, flib, rr, mm, 100, 5, "graph", 0, a_seed=1)
+                config_matrix.setdefault(rr["workload"], {})[str(mm)] = matrix_entry(rr, mm, tt)
+
+        config_matrix.setdefault(args.workload, {})[str(m)] = matrix_entry(r, m, t)
+        matrix_legs(r)
         free_ring(ctx, r)
         gemv_4096 = {}
         for wl in ("c1_i8", "i4_4096", "f8_4096"):
@@ -793,6 +824,15 @@ def main() -> int:
                     "f16x1": gemm_summary(r2, 256, time_matmul(ctx, flib, r2, 256, 200, r2["ring"], "eager", flib.FLAG_ACT_F16_SINGLE, a_seed=1))}
             if wl == "c1_i8":
                 gemm_m256["c1_i8_i8act"] = time_i8act(ctx, flib, r2, 256)
+                config_matrix.setdefault(wl, {})["1"] = matrix_entry(r2, 1, t2)
+                if args.workload != wl:
+                    matrix_legs(r2)
+            free_ring(ctx, r2)
+        for wl in ("c3_i4cb", "c4_f8_up", "c4_f8_down", "c4_f4_up", "c4_f4_down"):
+            if wl == args.workload:
+                continue
+            r2 = make_ring(ctx, fastnn_amd, flib, wl, 0)
+            matrix_legs(r2)
             free_ring(ctx, r2)
 
     # the composite configurations (conv list, conv plan, MLP stack), each its own short run: ms per forward
@@ -824,6 +864,7 @@ def main() -> int:
         "cpu_baseline": cpu,
         "gemv_4096": gemv_4096,
         "gemm_m256": gemm_m256,
+        "config_matrix": config_matrix,
         "composites": composites,
         "gb_per_s": round(gbs, 1), "tflop_per_s": round(tops, 3),
         "event_ms_total": round(t["event_ms_total"], 4), "wall_ms_total": round(t["wall_ms_total"], 4),
