@@ -145,6 +145,7 @@ const OptionSpec kOptions[FNN_OPT_COUNT] = {
     {17, 1, 32},      // FNN_OPT_STREAM_MIN_M
     {32, 0, 32},      // FNN_OPT_STREAM_MAX_M
     {0, 0, 0xffff},   // FNN_OPT_STREAM_SHAPE
+    {0, 0, 4},        // FNN_OPT_DIGIT_PLANES
 };
 
 #define HIP_TRY(ctx, code, expr)                                                              \

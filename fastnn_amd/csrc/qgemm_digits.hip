@@ -55,18 +55,19 @@ __device__ __forceinline__ void transpose4(uint32_t a, uint32_t b, uint32_t c, u
 }
 
 // One workgroup per activation row slot: row statistics, then the DIG digit planes of the row in the tile-major
-// operand layout.  Operand row of (activation row m, plane j): (m / RPB) * 32 + j * RPB + m % RPB, RPB = 32 / DIG.
+// operand layout.  Operand row of (activation row m, plane j): (m / RPB) * 32 + j * RPB + m % RPB, RPB = 32 / DIG, for
+// two and four planes; with three planes ((m / 8) * 3 + j) * 8 + m % 8 (groups of 24 rows: 8 activation rows x 3 planes).
 // IL: the nibble decoders deliver k = 0,2,4,6,1,3,5,7 of each 8, and the activations are stored in that order.
 template <int DIG, bool IL>
 __global__ void __launch_bounds__(256) digit_prep_kernel(DigitArgs p)
 {
-    constexpr int RPB = 32 / DIG;
-    constexpr uint32_t BIAS = DIG == 4 ? 0x80808080u : 0x00008080u;
+    constexpr int RPB = DIG == 3 ? 8 : 32 / DIG;
+    constexpr uint32_t BIAS = DIG == 4 ? 0x80808080u : (DIG == 3 ? 0x00808080u : 0x00008080u);
     __shared__ float red[2][4];
     const int64_t m = blockIdx.x;
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const int64_t nchunks = p.kpad / 16;
-    const int64_t row0 = (m / RPB) * 32 + m % RPB;
+    const int64_t row0 = DIG == 3 ? (m / 8) * 24 + m % 8 : (m / RPB) * 32 + m % RPB;
     auto chunk_at = [&](int j, int64_t c) { return p.planes + (((c >> 3) * p.rows_pad + row0 + j * RPB) * KB + (c & 7) * 16); };
     if (m >= p.m) {   // padding rows of the last tile
         const uint4 z = make_uint4(0, 0, 0, 0);
@@ -126,7 +127,7 @@ __global__ void __launch_bounds__(256) digit_prep_kernel(DigitArgs p)
     if (mx > 0.0f) {
         int ex;
         (void)frexpf(mx, &ex);            // mx = f * 2^ex, f in [0.5, 1)
-        e = (DIG == 4 ? 30 : 14) - ex;    // |x * 2^e| < 2^30 (2^14 with two planes)
+        e = (DIG == 4 ? 30 : (DIG == 3 ? 22 : 14)) - ex;    // |x * 2^e| < 2^30 (2^22 with three planes, 2^14 with two)
     }
     auto convert = [&](int64_t c, const float (&v)[16]) {
         uint32_t t[16];
@@ -306,6 +307,91 @@ int run_digits(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const Q
     return FNN_OK;
 }
 
+
+// Three digit planes: rint(x * 2^e) with |v| < 2^22 per row.  A quarter less matrix-core work and activation operand
+// traffic than four planes for 2e-5 of max|ref| stated (about 3e-6 measured on rows with 200x outliers; the four-plane
+// form holds 4e-6).  Operand rows come in groups of 24, so a wave owns three MFMA blocks: tiles of 192 operand rows
+// (64 activation rows) x 128 weight rows on four waves, x 256 on eight for 4-bit weights with many column tiles.
+template <int DT>
+int run_digits3(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &q)
+{
+    constexpr bool IL = DecI<DT>::INTERLEAVED;
+    constexpr bool W4 = DecI<DT>::WPS == 2;
+    const int64_t M = q.m, N = q.n, K = q.k;
+    const int64_t kpad = (K + KB - 1) / KB * KB;
+    const int iters = (int)(kpad / KB);
+    const int bm = 192, act_rows = 64;
+    // tile forms: 0 = 192 x 128 on four waves, 1 = 192 x 256 on eight (4-bit weights), 2 = 192 x 128 on eight (twice the
+    // waves requesting the operands).  By shape: 4-bit weights take the wide tiles while those still cover the chip.
+    int form = 2;
+    if (W4 && (N + 255) / 256 * ((M + 63) / 64) >= 160) form = 1;
+    const int64_t opt_cfg = fnn_ctx_option(ctx, FNN_OPT_TILE_SHAPE);
+    if (opt_cfg >= 0 && opt_cfg <= 2 && (opt_cfg != 1 || W4)) form = (int)opt_cfg;
+    const int wide = form == 1;
+    const int bn = wide ? 256 : 128;
+    const int mtiles = (int)((M + act_rows - 1) / act_rows), ntiles = (int)((N + bn - 1) / bn);
+    const int64_t tiles = (int64_t)mtiles * ntiles;
+    // K split: as many workgroups as fit one round over the 256 CUs, never more (4096 x 11008 at M = 256, 172 tiles:
+    // 47 us unsplit, 66 us in two splits; 4096 x 4096 at M = 128, 64 tiles: 23 us in four splits, 31 us unsplit)
+    int splits = (int)(256 / tiles);
+    if (splits > iters / 4) splits = iters / 4;   // four stages or more per workgroup
+    if (splits < 1) splits = 1;
+    const int opt_split = (int)fnn_ctx_option(ctx, FNN_OPT_TILE_SPLIT);
+    if (opt_split > 0) splits = opt_split;
+    if (splits > iters) splits = iters;
+    const int ips = (iters + splits - 1) / splits;
+    splits = (iters + ips - 1) / ips;   // no empty split
+    const int64_t rows_pad = (int64_t)mtiles * bm, m_pad = (int64_t)mtiles * act_rows;
+
+    const size_t a_bytes = (size_t)rows_pad * kpad;
+    const size_t meta_off = (a_bytes + 255) / 256 * 256;
+    void *ws0 = nullptr, *ws1 = nullptr;
+    int rc;
+    if ((rc = fnn_ctx_ensure_tmp(ctx, 0, meta_off + (size_t)m_pad * 8 + 256, &ws0))) return rc;
+    if (splits > 1 && (rc = fnn_ctx_ensure_tmp(ctx, 1, (size_t)splits * M * N * 4, &ws1))) return rc;
+
+    DigitArgs d;
+    d.a = q.a;
+    d.planes = (int8_t *)ws0;
+    d.rexp = (int *)((char *)ws0 + meta_off);
+    d.xsum = (float *)(d.rexp + m_pad);
+    d.m = M; d.k = K; d.kpad = kpad; d.rows_pad = rows_pad;
+    hipLaunchKernelGGL((digit_prep_kernel<3, IL>), dim3((unsigned)m_pad), dim3(256), 0, s, d);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, hipGetErrorString(e));
+
+    TileArgs t = {};
+    t.words = q.words;
+    t.zero_chunk = q.words + w->rows * q.kp;    // the zeroed margin behind the last row
+    t.scales = q.scales; t.zeros = q.zeros; t.bias = q.bias;
+    t.ap = reinterpret_cast<const _Float16 *>(d.planes);
+    t.rexp = d.rexp; t.xsum = d.xsum;
+    t.out = q.out; t.part = (float *)ws1;
+    if (FnnResidualIo *res = fnn_ctx_residual_io(ctx); splits > 1 && res->residual && res->of_out == q.out && res->elems == (uint64_t)(M * N)) {
+        t.residual = res->residual; t.sum_out = res->sum_out;
+        res->used = 1;
+    }
+    t.m = M; t.n = N; t.kp = q.kp; t.kpad = kpad; t.rows_pad = rows_pad;
+    t.act = q.act; t.splits = splits; t.iters = iters; t.ips = ips; t.mtiles = mtiles; t.ntiles = ntiles;
+    // ring depth: four stages (24 KB of planes + 8 or 16 KB of weights each; the 8-bit and the wide forms fill the LDS)
+    if (form == 1) {
+        if constexpr (W4) e = launch_digit_tile<DT, 2, 4, 3, 2, 4, 3>(t, s);
+        else e = hipErrorInvalidValue;
+    } else if (form == 2) e = launch_digit_tile<DT, 2, 4, 3, 1, 4, 3>(t, s);
+    else e = launch_digit_tile<DT, 2, 2, 3, 2, 4, 3>(t, s);
+    if (e != hipSuccess) return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, hipGetErrorString(e));
+    if (splits > 1) {
+        const int64_t colb = (N + 255) / 256;
+        int64_t rowb = (2048 + colb - 1) / colb;   // about 2048 workgroups
+        if (rowb > M) rowb = M;
+        if (rowb > 65535) rowb = 65535;
+        hipLaunchKernelGGL(splitk_epilogue_kernel, dim3((unsigned)colb, (unsigned)rowb), dim3(256), 0, s, t, 0);
+        e = hipGetLastError();
+        if (e != hipSuccess) return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, hipGetErrorString(e));
+    }
+    return FNN_OK;
+}
+
 }  // namespace
 
 int fnn_digits_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &q, int flags, bool *handled)
@@ -326,9 +412,25 @@ int fnn_digits_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w,
     // faster than one f16 row but measured 1.9e-3 on rows with a few 200x outliers, where a float rounding per
     // element keeps 2.4e-4; three planes cost what the f16 row costs.
     if (flags & FNN_FLAG_ACT_F16_SINGLE) return FNN_OK;
+    // Planes by shape: three wherever they measured faster than four, i.e. 4-bit weights at every M (4096 x 11008: M = 64
+    // 26.3 against 29.3 us, M = 128 30.9 against 40.2, M = 256 47.2 against 54.9, M = 1024 139 against 168) and 8-bit
+    // weights from M = 96 (4096 x 4096: M = 64 21.6 against 19.1, M = 128 23.1 against 24.2, M = 512 40.7 against 49.7).
+    int64_t planes = fnn_ctx_option(ctx, FNN_OPT_DIGIT_PLANES);
+    if (planes != 3 && planes != 4) planes = (dt == FNN_DT_I8 && q.m < 96) ? 4 : 3;
     // 8-bit weights decode to f16 with one permute per pair, so at four planes the int8 form only ties the f16 tiles
-    // (hi + lo rows) and falls 4-5 % behind them from M = 1024 on (4096 x 4096: 93 vs 89 us, M = 2048: 172 vs 164)
-    if (dt == FNN_DT_I8 && q.m >= 768 && fnn_ctx_option(ctx, FNN_OPT_GEMM_INT8_MIN_M) <= 17) return FNN_OK;
+    // (hi + lo rows) and falls 4-5 % behind them from M = 1024 on (4096 x 4096: 93 vs 89 us, M = 2048: 172 vs 164); at
+    // three planes it stays ahead (M = 1024: 70 against 86 us, M = 2048: 128 against 160)
+    if (planes == 4 && dt == FNN_DT_I8 && q.m >= 768 && fnn_ctx_option(ctx, FNN_OPT_GEMM_INT8_MIN_M) <= 17) return FNN_OK;
+    if (planes == 3) {
+        switch (dt) {
+        case FNN_DT_I8: rc = run_digits3<FNN_DT_I8>(ctx, s, w, qa); break;
+        case FNN_DT_I4: rc = run_digits3<FNN_DT_I4>(ctx, s, w, qa); break;
+        default: rc = run_digits3<FNN_DT_U4>(ctx, s, w, qa); break;
+        }
+        if (rc) return rc;
+        *handled = true;
+        return FNN_OK;
+    }
     switch (dt) {
     case FNN_DT_I8: rc = run_digits<FNN_DT_I8, 4>(ctx, s, w, qa); break;
     case FNN_DT_I4: rc = run_digits<FNN_DT_I4, 4>(ctx, s, w, qa); break;

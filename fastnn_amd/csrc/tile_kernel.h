@@ -96,14 +96,17 @@ __device__ __forceinline__ void wait_loads_but()
 // DIG > 0 (with INT8): the activation operand holds DIG balanced base-256 digit planes of f32 activations
 //               scaled per row by 2^rexp: a 32-row MFMA block = 32/DIG activation rows x DIG planes (plane j in
 //               block rows [j*32/DIG, (j+1)*32/DIG)), so a lane holds every plane's exact i32 sum of its outputs
-//               and recombines them, sum_j 256^j * acc_j, before the float epilogue.
+//               and recombines them, sum_j 256^j * acc_j, before the float epilogue.  DIG = 3: eight activation
+//               rows x 3 planes form a group of 24 operand rows (plane j in rows [8j, 8j + 8) of the group); the
+//               8-row slabs of a lane's accumulators then alternate plane by plane, three MFMA blocks per four groups.
 // CONV (with INT8, DIG = 0): the rows are im2col rows (image, pixel); the accumulators are turned into the
 //               convolution's outputs here (conv_dequant) and stored NCHW, four consecutive pixels of a channel
 //               per lane and store where the image size allows.
 template <int DT, int WGM, int WGN, int TM, int TN, bool PRECISE, int NS, bool INT8 = false, int DIG = 0, bool CONV = false, bool CRNG = false>
 __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
 {
-    static_assert(DIG == 0 || (INT8 && (DIG == 2 || DIG == 4)), "digit planes ride on the int8 operands");
+    static_assert(DIG == 0 || (INT8 && (DIG == 2 || DIG == 3 || DIG == 4)), "digit planes ride on the int8 operands");
+    static_assert(DIG != 3 || TM % 3 == 0, "three planes: a wave's rows are whole groups of 24 operand rows (8 activation rows x 3 planes)");
     static_assert(!CONV || (INT8 && DIG == 0), "the conv epilogue belongs to the plain int8 kernel");
     static_assert(!CRNG || CONV, "output ranges come from the conv epilogue");   // CRNG: p.cv.range_out is set
     // Codebook weights (w[n,k] = bscale[n, k/32] * table[nibble], src/packed_tensor.rs:469-521) are decoded here:
@@ -526,7 +529,63 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
 
     // ---- epilogue.  acc[i] of a 32x32 block: row (i/4)*8 + h*4 + i%4, column lr.  With hi/lo
     // operands a block holds 16 output rows: hi in rows 0..15 (i < 8), lo in rows 16..31 (i + 8).
-    if constexpr (INT8 && DIG > 0) {
+    if constexpr (INT8 && DIG == 3) {
+        // slab q of the wave (operand rows 8q .. 8q + 7, q = tm*4 + i/4) = plane q % 3 of the activation rows
+        // 8 (q/3) .. + 7; a lane holds rows 4h + t of every slab in acc[q / 4][tn][(q % 4) * 4 + t]
+        constexpr int SHIFT = (DT == FNN_DT_I4) ? 4 : 0;   // 4-bit signed lanes entered as 16*q
+        constexpr int GR = TM * 4 / 3;                      // groups of 8 activation rows per wave
+        const int64_t mrow0 = ((int64_t)mt * BM + wm * TM * 32) / 3;
+        const bool split = p.splits > 1;
+        float sc[TN], zp[TN], bi[TN];
+#pragma unroll
+        for (int tn = 0; tn < TN; tn++) {
+            const int64_t n = n0 + (wn * TN + tn) * 32 + lr;
+            const bool ok = n < p.n && !split;
+            sc[tn] = ok ? p.scales[n] : 0.0f;
+            zp[tn] = ok ? p.zeros[n] : 0.0f;
+            bi[tn] = (ok && p.bias) ? p.bias[n] : 0.0f;
+        }
+        int rexp[GR][4];
+        float rxs[GR][4];
+#pragma unroll
+        for (int u = 0; u < GR; u++)
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                int64_t m = mrow0 + u * 8 + h * 4 + t;
+                if (m > p.m - 1) m = p.m - 1;
+                rexp[u][t] = p.rexp[m];
+                rxs[u][t] = split ? 0.0f : p.xsum[m];
+            }
+#pragma unroll
+        for (int u = 0; u < GR; u++)
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                const int64_t m = mrow0 + u * 8 + h * 4 + t;
+                if (m >= p.m) continue;
+                const int e = rexp[u][t];
+                const bool bad = e == INT_MIN;      // the row holds a non-finite activation
+#pragma unroll
+                for (int tn = 0; tn < TN; tn++) {
+                    const int64_t n = n0 + (wn * TN + tn) * 32 + lr;
+                    if (n >= p.n) continue;
+                    float v = 0.0f;
+#pragma unroll
+                    for (int j = 2; j >= 0; j--) {
+                        const int q = 3 * u + j;
+                        v = fmaf(v, 256.0f, (float)__float_as_int(acc[q >> 2][tn][(q & 3) * 4 + t]));
+                    }
+                    const float d = bad ? __builtin_nanf("") : ldexpf(v, -e - SHIFT);
+                    if (split) {
+                        p.part[((int64_t)z * p.m + m) * p.n + n] = d;
+                    } else {
+                        float o = d * sc[tn] + zp[tn] * rxs[u][t];
+                        if (p.bias) o = o + bi[tn];
+                        p.out[m * p.n + n] = fnn_activation(o, p.act);
+                    }
+                }
+            }
+        return;
+    } else if constexpr (INT8 && DIG > 0) {
         constexpr int RPB = 32 / DIG;        // activation rows per 32-row block
         constexpr int NR = RPB / 2;          // ... of which a lane holds NR (the other half belongs to lanes h ^ 1)
         constexpr int SHIFT = (DT == FNN_DT_I4) ? 4 : 0;   // 4-bit signed lanes entered as 16*q

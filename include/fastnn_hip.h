@@ -132,7 +132,10 @@ enum {
                                   /* it declines shapes with more column tiles x K splits than the chip holds at once            */
     FNN_OPT_STREAM_SHAPE = 21,    /* its launch shape: 0 (default) = by rule, else (splits << 8) | (row tiles per wave << 4) |   */
                                   /* (k-values per round / 256), splits = 0 meaning one round per workgroup                      */
-    FNN_OPT_COUNT = 22
+    FNN_OPT_DIGIT_PLANES = 22,    /* int8 matrix-core GEMM (M >= 17, I8 / I4 / U4 weights): activation digit planes, 3 (22 bits     */
+                                  /* below the row maximum, 2e-5 of max|ref| stated) or 4 (30 bits, 4e-6, a third more matrix-core */
+                                  /* work and operand traffic); 0 (default) = three wherever they measured faster                  */
+    FNN_OPT_COUNT = 23
 };
 int fnn_hip_set_option(fnn_hip_ctx *ctx, int option, int64_t value);
 int fnn_hip_get_option(fnn_hip_ctx *ctx, int option, int64_t *value);
