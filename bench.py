@@ -783,17 +783,29 @@ def main() -> int:
         gemm_m256 = {"m": 256, "unit": "TFLOP/s",
                      "note": "algorithmic flops 2*M*K*N over the whole call (activation preparation + GEMM kernels), eager "
                              "launches over the weight ring; 'default' (2e-5 agreement): I8 / I4 weights run on the int8 matrix "
-                             "cores over four exact activation digit planes (4x the algorithmic ops at the int8 rate), FP8 on "
+                             "cores over three exact activation digit planes (3x the algorithmic ops at the int8 rate), FP8 on "
                              "the f16 matrix cores with hi+lo f16 activation rows (2x the algorithmic flops); 'f16x1' (1e-3): "
                              "activations rounded to f16 once; frac is of the nominal dense f16 peak (2.5 PFLOP/s); "
                              "matrix_core_only = what a kernel of MFMAs alone (no memory traffic) sustains on this device"}
         mc = probe.mfma_ceiling(target_us=(40.0,))
         gemm_m256["matrix_core_only"] = {"f16_tflop_per_s": max(v["tops"] for v in mc["f16_32x32x16"].values()),
                                          "i8_top_per_s": max(v["tops"] for v in mc["i8_32x32x32"].values())}
+        def act_quant_leg(rr):
+            peak = "fp8" if rr["dtn"] == "f8" else "i8"
+            e = gemm_summary(rr, 256, time_matmul(ctx, flib, rr, 256, 200, rr["ring"], "eager", flib.FLAG_ACT_QUANT, a_seed=1), peak)
+            e["note"] = ("FNN_FLAG_ACT_QUANT, NOT parity with matmul_%s: activations quantised on the way in (%s), one plane on the "
+                         "%s matrix cores; frac is of the nominal dense %s peak" %
+                         (rr["dtn"], "E4M3, one power-of-two scale per row; within 5e-2 of max|ref|" if peak == "fp8" else
+                          "the reference's quantize_activations -> matmul_*_i8 chain, integer accumulators bit-exact against it",
+                          peak, peak))
+            return e
+
         if m != 256:
             gemm_m256[args.workload] = {
                 "default": gemm_summary(r, 256, time_matmul(ctx, flib, r, 256, 200, ring, "eager", 0, a_seed=1)),
                 "f16x1": gemm_summary(r, 256, time_matmul(ctx, flib, r, 256, 200, ring, "eager", flib.FLAG_ACT_F16_SINGLE, a_seed=1))}
+            if dtn in ("i8", "i4", "f8"):
+                gemm_m256[args.workload]["act_quant"] = act_quant_leg(r)
         # every (configuration, M) pair the benchmark configurations name, graph replay over the weight ring
         config_matrix = {"note": "time per call (HIP events on the launch stream, graph replay of whole trips round a weight ring "
                                  "larger than the Infinity Cache), algorithmic bytes / flops, fraction of the applicable roof: "
@@ -821,7 +833,8 @@ def main() -> int:
             if wl != "i4_4096":
                 gemm_m256[wl] = {
                     "default": gemm_summary(r2, 256, time_matmul(ctx, flib, r2, 256, 200, r2["ring"], "eager", 0, a_seed=1)),
-                    "f16x1": gemm_summary(r2, 256, time_matmul(ctx, flib, r2, 256, 200, r2["ring"], "eager", flib.FLAG_ACT_F16_SINGLE, a_seed=1))}
+                    "f16x1": gemm_summary(r2, 256, time_matmul(ctx, flib, r2, 256, 200, r2["ring"], "eager", flib.FLAG_ACT_F16_SINGLE, a_seed=1)),
+                    "act_quant": act_quant_leg(r2)}
             if wl == "c1_i8":
                 gemm_m256["c1_i8_i8act"] = time_i8act(ctx, flib, r2, 256)
                 config_matrix.setdefault(wl, {})["1"] = matrix_entry(r2, 1, t2)

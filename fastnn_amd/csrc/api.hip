@@ -561,6 +561,40 @@ int fnn_hip_qmatmul(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *a, i
         p.m = m; p.n = n; p.k = k; p.kp = w->kp; p.bpr = w->bpr; p.qblock = w->qblock; p.act = act;
         p.as_written = (flags & FNN_FLAG_I4CB_AS_WRITTEN) ? 1 : 0;
 
+        if (flags & FNN_FLAG_ACT_QUANT) {
+            if (ctx->static_mode) return fail(ctx, FNN_ERR_DISPATCH, "fnn_hip_qmatmul_static: flag not available here");
+            if (w->dtype != FNN_DT_I8 && w->dtype != FNN_DT_I4 && w->dtype != FNN_DT_F8)
+                return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "%s: FNN_FLAG_ACT_QUANT applies to I8, I4 and F8 weights", kn);
+            if (w->dtype == FNN_DT_F8) {
+                bool done = false;
+                int rc = fnn_fp8_actquant_qmatmul(ctx, ctx->stream, w, p, &done);
+                if (rc) return rc;
+                if (!done) return fail(ctx, FNN_ERR_UNSUPPORTED_OP, "%s: FNN_FLAG_ACT_QUANT needs K %% 128 == 0 and 16-byte aligned operands for F8 weights", kn);
+            } else {
+                // quantize_activations (dynamic: scale = max|x| / 127, zero 0) into a transient payload, then the
+                // I8-activation MatMul with the bias and the activation behind its formula
+                void *pl = nullptr;
+                int rc = fnn_ctx_ensure_tmp(ctx, 2, (size_t)(m * k) + 8 + 16, &pl);
+                if (rc) return rc;
+                HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_quantize_activations(da, m * k, 0.0f, 0.0f, (uint8_t *)pl, ctx->scratch, ctx->stream));
+                I8ActArgs q8;
+                q8.words = w->words; q8.scales = w->scales; q8.zeros = w->zeros; q8.payload = (const uint8_t *)pl; q8.out = dout;
+                q8.acc_out = nullptr; q8.m = m; q8.n = n; q8.k = k; q8.kp = w->kp;
+                q8.bias = dbias; q8.act = act;
+                bool done = false;
+                if (!(flags & FNN_FLAG_FORCE_GENERIC)) {
+                    rc = fnn_i8_tiled_matmul(ctx, ctx->stream, w, q8, &done);
+                    if (rc) return rc;
+                }
+                if (!done) HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qgemm_i8act_generic(w->dtype, q8, ctx->stream));
+            }
+            if (!dev) {
+                HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(out, dout, (size_t)(m * n) * 4, hipMemcpyDeviceToHost, ctx->stream));
+                HIP_TRY(ctx, FNN_ERR_DISPATCH, hipStreamSynchronize(ctx->stream));
+            }
+            return FNN_OK;
+        }
+
         // kernel choice: matrix-core kernel for every M (bandwidth-bound at small M); the FMA GEMV
         // serves the codebook type at M <= 4 and any weight when FNN_FLAG_PREFER_FMA asks for it;
         // the shape-agnostic kernel takes what is left (ragged rows, unaligned pointers).

@@ -10,6 +10,10 @@ struct I8ActArgs {
     float *out;             // [M,N]
     int32_t *acc_out;       // [M,N] or null
     int64_t m, n, k, kp;
+    // the activation-quantised mode of the f32-activation MatMul (FNN_FLAG_ACT_QUANT): bias + activation behind the
+    // I8-activation formula, as the instruction chain matmul_i8_i8 -> add -> act would apply them
+    const float *bias = nullptr;
+    int act = 0;
 };
 
 struct QConvArgs {

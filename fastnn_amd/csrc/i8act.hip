@@ -128,6 +128,8 @@ __global__ void __launch_bounds__(256) qgemm_i8act_generic_kernel(I8ActArgs p)
             res = dot * sw + zw * input_sum;
         }
         if (lane == 0) {
+            if (p.bias) res = res + p.bias[n];
+            res = fnn_activation(res, p.act);
             p.out[(m0 + m) * p.n + n] = res;
             if (p.acc_out) p.acc_out[(m0 + m) * p.n + n] = a_tot;
         }

@@ -41,6 +41,8 @@ uint32_t *fnn_ctx_stream_counters(fnn_hip_ctx *ctx);
 int fnn_digits_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &p, int flags, bool *handled);
 int fnn_tiled_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &p,
                       int flags, bool *handled);
+// FNN_FLAG_ACT_QUANT with F8 weights: activations rounded to E4M3 (one power-of-two scale per row), fp8 matrix cores
+int fnn_fp8_actquant_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &p, bool *handled);
 
 int64_t fnn_conv_operand_workgroups(const QConvArgs &p);
 // the implicit-GEMM convolution (qconv_implicit.hip): rows of one of its workgroups for this shape, and the call

@@ -82,7 +82,8 @@ __global__ void __launch_bounds__(256) i8_rows_operand_kernel(const int8_t *qa, 
 // formed here from the integer sums: sum (q_a*sa + za)*q_w = sa*acc + za*sum_k q_w.
 __global__ void __launch_bounds__(256) i8_matmul_epilogue_kernel(const int32_t *c, const uint8_t *payload, const int32_t *qsum,
                                                                  const int32_t *wsum, const float *scales, const float *zeros,
-                                                                 int64_t m, int64_t n, int64_t k, float *out, int32_t *acc_out, int splits)
+                                                                 int64_t m, int64_t n, int64_t k, float *out, int32_t *acc_out, int splits,
+                                                                 const float *bias, int act)
 {
     // a thread owns one output column (its weight constants stay in registers) and walks rows blockIdx.y, +gridDim.y, ...
     const float sa = reinterpret_cast<const float *>(payload)[0];
@@ -92,13 +93,16 @@ __global__ void __launch_bounds__(256) i8_matmul_epilogue_kernel(const int32_t *
     const float sw = scales[col], zw = zeros[col];
     const float zwsum = za * (float)wsum[col];
     const float kza = (float)k * za;
+    const float bs = bias ? bias[col] : 0.0f;
     for (int64_t r = blockIdx.y; r < m; r += gridDim.y) {
         const int64_t idx = r * n + col;
         int acc = c[idx];
         for (int z = 1; z < splits; z++) acc += c[(int64_t)z * m * n + idx];   // exact whatever the order
         const float input_sum = (float)qsum[r] * sa + kza;
         const float dot = (za != 0.0f) ? (float)acc * sa + zwsum : (float)acc * sa;
-        out[idx] = dot * sw + zw * input_sum;
+        float v = dot * sw + zw * input_sum;
+        if (bias) v = v + bs;
+        out[idx] = fnn_activation(v, act);
         if (acc_out) acc_out[idx] = (za != 0.0f) ? 0 : acc;
     }
 }
@@ -402,7 +406,7 @@ __global__ void __launch_bounds__(256) conv_epilogue_kernel(QConvArgs a, int g, 
     }
 }
 
-template <int DT, int WGM, int WGN, int TM, int TN, int NS, bool CONV = false, bool CRNG = false>
+template <int DT, int WGM, int WGN, int TM, int TN, int NS, bool CONV = false, bool CRNG = false, bool FP8 = false>
 hipError_t launch_i8_tile(const TileArgs &p, hipStream_t s)
 {
     if constexpr (CONV && !CRNG) {
@@ -411,7 +415,7 @@ hipError_t launch_i8_tile(const TileArgs &p, hipStream_t s)
     constexpr int WC = 2 * DecI<DT>::WPS;
     constexpr int BM = WGM * TM * 32, BN = WGN * TN * 32;
     constexpr size_t lds = (size_t)NS * (BM * 128 + BN * WC * 16);
-    auto kern = qgemm_tile_kernel<DT, WGM, WGN, TM, TN, false, NS, true, 0, CONV, CRNG>;
+    auto kern = qgemm_tile_kernel<DT, WGM, WGN, TM, TN, false, NS, true, 0, CONV, CRNG, FP8>;
     static std::atomic<uint64_t> lds_raised{0};
     hipError_t e = fnn_raise_lds_limit(lds_raised, reinterpret_cast<const void *>(kern), (int)lds);
     if (e != hipSuccess) return e;
@@ -487,6 +491,121 @@ hipError_t run_i8_gemm(const uint32_t *words, int64_t kp, int64_t rows_total, in
 
 }  // namespace
 
+// ---- FNN_FLAG_ACT_QUANT with F8 weights: f32 activations rounded to E4M3, fp8 matrix cores.
+// Row m is scaled by a power of two that brings its largest magnitude into [128, 256) (E4M3 reaches 448) and rounded
+// to nearest-even E4M3 by v_cvt_pk_fp8_f32; the bytes go into the tile-major operand layout of the int8 kernels.
+// No counterpart in fastnn (it has no fp8 activation quantiser): a fast mode with a stated tolerance.
+namespace {
+
+__global__ void __launch_bounds__(256) fp8_rows_operand_kernel(const float *a, int64_t m, int64_t k, int64_t kpad, int64_t rows_pad,
+                                                               int8_t *a8, float *rscale)
+{
+    __shared__ float red[4];
+    const int64_t r = blockIdx.x;
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    float mx = 0.0f;
+    if (r < m)
+        for (int64_t i = tid; i < k; i += 256) mx = fmaxf(mx, fabsf(a[r * k + i]));
+    mx = wave_max(mx);
+    if (lane == 0) red[wv] = mx;
+    __syncthreads();
+    mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    int ex = (int)((__float_as_uint(mx) >> 23) & 0xff) - 127 - 7;   // mx * 2^-ex in [128, 256)
+    if (mx == 0.0f) ex = 0;
+    ex = ex < -100 ? -100 : (ex > 120 ? 120 : ex);
+    const float inv = __uint_as_float((uint32_t)(127 - ex) << 23);
+    for (int64_t c = tid; c < kpad / 16; c += 256) {   // 16-byte chunk c of the row
+        uint32_t out[4] = {0, 0, 0, 0};
+        if (r < m) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                float v[4];
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const int64_t kk = c * 16 + q * 4 + j;
+                    v[j] = kk < k ? a[r * k + kk] * inv : 0.0f;
+                }
+                int w = __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], 0, false);
+                w = __builtin_amdgcn_cvt_pk_fp8_f32(v[2], v[3], w, true);
+                out[q] = (uint32_t)w;
+            }
+        }
+        const int64_t kb = c >> 3, cc = c & 7;
+        *reinterpret_cast<uint4 *>(a8 + (kb * rows_pad + r) * KB + cc * 16) = make_uint4(out[0], out[1], out[2], out[3]);
+    }
+    if (tid == 0 && r < m) rscale[r] = __uint_as_float((uint32_t)(127 + ex) << 23);
+}
+
+// out[m,n] = act((sum over splits of the f32 partial sums) * 2^e[m] * scale[n] + bias[n]), partials added in split order
+__global__ void __launch_bounds__(256) fp8_matmul_epilogue_kernel(const float *c, const float *rscale, const float *scales, const float *bias,
+                                                                  int64_t m, int64_t n, float *out, int splits, int act)
+{
+    const int64_t col = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (col >= n) return;
+    const float sw = scales[col];
+    const float bs = bias ? bias[col] : 0.0f;
+    for (int64_t r = blockIdx.y; r < m; r += gridDim.y) {
+        const int64_t idx = r * n + col;
+        float acc = c[idx];
+        for (int z = 1; z < splits; z++) acc += c[(int64_t)z * m * n + idx];
+        float v = (acc * rscale[r]) * sw;
+        if (bias) v = v + bs;
+        out[idx] = fnn_activation(v, act);
+    }
+}
+
+}  // namespace
+
+int fnn_fp8_actquant_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &q, bool *handled)
+{
+    *handled = false;
+    if (w->dtype != FNN_DT_F8) return FNN_OK;
+    if ((reinterpret_cast<uintptr_t>(q.words) & 15) || q.kp % 4 != 0) return FNN_OK;
+    if (q.m < 1 || q.m > (1 << 22) || q.n > (1 << 24) || q.k > (1 << 20)) return FNN_OK;
+    const int64_t kpad = (q.k + KB - 1) / KB * KB;
+    const int64_t rows_pad = (q.m + 127) / 128 * 128;
+    const size_t a_bytes = (size_t)rows_pad * kpad;
+    const size_t r_off = (a_bytes + 255) / 256 * 256;
+    const int64_t tiles = (rows_pad / 128) * ((q.n + 127) / 128);
+    const int iters = (int)(kpad / KB);
+    int splits = (int)(256 / (tiles > 0 ? tiles : 1));
+    if (splits > iters / 4) splits = iters / 4;
+    if (splits > 16) splits = 16;
+    if (splits < 1) splits = 1;
+    void *ws0 = nullptr, *ws1 = nullptr;
+    int rc;
+    if ((rc = fnn_ctx_ensure_tmp(ctx, 0, r_off + (size_t)rows_pad * 4 + 256, &ws0))) return rc;
+    if ((rc = fnn_ctx_ensure_tmp(ctx, 1, (size_t)splits * q.m * q.n * 4 + 256, &ws1))) return rc;
+    int8_t *a8 = (int8_t *)ws0;
+    float *rscale = (float *)((char *)ws0 + r_off);
+    hipLaunchKernelGGL(fp8_rows_operand_kernel, dim3((unsigned)rows_pad), dim3(256), 0, s, q.a, q.m, q.k, kpad, rows_pad, a8, rscale);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, hipGetErrorString(e));
+    TileArgs t = {};
+    t.words = q.words;
+    t.zero_chunk = q.words + w->rows * q.kp;   // the zeroed margin behind the last row
+    t.ap = reinterpret_cast<const _Float16 *>(a8);
+    t.c_i32 = (int32_t *)ws1; t.ldc = q.n;
+    t.m = q.m; t.n = q.n; t.kp = q.kp; t.kpad = kpad; t.rows_pad = rows_pad;
+    t.iters = iters;
+    t.ips = (iters + splits - 1) / splits;
+    t.splits = (iters + t.ips - 1) / t.ips;
+    t.mtiles = (int)(rows_pad / 128);
+    t.ntiles = (int)((q.n + 127) / 128);
+    e = launch_i8_tile<FNN_DT_I8, 2, 2, 2, 2, 3, false, false, true>(t, s);
+    if (e != hipSuccess) return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, hipGetErrorString(e));
+    const int64_t colb = (q.n + 255) / 256;
+    int64_t rowb = (4096 + colb - 1) / colb;
+    if (rowb > q.m) rowb = q.m;
+    if (rowb > 65535) rowb = 65535;
+    hipLaunchKernelGGL(fp8_matmul_epilogue_kernel, dim3((unsigned)colb, (unsigned)rowb), dim3(256), 0, s, (const float *)ws1, rscale, q.scales,
+                       q.bias, q.m, q.n, q.out, t.splits, q.act);
+    e = hipGetLastError();
+    if (e != hipSuccess) return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, hipGetErrorString(e));
+    *handled = true;
+    return FNN_OK;
+}
+
 int fnn_i8_tiled_matmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const I8ActArgs &p, bool *handled)
 {
     *handled = false;
@@ -542,7 +661,7 @@ int fnn_i8_tiled_matmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w
         if (rowb > p.m) rowb = p.m;
         if (rowb > 65535) rowb = 65535;
         hipLaunchKernelGGL(i8_matmul_epilogue_kernel, dim3((unsigned)colb, (unsigned)rowb), dim3(256), 0, s, c, p.payload, qsum, wm->row_qsum,
-                           p.scales, p.zeros, p.m, p.n, p.k, p.out, p.acc_out, splits);
+                           p.scales, p.zeros, p.m, p.n, p.k, p.out, p.acc_out, splits, p.bias, p.act);
         e = hipGetLastError();
     }
     if (e != hipSuccess) return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, hipGetErrorString(e));

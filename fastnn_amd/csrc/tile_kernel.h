@@ -102,9 +102,14 @@ __device__ __forceinline__ void wait_loads_but()
 // CONV (with INT8, DIG = 0): the rows are im2col rows (image, pixel); the accumulators are turned into the
 //               convolution's outputs here (conv_dequant) and stored NCHW, four consecutive pixels of a channel
 //               per lane and store where the image size allows.
-template <int DT, int WGM, int WGN, int TM, int TN, bool PRECISE, int NS, bool INT8 = false, int DIG = 0, bool CONV = false, bool CRNG = false>
+// FP8 (with INT8, DT = FNN_DT_I8, DIG = 0, no CONV): the bytes of both operands are OCP E4M3 values; the same pipeline
+//               with two v_mfma_f32_32x32x16_fp8_fp8 per step (the low and the high 8 bytes of a lane's 16) and f32
+//               accumulators, whose bits are stored where the int8 mode stores its integers.
+template <int DT, int WGM, int WGN, int TM, int TN, bool PRECISE, int NS, bool INT8 = false, int DIG = 0, bool CONV = false, bool CRNG = false,
+          bool FP8 = false>
 __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
 {
+    static_assert(!FP8 || (INT8 && DT == FNN_DT_I8 && DIG == 0 && !CONV), "the fp8 mode rides on the plain byte pipeline");
     static_assert(DIG == 0 || (INT8 && (DIG == 2 || DIG == 3 || DIG == 4)), "digit planes ride on the int8 operands");
     static_assert(DIG != 3 || TM % 3 == 0, "three planes: a wave's rows are whole groups of 24 operand rows (8 activation rows x 3 planes)");
     static_assert(!CONV || (INT8 && DIG == 0), "the conv epilogue belongs to the plain int8 kernel");
@@ -420,7 +425,12 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
             for (int tm = 0; tm < TM; tm++)
 #pragma unroll
                 for (int tn = 0; tn < TN; tn++)
-                    if constexpr (INT8) {
+                    if constexpr (FP8) {
+                        typedef long i64x2 __attribute__((ext_vector_type(2)));
+                        const i64x2 a2 = __builtin_bit_cast(i64x2, af[tm]), b2 = __builtin_bit_cast(i64x2, bf[tn]);
+                        acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(a2[0], b2[0], acc[tm][tn], 0, 0, 0);
+                        acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(a2[1], b2[1], acc[tm][tn], 0, 0, 0);
+                    } else if constexpr (INT8) {
                         acc[tm][tn] = __builtin_bit_cast(f32x16, __builtin_amdgcn_mfma_i32_32x32x32_i8(
                                                                      __builtin_bit_cast(i32x4, af[tm]), __builtin_bit_cast(i32x4, bf[tn]),
                                                                      __builtin_bit_cast(i32x16, acc[tm][tn]), 0, 0, 0));

@@ -22,6 +22,7 @@ FLAG_I4CB_AS_WRITTEN = 2
 FLAG_ACT_F16_SINGLE = 4
 FLAG_FORCE_GENERIC = 8
 FLAG_PREFER_FMA = 16
+FLAG_ACT_QUANT = 32
 OPT_CODEBOOK_CACHE = 1
 OPT_GEMV_ROW_TILES = 2
 OPT_ROWS16_ROW_TILES = 3

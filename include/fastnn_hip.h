@@ -61,7 +61,16 @@ enum {
     FNN_FLAG_ACT_F16_SINGLE = 1 << 2, /* MFMA path: round activations to f16 once (default keeps  */
                                       /* a second f16 residual term, i.e. ~22 mantissa bits)      */
     FNN_FLAG_FORCE_GENERIC = 1 << 3,  /* take the shape-agnostic kernel (testing aid)             */
-    FNN_FLAG_PREFER_FMA = 1 << 4      /* M <= 4: take the f32 FMA GEMV instead of the MFMA kernel */
+    FNN_FLAG_PREFER_FMA = 1 << 4,     /* M <= 4: take the f32 FMA GEMV instead of the MFMA kernel */
+    FNN_FLAG_ACT_QUANT = 1 << 5       /* fnn_hip_qmatmul, opt-in fast mode, NOT the result of matmul_i8 / matmul_i4 /   */
+                                      /* matmul_f8: the f32 activations are quantised on the way in.  I8 / I4 weights:  */
+                                      /* the reference's own chain quantize_activations (dynamic, one scale per tensor, */
+                                      /* src/backend/cpu/mod.rs:6928-7008) -> matmul_i8_i8 / matmul_i4_i8               */
+                                      /* (src/backend/cpu/microkernels/gemm.rs:1641-1975) -> + bias -> activation, one   */
+                                      /* int8 matrix-core plane, integer accumulators bit-exact against that chain.      */
+                                      /* F8 weights: activations rounded to E4M3 with one power-of-two scale per row,    */
+                                      /* fp8 matrix cores, f32 accumulation; within 5e-2 of max|ref| (3 mantissa bits).  */
+                                      /* Other weight types refuse the flag (FNN_ERR_UNSUPPORTED_OP).                    */
 };
 
 typedef struct fnn_hip_ctx fnn_hip_ctx;

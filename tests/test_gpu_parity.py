@@ -805,3 +805,77 @@ def test_full_size_configs_on_row_sample(ctx, orc, name, dt, k, n, ms):
         rhs = ctx.qmatmul(h, a, n).astype(np.float64) + ctx.qmatmul(h, a2, n).astype(np.float64)
         assert rel_err(lhs, rhs) <= 1e-5
     ctx.release(h)
+
+
+# --------------------------------------------------------------------------- FNN_FLAG_ACT_QUANT (opt-in fast mode)
+@pytest.mark.parametrize("dt", [flib.DT_I8, flib.DT_I4])
+@pytest.mark.parametrize("m,k,n", [(1, 256, 64), (7, 1000, 72), (64, 2048, 300), (256, 4096, 512)])
+def test_act_quant_mode_is_the_reference_i8_activation_chain(ctx, orc, dt, m, k, n):
+    """FNN_FLAG_ACT_QUANT with I8 / I4 weights = quantize_activations (dynamic scale max|x| / 127, zero 0) ->
+    matmul_i8_i8 / matmul_i4_i8 -> + bias -> activation.  Without bias and activation the call gives, bit for bit,
+    what the two entry points of that chain give one after the other (whose payload and integer accumulators are
+    bit-exact against the oracle in their own tests); with them it matches the oracle's chain to 1e-6 (same f32
+    formula; the activation's exponential differs in the last place).  It is NOT the result of matmul_i8: against the
+    f32-activation oracle the difference is the 8-bit activation rounding, a few 1e-3 of max|ref|."""
+    rng = np.random.default_rng(6100 + dt + m + k)
+    pw = fastnn_amd.quantize_weights(dt, _weights(rng, n, k))
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    bias = (rng.standard_normal(n) * 0.01).astype(np.float32)
+    h = ctx.register(pw)
+    po = to_oracle(orc, pw)
+    got = ctx.qmatmul(h, a, n, flags=flib.FLAG_ACT_QUANT)
+    payload = ctx.quantize_activations(a)
+    assert payload.tobytes() == orc.quantize_activations(a).tobytes()
+    two_calls = ctx.qmatmul_i8act(h, payload, m, n)
+    two_calls = two_calls[0] if isinstance(two_calls, tuple) else two_calls
+    assert np.array_equal(got, two_calls)
+    want = orc.qmatmul_i8act(po, orc.quantize_activations(a), m)
+    assert_close(got, want, 1e-6, f"act-quant {NAMES[dt]} {m}x{k}x{n}")
+    for act in (1, 3):
+        got_e = ctx.qmatmul(h, a, n, bias=bias, act=act, flags=flib.FLAG_ACT_QUANT)
+        assert_close(got_e, orc.act_fn((want + bias).astype(np.float32), act), 1e-6, f"epilogue {act}")
+        gen = ctx.qmatmul(h, a, n, bias=bias, act=act, flags=flib.FLAG_ACT_QUANT | flib.FLAG_FORCE_GENERIC)
+        assert_close(gen, got_e, 1e-6, "shape-agnostic kernel")
+    exact = orc.qmatmul(po, a, order=2)
+    err = rel_err(got, exact)
+    assert 1e-5 < err < 2e-2, err        # a different function from matmul_i8 / matmul_i4, close to it
+    ctx.release(h)
+
+
+@pytest.mark.parametrize("m,k,n", [(3, 256, 64), (64, 2048, 300), (256, 4096, 512), (130, 1024, 1100)])
+def test_act_quant_mode_fp8_matrix_cores(ctx, orc, m, k, n):
+    """FNN_FLAG_ACT_QUANT with F8 weights: each activation row is scaled by a power of two (row maximum into
+    [128, 256)) and rounded to nearest-even E4M3, v_mfma_f32_32x32x16_fp8_fp8 multiplies the E4M3 bytes of both
+    operands exactly and accumulates in f32.  Checked against the same computation in numpy (activations rounded to
+    E4M3 through torch's float8_e4m3fn, f64 product with the dequantised weights): 1e-4 of max|ref| (measured 2e-5,
+    spread evenly over the outputs: the fp8 matrix core aligns the products of a step with fewer guard bits than a
+    chain of f32 fused multiply-adds; a wrong scale, byte order or rounding mode would show as 1e-2); against the
+    f32-activation oracle the 3-bit mantissa of the activations shows: below 5e-2 of max|ref| (stated tolerance of
+    the mode).  Other weight types refuse the flag."""
+    import torch
+    rng = np.random.default_rng(6200 + m + k)
+    pw = fastnn_amd.quantize_weights(flib.DT_F8, _weights(rng, n, k))
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    a[0] *= 1e-3
+    a[m - 1] *= 3e4
+    bias = (rng.standard_normal(n) * 0.01).astype(np.float32)
+    h = ctx.register(pw)
+    po = to_oracle(orc, pw)
+    got = ctx.qmatmul(h, a, n, bias=bias, act=1, flags=flib.FLAG_ACT_QUANT)
+    mx = np.abs(a).max(axis=1)
+    ex = np.where(mx > 0, np.floor(np.log2(np.maximum(mx, 1e-300))) - 7, 0.0)
+    scaled = (a / (2.0 ** ex)[:, None]).astype(np.float32)
+    a8 = torch.from_numpy(scaled).to(torch.float8_e4m3fn).to(torch.float32).numpy().astype(np.float64) * (2.0 ** ex)[:, None]
+    deq = orc.dequant(po).astype(np.float64)
+    want = np.maximum(a8 @ deq.T + bias, 0.0)
+    assert_close(got, want, 1e-4, f"fp8 act-quant {m}x{k}x{n}")
+    exact = orc.qmatmul(po, a, order=2, bias=bias, act=1)
+    assert rel_err(got, exact) < 5e-2
+    ctx.release(h)
+    for dt in (flib.DT_U8, flib.DT_F4, flib.DT_I4CB):
+        pw2 = fastnn_amd.quantize_weights(dt, _weights(rng, 32, 64))
+        h2 = ctx.register(pw2)
+        with pytest.raises(flib.FnnError) as e:
+            ctx.qmatmul(h2, a[:, :64].copy(), 32, flags=flib.FLAG_ACT_QUANT)
+        assert e.value.kind == "UnsupportedOp"
+        ctx.release(h2)
