@@ -693,6 +693,39 @@ int fnn_hip_dequantize_activations(fnn_hip_ctx *ctx, const uint8_t *payload, uin
     });
 }
 
+int fnn_hip_quantize_activations_per_channel(fnn_hip_ctx *ctx, const float *x_dev, uint64_t x_len, uint64_t numel, uint32_t num_channels,
+                                             const float *scales, const float *zero_points, uint8_t *payload_dev, uint64_t payload_len)
+{
+    return guarded(ctx, "fnn_hip_quantize_activations_per_channel", [&]() -> int {
+        if (!ctx || !x_dev || !payload_dev || !scales || !zero_points)
+            return fail(ctx, FNN_ERR_DISPATCH, "quantize_activations (per channel): NULL argument");
+        if (num_channels == 0) return fail(ctx, FNN_ERR_DISPATCH, "quantize_activations (per channel): no channels");
+        if ((reinterpret_cast<uintptr_t>(payload_dev) & 3) || (reinterpret_cast<uintptr_t>(x_dev) & 3))
+            return fail(ctx, FNN_ERR_DISPATCH, "quantize_activations (per channel): the input and the payload must be 4-byte aligned");
+        const uint64_t header = 8 + (uint64_t)num_channels * 8;
+        if (payload_len < header)
+            return fail(ctx, FNN_ERR_DISPATCH, "quantize_activations (per channel): the payload holds %llu bytes, the header of %u channels takes %llu",
+                        (unsigned long long)payload_len, num_channels, (unsigned long long)header);
+        if (numel / num_channels > 0xffffffffull)
+            return fail(ctx, FNN_ERR_DISPATCH, "quantize_activations (per channel): %llu elements per channel do not fit the header's u32",
+                        (unsigned long long)(numel / num_channels));
+        HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_quantize_activations_per_channel(x_dev, x_len, numel, num_channels, scales, zero_points, payload_dev,
+                                                                              payload_len, ctx->stream));
+        return FNN_OK;
+    });
+}
+
+int fnn_hip_dequantize_activations_per_channel(fnn_hip_ctx *ctx, const uint8_t *payload_dev, uint64_t payload_len, float *out_dev, uint64_t out_len)
+{
+    return guarded(ctx, "fnn_hip_dequantize_activations_per_channel", [&]() -> int {
+        if (!ctx || ((!payload_dev || !out_dev) && out_len)) return fail(ctx, FNN_ERR_DISPATCH, "dequantize_activations (per channel): NULL argument");
+        if (reinterpret_cast<uintptr_t>(payload_dev) & 3) return fail(ctx, FNN_ERR_DISPATCH, "dequantize_activations (per channel): payload must be 4-byte aligned");
+        if (payload_len < 8) return fail(ctx, FNN_ERR_DISPATCH, "dequantize_activations (per channel): a payload of %llu bytes has no header", (unsigned long long)payload_len);
+        HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_dequantize_activations_per_channel(payload_dev, payload_len, out_dev, out_len, ctx->stream));
+        return FNN_OK;
+    });
+}
+
 int fnn_hip_qmatmul_i8act(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const uint8_t *payload,
                           int64_t m, float *out, int32_t *acc_out, int flags)
 {

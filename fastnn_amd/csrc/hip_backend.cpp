@@ -386,9 +386,23 @@ int run_quantize_activations(fnn_backend *b, const Instr &in)
 {
     uint64_t numel = in.params.empty() ? 0 : in.params[0];
     bool per_channel = in.params.size() > 1 && in.params[1] == 1 && in.params.size() > 2 && in.params[2] > 0;
-    if (per_channel) return fail(b, FNN_ERR_UNSUPPORTED_OP, "quantize_activations: per-channel payloads are not implemented on the GPU");
     if (in.inputs.empty()) return FNN_OK;
     const fnn_slice &xs = in.inputs[0];
+    if (per_channel) {
+        // params [numel, 1, nc, scale bits x nc, zero-point bits x nc] (src/backend/cpu/mod.rs:2335-2350)
+        const uint64_t nc = in.params[2];
+        if (nc > 0xffffffffull || in.params.size() < 3 + 2 * nc)
+            return fail(b, FNN_ERR_DISPATCH, "quantize_activations: %llu channels need %llu params, the instruction has %llu",
+                        (unsigned long long)nc, (unsigned long long)(3 + 2 * nc), (unsigned long long)in.params.size());
+        std::vector<float> sc(nc), zp(nc);
+        for (uint64_t c = 0; c < nc; c++) {
+            const uint32_t sb = (uint32_t)in.params[3 + c], zb = (uint32_t)in.params[3 + nc + c];
+            memcpy(&sc[c], &sb, 4);
+            memcpy(&zp[c], &zb, 4);
+        }
+        return lift(b, fnn_hip_quantize_activations_per_channel(b->ctx, (const float *)(b->arena + xs.offset), xs.size / 4, numel, (uint32_t)nc,
+                                                                sc.data(), zp.data(), b->arena + in.dst.offset, in.dst.size));
+    }
     if (in.dst.size < 8) return fail(b, FNN_ERR_DISPATCH, "quantize_activations: output slice has no room for the header");
     uint64_t cap = in.dst.size - 8;
     if (numel > cap) numel = cap;  // min(out_bytes.len() - header, numel)
@@ -409,8 +423,10 @@ int run_dequantize_activations(fnn_backend *b, const Instr &in)
 {
     uint64_t numel = in.params.empty() ? 0 : in.params[0];
     bool per_channel = in.params.size() > 2 && in.params[1] == 1 && in.params[2] > 0;
-    if (per_channel) return fail(b, FNN_ERR_UNSUPPORTED_OP, "dequantize_activations: per-channel payloads are not implemented on the GPU");
     if (in.inputs.empty()) return FNN_OK;
+    if (per_channel)   // (channel count, chunk and the scales come from the payload's header, as in the reference)
+        return lift(b, fnn_hip_dequantize_activations_per_channel(b->ctx, b->arena + in.inputs[0].offset, in.inputs[0].size,
+                                                                  (float *)(b->arena + in.dst.offset), in.dst.size / 4));
     const uint64_t out_len = in.dst.size / 4;
     if (numel > out_len) numel = out_len;   // out_f32.len().min(numel)
     return lift(b, fnn_hip_dequantize_activations(b->ctx, b->arena + in.inputs[0].offset, in.inputs[0].size,

@@ -103,6 +103,12 @@ __device__ __forceinline__ void conv_fold_partial_ranges(const float *part, int 
 hipError_t launch_quantize_activations(const float *x, int64_t numel, float scale, float zp,
                                        uint8_t *payload, float *scratch_partial, hipStream_t s);
 hipError_t launch_dequantize_activations(const uint8_t *payload, uint64_t payload_len, float *out, uint64_t n, hipStream_t s);
+// per-channel payloads ([nc u32][chunk u32][scales][zero points][chunk code bytes], chunk = numel / nc); scales and
+// zero_points are host arrays of nc values, the header is at most 4 GiB (checked by the caller)
+constexpr uint32_t PC_HEADER_VALS = 128;   // header values per launch of the header kernel
+hipError_t launch_quantize_activations_per_channel(const float *x, uint64_t x_len, uint64_t numel, uint32_t nc, const float *scales,
+                                                   const float *zero_points, uint8_t *payload, uint64_t payload_len, hipStream_t s);
+hipError_t launch_dequantize_activations_per_channel(const uint8_t *payload, uint64_t payload_len, float *out, uint64_t out_len, hipStream_t s);
 hipError_t launch_qgemm_i8act_generic(int dtype, const I8ActArgs &p, hipStream_t s);
 hipError_t launch_row_qsum(const fnn_hip_weight *w, int32_t *out, hipStream_t s);
 // phase 0: everything with the direct kernel; 1: range scan + scales; 2: the direct kernel only (scales present);

@@ -148,7 +148,94 @@ __global__ void __launch_bounds__(256) dequantize_act_kernel(const uint8_t *payl
     }
 }
 
+// ---- per-channel payloads, as the reference's loops write and read them (src/backend/cpu/mod.rs:6941-6975,
+// 7026-7061): header [num_channels u32][chunk u32][scale f32 x nc][zero point f32 x nc], chunk = numel / nc, and ONE
+// block of chunk code bytes behind it that every channel's loop addresses from its start (byte `local` of channel ch
+// is the code of x[ch * chunk + local]).  The quantiser's channels run in ascending order, so a byte keeps the code
+// of the last channel that has an element at that position; the dequantiser reads the same block for every channel.
+
+struct HeaderVals { float v[PC_HEADER_VALS]; };
+
+// scales [first, first + count) and their zero points into the header (values travel as kernel arguments)
+__global__ void __launch_bounds__(PC_HEADER_VALS) pc_header_kernel(uint8_t *payload, uint32_t nc, uint32_t chunk, uint32_t first,
+                                                                  uint32_t count, HeaderVals sc, HeaderVals zp)
+{
+    const uint32_t t = threadIdx.x;
+    if (first == 0 && t == 0) {
+        reinterpret_cast<uint32_t *>(payload)[0] = nc;
+        reinterpret_cast<uint32_t *>(payload)[1] = chunk;
+    }
+    if (t < count) {
+        reinterpret_cast<float *>(payload + 8)[first + t] = sc.v[t];
+        reinterpret_cast<float *>(payload + 8 + (size_t)nc * 4)[first + t] = zp.v[t];
+    }
+}
+
+__global__ void __launch_bounds__(256) quantize_act_pc_kernel(const float *x, uint64_t x_len, uint32_t nc, uint64_t chunk, uint8_t *payload,
+                                                              uint64_t payload_len)
+{
+    const uint64_t header = 8 + (uint64_t)nc * 8;
+    const float *sc = reinterpret_cast<const float *>(payload + 8), *zps = sc + nc;
+    for (uint64_t local = (uint64_t)blockIdx.x * 256 + threadIdx.x; local < chunk; local += (uint64_t)gridDim.x * 256) {
+        if (header + local >= payload_len || local >= x_len) break;   // no room for the byte / no channel has the element
+        uint64_t ch = (x_len - 1 - local) / chunk;   // the last channel whose element `local` lies inside the input
+        if (ch > nc - 1) ch = nc - 1;
+        const float scale = sc[ch], zp = zps[ch];
+        int qi = 0;
+        if (scale != 0.0f) {
+            const float t = roundf((x[ch * chunk + local] - zp) / scale);
+            qi = (t != t) ? 0 : (int)fminf(fmaxf(t, -128.0f), 127.0f);   // (a NaN casts to 0)
+        }
+        payload[header + local] = (uint8_t)(int8_t)qi;
+    }
+}
+
+__global__ void __launch_bounds__(256) dequantize_act_pc_kernel(const uint8_t *payload, uint64_t payload_len, float *out, uint64_t out_len)
+{
+    if (payload_len < 8) return;
+    const uint64_t nc = reinterpret_cast<const uint32_t *>(payload)[0], chunk = reinterpret_cast<const uint32_t *>(payload)[1];
+    const uint64_t data = 8 + nc * 8;
+    if (data > payload_len || chunk == 0) return;   // (a header that does not fit its payload: nothing is written)
+    const float *sc = reinterpret_cast<const float *>(payload + 8), *zps = sc + nc;
+    const uint64_t total = nc * chunk < out_len ? nc * chunk : out_len;
+    for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (uint64_t)gridDim.x * 256) {
+        const uint64_t ch = i / chunk, di = data + (i - ch * chunk);
+        const int q = di < payload_len ? (int)(int8_t)payload[di] : 0;
+        out[i] = __fadd_rn(__fmul_rn((float)q, sc[ch]), zps[ch]);
+    }
+}
+
 }  // namespace
+
+hipError_t launch_quantize_activations_per_channel(const float *x, uint64_t x_len, uint64_t numel, uint32_t nc, const float *scales,
+                                                   const float *zero_points, uint8_t *payload, uint64_t payload_len, hipStream_t s)
+{
+    const uint64_t chunk = numel / nc;
+    for (uint32_t first = 0; first < nc; first += PC_HEADER_VALS) {
+        const uint32_t count = nc - first < PC_HEADER_VALS ? nc - first : PC_HEADER_VALS;
+        HeaderVals sc, zp;
+        for (uint32_t i = 0; i < PC_HEADER_VALS; i++) {
+            sc.v[i] = i < count ? scales[first + i] : 0.0f;
+            zp.v[i] = i < count ? zero_points[first + i] : 0.0f;
+        }
+        hipLaunchKernelGGL(pc_header_kernel, dim3(1), dim3(PC_HEADER_VALS), 0, s, payload, nc, (uint32_t)chunk, first, count, sc, zp);
+    }
+    if (chunk > 0) {
+        uint64_t blocks = (chunk + 255) / 256;
+        if (blocks > 4096) blocks = 4096;
+        hipLaunchKernelGGL(quantize_act_pc_kernel, dim3((unsigned)blocks), dim3(256), 0, s, x, x_len, nc, chunk, payload, payload_len);
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_dequantize_activations_per_channel(const uint8_t *payload, uint64_t payload_len, float *out, uint64_t out_len, hipStream_t s)
+{
+    if (out_len == 0) return hipSuccess;
+    uint64_t blocks = (out_len + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(dequantize_act_pc_kernel, dim3((unsigned)blocks), dim3(256), 0, s, payload, payload_len, out, out_len);
+    return hipGetLastError();
+}
 
 hipError_t launch_dequantize_activations(const uint8_t *payload, uint64_t payload_len, float *out, uint64_t n, hipStream_t s)
 {

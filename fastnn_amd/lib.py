@@ -53,7 +53,7 @@ EXPORTED_SYMBOLS = [
     "fnn_hip_device_count", "fnn_hip_create", "fnn_hip_destroy", "fnn_hip_last_error", "fnn_hip_sync", "fnn_hip_set_option", "fnn_hip_get_option", "fnn_hip_stream",
     "fnn_hip_malloc", "fnn_hip_free", "fnn_hip_upload", "fnn_hip_download",
     "fnn_hip_weight_register", "fnn_hip_weight_lookup", "fnn_hip_weight_release", "fnn_hip_dequant",
-    "fnn_hip_qmatmul", "fnn_hip_qmatmul_static", "fnn_hip_quantize_activations", "fnn_hip_dequantize_activations", "fnn_hip_qmatmul_i8act", "fnn_hip_qconv2d", "fnn_hip_qconv2d_i8act",
+    "fnn_hip_qmatmul", "fnn_hip_qmatmul_static", "fnn_hip_quantize_activations", "fnn_hip_dequantize_activations", "fnn_hip_quantize_activations_per_channel", "fnn_hip_dequantize_activations_per_channel", "fnn_hip_qmatmul_i8act", "fnn_hip_qconv2d", "fnn_hip_qconv2d_i8act",
     "fnn_hip_timer_start", "fnn_hip_timer_stop",
     "fnn_hip_graph_begin", "fnn_hip_graph_end", "fnn_hip_graph_launch", "fnn_hip_graph_destroy",
     "fnn_hip_workspace_epoch",
@@ -151,6 +151,8 @@ def _prototype(l):
     l.fnn_hip_qmatmul.argtypes = [_vp, _vp, _vp, _i64, _vp, C.c_int, _vp, C.c_int]
     l.fnn_hip_qmatmul_static.argtypes = [_vp, _vp, _vp, _i64, _vp, C.c_int, _vp, C.c_int]
     l.fnn_hip_quantize_activations.argtypes = [_vp, _vp, _i64, C.c_float, C.c_float, _vp, C.c_int]
+    l.fnn_hip_quantize_activations_per_channel.argtypes = [_vp, _vp, C.c_uint64, C.c_uint64, C.c_uint32, _vp, _vp, _vp, C.c_uint64]
+    l.fnn_hip_dequantize_activations_per_channel.argtypes = [_vp, _vp, C.c_uint64, _vp, C.c_uint64]
     l.fnn_hip_qmatmul_i8act.argtypes = [_vp, _vp, _vp, _i64, _vp, _vp, C.c_int]
     l.fnn_hip_qconv2d.argtypes = [_vp, _vp, _vp, _i64, _i64, _i64, _i64, C.c_int, C.c_int, C.c_int, C.c_int,
                                   C.c_int, C.c_int, _vp, C.c_int, _vp, _vp, C.c_int]
@@ -416,6 +418,38 @@ class HipContext:
         self._check(self.lib.fnn_hip_quantize_activations(self.handle, _np_ptr(x), x.size, scale, zp,
                                                           _np_ptr(payload), 0))
         return payload
+
+    def quantize_activations_per_channel(self, x: np.ndarray, numel: int, scales, zero_points, payload: np.ndarray) -> np.ndarray:
+        """Per-channel "quantize_activations" over the f32 values `x` (all of them readable: x_len = x.size) into a copy
+        of `payload` (its bytes beyond what the kernel writes stay as passed in); returns the payload bytes."""
+        x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1)
+        sc = np.ascontiguousarray(scales, dtype=np.float32)
+        zp = np.ascontiguousarray(zero_points, dtype=np.float32)
+        assert sc.size == zp.size
+        payload = np.ascontiguousarray(payload, dtype=np.uint8)
+        dx, dp = self.to_device(x), self.to_device(payload)
+        try:
+            self._check(self.lib.fnn_hip_quantize_activations_per_channel(self.handle, _vp(dx.ptr), x.size, numel, sc.size, _np_ptr(sc),
+                                                                          _np_ptr(zp), _vp(dp.ptr), payload.size))
+            self.sync()
+            return dp.download(np.uint8, payload.size)
+        finally:
+            dx.free()
+            dp.free()
+
+    def dequantize_activations_per_channel(self, payload: np.ndarray, out: np.ndarray) -> np.ndarray:
+        """Per-channel "dequantize_activations" of `payload` over a copy of the f32 array `out` (values the kernel does
+        not write stay as passed in)."""
+        payload = np.ascontiguousarray(payload, dtype=np.uint8)
+        out = np.ascontiguousarray(out, dtype=np.float32).reshape(-1)
+        dp, do = self.to_device(payload), self.to_device(out)
+        try:
+            self._check(self.lib.fnn_hip_dequantize_activations_per_channel(self.handle, _vp(dp.ptr), payload.size, _vp(do.ptr), out.size))
+            self.sync()
+            return do.download(np.float32, out.size)
+        finally:
+            dp.free()
+            do.free()
 
     def qmatmul_i8act(self, wh, payload: np.ndarray, m: int, n: int, want_acc: bool = False, flags: int = 0):
         payload = np.ascontiguousarray(payload, dtype=np.uint8)

@@ -213,6 +213,24 @@ int fnn_hip_quantize_activations(fnn_hip_ctx *ctx, const float *x, int64_t numel
 int fnn_hip_dequantize_activations(fnn_hip_ctx *ctx, const uint8_t *payload, uint64_t payload_len,
                                    float *out, uint64_t n);
 
+/* kernels "quantize_activations" / "dequantize_activations", per-channel form (src/backend/cpu/mod.rs:6941-6975,
+ * 7026-7061), with the results those loops produce as written.  payload = [num_channels u32][chunk u32]
+ * [scale f32 x nc][zero point f32 x nc][chunk x i8], chunk = numel / num_channels: every channel's loop addresses the
+ * ONE block of chunk code bytes from its start, in ascending channel order, so byte `local` ends as the code of
+ * x[ch*chunk + local] under (scale[ch], zero[ch]) of the last channel ch with ch*chunk + local < x_len (code 0 where
+ * that scale is 0); bytes at or past payload_len are not written.  The dequantiser takes nc and chunk from the header
+ * and writes out[ch*chunk + local] = code[local]*scale[ch] + zero[ch] for ch*chunk + local < out_len (code 0 past the
+ * payload's end); a header that does not fit its payload (the reference panics) leaves `out` untouched.
+ * x_dev / payload_dev / out_dev are device pointers (4-byte aligned), scales / zero_points host arrays of num_channels
+ * values (passed on by value, so the call may be captured); x_len = f32 values readable at x_dev, out_len = f32 values
+ * writable at out_dev.  Queued on the context's stream.  FNN_ERR_DISPATCH: num_channels == 0, a payload too small for
+ * its header (the reference panics on both), chunk >= 2^32. */
+int fnn_hip_quantize_activations_per_channel(fnn_hip_ctx *ctx, const float *x_dev, uint64_t x_len, uint64_t numel,
+                                             uint32_t num_channels, const float *scales, const float *zero_points,
+                                             uint8_t *payload_dev, uint64_t payload_len);
+int fnn_hip_dequantize_activations_per_channel(fnn_hip_ctx *ctx, const uint8_t *payload_dev, uint64_t payload_len,
+                                               float *out_dev, uint64_t out_len);
+
 /* "matmul_i8_i8" / "matmul_i4_i8": gemm_cpu_flat_i8_i8x4 / gemm_cpu_flat_i8_i4x8
  * (src/backend/cpu/microkernels/gemm.rs:1641-1975).  acc_out (nullable, [M,N]
  * i32) receives the exact integer accumulators sum q_w*q_a when zp_a == 0. */

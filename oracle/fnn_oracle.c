@@ -22,6 +22,9 @@
  *   f32 MatMul ............. closed-form literals microkernels/tests.rs:369-763,
  *                            seeded end-to-end bounds tests/cpu_reference_oracle.rs
  *   I8-activation MatMul ... exact integers; literals microkernels/tests.rs:369-678
+ *   per-channel activation payloads ... hand-worked byte images (a later channel overwrites an earlier one's
+ *                            codes), the closed form "codes of the last channel in range", the per-tensor functions on
+ *                            one channel
  *   conv lowering .......... (I8 and I4 weights) equals float conv of dequantised operands; integer
  *                            accumulators exact; brute-force direct convolution; activation
  *                            quantiser re-derived in f32; flat-input special cases
@@ -931,6 +934,71 @@ void fnn_or_quantize_activations_calibrated(const float *x, size_t numel, float 
         float q = clampf(roundf((x[i] - zp) / scale), -128.0f, 127.0f);
         payload[8 + i] = (uint8_t)(int8_t)sat_i32(q, -128, 127);
     }
+}
+
+/* "quantize_activations", per-channel form (backend/cpu/mod.rs:6941-6975), loop for loop as written there:
+ * the header, then for every channel in ascending order its chunk of codes, each chunk written from the first
+ * byte behind the header (`header_offset + local`), so a later channel overwrites an earlier one.  x_len = length of
+ * the f32 input view, payload_len = length of the output byte view; bytes the loops do not reach keep their value.
+ * Returns -1 where the reference would panic on a slice index (header does not fit), else 0. */
+int fnn_or_quantize_activations_per_channel(const float *x, size_t x_len, size_t numel, size_t num_channels,
+                                            const float *scales, const float *zero_points, uint8_t *payload,
+                                            size_t payload_len)
+{
+    if (num_channels == 0) return -1;
+    size_t chunk_size = numel / num_channels;
+    size_t header_offset = 4 + 4 + num_channels * 8;
+    if (payload_len < header_offset) return -1;
+    uint32_t nc32 = (uint32_t)num_channels, chunk32 = (uint32_t)chunk_size;
+    memcpy(payload, &nc32, 4);
+    memcpy(payload + 4, &chunk32, 4);
+    size_t scale_start = 8, zp_start = 8 + num_channels * 4;
+    for (size_t ch = 0; ch < num_channels; ch++) {
+        float scale = scales[ch], zp = zero_points[ch];
+        memcpy(payload + scale_start + ch * 4, &scale, 4);
+        memcpy(payload + zp_start + ch * 4, &zp, 4);
+        size_t ch_start = ch * chunk_size;
+        size_t ch_end = ch_start + chunk_size < x_len ? ch_start + chunk_size : x_len;
+        for (size_t i = ch_start; i < ch_end; i++) {
+            size_t local = i - ch_start;
+            if (header_offset + local < payload_len) {
+                int8_t q = 0;
+                if (scale != 0.0f)
+                    q = (int8_t)sat_i32(clampf(roundf((x[i] - zp) / scale), -128.0f, 127.0f), -128, 127);
+                payload[header_offset + local] = (uint8_t)q;
+            }
+        }
+    }
+    return 0;
+}
+
+/* "dequantize_activations", per-channel form (backend/cpu/mod.rs:7026-7061): channel count and chunk from the
+ * header, out[ch*chunk + local] = (q[local] as f32)*scale[ch] + zp[ch], every channel reading the block behind the
+ * header from its start, q = 0 past the payload.  Returns -1 where the reference would panic (header slices past
+ * the payload), else 0. */
+int fnn_or_dequantize_activations_per_channel(const uint8_t *payload, size_t payload_len, float *out, size_t out_len)
+{
+    if (payload_len < 8) return -1;
+    uint32_t nc32, chunk32;
+    memcpy(&nc32, payload, 4);
+    memcpy(&chunk32, payload + 4, 4);
+    size_t nc = nc32, chunk_size = chunk32;
+    size_t data_start = 8 + nc * 8;
+    if (data_start > payload_len) return -1;
+    for (size_t ch = 0; ch < nc; ch++) {
+        float scale, zp;
+        memcpy(&scale, payload + 8 + ch * 4, 4);
+        memcpy(&zp, payload + 8 + nc * 4 + ch * 4, 4);
+        size_t ch_start = ch * chunk_size;
+        size_t ch_end = ch_start + chunk_size < out_len ? ch_start + chunk_size : out_len;
+        for (size_t i = ch_start; i < ch_end; i++) {
+            size_t di = data_start + (i - ch_start);
+            int8_t q = di < payload_len ? (int8_t)payload[di] : 0;
+            volatile float prod = (float)q * scale;   /* two roundings, no contraction */
+            out[i] = prod + zp;
+        }
+    }
+    return 0;
 }
 
 /* microkernels/gemm.rs:1641-1788 (I8 weights) and :1795-1975 (I4 weights),

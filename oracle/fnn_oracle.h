@@ -87,6 +87,10 @@ float fnn_or_act(float x, int act);
 void fnn_or_quantize_activations(const float *x, size_t numel, uint8_t *payload);
 /* "dequantize_activations", per-tensor form (backend/cpu/mod.rs:7063-7086) */
 void fnn_or_dequantize_activations(const uint8_t *payload, size_t payload_len, float *out, size_t n);
+int fnn_or_quantize_activations_per_channel(const float *x, size_t x_len, size_t numel, size_t num_channels,
+                                            const float *scales, const float *zero_points, uint8_t *payload,
+                                            size_t payload_len);
+int fnn_or_dequantize_activations_per_channel(const uint8_t *payload, size_t payload_len, float *out, size_t out_len);
 void fnn_or_quantize_activations_calibrated(const float *x, size_t numel, float scale, float zp,
                                             uint8_t *payload);
 int  fnn_or_qmatmul_i8act(int dt, const uint32_t *words, size_t n, size_t k,

@@ -119,6 +119,10 @@ def _proto(l):
     l.fnn_or_quantize_activations.argtypes = [_f32p, _sz, _u8p]
     l.fnn_or_dequantize_activations.argtypes = [_u8p, _sz, _f32p, _sz]
     l.fnn_or_quantize_activations_calibrated.argtypes = [_f32p, _sz, C.c_float, C.c_float, _u8p]
+    l.fnn_or_quantize_activations_per_channel.argtypes = [_f32p, _sz, _sz, _sz, _f32p, _f32p, _u8p, _sz]
+    l.fnn_or_quantize_activations_per_channel.restype = C.c_int
+    l.fnn_or_dequantize_activations_per_channel.argtypes = [_u8p, _sz, _f32p, _sz]
+    l.fnn_or_dequantize_activations_per_channel.restype = C.c_int
     l.fnn_or_qmatmul_i8act.argtypes = [C.c_int, _u32p, _sz, _sz, C.c_void_p, _sz, C.c_void_p, _sz,
                                        _u8p, _sz, _sz, _f32p, C.c_void_p]
     l.fnn_or_conv_out_size.argtypes = [_sz] * 5
@@ -292,6 +296,26 @@ def dequantize_activations(payload, n: int) -> np.ndarray:
     payload = np.ascontiguousarray(payload, np.uint8)
     out = np.zeros(n, np.float32)
     lib().fnn_or_dequantize_activations(payload, payload.size, out, n)
+    return out
+
+
+def quantize_activations_per_channel(x, numel: int, scales, zero_points, payload) -> np.ndarray:
+    """The per-channel loops over a copy of `payload` (bytes they do not reach keep their value); ValueError where
+    the reference would panic on a slice index."""
+    x = _f32(x).reshape(-1)
+    sc, zp = _f32(scales).reshape(-1), _f32(zero_points).reshape(-1)
+    assert sc.size == zp.size
+    payload = np.ascontiguousarray(payload, np.uint8).copy()
+    if lib().fnn_or_quantize_activations_per_channel(x, x.size, numel, sc.size, sc, zp, payload, payload.size) != 0:
+        raise ValueError("quantize_activations (per channel): the header does not fit the payload")
+    return payload
+
+
+def dequantize_activations_per_channel(payload, out) -> np.ndarray:
+    payload = np.ascontiguousarray(payload, np.uint8)
+    out = _f32(out).reshape(-1).copy()
+    if lib().fnn_or_dequantize_activations_per_channel(payload, payload.size, out, out.size) != 0:
+        raise ValueError("dequantize_activations (per channel): the header does not fit the payload")
     return out
 
 

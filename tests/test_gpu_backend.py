@@ -158,9 +158,46 @@ def test_quantize_then_dequantize_activations(be, orc, calibrated):
     want = orc.dequantize_activations(payload, x.size)
     assert np.array_equal(be.read_arena(*s_y, np.float32), want)
     assert np.array_equal(be.read_arena(*s_short, np.float32), want[:100])
+
+
+@pytest.mark.parametrize("nc,numel", [(4, 1000), (200, 200 * 11 + 3)])
+def test_per_channel_quantize_then_dequantize_activations_plan(be, orc, nc, numel):
+    """The per-channel instructions as the reference's compile emits them (src/backend/cpu/mod.rs:2319-2425: params
+    [numel, 1, nc, scale bits.., zero-point bits..] for both): payload and values bit-identical to the reference's
+    loops (src/backend/cpu/mod.rs:6941-6975, 7026-7061), eager and as a replayed graph; an instruction with too few
+    params and a payload slice without room for its header are dispatch errors (the reference panics on both)."""
+    rng = np.random.default_rng(23 + nc)
+    x = (rng.standard_normal(numel) * 2).astype(np.float32)
+    sc = rng.uniform(0.01, 0.1, nc).astype(np.float32)
+    zp = rng.uniform(-1, 1, nc).astype(np.float32)
+    chunk = numel // nc
+    a = Arena()
+    s_x, s_q, s_y, s_short = a.take(x.nbytes), a.take(8 + 8 * nc + chunk), a.take(x.nbytes), a.take(4 * (chunk + 3))
+    params = [numel, 1, nc] + [int(v) for v in sc.view(np.uint32)] + [int(v) for v in zp.view(np.uint32)]
+    plan = ExecutablePlan(a.top)
+    plan.call_kernel("quantize_activations", [s_x], s_q, params)
+    plan.call_kernel("dequantize_activations", [s_q], s_y, params)
+    plan.call_kernel("dequantize_activations", [s_q], s_short, params)
+    be.allocate_arena(a.top)
+    before_q = np.arange(s_q[1], dtype=np.uint32).astype(np.uint8)
+    before_y = np.full(numel, 5.0, np.float32)
+    want_q = orc.quantize_activations_per_channel(x, numel, sc, zp, before_q)
+    want_y = orc.dequantize_activations_per_channel(want_q, before_y)
+    for rep in range(3):
+        be.write_arena(s_x[0], x)
+        be.write_arena(s_q[0], before_q)
+        be.write_arena(s_y[0], before_y)
+        be.write_arena(s_short[0], before_y[:chunk + 3])
+        be.dispatch(plan)
+        assert np.array_equal(be.read_arena(*s_q), want_q), rep
+        assert np.array_equal(be.read_arena(*s_y, np.float32), want_y), rep
+        assert np.array_equal(be.read_arena(*s_short, np.float32), orc.dequantize_activations_per_channel(want_q, before_y[:chunk + 3])), rep
     with pytest.raises(flib.FnnError) as e:
-        be.dispatch(ExecutablePlan(a.top).call_kernel("dequantize_activations", [s_q], s_y, [x.size, 1, 4]))
-    assert e.value.kind == "UnsupportedOp"
+        be.dispatch(ExecutablePlan(a.top).call_kernel("quantize_activations", [s_x], s_q, params[:-1]))
+    assert e.value.kind == "Dispatch"
+    with pytest.raises(flib.FnnError) as e:
+        be.dispatch(ExecutablePlan(a.top).call_kernel("quantize_activations", [s_x], (s_q[0], 8 * nc), params))
+    assert e.value.kind == "Dispatch"
 
 
 @pytest.mark.parametrize("act,code", [("", 0), ("_relu", 1), ("_silu", 3)])

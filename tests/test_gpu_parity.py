@@ -487,6 +487,48 @@ def test_quantize_activations_bit_exact(ctx, orc, numel):
     assert ctx.quantize_activations(z).tobytes() == orc.quantize_activations(z).tobytes()
 
 
+@pytest.mark.parametrize("nc,numel", [(1, 1), (1, 300), (3, 100), (8, 8 * 4096), (300, 300 * 37 + 5), (64, 40), (5, 100003)])
+def test_per_channel_activation_payloads_bit_exact(ctx, orc, nc, numel):
+    """The per-channel "quantize_activations" / "dequantize_activations" payloads, byte for byte what the reference's
+    loops leave behind (src/backend/cpu/mod.rs:6941-6975, 7026-7061): whole inputs, an input view shorter than numel,
+    a payload that ends inside the code block, zero scales, non-finite values, more channels than one header launch
+    carries, fewer elements than channels (chunk = 0); bytes and values the loops do not reach keep what they held."""
+    rng = np.random.default_rng(900 + nc + numel)
+    x = (rng.standard_normal(numel) * 3).astype(np.float32)
+    if numel > 8:
+        x[[1, 3, 5]] = [np.nan, np.inf, -np.inf]
+    sc = rng.uniform(0.01, 0.1, nc).astype(np.float32)
+    zp = rng.uniform(-1, 1, nc).astype(np.float32)
+    if nc > 2:
+        sc[nc // 2] = 0.0
+    chunk = numel // nc
+    header = 8 + 8 * nc
+    fill = rng.integers(0, 256, header + chunk + 13).astype(np.uint8)
+    cases = [(x, fill), (x, fill[:header + chunk // 2]), (x, fill[:header])]
+    if numel > nc:
+        cases += [(x[:numel - chunk // 2 - 1], fill), (x[:max(1, chunk // 3)], fill)]
+    for xv, pl in cases:
+        want = orc.quantize_activations_per_channel(xv, numel, sc, zp, pl)
+        got = ctx.quantize_activations_per_channel(xv, numel, sc, zp, pl)
+        assert got.tobytes() == want.tobytes(), (xv.size, pl.size)
+    # the last channel under a zero scale: every code is 0
+    sc0 = sc.copy()
+    sc0[-1] = 0.0
+    assert ctx.quantize_activations_per_channel(x, numel, sc0, zp, fill).tobytes() == orc.quantize_activations_per_channel(x, numel, sc0, zp, fill).tobytes()
+    payload = orc.quantize_activations_per_channel(x, numel, sc, zp, fill)
+    old = rng.standard_normal(numel + 9).astype(np.float32)
+    for pl, out in [(payload, old), (payload, old[:max(1, numel - chunk // 2 - 1)]), (payload[:header + chunk // 2], old), (payload[:header], old)]:
+        want = orc.dequantize_activations_per_channel(pl, out)
+        got = ctx.dequantize_activations_per_channel(pl, out)
+        assert got.tobytes() == want.tobytes(), (pl.size, out.size)
+    with pytest.raises(flib.FnnError):   # the header does not fit: the reference panics
+        ctx.quantize_activations_per_channel(x, numel, sc, zp, fill[:header - 1])
+    # a header that claims more channels than the payload holds: nothing is written
+    bad = payload.copy()
+    bad[:4] = np.array([payload.size], np.uint32).view(np.uint8)
+    assert ctx.dequantize_activations_per_channel(bad, old).tobytes() == old.tobytes()
+
+
 @pytest.mark.parametrize("dt", [0, 1])
 @pytest.mark.parametrize("m,k,n", [(1, 64, 32), (3, 61, 10), (16, 256, 64), (40, 1000, 72), (128, 512, 256)])
 @pytest.mark.parametrize("zp", [0.0, 0.375])

@@ -129,3 +129,58 @@ def test_dequantize_activations_inverts_the_payload(orc):
     assert np.abs(orc.dequantize_activations(pl, 500) - x).max() <= 0.5 * s * (1 + 1e-6)
     short = orc.dequantize_activations(payload[:8 + 100], 120)
     assert np.array_equal(short[:100], got[:100]) and np.all(short[100:] == zp)
+
+
+def _pc_payload_image(nc, chunk, scales, zps, codes, tail=b""):
+    """[nc u32][chunk u32][scales][zero points][codes] written out by hand"""
+    return np.concatenate([np.array([nc, chunk], np.uint32).view(np.uint8), np.asarray(scales, np.float32).view(np.uint8),
+                           np.asarray(zps, np.float32).view(np.uint8), np.asarray(codes, np.int8).view(np.uint8),
+                           np.frombuffer(tail, np.uint8)])
+
+
+def test_per_channel_activation_payloads_as_the_reference_loops_write_them(orc):
+    """src/backend/cpu/mod.rs:6941-6975, 7026-7061: every channel's codes start at the first byte behind the header,
+    channels in ascending order, so the block ends as the codes of the last channel in range.  Byte images worked out
+    by hand; the closed form against the per-tensor quantiser on the last chunk; one channel = the per-tensor pair."""
+    x = np.array([1.0, 2.0, 3.0, 10.0, 20.0, 30.0], np.float32)
+    fill = np.full(24 + 6, 0xAA, np.uint8)
+    got = orc.quantize_activations_per_channel(x, 6, [1.0, 5.0], [0.0, 0.0], fill)
+    assert np.array_equal(got, _pc_payload_image(2, 3, [1.0, 5.0], [0.0, 0.0], [2, 4, 6], b"\xaa\xaa\xaa"))
+    # an input view one value short of numel: channel 1 reaches positions 0 and 1 only, position 2 keeps channel 0's code
+    got = orc.quantize_activations_per_channel(x[:5], 6, [1.0, 5.0], [0.0, 0.0], fill)
+    assert np.array_equal(got, _pc_payload_image(2, 3, [1.0, 5.0], [0.0, 0.0], [2, 4, 3], b"\xaa\xaa\xaa"))
+    # a zero scale gives code 0, a zero point shifts before the division, the clamp saturates; a payload that ends
+    # inside the block is filled as far as it goes
+    got = orc.quantize_activations_per_channel(x, 6, [1.0, 0.0], [0.0, 0.0], fill)
+    assert np.array_equal(got[24:27].view(np.int8), [0, 0, 0])
+    got = orc.quantize_activations_per_channel(x, 6, [1.0, 0.1], [0.0, 9.0], fill[:26])
+    assert np.array_equal(got, _pc_payload_image(2, 3, [1.0, 0.1], [0.0, 9.0], [10, 110]))
+    with pytest.raises(ValueError):
+        orc.quantize_activations_per_channel(x, 6, [1.0, 5.0], [0.0, 0.0], fill[:23])
+    # dequantiser: every channel reads the same block
+    img = _pc_payload_image(2, 3, [1.0, 5.0], [0.5, -1.0], [2, 4, 6])
+    out = orc.dequantize_activations_per_channel(img, np.full(7, 99.0, np.float32))
+    assert np.array_equal(out, [2.5, 4.5, 6.5, 9.0, 19.0, 29.0, 99.0])
+    out = orc.dequantize_activations_per_channel(img, np.full(5, 99.0, np.float32))
+    assert np.array_equal(out, [2.5, 4.5, 6.5, 9.0, 19.0])
+    out = orc.dequantize_activations_per_channel(img[:26], np.full(6, 99.0, np.float32))   # codes past the payload read as 0
+    assert np.array_equal(out, [2.5, 4.5, 0.5, 9.0, 19.0, -1.0])
+    with pytest.raises(ValueError):
+        orc.dequantize_activations_per_channel(img[:20], np.zeros(6, np.float32))
+    # closed form on random data
+    rng = np.random.default_rng(77)
+    for nc, numel in [(1, 64), (3, 100), (7, 7 * 33), (16, 16 * 5 + 3)]:
+        xr = (rng.standard_normal(numel) * 3).astype(np.float32)
+        sc = rng.uniform(0.01, 0.1, nc).astype(np.float32)
+        zp = rng.uniform(-1, 1, nc).astype(np.float32)
+        chunk = numel // nc
+        pl = orc.quantize_activations_per_channel(xr, numel, sc, zp, np.zeros(8 + 8 * nc + chunk, np.uint8))
+        last = xr[(nc - 1) * chunk:nc * chunk]
+        assert np.array_equal(pl[8 + 8 * nc:], orc.quantize_activations(last, float(sc[-1]), float(zp[-1]))[8:])
+        deq = orc.dequantize_activations_per_channel(pl, np.full(numel, 7.0, np.float32))
+        q = pl[8 + 8 * nc:].view(np.int8).astype(np.float32)
+        for ch in range(nc):
+            assert np.array_equal(deq[ch * chunk:(ch + 1) * chunk], q * sc[ch] + zp[ch])
+        assert np.all(deq[nc * chunk:] == 7.0)
+        if nc == 1:
+            assert np.array_equal(deq, orc.dequantize_activations(orc.quantize_activations(xr, float(sc[0]), float(zp[0])), numel))
