@@ -144,6 +144,29 @@ def test_qmatmul_matches_oracle(ctx, orc, dt, m, k, n):
     ctx.release(h)
 
 
+@pytest.mark.parametrize("dt", ALL_DT)
+@pytest.mark.parametrize("m,k,n", [(1, 512, 48), (20, 200, 37)])
+def test_oracle_packed_weights_through_the_device(ctx, orc, dt, m, k, n):
+    """The words, scales, zeros and codebook the ORACLE's quantiser produces, registered and multiplied on the device:
+    the product's host packer (which every other test here feeds to both sides) has to produce the same bytes, and
+    the device has to agree with the oracle on a weight image the product did not write."""
+    rng = np.random.default_rng(3300 + dt * 13 + k)
+    w = _weights(rng, n, k, "laplace" if dt == 7 else "normal")
+    w[1] = 0.0
+    w[2] = 0.015
+    po = orc.quantize(dt, w)
+    pw = fastnn_amd.quantize_weights(dt, w)
+    assert np.array_equal(pw.words, po.words) and pw.scales.tobytes() == po.scales.tobytes() and pw.zeros.tobytes() == po.zeros.tobytes()
+    if dt == 7:
+        assert pw.codebook.tobytes() == po.codebook.tobytes() and pw.qblock == po.qblock
+    theirs = flib.PackedWeight(po.dt, po.rows, po.inner, po.words, po.scales, po.zeros, po.qblock, po.codebook)
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    h = ctx.register(theirs)
+    assert_close(ctx.qmatmul(h, a, n), orc.qmatmul(po, a, order=2), TOL_F32, f"{NAMES[dt]} {m}x{k}x{n}")
+    assert ctx.dequant(h, n, k).tobytes() == orc.dequant(po).tobytes()
+    ctx.release(h)
+
+
 @pytest.mark.parametrize("dt", [0, 1, 2, 3, 4, 5, 6])
 @pytest.mark.parametrize("m,k,n", ROW_TILE_SHAPES)
 def test_qmatmul_row_tile_kernels(ctx, orc, dt, m, k, n):
