@@ -479,6 +479,14 @@ TileLayout tile_layout(fnn_hip_ctx *ctx, int64_t M, int64_t N, int64_t K, int fl
     if (meff > 64) cfg = (!dense && ((meff + 127) / 128) * ((N + 127) / 128) <= 128) ? 1 : 0;
     else if (meff == 64) cfg = 1;
     else cfg = 2;
+    // ... unless the 32-row tiles fill the chip in one round without a K split (192..256 of them: no reduction launch,
+    // no partial tiles).  FP8 2048 -> 8192: M = 33 19.0 -> 17.0 us, M = 64 19.4 -> 17.6; FP4: 17.9 -> 14.4, 18.4 -> 14.9;
+    // with fewer or more tiles than that the 64-row tiles and their split stay ahead (4096 x 4096 at M = 64: 19.7 against
+    // 21.6 us; 2048 -> 8192 at M = 96: 21.6 against 25.5).
+    if (cfg == 1 && !dense) {
+        const int64_t small_tiles = ((meff + 31) / 32) * ((N + 127) / 128);
+        if (small_tiles >= 192 && small_tiles <= 256) cfg = 2;
+    }
     const int64_t opt_cfg = fnn_ctx_option(ctx, FNN_OPT_TILE_SHAPE);
     // 3 (by option only): 256x128 with 8 waves of 64x64, two waves per SIMD.  Measured on FP8 4096 x 4096 and 2048 -> 8192
     // at M = 128 ... 1024: 0-30 % slower than the automatic choice, except where it turns the tile count into one whole
