@@ -483,7 +483,10 @@ TileLayout tile_layout(fnn_hip_ctx *ctx, int64_t M, int64_t N, int64_t K, int fl
     // no partial tiles).  FP8 2048 -> 8192: M = 33 19.0 -> 17.0 us, M = 64 19.4 -> 17.6; FP4: 17.9 -> 14.4, 18.4 -> 14.9;
     // with fewer or more tiles than that the 64-row tiles and their split stay ahead (4096 x 4096 at M = 64: 19.7 against
     // 21.6 us; 2048 -> 8192 at M = 96: 21.6 against 25.5).
-    if (cfg == 1 && !dense) {
+    // codebook weights decoded in the kernel: the 64-row tiles at every size (their loop is bound by the vector ALU, and
+    // four waves of 64 x 32 share it better than four of 64 x 64: M = 512 109.6 against 131.6 us, M = 1024 204 against 231)
+    if (DT == FNN_DT_I4CB && meff > 64) cfg = 1;
+    if (cfg == 1 && !dense && meff <= 128 && DT != FNN_DT_I4CB) {   // (measured for up to 64 activation rows; the codebook decode wants the larger tiles)
         const int64_t small_tiles = ((meff + 31) / 32) * ((N + 127) / 128);
         if (small_tiles >= 192 && small_tiles <= 256) cfg = 2;
     }
@@ -557,6 +560,9 @@ int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QM
         const double cost = per * t_stage * wgs + (sp > 1 ? 2.0 * sp * part_us : 0.0);
         if (cost < best * 0.995) { best = cost; splits = sp; }   // on a tie the coarser split wins
     }
+    // the dense operand (128 x 128 tiles, one workgroup per CU): as many splits as fill one round, no more (measured on
+    // 4096 x 4096: 96 tiles 58.0 us with 2 splits against 71.6 with the model's choice, 192 tiles 82.1 with none against 110)
+    if (dense && cfg == 0) splits = base >= 256 ? 1 : 256 / base;
     if (env_split > 0) splits = env_split;
     if (splits > iters / 4) splits = iters / 4 > 0 ? iters / 4 : 1;
     int ips = (iters + splits - 1) / splits;
@@ -823,7 +829,7 @@ int fnn_tiled_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, 
         // vector-ALU bound; the expanded operand's loop is the plain f16 one).
         const int64_t opt_exp = fnn_ctx_option(ctx, FNN_OPT_CODEBOOK_EXPANDED);
         const bool precise = !(flags & FNN_FLAG_ACT_F16_SINGLE);
-        const bool in_kernel = opt_exp == 0 ? (precise ? (q.m < 192 || q.m >= 512) : q.m <= 16) : opt_exp == 2;
+        const bool in_kernel = opt_exp == 0 ? (precise ? (q.m < 192 || q.m >= 1024) : q.m <= 16) : opt_exp == 2;
         if (q.qblock == 32 && in_kernel) {
             QMatmulArgs qa = q;
             int rc;
