@@ -647,6 +647,8 @@ def main() -> int:
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--fast-act16", action="store_true", help="single f16 rounding of activations on the MFMA path")
+    ap.add_argument("--act-quant", action="store_true", help="the opt-in activation-quantised mode (FNN_FLAG_ACT_QUANT; I8 / I4 / F8 weights, "
+                    "M >= 17): NOT parity with the default MatMul")
     ap.add_argument("--no-extra", "--no-m256", dest="no_extra", action="store_true",
                     help="skip the extra legs (K=N=4096 GEMVs, M=256 GEMMs)")
     ap.add_argument("--opt", action="append", default=[], metavar="NAME=VALUE",
@@ -676,6 +678,8 @@ def main() -> int:
 
     m = args.m
     flags = flib.FLAG_ACT_F16_SINGLE if args.fast_act16 else 0
+    if args.act_quant:
+        flags |= flib.FLAG_ACT_QUANT
     ctx = fastnn_amd.HipContext(0)
     opts = {}
     for name, ident, value in parsed_options(args, flib):
@@ -871,7 +875,7 @@ def main() -> int:
         "config": {"workload": f"{args.workload}: {dtn} weights [N={n},K={k}] per-channel, f32 activations "
                                f"[M={m},K={k}] ~N(0,1), bias={has_bias}, act={r['actn']}, seed 0",
                    "m": m, "k": k, "n": n, "weight_ring": ring, "ring_bytes": ring * wbytes, "trips": t["trips"],
-                   "launch": args.mode, "act_rounding": "f16x1" if args.fast_act16 else "default",
+                   "launch": args.mode, "act_rounding": "act_quant (not parity)" if args.act_quant else ("f16x1" if args.fast_act16 else "default"),
                    **({"options": opts} if opts else {})},
         "roofline": roofline,
         "cpu_baseline": cpu,

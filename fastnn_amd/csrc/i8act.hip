@@ -11,9 +11,15 @@ __global__ void __launch_bounds__(256) absmax_partial_kernel(const float *x, int
 {
     __shared__ float sm[4];
     float v = 0.0f;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < numel;
-         i += (int64_t)gridDim.x * blockDim.x)
-        v = fmaxf(v, fabsf(x[i]));  // fmaxf ignores NaN like f32::max
+    // (the maximum does not depend on the order: whole 16-byte groups first, the ragged end value by value)
+    const bool vec = (reinterpret_cast<uintptr_t>(x) & 15) == 0;
+    const int64_t n4 = vec ? numel / 4 : 0;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += (int64_t)gridDim.x * blockDim.x) {
+        const float4 t = reinterpret_cast<const float4 *>(x)[i];
+        v = fmaxf(v, fmaxf(fmaxf(fabsf(t.x), fabsf(t.y)), fmaxf(fabsf(t.z), fabsf(t.w))));  // fmaxf ignores NaN like f32::max
+    }
+    for (int64_t i = n4 * 4 + (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < numel; i += (int64_t)gridDim.x * blockDim.x)
+        v = fmaxf(v, fabsf(x[i]));
     v = wave_max(v);
     if ((threadIdx.x & 63) == 0) sm[threadIdx.x >> 6] = v;
     __syncthreads();
@@ -26,6 +32,13 @@ quantize_act_kernel(const float *x, int64_t numel, const float *partial, int npa
                     float zp, uint8_t *payload)
 {
     __shared__ float s_scale;
+    // the first 16-byte group of every thread is requested before the scale is formed (its latency and that of the
+    // partial maxima overlap)
+    const bool vec = ((reinterpret_cast<uintptr_t>(x) & 15) | (reinterpret_cast<uintptr_t>(payload) & 3)) == 0;
+    const int64_t n4 = vec ? numel / 4 : 0;
+    const int64_t first = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    float4 t0 = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    if (first < n4) t0 = reinterpret_cast<const float4 *>(x)[first];
     if (threadIdx.x < 64) {
         float scale = scale_in;
         if (partial) {
@@ -43,13 +56,20 @@ quantize_act_kernel(const float *x, int64_t numel, const float *partial, int npa
         reinterpret_cast<float *>(payload)[1] = zp;
     }
     int8_t *q = reinterpret_cast<int8_t *>(payload + 8);
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < numel;
-         i += (int64_t)gridDim.x * blockDim.x) {
-        const float t = roundf((x[i] - zp) / scale);
+    auto code = [&](float xv) {
+        const float t = roundf((xv - zp) / scale);
         // clamp keeps NaN and the saturating cast maps NaN to 0
-        const int qi = (t != t) ? 0 : (int)fminf(fmaxf(t, -128.0f), 127.0f);
-        q[i] = (int8_t)qi;
+        return (t != t) ? 0 : (int)fminf(fmaxf(t, -128.0f), 127.0f);
+    };
+    // four values per thread where the input allows 16-byte loads (the payload is 4-byte aligned): one load, one store
+    for (int64_t i = first; i < n4; i += (int64_t)gridDim.x * blockDim.x) {
+        const float4 t = i == first ? t0 : reinterpret_cast<const float4 *>(x)[i];
+        const uint32_t w = (uint32_t)(uint8_t)code(t.x) | ((uint32_t)(uint8_t)code(t.y) << 8) | ((uint32_t)(uint8_t)code(t.z) << 16) |
+                           ((uint32_t)(uint8_t)code(t.w) << 24);
+        reinterpret_cast<uint32_t *>(q)[i] = w;
     }
+    for (int64_t i = n4 * 4 + (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < numel; i += (int64_t)gridDim.x * blockDim.x)
+        q[i] = (int8_t)code(x[i]);
 }
 
 template <int DT>

@@ -85,25 +85,77 @@ __global__ void __launch_bounds__(256) i8_matmul_epilogue_kernel(const int32_t *
                                                                  int64_t m, int64_t n, int64_t k, float *out, int32_t *acc_out, int splits,
                                                                  const float *bias, int act)
 {
-    // a thread owns one output column (its weight constants stay in registers) and walks rows blockIdx.y, +gridDim.y, ...
+    // a thread owns four consecutive output columns (their weight constants stay in registers; 16-byte loads and stores
+    // where n % 4 == 0 and the buffers are aligned) and walks rows blockIdx.y, +gridDim.y, ...
     const float sa = reinterpret_cast<const float *>(payload)[0];
     const float za = reinterpret_cast<const float *>(payload)[1];
-    const int64_t col = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (col >= n) return;
-    const float sw = scales[col], zw = zeros[col];
-    const float zwsum = za * (float)wsum[col];
+    const int64_t col0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (col0 >= n) return;
+    const bool vec = col0 + 4 <= n && n % 4 == 0 &&
+                     ((reinterpret_cast<uintptr_t>(c) | reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(acc_out)) & 15) == 0;
+    float sw[4], zw[4], zwsum[4], bs[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const bool ok = col0 + j < n;
+        sw[j] = ok ? scales[col0 + j] : 0.0f;
+        zw[j] = ok ? zeros[col0 + j] : 0.0f;
+        zwsum[j] = ok ? za * (float)wsum[col0 + j] : 0.0f;
+        bs[j] = (ok && bias) ? bias[col0 + j] : 0.0f;
+    }
     const float kza = (float)k * za;
-    const float bs = bias ? bias[col] : 0.0f;
-    for (int64_t r = blockIdx.y; r < m; r += gridDim.y) {
-        const int64_t idx = r * n + col;
-        int acc = c[idx];
-        for (int z = 1; z < splits; z++) acc += c[(int64_t)z * m * n + idx];   // exact whatever the order
-        const float input_sum = (float)qsum[r] * sa + kza;
-        const float dot = (za != 0.0f) ? (float)acc * sa + zwsum : (float)acc * sa;
-        float v = dot * sw + zw * input_sum;
-        if (bias) v = v + bs;
-        out[idx] = fnn_activation(v, act);
-        if (acc_out) acc_out[idx] = (za != 0.0f) ? 0 : acc;
+    // two rows per trip: both rows' partial sums are requested before either row's arithmetic starts
+    for (int64_t r0 = (int64_t)blockIdx.y * 2; r0 < m; r0 += (int64_t)gridDim.y * 2) {
+        int acc[2][4] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
+        int qs[2] = {0, 0};
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+            const int64_t r = r0 + t;
+            if (r >= m) break;
+            const int64_t idx = r * n + col0;
+            qs[t] = qsum[r];
+            if (vec) {
+                const int4 v0 = *reinterpret_cast<const int4 *>(c + idx);
+                acc[t][0] = v0.x; acc[t][1] = v0.y; acc[t][2] = v0.z; acc[t][3] = v0.w;
+                for (int z = 1; z < splits; z++) {   // exact whatever the order
+                    const int4 u = *reinterpret_cast<const int4 *>(c + (int64_t)z * m * n + idx);
+                    acc[t][0] += u.x; acc[t][1] += u.y; acc[t][2] += u.z; acc[t][3] += u.w;
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    if (col0 + j < n) {
+                        acc[t][j] = c[idx + j];
+                        for (int z = 1; z < splits; z++) acc[t][j] += c[(int64_t)z * m * n + idx + j];
+                    }
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+            const int64_t r = r0 + t;
+            if (r >= m) break;
+            const int64_t idx = r * n + col0;
+            const float input_sum = (float)qs[t] * sa + kza;
+            float o[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const float dot = (za != 0.0f) ? (float)acc[t][j] * sa + zwsum[j] : (float)acc[t][j] * sa;
+                float v = dot * sw[j] + zw[j] * input_sum;
+                if (bias) v = v + bs[j];
+                o[j] = fnn_activation(v, act);
+                if (za != 0.0f) acc[t][j] = 0;
+            }
+            if (vec) {
+                *reinterpret_cast<float4 *>(out + idx) = make_float4(o[0], o[1], o[2], o[3]);
+                if (acc_out) *reinterpret_cast<int4 *>(acc_out + idx) = make_int4(acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    if (col0 + j < n) {
+                        out[idx + j] = o[j];
+                        if (acc_out) acc_out[idx + j] = acc[t][j];
+                    }
+            }
+        }
     }
 }
 
@@ -421,7 +473,7 @@ hipError_t launch_i8_tile(const TileArgs &p, hipStream_t s)
     if (e != hipSuccess) return e;
     // (a ring of three requests only the stages its K range has: one LDS buffer per stage, at most three)
     const int bufs = (NS == 3 && p.ips < NS) ? p.ips : NS;
-    hipLaunchKernelGGL(kern, dim3((unsigned)p.mtiles * p.ntiles * p.splits), dim3(256), lds / NS * bufs, s, p);
+    hipLaunchKernelGGL(kern, dim3((unsigned)p.mtiles * p.ntiles * p.splits), dim3(WGM * WGN * 64), lds / NS * bufs, s, p);
     return hipGetLastError();
 }
 
@@ -463,7 +515,7 @@ namespace {
 template <int DT>
 hipError_t run_i8_gemm(const uint32_t *words, int64_t kp, int64_t rows_total, int64_t n0, int64_t n, const int8_t *a8, int64_t m,
                        int64_t rows_pad, int64_t kpad, int32_t *c, int64_t ldc, hipStream_t s, int splits = 1, const TileArgs *conv = nullptr,
-                       bool small_tiles = false)
+                       bool small_tiles = false, int form = 0)
 {
     TileArgs t = {};
     if (conv) { t.cv = conv->cv; t.scales = conv->scales; t.zeros = conv->zeros; t.bias = conv->bias; t.act = conv->act; }
@@ -486,6 +538,11 @@ hipError_t run_i8_gemm(const uint32_t *words, int64_t kp, int64_t rows_total, in
         return conv ? launch_i8_tile<DT, 4, 1, 1, 2, 3, true>(t, s) : launch_i8_tile<DT, 4, 1, 1, 2, 3>(t, s);
     }
     t.ntiles = (int)((n + 127) / 128);
+    if (!conv && form == 1) return launch_i8_tile<DT, 2, 4, 2, 1, 3>(t, s);      // 128 x 128 on eight waves of 64 x 32
+    if (!conv && form == 2) {                                                    // 256 x 128 on eight waves of 64 x 64
+        t.mtiles = (int)((rows_pad + 255) / 256);
+        return launch_i8_tile<DT, 4, 2, 2, 2, 3>(t, s);
+    }
     return conv ? launch_i8_tile<DT, 2, 2, 2, 2, 3, true>(t, s) : launch_i8_tile<DT, 2, 2, 2, 2, 3>(t, s);
 }
 
@@ -504,8 +561,17 @@ __global__ void __launch_bounds__(256) fp8_rows_operand_kernel(const float *a, i
     const int64_t r = blockIdx.x;
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     float mx = 0.0f;
-    if (r < m)
-        for (int64_t i = tid; i < k; i += 256) mx = fmaxf(mx, fabsf(a[r * k + i]));
+    const bool vec = (k % 4 == 0) && ((reinterpret_cast<uintptr_t>(a) & 15) == 0);   // rows start on 16-byte boundaries
+    if (r < m) {
+        if (vec) {
+            for (int64_t i = tid; i < k / 4; i += 256) {
+                const float4 t = reinterpret_cast<const float4 *>(a + r * k)[i];
+                mx = fmaxf(mx, fmaxf(fmaxf(fabsf(t.x), fabsf(t.y)), fmaxf(fabsf(t.z), fabsf(t.w))));
+            }
+        } else {
+            for (int64_t i = tid; i < k; i += 256) mx = fmaxf(mx, fabsf(a[r * k + i]));
+        }
+    }
     mx = wave_max(mx);
     if (lane == 0) red[wv] = mx;
     __syncthreads();
@@ -520,10 +586,13 @@ __global__ void __launch_bounds__(256) fp8_rows_operand_kernel(const float *a, i
 #pragma unroll
             for (int q = 0; q < 4; q++) {
                 float v[4];
+                const int64_t k0 = c * 16 + q * 4;
+                if (vec && k0 + 4 <= k) {
+                    const float4 t = *reinterpret_cast<const float4 *>(a + r * k + k0);
+                    v[0] = t.x * inv; v[1] = t.y * inv; v[2] = t.z * inv; v[3] = t.w * inv;
+                } else {
 #pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    const int64_t kk = c * 16 + q * 4 + j;
-                    v[j] = kk < k ? a[r * k + kk] * inv : 0.0f;
+                    for (int j = 0; j < 4; j++) v[j] = k0 + j < k ? a[r * k + k0 + j] * inv : 0.0f;
                 }
                 int w = __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], 0, false);
                 w = __builtin_amdgcn_cvt_pk_fp8_f32(v[2], v[3], w, true);
@@ -540,17 +609,61 @@ __global__ void __launch_bounds__(256) fp8_rows_operand_kernel(const float *a, i
 __global__ void __launch_bounds__(256) fp8_matmul_epilogue_kernel(const float *c, const float *rscale, const float *scales, const float *bias,
                                                                   int64_t m, int64_t n, float *out, int splits, int act)
 {
-    const int64_t col = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (col >= n) return;
-    const float sw = scales[col];
-    const float bs = bias ? bias[col] : 0.0f;
-    for (int64_t r = blockIdx.y; r < m; r += gridDim.y) {
-        const int64_t idx = r * n + col;
-        float acc = c[idx];
-        for (int z = 1; z < splits; z++) acc += c[(int64_t)z * m * n + idx];
-        float v = (acc * rscale[r]) * sw;
-        if (bias) v = v + bs;
-        out[idx] = fnn_activation(v, act);
+    // a thread owns four consecutive columns (16-byte loads and stores where n % 4 == 0 and the buffers are aligned)
+    const int64_t col0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (col0 >= n) return;
+    const bool vec = col0 + 4 <= n && n % 4 == 0 && ((reinterpret_cast<uintptr_t>(c) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+    float sw[4], bs[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const bool ok = col0 + j < n;
+        sw[j] = ok ? scales[col0 + j] : 0.0f;
+        bs[j] = (ok && bias) ? bias[col0 + j] : 0.0f;
+    }
+    for (int64_t r0 = (int64_t)blockIdx.y * 2; r0 < m; r0 += (int64_t)gridDim.y * 2) {   // two rows per trip, loads first
+        float acc[2][4] = {{0.0f, 0.0f, 0.0f, 0.0f}, {0.0f, 0.0f, 0.0f, 0.0f}};
+        float rs[2] = {0.0f, 0.0f};
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+            const int64_t r = r0 + t;
+            if (r >= m) break;
+            const int64_t idx = r * n + col0;
+            rs[t] = rscale[r];
+            if (vec) {
+                const float4 v0 = *reinterpret_cast<const float4 *>(c + idx);
+                acc[t][0] = v0.x; acc[t][1] = v0.y; acc[t][2] = v0.z; acc[t][3] = v0.w;
+                for (int z = 1; z < splits; z++) {
+                    const float4 u = *reinterpret_cast<const float4 *>(c + (int64_t)z * m * n + idx);
+                    acc[t][0] += u.x; acc[t][1] += u.y; acc[t][2] += u.z; acc[t][3] += u.w;
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    if (col0 + j < n) {
+                        acc[t][j] = c[idx + j];
+                        for (int z = 1; z < splits; z++) acc[t][j] += c[(int64_t)z * m * n + idx + j];
+                    }
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+            const int64_t r = r0 + t;
+            if (r >= m) break;
+            const int64_t idx = r * n + col0;
+            float o[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                float v = (acc[t][j] * rs[t]) * sw[j];
+                if (bias) v = v + bs[j];
+                o[j] = fnn_activation(v, act);
+            }
+            if (vec) *reinterpret_cast<float4 *>(out + idx) = make_float4(o[0], o[1], o[2], o[3]);
+            else {
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    if (col0 + j < n) out[idx + j] = o[j];
+            }
+        }
     }
 }
 
@@ -570,7 +683,7 @@ int fnn_fp8_actquant_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weig
     const int iters = (int)(kpad / KB);
     int splits = (int)(256 / (tiles > 0 ? tiles : 1));
     if (splits > iters / 4) splits = iters / 4;
-    if (splits > 16) splits = 16;
+    if (splits > 4) splits = 4;   // (more partial matrices cost more than the idle CUs they fill)
     if (splits < 1) splits = 1;
     void *ws0 = nullptr, *ws1 = nullptr;
     int rc;
@@ -592,11 +705,11 @@ int fnn_fp8_actquant_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weig
     t.splits = (iters + t.ips - 1) / t.ips;
     t.mtiles = (int)(rows_pad / 128);
     t.ntiles = (int)((q.n + 127) / 128);
-    e = launch_i8_tile<FNN_DT_I8, 2, 2, 2, 2, 3, false, false, true>(t, s);
+    e = launch_i8_tile<FNN_DT_I8, 2, 4, 2, 1, 3, false, false, true>(t, s);   // 128 x 128 on eight waves (every wave loads)
     if (e != hipSuccess) return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, hipGetErrorString(e));
-    const int64_t colb = (q.n + 255) / 256;
+    const int64_t colb = (q.n + 1023) / 1024;   // (four columns per thread)
     int64_t rowb = (4096 + colb - 1) / colb;
-    if (rowb > q.m) rowb = q.m;
+    if (rowb > (q.m + 1) / 2) rowb = (q.m + 1) / 2;   // (two rows per thread and trip)
     if (rowb > 65535) rowb = 65535;
     hipLaunchKernelGGL(fp8_matmul_epilogue_kernel, dim3((unsigned)colb, (unsigned)rowb), dim3(256), 0, s, (const float *)ws1, rscale, q.scales,
                        q.bias, q.m, q.n, q.out, t.splits, q.act);
@@ -623,6 +736,16 @@ int fnn_i8_tiled_matmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w
     const int64_t tiles = (rows_pad / 128) * (p.n <= 64 ? (p.n + 63) / 64 : (p.n + 127) / 128);
     const int iters = (int)(kpad / KB);
     int splits = (int)(256 / (tiles > 0 ? tiles : 1));
+    // Tile form: 128 x 128 on eight waves of 64 x 32 (every wave issues loads: 4096 x 4096 at M = 256 25.7 -> 24.3 us, M = 128
+    // 21.9 -> 20.5), 256 x 128 on eight waves of 64 x 64 once those fill the chip unsplit (M = 2048: 90.6 -> 70.1 us);
+    // FNN_OPT_TILE_SHAPE 0 / 1 / 2 picks the four-wave tiles / either of these.
+    int form = (int)fnn_ctx_option(ctx, FNN_OPT_TILE_SHAPE);
+    if (form < 0 || form > 2) form = (rows_pad % 256 == 0 && (rows_pad / 256) * ((p.n + 127) / 128) >= 256) ? 2 : 1;
+    if (p.n <= 64) form = 0;
+    if (form == 2 && rows_pad % 256) form = 1;
+    if (form == 2) splits *= 2;
+    if (splits > 4) splits = 4;   // (more partial matrices cost more than the idle CUs they fill: M = 128 23.8 -> 20.5 us)
+    if (const int64_t forced = fnn_ctx_option(ctx, FNN_OPT_TILE_SPLIT); forced > 0) splits = (int)forced;
     if (splits > iters / 4) splits = iters / 4;
     if (splits > 16) splits = 16;
     if (splits < 1) splits = 1;
@@ -651,14 +774,14 @@ int fnn_i8_tiled_matmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w
                            reinterpret_cast<const int8_t *>(p.payload + 8), p.m, p.k, kpad, rows_pad, a8, qsum);
     hipError_t e = hipGetLastError();
     if (e == hipSuccess)
-        e = w->dtype == FNN_DT_I8 ? run_i8_gemm<FNN_DT_I8>(words, kp, w->rows, 0, p.n, a8, p.m, rows_pad, kpad, c, p.n, s, splits)
-                                  : run_i8_gemm<FNN_DT_I4>(words, kp, w->rows, 0, p.n, a8, p.m, rows_pad, kpad, c, p.n, s, splits);
+        e = w->dtype == FNN_DT_I8 ? run_i8_gemm<FNN_DT_I8>(words, kp, w->rows, 0, p.n, a8, p.m, rows_pad, kpad, c, p.n, s, splits, nullptr, false, form)
+                                  : run_i8_gemm<FNN_DT_I4>(words, kp, w->rows, 0, p.n, a8, p.m, rows_pad, kpad, c, p.n, s, splits, nullptr, false, form);
     if (e == hipSuccess) {
         const int ips = (iters + splits - 1) / splits;
         splits = (iters + ips - 1) / ips;   // as run_i8_gemm rounds it
-        const int64_t colb = (p.n + 255) / 256;
+        const int64_t colb = (p.n + 1023) / 1024;   // (four columns per thread)
         int64_t rowb = (4096 + colb - 1) / colb;   // about 4096 workgroups
-        if (rowb > p.m) rowb = p.m;
+        if (rowb > (p.m + 1) / 2) rowb = (p.m + 1) / 2;   // (two rows per thread and trip)
         if (rowb > 65535) rowb = 65535;
         hipLaunchKernelGGL(i8_matmul_epilogue_kernel, dim3((unsigned)colb, (unsigned)rowb), dim3(256), 0, s, c, p.payload, qsum, wm->row_qsum,
                            p.scales, p.zeros, p.m, p.n, p.k, p.out, p.acc_out, splits, p.bias, p.act);

@@ -104,6 +104,8 @@ enum {
     FNN_OPT_TILE_SHAPE = 5,       /* tiled GEMMs, tile shape; -1 (default) = by shape.  f16 tiles: 0 = 128x128, 1 = 64x128, */
                                   /* 2 = 32x128, 3 = 256x128 with 8 waves (8-bit weights); int8 digit-plane tiles:       */
                                   /* 0 = 128x128, 1 = 256x128, 2 = 256x128 / 8 waves, 3 = 256x256, 4 = 256x192 (8 waves, 4-bit) */
+                                  /* int8-activation GEMMs (matmul_*_i8, FNN_FLAG_ACT_QUANT): 0 = 128x128 on four waves,  */
+                                  /* 1 = 128x128 on eight, 2 = 256x128 on eight (whole 256-row tiles only)                */
     FNN_OPT_TILE_SPLIT = 6,       /* tiled GEMM: K split over this many workgroups; 0 (default) = cost model        */
     FNN_OPT_TILE_STAGES = 7,      /* tiled GEMMs: LDS ring depth where the shape has variants (3..6); 0 (default) = by shape */
     FNN_OPT_TILE_MIN_M = 8,       /* smallest M the tiled GEMM takes (default 5)                                    */

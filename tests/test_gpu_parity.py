@@ -572,6 +572,33 @@ def test_i8act_matmul_integer_exact(ctx, orc, dt, m, k, n, zp):
     ctx.release(h)
 
 
+@pytest.mark.parametrize("dt", [0, 1])
+@pytest.mark.parametrize("m,k,n", [(200, 1000, 130), (256, 512, 264), (300, 2048, 72)])
+def test_i8act_matmul_tile_forms(ctx, orc, dt, m, k, n):
+    """The three tile forms of the int8 matrix-core GEMM behind matmul_i8_i8 / matmul_i4_i8 (128 x 128 on four waves, on
+    eight waves, 256 x 128 on eight waves) and K splits of 1, 2 and 4: exact integer accumulators whatever the form,
+    with ragged N and K, row counts that are and are not whole 256-row tiles, bias and activation in the epilogue's
+    four-column groups (n % 4 != 0 included)."""
+    rng = np.random.default_rng(5100 + dt + k)
+    pw = fastnn_amd.quantize_weights(dt, _weights(rng, n, k))
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    payload = orc.quantize_activations(x)
+    h = ctx.register(pw)
+    want, want_acc = orc.qmatmul_i8act(to_oracle(orc, pw), payload, m, want_acc=True)
+    try:
+        for form in (0, 1, 2):
+            for split in (0, 1, 2, 4):
+                ctx.set_option(flib.OPT_TILE_SHAPE, form)
+                ctx.set_option(flib.OPT_TILE_SPLIT, split)
+                got, acc = ctx.qmatmul_i8act(h, payload, m, n, want_acc=True)
+                assert np.array_equal(acc, want_acc), (form, split)
+                assert_close(got, want, 1e-6, f"form {form} split {split}")
+    finally:
+        ctx.set_option(flib.OPT_TILE_SHAPE, -1)
+        ctx.set_option(flib.OPT_TILE_SPLIT, 0)
+    ctx.release(h)
+
+
 def test_i8act_literals_on_gpu(ctx, orc, golden):
     dts = {"i8": 0, "i4": 1}
     for c in golden["gemm_i8act"]["cases"]:
