@@ -272,15 +272,18 @@ hipError_t launch_quantize_activations(const float *x, int64_t numel, float scal
     int64_t blocks = (numel + 255) / 256;
     if (blocks > 1024) blocks = 1024;
     if (blocks < 1) blocks = 1;
+    int64_t pblocks = blocks;
     const float *partial = nullptr;
     if (!(scale > 0.0f)) {
-        hipLaunchKernelGGL(absmax_partial_kernel, dim3((unsigned)blocks), dim3(256), 0, s, x, numel,
+        // (at most 256 partial maxima: every workgroup of the quantiser reduces them again before its first code)
+        if (pblocks > 256) pblocks = 256;
+        hipLaunchKernelGGL(absmax_partial_kernel, dim3((unsigned)pblocks), dim3(256), 0, s, x, numel,
                            scratch_partial);
         partial = scratch_partial;
         zp = 0.0f;
     }
     hipLaunchKernelGGL(quantize_act_kernel, dim3((unsigned)blocks), dim3(256), 0, s, x, numel, partial,
-                       (int)blocks, scale, zp, payload);
+                       (int)pblocks, scale, zp, payload);
     return hipGetLastError();
 }
 

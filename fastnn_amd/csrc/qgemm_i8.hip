@@ -85,77 +85,25 @@ __global__ void __launch_bounds__(256) i8_matmul_epilogue_kernel(const int32_t *
                                                                  int64_t m, int64_t n, int64_t k, float *out, int32_t *acc_out, int splits,
                                                                  const float *bias, int act)
 {
-    // a thread owns four consecutive output columns (their weight constants stay in registers; 16-byte loads and stores
-    // where n % 4 == 0 and the buffers are aligned) and walks rows blockIdx.y, +gridDim.y, ...
+    // a thread owns one output column (its weight constants stay in registers) and walks rows blockIdx.y, +gridDim.y, ...
     const float sa = reinterpret_cast<const float *>(payload)[0];
     const float za = reinterpret_cast<const float *>(payload)[1];
-    const int64_t col0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
-    if (col0 >= n) return;
-    const bool vec = col0 + 4 <= n && n % 4 == 0 &&
-                     ((reinterpret_cast<uintptr_t>(c) | reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(acc_out)) & 15) == 0;
-    float sw[4], zw[4], zwsum[4], bs[4];
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-        const bool ok = col0 + j < n;
-        sw[j] = ok ? scales[col0 + j] : 0.0f;
-        zw[j] = ok ? zeros[col0 + j] : 0.0f;
-        zwsum[j] = ok ? za * (float)wsum[col0 + j] : 0.0f;
-        bs[j] = (ok && bias) ? bias[col0 + j] : 0.0f;
-    }
+    const int64_t col = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (col >= n) return;
+    const float sw = scales[col], zw = zeros[col];
+    const float zwsum = za * (float)wsum[col];
     const float kza = (float)k * za;
-    // two rows per trip: both rows' partial sums are requested before either row's arithmetic starts
-    for (int64_t r0 = (int64_t)blockIdx.y * 2; r0 < m; r0 += (int64_t)gridDim.y * 2) {
-        int acc[2][4] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
-        int qs[2] = {0, 0};
-#pragma unroll
-        for (int t = 0; t < 2; t++) {
-            const int64_t r = r0 + t;
-            if (r >= m) break;
-            const int64_t idx = r * n + col0;
-            qs[t] = qsum[r];
-            if (vec) {
-                const int4 v0 = *reinterpret_cast<const int4 *>(c + idx);
-                acc[t][0] = v0.x; acc[t][1] = v0.y; acc[t][2] = v0.z; acc[t][3] = v0.w;
-                for (int z = 1; z < splits; z++) {   // exact whatever the order
-                    const int4 u = *reinterpret_cast<const int4 *>(c + (int64_t)z * m * n + idx);
-                    acc[t][0] += u.x; acc[t][1] += u.y; acc[t][2] += u.z; acc[t][3] += u.w;
-                }
-            } else {
-#pragma unroll
-                for (int j = 0; j < 4; j++)
-                    if (col0 + j < n) {
-                        acc[t][j] = c[idx + j];
-                        for (int z = 1; z < splits; z++) acc[t][j] += c[(int64_t)z * m * n + idx + j];
-                    }
-            }
-        }
-#pragma unroll
-        for (int t = 0; t < 2; t++) {
-            const int64_t r = r0 + t;
-            if (r >= m) break;
-            const int64_t idx = r * n + col0;
-            const float input_sum = (float)qs[t] * sa + kza;
-            float o[4];
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const float dot = (za != 0.0f) ? (float)acc[t][j] * sa + zwsum[j] : (float)acc[t][j] * sa;
-                float v = dot * sw[j] + zw[j] * input_sum;
-                if (bias) v = v + bs[j];
-                o[j] = fnn_activation(v, act);
-                if (za != 0.0f) acc[t][j] = 0;
-            }
-            if (vec) {
-                *reinterpret_cast<float4 *>(out + idx) = make_float4(o[0], o[1], o[2], o[3]);
-                if (acc_out) *reinterpret_cast<int4 *>(acc_out + idx) = make_int4(acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
-            } else {
-#pragma unroll
-                for (int j = 0; j < 4; j++)
-                    if (col0 + j < n) {
-                        out[idx + j] = o[j];
-                        if (acc_out) acc_out[idx + j] = acc[t][j];
-                    }
-            }
-        }
+    const float bs = bias ? bias[col] : 0.0f;
+    for (int64_t r = blockIdx.y; r < m; r += gridDim.y) {
+        const int64_t idx = r * n + col;
+        int acc = c[idx];
+        for (int z = 1; z < splits; z++) acc += c[(int64_t)z * m * n + idx];   // exact whatever the order
+        const float input_sum = (float)qsum[r] * sa + kza;
+        const float dot = (za != 0.0f) ? (float)acc * sa + zwsum : (float)acc * sa;
+        float v = dot * sw + zw * input_sum;
+        if (bias) v = v + bs;
+        out[idx] = fnn_activation(v, act);
+        if (acc_out) acc_out[idx] = (za != 0.0f) ? 0 : acc;
     }
 }
 
@@ -779,9 +727,9 @@ int fnn_i8_tiled_matmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w
     if (e == hipSuccess) {
         const int ips = (iters + splits - 1) / splits;
         splits = (iters + ips - 1) / ips;   // as run_i8_gemm rounds it
-        const int64_t colb = (p.n + 1023) / 1024;   // (four columns per thread)
+        const int64_t colb = (p.n + 255) / 256;
         int64_t rowb = (4096 + colb - 1) / colb;   // about 4096 workgroups
-        if (rowb > (p.m + 1) / 2) rowb = (p.m + 1) / 2;   // (two rows per thread and trip)
+        if (rowb > p.m) rowb = p.m;
         if (rowb > 65535) rowb = 65535;
         hipLaunchKernelGGL(i8_matmul_epilogue_kernel, dim3((unsigned)colb, (unsigned)rowb), dim3(256), 0, s, c, p.payload, qsum, wm->row_qsum,
                            p.scales, p.zeros, p.m, p.n, p.k, p.out, p.acc_out, splits, p.bias, p.act);
