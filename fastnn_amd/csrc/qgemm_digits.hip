@@ -6,13 +6,14 @@
 //
 // The integer lanes of these weight types are int8 operands as they are (I8) or after one mask per word
 // (4-bit lanes), so the weight side needs no decode to f16.  The activations become exact integers first:
-// row m is scaled by a power of two, v = rint(x * 2^e) with |v| < 2^30, and written as four balanced base-256
+// row m is scaled by a power of two, v = rint(x * 2^e) with |v| < 2^30 (four planes) or 2^22 (three planes, the
+// default wherever they measured faster: see fnn_digits_qmatmul), and written as balanced base-256
 // digits, v = sum_j 256^j d_j with -128 <= d_j <= 127, one int8 plane per digit.
 // v_mfma_i32_32x32x32_i8 multiplies every plane with the weight lanes exactly; the planes of an output meet in
 // one lane (tile_kernel.h) and are recombined in f32 before the reference's affine epilogue.  Against the f16
 // form (hi + lo f16 rows, weights decoded to f16 per MFMA step) this is the same matrix-core time (four planes at
 // twice the f16 rate), a fraction of the vector instructions per stage, and a tighter result: the only rounding
-// before the epilogue is rint() at 2^-30 of the row's largest magnitude.
+// before the epilogue is rint() at 2^-30 (2^-22 with three planes) of the row's largest magnitude.
 //
 // Launches: digit_prep_kernel (once per call), qgemm_tile_kernel<int8, DIG>, and with K split over workgroups
 // splitk_epilogue_kernel (partials added in split order: results do not depend on scheduling).

@@ -113,7 +113,7 @@ enum {
                                   /* (activations as four exact base-256 digit rows, integer sums, no weight decode);  */
                                   /* 0: the f16 GEMV kernel takes them too                                             */
     FNN_OPT_GEMM_INT8 = 10,       /* 1 (default): M >= FNN_OPT_GEMM_INT8_MIN_M with I8 / I4 / U4 weights runs as an int8  */
-                                  /* matrix-core GEMM over four exact activation digit planes (not in the single-rounding */
+                                  /* matrix-core GEMM over three or four exact activation digit planes (not in the single-rounding */
                                   /* mode); 0: the f16 tiled GEMM takes them too                                          */
     FNN_OPT_GEMM_INT8_MIN_M = 11, /* smallest M of that path (default 17)                                                 */
     FNN_OPT_CODEBOOK_EXPANDED = 12, /* codebook weights with blocks of 32 at M >= 5: 0 (default) = by M (decoded inside the */
