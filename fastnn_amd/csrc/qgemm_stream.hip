@@ -34,7 +34,23 @@ bool plan_stream(int bits, bool int8, int64_t m, int64_t n, int64_t k, int64_t f
     // launches: no more workgroups than the chip holds at once (a second wave of
     // workgroups repeats every phase).  4096 x 4096 at M = 32: 14.4 against 17.9 us; 2048 -> 8192 FP8: 13.3 against 17.4;
     // 4096 x 11008 (688 workgroups): 25.0 against 23.5; M = 64 on 4096 x 4096: 21.3 against 20.0.
-    if (forced == 0 && ntiles * splits > 320) return false;
+    if (forced == 0 && ntiles * splits > 320) {
+        // Wide outputs: two row tiles per wave (256 weight rows per workgroup) and as few rounds per workgroup as keep the
+        // launch within one round of workgroups.  4096 x 11008 (43 column tiles): 4 splits x 2 rounds of 512, 172 workgroups,
+        // M = 17 19.2 us against 23.0 on the tiled path, M = 32 21.3 against 23.9 (8 splits x 1 round, 344 workgroups: 25.5).
+        if (mb * 2 > (int8 ? 4 : 8)) return false;
+        const int64_t ntiles2 = (n + FNN_STREAM_NW * 2 * 16 - 1) / (FNN_STREAM_NW * 2 * 16);
+        const int64_t total512 = (k + 511) / 512;
+        for (int64_t r2 = 1; r2 <= 4; r2++) {
+            const int64_t s2 = (total512 + r2 - 1) / r2;
+            if (s2 > 64 || (s2 - 1) * r2 >= total512) continue;   // (no empty split)
+            if (ntiles2 * s2 > 320) continue;
+            if (ntiles2 * s2 < 128) break;                        // (too few workgroups: the tiled path is ahead)
+            *out = StreamPlan{mb, 2, 512, (int)s2, (int)r2, (int)ntiles2};
+            return true;
+        }
+        return false;
+    }
     *out = StreamPlan{mb, rt, kr, (int)splits, (int)rounds, (int)ntiles};
     return true;
 }

@@ -363,6 +363,31 @@ def test_streaming_matmul_takes_the_default_route_and_propagates_non_finite_rows
         ctx.release(h)
 
 
+@pytest.mark.parametrize("dt", [flib.DT_I4, flib.DT_I8, flib.DT_F4])
+@pytest.mark.parametrize("m,k,n", [(20, 4096, 5200), (32, 2048, 10500), (17, 1536, 11008)])
+def test_streaming_matmul_wide_outputs(ctx, orc, dt, m, k, n):
+    """Wide outputs (more than 320 workgroups with one row tile per wave) run in the streaming kernel on two row tiles
+    per wave and one to three rounds per workgroup, picked by rule: against the oracle on a sample of output rows
+    (the first, a ragged last column tile, some in between), with bias and activation, and against the tiled path."""
+    rng = np.random.default_rng(5300 + dt + n)
+    pw = fastnn_amd.quantize_weights(dt, _weights(rng, n, k))
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    bias = (rng.standard_normal(n) * 0.01).astype(np.float32)
+    h = ctx.register(pw)
+    got = ctx.qmatmul(h, a, n, bias=bias, act=2)
+    ctx.set_option(flib.OPT_STREAM_MAX_M, 0)
+    try:
+        other = ctx.qmatmul(h, a, n, bias=bias, act=2)
+    finally:
+        ctx.set_option(flib.OPT_STREAM_MAX_M, 32)
+    assert not np.array_equal(got, other)          # (another kernel, another summation order)
+    assert_close(got, other, 2 * TOL_F32)
+    rows = np.unique(np.concatenate([np.arange(0, 40), np.arange(n - 300, n), rng.integers(0, n, 200)]))
+    want = orc.qmatmul(to_oracle(orc, slice_rows(pw, rows)), a, order=2, bias=bias[rows], act=2)
+    assert_close(got[:, rows], want, TOL_F32, f"{NAMES[dt]} {m}x{k}x{n}")
+    ctx.release(h)
+
+
 def test_int8_digit_plane_gemm_non_finite_rows(ctx, orc):
     """A row holding a NaN or an infinity cannot be written as integer digits: its exponent entry carries a flag and
     the whole output row is NaN (the float path gives NaN or inf there); the other rows are untouched."""
