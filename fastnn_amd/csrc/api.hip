@@ -146,6 +146,7 @@ const OptionSpec kOptions[FNN_OPT_COUNT] = {
     {32, 0, 32},      // FNN_OPT_STREAM_MAX_M
     {0, 0, 0xffff},   // FNN_OPT_STREAM_SHAPE
     {0, 0, 4},        // FNN_OPT_DIGIT_PLANES
+    {1, 0, 1},        // FNN_OPT_GEMV_TILE_MAJOR
 };
 
 #define HIP_TRY(ctx, code, expr)                                                              \
@@ -207,6 +208,7 @@ void free_weight(fnn_hip_weight *w)
     if (w->row_qsum) (void)hipFree(w->row_qsum);
     if (w->umean) (void)hipFree(w->umean);
     if (w->words4) (void)hipFree(w->words4);
+    if (w->words_tm) (void)hipFree(w->words_tm);
     if (w->dense16) (void)hipFree(w->dense16);
     delete w;
 }

@@ -32,6 +32,8 @@ struct fnn_hip_weight {
     float *umean;       // device; [rows] mean lane value per row, built on first single-pass GEMM use
     uint32_t *words4;   // device; rows re-strided to kp4 = ceil4(kp) words (+16 zero words) when kp % 4 != 0,
     int64_t kp4;        //         built on first use by a kernel that fetches 16-byte pieces of a row
+    uint32_t *words_tm; // device; the packed words in blocks of 16 rows x 64 bytes (row block major, then k block), rows padded to
+                        // whole blocks with zeros: the int8 GEMV's wave loads are one contiguous KB each; built on first use
     void *dense16;      // device; codebook type: rows expanded to f16 [hi(K) | lo(K)] + per-row scale tables, built on the
                         //         first MatMul with M >= 5 and kept (the CPU path keeps an f32 copy: packed_tensor.rs:469-521)
     int qblock;         // I4CB block length along inner

@@ -38,6 +38,8 @@ struct DotArgs {
     int act;
     int nslice;   // slices of 512 k-values covering K
     int ntiles;   // row tiles of 16
+    const uint32_t *words_tm;   // non-null: the same words in blocks of 16 rows x 64 bytes, [row block][k block][row][64 bytes]
+    int64_t kb64;               // ... k blocks per row
 };
 
 constexpr int SL = 512;   // k-values per slice
@@ -89,7 +91,8 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t raw_buffer(const void *base, u
 }
 
 // MM activation rows per chunk (1, 2, 4), MC chunks (MC > 1 only with MM = 4): M <= MM * MC
-template <int DT, int MM, int NW, int RT, int MC = 1>
+// TMAJ: the packed words come from the tile-major copy (a wave load = the contiguous KB of one 16-row x 64-byte block)
+template <int DT, int MM, int NW, int RT, int MC = 1, bool TMAJ = false>
 __global__ void __launch_bounds__(NW * 64) qgemv_i8dot_kernel(DotArgs p)
 {
     using W = Int8Op<DT>;
@@ -114,11 +117,13 @@ __global__ void __launch_bounds__(NW * 64) qgemv_i8dot_kernel(DotArgs p)
     uint4 *frag = lds_dyn + wv * (NSTEP * R4 * 4);
 
     // the tile's 16 weight rows (rows past N read as zero) and the activation rows (rows past M read as zero)
-    const __amdgpu_buffer_rsrc_t wbuf = raw_buffer(p.words + n0 * kp, (uint64_t)(N - n0) * (uint64_t)kp * 4);
+    const __amdgpu_buffer_rsrc_t wbuf = TMAJ ? raw_buffer(p.words_tm + (n0 / 16) * p.kb64 * 256, (uint64_t)((N + 15) / 16 - n0 / 16) * (uint64_t)p.kb64 * 1024)
+                                             : raw_buffer(p.words + n0 * kp, (uint64_t)(N - n0) * (uint64_t)kp * 4);
     // one descriptor over the M activation rows: row m starts at byte m*K*4 (below 4 GiB, checked on the host)
     const __amdgpu_buffer_rsrc_t abuf = raw_buffer(p.a, (uint64_t)mreal * (uint64_t)K * 4);
     const uint32_t arow = (uint32_t)K * 4;
-    const uint32_t wlane = (uint32_t)ln * (uint32_t)kp * 4 + (uint32_t)g * 16;   // 16 rows of kp words: below 4 GiB (checked on the host)
+    const uint32_t wlane = TMAJ ? (uint32_t)ln * 64 + (uint32_t)g * 16
+                                : (uint32_t)ln * (uint32_t)kp * 4 + (uint32_t)g * 16;   // 16 rows of kp words: below 4 GiB (checked on the host)
 
     // the thread that finishes output (row tile r, m, column c): tid = (r*MM + m)*16 + c; its epilogue operands are
     // requested first
@@ -168,12 +173,15 @@ __global__ void __launch_bounds__(NW * 64) qgemv_i8dot_kernel(DotArgs p)
             xa[m][1] = __builtin_amdgcn_raw_buffer_load_b128(abuf, aoff + (uint32_t)m * astep + 16, 0, 0);
         }
         u32x4 wq[RT][LOADS];
-        const uint32_t woff = wlane + (uint32_t)slice * (LOADS * 64);
+        // (tile-major: k block slice * LOADS + l of row block r; a slice past K lands in the next row block or past the
+        // buffer, and its activation digits are zero)
+        const uint32_t woff = TMAJ ? wlane + (uint32_t)slice * (LOADS * 1024) : wlane + (uint32_t)slice * (LOADS * 64);
+        const uint32_t rstep = TMAJ ? (uint32_t)p.kb64 * 1024 : 16 * (uint32_t)kp * 4, lstep = TMAJ ? 1024 : 64;
 #pragma unroll
         for (int r = 0; r < RT; r++)
 #pragma unroll
             for (int l = 0; l < LOADS; l++)
-                wq[r][l] = __builtin_amdgcn_raw_buffer_load_b128(wbuf, woff + (uint32_t)r * 16 * (uint32_t)kp * 4 + l * 64, 0, 0);
+                wq[r][l] = __builtin_amdgcn_raw_buffer_load_b128(wbuf, woff + (uint32_t)r * rstep + l * lstep, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
 
 #pragma unroll
@@ -315,7 +323,8 @@ hipError_t launch_rt(DotArgs p, hipStream_t s, bool *handled)
     p.nslice = (int)((p.k + SL - 1) / SL);
     p.ntiles = (int)((p.n + 16 * RT - 1) / (16 * RT));
     const size_t lds = (size_t)NW * NSTEP * 4 * MM * 4 * 16;    // 2 KiB per wave and activation row of a chunk
-    hipLaunchKernelGGL((qgemv_i8dot_kernel<DT, MM, NW, RT, MC>), dim3((unsigned)p.ntiles), dim3(NW * 64), lds, s, p);
+    if (p.words_tm) hipLaunchKernelGGL((qgemv_i8dot_kernel<DT, MM, NW, RT, MC, true>), dim3((unsigned)p.ntiles), dim3(NW * 64), lds, s, p);
+    else hipLaunchKernelGGL((qgemv_i8dot_kernel<DT, MM, NW, RT, MC>), dim3((unsigned)p.ntiles), dim3(NW * 64), lds, s, p);
     *handled = true;
     return hipGetLastError();
 }
@@ -341,6 +350,20 @@ hipError_t launch_dt(const DotArgs &p, int rt, hipStream_t s, bool *handled)
     return shortk ? launch_nw<DT, 4, 4>(p, rt, s, handled) : launch_nw<DT, 4, 8>(p, rt, s, handled);
 }
 
+// row-major packed words -> blocks of 16 rows x 64 bytes; one thread per 16-byte piece of the destination
+__global__ void __launch_bounds__(256) tile_major_kernel(const uint32_t *src, int64_t rows, int64_t kp, int64_t kb64, u32x4 *dst)
+{
+    const int64_t total = (rows + 15) / 16 * kb64 * 64;   // 16-byte pieces
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+        const int64_t blk = i >> 6, rb = blk / kb64, kb = blk % kb64;
+        const int ln = (int)((i >> 2) & 15), g = (int)(i & 3);
+        const int64_t row = rb * 16 + ln;
+        u32x4 v = {0u, 0u, 0u, 0u};
+        if (row < rows) v = *reinterpret_cast<const u32x4 *>(src + row * kp + kb * 16 + g * 4);
+        dst[i] = v;
+    }
+}
+
 }  // namespace
 
 int fnn_i8dot_qgemv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &q, bool *handled)
@@ -357,6 +380,23 @@ int fnn_i8dot_qgemv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, co
     p.words = q.words; p.scales = q.scales; p.zeros = q.zeros; p.a = q.a; p.bias = q.bias; p.out = q.out;
     p.m = q.m; p.n = q.n; p.k = q.k; p.kp = q.kp; p.act = q.act;
     p.nslice = p.ntiles = 0;
+    p.words_tm = nullptr; p.kb64 = 0;
+    // the tile-major copy of the words (FNN_OPT_GEMV_TILE_MAJOR): rows of whole 64-byte blocks, the registered row-major words
+    if (fnn_ctx_option(ctx, FNN_OPT_GEMV_TILE_MAJOR) == 1 && q.words == w->words && q.kp % 16 == 0 &&
+        ((q.n + 15) / 16) * q.kp * 64 < (int64_t)0xFFFFFF00) {
+        fnn_hip_weight *wm = const_cast<fnn_hip_weight *>(w);
+        if (!wm->words_tm && !fnn_ctx_no_alloc(ctx)) {
+            const int64_t words_tm = (w->rows + 15) / 16 * 16 * q.kp;
+            if (hipMalloc((void **)&wm->words_tm, (size_t)words_tm * 4 + 256) != hipSuccess)
+                return fnn_ctx_fail(ctx, FNN_ERR_MEMORY, "out of device memory (tile-major weight rows)");
+            int64_t blocks = (words_tm / 4 + 255) / 256;
+            if (blocks > 4096) blocks = 4096;
+            hipLaunchKernelGGL(tile_major_kernel, dim3((unsigned)blocks), dim3(256), 0, s, w->words, w->rows, q.kp, q.kp / 16,
+                               reinterpret_cast<u32x4 *>(wm->words_tm));
+            if (hipGetLastError() != hipSuccess) return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, "building the tile-major weight rows failed");
+        }
+        if (wm->words_tm) { p.words_tm = wm->words_tm; p.kb64 = q.kp / 16; }
+    }
     // Row tiles (of 16 weight rows) per workgroup: a workgroup converts the activation rows once for all of its tiles,
     // and the workgroups should come in whole rounds over the 256 CUs: cost ~ rounds * (rows to convert + tiles).
     // Measured on N = 11008, K = 4096 (I4): M = 1 6.8 / 7.7 / 6.8 us with 1 / 2 / 3 tiles, M = 2 8.0 / 8.3 / 6.8,

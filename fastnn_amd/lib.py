@@ -45,6 +45,7 @@ OPT_STREAM_MIN_M = 19
 OPT_STREAM_MAX_M = 20
 OPT_STREAM_SHAPE = 21
 OPT_DIGIT_PLANES = 22
+OPT_GEMV_TILE_MAJOR = 23
 
 STATUS_NAMES = {0: "Ok", 1: "Dispatch", 2: "Memory", 3: "UnsupportedOp", 4: "Compilation"}
 

@@ -146,7 +146,12 @@ enum {
     FNN_OPT_DIGIT_PLANES = 22,    /* int8 matrix-core GEMM (M >= 17, I8 / I4 / U4 weights): activation digit planes, 3 (22 bits     */
                                   /* below the row maximum, 2e-5 of max|ref| stated) or 4 (30 bits, 4e-6, a third more matrix-core */
                                   /* work and operand traffic); 0 (default) = three wherever they measured faster                  */
-    FNN_OPT_COUNT = 23
+    FNN_OPT_GEMV_TILE_MAJOR = 23, /* int8 GEMV (M <= 8, I8 / I4 / U4 weights): 1 (default) = read the packed words from a second   */
+                                  /* device copy laid out in blocks of 16 rows x 64 bytes (one contiguous KB per wave load: same   */
+                                  /* bits, C1 M=1 5.97 -> 5.15 us, C2 6.70 -> 6.41), built on the weight's first such call and     */
+                                  /* kept with it (once more the packed bytes; rows of whole 64-byte blocks only; a call that may  */
+                                  /* not allocate uses the row-major words until the copy exists); 0 = row-major words only        */
+    FNN_OPT_COUNT = 24
 };
 int fnn_hip_set_option(fnn_hip_ctx *ctx, int option, int64_t value);
 int fnn_hip_get_option(fnn_hip_ctx *ctx, int option, int64_t *value);

@@ -212,10 +212,16 @@ def test_int8_gemv_kernel(ctx, orc, dt, m, k, n):
         for rt in (1, 2, 3):               # any number of row tiles per workgroup gives the same bits
             ctx.set_option(flib.OPT_GEMV_ROW_TILES, rt)
             assert np.array_equal(ctx.qmatmul(h, a, n, bias=bias, act=3), got), f"{rt} row tiles"
+            # ... and so does either layout of the packed words (the tile-major copy, default where the rows are whole
+            # 64-byte blocks, and the row-major words)
+            ctx.set_option(flib.OPT_GEMV_TILE_MAJOR, 0)
+            assert np.array_equal(ctx.qmatmul(h, a, n, bias=bias, act=3), got), f"{rt} row tiles, row-major words"
+            ctx.set_option(flib.OPT_GEMV_TILE_MAJOR, 1)
     finally:
         ctx.set_option(flib.OPT_GEMV_ROW_TILES, 0)
         ctx.set_option(flib.OPT_GEMV_INT8, 1)
         ctx.set_option(flib.OPT_GEMV_INT8_MAX_M, 8)
+        ctx.set_option(flib.OPT_GEMV_TILE_MAJOR, 1)
     ctx.release(h)
 
 
