@@ -59,6 +59,8 @@ int fnn_mfma_qgemv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, con
 // M <= 4, integer weights (I8, I4, U4): int8 matrix cores, activations as three exact base-256 digit rows, one
 // workgroup per CU walking the row tiles (no decode arithmetic, activations converted once per workgroup).
 int fnn_i8dot_qgemv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &p, bool *handled);
+// tile-major copy of the packed words for the GEMV kernels (blocks of 16 rows x 64 bytes), null where it does not apply
+int fnn_tile_major_words(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &q, const uint32_t **words_tm, int64_t *kb64);
 
 // 9 <= M <= 16: the same organisation with the 16 activation rows as the MFMA operand rows, loaded straight
 // into registers (no preparation or reduction launch).

@@ -366,6 +366,29 @@ __global__ void __launch_bounds__(256) tile_major_kernel(const uint32_t *src, in
 
 }  // namespace
 
+// The tile-major copy of a weight's packed words (FNN_OPT_GEMV_TILE_MAJOR) for the GEMV kernels: *words_tm = null where it
+// does not apply (option off, rows that are not whole 64-byte blocks, a call on part of a weight, or the copy does not
+// exist yet and this call may not allocate), else the copy (built here on first use) and *kb64 = 64-byte blocks per row.
+int fnn_tile_major_words(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &q, const uint32_t **words_tm, int64_t *kb64)
+{
+    *words_tm = nullptr;
+    *kb64 = 0;
+    if (fnn_ctx_option(ctx, FNN_OPT_GEMV_TILE_MAJOR) != 1 || q.words != w->words || q.kp != w->kp || q.kp % 16 != 0 || q.n != w->rows) return FNN_OK;
+    fnn_hip_weight *wm = const_cast<fnn_hip_weight *>(w);
+    if (!wm->words_tm && !fnn_ctx_no_alloc(ctx)) {
+        const int64_t nwords = (w->rows + 15) / 16 * 16 * w->kp;
+        if (hipMalloc((void **)&wm->words_tm, (size_t)nwords * 4 + 256) != hipSuccess)
+            return fnn_ctx_fail(ctx, FNN_ERR_MEMORY, "out of device memory (tile-major weight rows)");
+        int64_t blocks = (nwords / 4 + 255) / 256;
+        if (blocks > 4096) blocks = 4096;
+        hipLaunchKernelGGL(tile_major_kernel, dim3((unsigned)blocks), dim3(256), 0, s, w->words, w->rows, w->kp, w->kp / 16,
+                           reinterpret_cast<u32x4 *>(wm->words_tm));
+        if (hipGetLastError() != hipSuccess) return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, "building the tile-major weight rows failed");
+    }
+    if (wm->words_tm) { *words_tm = wm->words_tm; *kb64 = w->kp / 16; }
+    return FNN_OK;
+}
+
 int fnn_i8dot_qgemv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &q, bool *handled)
 {
     *handled = false;
@@ -381,22 +404,7 @@ int fnn_i8dot_qgemv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, co
     p.m = q.m; p.n = q.n; p.k = q.k; p.kp = q.kp; p.act = q.act;
     p.nslice = p.ntiles = 0;
     p.words_tm = nullptr; p.kb64 = 0;
-    // the tile-major copy of the words (FNN_OPT_GEMV_TILE_MAJOR): rows of whole 64-byte blocks, the registered row-major words
-    if (fnn_ctx_option(ctx, FNN_OPT_GEMV_TILE_MAJOR) == 1 && q.words == w->words && q.kp % 16 == 0 &&
-        ((q.n + 15) / 16) * q.kp * 64 < (int64_t)0xFFFFFF00) {
-        fnn_hip_weight *wm = const_cast<fnn_hip_weight *>(w);
-        if (!wm->words_tm && !fnn_ctx_no_alloc(ctx)) {
-            const int64_t words_tm = (w->rows + 15) / 16 * 16 * q.kp;
-            if (hipMalloc((void **)&wm->words_tm, (size_t)words_tm * 4 + 256) != hipSuccess)
-                return fnn_ctx_fail(ctx, FNN_ERR_MEMORY, "out of device memory (tile-major weight rows)");
-            int64_t blocks = (words_tm / 4 + 255) / 256;
-            if (blocks > 4096) blocks = 4096;
-            hipLaunchKernelGGL(tile_major_kernel, dim3((unsigned)blocks), dim3(256), 0, s, w->words, w->rows, q.kp, q.kp / 16,
-                               reinterpret_cast<u32x4 *>(wm->words_tm));
-            if (hipGetLastError() != hipSuccess) return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, "building the tile-major weight rows failed");
-        }
-        if (wm->words_tm) { p.words_tm = wm->words_tm; p.kb64 = q.kp / 16; }
-    }
+    if (int rc = fnn_tile_major_words(ctx, s, w, q, &p.words_tm, &p.kb64)) return rc;
     // Row tiles (of 16 weight rows) per workgroup: a workgroup converts the activation rows once for all of its tiles,
     // and the workgroups should come in whole rounds over the 256 CUs: cost ~ rounds * (rows to convert + tiles).
     // Measured on N = 11008, K = 4096 (I4): M = 1 6.8 / 7.7 / 6.8 us with 1 / 2 / 3 tiles, M = 2 8.0 / 8.3 / 6.8,

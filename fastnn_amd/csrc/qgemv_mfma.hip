@@ -40,13 +40,16 @@ struct GemvArgs {
     float *out;
     int64_t m, n, k, kp;
     int act;
+    const uint32_t *words_tm;   // non-null: the words in blocks of 16 rows x 64 bytes ([row block][k block][row][64 bytes]),
+    int64_t kb64;               // kb64 k blocks per row: a wave load is then one contiguous KB
 };
 
 constexpr int GV_NW = 8;        // waves per workgroup
 constexpr int GV_SLICE = 512;   // k-values per wave and round (64 groups of 8: one per lane)
 constexpr int GV_MMAX = 8;
 
-template <int DT, int RT, int MM, bool SINGLE, int NW>
+// TMAJ: the packed words come from the tile-major copy (a wave load = the contiguous KB of one 16-row x 64-byte block)
+template <int DT, int RT, int MM, bool SINGLE, int NW, bool TMAJ = false>
 __global__ void __launch_bounds__(NW * 64) qgemv_mfma_kernel(GemvArgs p)
 {
     using D = DecH<DT>;
@@ -80,7 +83,7 @@ __global__ void __launch_bounds__(NW * 64) qgemv_mfma_kernel(GemvArgs p)
     for (int r = 0; r < RT; r++) {
         int64_t row = n0 + r * 16 + ln;
         if (row > N - 1) row = N - 1;
-        wrow[r] = p.words + row * kp;
+        wrow[r] = TMAJ ? p.words_tm + ((row >> 4) * p.kb64) * 256 + (row & 15) * 16 : p.words + row * kp;
     }
 
     // epilogue operands of the output this thread will finish (idx = tid): requested now,
@@ -133,9 +136,15 @@ __global__ void __launch_bounds__(NW * 64) qgemv_mfma_kernel(GemvArgs p)
         for (int r = 0; r < RT; r++)
 #pragma unroll
             for (int t = 0; t < TPW; t++) {
-                const int64_t woff = wbase + t * 16 + g * 4;
-                const bool ok = woff + 4 <= kp;           // kp % 4 == 0, kp >= 4
-                const uint4 v = *reinterpret_cast<const uint4 *>(wrow[r] + (ok ? woff : kp - 4));
+                int64_t woff;
+                if constexpr (TMAJ) {   // k block min(wbase/16 + t, kb64 - 1) of the row's blocks (1 KB apart), words g*4 of its 64 bytes
+                    const int64_t kb = (wbase >> 4) + t;
+                    woff = (kb < p.kb64 ? kb : p.kb64 - 1) * 256 + g * 4;
+                } else {
+                    woff = wbase + t * 16 + g * 4;
+                    if (woff + 4 > kp) woff = kp - 4;     // kp % 4 == 0, kp >= 4
+                }
+                const uint4 v = *reinterpret_cast<const uint4 *>(wrow[r] + woff);
                 wq[r][t * 4 + 0] = v.x; wq[r][t * 4 + 1] = v.y; wq[r][t * 4 + 2] = v.z; wq[r][t * 4 + 3] = v.w;
             }
         // every request of the round is issued before anything waits: the activations (oldest requests) are
@@ -244,22 +253,26 @@ __global__ void __launch_bounds__(NW * 64) qgemv_mfma_kernel(GemvArgs p)
     }
 }
 
-template <int DT, int RT, bool SINGLE, int NW>
+template <int DT, int RT, bool SINGLE, int NW, bool TMAJ = false>
 void launch_rt(const GemvArgs &p, hipStream_t s)
 {
+    // the tile-major variants exist for the 8-bit types this kernel is the default for (hi + lo activations)
+    if constexpr (!TMAJ && !SINGLE && (DT == FNN_DT_U8 || DT == FNN_DT_F8 || DT == FNN_DT_F8R)) {
+        if (p.words_tm) return launch_rt<DT, RT, SINGLE, NW, true>(p, s);
+    }
     const dim3 grid((unsigned)((p.n + RT * 16 - 1) / (RT * 16))), blk(NW * 64);
     // operand fragments: waves x 16 steps x rows x 4 groups x 16 bytes
     const int mm = p.m <= 1 ? 1 : (p.m <= 2 ? 2 : (p.m <= 4 ? 4 : 8));
     const size_t lds = (size_t)NW * 16 * (SINGLE ? mm : 2 * mm) * 4 * 16;
-    if (mm == 1) hipLaunchKernelGGL((qgemv_mfma_kernel<DT, RT, 1, SINGLE, NW>), grid, blk, lds, s, p);
-    else if (mm == 2) hipLaunchKernelGGL((qgemv_mfma_kernel<DT, RT, 2, SINGLE, NW>), grid, blk, lds, s, p);
+    if (mm == 1) hipLaunchKernelGGL((qgemv_mfma_kernel<DT, RT, 1, SINGLE, NW, TMAJ>), grid, blk, lds, s, p);
+    else if (mm == 2) hipLaunchKernelGGL((qgemv_mfma_kernel<DT, RT, 2, SINGLE, NW, TMAJ>), grid, blk, lds, s, p);
     else if (mm == 4) {
-        auto kern = qgemv_mfma_kernel<DT, RT, 4, SINGLE, NW>;
+        auto kern = qgemv_mfma_kernel<DT, RT, 4, SINGLE, NW, TMAJ>;
         static std::atomic<uint64_t> lds_raised{0};   // up to 64 KiB of dynamic LDS plus the static reduction buffers
         (void)fnn_raise_lds_limit(lds_raised, reinterpret_cast<const void *>(kern), 96 * 1024);
         hipLaunchKernelGGL(kern, grid, blk, lds, s, p);
     } else {
-        auto kern = qgemv_mfma_kernel<DT, RT, 8, SINGLE, NW>;
+        auto kern = qgemv_mfma_kernel<DT, RT, 8, SINGLE, NW, TMAJ>;
         static std::atomic<uint64_t> lds_raised{0};   // up to 128 KiB of dynamic LDS: one workgroup per CU
         (void)fnn_raise_lds_limit(lds_raised, reinterpret_cast<const void *>(kern), 128 * 1024);
         hipLaunchKernelGGL(kern, grid, blk, lds, s, p);
@@ -322,6 +335,9 @@ int fnn_mfma_qgemv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, con
     p.words = q.words; p.scales = q.scales; p.zeros = q.zeros; p.a = q.a; p.bias = q.bias; p.out = q.out;
     p.m = q.m; p.n = q.n; p.k = q.k; p.kp = q.kp; p.act = q.act;
     const bool single = (flags & FNN_FLAG_ACT_F16_SINGLE) != 0;
+    p.words_tm = nullptr; p.kb64 = 0;
+    if (!single && (w->dtype == FNN_DT_U8 || w->dtype == FNN_DT_F8 || w->dtype == FNN_DT_F8R))
+        if (int rc = fnn_tile_major_words(ctx, s, w, q, &p.words_tm, &p.kb64)) return rc;
     p.umean = nullptr;
     if (single) {
         int rc = fnn_row_means(ctx, s, w, &p.umean);
