@@ -12,6 +12,8 @@ struct StreamArgs {
     uint32_t *count;         // splits > 1: one arrival counter per column tile, zero between launches
     int64_t m, n, k, kp;
     int act, splits, rounds, ntiles;
+    const uint32_t *words_tm;   // non-null: the words in blocks of 16 rows x 64 bytes ([row block][k block][row][64 bytes]),
+    int64_t kb64;               // kb64 k blocks per row: a wave load is one contiguous KB
 };
 
 constexpr int FNN_STREAM_NW = 8;   // waves per workgroup

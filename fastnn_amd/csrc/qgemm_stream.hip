@@ -84,6 +84,7 @@ int fnn_stream_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w,
     p.part = nullptr; p.count = fnn_ctx_stream_counters(ctx);
     p.m = q.m; p.n = q.n; p.k = q.k; p.kp = q.kp;
     p.act = q.act; p.splits = pl.splits; p.rounds = pl.rounds; p.ntiles = pl.ntiles;
+    if (int rc = fnn_tile_major_words(ctx, s, w, q, &p.words_tm, &p.kb64)) return rc;
     if (pl.splits > 1) {
         const size_t wgf = (size_t)pl.mb * pl.rt * 4 * FNN_STREAM_NW * 64 + 16 * pl.mb;
         void *ws = nullptr;

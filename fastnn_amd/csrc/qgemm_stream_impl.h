@@ -97,7 +97,8 @@ __device__ __forceinline__ void transpose4(uint32_t a, uint32_t b, uint32_t c, u
 }
 
 // MB: blocks of 16 activation rows (M <= 16*MB); RT: row tiles of 16 weight rows per wave; KR: k-values per round
-template <int DT, int MB, int RT, int KR>
+// TMAJ: the packed words come from the tile-major copy (p.words_tm)
+template <int DT, int MB, int RT, int KR, bool TMAJ = false>
 __global__ void __launch_bounds__(NW * 64) qgemm_stream_kernel(StreamArgs p)
 {
     using T = StreamType<DT>;
@@ -132,9 +133,11 @@ __global__ void __launch_bounds__(NW * 64) qgemm_stream_kernel(StreamArgs p)
     const int64_t n0 = (int64_t)nt * NT;
     const int64_t kbeg = (int64_t)ks * p.rounds * KR;
 
-    const __amdgpu_buffer_rsrc_t wbuf = raw_buffer(p.words + n0 * kp, (uint64_t)(N - n0) * (uint64_t)kp * 4);
+    const __amdgpu_buffer_rsrc_t wbuf = TMAJ ? raw_buffer(p.words_tm + (n0 / 16) * p.kb64 * 256, (uint64_t)((N + 15) / 16 - n0 / 16) * (uint64_t)p.kb64 * 1024)
+                                             : raw_buffer(p.words + n0 * kp, (uint64_t)(N - n0) * (uint64_t)kp * 4);
     const __amdgpu_buffer_rsrc_t abuf = raw_buffer(p.a, (uint64_t)mreal * (uint64_t)K * 4);
-    const uint32_t wlane = (uint32_t)(wv * RT * 16 + ln) * (uint32_t)kp * 4 + (uint32_t)g * 16;
+    const uint32_t wlane = TMAJ ? (uint32_t)(wv * RT) * (uint32_t)p.kb64 * 1024 + (uint32_t)ln * 64 + (uint32_t)g * 16
+                                : (uint32_t)(wv * RT * 16 + ln) * (uint32_t)kp * 4 + (uint32_t)g * 16;
 
     float e_scale[RT], e_zero[RT], e_bias[RT];   // epilogue operands of this lane's columns
     float tot[MB][RT][4];
@@ -175,7 +178,9 @@ __global__ void __launch_bounds__(NW * 64) qgemm_stream_kernel(StreamArgs p)
                 // a lane load wholly past K leaves the buffer and reads as zero (a row's bytes past K would be the next
                 // row's); the f16 types require K % CHUNK == 0, so no load of theirs straddles K, and the int8 types
                 // meet zero digits there
-                const uint32_t off = k0 + l * CHUNK < K ? wlane + (uint32_t)r * 16 * (uint32_t)kp * 4 + wk + l * 64 : 0xFFFFFF00u;
+                const uint32_t off = !(k0 + l * CHUNK < K) ? 0xFFFFFF00u
+                                     : TMAJ ? wlane + ((uint32_t)r * (uint32_t)p.kb64 + (wk >> 6) + l) * 1024
+                                            : wlane + (uint32_t)r * 16 * (uint32_t)kp * 4 + wk + l * 64;
                 wq[r][l] = __builtin_amdgcn_raw_buffer_load_b128(wbuf, off, 0, 0);
             }
         __builtin_amdgcn_sched_barrier(0);
@@ -511,16 +516,19 @@ size_t stream_lds_bytes()
     return (size_t)LOADS * SUB * MB * 64 * 16;
 }
 
-template <int DT, int MB, int RT, int KR>
+template <int DT, int MB, int RT, int KR, bool TMAJ = false>
 hipError_t launch_stream(const StreamArgs &p, hipStream_t s)
 {
+    if constexpr (!TMAJ) {
+        if (p.words_tm) return launch_stream<DT, MB, RT, KR, true>(p, s);
+    }
     static std::atomic<uint64_t> raised{0};
     const size_t lds = stream_lds_bytes<DT, MB, RT, KR>();
     if (lds > 48 * 1024) {
-        hipError_t e = fnn_raise_lds_limit(raised, (const void *)qgemm_stream_kernel<DT, MB, RT, KR>, (int)lds);
+        hipError_t e = fnn_raise_lds_limit(raised, (const void *)qgemm_stream_kernel<DT, MB, RT, KR, TMAJ>, (int)lds);
         if (e != hipSuccess) return e;
     }
-    hipLaunchKernelGGL((qgemm_stream_kernel<DT, MB, RT, KR>), dim3((unsigned)(p.ntiles * p.splits)), dim3(NW * 64), lds, s, p);
+    hipLaunchKernelGGL((qgemm_stream_kernel<DT, MB, RT, KR, TMAJ>), dim3((unsigned)(p.ntiles * p.splits)), dim3(NW * 64), lds, s, p);
     return hipGetLastError();
 }
 

@@ -146,11 +146,13 @@ enum {
     FNN_OPT_DIGIT_PLANES = 22,    /* int8 matrix-core GEMM (M >= 17, I8 / I4 / U4 weights): activation digit planes, 3 (22 bits     */
                                   /* below the row maximum, 2e-5 of max|ref| stated) or 4 (30 bits, 4e-6, a third more matrix-core */
                                   /* work and operand traffic); 0 (default) = three wherever they measured faster                  */
-    FNN_OPT_GEMV_TILE_MAJOR = 23, /* int8 GEMV (M <= 8, I8 / I4 / U4 weights): 1 (default) = read the packed words from a second   */
-                                  /* device copy laid out in blocks of 16 rows x 64 bytes (one contiguous KB per wave load: same   */
-                                  /* bits, C1 M=1 5.97 -> 5.15 us, C2 6.70 -> 6.41), built on the weight's first such call and     */
-                                  /* kept with it (once more the packed bytes; rows of whole 64-byte blocks only; a call that may  */
-                                  /* not allocate uses the row-major words until the copy exists); 0 = row-major words only        */
+    FNN_OPT_GEMV_TILE_MAJOR = 23, /* the kernels that stream the packed words straight into matrix-core operand registers (M <= 8: */
+                                  /* I8 / I4 / U4 / U8 / F8 / F8R weights; the one-launch kernel for 17 <= M <= 32: every type):   */
+                                  /* 1 (default) = read them from a second device copy laid out in blocks of 16 rows x 64 bytes    */
+                                  /* (one contiguous KB per wave load: same bits, C1 M=1 5.97 -> 5.15 us, C2 6.70 -> 6.41, FP8     */
+                                  /* 4096 x 4096 5.90 -> 5.40), built on the weight's first such call and kept with it (once more  */
+                                  /* the packed bytes; rows of whole 64-byte blocks only; a call that may not allocate uses the    */
+                                  /* row-major words until the copy exists); 0 = row-major words only                              */
     FNN_OPT_COUNT = 24
 };
 int fnn_hip_set_option(fnn_hip_ctx *ctx, int option, int64_t value);

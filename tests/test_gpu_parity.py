@@ -356,6 +356,11 @@ def test_streaming_matmul_takes_the_default_route_and_propagates_non_finite_rows
         assert_close(clean, want, TOL_F32)
         assert_close(other, want, TOL_F32)
         assert not np.array_equal(clean, other)
+        ctx.set_option(flib.OPT_GEMV_TILE_MAJOR, 0)   # the same kernel on the row-major words: the same bits
+        try:
+            assert np.array_equal(ctx.qmatmul(h, a, n), clean)
+        finally:
+            ctx.set_option(flib.OPT_GEMV_TILE_MAJOR, 1)
         a[0, 700] = np.nan
         a[20, 3] = np.inf
         a[31, 2047] = -np.inf
