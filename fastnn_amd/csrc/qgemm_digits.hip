@@ -267,6 +267,9 @@ int run_digits(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const Q
 
     TileArgs t = {};
     t.words = q.words;
+    if constexpr (DecI<DT>::WPS == 2) {   // 4-bit weights: 64 bytes per row and stage, one block of the tile-major copy
+        if (int rc = fnn_tile_major_words(ctx, s, w, q, &t.words_tm, &t.kb64)) return rc;
+    }
     t.zero_chunk = q.words + w->rows * q.kp;    // the zeroed margin behind the last row
     t.scales = q.scales; t.zeros = q.zeros; t.bias = q.bias;
     t.ap = reinterpret_cast<const _Float16 *>(d.planes);
@@ -363,6 +366,9 @@ int run_digits3(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const 
 
     TileArgs t = {};
     t.words = q.words;
+    if constexpr (DecI<DT>::WPS == 2) {   // 4-bit weights: 64 bytes per row and stage, one block of the tile-major copy
+        if (int rc = fnn_tile_major_words(ctx, s, w, q, &t.words_tm, &t.kb64)) return rc;
+    }
     t.zero_chunk = q.words + w->rows * q.kp;    // the zeroed margin behind the last row
     t.scales = q.scales; t.zeros = q.zeros; t.bias = q.bias;
     t.ap = reinterpret_cast<const _Float16 *>(d.planes);

@@ -610,8 +610,12 @@ int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QM
         if (e != hipSuccess) return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, hipGetErrorString(e));
     }
 
-    TileArgs t;
+    TileArgs t = {};
     t.words = q.words;
+    if constexpr (DT != DT_F16_DENSE && DT != FNN_DT_I4CB && DecH<DT>::WPS == 2) {   // 8-bit types: 64 bytes per row and stage, one block of the tile-major copy
+        if (!dense)
+            if (int rc2 = fnn_tile_major_words(ctx, s, w, q, &t.words_tm, &t.kb64)) return rc2;
+    }
     t.zero_chunk = q.words + w->rows * q.kp;    // the zeroed margin behind the last row
     t.scales = q.scales; t.zeros = q.zeros; t.umean = want_umean ? wm->umean : nullptr; t.bias = q.bias;
     t.ap = pa.ap; t.rexp = pa.rexp; t.xsum = pa.xsum; t.esum = pa.esum;

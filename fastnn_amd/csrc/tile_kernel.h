@@ -7,6 +7,10 @@
 
 struct TileArgs {
     const uint32_t *words;
+    // non-null (weight types with 64 bytes per row and stage only): the words in blocks of 16 rows x 64 bytes,
+    // [row block][k block][row][64 bytes], kb64 k blocks per row: a wave's 64 chunk loads of a stage are one contiguous KB
+    const uint32_t *words_tm = nullptr;
+    int64_t kb64 = 0;
     const uint32_t *zero_chunk;   // 16 zero bytes: source of weight chunks past the end of a row
     const float *scales, *zeros, *umean, *bias;
     const _Float16 *ap;
@@ -247,6 +251,7 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
         a_src[j] = p.ap + ((int64_t)mt * BM + row) * 64 + g * 8 - (j & 3) * 512;   // (biased: see load_group_to_lds16)
     }
     // weights: chunk (row, c) lives at slot row*WC + (c ^ swz(row)); rows past N repeat the last row
+    const bool tmaj = WC == 4 && !CB && p.words_tm != nullptr;   // (uniform)
     const uint32_t *w_src[W_LPW];
     int w_chunk[W_LPW];
 #pragma unroll
@@ -258,8 +263,10 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
         int64_t grow = n0 + row;
         if (grow > p.n - 1) grow = p.n - 1;
         w_src[j] = p.words + grow * p.kp + c * 4 - (j & 3) * 256;                  // (biased likewise)
+        if (tmaj) w_src[j] = p.words_tm + (((grow >> 4) * p.kb64) << 8) + ((grow & 15) << 4) + c * 4 - (j & 3) * 256;
         w_chunk[j] = c * 4;
     }
+    const int w_stride = tmaj ? 256 : WC * 4;   // words between consecutive stages of a row (tile-major: one block on)
     const int64_t a_step = p.rows_pad * 64;   // elements between consecutive k blocks
     const unsigned a_dst = __builtin_amdgcn_readfirstlane(lds0 + wv * A_LPW * 1024);
     const unsigned w_dst = __builtin_amdgcn_readfirstlane(lds0 + A_BYTES + wv * W_LPW * 1024);
@@ -272,7 +279,7 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
 #pragma unroll
     for (int j = 0; j < A_LPW; j++) a_src[j] += (int64_t)(DENSE ? it0 % p.a_wrap : it0) * a_step;
 #pragma unroll
-    for (int j = 0; j < W_LPW; j++) w_src[j] += (int64_t)it0 * (WC * 4);
+    for (int j = 0; j < W_LPW; j++) w_src[j] += (int64_t)it0 * w_stride;
     int a_pos = DENSE ? it0 % p.a_wrap : 0;       // position inside the activation sweep
     const bool ragged = !DENSE && (p.kp % (WC * 4)) != 0;
     bool w_past[W_LPW];   // this lane's chunk of the last stage lies behind the end of the row
@@ -316,7 +323,7 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
             a_pos = 0;
             astep = -(int64_t)(p.a_wrap - 1) * a_step;
         }
-        const int wstep = more ? WC * 4 : 0;
+        const int wstep = more ? w_stride : 0;
 #pragma unroll
         for (int j = 0; j < A_LPW; j++) a_src[j] += astep;
 #pragma unroll

@@ -399,6 +399,27 @@ def test_streaming_matmul_wide_outputs(ctx, orc, dt, m, k, n):
     ctx.release(h)
 
 
+@pytest.mark.parametrize("dt", [flib.DT_I8, flib.DT_I4, flib.DT_U4, flib.DT_U8, flib.DT_F8, flib.DT_F8R, flib.DT_F4])
+@pytest.mark.parametrize("m,k,n", [(1, 2048, 300), (6, 4096, 1000), (24, 2048, 1100), (40, 2048, 300), (200, 1024, 520)])
+def test_tile_major_copy_of_the_words_gives_the_same_bits(ctx, orc, dt, m, k, n):
+    """The kernels that read the packed words from the tile-major copy (blocks of 16 rows x 64 bytes: the GEMV kernels,
+    the streaming kernel, the tile kernels of the weight types with 64 bytes per row and stage) against the same
+    kernels on the row-major words: identical outputs, ragged N (a partial last row block), and the oracle's bound."""
+    rng = np.random.default_rng(6100 + dt * 7 + m)
+    pw = fastnn_amd.quantize_weights(dt, _weights(rng, n, k))
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    bias = (rng.standard_normal(n) * 0.01).astype(np.float32)
+    h = ctx.register(pw)
+    got = ctx.qmatmul(h, a, n, bias=bias, act=1)
+    ctx.set_option(flib.OPT_GEMV_TILE_MAJOR, 0)
+    try:
+        assert np.array_equal(ctx.qmatmul(h, a, n, bias=bias, act=1), got)
+    finally:
+        ctx.set_option(flib.OPT_GEMV_TILE_MAJOR, 1)
+    assert_close(got, orc.qmatmul(to_oracle(orc, pw), a, order=2, bias=bias, act=1), TOL_F32, f"{NAMES[dt]} {m}x{k}x{n}")
+    ctx.release(h)
+
+
 def test_int8_digit_plane_gemm_non_finite_rows(ctx, orc):
     """A row holding a NaN or an infinity cannot be written as integer digits: its exponent entry carries a flag and
     the whole output row is NaN (the float path gives NaN or inf there); the other rows are untouched."""
