@@ -36,11 +36,14 @@ struct Rows16Args {
     float *out;
     int64_t m, n, k, kp;
     int act;
+    const uint32_t *words_tm;   // non-null: the words in blocks of 16 rows x 64 bytes ([row block][k block][row][64 bytes]),
+    int64_t kb64;               // kb64 k blocks per row: a wave load of packed bytes is then one contiguous KB
 };
 
 constexpr int R16_SLICE = 512;   // k-values per wave and round
 
-template <int DT, int RT, bool SINGLE, int NW>
+// TMAJ: the packed words come from the tile-major copy (p.words_tm)
+template <int DT, int RT, bool SINGLE, int NW, bool TMAJ = false>
 __global__ void __launch_bounds__(NW * 64) qgemv_rows16_kernel(Rows16Args p)
 {
     using D = DecH<DT>;
@@ -77,7 +80,7 @@ __global__ void __launch_bounds__(NW * 64) qgemv_rows16_kernel(Rows16Args p)
     for (int r = 0; r < RT; r++) {
         int64_t row = n0 + r * 16 + ln;
         if (row > N - 1) row = N - 1;
-        wrow[r] = p.words + row * kp;
+        wrow[r] = TMAJ ? p.words_tm + ((row >> 4) * p.kb64) * 256 + (row & 15) * 16 : p.words + row * kp;
     }
     const float *arow[PPT];
     bool row_live[PPT];
@@ -125,9 +128,15 @@ __global__ void __launch_bounds__(NW * 64) qgemv_rows16_kernel(Rows16Args p)
         for (int r = 0; r < RT; r++)
 #pragma unroll
             for (int t = 0; t < TPW; t++) {
-                const int64_t woff = wbase + t * 16 + g * 4;
-                const bool ok = woff + 4 <= kp;
-                const uint4 v = *reinterpret_cast<const uint4 *>(wrow[r] + (ok ? woff : kp - 4));
+                int64_t woff;
+                if constexpr (TMAJ) {   // k block min(wbase/16 + t, kb64 - 1) of the row's blocks (1 KB apart), words g*4 of its 64 bytes
+                    const int64_t kb = (wbase >> 4) + t;
+                    woff = (kb < p.kb64 ? kb : p.kb64 - 1) * 256 + g * 4;
+                } else {
+                    woff = wbase + t * 16 + g * 4;
+                    if (woff + 4 > kp) woff = kp - 4;
+                }
+                const uint4 v = *reinterpret_cast<const uint4 *>(wrow[r] + woff);
                 wq[r][t * 4 + 0] = v.x; wq[r][t * 4 + 1] = v.y; wq[r][t * 4 + 2] = v.z; wq[r][t * 4 + 3] = v.w;
             }
         __builtin_amdgcn_sched_barrier(0);   // every request of the round is out before anything waits
@@ -272,11 +281,14 @@ inline int rows16_tiles(int64_t n, int forced)
     return best;
 }
 
-template <int DT, int RT, bool SINGLE, int NW>
+template <int DT, int RT, bool SINGLE, int NW, bool TMAJ = false>
 void launch_rt(const Rows16Args &p, hipStream_t s)
 {
+    if constexpr (!TMAJ && !SINGLE) {   // (the tile-major variants exist for the default activation mode)
+        if (p.words_tm) return launch_rt<DT, RT, SINGLE, NW, true>(p, s);
+    }
     const dim3 grid((unsigned)((p.n + RT * 16 - 1) / (RT * 16))), blk(NW * 64);
-    hipLaunchKernelGGL((qgemv_rows16_kernel<DT, RT, SINGLE, NW>), grid, blk, 0, s, p);
+    hipLaunchKernelGGL((qgemv_rows16_kernel<DT, RT, SINGLE, NW, TMAJ>), grid, blk, 0, s, p);
 }
 
 template <int DT, bool SINGLE, int NW>
@@ -317,9 +329,12 @@ int fnn_mfma_rows16(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, co
     p.m = q.m; p.n = q.n; p.k = q.k; p.kp = q.kp; p.act = q.act;
     const bool single = (flags & FNN_FLAG_ACT_F16_SINGLE) != 0;
     p.umean = nullptr;
+    p.words_tm = nullptr; p.kb64 = 0;
     if (single) {
         int rc = fnn_row_means(ctx, s, w, &p.umean);
         if (rc) return rc;
+    } else if (int rc = fnn_tile_major_words(ctx, s, w, q, &p.words_tm, &p.kb64)) {
+        return rc;
     }
     const int rt = (int)fnn_ctx_option(ctx, FNN_OPT_ROWS16_ROW_TILES);   // 0: by the cost model
     hipError_t e;

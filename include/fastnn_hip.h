@@ -147,7 +147,7 @@ enum {
                                   /* below the row maximum, 2e-5 of max|ref| stated) or 4 (30 bits, 4e-6, a third more matrix-core */
                                   /* work and operand traffic); 0 (default) = three wherever they measured faster                  */
     FNN_OPT_GEMV_TILE_MAJOR = 23, /* the kernels that stream the packed words straight into matrix-core operand registers (M <= 8: */
-                                  /* I8 / I4 / U4 / U8 / F8 / F8R weights; the one-launch kernel for 17 <= M <= 32: every type)    */
+                                  /* I8 / I4 / U4 / U8 / F8 / F8R weights; 9 <= M <= 32: every per-channel type)                   */
                                   /* and the tile kernels of the types with 64 bytes per row and stage (I4 / U4 digit planes,      */
                                   /* U8 / F8 / F8R):                                                                               */
                                   /* 1 (default) = read them from a second device copy laid out in blocks of 16 rows x 64 bytes    */

@@ -400,7 +400,7 @@ def test_streaming_matmul_wide_outputs(ctx, orc, dt, m, k, n):
 
 
 @pytest.mark.parametrize("dt", [flib.DT_I8, flib.DT_I4, flib.DT_U4, flib.DT_U8, flib.DT_F8, flib.DT_F8R, flib.DT_F4])
-@pytest.mark.parametrize("m,k,n", [(1, 2048, 300), (6, 4096, 1000), (24, 2048, 1100), (40, 2048, 300), (200, 1024, 520)])
+@pytest.mark.parametrize("m,k,n", [(1, 2048, 300), (6, 4096, 1000), (12, 2048, 1100), (16, 8192, 72), (24, 2048, 1100), (40, 2048, 300), (200, 1024, 520)])
 def test_tile_major_copy_of_the_words_gives_the_same_bits(ctx, orc, dt, m, k, n):
     """The kernels that read the packed words from the tile-major copy (blocks of 16 rows x 64 bytes: the GEMV kernels,
     the streaming kernel, the tile kernels of the weight types with 64 bytes per row and stage) against the same
