@@ -612,7 +612,7 @@ int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QM
 
     TileArgs t = {};
     t.words = q.words;
-    if constexpr (DT != DT_F16_DENSE && DT != FNN_DT_I4CB && DecH<DT>::WPS == 2) {   // 8-bit types: 64 bytes per row and stage, one block of the tile-major copy
+    if constexpr (DT != DT_F16_DENSE && DT != FNN_DT_I4CB && (DecH<DT>::WPS == 2 || DecH<DT>::WPS == 1)) {   // 64 (8-bit types) or 32 bytes (4-bit) per row and stage: a block or half a block of the tile-major copy
         if (!dense)
             if (int rc2 = fnn_tile_major_words(ctx, s, w, q, &t.words_tm, &t.kb64)) return rc2;
     }

@@ -251,7 +251,8 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
         a_src[j] = p.ap + ((int64_t)mt * BM + row) * 64 + g * 8 - (j & 3) * 512;   // (biased: see load_group_to_lds16)
     }
     // weights: chunk (row, c) lives at slot row*WC + (c ^ swz(row)); rows past N repeat the last row
-    const bool tmaj = WC == 4 && !CB && p.words_tm != nullptr;   // (uniform)
+    // tile-major copy: 64 bytes per row and stage = one block per stage (WC == 4); 32 bytes = half a block (WC == 2)
+    const bool tmaj = (WC == 4 || WC == 2) && !CB && p.words_tm != nullptr;   // (uniform)
     const uint32_t *w_src[W_LPW];
     int w_chunk[W_LPW];
 #pragma unroll
@@ -266,7 +267,7 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
         if (tmaj) w_src[j] = p.words_tm + (((grow >> 4) * p.kb64) << 8) + ((grow & 15) << 4) + c * 4 - (j & 3) * 256;
         w_chunk[j] = c * 4;
     }
-    const int w_stride = tmaj ? 256 : WC * 4;   // words between consecutive stages of a row (tile-major: one block on)
+    const int w_stride = tmaj ? 256 : WC * 4;   // words between consecutive stages of a row (tile-major, WC == 4: one block on)
     const int64_t a_step = p.rows_pad * 64;   // elements between consecutive k blocks
     const unsigned a_dst = __builtin_amdgcn_readfirstlane(lds0 + wv * A_LPW * 1024);
     const unsigned w_dst = __builtin_amdgcn_readfirstlane(lds0 + A_BYTES + wv * W_LPW * 1024);
@@ -279,7 +280,7 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
 #pragma unroll
     for (int j = 0; j < A_LPW; j++) a_src[j] += (int64_t)(DENSE ? it0 % p.a_wrap : it0) * a_step;
 #pragma unroll
-    for (int j = 0; j < W_LPW; j++) w_src[j] += (int64_t)it0 * w_stride;
+    for (int j = 0; j < W_LPW; j++) w_src[j] += (tmaj && WC == 2) ? (int64_t)(it0 >> 1) * 256 + (it0 & 1) * 8 : (int64_t)it0 * w_stride;
     int a_pos = DENSE ? it0 % p.a_wrap : 0;       // position inside the activation sweep
     const bool ragged = !DENSE && (p.kp % (WC * 4)) != 0;
     bool w_past[W_LPW];   // this lane's chunk of the last stage lies behind the end of the row
@@ -323,7 +324,8 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
             a_pos = 0;
             astep = -(int64_t)(p.a_wrap - 1) * a_step;
         }
-        const int wstep = more ? w_stride : 0;
+        // (half blocks: from the even half to the odd half of a block 32 bytes, from there to the next block 1024 - 32)
+        const int wstep = !more ? 0 : ((tmaj && WC == 2) ? ((it & 1) ? 248 : 8) : w_stride);
 #pragma unroll
         for (int j = 0; j < A_LPW; j++) a_src[j] += astep;
 #pragma unroll

@@ -148,8 +148,8 @@ enum {
                                   /* work and operand traffic); 0 (default) = three wherever they measured faster                  */
     FNN_OPT_GEMV_TILE_MAJOR = 23, /* the kernels that stream the packed words straight into matrix-core operand registers (M <= 8: */
                                   /* I8 / I4 / U4 / U8 / F8 / F8R weights; 9 <= M <= 32: every per-channel type)                   */
-                                  /* and the tile kernels of the types with 64 bytes per row and stage (I4 / U4 digit planes,      */
-                                  /* U8 / F8 / F8R):                                                                               */
+                                  /* and the tile kernels of the types with 64 or 32 bytes per row and stage (I4 / U4 digit        */
+                                  /* planes, U8 / F8 / F8R / F4):                                                                  */
                                   /* 1 (default) = read them from a second device copy laid out in blocks of 16 rows x 64 bytes    */
                                   /* (one contiguous KB per wave load: same bits, C1 M=1 5.97 -> 5.15 us, C2 6.70 -> 6.41, FP8     */
                                   /* 4096 x 4096 5.90 -> 5.40), built on the weight's first such call and kept with it (once more  */
