@@ -13,7 +13,8 @@
 // tiles x splits).  Per round:
 //   1. every wave requests its packed bytes (16 rows x KR values per row tile, raw buffer loads: rows past N and
 //      bytes past the buffer read as zero) and its share of the activation block (16*MB rows x KR values, split in
-//      units of 16 rows x one lane load of weights);
+//      units of 16 rows x one lane load of weights; the four lanes of a row load 64 contiguous bytes per
+//      instruction, and step 3 scatters each register to the fragment of the lane that multiplies it);
 //   2. row maxima and row sums of the round meet in LDS; every row gets one power-of-two scale per round;
 //   3. the units are converted into MFMA operand fragments in LDS, laid out so that a fragment is 64 lanes x 16
 //      contiguous bytes (conflict-free reads, no swizzle):
@@ -153,19 +154,23 @@ __global__ void __launch_bounds__(NW * 64) qgemm_stream_kernel(StreamArgs p)
         const int64_t k0 = kbeg + (int64_t)round * KR;
         // ---- 1. requests: this wave's activation units first (they come from the L2 and their conversion must not
         // wait for the packed bytes behind them: loads return in order), then the packed bytes, the long pole
+        // Load j of a unit covers, for every row, 64 contiguous bytes with the four lanes of the row (lane (ln, g): the
+        // four values k = chunk + 16 j + 4 g ..), so neighbouring lanes consume neighbouring pieces of a line; the values a
+        // lane converts are therefore not the ones its own weight bytes meet, and the conversion below writes every
+        // register's digits (or halves) where the lane that multiplies them will read them.
         u32x4 xr[UPW][FPL / 4];
 #pragma unroll
         for (int u = 0; u < UPW; u++) {
             const int unit = wv + u * NW;
             const int c = unit % LOADS, b = unit / LOADS;
             const int row = b * 16 + ln;
-            const int64_t kk = k0 + c * CHUNK + g * FPL;
+            const int64_t kk = k0 + c * CHUNK + g * 4;
 #pragma unroll
             for (int j = 0; j < FPL / 4; j++) {
                 // K % 8 == 0: a 16-byte piece lies wholly inside or wholly past K; past K (or past the units of the
                 // round) the offset leaves the buffer and the load returns zero
-                const bool ok = unit < UNITS && row < mreal && kk + j * 4 < K;
-                const uint32_t off = ok ? (uint32_t)(((int64_t)row * K + kk + j * 4) * 4) : 0xFFFFFF00u;
+                const bool ok = unit < UNITS && row < mreal && kk + j * 16 < K;
+                const uint32_t off = ok ? (uint32_t)(((int64_t)row * K + kk + j * 16) * 4) : 0xFFFFFF00u;
                 xr[u][j] = __builtin_amdgcn_raw_buffer_load_b128(abuf, off, 0, 0);
             }
         }
@@ -245,12 +250,9 @@ __global__ void __launch_bounds__(NW * 64) qgemm_stream_kernel(StreamArgs p)
 #pragma unroll
             for (int cc = 0; cc < LOADS; cc++) mx = fmaxf(mx, pmax[cc][b * 16 + ln]);
             int ex = (int)((__float_as_uint(mx) >> 23) & 0xff) - 127;
-            float x[FPL];
-#pragma unroll
-            for (int j = 0; j < FPL / 4; j++)
-#pragma unroll
-                for (int e = 0; e < 4; e++) x[j * 4 + e] = __uint_as_float(xr[u][j][e]);
-            uint4 *dst = frag + ((size_t)(c * SUB) * MB + b) * 64 + lane;   // fragment `sub` at dst[sub * MB * 64]
+            // register j holds the values f0 .. f0 + 3 of the unit's chunk, f0 = 16 j + 4 g: they belong to the k group
+            // f0 / FPL of the row (the lane (ln, f0 / FPL) of the MFMA operand), local index f0 % FPL
+            unsigned char *fbase = reinterpret_cast<unsigned char *>(frag + ((size_t)(c * SUB) * MB + b) * 64);   // fragment `sub` MB * 1024 bytes further
             if constexpr (INT8) {
                 ex = mx == 0.0f ? 0 : ex - 21;
                 // v = rint(x * 2^-e), |v| < 2^22.  Its balanced base-256 digits (each in [-128, 127], v = sum d_j 256^j,
@@ -260,46 +262,53 @@ __global__ void __launch_bounds__(NW * 64) qgemm_stream_kernel(StreamArgs p)
                 // offset are one constant.  2^-e is applied as an exact factor in two steps (e spans -148 .. 106).
                 const int e1 = -ex / 2, e2 = -ex - e1;
                 const float f1 = __uint_as_float((uint32_t)(127 + e1) << 23), f2 = __uint_as_float((uint32_t)(127 + e2) << 23);
-                uint32_t dg[FPL];
 #pragma unroll
-                for (int j = 0; j < FPL; j++)
-                    dg[j] = (__float_as_uint(__builtin_fmaf(x[j] * f1, f2, 12582912.0f)) + (0x00808080u - 0x4B400000u)) ^ 0x00808080u;
-                uint32_t pl[PAR][3][4];   // [parity][plane][word]
+                for (int j = 0; j < FPL / 4; j++) {
+                    uint32_t dg[4];
 #pragma unroll
-                for (int w = 0; w < 4; w++) {
-                    uint32_t t[4];
+                    for (int e = 0; e < 4; e++)
+                        dg[e] = (__float_as_uint(__builtin_fmaf(__uint_as_float(xr[u][j][e]) * f1, f2, 12582912.0f)) + (0x00808080u - 0x4B400000u)) ^ 0x00808080u;
+                    const int f0 = j * 16 + g * 4, owner = f0 / FPL, li = f0 % FPL;
+                    unsigned char *dl = fbase + (owner * 16 + ln) * 16;
                     if constexpr (PAR == 1) {
-                        // bytes 4w..4w+3 of the lane load are k = 4w..4w+3
-                        transpose4(dg[4 * w], dg[4 * w + 1], dg[4 * w + 2], dg[4 * w + 3], t);
-                        pl[0][0][w] = t[0]; pl[0][1][w] = t[1]; pl[0][2][w] = t[2];
+                        // bytes 4w .. 4w + 3 of the owner's lane load are k = 4w .. 4w + 3: word w = li / 4 of each plane
+                        uint32_t t[4];
+                        transpose4(dg[0], dg[1], dg[2], dg[3], t);
+#pragma unroll
+                        for (int pln = 0; pln < 3; pln++) *reinterpret_cast<uint32_t *>(dl + (size_t)pln * MB * 1024 + (li / 4) * 4) = t[pln];
                     } else {
-                        // word w of the lane load holds k = 8w..8w+7: low nibbles are the even, high nibbles the odd ones
-                        transpose4(dg[8 * w], dg[8 * w + 2], dg[8 * w + 4], dg[8 * w + 6], t);
-                        pl[0][0][w] = t[0]; pl[0][1][w] = t[1]; pl[0][2][w] = t[2];
-                        transpose4(dg[8 * w + 1], dg[8 * w + 3], dg[8 * w + 5], dg[8 * w + 7], t);
-                        pl[PAR - 1][0][w] = t[0]; pl[PAR - 1][1][w] = t[1]; pl[PAR - 1][2][w] = t[2];
+                        // word w = li / 8 of the owner's lane load holds k = 8w .. 8w + 7, low nibbles the even, high nibbles the
+                        // odd ones: these four values are elements (li % 8) / 2 and + 1 of the word's even and of its odd operand
+                        const int wbyte = (li / 8) * 4 + ((li % 8) / 2);
+#pragma unroll
+                        for (int pln = 0; pln < 3; pln++) {
+                            const uint32_t sel = 0x0c0c0400u + 0x0101u * pln;   // byte `pln` of the second, then of the first operand
+                            const uint32_t ev = __builtin_amdgcn_perm(dg[2], dg[0], sel), od = __builtin_amdgcn_perm(dg[3], dg[1], sel);
+                            *reinterpret_cast<uint16_t *>(dl + (size_t)pln * MB * 1024 + wbyte) = (uint16_t)ev;
+                            *reinterpret_cast<uint16_t *>(dl + (size_t)(3 + pln) * MB * 1024 + wbyte) = (uint16_t)od;
+                        }
                     }
                 }
-#pragma unroll
-                for (int q = 0; q < PAR; q++)
-#pragma unroll
-                    for (int j = 0; j < 3; j++) dst[(q * 3 + j) * MB * 64] = uint4{pl[q][j][0], pl[q][j][1], pl[q][j][2], pl[q][j][3]};
             } else {
                 ex = mx == 0.0f ? 0 : ex - 14;
                 ex = ex < -100 ? -100 : (ex > 120 ? 120 : ex);
                 const float inv = __uint_as_float((uint32_t)(127 - ex) << 23);
 #pragma unroll
-                for (int s = 0; s < SPL; s++) {
-                    f16x8 hi, lo;
+                for (int j = 0; j < FPL / 4; j++) {
+                    typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+                    f16x4 hi, lo;
 #pragma unroll
-                    for (int e = 0; e < 8; e++) {
-                        const float v = x[s * 8 + e] * inv;
+                    for (int e = 0; e < 4; e++) {
+                        const float v = __uint_as_float(xr[u][j][e]) * inv;
                         const _Float16 h = (_Float16)v;
                         hi[e] = h;
                         lo[e] = (_Float16)(v - (float)h);
                     }
-                    dst[(s * 2) * MB * 64] = __builtin_bit_cast(uint4, hi);
-                    dst[(s * 2 + 1) * MB * 64] = __builtin_bit_cast(uint4, lo);
+                    // MFMA step li / 8 of the owner's lane load, halves (li % 8) .. + 3 of its hi and of its lo fragment
+                    const int f0 = j * 16 + g * 4, owner = f0 / FPL, li = f0 % FPL;
+                    unsigned char *dl = fbase + (owner * 16 + ln) * 16 + (li % 8) * 2;
+                    *reinterpret_cast<f16x4 *>(dl + (size_t)((li / 8) * 2) * MB * 1024) = hi;
+                    *reinterpret_cast<f16x4 *>(dl + (size_t)((li / 8) * 2 + 1) * MB * 1024) = lo;
                 }
             }
         }
