@@ -19,7 +19,7 @@ LIB = os.path.join(HERE, "libfastnn_hip.so")
 
 HIP_SOURCES = ["api.hip", "qgemv.hip", "qgemm_generic.hip", "qgemm_tiled.hip", "qgemm_i8.hip", "qgemm_digits.hip", "qgemv_mfma.hip", "qgemv_i8dot.hip", "qgemv_rows16.hip", "i8act.hip", "qconv.hip", "qconv_float.hip", "qconv_implicit.hip", "eltwise.hip",
                "qgemm_stream.hip", "qgemm_stream_i8.hip", "qgemm_stream_i4.hip", "qgemm_stream_u4.hip", "qgemm_stream_u8.hip",
-               "qgemm_stream_f8.hip", "qgemm_stream_f8r.hip", "qgemm_stream_f4.hip"]
+               "qgemm_stream_f8.hip", "qgemm_stream_f8r.hip", "qgemm_stream_f4.hip", "qgemm_stream_i4cb.hip"]
 HOST_SOURCES = ["quantize_host.cpp", "hip_backend.cpp"]
 
 # -ffp-contract=off: the integer/quantisation formulas must evaluate exactly as written;

@@ -14,6 +14,19 @@ __device__ __forceinline__ f16x8 pack8(uint32_t a, uint32_t b, uint32_t c, uint3
     return __builtin_bit_cast(f16x8, u32x4{a, b, c, d});
 }
 
+// power of two that brings the largest table magnitude into [2^14, 2^15): the f16 hi + lo split of the scaled table
+// then carries ~22 bits of every entry (every thread computes the same value from the 16 cached floats)
+__device__ __forceinline__ int codebook_exp(const float *cb)
+{
+    float mx = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; i++) mx = fmaxf(mx, fabsf(cb[i]));
+    if (!(mx > 0.0f) || !(mx < __builtin_huge_valf())) return 0;
+    int ex;
+    (void)frexpf(mx, &ex);
+    return 15 - ex;
+}
+
 // Decoders: one MFMA step = 8 k-values of one weight row as f16x8.  `w` points at the
 // lane's packed words for the step (1 word for 4-bit types, 2 for 8-bit types).
 // PERM tells in which order the 8 k-values land in the operand (the activation fragments

@@ -4,7 +4,9 @@
 
 struct StreamArgs {
     const uint32_t *words;
-    const float *scales, *zeros, *a, *bias;
+    const float *scales, *zeros, *a, *bias;   // codebook weights: scales = block scales [n][bpr], zeros unused
+    const float *codebook;   // codebook weights: the 16 table values
+    int64_t bpr;             // ... blocks of 32 values per row
     float *out;
     const float *residual;   // a plan's Add behind this MatMul: sum_out[i] = out[i] + residual[i], or null
     float *sum_out;
@@ -30,3 +32,4 @@ hipError_t fnn_stream_launch_u8(const StreamPlan &pl, const StreamArgs &p, hipSt
 hipError_t fnn_stream_launch_f8(const StreamPlan &pl, const StreamArgs &p, hipStream_t s);
 hipError_t fnn_stream_launch_f8r(const StreamPlan &pl, const StreamArgs &p, hipStream_t s);
 hipError_t fnn_stream_launch_f4(const StreamPlan &pl, const StreamArgs &p, hipStream_t s);
+hipError_t fnn_stream_launch_i4cb(const StreamPlan &pl, const StreamArgs &p, hipStream_t s);

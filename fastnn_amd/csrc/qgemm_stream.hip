@@ -9,10 +9,10 @@ namespace {
 // RT, KR, splits and rounds from FNN_OPT_STREAM_SHAPE or by rule (MB follows from M).  The phases of a round (requests,
 // conversion, matrix cores) follow one another inside a workgroup, so a workgroup does one round where it can: one row
 // tile per wave, K / KR splits, and KR = 512 while that still gives the 256 CUs a workgroup each.
-bool plan_stream(int bits, bool int8, int64_t m, int64_t n, int64_t k, int64_t forced, StreamPlan *out)
+bool plan_stream(int bits, int max_tiles, int max_mb, int64_t m, int64_t n, int64_t k, int64_t forced, StreamPlan *out)
 {
     const int mb = (int)((m + 15) / 16);
-    if (mb < 1 || mb > 2) return false;   // (three and four blocks measured slower than the tiled path)
+    if (mb < 1 || mb > max_mb) return false;
     int rt = 1, kr = 512;
     const int64_t nt1 = (n + FNN_STREAM_NW * 16 - 1) / (FNN_STREAM_NW * 16);
     if (nt1 * ((k + 511) / 512) < 224) kr = 256;
@@ -23,7 +23,7 @@ bool plan_stream(int bits, bool int8, int64_t m, int64_t n, int64_t k, int64_t f
         splits = forced >> 8;
         if (rt < 1 || rt > 2 || (kr != 256 && kr != 512)) return false;
     }
-    if (mb * rt > (int8 ? 4 : 8)) return false;   // accumulator tiles that fit the registers
+    if (mb * rt > max_tiles) return false;   // accumulator tiles that fit the registers
     const int64_t kr_total = (k + kr - 1) / kr;   // rounds over all of K
     if (splits == 0) splits = kr_total > 64 ? 64 : kr_total;
     if (splits > kr_total || splits > 64) return false;
@@ -38,7 +38,7 @@ bool plan_stream(int bits, bool int8, int64_t m, int64_t n, int64_t k, int64_t f
         // Wide outputs: two row tiles per wave (256 weight rows per workgroup) and as few rounds per workgroup as keep the
         // launch within one round of workgroups.  4096 x 11008 (43 column tiles): 4 splits x 2 rounds of 512, 172 workgroups,
         // M = 17 19.2 us against 23.0 on the tiled path, M = 32 21.3 against 23.9 (8 splits x 1 round, 344 workgroups: 25.5).
-        if (mb * 2 > (int8 ? 4 : 8)) return false;
+        if (mb * 2 > max_tiles) return false;
         const int64_t ntiles2 = (n + FNN_STREAM_NW * 2 * 16 - 1) / (FNN_STREAM_NW * 2 * 16);
         const int64_t total512 = (k + 511) / 512;
         for (int64_t r2 = 1; r2 <= 4; r2++) {
@@ -60,12 +60,20 @@ bool plan_stream(int bits, bool int8, int64_t m, int64_t n, int64_t k, int64_t f
 int fnn_stream_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QMatmulArgs &q, int flags, bool *handled)
 {
     *handled = false;
-    const int64_t lo = fnn_ctx_option(ctx, FNN_OPT_STREAM_MIN_M), hi = fnn_ctx_option(ctx, FNN_OPT_STREAM_MAX_M);
-    if (q.m < lo || q.m > hi || q.m > 32 || q.n < 1) return FNN_OK;
-    if (flags & FNN_FLAG_ACT_F16_SINGLE) return FNN_OK;
+    int64_t lo = fnn_ctx_option(ctx, FNN_OPT_STREAM_MIN_M), hi = fnn_ctx_option(ctx, FNN_OPT_STREAM_MAX_M);
     const int dt = w->dtype;
+    const bool cb = dt == FNN_DT_I4CB;
+    // Per-channel types: up to two blocks of 16 activation rows (three and four measured slower than the tiled path).
+    // Codebook weights: the tiled path decodes them on the vector ALU inside its loop and is far from the memory bound,
+    // so the range is wider, 5 <= M <= 64 with the options at their defaults.
+    if (cb) { lo = lo < 5 ? lo : 5; hi = hi >= 32 ? 64 : hi; }
+    if (q.m < lo || q.m > hi || q.m > (cb ? 64 : 32) || q.n < 1) return FNN_OK;
+    if (flags & FNN_FLAG_ACT_F16_SINGLE) return FNN_OK;
     const bool int_type = dt == FNN_DT_I8 || dt == FNN_DT_I4 || dt == FNN_DT_U4;
-    if (dt == FNN_DT_I4CB) return FNN_OK;
+    if (cb && fnn_ctx_option(ctx, FNN_OPT_CODEBOOK_EXPANDED) != 0) return FNN_OK;   // (the option names a form of the tiled path)
+    if (cb && (q.as_written || q.qblock != 32 || q.k % 128 != 0 || q.bpr != q.k / 32 || (reinterpret_cast<uintptr_t>(q.scales) & 15) ||
+               q.bpr * 4 * 256 >= (int64_t)1 << 31)) return FNN_OK;
+    if (dt < FNN_DT_I8 || (dt > FNN_DT_F4 && !cb)) return FNN_OK;
     if (int_type && fnn_ctx_option(ctx, FNN_OPT_GEMM_INT8) == 0) return FNN_OK;
     if (q.kp % 4 != 0 || q.k % 8 != 0 || q.k < 8) return FNN_OK;
     // the f16 types multiply whatever bytes a lane load holds: every load must lie wholly inside or wholly past K
@@ -75,11 +83,12 @@ int fnn_stream_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w,
     if (q.kp * 4 * 256 >= (int64_t)1 << 31 || q.m * q.k * 4 >= (int64_t)0xFFFFFF00 || q.k >= (int64_t)1 << 28) return FNN_OK;
     StreamPlan pl;
     const int64_t forced = fnn_ctx_option(ctx, FNN_OPT_STREAM_SHAPE);
-    const int bits = (dt == FNN_DT_I4 || dt == FNN_DT_U4 || dt == FNN_DT_F4) ? 4 : 8;
-    if (!plan_stream(bits, int_type, q.m, q.n, q.k, forced, &pl)) return FNN_OK;
+    const int bits = (dt == FNN_DT_I4 || dt == FNN_DT_U4 || dt == FNN_DT_F4 || cb) ? 4 : 8;
+    if (!plan_stream(bits, int_type ? 4 : (cb ? 6 : 8), cb ? 4 : 2, q.m, q.n, q.k, forced, &pl)) return FNN_OK;
     if (pl.ntiles > FNN_STREAM_COUNTERS) return FNN_OK;
     StreamArgs p;
     p.words = q.words; p.scales = q.scales; p.zeros = q.zeros; p.a = q.a; p.bias = q.bias; p.out = q.out;
+    p.codebook = cb ? q.codebook : nullptr; p.bpr = cb ? q.bpr : 0;
     p.residual = nullptr; p.sum_out = nullptr;
     p.part = nullptr; p.count = fnn_ctx_stream_counters(ctx);
     p.m = q.m; p.n = q.n; p.k = q.k; p.kp = q.kp;
@@ -104,6 +113,7 @@ int fnn_stream_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w,
     case FNN_DT_U8: e = fnn_stream_launch_u8(pl, p, s); break;
     case FNN_DT_F8: e = fnn_stream_launch_f8(pl, p, s); break;
     case FNN_DT_F8R: e = fnn_stream_launch_f8r(pl, p, s); break;
+    case FNN_DT_I4CB: e = fnn_stream_launch_i4cb(pl, p, s); break;
     default: e = fnn_stream_launch_f4(pl, p, s); break;
     }
     if (e != hipSuccess) return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, hipGetErrorString(e));

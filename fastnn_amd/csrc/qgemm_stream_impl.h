@@ -22,6 +22,10 @@
 //          v_mfma_i32_16x16x64_i8 against the packed bytes as they are (4-bit lanes: one mask / shift-mask per word);
 //        U8 / F8 / F8R / F4 weights: f16 hi + lo of x * 2^-e (about 22 mantissa bits) for v_mfma_f32_16x16x32_f16
 //          against the weights decoded to f16 in registers (exact for every one of these types);
+//        codebook weights (blocks of 32 values with an f32 scale each, 16 table values): the same activation halves
+//          against the f16 hi and lo of the table value (scaled by one power of two) that a nibble looks up in a
+//          16-word LDS table; one MFMA step is one block, its sum is folded into the running sum with the block's
+//          scale: sum_blk s_blk * sum_k table[q] * a, the reference's association (src/packed_tensor.rs:469-521);
 //   4. every wave multiplies its row tiles with all MB activation blocks; integer plane sums are exact and are
 //      recombined in f32 once per round.
 // Split K: a workgroup stores its partial accumulator registers and row sums with agent-scope (write-through)
@@ -54,6 +58,7 @@ template <> struct StreamType<FNN_DT_U8> { static constexpr int BITS = 8; static
 template <> struct StreamType<FNN_DT_F8> { static constexpr int BITS = 8; static constexpr bool INT8 = false; static constexpr float POST = 1.0f; };
 template <> struct StreamType<FNN_DT_F8R> { static constexpr int BITS = 8; static constexpr bool INT8 = false; static constexpr float POST = 1.0f; };
 template <> struct StreamType<FNN_DT_F4> { static constexpr int BITS = 4; static constexpr bool INT8 = false; static constexpr float POST = 1.0f; };
+template <> struct StreamType<FNN_DT_I4CB> { static constexpr int BITS = 4; static constexpr bool INT8 = false; static constexpr float POST = 1.0f; };
 
 // int8 operand of one MFMA from the four words of a lane load (4-bit types: even nibbles, then odd nibbles)
 template <int DT>
@@ -104,6 +109,7 @@ __global__ void __launch_bounds__(NW * 64) qgemm_stream_kernel(StreamArgs p)
 {
     using T = StreamType<DT>;
     constexpr bool INT8 = T::INT8;
+    constexpr bool CB = DT == FNN_DT_I4CB;           // nibbles look up a 16-entry table; one f32 scale per 32 values
     constexpr int BITS = T::BITS;
     constexpr int LOADS = KR * BITS / 8 / 64;        // 16-byte lane loads per weight row tile and round
     constexpr int FPL = 128 / BITS;                  // activations a lane converts per unit: those its 16 weight bytes meet
@@ -117,7 +123,7 @@ __global__ void __launch_bounds__(NW * 64) qgemm_stream_kernel(StreamArgs p)
     constexpr int NT = NW * RT * 16;                 // weight rows of a workgroup
     constexpr int SLOTS = MB * RT * 4;               // accumulator registers per thread
     static_assert(LOADS >= 1 && KR % CHUNK == 0, "a round is whole lane loads");
-    static_assert(INT8 || !DecH<DT>::INTERLEAVED, "operand order of the f16 decoders used here is the memory order");
+    if constexpr (!INT8 && !CB) static_assert(!DecH<DT>::INTERLEAVED, "operand order of the f16 decoders used here is the memory order");
 
     extern __shared__ __attribute__((aligned(16))) uint4 frag[];   // [LOADS][SUB][MB][64 lanes]
     __shared__ float pmax[LOADS][ROWS], psum[LOADS][ROWS];
@@ -125,6 +131,7 @@ __global__ void __launch_bounds__(NW * 64) qgemm_stream_kernel(StreamArgs p)
     __shared__ int cse[ROWS];        // int8 path: e per row, INT_MIN marks a row with a non-finite activation
     __shared__ float xs[ROWS];       // row sums over the workgroup's K range (over all of K after the reduction)
     __shared__ int last_flag;
+    __shared__ uint32_t cbt[16];     // codebook weights: f16 hi | f16 lo << 16 of table value * 2^cb_exp
 
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const int ln = lane & 15, g = lane >> 4;
@@ -139,6 +146,19 @@ __global__ void __launch_bounds__(NW * 64) qgemm_stream_kernel(StreamArgs p)
     const __amdgpu_buffer_rsrc_t abuf = raw_buffer(p.a, (uint64_t)mreal * (uint64_t)K * 4);
     const uint32_t wlane = TMAJ ? (uint32_t)(wv * RT) * (uint32_t)p.kb64 * 1024 + (uint32_t)ln * 64 + (uint32_t)g * 16
                                 : (uint32_t)(wv * RT * 16 + ln) * (uint32_t)kp * 4 + (uint32_t)g * 16;
+
+    // codebook weights: the block scales of the workgroup's rows, [row][bpr]; the table
+    const __amdgpu_buffer_rsrc_t sbuf = raw_buffer(CB ? p.scales + n0 * p.bpr : p.scales, CB ? (uint64_t)(N - n0) * (uint64_t)p.bpr * 4 : 0);
+    int cb_exp = 0;
+    if constexpr (CB) {
+        cb_exp = codebook_exp(p.codebook);
+        if (tid < 16) {
+            const float v = ldexpf(p.codebook[tid], cb_exp);
+            const _Float16 h = (_Float16)v, l = (_Float16)(v - (float)h);
+            cbt[tid] = (uint32_t)__builtin_bit_cast(uint16_t, h) | ((uint32_t)__builtin_bit_cast(uint16_t, l) << 16);
+        }
+        // (the first barrier of the first round orders these writes before the first look-up)
+    }
 
     float e_scale[RT], e_zero[RT], e_bias[RT];   // epilogue operands of this lane's columns
     float tot[MB][RT][4];
@@ -188,6 +208,19 @@ __global__ void __launch_bounds__(NW * 64) qgemm_stream_kernel(StreamArgs p)
                                             : wlane + (uint32_t)r * 16 * (uint32_t)kp * 4 + wk + l * 64;
                 wq[r][l] = __builtin_amdgcn_raw_buffer_load_b128(wbuf, off, 0, 0);
             }
+        // codebook weights: the scales of the four blocks a lane load of a row covers (the four lanes of a row ask for
+        // the same 16 bytes)
+        u32x4 bsq[CB ? RT : 1][CB ? LOADS : 1];
+        if constexpr (CB) {
+#pragma unroll
+            for (int r = 0; r < RT; r++)
+#pragma unroll
+                for (int l = 0; l < LOADS; l++) {
+                    const uint32_t off = !(k0 + l * CHUNK < K) ? 0xFFFFFF00u
+                                                               : (uint32_t)((wv * RT + r) * 16 + ln) * (uint32_t)p.bpr * 4 + (uint32_t)((k0 >> 5) + l * 4) * 4;
+                    bsq[r][l] = __builtin_amdgcn_raw_buffer_load_b128(sbuf, off, 0, 0);
+                }
+        }
         __builtin_amdgcn_sched_barrier(0);
 
         if (round == 0) {   // requested behind the first round's operands: needed last, and loads return in order
@@ -195,8 +228,8 @@ __global__ void __launch_bounds__(NW * 64) qgemm_stream_kernel(StreamArgs p)
             for (int r = 0; r < RT; r++) {
                 const int64_t n = n0 + (wv * RT + r) * 16 + ln;
                 const bool ok = n < N;
-                e_scale[r] = p.scales[ok ? n : 0];
-                e_zero[r] = p.zeros[ok ? n : 0];
+                e_scale[r] = CB ? ldexpf(1.0f, -cb_exp) : p.scales[ok ? n : 0];   // (block scales are applied in the loop)
+                e_zero[r] = CB ? 0.0f : p.zeros[ok ? n : 0];
                 e_bias[r] = p.bias ? p.bias[ok ? n : 0] : 0.0f;
             }
         }
@@ -305,10 +338,12 @@ __global__ void __launch_bounds__(NW * 64) qgemm_stream_kernel(StreamArgs p)
                         lo[e] = (_Float16)(v - (float)h);
                     }
                     // MFMA step li / 8 of the owner's lane load, halves (li % 8) .. + 3 of its hi and of its lo fragment
-                    const int f0 = j * 16 + g * 4, owner = f0 / FPL, li = f0 % FPL;
-                    unsigned char *dl = fbase + (owner * 16 + ln) * 16 + (li % 8) * 2;
-                    *reinterpret_cast<f16x4 *>(dl + (size_t)((li / 8) * 2) * MB * 1024) = hi;
-                    *reinterpret_cast<f16x4 *>(dl + (size_t)((li / 8) * 2 + 1) * MB * 1024) = lo;
+                    // (codebook weights: a step is one block of 32 values, the owner holds its values 8 * owner ..)
+                    const int f0 = j * 16 + g * 4;
+                    const int owner = CB ? (f0 % 32) / 8 : f0 / FPL, step = CB ? f0 / 32 : (f0 % FPL) / 8;
+                    unsigned char *dl = fbase + (owner * 16 + ln) * 16 + (f0 % 8) * 2;
+                    *reinterpret_cast<f16x4 *>(dl + (size_t)(step * 2) * MB * 1024) = hi;
+                    *reinterpret_cast<f16x4 *>(dl + (size_t)(step * 2 + 1) * MB * 1024) = lo;
                 }
             }
         }
@@ -356,6 +391,85 @@ __global__ void __launch_bounds__(NW * 64) qgemm_stream_kernel(StreamArgs p)
                         const float v = fmaf(fmaf((float)acc[2][b][r][i], 256.0f, (float)acc[1][b][r][i]), 256.0f, (float)acc[0][b][r][i]);
                         tot[b][r][i] += ee[i] == INT_MIN ? __uint_as_float(0x7fc00000u) : ldexpf(v, ee[i]);
                     }
+            }
+        } else if constexpr (CB) {
+            // A lane load holds the four words of ONE block of its row, lane (ln, g) that of block 4 l + g; an MFMA step
+            // must be one block over all four k groups, so the words are transposed across the groups: afterwards word s
+            // of lane (ln, g) is word g (values 8 g .. 8 g + 7) of block 4 l + s.
+#pragma unroll
+            for (int r = 0; r < RT; r++)
+#pragma unroll
+                for (int l = 0; l < LOADS; l++) {
+                    // rows 2, 3 of the first operand <-> rows 0, 1 of the second; then odd rows <-> even rows (a row: 16 lanes)
+                    const auto s02 = __builtin_amdgcn_permlane32_swap(wq[r][l][0], wq[r][l][2], false, false);
+                    const auto s13 = __builtin_amdgcn_permlane32_swap(wq[r][l][1], wq[r][l][3], false, false);
+                    const auto t01 = __builtin_amdgcn_permlane16_swap(s02[0], s13[0], false, false);
+                    const auto t23 = __builtin_amdgcn_permlane16_swap(s02[1], s13[1], false, false);
+                    wq[r][l] = u32x4{t01[0], t01[1], t23[0], t23[1]};
+                }
+            constexpr int ITEMS = LOADS * SPL * MB;       // (lane load, block, activation block): a hi and a lo fragment each
+            constexpr int DEPTH = ITEMS < 3 ? ITEMS : 3;
+            f32x4 acc[MB][RT];
+#pragma unroll
+            for (int b = 0; b < MB; b++)
+#pragma unroll
+                for (int r = 0; r < RT; r++) acc[b][r] = f32x4{0.f, 0.f, 0.f, 0.f};
+            uint4 rhi[DEPTH], rlo[DEPTH];
+#pragma unroll
+            for (int i = 0; i < DEPTH; i++) {
+                const int b = i % MB, ls = i / MB;
+                rhi[i] = frd[((ls * 2) * MB + b) * 64];
+                rlo[i] = frd[((ls * 2 + 1) * MB + b) * 64];
+            }
+            f16x8 bwh[RT], bwl[RT];
+            float bsc[RT];
+#pragma unroll
+            for (int i = 0; i < ITEMS; i++) {
+                const int b = i % MB, ls = i / MB, sidx = ls % SPL, l = ls / SPL;
+                if (b == 0) {
+#pragma unroll
+                    for (int r = 0; r < RT; r++) {
+                        const uint32_t w = wq[r][l][sidx];
+                        uint32_t d[8];
+                        d[0] = cbt[w & 15u];
+#pragma unroll
+                        for (int j = 1; j < 8; j++) d[j] = cbt[(w >> (4 * j)) & 15u];
+                        uint32_t h4[4], l4[4];
+#pragma unroll
+                        for (int j = 0; j < 4; j++) {
+                            h4[j] = __builtin_amdgcn_perm(d[2 * j + 1], d[2 * j], 0x05040100u);   // low halves: hi parts
+                            l4[j] = __builtin_amdgcn_perm(d[2 * j + 1], d[2 * j], 0x07060302u);   // high halves: lo parts
+                        }
+                        bwh[r] = __builtin_bit_cast(f16x8, u32x4{h4[0], h4[1], h4[2], h4[3]});
+                        bwl[r] = __builtin_bit_cast(f16x8, u32x4{l4[0], l4[1], l4[2], l4[3]});
+                        bsc[r] = __uint_as_float(bsq[r][l][sidx]);
+                    }
+                }
+                const f16x8 ahi = __builtin_bit_cast(f16x8, rhi[i % DEPTH]);
+                const f16x8 alo = __builtin_bit_cast(f16x8, rlo[i % DEPTH]);
+                if (i + DEPTH < ITEMS) {
+                    const int nb = (i + DEPTH) % MB, nls = (i + DEPTH) / MB;
+                    rhi[i % DEPTH] = frd[((nls * 2) * MB + nb) * 64];
+                    rlo[i % DEPTH] = frd[((nls * 2 + 1) * MB + nb) * 64];
+                }
+#pragma unroll
+                for (int r = 0; r < RT; r++) {
+                    // the block's sum (the lo x lo product is below 2^-22 of the terms), then the block scale
+                    f32x4 blk = __builtin_amdgcn_mfma_f32_16x16x32_f16(alo, bwh[r], f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                    blk = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahi, bwl[r], blk, 0, 0, 0);
+                    blk = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahi, bwh[r], blk, 0, 0, 0);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) acc[b][r][e] = fmaf(bsc[r], blk[e], acc[b][r][e]);
+                }
+            }
+#pragma unroll
+            for (int b = 0; b < MB; b++) {
+                const float4 c4 = *reinterpret_cast<const float4 *>(&csc[b * 16 + g * 4]);
+                const float cc[4] = {c4.x, c4.y, c4.z, c4.w};
+#pragma unroll
+                for (int r = 0; r < RT; r++)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) tot[b][r][i] = fmaf(acc[b][r][i], cc[i], tot[b][r][i]);
             }
         } else {
             using D = DecH<DT>;
@@ -497,7 +611,7 @@ __global__ void __launch_bounds__(NW * 64) qgemm_stream_kernel(StreamArgs p)
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 const float dot = tot[b][r][i] * T::POST;
-                v[i] = dot * e_scale[r] + e_zero[r] * xx[i];
+                v[i] = CB ? dot * e_scale[r] : dot * e_scale[r] + e_zero[r] * xx[i];
                 if (p.bias) v[i] = v[i] + e_bias[r];
                 v[i] = fnn_activation(v[i], p.act);
             }
@@ -545,7 +659,7 @@ template <int DT, int MB>
 hipError_t launch_mb(const StreamPlan &pl, const StreamArgs &p, hipStream_t s)
 {
     using T = StreamType<DT>;
-    constexpr int kTiles = T::INT8 ? 4 : 8;   // MB * RT accumulator tiles (x 3 planes on the int8 path) that fit the registers
+    constexpr int kTiles = T::INT8 ? 4 : (DT == FNN_DT_I4CB ? 6 : 8);   // MB * RT accumulator tiles (x 3 planes on the int8 path) that fit the registers
     if (pl.rt == 2) {
         if constexpr (MB * 2 <= kTiles) {
             if (pl.kr == 512) return launch_stream<DT, MB, 2, 512>(p, s);
@@ -561,9 +675,11 @@ hipError_t launch_mb(const StreamPlan &pl, const StreamArgs &p, hipStream_t s)
 template <int DT>
 hipError_t launch_dt(const StreamPlan &pl, const StreamArgs &p, hipStream_t s)
 {
-    switch (pl.mb) {   // (three and four blocks measured slower than the tiled path for every shape: not built)
+    switch (pl.mb) {   // (three and four blocks measured slower than the tiled path for every per-channel type: built for the codebook type only)
     case 1: return launch_mb<DT, 1>(pl, p, s);
     case 2: return launch_mb<DT, 2>(pl, p, s);
+    case 3: if constexpr (DT == FNN_DT_I4CB) return launch_mb<DT, 3>(pl, p, s); else return hipErrorInvalidValue;
+    case 4: if constexpr (DT == FNN_DT_I4CB) return launch_mb<DT, 4>(pl, p, s); else return hipErrorInvalidValue;
     default: return hipErrorInvalidValue;
     }
 }

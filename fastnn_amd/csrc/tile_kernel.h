@@ -49,19 +49,6 @@ struct TileArgs {
     } cv;
 };
 
-// power of two that brings the largest table magnitude into [2^14, 2^15): the f16 hi + lo split of the scaled table
-// then carries ~22 bits of every entry (every thread computes the same value from the 16 cached floats)
-__device__ __forceinline__ int codebook_exp(const float *cb)
-{
-    float mx = 0.0f;
-#pragma unroll
-    for (int i = 0; i < 16; i++) mx = fmaxf(mx, fabsf(cb[i]));
-    if (!(mx > 0.0f) || !(mx < __builtin_huge_valf())) return 0;
-    int ex;
-    (void)frexpf(mx, &ex);
-    return 15 - ex;
-}
-
 // HBM -> LDS without passing registers: lane i of the wave stores its 16 bytes at
 // LDS address m0 + 16*i.  The compiler does not see these loads: waits are placed by hand.
 __device__ __forceinline__ void load_to_lds16(const void *gptr, unsigned lds_wave_base)

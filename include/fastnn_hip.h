@@ -116,9 +116,10 @@ enum {
                                   /* matrix-core GEMM over three or four exact activation digit planes (not in the single-rounding */
                                   /* mode); 0: the f16 tiled GEMM takes them too                                          */
     FNN_OPT_GEMM_INT8_MIN_M = 11, /* smallest M of that path (default 17)                                                 */
-    FNN_OPT_CODEBOOK_EXPANDED = 12, /* codebook weights with blocks of 32 at M >= 5: 0 (default) = by M (decoded inside the */
-                                  /* tiled GEMM where that measured faster), 1 = always through the expanded f16 hi + lo  */
-                                  /* operand (FNN_OPT_CODEBOOK_CACHE), 2 = always decoded inside the tiled GEMM           */
+    FNN_OPT_CODEBOOK_EXPANDED = 12, /* codebook weights with blocks of 32 at M >= 5: 0 (default) = by M (the streaming       */
+                                  /* MatMul up to M = 64, beyond it decoded inside the tiled GEMM where that measured      */
+                                  /* faster), 1 = always the tiled GEMM on the expanded f16 hi + lo operand                */
+                                  /* (FNN_OPT_CODEBOOK_CACHE), 2 = always decoded inside the tiled GEMM                    */
     FNN_OPT_GEMV_INT8_MAX_M = 13, /* largest M the int8 GEMV kernel takes, 1..16 (default 8: beyond that the f16 16-row      */
                                   /* kernel measured faster, the activation chunks being converted one after the other)   */
     FNN_OPT_CONV_EPILOGUE = 14,   /* quantised Conv2d (I8 / I4 weights) on the int8 matrix cores: 0 (default) = by size,      */
@@ -140,7 +141,9 @@ enum {
     FNN_OPT_STREAM_MIN_M = 19,    /* smallest and largest M of the one-launch streaming MatMul (weights straight into the      */
     FNN_OPT_STREAM_MAX_M = 20,    /* matrix-core operand registers, activations converted in the kernel, K split reduced by the  */
                                   /* last workgroup to arrive): defaults 17 and 32, 1..32; MAX_M = 0 switches it off.  By rule   */
-                                  /* it declines shapes with more column tiles x K splits than the chip holds at once            */
+                                  /* it declines shapes with more column tiles x K splits than the chip holds at once.           */
+                                  /* Codebook weights with blocks of 32 (K % 128 == 0): with MAX_M at 32 the kernel takes        */
+                                  /* min(MIN_M, 5) <= M <= 64 (a smaller MAX_M is taken as it is)                                */
     FNN_OPT_STREAM_SHAPE = 21,    /* its launch shape: 0 (default) = by rule, else (splits << 8) | (row tiles per wave << 4) |   */
                                   /* (k-values per round / 256), splits = 0 meaning one round per workgroup                      */
     FNN_OPT_DIGIT_PLANES = 22,    /* int8 matrix-core GEMM (M >= 17, I8 / I4 / U4 weights): activation digit planes, 3 (22 bits     */

@@ -374,6 +374,46 @@ def test_streaming_matmul_takes_the_default_route_and_propagates_non_finite_rows
         ctx.release(h)
 
 
+@pytest.mark.parametrize("m,k,n", [(5, 4096, 520), (16, 1024, 300), (17, 2048, 1100), (32, 4096, 2048), (33, 1536, 260), (48, 2048, 1100),
+                                   (64, 4096, 1024), (64, 128, 4400), (50, 2048, 5000)])
+def test_streaming_matmul_codebook_weights(ctx, orc, m, k, n):
+    """Codebook weights with blocks of 32 at 5 <= M <= 64 (K % 128 == 0) run in the streaming kernel: a matrix-core step
+    is one block (the lane loads are transposed across the k groups), its sum is folded with the block scale -- the
+    reference's association.  Every launch form within the MatMul bound of the oracle (rows with a 200x dynamic range,
+    an all-zero row, ragged N, bias + SiLU), the same bits on every call and on either layout of the words, and another
+    kernel than the tiled path's (which FNN_OPT_CODEBOOK_EXPANDED = 2 selects)."""
+    rng = np.random.default_rng(5400 + m + k)
+    pw = fastnn_amd.quantize_weights(flib.DT_I4CB, _weights(rng, n, k, "laplace"))
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    a[:, ::89] *= 200.0
+    a[m // 2] = 0.0
+    bias = (rng.standard_normal(n) * 0.01).astype(np.float32)
+    h = ctx.register(pw)
+    want = orc.qmatmul(to_oracle(orc, pw), a, order=2, bias=bias, act=3)
+    try:
+        for form in STREAM_FORMS:
+            ctx.set_option(flib.OPT_STREAM_SHAPE, form)
+            got = ctx.qmatmul(h, a, n, bias=bias, act=3)
+            assert_close(got, want, TOL_F32, f"stream codebook {m}x{k}x{n} form {form:#x}")
+            assert np.array_equal(got, ctx.qmatmul(h, a, n, bias=bias, act=3)), f"form {form:#x}: two calls differ"
+            if form in (0, 0x112):
+                ctx.set_option(flib.OPT_GEMV_TILE_MAJOR, 0)
+                assert np.array_equal(got, ctx.qmatmul(h, a, n, bias=bias, act=3)), f"form {form:#x}: the layouts differ"
+                ctx.set_option(flib.OPT_GEMV_TILE_MAJOR, 1)
+        ctx.set_option(flib.OPT_STREAM_SHAPE, 0)
+        by_rule = ctx.qmatmul(h, a, n, bias=bias, act=3)
+        ctx.set_option(flib.OPT_CODEBOOK_EXPANDED, 2)
+        tiled = ctx.qmatmul(h, a, n, bias=bias, act=3)
+        assert_close(tiled, want, TOL_F32)
+        if n * ((k + 511) // 512) <= 320 * 128:      # (the rule declines launches of more than 320 workgroups)
+            assert not np.array_equal(by_rule, tiled)
+    finally:
+        ctx.set_option(flib.OPT_STREAM_SHAPE, 0)
+        ctx.set_option(flib.OPT_GEMV_TILE_MAJOR, 1)
+        ctx.set_option(flib.OPT_CODEBOOK_EXPANDED, 0)
+    ctx.release(h)
+
+
 @pytest.mark.parametrize("dt", [flib.DT_I4, flib.DT_I8, flib.DT_F4])
 @pytest.mark.parametrize("m,k,n", [(20, 4096, 5200), (32, 2048, 10500), (17, 1536, 11008)])
 def test_streaming_matmul_wide_outputs(ctx, orc, dt, m, k, n):
