@@ -59,7 +59,8 @@ def test_static_entry_point_matches_the_allocating_one(orc):
 def test_static_entry_point_reuses_side_tables_but_never_builds_them(orc):
     """A codebook weight at M >= 5 run through its expanded f16 operand (by option) needs the expansion: built by
     fnn_hip_qmatmul on first use, refused with a message by the static entry point before that, used by it afterwards.
-    Decoded inside the tiled GEMM (the default at this M) it needs no side table and works at once."""
+    Decoded inside the kernel (the default at this M: the streaming kernel, on the row-major words as long as their
+    tile-major copy does not exist) it needs no side table and works at once, with the bits the other entry point gives."""
     rng = np.random.default_rng(14)
     n, k, m = 256, 512, 48
     pw = fastnn_amd.quantize_weights(flib.DT_I4CB, (rng.laplace(0, 0.02, (n, k))).astype(np.float32))
