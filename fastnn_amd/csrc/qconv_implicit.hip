@@ -20,8 +20,11 @@ struct ImplicitArgs {
     int g, kk, vec4;
 };
 
-template <int DT, int TN, int PW, int KW, bool RNG>
-__global__ void __launch_bounds__(64 * PW * KW) conv_implicit_kernel(ImplicitArgs p)
+constexpr int TAP_TABLE = 2048;   // taps (K rounded up to whole steps of 32) whose geometry is tabulated once per workgroup
+
+// TAB: K (rounded up to whole steps) fits the tap table
+template <int DT, int TN, int PW, int KW, bool RNG, bool TAB>
+__global__ void __launch_bounds__(64 * PW * KW, TAB ? 4 : 2) conv_implicit_kernel(ImplicitArgs p)   // (TAB: four waves per SIMD, at most 128 registers)
 {
     constexpr int NW = PW * KW;
     constexpr bool W4 = DT == FNN_DT_I4;
@@ -36,6 +39,8 @@ __global__ void __launch_bounds__(64 * PW * KW) conv_implicit_kernel(ImplicitArg
     __shared__ float s_rng[PW][4];
     __shared__ int s_cnt;
     __shared__ int r_img[PW][32];
+    // offset inside the slab and validity bits needed per tap, where K fits
+    __shared__ __attribute__((aligned(16))) uint32_t tap_offs[TAB ? TAP_TABLE : 4], tap_needs[TAB ? TAP_TABLE : 4];
 
     const int tid = threadIdx.x, lane = tid & 63;
     if constexpr (RNG) {
@@ -133,6 +138,21 @@ __global__ void __launch_bounds__(64 * PW * KW) conv_implicit_kernel(ImplicitArg
 
     const int nsteps = (kk + 31) / 32;
     const uint32_t bperm = (uint32_t)(hf * 16) * 4;   // this lane's 16 taps sit in lanes 16*hf .. 16*hf + 15 of the geometry
+    // The geometry of a tap does not depend on the pixel: with K up to TAP_TABLE taps it is worked out once per
+    // workgroup; a lane then reads its 16 taps of a step from the table (two addresses per wave: broadcast reads).
+    // A wave all of whose pixels exist and have every kernel row and column inside the image skips the validity test.
+    if constexpr (TAB) {
+        for (int e0 = tid; e0 < nsteps * 32; e0 += 64 * NW) {
+            const uint32_t e = (uint32_t)e0;
+            const uint32_t ic = p.dv.khw.div(e), rem = e - ic * (uint32_t)(a.kh * a.kw);
+            const uint32_t i = p.dv.kw.div(rem), j = rem - i * (uint32_t)a.kw;
+            tap_offs[e0] = ((ic * (uint32_t)hh + i * (uint32_t)a.dil) * (uint32_t)ww + j * (uint32_t)a.dil) * 4;
+            tap_needs[e0] = (int)e < kk ? ((1u << i) | (0x10000u << j)) : 0x80000000u;
+        }
+        __syncthreads();
+    }
+    const uint32_t all_bits = ((1u << a.kh) - 1u) | (((1u << a.kw) - 1u) << 16);
+    const bool inside = __builtin_amdgcn_ballot_w64(okbits != all_bits) == 0;   // (wave-uniform)
     i32x16 acc[TN];
 #pragma unroll
     for (int tn = 0; tn < TN; tn++)
@@ -150,14 +170,39 @@ __global__ void __launch_bounds__(64 * PW * KW) conv_implicit_kernel(ImplicitArg
         tap_need = (int)e < kk ? ((1u << i) | (0x10000u << j)) : 0x80000000u;
     };
     auto fetch = [&](int s, float(&v)[16], u32x4(&wq)[TN]) {
-        uint32_t tap_off, tap_need;
-        geometry(s, tap_off, tap_need);
+        if constexpr (TAB) {
+            // the lane's 16 taps are 64 contiguous bytes of either table: four 16-byte reads (two addresses per wave)
+            const u32x4 *po = reinterpret_cast<const u32x4 *>(tap_offs + 32 * s + 16 * hf);
+            if (inside && 32 * s + 32 <= kk) {
 #pragma unroll
-        for (int t = 0; t < 16; t++) {
-            const uint32_t soff = (uint32_t)__builtin_amdgcn_ds_bpermute((int)(bperm + 4 * t), (int)tap_off);
-            const uint32_t need = (uint32_t)__builtin_amdgcn_ds_bpermute((int)(bperm + 4 * t), (int)tap_need);
-            const uint32_t vo = (okbits & need) == need ? lane_base + soff : ~0u;
-            v[t] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xbuf, vo, 0, 0));
+                for (int t4 = 0; t4 < 4; t4++) {
+                    const u32x4 o4 = po[t4];
+#pragma unroll
+                    for (int t = 0; t < 4; t++)
+                        v[t4 * 4 + t] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xbuf, lane_base + o4[t], 0, 0));
+                }
+            } else {
+                const u32x4 *pn = reinterpret_cast<const u32x4 *>(tap_needs + 32 * s + 16 * hf);
+#pragma unroll
+                for (int t4 = 0; t4 < 4; t4++) {
+                    const u32x4 o4 = po[t4], n4 = pn[t4];
+#pragma unroll
+                    for (int t = 0; t < 4; t++) {
+                        const uint32_t vo = (okbits & n4[t]) == n4[t] ? lane_base + o4[t] : ~0u;
+                        v[t4 * 4 + t] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xbuf, vo, 0, 0));
+                    }
+                }
+            }
+        } else {
+            uint32_t tap_off, tap_need;
+            geometry(s, tap_off, tap_need);
+#pragma unroll
+            for (int t = 0; t < 16; t++) {
+                const uint32_t soff = (uint32_t)__builtin_amdgcn_ds_bpermute((int)(bperm + 4 * t), (int)tap_off);
+                const uint32_t need = (uint32_t)__builtin_amdgcn_ds_bpermute((int)(bperm + 4 * t), (int)tap_need);
+                const uint32_t vo = (okbits & need) == need ? lane_base + soff : ~0u;
+                v[t] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xbuf, vo, 0, 0));
+            }
         }
 #pragma unroll
         for (int tn = 0; tn < TN; tn++) {
@@ -424,8 +469,14 @@ hipError_t launch_implicit(const ImplicitArgs &p, int64_t rows, int64_t ocg, hip
     constexpr size_t lds = (size_t)PW * (KW - 1) * (TN * 16 + 1) * 64 * 4;
     static_assert(lds <= 48 * 1024, "the K slices meet in the default LDS allowance");
     const dim3 grid((unsigned)((rows + 32 * PW - 1) / (32 * PW)), (unsigned)((ocg + TN * 32 - 1) / (TN * 32)));
-    if (p.a.range_out) hipLaunchKernelGGL((conv_implicit_kernel<DT, TN, PW, KW, true>), grid, dim3(64 * PW * KW), lds, s, p);
-    else hipLaunchKernelGGL((conv_implicit_kernel<DT, TN, PW, KW, false>), grid, dim3(64 * PW * KW), lds, s, p);
+    const bool tab = (p.kk + 31) / 32 * 32 <= TAP_TABLE;
+    if (p.a.range_out) {
+        if (tab) hipLaunchKernelGGL((conv_implicit_kernel<DT, TN, PW, KW, true, true>), grid, dim3(64 * PW * KW), lds, s, p);
+        else hipLaunchKernelGGL((conv_implicit_kernel<DT, TN, PW, KW, true, false>), grid, dim3(64 * PW * KW), lds, s, p);
+    } else {
+        if (tab) hipLaunchKernelGGL((conv_implicit_kernel<DT, TN, PW, KW, false, true>), grid, dim3(64 * PW * KW), lds, s, p);
+        else hipLaunchKernelGGL((conv_implicit_kernel<DT, TN, PW, KW, false, false>), grid, dim3(64 * PW * KW), lds, s, p);
+    }
     return hipGetLastError();
 }
 

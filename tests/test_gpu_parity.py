@@ -763,6 +763,8 @@ IMPLICIT_CONVS = CONVS + [
     dict(b=1, c=20, h=30, w=33, oc=40, kh=3, kw=3, stride=2, pad=1, dil=1, groups=1),    # two k slices, odd pixel count
     dict(b=3, c=64, h=7, w=9, oc=70, kh=3, kw=3, stride=1, pad=1, dil=1, groups=1),      # four k slices, blocks over three images
     dict(b=2, c=6, h=50, w=46, oc=12, kh=5, kw=5, stride=1, pad=2, dil=1, groups=2),     # groups, K past a step's end
+    dict(b=1, c=230, h=12, w=14, oc=20, kh=3, kw=3, stride=1, pad=1, dil=1, groups=1),   # K = 2070: more taps than the geometry table holds
+    dict(b=2, c=16, h=36, w=34, oc=16, kh=3, kw=3, stride=1, pad=0, dil=2, groups=1),    # no padding: every tap of every pixel inside the image
 ]
 
 
