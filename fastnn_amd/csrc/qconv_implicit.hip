@@ -281,11 +281,15 @@ __global__ void __launch_bounds__(64 * PW * KW, TAB ? 4 : 2) conv_implicit_kerne
 
     // this lane's channel constants: requested when the K loop is done (not earlier: they would take registers the
     // loop's loads in flight need), so that they travel while the K slices meet
+    // Up to 16 channels in a 32-channel column block: the lanes of channels 16 .. 31 would sit out the epilogue, so
+    // they take over half of the pixels of the lane 16 below (`share`: lane lr works on channel lr & 15).
+    const bool share = TN == 1 && ocg <= 16;   // (uniform)
+    const int lch = share ? (lr & 15) : lr;
     float sw[TN], zw[TN], bi[TN];
     int wq_[TN];
 #pragma unroll
     for (int tn = 0; tn < TN; tn++) {
-        const int64_t n = n0 + tn * 32 + lr;
+        const int64_t n = n0 + tn * 32 + lch;
         const bool ok = kw == 0 && n < ocg;
         const int64_t ch = (int64_t)g * ocg + (ok ? n : 0);
         sw[tn] = ok ? a.scales[ch] : 0.0f;
@@ -342,8 +346,19 @@ __global__ void __launch_bounds__(64 * PW * KW, TAB ? 4 : 2) conv_implicit_kerne
         const bool has_bias = a.bias != nullptr;
         float *y = a.y + (int64_t)g * ocg * np;
         int32_t *acc_out = a.acc_out ? a.acc_out + (int64_t)g * ocg * np : nullptr;
+        if constexpr (TN == 1) {
+            if (share) {
+                // rows of 16 lanes: (k half 0, channels 0-15), (0, 16-31), (1, 0-15), (1, 16-31).  Registers 8 .. 15 (pixel
+                // groups 2 and 3) of the even rows move into registers 0 .. 7 of the odd rows above them
 #pragma unroll
-        for (int ig = 0; ig < 4; ig++) {
+                for (int i = 0; i < 8; i++)
+                    acc[0][i] = (int)__builtin_amdgcn_permlane16_swap((uint32_t)acc[0][i], (uint32_t)acc[0][i + 8], false, false)[0];
+            }
+        }
+#pragma unroll
+        for (int igl = 0; igl < 4; igl++) {
+            if (share && igl >= 2) break;
+            const int ig = share ? igl + 2 * (lr >> 4) : igl;   // pixel group of registers 4 igl .. 4 igl + 3
             const int rr0 = ig * 8 + hf * 4;
             const int64_t r0 = r_first + pw * 32 + rr0;
             if (r0 >= rows) continue;
@@ -356,7 +371,7 @@ __global__ void __launch_bounds__(64 * PW * KW, TAB ? 4 : 2) conv_implicit_kerne
             }
 #pragma unroll
             for (int tn = 0; tn < TN; tn++) {
-                const int64_t n = n0 + tn * 32 + lr;
+                const int64_t n = n0 + tn * 32 + lch;
                 if (n >= ocg) continue;
                 float v[4];
                 int av[4], bq[4];
@@ -365,7 +380,7 @@ __global__ void __launch_bounds__(64 * PW * KW, TAB ? 4 : 2) conv_implicit_kerne
                 for (int j = 1; j < 4; j++) bq[j] = (p.vec4 || !has_bias) ? bq[0] : conv_bias_q(bi[tn], rsa[j], sw[tn]);
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
-                    int ai = acc[tn][ig * 4 + j];
+                    int ai = acc[tn][igl * 4 + j];
                     if (W4) ai >>= 4;
                     v[j] = conv_dequant(ai, rsa[j], rza[j], rs[j], sw[tn], zw[tn], sw[tn] * (float)wq_[tn], bq[j], kk, a.act, &av[j]);
                 }
@@ -386,7 +401,7 @@ __global__ void __launch_bounds__(64 * PW * KW, TAB ? 4 : 2) conv_implicit_kerne
                     const int64_t o = r_off[pw][rr0] + n * np;
                     if constexpr (TN > 1) {   // stored below, channel by channel
 #pragma unroll
-                        for (int j = 0; j < 4; j++) acc[tn][ig * 4 + j] = __float_as_int(v[j]);
+                        for (int j = 0; j < 4; j++) acc[tn][igl * 4 + j] = __float_as_int(v[j]);
                     } else {
                         *reinterpret_cast<float4 *>(y + o) = make_float4(v[0], v[1], v[2], v[3]);
                     }
