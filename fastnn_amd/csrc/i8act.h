@@ -55,8 +55,9 @@ __device__ __forceinline__ int conv_bias_q(float bias, float sa, float sw)
     const float x = bias / (sa * sw);
     return (int)(x + __builtin_copysignf(0.49999997f, x));
 }
-__device__ __forceinline__ float conv_dequant(int acc_in, float sa, float za, float rsum, float sw, float zw, float wt,
-                                              int bias_q, int kk, int act, int *acc_out)
+// (the affine part alone; the activation follows, conv_act / conv_act4)
+__device__ __forceinline__ float conv_affine(int acc_in, float sa, float za, float rsum, float sw, float zw, float wt,
+                                             int bias_q, int kk, int *acc_out)
 {
     const float sab = sa * sw;
     const int accv = acc_in + bias_q;
@@ -65,11 +66,34 @@ __device__ __forceinline__ float conv_dequant(int acc_in, float sa, float za, fl
     val = val + zw * rsum;
     val = val + za * wt;
     val = val + zp_prod * (float)kk;
+    *acc_out = accv;
+    return val;
+}
+__device__ __forceinline__ float conv_act(float val, int act)
+{
     if (act == FNN_ACT_RELU) val = fmaxf(val, 0.0f);
     else if (act == FNN_ACT_SILU) val = fnn_sigmoid_times(val, val);
     else if (act == FNN_ACT_GELU) val = fnn_sigmoid_times(val, 2.0f * (val * 0.7978846f * (1.0f + 0.044715f * val * val)));   // = 0.5 v (1 + tanh(.))
-    *acc_out = accv;
     return val;
+}
+// the same on four outputs with one test of the (uniform) activation code
+__device__ __forceinline__ void conv_act4(float (&v)[4], int act)
+{
+    if (act == FNN_ACT_RELU) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) v[j] = fmaxf(v[j], 0.0f);
+    } else if (act == FNN_ACT_SILU) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) v[j] = fnn_sigmoid_times(v[j], v[j]);
+    } else if (act == FNN_ACT_GELU) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) v[j] = fnn_sigmoid_times(v[j], 2.0f * (v[j] * 0.7978846f * (1.0f + 0.044715f * v[j] * v[j])));
+    }
+}
+__device__ __forceinline__ float conv_dequant(int acc_in, float sa, float za, float rsum, float sw, float zw, float wt,
+                                              int bias_q, int kk, int act, int *acc_out)
+{
+    return conv_act(conv_affine(acc_in, sa, za, rsum, sw, zw, wt, bias_q, kk, acc_out), act);
 }
 
 // min / max over nparts (min, max) pairs at part (16-byte aligned) by the nthr threads of a workgroup, folded into

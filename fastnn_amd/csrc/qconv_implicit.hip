@@ -382,8 +382,9 @@ __global__ void __launch_bounds__(64 * PW * KW, TAB ? 4 : 2) conv_implicit_kerne
                 for (int j = 0; j < 4; j++) {
                     int ai = acc[tn][igl * 4 + j];
                     if (W4) ai >>= 4;
-                    v[j] = conv_dequant(ai, rsa[j], rza[j], rs[j], sw[tn], zw[tn], sw[tn] * (float)wq_[tn], bq[j], kk, a.act, &av[j]);
+                    v[j] = conv_affine(ai, rsa[j], rza[j], rs[j], sw[tn], zw[tn], sw[tn] * (float)wq_[tn], bq[j], kk, &av[j]);
                 }
+                conv_act4(v, a.act);
                 if constexpr (RNG) {
                     if (rng_plain) {   // (workgroup-uniform) every pixel of the block exists and lies in one image
                         mn0 = fminf(fminf(mn0, fminf(v[0], v[1])), fminf(v[2], v[3]));

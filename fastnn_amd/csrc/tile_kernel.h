@@ -689,8 +689,9 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
                         const float bits = acc[tm][tn][ig * 4 + j];
                         int a = __float_as_int(bits);
                         if constexpr (DT == FNN_DT_I4) a >>= 4;
-                        v[j] = conv_dequant(a, sa[j], za[j], rs[j], sw[tn], zw[tn], wt[tn], bq[j], p.cv.kk, p.act, &av[j]);
+                        v[j] = conv_affine(a, sa[j], za[j], rs[j], sw[tn], zw[tn], wt[tn], bq[j], p.cv.kk, &av[j]);
                     }
+                    conv_act4(v, p.act);
                     if constexpr (CRNG) {
                         if (rng_plain) {   // (workgroup-uniform) every row of the tile exists and lies in one image
                             mn0 = fminf(fminf(mn0, fminf(v[0], v[1])), fminf(v[2], v[3]));
