@@ -547,8 +547,10 @@ bool fnn_implicit_conv_takes(const fnn_hip_weight *w, const QConvArgs &p, int op
     if (option != 1) {
         // one pass over the pixels per 32 * tn channels: ahead of the pair while the channels fit one or two MFMA
         // columns and the launch has pixels enough to fill the chip
+        // (YOLOv8n-shaped layers, us, implicit / pair: 33-64 channels at 25 600 pixels 18.6 / 20.7, 23.6 / 25.9; at 6400
+        // pixels 14.7 / 12.6, 13.7 / 10.6; 128 channels and more: 38.1 / 32.2, 46.1 / 25.1, 16.4 / 14.7)
         if (ocg > 64) return false;
-        if (rows < (tn == 1 ? 2048 : 65536)) return false;
+        if (rows < (tn == 1 ? 2048 : 12800)) return false;
     }
     if (wg_rows) *wg_rows = wr;
     if (wgs) *wgs = ((rows + wr - 1) / wr) * ((ocg + tn * 32 - 1) / (tn * 32));
