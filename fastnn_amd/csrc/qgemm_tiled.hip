@@ -490,6 +490,10 @@ TileLayout tile_layout(fnn_hip_ctx *ctx, int64_t M, int64_t N, int64_t K, int fl
         const int64_t small_tiles = ((meff + 31) / 32) * ((N + 127) / 128);
         if (small_tiles >= 192 && small_tiles <= 256) cfg = 2;
     }
+    // the dense (expanded codebook) operand from 1024 effective rows on: 256 x 128 tiles on eight waves (twice the waves
+    // that fetch a stage's bytes, and half the weight bytes per row tile).  4096 x 4096, us, 128 x 128 / 256 x 128 tiles:
+    // M = 640 225 / 137, 768 223 / 140, 1024 225 / 155, 2048 436 / 289, 4096 871 / 562; up to M = 512 no gain (91.4 / 91.9)
+    if (dense && meff > 1024) cfg = 3;
     const int64_t opt_cfg = fnn_ctx_option(ctx, FNN_OPT_TILE_SHAPE);
     // 3 (by option only): 256x128 with 8 waves of 64x64, two waves per SIMD.  Measured on FP8 4096 x 4096 and 2048 -> 8192
     // at M = 128 ... 1024: 0-30 % slower than the automatic choice, except where it turns the tile count into one whole
@@ -500,7 +504,7 @@ TileLayout tile_layout(fnn_hip_ctx *ctx, int64_t M, int64_t N, int64_t K, int fl
     // wave loading) measured 10-40 % slower than the 4-wave tiles at every K split; these calls are bound by their
     // three dependent launches (activation preparation, tiles, split-K reduction), not by delivery.
     if (opt_cfg >= 0 && opt_cfg <= 3) cfg = (int)opt_cfg;
-    if (cfg == 3 && (DecH<DT>::WPS < 2 || dense)) cfg = 0;  // (8-bit weights only: a stage of 4-bit rows has too few 16-byte chunks for 8 waves)
+    if (cfg == 3 && DecH<DT>::WPS < 2) cfg = 0;  // (8-bit weights only: a stage of 4-bit rows has too few 16-byte chunks for 8 waves)
     L.precise = precise; L.cfg = cfg;
     L.bm = cfg == 3 ? 256 : (cfg == 0 ? 128 : (cfg == 1 ? 64 : 32));
     L.mtiles = (int)((meff + L.bm - 1) / L.bm);
@@ -563,6 +567,12 @@ int run_tiled(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, const QM
     // the dense operand (128 x 128 tiles, one workgroup per CU): as many splits as fill one round, no more (measured on
     // 4096 x 4096: 96 tiles 58.0 us with 2 splits against 71.6 with the model's choice, 192 tiles 82.1 with none against 110)
     if (dense && cfg == 0) splits = base >= 256 ? 1 : 256 / base;
+    // ... and on its 256 x 128 tiles: two splits only where they save a round of workgroups (M = 1536: 245 against 265 us;
+    // M = 1024, 2048, 4096: one split 155 / 289 / 562 against 169 / 316 / 640)
+    if (dense && cfg == 3) {
+        const double r1 = (double)((base + 255) / 256), r2 = (double)((2 * base + 255) / 256) / 2.0 + 0.1;
+        splits = r2 < r1 ? 2 : 1;
+    }
     if (env_split > 0) splits = env_split;
     if (splits > iters / 4) splits = iters / 4 > 0 ? iters / 4 : 1;
     int ips = (iters + splits - 1) / splits;
@@ -828,12 +838,13 @@ int fnn_tiled_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, 
         // of the 32 of the expanded f16 hi + lo operand, and no expansion is kept with the weight); other block
         // sizes, or by option, the expanded operand.  Measured on 4096 x 4096 (us, in-kernel / expanded): M = 5 ... 16
         // 19-20 / 23-26, M = 32 23.3 / 24.5, M = 64 30.5 / 31.5, M = 128 41.2 / 42.4, M = 256 65.8 / 58.4, M = 1024
-        // 191 / 207; single rounding: M <= 16 20 / 24-27, M = 64 30.1 / 27.2, M = 256 48.3 / 46.2, M = 1024 119 / 99
+        // 191 / 207 (155 on the 256 x 128 tiles the expanded operand takes from M = 513 on; M = 640: 142 / 137, M = 2048:
+        // 372 / 289); single rounding: M <= 16 20 / 24-27, M = 64 30.1 / 27.2, M = 256 48.3 / 46.2, M = 1024 119 / 99
         // (the per-block fold of the accumulator, 2 x 64 FMAs per wave and stage, and the look-ups make the loop
         // vector-ALU bound; the expanded operand's loop is the plain f16 one).
         const int64_t opt_exp = fnn_ctx_option(ctx, FNN_OPT_CODEBOOK_EXPANDED);
         const bool precise = !(flags & FNN_FLAG_ACT_F16_SINGLE);
-        const bool in_kernel = opt_exp == 0 ? (precise ? (q.m < 192 || q.m >= 1024) : q.m <= 16) : opt_exp == 2;
+        const bool in_kernel = opt_exp == 0 ? (precise ? q.m < 192 : q.m <= 16) : opt_exp == 2;
         if (q.qblock == 32 && in_kernel) {
             QMatmulArgs qa = q;
             int rc;
