@@ -139,7 +139,7 @@ const OptionSpec kOptions[FNN_OPT_COUNT] = {
     {8, 1, 16},       // FNN_OPT_GEMV_INT8_MAX_M
     {0, 0, 3},        // FNN_OPT_CONV_EPILOGUE
     {1, 0, 1},        // FNN_OPT_CONV_RANGES
-    {0, 0, 2},        // FNN_OPT_CONV_IMPLICIT
+    {0, 0, 3},        // FNN_OPT_CONV_IMPLICIT
     {1, 0, 1},        // FNN_OPT_FUSE_RESIDUAL
     {1, 0, 1},        // FNN_OPT_FUSE_PREP
     {17, 1, 32},      // FNN_OPT_STREAM_MIN_M

@@ -131,7 +131,8 @@ enum {
                                   /* every convolution scans                                                               */
     FNN_OPT_CONV_IMPLICIT = 16,   /* quantised Conv2d (I8 / I4 weights, f32 input): 1 = one implicit-GEMM kernel (im2col taps    */
                                   /* fetched and quantised in the GEMM's operand registers, no int8 operand in memory), 2 = the */
-                                  /* operand kernel + GEMM pair, 0 (default) = by shape                                         */
+                                  /* operand kernel + GEMM pair, 3 = the fused kernel (a workgroup quantises 32 pixels once     */
+                                  /* into LDS and runs all output channels against them; K up to 1280), 0 (default) = by shape  */
     FNN_OPT_FUSE_RESIDUAL = 17,   /* plans: 1 (default) = a MatMul whose output the next instruction adds to another tensor       */
                                   /* stores that sum from its own last kernel where it can (the Add instruction is then skipped; */
                                   /* same f32 addition, identical results), 0 = every Add runs as its own launch                 */

@@ -765,17 +765,21 @@ IMPLICIT_CONVS = CONVS + [
     dict(b=2, c=6, h=50, w=46, oc=12, kh=5, kw=5, stride=1, pad=2, dil=1, groups=2),     # groups, K past a step's end
     dict(b=1, c=230, h=12, w=14, oc=20, kh=3, kw=3, stride=1, pad=1, dil=1, groups=1),   # K = 2070: more taps than the geometry table holds
     dict(b=2, c=16, h=36, w=34, oc=16, kh=3, kw=3, stride=1, pad=0, dil=2, groups=1),    # no padding: every tap of every pixel inside the image
+    dict(b=2, c=96, h=13, w=11, oc=300, kh=3, kw=3, stride=1, pad=1, dil=1, groups=1),   # many channels: ten blocks of 32 (fused: two per wave), K = 864
+    dict(b=3, c=128, h=10, w=10, oc=136, kh=1, kw=1, stride=1, pad=0, dil=1, groups=1),  # 1x1, a ragged last channel block, blocks over two images
 ]
 
 
 @pytest.mark.parametrize("cfg", IMPLICIT_CONVS)
 @pytest.mark.parametrize("act", [0, 3])
 @pytest.mark.parametrize("wdt", [flib.DT_I8, flib.DT_I4])
-@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("mode", [0, 1, 3])
 def test_qconv2d_implicit_gemm(ctx, orc, cfg, act, wdt, mode):
-    """The kernel that fetches and quantises the im2col taps in the MFMA operand registers (no int8 operand in
-    memory): the same accumulators as conv2d_packed_i8x4 / conv2d_packed_i4x8, bit for bit.  mode 1: wherever it can
-    run; mode 0: where the library picks it by shape (the larger of these cases)."""
+    """The kernels that fetch and quantise the im2col taps themselves (no int8 operand in memory): the same
+    accumulators as conv2d_packed_i8x4 / conv2d_packed_i4x8, bit for bit.  mode 1: the implicit kernel (taps straight
+    into the MFMA operand registers, a pass over the pixels per channel block) wherever it can run; mode 3: the fused
+    kernel (a workgroup quantises 32 pixels once into LDS and runs all channels against them) wherever it can run;
+    mode 0: what the library picks by shape."""
     ctx.set_option(flib.OPT_CONV_IMPLICIT, mode)
     try:
         rng = np.random.default_rng(6100 + cfg["c"])
