@@ -6,6 +6,8 @@
 // A operand of v_mfma_i32_32x32x32_i8; the weight rows come as 16-byte loads in operand order.  KW waves of a
 // workgroup split the K range of the same pixels and add their exact i32 accumulators through LDS; the first of them
 // applies the reference's float formula (conv_dequant) and stores NCHW, four pixels of a channel per store.
+// Layers with many output channels run as conv_fused_kernel (below): the pixels quantised once into LDS, the waves
+// of a workgroup sharing the channel blocks.
 #include "mfma.h"
 #include "dech.h"
 #include "range_io.h"
