@@ -282,7 +282,7 @@ def test_yolo_graph_node_by_node_against_oracle(orc, batch, size):
         ex.close()
 
 
-@pytest.mark.parametrize("implicit", [0, 1, 2])
+@pytest.mark.parametrize("implicit", [0, 1, 2, 3])
 @pytest.mark.parametrize("batch,size", [(3, 160), (1, 224)])
 def test_conv_activation_ranges_from_the_producing_instruction(orc, batch, size, implicit):
     """A quantised Conv2d in a plan takes min / max of its input from partial pairs the instruction before it left
@@ -291,7 +291,8 @@ def test_conv_activation_ranges_from_the_producing_instruction(orc, batch, size,
     with every convolution scanning its own input; the sizes make output tiles straddle images (20 x 20 = 400 rows
     per image against 64-row tiles) and fall below one tile (5 x 5), where the producer leaves nothing and the
     consumer scans.  implicit: which convolution kernel leaves and takes the pairs (0 = chosen by shape, 1 = the
-    implicit-GEMM kernel wherever it runs, 2 = the operand kernel + GEMM pair everywhere)."""
+    implicit-GEMM kernel wherever it runs, 2 = the operand kernel + GEMM pair everywhere, 3 = the fused kernel wherever it
+    runs)."""
     rng = np.random.default_rng(11)
     nodes, params, shape, outs = bench.yolo_graph(batch, rng, size=size)
     x = rng.uniform(0, 1, shape).astype(np.float32)
@@ -445,7 +446,7 @@ def test_random_conv_graphs_equal_under_every_range_and_kernel_choice(seed):
         shape = (b, c0, h, w)
         x = rng.uniform(-1, 1, shape).astype(np.float32)
         res = {}
-        for ranges, implicit, fuse in [(0, 0, 0), (1, 0, 1), (1, 1, 1), (1, 2, 1), (0, 1, 1), (1, 0, 0), (0, 2, 1)]:
+        for ranges, implicit, fuse in [(0, 0, 0), (1, 0, 1), (1, 1, 1), (1, 2, 1), (0, 1, 1), (1, 0, 0), (0, 2, 1), (1, 3, 1), (0, 3, 0)]:
             ex = AotExecutor(nodes, params, ["x"], [cur], {"x": shape}, quantize=8)
             try:
                 ex.set_option(flib.OPT_CONV_RANGES, ranges)
