@@ -54,7 +54,9 @@ __global__ void __launch_bounds__(64 * PW * KW, TAB ? 4 : 2) conv_implicit_kerne
     const int g = p.g, kk = p.kk;
     const uint32_t np = (uint32_t)(a.ho * a.wo), wo = (uint32_t)a.wo;
     const int64_t rows = a.b * (int64_t)np;
-    const int cg = (int)a.c / a.groups, ocg = (int)(a.oc / a.groups);
+    // (quotients of launch constants: kept in scalar registers, so that what is built from them -- the buffer
+    // descriptors above all -- needs no per-lane check)
+    const int cg = __builtin_amdgcn_readfirstlane((int)a.c / a.groups), ocg = __builtin_amdgcn_readfirstlane((int)(a.oc / a.groups));
     const int64_t r_first = (int64_t)blockIdx.x * (32 * PW);
     const int64_t n0 = (int64_t)blockIdx.y * (TN * 32);
     const uint32_t nn0 = p.dv.np.div((uint32_t)(r_first < rows ? r_first : 0));   // image of the workgroup's first row
@@ -516,7 +518,9 @@ __global__ void __launch_bounds__(256) conv_fused_kernel(ImplicitArgs p)
     const int g = p.g, kk = p.kk;
     const uint32_t np = (uint32_t)(a.ho * a.wo), wo = (uint32_t)a.wo;
     const int64_t rows = a.b * (int64_t)np;
-    const int cg = (int)a.c / a.groups, ocg = (int)(a.oc / a.groups);
+    // (quotients of launch constants: kept in scalar registers, so that what is built from them -- the buffer
+    // descriptors above all -- needs no per-lane check)
+    const int cg = __builtin_amdgcn_readfirstlane((int)a.c / a.groups), ocg = __builtin_amdgcn_readfirstlane((int)(a.oc / a.groups));
     const int64_t r_first = (int64_t)blockIdx.x * 32;
     const uint32_t nn0 = p.dv.np.div((uint32_t)(r_first < rows ? r_first : 0));   // image of the workgroup's first row
 
