@@ -767,6 +767,7 @@ IMPLICIT_CONVS = CONVS + [
     dict(b=2, c=16, h=36, w=34, oc=16, kh=3, kw=3, stride=1, pad=0, dil=2, groups=1),    # no padding: every tap of every pixel inside the image
     dict(b=2, c=96, h=13, w=11, oc=300, kh=3, kw=3, stride=1, pad=1, dil=1, groups=1),   # many channels: ten blocks of 32 (fused: two per wave), K = 864
     dict(b=3, c=128, h=10, w=10, oc=136, kh=1, kw=1, stride=1, pad=0, dil=1, groups=1),  # 1x1, a ragged last channel block, blocks over two images
+    dict(b=1, c=140, h=9, w=9, oc=72, kh=3, kw=3, stride=1, pad=1, dil=1, groups=1),     # K = 1260: the most steps the fused kernel holds in LDS
 ]
 
 
