@@ -977,7 +977,7 @@ bool fnn_implicit_conv_takes(const fnn_hip_weight *w, const QConvArgs &p, int op
     const int64_t rows = p.b * p.ho * p.wo, ocg = p.oc / p.groups;
     int tn, kw, wr;
     implicit_shape(p, &tn, &kw, &wr);
-    if (form == 2) { wr = 32; tn = 1 << 20; }   // (one workgroup per 32 pixels, whatever the channels)
+    if (form == 2) wr = 32;   // (one workgroup per 32 pixels, whatever the channels)
     if (wg_rows) *wg_rows = wr;
     if (wgs) *wgs = ((rows + wr - 1) / wr) * (form == 2 ? 1 : (ocg + tn * 32 - 1) / (tn * 32));
     return true;
