@@ -106,7 +106,7 @@ class ExecutablePlan:
 
     @property
     def residuals_fused(self) -> int:
-        """add_f32 instructions whose sum the MatMul before them stored (no launch of their own)."""
+        """add_f32 instructions whose sum the MatMul or Conv2d before them stored (no launch of their own)."""
         return int(self.lib.fnn_plan_residuals_fused(self.handle))
 
     @property

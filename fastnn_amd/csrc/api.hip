@@ -881,6 +881,11 @@ int fnn_hip_qconv2d(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *x, i
             if (rio.out_table) rio.out_failed = 1;
             HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qconv2d_i8(p, ctx->stream, 0, nullptr));
         } else {
+            // an Add of the plan rides along (range_io.h): the kernels whose epilogue holds y in registers store the sum
+            // as well and say so; the ranges they leave are then those of the sum
+            if (const FnnResidualIo &res = ctx->residual; dev && res.residual && res.sum_out && res.of_out == dy && res.elems == (uint64_t)(b * oc * ho * wo)) {
+                p.residual = res.residual; p.sum_out = res.sum_out;
+            }
             // the caller asks for partial ranges of y (range_io.h): the epilogue inside the GEMM kernel leaves them
             const bool want_out = rio.out_table && dev && rio.out_parts == 0;
             if (want_out && rio.out_images == (uint64_t)b && rio.out_image_elems == (uint64_t)(oc * ho * wo)) {

@@ -60,6 +60,7 @@ struct Instr {
     bool clobbered = false;  // WriteConst only: another instruction of the plan writes into dst
     int add_operand = -1;    // MatMul whose output the next instruction (an add_f32) adds to a tensor: index (0 / 1) of that
                              // tensor among the Add's inputs, found by analyse(); -1: nothing to fuse
+    bool add_is_conv = false;   // ... the same for a quantised Conv2d (the sum's value ranges then come from its kernel)
 };
 
 bool overlaps(const fnn_slice &a, const fnn_slice &b)
@@ -779,7 +780,12 @@ int run_call_with_ranges(fnn_backend *b, fnn_plan *p, size_t idx)
     *rio = FnnRangeIo{};
     int64_t enabled = 1;
     fnn_hip_get_option(b->ctx, FNN_OPT_CONV_RANGES, &enabled);
-    if (!enabled) return run_call(b, in);
+    FnnResidualIo *res = fnn_ctx_residual_io(b->ctx);
+    const bool for_sum = in.add_is_conv && res->residual != nullptr;
+    if (!enabled) {
+        if (for_sum) drop_ranges_overlapping(b, p->instrs[idx + 1].dst);
+        return run_call(b, in);
+    }
     // consumer: a convolution whose input slice is described by a live table
     ConvInput ci;
     if (ranged_conv_input(in, &ci)) {
@@ -790,14 +796,19 @@ int run_call_with_ranges(fnn_backend *b, fnn_plan *p, size_t idx)
                 break;
             }
     }
-    // producer: some later convolution reads exactly what this instruction writes, before anything overwrites it
+    // producer: some later convolution reads exactly what this instruction writes, before anything overwrites it.  A
+    // convolution that carries the Add behind it asks on the Add's behalf: a kernel that stores the sum leaves the
+    // sum's ranges (one that does not leaves those of its own output, which are then of no use: the Add runs and
+    // asks again)
     fnn_slice covered{0, 0};
-    if (leaves_ranges(in)) request_ranges(b, p, idx, &covered);
+    if (for_sum) request_ranges(b, p, idx + 1, &covered);
+    else if (leaves_ranges(in)) request_ranges(b, p, idx, &covered);
     drop_ranges_overlapping(b, in.dst);
     if (in.has_secondary) drop_ranges_overlapping(b, in.secondary);
+    if (for_sum) drop_ranges_overlapping(b, p->instrs[idx + 1].dst);
     const int st = run_call(b, in);
     if (st == FNN_OK && rio->in_used) p->ranges_used++;
-    if (st == FNN_OK) note_ranges(b, covered);
+    if (st == FNN_OK && (!for_sum || res->used)) note_ranges(b, covered);
     *rio = FnnRangeIo{};
     return st;
 }
@@ -829,18 +840,24 @@ void analyse(fnn_plan *p)
             p->writes.push_back(r);
         }
     }
-    // MatMul followed by an Add of its whole output and another tensor of the same size: candidates for one call.
-    // Not when a quantised Conv2d reads the sum (the Add then leaves that convolution's activation ranges) and not
-    // when the sum overlaps the MatMul's own output or partly overlaps the other operand.
+    // MatMul (or quantised Conv2d with integer weights) followed by an Add of its whole output and another tensor of
+    // the same size: candidates for one call.  A MatMul not when a quantised Conv2d reads the sum (the Add then leaves
+    // that convolution's activation ranges; a Conv2d that stores the sum leaves them itself); neither when the sum
+    // overlaps the call's own output or any of its inputs (workgroups still read them while others store sums), or
+    // partly overlaps the other operand.
     for (size_t i = 0; i + 1 < p->instrs.size(); i++) {
         Instr &mm = p->instrs[i];
         const Instr &ad = p->instrs[i + 1];
         mm.add_operand = -1;
+        mm.add_is_conv = false;
         if (mm.kind != K_CALL || ad.kind != K_CALL || ad.kernel != "add_f32" || ad.inputs.size() != 2) continue;
         const KernelName kn = split_activation(mm.kernel);
         uint64_t mkn[3];
-        if (matmul_dtype(kn.base) < 0 || !static_mkn(mm, mkn)) continue;
-        const uint64_t bytes = mkn[0] * mkn[2] * 4;
+        uint64_t bytes = 0;
+        const bool is_conv = (kn.base == "conv2d_i8" || kn.base == "conv2d_i4") && mm.meta.present && mm.meta.codebook.empty();
+        if (is_conv) bytes = mm.dst.size;
+        else if (matmul_dtype(kn.base) >= 0 && static_mkn(mm, mkn)) bytes = mkn[0] * mkn[2] * 4;
+        else continue;
         if (bytes == 0 || mm.dst.size != bytes || ad.dst.size != bytes) continue;
         int other = -1;
         for (int k = 0; k < 2; k++)
@@ -850,12 +867,15 @@ void analyse(fnn_plan *p)
         if (overlaps(res, mm.dst) || overlaps(ad.dst, mm.dst)) continue;
         if (overlaps(ad.dst, res) && ad.dst.offset != res.offset) continue;
         if (ad.dst.offset % 4 || res.offset % 4) continue;
+        bool reads_sum_slot = false;
+        for (const auto &mi : mm.inputs) reads_sum_slot = reads_sum_slot || overlaps(mi, ad.dst);
+        if (reads_sum_slot) continue;
         bool feeds_conv = false;
-        for (size_t j = i + 2; j < p->instrs.size() && !feeds_conv; j++) {
+        for (size_t j = i + 2; j < p->instrs.size() && !feeds_conv && !is_conv; j++) {
             ConvInput cj;
             feeds_conv = ranged_conv_input(p->instrs[j], &cj) && overlaps(p->instrs[j].inputs[0], ad.dst);
         }
-        if (!feeds_conv) mm.add_operand = other;
+        if (!feeds_conv) { mm.add_operand = other; mm.add_is_conv = is_conv; }
     }
     p->analysed = true;
 }
@@ -878,9 +898,10 @@ void note_dispatched(fnn_backend *b, fnn_plan *p)
 int run_instr(fnn_backend *b, fnn_plan *p, size_t idx, bool consts_resident)
 {
     Instr &in = p->instrs[idx];
-    if (idx == p->add_done) {   // the MatMul before this Add has stored the sum already
+    if (idx == p->add_done) {   // the call before this Add has stored the sum already
         p->add_done = (size_t)-1;
-        drop_ranges_overlapping(b, in.dst);
+        // (a convolution dropped the stale ranges of the sum's slot before it ran and may have noted the sum's own)
+        if (!p->instrs[idx - 1].add_is_conv) drop_ranges_overlapping(b, in.dst);
         return FNN_OK;
     }
     p->add_done = (size_t)-1;
@@ -926,7 +947,7 @@ int run_instr(fnn_backend *b, fnn_plan *p, size_t idx, bool consts_resident)
         int64_t fuse = 1, hand = 1;
         fnn_hip_get_option(b->ctx, FNN_OPT_FUSE_RESIDUAL, &fuse);
         fnn_hip_get_option(b->ctx, FNN_OPT_FUSE_PREP, &hand);
-        // the Add behind this MatMul rides along: the MatMul's last kernel stores the sum too where it can
+        // the Add behind this MatMul (Conv2d) rides along: the call's last kernel stores the sum too where it can
         bool with_res = in.add_operand >= 0 && fuse && idx + 1 < p->instrs.size();
         if (with_res) {
             const Instr &ad = p->instrs[idx + 1];

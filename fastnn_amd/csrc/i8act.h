@@ -40,6 +40,10 @@ struct QConvArgs {
                              // the padding still has to join them
     float *range_out;        // non-null: partial (min, max) pairs of y per image go here, [B][range_out_stride][2]
     int range_out_stride;
+    // a plan's Add behind this convolution (range_io.h, FnnResidualIo): sum_out = y + residual, same shape as y, stored
+    // by the kernels whose epilogue holds the outputs in registers; the partial ranges are then those of the sums
+    const float *residual = nullptr;
+    float *sum_out = nullptr;
 };
 constexpr int QCONV_NPART = 512;
 // divisors of the im2col index arithmetic: pixels per image, output width, kernel area, kernel width

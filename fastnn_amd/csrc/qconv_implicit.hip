@@ -350,6 +350,8 @@ __global__ void __launch_bounds__(64 * PW * KW, TAB ? 4 : 2) conv_implicit_kerne
         const bool has_bias = a.bias != nullptr;
         float *y = a.y + (int64_t)g * ocg * np;
         int32_t *acc_out = a.acc_out ? a.acc_out + (int64_t)g * ocg * np : nullptr;
+        const float *residual = a.residual ? a.residual + (int64_t)g * ocg * np : nullptr;
+        float *sum_out = a.sum_out + (int64_t)g * ocg * np;
         if constexpr (TN == 1) {
             if (share) {
                 // rows of 16 lanes: (k half 0, channels 0-15), (0, 16-31), (1, 0-15), (1, 16-31).  Registers 8 .. 15 (pixel
@@ -389,6 +391,34 @@ __global__ void __launch_bounds__(64 * PW * KW, TAB ? 4 : 2) conv_implicit_kerne
                     v[j] = conv_affine(ai, rsa[j], rza[j], rs[j], sw[tn], zw[tn], sw[tn] * (float)wq_[tn], bq[j], kk, &av[j]);
                 }
                 conv_act4(v, a.act);
+                // a.residual: the Add behind this convolution; v becomes the sums, whose ranges travel on instead of y's
+                if (p.vec4) {
+                    const int64_t o = r_off[pw][rr0] + n * np;
+                    if constexpr (TN > 1) {   // stored below, channel by channel
+#pragma unroll
+                        for (int j = 0; j < 4; j++) acc[tn][igl * 4 + j] = __float_as_int(v[j]);
+                    } else {
+                        *reinterpret_cast<float4 *>(y + o) = make_float4(v[0], v[1], v[2], v[3]);
+                    }
+                    if (acc_out) *reinterpret_cast<int4 *>(acc_out + o) = make_int4(av[0], av[1], av[2], av[3]);
+                    if (residual) {
+                        const float4 r4 = *reinterpret_cast<const float4 *>(residual + o);
+                        v[0] = v[0] + r4.x; v[1] = v[1] + r4.y; v[2] = v[2] + r4.z; v[3] = v[3] + r4.w;
+                        *reinterpret_cast<float4 *>(sum_out + o) = make_float4(v[0], v[1], v[2], v[3]);
+                    }
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        if (r0 + j >= rows) continue;
+                        const int64_t o = r_off[pw][rr0 + j] + n * np;
+                        y[o] = v[j];
+                        if (acc_out) acc_out[o] = av[j];
+                        if (residual) {
+                            v[j] = v[j] + residual[o];
+                            sum_out[o] = v[j];
+                        }
+                    }
+                }
                 if constexpr (RNG) {
                     if (rng_plain) {   // (workgroup-uniform) every pixel of the block exists and lies in one image
                         mn0 = fminf(fminf(mn0, fminf(v[0], v[1])), fminf(v[2], v[3]));
@@ -400,24 +430,6 @@ __global__ void __launch_bounds__(64 * PW * KW, TAB ? 4 : 2) conv_implicit_kerne
                             if (rng_two && r_img[pw][rr0 + j]) { mn1 = fminf(mn1, v[j]); mx1 = fmaxf(mx1, v[j]); }
                             else { mn0 = fminf(mn0, v[j]); mx0 = fmaxf(mx0, v[j]); }
                         }
-                    }
-                }
-                if (p.vec4) {
-                    const int64_t o = r_off[pw][rr0] + n * np;
-                    if constexpr (TN > 1) {   // stored below, channel by channel
-#pragma unroll
-                        for (int j = 0; j < 4; j++) acc[tn][igl * 4 + j] = __float_as_int(v[j]);
-                    } else {
-                        *reinterpret_cast<float4 *>(y + o) = make_float4(v[0], v[1], v[2], v[3]);
-                    }
-                    if (acc_out) *reinterpret_cast<int4 *>(acc_out + o) = make_int4(av[0], av[1], av[2], av[3]);
-                } else {
-#pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        if (r0 + j >= rows) continue;
-                        const int64_t o = r_off[pw][rr0 + j] + n * np;
-                        y[o] = v[j];
-                        if (acc_out) acc_out[o] = av[j];
                     }
                 }
             }
@@ -700,6 +712,8 @@ __global__ void __launch_bounds__(256) conv_fused_kernel(ImplicitArgs p)
     const bool has_bias = a.bias != nullptr;
     float *y = a.y + (int64_t)g * ocg * np;
     int32_t *acc_out = a.acc_out ? a.acc_out + (int64_t)g * ocg * np : nullptr;
+    const float *residual = a.residual ? a.residual + (int64_t)g * ocg * np : nullptr;
+    float *sum_out = a.sum_out + (int64_t)g * ocg * np;
     const int nblocks = (ocg + TN * 32 - 1) / (TN * 32);
     for (int cb = wv; cb < nblocks; cb += NW) {
         const int n0 = cb * (TN * 32);
@@ -794,6 +808,29 @@ __global__ void __launch_bounds__(256) conv_fused_kernel(ImplicitArgs p)
                     v[j] = conv_affine(ai, rsa[j], rza[j], rs[j], sw[tn], zw[tn], sw[tn] * (float)wq_[tn], bq[j], kk, &av[j]);
                 }
                 conv_act4(v, a.act);
+                // a.residual: the Add behind this convolution; v becomes the sums, whose ranges travel on instead of y's
+                if (p.vec4) {
+                    const int64_t o = r_off[rr0] + n * np;
+                    *reinterpret_cast<float4 *>(y + o) = make_float4(v[0], v[1], v[2], v[3]);
+                    if (acc_out) *reinterpret_cast<int4 *>(acc_out + o) = make_int4(av[0], av[1], av[2], av[3]);
+                    if (residual) {
+                        const float4 r4 = *reinterpret_cast<const float4 *>(residual + o);
+                        v[0] = v[0] + r4.x; v[1] = v[1] + r4.y; v[2] = v[2] + r4.z; v[3] = v[3] + r4.w;
+                        *reinterpret_cast<float4 *>(sum_out + o) = make_float4(v[0], v[1], v[2], v[3]);
+                    }
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        if (r0 + j >= rows) continue;
+                        const int64_t o = r_off[rr0 + j] + n * np;
+                        y[o] = v[j];
+                        if (acc_out) acc_out[o] = av[j];
+                        if (residual) {
+                            v[j] = v[j] + residual[o];
+                            sum_out[o] = v[j];
+                        }
+                    }
+                }
                 if constexpr (RNG) {
                     if (rng_plain) {   // (workgroup-uniform) every pixel of the block exists and lies in one image
                         mn0 = fminf(fminf(mn0, fminf(v[0], v[1])), fminf(v[2], v[3]));
@@ -805,19 +842,6 @@ __global__ void __launch_bounds__(256) conv_fused_kernel(ImplicitArgs p)
                             if (rng_two && r_img[rr0 + j]) { mn1 = fminf(mn1, v[j]); mx1 = fmaxf(mx1, v[j]); }
                             else { mn0 = fminf(mn0, v[j]); mx0 = fmaxf(mx0, v[j]); }
                         }
-                    }
-                }
-                if (p.vec4) {
-                    const int64_t o = r_off[rr0] + n * np;
-                    *reinterpret_cast<float4 *>(y + o) = make_float4(v[0], v[1], v[2], v[3]);
-                    if (acc_out) *reinterpret_cast<int4 *>(acc_out + o) = make_int4(av[0], av[1], av[2], av[3]);
-                } else {
-#pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        if (r0 + j >= rows) continue;
-                        const int64_t o = r_off[rr0 + j] + n * np;
-                        y[o] = v[j];
-                        if (acc_out) acc_out[o] = av[j];
                     }
                 }
             }
@@ -998,7 +1022,10 @@ int fnn_i8_implicit_conv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *
     ia.a = p;
     ia.dv = ConvDivs{fast_div((uint32_t)np), fast_div((uint32_t)p.wo), fast_div((uint32_t)(p.kh * p.kw)), fast_div((uint32_t)p.kw)};
     ia.kk = (int)kk;
-    ia.vec4 = (np % 4 == 0 && (reinterpret_cast<uintptr_t>(p.y) & 15) == 0 && (!p.acc_out || (reinterpret_cast<uintptr_t>(p.acc_out) & 15) == 0)) ? 1 : 0;
+    const bool with_sum = p.residual && p.sum_out;
+    if (!with_sum) ia.a.residual = nullptr;
+    ia.vec4 = (np % 4 == 0 && (reinterpret_cast<uintptr_t>(p.y) & 15) == 0 && (!p.acc_out || (reinterpret_cast<uintptr_t>(p.acc_out) & 15) == 0) &&
+               (!with_sum || ((reinterpret_cast<uintptr_t>(p.residual) | reinterpret_cast<uintptr_t>(p.sum_out)) & 15) == 0)) ? 1 : 0;
     if (form == 2) wg_rows = 32;
     const int64_t parts = (np / wg_rows + 2) * (form == 2 ? 1 : (ocg + tn * 32 - 1) / (tn * 32));
     if (p.range_out && p.groups == 1 && np >= wg_rows && parts <= p.range_out_stride) fnn_ctx_range_io(ctx)->out_parts = (int)parts;
@@ -1015,6 +1042,7 @@ int fnn_i8_implicit_conv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *
         }
         if (e != hipSuccess) return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, hipGetErrorString(e));
     }
+    if (with_sum) fnn_ctx_residual_io(ctx)->used = 1;   // the epilogue stored y + residual as well
     *handled = true;
     return FNN_OK;
 }

@@ -802,7 +802,9 @@ int fnn_i8_tiled_conv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, 
     const bool fused = !p.payload_i4 && opt_fused != 2;
     const int64_t tiles128 = (rows_pad / 128) * (ocg <= 64 ? 1 : (ocg + 127) / 128);
     const bool small_tiles = tiles128 <= 256 && opt_fused != 3;   // less than one 128-row tile per CU
-    const bool vec4 = np % 4 == 0 && (reinterpret_cast<uintptr_t>(p.y) & 15) == 0 && (!p.acc_out || (reinterpret_cast<uintptr_t>(p.acc_out) & 15) == 0);
+    const bool with_sum = fused && p.residual && p.sum_out;   // (the epilogue kernel of its own leaves the Add to its caller)
+    const bool vec4 = np % 4 == 0 && (reinterpret_cast<uintptr_t>(p.y) & 15) == 0 && (!p.acc_out || (reinterpret_cast<uintptr_t>(p.acc_out) & 15) == 0) &&
+                      (!with_sum || ((reinterpret_cast<uintptr_t>(p.residual) | reinterpret_cast<uintptr_t>(p.sum_out)) & 15) == 0);
     for (int g = 0; g < p.groups; g++) {
         const dim3 grid((unsigned)(rows_pad / 64), (unsigned)nq);
         const bool w4 = p.wbits == 4;
@@ -827,7 +829,8 @@ int fnn_i8_tiled_conv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, 
             cv.cv.actq = p.actq; cv.cv.qsum = qsum; cv.cv.row_qsum = p.row_qsum + g * ocg;
             cv.cv.oc = p.oc; cv.cv.np = (uint32_t)np; cv.cv.nq = nq; cv.cv.groups = p.groups; cv.cv.g = g; cv.cv.kk = (int)kk;
             cv.cv.vec4 = vec4 ? 1 : 0;
-            // partial ranges of y for the next convolution: one group, and tiles that meet at most two images
+            if (with_sum) { cv.cv.residual = p.residual + g * ocg * np; cv.cv.sum_out = p.sum_out + g * ocg * np; }
+            // partial ranges of y (of the sums, with a residual) for the next convolution: one group, and tiles that meet at most two images
             const int64_t bm = small_tiles ? 64 : 128;
             const int64_t ntl = small_tiles ? (ocg + 63) / 64 : (ocg <= 64 ? 1 : (ocg + 127) / 128);
             const int64_t parts = (np / bm + 2) * ntl;
@@ -846,6 +849,7 @@ int fnn_i8_tiled_conv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, 
         }
         if (e != hipSuccess) return fnn_ctx_fail(ctx, FNN_ERR_DISPATCH, hipGetErrorString(e));
     }
+    if (with_sum) fnn_ctx_residual_io(ctx)->used = 1;
     *handled = true;
     return FNN_OK;
 }

@@ -29,15 +29,15 @@ struct FnnRangeIo {
 FnnRangeIo *fnn_ctx_range_io(fnn_hip_ctx *ctx);
 bool fnn_ctx_capturing(fnn_hip_ctx *ctx);   // a HIP graph is being recorded on the context's stream: no allocation
 
-// A residual that travels with a MatMul call: a plan's MatMul followed by an Add of its output and another tensor
-// can finish as one call.  The caller states the other operand and where the sum goes before the MatMul call (which
+// A residual that travels with a MatMul or quantised Conv2d call: a plan's MatMul (Conv2d) followed by an Add of its
+// output and another tensor can finish as one call.  The caller states the other operand and where the sum goes before the MatMul call (which
 // still writes its own output); `used` tells afterwards whether the call's last kernel stored the sum as well (then
 // sum_out[i] = out[i] + residual[i], the same f32 addition the Add would have done), else the caller runs the Add.
 struct FnnResidualIo {
     const float *residual = nullptr;
     float *sum_out = nullptr;
-    const float *of_out = nullptr;   // the MatMul output the request is about
-    uint64_t elems = 0;              // M * N
+    const float *of_out = nullptr;   // the MatMul (Conv2d) output the request is about
+    uint64_t elems = 0;              // M * N (B * OC * HO * WO)
     int used = 0;
 };
 FnnResidualIo *fnn_ctx_residual_io(fnn_hip_ctx *ctx);

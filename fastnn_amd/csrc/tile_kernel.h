@@ -46,6 +46,9 @@ struct TileArgs {
         // (mt - first tile of the image) * ntiles + nt of every image it meets, (np / BM + 2) * ntiles pairs per image
         float *range_out;
         int range_stride;
+        // non-null: sum_out = y + residual as well (same layout as y); range_out then describes the sums
+        const float *residual;
+        float *sum_out;
     } cv;
 };
 
@@ -692,6 +695,28 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
                         v[j] = conv_affine(a, sa[j], za[j], rs[j], sw[tn], zw[tn], wt[tn], bq[j], p.cv.kk, &av[j]);
                     }
                     conv_act4(v, p.act);
+                    if (p.cv.vec4) {
+                        const int64_t o = cv_off[rr0] + n * np;
+                        *reinterpret_cast<float4 *>(p.cv.y + o) = make_float4(v[0], v[1], v[2], v[3]);
+                        if (p.cv.acc_out) *reinterpret_cast<int4 *>(p.cv.acc_out + o) = make_int4(av[0], av[1], av[2], av[3]);
+                        if (p.cv.residual) {   // the Add behind this convolution: v becomes the sums (their ranges travel on)
+                            const float4 r4 = *reinterpret_cast<const float4 *>(p.cv.residual + o);
+                            v[0] = v[0] + r4.x; v[1] = v[1] + r4.y; v[2] = v[2] + r4.z; v[3] = v[3] + r4.w;
+                            *reinterpret_cast<float4 *>(p.cv.sum_out + o) = make_float4(v[0], v[1], v[2], v[3]);
+                        }
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < 4; j++) {
+                            if (r0 + j >= p.m) continue;
+                            const int64_t o = cv_off[rr0 + j] + n * np;
+                            p.cv.y[o] = v[j];
+                            if (p.cv.acc_out) p.cv.acc_out[o] = av[j];
+                            if (p.cv.residual) {
+                                v[j] = v[j] + p.cv.residual[o];
+                                p.cv.sum_out[o] = v[j];
+                            }
+                        }
+                    }
                     if constexpr (CRNG) {
                         if (rng_plain) {   // (workgroup-uniform) every row of the tile exists and lies in one image
                             mn0 = fminf(fminf(mn0, fminf(v[0], v[1])), fminf(v[2], v[3]));
@@ -703,19 +728,6 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
                                 if (second[j]) { mn1 = fminf(mn1, v[j]); mx1 = fmaxf(mx1, v[j]); }
                                 else { mn0 = fminf(mn0, v[j]); mx0 = fmaxf(mx0, v[j]); }
                             }
-                        }
-                    }
-                    if (p.cv.vec4) {
-                        const int64_t o = cv_off[rr0] + n * np;
-                        *reinterpret_cast<float4 *>(p.cv.y + o) = make_float4(v[0], v[1], v[2], v[3]);
-                        if (p.cv.acc_out) *reinterpret_cast<int4 *>(p.cv.acc_out + o) = make_int4(av[0], av[1], av[2], av[3]);
-                    } else {
-#pragma unroll
-                        for (int j = 0; j < 4; j++) {
-                            if (r0 + j >= p.m) continue;
-                            const int64_t o = cv_off[rr0 + j] + n * np;
-                            p.cv.y[o] = v[j];
-                            if (p.cv.acc_out) p.cv.acc_out[o] = av[j];
                         }
                     }
                 }

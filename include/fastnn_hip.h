@@ -133,9 +133,9 @@ enum {
                                   /* fetched and quantised in the GEMM's operand registers, no int8 operand in memory), 2 = the */
                                   /* operand kernel + GEMM pair, 3 = the fused kernel (a workgroup quantises 32 pixels once     */
                                   /* into LDS and runs all output channels against them; K up to 1280), 0 (default) = by shape  */
-    FNN_OPT_FUSE_RESIDUAL = 17,   /* plans: 1 (default) = a MatMul whose output the next instruction adds to another tensor       */
-                                  /* stores that sum from its own last kernel where it can (the Add instruction is then skipped; */
-                                  /* same f32 addition, identical results), 0 = every Add runs as its own launch                 */
+    FNN_OPT_FUSE_RESIDUAL = 17,   /* plans: 1 (default) = a MatMul or quantised Conv2d whose output the next instruction adds to  */
+                                  /* another tensor stores that sum from its own last kernel where it can (the Add instruction   */
+                                  /* is then skipped; same f32 addition, identical results), 0 = every Add runs as its own launch */
     FNN_OPT_FUSE_PREP = 18,       /* plans: 1 (default) = a MatMul at 17 <= M whose result the next instruction multiplies (f16    */
                                   /* matrix-core weight types) leaves that MatMul's prepared activation operand behind, which  */
                                   /* then skips its own preparation launch (same conversion code, identical results); 0 = off  */

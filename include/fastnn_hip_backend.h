@@ -137,7 +137,7 @@ int fnn_plan_replayed(const fnn_plan *p);
  * fastnn: lets tests and tools see which path ran). */
 uint64_t fnn_plan_ranges_used(const fnn_plan *p);
 /* add_f32 instructions of the plan that, on its last pass (or in its recorded graph), did not run as a launch of
- * their own because the MatMul before them stored the sum (FNN_OPT_FUSE_RESIDUAL; no counterpart in fastnn). */
+ * their own because the MatMul or Conv2d before them stored the sum (FNN_OPT_FUSE_RESIDUAL; no counterpart in fastnn). */
 uint64_t fnn_plan_residuals_fused(const fnn_plan *p);
 /* MatMul instructions of the plan that, on its last pass (or in its recorded graph), found their activation operand
  * prepared by the split-K reduction of the MatMul before them (FNN_OPT_FUSE_PREP; no counterpart in fastnn). */

@@ -932,6 +932,81 @@ def test_matmul_followed_by_residual_add_runs_as_one_call(be, orc, wdt, kname):
         assert np.array_equal(view(s), view(s_y[0]) + r)
 
 
+@pytest.mark.parametrize("implicit", [0, 1, 2, 3])
+@pytest.mark.parametrize("wdt,kname,geom", [
+    (flib.DT_I8, "conv2d_i8_silu", (3, 16, 20, 20, 24, 3)),    # (images, C, H, W, OC, kernel side)
+    (flib.DT_I4, "conv2d_i4", (2, 8, 9, 9, 40, 3)),            # 81 pixels per image: outputs stored one by one
+    (flib.DT_I8, "conv2d_i8_relu", (2, 32, 12, 12, 136, 1)),   # more than 128 channels
+    (flib.DT_I8, "conv2d_i8", (1, 144, 16, 16, 16, 3)),        # K = 1296: beyond the kernel that holds its operands in LDS
+])
+def test_conv_followed_by_residual_add_runs_as_one_call(be, orc, implicit, wdt, kname, geom):
+    """A quantised Conv2d whose output the next instruction adds to another tensor stores the sum from its epilogue
+    (FNN_OPT_FUSE_RESIDUAL, the Add is skipped), in each of its kernel forms: the whole arena is, bit for bit, what
+    the instructions give on their own, including the convolution that reads a sum (whose activation ranges then
+    come from the fused epilogue, not from the Add).  The sum overwriting the convolution's output or its input
+    still runs the Add."""
+    rng = np.random.default_rng(211 + wdt + geom[1])
+    n, c, h, w, oc, k = geom
+    hw, kk = h * w, c * k * k
+    x = rng.uniform(-1, 1, (n, c, h, w)).astype(np.float32)
+    r = rng.standard_normal((n, oc, h, w)).astype(np.float32)
+    pw = fastnn_amd.quantize_weights(wdt, (rng.standard_normal((oc, kk)) * np.sqrt(2.0 / kk)).astype(np.float32))
+    bias = (rng.standard_normal(oc) * 0.05).astype(np.float32)
+    pw2 = fastnn_amd.quantize_weights(flib.DT_I8, (rng.standard_normal((8, oc)) * np.sqrt(2.0 / oc)).astype(np.float32))
+    pwx = fastnn_amd.quantize_weights(flib.DT_I8, (rng.standard_normal((c, c)) * np.sqrt(2.0 / c)).astype(np.float32))
+    a = Arena()
+    ybytes = n * oc * hw * 4
+    s_x, s_r, s_w, s_b, s_w2, s_wx = a.take(x.nbytes), a.take(r.nbytes), a.take(pw.words.nbytes), a.take(bias.nbytes), a.take(pw2.words.nbytes), a.take(pwx.words.nbytes)
+    s_y = [a.take(ybytes) for _ in range(5)]
+    s_sum = [a.take(ybytes) for _ in range(5)]
+    s_r2, s_next, s_x2, s_y5 = a.take(r.nbytes), [a.take(n * 8 * hw * 4) for _ in range(2)], a.take(x.nbytes), a.take(x.nbytes)
+    plan = ExecutablePlan(a.top).write_const(s_w[0], pw.words).write_const(s_b[0], bias).write_const(s_w2[0], pw2.words).write_const(s_wx[0], pwx.words)
+    cv = lambda dst, src=s_x: plan.call_kernel(kname, [src, s_w, s_b], dst, [1, k // 2, 1, 1, c, h, w, k, k], meta_of(pw, [oc, c, k, k]))
+    reader = lambda src, dst: plan.call_kernel("conv2d_i8", [src, s_w2], dst, [1, 0, 1, 1, oc, h, w, 1, 1], meta_of(pw2, [8, oc, 1, 1]))
+    cv(s_y[0]); plan.call_kernel("add_f32", [s_y[0], s_r], s_sum[0], [n * oc * hw])       # convolution output first
+    reader(s_sum[0], s_next[0])                                                            # ... and a convolution reads the sum
+    cv(s_y[1]); plan.call_kernel("add_f32", [s_r, s_y[1]], s_sum[1], [n * oc * hw])       # ... second
+    plan.memcopy(s_r2, s_r)
+    cv(s_y[2]); plan.call_kernel("add_f32", [s_y[2], s_r2], s_r2, [n * oc * hw])          # the sum replaces the other operand
+    reader(s_r2, s_next[1])
+    cv(s_y[3]); plan.call_kernel("add_f32", [s_y[3], s_r], s_y[3], [n * oc * hw])         # ... replaces the convolution's output: not fused
+    # x2 = x2 + conv(x2) with C -> C channels: the sum would land where workgroups still read their taps: not fused
+    plan.memcopy(s_x2, s_x)
+    plan.call_kernel("conv2d_i8", [s_x2, s_wx], s_y5, [1, 0, 1, 1, c, h, w, 1, 1], meta_of(pwx, [c, c, 1, 1]))
+    plan.call_kernel("add_f32", [s_y5, s_x2], s_x2, [n * c * hw])
+    be.allocate_arena(a.top)
+    be.write_arena(s_x[0], x)
+    be.write_arena(s_r[0], r)
+    got, used = {}, {}
+    try:
+        be.set_option(flib.OPT_CONV_IMPLICIT, implicit)
+        for fuse in (1, 0):
+            be.set_option(flib.OPT_FUSE_RESIDUAL, fuse)
+            be.dispatch(plan)
+            first = be.read_arena(0, a.top).copy()
+            be.dispatch(plan)
+            assert plan.replayed
+            got[fuse] = be.read_arena(0, a.top).copy()
+            used[fuse] = plan.ranges_used
+            assert np.array_equal(first, got[fuse]), "replay differs from the first dispatch"
+            assert plan.residuals_fused == (3 if fuse else 0)
+    finally:
+        be.set_option(flib.OPT_FUSE_RESIDUAL, 1)
+        be.set_option(flib.OPT_CONV_IMPLICIT, 0)
+    assert np.array_equal(got[1], got[0])
+    # both readers take the ranges of the sums from the Add, or from the fused epilogue when an image holds at least a
+    # workgroup's pixels (the third taker is the convolution behind the copy of x)
+    assert used[0] == 3 and used[1] <= 3 and (hw < 256 or used[1] == 3), used
+    view = lambda s, ch=oc: got[1][s[0]:s[0] + s[1]].view(np.float32).reshape(n, ch, h, w)
+    act = {"silu": flib.ACT_SILU, "relu": flib.ACT_RELU}.get(kname.split("_")[-1], 0)
+    want_y = orc.qconv2d_i8(x, to_oracle(orc, pw), k, k, 1, k // 2, 1, 1, bias=bias, act=act)
+    for i in range(3):
+        assert_close(view(s_y[i]), want_y, 1e-5, f"convolution output {i}")
+    for s in (s_sum[0], s_sum[1], s_r2, s_y[3]):
+        assert np.array_equal(view(s), view(s_y[0]) + r)
+    assert np.array_equal(view(s_x2, c), view(s_y5, c) + x)
+
+
 @pytest.mark.parametrize("m", [64, 40])
 @pytest.mark.parametrize("single", [0, 1])
 def test_matmul_chain_hands_the_prepared_operand_on(be, orc, m, single):
