@@ -932,6 +932,27 @@ def test_matmul_followed_by_residual_add_runs_as_one_call(be, orc, wdt, kname):
         assert np.array_equal(view(s), view(s_y[0]) + r)
 
 
+def test_residual_add_onto_the_matmul_input_stays_an_instruction(be, orc):
+    """x = x + MatMul(x) with the sum written over x: workgroups of the MatMul still read x while others would store
+    sums, so the Add is not folded into the MatMul's last kernel."""
+    rng = np.random.default_rng(5)
+    m, d = 48, 512
+    x = rng.standard_normal((m, d)).astype(np.float32)
+    pw = fastnn_amd.quantize_weights(flib.DT_I8, _w(rng, d, d))
+    a = Arena()
+    s_x, s_w, s_y = a.take(x.nbytes), a.take(pw.words.nbytes), a.take(x.nbytes)
+    plan = ExecutablePlan(a.top).write_const(s_w[0], pw.words)
+    plan.call_kernel("matmul_i8", [s_x, s_w], s_y, [m, d, d], meta_of(pw)).call_kernel("add_f32", [s_y, s_x], s_x, [m * d])
+    be.allocate_arena(a.top)
+    for it in range(2):
+        be.write_arena(s_x[0], x)
+        be.dispatch(plan)
+        assert plan.residuals_fused == 0
+        y = be.read_arena(*s_y, np.float32).reshape(m, d)
+        assert_close(y, orc.qmatmul(to_oracle(orc, pw), x), 2e-5, "MatMul output")
+        assert np.array_equal(be.read_arena(*s_x, np.float32).reshape(m, d), y + x)
+
+
 @pytest.mark.parametrize("implicit", [0, 1, 2, 3])
 @pytest.mark.parametrize("wdt,kname,geom", [
     (flib.DT_I8, "conv2d_i8_silu", (3, 16, 20, 20, 24, 3)),    # (images, C, H, W, OC, kernel side)
