@@ -608,16 +608,16 @@ int fnn_hip_qmatmul(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *a, i
                 int rc = fnn_i8dot_qgemv(ctx, ctx->stream, w, p, &handled);
                 if (rc) return rc;
             }
+            if (!handled) {   // (17 <= M <= 32 and, for few columns under a long K, from M = 5)
+                int rc = fnn_stream_qmatmul(ctx, ctx->stream, w, p, flags, &handled);
+                if (rc) return rc;
+            }
             if (!handled) {
                 int rc = fnn_mfma_qgemv(ctx, ctx->stream, w, p, flags, &handled);
                 if (rc) return rc;
             }
             if (!handled) {
                 int rc = fnn_mfma_rows16(ctx, ctx->stream, w, p, flags, &handled);
-                if (rc) return rc;
-            }
-            if (!handled) {
-                int rc = fnn_stream_qmatmul(ctx, ctx->stream, w, p, flags, &handled);
                 if (rc) return rc;
             }
             if (!handled) {

@@ -374,6 +374,35 @@ def test_streaming_matmul_takes_the_default_route_and_propagates_non_finite_rows
         ctx.release(h)
 
 
+@pytest.mark.parametrize("dt", [flib.DT_I8, flib.DT_I4, flib.DT_U8, flib.DT_F8, flib.DT_F4])
+@pytest.mark.parametrize("m,k,n", [(5, 2048, 512), (8, 4096, 1000), (12, 8192, 2048), (16, 4096, 768)])
+def test_streaming_matmul_narrow_outputs_from_m5(ctx, orc, dt, m, k, n):
+    """Few output columns under a long K (N <= 2048, K >= 4 N): the streaming kernel takes 5 <= M <= 16 as well (the
+    one-launch kernels for those M give a workgroup whole rows, too few workgroups here).  Against the oracle with
+    bias + SiLU, the same bits on two calls, and another kernel than the one that runs with the streaming kernel off
+    (at M <= 8 the int8 GEMV serves the integer types either way)."""
+    rng = np.random.default_rng(5500 + dt * 11 + m)
+    pw = fastnn_amd.quantize_weights(dt, _weights(rng, n, k))
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    a[:, ::97] *= 150.0
+    a[m // 2] = 0.0
+    bias = (rng.standard_normal(n) * 0.01).astype(np.float32)
+    h = ctx.register(pw)
+    want = orc.qmatmul(to_oracle(orc, pw), a, order=2, bias=bias, act=3)
+    got = ctx.qmatmul(h, a, n, bias=bias, act=3)
+    assert_close(got, want, TOL_F32, f"narrow {NAMES[dt]} {m}x{k}x{n}")
+    assert np.array_equal(got, ctx.qmatmul(h, a, n, bias=bias, act=3))
+    ctx.set_option(flib.OPT_STREAM_MAX_M, 0)
+    try:
+        other = ctx.qmatmul(h, a, n, bias=bias, act=3)
+    finally:
+        ctx.set_option(flib.OPT_STREAM_MAX_M, 32)
+    assert_close(other, want, TOL_F32)
+    if m > 8 or dt in (flib.DT_U8, flib.DT_F8, flib.DT_F4):
+        assert not np.array_equal(got, other), "the streaming kernel did not take the call"
+    ctx.release(h)
+
+
 @pytest.mark.parametrize("m,k,n", [(5, 4096, 520), (16, 1024, 300), (17, 2048, 1100), (32, 4096, 2048), (33, 1536, 260), (48, 2048, 1100),
                                    (64, 4096, 1024), (64, 128, 4400), (50, 2048, 5000)])
 def test_streaming_matmul_codebook_weights(ctx, orc, m, k, n):
