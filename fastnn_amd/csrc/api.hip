@@ -604,12 +604,12 @@ int fnn_hip_qmatmul(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *a, i
         if (!(flags & FNN_FLAG_FORCE_GENERIC)) {
             const bool fma_first = (flags & FNN_FLAG_PREFER_FMA) || w->dtype == FNN_DT_I4CB;
             if (fma_first) HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qgemv(w->dtype, p, ctx->stream, &handled));
-            if (!handled && !(flags & FNN_FLAG_ACT_F16_SINGLE)) {
-                int rc = fnn_i8dot_qgemv(ctx, ctx->stream, w, p, &handled);
+            if (!handled) {   // (17 <= M <= 32 and, for a long K over few columns, from M = 9 or 5)
+                int rc = fnn_stream_qmatmul(ctx, ctx->stream, w, p, flags, &handled);
                 if (rc) return rc;
             }
-            if (!handled) {   // (17 <= M <= 32 and, for few columns under a long K, from M = 5)
-                int rc = fnn_stream_qmatmul(ctx, ctx->stream, w, p, flags, &handled);
+            if (!handled && !(flags & FNN_FLAG_ACT_F16_SINGLE)) {
+                int rc = fnn_i8dot_qgemv(ctx, ctx->stream, w, p, &handled);
                 if (rc) return rc;
             }
             if (!handled) {

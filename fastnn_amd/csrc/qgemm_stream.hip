@@ -67,10 +67,15 @@ int fnn_stream_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w,
     // Codebook weights: the tiled path decodes them on the vector ALU inside its loop and is far from the memory bound,
     // so the range is wider, 5 <= M <= 64 with the options at their defaults.
     if (cb) { lo = lo < 5 ? lo : 5; hi = hi >= 32 ? 64 : hi; }
-    // Few output columns under a long K (the down projection of an MLP): the one-launch kernels for M <= 16 give every
-    // workgroup whole rows, 128 workgroups or fewer here, while this kernel splits K over the chip
-    // (2048 x 8192 FP8, M = 9 .. 16: 12.1-12.4 against 15.5-15.8 us).  Not when the option was raised above its default.
-    if (!cb && lo <= 17 && q.n <= 2048 && q.k >= 4 * q.n) lo = lo < 5 ? lo : 5;
+    // A long K over few output columns (the down projection of an MLP): the one-launch kernels for M <= 16 give every
+    // workgroup whole rows -- few workgroups, each converting M x K activations -- while this kernel splits K over the
+    // chip and its time hardly depends on M.  From M = 9 where K >= 2 N (11008 -> 4096 I4: 16.9-17.2 against 22.7-23.6 us)
+    // and from M = 5 where N <= 2048 and K >= 4 N (8192 -> 2048 FP8: 12.0-12.4 against 13.0-15.8 us; 16384 -> 1024 I4:
+    // 13.7 against 20.2-20.8 us).  Not when the option was raised above its default.
+    if (!cb && lo <= 17) {
+        if (q.k >= 2 * q.n) lo = lo < 9 ? lo : 9;
+        if (q.n <= 2048 && q.k >= 4 * q.n) lo = lo < 5 ? lo : 5;
+    }
     if (q.m < lo || q.m > hi || q.m > (cb ? 64 : 32) || q.n < 1) return FNN_OK;
     if (flags & FNN_FLAG_ACT_F16_SINGLE) return FNN_OK;
     const bool int_type = dt == FNN_DT_I8 || dt == FNN_DT_I4 || dt == FNN_DT_U4;

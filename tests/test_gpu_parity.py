@@ -375,12 +375,12 @@ def test_streaming_matmul_takes_the_default_route_and_propagates_non_finite_rows
 
 
 @pytest.mark.parametrize("dt", [flib.DT_I8, flib.DT_I4, flib.DT_U8, flib.DT_F8, flib.DT_F4])
-@pytest.mark.parametrize("m,k,n", [(5, 2048, 512), (8, 4096, 1000), (12, 8192, 2048), (16, 4096, 768)])
+@pytest.mark.parametrize("m,k,n", [(5, 2048, 512), (8, 4096, 1000), (12, 8192, 2048), (16, 4096, 768), (9, 4096, 2040), (16, 5504, 2600)])
 def test_streaming_matmul_narrow_outputs_from_m5(ctx, orc, dt, m, k, n):
-    """Few output columns under a long K (N <= 2048, K >= 4 N): the streaming kernel takes 5 <= M <= 16 as well (the
-    one-launch kernels for those M give a workgroup whole rows, too few workgroups here).  Against the oracle with
-    bias + SiLU, the same bits on two calls, and another kernel than the one that runs with the streaming kernel off
-    (at M <= 8 the int8 GEMV serves the integer types either way)."""
+    """A long K over few output columns: the streaming kernel takes 9 <= M <= 16 where K >= 2 N and 5 <= M <= 16 where
+    N <= 2048 and K >= 4 N (the one-launch kernels for those M give a workgroup whole rows: few workgroups, each
+    converting all activations).  Against the oracle with bias + SiLU, the same bits on two calls, and another kernel
+    than the one that runs with the streaming kernel off."""
     rng = np.random.default_rng(5500 + dt * 11 + m)
     pw = fastnn_amd.quantize_weights(dt, _weights(rng, n, k))
     a = rng.standard_normal((m, k)).astype(np.float32)
@@ -398,8 +398,7 @@ def test_streaming_matmul_narrow_outputs_from_m5(ctx, orc, dt, m, k, n):
     finally:
         ctx.set_option(flib.OPT_STREAM_MAX_M, 32)
     assert_close(other, want, TOL_F32)
-    if m > 8 or dt in (flib.DT_U8, flib.DT_F8, flib.DT_F4):
-        assert not np.array_equal(got, other), "the streaming kernel did not take the call"
+    assert not np.array_equal(got, other), "the streaming kernel did not take the call"
     ctx.release(h)
 
 
