@@ -649,6 +649,8 @@ def main() -> int:
     ap.add_argument("--fast-act16", action="store_true", help="single f16 rounding of activations on the MFMA path")
     ap.add_argument("--act-quant", action="store_true", help="the opt-in activation-quantised mode (FNN_FLAG_ACT_QUANT; I8 / I4 / F8 weights, "
                     "M >= 17): NOT parity with the default MatMul")
+    ap.add_argument("--i8act", action="store_true", help="time only matmul_i8_i8 / matmul_i4_i8 (an int8 activation payload, resident) at "
+                    "--m on the workload's weights, eager launches (the gemm_m256.c1_i8_i8act leg on its own, for kernel traces)")
     ap.add_argument("--no-extra", "--no-m256", dest="no_extra", action="store_true",
                     help="skip the extra legs (K=N=4096 GEMVs, M=256 GEMMs)")
     ap.add_argument("--opt", action="append", default=[], metavar="NAME=VALUE",
@@ -727,6 +729,18 @@ def main() -> int:
                           "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
                           "config": {"workload": f"probe {args.probe}", "bytes_per_launch": nb, "weight_ring": ring}}))
         ctx.graph_destroy(graph)
+        ctx.close()
+        return 0
+
+    if args.i8act:
+        if dtn not in ("i8", "i4"):
+            raise SystemExit("--i8act: the I8-activation MatMul takes I8 and I4 weights")
+        t8 = time_i8act(ctx, flib, r, m, max(args.steps, 20))
+        print(json.dumps({"metric": f"matmul_{dtn}_i8 at M={m} (int8 activation payload x packed weights, eager launches over the weight ring)",
+                          "value": t8["top_per_s"], "unit": "TOP/s", "n_gpus": 1, "steps": t8["calls"], "warmup": ring, "ms_per_step": round(t8["us"] * 1e-3, 6),
+                          "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "i8/i32", "data": "synthetic",
+                          "config": {"workload": args.workload, "m": m, "k": k, "n": n, "options": opts}, "frac_of_int8_peak": t8["frac"]}))
+        free_ring(ctx, r)
         ctx.close()
         return 0
 
