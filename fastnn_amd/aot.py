@@ -74,20 +74,29 @@ def _attr_int(node: dict, *keys: str, default: int) -> int:
 
 
 class _Value:
-    __slots__ = ("shape", "slot")
+    __slots__ = ("shape", "slot", "view_of")
 
-    def __init__(self, shape: Sequence[int], slot):
+    def __init__(self, shape: Sequence[int], slot, view_of=None):
         self.shape = tuple(int(d) for d in shape)
         self.slot = slot
+        self.view_of = view_of     # (name of the value whose slot holds this one, byte offset inside it) or None
+
+    @property
+    def nbytes(self) -> int:
+        return int(np.prod(self.shape, dtype=np.int64)) * 4
 
 
 class AotExecutor:
     """Compiles the node list into an ExecutablePlan once; forward() writes the inputs into the arena,
-    dispatches (graph replay from the second call on) and reads the outputs."""
+    dispatches (graph replay from the second call on) and reads the outputs.
+
+    concat_in_place (default on): the parts of a Concat with one outer block (a channel Concat of one image) get
+    their slots inside the Concat's result, so their producers store there and the Concat copies only the parts
+    that cannot move (a graph input, a value that lives in another Concat already, a part that comes twice)."""
 
     def __init__(self, nodes: Sequence[Dict[str, str]], params: Dict[str, np.ndarray], input_names: Sequence[str],
                  output_names: Sequence[str], input_shapes: Optional[Dict[str, Sequence[int]]] = None, quantize=None,
-                 device: int = 0):
+                 device: int = 0, concat_in_place: bool = True):
         self.weight_dtype = weight_dtype_of(quantize)
         if self.weight_dtype is None:
             raise FnnError(3, "AotExecutor: only quantised weights run on this backend (quantize=None / 'f32' is the f32 path)")
@@ -100,14 +109,28 @@ class AotExecutor:
                 raise FnnError(4, f"AotExecutor: input_shapes must give the shape of '{n}'")
             if any(int(d) < 0 for d in shapes[n]):
                 raise FnnError(3, f"AotExecutor: symbolic dimension in the shape of '{n}' (static shapes only)")
-        self._top = 0
-        self._values: Dict[str, _Value] = {}
-        self.instructions: List[tuple] = []     # (kernel_name, input names, output name, params): for inspection
-        self._consts: List[tuple] = []          # (offset, array)
-        self._calls: List[tuple] = []           # (kernel, [slots], slot, params, meta)
-        for n in self.input_names:
-            self._new_value(n, shapes[n])
-        self._lower([dict(n) for n in nodes])
+        # Two passes when a Concat joins its parts in one outer block (a channel concat of one image): the first gives
+        # every value its shape, then the values that are such parts get their slot INSIDE the Concat result's slot
+        # (the producers store there, the Concat copies nothing), and the second pass lowers with those slots
+        self._placement: Dict[str, tuple] = {}  # value name -> (name of the Concat result, byte offset inside it)
+        self._sizes: Dict[str, int] = {}
+        self._reserved: Dict[str, tuple] = {}
+        for lowering in (0, 1):
+            self._top = 0
+            self._values: Dict[str, _Value] = {}
+            self.instructions: List[tuple] = []     # (kernel_name, input names, output name, params): for inspection
+            self._consts: List[tuple] = []          # (offset, array)
+            self._calls: List[tuple] = []           # (kernel, [slots], slot, params, meta)
+            self._reserved = {}
+            for n in self.input_names:
+                self._new_value(n, shapes[n])
+            self._lower([dict(n) for n in nodes])
+            if lowering == 1 or not concat_in_place:
+                break
+            self._placement = self._place_concat_parts([dict(n) for n in nodes])
+            if not self._placement:
+                break
+            self._sizes = {k: v.nbytes for k, v in self._values.items()}
         for n in self.output_names:
             if n not in self._values:
                 raise FnnError(4, f"AotExecutor: output '{n}' is produced by no node")
@@ -120,10 +143,77 @@ class AotExecutor:
         self._top += (int(nbytes) + 63) // 64 * 64
         return (off, int(nbytes))
 
+    def _slot_for(self, name: str, nbytes: int):
+        """A value's slot: inside the slot of the Concat result it is a part of (reserved on first use), the slot
+        reserved for it by one of its parts, or a new one."""
+        if name in self._reserved:
+            return self._reserved[name]
+        if name in self._placement:
+            parent, off = self._placement[name]
+            base = self._slot_for(parent, self._sizes[parent])
+            slot = (base[0] + off, int(nbytes))
+        else:
+            slot = self._take(nbytes)
+        self._reserved[name] = slot
+        return slot
+
     def _new_value(self, name: str, shape) -> _Value:
-        v = _Value(shape, self._take(int(np.prod(shape, dtype=np.int64)) * 4))
+        v = _Value(shape, self._slot_for(name, int(np.prod(shape, dtype=np.int64)) * 4))
         self._values[name] = v
         return v
+
+    def _root_of(self, name: str):
+        """(value that owns the slot `name` lives in, byte offset of `name` inside it)."""
+        off = 0
+        while self._values[name].view_of is not None:
+            name, o = self._values[name].view_of
+            off += o
+        return name, off
+
+    def _place_concat_parts(self, nodes: List[dict]) -> Dict[str, tuple]:
+        """After a first lowering: which values can live inside the slot of a Concat result.  A Concat with one
+        outer block lays its parts end to end; a part (or the value a part is a Split view of) takes that place
+        when it is produced by an instruction of the plan, is not placed already, lands 64-byte aligned, and all
+        of its bytes are parts of this Concat at the same relative position."""
+        placed: Dict[str, tuple] = {}
+        for nd in nodes:
+            if nd.get("op_type") != "Concat":
+                continue
+            ins, outs = _names(nd.get("inputs")), _names(nd.get("outputs"))
+            if not outs or outs[0] not in self._values or any(i not in self._values for i in ins):
+                continue
+            out = self._values[outs[0]]
+            rank = len(out.shape)
+            axis = _attr_int(nd, "axis", default=0)
+            axis = axis + rank if axis < 0 else axis
+            axis = min(max(axis, 0), rank - 1)
+            if int(np.prod(out.shape[:axis], dtype=np.int64)) != 1:
+                continue
+            claims: Dict[str, tuple] = {}       # root -> (offset of the root inside the result, [(first byte, size) of its parts])
+            off = 0
+            for x in ins:
+                size = self._values[x].nbytes
+                root, delta = self._root_of(x)
+                want = off - delta
+                if root in claims and claims[root][0] == want:
+                    claims[root][1].append((delta, size))
+                elif root not in claims and root not in placed and root not in self.input_names and root != outs[0]:
+                    claims[root] = (want, [(delta, size)])
+                off += size
+            spans = []
+            for root, (want, parts) in claims.items():
+                rsize = self._values[root].nbytes
+                covered, end = True, 0
+                for d, s in sorted(parts):
+                    covered = covered and d <= end
+                    end = max(end, d + s)
+                if not (covered and end >= rsize and want >= 0 and want % 64 == 0 and want + rsize <= out.nbytes):
+                    continue
+                if any(want < o + s and o < want + rsize for o, s in spans):
+                    continue
+                spans.append((want, rsize))
+                placed[root] = (outs[0], want)
+        return placed
 
     def _const_slot(self, arr: np.ndarray):
         slot = self._take(arr.nbytes)
@@ -191,7 +281,23 @@ class AotExecutor:
                 out = self._new_value(outs[0], shape)
                 inner = int(np.prod(shape[axis + 1:], dtype=np.int64))
                 outer = int(np.prod(shape[:axis], dtype=np.int64))
-                self._emit("concat", ins, outs[0], [v.slot for v in vals], out.slot, [axis, inner, outer])
+                # parts that live at their place inside the result already (their producers stored them there) are
+                # not copied; each run of the others is one concat into its stretch of the result
+                run, run_at, off = [], 0, 0
+                for name, v in list(zip(ins, vals)) + [(None, None)]:
+                    at_home = v is not None and outer == 1 and v.slot == (out.slot[0] + off, v.nbytes)
+                    if (v is None or at_home) and run:
+                        size = sum(r.nbytes for _, r in run)
+                        self._emit("concat", [n for n, _ in run], outs[0], [r.slot for _, r in run],
+                                   out.slot if size == out.nbytes else (out.slot[0] + run_at, size), [axis, inner, outer])
+                        run = []
+                    if v is None:
+                        break
+                    if not at_home:
+                        if not run:
+                            run_at = off
+                        run.append((name, v))
+                    off += v.nbytes
             elif op == "Split":
                 # one slice_f32 per output (src/onnx/converter.rs:549-612): explicit `split` sizes, else equal
                 # parts with the remainder in the last one
@@ -216,7 +322,7 @@ class AotExecutor:
                     if outer == 1 and byte0 % 64 == 0:
                         # one outer block: the part is a contiguous, aligned range of the input's slot; values are
                         # never overwritten (one slot per value), so it needs no copy
-                        self._values[o] = _Value(shape, (a.slot[0] + byte0, sz * inner * 4))
+                        self._values[o] = _Value(shape, (a.slot[0] + byte0, sz * inner * 4), view_of=(ins[0], byte0))
                     else:
                         out = self._new_value(o, shape)
                         self._emit("slice_f32", ins, o, [a.slot], out.slot, [axis, start, start + sz, inner])

@@ -886,10 +886,13 @@ int fnn_hip_qconv2d(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *x, i
             if (const FnnResidualIo &res = ctx->residual; dev && res.residual && res.sum_out && res.of_out == dy && res.elems == (uint64_t)(b * oc * ho * wo)) {
                 p.residual = res.residual; p.sum_out = res.sum_out;
             }
-            // the caller asks for partial ranges of y (range_io.h): the epilogue inside the GEMM kernel leaves them
-            const bool want_out = rio.out_table && dev && rio.out_parts == 0;
+            // the caller asks for partial ranges of y (range_io.h): the epilogue inside the GEMM kernel leaves them.
+            // Pairs already in place (y is one part of a one-image tensor that several calls write): behind them.
+            const int range_base = rio.out_parts;
+            const bool want_out = rio.out_table && dev && (range_base == 0 || (b == 1 && range_base < rio.out_stride));
+            rio.out_parts = 0;
             if (want_out && rio.out_images == (uint64_t)b && rio.out_image_elems == (uint64_t)(oc * ho * wo)) {
-                p.range_out = rio.out_table; p.range_out_stride = rio.out_stride;
+                p.range_out = rio.out_table + 2 * (size_t)range_base; p.range_out_stride = rio.out_stride - range_base;
             }
             // Activation ranges: from the partial pairs the producer of x left (usable when the im2col matrix holds
             // every input value, i.e. every input row and column is reached by some tap, and the group is the whole
@@ -929,7 +932,8 @@ int fnn_hip_qconv2d(fnn_hip_ctx *ctx, const fnn_hip_weight *w, const float *x, i
                 p.nparts = 0;
                 HIP_TRY(ctx, FNN_ERR_DISPATCH, launch_qconv2d_i8(p, ctx->stream, 2, nullptr));
             }
-            if (want_out && rio.out_parts == 0) rio.out_failed = 1;   // y is written, its ranges are not
+            if (rio.out_table && dev && rio.out_parts == 0) rio.out_failed = 1;   // y is written, its ranges are not
+            rio.out_parts += range_base;
         }
         if (!dev) {
             HIP_TRY(ctx, FNN_ERR_MEMORY, hipMemcpyAsync(y, dy, yout, hipMemcpyDeviceToHost, ctx->stream));

@@ -162,8 +162,13 @@ struct fnn_backend {
     // pass ends.
     struct RangeTable { float *dev = nullptr; uint64_t images = 0; };
     struct LiveRange { fnn_slice slice; const float *table; int parts; uint64_t image_elems, images; };
+    // A one-image tensor that several instructions write part by part (producers that store straight into the slot of
+    // a later Concat's result): each leaves its pairs behind those of the parts before it; the entry becomes a live
+    // range once disjoint parts cover the whole slice, and is void as soon as anything else writes into it.
+    struct PendingRange { fnn_slice slice; float *table; int parts; std::vector<fnn_slice> written; bool failed; uint64_t image_elems; };
     std::map<std::pair<uint64_t, uint64_t>, RangeTable> range_tables;
     std::vector<LiveRange> live_ranges;
+    std::vector<PendingRange> pending_ranges;
 };
 constexpr int kRangeStride = 2048;   // pairs per image a table has room for
 
@@ -716,59 +721,125 @@ bool leaves_ranges(const Instr &in)
     return (kn.base == "conv2d_i8" || kn.base == "conv2d_i4") && in.meta.present && in.meta.codebook.empty();
 }
 
-void drop_ranges_overlapping(fnn_backend *b, const fnn_slice &s)
+// (`contributes_to`: the pending entry that the write into `s` adds its own pairs to, which it does not void)
+void drop_ranges_overlapping(fnn_backend *b, const fnn_slice &s, int contributes_to = -1)
 {
     if (!s.size) return;
     auto &v = b->live_ranges;
     v.erase(std::remove_if(v.begin(), v.end(), [&](const fnn_backend::LiveRange &r) { return overlaps(r.slice, s); }), v.end());
+    for (size_t q = 0; q < b->pending_ranges.size(); q++)
+        if ((int)q != contributes_to && overlaps(b->pending_ranges[q].slice, s)) b->pending_ranges[q].failed = true;
+}
+
+void clear_ranges(fnn_backend *b)
+{
+    b->live_ranges.clear();
+    b->pending_ranges.clear();
+}
+
+// a device table of `images` x kRangeStride pairs under `key` (null: none can be had right now)
+float *range_table(fnn_backend *b, fnn_plan *p, std::pair<uint64_t, uint64_t> key, uint64_t images)
+{
+    if (b->range_tables.size() > 1024 && !fnn_ctx_capturing(b->ctx)) {
+        // plans come and go on a long-lived backend: the tables of the others are dropped (they get new
+        // ones on their next pass)
+        for (auto it = b->range_tables.begin(); it != b->range_tables.end();) {
+            if (it->first.first == p->uid) { ++it; continue; }
+            if (it->second.dev) fnn_hip_free(b->ctx, it->second.dev);
+            it = b->range_tables.erase(it);
+        }
+        b->weights_epoch++;   // captured graphs may hold a dropped table
+    }
+    auto &t = b->range_tables[key];
+    if (t.dev && t.images < images && !fnn_ctx_capturing(b->ctx)) {
+        fnn_hip_free(b->ctx, t.dev);
+        t.dev = nullptr;
+        b->weights_epoch++;   // a captured graph may hold the old table
+    }
+    if (!t.dev && !fnn_ctx_capturing(b->ctx)) {
+        void *d = nullptr;
+        if (fnn_hip_malloc(b->ctx, (size_t)images * kRangeStride * 8, &d) == FNN_OK) { t.dev = (float *)d; t.images = images; }
+    }
+    return (t.dev && t.images >= images) ? t.dev : nullptr;
 }
 
 // If a later convolution of the plan reads what instruction `idx` writes (from the first byte of its output slice,
 // before anything overwrites it), asks the next call on the context for the partial ranges that convolution
-// needs; *covered = the convolution's input slice.
-void request_ranges(fnn_backend *b, fnn_plan *p, size_t idx, fnn_slice *covered)
+// needs; *covered = the convolution's input slice.  If a later convolution of ONE image reads a slice of which `idx`
+// writes a part (the slot of a Concat result that its producers fill in place), the request is for the part, behind
+// the pairs of the parts before it; *pending = the entry that collects them (-1: none).  The pairs of a part also
+// serve a convolution that reads just that part (note_ranges), so this form goes first.
+void request_ranges(fnn_backend *b, fnn_plan *p, size_t idx, fnn_slice *covered, int *pending)
 {
     const Instr &in = p->instrs[idx];
     FnnRangeIo *rio = fnn_ctx_range_io(b->ctx);
+    *pending = -1;
     if (!in.dst.size) return;
-    for (size_t j = idx + 1; j < p->instrs.size(); j++) {
+    size_t exact = (size_t)-1, whole = (size_t)-1;
+    ConvInput ce{0, 0}, cw{0, 0};
+    for (size_t j = idx + 1; j < p->instrs.size() && whole == (size_t)-1; j++) {
         const Instr &nx = p->instrs[j];
         ConvInput cj;
-        if (ranged_conv_input(nx, &cj) && nx.inputs[0].offset == in.dst.offset && nx.inputs[0].size <= in.dst.size && cj.images <= 65535) {
-            if (b->range_tables.size() > 1024 && !fnn_ctx_capturing(b->ctx)) {
-                // plans come and go on a long-lived backend: the tables of the others are dropped (they get new
-                // ones on their next pass)
-                for (auto it = b->range_tables.begin(); it != b->range_tables.end();) {
-                    if (it->first.first == p->uid) { ++it; continue; }
-                    if (it->second.dev) fnn_hip_free(b->ctx, it->second.dev);
-                    it = b->range_tables.erase(it);
-                }
-                b->weights_epoch++;   // captured graphs may hold a dropped table
-            }
-            auto &t = b->range_tables[{p->uid, idx}];
-            if (t.dev && t.images < cj.images && !fnn_ctx_capturing(b->ctx)) {
-                fnn_hip_free(b->ctx, t.dev);
-                t.dev = nullptr;
-                b->weights_epoch++;   // a captured graph may hold the old table
-            }
-            if (!t.dev && !fnn_ctx_capturing(b->ctx)) {
-                void *d = nullptr;
-                if (fnn_hip_malloc(b->ctx, (size_t)cj.images * kRangeStride * 8, &d) == FNN_OK) { t.dev = (float *)d; t.images = cj.images; }
-            }
-            if (t.dev && t.images >= cj.images) {
-                rio->out_table = t.dev; rio->out_stride = kRangeStride;
-                rio->out_image_elems = cj.image_elems; rio->out_images = cj.images;
-                *covered = nx.inputs[0];
-            }
-            return;
+        if (ranged_conv_input(nx, &cj)) {
+            const fnn_slice &cs = nx.inputs[0];
+            if (exact == (size_t)-1 && cs.offset == in.dst.offset && cs.size <= in.dst.size && cj.images <= 65535) { exact = j; ce = cj; }
+            if (cj.images == 1 && in.dst.size % 4 == 0 && in.dst.size < cs.size && in.dst.offset >= cs.offset &&
+                in.dst.offset + in.dst.size <= cs.offset + cs.size) { whole = j; cw = cj; }
         }
-        if (overlaps(nx.dst, in.dst) || (nx.has_secondary && overlaps(nx.secondary, in.dst))) return;
+        if (overlaps(nx.dst, in.dst) || (nx.has_secondary && overlaps(nx.secondary, in.dst))) break;
+    }
+    if (whole != (size_t)-1 && (exact == (size_t)-1 || ce.images == 1)) {
+        const fnn_slice &cs = p->instrs[whole].inputs[0];
+        int at = -1;
+        for (size_t q = 0; q < b->pending_ranges.size(); q++)
+            if (b->pending_ranges[q].slice.offset == cs.offset && b->pending_ranges[q].slice.size == cs.size) at = (int)q;
+        if (at < 0) {
+            // (keyed by the consumer, apart from the producers' tables: bit 63)
+            if (float *t = range_table(b, p, {p->uid, (uint64_t)whole | (1ull << 63)}, 1)) {
+                b->pending_ranges.push_back(fnn_backend::PendingRange{cs, t, 0, {}, false, cw.image_elems});
+                at = (int)b->pending_ranges.size() - 1;
+            }
+        }
+        if (at >= 0) {
+            auto &pr = b->pending_ranges[(size_t)at];
+            for (const auto &w : pr.written)
+                if (overlaps(w, in.dst)) pr.failed = true;   // a part written twice: the pairs of the first are stale
+            if (!pr.failed && pr.parts < kRangeStride) {
+                rio->out_table = pr.table; rio->out_stride = kRangeStride; rio->out_parts = pr.parts;
+                rio->out_image_elems = in.dst.size / 4; rio->out_images = 1;
+                *covered = in.dst;
+                *pending = at;
+                return;
+            }
+        }
+    }
+    if (exact != (size_t)-1) {
+        if (float *t = range_table(b, p, {p->uid, idx}, ce.images)) {
+            rio->out_table = t; rio->out_stride = kRangeStride;
+            rio->out_image_elems = ce.image_elems; rio->out_images = ce.images;
+            *covered = p->instrs[exact].inputs[0];
+        }
     }
 }
 
-void note_ranges(fnn_backend *b, const fnn_slice &covered)
+void note_ranges(fnn_backend *b, const fnn_slice &covered, int pending)
 {
     FnnRangeIo *rio = fnn_ctx_range_io(b->ctx);
+    if (pending >= 0 && (size_t)pending < b->pending_ranges.size()) {
+        auto &pr = b->pending_ranges[(size_t)pending];
+        if (!rio->out_table || rio->out_failed || rio->out_parts <= pr.parts) { pr.failed = true; return; }
+        // the part's own pairs describe it to a convolution that reads just the part
+        b->live_ranges.push_back(fnn_backend::LiveRange{covered, pr.table + 2 * (size_t)pr.parts, rio->out_parts - pr.parts, covered.size / 4, 1});
+        pr.parts = rio->out_parts;
+        pr.written.push_back(covered);
+        uint64_t bytes = 0;
+        for (const auto &w : pr.written) bytes += w.size;   // (disjoint: checked when each was requested)
+        if (bytes == pr.slice.size) {
+            b->live_ranges.push_back(fnn_backend::LiveRange{pr.slice, pr.table, pr.parts, pr.image_elems, 1});
+            b->pending_ranges.erase(b->pending_ranges.begin() + pending);
+        }
+        return;
+    }
     if (rio->out_table && rio->out_parts > 0 && !rio->out_failed)
         b->live_ranges.push_back(fnn_backend::LiveRange{covered, rio->out_table, rio->out_parts, rio->out_image_elems, rio->out_images});
 }
@@ -801,14 +872,16 @@ int run_call_with_ranges(fnn_backend *b, fnn_plan *p, size_t idx)
     // sum's ranges (one that does not leaves those of its own output, which are then of no use: the Add runs and
     // asks again)
     fnn_slice covered{0, 0};
-    if (for_sum) request_ranges(b, p, idx + 1, &covered);
-    else if (leaves_ranges(in)) request_ranges(b, p, idx, &covered);
-    drop_ranges_overlapping(b, in.dst);
+    int pending = -1;
+    if (for_sum) request_ranges(b, p, idx + 1, &covered, &pending);
+    else if (leaves_ranges(in)) request_ranges(b, p, idx, &covered, &pending);
+    drop_ranges_overlapping(b, in.dst, for_sum ? -1 : pending);
     if (in.has_secondary) drop_ranges_overlapping(b, in.secondary);
-    if (for_sum) drop_ranges_overlapping(b, p->instrs[idx + 1].dst);
+    if (for_sum) drop_ranges_overlapping(b, p->instrs[idx + 1].dst, pending);
     const int st = run_call(b, in);
     if (st == FNN_OK && rio->in_used) p->ranges_used++;
-    if (st == FNN_OK && (!for_sum || res->used)) note_ranges(b, covered);
+    if (st == FNN_OK && (!for_sum || res->used)) note_ranges(b, covered, pending);
+    else if (pending >= 0) b->pending_ranges[(size_t)pending].failed = true;
     *rio = FnnRangeIo{};
     return st;
 }
@@ -907,7 +980,7 @@ int run_instr(fnn_backend *b, fnn_plan *p, size_t idx, bool consts_resident)
     p->add_done = (size_t)-1;
     const bool offered_here = p->prep_ready == idx;   // the call before this one prepared this MatMul's operand
     p->prep_ready = (size_t)-1;
-    if (in.kind != K_CALL) drop_ranges_overlapping(b, in.kind == K_WRITE_CONST ? fnn_slice{in.dst.offset, in.data.size()} : in.dst);
+    if (in.kind != K_CALL && in.kind != K_MEMCOPY) drop_ranges_overlapping(b, in.kind == K_WRITE_CONST ? fnn_slice{in.dst.offset, in.data.size()} : in.dst);
     switch (in.kind) {
     case K_WRITE_CONST: {
         fnn_slice d{in.dst.offset, in.data.size()};
@@ -932,11 +1005,13 @@ int run_instr(fnn_backend *b, fnn_plan *p, size_t idx, bool consts_resident)
         int64_t ranges_on = 1;
         fnn_hip_get_option(b->ctx, FNN_OPT_CONV_RANGES, &ranges_on);
         fnn_slice covered{0, 0};
-        if (ranges_on && n == in.dst.size && n % 4 == 0 && d.offset % 4 == 0 && s.offset % 4 == 0) request_ranges(b, p, idx, &covered);
+        int pending = -1;
+        if (ranges_on && n == in.dst.size && n % 4 == 0 && d.offset % 4 == 0 && s.offset % 4 == 0) request_ranges(b, p, idx, &covered, &pending);
+        drop_ranges_overlapping(b, in.dst, pending);
         if (rio->out_table && covered.size == n) {
             const uint64_t per = rio->out_image_elems, imgs = rio->out_images;
             int st = lift(b, fnn_hip_copy2d_f32(b->ctx, (float *)(b->arena + d.offset), per, n / 4, (const float *)(b->arena + s.offset), per, n / 4, per, imgs));
-            if (st == FNN_OK) note_ranges(b, covered);
+            if (st == FNN_OK) note_ranges(b, covered, pending);
             *rio = FnnRangeIo{};
             return st;
         }
@@ -1047,14 +1122,14 @@ int dispatch_impl(fnn_backend *b, fnn_plan *p, uint64_t *elapsed_ns, uint64_t n_
         const uint64_t w0 = b->weights_epoch, s0 = fnn_hip_workspace_epoch(b->ctx), c0 = b->scratch_epoch;
         if (fnn_hip_graph_begin(b->ctx) == FNN_OK) {
             int st = FNN_OK;
-            b->live_ranges.clear();
+            clear_ranges(b);
             p->ranges_used = 0;
             p->residuals_fused = 0;
             p->operands_handed = 0;
             p->add_done = (size_t)-1;
             p->prep_ready = (size_t)-1;
             for (size_t i = 0; i < p->instrs.size() && st == FNN_OK; i++) st = run_instr(b, p, i, true);
-            b->live_ranges.clear();
+            clear_ranges(b);
             fnn_hip_graph *g = nullptr;
             int en = fnn_hip_graph_end(b->ctx, &g);
             if (st == FNN_OK && en == FNN_OK && g && w0 == b->weights_epoch && s0 == fnn_hip_workspace_epoch(b->ctx) && c0 == b->scratch_epoch) {
@@ -1080,7 +1155,7 @@ int dispatch_impl(fnn_backend *b, fnn_plan *p, uint64_t *elapsed_ns, uint64_t n_
         return st;
     }
 
-    b->live_ranges.clear();   // ranges never outlive a pass: between passes anyone may write into the arena
+    clear_ranges(b);   // ranges never outlive a pass: between passes anyone may write into the arena
     if (first == 0) { p->ranges_used = 0; p->residuals_fused = 0; p->operands_handed = 0; }
     p->add_done = (size_t)-1;
     p->prep_ready = (size_t)-1;

@@ -80,12 +80,58 @@ def test_conv_lowering():
         {"name": "up", "op_type": "Resize", "inputs": "[k]", "outputs": "[y]", "mode": "nearest", "scale_h": "2", "scale_w": "2"},
     ]
     params = {"w": rng.standard_normal((8, 3, 3, 3)).astype(np.float32), "b": np.zeros(8, np.float32)}
-    ex = AotExecutor(nodes, params, ["x"], ["y"], {"x": [1, 3, 16, 16]}, quantize="i8")
+    ex = AotExecutor(nodes, params, ["x"], ["y"], {"x": [1, 3, 16, 16]}, quantize="i8", concat_in_place=False)
     assert [i[0] for i in ex.instructions] == ["conv2d_i8_silu", "pool_f32", "concat", "upsample_nearest2d"]
     assert ex.instructions[0][3] == [2, 1, 1, 1, 3, 16, 16, 3, 3]
     assert ex.instructions[1][3] == [5, 1, 2, 1, 1, 8, 8, 8]
     assert ex.instructions[2][3] == [1, 64, 1]
     assert ex.instructions[3][3] == [2, 2, 8, 8]
+    # by default the parts of a one-image channel Concat live inside its result: the conv and the pool store there
+    ex = AotExecutor(nodes, params, ["x"], ["y"], {"x": [1, 3, 16, 16]}, quantize="i8")
+    assert [i[0] for i in ex.instructions] == ["conv2d_i8_silu", "pool_f32", "upsample_nearest2d"]
+    k, s, m = ex._values["k"].slot, ex._values["s"].slot, ex._values["m"].slot
+    assert s == (k[0], 8 * 64 * 4) and m == (k[0] + 8 * 64 * 4, 8 * 64 * 4) and k[1] == 16 * 64 * 4
+    # a batch of two: the parts interleave per image, the Concat copies
+    ex = AotExecutor(nodes, params, ["x"], ["y"], {"x": [2, 3, 16, 16]}, quantize="i8")
+    assert [i[0] for i in ex.instructions] == ["conv2d_i8_silu", "pool_f32", "concat", "upsample_nearest2d"]
+
+
+def _concat_graph():
+    """conv -> Split -> conv on one half -> Concat(a, b, t) -> conv -> Concat(x, u, t, u)."""
+    rng = np.random.default_rng(2)
+    conv = lambda name, x, y: [{"name": name, "op_type": "Conv", "inputs": f"[{x}, w{name}]", "outputs": f"[{y}]", "strides": "1", "pads": "0"}]
+    params = {}
+    def w(name, c, oc):
+        params["w" + name] = (rng.standard_normal((oc, c, 1, 1)) * 0.3).astype(np.float32)
+    nodes = []
+    w("c0", 16, 32); nodes += conv("c0", "x", "y")
+    nodes += [{"name": "sp", "op_type": "Split", "inputs": "[y]", "outputs": "[a, b]", "axis": "1"}]
+    w("c1", 16, 16); nodes += conv("c1", "b", "t")
+    nodes += [{"name": "k1", "op_type": "Concat", "inputs": "[a, b, t]", "outputs": "[k]", "axis": "1"}]       # y and t in place
+    w("c2", 48, 16); nodes += conv("c2", "k", "u")
+    nodes += [{"name": "k2", "op_type": "Concat", "inputs": "[x, u, t, u]", "outputs": "[z]", "axis": "1"}]   # only the first u in place
+    return nodes, params
+
+
+def test_concat_parts_in_place():
+    """Which parts of a one-image Concat get their slot inside its result: values produced by an instruction, the
+    value whose Split views are consecutive parts (a C2f block: the views follow it), not the graph input, not a
+    value that already lives in another Concat, not a part that comes twice; what is left is copied by a Concat
+    over its stretch of the result."""
+    nodes, params = _concat_graph()
+    ex = AotExecutor(nodes, params, ["x"], ["z"], {"x": [1, 16, 8, 8]}, quantize=8)
+    names = [i[0] for i in ex.instructions]
+    assert names == ["conv2d_i8", "conv2d_i8", "conv2d_i8", "concat", "concat"], names
+    v = lambda n: ex._values[n].slot
+    part = 16 * 64 * 4
+    assert v("y") == (v("k")[0], 2 * part) and v("a") == (v("k")[0], part) and v("b") == (v("k")[0] + part, part)
+    assert v("t") == (v("k")[0] + 2 * part, part)
+    assert v("u") == (v("z")[0] + part, part)
+    # the two copies: x into the first stretch of z, (t, u) into the last two
+    assert ex._calls[3][1] == [v("x")] and ex._calls[3][2] == (v("z")[0], part)
+    assert ex._calls[4][1] == [v("t"), v("u")] and ex._calls[4][2] == (v("z")[0] + 2 * part, 2 * part)
+    off = AotExecutor(nodes, params, ["x"], ["z"], {"x": [1, 16, 8, 8]}, quantize=8, concat_in_place=False)
+    assert [i[0] for i in off.instructions] == ["conv2d_i8", "conv2d_i8", "concat", "conv2d_i8", "concat"]
 
 
 @pytest.mark.gpu
@@ -135,3 +181,32 @@ def test_forward_conv_graph(orc):
         assert_close(got, want, 1e-5, "conv graph")
     finally:
         ex.close()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("side", [32, 8])
+def test_forward_with_concat_parts_in_place(side):
+    """The same graph with the parts stored in place and with every Concat copying: every value equal bit for bit.
+    The convolution that reads k takes its ranges from the pairs that the producers of k's parts left one after the
+    other (no instruction writes k as a whole), on tiles of the 32 x 32 map and on the single tile of the 8 x 8 map."""
+    nodes, params = _concat_graph()
+    rng = np.random.default_rng(3)
+    x = rng.uniform(-1, 1, (1, 16, side, side)).astype(np.float32)
+    outs = ["z", "k", "u", "t", "y"]
+    got, used = {}, {}
+    for in_place in (True, False):
+        ex = AotExecutor(nodes, params, ["x"], outs, {"x": list(x.shape)}, quantize=8, concat_in_place=in_place)
+        try:
+            first = ex.forward({"x": x})
+            again = ex.forward({"x": x})
+            assert ex.replayed
+            for n in outs:
+                assert np.array_equal(first[n], again[n]), n
+            got[in_place], used[in_place] = again, ex.ranges_used
+        finally:
+            ex.close()
+    for n in outs:
+        assert np.array_equal(got[True][n], got[False][n]), n
+    assert np.array_equal(got[True]["k"], np.concatenate([got[True]["y"], got[True]["t"]], axis=1))
+    assert np.array_equal(got[True]["z"], np.concatenate([x, got[True]["u"], got[True]["t"], got[True]["u"]], axis=1))
+    assert used[False] == 1 and used[True] == 1, used

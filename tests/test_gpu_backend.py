@@ -932,6 +932,66 @@ def test_matmul_followed_by_residual_add_runs_as_one_call(be, orc, wdt, kname):
         assert np.array_equal(view(s), view(s_y[0]) + r)
 
 
+@pytest.mark.parametrize("case", ["parts", "memcopy part", "part without pairs", "part rewritten", "overwritten after", "gap"])
+def test_conv_ranges_collected_part_by_part(be, orc, case):
+    """A one-image tensor that several instructions write part by part (the slot of a Concat result filled in place):
+    each producer leaves its pairs behind those of the parts before it, and the convolution that reads the whole
+    tensor takes them once disjoint parts cover it -- not when a part comes from an instruction that leaves no
+    pairs, is overwritten afterwards, or is missing; a part that is written again before anything reads it counts with
+    its last writer (the first one's values are never read, so it is asked for nothing).  A convolution that reads just
+    one part takes that part's pairs.  Either way the arena equals, bit for bit, the one with every convolution scanning."""
+    rng = np.random.default_rng(31)
+    c, h, w = 16, 32, 32
+    half = (c // 2) * h * w
+    a0 = rng.standard_normal(half).astype(np.float32)
+    a1 = (rng.standard_normal(half) * 3).astype(np.float32)
+    pw = fastnn_amd.quantize_weights(flib.DT_I8, (rng.standard_normal((8, c)) * 0.3).astype(np.float32))
+    ph = fastnn_amd.quantize_weights(flib.DT_I8, (rng.standard_normal((8, c // 2)) * 0.3).astype(np.float32))
+    a = Arena()
+    s_a0, s_a1, s_w, s_wh = a.take(half * 4), a.take(half * 4), a.take(pw.words.nbytes), a.take(ph.words.nbytes)
+    s_t = a.take(2 * half * 4)
+    s_p0, s_p1 = (s_t[0], half * 4), (s_t[0] + half * 4, half * 4)
+    s_y, s_yh = a.take(8 * h * w * 4), a.take(8 * h * w * 4)
+    plan = ExecutablePlan(a.top).write_const(s_w[0], pw.words).write_const(s_wh[0], ph.words)
+    plan.call_kernel("relu_f32", [s_a0], s_p0, [half])
+    if case == "memcopy part":
+        plan.memcopy(s_p1, s_a1)
+    elif case == "part without pairs":
+        plan.fill(s_p1[0], s_p1[1], 0.25)
+    elif case != "gap":
+        plan.call_kernel("silu_f32", [s_a1], s_p1, [half])
+    if case == "part rewritten":
+        plan.call_kernel("gelu_f32", [s_a1], s_p0, [half])
+    if case == "overwritten after":
+        plan.fill(s_p0[0] + 64, 64, 9.0)
+    plan.call_kernel("conv2d_i8", [s_p0, s_wh], s_yh, [1, 0, 1, 1, c // 2, h, w, 1, 1], meta_of(ph, [8, c // 2, 1, 1]))   # reads one part
+    plan.call_kernel("conv2d_i8", [s_t, s_w], s_y, [1, 0, 1, 1, c, h, w, 1, 1], meta_of(pw, [8, c, 1, 1]))               # reads the whole
+    be.allocate_arena(a.top)
+    got, used = {}, {}
+    try:
+        for on in (1, 0):
+            be.set_option(flib.OPT_CONV_RANGES, on)
+            be.write_arena(0, np.zeros(a.top, np.uint8))
+            be.write_arena(s_a0[0], a0)
+            be.write_arena(s_a1[0], a1)
+            be.dispatch(plan)
+            first = be.read_arena(0, a.top).copy()
+            be.dispatch(plan)
+            assert plan.replayed
+            got[on], used[on] = be.read_arena(0, a.top).copy(), plan.ranges_used
+            assert np.array_equal(first, got[on]), "replay differs from the first dispatch"
+    finally:
+        be.set_option(flib.OPT_CONV_RANGES, 1)
+    assert np.array_equal(got[1], got[0])
+    # the reader of the part: its pairs hold unless the Fill wrote into the part; the reader of the whole: only with
+    # both parts from producers that leave pairs and nothing written after them
+    want = {"parts": 2, "memcopy part": 2, "part without pairs": 1, "part rewritten": 2, "overwritten after": 0, "gap": 1}[case]
+    assert used[0] == 0 and used[1] == want, (case, used)
+    t = got[1][s_t[0]:s_t[0] + s_t[1]].view(np.float32).reshape(1, c, h, w)
+    y = got[1][s_y[0]:s_y[0] + s_y[1]].view(np.float32).reshape(1, 8, h, w)
+    assert_close(y, orc.qconv2d_i8(t, to_oracle(orc, pw), 1, 1, 1, 0, 1, 1), 1e-5, case)
+
+
 def test_residual_add_onto_the_matmul_input_stays_an_instruction(be, orc):
     """x = x + MatMul(x) with the sum written over x: workgroups of the MatMul still read x while others would store
     sums, so the Add is not folded into the MatMul's last kernel."""

@@ -298,10 +298,12 @@ def test_conv_activation_ranges_from_the_producing_instruction(orc, batch, size,
     x = rng.uniform(0, 1, shape).astype(np.float32)
     results = {}
     used = {}
-    for on in (1, 0):
-        ex = AotExecutor(nodes, params, ["x"], outs, {"x": shape}, quantize=8)
+    # (2: with the parts of every Concat copied, as the plan of a batch has them anyway; 1 and 0: parts of a
+    # one-image Concat stored in place by their producers, whose pairs then arrive part by part)
+    for on in (1, 0, 2):
+        ex = AotExecutor(nodes, params, ["x"], outs, {"x": shape}, quantize=8, concat_in_place=on != 2)
         try:
-            ex.set_option(flib.OPT_CONV_RANGES, on)
+            ex.set_option(flib.OPT_CONV_RANGES, 1 if on else 0)
             ex.set_option(flib.OPT_CONV_IMPLICIT, implicit)
             first = ex.forward({"x": x})
             again = ex.forward({"x": x})
@@ -315,9 +317,12 @@ def test_conv_activation_ranges_from_the_producing_instruction(orc, batch, size,
         finally:
             ex.close()
     assert used[0] == 0
-    assert used[1] >= 30, used   # every conv but the first has a producer in the plan; the smallest maps fall back
+    # every conv but the first has a producer in the plan; the smallest maps fall back, and a part without pairs
+    # leaves the reader of the whole in-place Concat to its own scan
+    assert used[2] >= 30 and used[1] >= 28, used
     for name in outs:
         assert np.array_equal(results[1][name], results[0][name]), name
+        assert np.array_equal(results[1][name], results[2][name]), name
 
 
 def test_conv_activation_ranges_odd_shapes_and_every_producer(orc):
@@ -446,19 +451,21 @@ def test_random_conv_graphs_equal_under_every_range_and_kernel_choice(seed):
         shape = (b, c0, h, w)
         x = rng.uniform(-1, 1, shape).astype(np.float32)
         res = {}
-        for ranges, implicit, fuse in [(0, 0, 0), (1, 0, 1), (1, 1, 1), (1, 2, 1), (0, 1, 1), (1, 0, 0), (0, 2, 1), (1, 3, 1), (0, 3, 0)]:
-            ex = AotExecutor(nodes, params, ["x"], [cur], {"x": shape}, quantize=8)
+        # (the fourth entry: parts of a one-image Concat stored in place by their producers, or copied by the Concat)
+        for ranges, implicit, fuse, in_place in [(0, 0, 0, 0), (1, 0, 1, 1), (1, 1, 1, 1), (1, 2, 1, 0), (0, 1, 1, 1), (1, 0, 0, 1), (0, 2, 1, 1),
+                                                 (1, 3, 1, 0), (0, 3, 0, 1), (1, 0, 1, 0)]:
+            ex = AotExecutor(nodes, params, ["x"], [cur], {"x": shape}, quantize=8, concat_in_place=bool(in_place))
             try:
                 ex.set_option(flib.OPT_CONV_RANGES, ranges)
                 ex.set_option(flib.OPT_CONV_IMPLICIT, implicit)
                 ex.set_option(flib.OPT_FUSE_RESIDUAL, fuse)   # (the Add behind a convolution rides in its epilogue)
                 first = ex.forward({"x": x})[cur]
                 again = ex.forward({"x": x})[cur]
-                assert np.array_equal(first, again), (case, ranges, implicit, fuse, "replay differs from the first dispatch")
+                assert np.array_equal(first, again), (case, ranges, implicit, fuse, in_place, "replay differs from the first dispatch")
                 assert ranges or ex.ranges_used == 0
                 assert fuse or ex.residuals_fused == 0
-                res[(ranges, implicit, fuse)] = again
+                res[(ranges, implicit, fuse, in_place)] = again
             finally:
                 ex.close()
         for key, val in res.items():
-            assert np.array_equal(val, res[(0, 0, 0)]), (case, key, shape, len(nodes))
+            assert np.array_equal(val, res[(0, 0, 0, 0)]), (case, key, shape, len(nodes))
