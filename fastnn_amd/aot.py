@@ -122,9 +122,11 @@ class AotExecutor:
             self._consts: List[tuple] = []          # (offset, array)
             self._calls: List[tuple] = []           # (kernel, [slots], slot, params, meta)
             self._reserved = {}
+            self._split_of: Dict[str, tuple] = {}   # copied Split part -> (source, axis, first index, indices, source's size along axis)
             for n in self.input_names:
                 self._new_value(n, shapes[n])
             self._lower([dict(n) for n in nodes])
+            self._drop_unread()
             if lowering == 1 or not concat_in_place:
                 break
             self._placement = self._place_concat_parts([dict(n) for n in nodes])
@@ -161,6 +163,41 @@ class AotExecutor:
         v = _Value(shape, self._slot_for(name, int(np.prod(shape, dtype=np.int64)) * 4))
         self._values[name] = v
         return v
+
+    def _drop_unread(self):
+        """Instructions whose result nothing reads (no later instruction, no view of it, not a graph output) are
+        taken out: the copy of a Split part that only a Concat wanted, once that Concat reads the Split's source."""
+        inside: Dict[str, list] = {}     # Concat result -> the values stored in place inside it
+        for child, (parent, _) in self._placement.items():
+            inside.setdefault(parent, []).append(child)
+        needed = set()
+
+        def need(name):
+            name = self._root_of(name)[0]
+            if name not in needed:
+                needed.add(name)
+                for child in inside.get(name, []):
+                    if child in self._values:
+                        need(child)
+
+        for n in self.output_names:
+            if n in self._values:
+                need(n)
+        keep = [False] * len(self.instructions)
+        for idx in range(len(self.instructions) - 1, -1, -1):
+            _, ins, out, _ = self.instructions[idx]
+            if out in needed:
+                keep[idx] = True
+                for i in ins:
+                    if i in self._values:
+                        need(i)
+        self._dropped = set(x[2] for x, k in zip(self.instructions, keep) if not k)
+        self.instructions = [x for x, k in zip(self.instructions, keep) if k]
+        self._calls = [x for x, k in zip(self._calls, keep) if k]
+
+    def kept(self, name: str) -> bool:
+        """False for a value that no instruction of the plan writes (nothing reads it and it is no output)."""
+        return name in self._values and name not in self._dropped
 
     def _root_of(self, name: str):
         """(value that owns the slot `name` lives in, byte offset of `name` inside it)."""
@@ -271,11 +308,29 @@ class AotExecutor:
                 out = self._new_value(outs[0], (n, c, ho, wo))
                 self._emit("pool_f32", ins, outs[0], [a.slot], out.slot, [k, s, p, 1 if op == "MaxPool" else 0, n, c, h, w])
             elif op == "Concat":
-                vals = [self._val(i) for i in ins]
-                rank = len(vals[0].shape)
+                rank = len(self._val(ins[0]).shape)
                 axis = _attr_int(nd, "axis", default=0)
                 axis = axis + rank if axis < 0 else axis
                 axis = min(max(axis, 0), rank - 1)
+                # consecutive parts that are, in order, ALL the copied parts of one Split along this axis: the Split's
+                # source is read instead (the copies of parts that nothing else reads are then dropped)
+                merged, i = [], 0
+                while i < len(ins):
+                    sp = self._split_of.get(ins[i])
+                    if sp and sp[1] == axis and sp[2] == 0:
+                        j, at = i, 0
+                        while j < len(ins) and self._split_of.get(ins[j], (None,))[0] == sp[0] and self._split_of[ins[j]][1] == axis and \
+                                self._split_of[ins[j]][2] == at:
+                            at += self._split_of[ins[j]][3]
+                            j += 1
+                        if at == sp[4]:
+                            merged.append(sp[0])
+                            i = j
+                            continue
+                    merged.append(ins[i])
+                    i += 1
+                ins = merged
+                vals = [self._val(i) for i in ins]
                 shape = list(vals[0].shape)
                 shape[axis] = sum(v.shape[axis] for v in vals)
                 out = self._new_value(outs[0], shape)
@@ -326,6 +381,7 @@ class AotExecutor:
                     else:
                         out = self._new_value(o, shape)
                         self._emit("slice_f32", ins, o, [a.slot], out.slot, [axis, start, start + sz, inner])
+                        self._split_of[o] = (ins[0], axis, start, sz, a.shape[axis])
                     start += sz
             elif op == "Resize":
                 a = self._val(ins[0])
@@ -517,6 +573,9 @@ class AotExecutor:
         self._backend.dispatch(self._plan)
 
     def read_output(self, name: str) -> np.ndarray:
+        """A graph output, or any other value the plan computes (every value keeps its slot)."""
+        if name in self._dropped:
+            raise FnnError(4, f"AotExecutor: '{name}' is not computed: nothing reads it; name it in output_names to keep it")
         v = self._values[name]
         return self._backend.read_arena(*v.slot, np.float32).reshape(v.shape).copy()
 

@@ -183,6 +183,21 @@ def test_forward_conv_graph(orc):
         ex.close()
 
 
+def test_concat_of_all_split_parts_reads_the_split_source():
+    """A batch of two: the parts of a channel Split are copies.  A Concat that joins all of them, in order, reads the
+    Split's input instead, and the copy of a part that nothing else reads is not made (reading it says so)."""
+    nodes, params = _concat_graph()
+    ex = AotExecutor(nodes, params, ["x"], ["z"], {"x": [2, 16, 8, 8]}, quantize=8)
+    names = [(i[0], i[1], i[2]) for i in ex.instructions]
+    assert names == [("conv2d_i8", ["x", "wc0"], "y"), ("slice_f32", ["y"], "b"), ("conv2d_i8", ["b", "wc1"], "t"),
+                     ("concat", ["y", "t"], "k"), ("conv2d_i8", ["k", "wc2"], "u"), ("concat", ["x", "u", "t", "u"], "z")], names
+    assert ex.kept("b") and not ex.kept("a")
+    with pytest.raises(flib.FnnError):
+        ex.read_output("a")
+    keep_a = AotExecutor(nodes, params, ["x"], ["z", "a"], {"x": [2, 16, 8, 8]}, quantize=8)
+    assert [i[0] for i in keep_a.instructions].count("slice_f32") == 2 and keep_a.kept("a")
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("side", [32, 8])
 def test_forward_with_concat_parts_in_place(side):
