@@ -161,7 +161,8 @@ struct fnn_backend {
     // `slice` are exactly what the table describes, and lasts until something writes into the slice or the dispatch
     // pass ends.
     struct RangeTable { float *dev = nullptr; uint64_t images = 0; };
-    struct LiveRange { fnn_slice slice; const float *table; int parts; uint64_t image_elems, images; };
+    // (tile_elems > 0: the pairs come in groups of tile_pairs, one group per tile_elems values of the slice, in order)
+    struct LiveRange { fnn_slice slice; const float *table; int parts; uint64_t image_elems, images; uint64_t tile_elems = 0; int tile_pairs = 0; };
     // A one-image tensor that several instructions write part by part (producers that store straight into the slot of
     // a later Concat's result): each leaves its pairs behind those of the parts before it; the entry becomes a live
     // range once disjoint parts cover the whole slice, and is void as soon as anything else writes into it.
@@ -776,6 +777,7 @@ void request_ranges(fnn_backend *b, fnn_plan *p, size_t idx, fnn_slice *covered,
     *pending = -1;
     if (!in.dst.size) return;
     size_t exact = (size_t)-1, whole = (size_t)-1;
+    bool some = false;   // a convolution of one image reads some of what `idx` writes (one half of a Split that is a view)
     ConvInput ce{0, 0}, cw{0, 0};
     for (size_t j = idx + 1; j < p->instrs.size() && whole == (size_t)-1; j++) {
         const Instr &nx = p->instrs[j];
@@ -785,9 +787,12 @@ void request_ranges(fnn_backend *b, fnn_plan *p, size_t idx, fnn_slice *covered,
             if (exact == (size_t)-1 && cs.offset == in.dst.offset && cs.size <= in.dst.size && cj.images <= 65535) { exact = j; ce = cj; }
             if (cj.images == 1 && in.dst.size % 4 == 0 && in.dst.size < cs.size && in.dst.offset >= cs.offset &&
                 in.dst.offset + in.dst.size <= cs.offset + cs.size) { whole = j; cw = cj; }
+            if (cj.images == 1 && cs.size < in.dst.size && cs.offset >= in.dst.offset && cs.offset + cs.size <= in.dst.offset + in.dst.size) some = true;
         }
         if (overlaps(nx.dst, in.dst) || (nx.has_secondary && overlaps(nx.secondary, in.dst))) break;
     }
+    // (a reader of the first bytes only is served like any reader of some of them)
+    if (exact != (size_t)-1 && ce.images == 1 && ce.image_elems * 4 < in.dst.size) exact = (size_t)-1;
     if (whole != (size_t)-1 && (exact == (size_t)-1 || ce.images == 1)) {
         const fnn_slice &cs = p->instrs[whole].inputs[0];
         int at = -1;
@@ -819,6 +824,13 @@ void request_ranges(fnn_backend *b, fnn_plan *p, size_t idx, fnn_slice *covered,
             rio->out_image_elems = ce.image_elems; rio->out_images = ce.images;
             *covered = p->instrs[exact].inputs[0];
         }
+    } else if (some && in.dst.size % 4 == 0) {
+        // the whole result as one image: a producer that groups its pairs by channel block serves the readers of blocks
+        if (float *t = range_table(b, p, {p->uid, idx}, 1)) {
+            rio->out_table = t; rio->out_stride = kRangeStride;
+            rio->out_image_elems = in.dst.size / 4; rio->out_images = 1;
+            *covered = in.dst;
+        }
     }
 }
 
@@ -829,7 +841,8 @@ void note_ranges(fnn_backend *b, const fnn_slice &covered, int pending)
         auto &pr = b->pending_ranges[(size_t)pending];
         if (!rio->out_table || rio->out_failed || rio->out_parts <= pr.parts) { pr.failed = true; return; }
         // the part's own pairs describe it to a convolution that reads just the part
-        b->live_ranges.push_back(fnn_backend::LiveRange{covered, pr.table + 2 * (size_t)pr.parts, rio->out_parts - pr.parts, covered.size / 4, 1});
+        b->live_ranges.push_back(fnn_backend::LiveRange{covered, pr.table + 2 * (size_t)pr.parts, rio->out_parts - pr.parts, covered.size / 4, 1,
+                                                        rio->out_tile_elems, rio->out_tile_pairs});
         pr.parts = rio->out_parts;
         pr.written.push_back(covered);
         uint64_t bytes = 0;
@@ -841,7 +854,8 @@ void note_ranges(fnn_backend *b, const fnn_slice &covered, int pending)
         return;
     }
     if (rio->out_table && rio->out_parts > 0 && !rio->out_failed)
-        b->live_ranges.push_back(fnn_backend::LiveRange{covered, rio->out_table, rio->out_parts, rio->out_image_elems, rio->out_images});
+        b->live_ranges.push_back(fnn_backend::LiveRange{covered, rio->out_table, rio->out_parts, rio->out_image_elems, rio->out_images,
+                                                        rio->out_images == 1 ? rio->out_tile_elems : 0, rio->out_tile_pairs});
 }
 
 int run_call_with_ranges(fnn_backend *b, fnn_plan *p, size_t idx)
@@ -860,10 +874,23 @@ int run_call_with_ranges(fnn_backend *b, fnn_plan *p, size_t idx)
     // consumer: a convolution whose input slice is described by a live table
     ConvInput ci;
     if (ranged_conv_input(in, &ci)) {
+        const fnn_slice &xs = in.inputs[0];
         for (const auto &r : b->live_ranges)
-            if (r.slice.offset == in.inputs[0].offset && r.slice.size == in.inputs[0].size && r.image_elems == ci.image_elems &&
-                r.images == ci.images) {
+            if (r.slice.offset == xs.offset && r.slice.size == xs.size && r.image_elems == ci.image_elems && r.images == ci.images) {
                 rio->in_table = r.table; rio->in_stride = kRangeStride; rio->in_parts = r.parts;
+                break;
+            }
+        // ... or whole channel blocks of a one-image tensor whose producer grouped its pairs by channel block (one half
+        // of a Split that is a view into the convolution output it splits)
+        if (!rio->in_table && ci.images == 1)
+            for (const auto &r : b->live_ranges) {
+                const uint64_t tb = r.tile_elems * 4;
+                if (r.images != 1 || tb == 0 || r.tile_pairs <= 0 || xs.offset < r.slice.offset || xs.offset + xs.size > r.slice.offset + r.slice.size) continue;
+                const uint64_t at = xs.offset - r.slice.offset;
+                if (at % tb || xs.size % tb || xs.size != ci.image_elems * 4) continue;
+                const uint64_t t0 = at / tb, nt = xs.size / tb;
+                if ((t0 + nt) * (uint64_t)r.tile_pairs > (uint64_t)r.parts) continue;
+                rio->in_table = r.table + 2 * t0 * (uint64_t)r.tile_pairs; rio->in_stride = kRangeStride; rio->in_parts = (int)(nt * (uint64_t)r.tile_pairs);
                 break;
             }
     }

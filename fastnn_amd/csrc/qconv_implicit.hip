@@ -20,6 +20,7 @@ struct ImplicitArgs {
     QConvArgs a;
     ConvDivs dv;
     int g, kk, vec4;
+    int rng_blocks;   // conv_fused_kernel: > 1 = that many channel blocks, one per wave, each with its own range pairs
 };
 
 constexpr int TAP_TABLE = 2048;   // taps (K rounded up to whole steps of 32) whose geometry is tabulated once per workgroup
@@ -477,18 +478,19 @@ __global__ void __launch_bounds__(64 * PW * KW, TAB ? 4 : 2) conv_implicit_kerne
             constexpr uint32_t BM = 32 * PW;
             const uint32_t row_z = (uint32_t)(r_first + BM - 1 < rows ? r_first + BM - 1 : rows - 1);
             const uint32_t img_end = (nn0 + 1) * np - 1;
-            const int nt = (int)blockIdx.y, ntiles = (int)gridDim.y;
+            const int nt = (int)blockIdx.y;
             const int slot = (int)(blockIdx.x - (nn0 * np) / BM), per_m = (int)(np / BM) + 2;
             const int fill = row_z >= img_end ? slot + 1 : per_m;
-            float *row = a.range_out + (int64_t)nn0 * a.range_out_stride * 2;
-            float *dst = row + ((int64_t)slot * ntiles + nt) * 2;
+            // (the pairs of a channel block lie together: a reader of some of the channels takes its blocks' pairs)
+            float *row = a.range_out + (int64_t)nn0 * a.range_out_stride * 2 + (int64_t)nt * per_m * 2;
+            float *dst = row + (int64_t)slot * 2;
             dst[0] = mn0; dst[1] = mx0;
             if (rng_two) {   // the next image starts in this block: its pair 0
-                float *d1 = row + ((int64_t)a.range_out_stride + nt) * 2;
+                float *d1 = row + (int64_t)a.range_out_stride * 2;
                 d1[0] = mn1; d1[1] = mx1;
             }
             for (int j = fill; j < per_m; j++) {
-                float *d2 = row + ((int64_t)j * ntiles + nt) * 2;
+                float *d2 = row + (int64_t)j * 2;
                 d2[0] = INFINITY; d2[1] = -INFINITY;
             }
         }
@@ -849,8 +851,9 @@ __global__ void __launch_bounds__(256) conv_fused_kernel(ImplicitArgs p)
     }
     if constexpr (RNG) {
         if (r_first >= rows) return;   // (workgroup-uniform)
-        // one pair per workgroup (block of 32 pixels, all channels): pair (block - first block of the image) of every
-        // image the block meets, np / 32 + 2 pairs per image; the waves leave theirs in LDS, the last to arrive writes
+        // one pair per workgroup (block of 32 pixels) and channel group: pair (block - first block of the image) of
+        // every image the block meets, np / 32 + 2 pairs per image and group; the waves leave theirs in LDS, the last to
+        // arrive writes
         mn0 = wave_min(mn0); mx0 = wave_max(mx0);
         if (rng_two) { mn1 = wave_min(mn1); mx1 = wave_max(mx1); }
         int arrived = 0;
@@ -861,27 +864,35 @@ __global__ void __launch_bounds__(256) conv_fused_kernel(ImplicitArgs p)
             __threadfence_block();
         }
         if (lane == 0 && arrived == NW - 1) {
-            mn0 = s_rng[0][0]; mx0 = s_rng[0][1]; mn1 = s_rng[0][2]; mx1 = s_rng[0][3];
-#pragma unroll
-            for (int w2 = 1; w2 < NW; w2++) {
-                mn0 = fminf(mn0, s_rng[w2][0]); mx0 = fmaxf(mx0, s_rng[w2][1]);
-                mn1 = fminf(mn1, s_rng[w2][2]); mx1 = fmaxf(mx1, s_rng[w2][3]);
-            }
             constexpr uint32_t BM = 32;
             const uint32_t row_z = (uint32_t)(r_first + BM - 1 < rows ? r_first + BM - 1 : rows - 1);
             const uint32_t img_end = (nn0 + 1) * np - 1;
             const int slot = (int)(blockIdx.x - (nn0 * np) / BM), per_m = (int)(np / BM) + 2;
             const int fill = row_z >= img_end ? slot + 1 : per_m;
-            float *row = a.range_out + (int64_t)nn0 * a.range_out_stride * 2;
-            float *dst = row + (int64_t)slot * 2;
-            dst[0] = mn0; dst[1] = mx0;
-            if (rng_two) {   // the next image starts in this block: its pair 0
-                float *d1 = row + (int64_t)a.range_out_stride * 2;
-                d1[0] = mn1; d1[1] = mx1;
-            }
-            for (int j = fill; j < per_m; j++) {
-                float *d2 = row + (int64_t)j * 2;
-                d2[0] = INFINITY; d2[1] = -INFINITY;
+            // p.rng_blocks > 1 (at most one channel block per wave): wave w's pair is that of channel block w, and the
+            // pairs of a block lie together (a reader of some of the channels takes its blocks' pairs); else one pair
+            // for all channels
+            const int groups = p.rng_blocks > 1 ? p.rng_blocks : 1;
+            for (int gq = 0; gq < groups; gq++) {
+                float m0 = s_rng[gq][0], x0 = s_rng[gq][1], m1 = s_rng[gq][2], x1 = s_rng[gq][3];
+                if (groups == 1) {
+#pragma unroll
+                    for (int w2 = 1; w2 < NW; w2++) {
+                        m0 = fminf(m0, s_rng[w2][0]); x0 = fmaxf(x0, s_rng[w2][1]);
+                        m1 = fminf(m1, s_rng[w2][2]); x1 = fmaxf(x1, s_rng[w2][3]);
+                    }
+                }
+                float *row = a.range_out + (int64_t)nn0 * a.range_out_stride * 2 + (int64_t)gq * per_m * 2;
+                float *dst = row + (int64_t)slot * 2;
+                dst[0] = m0; dst[1] = x0;
+                if (rng_two) {   // the next image starts in this block: its pair 0
+                    float *d1 = row + (int64_t)a.range_out_stride * 2;
+                    d1[0] = m1; d1[1] = x1;
+                }
+                for (int j = fill; j < per_m; j++) {
+                    float *d2 = row + (int64_t)j * 2;
+                    d2[0] = INFINITY; d2[1] = -INFINITY;
+                }
             }
         }
     }
@@ -1027,9 +1038,20 @@ int fnn_i8_implicit_conv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *
     ia.vec4 = (np % 4 == 0 && (reinterpret_cast<uintptr_t>(p.y) & 15) == 0 && (!p.acc_out || (reinterpret_cast<uintptr_t>(p.acc_out) & 15) == 0) &&
                (!with_sum || ((reinterpret_cast<uintptr_t>(p.residual) | reinterpret_cast<uintptr_t>(p.sum_out)) & 15) == 0)) ? 1 : 0;
     if (form == 2) wg_rows = 32;
-    const int64_t parts = (np / wg_rows + 2) * (form == 2 ? 1 : (ocg + tn * 32 - 1) / (tn * 32));
-    if (p.range_out && p.groups == 1 && np >= wg_rows && parts <= p.range_out_stride) fnn_ctx_range_io(ctx)->out_parts = (int)parts;
-    else ia.a.range_out = nullptr;
+    // range pairs: per channel block (of the implicit form's column tiles; of the fused form's waves when every wave
+    // has at most one block), np / wg_rows + 2 pairs per image and block
+    const int block_ch = form == 2 ? (ocg > 128 ? 64 : 32) : tn * 32;
+    const int64_t nblocks = (ocg + block_ch - 1) / block_ch;
+    ia.rng_blocks = (form == 2 && nblocks <= 4) ? (int)nblocks : 1;
+    const int64_t groups_of_pairs = form == 2 ? ia.rng_blocks : nblocks;
+    const int64_t parts = (np / wg_rows + 2) * groups_of_pairs;
+    if (p.range_out && p.groups == 1 && np >= wg_rows && parts <= p.range_out_stride) {
+        FnnRangeIo *rio = fnn_ctx_range_io(ctx);
+        rio->out_parts = (int)parts;
+        if (groups_of_pairs == nblocks) { rio->out_tile_elems = (uint64_t)block_ch * (uint64_t)np; rio->out_tile_pairs = (int)(np / wg_rows + 2); }
+    } else {
+        ia.a.range_out = nullptr;
+    }
     for (int g = 0; g < p.groups; g++) {
         ia.g = g;
         hipError_t e;

@@ -836,7 +836,10 @@ int fnn_i8_tiled_conv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w, 
             const int64_t parts = (np / bm + 2) * ntl;
             if (p.range_out && p.groups == 1 && np >= bm && parts <= p.range_out_stride) {
                 cv.cv.range_out = p.range_out; cv.cv.range_stride = p.range_out_stride;
-                fnn_ctx_range_io(ctx)->out_parts = (int)parts;
+                FnnRangeIo *rio = fnn_ctx_range_io(ctx);
+                rio->out_parts = (int)parts;
+                rio->out_tile_elems = (uint64_t)(small_tiles || ocg <= 64 ? 64 : 128) * (uint64_t)np;   // (the pairs of a column tile lie together)
+                rio->out_tile_pairs = (int)(np / bm + 2);
             }
         }
         if (e == hipSuccess)

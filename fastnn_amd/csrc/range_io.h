@@ -20,6 +20,11 @@ struct FnnRangeIo {
     int out_parts = 0;        // pairs per image in place: a call appends behind them (a tensor written by several calls,
                               // e.g. the parts of a concat) and adds what it wrote; 0 after a single call: none
     int out_failed = 0;       // answer: a call wrote values of the tensor without leaving their ranges
+    // answer of a convolution: the pairs it left are grouped by blocks of output channels, out_tile_pairs pairs per
+    // block and image, block after block; a block is out_tile_elems values of an image (channels x pixels).  A reader
+    // of whole blocks of a ONE-image tensor takes just their pairs.  0: not grouped
+    uint64_t out_tile_elems = 0;
+    int out_tile_pairs = 0;
     // offer to the next quantised Conv2d: partial ranges of its input, one image per batch entry
     const float *in_table = nullptr;
     int in_stride = 0, in_parts = 0;

@@ -43,7 +43,7 @@ struct TileArgs {
         int vec4;                  // np % 4 == 0 and 16-byte aligned outputs: four pixels per store
         // non-null (only with np >= rows of a tile, so that a tile meets at most two images): partial (min, max)
         // pairs of the values this launch stores, [image][range_stride][2]; the tile (mt, nt) fills pair
-        // (mt - first tile of the image) * ntiles + nt of every image it meets, (np / BM + 2) * ntiles pairs per image
+        // nt * (np / BM + 2) + (mt - first tile of the image) of every image it meets, (np / BM + 2) * ntiles pairs per image
         float *range_out;
         int range_stride;
         // non-null: sum_out = y + residual as well (same layout as y); range_out then describes the sums
@@ -743,15 +743,16 @@ __global__ void __launch_bounds__(WGM * WGN * 64) qgemm_tile_kernel(TileArgs p)
                     mn0 = fminf(mn0, cv_red[w2][0]); mx0 = fmaxf(mx0, cv_red[w2][1]);
                     mn1 = fminf(mn1, cv_red[w2][2]); mx1 = fmaxf(mx1, cv_red[w2][3]);
                 }
-                float *row = p.cv.range_out + (int64_t)rng_img * p.cv.range_stride * 2;
-                float *dst = row + ((int64_t)rng_slot * p.ntiles + nt) * 2;
+                // (the pairs of a column tile lie together: a reader of some of the channels takes its tiles' pairs)
+                float *row = p.cv.range_out + (int64_t)rng_img * p.cv.range_stride * 2 + (int64_t)nt * rng_per_m * 2;
+                float *dst = row + (int64_t)rng_slot * 2;
                 dst[0] = mn0; dst[1] = mx0;
                 if (rng_two) {   // the next image starts in this tile: its pair 0
-                    float *d1 = row + ((int64_t)p.cv.range_stride + nt) * 2;
+                    float *d1 = row + (int64_t)p.cv.range_stride * 2;
                     d1[0] = mn1; d1[1] = mx1;
                 }
                 for (int j = rng_fill; j < rng_per_m; j++) {   // the image of the first row ends here: its unused pairs
-                    float *d2 = row + ((int64_t)j * p.ntiles + nt) * 2;
+                    float *d2 = row + (int64_t)j * 2;
                     d2[0] = INFINITY; d2[1] = -INFINITY;
                 }
             }

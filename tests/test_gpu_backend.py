@@ -992,6 +992,60 @@ def test_conv_ranges_collected_part_by_part(be, orc, case):
     assert_close(y, orc.qconv2d_i8(t, to_oracle(orc, pw), 1, 1, 1, 0, 1, 1), 1e-5, case)
 
 
+@pytest.mark.parametrize("implicit", [0, 1, 2, 3])
+@pytest.mark.parametrize("oc,side", [(64, 40), (128, 20), (256, 20), (32, 48)])
+def test_conv_ranges_of_a_channel_half(be, orc, implicit, oc, side):
+    """The two halves of a one-image convolution output read in place by two convolutions (a Split that is a view):
+    the producer groups its range pairs by channel block, so a reader of whole blocks takes just their pairs instead of
+    scanning -- where a half is whole blocks of the kernel form that ran; either way the arena equals the one with
+    every convolution scanning."""
+    rng = np.random.default_rng(41 + oc)
+    c, h, w = 16, side, side
+    x = rng.uniform(-1, 1, (1, c, h, w)).astype(np.float32)
+    pw = fastnn_amd.quantize_weights(flib.DT_I8, (rng.standard_normal((oc, c)) * 0.3).astype(np.float32))
+    bias = (rng.standard_normal(oc) * 0.1).astype(np.float32)
+    ph = [fastnn_amd.quantize_weights(flib.DT_I8, (rng.standard_normal((8, oc // 2)) * 0.2).astype(np.float32)) for _ in range(2)]
+    a = Arena()
+    s_x, s_w, s_b = a.take(x.nbytes), a.take(pw.words.nbytes), a.take(bias.nbytes)
+    s_wh = [a.take(p.words.nbytes) for p in ph]
+    s_y = a.take(oc * h * w * 4)
+    half = (oc // 2) * h * w * 4
+    s_h = [(s_y[0], half), (s_y[0] + half, half)]
+    s_o = [a.take(8 * h * w * 4) for _ in range(2)]
+    plan = ExecutablePlan(a.top).write_const(s_w[0], pw.words).write_const(s_b[0], bias)
+    for k in range(2):
+        plan.write_const(s_wh[k][0], ph[k].words)
+    plan.call_kernel("conv2d_i8_silu", [s_x, s_w, s_b], s_y, [1, 0, 1, 1, c, h, w, 1, 1], meta_of(pw, [oc, c, 1, 1]))
+    for k in range(2):
+        plan.call_kernel("conv2d_i8", [s_h[k], s_wh[k]], s_o[k], [1, 0, 1, 1, oc // 2, h, w, 1, 1], meta_of(ph[k], [8, oc // 2, 1, 1]))
+    be.allocate_arena(a.top)
+    be.write_arena(s_x[0], x)
+    got, used = {}, {}
+    try:
+        be.set_option(flib.OPT_CONV_IMPLICIT, implicit)
+        for on in (1, 0):
+            be.set_option(flib.OPT_CONV_RANGES, on)
+            be.dispatch(plan)
+            first = be.read_arena(0, a.top).copy()
+            be.dispatch(plan)
+            assert plan.replayed
+            got[on], used[on] = be.read_arena(0, a.top).copy(), plan.ranges_used
+            assert np.array_equal(first, got[on]), "replay differs from the first dispatch"
+    finally:
+        be.set_option(flib.OPT_CONV_RANGES, 1)
+        be.set_option(flib.OPT_CONV_IMPLICIT, 0)
+    assert np.array_equal(got[1], got[0])
+    assert used[0] == 0 and used[1] in (0, 2), used
+    # the fused kernel has blocks of 32 channels (64 from 129 channels on), the tiles of the GEMM pair 64 or 128
+    if (implicit == 3 and oc >= 64) or (implicit == 2 and oc >= 128):
+        assert used[1] == 2, used
+    y = got[1][s_y[0]:s_y[0] + s_y[1]].view(np.float32).reshape(1, oc, h, w)
+    for k in range(2):
+        o = got[1][s_o[k][0]:s_o[k][0] + s_o[k][1]].view(np.float32).reshape(1, 8, h, w)
+        part = np.ascontiguousarray(y[:, k * (oc // 2):(k + 1) * (oc // 2)])
+        assert_close(o, orc.qconv2d_i8(part, to_oracle(orc, ph[k]), 1, 1, 1, 0, 1, 1), 1e-5, f"half {k}")
+
+
 def test_residual_add_onto_the_matmul_input_stays_an_instruction(be, orc):
     """x = x + MatMul(x) with the sum written over x: workgroups of the MatMul still read x while others would store
     sums, so the Add is not folded into the MatMul's last kernel."""
