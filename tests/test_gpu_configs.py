@@ -397,7 +397,7 @@ def test_conv_activation_ranges_odd_shapes_and_every_producer(orc):
         assert np.array_equal(results[1][name], results[0][name]), name
 
 
-@pytest.mark.parametrize("seed", [21, 22])
+@pytest.mark.parametrize("seed", [21, 22, 23])
 def test_random_conv_graphs_equal_under_every_range_and_kernel_choice(seed):
     """Random graphs of 3 x 3 / 1 x 1 / strided convolutions with MaxPool, Resize, residual Add, ReLU and Concat
     between them (batch 1-3, maps of 9-40 pixels a side, 8-96 channels): the output of the plan is the same, bit for
@@ -425,7 +425,7 @@ def test_random_conv_graphs_equal_under_every_range_and_kernel_choice(seed):
 
         cur, cc, ch, cw = "x", c0, h, w
         for _ in range(int(rng.integers(3, 8))):
-            kind = rng.choice(["conv3", "conv1", "conv3s2", "pool", "up", "res", "relu", "cat"], p=[0.3, 0.2, 0.1, 0.08, 0.07, 0.1, 0.05, 0.1])
+            kind = rng.choice(["conv3", "conv1", "conv3s2", "pool", "up", "res", "relu", "cat", "c2f"], p=[0.25, 0.2, 0.1, 0.08, 0.07, 0.1, 0.05, 0.08, 0.07])
             if kind in ("conv3", "conv1", "conv3s2"):
                 oc, k = int(rng.choice([8, 16, 24, 40, 64, 96])), (1 if kind == "conv1" else 3)
                 s = 2 if kind == "conv3s2" and min(ch, cw) >= 8 else 1
@@ -451,6 +451,14 @@ def test_random_conv_graphs_equal_under_every_range_and_kernel_choice(seed):
                 t, y = conv(cur, cc, 8, 1, 1, 0), uid("k")
                 nodes.append({"name": y, "op_type": "Concat", "inputs": f"[{cur}, {t}]", "outputs": f"[{y}]", "axis": "1"})
                 cur, cc = y, cc + 8
+            elif kind == "c2f":   # conv, channel Split, a residual block on the second half, Concat of the halves and the sum
+                oc = int(rng.choice([16, 32, 64, 128]))
+                y0, ha, hb, r, y = conv(cur, cc, oc, 1, 1, 0), uid("h"), uid("h"), uid("a"), uid("k")
+                nodes.append({"name": uid("sp"), "op_type": "Split", "inputs": f"[{y0}]", "outputs": f"[{ha}, {hb}]", "axis": "1"})
+                t = conv(conv(hb, oc // 2, oc // 2, 3, 1, 1), oc // 2, oc // 2, 3, 1, 1)
+                nodes.append({"name": r, "op_type": "Add", "inputs": f"[{hb}, {t}]", "outputs": f"[{r}]"})
+                nodes.append({"name": y, "op_type": "Concat", "inputs": f"[{ha}, {hb}, {r}]", "outputs": f"[{y}]", "axis": "1"})
+                cur, cc = y, oc + oc // 2
         cur = conv(cur, cc, 8, 3, 1, 1)
         shape = (b, c0, h, w)
         x = rng.uniform(-1, 1, shape).astype(np.float32)
