@@ -1042,7 +1042,7 @@ int fnn_i8_implicit_conv(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *
     // has at most one block), np / wg_rows + 2 pairs per image and block
     const int block_ch = form == 2 ? (ocg > 128 ? 64 : 32) : tn * 32;
     const int64_t nblocks = (ocg + block_ch - 1) / block_ch;
-    ia.rng_blocks = (form == 2 && nblocks <= 4) ? (int)nblocks : 1;
+    ia.rng_blocks = (form == 2 && nblocks <= 4 && (np / wg_rows + 2) * nblocks <= p.range_out_stride) ? (int)nblocks : 1;   // (else one pair for all channels)
     const int64_t groups_of_pairs = form == 2 ? ia.rng_blocks : nblocks;
     const int64_t parts = (np / wg_rows + 2) * groups_of_pairs;
     if (p.range_out && p.groups == 1 && np >= wg_rows && parts <= p.range_out_stride) {
