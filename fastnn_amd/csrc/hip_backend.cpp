@@ -907,8 +907,9 @@ int run_call_with_ranges(fnn_backend *b, fnn_plan *p, size_t idx)
     if (for_sum) drop_ranges_overlapping(b, p->instrs[idx + 1].dst, pending);
     const int st = run_call(b, in);
     if (st == FNN_OK && rio->in_used) p->ranges_used++;
+    // (a convolution that did not take the Add along has written nothing into the sum's slot: the Add runs next and
+    // leaves the sum's pairs itself)
     if (st == FNN_OK && (!for_sum || res->used)) note_ranges(b, covered, pending);
-    else if (pending >= 0) b->pending_ranges[(size_t)pending].failed = true;
     *rio = FnnRangeIo{};
     return st;
 }
