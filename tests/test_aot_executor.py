@@ -113,6 +113,35 @@ def _concat_graph():
     return nodes, params
 
 
+def _nested_concat_graph():
+    """Concat results inside Concat results: k1 = (pa, pb), k2 = (k1, pc), z = (k2, pool(k2), pa)."""
+    rng = np.random.default_rng(4)
+    params = {}
+    def conv(name, x, y, c, oc):
+        params["w" + name] = (rng.standard_normal((oc, c, 1, 1)) * 0.3).astype(np.float32)
+        return {"name": name, "op_type": "Conv", "inputs": f"[{x}, w{name}]", "outputs": f"[{y}]", "strides": "1", "pads": "0"}
+    nodes = [conv("a", "x", "pa", 16, 16), conv("b", "x", "pb", 16, 16),
+             {"name": "k1", "op_type": "Concat", "inputs": "[pa, pb]", "outputs": "[k1]", "axis": "1"},
+             conv("c", "k1", "pc", 32, 16),
+             {"name": "k2", "op_type": "Concat", "inputs": "[k1, pc]", "outputs": "[k2]", "axis": "1"},
+             {"name": "p", "op_type": "MaxPool", "inputs": "[k2]", "outputs": "[m]", "kernel_shape": "5", "strides": "1", "pads": "2"},
+             {"name": "k3", "op_type": "Concat", "inputs": "[k2, m, pa]", "outputs": "[z]", "axis": "1"}]
+    return nodes, params
+
+
+def test_nested_concat_parts_in_place():
+    nodes, params = _nested_concat_graph()
+    ex = AotExecutor(nodes, params, ["x"], ["z", "k1"], {"x": [1, 16, 8, 8]}, quantize=8)
+    assert [(i[0], i[1]) for i in ex.instructions] == [("conv2d_i8", ["x", "wa"]), ("conv2d_i8", ["x", "wb"]), ("conv2d_i8", ["k1", "wc"]),
+                                                       ("pool_f32", ["k2"]), ("concat", ["pa"])]
+    v = lambda n: ex._values[n].slot
+    part = 16 * 64 * 4
+    z0 = v("z")[0]
+    assert v("k2") == (z0, 3 * part) and v("k1") == (z0, 2 * part) and v("pa") == (z0, part) and v("pb") == (z0 + part, part)
+    assert v("pc") == (z0 + 2 * part, part) and v("m") == (z0 + 3 * part, 3 * part) and v("z")[1] == 7 * part
+    assert ex._calls[4][2] == (z0 + 6 * part, part)   # the second pa: copied into the last stretch
+
+
 def test_concat_parts_in_place():
     """Which parts of a one-image Concat get their slot inside its result: values produced by an instruction, the
     value whose Split views are consecutive parts (a C2f block: the views follow it), not the graph input, not a
@@ -196,6 +225,27 @@ def test_concat_of_all_split_parts_reads_the_split_source():
         ex.read_output("a")
     keep_a = AotExecutor(nodes, params, ["x"], ["z", "a"], {"x": [2, 16, 8, 8]}, quantize=8)
     assert [i[0] for i in keep_a.instructions].count("slice_f32") == 2 and keep_a.kept("a")
+
+
+@pytest.mark.gpu
+def test_forward_with_nested_concat_parts_in_place():
+    """Concat results placed inside Concat results: every value equal, bit for bit, to the plan that copies."""
+    nodes, params = _nested_concat_graph()
+    x = np.random.default_rng(5).uniform(-1, 1, (1, 16, 24, 24)).astype(np.float32)
+    outs = ["z", "k2", "k1", "m", "pc", "pb", "pa"]
+    got = {}
+    for in_place in (True, False):
+        ex = AotExecutor(nodes, params, ["x"], outs, {"x": list(x.shape)}, quantize=8, concat_in_place=in_place)
+        try:
+            ex.forward({"x": x})
+            got[in_place] = ex.forward({"x": x})
+            assert ex.replayed
+        finally:
+            ex.close()
+    for n in outs:
+        assert np.array_equal(got[True][n], got[False][n]), n
+    g = got[True]
+    assert np.array_equal(g["z"], np.concatenate([g["pa"], g["pb"], g["pc"], g["m"], g["pa"]], axis=1))
 
 
 @pytest.mark.gpu
