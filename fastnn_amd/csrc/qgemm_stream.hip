@@ -69,16 +69,18 @@ int fnn_stream_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w,
     if (cb) { lo = lo < 5 ? lo : 5; hi = hi >= 32 ? 64 : hi; }
     // A long K over few output columns (the down projection of an MLP): the one-launch kernels for M <= 16 give every
     // workgroup whole rows -- few workgroups, each converting M x K activations -- while this kernel splits K over the
-    // chip and its time hardly depends on M.  From M = 9 where K >= 2 N (11008 -> 4096 I4: 16.9-17.2 against 22.7-23.6 us)
-    // and from M = 5 where N <= 2048 and K >= 4 N (8192 -> 2048 FP8: 12.0-12.4 against 13.0-15.8 us; 16384 -> 1024 I4:
-    // 13.7 against 20.2-20.8 us).  Not when the option was raised above its default.
+    // chip and its time hardly depends on M.  From M = 9 where K >= 4 N, or K >= 2 N from K = 8192 on (11008 -> 4096 I4:
+    // 16.7-17.2 against 22.1-23.6 us; 4096 -> 1024 I8: 8.7 against 9.5; but 4096 -> 2048: 10.6 against 9.7, left out);
+    // from M = 5 only where N <= 2048 and K >= 4 N with K >= 8192 (f16 types: 8192 -> 2048 FP8 12.0-12.2 against
+    // 13.0-13.3 us) or K >= 16384 (types of the int8 GEMV, which is the better kernel below that: 16384 -> 1024 I4 13.7
+    // against 20.2-20.8 us, 8192 -> 1024 I4 13.2 against 11.4).  Not when the option was raised above its default.
+    const bool int_type = dt == FNN_DT_I8 || dt == FNN_DT_I4 || dt == FNN_DT_U4;
     if (!cb && lo <= 17) {
-        if (q.k >= 2 * q.n) lo = lo < 9 ? lo : 9;
-        if (q.n <= 2048 && q.k >= 4 * q.n) lo = lo < 5 ? lo : 5;
+        if (q.k >= 4 * q.n || (q.k >= 2 * q.n && q.k >= 8192)) lo = lo < 9 ? lo : 9;
+        if (q.n <= 2048 && q.k >= 4 * q.n && q.k >= (int_type ? 16384 : 8192)) lo = lo < 5 ? lo : 5;
     }
     if (q.m < lo || q.m > hi || q.m > (cb ? 64 : 32) || q.n < 1) return FNN_OK;
     if (flags & FNN_FLAG_ACT_F16_SINGLE) return FNN_OK;
-    const bool int_type = dt == FNN_DT_I8 || dt == FNN_DT_I4 || dt == FNN_DT_U4;
     if (cb && fnn_ctx_option(ctx, FNN_OPT_CODEBOOK_EXPANDED) != 0) return FNN_OK;   // (the option names a form of the tiled path)
     if (cb && (q.as_written || q.qblock != 32 || q.k % 128 != 0 || q.bpr != q.k / 32 || (reinterpret_cast<uintptr_t>(q.scales) & 15) ||
                q.bpr * 4 * 256 >= (int64_t)1 << 31)) return FNN_OK;

@@ -377,12 +377,13 @@ def test_streaming_matmul_takes_the_default_route_and_propagates_non_finite_rows
 
 
 @pytest.mark.parametrize("dt", [flib.DT_I8, flib.DT_I4, flib.DT_U8, flib.DT_F8, flib.DT_F4])
-@pytest.mark.parametrize("m,k,n", [(5, 2048, 512), (8, 4096, 1000), (12, 8192, 2048), (16, 4096, 768), (9, 4096, 2040), (16, 5504, 2600)])
+@pytest.mark.parametrize("m,k,n", [(5, 8192, 512), (8, 16384, 256), (12, 8192, 2048), (16, 4096, 768), (9, 8192, 4000), (16, 4096, 2040), (8, 4096, 1000)])
 def test_streaming_matmul_narrow_outputs_from_m5(ctx, orc, dt, m, k, n):
-    """A long K over few output columns: the streaming kernel takes 9 <= M <= 16 where K >= 2 N and 5 <= M <= 16 where
-    N <= 2048 and K >= 4 N (the one-launch kernels for those M give a workgroup whole rows: few workgroups, each
-    converting all activations).  Against the oracle with bias + SiLU, the same bits on two calls, and another kernel
-    than the one that runs with the streaming kernel off."""
+    """A long K over few output columns: the streaming kernel takes 9 <= M <= 16 where K >= 4 N (K >= 2 N from K = 8192
+    on) and 5 <= M <= 8 where N <= 2048, K >= 4 N and K >= 8192 (16384 for the types of the int8 GEMV): the one-launch
+    kernels for those M give a workgroup whole rows, few workgroups here, each converting all activations.  Against the
+    oracle with bias + SiLU, the same bits on two calls, and another kernel than the one that runs with the streaming
+    kernel off exactly where the rule says so."""
     rng = np.random.default_rng(5500 + dt * 11 + m)
     pw = fastnn_amd.quantize_weights(dt, _weights(rng, n, k))
     a = rng.standard_normal((m, k)).astype(np.float32)
@@ -400,7 +401,9 @@ def test_streaming_matmul_narrow_outputs_from_m5(ctx, orc, dt, m, k, n):
     finally:
         ctx.set_option(flib.OPT_STREAM_MAX_M, 32)
     assert_close(other, want, TOL_F32)
-    assert not np.array_equal(got, other), "the streaming kernel did not take the call"
+    int_type = dt in (flib.DT_I8, flib.DT_I4)
+    takes = (m >= 9 and (k >= 4 * n or (k >= 2 * n and k >= 8192))) or (n <= 2048 and k >= 4 * n and k >= (16384 if int_type else 8192))
+    assert np.array_equal(got, other) != takes, "the streaming kernel " + ("did not take" if takes else "took") + " the call"
     ctx.release(h)
 
 
