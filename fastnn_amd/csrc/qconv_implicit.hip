@@ -983,6 +983,9 @@ int implicit_form(const fnn_hip_weight *w, const QConvArgs &p, int option)
     // the pixels fill the chip several times (102 400 pixels, 64 channels: 18.3 / 28.1 / 23.0).
     if (ocg <= 32 && rows >= 2048) return 1;
     if (ocg <= 64 && rows >= 65536) return 1;
+    // ... or, whatever the channels, a K of one or two steps under many pixels: nothing to save by quantising once
+    // (25 088 pixels, 64 -> 256 1x1: 20.8 / 26.6 / 23.9)
+    if (kk <= 64 && rows >= 12800) return 1;
     // The fused kernel quantises once for all channels: ahead from 33 channels on where its workgroups (32 pixels each)
     // fill half the chip (25 600 pixels: 64 -> 64 3x3 18.6 / 20.9 / 15.7, 384 -> 128 1x1 23.3 / 25.3 / 18.9, 64 -> 128 3x3
     // stride 2 38.1 / 32.0 / 25.5; not 128 -> 256 3x3 at 6400 pixels: 46 / 25 / 28), and with fewer workgroups while a
@@ -992,7 +995,7 @@ int implicit_form(const fnn_hip_weight *w, const QConvArgs &p, int option)
         const int64_t wgs = (rows + 31) / 32, nsteps = (kk + 31) / 32, passes = (ocg + 127) / 128;
         if (wgs >= 128) {
             if (!(ocg > 128 && nsteps > 18)) return 2;
-        } else if (nsteps * passes <= 12) {
+        } else if (nsteps * passes <= 12 || (wgs >= 96 && nsteps * passes <= 20)) {   // (3136 pixels, 64 -> 64 3x3: 14.6 / 14.9 / 12.9)
             return 2;
         }
     }
