@@ -36,7 +36,7 @@ bool plan_stream(int bits, int max_tiles, int max_mb, int64_t m, int64_t n, int6
     // 4096 x 11008 (688 workgroups): 25.0 against 23.5; M = 64 on 4096 x 4096: 21.3 against 20.0.
     if (forced == 0 && ntiles * splits > 320) {
         // Wide outputs: two row tiles per wave (256 weight rows per workgroup) and as few rounds per workgroup as keep the
-        // launch within one round of workgroups.  4096 x 11008 (43 column tiles): 4 splits x 2 rounds of 512, 172 workgroups,
+        // launch within one round of workgroups (one workgroup of this form per CU: at most 256).  4096 x 11008 (43 column tiles): 4 splits x 2 rounds of 512, 172 workgroups,
         // M = 17 19.2 us against 23.0 on the tiled path, M = 32 21.3 against 23.9 (8 splits x 1 round, 344 workgroups: 25.5).
         if (mb * 2 > max_tiles) return false;
         const int64_t ntiles2 = (n + FNN_STREAM_NW * 2 * 16 - 1) / (FNN_STREAM_NW * 2 * 16);
@@ -44,7 +44,7 @@ bool plan_stream(int bits, int max_tiles, int max_mb, int64_t m, int64_t n, int6
         for (int64_t r2 = 1; r2 <= 4; r2++) {
             const int64_t s2 = (total512 + r2 - 1) / r2;
             if (s2 > 64 || (s2 - 1) * r2 >= total512) continue;   // (no empty split)
-            if (ntiles2 * s2 > 320) continue;
+            if (ntiles2 * s2 > 256) continue;   // (one workgroup of this form per CU: 270 workgroups on 5120 x 13824 ran 33.7 us against 28.0 on the tiled path)
             if (ntiles2 * s2 < 128) break;                        // (too few workgroups: the tiled path is ahead)
             *out = StreamPlan{mb, 2, 512, (int)s2, (int)r2, (int)ntiles2};
             return true;
