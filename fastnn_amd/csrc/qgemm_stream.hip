@@ -76,6 +76,12 @@ int fnn_stream_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w,
     // against 20.2-20.8 us, 8192 -> 1024 I4 13.2 against 11.4).  Not when the option was raised above its default.
     const bool int_type = dt == FNN_DT_I8 || dt == FNN_DT_I4 || dt == FNN_DT_U4;
     if (!cb && lo <= 17) {
+        // ... and from M = 9 where K leaves the eight waves of the kernel for 9 <= M <= 16 a ragged last round (its waves
+        // take slices of 512 k-values in turn: 9, 10 or 12 slices are two rounds with half of the waves idle in the
+        // second).  5120 x 13824 I4: 18.0-19.0 against 32.7-34.0 us; 5120 x 5120: 13.4-13.7 against 17.0; 6144 x 6144: 14.4-14.9
+        // against 17.1-17.5; 3072 (six slices, one round) stays: 9.8 against 10.8-11.2.
+        const int64_t nsl = (q.k + 511) / 512, rnds = (nsl + 7) / 8;
+        if (rnds >= 2 && nsl * 4 <= rnds * 8 * 3) lo = lo < 9 ? lo : 9;
         if (q.k >= 4 * q.n || (q.k >= 2 * q.n && q.k >= 8192)) lo = lo < 9 ? lo : 9;
         if (q.n <= 2048 && q.k >= 4 * q.n && q.k >= (int_type ? 16384 : 8192)) lo = lo < 5 ? lo : 5;
     }

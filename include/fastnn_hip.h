@@ -146,7 +146,8 @@ enum {
                                   /* Codebook weights with blocks of 32 (K % 128 == 0): with MAX_M at 32 the kernel takes        */
                                   /* min(MIN_M, 5) <= M <= 64 (a smaller MAX_M is taken as it is).  A long K over few output     */
                                   /* columns, with MIN_M not above its default: from M = 9 where K >= 4 N (K >= 2 N from         */
-                                  /* K = 8192 on), from M = 5 where N <= 2048, K >= 4 N and K >= 8192 (16384 for I8 / I4 / U4)   */
+                                  /* K = 8192 on), from M = 5 where N <= 2048, K >= 4 N and K >= 8192 (16384 for I8 / I4 / U4);  */
+                                  /* from M = 9 also where K / 512 fills the last of two or more rounds of eight at most half    */
     FNN_OPT_STREAM_SHAPE = 21,    /* its launch shape: 0 (default) = by rule, else (splits << 8) | (row tiles per wave << 4) |   */
                                   /* (k-values per round / 256), splits = 0 meaning one round per workgroup                      */
     FNN_OPT_DIGIT_PLANES = 22,    /* int8 matrix-core GEMM (M >= 17, I8 / I4 / U4 weights): activation digit planes, 3 (22 bits     */
