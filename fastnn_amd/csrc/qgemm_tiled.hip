@@ -490,10 +490,22 @@ TileLayout tile_layout(fnn_hip_ctx *ctx, int64_t M, int64_t N, int64_t K, int fl
         const int64_t small_tiles = ((meff + 31) / 32) * ((N + 127) / 128);
         if (small_tiles >= 192 && small_tiles <= 256) cfg = 2;
     }
-    // the dense (expanded codebook) operand from 1024 effective rows on: 256 x 128 tiles on eight waves (twice the waves
-    // that fetch a stage's bytes, and half the weight bytes per row tile).  4096 x 4096, us, 128 x 128 / 256 x 128 tiles:
-    // M = 640 225 / 137, 768 223 / 140, 1024 225 / 155, 2048 436 / 289, 4096 871 / 562; up to M = 512 no gain (91.4 / 91.9)
-    if (dense && meff > 1024) cfg = 3;
+    // the dense (expanded codebook) operand: 256 x 128 tiles on eight waves (twice the waves that fetch a stage's bytes,
+    // and half the weight bytes per row tile) where they need fewer rounds of workgroups.  In units of a 128 x 128 tile's
+    // sweep over K: rounds of 256 workgroups x the share of K per workgroup, a 256 x 128 tile 1.36 of it, plus 0.13 / 0.35
+    // for the partial tiles of a K split (the rules further down).  us, 128 x 128 / 256 x 128 tiles, 4096 x 4096:
+    // M = 256 57 / 86, 384 80 / 92, 512 91 / 92, 640 225 / 137, 1024 225 / 155, 2048 436 / 289, 4096 871 / 562;
+    // 4096 x 11008: M = 192 211 / 151, 256 228 / 152, 384 307 / 230, 512 335 / 247; 11008 x 4096: M = 256 154 / 219; 8192 x 8192: M = 256
+    // 188 / 185, 384 473 / 295, 512 478 / 318, 1024 910 / 607
+    if (dense && meff > 128) {
+        const int64_t nt = (N + 127) / 128, t0 = ((meff + 127) / 128) * nt, t3 = ((meff + 255) / 256) * nt;
+        const int64_t s0 = t0 >= 256 ? 1 : 256 / t0;
+        const double c0 = (double)((t0 * s0 + 255) / 256) / (double)s0 + (s0 > 1 ? 0.13 : 0.0);
+        const double r1 = (double)((t3 + 255) / 256), r2 = (double)((2 * t3 + 255) / 256) / 2.0 + 0.1;
+        const int64_t s3 = r2 < r1 ? 2 : 1;
+        const double c3 = 1.36 * (double)((t3 * s3 + 255) / 256) / (double)s3 + (s3 > 1 ? 0.35 : 0.0);
+        if (c3 < c0) cfg = 3;
+    }
     const int64_t opt_cfg = fnn_ctx_option(ctx, FNN_OPT_TILE_SHAPE);
     // 3 (by option only): 256x128 with 8 waves of 64x64, two waves per SIMD.  Measured on FP8 4096 x 4096 and 2048 -> 8192
     // at M = 128 ... 1024: 0-30 % slower than the automatic choice, except where it turns the tile count into one whole
