@@ -424,10 +424,14 @@ int fnn_digits_qmatmul(fnn_hip_ctx *ctx, hipStream_t s, const fnn_hip_weight *w,
     // faster than one f16 row but measured 1.9e-3 on rows with a few 200x outliers, where a float rounding per
     // element keeps 2.4e-4; three planes cost what the f16 row costs.
     if (flags & FNN_FLAG_ACT_F16_SINGLE) return FNN_OK;
+    // Small weights stay with the f16 tiles as well (by rule; FNN_OPT_DIGIT_PLANES = 3 or 4 or FNN_OPT_GEMM_INT8_MIN_M
+    // below its default still bring them here): 1024 x 1024 I4 at M = 48 / 256 / 1024 14.6 / 16.2 / 22.3 us here against 12.9 / 13.6 / 15.9 there, 2048 x 2048 I8
+    // at M = 64 / 512 16.4 / 26.6 against 15.1 / 22.0; from 3072 x 3072 and 8192 x 1024 on this path is ahead
+    int64_t planes = fnn_ctx_option(ctx, FNN_OPT_DIGIT_PLANES);
+    if (planes != 3 && planes != 4 && q.n * q.k <= (int64_t)2048 * 2048 && fnn_ctx_option(ctx, FNN_OPT_GEMM_INT8_MIN_M) >= 17) return FNN_OK;
     // Planes by shape: three wherever they measured faster than four, i.e. 4-bit weights at every M (4096 x 11008: M = 64
     // 26.3 against 29.3 us, M = 128 30.9 against 40.2, M = 256 47.2 against 54.9, M = 1024 139 against 168) and 8-bit
     // weights from M = 96 (4096 x 4096: M = 64 21.6 against 19.1, M = 128 23.1 against 24.2, M = 512 40.7 against 49.7).
-    int64_t planes = fnn_ctx_option(ctx, FNN_OPT_DIGIT_PLANES);
     if (planes != 3 && planes != 4) planes = (dt == FNN_DT_I8 && q.m < 96) ? 4 : 3;
     // 8-bit weights decode to f16 with one permute per pair, so at four planes the int8 form only ties the f16 tiles
     // (hi + lo rows) and falls 4-5 % behind them from M = 1024 on (4096 x 4096: 93 vs 89 us, M = 2048: 172 vs 164); at

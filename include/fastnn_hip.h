@@ -114,7 +114,9 @@ enum {
                                   /* 0: the f16 GEMV kernel takes them too                                             */
     FNN_OPT_GEMM_INT8 = 10,       /* 1 (default): M >= FNN_OPT_GEMM_INT8_MIN_M with I8 / I4 / U4 weights runs as an int8  */
                                   /* matrix-core GEMM over three or four exact activation digit planes (not in the single-rounding */
-                                  /* mode); 0: the f16 tiled GEMM takes them too                                          */
+                                  /* mode, and by rule not weights of up to 2048 x 2048 elements, which the f16 tiles    */
+                                  /* serve faster: FNN_OPT_DIGIT_PLANES = 3 / 4 or a smaller MIN_M brings them here);     */
+                                  /* 0: the f16 tiled GEMM takes them too                                                 */
     FNN_OPT_GEMM_INT8_MIN_M = 11, /* smallest M of that path (default 17)                                                 */
     FNN_OPT_CODEBOOK_EXPANDED = 12, /* codebook weights with blocks of 32 at M >= 5: 0 (default) = by M (the streaming       */
                                   /* MatMul up to M = 64, beyond it decoded inside the tiled GEMM where that measured      */

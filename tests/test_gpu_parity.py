@@ -501,11 +501,15 @@ def test_int8_digit_plane_gemm_non_finite_rows(ctx, orc):
     pw = fastnn_amd.quantize_weights(flib.DT_I4, _weights(rng, n, k))
     a = rng.standard_normal((m, k)).astype(np.float32)
     h = ctx.register(pw)
-    clean = ctx.qmatmul(h, a, n)
-    a[0, 700] = np.nan
-    a[20, 3] = np.inf
-    a[32, 1023] = -np.inf
-    got = ctx.qmatmul(h, a, n)
+    ctx.set_option(flib.OPT_DIGIT_PLANES, 3)   # (weights this small go to the f16 tiles by rule)
+    try:
+        clean = ctx.qmatmul(h, a, n)
+        a[0, 700] = np.nan
+        a[20, 3] = np.inf
+        a[32, 1023] = -np.inf
+        got = ctx.qmatmul(h, a, n)
+    finally:
+        ctx.set_option(flib.OPT_DIGIT_PLANES, 0)
     for r in (0, 20, 32):
         assert np.isnan(got[r]).all()
     keep = [r for r in range(m) if r not in (0, 20, 32)]
